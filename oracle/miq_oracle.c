@@ -1,0 +1,714 @@
+/*
+ * TEST INFRASTRUCTURE ONLY.
+ *
+ * CPU restatement, in plain C, of the arithmetic of the reference's quantization-simulation hot path
+ * (the v1 / DlQuantization CPU loops and the v2 torch formulas).  It exists so that the HIP kernels can be
+ * compared bit-for-bit with an independent, single-threaded statement of the same arithmetic.  Nothing in the
+ * product package links, loads or calls this file: only tests/, the smoke check and the bench's CPU-baseline
+ * leg do.
+ *
+ * Every function names the reference lines it follows.  Paths are relative to the reference root:
+ *   DLQ   = ModelOptimizations/DlQuantization
+ *   TSRC  = TrainingExtensions/torch/src
+ *   TORCH = TrainingExtensions/torch/src/python/aimet_torch
+ *
+ * Build: gcc -O2 -std=c11 -ffp-contract=off -fno-fast-math (see oracle/Makefile).  The float/double/int type of
+ * every intermediate below is deliberate: it is the type the reference's C++ expression has after the usual
+ * arithmetic conversions with DTYPE = float.
+ *
+ * Pin status (what each function is checked against lives in tests/test_oracle_*.py):
+ *   every function here is pinned by the reference's own golden vectors and/or by the compiled reference
+ *   (oracle/_ref), except where its comment says "parity unpinned".
+ */
+#include <float.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_PDF_SIZE 512 /* DLQ/src/math_functions.hpp:80 */
+
+/* std::max(a, b) and std::min(a, b) exactly as libstdc++ evaluates them (this fixes which operand survives a NaN);
+ * the arguments below are always written in the reference's order. */
+#define STD_MAX(a, b) (((a) < (b)) ? (b) : (a))
+#define STD_MIN(a, b) (((b) < (a)) ? (b) : (a))
+
+typedef struct
+{
+    double min, max, delta, offset;
+    int bw;
+} orc_encoding; /* DLQ/include/DlQuantization/Quantization.hpp:113-120 */
+
+typedef struct
+{
+    double xLeft[ORC_PDF_SIZE];
+    double pdf[ORC_PDF_SIZE];
+    int iterations;
+    int initialized;   /* xLeft.size() != 0 in the reference */
+    int stats_updated; /* _statsUpdated */
+} orc_pdf;             /* DLQ/src/math_functions.hpp:59-67 + TfEnhancedEncodingAnalyzer.h:98-99 */
+
+/* ------------------------------------------------------------------------------------------------------------
+ * bf16 <-> f32 (round to nearest even), the conversion torch's .to(torch.bfloat16) performs
+ * (TORCH/v1/tensor_quantizer.py:1129-1138 upcasts the input and casts the result back).
+ * ---------------------------------------------------------------------------------------------------------- */
+float orc_bf16_to_f32(uint16_t h)
+{
+    uint32_t u = ((uint32_t) h) << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+uint16_t orc_f32_to_bf16(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) /* NaN: quiet it, keep sign */
+        return (uint16_t) ((u >> 16) | 0x0040u);
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;
+    return (uint16_t) (u >> 16);
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * a2  encoding from (min, max, bw)
+ * ---------------------------------------------------------------------------------------------------------- */
+
+/* DLQ/src/quantization_utils.cpp:145-156, EPSILON = 1e-5 (quantization_utils.hpp:51) */
+void orc_gate_min_max(double* mn, double* mx)
+{
+    *mn = fmin(*mn, 0.0);
+    *mx = fmax(*mx, 0.0);
+    *mx = fmax(*mx, *mn + 1e-5);
+}
+
+/* DLQ/src/TensorQuantizationSim.cpp:62-92 (generateScaleOffset + fillEncodingInfo),
+ * DLQ/src/trim_functions.cpp:61-73 (computeDelta / computeOffset: C round(), half away from zero) */
+void orc_fill_encoding_info(int bw, double mn, double mx, orc_encoding* e)
+{
+    orc_gate_min_max(&mn, &mx);
+    double numSteps = pow(2, bw) - 1;
+    if (mn == -mx)
+        numSteps -= 1;
+    double delta  = (mx - mn) / numSteps;
+    double offset = round(mn / delta);
+    e->bw         = bw;
+    e->delta      = delta;
+    e->offset     = offset;
+    e->min        = offset * delta;
+    e->max        = delta * numSteps + e->min;
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * a3  per-element quantize / dequantize, DTYPE = float
+ * ---------------------------------------------------------------------------------------------------------- */
+
+/* DLQ/src/trim_functions.cpp:141-165 with ROUND_NEAREST: clamp, scale, subtract offset, roundf */
+static inline float orc_quantize_value(float x, float mn, float mx, float delta, float offset)
+{
+    float t = fmaxf(fminf(x, mx), mn);
+    t       = t / delta - offset;
+    return roundf(t);
+}
+
+/* DLQ/src/trim_functions.cpp:167-171 */
+static inline float orc_dequantize_value(float q, float delta, float offset)
+{
+    return delta * (q + offset);
+}
+
+/* DLQ/src/TensorQuantizationSim.cpp:104-114 -> trim_functions.cpp:174-182 */
+void orc_qdq_per_tensor_f32(const float* in, int64_t n, float* out, double encMin, double encMax, int bw)
+{
+    orc_encoding e;
+    orc_fill_encoding_info(bw, encMin, encMax, &e);
+    float mn = (float) e.min, mx = (float) e.max, d = (float) e.delta, o = (float) e.offset;
+    for (int64_t i = 0; i < n; ++i)
+        out[i] = orc_dequantize_value(orc_quantize_value(in[i], mn, mx, d, o), d, o);
+}
+
+/* DLQ/src/TensorQuantizationSim.cpp:116-126 -> trim_functions.cpp:203-218.
+ * shift = 2^(bw-1) as unsigned int; out[i] -= shift is a float subtraction. */
+void orc_quantize_per_tensor_f32(const float* in, int64_t n, float* out, double encMin, double encMax, int bw,
+                                 int shiftToSigned)
+{
+    orc_encoding e;
+    orc_fill_encoding_info(bw, encMin, encMax, &e);
+    float mn = (float) e.min, mx = (float) e.max, d = (float) e.delta, o = (float) e.offset;
+    unsigned int shift = 0;
+    if (shiftToSigned)
+        shift = (unsigned int) pow(2, bw - 1);
+    for (int64_t i = 0; i < n; ++i)
+    {
+        float q = orc_quantize_value(in[i], mn, mx, d, o);
+        q -= (float) shift;
+        out[i] = q;
+    }
+}
+
+/* Same arithmetic with bf16 storage: upcast, QDQ in float, round the result back to bf16
+ * (TORCH/v1/tensor_quantizer.py:1129-1138). */
+void orc_qdq_per_tensor_bf16(const uint16_t* in, int64_t n, uint16_t* out, double encMin, double encMax, int bw)
+{
+    orc_encoding e;
+    orc_fill_encoding_info(bw, encMin, encMax, &e);
+    float mn = (float) e.min, mx = (float) e.max, d = (float) e.delta, o = (float) e.offset;
+    for (int64_t i = 0; i < n; ++i)
+    {
+        float x = orc_bf16_to_f32(in[i]);
+        out[i]  = orc_f32_to_bf16(orc_dequantize_value(orc_quantize_value(x, mn, mx, d, o), d, o));
+    }
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * a5  per-channel QDQ
+ * ---------------------------------------------------------------------------------------------------------- */
+
+/* TSRC/AimetTensorQuantizer.cpp:209-227, 268-297: the per-channel parameters are derived with float32 tensor ops:
+ * minimum/maximum with 0, max >= min + 1e-5 (added in float), delta = (max - min) / numSteps,
+ * offset = at::round(min / delta) which rounds half to even.  numSteps comes from encodings[0] only. */
+void orc_per_channel_params_f32(const double* encMin, const double* encMax, int64_t numChannel, int bw, float* mn,
+                                float* mx, float* delta, float* offset)
+{
+    double numSteps = pow(2, bw) - 1;
+    if (encMin[0] == -encMax[0])
+        numSteps -= 1;
+    float numStepsF = (float) numSteps;
+    for (int64_t c = 0; c < numChannel; ++c)
+    {
+        float lo  = (float) encMin[c];
+        float hi  = (float) encMax[c];
+        lo        = (lo < 0.0f) ? lo : 0.0f;
+        hi        = (hi > 0.0f) ? hi : 0.0f;
+        float eps = lo + 1e-5f;
+        hi        = (hi > eps) ? hi : eps;
+        float d   = (hi - lo) / numStepsF;
+        mn[c]     = lo;
+        mx[c]     = hi;
+        delta[c]  = d;
+        offset[c] = rintf(lo / d);
+    }
+}
+
+/* DLQ/src/trim_functions.cpp:698-709 */
+void orc_qdq_per_channel_f32(const float* in, int64_t numChannel, int64_t numElement, int64_t numElementPerChannel,
+                             float* out, const float* mn, const float* mx, const float* delta, const float* offset)
+{
+    for (int64_t i = 0; i < numElement; ++i)
+    {
+        int64_t c = (i / numElementPerChannel) % numChannel;
+        out[i] = orc_dequantize_value(orc_quantize_value(in[i], mn[c], mx[c], delta[c], offset[c]), delta[c], offset[c]);
+    }
+}
+
+/* quantize only (the float-valued grid index), per channel; used to pin integer codes */
+void orc_quantize_per_channel_f32(const float* in, int64_t numChannel, int64_t numElement,
+                                  int64_t numElementPerChannel, float* out, const float* mn, const float* mx,
+                                  const float* delta, const float* offset)
+{
+    for (int64_t i = 0; i < numElement; ++i)
+    {
+        int64_t c = (i / numElementPerChannel) % numChannel;
+        out[i]    = orc_quantize_value(in[i], mn[c], mx[c], delta[c], offset[c]);
+    }
+}
+
+void orc_qdq_per_channel_bf16(const uint16_t* in, int64_t numChannel, int64_t numElement,
+                              int64_t numElementPerChannel, uint16_t* out, const float* mn, const float* mx,
+                              const float* delta, const float* offset)
+{
+    for (int64_t i = 0; i < numElement; ++i)
+    {
+        int64_t c = (i / numElementPerChannel) % numChannel;
+        float x   = orc_bf16_to_f32(in[i]);
+        out[i]    = orc_f32_to_bf16(
+            orc_dequantize_value(orc_quantize_value(x, mn[c], mx[c], delta[c], offset[c]), delta[c], offset[c]));
+    }
+}
+
+/* DLQ/src/trim_functions.cpp:634-660: numpy-style broadcast of the encoding over the input.
+ * The reference keeps the running remainder and the indices in `int`. */
+void orc_qdq_broadcast_f32(const float* in, float* out, int64_t numElement, int64_t numDims,
+                           const int64_t* inputStrides, const int64_t* encodingStrides, const float* mn,
+                           const float* mx, const float* delta, const float* offset)
+{
+    for (int64_t i = 0; i < numElement; ++i)
+    {
+        int encIdx    = 0;
+        int remainder = (int) i;
+        for (int64_t dim = 0; dim < numDims; ++dim)
+        {
+            int dimIdx = (int) (remainder / inputStrides[dim]);
+            remainder  = (int) (remainder - dimIdx * inputStrides[dim]);
+            encIdx += (int) (encodingStrides[dim] * dimIdx);
+        }
+        out[i] = orc_dequantize_value(orc_quantize_value(in[i], mn[encIdx], mx[encIdx], delta[encIdx], offset[encIdx]),
+                                      delta[encIdx], offset[encIdx]);
+    }
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * a6  straight-through backward of the v1 path
+ * TORCH/v1/quantsim_straight_through_grad.py:91-118: grad * ((min <= x) & (x <= max)), both ends inclusive,
+ * min/max being the encoding's stored values converted to float32.
+ * ---------------------------------------------------------------------------------------------------------- */
+void orc_ste_bwd_per_tensor_f32(const float* x, const float* gout, float* gin, int64_t n, float mn, float mx)
+{
+    for (int64_t i = 0; i < n; ++i)
+        gin[i] = gout[i] * (float) ((mn <= x[i]) && (x[i] <= mx));
+}
+
+void orc_ste_bwd_per_channel_f32(const float* x, const float* gout, float* gin, int64_t numChannel,
+                                 int64_t numElement, int64_t numElementPerChannel, const float* mn, const float* mx)
+{
+    for (int64_t i = 0; i < numElement; ++i)
+    {
+        int64_t c = (i / numElementPerChannel) % numChannel;
+        gin[i]    = gout[i] * (float) ((mn[c] <= x[i]) && (x[i] <= mx[c]));
+    }
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * a9  min/max statistics and the TF (min/max) encoding
+ * ---------------------------------------------------------------------------------------------------------- */
+
+/* DLQ/src/math_functions.cpp:328-347: std::min/std::max against a running value that starts at -/+DBL_MAX cast
+ * to float (= -/+inf); NaN inputs never replace the running value. */
+void orc_minmax_f32(const float* in, int64_t n, float* mnOut, float* mxOut)
+{
+    float mx = -INFINITY, mn = INFINITY;
+    for (int64_t i = 0; i < n; ++i)
+    {
+        mx = STD_MAX(mx, in[i]);
+        mn = STD_MIN(mn, in[i]);
+    }
+    *mnOut = mn;
+    *mxOut = mx;
+}
+
+/* DLQ/src/quantization_utils.cpp:58-143 */
+void orc_get_computed_encodings(int bw, double mn, double mx, int sym, int strict, int unsignedSym, orc_encoding* e)
+{
+    double numSteps = pow(2, bw) - 1;
+    if (sym && strict)
+        numSteps -= 1;
+    e->bw = bw;
+    if (isinf(mn))
+        mn = -(double) FLT_MAX;
+    if (isinf(mx))
+        mx = (double) FLT_MAX;
+
+    if (sym && ((mn < 0.0) || !unsignedSym))
+    {
+        mx                       = fmax(fabs(mx), fabs(mn));
+        unsigned int numPosSteps = (unsigned int) floor(numSteps / 2);
+        e->delta                 = mx / numPosSteps;
+        e->offset                = -ceil(numSteps / 2);
+        e->min                   = fmax(e->offset * e->delta, -(double) FLT_MAX);
+        e->max                   = fmin(e->delta * numPosSteps, (double) FLT_MAX);
+        return;
+    }
+    e->delta = (mx - mn) / numSteps;
+    if (mn < 0 && mx > 0)
+    {
+        double bZero = round(-mn / e->delta);
+        bZero        = fmin(numSteps, fmax(0.0, bZero));
+        e->offset    = -bZero;
+    }
+    else
+    {
+        e->offset = round(mn / e->delta);
+        e->min    = mn;
+        e->max    = mx;
+        return;
+    }
+    double t = e->delta * e->offset;
+    if (t >= -(double) FLT_MAX && t <= (double) FLT_MAX)
+        e->min = t;
+    else
+        e->min = -(double) FLT_MAX;
+    e->max = mx - mn + e->min;
+    if (e->max > (double) FLT_MAX)
+        e->max = (double) FLT_MAX;
+}
+
+/* DLQ/src/TfEncodingAnalyzer.cpp:80-101, MIN_RANGE = 0.01 (TfEncodingAnalyzer.h:81) */
+void orc_tf_compute_encoding(double accMin, double accMax, int bw, int sym, int strict, int unsignedSym,
+                             orc_encoding* e)
+{
+    double newMin = fmin(0.0, accMin);
+    double newMax = fmax(0.0, accMax);
+    newMax        = fmax(newMax, newMin + 0.01);
+    orc_get_computed_encodings(bw, newMin, newMax, sym, strict, unsignedSym, e);
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * a10  512-bucket PDF accumulation (signed_vals = true, the only mode the TF-Enhanced analyzer uses)
+ * ---------------------------------------------------------------------------------------------------------- */
+void orc_pdf_reset(orc_pdf* p)
+{
+    memset(p, 0, sizeof(*p));
+}
+
+/* DLQ/src/math_functions.cpp:208-241 */
+static void orc_initialize_pdf(orc_pdf* p, float minVal, float maxVal)
+{
+    if (minVal == maxVal)
+    {
+        float t = minVal + (float) 0.01;
+        maxVal  = STD_MAX(maxVal, t);
+    }
+    float center = (maxVal + minVal) / 2;
+    float lo     = center - 3 * (center - minVal);
+    float hi     = center + 3 * (maxVal - center);
+    minVal       = STD_MAX(-FLT_MAX, lo);
+    maxVal       = STD_MIN(FLT_MAX, hi);
+    double bucket = ((double) maxVal - (double) minVal) / ORC_PDF_SIZE;
+    for (int i = 0; i < ORC_PDF_SIZE; ++i)
+    {
+        p->xLeft[i] = minVal + i * bucket;
+        p->pdf[i]   = 0.0;
+    }
+    p->iterations  = 0;
+    p->initialized = 1;
+}
+
+/* DLQ/src/math_functions.cpp:368-384.  The reference converts the rounded float straight to int, which for NaN and
+ * for values beyond the int range is the x86 "integer indefinite" INT_MIN and is therefore dropped by the range
+ * test; comparing in float before converting gives the same outcome without relying on that. */
+void orc_histogram_f32(const float* data, int64_t n, uint32_t* hist, float bucket, float pdfOffset)
+{
+    for (int64_t i = 0; i < n; ++i)
+    {
+        float r = roundf(data[i] / bucket - pdfOffset);
+        if (r >= 0.0f && r < (float) ORC_PDF_SIZE)
+            hist[(int) r] += 1;
+    }
+}
+
+/* DLQ/src/math_functions.cpp:244-288 + TfEnhancedEncodingAnalyzer.cpp:68-76.
+ * histOut (may be NULL) receives this batch's 512 integer bin counts. */
+void orc_pdf_update_f32(orc_pdf* p, const float* data, int64_t n, uint32_t* histOut)
+{
+    uint32_t hist[ORC_PDF_SIZE];
+    memset(hist, 0, sizeof(hist));
+    if (histOut)
+        memset(histOut, 0, sizeof(hist));
+    p->stats_updated = 1;
+    if (!p->initialized)
+    {
+        float mn, mx;
+        orc_minmax_f32(data, n, &mn, &mx);
+        if (mn == 0 && mx == 0)
+            return;
+        orc_initialize_pdf(p, mn, mx);
+    }
+    float bucket    = (float) (p->xLeft[1] - p->xLeft[0]);
+    float minVal    = (float) p->xLeft[0];
+    float pdfOffset = minVal / bucket;
+    orc_histogram_f32(data, n, hist, bucket, pdfOffset);
+    int cnt = (int) n;
+    for (int i = 0; i < ORC_PDF_SIZE; ++i)
+    {
+        double prob = (double) hist[i] / (double) cnt;
+        p->pdf[i]   = (p->pdf[i] * p->iterations + prob) / (p->iterations + 1);
+    }
+    p->iterations++;
+    if (histOut)
+        memcpy(histOut, hist, sizeof(hist));
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * a11  TF-Enhanced (SQNR) candidate search
+ * ---------------------------------------------------------------------------------------------------------- */
+
+/* DLQ/src/TfEnhancedEncodingAnalyzer.cpp:255-291, MIN_RANGE = 0.01 (.h:105) */
+void orc_tfe_find_range(const orc_pdf* p, float* minOut, float* maxOut)
+{
+    float minVal = (float) p->xLeft[0];
+    float maxVal = (float) p->xLeft[ORC_PDF_SIZE - 1];
+    for (int i = 0; i < ORC_PDF_SIZE; ++i)
+        if (p->pdf[i] > 0)
+        {
+            minVal = (float) p->xLeft[i];
+            break;
+        }
+    for (int i = ORC_PDF_SIZE - 1; i > 0; --i)
+        if (p->pdf[i] > 0)
+        {
+            maxVal = (float) p->xLeft[i];
+            break;
+        }
+    minVal  = STD_MIN(minVal, 0.0f);
+    maxVal  = STD_MAX(maxVal, 0.0f);
+    float t = minVal + (float) 0.01;
+    maxVal  = STD_MAX(maxVal, t);
+    *minOut = minVal;
+    *maxOut = maxVal;
+}
+
+/* DLQ/src/TfEnhancedEncodingAnalyzer.cpp:149-175 */
+static int orc_tfe_clamp_to_observed(float obsMin, float obsMax, float numSteps, float* testDelta, int* testOffset)
+{
+    float tMin = *testDelta * (float) *testOffset;
+    tMin       = STD_MAX(tMin, -FLT_MAX);
+    float tMax = *testDelta * ((float) *testOffset + numSteps);
+    tMax       = STD_MIN(tMax, FLT_MAX);
+    if ((tMin < obsMin) && (tMax > obsMax))
+        return 0;
+    tMin = STD_MAX(obsMin, tMin);
+    tMax = STD_MIN(obsMax, tMax);
+    if (tMin == tMax)
+        return 0;
+    *testDelta  = (float) (((double) tMax - tMin) / numSteps);
+    *testOffset = (int) roundf(tMin / *testDelta);
+    return 1;
+}
+
+/* DLQ/src/TfEnhancedEncodingAnalyzer.cpp:177-214.  The delta factor f is a float that is advanced by adding the
+ * double 1/16 and rounding back to float; the loop bound is compared in double. */
+static int orc_tfe_pick_asymmetric(float obsMin, float obsMax, float numSteps, float* deltas, int* offsets, int maxOut)
+{
+    int n          = 0;
+    float obsDelta = (float) (((double) obsMax - (double) obsMin) / numSteps);
+    int obsOffset  = (int) roundf(obsMin / obsDelta);
+    float t        = obsDelta * (float) obsOffset;
+    obsMin         = STD_MAX(t, -FLT_MAX);
+    t              = obsDelta * ((float) obsOffset + numSteps);
+    obsMax         = STD_MIN(t, FLT_MAX);
+    float deltaMax = obsDelta;
+    for (float f = (float) (1.0 / 16); (double) f <= 1 + 1.0 / 16; f = (float) ((double) f + 1.0 / 16))
+    {
+        for (int i = 0; i <= 20; ++i)
+        {
+            float testDelta = f * deltaMax;
+            int testOffset  = (int) ((double) (-numSteps) + (double) numSteps / 20.0 * i);
+            if (!orc_tfe_clamp_to_observed(obsMin, obsMax, numSteps, &testDelta, &testOffset))
+                continue;
+            if (n < maxOut)
+            {
+                deltas[n]  = testDelta;
+                offsets[n] = testOffset;
+            }
+            ++n;
+        }
+    }
+    if (n < maxOut)
+    {
+        deltas[n]  = obsDelta;
+        offsets[n] = obsOffset;
+    }
+    ++n;
+    return n;
+}
+
+/* DLQ/src/TfEnhancedEncodingAnalyzer.cpp:216-253 */
+static int orc_tfe_pick_symmetric(float minVal, float maxVal, float numSteps, int unsignedSym, float* deltas,
+                                  int* offsets, int maxOut)
+{
+    int n = 0;
+    float deltaMax;
+    int testOffset;
+    if ((minVal == 0.0) && unsignedSym)
+    {
+        deltaMax   = maxVal / numSteps;
+        testOffset = 0;
+    }
+    else
+    {
+        float a    = fabsf(maxVal), b = fabsf(minVal);
+        float absM = STD_MAX(a, b);
+        deltaMax   = (float) (absM / (numSteps / 2.0));
+        testOffset = (int) floorf(-numSteps / 2);
+    }
+    for (float f = (float) (1.0 / 100); (double) f <= 1 + 1.0 / 100; f = (float) ((double) f + 1.0 / 100))
+    {
+        if (n < maxOut)
+        {
+            deltas[n]  = f * deltaMax;
+            offsets[n] = testOffset;
+        }
+        ++n;
+    }
+    return n;
+}
+
+/* Candidate list exactly as DLQ/src/TfEnhancedEncodingAnalyzer.cpp:357-381 builds it; returns the count. */
+int orc_tfe_candidates(const orc_pdf* p, int bw, int sym, int strict, int unsignedSym, float* deltas, int* offsets,
+                       int maxOut)
+{
+    float minVal, maxVal;
+    orc_tfe_find_range(p, &minVal, &maxVal);
+    float numSteps = (float) (pow(2, bw) - 1);
+    if (sym)
+    {
+        if (strict)
+            numSteps -= 1;
+        return orc_tfe_pick_symmetric(minVal, maxVal, numSteps, unsignedSym, deltas, offsets, maxOut);
+    }
+    return orc_tfe_pick_asymmetric(minVal, maxVal, numSteps, deltas, offsets, maxOut);
+}
+
+/* DLQ/src/TfEnhancedEncodingAnalyzer.cpp:293-355, GAMMA = 3.0 (.h:102).  pow(v, 2) of the reference is v*v. */
+double orc_tfe_cost(const orc_pdf* p, int bw, float delta, int offset)
+{
+    float minVal   = delta * (float) offset;
+    float stepSize = (float) (pow(2, bw) - 1);
+    float maxVal   = delta * ((float) offset + stepSize);
+    float pdfStart = (float) p->xLeft[0];
+    double pdfStep = p->xLeft[1] - p->xLeft[0];
+    int minInd     = (int) floor((minVal - pdfStart) / pdfStep);
+    minInd         = (minInd < 0) ? 0 : minInd;
+    minInd         = (minInd > ORC_PDF_SIZE - 1) ? ORC_PDF_SIZE - 1 : minInd;
+    int maxInd     = (int) floor((maxVal - pdfStart) / pdfStep);
+    maxInd         = (maxInd < 0) ? 0 : maxInd;
+    maxInd         = (maxInd > ORC_PDF_SIZE - 1) ? ORC_PDF_SIZE - 1 : maxInd;
+
+    double satBottom = 0;
+    float minMid     = (float) (pdfStart + (minInd * pdfStep) + pdfStep / 2);
+    for (int i = 0; i < minInd; ++i)
+    {
+        double mid = pdfStart + i * pdfStep + pdfStep / 2;
+        double d   = mid - minMid;
+        satBottom += p->pdf[i] * (d * d);
+    }
+    double satTop = 0;
+    float maxMid  = (float) (pdfStart + (maxInd * pdfStep) + pdfStep / 2);
+    for (int i = maxInd; i < ORC_PDF_SIZE; ++i)
+    {
+        double mid = pdfStart + i * pdfStep + pdfStep / 2;
+        double d   = mid - maxMid;
+        satTop += p->pdf[i] * (d * d);
+    }
+    double quant = 0;
+    for (int i = minInd; i < maxInd; ++i)
+    {
+        float fv    = (float) (pdfStart + i * pdfStep + pdfStep / 2);
+        int q       = (int) roundf(fv / delta - (float) offset);
+        float dq    = delta * (float) (q + offset);
+        double diff = (double) (fv - dq);
+        quant += p->pdf[i] * (diff * diff);
+    }
+    double sqnr = 3.0 * (satBottom + satTop) + quant;
+    return (sqnr < DBL_MAX) ? sqnr : DBL_MAX;
+}
+
+/* DLQ/src/TfEnhancedEncodingAnalyzer.cpp:78-147, 357-397.
+ * costsOut / bestIdxOut are optional (NULL) and report every candidate's cost and the winner's position. */
+void orc_tfe_compute_encoding(const orc_pdf* p, int bw, int sym, int strict, int unsignedSym, orc_encoding* e,
+                              double* costsOut, int* bestIdxOut)
+{
+    memset(e, 0, sizeof(*e));
+    float numSteps = (float) (pow(2, bw) - 1);
+    if (bestIdxOut)
+        *bestIdxOut = -1;
+    if (!p->initialized)
+    {
+        if (p->stats_updated)
+        {
+            e->min    = -1;
+            e->max    = 1;
+            e->delta  = (e->max - e->min) / (int) numSteps;
+            e->offset = floor(e->min / e->delta);
+            e->min    = e->offset * e->delta;
+            e->max    = e->min + (int) numSteps * e->delta;
+            e->bw     = bw;
+        }
+        return;
+    }
+    enum { MAXC = 512 };
+    float deltas[MAXC];
+    int offsets[MAXC];
+    int n = orc_tfe_candidates(p, bw, sym, strict, unsignedSym, deltas, offsets, MAXC);
+    if (sym && strict)
+        numSteps -= 1;
+    float bestDelta = -1;
+    int bestOffset  = -1;
+    double bestCost = DBL_MAX;
+    for (int i = 0; i < n; ++i)
+    {
+        double cost = orc_tfe_cost(p, bw, deltas[i], offsets[i]);
+        if (costsOut)
+            costsOut[i] = cost;
+        if (cost < bestCost)
+        {
+            bestCost   = cost;
+            bestDelta  = deltas[i];
+            bestOffset = offsets[i];
+            if (bestIdxOut)
+                *bestIdxOut = i;
+        }
+    }
+    float bMin = bestDelta * (float) bestOffset;
+    bMin       = STD_MAX(bMin, -FLT_MAX);
+    float bMax = bestDelta * ((float) bestOffset + numSteps);
+    bMax       = STD_MIN(bMax, FLT_MAX);
+    e->delta   = bestDelta;
+    e->offset  = bestOffset;
+    e->bw      = bw;
+    e->min     = bMin;
+    e->max     = bMax;
+}
+
+/* ------------------------------------------------------------------------------------------------------------
+ * a7  v2 quantize-dequantize (TORCH/v2/quantization/affine/backends/torch_builtins.py:303-344), float32 internal
+ * dtype.  scale/offset are per "channel" with channel = (i / numElementPerChannel) % numChannel, which covers the
+ * per-tensor ([1]) and per-output-channel ([C,1,...]) broadcast shapes.  torch.round is half-to-even (rintf under
+ * the default rounding mode).  maskOut (optional) receives 1 where qmin <= round(x/s) - o <= qmax.
+ * ---------------------------------------------------------------------------------------------------------- */
+void orc_v2_qdq_f32(const float* in, int64_t numChannel, int64_t numElement, int64_t numElementPerChannel,
+                    float* out, float* codesOut, uint8_t* maskOut, const float* scale, const float* offset, int qmin,
+                    int qmax)
+{
+    for (int64_t i = 0; i < numElement; ++i)
+    {
+        int64_t c  = (i / numElementPerChannel) % numChannel;
+        float r    = rintf(in[i] / scale[c]) - offset[c];
+        int inside = ((float) qmin <= r) && (r <= (float) qmax);
+        float q    = r;
+        if (q < (float) qmin)
+            q = (float) qmin;
+        if (q > (float) qmax)
+            q = (float) qmax;
+        if (codesOut)
+            codesOut[i] = q;
+        if (maskOut)
+            maskOut[i] = (uint8_t) inside;
+        if (out)
+            out[i] = (q + offset[c]) * scale[c];
+    }
+}
+
+void orc_v2_qdq_bf16(const uint16_t* in, int64_t numChannel, int64_t numElement, int64_t numElementPerChannel,
+                     uint16_t* out, uint8_t* maskOut, const float* scale, const float* offset, int qmin, int qmax)
+{
+    for (int64_t i = 0; i < numElement; ++i)
+    {
+        int64_t c  = (i / numElementPerChannel) % numChannel;
+        float r    = rintf(orc_bf16_to_f32(in[i]) / scale[c]) - offset[c];
+        int inside = ((float) qmin <= r) && (r <= (float) qmax);
+        float q    = r;
+        if (q < (float) qmin)
+            q = (float) qmin;
+        if (q > (float) qmax)
+            q = (float) qmax;
+        if (maskOut)
+            maskOut[i] = (uint8_t) inside;
+        out[i] = orc_f32_to_bf16((q + offset[c]) * scale[c]);
+    }
+}
+
+/* torch_builtins.py:329-344: tensor_grad = grad * mask */
+void orc_v2_qdq_bwd_f32(const float* in, const float* gout, int64_t numChannel, int64_t numElement,
+                        int64_t numElementPerChannel, float* gin, const float* scale, const float* offset, int qmin,
+                        int qmax)
+{
+    for (int64_t i = 0; i < numElement; ++i)
+    {
+        int64_t c  = (i / numElementPerChannel) % numChannel;
+        float r    = rintf(in[i] / scale[c]) - offset[c];
+        int inside = ((float) qmin <= r) && (r <= (float) qmax);
+        gin[i]     = gout[i] * (float) inside;
+    }
+}
