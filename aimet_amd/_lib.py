@@ -1,0 +1,96 @@
+"""ctypes binding of libmiq.so (the C ABI declared in include/miq.h).
+
+The library is the only compute path of this package: if it has not been built the import fails with an error that
+says how to build it.  There is no CPU or eager-PyTorch fallback.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmiq.so")
+
+OK = 0
+ROUND_NEAREST, ROUND_STOCHASTIC = 0, 1
+QUANTIZATION_TF, QUANTIZATION_TF_ENHANCED = 0, 1
+PDF_SIZE = 512
+
+
+class MiqError(RuntimeError):
+    """A libmiq entry point returned a non-zero status."""
+
+
+class Encoding(C.Structure):
+    """struct miq_encoding == DlQuantization::TfEncoding"""
+    _fields_ = [("min", C.c_double), ("max", C.c_double), ("delta", C.c_double), ("offset", C.c_double),
+                ("bw", C.c_int)]
+
+
+_p = C.c_void_p
+_i64 = C.c_int64
+_int = C.c_int
+_dbl = C.c_double
+_flt = C.c_float
+
+_SIGNATURES = {
+    "miq_version": ([], _int),
+    "miq_last_error": ([], C.c_char_p),
+    "miq_fill_encoding_info": ([_int, _dbl, _dbl, C.POINTER(Encoding)], _int),
+    "miq_get_computed_encodings": ([_int, _dbl, _dbl, _int, _int, _int, C.POINTER(Encoding)], _int),
+    "miq_qdq_per_tensor_f32": ([_p, _p, _i64, _dbl, _dbl, _int, _int, _p], _int),
+    "miq_qdq_per_tensor_bf16": ([_p, _p, _i64, _dbl, _dbl, _int, _int, _p], _int),
+    "miq_quantize_per_tensor_f32": ([_p, _p, _i64, _dbl, _dbl, _int, _int, _int, _p], _int),
+    "miq_qdq_codes_per_tensor_f32": ([_p, _p, _p, _i64, _dbl, _dbl, _int, _int, _p], _int),
+    "miq_per_channel_params_f32": ([_p, _p, _i64, _dbl, _p, _p, _p, _p, _p], _int),
+    "miq_qdq_per_channel_f32": ([_p, _p, _i64, _i64, _i64, _p, _p, _p, _p, _int, _p], _int),
+    "miq_qdq_per_channel_bf16": ([_p, _p, _i64, _i64, _i64, _p, _p, _p, _p, _int, _p], _int),
+    "miq_qdq_codes_per_channel_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _p, _p, _int, _int, _p], _int),
+    "miq_qdq_broadcast_f32": ([_p, _p, _i64, _i64, C.POINTER(_i64), C.POINTER(_i64), _p, _p, _p, _p, _p], _int),
+    "miq_ste_bwd_per_tensor_f32": ([_p, _p, _p, _i64, _flt, _flt, _p], _int),
+    "miq_ste_bwd_per_tensor_bf16": ([_p, _p, _p, _i64, _flt, _flt, _p], _int),
+    "miq_ste_bwd_per_channel_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _p], _int),
+    "miq_ste_bwd_per_channel_bf16": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _p], _int),
+    "miq_v2_qdq_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p], _int),
+    "miq_v2_qdq_bf16": ([_p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p], _int),
+    "miq_v2_qdq_bwd_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p], _int),
+    "miq_v2_qdq_bwd_bf16": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p], _int),
+    "miq_minmax_f32": ([_p, _i64, _p, _p], _int),
+    "miq_minmax_per_channel_f32": ([_p, _i64, _i64, _i64, _p, _p], _int),
+    "miq_analyzer_create": ([_int, C.POINTER(_p)], _int),
+    "miq_analyzer_destroy": ([_p], _int),
+    "miq_analyzer_reset": ([_p, _p], _int),
+    "miq_analyzer_update_stats_f32": ([_p, _p, _i64, _p], _int),
+    "miq_analyzer_compute_encoding": ([_p, _int, _int, _int, _int, C.POINTER(Encoding), C.POINTER(_int), _p], _int),
+    "miq_analyzer_get_stats_histogram": ([_p, _p, _p, C.POINTER(_int), _p], _int),
+    "miq_analyzer_last_batch_counts": ([_p, _p, _p], _int),
+    "miq_analyzer_last_search": ([_p, _p, _p, _p, _int, C.POINTER(_int), C.POINTER(_int), _p], _int),
+}
+
+# Entry points declared in include/miq.h; the loader insists on every one of them.
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: the HIP kernels have not been built. Build them with "
+            "`make -C aimet_amd/csrc` (or `python -c 'import __graft_entry__ as g; g.build()'`). "
+            "This package has no CPU fallback.")
+    lib = C.CDLL(LIB_PATH)
+    for name, (argtypes, restype) in _SIGNATURES.items():
+        try:
+            fn = getattr(lib, name)
+        except AttributeError as exc:
+            raise ImportError(f"{LIB_PATH} does not export {name}; rebuild it") from exc
+        fn.argtypes = argtypes
+        fn.restype = restype
+    return lib
+
+
+lib = _load()
+
+
+def check(status):
+    """Raise MiqError for a non-zero status (RuntimeError subclass, like the reference's pybind exceptions)."""
+    if status != OK:
+        msg = lib.miq_last_error()
+        raise MiqError(f"libmiq status {status}: {msg.decode() if msg else ''}")

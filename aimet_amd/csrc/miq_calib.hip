@@ -1,0 +1,1029 @@
+// Calibration kernels for gfx950: fused min/max reduction, 512-bucket histogram (PDF) accumulation and the
+// TF-Enhanced (SQNR) delta/offset candidate search.
+//
+// Reference arithmetic followed here (paths relative to the reference root, DLQ = ModelOptimizations/DlQuantization):
+//   GetMin/GetMax                    DLQ/src/math_functions.cpp:328-347
+//   InitializePdf / UpdatePdf        DLQ/src/math_functions.cpp:208-288
+//   GetHistogram_cpu                 DLQ/src/math_functions.cpp:368-384
+//   TfEncodingAnalyzer               DLQ/src/TfEncodingAnalyzer.cpp:59-101
+//   TfEnhancedEncodingAnalyzer       DLQ/src/TfEnhancedEncodingAnalyzer.cpp:78-397
+//
+// Design: every statistic lives in one device-resident state block per analyzer.  update_stats is one streaming
+// kernel per batch in steady state (the first batch adds a min/max pass); the workgroup that finishes last folds
+// the batch's integer bin counts into the running PDF, so nothing is copied to the host and nothing synchronises
+// until an encoding is asked for.  Bin counts are integers, hence independent of the order in which lanes add them.
+// The histogram is privatised in LDS: 16 interleaved copies of the 512 bins per workgroup, lane l using copy
+// l mod 16, so that even when every sample of a wavefront falls into one bin (post-ReLU data) at most two lanes
+// meet on an address.
+#include "miq_common.h"
+
+#include <cfloat>
+#include <cmath>
+#include <cstring>
+#include <new>
+
+namespace miq
+{
+namespace
+{
+constexpr int kPdf      = MIQ_PDF_SIZE;
+constexpr int kMaxCand  = 512;
+constexpr int kCopies   = 16;
+constexpr int kHistGrid = 2048;   // upper bound on histogram workgroups (8 per CU)
+
+// float <-> unsigned key whose integer order is the float order (for atomicMin/atomicMax)
+__host__ __device__ inline uint32_t f2ord(float f)
+{
+    uint32_t u;
+#ifdef __HIP_DEVICE_COMPILE__
+    u = __float_as_uint(f);
+#else
+    memcpy(&u, &f, 4);
+#endif
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__host__ __device__ inline float ord2f(uint32_t o)
+{
+    uint32_t u = (o & 0x80000000u) ? (o & 0x7fffffffu) : ~o;
+#ifdef __HIP_DEVICE_COMPILE__
+    return __uint_as_float(u);
+#else
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+#endif
+}
+constexpr uint32_t kOrdPosInf = 0xff800000u;   // f2ord(+inf)
+constexpr uint32_t kOrdNegInf = 0x007fffffu;   // f2ord(-inf)
+
+struct DevState
+{
+    // batch min/max accumulators (ordered keys), consumed and re-armed by the last workgroup of the min/max pass
+    uint32_t min_key, max_key;
+    uint32_t ticket_minmax, ticket_hist, ticket_search;
+    int stats_updated;   // _statsUpdated
+    // TF analyzer: accumulated range in double (TfEncodingAnalyzer.h:84-90)
+    double acc_min, acc_max;
+    // TF-Enhanced analyzer
+    int initialized;   // PDF range fixed (xLeft.size() != 0 in the reference)
+    int iterations;
+    float bucket_f, pdf_offset_f;
+    double xLeft[kPdf];
+    double pdf[kPdf];
+    uint32_t counts[kPdf];        // current batch; zero between batches
+    uint32_t last_counts[kPdf];   // copy of the last folded batch (inspection)
+    // search scratch and result
+    float cand_delta[kMaxCand];
+    int cand_offset[kMaxCand];
+    int cand_valid[kMaxCand];
+    double cand_cost[kMaxCand];
+    int n_cand;
+    int best_index;
+    double enc_min, enc_max, enc_delta, enc_offset;
+    int enc_bw;
+};
+
+// relaxed agent-scope loads: used by the workgroup that finishes last to read what the others published
+template <typename T>
+__device__ __forceinline__ T agent_load(const T* p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ float wave_min(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v = fminf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+
+// ---------------------------------------------------------------------------------------------------- min / max
+// mode kMinMaxTf : TF analyzer   -> fold the batch range into acc_min / acc_max
+// mode kMinMaxTfe: TF-Enhanced   -> if the PDF is not initialised yet, derive its range from this batch
+enum
+{
+    kMinMaxTf  = 1,
+    kMinMaxTfe = 2
+};
+
+__device__ void initialize_pdf(DevState* st, float min_val, float max_val)
+{
+    // DLQ/src/math_functions.cpp:208-241 with signed_vals = true, DTYPE = float
+    if (min_val == max_val)
+    {
+        const float t = min_val + (float) 0.01;
+        max_val       = (max_val < t) ? t : max_val;
+    }
+    const float center = (max_val + min_val) / 2;
+    const float lo     = center - 3 * (center - min_val);
+    const float hi     = center + 3 * (max_val - center);
+    min_val            = (-FLT_MAX < lo) ? lo : -FLT_MAX;
+    max_val            = (hi < FLT_MAX) ? hi : FLT_MAX;
+    const double bucket = ((double) max_val - (double) min_val) / kPdf;
+    for (int i = threadIdx.x; i < kPdf; i += blockDim.x)
+    {
+        st->xLeft[i] = min_val + i * bucket;
+        st->pdf[i]   = 0.0;
+    }
+    if (threadIdx.x == 0)
+    {
+        // x_left[1] - x_left[0] and x_left[0], rounded to float, drive the bucket index of every later batch
+        const double x0   = min_val + 0 * bucket;
+        const double x1   = min_val + 1 * bucket;
+        const float bf    = (float) (x1 - x0);
+        st->bucket_f      = bf;
+        st->pdf_offset_f  = (float) x0 / bf;
+        st->iterations    = 0;
+        st->initialized   = 1;
+    }
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void minmax_kernel(const float* __restrict__ in, int64_t n, DevState* st,
+                                                        int mode)
+{
+    if (mode == kMinMaxTfe && st->initialized)
+        return;   // range already fixed: later batches need no min/max pass
+    float mn = INFINITY, mx = -INFINITY;
+    if (VEC)
+    {
+        const int64_t nvec = n / 4;
+        const float4* v    = reinterpret_cast<const float4*>(in);
+        for (int64_t i = (int64_t) blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (int64_t) gridDim.x * kBlock)
+        {
+            const float4 a = v[i];
+            mn             = fminf(fminf(mn, a.x), fminf(a.y, fminf(a.z, a.w)));
+            mx             = fmaxf(fmaxf(mx, a.x), fmaxf(a.y, fmaxf(a.z, a.w)));
+        }
+        if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * 4))
+        {
+            const float a = in[nvec * 4 + threadIdx.x];
+            mn            = fminf(mn, a);
+            mx            = fmaxf(mx, a);
+        }
+    }
+    else
+    {
+        for (int64_t i = (int64_t) blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t) gridDim.x * kBlock)
+        {
+            const float a = in[i];
+            mn            = fminf(mn, a);
+            mx            = fmaxf(mx, a);
+        }
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    __shared__ float smn[kBlock / 64], smx[kBlock / 64];
+    __shared__ bool is_last;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0)
+    {
+        smn[wave] = mn;
+        smx[wave] = mx;
+    }
+    __syncthreads();
+    uint32_t* kmin = &st->min_key;
+    uint32_t* kmax = &st->max_key;
+    uint32_t* tick = &st->ticket_minmax;
+    if (threadIdx.x == 0)
+    {
+        for (int w = 1; w < kBlock / 64; ++w)
+        {
+            mn = fminf(mn, smn[w]);
+            mx = fmaxf(mx, smx[w]);
+        }
+        atomicMin(kmin, f2ord(mn));
+        atomicMax(kmax, f2ord(mx));
+        __threadfence();
+        const uint32_t t = atomicAdd(tick, 1u);
+        is_last          = (t == gridDim.x - 1);
+    }
+    __syncthreads();
+    if (!is_last)
+        return;
+    __threadfence();
+    const float gmn = ord2f(agent_load(kmin));
+    const float gmx = ord2f(agent_load(kmax));
+    __syncthreads();   // everyone holds gmn/gmx before the keys are re-armed
+    if (threadIdx.x == 0)
+    {
+        st->min_key       = kOrdPosInf;
+        st->max_key       = kOrdNegInf;
+        st->ticket_minmax = 0;
+        st->stats_updated = 1;
+    }
+    if (mode == kMinMaxTf)
+    {
+        if (threadIdx.x == 0)
+        {
+            // DLQ/src/TfEncodingAnalyzer.cpp:59-71
+            const double cmn = (double) gmn, cmx = (double) gmx;
+            st->acc_min = (cmn < st->acc_min) ? cmn : st->acc_min;
+            st->acc_max = (st->acc_max < cmx) ? cmx : st->acc_max;
+        }
+        return;
+    }
+    // TF-Enhanced: DLQ/src/math_functions.cpp:248-262
+    if (gmn == 0 && gmx == 0)
+        return;   // an all-zero batch cannot fix a range; the PDF stays uninitialised and this batch is not counted
+    initialize_pdf(st, gmn, gmx);
+}
+
+// per-channel min/max: partial reductions meet in `keys` (uint32[2C], ordered keys) through atomics
+__global__ void fill_keys_kernel(uint32_t* keys, int64_t c)
+{
+    const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < c)
+    {
+        keys[i]     = kOrdPosInf;
+        keys[c + i] = kOrdNegInf;
+    }
+}
+__global__ void decode_keys_kernel(uint32_t* keys, int64_t c2)
+{
+    const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < c2)
+        reinterpret_cast<float*>(keys)[i] = ord2f(keys[i]);
+}
+// one workgroup per (row, chunk); row = outer * C + c, every row has n_per_channel contiguous elements
+__global__ __launch_bounds__(kBlock) void minmax_rows_kernel(const float* __restrict__ in, int64_t num_channel,
+                                                             int64_t n_per_channel, int64_t chunk,
+                                                             uint32_t chunks_per_row, uint32_t* keys)
+{
+    const int64_t row   = blockIdx.x / chunks_per_row;
+    const int64_t c     = row % num_channel;
+    const int64_t begin = (int64_t) (blockIdx.x % chunks_per_row) * chunk;
+    int64_t end         = begin + chunk;
+    if (end > n_per_channel)
+        end = n_per_channel;
+    const float* p = in + row * n_per_channel;
+    float mn = INFINITY, mx = -INFINITY;
+    for (int64_t i = begin + threadIdx.x; i < end; i += kBlock)
+    {
+        const float a = p[i];
+        mn            = fminf(mn, a);
+        mx            = fmaxf(mx, a);
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    __shared__ float smn[kBlock / 64], smx[kBlock / 64];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0)
+    {
+        smn[wave] = mn;
+        smx[wave] = mx;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        for (int w = 1; w < kBlock / 64; ++w)
+        {
+            mn = fminf(mn, smn[w]);
+            mx = fmaxf(mx, smx[w]);
+        }
+        atomicMin(&keys[c], f2ord(mn));
+        atomicMax(&keys[num_channel + c], f2ord(mx));
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------- histogram
+__device__ __forceinline__ void hist_add(uint32_t* lds, float x, float bucket, float off, int copy)
+{
+    // DLQ/src/math_functions.cpp:375-382; the range test is done on the rounded float so that NaN and values
+    // beyond the int range are dropped, as they are on the reference's CPU path
+    const float r = roundf(x / bucket - off);
+    if (r >= 0.0f && r < (float) kPdf)
+        atomicAdd(&lds[(int) r * kCopies + copy], 1u);
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ in, int64_t n, DevState* st)
+{
+    if (!st->initialized)
+        return;   // only all-zero batches so far: the reference returns without touching the PDF
+    __shared__ uint32_t lds[kPdf * kCopies];
+    __shared__ bool is_last;
+    for (int i = threadIdx.x; i < kPdf * kCopies; i += kBlock)
+        lds[i] = 0;
+    __syncthreads();
+    const float bucket = st->bucket_f;
+    const float off    = st->pdf_offset_f;
+    const int copy     = threadIdx.x & (kCopies - 1);
+    if (VEC)
+    {
+        const int64_t nvec   = n / 4;
+        const float4* v      = reinterpret_cast<const float4*>(in);
+        const int64_t stride = (int64_t) gridDim.x * kBlock * kUnroll;
+        for (int64_t base = (int64_t) blockIdx.x * kBlock * kUnroll; base < nvec; base += stride)
+        {
+            float4 a[kUnroll];
+            bool live[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+            {
+                const int64_t i = base + u * kBlock + threadIdx.x;
+                live[u]         = i < nvec;
+                if (live[u])
+                    a[u] = v[i];
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+            {
+                if (!live[u])
+                    continue;
+                hist_add(lds, a[u].x, bucket, off, copy);
+                hist_add(lds, a[u].y, bucket, off, copy);
+                hist_add(lds, a[u].z, bucket, off, copy);
+                hist_add(lds, a[u].w, bucket, off, copy);
+            }
+        }
+        if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * 4))
+            hist_add(lds, in[nvec * 4 + threadIdx.x], bucket, off, copy);
+    }
+    else
+    {
+        for (int64_t i = (int64_t) blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t) gridDim.x * kBlock)
+            hist_add(lds, in[i], bucket, off, copy);
+    }
+    __syncthreads();
+    for (int b = threadIdx.x; b < kPdf; b += kBlock)
+    {
+        uint32_t s = 0;
+#pragma unroll
+        for (int c = 0; c < kCopies; ++c)
+            s += lds[b * kCopies + c];
+        if (s)
+            atomicAdd(&st->counts[b], s);
+    }
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        const uint32_t t = atomicAdd(&st->ticket_hist, 1u);
+        is_last          = (t == gridDim.x - 1);
+    }
+    __syncthreads();
+    if (!is_last)
+        return;
+    __threadfence();
+    // fold this batch into the running PDF: DLQ/src/math_functions.cpp:279-287 (cnt is an int in the reference)
+    const int it     = st->iterations;
+    const double cnt = (double) (int) n;
+    for (int b = threadIdx.x; b < kPdf; b += kBlock)
+    {
+        const uint32_t c   = atomicExch(&st->counts[b], 0u);
+        st->last_counts[b] = c;
+        const double prob  = (double) c / cnt;
+        st->pdf[b]         = (st->pdf[b] * it + prob) / (it + 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        st->iterations  = it + 1;
+        st->ticket_hist = 0;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ SQNR search
+struct SearchArgs
+{
+    int bw;
+    int sym, strict, uns;
+    float num_steps_cand;   // 2^bw - 1, minus 1 for strict symmetric (candidate generation and final min/max)
+    float step_size_cost;   // 2^bw - 1 (the cost function never reduces it)
+    int n_cand;             // grid size: 17*21 + 1 asymmetric, number of float steps of 0.01 symmetric
+    int n_delta;            // 17 or the symmetric count
+};
+
+__device__ __forceinline__ float std_max(float a, float b)
+{
+    return (a < b) ? b : a;   // std::max(a, b)
+}
+__device__ __forceinline__ float std_min(float a, float b)
+{
+    return (b < a) ? b : a;   // std::min(a, b)
+}
+
+// One wavefront per candidate.  Lanes evaluate the per-bucket error terms in parallel; the three sums of the
+// cost are then accumulated by one lane in bucket order, the order the reference's loops use, so that costs are
+// bit-identical to the CPU result and ties between candidates resolve identically.
+__global__ __launch_bounds__(64) void tfe_search_kernel(DevState* st, SearchArgs a)
+{
+    const int cand = blockIdx.x;
+    const int lane = threadIdx.x;
+    __shared__ double term[kPdf];
+    __shared__ bool is_last;
+
+    if (st->initialized)
+    {
+        // ---- range of the aggregate stats: DLQ/src/TfEnhancedEncodingAnalyzer.cpp:255-291
+        int first = -1, last = -1;
+#pragma unroll
+        for (int k = 0; k < kPdf / 64; ++k)
+        {
+            const uint64_t m = __ballot(st->pdf[k * 64 + lane] > 0);
+            if (m)
+            {
+                if (first < 0)
+                    first = k * 64 + __builtin_ctzll(m);
+                const uint64_t m1 = (k == 0) ? (m & ~1ull) : m;   // the downward scan stops above bucket 0
+                if (m1)
+                    last = k * 64 + 63 - __builtin_clzll(m1);
+            }
+        }
+        float minVal = (float) st->xLeft[first < 0 ? 0 : first];
+        float maxVal = (float) st->xLeft[last < 0 ? kPdf - 1 : last];
+        minVal       = std_min(minVal, 0.0f);
+        maxVal       = std_max(maxVal, 0.0f);
+        maxVal       = std_max(maxVal, minVal + (float) 0.01);
+
+        // ---- this wavefront's candidate
+        float delta = 0.f;
+        int offset  = 0;
+        bool valid  = true;
+        const float numSteps = a.num_steps_cand;
+        if (a.sym)
+        {
+            // DLQ/src/TfEnhancedEncodingAnalyzer.cpp:216-253
+            float deltaMax;
+            if ((minVal == 0.0) && a.uns)
+            {
+                deltaMax = maxVal / numSteps;
+                offset   = 0;
+            }
+            else
+            {
+                const float absMax = std_max(fabsf(maxVal), fabsf(minVal));
+                deltaMax           = (float) (absMax / (numSteps / 2.0));
+                offset             = (int) floorf(-numSteps / 2);
+            }
+            float f = (float) (1.0 / 100);
+            for (int k = 0; k < cand; ++k)
+                f = (float) ((double) f + 1.0 / 100);
+            delta = f * deltaMax;
+        }
+        else
+        {
+            // DLQ/src/TfEnhancedEncodingAnalyzer.cpp:177-214
+            const float obsDelta = (float) (((double) maxVal - (double) minVal) / numSteps);
+            const int obsOffset  = (int) roundf(minVal / obsDelta);
+            const float obsMin   = std_max(obsDelta * (float) obsOffset, -FLT_MAX);
+            const float obsMax   = std_min(obsDelta * ((float) obsOffset + numSteps), FLT_MAX);
+            if (cand == a.n_cand - 1)
+            {
+                delta  = obsDelta;
+                offset = obsOffset;
+            }
+            else
+            {
+                const int fi = cand / 21, oi = cand % 21;
+                float f = (float) (1.0 / 16);
+                for (int k = 0; k < fi; ++k)
+                    f = (float) ((double) f + 1.0 / 16);
+                delta  = f * obsDelta;
+                offset = (int) ((double) (-numSteps) + (double) numSteps / 20.0 * oi);
+                // clamp to the observed range: DLQ/src/TfEnhancedEncodingAnalyzer.cpp:149-175
+                float tMin = std_max(delta * (float) offset, -FLT_MAX);
+                float tMax = std_min(delta * ((float) offset + numSteps), FLT_MAX);
+                if ((tMin < obsMin) && (tMax > obsMax))
+                    valid = false;
+                else
+                {
+                    tMin = std_max(obsMin, tMin);
+                    tMax = std_min(obsMax, tMax);
+                    if (tMin == tMax)
+                        valid = false;
+                    else
+                    {
+                        delta  = (float) (((double) tMax - tMin) / numSteps);
+                        offset = (int) roundf(tMin / delta);
+                    }
+                }
+            }
+        }
+
+        // ---- cost: DLQ/src/TfEnhancedEncodingAnalyzer.cpp:293-355
+        double cost = 0;
+        if (valid)
+        {
+            const float cMin      = delta * (float) offset;
+            const float stepSize  = a.step_size_cost;
+            const float cMax      = delta * ((float) offset + stepSize);
+            const float pdfStart  = (float) st->xLeft[0];
+            const double pdfStep  = st->xLeft[1] - st->xLeft[0];
+            int minInd            = (int) floor((cMin - pdfStart) / pdfStep);
+            minInd                = minInd < 0 ? 0 : (minInd > kPdf - 1 ? kPdf - 1 : minInd);
+            int maxInd            = (int) floor((cMax - pdfStart) / pdfStep);
+            maxInd                = maxInd < 0 ? 0 : (maxInd > kPdf - 1 ? kPdf - 1 : maxInd);
+            const float minMid    = (float) (pdfStart + (minInd * pdfStep) + pdfStep / 2);
+            const float maxMid    = (float) (pdfStart + (maxInd * pdfStep) + pdfStep / 2);
+#pragma unroll
+            for (int k = 0; k < kPdf / 64; ++k)
+            {
+                const int i      = k * 64 + lane;
+                const double p   = st->pdf[i];
+                const double mid = pdfStart + i * pdfStep + pdfStep / 2;
+                double t;
+                if (i < minInd)
+                {
+                    const double d = mid - minMid;
+                    t              = p * (d * d);
+                }
+                else if (i >= maxInd)
+                {
+                    const double d = mid - maxMid;
+                    t              = p * (d * d);
+                }
+                else
+                {
+                    const float fv   = (float) mid;
+                    const int q      = (int) roundf(fv / delta - (float) offset);
+                    const float dq   = delta * (float) (q + offset);
+                    const double d   = (double) (fv - dq);
+                    t                = p * (d * d);
+                }
+                term[i] = t;
+            }
+            __syncthreads();
+            // lanes 0,1,2 each accumulate one of the three sums in ascending bucket order
+            double acc = 0;
+            if (lane == 0)
+                for (int i = 0; i < minInd; ++i)
+                    acc += term[i];
+            else if (lane == 1)
+                for (int i = maxInd; i < kPdf; ++i)
+                    acc += term[i];
+            else if (lane == 2)
+                for (int i = minInd; i < maxInd; ++i)
+                    acc += term[i];
+            const double satBottom = __shfl(acc, 0);
+            const double satTop    = __shfl(acc, 1);
+            const double quant     = __shfl(acc, 2);
+            cost                   = 3.0 * (satBottom + satTop) + quant;
+            cost                   = (cost < DBL_MAX) ? cost : DBL_MAX;   // std::min(sqnr, max())
+        }
+        if (lane == 0)
+        {
+            st->cand_delta[cand]  = delta;
+            st->cand_offset[cand] = offset;
+            st->cand_valid[cand]  = valid ? 1 : 0;
+            st->cand_cost[cand]   = cost;
+        }
+    }
+    __threadfence();
+    __syncthreads();
+    if (lane == 0)
+    {
+        const uint32_t t = atomicAdd(&st->ticket_search, 1u);
+        is_last          = (t == gridDim.x - 1);
+    }
+    __syncthreads();
+    if (!is_last)
+        return;
+    __threadfence();
+
+    // ---- last wavefront: pick the winner (first strict minimum) and form the encoding
+    if (lane == 0)
+    {
+        st->ticket_search = 0;
+        st->n_cand        = st->initialized ? a.n_cand : 0;
+    }
+    if (!st->initialized)
+    {
+        if (lane == 0)
+        {
+            st->best_index = -1;
+            if (st->stats_updated)
+            {
+                // only zeros were seen: DLQ/src/TfEnhancedEncodingAnalyzer.cpp:85-100
+                const float ns    = a.step_size_cost;
+                double mn = -1, mx = 1;
+                const double d = (mx - mn) / (int) ns;
+                const double o = floor(mn / d);
+                mn             = o * d;
+                mx             = mn + (int) ns * d;
+                st->enc_min = mn, st->enc_max = mx, st->enc_delta = d, st->enc_offset = o;
+                st->enc_bw = a.bw;
+            }
+            else
+            {
+                st->enc_min = st->enc_max = st->enc_delta = st->enc_offset = 0;
+                st->enc_bw                                                = 0;
+            }
+        }
+        return;
+    }
+    double best = DBL_MAX;
+    int bidx    = 0x7fffffff;
+    for (int c = lane; c < a.n_cand; c += 64)
+    {
+        const double cost = agent_load(&st->cand_cost[c]);
+        const int v       = agent_load(&st->cand_valid[c]);
+        if (v && cost < best)
+        {
+            best = cost;
+            bidx = c;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        const double ob = __shfl_xor(best, o);
+        const int oi    = __shfl_xor(bidx, o);
+        if (ob < best || (ob == best && oi < bidx))
+        {
+            best = ob;
+            bidx = oi;
+        }
+    }
+    if (lane == 0)
+    {
+        float bestDelta = -1;
+        int bestOffset  = -1;
+        if (bidx != 0x7fffffff && best < DBL_MAX)
+        {
+            bestDelta  = agent_load(&st->cand_delta[bidx]);
+            bestOffset = agent_load(&st->cand_offset[bidx]);
+        }
+        else
+            bidx = -1;
+        // DLQ/src/TfEnhancedEncodingAnalyzer.cpp:383-396
+        const float bMin = std_max(bestDelta * (float) bestOffset, -FLT_MAX);
+        const float bMax = std_min(bestDelta * ((float) bestOffset + a.num_steps_cand), FLT_MAX);
+        st->enc_delta    = bestDelta;
+        st->enc_offset   = bestOffset;
+        st->enc_bw       = a.bw;
+        st->enc_min      = bMin;
+        st->enc_max      = bMax;
+        st->best_index   = bidx;
+    }
+}
+
+__global__ void reset_state_kernel(DevState* st)
+{
+    const int i = threadIdx.x;   // launched with kPdf threads
+    if (i == 0)
+    {
+        st->min_key       = kOrdPosInf;
+        st->max_key       = kOrdNegInf;
+        st->ticket_minmax = st->ticket_hist = st->ticket_search = 0;
+        st->stats_updated                                       = 0;
+        st->acc_min                                             = DBL_MAX;
+        st->acc_max                                             = -DBL_MAX;
+        st->initialized = st->iterations = 0;
+        st->bucket_f = st->pdf_offset_f = 0.f;
+        st->n_cand                      = 0;
+        st->best_index                  = -1;
+        st->enc_min = st->enc_max = st->enc_delta = st->enc_offset = 0;
+        st->enc_bw                                                 = 0;
+    }
+    st->xLeft[i]       = 0;
+    st->pdf[i]         = 0;
+    st->counts[i]      = 0;
+    st->last_counts[i] = 0;
+}
+
+int minmax_grid(int64_t n)
+{
+    int64_t blocks = (n / 4 + (int64_t) kBlock * kUnroll - 1) / ((int64_t) kBlock * kUnroll);
+    if (blocks < 1)
+        blocks = 1;
+    if (blocks > kHistGrid)
+        blocks = kHistGrid;
+    return (int) blocks;
+}
+}   // namespace
+}   // namespace miq
+
+using namespace miq;
+
+struct miq_analyzer
+{
+    int mode;
+    int device;
+    DevState* st;        // device
+    void* pinned;        // host staging (pinned) for read-backs
+    bool stats_updated;  // host mirror of _isEncodingValid / _statsUpdated
+    bool range_known;    // host knows the PDF range has been fixed, so no further min/max pass is queued
+    hipEvent_t probe;    // marks the completion of an asynchronous read of DevState::initialized
+    bool probe_pending;
+    int* probe_flag;     // pinned host word receiving that read
+    int last_bw;
+};
+
+extern "C" {
+
+static int launch_minmax_rows(const float* in, int64_t num_channel, int64_t rows, int64_t n_per_channel,
+                              uint32_t* keys, hipStream_t s)
+{
+    // keys: uint32[2C] ordered keys (min block then max block); decoded in place to float at the end
+    hipLaunchKernelGGL(fill_keys_kernel, dim3((unsigned) ((num_channel + kBlock - 1) / kBlock)), dim3(kBlock), 0, s,
+                       keys, num_channel);
+    if (rows > 0)
+    {
+        int64_t chunk = (int64_t) kBlock * 16;
+        int64_t bx    = (n_per_channel + chunk - 1) / chunk;
+        if (rows * bx > (1ll << 20))
+        {
+            // keep the grid modest for very long rows: fewer, longer chunks
+            bx    = ((1ll << 20) + rows - 1) / rows;
+            chunk = (n_per_channel + bx - 1) / bx;
+            bx    = (n_per_channel + chunk - 1) / chunk;
+        }
+        MIQ_CHECK_ARG(rows * bx < (1ll << 31), "too many rows for one launch");
+        hipLaunchKernelGGL(minmax_rows_kernel, dim3((unsigned) (rows * bx)), dim3(kBlock), 0, s, in, num_channel,
+                           n_per_channel, chunk, (uint32_t) bx, keys);
+    }
+    hipLaunchKernelGGL(decode_keys_kernel, dim3((unsigned) ((2 * num_channel + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                       s, keys, 2 * num_channel);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int miq_minmax_f32(const float* in, int64_t n, float* out_min_max, void* stream)
+{
+    MIQ_CHECK_ARG(n >= 0 && out_min_max && (n == 0 || in), "null pointer or negative count");
+    return launch_minmax_rows(in, 1, n > 0 ? 1 : 0, n > 0 ? n : 1, reinterpret_cast<uint32_t*>(out_min_max),
+                              (hipStream_t) stream);
+}
+
+int miq_minmax_per_channel_f32(const float* in, int64_t num_channel, int64_t num_element,
+                               int64_t num_element_per_channel, float* out_min_max, void* stream)
+{
+    MIQ_CHECK_ARG(num_channel > 0 && num_element_per_channel > 0 && num_element >= 0 && out_min_max,
+                  "bad channel geometry or null output");
+    MIQ_CHECK_ARG(num_element == 0 || in, "null input");
+    MIQ_CHECK_ARG(num_element % num_element_per_channel == 0,
+                  "num_element must be a multiple of num_element_per_channel");
+    return launch_minmax_rows(in, num_channel, num_element / num_element_per_channel, num_element_per_channel,
+                              reinterpret_cast<uint32_t*>(out_min_max), (hipStream_t) stream);
+}
+
+int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
+{
+    MIQ_CHECK_ARG(out != nullptr, "null output handle");
+    if (quantization_mode != MIQ_QUANTIZATION_TF && quantization_mode != MIQ_QUANTIZATION_TF_ENHANCED)
+    {
+        set_error("quantization mode %d is not implemented (only TF and TF_ENHANCED are)", quantization_mode);
+        return MIQ_ERR_UNSUPPORTED;
+    }
+    miq_analyzer* a = new (std::nothrow) miq_analyzer();
+    MIQ_CHECK_ARG(a != nullptr, "out of host memory");
+    a->mode          = quantization_mode;
+    a->st            = nullptr;
+    a->pinned        = nullptr;
+    a->stats_updated = false;
+    a->range_known   = false;
+    a->probe         = nullptr;
+    a->probe_pending = false;
+    a->probe_flag    = nullptr;
+    a->last_bw       = 0;
+    hipError_t e     = hipGetDevice(&a->device);
+    if (e == hipSuccess)
+        e = hipMalloc((void**) &a->st, sizeof(DevState));
+    if (e == hipSuccess)
+        e = hipHostMalloc(&a->pinned, sizeof(DevState) + 64, hipHostMallocDefault);
+    if (e == hipSuccess)
+        e = hipEventCreateWithFlags(&a->probe, hipEventDisableTiming);
+    if (e != hipSuccess)
+    {
+        set_error("analyzer allocation failed: %s", hipGetErrorString(e));
+        if (a->st)
+            (void) hipFree(a->st);
+        if (a->pinned)
+            (void) hipHostFree(a->pinned);
+        delete a;
+        return MIQ_ERR_HIP;
+    }
+    a->probe_flag  = reinterpret_cast<int*>(static_cast<char*>(a->pinned) + sizeof(DevState));
+    *a->probe_flag = 0;
+    hipLaunchKernelGGL(reset_state_kernel, dim3(1), dim3(kPdf), 0, (hipStream_t) nullptr, a->st);
+    e = hipStreamSynchronize(nullptr);
+    if (e != hipSuccess)
+    {
+        set_error("analyzer initialisation failed: %s", hipGetErrorString(e));
+        (void) hipFree(a->st);
+        (void) hipHostFree(a->pinned);
+        (void) hipEventDestroy(a->probe);
+        delete a;
+        return MIQ_ERR_HIP;
+    }
+    *out = a;
+    return MIQ_OK;
+}
+
+int miq_analyzer_destroy(miq_analyzer* a)
+{
+    if (!a)
+        return MIQ_OK;
+    if (a->probe_pending)
+        (void) hipEventSynchronize(a->probe);
+    (void) hipEventDestroy(a->probe);
+    (void) hipFree(a->st);
+    (void) hipHostFree(a->pinned);
+    delete a;
+    return MIQ_OK;
+}
+
+int miq_analyzer_reset(miq_analyzer* a, void* stream)
+{
+    MIQ_CHECK_ARG(a != nullptr, "null analyzer");
+    hipLaunchKernelGGL(reset_state_kernel, dim3(1), dim3(kPdf), 0, (hipStream_t) stream, a->st);
+    MIQ_CHECK_LAUNCH();
+    a->stats_updated = false;
+    a->range_known   = false;
+    if (a->probe_pending)
+    {
+        // a read of the pre-reset state may still be in flight; its answer must not be believed afterwards
+        MIQ_CHECK_HIP(hipEventSynchronize(a->probe));
+        a->probe_pending = false;
+    }
+    *a->probe_flag = 0;
+    return MIQ_OK;
+}
+
+int miq_analyzer_update_stats_f32(miq_analyzer* a, const float* data, int64_t n, void* stream)
+{
+    MIQ_CHECK_ARG(a != nullptr, "null analyzer");
+    MIQ_CHECK_ARG(n > 0 && data, "update_stats needs a non-empty tensor");
+    hipStream_t s  = (hipStream_t) stream;
+    const bool vec = aligned16(data);
+    a->stats_updated = true;
+    const int grid = minmax_grid(n);
+    if (a->mode == MIQ_QUANTIZATION_TF)
+    {
+        if (vec)
+            hipLaunchKernelGGL(minmax_kernel<true>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st, kMinMaxTf);
+        else
+            hipLaunchKernelGGL(minmax_kernel<false>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st, kMinMaxTf);
+        MIQ_CHECK_LAUNCH();
+        return MIQ_OK;
+    }
+    if (!a->range_known && a->probe_pending && hipEventQuery(a->probe) == hipSuccess)
+    {
+        a->probe_pending = false;
+        a->range_known   = (*a->probe_flag != 0);
+    }
+    if (!a->range_known)
+    {
+        // The range is fixed by the first batch that is not all zeros.  Whether that has happened is device state;
+        // the pass below returns at once when it has, and the host stops queuing it once an asynchronous read of
+        // that flag (queued after each batch until it answers yes) has landed.  Nothing here blocks.
+        if (vec)
+            hipLaunchKernelGGL(minmax_kernel<true>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st, kMinMaxTfe);
+        else
+            hipLaunchKernelGGL(minmax_kernel<false>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st, kMinMaxTfe);
+    }
+    if (vec)
+        hipLaunchKernelGGL(hist_kernel<true>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st);
+    else
+        hipLaunchKernelGGL(hist_kernel<false>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st);
+    MIQ_CHECK_LAUNCH();
+    if (!a->range_known && !a->probe_pending)
+    {
+        MIQ_CHECK_HIP(hipMemcpyAsync(a->probe_flag, &a->st->initialized, sizeof(int), hipMemcpyDeviceToHost, s));
+        MIQ_CHECK_HIP(hipEventRecord(a->probe, s));
+        a->probe_pending = true;
+    }
+    return MIQ_OK;
+}
+
+static int read_state(miq_analyzer* a, hipStream_t s)
+{
+    MIQ_CHECK_HIP(hipMemcpyAsync(a->pinned, a->st, sizeof(DevState), hipMemcpyDeviceToHost, s));
+    MIQ_CHECK_HIP(hipStreamSynchronize(s));
+    const DevState* h = static_cast<const DevState*>(a->pinned);
+    if (h->initialized)
+        a->range_known = true;
+    return MIQ_OK;
+}
+
+int miq_analyzer_compute_encoding(miq_analyzer* a, int bw, int use_symmetric, int use_strict_symmetric,
+                                  int use_unsigned_symmetric, miq_encoding* out, int* is_valid, void* stream)
+{
+    MIQ_CHECK_ARG(a && out && is_valid, "null argument");
+    MIQ_CHECK_ARG(bw >= 1 && bw <= 32, "bitwidth must be in [1, 32] (got %d)", bw);
+    hipStream_t s = (hipStream_t) stream;
+    memset(out, 0, sizeof(*out));
+    *is_valid = a->stats_updated ? 1 : 0;
+    if (!a->stats_updated)
+        return MIQ_OK;   // AimetTensorQuantizer::getEncoding returns a default encoding and valid = false
+    if (a->mode == MIQ_QUANTIZATION_TF)
+    {
+        if (int rc = read_state(a, s))
+            return rc;
+        const DevState* h = static_cast<const DevState*>(a->pinned);
+        // DLQ/src/TfEncodingAnalyzer.cpp:80-101 (MIN_RANGE = 0.01)
+        double lo = std::min(0.0, h->acc_min);
+        double hi = std::max(0.0, h->acc_max);
+        hi        = std::max(hi, lo + 0.01);
+        return miq_get_computed_encodings(bw, lo, hi, use_symmetric, use_strict_symmetric, use_unsigned_symmetric, out);
+    }
+    SearchArgs sa{};
+    sa.bw             = bw;
+    sa.sym            = use_symmetric ? 1 : 0;
+    sa.strict         = use_strict_symmetric ? 1 : 0;
+    sa.uns            = use_unsigned_symmetric ? 1 : 0;
+    sa.step_size_cost = (float) (std::pow(2, bw) - 1);
+    sa.num_steps_cand = sa.step_size_cost;
+    if (sa.sym && sa.strict)
+        sa.num_steps_cand -= 1;
+    if (sa.sym)
+    {
+        // the delta factor advances by adding the double 0.01 to a float; how many steps fit below 1.01 is decided
+        // by that float arithmetic (DLQ/src/TfEnhancedEncodingAnalyzer.cpp:248)
+        int cnt = 0;
+        for (float f = (float) (1.0 / 100); (double) f <= 1 + 1.0 / 100; f = (float) ((double) f + 1.0 / 100))
+            ++cnt;
+        sa.n_delta = cnt;
+        sa.n_cand  = cnt;
+    }
+    else
+    {
+        int cnt = 0;
+        for (float f = (float) (1.0 / 16); (double) f <= 1 + 1.0 / 16; f = (float) ((double) f + 1.0 / 16))
+            ++cnt;
+        sa.n_delta = cnt;
+        sa.n_cand  = cnt * 21 + 1;
+    }
+    MIQ_CHECK_ARG(sa.n_cand <= kMaxCand, "internal: candidate grid too large");
+    hipLaunchKernelGGL(tfe_search_kernel, dim3(sa.n_cand), dim3(64), 0, s, a->st, sa);
+    MIQ_CHECK_LAUNCH();
+    if (int rc = read_state(a, s))
+        return rc;
+    const DevState* h = static_cast<const DevState*>(a->pinned);
+    out->min    = h->enc_min;
+    out->max    = h->enc_max;
+    out->delta  = h->enc_delta;
+    out->offset = h->enc_offset;
+    out->bw     = h->enc_bw;
+    a->last_bw  = bw;
+    return MIQ_OK;
+}
+
+int miq_analyzer_get_stats_histogram(miq_analyzer* a, double* x_left, double* pdf, int* num_buckets, void* stream)
+{
+    MIQ_CHECK_ARG(a && x_left && pdf && num_buckets, "null argument");
+    if (a->mode != MIQ_QUANTIZATION_TF_ENHANCED)
+    {
+        set_error("no histogram is kept by the TF (min/max) analyzer");
+        return MIQ_ERR_UNSUPPORTED;
+    }
+    if (int rc = read_state(a, (hipStream_t) stream))
+        return rc;
+    const DevState* h = static_cast<const DevState*>(a->pinned);
+    *num_buckets      = h->initialized ? kPdf : 0;
+    if (h->initialized)
+    {
+        memcpy(x_left, h->xLeft, sizeof(double) * kPdf);
+        memcpy(pdf, h->pdf, sizeof(double) * kPdf);
+    }
+    return MIQ_OK;
+}
+
+int miq_analyzer_last_batch_counts(miq_analyzer* a, uint32_t* counts, void* stream)
+{
+    MIQ_CHECK_ARG(a && counts, "null argument");
+    if (int rc = read_state(a, (hipStream_t) stream))
+        return rc;
+    memcpy(counts, static_cast<const DevState*>(a->pinned)->last_counts, sizeof(uint32_t) * kPdf);
+    return MIQ_OK;
+}
+
+int miq_analyzer_last_search(miq_analyzer* a, float* deltas, int32_t* offsets, double* costs, int cap, int* count,
+                             int* best_index, void* stream)
+{
+    MIQ_CHECK_ARG(a && deltas && offsets && costs && count && best_index && cap >= 0, "bad argument");
+    if (int rc = read_state(a, (hipStream_t) stream))
+        return rc;
+    const DevState* h = static_cast<const DevState*>(a->pinned);
+    // compact to the candidates the reference would have kept, in its order
+    int n = 0, best = -1;
+    for (int c = 0; c < h->n_cand; ++c)
+    {
+        if (!h->cand_valid[c])
+            continue;
+        if (c == h->best_index)
+            best = n;
+        if (n < cap)
+        {
+            deltas[n]  = h->cand_delta[c];
+            offsets[n] = h->cand_offset[c];
+            costs[n]   = h->cand_cost[c];
+        }
+        ++n;
+    }
+    *count      = n;
+    *best_index = best;
+    return MIQ_OK;
+}
+
+}   // extern "C"

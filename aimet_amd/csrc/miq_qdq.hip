@@ -1,0 +1,797 @@
+// Quantize-dequantize (fake-quant) forward and straight-through backward kernels for gfx950.
+//
+// One streaming kernel template serves every variant.  Each lane moves 16-byte vectors (4 x f32 or 8 x bf16),
+// kUnroll of them in flight, so a 256-lane workgroup covers a contiguous tile of 4096 (f32) or 8192 (bf16)
+// elements.  Per-tensor parameters travel as kernel arguments (scalar registers).  Per-channel parameters are
+// staged once per workgroup into an LDS window that holds just the channel rows the tile touches
+// (tile / elements-per-channel + 2 rows), and the row of a vector is found with one multiply-high (the divisor is
+// launch-invariant), so no per-element integer division or dependent global loads remain.
+//
+// Arithmetic is the reference's, operation for operation, in float32 with IEEE division and no contraction:
+//   v1  (DlQuantization): t = fmax(fmin(x, max), min); q = roundf(t / delta - offset); y = delta * (q + offset)
+//       ModelOptimizations/DlQuantization/src/trim_functions.cpp:141-182, 698-709
+//   v2  (aimet_torch.v2): r = rint(x / scale) - offset; y = (clamp(r, qmin, qmax) + offset) * scale
+//       TrainingExtensions/torch/src/python/aimet_torch/v2/quantization/affine/backends/torch_builtins.py:303-344
+#include "miq_common.h"
+
+#include <cmath>
+
+namespace miq
+{
+namespace
+{
+// ------------------------------------------------------------------------------------------------ IO vector types
+template <typename IO>
+struct IOTraits;
+
+template <>
+struct IOTraits<float>
+{
+    using Vec                = float4;
+    static constexpr int VEC = 4;
+    __device__ static void unpack(const Vec& v, float* f)
+    {
+        f[0] = v.x;
+        f[1] = v.y;
+        f[2] = v.z;
+        f[3] = v.w;
+    }
+    __device__ static Vec pack(const float* f)
+    {
+        return make_float4(f[0], f[1], f[2], f[3]);
+    }
+    __device__ static float load1(const float* p)
+    {
+        return *p;
+    }
+    __device__ static void store1(float* p, float v)
+    {
+        *p = v;
+    }
+};
+
+template <>
+struct IOTraits<uint16_t>
+{
+    using Vec                = uint4;
+    static constexpr int VEC = 8;
+    __device__ static void unpack(const Vec& v, float* f)
+    {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            f[2 * i]     = __uint_as_float(w[i] << 16);
+            f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+    __device__ static Vec pack(const float* f)
+    {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            w[i] = f32_to_bf16(f[2 * i]) | (f32_to_bf16(f[2 * i + 1]) << 16);
+        return make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    __device__ static float load1(const uint16_t* p)
+    {
+        return bf16_to_f32(*p);
+    }
+    __device__ static void store1(uint16_t* p, float v)
+    {
+        *p = (uint16_t) f32_to_bf16(v);
+    }
+};
+
+// -------------------------------------------------------------------------------------------------- the operations
+// Channel parameter sources (device pointers) and per-tensor values; which fields an op reads is up to the op.
+struct ParamSrc
+{
+    const float* a;   // v1: min      v2: scale
+    const float* b;   // v1: max      v2: offset
+    const float* c;   // v1: delta
+    const float* d;   // v1: offset
+    float4 scalar;    // per-tensor: the same four values
+    int qmin, qmax;   // v2 grid
+    float shift;      // v1 quantize-only: 2^(bw-1) or 0
+    int ishift;       // the same as an integer, for byte codes
+};
+
+struct OpV1
+{
+    using P = float4;   // min, max, delta, offset
+    __device__ static P load(const ParamSrc& s, uint32_t ch)
+    {
+        return make_float4(s.a[ch], s.b[ch], s.c[ch], s.d[ch]);
+    }
+    __device__ static float quant(const P& p, float x)
+    {
+        float t = fmaxf(fminf(x, p.y), p.x);
+        t       = t / p.z - p.w;
+        return roundf(t);
+    }
+};
+
+// y = QDQ(x); optional byte codes
+struct OpV1Qdq : OpV1
+{
+    static constexpr int NIN = 1;
+    using Code               = uint8_t;
+    __device__ static float apply(const ParamSrc& s, const P& p, float x, float, int& code)
+    {
+        float q = quant(p, x);
+        code    = (int) q - s.ishift;
+        return p.z * (q + p.w);
+    }
+};
+
+// y = grid index - shift (float valued), reference quantizeToFxp
+struct OpV1Quantize : OpV1
+{
+    static constexpr int NIN = 1;
+    using Code               = uint8_t;
+    __device__ static float apply(const ParamSrc& s, const P& p, float x, float, int& code)
+    {
+        float q = quant(p, x);
+        code    = 0;
+        return q - s.shift;
+    }
+};
+
+// gin = g * (min <= x <= max)
+struct OpV1Ste
+{
+    using P                  = float2;   // min, max
+    static constexpr int NIN = 2;
+    using Code               = uint8_t;
+    __device__ static P load(const ParamSrc& s, uint32_t ch)
+    {
+        return make_float2(s.a[ch], s.b[ch]);
+    }
+    __device__ static float apply(const ParamSrc&, const P& p, float x, float g, int& code)
+    {
+        code = 0;
+        return g * (float) ((p.x <= x) && (x <= p.y));
+    }
+};
+
+struct OpV2
+{
+    using P = float2;   // scale, offset
+    __device__ static P load(const ParamSrc& s, uint32_t ch)
+    {
+        return make_float2(s.a[ch], s.b[ch]);
+    }
+};
+
+struct OpV2Qdq : OpV2
+{
+    static constexpr int NIN = 1;
+    using Code               = int32_t;
+    __device__ static float apply(const ParamSrc& s, const P& p, float x, float, int& code)
+    {
+        float r = rintf(x / p.x) - p.y;
+        // torch.clamp semantics: NaN stays NaN
+        float q = r;
+        q       = (q < (float) s.qmin) ? (float) s.qmin : q;
+        q       = (q > (float) s.qmax) ? (float) s.qmax : q;
+        code    = (int) q;
+        return (q + p.y) * p.x;
+    }
+};
+
+struct OpV2Bwd : OpV2
+{
+    static constexpr int NIN = 2;
+    using Code               = int32_t;
+    __device__ static float apply(const ParamSrc& s, const P& p, float x, float g, int& code)
+    {
+        float r = rintf(x / p.x) - p.y;
+        code    = 0;
+        return g * (float) (((float) s.qmin <= r) && (r <= (float) s.qmax));
+    }
+};
+
+template <typename OP>
+__device__ typename OP::P scalar_params(const ParamSrc& s);
+template <>
+__device__ float4 scalar_params<OpV1Qdq>(const ParamSrc& s)
+{
+    return s.scalar;
+}
+template <>
+__device__ float4 scalar_params<OpV1Quantize>(const ParamSrc& s)
+{
+    return s.scalar;
+}
+template <>
+__device__ float2 scalar_params<OpV1Ste>(const ParamSrc& s)
+{
+    return make_float2(s.scalar.x, s.scalar.y);
+}
+// v2 per-tensor: scale/offset are one-element device tensors; the load is wave-uniform (scalar load)
+template <>
+__device__ float2 scalar_params<OpV2Qdq>(const ParamSrc& s)
+{
+    return make_float2(s.a[0], s.b[0]);
+}
+template <>
+__device__ float2 scalar_params<OpV2Bwd>(const ParamSrc& s)
+{
+    return make_float2(s.a[0], s.b[0]);
+}
+
+// ----------------------------------------------------------------------------------------------------- the kernels
+template <typename IO, typename CodeT>
+struct EwPtrs
+{
+    const IO* x;
+    const IO* g;    // second input (backward), else unused
+    IO* y;          // may be null when only codes are wanted
+    CodeT* codes;   // may be null
+};
+
+constexpr int kWin = 264;   // LDS window rows; host guarantees tile / elements-per-channel + 2 <= kWin
+
+template <typename CodeT, int VEC>
+__device__ __forceinline__ void store_codes(CodeT* dst, const int* c);
+
+template <>
+__device__ __forceinline__ void store_codes<uint8_t, 4>(uint8_t* dst, const int* c)
+{
+    uint32_t w = (uint32_t) (c[0] & 0xff) | ((uint32_t) (c[1] & 0xff) << 8) | ((uint32_t) (c[2] & 0xff) << 16) |
+                 ((uint32_t) (c[3] & 0xff) << 24);
+    *reinterpret_cast<uint32_t*>(dst) = w;
+}
+template <>
+__device__ __forceinline__ void store_codes<uint8_t, 8>(uint8_t* dst, const int* c)
+{
+    store_codes<uint8_t, 4>(dst, c);
+    store_codes<uint8_t, 4>(dst + 4, c + 4);
+}
+template <>
+__device__ __forceinline__ void store_codes<int32_t, 4>(int32_t* dst, const int* c)
+{
+    *reinterpret_cast<int4*>(dst) = make_int4(c[0], c[1], c[2], c[3]);
+}
+template <>
+__device__ __forceinline__ void store_codes<int32_t, 8>(int32_t* dst, const int* c)
+{
+    store_codes<int32_t, 4>(dst, c);
+    store_codes<int32_t, 4>(dst + 4, c + 4);
+}
+
+// Vectorised tile kernel.  Requires 16-byte aligned pointers; n < 2^31 when PER_CHANNEL.
+template <typename IO, typename OP, bool PER_CHANNEL>
+__global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::Code> ptr, ParamSrc src, int64_t n,
+                                                        uint32_t num_channel, FastDiv fd)
+{
+    using T                 = IOTraits<IO>;
+    using Vec               = typename T::Vec;
+    using P                 = typename OP::P;
+    constexpr int VEC       = T::VEC;
+    constexpr uint32_t TILE = kBlock * kUnroll * VEC;
+    const int64_t e_base    = (int64_t) blockIdx.x * TILE;
+    const int64_t nvec      = n / VEC;
+
+    __shared__ P win[PER_CHANNEL ? kWin : 1];
+    uint32_t rem0 = 0;
+    P pt;
+    if constexpr (PER_CHANNEL)
+    {
+        const uint32_t eb   = (uint32_t) e_base;
+        const uint32_t row0 = fastdiv(eb, fd);
+        rem0                = eb - row0 * fd.d;
+        const uint32_t ee   = (uint32_t) (((int64_t) eb + TILE < n) ? eb + TILE : n);
+        const uint32_t row1 = fastdiv(ee - 1, fd);
+        for (uint32_t r = threadIdx.x; r <= row1 - row0; r += kBlock)
+            win[r] = OP::load(src, (row0 + r) % num_channel);
+        __syncthreads();
+    }
+    else
+    {
+        pt = scalar_params<OP>(src);
+    }
+
+    Vec vx[kUnroll], vg[kUnroll];
+    bool live[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+    {
+        const int64_t v = e_base / VEC + (int64_t) u * kBlock + threadIdx.x;
+        live[u]         = v < nvec;
+        if (live[u])
+        {
+            vx[u] = reinterpret_cast<const Vec*>(ptr.x)[v];
+            if constexpr (OP::NIN == 2)
+                vg[u] = reinterpret_cast<const Vec*>(ptr.g)[v];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+    {
+        if (!live[u])
+            continue;
+        const uint32_t le = ((uint32_t) u * kBlock + threadIdx.x) * VEC;
+        const int64_t v   = e_base / VEC + (int64_t) u * kBlock + threadIdx.x;
+        float fx[VEC], fg[VEC], fy[VEC];
+        int code[VEC];
+        T::unpack(vx[u], fx);
+        if constexpr (OP::NIN == 2)
+            T::unpack(vg[u], fg);
+        if constexpr (PER_CHANNEL)
+        {
+            const uint32_t t   = rem0 + le;
+            const uint32_t lr  = fastdiv(t, fd);
+            const uint32_t rem = t - lr * fd.d;
+            if (rem + VEC <= fd.d)
+            {
+                const P p = win[lr];
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                    fy[j] = OP::apply(src, p, fx[j], OP::NIN == 2 ? fg[j] : 0.f, code[j]);
+            }
+            else
+            {
+                // the vector straddles one channel boundary (elements-per-channel is not a multiple of VEC)
+#pragma unroll
+                for (int j = 0; j < VEC; ++j)
+                {
+                    const P p = win[lr + ((rem + j >= fd.d) ? 1u : 0u)];
+                    fy[j]     = OP::apply(src, p, fx[j], OP::NIN == 2 ? fg[j] : 0.f, code[j]);
+                }
+            }
+        }
+        else
+        {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+                fy[j] = OP::apply(src, pt, fx[j], OP::NIN == 2 ? fg[j] : 0.f, code[j]);
+        }
+        if (ptr.y)
+            reinterpret_cast<Vec*>(ptr.y)[v] = T::pack(fy);
+        if (ptr.codes)
+            store_codes<typename OP::Code, VEC>(ptr.codes + v * VEC, code);
+    }
+    // the n % VEC trailing elements
+    if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * VEC))
+    {
+        const int64_t e = nvec * VEC + threadIdx.x;
+        P p;
+        if constexpr (PER_CHANNEL)
+            p = OP::load(src, (uint32_t) ((e / fd.d) % num_channel));
+        else
+            p = pt;
+        int code;
+        const float y = OP::apply(src, p, T::load1(ptr.x + e), OP::NIN == 2 ? T::load1(ptr.g + e) : 0.f, code);
+        if (ptr.y)
+            T::store1(ptr.y + e, y);
+        if (ptr.codes)
+            ptr.codes[e] = (typename OP::Code) code;
+    }
+}
+
+// Fallback for unaligned pointers, tiny channels (elements-per-channel < 16) and n >= 2^31: one element per lane,
+// grid-stride, 64-bit indexing, parameters read through the cache.
+template <typename IO, typename OP, bool PER_CHANNEL>
+__global__ __launch_bounds__(kBlock) void ew_scalar_kernel(EwPtrs<IO, typename OP::Code> ptr, ParamSrc src, int64_t n,
+                                                           int64_t num_channel, int64_t n_per_channel)
+{
+    using T = IOTraits<IO>;
+    using P = typename OP::P;
+    for (int64_t e = (int64_t) blockIdx.x * kBlock + threadIdx.x; e < n; e += (int64_t) gridDim.x * kBlock)
+    {
+        P p;
+        if constexpr (PER_CHANNEL)
+            p = OP::load(src, (uint32_t) ((e / n_per_channel) % num_channel));
+        else
+            p = scalar_params<OP>(src);
+        int code;
+        const float y = OP::apply(src, p, T::load1(ptr.x + e), OP::NIN == 2 ? T::load1(ptr.g + e) : 0.f, code);
+        if (ptr.y)
+            T::store1(ptr.y + e, y);
+        if (ptr.codes)
+            ptr.codes[e] = (typename OP::Code) code;
+    }
+}
+
+template <typename IO, typename OP, bool PER_CHANNEL>
+int launch_ew(EwPtrs<IO, typename OP::Code> ptr, const ParamSrc& src, int64_t n, int64_t num_channel,
+              int64_t n_per_channel, hipStream_t stream)
+{
+    if (n == 0)
+        return MIQ_OK;
+    using T                = IOTraits<IO>;
+    constexpr int64_t TILE = (int64_t) kBlock * kUnroll * T::VEC;
+    bool vec_ok = aligned16(ptr.x) && (OP::NIN == 1 || aligned16(ptr.g)) && (!ptr.y || aligned16(ptr.y)) &&
+                  (!ptr.codes || aligned16(ptr.codes));
+    if (PER_CHANNEL)
+        vec_ok = vec_ok && n < (1ll << 31) && n_per_channel < (1ll << 31) &&
+                 (TILE / n_per_channel + 2 <= kWin);
+    if (vec_ok)
+    {
+        const int64_t blocks = (n + TILE - 1) / TILE;
+        FastDiv fd           = make_fastdiv(PER_CHANNEL ? (uint32_t) n_per_channel : 1u);
+        hipLaunchKernelGGL((ew_vec_kernel<IO, OP, PER_CHANNEL>), dim3((unsigned) blocks), dim3(kBlock), 0, stream, ptr,
+                           src, n, (uint32_t) num_channel, fd);
+    }
+    else
+    {
+        int64_t blocks = (n + kBlock - 1) / kBlock;
+        if (blocks > 65536)
+            blocks = 65536;
+        hipLaunchKernelGGL((ew_scalar_kernel<IO, OP, PER_CHANNEL>), dim3((unsigned) blocks), dim3(kBlock), 0, stream,
+                           ptr, src, n, num_channel, n_per_channel);
+    }
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int check_round(int rounding_mode)
+{
+    if (rounding_mode == MIQ_ROUND_NEAREST)
+        return MIQ_OK;
+    if (rounding_mode == MIQ_ROUND_STOCHASTIC)
+    {
+        set_error("stochastic rounding is not implemented (the reference's is not reproducible by design)");
+        return MIQ_ERR_UNSUPPORTED;
+    }
+    set_error("unknown rounding mode %d", rounding_mode);
+    return MIQ_ERR_INVALID_ARG;
+}
+
+int check_channels(int64_t num_channel, int64_t num_element, int64_t n_per_channel)
+{
+    MIQ_CHECK_ARG(num_channel > 0 && num_channel < (1ll << 31), "num_channel must be in [1, 2^31)");
+    MIQ_CHECK_ARG(n_per_channel > 0, "num_element_per_channel must be positive");
+    MIQ_CHECK_ARG(num_element >= 0, "num_element must be non-negative");
+    return MIQ_OK;
+}
+
+ParamSrc per_tensor_src(const miq_encoding& e)
+{
+    ParamSrc s{};
+    s.scalar = make_float4((float) e.min, (float) e.max, (float) e.delta, (float) e.offset);
+    return s;
+}
+
+// per-channel parameter recipe, float32, operation for operation as the ATen sequence of the reference
+__global__ void per_channel_params_kernel(const float* enc_min, const float* enc_max, int64_t c, float num_steps,
+                                          float* omin, float* omax, float* odelta, float* ooffset)
+{
+    const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= c)
+        return;
+    float lo = enc_min[i], hi = enc_max[i];
+    // torch.minimum / torch.maximum propagate NaN
+    lo        = (lo != lo) ? lo : fminf(lo, 0.f);
+    hi        = (hi != hi) ? hi : fmaxf(hi, 0.f);
+    float eps = lo + 1e-5f;
+    hi        = (hi != hi || eps != eps) ? (hi + eps) : fmaxf(hi, eps);
+    float d   = (hi - lo) / num_steps;
+    omin[i]   = lo;
+    omax[i]   = hi;
+    odelta[i] = d;
+    ooffset[i] = rintf(lo / d);
+}
+
+struct BcastArgs
+{
+    int64_t istride[8];
+    int64_t estride[8];
+    int ndims;
+};
+
+// numpy-style broadcast of the encoding (DlQuantization/src/trim_functions.cpp:634-660); the reference keeps the
+// running remainder and the indices in `int`, so this path is defined for fewer than 2^31 elements.
+__global__ __launch_bounds__(kBlock) void qdq_broadcast_kernel(const float* in, float* out, int64_t n, BcastArgs b,
+                                                               const float* mn, const float* mx, const float* delta,
+                                                               const float* offset)
+{
+    for (int64_t e = (int64_t) blockIdx.x * kBlock + threadIdx.x; e < n; e += (int64_t) gridDim.x * kBlock)
+    {
+        int enc = 0;
+        int rem = (int) e;
+        for (int d = 0; d < b.ndims; ++d)
+        {
+            int idx = (int) (rem / b.istride[d]);
+            rem     = (int) (rem - idx * b.istride[d]);
+            enc += (int) (b.estride[d] * idx);
+        }
+        const float4 p = make_float4(mn[enc], mx[enc], delta[enc], offset[enc]);
+        const float q  = OpV1::quant(p, in[e]);
+        out[e]         = p.z * (q + p.w);
+    }
+}
+static ParamSrc v1_channel_src(const float* mn, const float* mx, const float* d, const float* o)
+{
+    ParamSrc s{};
+    s.a = mn;
+    s.b = mx;
+    s.c = d;
+    s.d = o;
+    return s;
+}
+
+static int check_v2(int64_t num_channel, int64_t num_element, int64_t npc, const float* scale, const float* offset,
+                    int qmin, int qmax)
+{
+    if (int rc = check_channels(num_channel, num_element, npc))
+        return rc;
+    MIQ_CHECK_ARG(scale && offset, "null scale/offset pointer");
+    MIQ_CHECK_ARG(qmin <= qmax, "qmin (%d) must be smaller than or equal to qmax (%d)", qmin, qmax);
+    // float32 must represent the grid exactly (torch_builtins.py:52-69)
+    MIQ_CHECK_ARG(qmin > -(1 << 24) && qmax < (1 << 24), "float32 is unable to represent the grid [%d, %d]", qmin,
+                  qmax);
+    return MIQ_OK;
+}
+
+template <typename IO, typename OP>
+static int launch_v2(EwPtrs<IO, int32_t> p, const ParamSrc& s, int64_t n, int64_t num_channel, int64_t npc,
+                     hipStream_t stream)
+{
+    if (num_channel == 1)
+        return launch_ew<IO, OP, false>(p, s, n, 1, 1, stream);
+    return launch_ew<IO, OP, true>(p, s, n, num_channel, npc, stream);
+}
+
+static ParamSrc v2_src(const float* scale, const float* offset, int qmin, int qmax)
+{
+    ParamSrc s{};
+    s.a    = scale;
+    s.b    = offset;
+    s.qmin = qmin;
+    s.qmax = qmax;
+    return s;
+}
+}   // namespace
+}   // namespace miq
+
+using namespace miq;
+
+extern "C" {
+
+int miq_qdq_per_tensor_f32(const float* in, float* out, int64_t n, double enc_min, double enc_max, int bw,
+                           int rounding_mode, void* stream)
+{
+    MIQ_CHECK_ARG(n >= 0 && (n == 0 || (in && out)), "null tensor pointer or negative count");
+    if (int rc = check_round(rounding_mode))
+        return rc;
+    miq_encoding e;
+    if (int rc = miq_fill_encoding_info(bw, enc_min, enc_max, &e))
+        return rc;
+    EwPtrs<float, uint8_t> p{in, nullptr, out, nullptr};
+    return launch_ew<float, OpV1Qdq, false>(p, per_tensor_src(e), n, 1, 1, (hipStream_t) stream);
+}
+
+int miq_qdq_per_tensor_bf16(const uint16_t* in, uint16_t* out, int64_t n, double enc_min, double enc_max, int bw,
+                            int rounding_mode, void* stream)
+{
+    MIQ_CHECK_ARG(n >= 0 && (n == 0 || (in && out)), "null tensor pointer or negative count");
+    if (int rc = check_round(rounding_mode))
+        return rc;
+    miq_encoding e;
+    if (int rc = miq_fill_encoding_info(bw, enc_min, enc_max, &e))
+        return rc;
+    EwPtrs<uint16_t, uint8_t> p{in, nullptr, out, nullptr};
+    return launch_ew<uint16_t, OpV1Qdq, false>(p, per_tensor_src(e), n, 1, 1, (hipStream_t) stream);
+}
+
+int miq_quantize_per_tensor_f32(const float* in, float* out, int64_t n, double enc_min, double enc_max, int bw,
+                                int rounding_mode, int shift_to_signed, void* stream)
+{
+    MIQ_CHECK_ARG(n >= 0 && (n == 0 || (in && out)), "null tensor pointer or negative count");
+    if (int rc = check_round(rounding_mode))
+        return rc;
+    miq_encoding e;
+    if (int rc = miq_fill_encoding_info(bw, enc_min, enc_max, &e))
+        return rc;
+    ParamSrc s = per_tensor_src(e);
+    // DlQuantization/src/trim_functions.cpp:207-216: shift = 2^(bw-1) held in an unsigned int, subtracted in float
+    unsigned int shift = shift_to_signed ? (unsigned int) std::pow(2, bw - 1) : 0u;
+    s.shift            = (float) shift;
+    EwPtrs<float, uint8_t> p{in, nullptr, out, nullptr};
+    return launch_ew<float, OpV1Quantize, false>(p, s, n, 1, 1, (hipStream_t) stream);
+}
+
+int miq_qdq_codes_per_tensor_f32(const float* in, float* out, uint8_t* codes, int64_t n, double enc_min,
+                                 double enc_max, int bw, int shift_to_signed, void* stream)
+{
+    MIQ_CHECK_ARG(n >= 0 && (n == 0 || (in && codes)), "null tensor pointer or negative count");
+    MIQ_CHECK_ARG(bw >= 1 && bw <= 8, "byte codes need 1 <= bw <= 8 (got %d)", bw);
+    miq_encoding e;
+    if (int rc = miq_fill_encoding_info(bw, enc_min, enc_max, &e))
+        return rc;
+    ParamSrc s = per_tensor_src(e);
+    s.ishift   = shift_to_signed ? (1 << (bw - 1)) : 0;
+    EwPtrs<float, uint8_t> p{in, nullptr, out, codes};
+    return launch_ew<float, OpV1Qdq, false>(p, s, n, 1, 1, (hipStream_t) stream);
+}
+
+int miq_per_channel_params_f32(const float* enc_min, const float* enc_max, int64_t num_channel, double num_steps,
+                               float* out_min, float* out_max, float* out_delta, float* out_offset, void* stream)
+{
+    MIQ_CHECK_ARG(num_channel > 0 && enc_min && enc_max && out_min && out_max && out_delta && out_offset,
+                  "null pointer or non-positive channel count");
+    MIQ_CHECK_ARG(num_steps > 0, "num_steps must be positive");
+    const int64_t blocks = (num_channel + kBlock - 1) / kBlock;
+    hipLaunchKernelGGL(per_channel_params_kernel, dim3((unsigned) blocks), dim3(kBlock), 0, (hipStream_t) stream,
+                       enc_min, enc_max, num_channel, (float) num_steps, out_min, out_max, out_delta, out_offset);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+
+int miq_qdq_per_channel_f32(const float* in, float* out, int64_t num_channel, int64_t num_element,
+                            int64_t num_element_per_channel, const float* enc_min, const float* enc_max,
+                            const float* enc_delta, const float* enc_offset, int rounding_mode, void* stream)
+{
+    if (int rc = check_channels(num_channel, num_element, num_element_per_channel))
+        return rc;
+    MIQ_CHECK_ARG(num_element == 0 || (in && out && enc_min && enc_max && enc_delta && enc_offset), "null pointer");
+    if (int rc = check_round(rounding_mode))
+        return rc;
+    EwPtrs<float, uint8_t> p{in, nullptr, out, nullptr};
+    return launch_ew<float, OpV1Qdq, true>(p, v1_channel_src(enc_min, enc_max, enc_delta, enc_offset), num_element,
+                                           num_channel, num_element_per_channel, (hipStream_t) stream);
+}
+
+int miq_qdq_per_channel_bf16(const uint16_t* in, uint16_t* out, int64_t num_channel, int64_t num_element,
+                             int64_t num_element_per_channel, const float* enc_min, const float* enc_max,
+                             const float* enc_delta, const float* enc_offset, int rounding_mode, void* stream)
+{
+    if (int rc = check_channels(num_channel, num_element, num_element_per_channel))
+        return rc;
+    MIQ_CHECK_ARG(num_element == 0 || (in && out && enc_min && enc_max && enc_delta && enc_offset), "null pointer");
+    if (int rc = check_round(rounding_mode))
+        return rc;
+    EwPtrs<uint16_t, uint8_t> p{in, nullptr, out, nullptr};
+    return launch_ew<uint16_t, OpV1Qdq, true>(p, v1_channel_src(enc_min, enc_max, enc_delta, enc_offset), num_element,
+                                              num_channel, num_element_per_channel, (hipStream_t) stream);
+}
+
+int miq_qdq_codes_per_channel_f32(const float* in, float* out, uint8_t* codes, int64_t num_channel,
+                                  int64_t num_element, int64_t num_element_per_channel, const float* enc_min,
+                                  const float* enc_max, const float* enc_delta, const float* enc_offset,
+                                  int shift_to_signed, int bw, void* stream)
+{
+    if (int rc = check_channels(num_channel, num_element, num_element_per_channel))
+        return rc;
+    MIQ_CHECK_ARG(num_element == 0 || (in && codes && enc_min && enc_max && enc_delta && enc_offset), "null pointer");
+    MIQ_CHECK_ARG(bw >= 1 && bw <= 8, "byte codes need 1 <= bw <= 8 (got %d)", bw);
+    ParamSrc s = v1_channel_src(enc_min, enc_max, enc_delta, enc_offset);
+    s.ishift   = shift_to_signed ? (1 << (bw - 1)) : 0;
+    EwPtrs<float, uint8_t> p{in, nullptr, out, codes};
+    return launch_ew<float, OpV1Qdq, true>(p, s, num_element, num_channel, num_element_per_channel,
+                                           (hipStream_t) stream);
+}
+
+int miq_qdq_broadcast_f32(const float* in, float* out, int64_t num_element, int64_t num_dims,
+                          const int64_t* input_strides, const int64_t* encoding_strides, const float* enc_min,
+                          const float* enc_max, const float* enc_delta, const float* enc_offset, void* stream)
+{
+    MIQ_CHECK_ARG(num_element >= 0 && num_element < (1ll << 31), "num_element must be in [0, 2^31)");
+    MIQ_CHECK_ARG(num_dims >= 1 && num_dims <= 8, "num_dims must be in [1, 8]");
+    MIQ_CHECK_ARG(input_strides && encoding_strides, "null stride array");
+    MIQ_CHECK_ARG(num_element == 0 || (in && out && enc_min && enc_max && enc_delta && enc_offset), "null pointer");
+    if (num_element == 0)
+        return MIQ_OK;
+    BcastArgs b{};
+    b.ndims = (int) num_dims;
+    for (int d = 0; d < b.ndims; ++d)
+    {
+        MIQ_CHECK_ARG(input_strides[d] > 0, "input strides must be positive");
+        b.istride[d] = input_strides[d];
+        b.estride[d] = encoding_strides[d];
+    }
+    int64_t blocks = (num_element + kBlock - 1) / kBlock;
+    if (blocks > 65536)
+        blocks = 65536;
+    hipLaunchKernelGGL(qdq_broadcast_kernel, dim3((unsigned) blocks), dim3(kBlock), 0, (hipStream_t) stream, in, out,
+                       num_element, b, enc_min, enc_max, enc_delta, enc_offset);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int miq_ste_bwd_per_tensor_f32(const float* x, const float* grad_out, float* grad_in, int64_t n, float enc_min,
+                               float enc_max, void* stream)
+{
+    MIQ_CHECK_ARG(n >= 0 && (n == 0 || (x && grad_out && grad_in)), "null tensor pointer or negative count");
+    ParamSrc s{};
+    s.scalar = make_float4(enc_min, enc_max, 0.f, 0.f);
+    EwPtrs<float, uint8_t> p{x, grad_out, grad_in, nullptr};
+    return launch_ew<float, OpV1Ste, false>(p, s, n, 1, 1, (hipStream_t) stream);
+}
+
+int miq_ste_bwd_per_tensor_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* grad_in, int64_t n,
+                                float enc_min, float enc_max, void* stream)
+{
+    MIQ_CHECK_ARG(n >= 0 && (n == 0 || (x && grad_out && grad_in)), "null tensor pointer or negative count");
+    ParamSrc s{};
+    s.scalar = make_float4(enc_min, enc_max, 0.f, 0.f);
+    EwPtrs<uint16_t, uint8_t> p{x, grad_out, grad_in, nullptr};
+    return launch_ew<uint16_t, OpV1Ste, false>(p, s, n, 1, 1, (hipStream_t) stream);
+}
+
+int miq_ste_bwd_per_channel_f32(const float* x, const float* grad_out, float* grad_in, int64_t num_channel,
+                                int64_t num_element, int64_t num_element_per_channel, const float* enc_min,
+                                const float* enc_max, void* stream)
+{
+    if (int rc = check_channels(num_channel, num_element, num_element_per_channel))
+        return rc;
+    MIQ_CHECK_ARG(num_element == 0 || (x && grad_out && grad_in && enc_min && enc_max), "null pointer");
+    ParamSrc s{};
+    s.a = enc_min;
+    s.b = enc_max;
+    EwPtrs<float, uint8_t> p{x, grad_out, grad_in, nullptr};
+    return launch_ew<float, OpV1Ste, true>(p, s, num_element, num_channel, num_element_per_channel,
+                                           (hipStream_t) stream);
+}
+
+int miq_ste_bwd_per_channel_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* grad_in,
+                                 int64_t num_channel, int64_t num_element, int64_t num_element_per_channel,
+                                 const float* enc_min, const float* enc_max, void* stream)
+{
+    if (int rc = check_channels(num_channel, num_element, num_element_per_channel))
+        return rc;
+    MIQ_CHECK_ARG(num_element == 0 || (x && grad_out && grad_in && enc_min && enc_max), "null pointer");
+    ParamSrc s{};
+    s.a = enc_min;
+    s.b = enc_max;
+    EwPtrs<uint16_t, uint8_t> p{x, grad_out, grad_in, nullptr};
+    return launch_ew<uint16_t, OpV1Ste, true>(p, s, num_element, num_channel, num_element_per_channel,
+                                              (hipStream_t) stream);
+}
+
+
+
+
+int miq_v2_qdq_f32(const float* in, float* out, int32_t* codes, int64_t num_channel, int64_t num_element,
+                   int64_t num_element_per_channel, const float* scale, const float* offset, int qmin, int qmax,
+                   void* stream)
+{
+    if (int rc = check_v2(num_channel, num_element, num_element_per_channel, scale, offset, qmin, qmax))
+        return rc;
+    MIQ_CHECK_ARG(num_element == 0 || (in && (out || codes)), "null pointer");
+    EwPtrs<float, int32_t> p{in, nullptr, out, codes};
+    return launch_v2<float, OpV2Qdq>(p, v2_src(scale, offset, qmin, qmax), num_element, num_channel,
+                                     num_element_per_channel, (hipStream_t) stream);
+}
+
+int miq_v2_qdq_bf16(const uint16_t* in, uint16_t* out, int64_t num_channel, int64_t num_element,
+                    int64_t num_element_per_channel, const float* scale, const float* offset, int qmin, int qmax,
+                    void* stream)
+{
+    if (int rc = check_v2(num_channel, num_element, num_element_per_channel, scale, offset, qmin, qmax))
+        return rc;
+    MIQ_CHECK_ARG(num_element == 0 || (in && out), "null pointer");
+    EwPtrs<uint16_t, int32_t> p{in, nullptr, out, nullptr};
+    return launch_v2<uint16_t, OpV2Qdq>(p, v2_src(scale, offset, qmin, qmax), num_element, num_channel,
+                                        num_element_per_channel, (hipStream_t) stream);
+}
+
+int miq_v2_qdq_bwd_f32(const float* x, const float* grad_out, float* grad_in, int64_t num_channel,
+                       int64_t num_element, int64_t num_element_per_channel, const float* scale,
+                       const float* offset, int qmin, int qmax, void* stream)
+{
+    if (int rc = check_v2(num_channel, num_element, num_element_per_channel, scale, offset, qmin, qmax))
+        return rc;
+    MIQ_CHECK_ARG(num_element == 0 || (x && grad_out && grad_in), "null pointer");
+    EwPtrs<float, int32_t> p{x, grad_out, grad_in, nullptr};
+    return launch_v2<float, OpV2Bwd>(p, v2_src(scale, offset, qmin, qmax), num_element, num_channel,
+                                     num_element_per_channel, (hipStream_t) stream);
+}
+
+int miq_v2_qdq_bwd_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* grad_in, int64_t num_channel,
+                        int64_t num_element, int64_t num_element_per_channel, const float* scale,
+                        const float* offset, int qmin, int qmax, void* stream)
+{
+    if (int rc = check_v2(num_channel, num_element, num_element_per_channel, scale, offset, qmin, qmax))
+        return rc;
+    MIQ_CHECK_ARG(num_element == 0 || (x && grad_out && grad_in), "null pointer");
+    EwPtrs<uint16_t, int32_t> p{x, grad_out, grad_in, nullptr};
+    return launch_v2<uint16_t, OpV2Bwd>(p, v2_src(scale, offset, qmin, qmax), num_element, num_channel,
+                                        num_element_per_channel, (hipStream_t) stream);
+}
+
+}   // extern "C"

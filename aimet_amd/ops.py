@@ -1,0 +1,293 @@
+"""Tensor-level entry points over the libmiq C ABI.
+
+Every function takes CUDA(HIP) tensors, launches on torch's *current* stream of the tensor's device and returns
+without synchronising (except the analyzer read-backs, which must).  torch is used for device memory and streams
+only; there is no torch-op fallback: tensors that are not on a GPU are rejected.
+"""
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import Encoding, check, lib
+
+_F32, _BF16 = torch.float32, torch.bfloat16
+
+
+def _stream(t):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _require_gpu(*tensors):
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("aimet_amd kernels run on the GPU only; got a tensor on " + str(t.device))
+        if t.device != tensors[0].device:
+            raise RuntimeError(f"tensors are on different devices: {t.device} vs {tensors[0].device}")
+
+
+def _suffix(t):
+    if t.dtype == _F32:
+        return "f32"
+    if t.dtype == _BF16:
+        return "bf16"
+    raise RuntimeError(f"unsupported dtype {t.dtype}: float32 and bfloat16 are implemented")
+
+
+def _params_f32(t, like):
+    return t.to(device=like.device, dtype=_F32).contiguous()
+
+
+# ---------------------------------------------------------------------------------------------------------- host math
+def fill_encoding_info(bw, enc_min, enc_max):
+    e = Encoding()
+    check(lib.miq_fill_encoding_info(int(bw), float(enc_min), float(enc_max), C.byref(e)))
+    return e
+
+
+def get_computed_encodings(bw, mn, mx, symmetric, strict_symmetric, unsigned_symmetric):
+    e = Encoding()
+    check(lib.miq_get_computed_encodings(int(bw), float(mn), float(mx), int(symmetric), int(strict_symmetric),
+                                         int(unsigned_symmetric), C.byref(e)))
+    return e
+
+
+# ------------------------------------------------------------------------------------------------------------ v1 QDQ
+def qdq_per_tensor(x, enc_min, enc_max, bw, rounding_mode=_lib.ROUND_NEAREST, out=None):
+    """DlQuantization per-tensor quantize-dequantize; float32 or bfloat16 storage, float32 arithmetic."""
+    _require_gpu(x, out)
+    x = x.contiguous()
+    out = torch.empty_like(x) if out is None else out
+    fn = getattr(lib, "miq_qdq_per_tensor_" + _suffix(x))
+    with torch.cuda.device(x.device):
+        check(fn(_ptr(x), _ptr(out), x.numel(), float(enc_min), float(enc_max), int(bw), int(rounding_mode),
+                 _stream(x)))
+    return out
+
+
+def quantize_per_tensor(x, enc_min, enc_max, bw, shift_to_signed, rounding_mode=_lib.ROUND_NEAREST):
+    """Float-valued grid indices (minus 2^(bw-1) when shift_to_signed)."""
+    _require_gpu(x)
+    x = x.to(_F32).contiguous()
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        check(lib.miq_quantize_per_tensor_f32(_ptr(x), _ptr(out), x.numel(), float(enc_min), float(enc_max), int(bw),
+                                              int(rounding_mode), int(bool(shift_to_signed)), _stream(x)))
+    return out
+
+
+def qdq_codes_per_tensor(x, enc_min, enc_max, bw, shift_to_signed=False, want_dequant=True):
+    """One pass producing (dequantized or None, byte codes): uint8 grid index, or int8 when shift_to_signed."""
+    _require_gpu(x)
+    x = x.to(_F32).contiguous()
+    out = torch.empty_like(x) if want_dequant else None
+    codes = torch.empty(x.shape, dtype=torch.int8 if shift_to_signed else torch.uint8, device=x.device)
+    with torch.cuda.device(x.device):
+        check(lib.miq_qdq_codes_per_tensor_f32(_ptr(x), _ptr(out), _ptr(codes), x.numel(), float(enc_min),
+                                               float(enc_max), int(bw), int(bool(shift_to_signed)), _stream(x)))
+    return out, codes
+
+
+def per_channel_params(enc_min, enc_max, num_steps):
+    """(min, max, delta, offset) float32 device vectors from raw per-channel min/max (float32 tensors on the GPU)."""
+    _require_gpu(enc_min, enc_max)
+    enc_min, enc_max = enc_min.to(_F32).contiguous(), enc_max.to(_F32).contiguous()
+    c = enc_min.numel()
+    outs = torch.empty(4, c, dtype=_F32, device=enc_min.device)
+    with torch.cuda.device(enc_min.device):
+        check(lib.miq_per_channel_params_f32(_ptr(enc_min), _ptr(enc_max), c, float(num_steps), _ptr(outs[0]),
+                                             _ptr(outs[1]), _ptr(outs[2]), _ptr(outs[3]), _stream(enc_min)))
+    return outs[0], outs[1], outs[2], outs[3]
+
+
+def qdq_per_channel(x, num_channel, n_per_channel, mn, mx, delta, offset, rounding_mode=_lib.ROUND_NEAREST,
+                    out=None):
+    _require_gpu(x, mn, mx, delta, offset, out)
+    x = x.contiguous()
+    out = torch.empty_like(x) if out is None else out
+    fn = getattr(lib, "miq_qdq_per_channel_" + _suffix(x))
+    mn, mx, delta, offset = (_params_f32(p, x) for p in (mn, mx, delta, offset))
+    with torch.cuda.device(x.device):
+        check(fn(_ptr(x), _ptr(out), int(num_channel), x.numel(), int(n_per_channel), _ptr(mn), _ptr(mx),
+                 _ptr(delta), _ptr(offset), int(rounding_mode), _stream(x)))
+    return out
+
+
+def qdq_codes_per_channel(x, num_channel, n_per_channel, mn, mx, delta, offset, bw, shift_to_signed=False,
+                          want_dequant=True):
+    _require_gpu(x, mn, mx, delta, offset)
+    x = x.to(_F32).contiguous()
+    out = torch.empty_like(x) if want_dequant else None
+    codes = torch.empty(x.shape, dtype=torch.int8 if shift_to_signed else torch.uint8, device=x.device)
+    mn, mx, delta, offset = (_params_f32(p, x) for p in (mn, mx, delta, offset))
+    with torch.cuda.device(x.device):
+        check(lib.miq_qdq_codes_per_channel_f32(_ptr(x), _ptr(out), _ptr(codes), int(num_channel), x.numel(),
+                                                int(n_per_channel), _ptr(mn), _ptr(mx), _ptr(delta), _ptr(offset),
+                                                int(bool(shift_to_signed)), int(bw), _stream(x)))
+    return out, codes
+
+
+def qdq_broadcast(x, input_strides, encoding_strides, mn, mx, delta, offset):
+    _require_gpu(x, mn, mx, delta, offset)
+    x = x.to(_F32).contiguous()
+    out = torch.empty_like(x)
+    nd = len(input_strides)
+    ist = (C.c_int64 * nd)(*[int(v) for v in input_strides])
+    est = (C.c_int64 * nd)(*[int(v) for v in encoding_strides])
+    mn, mx, delta, offset = (_params_f32(p, x) for p in (mn, mx, delta, offset))
+    with torch.cuda.device(x.device):
+        check(lib.miq_qdq_broadcast_f32(_ptr(x), _ptr(out), x.numel(), nd, ist, est, _ptr(mn), _ptr(mx), _ptr(delta),
+                                        _ptr(offset), _stream(x)))
+    return out
+
+
+def ste_bwd_per_tensor(x, grad_out, enc_min, enc_max, out=None):
+    _require_gpu(x, grad_out, out)
+    x, grad_out = x.contiguous(), grad_out.to(x.dtype).contiguous()
+    gin = torch.empty_like(x) if out is None else out
+    fn = getattr(lib, "miq_ste_bwd_per_tensor_" + _suffix(x))
+    with torch.cuda.device(x.device):
+        check(fn(_ptr(x), _ptr(grad_out), _ptr(gin), x.numel(), float(enc_min), float(enc_max), _stream(x)))
+    return gin
+
+
+def ste_bwd_per_channel(x, grad_out, num_channel, n_per_channel, enc_min, enc_max, out=None):
+    _require_gpu(x, grad_out, enc_min, enc_max, out)
+    x, grad_out = x.contiguous(), grad_out.to(x.dtype).contiguous()
+    gin = torch.empty_like(x) if out is None else out
+    fn = getattr(lib, "miq_ste_bwd_per_channel_" + _suffix(x))
+    enc_min, enc_max = _params_f32(enc_min, x), _params_f32(enc_max, x)
+    with torch.cuda.device(x.device):
+        check(fn(_ptr(x), _ptr(grad_out), _ptr(gin), int(num_channel), x.numel(), int(n_per_channel), _ptr(enc_min),
+                 _ptr(enc_max), _stream(x)))
+    return gin
+
+
+# ------------------------------------------------------------------------------------------------------------ v2 QDQ
+def v2_qdq(x, num_channel, n_per_channel, scale, offset, qmin, qmax, want_codes=False):
+    _require_gpu(x, scale, offset)
+    x = x.contiguous()
+    scale, offset = _params_f32(scale, x).reshape(-1), _params_f32(offset, x).reshape(-1)
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        if x.dtype == _F32:
+            codes = torch.empty(x.shape, dtype=torch.int32, device=x.device) if want_codes else None
+            check(lib.miq_v2_qdq_f32(_ptr(x), _ptr(out), _ptr(codes), int(num_channel), x.numel(), int(n_per_channel),
+                                     _ptr(scale), _ptr(offset), int(qmin), int(qmax), _stream(x)))
+            return (out, codes) if want_codes else out
+        if x.dtype == _BF16 and not want_codes:
+            check(lib.miq_v2_qdq_bf16(_ptr(x), _ptr(out), int(num_channel), x.numel(), int(n_per_channel),
+                                      _ptr(scale), _ptr(offset), int(qmin), int(qmax), _stream(x)))
+            return out
+    raise RuntimeError(f"unsupported dtype {x.dtype} for v2 quantize-dequantize")
+
+
+def v2_qdq_bwd(x, grad_out, num_channel, n_per_channel, scale, offset, qmin, qmax):
+    _require_gpu(x, grad_out, scale, offset)
+    x, grad_out = x.contiguous(), grad_out.to(x.dtype).contiguous()
+    scale, offset = _params_f32(scale, x).reshape(-1), _params_f32(offset, x).reshape(-1)
+    gin = torch.empty_like(x)
+    fn = getattr(lib, "miq_v2_qdq_bwd_" + _suffix(x))
+    with torch.cuda.device(x.device):
+        check(fn(_ptr(x), _ptr(grad_out), _ptr(gin), int(num_channel), x.numel(), int(n_per_channel), _ptr(scale),
+                 _ptr(offset), int(qmin), int(qmax), _stream(x)))
+    return gin
+
+
+# -------------------------------------------------------------------------------------------------------- statistics
+def minmax(x):
+    """float32 device tensor [min, max] of x (NaN ignored); asynchronous."""
+    _require_gpu(x)
+    x = x.to(_F32).contiguous()
+    out = torch.empty(2, dtype=_F32, device=x.device)
+    with torch.cuda.device(x.device):
+        check(lib.miq_minmax_f32(_ptr(x), x.numel(), _ptr(out), _stream(x)))
+    return out
+
+
+def minmax_per_channel(x, num_channel, n_per_channel):
+    """float32 device tensor [2, C]: row 0 = per-channel min, row 1 = per-channel max."""
+    _require_gpu(x)
+    x = x.to(_F32).contiguous()
+    out = torch.empty(2, num_channel, dtype=_F32, device=x.device)
+    with torch.cuda.device(x.device):
+        check(lib.miq_minmax_per_channel_f32(_ptr(x), int(num_channel), x.numel(), int(n_per_channel), _ptr(out),
+                                             _stream(x)))
+    return out
+
+
+class Analyzer:
+    """Device-resident encoding analyzer (TF min/max or TF-Enhanced 512-bucket PDF + SQNR search)."""
+
+    def __init__(self, mode, device=None):
+        self.mode = int(mode)
+        self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        if self.device.type != "cuda":
+            raise RuntimeError("an Analyzer lives on a GPU")
+        h = C.c_void_p()
+        with torch.cuda.device(self.device):
+            check(lib.miq_analyzer_create(self.mode, C.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            lib.miq_analyzer_destroy(h)
+
+    def _s(self):
+        return C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def reset(self):
+        with torch.cuda.device(self.device):
+            check(lib.miq_analyzer_reset(self._h, self._s()))
+
+    def update_stats(self, x):
+        _require_gpu(x)
+        if x.device != self.device:
+            raise RuntimeError(f"analyzer lives on {self.device}, tensor on {x.device}")
+        x = x.to(_F32).contiguous()
+        with torch.cuda.device(self.device):
+            check(lib.miq_analyzer_update_stats_f32(self._h, _ptr(x), x.numel(), self._s()))
+        # keep x alive until the kernels that read it have been queued behind it on the same stream
+        x.record_stream(torch.cuda.current_stream(self.device))
+
+    def compute_encoding(self, bw, symmetric=False, strict_symmetric=False, unsigned_symmetric=False):
+        """returns (Encoding, is_valid)"""
+        e, valid = Encoding(), C.c_int(0)
+        with torch.cuda.device(self.device):
+            check(lib.miq_analyzer_compute_encoding(self._h, int(bw), int(bool(symmetric)),
+                                                    int(bool(strict_symmetric)), int(bool(unsigned_symmetric)),
+                                                    C.byref(e), C.byref(valid), self._s()))
+        return e, bool(valid.value)
+
+    def get_stats_histogram(self):
+        import numpy as np
+        xl, pdf = np.zeros(_lib.PDF_SIZE), np.zeros(_lib.PDF_SIZE)
+        n = C.c_int(0)
+        with torch.cuda.device(self.device):
+            check(lib.miq_analyzer_get_stats_histogram(self._h, xl.ctypes.data, pdf.ctypes.data, C.byref(n),
+                                                       self._s()))
+        return xl[:n.value], pdf[:n.value]
+
+    def last_batch_counts(self):
+        import numpy as np
+        counts = np.zeros(_lib.PDF_SIZE, np.uint32)
+        with torch.cuda.device(self.device):
+            check(lib.miq_analyzer_last_batch_counts(self._h, counts.ctypes.data, self._s()))
+        return counts
+
+    def last_search(self):
+        import numpy as np
+        cap = 512
+        d, o, c = np.zeros(cap, np.float32), np.zeros(cap, np.int32), np.zeros(cap, np.float64)
+        n, best = C.c_int(0), C.c_int(-1)
+        with torch.cuda.device(self.device):
+            check(lib.miq_analyzer_last_search(self._h, d.ctypes.data, o.ctypes.data, c.ctypes.data, cap, C.byref(n),
+                                               C.byref(best), self._s()))
+        return d[:n.value], o[:n.value], c[:n.value], best.value

@@ -1,0 +1,204 @@
+/*
+ * libmiq -- C ABI of the MI355X (gfx950) quantization-simulation kernels.
+ *
+ * Every entry point takes plain pointers and sizes (device pointers unless a parameter says "host"), an explicit
+ * `void* stream` (a hipStream_t; NULL = the default stream) and returns an int status: MIQ_OK (0) or a negative
+ * MIQ_ERR_* code, in which case miq_last_error() holds a message for the calling thread.  Nothing throws across
+ * this boundary.  Kernels are enqueued asynchronously on `stream`; the caller owns every buffer and keeps it alive
+ * until the stream has passed the call.  In-place operation (out == in) is allowed for every elementwise call.
+ * Element counts are 64-bit.
+ *
+ * Each declaration names the reference interface it replaces (paths relative to the reference root;
+ * DLQ = ModelOptimizations/DlQuantization, TSRC = TrainingExtensions/torch/src,
+ * TORCH = TrainingExtensions/torch/src/python/aimet_torch).
+ */
+#ifndef MIQ_H
+#define MIQ_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MIQ_OK 0
+#define MIQ_ERR_INVALID_ARG (-1)
+#define MIQ_ERR_HIP (-2)
+#define MIQ_ERR_UNSUPPORTED (-3)
+
+/* DLQ/include/DlQuantization/Quantization.hpp:145-149 (RoundingMode).  Only nearest is implemented: the
+ * reference's stochastic mode seeds from clock() per element and is not reproducible by design. */
+#define MIQ_ROUND_NEAREST 0
+#define MIQ_ROUND_STOCHASTIC 1
+
+/* DLQ/include/DlQuantization/Quantization.hpp:83-105 (QuantizationMode) */
+#define MIQ_QUANTIZATION_TF 0
+#define MIQ_QUANTIZATION_TF_ENHANCED 1
+
+#define MIQ_PDF_SIZE 512 /* DLQ/src/math_functions.hpp:80 */
+
+/* DLQ/include/DlQuantization/Quantization.hpp:113-120 (struct TfEncoding); same field order and types. */
+typedef struct miq_encoding
+{
+    double min;
+    double max;
+    double delta;
+    double offset;
+    int bw;
+} miq_encoding;
+
+const char* miq_last_error(void);
+/* Library/ABI version, bumped when a signature changes. */
+int miq_version(void);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * Host-side encoding arithmetic (double precision, no device work)
+ * ------------------------------------------------------------------------------------------------------------- */
+
+/* ITensorQuantizationSim<float>::fillEncodingInfo / generateScaleOffset
+ * (DLQ/include/DlQuantization/ITensorQuantizationSim.h:102-105, DLQ/src/TensorQuantizationSim.cpp:62-92). */
+int miq_fill_encoding_info(int bw, double enc_min, double enc_max, miq_encoding* out /* host */);
+
+/* getComputedEncodings (DLQ/src/quantization_utils.cpp:58-143): (min, max) -> TF encoding. */
+int miq_get_computed_encodings(int bw, double mn, double mx, int use_symmetric, int use_strict_symmetric,
+                               int use_unsigned_symmetric, miq_encoding* out /* host */);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * v1 (DlQuantization) quantize-dequantize: clamp to [min,max], x/delta - offset, round half away from zero,
+ * delta*(q+offset); all in float32
+ * ------------------------------------------------------------------------------------------------------------- */
+
+/* ITensorQuantizationSim<float>::quantizeDequantizeTensor(in, cnt, out, encMin, encMax, bw, roundMode, use_cuda, stream)
+ * (ITensorQuantizationSim.h:49-55, DLQ/src/TensorQuantizationSim.cpp:104-114; kernel DLQ/src/trim_functions.cu:46-60).
+ * As in the reference, delta/offset are re-derived from (enc_min, enc_max, bw). */
+int miq_qdq_per_tensor_f32(const float* in, float* out, int64_t n, double enc_min, double enc_max, int bw,
+                           int rounding_mode, void* stream);
+/* Same arithmetic with bfloat16 storage (the reference's caller upcasts to float32 and casts the result back:
+ * TORCH/v1/tensor_quantizer.py:1129-1138); the conversion passes are fused into the kernel. */
+int miq_qdq_per_tensor_bf16(const uint16_t* in, uint16_t* out, int64_t n, double enc_min, double enc_max, int bw,
+                            int rounding_mode, void* stream);
+
+/* ITensorQuantizationSim<float>::quantizeTensor(..., shiftToSigned) (ITensorQuantizationSim.h:57-59,
+ * DLQ/src/TensorQuantizationSim.cpp:116-126; kernel DLQ/src/trim_functions.cu:62-76): float-valued grid indices. */
+int miq_quantize_per_tensor_f32(const float* in, float* out, int64_t n, double enc_min, double enc_max, int bw,
+                                int rounding_mode, int shift_to_signed, void* stream);
+
+/* One pass that writes the dequantized tensor (out may be NULL) and the integer codes as bytes (bw <= 8):
+ * uint8 grid index, or int8 (index - 2^(bw-1)) when shift_to_signed.  Fuses the two reference calls above. */
+int miq_qdq_codes_per_tensor_f32(const float* in, float* out, uint8_t* codes, int64_t n, double enc_min,
+                                 double enc_max, int bw, int shift_to_signed, void* stream);
+
+/* Per-channel parameter recipe of AimetTensorQuantizer::quantizeDequantizePerChannel
+ * (TSRC/AimetTensorQuantizer.cpp:209-227, 268-297): from per-channel (min,max) in float32, gate to include zero,
+ * delta = (max-min)/num_steps, offset = round-half-even(min/delta).  enc_min/enc_max: device float[C] (raw encoding
+ * values); the four outputs are device float[C].  num_steps = 2^bw - 1, minus 1 iff encodings[0].min == -encodings[0].max. */
+int miq_per_channel_params_f32(const float* enc_min, const float* enc_max, int64_t num_channel, double num_steps,
+                               float* out_min, float* out_max, float* out_delta, float* out_offset, void* stream);
+
+/* ITensorQuantizationSim<float>::quantizeDequantizeTensorPerChannel(in, numChannel, numElement, numElementPerChannel,
+ * out, encMin*, encMax*, encDelta*, encOffset*, roundMode, useCuda, stream) (ITensorQuantizationSim.h:107-118,
+ * DLQ/src/TensorQuantizationSim.cpp:300-317; kernel DLQ/src/trim_functions.cu:78-92):
+ * channel(i) = (i / num_element_per_channel) % num_channel. */
+int miq_qdq_per_channel_f32(const float* in, float* out, int64_t num_channel, int64_t num_element,
+                            int64_t num_element_per_channel, const float* enc_min, const float* enc_max,
+                            const float* enc_delta, const float* enc_offset, int rounding_mode, void* stream);
+int miq_qdq_per_channel_bf16(const uint16_t* in, uint16_t* out, int64_t num_channel, int64_t num_element,
+                             int64_t num_element_per_channel, const float* enc_min, const float* enc_max,
+                             const float* enc_delta, const float* enc_offset, int rounding_mode, void* stream);
+/* As above, also writing the 8-bit grid indices (out may be NULL). */
+int miq_qdq_codes_per_channel_f32(const float* in, float* out, uint8_t* codes, int64_t num_channel,
+                                  int64_t num_element, int64_t num_element_per_channel, const float* enc_min,
+                                  const float* enc_max, const float* enc_delta, const float* enc_offset,
+                                  int shift_to_signed, int bw, void* stream);
+
+/* quantizeDequantizeBroadcast<float> (DLQ/include/DlQuantization/Quantization.hpp:209-222, kernel
+ * DLQ/src/trim_functions.cu:96-122).  input_strides / encoding_strides are HOST arrays of length num_dims
+ * (num_dims <= 8); they travel as kernel arguments instead of device-resident arrays. */
+int miq_qdq_broadcast_f32(const float* in, float* out, int64_t num_element, int64_t num_dims,
+                          const int64_t* input_strides /* host */, const int64_t* encoding_strides /* host */,
+                          const float* enc_min, const float* enc_max, const float* enc_delta,
+                          const float* enc_offset, void* stream);
+
+/* Straight-through backward of the v1 path, compute_dloss_by_dx
+ * (TORCH/v1/quantsim_straight_through_grad.py:91-118): grad_in = grad_out * (min <= x && x <= max). */
+int miq_ste_bwd_per_tensor_f32(const float* x, const float* grad_out, float* grad_in, int64_t n, float enc_min,
+                               float enc_max, void* stream);
+int miq_ste_bwd_per_tensor_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* grad_in, int64_t n,
+                                float enc_min, float enc_max, void* stream);
+int miq_ste_bwd_per_channel_f32(const float* x, const float* grad_out, float* grad_in, int64_t num_channel,
+                                int64_t num_element, int64_t num_element_per_channel, const float* enc_min,
+                                const float* enc_max, void* stream);
+int miq_ste_bwd_per_channel_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* grad_in,
+                                 int64_t num_channel, int64_t num_element, int64_t num_element_per_channel,
+                                 const float* enc_min, const float* enc_max, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * v2 quantize-dequantize (TORCH/v2/quantization/affine/backends/torch_builtins.py:290-344, QuantDequantFunc):
+ * r = round-half-even(x/scale) - offset; mask = qmin <= r <= qmax; y = (clamp(r,qmin,qmax) + offset) * scale,
+ * computed in float32.  scale/offset: device float[num_channel], channel(i) = (i / num_element_per_channel) %
+ * num_channel (num_channel = 1 for per-tensor).  out and codes may each be NULL; codes are int32 grid values.
+ * ------------------------------------------------------------------------------------------------------------- */
+int miq_v2_qdq_f32(const float* in, float* out, int32_t* codes, int64_t num_channel, int64_t num_element,
+                   int64_t num_element_per_channel, const float* scale, const float* offset, int qmin, int qmax,
+                   void* stream);
+int miq_v2_qdq_bf16(const uint16_t* in, uint16_t* out, int64_t num_channel, int64_t num_element,
+                    int64_t num_element_per_channel, const float* scale, const float* offset, int qmin, int qmax,
+                    void* stream);
+/* Backward w.r.t. the input (torch_builtins.py:329-344, tensor_grad = grad * mask); the mask is recomputed from x. */
+int miq_v2_qdq_bwd_f32(const float* x, const float* grad_out, float* grad_in, int64_t num_channel,
+                       int64_t num_element, int64_t num_element_per_channel, const float* scale,
+                       const float* offset, int qmin, int qmax, void* stream);
+int miq_v2_qdq_bwd_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* grad_in, int64_t num_channel,
+                        int64_t num_element, int64_t num_element_per_channel, const float* scale,
+                        const float* offset, int qmin, int qmax, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * Calibration statistics
+ * ------------------------------------------------------------------------------------------------------------- */
+
+/* GetMin + GetMax (DLQ/src/math_functions.cpp:328-347; GPU twins math_functions.cu:52-64) fused into one pass.
+ * out_min_max: device float[2] = {min, max}; NaN elements are ignored, an empty input yields {+inf, -inf}. */
+int miq_minmax_f32(const float* in, int64_t n, float* out_min_max, void* stream);
+/* Per-channel form used for per-channel min/max (TF) encodings: out is device float[2*num_channel] laid out
+ * {min_0..min_{C-1}, max_0..max_{C-1}}; channel(i) = (i / num_element_per_channel) % num_channel. */
+int miq_minmax_per_channel_f32(const float* in, int64_t num_channel, int64_t num_element,
+                               int64_t num_element_per_channel, float* out_min_max, void* stream);
+
+/* Encoding analyzer object = IQuantizationEncodingAnalyzer<float>
+ * (DLQ/include/DlQuantization/IQuantizationEncodingAnalyzer.hpp:48-126) as instantiated by
+ * getEncodingAnalyzerInstance<float>(mode) (DLQ/src/QuantizerFactory.cpp:74-97) for QUANTIZATION_TF
+ * (TfEncodingAnalyzer, DLQ/src/TfEncodingAnalyzer.cpp:59-101) and QUANTIZATION_TF_ENHANCED
+ * (TfEnhancedEncodingAnalyzer, DLQ/src/TfEnhancedEncodingAnalyzer.cpp:68-397).  All statistics (running min/max,
+ * the 512-bucket PDF, its range and iteration count) live in device memory owned by the object on the device that
+ * was current at creation; update_stats enqueues work and never synchronises.  compute_encoding synchronises
+ * `stream` once to read the result back.  An object must not be used from two threads at once. */
+typedef struct miq_analyzer miq_analyzer;
+int miq_analyzer_create(int quantization_mode, miq_analyzer** out);
+int miq_analyzer_destroy(miq_analyzer* a);
+/* resetEncodingStats (TSRC/AimetTensorQuantizer.cpp:85-92) */
+int miq_analyzer_reset(miq_analyzer* a, void* stream);
+/* updateStats(tensor, tensorSize, mode, allocator) (IQuantizationEncodingAnalyzer.hpp:59-69) */
+int miq_analyzer_update_stats_f32(miq_analyzer* a, const float* data, int64_t n, void* stream);
+/* computeEncoding(bw, useSymmetricEncodings, useStrictSymmetric, useUnsignedSymmetric)
+ * (IQuantizationEncodingAnalyzer.hpp:71-93) + the validity flag of AimetTensorQuantizer::getEncoding
+ * (TSRC/AimetTensorQuantizer.cpp:180-192): *is_valid = 0 when no statistics were ever supplied. */
+int miq_analyzer_compute_encoding(miq_analyzer* a, int bw, int use_symmetric, int use_strict_symmetric,
+                                  int use_unsigned_symmetric, miq_encoding* out /* host */, int* is_valid /* host */,
+                                  void* stream);
+/* getStatsHistogram() (IQuantizationEncodingAnalyzer.hpp:95-102): 512 (xLeft, pdf) pairs into host arrays.
+ * Returns MIQ_ERR_UNSUPPORTED for a TF analyzer (the reference asserts) and writes *num_buckets = 0 while the PDF
+ * has not been initialised. */
+int miq_analyzer_get_stats_histogram(miq_analyzer* a, double* x_left /* host[512] */, double* pdf /* host[512] */,
+                                     int* num_buckets /* host */, void* stream);
+/* Test/inspection hooks: the integer bin counts of the most recent update_stats call (host uint32[512]) and the
+ * TF-Enhanced candidate list with every candidate's cost from the most recent compute_encoding call
+ * (host arrays of capacity `cap`; *count receives the number of candidates, *best_index the winner). */
+int miq_analyzer_last_batch_counts(miq_analyzer* a, uint32_t* counts /* host[512] */, void* stream);
+int miq_analyzer_last_search(miq_analyzer* a, float* deltas /* host */, int32_t* offsets /* host */,
+                             double* costs /* host */, int cap, int* count /* host */, int* best_index /* host */,
+                             void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MIQ_H */

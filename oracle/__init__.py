@@ -217,7 +217,7 @@ class _Oracle:
         u = x.view(np.uint32).astype(np.uint64)
         nan = (u & 0x7fffffff) > 0x7f800000
         r = ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
-        r[nan] = ((u[nan] >> 16) | 0x40).astype(np.uint16)
+        r[nan] = 0x7fc0
         return r
 
     @staticmethod

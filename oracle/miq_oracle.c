@@ -64,8 +64,8 @@ uint16_t orc_f32_to_bf16(float f)
 {
     uint32_t u;
     memcpy(&u, &f, 4);
-    if ((u & 0x7fffffffu) > 0x7f800000u) /* NaN: quiet it, keep sign */
-        return (uint16_t) ((u >> 16) | 0x0040u);
+    if ((u & 0x7fffffffu) > 0x7f800000u) /* NaN -> 0x7FC0, as c10::BFloat16's round_to_nearest_even does */
+        return (uint16_t) 0x7fc0u;
     uint32_t lsb = (u >> 16) & 1u;
     u += 0x7fffu + lsb;
     return (uint16_t) (u >> 16);

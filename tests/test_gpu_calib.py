@@ -1,0 +1,195 @@
+"""GPU parity of the calibration kernels (min/max, 512-bucket PDF, TF-Enhanced search) against the CPU oracle,
+through the C ABI.  Bin counts, PDF, candidate lists, costs and the chosen encoding must be identical."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TF, TFE = 0, 1
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from aimet_amd import ops as o
+    return o
+
+
+def _gpu(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _relu_pareto(seed, n):
+    """|N(0,1)| with a 0.5 % Pareto(alpha=2, x_m=1) tail: the post-ReLU activation model of the calibration config."""
+    rng = np.random.default_rng(seed)
+    x = np.abs(rng.standard_normal(n)).astype(np.float32)
+    tail = rng.random(n) < 0.005
+    x[tail] = (1.0 / np.sqrt(1.0 - rng.random(int(tail.sum())))).astype(np.float32)
+    return x
+
+
+def _check_tfe(ops, oracle, batches, modes=((8, 0, 0, 0), (8, 1, 0, 0), (8, 1, 1, 0), (8, 1, 0, 1), (4, 0, 0, 0))):
+    an = ops.Analyzer(TFE)
+    pdf = oracle.new_pdf()
+    for b in batches:
+        an.update_stats(_gpu(b))
+        hist = pdf.update(b)
+        if pdf.initialized:
+            assert np.array_equal(an.last_batch_counts(), hist)
+    xl, p = an.get_stats_histogram()
+    if pdf.initialized:
+        assert np.array_equal(xl, pdf.x_left())
+        assert np.array_equal(p, pdf.pdf())
+    else:
+        assert xl.size == 0
+    for bw, sym, strict, uns in modes:
+        enc, valid = an.compute_encoding(bw, sym, strict, uns)
+        oenc, ocosts, obest = pdf.compute_encoding(bw, sym, strict, uns)
+        assert valid
+        assert (enc.min, enc.max, enc.delta, enc.offset, enc.bw) == oenc.astuple(), (bw, sym, strict, uns)
+        if pdf.initialized:
+            d, o, c, best = an.last_search()
+            od, oo = pdf.candidates(bw, sym, strict, uns)
+            assert np.array_equal(d.view(np.uint32), od.view(np.uint32)) and np.array_equal(o, oo)
+            assert np.array_equal(c.view(np.uint64), ocosts[:len(od)].view(np.uint64))   # costs bit-identical
+            assert best == obest
+    return an
+
+
+def test_minmax(ops, oracle):
+    for n in (1, 5, 1023, 100003, 1 << 22):
+        rng = np.random.default_rng(n)
+        x = (rng.standard_normal(n) * 3).astype(np.float32)
+        if n > 10:
+            x[3] = np.nan
+        got = ops.minmax(_gpu(x)).cpu().numpy()
+        mn, mx = oracle.minmax(x)
+        assert got[0] == mn and got[1] == mx
+    x = np.full(7, np.nan, np.float32)
+    got = ops.minmax(_gpu(x)).cpu().numpy()
+    assert got[0] == np.inf and got[1] == -np.inf
+
+
+def test_minmax_per_channel(ops):
+    g = torch.Generator().manual_seed(3)
+    for shape, axis in (((64, 300), 0), ((3, 16, 50), 1), ((11008, 4096), 0), ((5, 7, 3, 3), 1)):
+        x = torch.randn(shape, generator=g)
+        c = shape[axis]
+        npc = int(np.prod(shape[axis + 1:]))
+        got = ops.minmax_per_channel(x.cuda(), c, npc).cpu()
+        dims = [d for d in range(len(shape)) if d != axis]
+        assert torch.equal(got[0], x.amin(dim=dims)) and torch.equal(got[1], x.amax(dim=dims))
+
+
+def test_tf_analyzer(ops, oracle):
+    an = ops.Analyzer(TF)
+    e, valid = an.compute_encoding(8)
+    assert not valid
+    rng = np.random.default_rng(4)
+    acc_min, acc_max = np.inf, -np.inf
+    for i in range(3):
+        x = (rng.standard_normal(50001) * (i + 1)).astype(np.float32)
+        an.update_stats(_gpu(x))
+        acc_min, acc_max = min(acc_min, float(x.min())), max(acc_max, float(x.max()))
+    for bw in (4, 8):
+        for sym, strict, uns in ((0, 0, 0), (1, 0, 0), (1, 1, 0), (1, 0, 1)):
+            e, valid = an.compute_encoding(bw, sym, strict, uns)
+            o = oracle.tf_compute_encoding(acc_min, acc_max, bw, sym, strict, uns)
+            assert valid and (e.min, e.max, e.delta, e.offset, e.bw) == o.astuple()
+    an.reset()
+    assert not an.compute_encoding(8)[1]
+
+
+def test_tfe_known_answer_n22(ops, oracle, vectors, n22):
+    v = vectors["tf_enhanced_n22"]
+    an = _check_tfe(ops, oracle, [n22])
+    enc, _ = an.compute_encoding(8)
+    assert enc.min == pytest.approx(v["exp_min"], abs=v["atol"]) and enc.max == pytest.approx(v["exp_max"], abs=v["atol"])
+    y = ops.qdq_per_tensor(torch.full((16,), 5.0, device="cuda"), enc.min, enc.max, 8)
+    assert float(y[0]) == pytest.approx(v["qdq_of_5"], abs=1e-3)
+
+
+def test_tfe_multi_batch_relu_pareto(ops, oracle):
+    _check_tfe(ops, oracle, [_relu_pareto(1003 + b, 200000 + 3 * b) for b in range(5)])
+
+
+def test_tfe_outliers_nan_dropped(ops, oracle):
+    rng = np.random.default_rng(6)
+    b0 = (rng.standard_normal(100000)).astype(np.float32)
+    b1 = b0.copy()
+    b1[:10] = 1e6
+    b1[10:15] = np.nan
+    b1[15:20] = -np.inf
+    an = _check_tfe(ops, oracle, [b0, b1], modes=((8, 0, 0, 0),))
+    assert an.last_batch_counts().sum() == b1.size - 20
+
+
+def test_tfe_all_zero_batches_then_data(ops, oracle, vectors):
+    v = vectors["tf_enhanced_all_zeros"]
+    an = ops.Analyzer(TFE)
+    e, valid = an.compute_encoding(8)
+    assert not valid                                   # nothing seen yet
+    an.update_stats(torch.zeros(1000, device="cuda"))
+    e, valid = an.compute_encoding(8)
+    assert valid and e.offset == v["offset"]
+    assert e.min == pytest.approx(v["exp_min"], abs=v["atol"]) and e.max == pytest.approx(v["exp_max"], abs=v["atol"])
+    assert an.get_stats_histogram()[0].size == 0
+    _check_tfe(ops, oracle, [np.zeros(64, np.float32), _relu_pareto(7, 30000), np.zeros(64, np.float32)])
+
+
+def test_tfe_constant_and_tiny(ops, oracle):
+    _check_tfe(ops, oracle, [np.full(100, 4.0, np.float32)], modes=((8, 0, 0, 0),))
+    _check_tfe(ops, oracle, [np.full(100, -5.0, np.float32)], modes=((8, 0, 0, 0),))
+    _check_tfe(ops, oracle, [np.array([0.25], np.float32), np.array([0.25, 0.3, -0.1], np.float32)])
+
+
+def test_tfe_reset_and_unaligned(ops, oracle):
+    an = ops.Analyzer(TFE)
+    x = _relu_pareto(8, 50001)
+    an.update_stats(_gpu(x))
+    an.reset()
+    y = (np.random.default_rng(9).standard_normal(40003)).astype(np.float32)
+    base = _gpu(np.concatenate([np.zeros(1, np.float32), y]))
+    an.update_stats(base[1:])                          # 4-byte aligned only
+    pdf = oracle.new_pdf()
+    hist = pdf.update(y)
+    assert np.array_equal(an.last_batch_counts(), hist)
+    enc, _ = an.compute_encoding(8)
+    assert (enc.min, enc.max, enc.delta, enc.offset, enc.bw) == pdf.compute_encoding(8)[0].astuple()
+
+
+def test_cfg3_full_size_properties(ops, oracle):
+    """16 batches of [32,256,28,28] on the GPU: counts of every batch sum to the batch size minus the dropped samples,
+    the PDF sums to the kept fraction, and a sub-sampled oracle run agrees on the first batch bit for bit."""
+    n = 32 * 256 * 28 * 28
+    an = ops.Analyzer(TFE)
+    g = torch.Generator(device="cuda")
+    first = None
+    kept = []
+    for b in range(16):
+        g.manual_seed(1003 + b)
+        x = torch.randn(n, device="cuda", generator=g).abs_()
+        u = torch.rand(n, device="cuda", generator=g)
+        t = torch.rand(n, device="cuda", generator=g)
+        x = torch.where(u < 0.005, (1 - t).rsqrt(), x)
+        an.update_stats(x)
+        if b == 0:
+            first = x.cpu().numpy()
+            counts0 = an.last_batch_counts()
+        if b in (0, 7, 15):
+            c = an.last_batch_counts()
+            xl, _ = an.get_stats_histogram()
+            bucket = np.float32(xl[1] - xl[0])
+            off = np.float32(xl[0]) / bucket
+            r = torch.round(x / float(bucket) - float(off))   # not bit-exact near ties; used only for the drop count
+            kept.append((int(c.sum()), int(((r >= 0) & (r < 512)).sum())))
+    for got, approx in kept:
+        assert abs(got - approx) <= 64                 # samples within rounding distance of the range ends
+    pdf = oracle.new_pdf()
+    hist = pdf.update(first)
+    assert np.array_equal(counts0, hist)               # first batch: bit-exact against the oracle at full size
+    xl, p = an.get_stats_histogram()
+    assert np.array_equal(xl, pdf.x_left())
+    assert 0.99 < p.sum() <= 1.0 + 1e-12
+    enc, valid = an.compute_encoding(8)
+    assert valid and enc.delta > 0 and enc.min <= 0 <= enc.max
