@@ -18,6 +18,7 @@
 #include "miq_common.h"
 
 #include <cfloat>
+#include <cstddef>
 #include <cmath>
 #include <cstring>
 #include <new>
@@ -29,7 +30,10 @@ namespace
 constexpr int kPdf      = MIQ_PDF_SIZE;
 constexpr int kMaxCand  = 512;
 constexpr int kCopies   = 16;
-constexpr int kHistGrid = 2048;   // upper bound on histogram workgroups (8 per CU)
+constexpr int kMaxGrid  = 1024;   // upper bound on streaming workgroups (4 per CU): each lane keeps several 16-byte
+                                  // loads in flight, so this many waves already cover the HBM latency
+constexpr int kReplicas = 32;     // global count replicas: workgroup b merges into replica b % kReplicas, so at most
+                                  // kMaxGrid / kReplicas atomics ever meet on one address
 
 // float <-> unsigned key whose integer order is the float order (for atomicMin/atomicMax)
 __host__ __device__ inline uint32_t f2ord(float f)
@@ -56,32 +60,38 @@ __host__ __device__ inline float ord2f(uint32_t o)
 constexpr uint32_t kOrdPosInf = 0xff800000u;   // f2ord(+inf)
 constexpr uint32_t kOrdNegInf = 0x007fffffu;   // f2ord(-inf)
 
+// Layout: a small head that every read-back needs, then the inspection block (PDF, last counts, search scratch),
+// then device-only accumulators.  Read-backs copy a prefix, never the accumulators.
 struct DevState
 {
-    // batch min/max accumulators (ordered keys), consumed and re-armed by the last workgroup of the min/max pass
-    uint32_t min_key, max_key;
-    uint32_t ticket_minmax, ticket_hist, ticket_search;
+    // ---- head
+    uint32_t ticket_search;
     int stats_updated;   // _statsUpdated
-    // TF analyzer: accumulated range in double (TfEncodingAnalyzer.h:84-90)
-    double acc_min, acc_max;
-    // TF-Enhanced analyzer
-    int initialized;   // PDF range fixed (xLeft.size() != 0 in the reference)
+    int minmax_valid;    // the min/max pass of this batch ran (it returns at once when the PDF range is fixed)
+    int initialized;     // PDF range fixed (xLeft.size() != 0 in the reference)
     int iterations;
     float bucket_f, pdf_offset_f;
+    int n_cand;
+    int best_index;
+    int enc_bw;
+    uint32_t batch_seq[2];   // update-call number whose counts sit in counts[i]; 0 = none pending
+    int64_t batch_n[2];      // element count of that batch
+    double acc_min, acc_max; // TF analyzer: accumulated range in double (TfEncodingAnalyzer.h:84-90)
+    double enc_min, enc_max, enc_delta, enc_offset;
+    // ---- inspection block
     double xLeft[kPdf];
     double pdf[kPdf];
-    uint32_t counts[kPdf];        // current batch; zero between batches
-    uint32_t last_counts[kPdf];   // copy of the last folded batch (inspection)
-    // search scratch and result
+    uint32_t last_counts[kPdf];   // the last folded batch
     float cand_delta[kMaxCand];
     int cand_offset[kMaxCand];
     int cand_valid[kMaxCand];
     double cand_cost[kMaxCand];
-    int n_cand;
-    int best_index;
-    double enc_min, enc_max, enc_delta, enc_offset;
-    int enc_bw;
+    // ---- device-only accumulators
+    uint32_t counts[2][kReplicas][kPdf];   // two batches in flight (filling / being folded), replicated; zero when idle
+    float2 partial[kMaxGrid];              // per-workgroup (min, max) of the batch in flight
 };
+constexpr size_t kHeadBytes    = offsetof(DevState, xLeft);
+constexpr size_t kInspectBytes = offsetof(DevState, counts);
 
 // relaxed agent-scope loads: used by the workgroup that finishes last to read what the others published
 template <typename T>
@@ -146,6 +156,8 @@ __device__ void initialize_pdf(DevState* st, float min_val, float max_val)
     }
 }
 
+// Pass 1: every workgroup reduces its share and stores one (min, max) pair -- plain stores, no atomics, because
+// same-address device atomics from a thousand workgroups serialise at roughly 15 ns each on this part.
 template <bool VEC>
 __global__ __launch_bounds__(kBlock) void minmax_kernel(const float* __restrict__ in, int64_t n, DevState* st,
                                                         int mode)
@@ -155,13 +167,24 @@ __global__ __launch_bounds__(kBlock) void minmax_kernel(const float* __restrict_
     float mn = INFINITY, mx = -INFINITY;
     if (VEC)
     {
-        const int64_t nvec = n / 4;
-        const float4* v    = reinterpret_cast<const float4*>(in);
-        for (int64_t i = (int64_t) blockIdx.x * kBlock + threadIdx.x; i < nvec; i += (int64_t) gridDim.x * kBlock)
+        const int64_t nvec   = n / 4;
+        const float4* v      = reinterpret_cast<const float4*>(in);
+        const int64_t stride = (int64_t) gridDim.x * kBlock * kUnroll;
+        for (int64_t base = (int64_t) blockIdx.x * kBlock * kUnroll; base < nvec; base += stride)
         {
-            const float4 a = v[i];
-            mn             = fminf(fminf(mn, a.x), fminf(a.y, fminf(a.z, a.w)));
-            mx             = fmaxf(fmaxf(mx, a.x), fmaxf(a.y, fmaxf(a.z, a.w)));
+            float4 a[kUnroll];
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+            {
+                const int64_t i = base + u * kBlock + threadIdx.x;
+                a[u] = (i < nvec) ? v[i] : make_float4(NAN, NAN, NAN, NAN);   // fminf/fmaxf skip NaN
+            }
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+            {
+                mn = fminf(fminf(mn, a[u].x), fminf(a[u].y, fminf(a[u].z, a[u].w)));
+                mx = fmaxf(fmaxf(mx, a[u].x), fmaxf(a[u].y, fmaxf(a[u].z, a[u].w)));
+            }
         }
         if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * 4))
         {
@@ -182,7 +205,6 @@ __global__ __launch_bounds__(kBlock) void minmax_kernel(const float* __restrict_
     mn = wave_min(mn);
     mx = wave_max(mx);
     __shared__ float smn[kBlock / 64], smx[kBlock / 64];
-    __shared__ bool is_last;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     if (lane == 0)
     {
@@ -190,9 +212,6 @@ __global__ __launch_bounds__(kBlock) void minmax_kernel(const float* __restrict_
         smx[wave] = mx;
     }
     __syncthreads();
-    uint32_t* kmin = &st->min_key;
-    uint32_t* kmax = &st->max_key;
-    uint32_t* tick = &st->ticket_minmax;
     if (threadIdx.x == 0)
     {
         for (int w = 1; w < kBlock / 64; ++w)
@@ -200,24 +219,43 @@ __global__ __launch_bounds__(kBlock) void minmax_kernel(const float* __restrict_
             mn = fminf(mn, smn[w]);
             mx = fmaxf(mx, smx[w]);
         }
-        atomicMin(kmin, f2ord(mn));
-        atomicMax(kmax, f2ord(mx));
-        __threadfence();
-        const uint32_t t = atomicAdd(tick, 1u);
-        is_last          = (t == gridDim.x - 1);
+        st->partial[blockIdx.x] = make_float2(mn, mx);
+        if (blockIdx.x == 0)
+            st->minmax_valid = 1;
+    }
+}
+
+// Pass 2 (one workgroup of kBlock lanes): fold the per-workgroup pairs and apply the analyzer's rule.
+__global__ __launch_bounds__(kBlock) void minmax_finalize_kernel(DevState* st, int grid, int mode)
+{
+    if (!st->minmax_valid)
+        return;
+    float mn = INFINITY, mx = -INFINITY;
+    for (int i = threadIdx.x; i < grid; i += kBlock)
+    {
+        const float2 p = st->partial[i];
+        mn             = fminf(mn, p.x);
+        mx             = fmaxf(mx, p.y);
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    __shared__ float smn[kBlock / 64], smx[kBlock / 64];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0)
+    {
+        smn[wave] = mn;
+        smx[wave] = mx;
     }
     __syncthreads();
-    if (!is_last)
-        return;
-    __threadfence();
-    const float gmn = ord2f(agent_load(kmin));
-    const float gmx = ord2f(agent_load(kmax));
-    __syncthreads();   // everyone holds gmn/gmx before the keys are re-armed
+    float gmn = smn[0], gmx = smx[0];
+    for (int w = 1; w < kBlock / 64; ++w)
+    {
+        gmn = fminf(gmn, smn[w]);
+        gmx = fmaxf(gmx, smx[w]);
+    }
     if (threadIdx.x == 0)
     {
-        st->min_key       = kOrdPosInf;
-        st->max_key       = kOrdNegInf;
-        st->ticket_minmax = 0;
+        st->minmax_valid  = 0;
         st->stats_updated = 1;
     }
     if (mode == kMinMaxTf)
@@ -295,91 +333,33 @@ __global__ __launch_bounds__(kBlock) void minmax_rows_kernel(const float* __rest
 }
 
 // ---------------------------------------------------------------------------------------------------- histogram
+// Adds one sample to the workgroup's LDS histogram.  Row kPdf is a sink for dropped samples, so the add is
+// unconditional (no divergent branch per element).
 __device__ __forceinline__ void hist_add(uint32_t* lds, float x, float bucket, float off, int copy)
 {
     // DLQ/src/math_functions.cpp:375-382; the range test is done on the rounded float so that NaN and values
     // beyond the int range are dropped, as they are on the reference's CPU path
-    const float r = roundf(x / bucket - off);
-    if (r >= 0.0f && r < (float) kPdf)
-        atomicAdd(&lds[(int) r * kCopies + copy], 1u);
+    const float r  = roundf(x / bucket - off);
+    const bool ok  = (r >= 0.0f && r < (float) kPdf);
+    const int row  = ok ? (int) r : kPdf;
+    atomicAdd(&lds[row * kCopies + copy], 1u);
 }
 
-template <bool VEC>
-__global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ in, int64_t n, DevState* st)
+// Folds the counts of one finished batch into the running PDF (DLQ/src/math_functions.cpp:279-287; the element
+// count is an int in the reference) and clears them.  Run by one workgroup.
+__device__ void fold_batch(DevState* st, int buf)
 {
-    if (!st->initialized)
-        return;   // only all-zero batches so far: the reference returns without touching the PDF
-    __shared__ uint32_t lds[kPdf * kCopies];
-    __shared__ bool is_last;
-    for (int i = threadIdx.x; i < kPdf * kCopies; i += kBlock)
-        lds[i] = 0;
-    __syncthreads();
-    const float bucket = st->bucket_f;
-    const float off    = st->pdf_offset_f;
-    const int copy     = threadIdx.x & (kCopies - 1);
-    if (VEC)
-    {
-        const int64_t nvec   = n / 4;
-        const float4* v      = reinterpret_cast<const float4*>(in);
-        const int64_t stride = (int64_t) gridDim.x * kBlock * kUnroll;
-        for (int64_t base = (int64_t) blockIdx.x * kBlock * kUnroll; base < nvec; base += stride)
-        {
-            float4 a[kUnroll];
-            bool live[kUnroll];
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
-            {
-                const int64_t i = base + u * kBlock + threadIdx.x;
-                live[u]         = i < nvec;
-                if (live[u])
-                    a[u] = v[i];
-            }
-#pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
-            {
-                if (!live[u])
-                    continue;
-                hist_add(lds, a[u].x, bucket, off, copy);
-                hist_add(lds, a[u].y, bucket, off, copy);
-                hist_add(lds, a[u].z, bucket, off, copy);
-                hist_add(lds, a[u].w, bucket, off, copy);
-            }
-        }
-        if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * 4))
-            hist_add(lds, in[nvec * 4 + threadIdx.x], bucket, off, copy);
-    }
-    else
-    {
-        for (int64_t i = (int64_t) blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t) gridDim.x * kBlock)
-            hist_add(lds, in[i], bucket, off, copy);
-    }
-    __syncthreads();
-    for (int b = threadIdx.x; b < kPdf; b += kBlock)
-    {
-        uint32_t s = 0;
-#pragma unroll
-        for (int c = 0; c < kCopies; ++c)
-            s += lds[b * kCopies + c];
-        if (s)
-            atomicAdd(&st->counts[b], s);
-    }
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0)
-    {
-        const uint32_t t = atomicAdd(&st->ticket_hist, 1u);
-        is_last          = (t == gridDim.x - 1);
-    }
-    __syncthreads();
-    if (!is_last)
-        return;
-    __threadfence();
-    // fold this batch into the running PDF: DLQ/src/math_functions.cpp:279-287 (cnt is an int in the reference)
     const int it     = st->iterations;
-    const double cnt = (double) (int) n;
-    for (int b = threadIdx.x; b < kPdf; b += kBlock)
+    const double cnt = (double) (int) st->batch_n[buf];
+    for (int b = threadIdx.x; b < kPdf; b += blockDim.x)
     {
-        const uint32_t c   = atomicExch(&st->counts[b], 0u);
+        uint32_t c = 0;
+#pragma unroll 8
+        for (int r = 0; r < kReplicas; ++r)
+        {
+            c += st->counts[buf][r][b];
+            st->counts[buf][r][b] = 0;
+        }
         st->last_counts[b] = c;
         const double prob  = (double) c / cnt;
         st->pdf[b]         = (st->pdf[b] * it + prob) / (it + 1);
@@ -387,8 +367,113 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
     __syncthreads();
     if (threadIdx.x == 0)
     {
-        st->iterations  = it + 1;
-        st->ticket_hist = 0;
+        st->iterations     = it + 1;
+        st->batch_seq[buf] = 0;
+    }
+}
+
+// One launch per batch.  Workgroups 0 .. gridDim.x-2 stream the tensor into counts[buf]; the extra last workgroup
+// meanwhile folds the previous batch (counts[1-buf], if that batch was accumulated) into the PDF and stamps this
+// batch as pending, so no second launch and no cross-workgroup hand-shake is needed.  `seq` numbers the update
+// calls of this analyzer; a buffer is pending iff its stamp equals the sequence number of the call that filled it.
+// With from_args the bucket width and offset arrive as kernel arguments (the host has learnt them); otherwise
+// they are read from the device state, which also says whether a range exists at all.
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ in, int64_t n, DevState* st, int buf,
+                                                      uint32_t seq, int from_args, float bucket_arg, float off_arg)
+{
+    const bool fold_group = (blockIdx.x == gridDim.x - 1);
+    const int data_groups = gridDim.x - 1;
+    if (fold_group)
+    {
+        if (st->batch_seq[1 - buf] != 0 && st->batch_seq[1 - buf] == seq - 1)
+            fold_batch(st, 1 - buf);
+        if (threadIdx.x == 0 && st->initialized)
+        {
+            st->batch_seq[buf] = seq;
+            st->batch_n[buf]   = n;
+        }
+        return;
+    }
+    __shared__ uint32_t lds[(kPdf + 1) * kCopies];
+    const int64_t nvec   = n / 4;
+    const float4* v      = reinterpret_cast<const float4*>(in);
+    const int64_t stride = (int64_t) data_groups * kBlock * kUnroll;
+    int64_t base         = (int64_t) blockIdx.x * kBlock * kUnroll;
+    float4 a[kUnroll];
+    // first tile's loads go out before anything else: they overlap the state read and the LDS clear
+    if (VEC)
+    {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+        {
+            const int64_t i = base + u * kBlock + threadIdx.x;
+            a[u] = (i < nvec) ? v[i] : make_float4(NAN, NAN, NAN, NAN);   // NaN is dropped by hist_add
+        }
+    }
+    float bucket = bucket_arg, off = off_arg;
+    if (!from_args)
+    {
+        if (!st->initialized)
+            return;   // only all-zero batches so far: the reference returns without touching the PDF
+        bucket = st->bucket_f;
+        off    = st->pdf_offset_f;
+    }
+    for (int i = threadIdx.x; i < (kPdf + 1) * kCopies; i += kBlock)
+        lds[i] = 0;
+    __syncthreads();
+    const int copy = threadIdx.x & (kCopies - 1);
+    if (VEC)
+    {
+        while (true)
+        {
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+            {
+                hist_add(lds, a[u].x, bucket, off, copy);
+                hist_add(lds, a[u].y, bucket, off, copy);
+                hist_add(lds, a[u].z, bucket, off, copy);
+                hist_add(lds, a[u].w, bucket, off, copy);
+            }
+            base += stride;
+            if (base >= nvec)
+                break;
+#pragma unroll
+            for (int u = 0; u < kUnroll; ++u)
+            {
+                const int64_t i = base + u * kBlock + threadIdx.x;
+                a[u] = (i < nvec) ? v[i] : make_float4(NAN, NAN, NAN, NAN);
+            }
+        }
+        if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * 4))
+            hist_add(lds, in[nvec * 4 + threadIdx.x], bucket, off, copy);
+    }
+    else
+    {
+        for (int64_t i = (int64_t) blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t) data_groups * kBlock)
+            hist_add(lds, in[i], bucket, off, copy);
+    }
+    __syncthreads();
+    uint32_t* dst = st->counts[buf][blockIdx.x % kReplicas];
+    for (int b = threadIdx.x; b < kPdf; b += kBlock)
+    {
+        uint32_t s = 0;
+#pragma unroll
+        for (int c = 0; c < kCopies; ++c)
+            s += lds[b * kCopies + c];
+        if (s)
+            atomicAdd(&dst[b], s);
+    }
+}
+
+// Folds whichever batch is still pending (at most one).  Queued before anything reads the PDF.
+__global__ __launch_bounds__(kBlock) void hist_flush_kernel(DevState* st, uint32_t seq)
+{
+    for (int buf = 0; buf < 2; ++buf)
+    {
+        if (st->batch_seq[buf] != 0 && st->batch_seq[buf] == seq)
+            fold_batch(st, buf);
+        __syncthreads();
     }
 }
 
@@ -412,17 +497,40 @@ __device__ __forceinline__ float std_min(float a, float b)
     return (b < a) ? b : a;   // std::min(a, b)
 }
 
+// Sum of term[lo..hi) in ascending index order.  Eight loads are issued ahead of the eight dependent adds.
+__device__ __forceinline__ double ordered_sum(const double* term, int lo, int hi)
+{
+    double acc = 0;
+    int i      = lo;
+    for (; i + 8 <= hi; i += 8)
+    {
+        double t[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            t[k] = term[i + k];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            acc += t[k];
+    }
+    for (; i < hi; ++i)
+        acc += term[i];
+    return acc;
+}
+
 // One wavefront per candidate.  Lanes evaluate the per-bucket error terms in parallel; the three sums of the
 // cost are then accumulated by one lane in bucket order, the order the reference's loops use, so that costs are
 // bit-identical to the CPU result and ties between candidates resolve identically.
-__global__ __launch_bounds__(64) void tfe_search_kernel(DevState* st, SearchArgs a)
+__global__ __launch_bounds__(kBlock) void tfe_search_kernel(DevState* st, SearchArgs a)
 {
-    const int cand = blockIdx.x;
-    const int lane = threadIdx.x;
-    __shared__ double term[kPdf];
+    constexpr int kWaves = kBlock / 64;
+    const int wave       = threadIdx.x >> 6;
+    const int cand       = blockIdx.x * kWaves + wave;   // one wavefront per candidate
+    const int lane       = threadIdx.x & 63;
+    __shared__ double term_all[kWaves][kPdf];
     __shared__ bool is_last;
+    double* term = term_all[wave];
 
-    if (st->initialized)
+    if (st->initialized && cand < a.n_cand)
     {
         // ---- range of the aggregate stats: DLQ/src/TfEnhancedEncodingAnalyzer.cpp:255-291
         int first = -1, last = -1;
@@ -552,22 +660,14 @@ __global__ __launch_bounds__(64) void tfe_search_kernel(DevState* st, SearchArgs
                 }
                 term[i] = t;
             }
-            __syncthreads();
-            // lanes 0,1,2 each accumulate one of the three sums in ascending bucket order
-            double acc = 0;
-            if (lane == 0)
-                for (int i = 0; i < minInd; ++i)
-                    acc += term[i];
-            else if (lane == 1)
-                for (int i = maxInd; i < kPdf; ++i)
-                    acc += term[i];
-            else if (lane == 2)
-                for (int i = minInd; i < maxInd; ++i)
-                    acc += term[i];
-            const double satBottom = __shfl(acc, 0);
-            const double satTop    = __shfl(acc, 1);
-            const double quant     = __shfl(acc, 2);
-            cost                   = 3.0 * (satBottom + satTop) + quant;
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // LDS writes of this wavefront have landed (lgkmcnt = 0)
+            // The three sums are accumulated in ascending bucket order, the order of the reference's loops.  Every
+            // lane runs the same chain (uniform bounds, LDS broadcast reads), so no cross-lane traffic is needed.
+            const double satBottom = ordered_sum(term, 0, minInd);
+            const double satTop    = ordered_sum(term, maxInd, kPdf);
+            const double quant     = ordered_sum(term, minInd, maxInd);
+            cost = 3.0 * (satBottom + satTop) + quant;
             cost                   = (cost < DBL_MAX) ? cost : DBL_MAX;   // std::min(sqnr, max())
         }
         if (lane == 0)
@@ -580,13 +680,13 @@ __global__ __launch_bounds__(64) void tfe_search_kernel(DevState* st, SearchArgs
     }
     __threadfence();
     __syncthreads();
-    if (lane == 0)
+    if (threadIdx.x == 0)
     {
         const uint32_t t = atomicAdd(&st->ticket_search, 1u);
         is_last          = (t == gridDim.x - 1);
     }
     __syncthreads();
-    if (!is_last)
+    if (!is_last || wave != 0)
         return;
     __threadfence();
 
@@ -672,12 +772,11 @@ __global__ void reset_state_kernel(DevState* st)
     const int i = threadIdx.x;   // launched with kPdf threads
     if (i == 0)
     {
-        st->min_key       = kOrdPosInf;
-        st->max_key       = kOrdNegInf;
-        st->ticket_minmax = st->ticket_hist = st->ticket_search = 0;
-        st->stats_updated                                       = 0;
-        st->acc_min                                             = DBL_MAX;
-        st->acc_max                                             = -DBL_MAX;
+        st->ticket_search = 0;
+        st->stats_updated = 0;
+        st->minmax_valid  = 0;
+        st->acc_min       = DBL_MAX;
+        st->acc_max       = -DBL_MAX;
         st->initialized = st->iterations = 0;
         st->bucket_f = st->pdf_offset_f = 0.f;
         st->n_cand                      = 0;
@@ -687,17 +786,23 @@ __global__ void reset_state_kernel(DevState* st)
     }
     st->xLeft[i]       = 0;
     st->pdf[i]         = 0;
-    st->counts[i]      = 0;
+    for (int r = 0; r < kReplicas; ++r)
+        st->counts[0][r][i] = st->counts[1][r][i] = 0;
     st->last_counts[i] = 0;
+    if (i < 2)
+    {
+        st->batch_seq[i] = 0;
+        st->batch_n[i]   = 0;
+    }
 }
 
-int minmax_grid(int64_t n)
+int stream_grid(int64_t n)
 {
     int64_t blocks = (n / 4 + (int64_t) kBlock * kUnroll - 1) / ((int64_t) kBlock * kUnroll);
     if (blocks < 1)
         blocks = 1;
-    if (blocks > kHistGrid)
-        blocks = kHistGrid;
+    if (blocks > kMaxGrid)
+        blocks = kMaxGrid;
     return (int) blocks;
 }
 }   // namespace
@@ -715,7 +820,9 @@ struct miq_analyzer
     bool range_known;    // host knows the PDF range has been fixed, so no further min/max pass is queued
     hipEvent_t probe;    // marks the completion of an asynchronous read of DevState::initialized
     bool probe_pending;
-    int* probe_flag;     // pinned host word receiving that read
+    int* probe_flag;     // pinned host words receiving that read: {initialized, iterations, bucket_f, pdf_offset_f}
+    float bucket_f, pdf_offset_f;   // valid once range_known
+    uint32_t seq;        // number of TF-Enhanced update calls since the last reset
     int last_bw;
 };
 
@@ -785,12 +892,14 @@ int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
     a->probe         = nullptr;
     a->probe_pending = false;
     a->probe_flag    = nullptr;
+    a->bucket_f = a->pdf_offset_f = 0.f;
+    a->seq           = 0;
     a->last_bw       = 0;
     hipError_t e     = hipGetDevice(&a->device);
     if (e == hipSuccess)
         e = hipMalloc((void**) &a->st, sizeof(DevState));
     if (e == hipSuccess)
-        e = hipHostMalloc(&a->pinned, sizeof(DevState) + 64, hipHostMallocDefault);
+        e = hipHostMalloc(&a->pinned, kInspectBytes + 64, hipHostMallocDefault);   // + 4 probe words
     if (e == hipSuccess)
         e = hipEventCreateWithFlags(&a->probe, hipEventDisableTiming);
     if (e != hipSuccess)
@@ -803,7 +912,7 @@ int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
         delete a;
         return MIQ_ERR_HIP;
     }
-    a->probe_flag  = reinterpret_cast<int*>(static_cast<char*>(a->pinned) + sizeof(DevState));
+    a->probe_flag  = reinterpret_cast<int*>(static_cast<char*>(a->pinned) + kInspectBytes);
     *a->probe_flag = 0;
     hipLaunchKernelGGL(reset_state_kernel, dim3(1), dim3(kPdf), 0, (hipStream_t) nullptr, a->st);
     e = hipStreamSynchronize(nullptr);
@@ -840,6 +949,7 @@ int miq_analyzer_reset(miq_analyzer* a, void* stream)
     MIQ_CHECK_LAUNCH();
     a->stats_updated = false;
     a->range_known   = false;
+    a->seq           = 0;
     if (a->probe_pending)
     {
         // a read of the pre-reset state may still be in flight; its answer must not be believed afterwards
@@ -857,20 +967,26 @@ int miq_analyzer_update_stats_f32(miq_analyzer* a, const float* data, int64_t n,
     hipStream_t s  = (hipStream_t) stream;
     const bool vec = aligned16(data);
     a->stats_updated = true;
-    const int grid = minmax_grid(n);
+    const int grid = stream_grid(n);
     if (a->mode == MIQ_QUANTIZATION_TF)
     {
         if (vec)
             hipLaunchKernelGGL(minmax_kernel<true>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st, kMinMaxTf);
         else
             hipLaunchKernelGGL(minmax_kernel<false>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st, kMinMaxTf);
+        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(1), dim3(kBlock), 0, s, a->st, grid, kMinMaxTf);
         MIQ_CHECK_LAUNCH();
         return MIQ_OK;
     }
     if (!a->range_known && a->probe_pending && hipEventQuery(a->probe) == hipSuccess)
     {
         a->probe_pending = false;
-        a->range_known   = (*a->probe_flag != 0);
+        if (a->probe_flag[0] != 0)
+        {
+            a->range_known = true;
+            memcpy(&a->bucket_f, &a->probe_flag[2], sizeof(float));
+            memcpy(&a->pdf_offset_f, &a->probe_flag[3], sizeof(float));
+        }
     }
     if (!a->range_known)
     {
@@ -881,28 +997,49 @@ int miq_analyzer_update_stats_f32(miq_analyzer* a, const float* data, int64_t n,
             hipLaunchKernelGGL(minmax_kernel<true>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st, kMinMaxTfe);
         else
             hipLaunchKernelGGL(minmax_kernel<false>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st, kMinMaxTfe);
+        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(1), dim3(kBlock), 0, s, a->st, grid, kMinMaxTfe);
     }
+    a->seq += 1;
+    const int buf       = (int) (a->seq & 1u);
+    const int from_args = a->range_known ? 1 : 0;
     if (vec)
-        hipLaunchKernelGGL(hist_kernel<true>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st);
+        hipLaunchKernelGGL(hist_kernel<true>, dim3(grid + 1), dim3(kBlock), 0, s, data, n, a->st, buf, a->seq, from_args,
+                           a->bucket_f, a->pdf_offset_f);
     else
-        hipLaunchKernelGGL(hist_kernel<false>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st);
+        hipLaunchKernelGGL(hist_kernel<false>, dim3(grid + 1), dim3(kBlock), 0, s, data, n, a->st, buf, a->seq,
+                           from_args, a->bucket_f, a->pdf_offset_f);
     MIQ_CHECK_LAUNCH();
     if (!a->range_known && !a->probe_pending)
     {
-        MIQ_CHECK_HIP(hipMemcpyAsync(a->probe_flag, &a->st->initialized, sizeof(int), hipMemcpyDeviceToHost, s));
+        // {initialized, iterations, bucket_f, pdf_offset_f} are adjacent in DevState
+        MIQ_CHECK_HIP(hipMemcpyAsync(a->probe_flag, &a->st->initialized, 4 * sizeof(int), hipMemcpyDeviceToHost, s));
         MIQ_CHECK_HIP(hipEventRecord(a->probe, s));
         a->probe_pending = true;
     }
     return MIQ_OK;
 }
 
-static int read_state(miq_analyzer* a, hipStream_t s)
+static int flush_pending(miq_analyzer* a, hipStream_t s)
 {
-    MIQ_CHECK_HIP(hipMemcpyAsync(a->pinned, a->st, sizeof(DevState), hipMemcpyDeviceToHost, s));
+    if (a->mode == MIQ_QUANTIZATION_TF_ENHANCED && a->seq != 0)
+    {
+        hipLaunchKernelGGL(hist_flush_kernel, dim3(1), dim3(kBlock), 0, s, a->st, a->seq);
+        MIQ_CHECK_LAUNCH();
+    }
+    return MIQ_OK;
+}
+
+static int read_state(miq_analyzer* a, hipStream_t s, size_t bytes = kInspectBytes)
+{
+    MIQ_CHECK_HIP(hipMemcpyAsync(a->pinned, a->st, bytes, hipMemcpyDeviceToHost, s));
     MIQ_CHECK_HIP(hipStreamSynchronize(s));
     const DevState* h = static_cast<const DevState*>(a->pinned);
     if (h->initialized)
-        a->range_known = true;
+    {
+        a->range_known  = true;
+        a->bucket_f     = h->bucket_f;
+        a->pdf_offset_f = h->pdf_offset_f;
+    }
     return MIQ_OK;
 }
 
@@ -918,7 +1055,7 @@ int miq_analyzer_compute_encoding(miq_analyzer* a, int bw, int use_symmetric, in
         return MIQ_OK;   // AimetTensorQuantizer::getEncoding returns a default encoding and valid = false
     if (a->mode == MIQ_QUANTIZATION_TF)
     {
-        if (int rc = read_state(a, s))
+        if (int rc = read_state(a, s, kHeadBytes))
             return rc;
         const DevState* h = static_cast<const DevState*>(a->pinned);
         // DLQ/src/TfEncodingAnalyzer.cpp:80-101 (MIN_RANGE = 0.01)
@@ -955,9 +1092,12 @@ int miq_analyzer_compute_encoding(miq_analyzer* a, int bw, int use_symmetric, in
         sa.n_cand  = cnt * 21 + 1;
     }
     MIQ_CHECK_ARG(sa.n_cand <= kMaxCand, "internal: candidate grid too large");
-    hipLaunchKernelGGL(tfe_search_kernel, dim3(sa.n_cand), dim3(64), 0, s, a->st, sa);
+    if (int rc = flush_pending(a, s))
+        return rc;
+    hipLaunchKernelGGL(tfe_search_kernel, dim3((sa.n_cand + kBlock / 64 - 1) / (kBlock / 64)), dim3(kBlock), 0, s, a->st,
+                       sa);
     MIQ_CHECK_LAUNCH();
-    if (int rc = read_state(a, s))
+    if (int rc = read_state(a, s, kHeadBytes))
         return rc;
     const DevState* h = static_cast<const DevState*>(a->pinned);
     out->min    = h->enc_min;
@@ -977,6 +1117,8 @@ int miq_analyzer_get_stats_histogram(miq_analyzer* a, double* x_left, double* pd
         set_error("no histogram is kept by the TF (min/max) analyzer");
         return MIQ_ERR_UNSUPPORTED;
     }
+    if (int rc = flush_pending(a, (hipStream_t) stream))
+        return rc;
     if (int rc = read_state(a, (hipStream_t) stream))
         return rc;
     const DevState* h = static_cast<const DevState*>(a->pinned);
@@ -992,6 +1134,8 @@ int miq_analyzer_get_stats_histogram(miq_analyzer* a, double* x_left, double* pd
 int miq_analyzer_last_batch_counts(miq_analyzer* a, uint32_t* counts, void* stream)
 {
     MIQ_CHECK_ARG(a && counts, "null argument");
+    if (int rc = flush_pending(a, (hipStream_t) stream))
+        return rc;
     if (int rc = read_state(a, (hipStream_t) stream))
         return rc;
     memcpy(counts, static_cast<const DevState*>(a->pinned)->last_counts, sizeof(uint32_t) * kPdf);

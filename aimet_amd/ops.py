@@ -230,6 +230,8 @@ class Analyzer:
         self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
         if self.device.type != "cuda":
             raise RuntimeError("an Analyzer lives on a GPU")
+        if self.device.index is None:
+            self.device = torch.device("cuda", torch.cuda.current_device())
         h = C.c_void_p()
         with torch.cuda.device(self.device):
             check(lib.miq_analyzer_create(self.mode, C.byref(h)))
@@ -248,14 +250,20 @@ class Analyzer:
             check(lib.miq_analyzer_reset(self._h, self._s()))
 
     def update_stats(self, x):
-        _require_gpu(x)
-        if x.device != self.device:
+        """Queue one batch.  Lean on purpose: a batch of a few MB takes microseconds on the device, so the Python
+        cost of this call is what bounds calibration throughput."""
+        if not x.is_cuda or x.device != self.device:
             raise RuntimeError(f"analyzer lives on {self.device}, tensor on {x.device}")
-        x = x.to(_F32).contiguous()
-        with torch.cuda.device(self.device):
-            check(lib.miq_analyzer_update_stats_f32(self._h, _ptr(x), x.numel(), self._s()))
-        # keep x alive until the kernels that read it have been queued behind it on the same stream
-        x.record_stream(torch.cuda.current_stream(self.device))
+        if x.dtype != _F32 or not x.is_contiguous():
+            x = x.to(_F32).contiguous()
+        # x was produced on (or converted on) the current stream and the kernels are queued on the same stream, so
+        # the caching allocator cannot hand its memory to anyone else before they have run
+        if torch.cuda.current_device() == self.device.index:
+            check(lib.miq_analyzer_update_stats_f32(self._h, x.data_ptr(), x.numel(),
+                                                    torch.cuda.current_stream().cuda_stream))
+        else:
+            with torch.cuda.device(self.device):
+                check(lib.miq_analyzer_update_stats_f32(self._h, x.data_ptr(), x.numel(), self._s()))
 
     def compute_encoding(self, bw, symmetric=False, strict_symmetric=False, unsigned_symmetric=False):
         """returns (Encoding, is_valid)"""
