@@ -44,7 +44,7 @@ inline bool aligned16(const void* p)
 }
 
 constexpr int kBlock  = 256;   // 4 wavefronts of 64 lanes
-constexpr int kUnroll = 4;     // 16-byte vectors in flight per lane
+constexpr int kUnroll = 2;     // 16-byte vectors in flight per lane (measured: 2 beats 4 and 8 for streaming)
 
 // ---- unsigned division of a 31-bit value by a launch-invariant divisor --------------------------------------
 // For n < 2^31 and 1 <= d < 2^31:  n / d == (n * magic) >> (31 + s)  with s = ceil(log2 d),

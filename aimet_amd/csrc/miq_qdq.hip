@@ -13,6 +13,7 @@
 //   v2  (aimet_torch.v2): r = rint(x / scale) - offset; y = (clamp(r, qmin, qmax) + offset) * scale
 //       TrainingExtensions/torch/src/python/aimet_torch/v2/quantization/affine/backends/torch_builtins.py:303-344
 #include "miq_common.h"
+#include "miq_fastmath.h"
 
 #include <cmath>
 
@@ -21,6 +22,32 @@ namespace miq
 namespace
 {
 // ------------------------------------------------------------------------------------------------ IO vector types
+// Streaming accesses are marked non-temporal: every byte is touched exactly once, and on this part that alone is
+// worth about 10 % of bandwidth for both the read-once inputs and the write-once outputs.
+typedef float nt_f4 __attribute__((ext_vector_type(4)));
+typedef unsigned int nt_u4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float4 stream_load(const float4* p)
+{
+    const nt_f4 v = __builtin_nontemporal_load(reinterpret_cast<const nt_f4*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint4 stream_load(const uint4* p)
+{
+    const nt_u4 v = __builtin_nontemporal_load(reinterpret_cast<const nt_u4*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void stream_store(float4* p, const float4& v)
+{
+    const nt_f4 w = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(w, reinterpret_cast<nt_f4*>(p));
+}
+__device__ __forceinline__ void stream_store(uint4* p, const uint4& v)
+{
+    const nt_u4 w = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(w, reinterpret_cast<nt_u4*>(p));
+}
+
 template <typename IO>
 struct IOTraits;
 
@@ -92,22 +119,45 @@ struct ParamSrc
     const float* c;   // v1: delta
     const float* d;   // v1: offset
     float4 scalar;    // per-tensor: the same four values
+    float scalar_rcp; // per-tensor: RN(1/delta), or 0 when delta is outside the fast-division contract
     int qmin, qmax;   // v2 grid
     float shift;      // v1 quantize-only: 2^(bw-1) or 0
     int ishift;       // the same as an integer, for byte codes
 };
 
+// v1 channel parameters.  rcp = RN(1/delta) when delta lies inside the contract of div_by_invariant, else 0, in
+// which case the quotient is formed with the ordinary division (both give the same bits; see miq_fastmath.h).
+struct V1P
+{
+    float mn, mx, delta, offset, rcp;
+};
+
+// RN(1/d) if every quotient this channel can form stays inside the contract of div_by_invariant, else 0
+__device__ __forceinline__ float safe_rcp(float d, float bound)
+{
+    return (fastdiv_divisor_ok(d) && bound <= kFastDivMaxDividend) ? 1.0f / d : 0.0f;
+}
+
 struct OpV1
 {
-    using P = float4;   // min, max, delta, offset
+    using P = V1P;
     __device__ static P load(const ParamSrc& s, uint32_t ch)
     {
-        return make_float4(s.a[ch], s.b[ch], s.c[ch], s.d[ch]);
+        const float mn = s.a[ch], mx = s.b[ch], d = s.c[ch];
+        // the dividend is clamped to [mn, mx] first, so max(|mn|, |mx|) bounds it
+        return P{mn, mx, d, s.d[ch], safe_rcp(d, fmaxf(fabsf(mn), fabsf(mx)))};
     }
+    // one decision per vector, not per element: whether the fast exact quotient may be used
+    __device__ static bool fast_ok(const P& p, const float*, int)
+    {
+        return p.rcp != 0.0f;
+    }
+    template <bool FAST>
     __device__ static float quant(const P& p, float x)
     {
-        float t = fmaxf(fminf(x, p.y), p.x);
-        t       = t / p.z - p.w;
+        float t = fmaxf(fminf(x, p.mx), p.mn);
+        t       = FAST ? div_by_invariant(t, p.delta, p.rcp) : t / p.delta;
+        t       = t - p.offset;
         return roundf(t);
     }
 };
@@ -117,11 +167,12 @@ struct OpV1Qdq : OpV1
 {
     static constexpr int NIN = 1;
     using Code               = uint8_t;
+    template <bool FAST>
     __device__ static float apply(const ParamSrc& s, const P& p, float x, float, int& code)
     {
-        float q = quant(p, x);
+        float q = quant<FAST>(p, x);
         code    = (int) q - s.ishift;
-        return p.z * (q + p.w);
+        return p.delta * (q + p.offset);
     }
 };
 
@@ -130,9 +181,10 @@ struct OpV1Quantize : OpV1
 {
     static constexpr int NIN = 1;
     using Code               = uint8_t;
+    template <bool FAST>
     __device__ static float apply(const ParamSrc& s, const P& p, float x, float, int& code)
     {
-        float q = quant(p, x);
+        float q = quant<FAST>(p, x);
         code    = 0;
         return q - s.shift;
     }
@@ -148,6 +200,11 @@ struct OpV1Ste
     {
         return make_float2(s.a[ch], s.b[ch]);
     }
+    __device__ static bool fast_ok(const P&, const float*, int)
+    {
+        return true;   // no division in this op
+    }
+    template <bool FAST>
     __device__ static float apply(const ParamSrc&, const P& p, float x, float g, int& code)
     {
         code = 0;
@@ -155,12 +212,33 @@ struct OpV1Ste
     }
 };
 
+struct V2P
+{
+    float scale, offset, rcp;
+};
+
 struct OpV2
 {
-    using P = float2;   // scale, offset
+    using P = V2P;
     __device__ static P load(const ParamSrc& s, uint32_t ch)
     {
-        return make_float2(s.a[ch], s.b[ch]);
+        const float sc = s.a[ch];
+        return P{sc, s.b[ch], safe_rcp(sc, 0.0f)};
+    }
+    // x is not clamped before the division here, so the dividend bound is checked on the vector's largest |x|
+    __device__ static bool fast_ok(const P& p, const float* x, int n)
+    {
+        float m = 0.0f;
+        for (int j = 0; j < n; ++j)
+            m = fmaxf(m, fabsf(x[j]));   // NaN elements are skipped: they give NaN on either path
+        return p.rcp != 0.0f && m <= kFastDivMaxDividend;
+    }
+    // round-half-even(x / scale) - offset
+    template <bool FAST>
+    __device__ static float grid(const P& p, float x)
+    {
+        const float q = FAST ? div_by_invariant(x, p.scale, p.rcp) : x / p.scale;
+        return rintf(q) - p.offset;
     }
 };
 
@@ -168,15 +246,16 @@ struct OpV2Qdq : OpV2
 {
     static constexpr int NIN = 1;
     using Code               = int32_t;
+    template <bool FAST>
     __device__ static float apply(const ParamSrc& s, const P& p, float x, float, int& code)
     {
-        float r = rintf(x / p.x) - p.y;
+        float r = grid<FAST>(p, x);
         // torch.clamp semantics: NaN stays NaN
         float q = r;
         q       = (q < (float) s.qmin) ? (float) s.qmin : q;
         q       = (q > (float) s.qmax) ? (float) s.qmax : q;
         code    = (int) q;
-        return (q + p.y) * p.x;
+        return (q + p.offset) * p.scale;
     }
 };
 
@@ -184,9 +263,10 @@ struct OpV2Bwd : OpV2
 {
     static constexpr int NIN = 2;
     using Code               = int32_t;
+    template <bool FAST>
     __device__ static float apply(const ParamSrc& s, const P& p, float x, float g, int& code)
     {
-        float r = rintf(x / p.x) - p.y;
+        float r = grid<FAST>(p, x);
         code    = 0;
         return g * (float) (((float) s.qmin <= r) && (r <= (float) s.qmax));
     }
@@ -195,14 +275,14 @@ struct OpV2Bwd : OpV2
 template <typename OP>
 __device__ typename OP::P scalar_params(const ParamSrc& s);
 template <>
-__device__ float4 scalar_params<OpV1Qdq>(const ParamSrc& s)
+__device__ V1P scalar_params<OpV1Qdq>(const ParamSrc& s)
 {
-    return s.scalar;
+    return V1P{s.scalar.x, s.scalar.y, s.scalar.z, s.scalar.w, s.scalar_rcp};
 }
 template <>
-__device__ float4 scalar_params<OpV1Quantize>(const ParamSrc& s)
+__device__ V1P scalar_params<OpV1Quantize>(const ParamSrc& s)
 {
-    return s.scalar;
+    return V1P{s.scalar.x, s.scalar.y, s.scalar.z, s.scalar.w, s.scalar_rcp};
 }
 template <>
 __device__ float2 scalar_params<OpV1Ste>(const ParamSrc& s)
@@ -211,14 +291,33 @@ __device__ float2 scalar_params<OpV1Ste>(const ParamSrc& s)
 }
 // v2 per-tensor: scale/offset are one-element device tensors; the load is wave-uniform (scalar load)
 template <>
-__device__ float2 scalar_params<OpV2Qdq>(const ParamSrc& s)
+__device__ V2P scalar_params<OpV2Qdq>(const ParamSrc& s)
 {
-    return make_float2(s.a[0], s.b[0]);
+    return OpV2::load(s, 0);
 }
 template <>
-__device__ float2 scalar_params<OpV2Bwd>(const ParamSrc& s)
+__device__ V2P scalar_params<OpV2Bwd>(const ParamSrc& s)
 {
-    return make_float2(s.a[0], s.b[0]);
+    return OpV2::load(s, 0);
+}
+
+// Applies OP to N elements that share one parameter set; the fast/plain quotient decision is taken once.
+template <typename OP, int N, bool TWO_IN>
+__device__ __forceinline__ void apply_n(const ParamSrc& s, const typename OP::P& p, const float* fx, const float* fg,
+                                        float* fy, int* code)
+{
+    if (OP::fast_ok(p, fx, N))
+    {
+#pragma unroll
+        for (int j = 0; j < N; ++j)
+            fy[j] = OP::template apply<true>(s, p, fx[j], TWO_IN ? fg[j] : 0.f, code[j]);
+    }
+    else
+    {
+#pragma unroll
+        for (int j = 0; j < N; ++j)
+            fy[j] = OP::template apply<false>(s, p, fx[j], TWO_IN ? fg[j] : 0.f, code[j]);
+    }
 }
 
 // ----------------------------------------------------------------------------------------------------- the kernels
@@ -274,25 +373,7 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
     const int64_t e_base    = (int64_t) blockIdx.x * TILE;
     const int64_t nvec      = n / VEC;
 
-    __shared__ P win[PER_CHANNEL ? kWin : 1];
-    uint32_t rem0 = 0;
-    P pt;
-    if constexpr (PER_CHANNEL)
-    {
-        const uint32_t eb   = (uint32_t) e_base;
-        const uint32_t row0 = fastdiv(eb, fd);
-        rem0                = eb - row0 * fd.d;
-        const uint32_t ee   = (uint32_t) (((int64_t) eb + TILE < n) ? eb + TILE : n);
-        const uint32_t row1 = fastdiv(ee - 1, fd);
-        for (uint32_t r = threadIdx.x; r <= row1 - row0; r += kBlock)
-            win[r] = OP::load(src, (row0 + r) % num_channel);
-        __syncthreads();
-    }
-    else
-    {
-        pt = scalar_params<OP>(src);
-    }
-
+    // 1. the tile's loads go out first; everything below overlaps their latency
     Vec vx[kUnroll], vg[kUnroll];
     bool live[kUnroll];
 #pragma unroll
@@ -302,11 +383,43 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
         live[u]         = v < nvec;
         if (live[u])
         {
-            vx[u] = reinterpret_cast<const Vec*>(ptr.x)[v];
+            vx[u] = stream_load(reinterpret_cast<const Vec*>(ptr.x) + v);
             if constexpr (OP::NIN == 2)
-                vg[u] = reinterpret_cast<const Vec*>(ptr.g)[v];
+                vg[u] = stream_load(reinterpret_cast<const Vec*>(ptr.g) + v);
         }
     }
+
+    // 2. parameters: kernel arguments (per-tensor), scalar loads when the whole tile lies in one channel row (the
+    //    usual case for weights: a row is at least a tile long), else the LDS window of the rows the tile touches
+    __shared__ P win[PER_CHANNEL ? kWin : 1];
+    uint32_t rem0   = 0;
+    bool one_row    = true;
+    P pt;
+    if constexpr (PER_CHANNEL)
+    {
+        const uint32_t eb   = (uint32_t) e_base;
+        const uint32_t row0 = fastdiv(eb, fd);
+        rem0                = eb - row0 * fd.d;
+        const uint32_t ee   = (uint32_t) (((int64_t) eb + TILE < n) ? eb + TILE : n);
+        const uint32_t row1 = fastdiv(ee - 1, fd);
+        one_row             = (row0 == row1);   // workgroup-uniform
+        if (one_row)
+        {
+            pt = OP::load(src, row0 % num_channel);
+        }
+        else
+        {
+            for (uint32_t r = threadIdx.x; r <= row1 - row0; r += kBlock)
+                win[r] = OP::load(src, (row0 + r) % num_channel);
+            __syncthreads();
+        }
+    }
+    else
+    {
+        pt = scalar_params<OP>(src);
+    }
+
+    // 3. compute and store
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
     {
@@ -319,7 +432,11 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
         T::unpack(vx[u], fx);
         if constexpr (OP::NIN == 2)
             T::unpack(vg[u], fg);
-        if constexpr (PER_CHANNEL)
+        if (one_row)
+        {
+            apply_n<OP, VEC, OP::NIN == 2>(src, pt, fx, fg, fy, code);
+        }
+        else
         {
             const uint32_t t   = rem0 + le;
             const uint32_t lr  = fastdiv(t, fd);
@@ -327,9 +444,7 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
             if (rem + VEC <= fd.d)
             {
                 const P p = win[lr];
-#pragma unroll
-                for (int j = 0; j < VEC; ++j)
-                    fy[j] = OP::apply(src, p, fx[j], OP::NIN == 2 ? fg[j] : 0.f, code[j]);
+                apply_n<OP, VEC, OP::NIN == 2>(src, p, fx, fg, fy, code);
             }
             else
             {
@@ -338,18 +453,12 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
                 for (int j = 0; j < VEC; ++j)
                 {
                     const P p = win[lr + ((rem + j >= fd.d) ? 1u : 0u)];
-                    fy[j]     = OP::apply(src, p, fx[j], OP::NIN == 2 ? fg[j] : 0.f, code[j]);
+                    fy[j]     = OP::template apply<false>(src, p, fx[j], OP::NIN == 2 ? fg[j] : 0.f, code[j]);
                 }
             }
         }
-        else
-        {
-#pragma unroll
-            for (int j = 0; j < VEC; ++j)
-                fy[j] = OP::apply(src, pt, fx[j], OP::NIN == 2 ? fg[j] : 0.f, code[j]);
-        }
         if (ptr.y)
-            reinterpret_cast<Vec*>(ptr.y)[v] = T::pack(fy);
+            stream_store(reinterpret_cast<Vec*>(ptr.y) + v, T::pack(fy));
         if (ptr.codes)
             store_codes<typename OP::Code, VEC>(ptr.codes + v * VEC, code);
     }
@@ -363,7 +472,8 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
         else
             p = pt;
         int code;
-        const float y = OP::apply(src, p, T::load1(ptr.x + e), OP::NIN == 2 ? T::load1(ptr.g + e) : 0.f, code);
+        const float y =
+            OP::template apply<false>(src, p, T::load1(ptr.x + e), OP::NIN == 2 ? T::load1(ptr.g + e) : 0.f, code);
         if (ptr.y)
             T::store1(ptr.y + e, y);
         if (ptr.codes)
@@ -387,7 +497,8 @@ __global__ __launch_bounds__(kBlock) void ew_scalar_kernel(EwPtrs<IO, typename O
         else
             p = scalar_params<OP>(src);
         int code;
-        const float y = OP::apply(src, p, T::load1(ptr.x + e), OP::NIN == 2 ? T::load1(ptr.g + e) : 0.f, code);
+        const float y =
+            OP::template apply<false>(src, p, T::load1(ptr.x + e), OP::NIN == 2 ? T::load1(ptr.g + e) : 0.f, code);
         if (ptr.y)
             T::store1(ptr.y + e, y);
         if (ptr.codes)
@@ -452,6 +563,9 @@ ParamSrc per_tensor_src(const miq_encoding& e)
 {
     ParamSrc s{};
     s.scalar = make_float4((float) e.min, (float) e.max, (float) e.delta, (float) e.offset);
+    // IEEE single division on the host gives the same correctly rounded reciprocal the device would compute
+    const float bound = std::fmax(std::fabs(s.scalar.x), std::fabs(s.scalar.y));
+    s.scalar_rcp      = (fastdiv_divisor_ok(s.scalar.z) && bound <= kFastDivMaxDividend) ? 1.0f / s.scalar.z : 0.0f;
     return s;
 }
 
@@ -498,9 +612,9 @@ __global__ __launch_bounds__(kBlock) void qdq_broadcast_kernel(const float* in, 
             rem     = (int) (rem - idx * b.istride[d]);
             enc += (int) (b.estride[d] * idx);
         }
-        const float4 p = make_float4(mn[enc], mx[enc], delta[enc], offset[enc]);
-        const float q  = OpV1::quant(p, in[e]);
-        out[e]         = p.z * (q + p.w);
+        const V1P p   = V1P{mn[enc], mx[enc], delta[enc], offset[enc], 0.0f};
+        const float q = OpV1::quant<false>(p, in[e]);
+        out[e]        = p.delta * (q + p.offset);
     }
 }
 static ParamSrc v1_channel_src(const float* mn, const float* mx, const float* d, const float* o)
