@@ -1,0 +1,325 @@
+"""QuantizationSimModel of the v1 path.
+
+Mirrors the user-facing surface of TrainingExtensions/torch/src/python/aimet_torch/v1/quantsim.py
+(constructor :225-307, compute_encodings :381-448, encodings export :486-576) and the quantizer-configuration
+semantics of TrainingExtensions/torch/src/python/aimet_torch/quantsim_config/quantsim_config.py:291-593 for the JSON
+keys that matter to this path: defaults (ops / params / strict_symmetric / unsigned_symmetric /
+per_channel_quantization), params, op_type, supergroups, model_input, model_output.
+
+The reference discovers the graph with torch.jit.trace (ConnectedGraph).  Here one forward pass with hooks on the
+leaf modules records the execution order and which module produced / consumed each tensor; that is enough to apply
+the supergroup and model-input rules to models built from modules (functional ``+`` needs the ``Add`` module of
+aimet_amd.v1.nn.modules.custom, as in the reference).
+"""
+import copy
+import json
+import os
+from typing import Dict, List, Tuple, Union
+
+import torch
+from torch import nn
+
+from ..common.defs import QuantizationDataType, QuantScheme
+from .nn.modules import custom
+from .qc_quantize_op import QcQuantizeOpMode, QcQuantizeWrapper, StaticGridQuantWrapper
+
+# same rules as the reference's aimet_common/quantsim_config/default_config.json
+DEFAULT_CONFIG = {
+    "defaults": {"ops": {"is_output_quantized": "True"},
+                 "params": {"is_quantized": "True", "is_symmetric": "True"},
+                 "strict_symmetric": "False", "per_channel_quantization": "False"},
+    "params": {"bias": {"is_quantized": "False"}},
+    "op_type": {"Dropout": {"is_output_quantized": "False"}, "Flatten": {"is_output_quantized": "False"}},
+    "supergroups": [{"op_list": ["Conv", "Relu"]}, {"op_list": ["ConvTranspose", "Relu"]},
+                    {"op_list": ["Conv", "Clip"]}, {"op_list": ["Add", "Relu"]}, {"op_list": ["Gemm", "Relu"]}],
+    "model_input": {"is_input_quantized": "True"},
+    "model_output": {},
+}
+
+_OP_TYPES = (
+    ((nn.ConvTranspose1d, nn.ConvTranspose2d, nn.ConvTranspose3d), "ConvTranspose"),
+    ((nn.Conv1d, nn.Conv2d, nn.Conv3d), "Conv"),
+    ((nn.Linear,), "Gemm"),
+    ((nn.ReLU,), "Relu"),
+    ((nn.ReLU6, nn.Hardtanh), "Clip"),
+    ((nn.BatchNorm1d, nn.BatchNorm2d, nn.BatchNorm3d), "BatchNormalization"),
+    ((nn.MaxPool1d, nn.MaxPool2d, nn.MaxPool3d), "MaxPool"),
+    ((nn.AvgPool1d, nn.AvgPool2d, nn.AvgPool3d), "AveragePool"),
+    ((nn.AdaptiveAvgPool1d, nn.AdaptiveAvgPool2d), "GlobalAveragePool"),
+    ((nn.Dropout, nn.Dropout2d), "Dropout"),
+    ((nn.Flatten,), "Flatten"),
+    ((nn.Sigmoid,), "Sigmoid"),
+    ((nn.Tanh,), "Tanh"),
+    ((nn.Softmax,), "Softmax"),
+    ((nn.LayerNorm,), "LayerNormalization"),
+    ((custom.Add,), "Add"),
+    ((custom.Subtract,), "Sub"),
+    ((custom.Multiply,), "Mul"),
+    ((custom.Concat,), "Concat"),
+)
+
+
+def _op_type(module: nn.Module) -> str:
+    for classes, name in _OP_TYPES:
+        if isinstance(module, classes):
+            return name
+    return type(module).__name__
+
+
+def _flag(d: dict, key: str, default=None):
+    if key not in d:
+        return default
+    return str(d[key]) == "True"
+
+
+class QuantizationSimModel:
+    """Adds quantization simulation ops to a model for off-target simulation of quantized inference accuracy."""
+
+    # pylint: disable=too-many-arguments
+    def __init__(self, model: nn.Module, dummy_input: Union[torch.Tensor, Tuple],
+                 quant_scheme: Union[str, QuantScheme] = QuantScheme.post_training_tf_enhanced,
+                 rounding_mode: str = 'nearest', default_output_bw: int = 8, default_param_bw: int = 8,
+                 in_place: bool = False, config_file: str = None,
+                 default_data_type: QuantizationDataType = QuantizationDataType.int):
+        if isinstance(quant_scheme, str):
+            quant_scheme = {'tf': QuantScheme.post_training_tf,
+                            'tf_enhanced': QuantScheme.post_training_tf_enhanced}[quant_scheme]
+        if quant_scheme not in (QuantScheme.post_training_tf, QuantScheme.post_training_tf_enhanced):
+            raise ValueError(f"quant_scheme {quant_scheme} is not implemented (tf and tf_enhanced are)")
+        if rounding_mode not in ('nearest', 'stochastic'):
+            raise ValueError('Parameter round mode can only be nearest or stochastic')
+        if default_param_bw < 4 or default_param_bw > 32 or default_output_bw < 4 or default_output_bw > 32:
+            raise ValueError('Default bitwidth for parameters and activations must be between 4 and 32')
+        if default_data_type != QuantizationDataType.int:
+            raise ValueError('only QuantizationDataType.int is implemented')
+        self.model = model if in_place else copy.deepcopy(model)
+        self._quant_scheme = quant_scheme
+        self._rounding_mode = rounding_mode
+        self._default_output_bw = default_output_bw
+        self._default_param_bw = default_param_bw
+        self._config = DEFAULT_CONFIG if config_file is None else self._load_config(config_file)
+        dummy_input = dummy_input if isinstance(dummy_input, (tuple, list)) else (dummy_input,)
+        self._graph = self._trace(self.model, dummy_input)
+        self._add_quantization_wrappers()
+        self._configure_quantization_ops()
+
+    # ------------------------------------------------------------------------------------------------ construction
+    @staticmethod
+    def _load_config(config_file: str) -> dict:
+        with open(config_file) as f:
+            return json.load(f)
+
+    @staticmethod
+    def _is_leaf(module: nn.Module) -> bool:
+        return len(list(module.children())) == 0
+
+    def _trace(self, model: nn.Module, dummy_input: Tuple):
+        """One hooked forward pass: execution order of the leaf modules and tensor producers / consumers."""
+        records, handles = [], []
+        producer: Dict[int, str] = {}
+        consumers: Dict[int, List[str]] = {}
+        keep_alive = []
+        names = {m: n for n, m in model.named_modules()}
+        for t in dummy_input:
+            if isinstance(t, torch.Tensor):
+                producer[id(t)] = "__model_input__"
+
+        def hook(module, inputs, output):
+            name = names[module]
+            ins = [t for t in inputs if isinstance(t, torch.Tensor)]
+            outs = [t for t in (output if isinstance(output, (tuple, list)) else (output,))
+                    if isinstance(t, torch.Tensor)]
+            keep_alive.extend(ins + outs)            # ids stay unique while the pass runs
+            for t in ins:
+                consumers.setdefault(id(t), []).append(name)
+            records.append({"name": name, "module": module, "type": _op_type(module),
+                            "inputs": [producer.get(id(t)) for t in ins], "in_ids": [id(t) for t in ins],
+                            "out_ids": [id(t) for t in outs], "num_inputs": max(1, len(ins)),
+                            "num_outputs": max(1, len(outs))})
+            for t in outs:
+                producer[id(t)] = name
+
+        for module in model.modules():
+            if self._is_leaf(module) and module is not model:
+                handles.append(module.register_forward_hook(hook))
+        was_training = model.training
+        model.eval()
+        try:
+            with torch.no_grad():
+                out = model(*dummy_input)
+        finally:
+            for h in handles:
+                h.remove()
+            model.train(was_training)
+        outs = out if isinstance(out, (tuple, list)) else (out,)
+        model_outputs = {producer.get(id(t)) for t in outs if isinstance(t, torch.Tensor)}
+        for r in records:
+            r["consumers"] = [c for oid in r["out_ids"] for c in consumers.get(oid, [])]
+            r["is_model_output"] = r["name"] in model_outputs
+        return records
+
+    def _add_quantization_wrappers(self):
+        seen = set()
+        for rec in self._graph:
+            if rec["name"] in seen:
+                raise RuntimeError(f"module {rec['name']} is used more than once in the forward pass; "
+                                   "give each use its own module")
+            seen.add(rec["name"])
+            wrapper = StaticGridQuantWrapper(rec["module"], self._default_param_bw, self._default_output_bw,
+                                             self._rounding_mode, self._quant_scheme, num_inputs=rec["num_inputs"],
+                                             num_outputs=rec["num_outputs"])
+            rec["wrapper"] = wrapper
+            parent = self.model
+            *path, leaf = rec["name"].split('.')
+            for p in path:
+                parent = getattr(parent, p)
+            setattr(parent, leaf, wrapper)
+
+    def _configure_quantization_ops(self):
+        """Precedence as in the reference: defaults -> params -> op_type -> supergroups -> model_input -> model_output."""
+        cfg = self._config
+        defaults = cfg.get("defaults", {})
+        out_q = _flag(defaults.get("ops", {}), "is_output_quantized", False)
+        in_q = _flag(defaults.get("ops", {}), "is_input_quantized", False)
+        act_sym = _flag(defaults.get("ops", {}), "is_symmetric", False)
+        par_q = _flag(defaults.get("params", {}), "is_quantized", False)
+        par_sym = _flag(defaults.get("params", {}), "is_symmetric", False)
+        strict = _flag(defaults, "strict_symmetric", False)
+        unsigned = _flag(defaults, "unsigned_symmetric", False)
+        per_channel = _flag(defaults, "per_channel_quantization", False)
+        by_name = {r["name"]: r for r in self._graph}
+        for rec in self._graph:
+            w: StaticGridQuantWrapper = rec["wrapper"]
+            op_cfg = cfg.get("op_type", {}).get(rec["type"], {})
+            w.enable_output_quantizers(_flag(op_cfg, "is_output_quantized", out_q))
+            w.enable_input_quantizers(_flag(op_cfg, "is_input_quantized", in_q))
+            for q in w.input_quantizers + w.output_quantizers:
+                q.use_symmetric_encodings = _flag(op_cfg, "is_symmetric", act_sym)
+                q.use_strict_symmetric, q.use_unsigned_symmetric = strict, unsigned
+            for pname, q in w.param_quantizers.items():
+                pcfg = dict(cfg.get("params", {}).get(pname, {}))
+                pcfg.update(op_cfg.get("params", {}).get(pname, {}))
+                q.enabled = _flag(pcfg, "is_quantized", par_q)
+                q.use_symmetric_encodings = _flag(pcfg, "is_symmetric", par_sym)
+                q.use_strict_symmetric, q.use_unsigned_symmetric = strict, unsigned
+            if rec["type"] == "BatchNormalization":
+                w.enable_param_quantizers(False, None)        # BN statistics are never quantized
+            if _flag(op_cfg, "per_channel_quantization", per_channel) and w.param_quantizers:
+                w.enable_per_channel_quantization()
+        # supergroups: inside a matched chain only the last op keeps its output quantizer
+        for group in cfg.get("supergroups", []):
+            ops_list = group["op_list"]
+            for rec in self._graph:
+                chain, cur = [rec], rec
+                for want in ops_list[1:]:
+                    nxt = [by_name[c] for c in set(cur["consumers"])]
+                    if len(nxt) != 1 or nxt[0]["type"] != want or cur["is_model_output"]:
+                        chain = None
+                        break
+                    cur = nxt[0]
+                    chain.append(cur)
+                if chain is None or rec["type"] != ops_list[0]:
+                    continue
+                for member in chain[:-1]:
+                    member["wrapper"].enable_output_quantizers(False)
+                for member in chain[1:]:
+                    member["wrapper"].enable_input_quantizers(False)
+        if _flag(cfg.get("model_input", {}), "is_input_quantized", False):
+            for rec in self._graph:
+                for idx, src in enumerate(rec["inputs"]):
+                    if src == "__model_input__" and idx < len(rec["wrapper"].input_quantizers):
+                        rec["wrapper"].input_quantizers[idx].enabled = True
+        if _flag(cfg.get("model_output", {}), "is_output_quantized", False):
+            for rec in self._graph:
+                if rec["is_model_output"]:
+                    rec["wrapper"].enable_output_quantizers(True)
+
+    # --------------------------------------------------------------------------------------------------- usage
+    def quant_wrappers(self):
+        """Generator of (name, wrapper) in the model."""
+        for name, module in self.model.named_modules():
+            if isinstance(module, QcQuantizeWrapper):
+                yield name, module
+
+    _get_qc_quantized_layers = staticmethod(lambda model: [(n, m) for n, m in model.named_modules()
+                                                           if isinstance(m, QcQuantizeWrapper)])
+
+    def __str__(self):
+        lines = ["-------------------------", "Quantized Model Report", "-------------------------"]
+        for name, w in self.quant_wrappers():
+            lines.append(f"Layer: {name}")
+            lines.append(f"  inputs : {[(q.enabled, q.bitwidth) for q in w.input_quantizers]}")
+            lines.append(f"  params : {{{', '.join(f'{k}: ({q.enabled}, {q.bitwidth})' for k, q in w.param_quantizers.items())}}}")
+            lines.append(f"  outputs: {[(q.enabled, q.bitwidth) for q in w.output_quantizers]}")
+        return "\n".join(lines)
+
+    def compute_encodings(self, forward_pass_callback, forward_pass_callback_args):
+        """Runs `forward_pass_callback(model, args)` in ANALYSIS mode, then computes every encoding and switches the
+        wrappers to ACTIVE (reference :425-448)."""
+        layers = self._get_qc_quantized_layers(self.model)
+        for _, layer in layers:
+            layer.reset_encodings()
+            layer.set_mode(QcQuantizeOpMode.ANALYSIS)
+        was_training = self.model.training
+        self.model.eval()
+        try:
+            with torch.no_grad():
+                forward_pass_callback(self.model, forward_pass_callback_args)
+        finally:
+            self.model.train(was_training)
+        for _, layer in layers:
+            layer.compute_encoding()
+            layer.set_mode(QcQuantizeOpMode.ACTIVE)
+
+    # ------------------------------------------------------------------------------------ encodings on disk
+    @staticmethod
+    def _encoding_dict(enc, symmetric: bool) -> dict:
+        # the reference's legacy format (aimet_torch/utils.py:1140-1170)
+        return {'min': enc.min, 'max': enc.max, 'scale': enc.delta, 'offset': int(enc.offset), 'bitwidth': enc.bw,
+                'is_symmetric': str(symmetric), 'dtype': 'int'}
+
+    def get_encodings_dict(self) -> dict:
+        param_enc, act_enc = {}, {}
+        for name, w in self.quant_wrappers():
+            for pname, q in w.param_quantizers.items():
+                if q.enabled and q.encoding is not None:
+                    encs = q.encoding if isinstance(q.encoding, list) else [q.encoding]
+                    param_enc[f"{name}.{pname}"] = [self._encoding_dict(e, q.use_symmetric_encodings) for e in encs]
+            entry = {}
+            for kind, qs in (('input', w.input_quantizers), ('output', w.output_quantizers)):
+                for i, q in enumerate(qs):
+                    if q.enabled and q.encoding is not None:
+                        entry.setdefault(kind, {})[str(i)] = self._encoding_dict(q.encoding,
+                                                                                 q.use_symmetric_encodings)
+            if entry:
+                act_enc[name] = entry
+        return {'version': '0.6.1', 'activation_encodings': act_enc, 'param_encodings': param_enc,
+                'quantizer_args': {'activation_bitwidth': self._default_output_bw,
+                                   'param_bitwidth': self._default_param_bw, 'dtype': 'int',
+                                   'quant_scheme': self._quant_scheme.name}}
+
+    def export_encodings(self, path: str, filename_prefix: str) -> str:
+        os.makedirs(path, exist_ok=True)
+        file = os.path.join(path, filename_prefix + '.encodings')
+        with open(file, 'w') as f:
+            json.dump(self.get_encodings_dict(), f, sort_keys=True, indent=4)
+        return file
+
+    def set_and_freeze_param_encodings(self, encoding_path: str):
+        """Loads parameter encodings written by export_encodings / Adaround and freezes them
+        (reference quantsim.py:1695-1756, qc_quantize_op.py:499-560)."""
+        from ..common import libpymo
+        with open(encoding_path) as f:
+            data = json.load(f)
+        param_encodings = data.get('param_encodings', data)
+        for name, w in self.quant_wrappers():
+            for pname, q in w.param_quantizers.items():
+                key = f"{name}.{pname}"
+                if key in param_encodings:
+                    encs = [libpymo.TfEncoding(e['min'], e['max'], e['scale'], e['offset'], e['bitwidth'])
+                            for e in param_encodings[key]]
+                    q.enabled = True
+                    q.bitwidth = encs[0].bw
+                    q.use_symmetric_encodings = param_encodings[key][0]['is_symmetric'] == 'True'
+                    q.encoding = encs if isinstance(q.encoding, list) or len(encs) > 1 else encs[0]
+                    q.freeze_encoding()

@@ -1,0 +1,163 @@
+"""``hip_gfx950``: the v2 affine quantization backend on hand-written HIP kernels.
+
+Same functions, argument meaning and error behaviour as the reference's torch_builtins backend
+(TrainingExtensions/torch/src/python/aimet_torch/v2/quantization/affine/backends/torch_builtins.py:52-344):
+
+    quantize            out = clamp(round_half_even(x / scale) - offset, qmin, qmax)
+    dequantize          out = (x + offset) * scale
+    quantize_dequantize out = (clamp(round_half_even(x / scale) - offset, qmin, qmax) + offset) * scale
+
+The forward of quantize / quantize_dequantize is one fused kernel (the reference runs about seven elementwise ATen
+kernels and saves a bool mask); the input gradient is one fused kernel that recomputes the mask from the saved
+input.  float32 and bfloat16 tensors are computed in float32, as the reference does for 4- and 8-bit grids; other
+float types are upcast to float32.  Scale / offset must be per-tensor or per-channel along one axis (numpy-style
+broadcast); block quantization (`block_size`) and multi-axis scales are not implemented.
+
+Gradients w.r.t. scale and offset (range learning) are formed with tensor ops from the same formulas
+(torch_builtins.py:329-344); they are not on the measured hot path.
+"""
+from typing import List, Optional
+
+import torch
+
+from ..... import ops
+from ....utils import _is_expandable
+
+
+def _is_value_representable(dtype: torch.dtype, value: int) -> bool:
+    r = torch.tensor(value, dtype=dtype)
+    return bool(r.isfinite()) and int(r.long()) == value
+
+
+def _is_grid_representable(dtype: torch.dtype, qmin: int, qmax: int) -> bool:
+    return all(_is_value_representable(dtype, v) for v in (qmax, qmax - 1, qmin + 1, qmin))
+
+
+def _validate_arguments(tensor, scale, offset, qmin=None, qmax=None, block_size=None):
+    if block_size is not None:
+        raise RuntimeError("block_size is not implemented by the hip_gfx950 backend")
+    if not _is_expandable(scale.shape, tensor.shape):
+        raise RuntimeError(f"Scale of shape {scale.shape} cannot be expanded like input tensor of shape "
+                           f"{tensor.shape}")
+    if tensor.device != scale.device or tensor.device != offset.device:
+        raise RuntimeError(f"Expected all tensors to be on the same device, but found {tensor.device}, "
+                           f"{scale.device} and {offset.device}")
+    if qmin is not None and qmax is not None and qmin > qmax:
+        raise RuntimeError(f"qmin ({qmin}) must be smaller than or equal to qmax ({qmax})")
+
+
+def _channel_geometry(tensor_shape, scale_shape):
+    """(num_channel, n_per_channel) of a scale that is per-tensor or varies along exactly one axis."""
+    padded = (1,) * (len(tensor_shape) - len(scale_shape)) + tuple(scale_shape)
+    axes = [a for a, d in enumerate(padded) if d != 1]
+    if not axes:
+        n = 1
+        for d in tensor_shape:
+            n *= d
+        return 1, max(n, 1)
+    if len(axes) > 1:
+        raise RuntimeError(f"scale of shape {tuple(scale_shape)} varies along more than one axis: not implemented by "
+                           "the hip_gfx950 backend")
+    axis = axes[0]
+    npc = 1
+    for d in tensor_shape[axis + 1:]:
+        npc *= d
+    return tensor_shape[axis], npc
+
+
+def _reduce_like(grad: torch.Tensor, shape) -> torch.Tensor:
+    return grad.sum_to_size(shape) if tuple(grad.shape) != tuple(shape) else grad
+
+
+class _QuantDequantFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, tensor, scale, offset, qmin, qmax):  # pylint: disable=arguments-differ
+        c, npc = _channel_geometry(tensor.shape, scale.shape)
+        out = ops.v2_qdq(tensor, c, npc, scale, offset, qmin, qmax)
+        ctx.geom = (c, npc, qmin, qmax)
+        ctx.save_for_backward(tensor, scale, offset)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):  # pylint: disable=arguments-differ
+        tensor, scale, offset = ctx.saved_tensors
+        c, npc, qmin, qmax = ctx.geom
+        tensor_grad = scale_grad = offset_grad = None
+        if ctx.needs_input_grad[0]:
+            tensor_grad = ops.v2_qdq_bwd(tensor, grad, c, npc, scale, offset, qmin, qmax)
+        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+            s, o = scale.to(torch.float32), offset.to(torch.float32)
+            x = tensor.to(torch.float32) / s
+            x_round = torch.round(x) - o
+            mask = (qmin <= x_round) & (x_round <= qmax)
+            g = grad.to(torch.float32)
+            if ctx.needs_input_grad[1]:
+                scale_grad = _reduce_like(g * (torch.round(x).clamp(o + qmin, o + qmax) - x * mask),
+                                          scale.shape).to(scale.dtype)
+            if ctx.needs_input_grad[2]:
+                offset_grad = _reduce_like(g * (~mask * s), offset.shape).to(offset.dtype)
+        return tensor_grad, scale_grad, offset_grad, None, None
+
+
+class _QuantizeFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, tensor, scale, offset, qmin, qmax):  # pylint: disable=arguments-differ
+        c, npc = _channel_geometry(tensor.shape, scale.shape)
+        x = tensor.to(torch.float32)
+        _, codes = ops.v2_qdq(x, c, npc, scale, offset, qmin, qmax, want_codes=True)
+        ctx.geom = (c, npc, qmin, qmax)
+        ctx.save_for_backward(tensor, scale, offset)
+        return codes.to(tensor.dtype)
+
+    @staticmethod
+    def backward(ctx, grad):  # pylint: disable=arguments-differ
+        tensor, scale, offset = ctx.saved_tensors
+        c, npc, qmin, qmax = ctx.geom
+        # torch_builtins.py:236-246: masked_grad = grad * mask; d/dx = masked / scale;
+        # d/dscale = -(masked / scale) * (x / scale); d/doffset = -masked
+        masked = ops.v2_qdq_bwd(tensor.to(torch.float32), grad.to(torch.float32), c, npc, scale, offset, qmin, qmax)
+        s = scale.to(torch.float32)
+        tensor_grad = (masked / s).to(tensor.dtype) if ctx.needs_input_grad[0] else None
+        scale_grad = _reduce_like(-(masked / s) * (tensor.to(torch.float32) / s), scale.shape).to(scale.dtype) \
+            if ctx.needs_input_grad[1] else None
+        offset_grad = _reduce_like(-masked, offset.shape).to(offset.dtype) if ctx.needs_input_grad[2] else None
+        return tensor_grad, scale_grad, offset_grad, None, None
+
+
+def _prepare(tensor, scale, offset):
+    if not tensor.is_cuda:
+        raise RuntimeError("the hip_gfx950 backend computes on the GPU only; got a tensor on " + str(tensor.device))
+    if tensor.dtype not in (torch.float32, torch.bfloat16):
+        if not tensor.is_floating_point():
+            raise RuntimeError(f"expected a floating point tensor, got {tensor.dtype}")
+        return tensor.to(torch.float32), tensor.dtype
+    return tensor, None
+
+
+def quantize(tensor: torch.Tensor, scale: torch.Tensor, offset: torch.Tensor, qmin: int, qmax: int,
+             block_size: Optional[List] = None) -> torch.Tensor:
+    """Differentiable quantization: integer-valued output in the input's dtype."""
+    _validate_arguments(tensor, scale, offset, qmin, qmax, block_size)
+    if not _is_grid_representable(tensor.dtype, qmin, qmax):
+        raise RuntimeError(f"{tensor.dtype} is unable to represent quantized output of range [{qmin}, {qmax}].")
+    x, orig = _prepare(tensor, scale, offset)
+    out = _QuantizeFunc.apply(x, scale, offset, qmin, qmax)
+    return out.to(orig) if orig is not None else out
+
+
+def quantize_dequantize(tensor: torch.Tensor, scale: torch.Tensor, offset: torch.Tensor, qmin: int, qmax: int,
+                        block_size: Optional[List] = None) -> torch.Tensor:
+    """Differentiable quantize-dequantize (fake quantization)."""
+    _validate_arguments(tensor, scale, offset, qmin, qmax, block_size)
+    if not _is_grid_representable(torch.float32, qmin, qmax):
+        raise RuntimeError(f"{torch.float32} is unable to represent quantized output of range [{qmin}, {qmax}].")
+    x, orig = _prepare(tensor, scale, offset)
+    out = _QuantDequantFunc.apply(x, scale, offset, qmin, qmax)
+    return out.to(orig) if orig is not None else out
+
+
+def dequantize(tensor: torch.Tensor, scale: torch.Tensor, offset: torch.Tensor,
+               block_size: Optional[List] = None) -> torch.Tensor:
+    """(x + offset) * scale on an already quantized tensor; not a hot op (two elementwise tensor ops)."""
+    _validate_arguments(tensor, scale, offset, block_size=block_size)
+    return (tensor + offset.to(tensor.dtype)) * scale.to(tensor.dtype)

@@ -1,0 +1,233 @@
+"""v2 affine quantizer modules.
+
+Mirrors TrainingExtensions/torch/src/python/aimet_torch/v2/quantization/affine/quantizer.py: AffineQuantizerBase
+constructor signatures (:64-148), MinMaxQuantizer (:303-445: learnable ``min`` / ``max`` parameters, compute_encodings
+context, get_min / get_max / get_scale / get_offset / set_range), Quantize (:448-563) and QuantizeDequantize
+(:566-697).  The arithmetic is dispatched through the backend registry to the HIP kernels.
+"""
+import contextlib
+import functools
+from typing import Optional
+
+import torch
+from torch import nn
+
+from ...utils import StatisticsNotFoundError, _is_expandable, patch_attr, ste_round
+from ..encoding_analyzer import EncodingAnalyzer, MinMaxEncodingAnalyzer
+from .backends import _derive_qmin_qmax, quantize, quantize_dequantize
+
+
+class _AffineEncoding:
+    """Value object returned by get_encoding(): scale, offset, grid."""
+
+    def __init__(self, scale, offset, qmin, qmax, symmetry, block_size=None):
+        self.scale, self.offset, self.qmin, self.qmax = scale, offset, qmin, qmax
+        self.symmetry, self.block_size = symmetry, block_size
+
+    @property
+    def num_steps(self):
+        return self.qmax - self.qmin
+
+    @property
+    def bitwidth(self):
+        return (self.qmax - self.qmin).bit_length()
+
+    @property
+    def min(self):
+        return self.scale * (self.offset + self.qmin)
+
+    @property
+    def max(self):
+        return self.scale * (self.offset + self.qmax)
+
+
+class MinMaxQuantizer(nn.Module):
+    """Affine quantizer with min / max as trainable parameters."""
+
+    def __init__(self, shape, *args, **kwargs):
+        super().__init__()
+        if isinstance(shape, int):
+            shape = (shape,)
+        self.shape = tuple(shape)
+        # (qmin, qmax, symmetric[, encoding_analyzer[, block_size]]) or (bitwidth, symmetric[, encoding_analyzer[, block_size]])
+        args = list(args) + [None] * (5 - len(args))
+        arg0 = kwargs.pop('qmin', kwargs.pop('bitwidth', args[0]))
+        arg1 = kwargs.pop('qmax', args[1])
+        if arg1 is not None and not isinstance(arg1, bool):
+            qmin, qmax = arg0, arg1
+            symmetric = kwargs.pop('symmetric', args[2])
+            encoding_analyzer = kwargs.pop('encoding_analyzer', args[3])
+            block_size = kwargs.pop('block_size', args[4])
+            if qmin is None or qmax is None or symmetric is None:
+                raise TypeError("expected (shape, qmin, qmax, symmetric) or (shape, bitwidth, symmetric)")
+        else:
+            bitwidth = arg0
+            symmetric = kwargs.pop('symmetric', args[1])
+            if bitwidth is None or symmetric is None:
+                raise TypeError("expected (shape, qmin, qmax, symmetric) or (shape, bitwidth, symmetric)")
+            qmin, qmax = _derive_qmin_qmax(bitwidth=bitwidth, signed=symmetric)
+            encoding_analyzer = kwargs.pop('encoding_analyzer', args[2])
+            block_size = kwargs.pop('block_size', args[3])
+        if kwargs:
+            raise TypeError(f"{type(self).__qualname__}.__init__ got unexpected keyword argument: "
+                            f"{', '.join(kwargs)}")
+        if qmin >= qmax:
+            raise ValueError(f"qmax should be strictly larger than qmin. Got qmax={qmax}, qmin={qmin}")
+        if block_size is not None:
+            raise NotImplementedError("block_size is not implemented")
+        self.qmin, self.qmax = qmin, qmax
+        self._symmetric = symmetric
+        self.block_size = None
+        self.encoding_analyzer: EncodingAnalyzer = encoding_analyzer or MinMaxEncodingAnalyzer(self.shape)
+        if not _is_expandable(self.encoding_analyzer.observer.shape, self.shape):
+            raise RuntimeError(f'Encoding analyzer of shape {self.encoding_analyzer.observer.shape} '
+                               f'is incompatible with quantizer of shape {self.shape}.')
+        self.min = nn.Parameter(-torch.ones(self.shape))
+        self.max = nn.Parameter(torch.ones(self.shape))
+        self._initialized = False
+        self._allow_overwrite = True
+
+    # ---------------------------------------------------------------------------------------------- properties
+    @property
+    def symmetric(self) -> bool:
+        return self._symmetric
+
+    @symmetric.setter
+    def symmetric(self, symmetric: bool):
+        self._symmetric = symmetric
+
+    @property
+    def bitwidth(self) -> int:
+        return (self.qmax - self.qmin).bit_length()
+
+    @property
+    def signed(self) -> bool:
+        return self.qmin < 0
+
+    def is_initialized(self) -> bool:
+        return self._initialized
+
+    def __setattr__(self, name, value):
+        # assigning new min and max parameters by hand initialises the quantizer, as in the reference
+        if name in ('min', 'max') and '_initialized' in self.__dict__ and isinstance(value, nn.Parameter):
+            assigned = self.__dict__.setdefault('_assigned', set())
+            assigned.add(name)
+            if assigned >= {'min', 'max'}:
+                self.__dict__['_initialized'] = True
+        super().__setattr__(name, value)
+
+    def extra_repr(self) -> str:
+        return f'shape={self.shape}, qmin={self.qmin}, qmax={self.qmax}, symmetric={self.symmetric}'
+
+    # ------------------------------------------------------------------------------------------------ calibration
+    @contextlib.contextmanager
+    def compute_encodings(self):
+        """Observe inputs and set min / max from their statistics on exit; while inside, forward performs dynamic
+        quantization with the batch statistics (reference :317-374)."""
+        if not self._allow_overwrite:
+            yield
+            return
+        original_forward = self.forward
+
+        @functools.wraps(original_forward)
+        def forward_wrapper(input):  # pylint: disable=redefined-builtin
+            batch_statistics = self.encoding_analyzer.update_stats(input)
+            num_steps = self.qmax - self.qmin
+            dyn_min, dyn_max = self.encoding_analyzer.compute_encodings_from_stats(batch_statistics, num_steps,
+                                                                                   self.symmetric)
+            dyn_min = dyn_min.to(dtype=self.min.dtype, device=self.min.device).expand_as(self.min)
+            dyn_max = dyn_max.to(dtype=self.max.dtype, device=self.max.device).expand_as(self.max)
+            with patch_attr(self, 'min', dyn_min), patch_attr(self, 'max', dyn_max), \
+                    patch_attr(self, '_initialized', True):
+                return original_forward(input)
+
+        self.encoding_analyzer.reset_stats()
+        with patch_attr(self, 'forward', forward_wrapper):
+            yield
+        try:
+            num_steps = self.qmax - self.qmin
+            enc_min, enc_max = self.encoding_analyzer.compute_encodings(num_steps, self.symmetric)
+        except StatisticsNotFoundError:
+            return
+        if enc_min is None or enc_max is None:
+            return
+        self.set_range(enc_min, enc_max)
+
+    def set_range(self, min: torch.Tensor, max: torch.Tensor):  # pylint: disable=redefined-builtin
+        with torch.no_grad():
+            self.min.copy_(min)
+            self.max.copy_(max)
+        self._initialized = True
+
+    def get_scale(self, dtype=None) -> Optional[torch.Tensor]:
+        if not self.is_initialized():
+            return None
+        dtype = dtype or torch.float32
+        num_steps = self.qmax - self.qmin
+        return ((self.max.to(dtype) - self.min.to(dtype)) / num_steps).to(dtype)
+
+    def get_offset(self, dtype=None) -> Optional[torch.Tensor]:
+        if not self.is_initialized():
+            return None
+        dtype = dtype or torch.float32
+        if self.symmetric:
+            return torch.zeros_like(self.min, requires_grad=False, dtype=dtype)
+        return (ste_round(self.min.to(dtype) / self.get_scale(dtype)) - self.qmin).to(dtype)
+
+    def get_min(self, dtype=None) -> Optional[torch.Tensor]:
+        if not self.is_initialized():
+            return None
+        return self.get_scale(dtype) * (self.get_offset(dtype) + self.qmin)
+
+    def get_max(self, dtype=None) -> Optional[torch.Tensor]:
+        if not self.is_initialized():
+            return None
+        return self.get_scale(dtype) * (self.get_offset(dtype) + self.qmax)
+
+    def get_encoding(self) -> Optional[_AffineEncoding]:
+        if not self.is_initialized():
+            return None
+        return _AffineEncoding(self.get_scale(torch.float32), self.get_offset(torch.float32), self.qmin, self.qmax,
+                               self._symmetric, self.block_size)
+
+    @torch.no_grad()
+    def get_legacy_encodings(self):
+        if not self.is_initialized():
+            return None
+        enc = self.get_encoding()
+        mn, mx = enc.min.flatten().tolist(), enc.max.flatten().tolist()
+        sc, of = enc.scale.flatten().tolist(), enc.offset.flatten().tolist()
+        return [{'min': a, 'max': b, 'scale': s, 'offset': int(o), 'bitwidth': self.bitwidth, 'dtype': 'int',
+                 'is_symmetric': str(self.symmetric)} for a, b, s, o in zip(mn, mx, sc, of)]
+
+    @torch.no_grad()
+    def set_legacy_encodings(self, encodings):
+        bitwidth = encodings[0]['bitwidth']
+        symmetric = encodings[0]['is_symmetric'].lower() == 'true'
+        self.qmin, self.qmax = _derive_qmin_qmax(bitwidth=bitwidth, signed=symmetric)
+        self.symmetric = symmetric
+        dev = self.min.device
+        self.set_range(torch.tensor([e['min'] for e in encodings]).view(self.shape).to(dev),
+                       torch.tensor([e['max'] for e in encodings]).view(self.shape).to(dev))
+
+
+class Quantize(MinMaxQuantizer):
+    """out = clamp(round(input / scale) - offset, qmin, qmax)"""
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:  # pylint: disable=redefined-builtin
+        if not self.is_initialized():
+            raise RuntimeError('Failed to run Quantize since quantization parameters are not initialized.'
+                               ' Please initialize the quantization parameters using `compute_encodings()`.')
+        encoding = self.get_encoding()
+        return quantize(input, encoding.scale, encoding.offset, encoding.qmin, encoding.qmax)
+
+
+class QuantizeDequantize(MinMaxQuantizer):
+    """out = (clamp(round(input / scale) - offset, qmin, qmax) + offset) * scale"""
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:  # pylint: disable=redefined-builtin
+        if not self.is_initialized():
+            raise RuntimeError('Failed to run QuantizeDequantize since quantization parameters are not initialized.'
+                               ' Please initialize the quantization parameters using `compute_encodings()`.')
+        encoding = self.get_encoding()
+        return quantize_dequantize(input, encoding.scale, encoding.offset, encoding.qmin, encoding.qmax)
