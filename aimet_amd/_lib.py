@@ -63,6 +63,12 @@ _SIGNATURES = {
     "miq_analyzer_get_stats_histogram": ([_p, _p, _p, C.POINTER(_int), _p], _int),
     "miq_analyzer_last_batch_counts": ([_p, _p, _p], _int),
     "miq_analyzer_last_search": ([_p, _p, _p, _p, _int, C.POINTER(_int), C.POINTER(_int), _p], _int),
+    "miq_adaround_soft_round_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int, _p], _int),
+    "miq_adaround_init_alpha_f32": ([_p, _p, _i64, _i64, _i64, _p, _p], _int),
+    "miq_adaround_bwd_adam_f32": ([_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _flt, _flt, _flt,
+                                   _flt, _flt, _flt, _int, _p, _p], _int),
+    "miq_adaround_bwd_f32": ([_p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _flt, _flt, _p, _p], _int),
+    "miq_adaround_blocks": ([_i64], _int),
 }
 
 # Entry points declared in include/miq.h; the loader insists on every one of them.

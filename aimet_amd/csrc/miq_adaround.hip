@@ -1,0 +1,372 @@
+// AdaRound kernels for gfx950: soft/hard rounding forward, and the fused backward that turns dL/dW' into the Adam
+// update of alpha (rectified-sigmoid chain rule + rounding regulariser gradient + Adam step in one pass).
+//
+// Reference arithmetic (paths relative to the reference root,
+// ADA = TrainingExtensions/torch/src/python/aimet_torch/v1/adaround):
+//   apply_adaround              ADA/adaround_wrapper.py:124-149
+//   _generate_alpha_parameter   ADA/adaround_wrapper.py:211-224
+//   compute_round_loss          ADA/adaround_loss.py:82-111
+//   optimiser step              torch.optim.Adam (single-tensor form), ADA/adaround_optimizer.py:157-218
+//   constants zeta = 1.1, gamma = -0.1   TrainingExtensions/common/src/python/aimet_common/defs.py:302-306
+//
+// The reference runs about fifteen elementwise ATen kernels per iteration over weight-shaped tensors plus their
+// autograd twins; here the forward is one pass (read W, alpha; write W') and the backward one pass (read dW', W,
+// alpha, m, v; write alpha, m, v).
+#include "miq_common.h"
+
+#include <cmath>
+
+namespace miq
+{
+namespace
+{
+constexpr float kZetaMinusGamma = 1.2f;   // float32(1.1 - (-0.1)) = float32(1.2000000000000002)
+constexpr float kGamma          = -0.1f;
+
+struct AdaGeom
+{
+    int64_t n;
+    uint32_t num_channel;
+    FastDiv fd;          // elements per channel
+    const float* delta;  // [num_channel]
+    const float* offset; // [num_channel]
+    float clip_min, clip_max;
+};
+
+__device__ __forceinline__ uint32_t channel_of(int64_t e, const AdaGeom& g)
+{
+    // e < 2^31 on this path (checked by the host)
+    return fastdiv((uint32_t) e, g.fd) % g.num_channel;
+}
+
+__device__ __forceinline__ float sigmoidf_(float a)
+{
+    return 1.0f / (1.0f + expf(-a));
+}
+
+// h(alpha) and, optionally, the pieces the backward needs
+__device__ __forceinline__ float soft_h(float alpha, float& sig, float& inner)
+{
+    sig   = sigmoidf_(alpha);
+    inner = sig * kZetaMinusGamma + kGamma;
+    return fminf(fmaxf(inner, 0.0f), 1.0f);
+}
+
+template <bool SOFT>
+__global__ __launch_bounds__(kBlock) void soft_round_kernel(const float* __restrict__ w, const float* __restrict__ alpha,
+                                                            float* __restrict__ out, AdaGeom g)
+{
+    const int64_t nvec = g.n / 4;
+    const int64_t v    = (int64_t) blockIdx.x * kBlock + threadIdx.x;
+    if (v < nvec)
+    {
+        const float4 wv = reinterpret_cast<const float4*>(w)[v];
+        const float4 av = reinterpret_cast<const float4*>(alpha)[v];
+        const float ws[4] = {wv.x, wv.y, wv.z, wv.w};
+        const float as[4] = {av.x, av.y, av.z, av.w};
+        float ys[4];
+        const uint32_t c0 = channel_of(v * 4, g), c3 = channel_of(v * 4 + 3, g);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            const uint32_t c = (c0 == c3) ? c0 : channel_of(v * 4 + j, g);
+            const float d = g.delta[c], o = g.offset[c];
+            const float f = floorf(ws[j] / d);
+            float sig, inner;
+            const float h = SOFT ? soft_h(as[j], sig, inner) : (as[j] >= 0.0f ? 1.0f : 0.0f);
+            const float t = f + h;
+            const float q = fminf(fmaxf(t - o, g.clip_min), g.clip_max);
+            ys[j]         = (q + o) * d;
+        }
+        reinterpret_cast<float4*>(out)[v] = make_float4(ys[0], ys[1], ys[2], ys[3]);
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (g.n - nvec * 4))
+    {
+        const int64_t e  = nvec * 4 + threadIdx.x;
+        const uint32_t c = channel_of(e, g);
+        const float d = g.delta[c], o = g.offset[c];
+        const float f = floorf(w[e] / d);
+        float sig, inner;
+        const float h = SOFT ? soft_h(alpha[e], sig, inner) : (alpha[e] >= 0.0f ? 1.0f : 0.0f);
+        const float q = fminf(fmaxf(f + h - o, g.clip_min), g.clip_max);
+        out[e]        = (q + o) * d;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void init_alpha_kernel(const float* __restrict__ w, float* __restrict__ alpha,
+                                                            AdaGeom g)
+{
+    for (int64_t e = (int64_t) blockIdx.x * kBlock + threadIdx.x; e < g.n; e += (int64_t) gridDim.x * kBlock)
+    {
+        const float d    = g.delta[channel_of(e, g)];
+        const float s    = w[e] / d;
+        const float frac = s - floorf(s);
+        // alpha = -log((zeta - gamma) / (frac - gamma) - 1)
+        alpha[e] = -logf(kZetaMinusGamma / (frac - kGamma) - 1.0f);
+    }
+}
+
+struct AdamArgs
+{
+    float reg_param;
+    float beta;        // exponent of the regulariser; < 0 during warm start (no rounding loss)
+    float lr_over_bc1; // lr / (1 - beta1^t)
+    float bc2_sqrt;    // sqrt(1 - beta2^t)
+    float beta1, beta2, eps;
+};
+
+// dLoss/dalpha of one element: chain rule of apply_adaround (closed-interval clamp gradients, as torch.clamp) plus the
+// gradient of reg_param * (1 - |2h - 1|^beta); `reg` receives this element's regulariser term (0 in warm start)
+__device__ __forceinline__ float alpha_grad(float w, float gw, float alpha, float d, float o, const AdaGeom& g,
+                                            const AdamArgs& a, float& reg)
+{
+    const float f = floorf(w / d);
+    float sig, inner;
+    const float h      = soft_h(alpha, sig, inner);
+    const float t      = f + h - o;
+    const float pass_q = (t >= g.clip_min && t <= g.clip_max) ? 1.0f : 0.0f;
+    const float pass_h = (inner >= 0.0f && inner <= 1.0f) ? 1.0f : 0.0f;
+    const float dsig   = (1.0f - sig) * sig;
+    const float dh     = pass_h * kZetaMinusGamma * dsig;
+    float grad         = gw * d * pass_q * dh;
+    reg                = 0.0f;
+    if (a.beta >= 0.0f)
+    {
+        const float x   = 2.0f * h - 1.0f;
+        const float ax  = fabsf(x);
+        reg             = 1.0f - powf(ax, a.beta);
+        const float sgn = (x > 0.0f) ? 1.0f : ((x < 0.0f) ? -1.0f : 0.0f);
+        const float dp  = (ax > 0.0f) ? a.beta * powf(ax, a.beta - 1.0f) : 0.0f;
+        grad += -a.reg_param * dp * sgn * 2.0f * dh;
+    }
+    return grad;
+}
+
+// Adam (torch single-tensor form): lerp for the first moment, mul/addcmul for the second
+__device__ __forceinline__ void adam_update(float grad, float& alpha, float& m, float& v, const AdamArgs& a)
+{
+    m = m + (1.0f - a.beta1) * (grad - m);
+    v = v * a.beta2 + (1.0f - a.beta2) * grad * grad;
+    const float denom = sqrtf(v) / a.bc2_sqrt + a.eps;
+    alpha             = alpha - a.lr_over_bc1 * (m / denom);
+}
+
+// ADAM = true : alpha, m, v updated in place; grad_out (optional) receives dLoss/dalpha
+// ADAM = false: grad_out receives dLoss/dalpha; alpha, m, v untouched (m, v may be null)
+template <bool ADAM>
+__global__ __launch_bounds__(kBlock) void bwd_kernel(const float* __restrict__ w, const float* __restrict__ gw,
+                                                     float* __restrict__ alpha, float* __restrict__ m,
+                                                     float* __restrict__ v, float* __restrict__ grad_out, AdaGeom g,
+                                                     AdamArgs a, float* __restrict__ reg_partial)
+{
+    const int64_t nvec = g.n / 4;
+    const int64_t i    = (int64_t) blockIdx.x * kBlock + threadIdx.x;
+    float reg          = 0.0f;
+    if (i < nvec)
+    {
+        const float4 wv = reinterpret_cast<const float4*>(w)[i];
+        const float4 gv = reinterpret_cast<const float4*>(gw)[i];
+        const float4 av = reinterpret_cast<const float4*>(alpha)[i];
+        float4 mv = make_float4(0, 0, 0, 0), vv = mv;
+        if (ADAM)
+        {
+            mv = reinterpret_cast<const float4*>(m)[i];
+            vv = reinterpret_cast<const float4*>(v)[i];
+        }
+        const uint32_t c0 = channel_of(i * 4, g), c3 = channel_of(i * 4 + 3, g);
+        const float ws[4] = {wv.x, wv.y, wv.z, wv.w};
+        const float gs[4] = {gv.x, gv.y, gv.z, gv.w};
+        float as[4] = {av.x, av.y, av.z, av.w}, ms[4] = {mv.x, mv.y, mv.z, mv.w}, vs[4] = {vv.x, vv.y, vv.z, vv.w};
+        float gr[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+        {
+            const uint32_t c = (c0 == c3) ? c0 : channel_of(i * 4 + j, g);
+            float r;
+            gr[j] = alpha_grad(ws[j], gs[j], as[j], g.delta[c], g.offset[c], g, a, r);
+            reg += r;
+            if (ADAM)
+                adam_update(gr[j], as[j], ms[j], vs[j], a);
+        }
+        if (ADAM)
+        {
+            reinterpret_cast<float4*>(alpha)[i] = make_float4(as[0], as[1], as[2], as[3]);
+            reinterpret_cast<float4*>(m)[i]     = make_float4(ms[0], ms[1], ms[2], ms[3]);
+            reinterpret_cast<float4*>(v)[i]     = make_float4(vs[0], vs[1], vs[2], vs[3]);
+        }
+        if (grad_out)
+            reinterpret_cast<float4*>(grad_out)[i] = make_float4(gr[0], gr[1], gr[2], gr[3]);
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (g.n - nvec * 4))
+    {
+        const int64_t e  = nvec * 4 + threadIdx.x;
+        const uint32_t c = channel_of(e, g);
+        float r;
+        const float gr = alpha_grad(w[e], gw[e], alpha[e], g.delta[c], g.offset[c], g, a, r);
+        reg += r;
+        if (ADAM)
+            adam_update(gr, alpha[e], m[e], v[e], a);
+        if (grad_out)
+            grad_out[e] = gr;
+    }
+    if (reg_partial)
+    {
+        // per-workgroup partial of the regulariser sum, combined in a fixed order by the caller (deterministic)
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1)
+            reg += __shfl_xor(reg, o);
+        __shared__ float s[kBlock / 64];
+        if ((threadIdx.x & 63) == 0)
+            s[threadIdx.x >> 6] = reg;
+        __syncthreads();
+        if (threadIdx.x == 0)
+        {
+            float t = 0;
+            for (int k = 0; k < kBlock / 64; ++k)
+                t += s[k];
+            reg_partial[blockIdx.x] = t;
+        }
+    }
+}
+
+int make_geom(AdaGeom& g, int64_t num_channel, int64_t num_element, int64_t n_per_channel, const float* delta,
+              const float* offset, float clip_min, float clip_max)
+{
+    MIQ_CHECK_ARG(num_channel > 0 && n_per_channel > 0 && num_element >= 0, "bad channel geometry");
+    MIQ_CHECK_ARG(num_element < (1ll << 31) && n_per_channel < (1ll << 31) && num_channel < (1ll << 31),
+                  "AdaRound kernels take tensors of fewer than 2^31 elements");
+    MIQ_CHECK_ARG(delta && offset, "null delta/offset");
+    MIQ_CHECK_ARG(clip_min <= clip_max, "clip_min must not exceed clip_max");
+    g.n           = num_element;
+    g.num_channel = (uint32_t) num_channel;
+    g.fd          = make_fastdiv((uint32_t) n_per_channel);
+    g.delta       = delta;
+    g.offset      = offset;
+    g.clip_min    = clip_min;
+    g.clip_max    = clip_max;
+    return MIQ_OK;
+}
+
+int make_adam(AdamArgs& a, float reg_param, float beta, float lr, float beta1, float beta2, float eps, int step)
+{
+    MIQ_CHECK_ARG(beta1 >= 0.f && beta1 < 1.f && beta2 >= 0.f && beta2 < 1.f, "Adam betas must lie in [0, 1)");
+    a.reg_param = reg_param;
+    a.beta      = beta;
+    // bias corrections in double, as the Python floats of torch.optim.Adam are
+    const double bc1 = 1.0 - std::pow((double) beta1, (double) step);
+    const double bc2 = 1.0 - std::pow((double) beta2, (double) step);
+    a.lr_over_bc1    = (float) ((double) lr / bc1);
+    a.bc2_sqrt       = (float) std::sqrt(bc2);
+    a.beta1          = beta1;
+    a.beta2          = beta2;
+    a.eps            = eps;
+    return MIQ_OK;
+}
+
+inline unsigned vec_blocks(int64_t n)
+{
+    int64_t nvec = n / 4;
+    int64_t b    = (nvec + kBlock - 1) / kBlock;
+    return (unsigned) (b < 1 ? 1 : b);
+}
+}   // namespace
+}   // namespace miq
+
+using namespace miq;
+
+extern "C" {
+
+int miq_adaround_blocks(int64_t num_element)
+{
+    return (int) vec_blocks(num_element);
+}
+
+int miq_adaround_soft_round_f32(const float* weight, const float* alpha, float* out, int64_t num_channel,
+                                int64_t num_element, int64_t num_element_per_channel, const float* delta,
+                                const float* offset, float clip_min, float clip_max, int use_soft_rounding,
+                                void* stream)
+{
+    AdaGeom g;
+    if (int rc = make_geom(g, num_channel, num_element, num_element_per_channel, delta, offset, clip_min, clip_max))
+        return rc;
+    if (num_element == 0)
+        return MIQ_OK;
+    MIQ_CHECK_ARG(weight && alpha && out, "null tensor pointer");
+    MIQ_CHECK_ARG(aligned16(weight) && aligned16(alpha) && aligned16(out), "tensors must be 16-byte aligned");
+    if (use_soft_rounding)
+        hipLaunchKernelGGL(soft_round_kernel<true>, dim3(vec_blocks(num_element)), dim3(kBlock), 0,
+                           (hipStream_t) stream, weight, alpha, out, g);
+    else
+        hipLaunchKernelGGL(soft_round_kernel<false>, dim3(vec_blocks(num_element)), dim3(kBlock), 0,
+                           (hipStream_t) stream, weight, alpha, out, g);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int miq_adaround_init_alpha_f32(const float* weight, float* alpha, int64_t num_channel, int64_t num_element,
+                                int64_t num_element_per_channel, const float* delta, void* stream)
+{
+    AdaGeom g;
+    if (int rc = make_geom(g, num_channel, num_element, num_element_per_channel, delta, delta, 0.f, 0.f))
+        return rc;
+    if (num_element == 0)
+        return MIQ_OK;
+    MIQ_CHECK_ARG(weight && alpha, "null tensor pointer");
+    int64_t blocks = (num_element + kBlock - 1) / kBlock;
+    if (blocks > 65536)
+        blocks = 65536;
+    hipLaunchKernelGGL(init_alpha_kernel, dim3((unsigned) blocks), dim3(kBlock), 0, (hipStream_t) stream, weight, alpha,
+                       g);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int miq_adaround_bwd_f32(const float* weight, const float* grad_weight, const float* alpha, float* grad_alpha,
+                         int64_t num_channel, int64_t num_element, int64_t num_element_per_channel,
+                         const float* delta, const float* offset, float clip_min, float clip_max, float reg_param,
+                         float beta, float* reg_partial, void* stream)
+{
+    AdaGeom g;
+    if (int rc = make_geom(g, num_channel, num_element, num_element_per_channel, delta, offset, clip_min, clip_max))
+        return rc;
+    if (num_element == 0)
+        return MIQ_OK;
+    MIQ_CHECK_ARG(weight && grad_weight && alpha && grad_alpha, "null tensor pointer");
+    MIQ_CHECK_ARG(aligned16(weight) && aligned16(grad_weight) && aligned16(alpha) && aligned16(grad_alpha),
+                  "tensors must be 16-byte aligned");
+    AdamArgs a    = {};
+    a.reg_param   = reg_param;
+    a.beta        = beta;
+    hipLaunchKernelGGL(bwd_kernel<false>, dim3(vec_blocks(num_element)), dim3(kBlock), 0, (hipStream_t) stream, weight,
+                       grad_weight, const_cast<float*>(alpha), (float*) nullptr, (float*) nullptr, grad_alpha, g, a,
+                       reg_partial);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int miq_adaround_bwd_adam_f32(const float* weight, const float* grad_weight, float* alpha, float* exp_avg,
+                              float* exp_avg_sq, float* grad_alpha, int64_t num_channel, int64_t num_element,
+                              int64_t num_element_per_channel, const float* delta, const float* offset, float clip_min,
+                              float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
+                              float eps, int step, float* reg_partial, void* stream)
+{
+    AdaGeom g;
+    if (int rc = make_geom(g, num_channel, num_element, num_element_per_channel, delta, offset, clip_min, clip_max))
+        return rc;
+    if (num_element == 0)
+        return MIQ_OK;
+    MIQ_CHECK_ARG(weight && grad_weight && alpha && exp_avg && exp_avg_sq, "null tensor pointer");
+    MIQ_CHECK_ARG(aligned16(weight) && aligned16(grad_weight) && aligned16(alpha) && aligned16(exp_avg) &&
+                      aligned16(exp_avg_sq) && aligned16(grad_alpha),
+                  "tensors must be 16-byte aligned");
+    MIQ_CHECK_ARG(step >= 1, "Adam step count starts at 1");
+    AdamArgs a;
+    if (int rc = make_adam(a, reg_param, beta, lr, beta1, beta2, eps, step))
+        return rc;
+    hipLaunchKernelGGL(bwd_kernel<true>, dim3(vec_blocks(num_element)), dim3(kBlock), 0, (hipStream_t) stream, weight,
+                       grad_weight, alpha, exp_avg, exp_avg_sq, grad_alpha, g, a, reg_partial);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+}   // extern "C"

@@ -222,6 +222,70 @@ def minmax_per_channel(x, num_channel, n_per_channel):
     return out
 
 
+# ----------------------------------------------------------------------------------------------------------- AdaRound
+def _ada_check(weight, *others):
+    _require_gpu(weight, *others)
+    for t in (weight,) + others:
+        if t is None:
+            continue
+        if t.dtype != _F32 or not t.is_contiguous():
+            raise RuntimeError("AdaRound kernels take contiguous float32 tensors")
+
+
+def adaround_soft_round(weight, alpha, num_channel, n_per_channel, delta, offset, clip_min, clip_max,
+                        use_soft_rounding=True, out=None):
+    """(clamp(floor(w / delta) + h(alpha) - offset, clip_min, clip_max) + offset) * delta."""
+    _ada_check(weight, alpha, out)
+    out = torch.empty_like(weight) if out is None else out
+    with torch.cuda.device(weight.device):
+        check(lib.miq_adaround_soft_round_f32(_ptr(weight), _ptr(alpha), _ptr(out), int(num_channel), weight.numel(),
+                                              int(n_per_channel), _ptr(delta), _ptr(offset), float(clip_min),
+                                              float(clip_max), int(bool(use_soft_rounding)), _stream(weight)))
+    return out
+
+
+def adaround_init_alpha(weight, num_channel, n_per_channel, delta):
+    """alpha such that h(alpha) equals the fractional part of w / delta."""
+    _ada_check(weight)
+    alpha = torch.empty_like(weight)
+    with torch.cuda.device(weight.device):
+        check(lib.miq_adaround_init_alpha_f32(_ptr(weight), _ptr(alpha), int(num_channel), weight.numel(),
+                                              int(n_per_channel), _ptr(delta), _stream(weight)))
+    return alpha
+
+
+def adaround_blocks(num_element):
+    return int(lib.miq_adaround_blocks(int(num_element)))
+
+
+def adaround_bwd(weight, grad_weight, alpha, num_channel, n_per_channel, delta, offset, clip_min, clip_max,
+                 reg_param=0.0, beta=-1.0, reg_partial=None):
+    """dLoss/dW' -> dLoss/dalpha (rounding regulariser included when beta >= 0); returns the gradient."""
+    _ada_check(weight, grad_weight, alpha)
+    grad_alpha = torch.empty_like(alpha)
+    with torch.cuda.device(weight.device):
+        check(lib.miq_adaround_bwd_f32(_ptr(weight), _ptr(grad_weight), _ptr(alpha), _ptr(grad_alpha),
+                                       int(num_channel), weight.numel(), int(n_per_channel), _ptr(delta),
+                                       _ptr(offset), float(clip_min), float(clip_max), float(reg_param), float(beta),
+                                       _ptr(reg_partial), _stream(weight)))
+    return grad_alpha
+
+
+def adaround_bwd_adam(weight, grad_weight, alpha, exp_avg, exp_avg_sq, num_channel, n_per_channel, delta, offset,
+                      clip_min, clip_max, reg_param, beta, lr, beta1, beta2, eps, step, reg_partial=None,
+                      grad_alpha=None):
+    """dLoss/dW' -> Adam update of alpha (in place), rounding regulariser included when beta >= 0."""
+    _ada_check(weight, grad_weight, alpha, exp_avg, exp_avg_sq)
+    if reg_partial is not None and reg_partial.numel() < adaround_blocks(weight.numel()):
+        raise RuntimeError("reg_partial is too small")
+    with torch.cuda.device(weight.device):
+        check(lib.miq_adaround_bwd_adam_f32(_ptr(weight), _ptr(grad_weight), _ptr(alpha), _ptr(exp_avg),
+                                            _ptr(exp_avg_sq), _ptr(grad_alpha), int(num_channel), weight.numel(), int(n_per_channel),
+                                            _ptr(delta), _ptr(offset), float(clip_min), float(clip_max),
+                                            float(reg_param), float(beta), float(lr), float(beta1), float(beta2),
+                                            float(eps), int(step), _ptr(reg_partial), _stream(weight)))
+
+
 class Analyzer:
     """Device-resident encoding analyzer (TF min/max or TF-Enhanced 512-bucket PDF + SQNR search)."""
 

@@ -1,0 +1,144 @@
+"""Per-layer optimisation of the weight rounding.
+
+Mirrors AdaroundOptimizer of TrainingExtensions/torch/src/python/aimet_torch/v1/adaround/adaround_optimizer.py
+(adaround_module :66-113, _optimize_rounding :115-222, _compute_recons_metrics :224-251,
+_compute_output_with_adarounded_weights :253-283).  Per iteration the reference runs apply_adaround's elementwise ops,
+the layer, both losses, autograd through all of it and torch.optim.Adam -- some forty kernels over weight-shaped
+tensors.  Here an iteration is: one soft-rounding kernel (W, alpha -> W'), the layer forward and its weight gradient
+(torch, on W' as a leaf), and one fused kernel (dW', W, alpha, moments -> alpha, moments) that applies the chain rule
+of the soft rounding, adds the rounding regulariser's gradient and performs the Adam update.  The batch indices are
+drawn with torch.randperm on the host exactly as the reference draws them, so a seeded run visits the same batches.
+"""
+from typing import Any, Callable, Tuple, Union
+
+import torch
+import torch.nn.functional as functional
+
+from ... import ops, utils
+from .activation_sampler import ActivationSampler
+from .adaround_loss import AdaroundHyperParameters, AdaroundLoss
+from .adaround_wrapper import AdaroundWrapper
+
+BATCH_SIZE = 32
+ADAM_LR, ADAM_BETAS, ADAM_EPS = 1e-3, (0.9, 0.999), 1e-8      # torch.optim.Adam defaults, as the reference uses
+
+
+class AdaroundOptimizer:
+    """Optimizes the weight rounding of a quantized wrapper module."""
+
+    @classmethod
+    def adaround_module(cls, module: torch.nn.Module, quant_module: AdaroundWrapper, orig_model: torch.nn.Module,
+                        quant_model: torch.nn.Module, act_func: Union[torch.nn.Module, None], cached_dataset,
+                        forward_fn: Callable[[torch.nn.Module, Any], Any], opt_params: AdaroundHyperParameters,
+                        cached_quant_dataset=None):
+        # pylint: disable=too-many-arguments
+        assert isinstance(quant_module, AdaroundWrapper), '%s is not adaround wrapper module.' % quant_module
+        cls._optimize_rounding(module, quant_module, orig_model, quant_model, act_func, cached_dataset, forward_fn,
+                               opt_params, cached_quant_dataset)
+        # after optimisation the layer uses hard rounding
+        quant_module.use_soft_rounding = False
+
+    @classmethod
+    def _optimize_rounding(cls, module: torch.nn.Module, quant_module: AdaroundWrapper, orig_model: torch.nn.Module,
+                           quant_model: torch.nn.Module, act_func: Union[torch.nn.Module, None], cached_dataset,
+                           forward_fn: Callable[[torch.nn.Module, Any], Any], opt_params: AdaroundHyperParameters,
+                           cached_quant_dataset=None):
+        # pylint: disable=too-many-arguments, too-many-locals
+        assert isinstance(quant_module, AdaroundWrapper), '%s is not adaround wrapper module.' % quant_module
+        assert quant_module.use_soft_rounding, 'optimization should use soft rounding only.'
+        assert quant_module.alpha is not None, 'alpha parameter should be initialized.'
+
+        act_sampler = ActivationSampler(module, quant_module, orig_model, quant_model, forward_fn)
+        all_inp_data, all_orig_out_data = act_sampler.sample_all_acts(cached_dataset, cached_quant_dataset)
+        cls.optimize_rounding_on_cached_acts(quant_module, act_func, all_inp_data, all_orig_out_data, opt_params)
+
+    @classmethod
+    def optimize_rounding_on_cached_acts(cls, quant_module: AdaroundWrapper, act_func, all_inp_data: torch.Tensor,
+                                         all_orig_out_data: torch.Tensor, opt_params: AdaroundHyperParameters,
+                                         batches=None, first_iteration: int = 0):
+        """The iteration loop over activations that are already resident on the GPU.
+
+        `batches`: optional iterable of index tensors, one per iteration; by default opt_params.num_iterations batches
+        of torch.randperm(N)[:BATCH_SIZE] drawn from torch's global host generator.
+        Returns the Adam state (exp_avg, exp_avg_sq); alpha is updated in place and alpha.grad holds the last gradient.
+        """
+        # pylint: disable=too-many-arguments, too-many-locals
+        qm = quant_module
+        device = all_inp_data.device
+        weight = qm.weight.detach().to(torch.float32).contiguous()
+        alpha = qm.alpha.data
+        exp_avg = torch.zeros_like(alpha)
+        exp_avg_sq = torch.zeros_like(alpha)
+        grad_alpha = torch.empty_like(alpha)
+        if batches is None:
+            n = all_inp_data.size(0)
+            batches = (torch.randperm(n)[:BATCH_SIZE] for _ in range(opt_params.num_iterations))
+
+        step = 0
+        for k, indices in enumerate(batches):
+            iteration = first_iteration + k
+            indices = indices.to(device)
+            inp_data = all_inp_data[indices]
+            orig_out_data = all_orig_out_data[indices]
+
+            ada_weight = ops.adaround_soft_round(weight, alpha, qm.num_channel, qm.n_per_channel, qm.delta, qm.offset,
+                                                 qm.clip_min, qm.clip_max, True)
+            ada_weight.requires_grad_(True)
+            quant_out_data = cls._layer_output(qm.get_original_module(), inp_data, ada_weight)
+            if act_func is not None:
+                orig_out_data = act_func(orig_out_data)
+                quant_out_data = act_func(quant_out_data)
+            recon_loss = AdaroundLoss.compute_recon_loss(quant_out_data, orig_out_data)
+            grad_weight, = torch.autograd.grad(recon_loss, ada_weight)
+
+            if AdaroundLoss.in_warm_start(opt_params, iteration):
+                beta = -1.0
+            else:
+                beta = AdaroundLoss._compute_beta(opt_params.num_iterations, iteration,  # pylint: disable=protected-access
+                                                  opt_params.beta_range, opt_params.warm_start)
+            step += 1
+            ops.adaround_bwd_adam(weight, grad_weight.contiguous(), alpha, exp_avg, exp_avg_sq, qm.num_channel,
+                                  qm.n_per_channel, qm.delta, qm.offset, qm.clip_min, qm.clip_max,
+                                  opt_params.reg_param, beta, ADAM_LR, ADAM_BETAS[0], ADAM_BETAS[1], ADAM_EPS, step,
+                                  grad_alpha=grad_alpha)
+        if step:
+            qm.alpha.grad = grad_alpha
+        return exp_avg, exp_avg_sq
+
+    @classmethod
+    def _compute_recons_metrics(cls, quant_module: AdaroundWrapper, act_func, inp_data: torch.Tensor,
+                                out_data: torch.Tensor) -> Tuple[float, float]:
+        """MSE of the layer output under hard and under soft rounding: (recons_err_hard, recons_err_soft)."""
+        with torch.no_grad():
+            quant_module.use_soft_rounding = False
+            out_data_hard = cls._compute_output_with_adarounded_weights(quant_module, inp_data)
+            quant_module.use_soft_rounding = True
+            out_data_soft = cls._compute_output_with_adarounded_weights(quant_module, inp_data)
+            if act_func is not None:
+                out_data = act_func(out_data)
+                out_data_soft = act_func(out_data_soft)
+                out_data_hard = act_func(out_data_hard)
+            recons_err_soft = functional.mse_loss(out_data_soft, out_data)
+            recons_err_hard = functional.mse_loss(out_data_hard, out_data)
+        return float(recons_err_hard), float(recons_err_soft)
+
+    @staticmethod
+    def _layer_output(module: torch.nn.Module, inp_data: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+        if isinstance(module, torch.nn.Conv2d):
+            return functional.conv2d(inp_data, weight, bias=module.bias, stride=module.stride,
+                                     dilation=module.dilation, padding=module.padding, groups=module.groups)
+        if isinstance(module, torch.nn.ConvTranspose2d):
+            return functional.conv_transpose2d(inp_data, weight, bias=module.bias, stride=module.stride,
+                                               padding=module.padding, output_padding=module.output_padding,
+                                               groups=module.groups, dilation=module.dilation)
+        if isinstance(module, torch.nn.Linear):
+            return functional.linear(inp_data, weight, bias=module.bias)
+        raise ValueError('AdaRound is not supported for the module: ', module)
+
+    @classmethod
+    def _compute_output_with_adarounded_weights(cls, quant_module: AdaroundWrapper, inp_data: torch.Tensor):
+        """Output of the wrapped Conv2d / ConvTranspose2d / Linear computed with the adarounded weight."""
+        module = quant_module.get_original_module()
+        quant_module.to(inp_data.device)
+        adarounded_weights = quant_module.apply_adaround(quant_module.weight)
+        return cls._layer_output(module, inp_data, adarounded_weights)

@@ -271,6 +271,24 @@ class QuantizationSimModel:
             layer.compute_encoding()
             layer.set_mode(QcQuantizeOpMode.ACTIVE)
 
+    def exclude_layers_from_quantization(self, layers_to_exclude: List[nn.Module]):
+        """Replaces the given quantization wrappers by the modules they wrap (reference quantsim.py:1419-1433)."""
+        self._replace_wrappers(self.model, set(layers_to_exclude))
+
+    @classmethod
+    def _replace_wrappers(cls, module: nn.Module, only=None):
+        for name, child in list(module.named_children()):
+            if isinstance(child, QcQuantizeWrapper):
+                if only is None or child in only:
+                    setattr(module, name, child.get_original_module())
+            else:
+                cls._replace_wrappers(child, only)
+
+    @classmethod
+    def remove_quantization_wrappers(cls, module: nn.Module):
+        """Strips every quantization wrapper below `module` (reference SaveUtils.remove_quantization_wrappers)."""
+        cls._replace_wrappers(module, None)
+
     # ------------------------------------------------------------------------------------ encodings on disk
     @staticmethod
     def _encoding_dict(enc, symmetric: bool) -> dict:

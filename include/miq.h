@@ -198,6 +198,51 @@ int miq_analyzer_last_search(miq_analyzer* a, float* deltas /* host */, int32_t*
                              double* costs /* host */, int cap, int* count /* host */, int* best_index /* host */,
                              void* stream);
 
+/* ---------------------------------------------------------------------------------------------------------------
+ * AdaRound (ADA = TrainingExtensions/torch/src/python/aimet_torch/v1/adaround)
+ *
+ * All tensors are float32 in device memory; channel(i) = (i / num_element_per_channel) % num_channel selects the
+ * entry of the device vectors delta / offset (one entry for a per-tensor encoding).  clip_min / clip_max are the
+ * integer grid limits of AdaroundWrapper.apply_adaround (0 and 2^bw - 1, or -2^(bw-1) and 2^(bw-1) - 1 for the
+ * signed-symmetric grid).  Tensors of at most 2^31 - 1 elements.
+ * ------------------------------------------------------------------------------------------------------------- */
+
+/* AdaroundWrapper.apply_adaround (ADA/adaround_wrapper.py:124-149):
+ *   out = (clamp(floor(w / delta) + h(alpha) - offset, clip_min, clip_max) + offset) * delta
+ * with h = clamp(sigmoid(alpha) * (zeta - gamma) + gamma, 0, 1) when use_soft_rounding != 0 and h = (alpha >= 0)
+ * otherwise; zeta = 1.1, gamma = -0.1 (aimet_common/defs.py:302-306). */
+int miq_adaround_soft_round_f32(const float* weight, const float* alpha, float* out, int64_t num_channel,
+                                int64_t num_element, int64_t num_element_per_channel, const float* delta,
+                                const float* offset, float clip_min, float clip_max, int use_soft_rounding,
+                                void* stream);
+/* AdaroundWrapper._generate_alpha_parameter (ADA/adaround_wrapper.py:211-224):
+ *   alpha = -log((zeta - gamma) / (w / delta - floor(w / delta) - gamma) - 1) */
+int miq_adaround_init_alpha_f32(const float* weight, float* alpha, int64_t num_channel, int64_t num_element,
+                                int64_t num_element_per_channel, const float* delta, void* stream);
+/* One optimiser iteration's elementwise tail, fused (AdaroundOptimizer._optimize_rounding's loss.backward() +
+ * optimizer.step(), ADA/adaround_optimizer.py:190-218, for the part below the layer's own backward):
+ * given grad_weight = dLoss_recon/dW', computes dLoss/dalpha through apply_adaround's soft rounding (closed-interval
+ * clamp gradients, as torch.clamp), adds the gradient of the rounding regulariser
+ * reg_param * sum(1 - |2h - 1|^beta) (AdaroundLoss.compute_round_loss, ADA/adaround_loss.py:82-111) when beta >= 0
+ * (beta < 0 = warm-start period, regulariser off), and applies torch.optim.Adam's update (no weight decay, no
+ * amsgrad) to alpha with moments exp_avg / exp_avg_sq; `step` is the 1-based count of this update.
+ * grad_alpha: optional (may be null) device tensor receiving dLoss/dalpha, what alpha.grad holds in the reference.
+ * reg_partial: optional device float[miq_adaround_blocks(num_element)] receiving per-workgroup partial sums of
+ * (1 - |2h - 1|^beta) evaluated at the alpha *before* the update (summed and scaled by reg_param by the caller). */
+int miq_adaround_bwd_adam_f32(const float* weight, const float* grad_weight, float* alpha, float* exp_avg,
+                              float* exp_avg_sq, float* grad_alpha, int64_t num_channel, int64_t num_element,
+                              int64_t num_element_per_channel, const float* delta, const float* offset, float clip_min,
+                              float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
+                              float eps, int step, float* reg_partial, void* stream);
+/* The gradient alone (autograd of apply_adaround + compute_round_loss w.r.t. alpha), nothing updated: for callers
+ * that keep their own optimiser. */
+int miq_adaround_bwd_f32(const float* weight, const float* grad_weight, const float* alpha, float* grad_alpha,
+                         int64_t num_channel, int64_t num_element, int64_t num_element_per_channel,
+                         const float* delta, const float* offset, float clip_min, float clip_max, float reg_param,
+                         float beta, float* reg_partial, void* stream);
+/* Number of workgroups (= partial sums) miq_adaround_bwd_adam_f32 / miq_adaround_bwd_f32 use for num_element elements. */
+int miq_adaround_blocks(int64_t num_element);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,284 @@
+"""GPU parity of the AdaRound kernels and of the AdaRound flow against the CPU restatement of the reference
+(oracle/adaround_oracle.py: torch CPU ops, torch autograd and torch.optim.Adam), through the C ABI.
+
+Tolerances (float32 path, transcendental functions differ by an ulp or two between the GPU and the host libm):
+  adarounded weights   hard rounding: identical; soft rounding: |diff| <= 4 ulp(2^bw) * delta
+  alpha initialisation |diff| <= 2e-6 (alpha lies in [-2.4, 2.4])
+  gradients            1e-4 relative to the largest gradient magnitude
+  alpha after N Adam iterations  2e-5 absolute (lr = 1e-3, so this is 2 % of one step)
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import adaround_oracle as ada
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from aimet_amd import ops as o
+    return o
+
+
+def _case(seed, shape, ch_axis, per_channel, bw=4):
+    g = torch.Generator().manual_seed(seed)
+    weight = torch.randn(*shape, generator=g) * 0.05
+    num_channel = shape[ch_axis] if per_channel else 1
+    if per_channel:
+        red = [d for d in range(len(shape)) if d != ch_axis]
+        absmax = weight.abs().amax(dim=red)
+    else:
+        absmax = weight.abs().max().reshape(1)
+    # a grid a little narrower than the weight range, so that the clamp to [clip_min, clip_max] is exercised
+    delta = (absmax * 1.7 / (2 ** bw - 1)).float()
+    offset = torch.full((num_channel,), float(-2 ** (bw - 1)))
+    n_per_channel = int(np.prod(shape[ch_axis + 1:])) if per_channel else int(np.prod(shape))
+    return weight, delta, offset, num_channel, n_per_channel, 0.0, float(2 ** bw - 1)
+
+
+CASES = [((64, 96), 0, True), ((7, 5, 3, 3), 0, True), ((6, 8, 3, 3), 1, True), ((33, 17), 0, False),
+         ((1, 3), 0, True), ((512, 512), 0, True)]
+
+
+@pytest.mark.parametrize("shape,ch_axis,per_channel", CASES)
+def test_init_alpha_and_soft_round(ops, shape, ch_axis, per_channel):
+    weight, delta, offset, C, npc, cmin, cmax = _case(11, shape, ch_axis, per_channel)
+    d, o = ada.broadcast(delta, weight, ch_axis), ada.broadcast(offset, weight, ch_axis)
+    alpha_ref = ada.generate_alpha(weight, d)
+    wg, dg, og = weight.cuda(), delta.cuda(), offset.cuda()
+    alpha = ops.adaround_init_alpha(wg, C, npc, dg)
+    assert torch.allclose(alpha.cpu(), alpha_ref, atol=2e-6, rtol=0)
+    # same alpha on both sides from here on; perturb it so that h leaves the initial fractional part
+    torch.manual_seed(1)
+    alpha_ref = alpha_ref + torch.randn_like(alpha_ref) * 2.0
+    ag = alpha_ref.cuda()
+    hard = ops.adaround_soft_round(wg, ag, C, npc, dg, og, cmin, cmax, False).cpu()
+    assert torch.equal(hard, ada.apply_adaround(weight, alpha_ref, d, o, cmin, cmax, False))
+    soft = ops.adaround_soft_round(wg, ag, C, npc, dg, og, cmin, cmax, True).cpu()
+    soft_ref = ada.apply_adaround(weight, alpha_ref, d, o, cmin, cmax, True)
+    # floor(w/delta) + h is rounded to float32 at magnitudes up to 2^bw: a one-ulp difference in sigmoid moves the sum
+    # by one ulp of that magnitude, and the result by that times delta
+    assert torch.allclose(soft, soft_ref, atol=float(4 * 2.0 ** -23 * 16 * delta.max()), rtol=0)
+
+
+@pytest.mark.parametrize("shape,ch_axis,per_channel", CASES[:4])
+@pytest.mark.parametrize("beta", [-1.0, 20.0, 4.636038969321072, 2.0])
+def test_alpha_gradient(ops, shape, ch_axis, per_channel, beta):
+    weight, delta, offset, C, npc, cmin, cmax = _case(13, shape, ch_axis, per_channel)
+    d, o = ada.broadcast(delta, weight, ch_axis), ada.broadcast(offset, weight, ch_axis)
+    torch.manual_seed(2)
+    alpha = (ada.generate_alpha(weight, d) + torch.randn_like(weight) * 2.5).requires_grad_(True)
+    grad_w = torch.randn_like(weight)
+    reg_param = 0.01
+    loss = (ada.apply_adaround(weight, alpha, d, o, cmin, cmax, True) * grad_w).sum()
+    reg_ref = None
+    if beta >= 0:
+        h = ada.rectified_sigmoid(alpha)
+        reg_ref = torch.add(1, -(torch.add(2 * h, -1).abs()).pow(beta)).sum()
+        loss = loss + reg_param * reg_ref
+    loss.backward()
+    partial = torch.zeros(ops.adaround_blocks(weight.numel()), device="cuda")
+    got = ops.adaround_bwd(weight.cuda(), grad_w.cuda(), alpha.detach().cuda(), C, npc, delta.cuda(), offset.cuda(),
+                           cmin, cmax, reg_param, beta, partial).cpu()
+    scale = alpha.grad.abs().max().item()
+    assert torch.allclose(got, alpha.grad, atol=1e-4 * scale, rtol=1e-4)
+    # same zero pattern: the clamp masks are decided identically
+    assert torch.equal(got == 0, alpha.grad == 0)
+    if beta >= 0:
+        assert partial.sum().item() == pytest.approx(reg_ref.item(), rel=1e-5)
+
+
+class _Layer:
+    """What AdaroundOptimizer reads from an AdaroundWrapper, without a QuantizationSimModel around it."""
+
+    def __init__(self, module, alpha0, delta, offset, C, npc, cmin, cmax):
+        self._module = module
+        self.weight = module.weight
+        self.alpha = torch.nn.Parameter(alpha0.clone().cuda())
+        self.delta, self.offset = delta.cuda(), offset.cuda()
+        self.num_channel, self.n_per_channel, self.clip_min, self.clip_max = C, npc, cmin, cmax
+        self.use_soft_rounding = True
+
+    def get_original_module(self):
+        return self._module
+
+
+def _run_product_loop(kind, weight, alpha0, delta, offset, C, npc, cmin, cmax, all_inp, all_out, batches, hyper, act,
+                      conv_args):
+    from aimet_amd.v1.adaround.adaround_loss import AdaroundHyperParameters
+    from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
+    if kind == "linear":
+        module = torch.nn.Linear(weight.shape[1], weight.shape[0], bias=False)
+    else:
+        module = torch.nn.Conv2d(weight.shape[1], weight.shape[0], weight.shape[2], bias=False, **conv_args)
+    module.weight.data = weight.clone()
+    module.cuda()
+    layer = _Layer(module, alpha0, delta, offset, C, npc, cmin, cmax)
+    m, v = AdaroundOptimizer.optimize_rounding_on_cached_acts(layer, act, all_inp.cuda(), all_out.cuda(),
+                                                              AdaroundHyperParameters(*hyper), batches=batches)
+    return layer.alpha.detach().cpu(), m.cpu(), v.cpu(), layer.alpha.grad.cpu()
+
+
+@pytest.mark.parametrize("kind,act", [("linear", None), ("linear", torch.relu), ("conv2d", torch.relu)])
+def test_optimisation_trajectory(ops, kind, act):
+    iters = 40
+    hyper = (iters, 0.01, (20, 2), 0.2)
+    if kind == "linear":
+        shape, conv_args = (48, 64), {}
+        torch.manual_seed(21)
+        all_inp = torch.randn(128, 64)
+    else:
+        shape, conv_args = (8, 6, 3, 3), {"padding": 1}
+        torch.manual_seed(22)
+        all_inp = torch.randn(96, 6, 9, 9)
+    weight, delta, offset, C, npc, cmin, cmax = _case(17, shape, 0, True)
+    d = ada.broadcast(delta, weight, 0)
+    alpha0 = ada.generate_alpha(weight, d)
+    all_out = ada.layer_output(kind, all_inp, weight, **conv_args)          # the fp32 layer's output
+    batches = [torch.randperm(all_inp.size(0))[:32] for _ in range(iters)]
+    trace = []
+    a_ref, m_ref, v_ref, g_ref = ada.optimize_rounding(kind, weight, alpha0, delta, offset, cmin, cmax, all_inp,
+                                                       all_out, batches, *hyper, act=act, conv_args=conv_args,
+                                                       trace=trace)
+    a, m, v, g = _run_product_loop(kind, weight, alpha0, delta, offset, C, npc, cmin, cmax, all_inp, all_out, batches,
+                                   hyper, act, conv_args)
+    assert (a_ref - alpha0).abs().max() > 5e-3          # the loop did move alpha
+    assert torch.allclose(a, a_ref, atol=2e-5, rtol=0)
+    assert torch.allclose(g, g_ref, atol=1e-4 * g_ref.abs().max().item(), rtol=1e-3)
+    assert torch.allclose(m, m_ref, atol=1e-4 * m_ref.abs().max().item(), rtol=1e-3)
+    assert torch.allclose(v, v_ref, atol=1e-4 * v_ref.abs().max().item(), rtol=1e-3)
+
+
+class _TinyNet(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.conv1 = torch.nn.Conv2d(3, 8, 3, padding=1)
+        self.relu1 = torch.nn.ReLU(inplace=True)
+        self.pool = torch.nn.AdaptiveAvgPool2d(4)
+        self.flatten = torch.nn.Flatten()
+        self.fc = torch.nn.Linear(8 * 16, 10)
+
+    def forward(self, x):
+        return self.fc(self.flatten(self.pool(self.relu1(self.conv1(x)))))
+
+
+def _loader(n_batches, batch, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [(torch.randn(batch, 3, 8, 8, generator=g).cuda(), torch.zeros(batch)) for _ in range(n_batches)]
+
+
+def _forward_fn(model, inputs):
+    x, _ = inputs
+    return model(x)
+
+
+def test_reference_style_layer_optimisation(tmp_path):
+    """Shaped after TestAdaroundOptimizer._optimize_layer_rounding (test_adaround_optimizer.py:65-109): alpha changes,
+    alpha.grad is populated, and afterwards the layer uses hard rounding."""
+    from aimet_amd.v1.adaround.adaround_loss import AdaroundHyperParameters
+    from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
+    from aimet_amd.v1.adaround.adaround_weight import Adaround
+    from aimet_amd.v1.quantsim import QuantizationSimModel
+    from aimet_amd import utils
+    for warm_start in (1.0, 0.2):
+        torch.manual_seed(0)
+        model = _TinyNet().eval().cuda()
+        dummy = torch.randn(1, 3, 8, 8).cuda()
+        sim = QuantizationSimModel(model, dummy_input=dummy, quant_scheme='tf_enhanced', default_param_bw=4)
+        Adaround._compute_param_encodings(sim)
+        with Adaround._replace_quantization_layer(sim.model, "conv1") as wrapper:
+            wrapper.alpha = torch.nn.Parameter(torch.randn(wrapper.weight.shape).cuda())
+            before = wrapper.alpha.detach().clone()
+            cached = utils.CachedDataset(_loader(5, 10, 1), 5)
+            opt = AdaroundHyperParameters(num_iterations=10, reg_param=0.01, beta_range=(20, 2),
+                                          warm_start=warm_start)
+            AdaroundOptimizer.adaround_module(model.conv1, wrapper, model, sim.model, None, cached, _forward_fn, opt)
+            assert not torch.equal(before, wrapper.alpha.detach())
+            assert wrapper.alpha.grad is not None
+            assert wrapper.use_soft_rounding is False
+
+
+def test_recons_metrics_known_answer(vectors, ops):
+    """test_adaround_optimizer.py:122-196 on the GPU: TF-Enhanced encoding of a seeded weight, hard / soft
+    reconstruction errors and the reconstruction loss."""
+    from aimet_amd.v1.adaround.adaround_loss import AdaroundLoss
+    from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
+    from aimet_amd.v1.adaround.adaround_wrapper import AdaroundWrapper
+    from aimet_amd.v1.qc_quantize_op import StaticGridQuantWrapper
+    from aimet_amd.common.defs import QuantScheme
+    g = vectors["adaround"]["recons_metrics"]
+    np.random.seed(g["np_seed"])
+    weight = np.random.rand(*g["weight_shape"]).astype('float32')
+    conv = torch.nn.Conv2d(4, 4, 1, bias=False).cuda()
+    conv.weight.data = torch.from_numpy(weight).cuda()
+    qw = StaticGridQuantWrapper(conv, g["weight_bw"], 8, round_mode='nearest',
+                                quant_scheme=QuantScheme.post_training_tf_enhanced)
+    qw.param_quantizers['weight'].update_encoding_stats(conv.weight.data)
+    qw.param_quantizers['weight'].compute_encoding()
+    assert qw.param_quantizers['weight'].encoding.delta == pytest.approx(g["scale"], abs=10 ** -g["scale_places"])
+    inp = torch.from_numpy(np.random.rand(*g["inp_shape"]).astype('float32')).cuda()
+    out = torch.from_numpy(np.random.rand(*g["out_shape"]).astype('float32')).cuda()
+    wrapper = AdaroundWrapper(qw)
+    hard, soft = AdaroundOptimizer._compute_recons_metrics(wrapper, None, inp, out)
+    assert hard == pytest.approx(g["recons_err_hard"], abs=10 ** -g["places"])
+    assert soft == pytest.approx(g["recons_err_soft"], abs=10 ** -g["places"])
+    y = AdaroundOptimizer._compute_output_with_adarounded_weights(wrapper, inp)
+    assert AdaroundLoss.compute_recon_loss(y, out).item() == pytest.approx(g["recon_loss_soft"],
+                                                                           abs=10 ** -g["cuda_places"])
+
+
+def test_apply_adaround_end_to_end(tmp_path, oracle):
+    """Adaround.apply_adaround on a small conv + linear model against the same flow replayed with the CPU restatement:
+    same encodings file, same seeded batches, adarounded weights equal on the quantization grid."""
+    from aimet_amd.v1.adaround.adaround_weight import Adaround, AdaroundParameters
+    torch.manual_seed(0)
+    model = _TinyNet().eval().cuda()
+    dummy = torch.randn(1, 3, 8, 8).cuda()
+    loader = _loader(4, 16, 5)
+    iters = 30
+    params = AdaroundParameters(loader, num_batches=4, default_num_iterations=iters, forward_fn=_forward_fn)
+    torch.manual_seed(1234)
+    ada_model = Adaround.apply_adaround(model, dummy, params, str(tmp_path), "tiny", default_param_bw=4)
+    with open(os.path.join(str(tmp_path), "tiny.encodings")) as f:
+        enc = json.load(f)["param_encodings"]
+    assert set(enc) == {"conv1.weight", "fc.weight"}
+
+    # replay on the CPU
+    cpu = _TinyNet().eval()
+    cpu.load_state_dict({k: v.cpu() for k, v in model.state_dict().items()})
+    quant = _TinyNet().eval()
+    quant.load_state_dict(cpu.state_dict())
+    torch.manual_seed(1234)                     # the product drew its batches from the host generator seeded so
+    xs = torch.cat([b[0].cpu() for b in loader])
+    for name, kind, act, conv_args in (("conv1", "conv2d", torch.relu, {"padding": 1}), ("fc", "linear", None, {})):
+        e = enc[name + ".weight"][0]
+        assert e["bitwidth"] == 4
+        delta = torch.tensor([e["scale"]], dtype=torch.float32)
+        offset = torch.tensor([float(e["offset"])], dtype=torch.float32)
+        layer_fp, layer_q = getattr(cpu, name), getattr(quant, name)
+        with torch.no_grad():
+            if name == "conv1":
+                inp, out = xs, layer_fp(xs)
+            else:
+                inp = quant.flatten(quant.pool(torch.relu(quant.conv1(xs))))
+                out = layer_fp(cpu.flatten(cpu.pool(torch.relu(cpu.conv1(xs)))))
+        weight = layer_fp.weight.detach()
+        alpha0 = ada.generate_alpha(weight, delta.reshape(()))
+        batches = [torch.randperm(inp.size(0))[:32] for _ in range(iters)]
+        alpha, _, _, _ = ada.optimize_rounding(kind, weight, alpha0, delta, offset, 0, 15, inp, out, batches, iters,
+                                               0.01, (20, 2), 0.2, bias=layer_fp.bias.detach(), act=act,
+                                               conv_args=conv_args)
+        w_ref = ada.apply_adaround(weight, alpha, delta.reshape(()), offset.reshape(()), 0, 15, True)
+        got = getattr(ada_model, name).weight.detach().cpu()
+        assert torch.allclose(got, w_ref, atol=float(delta) * 2e-3, rtol=0), name
+        # later layers see this layer through its weight quantizer (same encoding, round to nearest)
+        w_seen = oracle.qdq_per_tensor(w_ref.numpy().reshape(-1), e["min"], e["max"], 4).reshape(w_ref.shape)
+        with torch.no_grad():
+            layer_q.weight.copy_(torch.from_numpy(w_seen))
+    assert not any(isinstance(m, torch.nn.Module) and type(m).__name__.endswith("Wrapper")
+                   for m in ada_model.modules())

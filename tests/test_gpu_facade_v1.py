@@ -1,0 +1,238 @@
+"""GPU tests of the v1 host-side interface (tensor quantizers, wrappers, QuantizationSimModel) against the CPU oracle.
+
+The cases follow the reference's own unit tests of this interface (TrainingExtensions/torch/test/python/
+test_tensor_quantizer.py, test_quantizer.py): statistics -> encoding -> quantize-dequantize -> straight-through
+gradient, per tensor and per channel, then the model-level flow compute_encodings / forward / export.
+Encodings and quantized values must be identical to the oracle's; nothing here is a tolerance test.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+pytestmark = pytest.mark.gpu
+
+@pytest.fixture(scope="module")
+def api():
+    from aimet_amd.common import libpymo
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1 import qc_quantize_op, quantsim, tensor_quantizer
+
+    class Api:
+        pass
+    a = Api()
+    a.libpymo, a.QuantScheme, a.qc, a.quantsim, a.tq = libpymo, QuantScheme, qc_quantize_op, quantsim, tensor_quantizer
+    a.nearest = libpymo.RoundingMode.ROUND_NEAREST
+    return a
+
+
+def _enc_tuple(e):
+    return (e.min, e.max, e.delta, e.offset, e.bw)
+
+
+@pytest.mark.parametrize("scheme", ["tf", "tfe"])
+@pytest.mark.parametrize("bw,sym", [(8, False), (8, True), (4, False)])
+def test_per_tensor_quantizer(api, oracle, scheme, bw, sym):
+    qs = api.QuantScheme.post_training_tf if scheme == "tf" else api.QuantScheme.post_training_tf_enhanced
+    q = api.tq.StaticGridPerTensorQuantizer(bw, api.nearest, qs, sym, enabled_by_default=True)
+    rng = np.random.default_rng(3)
+    batches = [(rng.standard_normal(20000) * s).astype(np.float32) for s in (1.0, 1.5)]
+    for b in batches:
+        q.update_encoding_stats(torch.from_numpy(b).cuda())
+    q.compute_encoding()
+    if scheme == "tf":
+        mn = min(float(b.min()) for b in batches)
+        mx = max(float(b.max()) for b in batches)
+        expect = oracle.tf_compute_encoding(mn, mx, bw, sym)
+    else:
+        pdf = oracle.new_pdf()
+        for b in batches:
+            pdf.update(b)
+        expect, _, _ = pdf.compute_encoding(bw, sym)
+    assert _enc_tuple(q.encoding) == expect.astuple()
+    x = (rng.standard_normal(5003) * 2).astype(np.float32)
+    xg = torch.from_numpy(x).cuda().requires_grad_(True)
+    y = q.quantize_dequantize(xg, api.nearest)
+    assert np.array_equal(y.detach().cpu().numpy(), oracle.qdq_per_tensor(x, expect.min, expect.max, bw))
+    g = rng.standard_normal(x.size).astype(np.float32)
+    y.backward(torch.from_numpy(g).cuda())
+    assert np.array_equal(xg.grad.cpu().numpy(), oracle.ste_bwd_per_tensor(x, g, expect.min, expect.max))
+    codes = q.quantize(torch.from_numpy(x).cuda(), api.nearest)
+    # quantize-only shifts to the signed range unless the quantizer is unsigned-symmetric
+    assert np.array_equal(codes.cpu().numpy(), oracle.quantize_per_tensor(x, expect.min, expect.max, bw, True))
+
+
+@pytest.mark.parametrize("scheme", ["tf", "tfe"])
+@pytest.mark.parametrize("shape,axis", [((16, 8, 3, 3), 0), ((6, 10, 3, 3), 1), ((32, 48), 0)])
+def test_per_channel_quantizer(api, oracle, scheme, shape, axis):
+    qs = api.QuantScheme.post_training_tf if scheme == "tf" else api.QuantScheme.post_training_tf_enhanced
+    q = api.tq.StaticGridPerChannelQuantizer(8, api.nearest, qs, True, num_channels=shape[axis],
+                                             enabled_by_default=True, ch_axis=axis)
+    rng = np.random.default_rng(5)
+    w = (rng.laplace(0, 0.02, size=shape)).astype(np.float32)
+    q.update_encoding_stats(torch.from_numpy(w).cuda())
+    q.compute_encoding()
+    expect = []
+    for c in range(shape[axis]):
+        sl = np.ascontiguousarray(np.take(w, c, axis=axis)).reshape(-1)
+        if scheme == "tf":
+            expect.append(oracle.tf_compute_encoding(float(sl.min()), float(sl.max()), 8, True))
+        else:
+            pdf = oracle.new_pdf()
+            pdf.update(sl)
+            expect.append(pdf.compute_encoding(8, True)[0])
+    assert [_enc_tuple(e) for e in q.encoding] == [e.astuple() for e in expect]
+    xg = torch.from_numpy(w * 1.3).cuda().requires_grad_(True)
+    y = q.quantize_dequantize(xg, api.nearest)
+    npc = int(np.prod(shape[axis + 1:]))
+    params = oracle.per_channel_params(np.array([e.min for e in expect], np.float32),
+                                       np.array([e.max for e in expect], np.float32), 8)
+    want = oracle.qdq_per_channel((w * 1.3).astype(np.float32).reshape(-1), shape[axis], npc, params)
+    assert np.array_equal(y.detach().cpu().numpy().reshape(-1), want)
+    g = rng.standard_normal(w.size).astype(np.float32)
+    y.backward(torch.from_numpy(g.reshape(shape)).cuda())
+    want_g = oracle.ste_bwd_per_channel((w * 1.3).astype(np.float32).reshape(-1), g, shape[axis], npc,
+                                        np.array([e.min for e in expect], np.float32),
+                                        np.array([e.max for e in expect], np.float32))
+    assert np.array_equal(xg.grad.cpu().numpy().reshape(-1), want_g)
+
+
+def test_cpu_tensors_are_rejected(api):
+    q = api.tq.StaticGridPerTensorQuantizer(8, api.nearest, api.QuantScheme.post_training_tf, False, True)
+    with pytest.raises(RuntimeError):
+        q.update_encoding_stats(torch.randn(10))
+
+
+def test_disabled_and_frozen_quantizers(api):
+    """test_tensor_quantizer.py: a disabled quantizer ignores statistics; a frozen one keeps its encoding."""
+    q = api.tq.StaticGridPerTensorQuantizer(8, api.nearest, api.QuantScheme.post_training_tf, False, True)
+    with pytest.raises(RuntimeError):
+        q.freeze_encoding()
+    q.update_encoding_stats(torch.randn(100).cuda())
+    q.compute_encoding()
+    first = _enc_tuple(q.encoding)
+    q.freeze_encoding()
+    q.reset_encoding_stats()
+    q.update_encoding_stats(torch.randn(100).cuda() * 10)
+    q.compute_encoding()
+    assert _enc_tuple(q.encoding) == first and q.is_encoding_frozen
+    with pytest.raises(RuntimeError):
+        q.encoding = q.encoding
+    # no statistics at all -> quantizer disables itself
+    q2 = api.tq.StaticGridPerTensorQuantizer(8, api.nearest, api.QuantScheme.post_training_tf, False, True)
+    q2.compute_encoding()
+    assert q2.enabled is False and q2.encoding is None
+
+
+class _Net(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.conv1 = nn.Conv2d(3, 8, 3, padding=1)
+        self.relu1 = nn.ReLU()
+        self.conv2 = nn.Conv2d(8, 8, 3, padding=1, bias=False)
+        self.bn = nn.BatchNorm2d(8)
+        self.flatten = nn.Flatten()
+        self.fc = nn.Linear(8 * 6 * 6, 5)
+
+    def forward(self, x):
+        x = self.relu1(self.conv1(x))
+        x = self.bn(self.conv2(x))
+        return self.fc(self.flatten(x))
+
+
+def _calibrate(model, batches):
+    for b in batches:
+        model(b)
+
+
+def test_quantsim_flow(api, oracle, tmp_path):
+    torch.manual_seed(0)
+    model = _Net().eval().cuda()
+    dummy = torch.randn(2, 3, 6, 6).cuda()
+    sim = api.quantsim.QuantizationSimModel(model, dummy_input=dummy, quant_scheme='tf_enhanced',
+                                            default_output_bw=8, default_param_bw=8)
+    w = dict(sim.quant_wrappers())
+    assert set(w) == {"conv1", "relu1", "conv2", "bn", "flatten", "fc"}
+    # default configuration: model input quantized, Conv+Relu supergroup, bias not quantized, Flatten transparent
+    assert w["conv1"].input_quantizers[0].enabled
+    assert not w["conv1"].output_quantizers[0].enabled
+    assert w["relu1"].output_quantizers[0].enabled
+    assert w["conv1"].param_quantizers["weight"].enabled and not w["conv1"].param_quantizers["bias"].enabled
+    assert not w["flatten"].output_quantizers[0].enabled
+    assert w["fc"].output_quantizers[0].enabled
+
+    batches = [torch.randn(4, 3, 6, 6).cuda() for _ in range(3)]
+    captured = []
+    handle = w["relu1"]._module_to_wrap.register_forward_hook(lambda m, i, o: captured.append(o.detach().cpu()))
+    sim.compute_encodings(_calibrate, batches)
+    handle.remove()
+    # the relu output quantizer saw exactly the captured activations
+    pdf = oracle.new_pdf()
+    for a in captured[:3]:
+        pdf.update(a.numpy().reshape(-1))
+    expect, _, _ = pdf.compute_encoding(8, False)
+    enc = w["relu1"].output_quantizers[0].encoding
+    assert _enc_tuple(enc) == expect.astuple()
+    # weight encodings: symmetric TF-Enhanced on the weight tensor
+    pdf = oracle.new_pdf()
+    pdf.update(model.conv2.weight.detach().cpu().numpy().reshape(-1))
+    expect_w, _, _ = pdf.compute_encoding(8, True)
+    assert _enc_tuple(w["conv2"].param_quantizers["weight"].encoding) == expect_w.astuple()
+
+    # forward in ACTIVE mode: the model output lies on the grid of the last output quantizer
+    x = torch.randn(4, 3, 6, 6).cuda()
+    with torch.no_grad():
+        y = sim.model(x)
+    e = w["fc"].output_quantizers[0].encoding
+    steps = y.double().cpu().numpy() / e.delta
+    assert np.abs(steps - np.round(steps)).max() < 1e-3
+    assert y.min().item() >= e.min - 1e-6 and y.max().item() <= e.max + 1e-6
+    # parameters are restored after the pass
+    assert torch.equal(sim.model.conv2._module_to_wrap.weight, model.conv2.weight)
+
+    # backward reaches the input and the parameters
+    x.requires_grad_(True)
+    sim.model(x).sum().backward()
+    assert x.grad is not None and torch.isfinite(x.grad).all()
+    assert sim.model.fc._module_to_wrap.weight.grad is not None
+
+    # export and re-import of parameter encodings
+    path = sim.export_encodings(str(tmp_path), "net")
+    with open(path) as f:
+        data = json.load(f)
+    assert "conv2.weight" in data["param_encodings"] and "relu1" in data["activation_encodings"]
+    assert data["param_encodings"]["conv2.weight"][0]["scale"] == expect_w.delta
+    sim2 = api.quantsim.QuantizationSimModel(model, dummy_input=dummy, quant_scheme='tf_enhanced')
+    sim2.set_and_freeze_param_encodings(path)
+    q = dict(sim2.quant_wrappers())["conv2"].param_quantizers["weight"]
+    assert q.is_encoding_frozen and q.encoding.delta == expect_w.delta
+
+
+def test_quantsim_per_channel_config(api, tmp_path):
+    cfg = {"defaults": {"ops": {"is_output_quantized": "True"},
+                        "params": {"is_quantized": "True", "is_symmetric": "True"},
+                        "per_channel_quantization": "True"},
+           "params": {"bias": {"is_quantized": "False"}}, "op_type": {}, "supergroups": [],
+           "model_input": {"is_input_quantized": "True"}, "model_output": {}}
+    p = os.path.join(str(tmp_path), "cfg.json")
+    with open(p, "w") as f:
+        json.dump(cfg, f)
+    torch.manual_seed(1)
+    model = _Net().eval().cuda()
+    dummy = torch.randn(2, 3, 6, 6).cuda()
+    sim = api.quantsim.QuantizationSimModel(model, dummy_input=dummy, quant_scheme='tf', config_file=p)
+    w = dict(sim.quant_wrappers())
+    assert isinstance(w["conv1"].param_quantizers["weight"], api.tq.StaticGridPerChannelQuantizer)
+    sim.compute_encodings(_calibrate, [torch.randn(4, 3, 6, 6).cuda()])
+    encs = w["conv1"].param_quantizers["weight"].encoding
+    assert len(encs) == 8
+    wt = model.conv1.weight.detach()
+    for c, e in enumerate(encs):
+        absmax = wt[c].abs().max().item()
+        assert e.max == pytest.approx(absmax, rel=1e-6)      # symmetric TF encoding: max = |w|max of the channel
+    with torch.no_grad():
+        y = sim.model(dummy)
+    assert torch.isfinite(y).all()
