@@ -28,6 +28,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
+# HBM bytes per launch at the main shape, from hardware counters (two rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE,
+# each scaled by what the same counter reads for a plain elementwise kernel of known traffic: x2.000 and x1.000).
+# The counter runs are separate from this program; these are their results for [11008,4096] fp32.
+MEASURED_TRAFFIC_BYTES = {"ste_bwd_per_channel_f32": 542.47e6, "qdq_fwd_per_channel_f32": 363.61e6}
+
 
 def _laplace_weights(torch, shape, seed, device):
     g = torch.Generator(device=device).manual_seed(seed)
@@ -220,7 +225,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--full", action="store_true", help="also measure every shape x dtype x bit-width cell")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default=None, help="internal: run one leg only (main|pt|calib) for profiling")
+    ap.add_argument("--only", default=None,
+                    help="run a subset of the legs, comma separated (main|pt|calib|copyref), for profiling")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
@@ -237,11 +243,25 @@ def main():
     main_shape = (11008, 4096)
     extra = {}
     res = None
-    if args.only in (None, "main"):
+    legs = None if args.only is None else set(args.only.split(","))
+
+    def want(leg):
+        return leg in legs if legs is not None else leg != "copyref"
+
+    if want("copyref"):
+        # a plain elementwise kernel of known traffic (reads 4 B, writes 4 B per element of the main shape): the
+        # yardstick that hardware-counter readings of the kernels above are scaled by
+        a = torch.randn(main_shape, device="cuda")
+        b = torch.empty_like(a)
+        for _ in range(10):
+            torch.add(a, 1.0, out=b)
+        torch.cuda.synchronize()
+        extra["copyref"] = {"elements": a.numel(), "bytes_read": 4 * a.numel(), "bytes_written": 4 * a.numel()}
+    if want("main"):
         res = bench_per_channel(torch, ops, main_shape, torch.float32, 8, args.steps, args.warmup, 1004)
-    if args.only in (None, "pt"):
+    if want("pt"):
         extra["per_tensor_act_int8"] = bench_per_tensor(torch, ops, max(20, args.steps), args.warmup)
-    if args.only in (None, "calib"):
+    if want("calib"):
         extra["tf_enhanced_calibration"] = bench_calibration(torch, ops, 5)
     if args.only is None:
         cells = [((11008, 4096), torch.bfloat16, 8), ((11008, 4096), torch.float32, 4)]
@@ -267,10 +287,12 @@ def main():
         "pct_hbm_peak": 100.0 * res["fwd_bwd_GBps"] / HBM_PEAK_GBPS,
         "roofline": {"bound": "hbm", "kernel": "ew_vec_kernel<float, OpV1Ste, per-channel> (STE backward)",
                      "achieved": res["bwd_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": res["bwd_GBps"] / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": res["bwd_GBps"] / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES["ste_bwd_per_channel_f32"],
                      "avg_launch_ms": res["bwd_ms"], "algorithmic_bytes_per_launch": 12 * n,
                      "forward_kernel": {"achieved": res["fwd_GBps"], "frac": res["fwd_GBps"] / HBM_PEAK_GBPS,
-                                        "avg_launch_ms": res["fwd_ms"], "algorithmic_bytes_per_launch": 8 * n}},
+                                        "avg_launch_ms": res["fwd_ms"], "algorithmic_bytes_per_launch": 8 * n,
+                                        "traffic": MEASURED_TRAFFIC_BYTES["qdq_fwd_per_channel_f32"]}},
     }
     if "tf_enhanced_calibration" in extra:
         line["calib_elements_per_s"] = extra["tf_enhanced_calibration"]["elements_per_s"]
