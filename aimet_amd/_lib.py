@@ -69,6 +69,12 @@ _SIGNATURES = {
                                    _flt, _flt, _flt, _int, _p, _p], _int),
     "miq_adaround_bwd_f32": ([_p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _flt, _flt, _p, _p], _int),
     "miq_adaround_blocks": ([_i64], _int),
+    "miq_adaround_linear_workspace_bytes": ([_i64, _i64], _i64),
+    "miq_adaround_linear_blocks": ([_i64, _i64], _int),
+    "miq_adaround_linear_fwd_f32": ([_p, _p, _p, _p, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
+                                     _p, _p, _p, _p, _p], _int),
+    "miq_adaround_linear_bwd_adam_f32": ([_p, _p, _p, _p, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
+                                          _flt, _flt, _flt, _flt, _flt, _flt, _int, _p, _p], _int),
 }
 
 # Entry points declared in include/miq.h; the loader insists on every one of them.

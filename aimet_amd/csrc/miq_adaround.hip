@@ -12,16 +12,34 @@
 // The reference runs about fifteen elementwise ATen kernels per iteration over weight-shaped tensors plus their
 // autograd twins; here the forward is one pass (read W, alpha; write W') and the backward one pass (read dW', W,
 // alpha, m, v; write alpha, m, v).
-#include "miq_common.h"
+#include "miq_adaround_math.h"
 
 #include <cmath>
 
 namespace miq
 {
+namespace ada
+{
+int make_adam(AdamArgs& a, float reg_param, float beta, float lr, float beta1, float beta2, float eps, int step)
+{
+    MIQ_CHECK_ARG(step >= 1, "Adam step count starts at 1");
+    MIQ_CHECK_ARG(beta1 >= 0.f && beta1 < 1.f && beta2 >= 0.f && beta2 < 1.f, "Adam betas must lie in [0, 1)");
+    a.reg_param = reg_param;
+    a.beta      = beta;
+    const double bc1 = 1.0 - std::pow((double) beta1, (double) step);
+    const double bc2 = 1.0 - std::pow((double) beta2, (double) step);
+    a.lr_over_bc1    = (float) ((double) lr / bc1);
+    a.bc2_sqrt       = (float) std::sqrt(bc2);
+    a.beta1          = beta1;
+    a.beta2          = beta2;
+    a.eps            = eps;
+    return MIQ_OK;
+}
+}   // namespace ada
+
 namespace
 {
-constexpr float kZetaMinusGamma = 1.2f;   // float32(1.1 - (-0.1)) = float32(1.2000000000000002)
-constexpr float kGamma          = -0.1f;
+using namespace ada;
 
 struct AdaGeom
 {
@@ -37,19 +55,6 @@ __device__ __forceinline__ uint32_t channel_of(int64_t e, const AdaGeom& g)
 {
     // e < 2^31 on this path (checked by the host)
     return fastdiv((uint32_t) e, g.fd) % g.num_channel;
-}
-
-__device__ __forceinline__ float sigmoidf_(float a)
-{
-    return 1.0f / (1.0f + expf(-a));
-}
-
-// h(alpha) and, optionally, the pieces the backward needs
-__device__ __forceinline__ float soft_h(float alpha, float& sig, float& inner)
-{
-    sig   = sigmoidf_(alpha);
-    inner = sig * kZetaMinusGamma + kGamma;
-    return fminf(fmaxf(inner, 0.0f), 1.0f);
 }
 
 template <bool SOFT>
@@ -70,13 +75,7 @@ __global__ __launch_bounds__(kBlock) void soft_round_kernel(const float* __restr
         for (int j = 0; j < 4; ++j)
         {
             const uint32_t c = (c0 == c3) ? c0 : channel_of(v * 4 + j, g);
-            const float d = g.delta[c], o = g.offset[c];
-            const float f = floorf(ws[j] / d);
-            float sig, inner;
-            const float h = SOFT ? soft_h(as[j], sig, inner) : (as[j] >= 0.0f ? 1.0f : 0.0f);
-            const float t = f + h;
-            const float q = fminf(fmaxf(t - o, g.clip_min), g.clip_max);
-            ys[j]         = (q + o) * d;
+            ys[j] = adarounded<SOFT>(ws[j], as[j], g.delta[c], g.offset[c], g.clip_min, g.clip_max);
         }
         reinterpret_cast<float4*>(out)[v] = make_float4(ys[0], ys[1], ys[2], ys[3]);
     }
@@ -84,12 +83,7 @@ __global__ __launch_bounds__(kBlock) void soft_round_kernel(const float* __restr
     {
         const int64_t e  = nvec * 4 + threadIdx.x;
         const uint32_t c = channel_of(e, g);
-        const float d = g.delta[c], o = g.offset[c];
-        const float f = floorf(w[e] / d);
-        float sig, inner;
-        const float h = SOFT ? soft_h(alpha[e], sig, inner) : (alpha[e] >= 0.0f ? 1.0f : 0.0f);
-        const float q = fminf(fmaxf(f + h - o, g.clip_min), g.clip_max);
-        out[e]        = (q + o) * d;
+        out[e] = adarounded<SOFT>(w[e], alpha[e], g.delta[c], g.offset[c], g.clip_min, g.clip_max);
     }
 }
 
@@ -104,51 +98,6 @@ __global__ __launch_bounds__(kBlock) void init_alpha_kernel(const float* __restr
         // alpha = -log((zeta - gamma) / (frac - gamma) - 1)
         alpha[e] = -logf(kZetaMinusGamma / (frac - kGamma) - 1.0f);
     }
-}
-
-struct AdamArgs
-{
-    float reg_param;
-    float beta;        // exponent of the regulariser; < 0 during warm start (no rounding loss)
-    float lr_over_bc1; // lr / (1 - beta1^t)
-    float bc2_sqrt;    // sqrt(1 - beta2^t)
-    float beta1, beta2, eps;
-};
-
-// dLoss/dalpha of one element: chain rule of apply_adaround (closed-interval clamp gradients, as torch.clamp) plus the
-// gradient of reg_param * (1 - |2h - 1|^beta); `reg` receives this element's regulariser term (0 in warm start)
-__device__ __forceinline__ float alpha_grad(float w, float gw, float alpha, float d, float o, const AdaGeom& g,
-                                            const AdamArgs& a, float& reg)
-{
-    const float f = floorf(w / d);
-    float sig, inner;
-    const float h      = soft_h(alpha, sig, inner);
-    const float t      = f + h - o;
-    const float pass_q = (t >= g.clip_min && t <= g.clip_max) ? 1.0f : 0.0f;
-    const float pass_h = (inner >= 0.0f && inner <= 1.0f) ? 1.0f : 0.0f;
-    const float dsig   = (1.0f - sig) * sig;
-    const float dh     = pass_h * kZetaMinusGamma * dsig;
-    float grad         = gw * d * pass_q * dh;
-    reg                = 0.0f;
-    if (a.beta >= 0.0f)
-    {
-        const float x   = 2.0f * h - 1.0f;
-        const float ax  = fabsf(x);
-        reg             = 1.0f - powf(ax, a.beta);
-        const float sgn = (x > 0.0f) ? 1.0f : ((x < 0.0f) ? -1.0f : 0.0f);
-        const float dp  = (ax > 0.0f) ? a.beta * powf(ax, a.beta - 1.0f) : 0.0f;
-        grad += -a.reg_param * dp * sgn * 2.0f * dh;
-    }
-    return grad;
-}
-
-// Adam (torch single-tensor form): lerp for the first moment, mul/addcmul for the second
-__device__ __forceinline__ void adam_update(float grad, float& alpha, float& m, float& v, const AdamArgs& a)
-{
-    m = m + (1.0f - a.beta1) * (grad - m);
-    v = v * a.beta2 + (1.0f - a.beta2) * grad * grad;
-    const float denom = sqrtf(v) / a.bc2_sqrt + a.eps;
-    alpha             = alpha - a.lr_over_bc1 * (m / denom);
 }
 
 // ADAM = true : alpha, m, v updated in place; grad_out (optional) receives dLoss/dalpha
@@ -183,7 +132,7 @@ __global__ __launch_bounds__(kBlock) void bwd_kernel(const float* __restrict__ w
         {
             const uint32_t c = (c0 == c3) ? c0 : channel_of(i * 4 + j, g);
             float r;
-            gr[j] = alpha_grad(ws[j], gs[j], as[j], g.delta[c], g.offset[c], g, a, r);
+            gr[j] = alpha_grad(ws[j], gs[j], as[j], g.delta[c], g.offset[c], g.clip_min, g.clip_max, a, r);
             reg += r;
             if (ADAM)
                 adam_update(gr[j], as[j], ms[j], vs[j], a);
@@ -202,7 +151,7 @@ __global__ __launch_bounds__(kBlock) void bwd_kernel(const float* __restrict__ w
         const int64_t e  = nvec * 4 + threadIdx.x;
         const uint32_t c = channel_of(e, g);
         float r;
-        const float gr = alpha_grad(w[e], gw[e], alpha[e], g.delta[c], g.offset[c], g, a, r);
+        const float gr = alpha_grad(w[e], gw[e], alpha[e], g.delta[c], g.offset[c], g.clip_min, g.clip_max, a, r);
         reg += r;
         if (ADAM)
             adam_update(gr, alpha[e], m[e], v[e], a);
@@ -212,20 +161,9 @@ __global__ __launch_bounds__(kBlock) void bwd_kernel(const float* __restrict__ w
     if (reg_partial)
     {
         // per-workgroup partial of the regulariser sum, combined in a fixed order by the caller (deterministic)
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1)
-            reg += __shfl_xor(reg, o);
-        __shared__ float s[kBlock / 64];
-        if ((threadIdx.x & 63) == 0)
-            s[threadIdx.x >> 6] = reg;
-        __syncthreads();
+        const float t = block_sum_256(reg);
         if (threadIdx.x == 0)
-        {
-            float t = 0;
-            for (int k = 0; k < kBlock / 64; ++k)
-                t += s[k];
             reg_partial[blockIdx.x] = t;
-        }
     }
 }
 
@@ -244,22 +182,6 @@ int make_geom(AdaGeom& g, int64_t num_channel, int64_t num_element, int64_t n_pe
     g.offset      = offset;
     g.clip_min    = clip_min;
     g.clip_max    = clip_max;
-    return MIQ_OK;
-}
-
-int make_adam(AdamArgs& a, float reg_param, float beta, float lr, float beta1, float beta2, float eps, int step)
-{
-    MIQ_CHECK_ARG(beta1 >= 0.f && beta1 < 1.f && beta2 >= 0.f && beta2 < 1.f, "Adam betas must lie in [0, 1)");
-    a.reg_param = reg_param;
-    a.beta      = beta;
-    // bias corrections in double, as the Python floats of torch.optim.Adam are
-    const double bc1 = 1.0 - std::pow((double) beta1, (double) step);
-    const double bc2 = 1.0 - std::pow((double) beta2, (double) step);
-    a.lr_over_bc1    = (float) ((double) lr / bc1);
-    a.bc2_sqrt       = (float) std::sqrt(bc2);
-    a.beta1          = beta1;
-    a.beta2          = beta2;
-    a.eps            = eps;
     return MIQ_OK;
 }
 
@@ -359,7 +281,6 @@ int miq_adaround_bwd_adam_f32(const float* weight, const float* grad_weight, flo
     MIQ_CHECK_ARG(aligned16(weight) && aligned16(grad_weight) && aligned16(alpha) && aligned16(exp_avg) &&
                       aligned16(exp_avg_sq) && aligned16(grad_alpha),
                   "tensors must be 16-byte aligned");
-    MIQ_CHECK_ARG(step >= 1, "Adam step count starts at 1");
     AdamArgs a;
     if (int rc = make_adam(a, reg_param, beta, lr, beta1, beta2, eps, step))
         return rc;

@@ -1,0 +1,365 @@
+// AdaRound iteration of a Linear layer with the soft rounding fused into MFMA GEMMs (gfx950).
+//
+// Reference (ADA = TrainingExtensions/torch/src/python/aimet_torch/v1/adaround), one iteration of
+// AdaroundOptimizer._optimize_rounding (ADA/adaround_optimizer.py:182-218) for torch.nn.Linear:
+//   W'   = apply_adaround(W)                                   ADA/adaround_wrapper.py:124-149
+//   out  = functional.linear(x[batch], W', bias)               ADA/adaround_optimizer.py:276-277
+//   loss = recon_loss(act(out), act(y[batch])) + round_loss    ADA/adaround_loss.py:70-111
+//   loss.backward(); Adam step on alpha
+//
+// With 32 rows per iteration the GEMMs are bandwidth-bound on the weight-shaped operands, so the point of fusing is
+// that W' and dLoss/dW' never exist in memory:
+//   lin_fwd_kernel   reads W and alpha once, forms W' in registers and feeds it to 16x16x4 fp32 MFMAs as the B
+//                    operand; the K dimension is split over workgroups, partial [32, O] products go to a workspace
+//   lin_loss_kernel  adds the partials in a fixed order (deterministic), bias, activation, and writes
+//                    G = dLoss_recon/dout = 2 (act(out) - act(y)) act'(out) / batch
+//   lin_bwd_kernel   forms dLoss/dW'[o][k] = sum_b G[b][o] x[b][k] as a rank-32 MFMA product in registers and runs
+//                    the alpha-gradient + regulariser + Adam epilogue on it (reads W, alpha, m, v; writes alpha, m, v)
+//
+// MFMA operand layout used below (v_mfma_f32_16x16x4_f32, one wavefront): lane l supplies A[m = l % 16][k = l / 16]
+// and B[k = l / 16][n = l % 16]; it receives D[m = 4 (l / 16) + i][n = l % 16] in element i of the accumulator.
+#include "miq_adaround_math.h"
+
+namespace miq
+{
+namespace
+{
+using namespace ada;
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kBatch   = 32;    // rows per iteration (BATCH_SIZE of ADA/adaround_optimizer.py:58)
+constexpr int kFwdOBlk = 64;    // output channels per forward workgroup
+constexpr int kFwdKBlk = 256;   // K extent per forward workgroup (64 per wavefront)
+constexpr int kBwdOBlk = 32;    // output channels per backward workgroup
+constexpr int kBwdKBlk = 256;   // K extent per backward workgroup (64 per wavefront)
+
+struct LinGeom
+{
+    int out_features, in_features;
+    int chan_stride;      // 1: delta/offset per output channel, 0: one entry for the whole tensor
+    const float* delta;
+    const float* offset;
+    float clip_min, clip_max;
+};
+
+__device__ __forceinline__ v4f mfma16(float a, float b, v4f c)
+{
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ v4f ldg4(const float* p)
+{
+    return *reinterpret_cast<const v4f*>(p);
+}
+
+__device__ __forceinline__ v4f ldg4_stream(const float* p)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const v4f*>(p));
+}
+
+// grid (O / 64, K / 256), 256 threads.  Wavefront w of a workgroup takes k in [256 by + 64 w, +64).
+__global__ __launch_bounds__(256) void lin_fwd_kernel(const float* __restrict__ W, const float* __restrict__ alpha,
+                                                      const float* __restrict__ X, const int* __restrict__ row_index,
+                                                      int64_t x_row_stride, float* __restrict__ partial, LinGeom g)
+{
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n = lane & 15, s = lane >> 4;
+    const int o_blk = blockIdx.x * kFwdOBlk;
+    const int k_blk = blockIdx.y * kFwdKBlk + wave * 64;
+    const int K     = g.in_features;
+
+    float d[4], off[4];
+    const float* wrow[4];
+    const float* arow[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+    {
+        const int o = o_blk + nt * 16 + n;
+        d[nt]       = g.delta[o * g.chan_stride];
+        off[nt]     = g.offset[o * g.chan_stride];
+        wrow[nt]    = W + (int64_t) o * K;
+        arow[nt]    = alpha + (int64_t) o * K;
+    }
+    const float* xrow[2];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+    {
+        const int b = mt * 16 + n;
+        xrow[mt]    = X + (int64_t) (row_index ? row_index[b] : b) * x_row_stride;
+    }
+
+    v4f acc[2][4];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+            acc[mt][nt] = (v4f) {0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll 2
+    for (int kk = 0; kk < 64; kk += 16)
+    {
+        const int k = k_blk + kk + 4 * s;
+        v4f w[4], al[4], a[2];
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+        {
+            w[nt]  = ldg4_stream(wrow[nt] + k);
+            al[nt] = ldg4_stream(arow[nt] + k);
+        }
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+            a[mt] = ldg4(xrow[mt] + k);
+        v4f wq[4];
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                wq[nt][t] = adarounded<true>(w[nt][t], al[nt][t], d[nt], off[nt], g.clip_min, g.clip_max);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+                    acc[mt][nt] = mfma16(a[mt][t], wq[nt][t], acc[mt][nt]);
+    }
+
+    // add the four wavefronts' products in wavefront order, then one partial tile per workgroup
+    __shared__ v4f red[4][8][64];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+            red[wave][mt * 4 + nt][lane] = acc[mt][nt];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < 8 * 64; idx += 256)
+    {
+        const int tile = idx >> 6, ln = idx & 63;
+        const v4f sum  = ((red[0][tile][ln] + red[1][tile][ln]) + red[2][tile][ln]) + red[3][tile][ln];
+        const int mt = tile >> 2, nt = tile & 3;
+        const int o  = o_blk + nt * 16 + (ln & 15);
+        const int b0 = mt * 16 + 4 * (ln >> 4);
+        float* dst   = partial + ((int64_t) blockIdx.y * kBatch + b0) * g.out_features + o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            dst[(int64_t) i * g.out_features] = sum[i];
+    }
+}
+
+// one thread per (b, o): out = sum_s partial[s][b][o] + bias[o]; G = 2 (act(out) - act(y)) act'(out) / batch
+__global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__ partial, int num_split,
+                                                       const float* __restrict__ bias, const float* __restrict__ Y,
+                                                       const int* __restrict__ row_index, int64_t y_row_stride,
+                                                       int out_features, int act, float* __restrict__ out,
+                                                       float* __restrict__ G, float* __restrict__ loss_partial)
+{
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    float sq      = 0.f;
+    if (idx < kBatch * out_features)
+    {
+        const int b = idx / out_features, o = idx - b * out_features;
+        float acc = 0.f;
+        for (int s = 0; s < num_split; ++s)
+            acc += partial[((int64_t) s * kBatch + b) * out_features + o];
+        if (bias)
+            acc += bias[o];
+        float y = Y[(int64_t) (row_index ? row_index[b] : b) * y_row_stride + o];
+        if (out)
+            out[idx] = acc;
+        float pass = 1.f, ao = acc;
+        if (act == 1)
+        {
+            pass = acc > 0.f ? 1.f : 0.f;
+            ao   = fmaxf(acc, 0.f);
+            y    = fmaxf(y, 0.f);
+        }
+        const float diff = ao - y;
+        sq               = diff * diff;
+        G[idx]           = 2.0f * diff * pass * (1.0f / kBatch);
+    }
+    if (loss_partial)
+    {
+        const float t = block_sum_256(sq);
+        if (threadIdx.x == 0)
+            loss_partial[blockIdx.x] = t * (1.0f / kBatch);
+    }
+}
+
+// grid (O / 32, K / 256), 256 threads.  Wavefront w takes k in [256 by + 64 w, +64): four 16-wide k tiles (the M
+// dimension of the MFMA) by two 16-wide o tiles (N); the batch is the MFMA's K dimension, 8 steps of 4.
+__global__ __launch_bounds__(256) void lin_bwd_kernel(const float* __restrict__ W, const float* __restrict__ G,
+                                                      const float* __restrict__ X, const int* __restrict__ row_index,
+                                                      int64_t x_row_stride, float* __restrict__ alpha,
+                                                      float* __restrict__ m, float* __restrict__ v,
+                                                      float* __restrict__ grad_out, LinGeom g, AdamArgs a,
+                                                      float* __restrict__ reg_partial)
+{
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n = lane & 15, s = lane >> 4;
+    const int o_blk = blockIdx.x * kBwdOBlk;
+    const int k_blk = blockIdx.y * kBwdKBlk + wave * 64;
+    const int K = g.in_features, O = g.out_features;
+
+    v4f acc[4][2];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+            acc[mt][nt] = (v4f) {0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+    for (int step = 0; step < 8; ++step)
+    {
+        const int b       = 4 * step + s;
+        const float* xrow = X + (int64_t) (row_index ? row_index[b] : b) * x_row_stride + k_blk + n;
+        const float* grow = G + (int64_t) b * O + o_blk + n;
+        float xa[4], gb[2];
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+            xa[mt] = xrow[mt * 16];
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+            gb[nt] = grow[nt * 16];
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+                acc[mt][nt] = mfma16(xa[mt], gb[nt], acc[mt][nt]);
+    }
+
+    // lane holds dW'[o = o_blk + 16 nt + n][k = k_blk + 16 mt + 4 s + i], i = 0..3: one 16-byte vector per tile
+    float reg = 0.f;
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt)
+    {
+        const int o   = o_blk + nt * 16 + n;
+        const float d = g.delta[o * g.chan_stride], off = g.offset[o * g.chan_stride];
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+        {
+            const int64_t e = (int64_t) o * K + k_blk + mt * 16 + 4 * s;
+            const v4f wv    = ldg4_stream(W + e);
+            const v4f av    = ldg4(alpha + e);
+            const v4f mv    = ldg4(m + e);
+            const v4f vv    = ldg4(v + e);
+            float as[4] = {av[0], av[1], av[2], av[3]}, ms[4] = {mv[0], mv[1], mv[2], mv[3]};
+            float vs[4] = {vv[0], vv[1], vv[2], vv[3]};
+            v4f gr;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                float r;
+                const float gi = alpha_grad(wv[i], acc[mt][nt][i], as[i], d, off, g.clip_min, g.clip_max, a, r);
+                reg += r;
+                adam_update(gi, as[i], ms[i], vs[i], a);
+                gr[i] = gi;
+            }
+            *reinterpret_cast<v4f*>(alpha + e) = (v4f) {as[0], as[1], as[2], as[3]};
+            *reinterpret_cast<v4f*>(m + e)     = (v4f) {ms[0], ms[1], ms[2], ms[3]};
+            *reinterpret_cast<v4f*>(v + e)     = (v4f) {vs[0], vs[1], vs[2], vs[3]};
+            if (grad_out)
+                *reinterpret_cast<v4f*>(grad_out + e) = gr;
+        }
+    }
+    if (reg_partial)
+    {
+        const float t = block_sum_256(reg);
+        if (threadIdx.x == 0)
+            reg_partial[blockIdx.y * gridDim.x + blockIdx.x] = t;
+    }
+}
+
+int make_lin_geom(LinGeom& g, int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
+                  const float* offset, float clip_min, float clip_max)
+{
+    MIQ_CHECK_ARG(out_features > 0 && in_features > 0, "bad layer shape");
+    MIQ_CHECK_ARG(out_features % kFwdOBlk == 0 && in_features % kFwdKBlk == 0,
+                  "the fused Linear path takes out_features that are a multiple of 64 and in_features that are a "
+                  "multiple of 256 (got %lld x %lld)", (long long) out_features, (long long) in_features);
+    MIQ_CHECK_ARG(out_features * in_features < (1ll << 31), "layer too large for the fused Linear path");
+    MIQ_CHECK_ARG(num_channel == 1 || num_channel == out_features,
+                  "delta/offset must have one entry, or one per output channel");
+    MIQ_CHECK_ARG(delta && offset, "null delta/offset");
+    MIQ_CHECK_ARG(clip_min <= clip_max, "clip_min must not exceed clip_max");
+    g.out_features = (int) out_features;
+    g.in_features  = (int) in_features;
+    g.chan_stride  = num_channel == 1 ? 0 : 1;
+    g.delta        = delta;
+    g.offset       = offset;
+    g.clip_min     = clip_min;
+    g.clip_max     = clip_max;
+    return MIQ_OK;
+}
+}   // namespace
+}   // namespace miq
+
+using namespace miq;
+
+extern "C" {
+
+int64_t miq_adaround_linear_workspace_bytes(int64_t out_features, int64_t in_features)
+{
+    if (out_features <= 0 || in_features <= 0)
+        return 0;
+    const int64_t splits = (in_features + kFwdKBlk - 1) / kFwdKBlk;
+    return splits * kBatch * out_features * (int64_t) sizeof(float);
+}
+
+int miq_adaround_linear_blocks(int64_t out_features, int64_t in_features)
+{
+    return (int) ((out_features / kBwdOBlk) * (in_features / kBwdKBlk));
+}
+
+int miq_adaround_linear_fwd_f32(const float* weight, const float* alpha, const float* x, const int32_t* row_index,
+                                int64_t x_row_stride, const float* target, int64_t target_row_stride,
+                                const float* bias, int64_t out_features, int64_t in_features, int64_t num_channel,
+                                const float* delta, const float* offset, float clip_min, float clip_max,
+                                int activation, float* workspace, float* out, float* grad_out, float* loss_partial,
+                                void* stream)
+{
+    LinGeom g;
+    if (int rc = make_lin_geom(g, out_features, in_features, num_channel, delta, offset, clip_min, clip_max))
+        return rc;
+    MIQ_CHECK_ARG(weight && alpha && x && target && workspace && grad_out, "null tensor pointer");
+    MIQ_CHECK_ARG(aligned16(weight) && aligned16(alpha) && aligned16(x) && (x_row_stride % 4) == 0,
+                  "weight, alpha and the rows of x must be 16-byte aligned");
+    MIQ_CHECK_ARG(x_row_stride >= in_features && target_row_stride >= out_features, "row stride shorter than a row");
+    MIQ_CHECK_ARG(activation == 0 || activation == 1, "activation must be 0 (none) or 1 (ReLU)");
+    const int splits = (int) (in_features / kFwdKBlk);
+    hipLaunchKernelGGL(lin_fwd_kernel, dim3((unsigned) (out_features / kFwdOBlk), (unsigned) splits), dim3(256), 0,
+                       (hipStream_t) stream, weight, alpha, x, row_index, x_row_stride, workspace, g);
+    MIQ_CHECK_LAUNCH();
+    const unsigned blocks = (unsigned) ((kBatch * out_features + 255) / 256);
+    hipLaunchKernelGGL(lin_loss_kernel, dim3(blocks), dim3(256), 0, (hipStream_t) stream, workspace, splits, bias, target,
+                       row_index, target_row_stride, (int) out_features, activation, out, grad_out, loss_partial);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int miq_adaround_linear_bwd_adam_f32(const float* weight, const float* grad_out, const float* x,
+                                     const int32_t* row_index, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                     float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
+                                     int64_t num_channel, const float* delta, const float* offset, float clip_min,
+                                     float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
+                                     float eps, int step, float* reg_partial, void* stream)
+{
+    LinGeom g;
+    if (int rc = make_lin_geom(g, out_features, in_features, num_channel, delta, offset, clip_min, clip_max))
+        return rc;
+    MIQ_CHECK_ARG(weight && grad_out && x && alpha && exp_avg && exp_avg_sq, "null tensor pointer");
+    MIQ_CHECK_ARG(aligned16(weight) && aligned16(alpha) && aligned16(exp_avg) && aligned16(exp_avg_sq) &&
+                      aligned16(grad_alpha),
+                  "tensors must be 16-byte aligned");
+    MIQ_CHECK_ARG(x_row_stride >= in_features, "row stride shorter than a row");
+    AdamArgs a;
+    if (int rc = make_adam(a, reg_param, beta, lr, beta1, beta2, eps, step))
+        return rc;
+    hipLaunchKernelGGL(lin_bwd_kernel, dim3((unsigned) (out_features / kBwdOBlk), (unsigned) (in_features / kBwdKBlk)),
+                       dim3(256), 0, (hipStream_t) stream, weight, grad_out, x, row_index, x_row_stride, alpha, exp_avg,
+                       exp_avg_sq, grad_alpha, g, a, reg_partial);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+}   // extern "C"

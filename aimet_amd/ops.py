@@ -286,6 +286,55 @@ def adaround_bwd_adam(weight, grad_weight, alpha, exp_avg, exp_avg_sq, num_chann
                                             float(eps), int(step), _ptr(reg_partial), _stream(weight)))
 
 
+def adaround_linear_supported(out_features, in_features, batch):
+    """Shapes the MFMA-fused Linear path takes."""
+    return batch == 32 and out_features % 64 == 0 and in_features % 256 == 0 and \
+        out_features * in_features < 2 ** 31
+
+
+def adaround_linear_workspace(out_features, in_features, device):
+    nbytes = int(lib.miq_adaround_linear_workspace_bytes(int(out_features), int(in_features)))
+    return torch.empty(nbytes // 4, dtype=_F32, device=device)
+
+
+def adaround_linear_blocks(out_features, in_features):
+    return int(lib.miq_adaround_linear_blocks(int(out_features), int(in_features)))
+
+
+def adaround_linear_fwd(weight, alpha, x, row_index, target, bias, num_channel, delta, offset, clip_min, clip_max,
+                        activation, workspace, grad_out, out=None, loss_partial=None):
+    """Fused apply_adaround + Linear forward + reconstruction-loss gradient for 32 rows of x / target."""
+    _ada_check(weight, alpha, workspace, grad_out, out)
+    _require_gpu(weight, x, target, bias, row_index)
+    if x.dtype != _F32 or target.dtype != _F32 or x.stride(-1) != 1 or target.stride(-1) != 1:
+        raise RuntimeError("x and target must be float32 with contiguous rows")
+    if row_index is not None and (row_index.dtype != torch.int32 or row_index.numel() != 32):
+        raise RuntimeError("row_index must hold 32 int32 row numbers")
+    o, k = weight.shape
+    with torch.cuda.device(weight.device):
+        check(lib.miq_adaround_linear_fwd_f32(_ptr(weight), _ptr(alpha), _ptr(x), _ptr(row_index), x.stride(0),
+                                              _ptr(target), target.stride(0), _ptr(bias), o, k, int(num_channel),
+                                              _ptr(delta), _ptr(offset), float(clip_min), float(clip_max),
+                                              int(activation), _ptr(workspace), _ptr(out), _ptr(grad_out),
+                                              _ptr(loss_partial), _stream(weight)))
+
+
+def adaround_linear_bwd_adam(weight, grad_out, x, row_index, alpha, exp_avg, exp_avg_sq, num_channel, delta, offset,
+                             clip_min, clip_max, reg_param, beta, lr, beta1, beta2, eps, step, reg_partial=None,
+                             grad_alpha=None):
+    """Fused dLoss/dW' = grad_out^T x (MFMA) + alpha gradient + regulariser + Adam update (alpha, moments in place)."""
+    _ada_check(weight, grad_out, alpha, exp_avg, exp_avg_sq, grad_alpha)
+    _require_gpu(weight, x, row_index)
+    o, k = weight.shape
+    with torch.cuda.device(weight.device):
+        check(lib.miq_adaround_linear_bwd_adam_f32(_ptr(weight), _ptr(grad_out), _ptr(x), _ptr(row_index),
+                                                   x.stride(0), _ptr(alpha), _ptr(exp_avg), _ptr(exp_avg_sq),
+                                                   _ptr(grad_alpha), o, k, int(num_channel), _ptr(delta),
+                                                   _ptr(offset), float(clip_min), float(clip_max), float(reg_param),
+                                                   float(beta), float(lr), float(beta1), float(beta2), float(eps),
+                                                   int(step), _ptr(reg_partial), _stream(weight)))
+
+
 class Analyzer:
     """Device-resident encoding analyzer (TF min/max or TF-Enhanced 512-bucket PDF + SQNR search)."""
 

@@ -26,6 +26,10 @@ ADAM_LR, ADAM_BETAS, ADAM_EPS = 1e-3, (0.9, 0.999), 1e-8      # torch.optim.Adam
 class AdaroundOptimizer:
     """Optimizes the weight rounding of a quantized wrapper module."""
 
+    # Linear layers whose shape the MFMA-fused kernels take (out % 64 == 0, in % 256 == 0, batch 32, no activation or
+    # ReLU) use them; everything else runs soft-round kernel + torch layer + fused backward/Adam kernel
+    use_fused_linear = True
+
     @classmethod
     def adaround_module(cls, module: torch.nn.Module, quant_module: AdaroundWrapper, orig_model: torch.nn.Module,
                         quant_model: torch.nn.Module, act_func: Union[torch.nn.Module, None], cached_dataset,
@@ -72,11 +76,42 @@ class AdaroundOptimizer:
         grad_alpha = torch.empty_like(alpha)
         if batches is None:
             n = all_inp_data.size(0)
-            batches = (torch.randperm(n)[:BATCH_SIZE] for _ in range(opt_params.num_iterations))
+            batches = [torch.randperm(n)[:BATCH_SIZE] for _ in range(opt_params.num_iterations)]
+        else:
+            batches = list(batches)
+        if not batches:
+            return exp_avg, exp_avg_sq
 
-        step = 0
+        def beta_of(iteration):
+            if AdaroundLoss.in_warm_start(opt_params, iteration):
+                return -1.0
+            return AdaroundLoss._compute_beta(opt_params.num_iterations, iteration,  # pylint: disable=protected-access
+                                              opt_params.beta_range, opt_params.warm_start)
+
+        activation = cls._fused_activation_code(act_func)
+        module = qm.get_original_module()
+        if cls.use_fused_linear and activation is not None and \
+                cls._fused_linear_applies(module, weight, qm, all_inp_data, all_orig_out_data, batches):
+            # soft rounding fused into the MFMA GEMMs: three launches per iteration, nothing weight-shaped is
+            # written except alpha and the Adam moments
+            index = torch.stack(batches).to(dtype=torch.int32, device=device).contiguous()
+            bias = None if module.bias is None else module.bias.detach().to(torch.float32).contiguous()
+            out_features, in_features = weight.shape
+            workspace = ops.adaround_linear_workspace(out_features, in_features, device)
+            grad_out = torch.empty(BATCH_SIZE, out_features, dtype=torch.float32, device=device)
+            for k in range(len(batches)):
+                ops.adaround_linear_fwd(weight, alpha, all_inp_data, index[k], all_orig_out_data, bias,
+                                        qm.num_channel, qm.delta, qm.offset, qm.clip_min, qm.clip_max, activation,
+                                        workspace, grad_out)
+                ops.adaround_linear_bwd_adam(weight, grad_out, all_inp_data, index[k], alpha, exp_avg, exp_avg_sq,
+                                             qm.num_channel, qm.delta, qm.offset, qm.clip_min, qm.clip_max,
+                                             opt_params.reg_param, beta_of(first_iteration + k), ADAM_LR,
+                                             ADAM_BETAS[0], ADAM_BETAS[1], ADAM_EPS, k + 1,
+                                             grad_alpha=grad_alpha if k == len(batches) - 1 else None)
+            qm.alpha.grad = grad_alpha
+            return exp_avg, exp_avg_sq
+
         for k, indices in enumerate(batches):
-            iteration = first_iteration + k
             indices = indices.to(device)
             inp_data = all_inp_data[indices]
             orig_out_data = all_orig_out_data[indices]
@@ -84,26 +119,39 @@ class AdaroundOptimizer:
             ada_weight = ops.adaround_soft_round(weight, alpha, qm.num_channel, qm.n_per_channel, qm.delta, qm.offset,
                                                  qm.clip_min, qm.clip_max, True)
             ada_weight.requires_grad_(True)
-            quant_out_data = cls._layer_output(qm.get_original_module(), inp_data, ada_weight)
+            quant_out_data = cls._layer_output(module, inp_data, ada_weight)
             if act_func is not None:
                 orig_out_data = act_func(orig_out_data)
                 quant_out_data = act_func(quant_out_data)
             recon_loss = AdaroundLoss.compute_recon_loss(quant_out_data, orig_out_data)
             grad_weight, = torch.autograd.grad(recon_loss, ada_weight)
-
-            if AdaroundLoss.in_warm_start(opt_params, iteration):
-                beta = -1.0
-            else:
-                beta = AdaroundLoss._compute_beta(opt_params.num_iterations, iteration,  # pylint: disable=protected-access
-                                                  opt_params.beta_range, opt_params.warm_start)
-            step += 1
             ops.adaround_bwd_adam(weight, grad_weight.contiguous(), alpha, exp_avg, exp_avg_sq, qm.num_channel,
                                   qm.n_per_channel, qm.delta, qm.offset, qm.clip_min, qm.clip_max,
-                                  opt_params.reg_param, beta, ADAM_LR, ADAM_BETAS[0], ADAM_BETAS[1], ADAM_EPS, step,
-                                  grad_alpha=grad_alpha)
-        if step:
-            qm.alpha.grad = grad_alpha
+                                  opt_params.reg_param, beta_of(first_iteration + k), ADAM_LR, ADAM_BETAS[0],
+                                  ADAM_BETAS[1], ADAM_EPS, k + 1,
+                                  grad_alpha=grad_alpha if k == len(batches) - 1 else None)
+        qm.alpha.grad = grad_alpha
         return exp_avg, exp_avg_sq
+
+    @staticmethod
+    def _fused_activation_code(act_func):
+        """0 / 1 for the activations the fused Linear kernels implement (none / ReLU), else None."""
+        if act_func is None:
+            return 0
+        if isinstance(act_func, torch.nn.ReLU) or act_func in (torch.relu, functional.relu):
+            return 1
+        return None
+
+    @staticmethod
+    def _fused_linear_applies(module, weight, qm, all_inp_data, all_orig_out_data, batches) -> bool:
+        if not isinstance(module, torch.nn.Linear) or weight.dim() != 2:
+            return False
+        out_features, in_features = weight.shape
+        per_channel_ok = qm.num_channel == 1 or (qm.num_channel == out_features and qm.n_per_channel == in_features)
+        data_ok = all(t.dim() == 2 and t.dtype == torch.float32 and t.stride(1) == 1 and t.stride(0) % 4 == 0 and
+                      t.data_ptr() % 16 == 0 for t in (all_inp_data, all_orig_out_data))
+        return per_channel_ok and data_ok and all(b.numel() == BATCH_SIZE for b in batches) and \
+            ops.adaround_linear_supported(out_features, in_features, BATCH_SIZE)
 
     @classmethod
     def _compute_recons_metrics(cls, quant_module: AdaroundWrapper, act_func, inp_data: torch.Tensor,
