@@ -64,6 +64,7 @@ _SIGNATURES = {
     "miq_analyzer_last_batch_counts": ([_p, _p, _p], _int),
     "miq_analyzer_last_search": ([_p, _p, _p, _p, _int, C.POINTER(_int), C.POINTER(_int), _p], _int),
     "miq_adaround_soft_round_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int, _p], _int),
+    "miq_adaround_floor_f32": ([_p, _p, _i64, _i64, _i64, _p, _p], _int),
     "miq_adaround_init_alpha_f32": ([_p, _p, _i64, _i64, _i64, _p, _p], _int),
     "miq_adaround_bwd_adam_f32": ([_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _flt, _flt, _flt,
                                    _flt, _flt, _flt, _int, _p, _p], _int),

@@ -29,7 +29,7 @@ int make_adam(AdamArgs& a, float reg_param, float beta, float lr, float beta1, f
     const double bc1 = 1.0 - std::pow((double) beta1, (double) step);
     const double bc2 = 1.0 - std::pow((double) beta2, (double) step);
     a.lr_over_bc1    = (float) ((double) lr / bc1);
-    a.bc2_sqrt       = (float) std::sqrt(bc2);
+    a.inv_bc2_sqrt   = (float) (1.0 / std::sqrt(bc2));
     a.beta1          = beta1;
     a.beta2          = beta2;
     a.eps            = eps;
@@ -85,6 +85,12 @@ __global__ __launch_bounds__(kBlock) void soft_round_kernel(const float* __restr
         const uint32_t c = channel_of(e, g);
         out[e] = adarounded<SOFT>(w[e], alpha[e], g.delta[c], g.offset[c], g.clip_min, g.clip_max);
     }
+}
+
+__global__ __launch_bounds__(kBlock) void floor_kernel(const float* __restrict__ w, float* __restrict__ out, AdaGeom g)
+{
+    for (int64_t e = (int64_t) blockIdx.x * kBlock + threadIdx.x; e < g.n; e += (int64_t) gridDim.x * kBlock)
+        out[e] = floorf(w[e] / g.delta[channel_of(e, g)]);
 }
 
 __global__ __launch_bounds__(kBlock) void init_alpha_kernel(const float* __restrict__ w, float* __restrict__ alpha,
@@ -221,6 +227,24 @@ int miq_adaround_soft_round_f32(const float* weight, const float* alpha, float* 
     else
         hipLaunchKernelGGL(soft_round_kernel<false>, dim3(vec_blocks(num_element)), dim3(kBlock), 0,
                            (hipStream_t) stream, weight, alpha, out, g);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int miq_adaround_floor_f32(const float* weight, float* weight_floor, int64_t num_channel, int64_t num_element,
+                           int64_t num_element_per_channel, const float* delta, void* stream)
+{
+    AdaGeom g;
+    if (int rc = make_geom(g, num_channel, num_element, num_element_per_channel, delta, delta, 0.f, 0.f))
+        return rc;
+    if (num_element == 0)
+        return MIQ_OK;
+    MIQ_CHECK_ARG(weight && weight_floor, "null tensor pointer");
+    int64_t blocks = (num_element + kBlock - 1) / kBlock;
+    if (blocks > 65536)
+        blocks = 65536;
+    hipLaunchKernelGGL(floor_kernel, dim3((unsigned) blocks), dim3(kBlock), 0, (hipStream_t) stream, weight, weight_floor,
+                       g);
     MIQ_CHECK_LAUNCH();
     return MIQ_OK;
 }

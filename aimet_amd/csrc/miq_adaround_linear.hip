@@ -9,7 +9,8 @@
 //
 // With 32 rows per iteration the GEMMs are bandwidth-bound on the weight-shaped operands, so the point of fusing is
 // that W' and dLoss/dW' never exist in memory:
-//   lin_fwd_kernel   reads W and alpha once, forms W' in registers and feeds it to 16x16x4 fp32 MFMAs as the B
+//   (W enters as F = floor(W / delta), computed once per layer: W and delta do not change during the optimisation)
+//   lin_fwd_kernel   reads F and alpha once, forms W' in registers and feeds it to 16x16x4 fp32 MFMAs as the B
 //                    operand; the K dimension is split over workgroups, partial [32, O] products go to a workspace
 //   lin_loss_kernel  adds the partials in a fixed order (deterministic), bias, activation, and writes
 //                    G = dLoss_recon/dout = 2 (act(out) - act(y)) act'(out) / batch
@@ -115,7 +116,7 @@ __global__ __launch_bounds__(256) void lin_fwd_kernel(const float* __restrict__ 
         for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
             for (int t = 0; t < 4; ++t)
-                wq[nt][t] = adarounded<true>(w[nt][t], al[nt][t], d[nt], off[nt], g.clip_min, g.clip_max);
+                wq[nt][t] = adarounded_f<true>(w[nt][t], al[nt][t], d[nt], off[nt], g.clip_min, g.clip_max);
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -250,7 +251,7 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const float* __restrict__ 
             for (int i = 0; i < 4; ++i)
             {
                 float r;
-                const float gi = alpha_grad(wv[i], acc[mt][nt][i], as[i], d, off, g.clip_min, g.clip_max, a, r);
+                const float gi = alpha_grad_f(wv[i], acc[mt][nt][i], as[i], d, off, g.clip_min, g.clip_max, a, r);
                 reg += r;
                 adam_update(gi, as[i], ms[i], vs[i], a);
                 gr[i] = gi;

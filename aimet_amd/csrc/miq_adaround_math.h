@@ -28,7 +28,7 @@ struct AdamArgs
     float reg_param;
     float beta;        // exponent of the regulariser; < 0 during warm start (no rounding loss)
     float lr_over_bc1; // lr / (1 - beta1^t)
-    float bc2_sqrt;    // sqrt(1 - beta2^t)
+    float inv_bc2_sqrt; // 1 / sqrt(1 - beta2^t)
     float beta1, beta2, eps;
 };
 
@@ -57,23 +57,28 @@ __device__ __forceinline__ float hard_h(float alpha)
     return alpha >= 0.0f ? 1.0f : 0.0f;
 }
 
+// `f` = floor(w / delta), an IEEE-exact division: it decides the grid point
 template <bool SOFT>
-__device__ __forceinline__ float adarounded(float w, float alpha, float d, float o, float clip_min, float clip_max)
+__device__ __forceinline__ float adarounded_f(float f, float alpha, float d, float o, float clip_min, float clip_max)
 {
-    const float f = floorf(w / d);
     float sig, inner;
     const float h = SOFT ? soft_h(alpha, sig, inner) : hard_h(alpha);
     const float q = fminf(fmaxf(f + h - o, clip_min), clip_max);
     return (q + o) * d;
 }
 
+template <bool SOFT>
+__device__ __forceinline__ float adarounded(float w, float alpha, float d, float o, float clip_min, float clip_max)
+{
+    return adarounded_f<SOFT>(floorf(w / d), alpha, d, o, clip_min, clip_max);
+}
+
 // dLoss/dalpha of one element from gw = dLoss_recon/dW': chain rule of `adarounded` (closed-interval clamp gradients,
 // as torch.clamp) plus the gradient of reg_param * (1 - |2h - 1|^beta); `reg` receives this element's regulariser
 // term (0 in warm start)
-__device__ __forceinline__ float alpha_grad(float w, float gw, float alpha, float d, float o, float clip_min,
-                                            float clip_max, const AdamArgs& a, float& reg)
+__device__ __forceinline__ float alpha_grad_f(float f, float gw, float alpha, float d, float o, float clip_min,
+                                              float clip_max, const AdamArgs& a, float& reg)
 {
-    const float f = floorf(w / d);
     float sig, inner;
     const float h      = soft_h(alpha, sig, inner);
     const float t      = f + h - o;
@@ -95,13 +100,21 @@ __device__ __forceinline__ float alpha_grad(float w, float gw, float alpha, floa
     return grad;
 }
 
+__device__ __forceinline__ float alpha_grad(float w, float gw, float alpha, float d, float o, float clip_min,
+                                            float clip_max, const AdamArgs& a, float& reg)
+{
+    return alpha_grad_f(floorf(w / d), gw, alpha, d, o, clip_min, clip_max, a, reg);
+}
+
 // lerp for the first moment, mul/addcmul for the second, as torch's single-tensor Adam orders them
 __device__ __forceinline__ void adam_update(float grad, float& alpha, float& m, float& v, const AdamArgs& a)
 {
     m = m + (1.0f - a.beta1) * (grad - m);
     v = v * a.beta2 + (1.0f - a.beta2) * grad * grad;
-    const float denom = sqrtf(v) / a.bc2_sqrt + a.eps;
-    alpha             = alpha - a.lr_over_bc1 * (m / denom);
+    // sqrt and the two divisions through the hardware's one-ulp sqrt / reciprocal: the step is lr-sized (1e-3), so the
+    // last-bit differences against exact division are ~1e-10 in alpha
+    const float denom = __builtin_amdgcn_sqrtf(v) * a.inv_bc2_sqrt + a.eps;
+    alpha             = alpha - a.lr_over_bc1 * (m * __builtin_amdgcn_rcpf(denom));
 }
 
 // bias corrections in double, as the Python floats of torch.optim.Adam are

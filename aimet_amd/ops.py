@@ -244,6 +244,16 @@ def adaround_soft_round(weight, alpha, num_channel, n_per_channel, delta, offset
     return out
 
 
+def adaround_floor(weight, num_channel, n_per_channel, delta):
+    """floor(w / delta): the alpha-independent part of apply_adaround, input of the fused Linear kernels."""
+    _ada_check(weight)
+    out = torch.empty_like(weight)
+    with torch.cuda.device(weight.device):
+        check(lib.miq_adaround_floor_f32(_ptr(weight), _ptr(out), int(num_channel), weight.numel(),
+                                         int(n_per_channel), _ptr(delta), _stream(weight)))
+    return out
+
+
 def adaround_init_alpha(weight, num_channel, n_per_channel, delta):
     """alpha such that h(alpha) equals the fractional part of w / delta."""
     _ada_check(weight)
@@ -301,38 +311,38 @@ def adaround_linear_blocks(out_features, in_features):
     return int(lib.miq_adaround_linear_blocks(int(out_features), int(in_features)))
 
 
-def adaround_linear_fwd(weight, alpha, x, row_index, target, bias, num_channel, delta, offset, clip_min, clip_max,
+def adaround_linear_fwd(weight_floor, alpha, x, row_index, target, bias, num_channel, delta, offset, clip_min, clip_max,
                         activation, workspace, grad_out, out=None, loss_partial=None):
     """Fused apply_adaround + Linear forward + reconstruction-loss gradient for 32 rows of x / target."""
-    _ada_check(weight, alpha, workspace, grad_out, out)
-    _require_gpu(weight, x, target, bias, row_index)
+    _ada_check(weight_floor, alpha, workspace, grad_out, out)
+    _require_gpu(weight_floor, x, target, bias, row_index)
     if x.dtype != _F32 or target.dtype != _F32 or x.stride(-1) != 1 or target.stride(-1) != 1:
         raise RuntimeError("x and target must be float32 with contiguous rows")
     if row_index is not None and (row_index.dtype != torch.int32 or row_index.numel() != 32):
         raise RuntimeError("row_index must hold 32 int32 row numbers")
-    o, k = weight.shape
-    with torch.cuda.device(weight.device):
-        check(lib.miq_adaround_linear_fwd_f32(_ptr(weight), _ptr(alpha), _ptr(x), _ptr(row_index), x.stride(0),
+    o, k = weight_floor.shape
+    with torch.cuda.device(weight_floor.device):
+        check(lib.miq_adaround_linear_fwd_f32(_ptr(weight_floor), _ptr(alpha), _ptr(x), _ptr(row_index), x.stride(0),
                                               _ptr(target), target.stride(0), _ptr(bias), o, k, int(num_channel),
                                               _ptr(delta), _ptr(offset), float(clip_min), float(clip_max),
                                               int(activation), _ptr(workspace), _ptr(out), _ptr(grad_out),
-                                              _ptr(loss_partial), _stream(weight)))
+                                              _ptr(loss_partial), _stream(weight_floor)))
 
 
-def adaround_linear_bwd_adam(weight, grad_out, x, row_index, alpha, exp_avg, exp_avg_sq, num_channel, delta, offset,
+def adaround_linear_bwd_adam(weight_floor, grad_out, x, row_index, alpha, exp_avg, exp_avg_sq, num_channel, delta, offset,
                              clip_min, clip_max, reg_param, beta, lr, beta1, beta2, eps, step, reg_partial=None,
                              grad_alpha=None):
     """Fused dLoss/dW' = grad_out^T x (MFMA) + alpha gradient + regulariser + Adam update (alpha, moments in place)."""
-    _ada_check(weight, grad_out, alpha, exp_avg, exp_avg_sq, grad_alpha)
-    _require_gpu(weight, x, row_index)
-    o, k = weight.shape
-    with torch.cuda.device(weight.device):
-        check(lib.miq_adaround_linear_bwd_adam_f32(_ptr(weight), _ptr(grad_out), _ptr(x), _ptr(row_index),
+    _ada_check(weight_floor, grad_out, alpha, exp_avg, exp_avg_sq, grad_alpha)
+    _require_gpu(weight_floor, x, row_index)
+    o, k = weight_floor.shape
+    with torch.cuda.device(weight_floor.device):
+        check(lib.miq_adaround_linear_bwd_adam_f32(_ptr(weight_floor), _ptr(grad_out), _ptr(x), _ptr(row_index),
                                                    x.stride(0), _ptr(alpha), _ptr(exp_avg), _ptr(exp_avg_sq),
                                                    _ptr(grad_alpha), o, k, int(num_channel), _ptr(delta),
                                                    _ptr(offset), float(clip_min), float(clip_max), float(reg_param),
                                                    float(beta), float(lr), float(beta1), float(beta2), float(eps),
-                                                   int(step), _ptr(reg_partial), _stream(weight)))
+                                                   int(step), _ptr(reg_partial), _stream(weight_floor)))
 
 
 class Analyzer:

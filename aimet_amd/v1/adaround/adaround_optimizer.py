@@ -94,16 +94,17 @@ class AdaroundOptimizer:
                 cls._fused_linear_applies(module, weight, qm, all_inp_data, all_orig_out_data, batches):
             # soft rounding fused into the MFMA GEMMs: three launches per iteration, nothing weight-shaped is
             # written except alpha and the Adam moments
+            weight_floor = ops.adaround_floor(weight, qm.num_channel, qm.n_per_channel, qm.delta)
             index = torch.stack(batches).to(dtype=torch.int32, device=device).contiguous()
             bias = None if module.bias is None else module.bias.detach().to(torch.float32).contiguous()
             out_features, in_features = weight.shape
             workspace = ops.adaround_linear_workspace(out_features, in_features, device)
             grad_out = torch.empty(BATCH_SIZE, out_features, dtype=torch.float32, device=device)
             for k in range(len(batches)):
-                ops.adaround_linear_fwd(weight, alpha, all_inp_data, index[k], all_orig_out_data, bias,
+                ops.adaround_linear_fwd(weight_floor, alpha, all_inp_data, index[k], all_orig_out_data, bias,
                                         qm.num_channel, qm.delta, qm.offset, qm.clip_min, qm.clip_max, activation,
                                         workspace, grad_out)
-                ops.adaround_linear_bwd_adam(weight, grad_out, all_inp_data, index[k], alpha, exp_avg, exp_avg_sq,
+                ops.adaround_linear_bwd_adam(weight_floor, grad_out, all_inp_data, index[k], alpha, exp_avg, exp_avg_sq,
                                              qm.num_channel, qm.delta, qm.offset, qm.clip_min, qm.clip_max,
                                              opt_params.reg_param, beta_of(first_iteration + k), ADAM_LR,
                                              ADAM_BETAS[0], ADAM_BETAS[1], ADAM_EPS, k + 1,

@@ -175,6 +175,117 @@ def bench_calibration(torch, ops, reps):
             "encoding": [enc.min, enc.max, enc.delta, enc.offset]}
 
 
+def _adaround_layer(torch, seed=1005, out_features=4096, in_features=4096, rows=2048):
+    """cfg5 objects: Linear [4096,4096] fp32, W ~ N(0, 0.02); X [2048,4096] ~ N(0,1); Y = X W^T; 4-bit per-channel."""
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.adaround.adaround_wrapper import AdaroundWrapper
+    from aimet_amd.v1.qc_quantize_op import StaticGridQuantWrapper
+    dev = torch.device("cuda", 0)
+    g = torch.Generator(device=dev).manual_seed(seed)
+    lin = torch.nn.Linear(in_features, out_features, bias=False).to(dev)
+    lin.weight.data = torch.randn(out_features, in_features, device=dev, generator=g) * 0.02
+    x = torch.randn(rows, in_features, device=dev, generator=g)
+    y = torch.nn.functional.linear(x, lin.weight.data)
+    qw = StaticGridQuantWrapper(lin, 4, 8, round_mode='nearest', quant_scheme=QuantScheme.post_training_tf,
+                                is_symmetric=True)
+    qw.enable_per_channel_quantization()
+    q = qw.param_quantizers['weight']
+    q.update_encoding_stats(lin.weight.data)
+    q.compute_encoding()
+    return AdaroundWrapper(qw), x, y
+
+
+def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
+    """AdaRound inner loop of one Linear [4096,4096] layer (cfg5): whole loop wall-clock through AdaroundOptimizer, then
+    the three kernels of one iteration timed with events."""
+    from aimet_amd.v1.adaround.adaround_loss import AdaroundHyperParameters
+    from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
+    wrapper, x, y = _adaround_layer(torch)
+    n = wrapper.weight.numel()
+    o, k = wrapper.weight.shape
+    params = AdaroundHyperParameters(iterations, 0.01, (20, 2), 0.2)
+    torch.manual_seed(1005)
+    batches = [torch.randperm(x.size(0))[:32] for _ in range(iterations)]
+    res = {"layer": [o, k], "rows_cached": x.size(0), "batch": 32, "bitwidth": 4, "iterations": iterations}
+    for name, fused in (("fused_mfma", True), ("elementwise_plus_torch_gemm", False)):
+        AdaroundOptimizer.use_fused_linear = fused
+        alpha0 = wrapper.alpha.data.clone()
+        AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, x, y, params, batches=batches[:20])  # warm-up
+        wrapper.alpha.data.copy_(alpha0)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, x, y, params, batches=batches)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        res[name] = {"ms_per_iteration": dt * 1e3 / iterations, "iterations_per_s": iterations / dt}
+        if not fused:
+            wrapper.alpha.data.copy_(alpha0)
+    AdaroundOptimizer.use_fused_linear = True
+
+    # per-kernel times of the fused iteration
+    w = ops.adaround_floor(wrapper.weight.detach(), wrapper.num_channel, wrapper.n_per_channel, wrapper.delta)
+    alpha = wrapper.alpha.data
+    m, v = torch.zeros_like(alpha), torch.zeros_like(alpha)
+    ws = ops.adaround_linear_workspace(o, k, w.device)
+    gout = torch.empty(32, o, device=w.device)
+    idx = torch.stack(batches[:timed_kernel_iters]).to(torch.int32).to(w.device)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(timed_kernel_iters)]
+    torch.cuda.synchronize()
+    for i in range(timed_kernel_iters):
+        ev[i][0].record()
+        ops.adaround_linear_fwd(w, alpha, x, idx[i], y, None, wrapper.num_channel, wrapper.delta, wrapper.offset,
+                                wrapper.clip_min, wrapper.clip_max, 0, ws, gout)
+        ev[i][1].record()
+        ops.adaround_linear_bwd_adam(w, gout, x, idx[i], alpha, m, v, wrapper.num_channel, wrapper.delta,
+                                     wrapper.offset, wrapper.clip_min, wrapper.clip_max, 0.01, 10.0, 1e-3, 0.9, 0.999,
+                                     1e-8, i + 1)
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    f = sum(e[0].elapsed_time(e[1]) for e in ev) / timed_kernel_iters
+    b = sum(e[1].elapsed_time(e[2]) for e in ev) / timed_kernel_iters
+    res["fused_kernels"] = {
+        "fwd_ms": f, "bwd_ms": b,
+        "fwd_algorithmic_bytes": 8 * n, "fwd_GBps": 8 * n / f / 1e6, "fwd_frac_hbm": 8 * n / f / 1e6 / HBM_PEAK_GBPS,
+        "fwd_mfma_TFLOPs": 2.0 * 32 * n / f / 1e9,
+        "bwd_algorithmic_bytes": 28 * n, "bwd_GBps": 28 * n / b / 1e6, "bwd_frac_hbm": 28 * n / b / 1e6 / HBM_PEAK_GBPS,
+        "bwd_mfma_TFLOPs": 2.0 * 32 * n / b / 1e9}
+    return res
+
+
+def torch_ops_adaround_baseline(torch, iterations=20):
+    """The same iteration written with stock torch ops + autograd + torch.optim.Adam on the GPU (what the reference's
+    Python does when run on PyTorch-ROCm): a comparison figure, not part of the product."""
+    wrapper, x, y = _adaround_layer(torch)
+    w = wrapper.weight.detach()
+    d, o = wrapper.delta.view(-1, 1), wrapper.offset.view(-1, 1)
+    alpha = torch.nn.Parameter(wrapper.alpha.data.clone())
+    opt = torch.optim.Adam([alpha])
+    torch.manual_seed(1005)
+
+    def step(it):
+        idx = torch.randperm(x.size(0))[:32].to(x.device)
+        opt.zero_grad()
+        h = torch.clamp(torch.sigmoid(alpha) * 1.2 - 0.1, 0, 1)
+        wq = (torch.clamp(torch.floor(w / d) + h - o, wrapper.clip_min, wrapper.clip_max) + o) * d
+        out = torch.nn.functional.linear(x[idx], wq)
+        recon = (torch.norm(out - y[idx], p="fro", dim=1) ** 2).mean()
+        h2 = torch.clamp(torch.sigmoid(alpha) * 1.2 - 0.1, 0, 1)
+        rnd = 0.01 * torch.add(1, -(torch.add(2 * h2, -1).abs()).pow(10.0)).sum()
+        (recon + rnd).backward()
+        opt.step()
+
+    for it in range(3):
+        step(it)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for it in range(iterations):
+        step(it)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    return {"ms_per_iteration": dt * 1e3 / iterations, "iterations": iterations,
+            "what": "torch elementwise ops + autograd + torch.optim.Adam on the same GPU"}
+
+
 def cpu_baseline_qdq(seconds=10.0):
     """Single-threaded oracle (C restatement of the reference CPU loops) on a [1024, 4096] slice of the workload."""
     import numpy as np
@@ -226,7 +337,7 @@ def main():
     ap.add_argument("--full", action="store_true", help="also measure every shape x dtype x bit-width cell")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run a subset of the legs, comma separated (main|pt|calib|copyref), for profiling")
+                    help="run a subset of the legs, comma separated (main|pt|calib|adaround|copyref), for profiling")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
@@ -263,6 +374,9 @@ def main():
         extra["per_tensor_act_int8"] = bench_per_tensor(torch, ops, max(20, args.steps), args.warmup)
     if want("calib"):
         extra["tf_enhanced_calibration"] = bench_calibration(torch, ops, 5)
+    if want("adaround"):
+        extra["adaround_linear_4096"] = bench_adaround(torch, ops, 1000 if args.only is None else args.steps)
+        extra["adaround_linear_4096"]["torch_ops_same_gpu"] = torch_ops_adaround_baseline(torch)
     if args.only is None:
         cells = [((11008, 4096), torch.bfloat16, 8), ((11008, 4096), torch.float32, 4)]
         if args.full:

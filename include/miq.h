@@ -215,6 +215,10 @@ int miq_adaround_soft_round_f32(const float* weight, const float* alpha, float* 
                                 int64_t num_element, int64_t num_element_per_channel, const float* delta,
                                 const float* offset, float clip_min, float clip_max, int use_soft_rounding,
                                 void* stream);
+/* weight_floor = floor(weight / delta) (ADA/adaround_wrapper.py:132), the part of apply_adaround that does not depend
+ * on alpha; the fused Linear entry points below take it in place of the weight. */
+int miq_adaround_floor_f32(const float* weight, float* weight_floor, int64_t num_channel, int64_t num_element,
+                           int64_t num_element_per_channel, const float* delta, void* stream);
 /* AdaroundWrapper._generate_alpha_parameter (ADA/adaround_wrapper.py:211-224):
  *   alpha = -log((zeta - gamma) / (w / delta - floor(w / delta) - gamma) - 1) */
 int miq_adaround_init_alpha_f32(const float* weight, float* alpha, int64_t num_channel, int64_t num_element,
@@ -249,7 +253,8 @@ int miq_adaround_blocks(int64_t num_element);
  * for torch.nn.Linear with a batch of exactly 32 rows (BATCH_SIZE, ADA/adaround_optimizer.py:58):
  *   fwd:  out = linear(x[rows], apply_adaround(W), bias);  grad_out = d recon_loss(act(out), act(target[rows])) / d out
  *   bwd:  dLoss/dW' = grad_out^T x[rows]  ->  alpha gradient + regulariser + Adam, as miq_adaround_bwd_adam_f32
- * weight, alpha, moments: [out_features, in_features] float32 row-major.  x: rows of in_features floats, row r at
+ * weight_floor (= floor(W / delta), from miq_adaround_floor_f32), alpha, moments: [out_features, in_features] float32
+ * row-major.  x: rows of in_features floats, row r at
  * x + r * x_row_stride; target likewise with out_features floats.  row_index: device int32[32] choosing the rows of x
  * and target (NULL = rows 0..31).  num_channel: 1 (per-tensor delta/offset) or out_features (per output channel).
  * Shapes: out_features % 64 == 0, in_features % 256 == 0, out_features * in_features < 2^31; other shapes return
@@ -265,13 +270,13 @@ int miq_adaround_linear_blocks(int64_t out_features, int64_t in_features);
  * grad_out: device float[32 * out_features] = 2 (act(out) - act(target)) act'(out) / 32, the gradient of
  * AdaroundLoss.compute_recon_loss (ADA/adaround_loss.py:70-80) w.r.t. out.
  * loss_partial (optional): device float[ceil(32 * out_features / 256)] partial sums of the reconstruction loss. */
-int miq_adaround_linear_fwd_f32(const float* weight, const float* alpha, const float* x, const int32_t* row_index,
+int miq_adaround_linear_fwd_f32(const float* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
                                 int64_t x_row_stride, const float* target, int64_t target_row_stride,
                                 const float* bias, int64_t out_features, int64_t in_features, int64_t num_channel,
                                 const float* delta, const float* offset, float clip_min, float clip_max,
                                 int activation, float* workspace, float* out, float* grad_out, float* loss_partial,
                                 void* stream);
-int miq_adaround_linear_bwd_adam_f32(const float* weight, const float* grad_out, const float* x,
+int miq_adaround_linear_bwd_adam_f32(const float* weight_floor, const float* grad_out, const float* x,
                                      const int32_t* row_index, int64_t x_row_stride, float* alpha, float* exp_avg,
                                      float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                      int64_t num_channel, const float* delta, const float* offset, float clip_min,

@@ -185,7 +185,9 @@ def test_fused_linear_forward_and_backward(ops, shape, per_channel, act):
     G = torch.empty(32, O, device="cuda")
     out = torch.empty(32, O, device="cuda")
     lp = torch.zeros((32 * O + 255) // 256, device="cuda")
-    ops.adaround_linear_fwd(wg, ag, Xg, ig, Yg, bg, C, dg, og, cmin, cmax, act, ws, G, out=out, loss_partial=lp)
+    fg = ops.adaround_floor(wg, C, npc, dg)
+    assert torch.equal(fg.cpu(), torch.floor(weight / d))
+    ops.adaround_linear_fwd(fg, ag, Xg, ig, Yg, bg, C, dg, og, cmin, cmax, act, ws, G, out=out, loss_partial=lp)
 
     # CPU restatement
     a_ref = alpha.clone().requires_grad_(True)
@@ -207,7 +209,7 @@ def test_fused_linear_forward_and_backward(ops, shape, per_channel, act):
     a1, m1, v1 = ag.clone(), m0.cuda(), v0.cuda()
     g1 = torch.empty_like(a1)
     rp1 = torch.zeros(ops.adaround_linear_blocks(O, K), device="cuda")
-    ops.adaround_linear_bwd_adam(wg, G, Xg, ig, a1, m1, v1, C, dg, og, cmin, cmax, reg_partial=rp1, grad_alpha=g1,
+    ops.adaround_linear_bwd_adam(fg, G, Xg, ig, a1, m1, v1, C, dg, og, cmin, cmax, reg_partial=rp1, grad_alpha=g1,
                                  **hyper)
     a2, m2, v2 = ag.clone(), m0.cuda(), v0.cuda()
     g2 = torch.empty_like(a2)
