@@ -1,0 +1,592 @@
+// v2 histogram observer + SQNR encoding search on gfx950.
+//
+// Reference (EA = TrainingExtensions/torch/src/python/aimet_torch/v2/quantization/encoding_analyzer.py):
+//   _HistogramObserver.collect_stats / _handle_inputs / _create_bin_edges      EA:131-205
+//   _HistogramObserver.merge_stats / _get_bin_num                              EA:207-262
+//   SqnrEncodingAnalyzer._pick_test_candidates*, _clamp_delta_offset_values    EA:594-660
+//   SqnrEncodingAnalyzer._estimate_clip_and_quant_noise, _select_best_candidates, compute_encodings_from_stats
+//                                                                              EA:566-592, 662-725
+// The reference's arithmetic is float32 torch ops (torch.histc for the binning); every float32 operation below is the
+// same IEEE operation in the same order, so bin counts, candidate grids and per-bin noise terms are identical.  The
+// only deliberate difference: the per-candidate sum over the bins is accumulated in double (torch.sum's float32
+// blocked summation order is not reproduced), so scores agree to rounding (about 1e-6 relative), not bit for bit.
+//
+// One update of the statistics reads the batch twice (finite min/max, then ONE binning pass that fills both the
+// batch's own histogram and the histogram over the merged range); the reference reads it about eight times
+// (isfinite x4, histc x2, comparisons x4) and re-bins the running histogram with per-element Python loops.
+#include "miq_common.h"
+#include "miq_fastmath.h"
+
+#include <cmath>
+
+namespace miq
+{
+namespace
+{
+constexpr int kMaxBins    = 4096;
+constexpr int kHistBlock  = 256;
+constexpr float kMinScale = 1.1920928955078125e-07f;   // torch.finfo(torch.float32).eps (EA:322)
+
+// ---- finite min / max per row --------------------------------------------------------------------------------
+// partial[(h * blocks + b) * 2 + {0,1}]
+__global__ __launch_bounds__(kHistBlock) void finite_minmax_kernel(const float* __restrict__ x, int64_t n_per_hist,
+                                                                   float* __restrict__ partial,
+                                                                   uint32_t* __restrict__ sums, int sums_per_hist)
+{
+    const int h = blockIdx.y;
+    // this launch also clears the count sums that the later kernels of the same update accumulate into
+    for (int i = blockIdx.x * kHistBlock + threadIdx.x; i < sums_per_hist; i += gridDim.x * kHistBlock)
+        sums[(int64_t) h * sums_per_hist + i] = 0;
+    const float* row = x + (int64_t) h * n_per_hist;
+    float lo = INFINITY, hi = -INFINITY;
+    for (int64_t i = (int64_t) blockIdx.x * kHistBlock + threadIdx.x; i < n_per_hist;
+         i += (int64_t) gridDim.x * kHistBlock)
+    {
+        const float v = row[i];
+        if (fabsf(v) < INFINITY)   // false for NaN and +-inf
+        {
+            lo = fminf(lo, v);
+            hi = fmaxf(hi, v);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        lo = fminf(lo, __shfl_xor(lo, o));
+        hi = fmaxf(hi, __shfl_xor(hi, o));
+    }
+    __shared__ float s[2][kHistBlock / 64];
+    if ((threadIdx.x & 63) == 0)
+    {
+        s[0][threadIdx.x >> 6] = lo;
+        s[1][threadIdx.x >> 6] = hi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        for (int k = 1; k < kHistBlock / 64; ++k)
+        {
+            lo = fminf(lo, s[0][k]);
+            hi = fmaxf(hi, s[1][k]);
+        }
+        float* p = partial + ((int64_t) h * gridDim.x + blockIdx.x) * 2;
+        p[0]     = lo;
+        p[1]     = hi;
+    }
+}
+
+// Binning ranges of one update, per histogram (device resident so that nothing waits for the host).
+struct Ranges
+{
+    float b_lo, b_hi;   // batch range = bin_edges[0], bin_edges[-1] of the batch's own histogram
+    float m_lo, m_hi;   // range torch.histc uses for the merged histogram
+    float new_min, new_max;   // merged (min, max) statistics
+    float old_min, old_max;   // statistics before this update
+    int   rebin;        // 1: the running histogram has to be re-binned into the merged range
+    int   pad;
+};
+
+// grid H, one wavefront per histogram: reduces the workgroups' (min, max), then lane 0 does the scalar work of
+// _create_bin_edges and of merge_stats' range logic
+__global__ __launch_bounds__(64) void ranges_kernel(const float* __restrict__ partial, int blocks, int num_bins,
+                                                    int has_stats, const float* __restrict__ state_minmax,
+                                                    float* __restrict__ batch_minmax, Ranges* __restrict__ ranges,
+                                                    int* __restrict__ bad_flag, int num_hist)
+{
+    const int h = blockIdx.x;
+    float lo = INFINITY, hi = -INFINITY;
+    for (int b = threadIdx.x; b < blocks; b += 64)
+    {
+        lo = fminf(lo, partial[((int64_t) h * blocks + b) * 2]);
+        hi = fmaxf(hi, partial[((int64_t) h * blocks + b) * 2 + 1]);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        lo = fminf(lo, __shfl_xor(lo, o));
+        hi = fmaxf(hi, __shfl_xor(hi, o));
+    }
+    if (threadIdx.x != 0)
+        return;
+    if (!(lo <= hi))
+    {
+        // no finite value at all: the reference raises ValueError here; reported when the statistics are next read
+        atomicOr(bad_flag, 1);
+        lo = 0.f;
+        hi = 0.f;
+    }
+    batch_minmax[2 * h]     = lo;
+    batch_minmax[2 * h + 1] = hi;
+    Ranges r;
+    // _create_bin_edges: equal min and max are widened by 0.5 each way; edges = arange(0, bins + 1) * step + min
+    float e_lo = lo, e_hi = hi;
+    if (e_hi == e_lo)
+    {
+        e_lo = e_lo - 0.5f;
+        e_hi = e_hi + 0.5f;
+    }
+    const float step = (e_hi - e_lo) / (float) num_bins;
+    r.b_lo           = 0.0f * step + e_lo;
+    r.b_hi           = (float) num_bins * step + e_lo;
+    r.old_min = r.old_max = 0.f;
+    r.rebin               = 0;
+    if (!has_stats)
+    {
+        r.new_min = lo;
+        r.new_max = hi;
+        r.m_lo    = r.b_lo;
+        r.m_hi    = r.b_hi;
+    }
+    else
+    {
+        r.old_min = state_minmax[2 * h];
+        r.old_max = state_minmax[2 * h + 1];
+        r.new_min = fminf(lo, r.old_min);
+        r.new_max = fmaxf(hi, r.old_max);
+        r.rebin   = !(r.new_min == r.old_min && r.new_max == r.old_max);
+        // torch.histc(min, max): equal bounds are widened by one each way
+        r.m_lo = r.new_min;
+        r.m_hi = r.new_max;
+        if (r.m_lo == r.m_hi)
+        {
+            r.m_lo -= 1.0f;
+            r.m_hi += 1.0f;
+        }
+    }
+    r.pad     = 0;
+    ranges[h] = r;
+}
+
+// torch.histc's bin of x in [lo, hi] (float32: (x - lo) * bins / (hi - lo), truncated; x == hi falls in the last
+// bin), followed by the observer's rule for what lies outside (below -> first bin, above -> last bin).  NaN: -1.
+struct Binner
+{
+    float lo, hi, width, recip, nbf;
+    int nb;
+    bool fast;
+
+    __device__ void init(float lo_, float hi_, int nb_)
+    {
+        lo    = lo_;
+        hi    = hi_;
+        nb    = nb_;
+        nbf   = (float) nb_;
+        width = hi_ - lo_;
+        fast  = fastdiv_divisor_ok(width);
+        recip = fast ? 1.0f / width : 0.f;
+    }
+
+    __device__ __forceinline__ int bin(float x) const
+    {
+        if (x != x)
+            return -1;
+        if (x < lo)
+            return 0;
+        if (x > hi)
+            return nb - 1;
+        const float a = (x - lo) * nbf;
+        const float q = (fast && a <= kFastDivMaxDividend) ? div_by_invariant(a, width, recip) : a / width;
+        int pos       = (int) q;
+        return pos >= nb ? nb - 1 : pos;
+    }
+};
+
+// grid (blocks, H).  Each workgroup bins its share of row h into LDS (batch range and merged range in one pass) and
+// stores its counts to its own slice of `partial` (plain stores: no atomics on global memory).
+// partial layout: [h][block][2][num_bins] uint32
+__global__ __launch_bounds__(kHistBlock) void hist2_kernel(const float* __restrict__ x, int64_t n_per_hist,
+                                                           int num_bins, int has_stats,
+                                                           const Ranges* __restrict__ ranges,
+                                                           uint32_t* __restrict__ partial)
+{
+    extern __shared__ uint32_t lds[];   // [2][num_bins]
+    const int h = blockIdx.y;
+    for (int i = threadIdx.x; i < 2 * num_bins; i += kHistBlock)
+        lds[i] = 0;
+    const Ranges r = ranges[h];
+    Binner bb, mb;
+    bb.init(r.b_lo, r.b_hi, num_bins);
+    mb.init(r.m_lo, r.m_hi, num_bins);
+    __syncthreads();
+    const float* row = x + (int64_t) h * n_per_hist;
+    for (int64_t i = (int64_t) blockIdx.x * kHistBlock + threadIdx.x; i < n_per_hist;
+         i += (int64_t) gridDim.x * kHistBlock)
+    {
+        const float v = row[i];
+        const int pb  = bb.bin(v);
+        if (pb >= 0)
+        {
+            atomicAdd(&lds[pb], 1u);
+            if (has_stats)
+                atomicAdd(&lds[num_bins + mb.bin(v)], 1u);
+        }
+    }
+    __syncthreads();
+    uint32_t* dst = partial + ((int64_t) h * gridDim.x + blockIdx.x) * 2 * num_bins;
+    for (int i = threadIdx.x; i < 2 * num_bins; i += kHistBlock)
+        dst[i] = lds[i];
+}
+
+// grid (ceil(2 bins / 256), slices, H): adds a slice of the workgroups' counts into sums[h][2][bins]
+__global__ __launch_bounds__(kHistBlock) void reduce_counts_kernel(const uint32_t* __restrict__ partial, int blocks,
+                                                                   int num_bins, uint32_t* __restrict__ sums)
+{
+    const int i = blockIdx.x * kHistBlock + threadIdx.x;
+    const int h = blockIdx.z;
+    if (i >= 2 * num_bins)
+        return;
+    const int per   = (blocks + gridDim.y - 1) / gridDim.y;
+    const int b0    = blockIdx.y * per;
+    const int b1    = min(blocks, b0 + per);
+    const uint32_t* p = partial + (int64_t) h * blocks * 2 * num_bins + i;
+    uint32_t acc    = 0;
+    for (int b = b0; b < b1; ++b)
+        acc += p[(int64_t) b * 2 * num_bins];
+    if (acc)
+        atomicAdd(&sums[(int64_t) h * 2 * num_bins + i], acc);
+}
+
+// grid H, 256 threads: writes the batch histogram, re-bins the running histogram when the
+// range grew (merge_stats, EA:222-251) and adds the batch's counts over the merged range.
+__global__ __launch_bounds__(kHistBlock) void merge_kernel(const uint32_t* __restrict__ sums, int num_bins,
+                                                           int has_stats,
+                                                           const Ranges* __restrict__ ranges,
+                                                           float* __restrict__ state_hist,
+                                                           float* __restrict__ state_minmax,
+                                                           float* __restrict__ batch_hist)
+{
+    __shared__ float upd[kMaxBins];
+    const int h    = blockIdx.x;
+    const Ranges r = ranges[h];
+    float* sh      = state_hist + (int64_t) h * num_bins;
+    float* bh      = batch_hist + (int64_t) h * num_bins;
+    const uint32_t* p = sums + (int64_t) h * 2 * num_bins;
+    for (int i = threadIdx.x; i < num_bins; i += kHistBlock)
+        upd[i] = 0.f;
+    __syncthreads();
+    if (has_stats && r.rebin)
+    {
+        const float nbf            = (float) num_bins;
+        const float dest_bin_width = (r.new_max - r.new_min) / nbf;
+        const float src_bin_width  = (r.old_max - r.old_min) / nbf;
+        for (int i = threadIdx.x; i < num_bins; i += kHistBlock)
+        {
+            const float cur           = sh[i];
+            const float src_bin_start = r.old_min + src_bin_width * (float) i;
+            int dest                  = (int) ((src_bin_start - r.new_min) / dest_bin_width);
+            dest                      = dest < num_bins - 1 ? dest : num_bins - 1;
+            const float dest_bin_end  = r.new_min + dest_bin_width * (float) (dest + 1);
+            const float split         = rintf(((dest_bin_end - src_bin_start) / src_bin_width) * cur);
+            const float first         = fminf(split, cur);
+            // counts are integer valued, so the order of these additions does not change the sums
+            atomicAdd(&upd[dest], first);
+            if (first < cur)
+            {
+                int other = (int) (((src_bin_start + dest_bin_width) - r.new_min) / dest_bin_width);
+                other     = other < num_bins - 1 ? other : num_bins - 1;
+                atomicAdd(&upd[other], cur - first);
+            }
+        }
+        __syncthreads();
+    }
+    for (int i = threadIdx.x; i < num_bins; i += kHistBlock)
+    {
+        const uint32_t cb = p[i], cm = p[num_bins + i];
+        bh[i]             = (float) cb;
+        if (!has_stats)
+            sh[i] = (float) cb;
+        else
+            sh[i] = (float) cm + (r.rebin ? upd[i] : sh[i]);
+    }
+    if (threadIdx.x == 0)
+    {
+        state_minmax[2 * h]     = r.new_min;
+        state_minmax[2 * h + 1] = r.new_max;
+    }
+}
+
+// ---- SQNR search ---------------------------------------------------------------------------------------------
+struct SearchArgs
+{
+    int num_bins, num_hist;
+    int symmetric;
+    int n_delta;        // asymmetric: delta candidates; symmetric: delta candidates
+    int n_offset;       // asymmetric: offsets from the arange + 1 observed; symmetric: 1
+    int n_arange;       // asymmetric: number of arange offsets
+    float num_steps;    // float32(num_steps)
+    double num_steps_d;
+    double offset_step; // num_steps / (num_offsets - 2)
+    float sym_offset;   // (-num_steps) // 2
+    float gamma;
+    int use_gamma;      // gamma != 1.0
+};
+
+// candidate c of histogram with gated (min_v, max_v): (delta, offset) exactly as the reference's tensor ops give them
+__device__ void candidate(const SearchArgs& a, float min_v, float max_v, int c, float& delta, float& offset)
+{
+    if (a.symmetric)
+    {
+        const float max_delta = 2.0f * fmaxf(max_v, -min_v) / a.num_steps;
+        delta                 = fmaxf(max_delta * (float) (c + 1) / (float) (a.n_delta - 1), kMinScale);
+        offset                = a.sym_offset;
+        return;
+    }
+    const int di = c / a.n_offset, oi = c - di * a.n_offset;
+    const float max_delta       = (max_v - min_v) / a.num_steps;
+    const float observed_offset = rintf(min_v / max_delta);
+    const float observed_min    = max_delta * observed_offset;
+    const float observed_max    = observed_min + max_delta * a.num_steps;
+    const float test_delta      = max_delta * (float) (di + 1) / (float) (a.n_delta - 1);
+    const float test_offset =
+        oi < a.n_arange ? rintf((float) (-a.num_steps_d + a.offset_step * (double) oi)) : observed_offset;
+    float test_min = test_delta * test_offset;
+    float test_max = test_min + test_delta * a.num_steps;
+    test_min       = fmaxf(observed_min, test_min);
+    test_max       = fminf(observed_max, test_max);
+    delta          = fmaxf((test_max - test_min) / a.num_steps, kMinScale);
+    offset         = rintf(test_min / delta);
+}
+
+__device__ __forceinline__ void gated_minmax(const float* minmax, int h, float num_steps, float eps_steps, float& mn,
+                                             float& mx)
+{
+    mn = fminf(minmax[2 * h], 0.0f);
+    mx = fmaxf(minmax[2 * h + 1], 0.0f);
+    mx = fmaxf(mx, mn + eps_steps);
+}
+
+// grid (candidate groups, H), 256 threads = 4 wavefronts, one candidate per wavefront at a time
+__global__ __launch_bounds__(256) void sqnr_noise_kernel(const float* __restrict__ hist,
+                                                         const float* __restrict__ minmax, SearchArgs a,
+                                                         float eps_steps, int cand_per_block,
+                                                         double* __restrict__ noise)
+{
+    __shared__ float s_mid[kMaxBins];
+    __shared__ float s_cnt[kMaxBins];
+    const int h = blockIdx.y, nb = a.num_bins;
+    // bin mid-points from the histogram's own edges: edges = arange * step + min (EA:197-205), mid-points EA:700-703
+    float lo = minmax[2 * h], hi = minmax[2 * h + 1];
+    if (hi == lo)
+    {
+        lo = lo - 0.5f;
+        hi = hi + 0.5f;
+    }
+    const float step       = (hi - lo) / (float) nb;
+    const float e0         = 0.0f * step + lo;
+    const float e1         = 1.0f * step + lo;
+    const float hist_delta = e1 - e0;
+    const float base       = e0 + hist_delta / 2.0f;
+    for (int i = threadIdx.x; i < nb; i += 256)
+    {
+        s_mid[i] = base + hist_delta * (float) i;
+        s_cnt[i] = hist[(int64_t) h * nb + i];
+    }
+    __syncthreads();
+    float mn, mx;
+    gated_minmax(minmax, h, a.num_steps, eps_steps, mn, mx);
+    const int ncand = a.n_delta * a.n_offset;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int c_end = min(ncand, (int) (blockIdx.x + 1) * cand_per_block);
+    for (int c = blockIdx.x * cand_per_block + wave; c < c_end; c += 4)
+    {
+        float delta, offset;
+        candidate(a, mn, mx, c, delta, offset);
+        double acc = 0.0;
+        for (int i = lane; i < nb; i += 64)
+        {
+            const float mid = s_mid[i];
+            float q         = rintf(mid / delta - offset);
+            const bool clip = q < 0.0f || q > a.num_steps;
+            q               = fminf(fmaxf(q, 0.0f), a.num_steps);
+            const float d   = (q + offset) * delta - mid;
+            float err       = d * d * s_cnt[i];
+            if (a.use_gamma && clip)
+                err = err * a.gamma;
+            acc += (double) err;
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1)
+            acc += __shfl_xor(acc, o);
+        if (lane == 0)
+            noise[(int64_t) h * ncand + c] = acc;
+    }
+}
+
+// grid H: first minimum in flattened (delta, offset) order, then min = offset * delta, max = min + num_steps * delta
+__global__ __launch_bounds__(64) void sqnr_pick_kernel(const double* __restrict__ noise,
+                                                       const float* __restrict__ minmax, SearchArgs a, float eps_steps,
+                                                       float* __restrict__ out_min, float* __restrict__ out_max,
+                                                       int* __restrict__ out_index)
+{
+    const int h = blockIdx.x, lane = threadIdx.x;
+    const int ncand = a.n_delta * a.n_offset;
+    double best = INFINITY;
+    int best_c  = 0x7fffffff;
+    for (int c = lane; c < ncand; c += 64)
+    {
+        const double v = noise[(int64_t) h * ncand + c];
+        if (v < best || (v == best && c < best_c))
+        {
+            best   = v;
+            best_c = c;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        const double ob = __shfl_xor(best, o);
+        const int oc    = __shfl_xor(best_c, o);
+        if (ob < best || (ob == best && oc < best_c))
+        {
+            best   = ob;
+            best_c = oc;
+        }
+    }
+    if (lane == 0)
+    {
+        if (best_c == 0x7fffffff)
+            best_c = 0;   // every score NaN: torch.min returns the first NaN's index; candidate 0 stands in for it
+        float mn, mx, delta, offset;
+        gated_minmax(minmax, h, a.num_steps, eps_steps, mn, mx);
+        candidate(a, mn, mx, best_c, delta, offset);
+        const float emin = offset * delta;
+        out_min[h]       = emin;
+        out_max[h]       = emin + a.num_steps * delta;
+        if (out_index)
+            out_index[h] = best_c;
+    }
+}
+
+int hist_blocks(int64_t num_hist, int64_t n_per_hist)
+{
+    // enough workgroups to fill 256 CUs a few times over, at least ~4K elements each
+    int64_t per_row = (n_per_hist + 4095) / 4096;
+    int64_t want    = (1024 + num_hist - 1) / num_hist;
+    int64_t b       = per_row < want ? per_row : want;
+    return (int) (b < 1 ? 1 : b);
+}
+
+int make_search(SearchArgs& a, int64_t num_hist, int num_bins, double num_steps, int symmetric, double gamma,
+                int asym_deltas, int sym_deltas, int offset_candidates)
+{
+    MIQ_CHECK_ARG(num_hist > 0 && num_hist < (1 << 30), "bad number of histograms");
+    MIQ_CHECK_ARG(num_bins > 0 && num_bins <= kMaxBins, "num_bins must lie in 1..%d", kMaxBins);
+    MIQ_CHECK_ARG(num_steps > 0, "The number of quantization bins cannot be less than or equal to 0.");
+    MIQ_CHECK_ARG(asym_deltas >= 2 && sym_deltas >= 2 && offset_candidates >= 3, "too few search candidates");
+    a.num_bins    = num_bins;
+    a.num_hist    = (int) num_hist;
+    a.symmetric   = symmetric != 0;
+    a.num_steps   = (float) num_steps;
+    a.num_steps_d = num_steps;
+    a.gamma       = (float) gamma;
+    a.use_gamma   = gamma != 1.0;
+    a.sym_offset  = (float) std::floor(-num_steps / 2.0);
+    a.offset_step = 0;
+    a.n_arange    = 0;
+    if (a.symmetric)
+    {
+        a.n_delta  = sym_deltas;
+        a.n_offset = 1;
+    }
+    else
+    {
+        // num_offsets = min(num_steps + 2, offset_candidates); arange(-num_steps, step, step): ceil((end - start) / step)
+        const double num_offsets = std::fmin(num_steps + 2.0, (double) offset_candidates);
+        a.offset_step            = num_steps / (num_offsets - 2.0);
+        a.n_arange               = (int) std::ceil((a.offset_step - (-num_steps)) / a.offset_step);
+        a.n_delta                = asym_deltas;
+        a.n_offset               = a.n_arange + 1;
+    }
+    return MIQ_OK;
+}
+}   // namespace
+}   // namespace miq
+
+using namespace miq;
+
+extern "C" {
+
+int64_t miq_v2_hist_workspace_bytes(int64_t num_hist, int64_t n_per_hist, int num_bins)
+{
+    if (num_hist <= 0 || n_per_hist <= 0 || num_bins <= 0)
+        return 0;
+    const int64_t blocks = hist_blocks(num_hist, n_per_hist);
+    // per-workgroup counts + their sums + per-workgroup (min, max) + the per-histogram ranges
+    return num_hist * blocks * 2 * (int64_t) num_bins * 4 + num_hist * 2 * (int64_t) num_bins * 4 +
+           num_hist * blocks * 2 * 4 + num_hist * (int64_t) sizeof(Ranges) + 256;
+}
+
+int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hist, int num_bins, int has_stats,
+                           float* state_hist, float* state_minmax, float* batch_hist, float* batch_minmax,
+                           int32_t* bad_flag, void* workspace, void* stream)
+{
+    MIQ_CHECK_ARG(num_hist > 0 && n_per_hist > 0, "empty input");
+    MIQ_CHECK_ARG(num_bins > 0 && num_bins <= kMaxBins, "num_bins must lie in 1..%d", kMaxBins);
+    MIQ_CHECK_ARG(num_hist <= 65535, "at most 65535 histograms per call");
+    MIQ_CHECK_ARG(data && state_hist && state_minmax && batch_hist && batch_minmax && bad_flag && workspace,
+                  "null pointer");
+    const int blocks = hist_blocks(num_hist, n_per_hist);
+    char* ws         = (char*) workspace;
+    uint32_t* counts = (uint32_t*) ws;
+    ws += num_hist * blocks * 2 * (int64_t) num_bins * 4;
+    uint32_t* sums = (uint32_t*) ws;
+    ws += num_hist * 2 * (int64_t) num_bins * 4;
+    float* mm_part = (float*) ws;
+    ws += num_hist * blocks * 2 * 4;
+    ws             = (char*) (((uintptr_t) ws + 15) & ~(uintptr_t) 15);
+    Ranges* ranges = (Ranges*) ws;
+    hipStream_t s  = (hipStream_t) stream;
+    hipLaunchKernelGGL(finite_minmax_kernel, dim3(blocks, (unsigned) num_hist), dim3(kHistBlock), 0, s, data, n_per_hist,
+                       mm_part, sums, 2 * num_bins);
+    MIQ_CHECK_LAUNCH();
+    hipLaunchKernelGGL(ranges_kernel, dim3((unsigned) num_hist), dim3(64), 0, s, mm_part, blocks, num_bins,
+                       has_stats, state_minmax, batch_minmax, ranges, bad_flag, (int) num_hist);
+    MIQ_CHECK_LAUNCH();
+    hipLaunchKernelGGL(hist2_kernel, dim3(blocks, (unsigned) num_hist), dim3(kHistBlock),
+                       2 * num_bins * sizeof(uint32_t), s, data, n_per_hist, num_bins, has_stats, ranges, counts);
+    MIQ_CHECK_LAUNCH();
+    const int slices = blocks < 32 ? blocks : 32;
+    hipLaunchKernelGGL(reduce_counts_kernel, dim3((2 * num_bins + kHistBlock - 1) / kHistBlock, slices, (unsigned) num_hist),
+                       dim3(kHistBlock), 0, s, counts, blocks, num_bins, sums);
+    MIQ_CHECK_LAUNCH();
+    hipLaunchKernelGGL(merge_kernel, dim3((unsigned) num_hist), dim3(kHistBlock), 0, s, sums, num_bins, has_stats, ranges,
+                       state_hist, state_minmax, batch_hist);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int miq_v2_sqnr_num_candidates(double num_steps, int symmetric, int asym_deltas, int sym_deltas, int offset_candidates)
+{
+    SearchArgs a;
+    if (make_search(a, 1, 1, num_steps, symmetric, 1.0, asym_deltas, sym_deltas, offset_candidates))
+        return -1;
+    return a.n_delta * a.n_offset;
+}
+
+int miq_v2_sqnr_search_f32(const float* hist, const float* minmax, int64_t num_hist, int num_bins, double num_steps,
+                           int symmetric, double gamma, int asym_deltas, int sym_deltas, int offset_candidates,
+                           float* out_min, float* out_max, double* noise, int32_t* best_index, void* stream)
+{
+    SearchArgs a;
+    if (int rc = make_search(a, num_hist, num_bins, num_steps, symmetric, gamma, asym_deltas, sym_deltas,
+                             offset_candidates))
+        return rc;
+    MIQ_CHECK_ARG(num_hist <= 65535, "at most 65535 histograms per call");
+    MIQ_CHECK_ARG(hist && minmax && out_min && out_max && noise, "null pointer");
+    const int ncand = a.n_delta * a.n_offset;
+    // MINIMUM_SCALE * num_steps is a Python float product, cast to float32 when added to the tensor
+    const float eps_steps = (float) ((double) kMinScale * num_steps);
+    // few histograms: spread one histogram's candidates over many workgroups
+    int cand_per_block = num_hist >= 256 ? ncand : 8;
+    const int groups   = (ncand + cand_per_block - 1) / cand_per_block;
+    hipStream_t s      = (hipStream_t) stream;
+    hipLaunchKernelGGL(sqnr_noise_kernel, dim3(groups, (unsigned) num_hist), dim3(256), 0, s, hist, minmax, a, eps_steps,
+                       cand_per_block, noise);
+    MIQ_CHECK_LAUNCH();
+    hipLaunchKernelGGL(sqnr_pick_kernel, dim3((unsigned) num_hist), dim3(64), 0, s, noise, minmax, a, eps_steps, out_min,
+                       out_max, best_index);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+}   // extern "C"

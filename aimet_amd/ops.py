@@ -222,6 +222,55 @@ def minmax_per_channel(x, num_channel, n_per_channel):
     return out
 
 
+# ------------------------------------------------------------------------------------- v2 histogram observer / SQNR
+def v2_hist_workspace(num_hist, n_per_hist, num_bins, device):
+    nbytes = int(lib.miq_v2_hist_workspace_bytes(int(num_hist), int(n_per_hist), int(num_bins)))
+    return torch.empty((nbytes + 3) // 4, dtype=torch.int32, device=device)
+
+
+def v2_hist_update(data, num_hist, num_bins, has_stats, state_hist, state_minmax, bad_flag, workspace):
+    """collect_stats + merge_stats of the v2 histogram observer for one batch; returns (batch_hist, batch_minmax)."""
+    _require_gpu(data, state_hist, state_minmax, bad_flag, workspace)
+    if data.dtype != _F32 or not data.is_contiguous():
+        raise RuntimeError("the histogram observer takes contiguous float32 data")
+    n_per_hist = data.numel() // num_hist
+    batch_hist = torch.empty(num_hist, num_bins, dtype=_F32, device=data.device)
+    batch_minmax = torch.empty(num_hist, 2, dtype=_F32, device=data.device)
+    with torch.cuda.device(data.device):
+        check(lib.miq_v2_hist_update_f32(_ptr(data), int(num_hist), int(n_per_hist), int(num_bins), int(has_stats),
+                                         _ptr(state_hist), _ptr(state_minmax), _ptr(batch_hist), _ptr(batch_minmax),
+                                         _ptr(bad_flag), _ptr(workspace), _stream(data)))
+    return batch_hist, batch_minmax
+
+
+def v2_sqnr_num_candidates(num_steps, symmetric, asym_deltas, sym_deltas, offset_candidates):
+    n = int(lib.miq_v2_sqnr_num_candidates(float(num_steps), int(symmetric), int(asym_deltas), int(sym_deltas),
+                                           int(offset_candidates)))
+    if n < 0:
+        raise _lib.MiqError(lib.miq_last_error().decode())
+    return n
+
+
+def v2_sqnr_search(hist, minmax, num_steps, symmetric, gamma, asym_deltas, sym_deltas, offset_candidates,
+                   want_details=False):
+    """SQNR search over the candidate grid; returns (min, max) device vectors [num_hist] (+ noise, best index)."""
+    _require_gpu(hist, minmax)
+    hist, minmax = hist.contiguous(), minmax.contiguous()
+    num_hist, num_bins = hist.shape
+    ncand = v2_sqnr_num_candidates(num_steps, symmetric, asym_deltas, sym_deltas, offset_candidates)
+    out = torch.empty(2, num_hist, dtype=_F32, device=hist.device)
+    noise = torch.empty(num_hist, ncand, dtype=torch.float64, device=hist.device)
+    best = torch.empty(num_hist, dtype=torch.int32, device=hist.device) if want_details else None
+    with torch.cuda.device(hist.device):
+        check(lib.miq_v2_sqnr_search_f32(_ptr(hist), _ptr(minmax), num_hist, num_bins, float(num_steps),
+                                         int(symmetric), float(gamma), int(asym_deltas), int(sym_deltas),
+                                         int(offset_candidates), _ptr(out[0]), _ptr(out[1]), _ptr(noise), _ptr(best),
+                                         _stream(hist)))
+    if want_details:
+        return out[0], out[1], noise, best
+    return out[0], out[1]
+
+
 # ----------------------------------------------------------------------------------------------------------- AdaRound
 def _ada_check(weight, *others):
     _require_gpu(weight, *others)

@@ -283,6 +283,35 @@ int miq_adaround_linear_bwd_adam_f32(const float* weight_floor, const float* gra
                                      float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
                                      float eps, int step, float* reg_partial, void* stream);
 
+/* ---------------------------------------------------------------------------------------------------------------
+ * v2 histogram observer + SQNR encoding analyzer
+ * (EA = TORCH/v2/quantization/encoding_analyzer.py).  State lives in caller-owned device buffers:
+ *   state_hist    float[num_hist * num_bins]   running histogram (integer-valued counts, as torch.histc returns)
+ *   state_minmax  float[num_hist * 2]          running {min, max} of the finite values
+ * Histogram h covers the contiguous slab data[h * n_per_hist, (h + 1) * n_per_hist) (per-tensor: num_hist = 1;
+ * per-channel along axis 0: num_hist = C).
+ * ------------------------------------------------------------------------------------------------------------- */
+
+int64_t miq_v2_hist_workspace_bytes(int64_t num_hist, int64_t n_per_hist, int num_bins);
+/* _HistogramObserver.collect_stats + merge_stats (EA:131-262) for one batch.  Writes the batch's own statistics
+ * (what collect_stats returns) to batch_hist / batch_minmax and merges them into state_* (has_stats = 0: the state is
+ * empty and becomes the batch's statistics).  bad_flag: device int32, set to 1 when a slab holds no finite value (the
+ * reference raises ValueError there; the caller checks the flag when it next reads results).  workspace: device
+ * buffer of miq_v2_hist_workspace_bytes.  Enqueues five kernels; never synchronises. */
+int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hist, int num_bins, int has_stats,
+                           float* state_hist, float* state_minmax, float* batch_hist, float* batch_minmax,
+                           int32_t* bad_flag, void* workspace, void* stream);
+/* Number of (delta, offset) candidates SqnrEncodingAnalyzer searches (EA:594-646); -1 on invalid arguments. */
+int miq_v2_sqnr_num_candidates(double num_steps, int symmetric, int asym_deltas, int sym_deltas,
+                               int offset_candidates);
+/* SqnrEncodingAnalyzer.compute_encodings_from_stats (EA:566-592): candidate grid (EA:594-660), expected noise of every
+ * candidate (EA:675-725, gamma-weighted clipping noise), first minimum wins; out_min / out_max: device float[num_hist].
+ * noise: device double[num_hist * num_candidates] (scratch and inspection: the score of every candidate);
+ * best_index (optional): device int32[num_hist]. */
+int miq_v2_sqnr_search_f32(const float* hist, const float* minmax, int64_t num_hist, int num_bins, double num_steps,
+                           int symmetric, double gamma, int asym_deltas, int sym_deltas, int offset_candidates,
+                           float* out_min, float* out_max, double* noise, int32_t* best_index, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,178 @@
+"""GPU parity of the v2 histogram observer and SQNR search against the CPU restatement of the reference
+(oracle/sqnr_oracle.py: torch CPU ops incl. torch.histc), through the C ABI.
+
+Bar: histogram counts, ranges and the chosen (min, max) identical; candidate scores within 1e-5 relative (they are
+summed in double on the GPU and in float32 by torch.sum on the CPU).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import sqnr_oracle as sq
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ea():
+    from aimet_amd.v2.quantization import encoding_analyzer
+    return encoding_analyzer
+
+
+def _batches(seed):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(30000, generator=g)
+    b = torch.randn(50000, generator=g) * 3 + 1            # range grows on both sides
+    c = torch.randn(20000, generator=g) * 0.2               # inside the range
+    d = torch.randn(1000, generator=g).abs() * 20           # grows on the right only
+    e = a.clone()
+    e[:4] = torch.tensor([float('inf'), -float('inf'), float('nan'), 1e30])
+    return [a, b, c, d, e]
+
+
+def _same_hist(dev, ref: sq.Histogram):
+    assert torch.equal(dev.histogram.cpu(), ref.histogram)
+    assert dev.min.item() == ref.min.item() and dev.max.item() == ref.max.item()
+    assert torch.equal(dev.bin_edges.cpu(), ref.bin_edges)
+
+
+@pytest.mark.parametrize("num_bins", [2048, 512, 100])
+def test_histograms_match_torch_histc_across_merges(ea, num_bins):
+    obs = ea._HistogramObserver((1,), num_bins)
+    ref = sq.SqnrAnalyzer(1, num_bins)
+    for x in _batches(1):
+        new = obs.collect_and_merge_stats(x.cuda())
+        ref_new = ref.update_stats(x)
+        _same_hist(new[0], ref_new[0])
+        _same_hist(obs.get_stats()[0], ref.stats[0])
+
+
+def test_edge_inputs(ea):
+    for x in (torch.full((1000,), 3.25), torch.zeros(77), torch.tensor([1.0]), torch.tensor([-2.0, 5.0]),
+              torch.arange(-100, 101) / 100):
+        obs = ea._HistogramObserver((1,), 2048)
+        ref = sq.SqnrAnalyzer(1, 2048)
+        for rep in range(2):                      # the second round merges an identical batch (equal min and max)
+            new = obs.collect_and_merge_stats(x.cuda())
+            ref_new = ref.update_stats(x)
+            _same_hist(new[0], ref_new[0])
+            _same_hist(obs.get_stats()[0], ref.stats[0])
+    obs = ea._HistogramObserver((1,), 16)
+    stats = obs.collect_and_merge_stats(torch.tensor([float('nan'), float('inf')]).cuda())
+    with pytest.raises(ValueError):
+        stats[0]
+    with pytest.raises(RuntimeError):
+        obs.collect_stats(torch.randn(10))        # CPU tensor
+
+
+def test_large_batch_counts(ea):
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(32 * 256 * 28 * 28 // 4, generator=g).abs()
+    obs = ea._HistogramObserver((1,), 2048)
+    new = obs.collect_and_merge_stats(x.cuda())
+    _same_hist(new[0], sq.collect_histogram(x, 2048))
+
+
+@pytest.mark.parametrize("symmetric", [False, True])
+@pytest.mark.parametrize("num_steps,gamma", [(255.0, 3.0), (255.0, 1.0), (15.0, 3.0), (65535.0, 3.0)])
+def test_search_matches_restatement(ea, symmetric, num_steps, gamma):
+    an = ea.SqnrEncodingAnalyzer((1,), gamma=gamma)
+    ref = sq.SqnrAnalyzer(1, 2048, gamma=gamma)
+    g = torch.Generator().manual_seed(7)
+    for scale, shift in ((1.0, 0.3), (2.0, -0.5)):
+        x = torch.randn(40000, generator=g) * scale + shift
+        x[:3] = torch.tensor([25.0, -14.0, 18.0])          # outliers: clipping is worth it
+        an.update_stats(x.cuda())
+        ref.update_stats(x)
+    rmin, rmax, rnoise = ref.compute_encodings(num_steps, symmetric)
+    st = an.observer.get_stats()
+    from aimet_amd import ops
+    gmin, gmax, gnoise, best = ops.v2_sqnr_search(st.hist, st.minmax, num_steps, symmetric, gamma, 17, 101, 21,
+                                                  want_details=True)
+    assert gnoise.shape == rnoise.shape
+    assert torch.allclose(gnoise.cpu().float(), rnoise, rtol=1e-5, atol=0)
+    ref_best = int(torch.argmin(rnoise[0]))
+    if int(best[0]) != ref_best:
+        # a near-tie resolved differently by the two summation orders: the scores must be indistinguishable
+        assert abs(rnoise[0, int(best[0])] - rnoise[0, ref_best]) <= 2e-6 * rnoise[0, ref_best]
+    else:
+        assert torch.equal(gmin.cpu(), rmin) and torch.equal(gmax.cpu(), rmax)
+    qmin, qmax = an.compute_encodings(num_steps, symmetric)
+    assert torch.equal(qmin, gmin.view(1)) and torch.equal(qmax, gmax.view(1))
+
+
+def test_per_channel(ea):
+    torch.manual_seed(10)
+    x = torch.randn(6, 3, 5, 100) * torch.linspace(0.5, 3, 6).view(6, 1, 1, 1)
+    shape = (6, 1, 1, 1)
+    an = ea.SqnrEncodingAnalyzer(shape)
+    ref = sq.SqnrAnalyzer(6, 2048)
+    for t in (x, x / 2, x * 1.5):
+        an.update_stats(t.cuda())
+        ref.update_stats(t)
+    st = an.observer.get_stats()
+    for i in range(6):
+        _same_hist(st[i], ref.stats[i])
+        assert st[i].min.item() == (x[i] * 1.5).min().item() and st[i].max.item() == (x[i] * 1.5).max().item()
+    qmin, qmax = an.compute_encodings(255.0, False)
+    rmin, rmax, _ = ref.compute_encodings(255.0, False)
+    assert qmin.shape == shape and qmax.shape == shape
+    assert torch.equal(qmin.cpu().view(-1), rmin) and torch.equal(qmax.cpu().view(-1), rmax)
+    with pytest.raises(RuntimeError):
+        ea.SqnrEncodingAnalyzer((1, 3, 1, 1)).update_stats(x.cuda())     # slabs not contiguous: not implemented
+
+
+def test_reference_cases_through_the_analyzer(ea):
+    # test_encoding_analyzer.py:659-674: equally spaced input, gamma = 1 -> the observed range exactly
+    x = torch.arange(-100, 101) / 100
+    an = ea.SqnrEncodingAnalyzer(shape=(1,), gamma=1)
+    observed_delta = torch.tensor(2 / 255.0)
+    observed_offset = torch.round(-1 / observed_delta)
+    observed_min = observed_offset * observed_delta
+    observed_max = observed_min + 255 * observed_delta
+    an.update_stats(x.cuda())
+    qmin, qmax = an.compute_encodings(num_steps=math.pow(2, 8) - 1, is_symmetric=False)
+    assert torch.equal(qmin.cpu(), observed_min.view((1,))) and torch.equal(qmax.cpu(), observed_max.view((1,)))
+    # :676-709: one severe outlier is clipped at 3/4 of its value
+    expected_delta = torch.Tensor([0.1])
+    outlier_val = (255 * expected_delta) / 0.75
+    n = round(12 * 255 * outlier_val.item() / expected_delta.item() - 12 * (255 ** 2))
+    an = ea.SqnrEncodingAnalyzer((1,), gamma=1.0)
+    torch.manual_seed(0)
+    an.update_stats((torch.rand((1, n)) * 255 * expected_delta).cuda())
+    an.update_stats(torch.Tensor([outlier_val]).view(1, 1).cuda())
+    qmin, qmax = an.compute_encodings(math.pow(2, 8) - 1, is_symmetric=False)
+    assert torch.allclose(qmin.cpu(), torch.Tensor([0])) and torch.allclose(qmax.cpu(), expected_delta * 255)
+    # no statistics / bad arguments
+    from aimet_amd.v2.utils import StatisticsNotFoundError
+    fresh = ea.SqnrEncodingAnalyzer((1,))
+    with pytest.raises(StatisticsNotFoundError):
+        fresh.compute_encodings(255, False)
+    with pytest.raises(ValueError):
+        an.compute_encodings(0, False)
+    with pytest.raises(ValueError):
+        ea.SqnrEncodingAnalyzer((1,), num_bins=0)
+    # dynamic encodings from the batch's own statistics
+    dmin, dmax = an.compute_dynamic_encodings(torch.randn(1000).cuda(), 255, False)
+    assert dmin.shape == (1,) and dmin.item() < 0 < dmax.item()
+
+
+def test_quantizer_with_sqnr_analyzer(ea):
+    """QuantizeDequantize calibrated by the SQNR analyzer (the injection point of the reference's quantizer ctor)."""
+    from aimet_amd.v2.quantization.affine import QuantizeDequantize
+    torch.manual_seed(3)
+    x = torch.randn(64, 128).cuda()
+    x[0, 0] = 40.0
+    q = QuantizeDequantize((), bitwidth=8, symmetric=False, encoding_analyzer=ea.SqnrEncodingAnalyzer(())).cuda()
+    with q.compute_encodings():
+        q(x)
+    assert q.is_initialized()
+    want_min, want_max = q.encoding_analyzer.compute_encodings(255, False)
+    # the quantizer snaps the range to its grid (offset rounding): within one step of the analyzer's answer
+    assert abs(q.get_min().item() - want_min.item()) <= q.get_scale().item()
+    assert abs(q.get_max().item() - want_max.item()) <= q.get_scale().item()
+    y = q(x)
+    inside = (x >= q.get_min()) & (x <= q.get_max())
+    assert (y - x)[inside].abs().max().item() <= 0.5 * q.get_scale().item() * 1.001
