@@ -10,8 +10,8 @@ last-level cache cannot serve the traffic.  One JSON line is printed:
 
   value            whole-job algorithmic GB/s of fwd+bwd (20 B/element: fwd reads x, writes y; bwd reads x and g,
                    writes gx) over the K timed steps
-  roofline         the dominant kernel (backward, 12 B/element) measured with HIP events around every launch of the
-                   timed region, against the 8 TB/s HBM peak
+  roofline         the dominant kernel (backward, 12 B/element): mean duration of K back-to-back launches bracketed
+                   by a HIP event pair on the launching stream, against the 8 TB/s HBM peak
   cpu_baseline     the single-threaded C restatement of the reference's CPU loops (oracle/), timed on this host on a
                    bounded sample of the same workload
   extra            the other cells of the measurement matrix (per-tensor activation QDQ, the weight shapes x dtypes x
@@ -56,26 +56,39 @@ def _sym_channel_params(torch, ops, w, c, npc, bw):
 
 
 def _time_fwd_bwd(torch, fwd, bwd, sets, steps, warmup):
-    """Runs warmup + steps passes, rotating buffer sets; returns (wall ms/step, mean fwd ms, mean bwd ms)."""
+    """Runs warmup + steps fwd+bwd passes, rotating buffer sets; returns (wall ms/step, mean fwd ms, mean bwd ms).
+
+    The step time is wall-clock over exactly `steps` passes between two synchronisations (one HIP event pair around
+    the same region cross-checks it).  The per-kernel durations come from two more regions of `steps` back-to-back
+    launches of that kernel alone, each bracketed by a HIP event pair on the launching stream: events between every
+    pair of launches would put a ~5 us bubble after each kernel and distort both numbers.
+    """
     for i in range(warmup):
         s = sets[i % len(sets)]
         fwd(s)
         bwd(s)
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    e = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    e[0].record()
     for i in range(steps):
         s = sets[i % len(sets)]
-        ev[i][0].record()
         fwd(s)
-        ev[i][1].record()
         bwd(s)
-        ev[i][2].record()
+    e[1].record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    f = sum(e[0].elapsed_time(e[1]) for e in ev) / steps
-    b = sum(e[1].elapsed_time(e[2]) for e in ev) / steps
-    return wall_ms, f, b
+    assert e[0].elapsed_time(e[1]) / steps <= wall_ms * 1.001
+    e[2].record()
+    for i in range(steps):
+        fwd(sets[i % len(sets)])
+    e[3].record()
+    e[4].record()
+    for i in range(steps):
+        bwd(sets[i % len(sets)])
+    e[5].record()
+    torch.cuda.synchronize()
+    return wall_ms, e[2].elapsed_time(e[3]) / steps, e[4].elapsed_time(e[5]) / steps
 
 
 def bench_per_channel(torch, ops, shape, dtype, bw, steps, warmup, seed, nsets=3):
