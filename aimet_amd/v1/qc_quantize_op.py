@@ -155,10 +155,12 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
     def forward(self, *inputs, **kwargs):
         quantized_inputs = self._quantize_activation(self.input_quantizers, list(inputs))
         shadow_params = self._quantize_dequantize_params()
-        quantized_inputs = SteGatingFuncForParameters.apply(self, *quantized_inputs)
-        # the custom function returns its inputs as they are; clone so that an in-place op of the wrapped module
-        # cannot corrupt the gradient bookkeeping of that view
-        quantized_inputs = [inp.clone() if isinstance(inp, torch.Tensor) else inp for inp in quantized_inputs]
+        if torch.is_grad_enabled():
+            quantized_inputs = SteGatingFuncForParameters.apply(self, *quantized_inputs)
+            # the custom function returns its inputs as they are; clone so that an in-place op of the wrapped module
+            # cannot corrupt the gradient bookkeeping of that view.  Without autograd there is nothing to gate and
+            # nothing to protect: no extra pass over the activations.
+            quantized_inputs = [inp.clone() if isinstance(inp, torch.Tensor) else inp for inp in quantized_inputs]
         wrapped_output = self._module_to_wrap(*quantized_inputs, **kwargs)
         self._restore_shadow_params(shadow_params)
         if not isinstance(wrapped_output, (List, Tuple)):
