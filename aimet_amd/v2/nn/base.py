@@ -1,0 +1,152 @@
+"""Quantized modules of the v2 path: a mixin that adds input / parameter / output quantizers to a torch module class.
+
+Mirrors BaseQuantizationMixin of TrainingExtensions/torch/src/python/aimet_torch/v2/nn/base.py (:60-262:
+__quant_init__, __call__, _patch_quantized_parameters, _compute_param_encodings, compute_param_encodings,
+compute_encodings, implements, from_module) and the fake-quantization forward of
+TrainingExtensions/torch/src/python/aimet_torch/v2/nn/fake_quant.py (quantize inputs, patch quantized parameters, run
+the base class' forward, quantize outputs).  The quantizers are the HIP-backed QuantizeDequantize modules.
+"""
+import contextlib
+import itertools
+from typing import Type
+
+import torch
+from torch import nn
+
+from ..quantization.affine.quantizer import MinMaxQuantizer
+from ..utils import patch_attr
+
+
+def _no_op(input):  # pylint: disable=redefined-builtin
+    return input
+
+
+class BaseQuantizationMixin:
+    """Mixin that implements quantization on top of regular torch modules."""
+
+    cls_to_qcls: dict = {}
+    qcls_to_cls: dict = {}
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.__quant_init__()
+
+    def __quant_init__(self):
+        """All quantizers start as None: one input, one output, one per parameter of the base module."""
+        self.param_quantizers = nn.ModuleDict({name: None for name, _ in self.named_parameters(recurse=False)})
+        self.input_quantizers = nn.ModuleList([None])
+        self.output_quantizers = nn.ModuleList([None])
+
+    def __call__(self, *args, **kwargs):
+        self._compute_param_encodings(overwrite=False)
+        return super().__call__(*args, **kwargs)
+
+    def _patch_quantized_parameters(self):
+        stack = contextlib.ExitStack()
+        for param_name, param_quantizer in self.param_quantizers.items():
+            if param_quantizer and param_quantizer.is_initialized():
+                stack.enter_context(patch_attr(self, param_name, param_quantizer(getattr(self, param_name))))
+        return stack
+
+    def _compute_param_encodings(self, overwrite: bool):
+        for param_name, param_quantizer in self.param_quantizers.items():
+            if not param_quantizer or not param_quantizer._allow_overwrite:  # pylint: disable=protected-access
+                continue
+            if not param_quantizer.is_initialized() or overwrite:
+                param = getattr(self, param_name)
+                if param is not None:
+                    with patch_attr(param_quantizer, "forward", _no_op), param_quantizer.compute_encodings():
+                        _ = param_quantizer(param)
+
+    def compute_param_encodings(self):
+        self._compute_param_encodings(overwrite=True)
+
+    @contextlib.contextmanager
+    def compute_encodings(self):
+        """Every quantizer of the layer observes what passes through it and computes its encoding on exit; input and
+        output quantizers are pass-through meanwhile (as in the v1 simulation)."""
+        self._compute_param_encodings(overwrite=True)
+        with contextlib.ExitStack() as stack:
+            for quantizer in itertools.chain(self.input_quantizers, self.output_quantizers):
+                if not isinstance(quantizer, MinMaxQuantizer) or not quantizer._allow_overwrite:  # pylint: disable=protected-access
+                    continue
+                stack.enter_context(patch_attr(quantizer, 'forward', _no_op))
+                stack.enter_context(quantizer.compute_encodings())
+            yield
+
+    def get_original_module(self) -> nn.Module:
+        """A plain module of the base class sharing this module's parameters and buffers."""
+        base_cls = type(self).qcls_to_cls[type(self)]
+        module = base_cls.__new__(base_cls)
+        module.__dict__ = {k: v for k, v in self.__dict__.items()}
+        module._modules = {k: v for k, v in self._modules.items()
+                           if k not in ('param_quantizers', 'input_quantizers', 'output_quantizers')}
+        module._parameters = dict(self._parameters)
+        module._buffers = dict(self._buffers)
+        return module
+
+    @classmethod
+    def implements(cls, module_cls):
+        """Decorator registering the quantized definition of a base class."""
+        def wrapper(quantized_cls):
+            cls.cls_to_qcls[module_cls] = quantized_cls
+            cls.qcls_to_cls[quantized_cls] = module_cls
+            return quantized_cls
+        return wrapper
+
+    @classmethod
+    def from_module(cls, module: nn.Module):
+        """Quantized module with the attributes, parameters and buffers of `module` (shared, not copied)."""
+        module_cls = type(module)
+        qtzn_module_cls = cls.cls_to_qcls.get(module_cls, None)
+        if not qtzn_module_cls:
+            raise RuntimeError(f'The quantized module definition of {module_cls} is not registered. '
+                               f'Please register the quantized module definition of {module_cls} '
+                               f'using `@{cls.__name__}.implements({module_cls.__name__})` decorator.')
+        qtzn_module = cls.__new__(qtzn_module_cls)
+        qtzn_module.__dict__ = module.__dict__.copy()
+        qtzn_module._modules = module._modules.copy()
+        qtzn_module._parameters = module._parameters.copy()
+        qtzn_module._buffers = module._buffers.copy()
+        qtzn_module.__quant_init__()
+        return qtzn_module
+
+
+class QuantizationMixin(BaseQuantizationMixin):
+    """Fake-quantization: quantize-dequantize inputs, parameters and outputs around the base class' forward."""
+
+    cls_to_qcls = {}
+    qcls_to_cls = {}
+
+    def forward(self, *args, **kwargs):
+        args = list(args)
+        for i, quantizer in enumerate(self.input_quantizers):
+            if quantizer and i < len(args) and isinstance(args[i], torch.Tensor) and args[i].is_floating_point():
+                args[i] = quantizer(args[i])
+        with self._patch_quantized_parameters():
+            output = super().forward(*args, **kwargs)
+        outputs = list(output) if isinstance(output, (tuple, list)) else [output]
+        for i, quantizer in enumerate(self.output_quantizers):
+            if quantizer and i < len(outputs) and isinstance(outputs[i], torch.Tensor) and \
+                    outputs[i].is_floating_point():
+                outputs[i] = quantizer(outputs[i])
+        return type(output)(outputs) if isinstance(output, (tuple, list)) else outputs[0]
+
+    @classmethod
+    def wrap(cls, module_cls: Type[nn.Module]):
+        """Creates (and registers) the quantized class of a single-input, single-output module class."""
+        if module_cls in cls.cls_to_qcls:
+            return cls.cls_to_qcls[module_cls]
+        quantized_cls = type(f"Quantized{module_cls.__name__}", (cls, module_cls), {})
+        return cls.implements(module_cls)(quantized_cls)
+
+
+for _cls in (nn.Linear, nn.Conv1d, nn.Conv2d, nn.Conv3d, nn.ConvTranspose1d, nn.ConvTranspose2d, nn.ConvTranspose3d,
+             nn.ReLU, nn.ReLU6, nn.Sigmoid, nn.Tanh, nn.Hardtanh, nn.MaxPool2d, nn.AvgPool2d, nn.AdaptiveAvgPool2d,
+             nn.Flatten, nn.Dropout, nn.BatchNorm2d, nn.LayerNorm, nn.GELU, nn.SiLU, nn.Softmax):
+    QuantizationMixin.wrap(_cls)
+
+QuantizedLinear = QuantizationMixin.cls_to_qcls[nn.Linear]
+QuantizedConv2d = QuantizationMixin.cls_to_qcls[nn.Conv2d]
+QuantizedConvTranspose2d = QuantizationMixin.cls_to_qcls[nn.ConvTranspose2d]
+QuantizedReLU = QuantizationMixin.cls_to_qcls[nn.ReLU]

@@ -403,3 +403,85 @@ def test_apply_adaround_end_to_end(tmp_path, oracle):
             layer_q.weight.copy_(torch.from_numpy(w_seen))
     assert not any(isinstance(m, torch.nn.Module) and type(m).__name__.endswith("Wrapper")
                    for m in ada_model.modules())
+
+
+def test_v2_quantized_modules_and_sim():
+    """v2 quantized modules: parameters and activations are quantize-dequantized around the base forward."""
+    from aimet_amd.v2.nn import QuantizationMixin, QuantizedLinear
+    from aimet_amd.v2.quantization.affine import QuantizeDequantize
+    from aimet_amd.v2.quantsim import QuantizationSimModel
+    torch.manual_seed(0)
+    lin = torch.nn.Linear(16, 8).cuda()
+    q = QuantizationMixin.from_module(lin)
+    assert isinstance(q, QuantizedLinear) and isinstance(q, torch.nn.Linear) and q.weight is lin.weight
+    x = torch.randn(4, 16).cuda()
+    assert torch.equal(q(x), lin(x))                         # no quantizers yet
+    q.param_quantizers['weight'] = QuantizeDequantize((), bitwidth=4, symmetric=True).cuda()
+    q.output_quantizers[0] = QuantizeDequantize((), bitwidth=8, symmetric=False).cuda()
+    with q.compute_encodings():
+        q(x)
+    wq = q.param_quantizers['weight']
+    assert wq.is_initialized() and q.output_quantizers[0].is_initialized()
+    want = q.output_quantizers[0](torch.nn.functional.linear(x, wq(lin.weight), lin.bias))
+    assert torch.equal(q(x), want)
+    assert q.weight is lin.weight                            # the patch is gone after the call
+    with pytest.raises(RuntimeError):
+        QuantizationMixin.from_module(torch.nn.Bilinear(2, 2, 2))
+    model = _TinyNet().eval().cuda()
+    sim = QuantizationSimModel(model, torch.randn(1, 3, 8, 8).cuda(), quant_scheme='tf', default_param_bw=8)
+    names = [n for n, _ in sim.qmodules()]
+    assert names == ["conv1", "relu1", "pool", "flatten", "fc"]
+    sim.compute_encodings(lambda m, a: m(a), torch.randn(8, 3, 8, 8).cuda())
+    y = sim.model(torch.randn(2, 3, 8, 8).cuda())
+    assert y.shape == (2, 10) and torch.isfinite(y).all()
+
+
+def test_v2_apply_adaround_end_to_end(tmp_path, oracle):
+    """aimet_amd.v2.adaround.Adaround.apply_adaround (signed grid of the symmetric v2 weight quantizers) against the
+    same flow replayed with the CPU restatement."""
+    from aimet_amd.v2.adaround import Adaround, AdaroundParameters, AdaroundWrapper
+    from aimet_amd.v2.nn import BaseQuantizationMixin
+    from aimet_amd.common.defs import QuantScheme
+    torch.manual_seed(0)
+    model = _TinyNet().eval().cuda()
+    dummy = torch.randn(1, 3, 8, 8).cuda()
+    loader = _loader(4, 16, 7)
+    iters = 30
+    params = AdaroundParameters(loader, num_batches=4, default_num_iterations=iters, forward_fn=_forward_fn)
+    torch.manual_seed(4321)
+    ada_model = Adaround.apply_adaround(model, dummy, params, str(tmp_path), "tiny2", default_param_bw=4,
+                                        default_quant_scheme=QuantScheme.post_training_tf)
+    assert not any(isinstance(m, (BaseQuantizationMixin, AdaroundWrapper)) for m in ada_model.modules())
+    with open(os.path.join(str(tmp_path), "tiny2.encodings")) as f:
+        enc = json.load(f)["param_encodings"]
+    assert set(enc) == {"conv1.weight", "fc.weight"}
+    cpu = _TinyNet().eval()
+    cpu.load_state_dict({k: v.cpu() for k, v in model.state_dict().items()})
+    quant = _TinyNet().eval()
+    quant.load_state_dict(cpu.state_dict())
+    torch.manual_seed(4321)
+    xs = torch.cat([b[0].cpu() for b in loader])
+    for name, kind, act, conv_args in (("conv1", "conv2d", torch.relu, {"padding": 1}), ("fc", "linear", None, {})):
+        e = enc[name + ".weight"][0]
+        assert e["bitwidth"] == 4 and e["is_symmetric"] == "True" and e["offset"] == 0
+        delta = torch.tensor([e["scale"]], dtype=torch.float32)
+        offset = torch.tensor([0.0])
+        layer_fp, layer_q = getattr(cpu, name), getattr(quant, name)
+        with torch.no_grad():
+            if name == "conv1":
+                inp, out = xs, layer_fp(xs)
+            else:
+                inp = quant.flatten(quant.pool(torch.relu(quant.conv1(xs))))
+                out = layer_fp(cpu.flatten(cpu.pool(torch.relu(cpu.conv1(xs)))))
+        weight = layer_fp.weight.detach()
+        alpha0 = ada.generate_alpha(weight, delta.reshape(()))
+        batches = [torch.randperm(inp.size(0))[:32] for _ in range(iters)]
+        alpha, _, _, _ = ada.optimize_rounding(kind, weight, alpha0, delta, offset, -8, 7, inp, out, batches, iters,
+                                               0.01, (20, 2), 0.2, bias=layer_fp.bias.detach(), act=act,
+                                               conv_args=conv_args)
+        w_ref = ada.apply_adaround(weight, alpha, delta.reshape(()), offset.reshape(()), -8, 7, True)
+        got = getattr(ada_model, name).weight.detach().cpu()
+        assert torch.allclose(got, w_ref, atol=float(delta) * 2e-3, rtol=0), name
+        w_seen, _, _ = oracle.v2_qdq(w_ref.numpy().reshape(-1), 1, w_ref.numel(), delta.numpy(), offset.numpy(), -8, 7)
+        with torch.no_grad():
+            layer_q.weight.copy_(torch.from_numpy(w_seen.reshape(w_ref.shape)))
