@@ -29,11 +29,9 @@ using namespace ada;
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kBatch   = 32;    // rows per iteration (BATCH_SIZE of ADA/adaround_optimizer.py:58)
-constexpr int kFwdOBlk = 64;    // output channels per forward workgroup
-constexpr int kFwdKBlk = 256;   // K extent per forward workgroup (64 per wavefront)
-constexpr int kBwdOBlk = 32;    // output channels per backward workgroup
-constexpr int kBwdKBlk = 256;   // K extent per backward workgroup (64 per wavefront)
+constexpr int kBatch  = 32;    // rows per iteration (BATCH_SIZE of ADA/adaround_optimizer.py:58)
+constexpr int kTileO  = 32;    // output channels per workgroup
+constexpr int kTileK  = 256;   // K extent per workgroup: one 1 KiB row segment per wavefront-wide 16-byte access
 
 struct LinGeom
 {
@@ -59,86 +57,100 @@ __device__ __forceinline__ v4f ldg4_stream(const float* p)
     return __builtin_nontemporal_load(reinterpret_cast<const v4f*>(p));
 }
 
-// grid (O / 64, K / 256), 256 threads.  Wavefront w of a workgroup takes k in [256 by + 64 w, +64).
-__global__ __launch_bounds__(256) void lin_fwd_kernel(const float* __restrict__ W, const float* __restrict__ alpha,
+constexpr int kLdsRow = kTileK + 4;   // floats per LDS tile row; the pad spreads the MFMA-layout accesses over banks
+
+// Both kernels work on a [32 o] x [256 k] tile of the weight-shaped tensors per workgroup and move it through LDS, so
+// that global memory is always touched in the streaming layout (lane l of a wavefront owns floats 4l..4l+3 of a 1 KiB
+// row segment: fully coalesced) while the MFMAs see their own operand / accumulator layout.
+// (Measured alternative: wavefront-private [16 o] x [128 k] tiles without workgroup barriers were 10-20 % slower.)
+
+// grid (O / 32, K / 256), 256 threads.
+__global__ __launch_bounds__(256) void lin_fwd_kernel(const float* __restrict__ F, const float* __restrict__ alpha,
                                                       const float* __restrict__ X, const int* __restrict__ row_index,
                                                       int64_t x_row_stride, float* __restrict__ partial, LinGeom g)
 {
+    __shared__ __attribute__((aligned(16))) float tile[kTileO * kLdsRow];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int n = lane & 15, s = lane >> 4;
-    const int o_blk = blockIdx.x * kFwdOBlk;
-    const int k_blk = blockIdx.y * kFwdKBlk + wave * 64;
+    const int o_blk = blockIdx.x * kTileO;
+    const int k_blk = blockIdx.y * kTileK;
     const int K     = g.in_features;
 
-    float d[4], off[4];
-    const float* wrow[4];
-    const float* arow[4];
+    // phase 1: adarounded weight tile, streaming layout: wavefront w forms rows 8w .. 8w+7
+    v4f f[8], al[8];
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt)
+    for (int j = 0; j < 8; ++j)
     {
-        const int o = o_blk + nt * 16 + n;
-        d[nt]       = g.delta[o * g.chan_stride];
-        off[nt]     = g.offset[o * g.chan_stride];
-        wrow[nt]    = W + (int64_t) o * K;
-        arow[nt]    = alpha + (int64_t) o * K;
+        const int64_t e = (int64_t) (o_blk + wave * 8 + j) * K + k_blk + 4 * lane;
+        f[j]            = ldg4_stream(F + e);
+        al[j]           = ldg4_stream(alpha + e);
     }
+    // the activations of this wavefront's MFMA k-range [64w, 64w + 64), fetched while the weights are in flight
     const float* xrow[2];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
     {
         const int b = mt * 16 + n;
-        xrow[mt]    = X + (int64_t) (row_index ? row_index[b] : b) * x_row_stride;
+        xrow[mt]    = X + (int64_t) (row_index ? row_index[b] : b) * x_row_stride + k_blk + wave * 64 + 4 * s;
     }
+    v4f a[4][2];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+            a[kk][mt] = ldg4(xrow[mt] + kk * 16);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+    {
+        const int r   = wave * 8 + j;
+        const int c   = (o_blk + r) * g.chan_stride;
+        const float d = g.delta[c], off = g.offset[c];
+        v4f wq;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            wq[t] = adarounded_f<true>(f[j][t], al[j][t], d, off, g.clip_min, g.clip_max);
+        *reinterpret_cast<v4f*>(&tile[r * kLdsRow + 4 * lane]) = wq;
+    }
+    __syncthreads();
 
-    v4f acc[2][4];
+    // phase 2: out[b][o] += x[b][k] W'[o][k] over this wavefront's 64 k
+    v4f acc[2][2];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
+        for (int nt = 0; nt < 2; ++nt)
             acc[mt][nt] = (v4f) {0.f, 0.f, 0.f, 0.f};
-
-#pragma unroll 2
-    for (int kk = 0; kk < 64; kk += 16)
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
     {
-        const int k = k_blk + kk + 4 * s;
-        v4f w[4], al[4], a[2];
+        const int col = wave * 64 + kk * 16 + 4 * s;
+        v4f wq[2];
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
-        {
-            w[nt]  = ldg4_stream(wrow[nt] + k);
-            al[nt] = ldg4_stream(arow[nt] + k);
-        }
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-            a[mt] = ldg4(xrow[mt] + k);
-        v4f wq[4];
-#pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-                wq[nt][t] = adarounded_f<true>(w[nt][t], al[nt][t], d[nt], off[nt], g.clip_min, g.clip_max);
+        for (int nt = 0; nt < 2; ++nt)
+            wq[nt] = *reinterpret_cast<const v4f*>(&tile[(nt * 16 + n) * kLdsRow + col]);
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int nt = 0; nt < 4; ++nt)
+            for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
                 for (int mt = 0; mt < 2; ++mt)
-                    acc[mt][nt] = mfma16(a[mt][t], wq[nt][t], acc[mt][nt]);
+                    acc[mt][nt] = mfma16(a[kk][mt][t], wq[nt][t], acc[mt][nt]);
     }
+    __syncthreads();   // every wavefront is done reading the weight tile: its memory now holds the partial products
 
-    // add the four wavefronts' products in wavefront order, then one partial tile per workgroup
-    __shared__ v4f red[4][8][64];
+    // add the four wavefronts' products in wavefront order, then one partial [32, 32] tile per workgroup
+    v4f* red = reinterpret_cast<v4f*>(tile);   // [4 waves][4 tiles][64 lanes]
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-        for (int nt = 0; nt < 4; ++nt)
-            red[wave][mt * 4 + nt][lane] = acc[mt][nt];
+        for (int nt = 0; nt < 2; ++nt)
+            red[(wave * 4 + mt * 2 + nt) * 64 + lane] = acc[mt][nt];
     __syncthreads();
-    for (int idx = threadIdx.x; idx < 8 * 64; idx += 256)
     {
-        const int tile = idx >> 6, ln = idx & 63;
-        const v4f sum  = ((red[0][tile][ln] + red[1][tile][ln]) + red[2][tile][ln]) + red[3][tile][ln];
-        const int mt = tile >> 2, nt = tile & 3;
+        const int t4 = threadIdx.x >> 6, ln = threadIdx.x & 63;   // tile index, lane within the tile
+        const v4f sum = ((red[(0 * 4 + t4) * 64 + ln] + red[(1 * 4 + t4) * 64 + ln]) + red[(2 * 4 + t4) * 64 + ln]) +
+                        red[(3 * 4 + t4) * 64 + ln];
+        const int mt = t4 >> 1, nt = t4 & 1;
         const int o  = o_blk + nt * 16 + (ln & 15);
         const int b0 = mt * 16 + 4 * (ln >> 4);
         float* dst   = partial + ((int64_t) blockIdx.y * kBatch + b0) * g.out_features + o;
@@ -187,20 +199,34 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
     }
 }
 
-// grid (O / 32, K / 256), 256 threads.  Wavefront w takes k in [256 by + 64 w, +64): four 16-wide k tiles (the M
-// dimension of the MFMA) by two 16-wide o tiles (N); the batch is the MFMA's K dimension, 8 steps of 4.
-__global__ __launch_bounds__(256) void lin_bwd_kernel(const float* __restrict__ W, const float* __restrict__ G,
+// grid (O / 32, K / 256), 256 threads.  Phase 1: wavefront w forms dLoss/dW' for k in [64w, 64w + 64) as four 16-wide k
+// tiles (the M dimension of the MFMA) by two 16-wide o tiles (N), the batch being the MFMA's K dimension (8 steps of
+// 4), and parks it in the LDS tile.  Phase 2: the alpha-gradient + regulariser + Adam epilogue in the streaming layout.
+__global__ __launch_bounds__(256) void lin_bwd_kernel(const float* __restrict__ F, const float* __restrict__ G,
                                                       const float* __restrict__ X, const int* __restrict__ row_index,
                                                       int64_t x_row_stride, float* __restrict__ alpha,
                                                       float* __restrict__ m, float* __restrict__ v,
                                                       float* __restrict__ grad_out, LinGeom g, AdamArgs a,
                                                       float* __restrict__ reg_partial)
 {
+    __shared__ __attribute__((aligned(16))) float tile[kTileO * kLdsRow];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int n = lane & 15, s = lane >> 4;
-    const int o_blk = blockIdx.x * kBwdOBlk;
-    const int k_blk = blockIdx.y * kBwdKBlk + wave * 64;
+    const int o_blk = blockIdx.x * kTileO;
+    const int k_blk = blockIdx.y * kTileK;
     const int K = g.in_features, O = g.out_features;
+
+    // the epilogue's first rows are requested before the MFMA phase so that they arrive while it runs
+    v4f fv[2], av[2], mv[2], vv[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+    {
+        const int64_t e = (int64_t) (o_blk + wave * 8 + j) * K + k_blk + 4 * lane;
+        fv[j]           = ldg4_stream(F + e);
+        av[j]           = ldg4(alpha + e);
+        mv[j]           = ldg4(m + e);
+        vv[j]           = ldg4(v + e);
+    }
 
     v4f acc[4][2];
 #pragma unroll
@@ -208,12 +234,11 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const float* __restrict__ 
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
             acc[mt][nt] = (v4f) {0.f, 0.f, 0.f, 0.f};
-
 #pragma unroll
     for (int step = 0; step < 8; ++step)
     {
         const int b       = 4 * step + s;
-        const float* xrow = X + (int64_t) (row_index ? row_index[b] : b) * x_row_stride + k_blk + n;
+        const float* xrow = X + (int64_t) (row_index ? row_index[b] : b) * x_row_stride + k_blk + wave * 64 + n;
         const float* grow = G + (int64_t) b * O + o_blk + n;
         float xa[4], gb[2];
 #pragma unroll
@@ -228,40 +253,50 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const float* __restrict__ 
             for (int nt = 0; nt < 2; ++nt)
                 acc[mt][nt] = mfma16(xa[mt], gb[nt], acc[mt][nt]);
     }
+    // lane holds dW'[o = 16 nt + n][k = 64 w + 16 mt + 4 s + i], i = 0..3
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+            *reinterpret_cast<v4f*>(&tile[(nt * 16 + n) * kLdsRow + wave * 64 + mt * 16 + 4 * s]) = acc[mt][nt];
+    __syncthreads();
 
-    // lane holds dW'[o = o_blk + 16 nt + n][k = k_blk + 16 mt + 4 s + i], i = 0..3: one 16-byte vector per tile
     float reg = 0.f;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+    for (int j = 0; j < 8; ++j)
     {
-        const int o   = o_blk + nt * 16 + n;
-        const float d = g.delta[o * g.chan_stride], off = g.offset[o * g.chan_stride];
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
+        const int r     = wave * 8 + j;
+        const int slot  = j & 1;
+        const int64_t e = (int64_t) (o_blk + r) * K + k_blk + 4 * lane;
+        const v4f f4 = fv[slot], a4 = av[slot], m4 = mv[slot], v4 = vv[slot];
+        if (j + 2 < 8)
         {
-            const int64_t e = (int64_t) o * K + k_blk + mt * 16 + 4 * s;
-            const v4f wv    = ldg4_stream(W + e);
-            const v4f av    = ldg4(alpha + e);
-            const v4f mv    = ldg4(m + e);
-            const v4f vv    = ldg4(v + e);
-            float as[4] = {av[0], av[1], av[2], av[3]}, ms[4] = {mv[0], mv[1], mv[2], mv[3]};
-            float vs[4] = {vv[0], vv[1], vv[2], vv[3]};
-            v4f gr;
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-            {
-                float r;
-                const float gi = alpha_grad_f(wv[i], acc[mt][nt][i], as[i], d, off, g.clip_min, g.clip_max, a, r);
-                reg += r;
-                adam_update(gi, as[i], ms[i], vs[i], a);
-                gr[i] = gi;
-            }
-            *reinterpret_cast<v4f*>(alpha + e) = (v4f) {as[0], as[1], as[2], as[3]};
-            *reinterpret_cast<v4f*>(m + e)     = (v4f) {ms[0], ms[1], ms[2], ms[3]};
-            *reinterpret_cast<v4f*>(v + e)     = (v4f) {vs[0], vs[1], vs[2], vs[3]};
-            if (grad_out)
-                *reinterpret_cast<v4f*>(grad_out + e) = gr;
+            const int64_t e2 = e + 2 * (int64_t) K;
+            fv[slot]         = ldg4_stream(F + e2);
+            av[slot]         = ldg4(alpha + e2);
+            mv[slot]         = ldg4(m + e2);
+            vv[slot]         = ldg4(v + e2);
         }
+        const int c   = (o_blk + r) * g.chan_stride;
+        const float d = g.delta[c], off = g.offset[c];
+        const v4f gw  = *reinterpret_cast<const v4f*>(&tile[r * kLdsRow + 4 * lane]);
+        float as[4] = {a4[0], a4[1], a4[2], a4[3]}, ms[4] = {m4[0], m4[1], m4[2], m4[3]};
+        float vs[4] = {v4[0], v4[1], v4[2], v4[3]};
+        v4f gr;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+        {
+            float rr;
+            const float gi = alpha_grad_f(f4[i], gw[i], as[i], d, off, g.clip_min, g.clip_max, a, rr);
+            reg += rr;
+            adam_update(gi, as[i], ms[i], vs[i], a);
+            gr[i] = gi;
+        }
+        *reinterpret_cast<v4f*>(alpha + e) = (v4f) {as[0], as[1], as[2], as[3]};
+        *reinterpret_cast<v4f*>(m + e)     = (v4f) {ms[0], ms[1], ms[2], ms[3]};
+        *reinterpret_cast<v4f*>(v + e)     = (v4f) {vs[0], vs[1], vs[2], vs[3]};
+        if (grad_out)
+            *reinterpret_cast<v4f*>(grad_out + e) = gr;
     }
     if (reg_partial)
     {
@@ -275,8 +310,8 @@ int make_lin_geom(LinGeom& g, int64_t out_features, int64_t in_features, int64_t
                   const float* offset, float clip_min, float clip_max)
 {
     MIQ_CHECK_ARG(out_features > 0 && in_features > 0, "bad layer shape");
-    MIQ_CHECK_ARG(out_features % kFwdOBlk == 0 && in_features % kFwdKBlk == 0,
-                  "the fused Linear path takes out_features that are a multiple of 64 and in_features that are a "
+    MIQ_CHECK_ARG(out_features % kTileO == 0 && in_features % kTileK == 0,
+                  "the fused Linear path takes out_features that are a multiple of 32 and in_features that are a "
                   "multiple of 256 (got %lld x %lld)", (long long) out_features, (long long) in_features);
     MIQ_CHECK_ARG(out_features * in_features < (1ll << 31), "layer too large for the fused Linear path");
     MIQ_CHECK_ARG(num_channel == 1 || num_channel == out_features,
@@ -303,13 +338,13 @@ int64_t miq_adaround_linear_workspace_bytes(int64_t out_features, int64_t in_fea
 {
     if (out_features <= 0 || in_features <= 0)
         return 0;
-    const int64_t splits = (in_features + kFwdKBlk - 1) / kFwdKBlk;
+    const int64_t splits = (in_features + kTileK - 1) / kTileK;
     return splits * kBatch * out_features * (int64_t) sizeof(float);
 }
 
 int miq_adaround_linear_blocks(int64_t out_features, int64_t in_features)
 {
-    return (int) ((out_features / kBwdOBlk) * (in_features / kBwdKBlk));
+    return (int) ((out_features / kTileO) * (in_features / kTileK));
 }
 
 int miq_adaround_linear_fwd_f32(const float* weight, const float* alpha, const float* x, const int32_t* row_index,
@@ -327,8 +362,8 @@ int miq_adaround_linear_fwd_f32(const float* weight, const float* alpha, const f
                   "weight, alpha and the rows of x must be 16-byte aligned");
     MIQ_CHECK_ARG(x_row_stride >= in_features && target_row_stride >= out_features, "row stride shorter than a row");
     MIQ_CHECK_ARG(activation == 0 || activation == 1, "activation must be 0 (none) or 1 (ReLU)");
-    const int splits = (int) (in_features / kFwdKBlk);
-    hipLaunchKernelGGL(lin_fwd_kernel, dim3((unsigned) (out_features / kFwdOBlk), (unsigned) splits), dim3(256), 0,
+    const int splits = (int) (in_features / kTileK);
+    hipLaunchKernelGGL(lin_fwd_kernel, dim3((unsigned) (out_features / kTileO), (unsigned) splits), dim3(256), 0,
                        (hipStream_t) stream, weight, alpha, x, row_index, x_row_stride, workspace, g);
     MIQ_CHECK_LAUNCH();
     const unsigned blocks = (unsigned) ((kBatch * out_features + 255) / 256);
@@ -356,7 +391,7 @@ int miq_adaround_linear_bwd_adam_f32(const float* weight, const float* grad_out,
     AdamArgs a;
     if (int rc = make_adam(a, reg_param, beta, lr, beta1, beta2, eps, step))
         return rc;
-    hipLaunchKernelGGL(lin_bwd_kernel, dim3((unsigned) (out_features / kBwdOBlk), (unsigned) (in_features / kBwdKBlk)),
+    hipLaunchKernelGGL(lin_bwd_kernel, dim3((unsigned) (out_features / kTileO), (unsigned) (in_features / kTileK)),
                        dim3(256), 0, (hipStream_t) stream, weight, grad_out, x, row_index, x_row_stride, alpha, exp_avg,
                        exp_avg_sq, grad_alpha, g, a, reg_partial);
     MIQ_CHECK_LAUNCH();

@@ -347,7 +347,7 @@ def adaround_bwd_adam(weight, grad_weight, alpha, exp_avg, exp_avg_sq, num_chann
 
 def adaround_linear_supported(out_features, in_features, batch):
     """Shapes the MFMA-fused Linear path takes."""
-    return batch == 32 and out_features % 64 == 0 and in_features % 256 == 0 and \
+    return batch == 32 and out_features % 32 == 0 and in_features % 256 == 0 and \
         out_features * in_features < 2 ** 31
 
 

@@ -26,7 +26,7 @@ ADAM_LR, ADAM_BETAS, ADAM_EPS = 1e-3, (0.9, 0.999), 1e-8      # torch.optim.Adam
 class AdaroundOptimizer:
     """Optimizes the weight rounding of a quantized wrapper module."""
 
-    # Linear layers whose shape the MFMA-fused kernels take (out % 64 == 0, in % 256 == 0, batch 32, no activation or
+    # Linear layers whose shape the MFMA-fused kernels take (out % 32 == 0, in % 256 == 0, batch 32, no activation or
     # ReLU) use them; everything else runs soft-round kernel + torch layer + fused backward/Adam kernel
     use_fused_linear = True
 

@@ -257,7 +257,7 @@ int miq_adaround_blocks(int64_t num_element);
  * row-major.  x: rows of in_features floats, row r at
  * x + r * x_row_stride; target likewise with out_features floats.  row_index: device int32[32] choosing the rows of x
  * and target (NULL = rows 0..31).  num_channel: 1 (per-tensor delta/offset) or out_features (per output channel).
- * Shapes: out_features % 64 == 0, in_features % 256 == 0, out_features * in_features < 2^31; other shapes return
+ * Shapes: out_features % 32 == 0, in_features % 256 == 0, out_features * in_features < 2^31; other shapes return
  * MIQ_ERR_INVALID_ARG and the caller uses the elementwise entry points around its own GEMM.
  * activation: 0 none, 1 ReLU (the act_func the reference applies to both outputs, ADA/adaround_optimizer.py:192-194).
  * ------------------------------------------------------------------------------------------------------------- */
