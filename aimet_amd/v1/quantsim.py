@@ -117,7 +117,7 @@ class QuantizationSimModel:
         """One hooked forward pass: execution order of the leaf modules and tensor producers / consumers."""
         records, handles = [], []
         producer: Dict[int, str] = {}
-        consumers: Dict[int, List[str]] = {}
+        consumers: Dict[str, List[str]] = {}      # producing module -> consuming modules
         keep_alive = []
         names = {m: n for n, m in model.named_modules()}
         for t in dummy_input:
@@ -131,7 +131,10 @@ class QuantizationSimModel:
                     if isinstance(t, torch.Tensor)]
             keep_alive.extend(ins + outs)            # ids stay unique while the pass runs
             for t in ins:
-                consumers.setdefault(id(t), []).append(name)
+                # resolved now, not afterwards: an in-place op returns the tensor it was given, so the tensor's id
+                # says nothing about who produced the value a later module reads
+                if id(t) in producer:
+                    consumers.setdefault(producer[id(t)], []).append(name)
             records.append({"name": name, "module": module, "type": _op_type(module),
                             "inputs": [producer.get(id(t)) for t in ins], "in_ids": [id(t) for t in ins],
                             "out_ids": [id(t) for t in outs], "num_inputs": max(1, len(ins)),
@@ -154,7 +157,7 @@ class QuantizationSimModel:
         outs = out if isinstance(out, (tuple, list)) else (out,)
         model_outputs = {producer.get(id(t)) for t in outs if isinstance(t, torch.Tensor)}
         for r in records:
-            r["consumers"] = [c for oid in r["out_ids"] for c in consumers.get(oid, [])]
+            r["consumers"] = list(consumers.get(r["name"], []))
             r["is_model_output"] = r["name"] in model_outputs
         return records
 

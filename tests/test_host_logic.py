@@ -1,0 +1,192 @@
+"""Host-side logic that needs no GPU: configuration of the simulation model, graph helpers of the AdaRound flow,
+argument handling of the v2 quantizers, the backend registry, and the failure behaviour of the loader."""
+import importlib
+import json
+import math
+import os
+
+import pytest
+import torch
+from torch import nn
+
+
+class _Net(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.conv1 = nn.Conv2d(3, 4, 3, padding=1)
+        self.relu1 = nn.ReLU(inplace=True)
+        self.conv2 = nn.Conv2d(4, 4, 3, padding=1)
+        self.bn = nn.BatchNorm2d(4)
+        self.drop = nn.Dropout(0.1)
+        self.flatten = nn.Flatten()
+        self.fc = nn.Linear(4 * 4 * 4, 5)
+        self.act = nn.ReLU()
+
+    def forward(self, x):
+        x = self.relu1(self.conv1(x))
+        x = self.drop(self.bn(self.conv2(x)))
+        return self.act(self.fc(self.flatten(x)))
+
+
+def test_quantsim_default_configuration():
+    """Which quantizers the default configuration switches on (reference default_config.json semantics: outputs
+    quantized, parameters symmetric, bias off, Conv+Relu / Gemm+Relu supergroups, model input quantized)."""
+    from aimet_amd.v1.quantsim import QuantizationSimModel
+    from aimet_amd.v1.qc_quantize_op import QcQuantizeOpMode, StaticGridQuantWrapper
+    model = _Net().eval()
+    sim = QuantizationSimModel(model, dummy_input=torch.randn(1, 3, 4, 4), default_param_bw=4, default_output_bw=16)
+    w = dict(sim.quant_wrappers())
+    assert list(w) == ["conv1", "relu1", "conv2", "bn", "drop", "flatten", "fc", "act"]
+    assert all(isinstance(x, StaticGridQuantWrapper) for x in w.values())
+    assert w["conv1"].input_quantizers[0].enabled and not w["conv2"].input_quantizers[0].enabled
+    assert not w["conv1"].output_quantizers[0].enabled and w["relu1"].output_quantizers[0].enabled   # Conv+Relu
+    assert w["conv2"].output_quantizers[0].enabled
+    assert not w["fc"].output_quantizers[0].enabled and w["act"].output_quantizers[0].enabled        # Gemm+Relu
+    assert not w["drop"].output_quantizers[0].enabled and not w["flatten"].output_quantizers[0].enabled
+    assert w["conv1"].param_quantizers["weight"].enabled and not w["conv1"].param_quantizers["bias"].enabled
+    assert not any(q.enabled for q in w["bn"].param_quantizers.values())
+    assert w["conv1"].param_quantizers["weight"].bitwidth == 4 and w["relu1"].output_quantizers[0].bitwidth == 16
+    assert w["conv1"].param_quantizers["weight"].use_symmetric_encodings
+    assert not w["relu1"].output_quantizers[0].use_symmetric_encodings
+    assert w["conv1"]._mode is QcQuantizeOpMode.ANALYSIS
+    # the original model is untouched; exclusion and stripping of wrappers
+    assert isinstance(model.conv1, nn.Conv2d)
+    sim.exclude_layers_from_quantization([w["bn"]])
+    assert isinstance(sim.model.bn, nn.BatchNorm2d)
+    QuantizationSimModel.remove_quantization_wrappers(sim.model)
+    assert not list(sim.quant_wrappers())
+    with pytest.raises(ValueError):
+        QuantizationSimModel(model, torch.randn(1, 3, 4, 4), default_param_bw=2)
+    with pytest.raises(ValueError):
+        QuantizationSimModel(model, torch.randn(1, 3, 4, 4), rounding_mode='up')
+
+
+def test_quantsim_config_file(tmp_path):
+    from aimet_amd.v1.quantsim import QuantizationSimModel
+    from aimet_amd.v1.tensor_quantizer import StaticGridPerChannelQuantizer
+    cfg = {"defaults": {"ops": {"is_output_quantized": "True", "is_symmetric": "True"},
+                        "params": {"is_quantized": "True", "is_symmetric": "False"},
+                        "strict_symmetric": "True", "per_channel_quantization": "True"},
+           "params": {"bias": {"is_quantized": "False"}},
+           "op_type": {"Relu": {"is_output_quantized": "False"}, "Conv": {"is_input_quantized": "True"}},
+           "supergroups": [], "model_input": {}, "model_output": {"is_output_quantized": "True"}}
+    path = os.path.join(str(tmp_path), "c.json")
+    with open(path, "w") as f:
+        json.dump(cfg, f)
+    sim = QuantizationSimModel(_Net().eval(), torch.randn(1, 3, 4, 4), quant_scheme='tf', config_file=path)
+    w = dict(sim.quant_wrappers())
+    assert isinstance(w["conv1"].param_quantizers["weight"], StaticGridPerChannelQuantizer)
+    assert len(w["conv1"].param_quantizers["weight"]._cppOp) == 4
+    assert w["conv2"].input_quantizers[0].enabled and w["conv1"].output_quantizers[0].enabled
+    assert not w["relu1"].output_quantizers[0].enabled
+    assert w["act"].output_quantizers[0].enabled                        # model output overrides the op-type rule
+    assert w["conv1"].output_quantizers[0].use_symmetric_encodings and w["conv1"].output_quantizers[0].use_strict_symmetric
+    assert not w["conv1"].param_quantizers["weight"].use_symmetric_encodings
+
+
+def test_graph_helpers():
+    from aimet_amd import utils
+    model = _Net().eval()
+    x = torch.randn(2, 3, 4, 4)
+    order = [n for n, _ in utils.get_ordered_list_of_modules(model, x)]
+    assert order == ["conv1", "relu1", "conv2", "bn", "drop", "flatten", "fc", "act"]
+    pairs = utils.get_module_act_func_pair(model, x)
+    assert pairs[model.conv1] is model.relu1          # through the in-place ReLU
+    assert pairs[model.conv2] is None and pairs[model.fc] is model.act
+    assert utils.get_named_module(model, "fc") is model.fc
+    loader = [(torch.randn(2, 3, 4, 4), torch.zeros(2)) for _ in range(3)]
+    cached = utils.CachedDataset(loader, 2)
+    assert len(cached) == 2 and cached[1][0] is loader[1][0]
+    with pytest.raises(ValueError):
+        utils.CachedDataset(loader, 4)
+    inp, out = utils.ModuleData(model, model.conv2, lambda m, b: m(b[0])).collect_inp_out_data(loader[0], True, True)
+    with torch.no_grad():
+        want_in = model.relu1(model.conv1(loader[0][0]))
+    assert torch.allclose(inp, want_in) and torch.allclose(out, model.conv2(want_in))
+
+
+def test_adaround_parameters_and_schedule():
+    from aimet_amd.v1.adaround.adaround_loss import AdaroundHyperParameters, AdaroundLoss
+    from aimet_amd.v1.adaround.adaround_weight import AdaroundParameters
+    with pytest.raises(ValueError):
+        AdaroundParameters([1, 2], num_batches=3)
+    p = AdaroundParameters([1, 2, 3], num_batches=2)
+    assert (p.num_iterations, p.reg_param, p.beta_range, p.warm_start) == (None, 0.01, (20, 2), 0.2)
+    # known answers of the reference's tests (test_adaround_loss.py:76-100)
+    assert AdaroundLoss._compute_beta(10000, 8000, (20, 2), 0.2) == 4.636038969321072
+    import numpy as np
+    np.random.seed(0)
+    alpha = torch.from_numpy(np.random.rand(1, 3, 12, 12))
+    hp = AdaroundHyperParameters(10000, 0.01, (20, 2), 0.2)
+    assert AdaroundLoss.compute_round_loss(alpha, hp, 10) == 0
+    assert AdaroundLoss.compute_round_loss(alpha, hp, 8000).item() == pytest.approx(4.266156963161077, abs=1e-5)
+    a, b = torch.rand(8, 3, 4, 4), torch.rand(8, 3, 4, 4)
+    assert AdaroundLoss.compute_recon_loss(a, b).item() == pytest.approx(
+        torch.nn.functional.mse_loss(a, b, reduction='none').sum(1).mean().item(), abs=1e-5)
+
+
+def test_v2_quantizer_arguments_and_registry():
+    from aimet_amd.v2.quantization.affine import QuantizeDequantize, backends
+    from aimet_amd.v2.quantization.affine.backends import _derive_qmin_qmax
+    assert _derive_qmin_qmax(bitwidth=8, signed=True) == (-128, 127)
+    assert _derive_qmin_qmax(bitwidth=4, signed=False) == (0, 15)
+    assert _derive_qmin_qmax(num_steps=254, signed=True) == (-127, 127)
+    q = QuantizeDequantize((4, 1), 8, True)
+    assert (q.qmin, q.qmax, q.symmetric, q.bitwidth, q.signed) == (-128, 127, True, 8, True)
+    q = QuantizeDequantize((), qmin=0, qmax=15, symmetric=False)
+    assert q.bitwidth == 4 and not q.signed and not q.is_initialized()
+    with pytest.raises(ValueError):
+        QuantizeDequantize((), qmin=5, qmax=5, symmetric=False)
+    with pytest.raises(TypeError):
+        QuantizeDequantize((), 8)
+    with pytest.raises(RuntimeError):
+        q(torch.randn(3))                                   # not initialised
+    q.set_range(torch.tensor(-1.0), torch.tensor(2.0))
+    assert q.is_initialized() and q.get_scale().item() == pytest.approx(3 / 15)
+    assert q.get_offset().item() == round(-1.0 / (3 / 15))
+    with pytest.raises(RuntimeError):
+        q(torch.randn(3))                                   # CPU tensor: the backend computes on the GPU only
+    with pytest.raises(RuntimeError):
+        backends.set_global_backend("nope")
+    with pytest.raises(RuntimeError):
+        backends.add_backend("hip_gfx950", object())
+    enc = q.get_legacy_encodings()
+    assert enc[0]["bitwidth"] == 4 and enc[0]["is_symmetric"] == "False"
+
+
+def test_v2_minmax_analyzer_formulas():
+    """MinMaxEncodingAnalyzer.compute_encodings_from_stats on CPU statistics (pure tensor arithmetic): the cases of
+    the reference's test_encoding_analyzer.py for min-max (zero included, symmetric grid, degenerate range)."""
+    from aimet_amd.v2.quantization.encoding_analyzer import MinMaxEncodingAnalyzer, _MinMaxRange
+    from aimet_amd.v2.utils import StatisticsNotFoundError
+    an = MinMaxEncodingAnalyzer((1,))
+    mn, mx = an.compute_encodings_from_stats(_MinMaxRange(torch.tensor([2.0]), torch.tensor([5.0])), 255, False)
+    assert mn.item() == 0 and mx.item() == 5
+    mn, mx = an.compute_encodings_from_stats(_MinMaxRange(torch.tensor([-3.0]), torch.tensor([5.0])), 255, True)
+    delta = max(5 / 127, 3 / 128)
+    assert mn.item() == pytest.approx(-128 * delta) and mx.item() == pytest.approx(127 * delta)
+    mn, mx = an.compute_encodings_from_stats(_MinMaxRange(torch.tensor([0.0]), torch.tensor([0.0])), 255, False)
+    assert mn.item() == 0 and mx.item() == pytest.approx(255 * torch.finfo(torch.float32).eps)
+    with pytest.raises(StatisticsNotFoundError):
+        an.compute_encodings(255, False)
+    with pytest.raises(ValueError):
+        an.compute_encodings_from_stats(_MinMaxRange(torch.tensor([0.0]), torch.tensor([1.0])), 0, False)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    """There is no CPU fallback: without libmiq.so the package's loader raises ImportError."""
+    import aimet_amd._lib as lib_mod
+    monkeypatch.setattr(lib_mod, "LIB_PATH", os.path.join(str(tmp_path), "libmiq.so"))
+    with pytest.raises(ImportError, match="no CPU fallback"):
+        lib_mod._load()
+
+
+def test_cpu_tensors_are_rejected_everywhere():
+    from aimet_amd import ops
+    x = torch.randn(16)
+    for call in (lambda: ops.qdq_per_tensor(x, -1.0, 1.0, 8), lambda: ops.minmax(x),
+                 lambda: ops.v2_qdq(x, 1, 16, torch.ones(1), torch.zeros(1), 0, 255),
+                 lambda: ops.adaround_init_alpha(x, 1, 16, torch.ones(1)),
+                 lambda: ops.Analyzer(1, torch.device("cpu")).update_stats(x)):
+        with pytest.raises((RuntimeError, AssertionError)):
+            call()
