@@ -71,7 +71,7 @@ _SIGNATURES = {
     "miq_adaround_bwd_f32": ([_p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _flt, _flt, _p, _p], _int),
     "miq_adaround_blocks": ([_i64], _int),
     "miq_v2_hist_workspace_bytes": ([_i64, _i64, _int], _i64),
-    "miq_v2_hist_update_f32": ([_p, _i64, _i64, _int, _int, _p, _p, _p, _p, _p, _p, _p], _int),
+    "miq_v2_hist_update_f32": ([_p, _i64, _i64, _int, _int, _int, _p, _p, _p, _p, _p, _p, _p], _int),
     "miq_v2_sqnr_num_candidates": ([_dbl, _int, _int, _int, _int], _int),
     "miq_v2_sqnr_search_f32": ([_p, _p, _i64, _int, _dbl, _int, _dbl, _int, _int, _int, _p, _p, _p, _p, _p], _int),
     "miq_adaround_linear_workspace_bytes": ([_i64, _i64], _i64),

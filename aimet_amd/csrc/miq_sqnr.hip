@@ -27,11 +27,14 @@ constexpr int kMaxBins    = 4096;
 constexpr int kHistBlock  = 256;
 constexpr float kMinScale = 1.1920928955078125e-07f;   // torch.finfo(torch.float32).eps (EA:322)
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+
 // ---- finite min / max per row --------------------------------------------------------------------------------
 // partial[(h * blocks + b) * 2 + {0,1}]
 __global__ __launch_bounds__(kHistBlock) void finite_minmax_kernel(const float* __restrict__ x, int64_t n_per_hist,
                                                                    float* __restrict__ partial,
-                                                                   uint32_t* __restrict__ sums, int sums_per_hist)
+                                                                   uint32_t* __restrict__ sums, int sums_per_hist,
+                                                                   int vec)
 {
     const int h = blockIdx.y;
     // this launch also clears the count sums that the later kernels of the same update accumulate into
@@ -39,15 +42,43 @@ __global__ __launch_bounds__(kHistBlock) void finite_minmax_kernel(const float* 
         sums[(int64_t) h * sums_per_hist + i] = 0;
     const float* row = x + (int64_t) h * n_per_hist;
     float lo = INFINITY, hi = -INFINITY;
-    for (int64_t i = (int64_t) blockIdx.x * kHistBlock + threadIdx.x; i < n_per_hist;
-         i += (int64_t) gridDim.x * kHistBlock)
-    {
-        const float v = row[i];
+    auto take = [&](float v) {
         if (fabsf(v) < INFINITY)   // false for NaN and +-inf
         {
             lo = fminf(lo, v);
             hi = fmaxf(hi, v);
         }
+    };
+    if (vec)
+    {
+        // 16-byte loads, four in flight per lane
+        const v4f* rv       = reinterpret_cast<const v4f*>(row);
+        const int64_t nvec  = n_per_hist / 4;
+        const int64_t stride = (int64_t) gridDim.x * kHistBlock * 4;
+        for (int64_t base = (int64_t) blockIdx.x * kHistBlock * 4; base < nvec; base += stride)
+        {
+            v4f a[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+            {
+                const int64_t i = base + u * kHistBlock + threadIdx.x;
+                a[u]            = i < nvec ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+            {
+                take(a[u][0]);
+                take(a[u][1]);
+                take(a[u][2]);
+                take(a[u][3]);
+            }
+        }
+    }
+    else
+    {
+        for (int64_t i = (int64_t) blockIdx.x * kHistBlock + threadIdx.x; i < n_per_hist;
+             i += (int64_t) gridDim.x * kHistBlock)
+            take(row[i]);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1)
@@ -82,42 +113,25 @@ struct Ranges
     float m_lo, m_hi;   // range torch.histc uses for the merged histogram
     float new_min, new_max;   // merged (min, max) statistics
     float old_min, old_max;   // statistics before this update
+    float batch_min, batch_max;   // finite (min, max) of the batch
     int   rebin;        // 1: the running histogram has to be re-binned into the merged range
     int   pad;
 };
 
-// grid H, one wavefront per histogram: reduces the workgroups' (min, max), then lane 0 does the scalar work of
-// _create_bin_edges and of merge_stats' range logic
-__global__ __launch_bounds__(64) void ranges_kernel(const float* __restrict__ partial, int blocks, int num_bins,
-                                                    int has_stats, const float* __restrict__ state_minmax,
-                                                    float* __restrict__ batch_minmax, Ranges* __restrict__ ranges,
-                                                    int* __restrict__ bad_flag, int num_hist)
+// The scalar work of _create_bin_edges and of merge_stats' range logic for one histogram, from the batch's finite
+// (min, max); `ok` is false when the batch held no finite value (the reference raises ValueError there).
+__device__ Ranges compute_ranges(float lo, float hi, int num_bins, int has_stats, const float* __restrict__ state_minmax,
+                                 int h, bool& ok)
 {
-    const int h = blockIdx.x;
-    float lo = INFINITY, hi = -INFINITY;
-    for (int b = threadIdx.x; b < blocks; b += 64)
+    ok = lo <= hi;
+    if (!ok)
     {
-        lo = fminf(lo, partial[((int64_t) h * blocks + b) * 2]);
-        hi = fmaxf(hi, partial[((int64_t) h * blocks + b) * 2 + 1]);
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1)
-    {
-        lo = fminf(lo, __shfl_xor(lo, o));
-        hi = fmaxf(hi, __shfl_xor(hi, o));
-    }
-    if (threadIdx.x != 0)
-        return;
-    if (!(lo <= hi))
-    {
-        // no finite value at all: the reference raises ValueError here; reported when the statistics are next read
-        atomicOr(bad_flag, 1);
         lo = 0.f;
         hi = 0.f;
     }
-    batch_minmax[2 * h]     = lo;
-    batch_minmax[2 * h + 1] = hi;
     Ranges r;
+    r.batch_min = lo;
+    r.batch_max = hi;
     // _create_bin_edges: equal min and max are widened by 0.5 each way; edges = arange(0, bins + 1) * step + min
     float e_lo = lo, e_hi = hi;
     if (e_hi == e_lo)
@@ -153,8 +167,7 @@ __global__ __launch_bounds__(64) void ranges_kernel(const float* __restrict__ pa
             r.m_hi += 1.0f;
         }
     }
-    r.pad     = 0;
-    ranges[h] = r;
+    return r;
 }
 
 // torch.histc's bin of x in [lo, hi] (float32: (x - lo) * bins / (hi - lo), truncated; x == hi falls in the last
@@ -191,65 +204,153 @@ struct Binner
     }
 };
 
-// grid (blocks, H).  Each workgroup bins its share of row h into LDS (batch range and merged range in one pass) and
-// stores its counts to its own slice of `partial` (plain stores: no atomics on global memory).
-// partial layout: [h][block][2][num_bins] uint32
-__global__ __launch_bounds__(kHistBlock) void hist2_kernel(const float* __restrict__ x, int64_t n_per_hist,
-                                                           int num_bins, int has_stats,
-                                                           const Ranges* __restrict__ ranges,
-                                                           uint32_t* __restrict__ partial)
+// grid (blocks, H).  Each workgroup first derives the binning ranges of histogram h from the (min, max) partials of the
+// previous launch (every workgroup repeats this small reduction: cheaper than a launch of its own), then bins its
+// share of row h into LDS -- the batch's own range and / or the merged range, in one pass over the data -- and stores
+// its counts to its own slice of `partial` (plain stores: no atomics on global memory).
+// LDS: [kinds][num_bins][copies] uint32, copy = lane % copies (lanes of a wavefront that hit the same bin spread out).
+// partial layout: [h][block][kinds][num_bins] uint32
+__global__ __launch_bounds__(kHistBlock) void hist_kernel(const float* __restrict__ x, int64_t n_per_hist, int num_bins,
+                                                          int has_stats, int count_batch, int count_merged,
+                                                          int copies, const float* __restrict__ mm_partial,
+                                                          const float* __restrict__ state_minmax,
+                                                          Ranges* __restrict__ ranges, float* __restrict__ batch_minmax,
+                                                          int* __restrict__ bad_flag, uint32_t* __restrict__ partial,
+                                                          int vec)
 {
-    extern __shared__ uint32_t lds[];   // [2][num_bins]
+    extern __shared__ uint32_t lds[];
+    __shared__ float s_mm[2][kHistBlock / 64];
     const int h = blockIdx.y;
-    for (int i = threadIdx.x; i < 2 * num_bins; i += kHistBlock)
+    const int kinds = count_batch + count_merged;
+    for (int i = threadIdx.x; i < kinds * num_bins * copies; i += kHistBlock)
         lds[i] = 0;
-    const Ranges r = ranges[h];
+    float lo = INFINITY, hi = -INFINITY;
+    for (int b = threadIdx.x; b < (int) gridDim.x; b += kHistBlock)
+    {
+        lo = fminf(lo, mm_partial[((int64_t) h * gridDim.x + b) * 2]);
+        hi = fmaxf(hi, mm_partial[((int64_t) h * gridDim.x + b) * 2 + 1]);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        lo = fminf(lo, __shfl_xor(lo, o));
+        hi = fmaxf(hi, __shfl_xor(hi, o));
+    }
+    if ((threadIdx.x & 63) == 0)
+    {
+        s_mm[0][threadIdx.x >> 6] = lo;
+        s_mm[1][threadIdx.x >> 6] = hi;
+    }
+    __syncthreads();
+    for (int k = 0; k < kHistBlock / 64; ++k)
+    {
+        lo = fminf(lo, s_mm[0][k]);
+        hi = fmaxf(hi, s_mm[1][k]);
+    }
+    bool ok;
+    const Ranges r = compute_ranges(lo, hi, num_bins, has_stats, state_minmax, h, ok);
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+    {
+        ranges[h] = r;
+        if (batch_minmax)
+        {
+            batch_minmax[2 * h]     = r.batch_min;
+            batch_minmax[2 * h + 1] = r.batch_max;
+        }
+        if (!ok)
+            atomicOr(bad_flag, 1);
+    }
     Binner bb, mb;
     bb.init(r.b_lo, r.b_hi, num_bins);
     mb.init(r.m_lo, r.m_hi, num_bins);
-    __syncthreads();
+    const int copy = threadIdx.x & (copies - 1);
+    uint32_t* lb   = lds + copy;                                        // batch-range counts
+    uint32_t* lm   = lds + (count_batch ? num_bins * copies : 0) + copy;   // merged-range counts
     const float* row = x + (int64_t) h * n_per_hist;
-    for (int64_t i = (int64_t) blockIdx.x * kHistBlock + threadIdx.x; i < n_per_hist;
-         i += (int64_t) gridDim.x * kHistBlock)
+    auto count = [&](float v) {
+        if (v != v)
+            return;
+        if (count_batch)
+            atomicAdd(&lb[bb.bin(v) * copies], 1u);
+        if (count_merged)
+            atomicAdd(&lm[mb.bin(v) * copies], 1u);
+    };
+    if (vec)
     {
-        const float v = row[i];
-        const int pb  = bb.bin(v);
-        if (pb >= 0)
+        const v4f* rv        = reinterpret_cast<const v4f*>(row);
+        const int64_t nvec   = n_per_hist / 4;
+        const int64_t stride = (int64_t) gridDim.x * kHistBlock * 2;
+        for (int64_t base = (int64_t) blockIdx.x * kHistBlock * 2; base < nvec; base += stride)
         {
-            atomicAdd(&lds[pb], 1u);
-            if (has_stats)
-                atomicAdd(&lds[num_bins + mb.bin(v)], 1u);
+            v4f a[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+            {
+                const int64_t i = base + u * kHistBlock + threadIdx.x;
+                a[u]            = i < nvec ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+            {
+                count(a[u][0]);
+                count(a[u][1]);
+                count(a[u][2]);
+                count(a[u][3]);
+            }
         }
     }
+    else
+    {
+        for (int64_t i = (int64_t) blockIdx.x * kHistBlock + threadIdx.x; i < n_per_hist;
+             i += (int64_t) gridDim.x * kHistBlock)
+            count(row[i]);
+    }
     __syncthreads();
-    uint32_t* dst = partial + ((int64_t) h * gridDim.x + blockIdx.x) * 2 * num_bins;
-    for (int i = threadIdx.x; i < 2 * num_bins; i += kHistBlock)
-        dst[i] = lds[i];
+    uint32_t* dst = partial + ((int64_t) h * gridDim.x + blockIdx.x) * kinds * num_bins;
+    for (int i = threadIdx.x; i < kinds * num_bins; i += kHistBlock)
+    {
+        uint32_t sum = 0;
+        for (int c = 0; c < copies; ++c)
+            sum += lds[i * copies + c];
+        dst[i] = sum;
+    }
 }
 
-// grid (ceil(2 bins / 256), slices, H): adds a slice of the workgroups' counts into sums[h][2][bins]
+// grid (ceil(width / 256), slices, H), width = kinds * bins: adds a slice of the workgroups' counts into sums[h][width]
 __global__ __launch_bounds__(kHistBlock) void reduce_counts_kernel(const uint32_t* __restrict__ partial, int blocks,
-                                                                   int num_bins, uint32_t* __restrict__ sums)
+                                                                   int width, uint32_t* __restrict__ sums)
 {
     const int i = blockIdx.x * kHistBlock + threadIdx.x;
     const int h = blockIdx.z;
-    if (i >= 2 * num_bins)
+    if (i >= width)
         return;
     const int per   = (blocks + gridDim.y - 1) / gridDim.y;
     const int b0    = blockIdx.y * per;
     const int b1    = min(blocks, b0 + per);
-    const uint32_t* p = partial + (int64_t) h * blocks * 2 * num_bins + i;
-    uint32_t acc    = 0;
-    for (int b = b0; b < b1; ++b)
-        acc += p[(int64_t) b * 2 * num_bins];
+    const uint32_t* p = partial + (int64_t) h * blocks * width + i;
+    // independent loads, eight in flight per lane
+    uint32_t acc = 0;
+    int b        = b0;
+    for (; b + 8 <= b1; b += 8)
+    {
+        uint32_t t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            t[u] = p[(int64_t) (b + u) * width];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            acc += t[u];
+    }
+    for (; b < b1; ++b)
+        acc += p[(int64_t) b * width];
     if (acc)
-        atomicAdd(&sums[(int64_t) h * 2 * num_bins + i], acc);
+        atomicAdd(&sums[(int64_t) h * width + i], acc);
 }
 
 // grid H, 256 threads: writes the batch histogram, re-bins the running histogram when the
 // range grew (merge_stats, EA:222-251) and adds the batch's counts over the merged range.
 __global__ __launch_bounds__(kHistBlock) void merge_kernel(const uint32_t* __restrict__ sums, int num_bins,
-                                                           int has_stats,
+                                                           int has_stats, int count_batch, int count_merged,
                                                            const Ranges* __restrict__ ranges,
                                                            float* __restrict__ state_hist,
                                                            float* __restrict__ state_minmax,
@@ -259,8 +360,9 @@ __global__ __launch_bounds__(kHistBlock) void merge_kernel(const uint32_t* __res
     const int h    = blockIdx.x;
     const Ranges r = ranges[h];
     float* sh      = state_hist + (int64_t) h * num_bins;
-    float* bh      = batch_hist + (int64_t) h * num_bins;
-    const uint32_t* p = sums + (int64_t) h * 2 * num_bins;
+    float* bh      = batch_hist ? batch_hist + (int64_t) h * num_bins : nullptr;
+    const uint32_t* p  = sums + (int64_t) h * (count_batch + count_merged) * num_bins;
+    const uint32_t* pm = p + (count_batch ? num_bins : 0);
     for (int i = threadIdx.x; i < num_bins; i += kHistBlock)
         upd[i] = 0.f;
     __syncthreads();
@@ -291,12 +393,12 @@ __global__ __launch_bounds__(kHistBlock) void merge_kernel(const uint32_t* __res
     }
     for (int i = threadIdx.x; i < num_bins; i += kHistBlock)
     {
-        const uint32_t cb = p[i], cm = p[num_bins + i];
-        bh[i]             = (float) cb;
+        if (count_batch && batch_hist)
+            bh[i] = (float) p[i];
         if (!has_stats)
-            sh[i] = (float) cb;
-        else
-            sh[i] = (float) cm + (r.rebin ? upd[i] : sh[i]);
+            sh[i] = (float) p[i];
+        else if (count_merged)
+            sh[i] = (float) pm[i] + (r.rebin ? upd[i] : sh[i]);
     }
     if (threadIdx.x == 0)
     {
@@ -459,9 +561,9 @@ __global__ __launch_bounds__(64) void sqnr_pick_kernel(const double* __restrict_
 
 int hist_blocks(int64_t num_hist, int64_t n_per_hist)
 {
-    // enough workgroups to fill 256 CUs a few times over, at least ~4K elements each
-    int64_t per_row = (n_per_hist + 4095) / 4096;
-    int64_t want    = (1024 + num_hist - 1) / num_hist;
+    // enough workgroups to fill 256 CUs three times over, at least ~8K elements each
+    int64_t per_row = (n_per_hist + 8191) / 8192;
+    int64_t want    = (768 + num_hist - 1) / num_hist;
     int64_t b       = per_row < want ? per_row : want;
     return (int) (b < 1 ? 1 : b);
 }
@@ -517,14 +619,19 @@ int64_t miq_v2_hist_workspace_bytes(int64_t num_hist, int64_t n_per_hist, int nu
 }
 
 int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hist, int num_bins, int has_stats,
-                           float* state_hist, float* state_minmax, float* batch_hist, float* batch_minmax,
-                           int32_t* bad_flag, void* workspace, void* stream)
+                           int want_batch_hist, float* state_hist, float* state_minmax, float* batch_hist,
+                           float* batch_minmax, int32_t* bad_flag, void* workspace, void* stream)
 {
     MIQ_CHECK_ARG(num_hist > 0 && n_per_hist > 0, "empty input");
     MIQ_CHECK_ARG(num_bins > 0 && num_bins <= kMaxBins, "num_bins must lie in 1..%d", kMaxBins);
     MIQ_CHECK_ARG(num_hist <= 65535, "at most 65535 histograms per call");
-    MIQ_CHECK_ARG(data && state_hist && state_minmax && batch_hist && batch_minmax && bad_flag && workspace,
-                  "null pointer");
+    MIQ_CHECK_ARG(data && state_hist && state_minmax && bad_flag && workspace, "null pointer");
+    MIQ_CHECK_ARG(!want_batch_hist || batch_hist, "batch_hist is needed when want_batch_hist is set");
+    // which histograms this pass fills: the batch's own range and / or the merged range
+    const int count_batch  = !has_stats || want_batch_hist;
+    const int count_merged = has_stats != 0;
+    const int kinds        = count_batch + count_merged;
+    const int copies       = kinds == 1 ? 4 : 2;   // LDS: kinds * bins * copies * 4 B <= 64 KiB at 4096 bins
     const int blocks = hist_blocks(num_hist, n_per_hist);
     char* ws         = (char*) workspace;
     uint32_t* counts = (uint32_t*) ws;
@@ -536,21 +643,21 @@ int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hi
     ws             = (char*) (((uintptr_t) ws + 15) & ~(uintptr_t) 15);
     Ranges* ranges = (Ranges*) ws;
     hipStream_t s  = (hipStream_t) stream;
+    const int vec  = (n_per_hist % 4 == 0) && aligned16(data);
+    const int width = kinds * num_bins;
     hipLaunchKernelGGL(finite_minmax_kernel, dim3(blocks, (unsigned) num_hist), dim3(kHistBlock), 0, s, data, n_per_hist,
-                       mm_part, sums, 2 * num_bins);
+                       mm_part, sums, width, vec);
     MIQ_CHECK_LAUNCH();
-    hipLaunchKernelGGL(ranges_kernel, dim3((unsigned) num_hist), dim3(64), 0, s, mm_part, blocks, num_bins,
-                       has_stats, state_minmax, batch_minmax, ranges, bad_flag, (int) num_hist);
-    MIQ_CHECK_LAUNCH();
-    hipLaunchKernelGGL(hist2_kernel, dim3(blocks, (unsigned) num_hist), dim3(kHistBlock),
-                       2 * num_bins * sizeof(uint32_t), s, data, n_per_hist, num_bins, has_stats, ranges, counts);
+    hipLaunchKernelGGL(hist_kernel, dim3(blocks, (unsigned) num_hist), dim3(kHistBlock),
+                       (size_t) width * copies * sizeof(uint32_t), s, data, n_per_hist, num_bins, has_stats, count_batch,
+                       count_merged, copies, mm_part, state_minmax, ranges, batch_minmax, bad_flag, counts, vec);
     MIQ_CHECK_LAUNCH();
     const int slices = blocks < 32 ? blocks : 32;
-    hipLaunchKernelGGL(reduce_counts_kernel, dim3((2 * num_bins + kHistBlock - 1) / kHistBlock, slices, (unsigned) num_hist),
-                       dim3(kHistBlock), 0, s, counts, blocks, num_bins, sums);
+    hipLaunchKernelGGL(reduce_counts_kernel, dim3((width + kHistBlock - 1) / kHistBlock, slices, (unsigned) num_hist),
+                       dim3(kHistBlock), 0, s, counts, blocks, width, sums);
     MIQ_CHECK_LAUNCH();
-    hipLaunchKernelGGL(merge_kernel, dim3((unsigned) num_hist), dim3(kHistBlock), 0, s, sums, num_bins, has_stats, ranges,
-                       state_hist, state_minmax, batch_hist);
+    hipLaunchKernelGGL(merge_kernel, dim3((unsigned) num_hist), dim3(kHistBlock), 0, s, sums, num_bins, has_stats,
+                       count_batch, count_merged, ranges, state_hist, state_minmax, want_batch_hist ? batch_hist : nullptr);
     MIQ_CHECK_LAUNCH();
     return MIQ_OK;
 }

@@ -228,18 +228,21 @@ def v2_hist_workspace(num_hist, n_per_hist, num_bins, device):
     return torch.empty((nbytes + 3) // 4, dtype=torch.int32, device=device)
 
 
-def v2_hist_update(data, num_hist, num_bins, has_stats, state_hist, state_minmax, bad_flag, workspace):
-    """collect_stats + merge_stats of the v2 histogram observer for one batch; returns (batch_hist, batch_minmax)."""
+def v2_hist_update(data, num_hist, num_bins, has_stats, state_hist, state_minmax, bad_flag, workspace,
+                   want_batch_hist=True):
+    """collect_stats + merge_stats of the v2 histogram observer for one batch; returns (batch_hist, batch_minmax)
+    (batch_hist is None when want_batch_hist is False)."""
     _require_gpu(data, state_hist, state_minmax, bad_flag, workspace)
     if data.dtype != _F32 or not data.is_contiguous():
         raise RuntimeError("the histogram observer takes contiguous float32 data")
     n_per_hist = data.numel() // num_hist
-    batch_hist = torch.empty(num_hist, num_bins, dtype=_F32, device=data.device)
+    batch_hist = torch.empty(num_hist, num_bins, dtype=_F32, device=data.device) if want_batch_hist else None
     batch_minmax = torch.empty(num_hist, 2, dtype=_F32, device=data.device)
     with torch.cuda.device(data.device):
         check(lib.miq_v2_hist_update_f32(_ptr(data), int(num_hist), int(n_per_hist), int(num_bins), int(has_stats),
-                                         _ptr(state_hist), _ptr(state_minmax), _ptr(batch_hist), _ptr(batch_minmax),
-                                         _ptr(bad_flag), _ptr(workspace), _stream(data)))
+                                         int(bool(want_batch_hist)), _ptr(state_hist), _ptr(state_minmax),
+                                         _ptr(batch_hist), _ptr(batch_minmax), _ptr(bad_flag), _ptr(workspace),
+                                         _stream(data)))
     return batch_hist, batch_minmax
 
 

@@ -177,6 +177,34 @@ class _DeviceHistograms:
         return (self[i] for i in range(len(self)))
 
 
+class _LazyBatchHistograms:
+    """Stands for the statistics of one batch; computes them (collect_stats) when first read."""
+
+    def __init__(self, observer, input_tensor: torch.Tensor):
+        self._observer, self._input, self._stats = observer, input_tensor, None
+
+    def _get(self) -> _DeviceHistograms:
+        if self._stats is None:
+            self._stats = self._observer.collect_stats(self._input)
+            self._input = None
+        return self._stats
+
+    hist = property(lambda self: self._get().hist)
+    minmax = property(lambda self: self._get().minmax)
+
+    def check(self):
+        self._get().check()
+
+    def __len__(self):
+        return self._observer.num_histograms
+
+    def __getitem__(self, index):
+        return self._get()[index]
+
+    def __iter__(self):
+        return iter(self._get())
+
+
 class _HistogramObserver:
     """Running histogram(s) of the observed tensors (percentile / SQNR calibration)."""
 
@@ -204,7 +232,7 @@ class _HistogramObserver:
         return input_tensor.detach().to(torch.float32).contiguous()
 
     @torch.no_grad()
-    def _update(self, input_tensor: torch.Tensor, merge: bool) -> _DeviceHistograms:
+    def _update(self, input_tensor: torch.Tensor, merge: bool, want_batch: bool = True):
         data = self._slabs(input_tensor)
         n_per_hist = data.numel() // self.num_histograms
         device = data.device
@@ -224,23 +252,29 @@ class _HistogramObserver:
             state_minmax = torch.empty(self.num_histograms, 2, dtype=torch.float32, device=device)
             has_stats = False
         batch_hist, batch_minmax = ops.v2_hist_update(data, self.num_histograms, self.num_bins, has_stats, state_hist,
-                                                      state_minmax, bad, self._workspace)
+                                                      state_minmax, bad, self._workspace,
+                                                      want_batch_hist=want_batch or not has_stats)
         if merge:
             self._state = _DeviceHistograms(state_hist, state_minmax, bad)
+        if batch_hist is None:
+            return None
         return _DeviceHistograms(batch_hist, batch_minmax, bad)
 
     def collect_stats(self, input_tensor: torch.Tensor) -> _DeviceHistograms:
         """The batch's own histogram(s); the running statistics are not touched."""
         return self._update(input_tensor, merge=False)
 
-    def collect_and_merge_stats(self, input_tensor: torch.Tensor) -> _DeviceHistograms:
-        """collect_stats followed by merge_stats in one pass over the input."""
-        return self._update(input_tensor, merge=True)
+    def collect_and_merge_stats(self, input_tensor: torch.Tensor):
+        """collect_stats followed by merge_stats.  The batch's own histogram is what only dynamic quantization inside
+        compute_encodings() reads, so it is formed when first looked at, from the tensor handed in here (which the
+        caller therefore must not modify in place before looking)."""
+        self._update(input_tensor, merge=True, want_batch=False)
+        return _LazyBatchHistograms(self, input_tensor)
 
     def merge_stats(self, new_stats_list, input_tensor: torch.Tensor):
         """Merges a batch into the running statistics (the batch histogram passed in is not needed: the merged-range
         histogram is recomputed from the input, as in the reference)."""
-        self._update(input_tensor, merge=True)
+        self._update(input_tensor, merge=True, want_batch=False)
 
     def get_stats(self):
         if self._state is None:

@@ -385,6 +385,46 @@ def bench_quantsim(torch, steps=10, batch=64):
             "images_per_s": batch / (sim_ms / 1e3), "fp32_images_per_s": batch / (fp32_ms / 1e3)}
 
 
+def bench_sqnr(torch, ops, reps=5):
+    """v2 SQNR analyzer on the calibration workload: 16 batches of [32,256,28,28] through the 2048-bin histogram
+    observer (finite min/max + one dual-range binning pass per batch), then the 8-bit asymmetric search."""
+    from aimet_amd.v2.quantization.encoding_analyzer import SqnrEncodingAnalyzer
+    dev = torch.device("cuda", 0)
+    n = 32 * 256 * 28 * 28
+    batches = []
+    for b in range(16):
+        g = torch.Generator(device=dev).manual_seed(1003 + b)
+        x = torch.randn(n, device=dev, generator=g).abs_()
+        u = torch.rand(n, device=dev, generator=g)
+        t = torch.rand(n, device=dev, generator=g)
+        batches.append(torch.where(u < 0.005, (1 - t).rsqrt(), x).contiguous())
+    an = SqnrEncodingAnalyzer((1,))
+    acc_ms, search_ms = [], []
+    for r in range(reps + 1):
+        an.reset_stats()
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        torch.cuda.synchronize()
+        e[0].record()
+        for x in batches:
+            an.update_stats(x)
+        e[1].record()
+        e[2].record()
+        mn, mx = an.compute_encodings(255.0, False)
+        e[3].record()
+        torch.cuda.synchronize()
+        if r:
+            acc_ms.append(e[0].elapsed_time(e[1]))
+            search_ms.append(e[2].elapsed_time(e[3]))
+    acc = sum(acc_ms) / len(acc_ms)
+    srch = sum(search_ms) / len(search_ms)
+    elems = 16 * n
+    # two passes over each batch: 8 B/element
+    return {"elements": elems, "num_bins": 2048, "accumulate_ms": acc, "search_ms": srch,
+            "elements_per_s": elems / ((acc + srch) / 1e3), "accumulate_GBps": 8.0 * elems / acc / 1e6,
+            "accumulate_frac_hbm": 8.0 * elems / acc / 1e6 / HBM_PEAK_GBPS,
+            "encoding": [float(mn), float(mx)]}
+
+
 def cpu_baseline_qdq(seconds=10.0):
     """Single-threaded oracle (C restatement of the reference CPU loops) on a [1024, 4096] slice of the workload."""
     import numpy as np
@@ -436,7 +476,7 @@ def main():
     ap.add_argument("--full", action="store_true", help="also measure every shape x dtype x bit-width cell")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run a subset of the legs, comma separated (main|pt|calib|quantsim|adaround|copyref), for profiling")
+                    help="run a subset of the legs, comma separated (main|pt|calib|sqnr|quantsim|adaround|copyref), for profiling")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
@@ -473,6 +513,8 @@ def main():
         extra["per_tensor_act_int8"] = bench_per_tensor(torch, ops, max(20, args.steps), args.warmup)
     if want("calib"):
         extra["tf_enhanced_calibration"] = bench_calibration(torch, ops, 5)
+    if want("sqnr"):
+        extra["v2_sqnr_calibration"] = bench_sqnr(torch, ops)
     if want("quantsim"):
         extra["quantsim_resnet50_shaped"] = bench_quantsim(torch)
     if want("adaround"):

@@ -297,10 +297,12 @@ int64_t miq_v2_hist_workspace_bytes(int64_t num_hist, int64_t n_per_hist, int nu
  * (what collect_stats returns) to batch_hist / batch_minmax and merges them into state_* (has_stats = 0: the state is
  * empty and becomes the batch's statistics).  bad_flag: device int32, set to 1 when a slab holds no finite value (the
  * reference raises ValueError there; the caller checks the flag when it next reads results).  workspace: device
- * buffer of miq_v2_hist_workspace_bytes.  Enqueues five kernels; never synchronises. */
+ * buffer of miq_v2_hist_workspace_bytes.  want_batch_hist = 0 skips the batch's own histogram (batch_hist may then be
+ * NULL; batch_minmax, optional, is still written): only callers that quantize dynamically with the batch's statistics
+ * read it.  Enqueues four kernels; never synchronises. */
 int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hist, int num_bins, int has_stats,
-                           float* state_hist, float* state_minmax, float* batch_hist, float* batch_minmax,
-                           int32_t* bad_flag, void* workspace, void* stream);
+                           int want_batch_hist, float* state_hist, float* state_minmax, float* batch_hist,
+                           float* batch_minmax, int32_t* bad_flag, void* workspace, void* stream);
 /* Number of (delta, offset) candidates SqnrEncodingAnalyzer searches (EA:594-646); -1 on invalid arguments. */
 int miq_v2_sqnr_num_candidates(double num_steps, int symmetric, int asym_deltas, int sym_deltas,
                                int offset_candidates);
