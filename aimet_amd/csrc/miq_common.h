@@ -93,5 +93,20 @@ __device__ __forceinline__ uint32_t f32_to_bf16(float f)
     return ((u & 0x7fffffffu) > 0x7f800000u) ? 0x7fc0u : r;
 }
 
+// two floats -> packed bf16 pair with the hardware's round-to-nearest-even conversion (v_cvt_pk_bf16_f32); NaN is
+// canonicalised to 0x7FC0 as above
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi)
+{
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const f2 v = {lo, hi};
+    uint32_t w = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2));
+    if (lo != lo)
+        w = (w & 0xffff0000u) | 0x7fc0u;
+    if (hi != hi)
+        w = (w & 0x0000ffffu) | 0x7fc00000u;
+    return w;
+}
+
 }   // namespace miq
 #endif

@@ -97,7 +97,7 @@ struct IOTraits<uint16_t>
         uint32_t w[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            w[i] = f32_to_bf16(f[2 * i]) | (f32_to_bf16(f[2 * i + 1]) << 16);
+            w[i] = f32x2_to_bf16x2(f[2 * i], f[2 * i + 1]);
         return make_uint4(w[0], w[1], w[2], w[3]);
     }
     __device__ static float load1(const uint16_t* p)
