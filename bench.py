@@ -214,6 +214,7 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
     from aimet_amd.v1.adaround.adaround_loss import AdaroundHyperParameters
     from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
     wrapper, x, y = _adaround_layer(torch)
+    timed_kernel_iters = min(timed_kernel_iters, iterations)
     n = wrapper.weight.numel()
     o, k = wrapper.weight.shape
     params = AdaroundHyperParameters(iterations, 0.01, (20, 2), 0.2)
