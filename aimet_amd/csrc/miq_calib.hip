@@ -353,11 +353,16 @@ __device__ void fold_batch(DevState* st, int buf)
     const double cnt = (double) (int) st->batch_n[buf];
     for (int b = threadIdx.x; b < kPdf; b += blockDim.x)
     {
+        // all replica loads in flight together, then the clears
+        uint32_t t[kReplicas];
+#pragma unroll
+        for (int r = 0; r < kReplicas; ++r)
+            t[r] = st->counts[buf][r][b];
         uint32_t c = 0;
-#pragma unroll 8
+#pragma unroll
         for (int r = 0; r < kReplicas; ++r)
         {
-            c += st->counts[buf][r][b];
+            c += t[r];
             st->counts[buf][r][b] = 0;
         }
         st->last_counts[b] = c;
@@ -382,8 +387,11 @@ template <bool VEC>
 __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ in, int64_t n, DevState* st, int buf,
                                                       uint32_t seq, int from_args, float bucket_arg, float off_arg)
 {
-    const bool fold_group = (blockIdx.x == gridDim.x - 1);
+    // workgroup 0 folds: it is dispatched first and runs beside the data workgroups (as the last one it would start only
+    // after a data workgroup had retired and would lengthen the launch by its own duration)
+    const bool fold_group = (blockIdx.x == 0);
     const int data_groups = gridDim.x - 1;
+    const int group       = (int) blockIdx.x - 1;
     if (fold_group)
     {
         if (st->batch_seq[1 - buf] != 0 && st->batch_seq[1 - buf] == seq - 1)
@@ -399,7 +407,7 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
     const int64_t nvec   = n / 4;
     const float4* v      = reinterpret_cast<const float4*>(in);
     const int64_t stride = (int64_t) data_groups * kBlock * kUnroll;
-    int64_t base         = (int64_t) blockIdx.x * kBlock * kUnroll;
+    int64_t base         = (int64_t) group * kBlock * kUnroll;
     float4 a[kUnroll];
     // first tile's loads go out before anything else: they overlap the state read and the LDS clear
     if (VEC)
@@ -445,16 +453,16 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
                 a[u] = (i < nvec) ? v[i] : make_float4(NAN, NAN, NAN, NAN);
             }
         }
-        if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * 4))
+        if (group == 0 && threadIdx.x < (uint32_t) (n - nvec * 4))
             hist_add(lds, in[nvec * 4 + threadIdx.x], bucket, off, copy);
     }
     else
     {
-        for (int64_t i = (int64_t) blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t) data_groups * kBlock)
+        for (int64_t i = (int64_t) group * kBlock + threadIdx.x; i < n; i += (int64_t) data_groups * kBlock)
             hist_add(lds, in[i], bucket, off, copy);
     }
     __syncthreads();
-    uint32_t* dst = st->counts[buf][blockIdx.x % kReplicas];
+    uint32_t* dst = st->counts[buf][group % kReplicas];
     for (int b = threadIdx.x; b < kPdf; b += kBlock)
     {
         uint32_t s = 0;
