@@ -453,6 +453,32 @@ def cpu_baseline_qdq(seconds=10.0):
                       "single-threaded C restatement of the reference CPU loops (oracle/miq_oracle.c)"}
 
 
+def cpu_reference_qdq_forward(seconds=5.0):
+    """The reference's own compiled C++ per-channel quantize-dequantize (oracle/_ref, built from the reference tree where
+    that tree exists) on the same [1024, 4096] slice: forward only (its backward is Python)."""
+    import numpy as np
+    import oracle
+    if oracle.ref is None:
+        return None
+    o, r = oracle.lib, oracle.ref
+    rng = np.random.default_rng(1004)
+    c, npc = 1024, 4096
+    u = rng.random((c, npc)) - 0.5
+    w = (-0.02 * np.sign(u) * np.log1p(-2 * np.abs(u))).astype(np.float32)
+    amax = np.abs(w).max(axis=1).astype(np.float64)
+    encs = [o.tf_compute_encoding(-a, a, 8, sym=True) for a in amax]
+    params = o.per_channel_params(np.array([e.min for e in encs]), np.array([e.max for e in encs]), 8)
+    n, reps = c * npc, 0
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        r.qdq_per_channel(w, c, npc, params)
+        reps += 1
+    dt = time.perf_counter() - t0
+    return {"value": 8.0 * n * reps / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "reference",
+            "sample": f"{reps} forward passes over a [1024,4096] fp32 slice, {dt:.1f} s, the reference's "
+                      "quantizeDequantizeTensorPerChannel compiled from its own sources"}
+
+
 def cpu_baseline_calibration(seconds=5.0):
     import numpy as np
     import oracle
@@ -557,6 +583,9 @@ def main():
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline_qdq()
         extra["cpu_baseline_calibration"] = cpu_baseline_calibration()
+        ref_fwd = cpu_reference_qdq_forward()
+        if ref_fwd is not None:
+            extra["cpu_reference_qdq_forward"] = ref_fwd
     line["extra"] = extra
     print(json.dumps(line))
 
