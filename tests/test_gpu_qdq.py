@@ -284,3 +284,40 @@ def test_idempotence_and_grid_membership_full_size(ops):
     assert torch.all((k - k.round()).abs() < 1e-3)
     assert k.round().min() >= -128 and k.round().max() <= 127
     assert torch.equal(mm[0], w.min(dim=1).values) and torch.equal(mm[1], w.max(dim=1).values)
+
+
+def test_more_than_2_31_elements(ops, oracle):
+    """Maximum sizes: 2^31 + 4099 elements (64-bit indexing in the kernels and in the channel arithmetic); slices at
+    the start, across the 2^31 boundary and at the end are compared with the oracle."""
+    n = (1 << 31) + 4099
+    free, _ = torch.cuda.mem_get_info()
+    if free < 3 * 4 * n:
+        pytest.skip("not enough device memory for a 2^31-element round trip")
+    g = torch.Generator(device="cuda").manual_seed(9)
+    x = torch.empty(n, device="cuda")
+    chunk = 1 << 28
+    for s in range(0, n, chunk):
+        x[s:s + chunk].normal_(generator=g)
+    spans = [(0, 100000), ((1 << 31) - 50000, (1 << 31) + 4099), (n - 70001, n)]
+    y = ops.qdq_per_tensor(x, -2.5, 3.0, 8)
+    for a, b in spans:
+        xs = x[a:b].cpu().numpy()
+        assert np.array_equal(y[a:b].cpu().numpy().view(np.uint32), oracle.qdq_per_tensor(xs, -2.5, 3.0, 8).view(np.uint32))
+    gx = ops.ste_bwd_per_tensor(x, y, -2.5, 3.0)
+    for a, b in spans:
+        assert np.array_equal(gx[a:b].cpu().numpy(),
+                              oracle.ste_bwd_per_tensor(x[a:b].cpu().numpy(), y[a:b].cpu().numpy(),
+                                                        np.float32(-2.5), np.float32(3.0)))
+    del y, gx
+    # per-channel: 7 channels of 613 consecutive elements, repeating (channel = (i / 613) % 7)
+    C, npc = 7, 613
+    emin = np.linspace(-3, -1, C).astype(np.float32)
+    emax = np.linspace(1, 3.5, C).astype(np.float32)
+    params = oracle.per_channel_params(emin, emax, 8)
+    gp = ops.per_channel_params(torch.from_numpy(emin).cuda(), torch.from_numpy(emax).cuda(), 255)
+    yc = ops.qdq_per_channel(x, C, npc, *gp)
+    for a, b in spans:
+        a0 = a - a % (C * npc)                      # start on a channel-0 boundary so the oracle sees the same phase
+        xs = x[a0:b].cpu().numpy()
+        want = oracle.qdq_per_channel(xs, C, npc, params)
+        assert np.array_equal(yc[a0:b].cpu().numpy().view(np.uint32), want.view(np.uint32))
