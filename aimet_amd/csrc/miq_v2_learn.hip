@@ -1,0 +1,316 @@
+// Backward of the v2 quantize-dequantize with learnable scale and offset, in one pass over x and grad.
+//
+// The reference forms three full-size intermediates and lets autograd reduce two of them to the parameter shape
+// (TrainingExtensions/torch/src/python/aimet_torch/v2/quantization/affine/backends/torch_builtins.py:329-344):
+//     q = x / scale;  r = round(q);  mask = qmin <= r - offset <= qmax
+//     tensor_grad = grad * mask
+//     scale_grad  = sum( grad * (clamp(r, offset + qmin, offset + qmax) - q * mask) )
+//     offset_grad = sum( grad * (~mask * scale) )
+// Here every element is read once: the workgroup streams a span of one channel row, writes tensor_grad, keeps the
+// two sums in registers, and stores one (scale, offset) partial per workgroup.  A second small kernel adds the
+// partials of each channel in double precision in a fixed order, so results do not depend on scheduling.
+//
+// Layout: the tensor is [outer][channel][elements-per-channel] in memory (outer = 1 for weights quantized along
+// axis 0, channel = 1 for per-tensor), so a "row" is one contiguous run that shares its parameters.
+#include "miq_common.h"
+#include "miq_fastmath.h"
+#include "miq_io.h"
+
+#include <cmath>
+
+namespace miq
+{
+namespace
+{
+struct LearnGeom
+{
+    uint32_t num_channel;
+    uint32_t chunks;        // workgroups per row
+    FastDiv chunks_div;
+    int64_t npc;            // elements per row
+    int64_t span;           // elements per workgroup (multiple of the vector width)
+    int64_t rows;           // outer * num_channel
+};
+
+struct LearnParams
+{
+    float scale, offset, rcp, lo, hi, qmin, qmax;
+};
+
+__device__ __forceinline__ LearnParams load_params(const float* scale, const float* offset, uint32_t ch, int qmin,
+                                                   int qmax)
+{
+    LearnParams p;
+    p.scale  = scale[ch];
+    p.offset = offset[ch];
+    p.rcp    = fastdiv_divisor_ok(p.scale) ? 1.0f / p.scale : 0.0f;
+    p.qmin   = (float) qmin;
+    p.qmax   = (float) qmax;
+    p.lo     = p.offset + p.qmin;
+    p.hi     = p.offset + p.qmax;
+    return p;
+}
+
+// one element: returns tensor_grad, adds this element's terms to the two sums
+template <bool FAST>
+__device__ __forceinline__ float learn_elem(const LearnParams& p, float x, float g, float& sg, float& og)
+{
+    const float q   = FAST ? div_by_invariant(x, p.scale, p.rcp) : x / p.scale;
+    const float r   = rintf(q);
+    const float rm  = r - p.offset;
+    const bool in   = (p.qmin <= rm) && (rm <= p.qmax);
+    const float m   = in ? 1.0f : 0.0f;
+    float c         = r;   // torch.clamp: NaN stays NaN
+    c               = (c < p.lo) ? p.lo : c;
+    c               = (c > p.hi) ? p.hi : c;
+    sg += g * (c - q * m);
+    og += g * ((1.0f - m) * p.scale);
+    return g * m;
+}
+
+template <typename IO, bool WRITE_GX>
+__device__ __forceinline__ void learn_vec(const LearnParams& p, const IO* x, const IO* g, IO* gx, int64_t at,
+                                          float& sg, float& og)
+{
+    using T = IOTraits<IO>;
+    float xf[T::VEC], gf[T::VEC], of[T::VEC];
+    T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(x + at)), xf);
+    T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(g + at)), gf);
+    float m = 0.0f;
+#pragma unroll
+    for (int j = 0; j < T::VEC; ++j)
+        m = fmaxf(m, fabsf(xf[j]));
+    if (p.rcp != 0.0f && m <= kFastDivMaxDividend)
+    {
+#pragma unroll
+        for (int j = 0; j < T::VEC; ++j)
+            of[j] = learn_elem<true>(p, xf[j], gf[j], sg, og);
+    }
+    else
+    {
+#pragma unroll
+        for (int j = 0; j < T::VEC; ++j)
+            of[j] = learn_elem<false>(p, xf[j], gf[j], sg, og);
+    }
+    if (WRITE_GX)
+        stream_store(reinterpret_cast<typename T::Vec*>(gx + at), T::pack(of));
+}
+
+template <typename IO, bool VECTOR, bool WRITE_GX>
+__global__ __launch_bounds__(kBlock) void learn_bwd_kernel(const IO* __restrict__ x, const IO* __restrict__ g,
+                                                           IO* __restrict__ gx, const float* __restrict__ scale,
+                                                           const float* __restrict__ offset, int qmin, int qmax,
+                                                           LearnGeom geo, float2* __restrict__ partial)
+{
+    using T              = IOTraits<IO>;
+    const uint32_t row   = fastdiv(blockIdx.x, geo.chunks_div);
+    const uint32_t chunk = blockIdx.x - row * geo.chunks;
+    const LearnParams p  = load_params(scale, offset, row % geo.num_channel, qmin, qmax);
+    const int64_t first  = (int64_t) chunk * geo.span;
+    const int64_t len    = min(geo.span, geo.npc - first);
+    const int64_t base   = (int64_t) row * geo.npc + first;
+    float sg = 0.0f, og = 0.0f;
+    if (VECTOR)
+    {
+        // len and base are multiples of the vector width on this path (checked by the host)
+        constexpr int64_t kStep = (int64_t) kBlock * T::VEC;
+        int64_t i               = (int64_t) threadIdx.x * T::VEC;
+        for (; i + kStep < len; i += 2 * kStep)
+        {
+            // two vectors per array in flight before the arithmetic starts
+            float xa[T::VEC], ga[T::VEC], xb[T::VEC], gb[T::VEC], oa[T::VEC], ob[T::VEC];
+            T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(x + base + i)), xa);
+            T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(x + base + i + kStep)), xb);
+            T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(g + base + i)), ga);
+            T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(g + base + i + kStep)), gb);
+            float m = 0.0f;
+#pragma unroll
+            for (int j = 0; j < T::VEC; ++j)
+                m = fmaxf(m, fmaxf(fabsf(xa[j]), fabsf(xb[j])));
+            if (p.rcp != 0.0f && m <= kFastDivMaxDividend)
+            {
+#pragma unroll
+                for (int j = 0; j < T::VEC; ++j)
+                {
+                    oa[j] = learn_elem<true>(p, xa[j], ga[j], sg, og);
+                    ob[j] = learn_elem<true>(p, xb[j], gb[j], sg, og);
+                }
+            }
+            else
+            {
+#pragma unroll
+                for (int j = 0; j < T::VEC; ++j)
+                {
+                    oa[j] = learn_elem<false>(p, xa[j], ga[j], sg, og);
+                    ob[j] = learn_elem<false>(p, xb[j], gb[j], sg, og);
+                }
+            }
+            if (WRITE_GX)
+            {
+                stream_store(reinterpret_cast<typename T::Vec*>(gx + base + i), T::pack(oa));
+                stream_store(reinterpret_cast<typename T::Vec*>(gx + base + i + kStep), T::pack(ob));
+            }
+        }
+        if (i < len)
+            learn_vec<IO, WRITE_GX>(p, x, g, gx, base + i, sg, og);
+    }
+    else
+    {
+        for (int64_t i = threadIdx.x; i < len; i += kBlock)
+        {
+            const float o = learn_elem<false>(p, T::load1(x + base + i), T::load1(g + base + i), sg, og);
+            if (WRITE_GX)
+                T::store1(gx + base + i, o);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        sg += __shfl_xor(sg, o);
+        og += __shfl_xor(og, o);
+    }
+    __shared__ float2 wave_sum[kBlock / 64];
+    if ((threadIdx.x & 63) == 0)
+        wave_sum[threadIdx.x >> 6] = make_float2(sg, og);
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        float a = 0.0f, b = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kBlock / 64; ++w)
+        {
+            a += wave_sum[w].x;
+            b += wave_sum[w].y;
+        }
+        partial[blockIdx.x] = make_float2(a, b);
+    }
+}
+
+// One wavefront per channel: adds the channel's partials (outer x chunks of them) in double.
+__global__ __launch_bounds__(64) void learn_reduce_kernel(const float2* __restrict__ partial, LearnGeom geo,
+                                                          uint32_t outer, float* __restrict__ scale_grad,
+                                                          float* __restrict__ offset_grad)
+{
+    const uint32_t ch = blockIdx.x;
+    double a = 0.0, b = 0.0;
+    for (uint32_t o = 0; o < outer; ++o)
+    {
+        const float2* row = partial + ((int64_t) o * geo.num_channel + ch) * geo.chunks;
+        for (uint32_t k = threadIdx.x; k < geo.chunks; k += 64)
+        {
+            const float2 v = row[k];
+            a += (double) v.x;
+            b += (double) v.y;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        a += __shfl_xor(a, o);
+        b += __shfl_xor(b, o);
+    }
+    if (threadIdx.x == 0)
+    {
+        if (scale_grad)
+            scale_grad[ch] = (float) a;
+        if (offset_grad)
+            offset_grad[ch] = (float) b;
+    }
+}
+
+// rows, chunks and span for a tensor of num_channel x npc rows repeated `outer` times
+int make_learn_geom(int64_t num_channel, int64_t n, int64_t npc, LearnGeom& geo, int64_t& outer)
+{
+    MIQ_CHECK_ARG(num_channel >= 1 && npc >= 1 && n >= 0, "non-positive channel geometry");
+    MIQ_CHECK_ARG(num_channel <= 0x7fffffff, "too many channels");
+    MIQ_CHECK_ARG(n % (num_channel * npc) == 0, "num_element is not a multiple of num_channel * elements per channel");
+    outer    = n / (num_channel * npc);
+    geo.rows = outer * num_channel;
+    geo.npc  = npc;
+    geo.num_channel = (uint32_t) num_channel;
+    // Spans of 8192 elements keep partials few; shorter ones when that would leave compute units idle.
+    int64_t span = 8192;
+    while (span > 2048 && geo.rows * ((npc + span - 1) / span) < 2048)
+        span /= 2;
+    const int64_t chunks = (npc + span - 1) / span;
+    MIQ_CHECK_ARG(geo.rows * chunks < 0x7fffffff, "tensor too large for one launch");
+    geo.span       = span;
+    geo.chunks     = (uint32_t) chunks;
+    geo.chunks_div = make_fastdiv((uint32_t) chunks);
+    return MIQ_OK;
+}
+
+template <typename IO>
+int launch_learn(const IO* x, const IO* g, IO* gx, int64_t num_channel, int64_t n, int64_t npc, const float* scale,
+                 const float* offset, int qmin, int qmax, float* scale_grad, float* offset_grad, void* workspace,
+                 hipStream_t stream)
+{
+    MIQ_CHECK_ARG(scale && offset, "null parameter pointer");
+    MIQ_CHECK_ARG(qmin <= qmax, "qmin must not exceed qmax");
+    MIQ_CHECK_ARG(scale_grad || offset_grad, "neither scale_grad nor offset_grad requested");
+    LearnGeom geo{};
+    int64_t outer = 0;
+    if (int rc = make_learn_geom(num_channel, n, npc, geo, outer))
+        return rc;
+    MIQ_CHECK_ARG(n == 0 || (x && g && workspace), "null pointer");
+    const bool vector = npc % IOTraits<IO>::VEC == 0 && aligned16(x) && aligned16(g) && (!gx || aligned16(gx));
+    float2* partial   = static_cast<float2*>(workspace);
+    // an empty tensor launches only the reduction, which then writes the zero sums
+    if (n > 0)
+    {
+        const dim3 grid((uint32_t) (geo.rows * geo.chunks));
+#define MIQ_LEARN(V, W)                                                                                                \
+    learn_bwd_kernel<IO, V, W><<<grid, kBlock, 0, stream>>>(x, g, gx, scale, offset, qmin, qmax, geo, partial)
+        if (vector && gx)
+            MIQ_LEARN(true, true);
+        else if (vector)
+            MIQ_LEARN(true, false);
+        else if (gx)
+            MIQ_LEARN(false, true);
+        else
+            MIQ_LEARN(false, false);
+#undef MIQ_LEARN
+        MIQ_CHECK_LAUNCH();
+    }
+    learn_reduce_kernel<<<dim3(geo.num_channel), 64, 0, stream>>>(partial, geo, (uint32_t) outer, scale_grad,
+                                                                  offset_grad);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+}   // namespace
+}   // namespace miq
+
+using namespace miq;
+
+extern "C" {
+
+int64_t miq_v2_qdq_bwd_params_workspace_bytes(int64_t num_channel, int64_t num_element,
+                                              int64_t num_element_per_channel)
+{
+    LearnGeom geo{};
+    int64_t outer = 0;
+    if (make_learn_geom(num_channel, num_element, num_element_per_channel, geo, outer) != MIQ_OK)
+        return 0;
+    const int64_t blocks = geo.rows * geo.chunks;
+    return (int64_t) sizeof(float2) * (blocks > 0 ? blocks : 1);
+}
+
+int miq_v2_qdq_bwd_params_f32(const float* x, const float* grad_out, float* grad_in, int64_t num_channel,
+                              int64_t num_element, int64_t num_element_per_channel, const float* scale,
+                              const float* offset, int qmin, int qmax, float* scale_grad, float* offset_grad,
+                              void* workspace, void* stream)
+{
+    return launch_learn<float>(x, grad_out, grad_in, num_channel, num_element, num_element_per_channel, scale, offset,
+                               qmin, qmax, scale_grad, offset_grad, workspace, (hipStream_t) stream);
+}
+
+int miq_v2_qdq_bwd_params_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* grad_in, int64_t num_channel,
+                               int64_t num_element, int64_t num_element_per_channel, const float* scale,
+                               const float* offset, int qmin, int qmax, float* scale_grad, float* offset_grad,
+                               void* workspace, void* stream)
+{
+    return launch_learn<uint16_t>(x, grad_out, grad_in, num_channel, num_element, num_element_per_channel, scale,
+                                  offset, qmin, qmax, scale_grad, offset_grad, workspace, (hipStream_t) stream);
+}
+
+}   // extern "C"

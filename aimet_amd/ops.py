@@ -200,6 +200,23 @@ def v2_qdq_bwd(x, grad_out, num_channel, n_per_channel, scale, offset, qmin, qma
     return gin
 
 
+def v2_qdq_bwd_params(x, grad_out, num_channel, n_per_channel, scale, offset, qmin, qmax, want_grad_in=True):
+    """(grad_in or None, scale_grad[C], offset_grad[C]) of the v2 quantize-dequantize in one pass; float32 sums."""
+    _require_gpu(x, grad_out, scale, offset)
+    x, grad_out = x.contiguous(), grad_out.to(x.dtype).contiguous()
+    scale, offset = _params_f32(scale, x).reshape(-1), _params_f32(offset, x).reshape(-1)
+    c, npc = int(num_channel), int(n_per_channel)
+    gin = torch.empty_like(x) if want_grad_in else None
+    grads = torch.empty(2, c, dtype=_F32, device=x.device)
+    ws = torch.empty(int(lib.miq_v2_qdq_bwd_params_workspace_bytes(c, x.numel(), npc)), dtype=torch.uint8,
+                     device=x.device)
+    fn = getattr(lib, "miq_v2_qdq_bwd_params_" + _suffix(x))
+    with torch.cuda.device(x.device):
+        check(fn(_ptr(x), _ptr(grad_out), _ptr(gin) if want_grad_in else None, c, x.numel(), npc, _ptr(scale),
+                 _ptr(offset), int(qmin), int(qmax), _ptr(grads[0]), _ptr(grads[1]), _ptr(ws), _stream(x)))
+    return gin, grads[0], grads[1]
+
+
 # -------------------------------------------------------------------------------------------------------- statistics
 def minmax(x):
     """float32 device tensor [min, max] of x (NaN ignored); asynchronous."""

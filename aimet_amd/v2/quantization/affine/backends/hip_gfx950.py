@@ -65,6 +65,11 @@ def _channel_geometry(tensor_shape, scale_shape):
     return tensor_shape[axis], npc
 
 
+# The one-pass backward gives each contiguous channel row to its own workgroups; below this row length that is
+# slower than torch's elementwise ops plus a reduction.
+_MIN_ROW_FOR_FUSED_PARAM_GRADS = 256
+
+
 def _reduce_like(grad: torch.Tensor, shape) -> torch.Tensor:
     return grad.sum_to_size(shape) if tuple(grad.shape) != tuple(shape) else grad
 
@@ -83,9 +88,16 @@ class _QuantDequantFunc(torch.autograd.Function):
         tensor, scale, offset = ctx.saved_tensors
         c, npc, qmin, qmax = ctx.geom
         tensor_grad = scale_grad = offset_grad = None
-        if ctx.needs_input_grad[0]:
-            tensor_grad = ops.v2_qdq_bwd(tensor, grad, c, npc, scale, offset, qmin, qmax)
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+            if c == 1 or npc >= _MIN_ROW_FOR_FUSED_PARAM_GRADS:
+                # x and grad are read once: tensor_grad and both parameter sums come out of the same pass
+                tensor_grad, sg, og = ops.v2_qdq_bwd_params(tensor, grad, c, npc, scale, offset, qmin, qmax,
+                                                            want_grad_in=ctx.needs_input_grad[0])
+                scale_grad = sg.reshape(scale.shape).to(scale.dtype) if ctx.needs_input_grad[1] else None
+                offset_grad = og.reshape(offset.shape).to(offset.dtype) if ctx.needs_input_grad[2] else None
+                return tensor_grad, scale_grad, offset_grad, None, None
+            # short channel rows (a scale that varies along one of the innermost axes): elementwise terms from
+            # torch, reduced to the parameter shape as autograd would
             s, o = scale.to(torch.float32), offset.to(torch.float32)
             x = tensor.to(torch.float32) / s
             x_round = torch.round(x) - o
@@ -96,6 +108,8 @@ class _QuantDequantFunc(torch.autograd.Function):
                                           scale.shape).to(scale.dtype)
             if ctx.needs_input_grad[2]:
                 offset_grad = _reduce_like(g * (~mask * s), offset.shape).to(offset.dtype)
+        if ctx.needs_input_grad[0]:
+            tensor_grad = ops.v2_qdq_bwd(tensor, grad, c, npc, scale, offset, qmin, qmax)
         return tensor_grad, scale_grad, offset_grad, None, None
 
 

@@ -426,6 +426,55 @@ def bench_sqnr(torch, ops, reps=5):
             "encoding": [float(mn), float(mx)]}
 
 
+def bench_v2_range_learning(torch, ops, steps=50):
+    """v2 quantize-dequantize backward with learnable scale and offset: the one-pass kernel (tensor_grad + both
+    parameter sums; 12 B per element) against the torch elementwise ops + reductions of the same expressions, on the
+    main weight shape (per channel) and the activation shape (per tensor)."""
+    dev = torch.device("cuda", 0)
+    out = {}
+    for name, shape, c in (("per_channel_11008x4096", (11008, 4096), 11008), ("per_tensor_32x64x56x56", (32, 64, 56, 56), 1)):
+        g = torch.Generator(device=dev).manual_seed(1006)
+        n = 1
+        for d in shape:
+            n *= d
+        npc = n // c
+        sets = [(torch.randn(c, npc, device=dev, generator=g) * 0.05, torch.randn(c, npc, device=dev, generator=g))
+                for _ in range(3)]
+        scale = (sets[0][0].abs().amax(dim=1) / 127).clamp_min(1e-6).contiguous()
+        offset = torch.zeros(c, device=dev)
+
+        def fused(k):
+            x, gr = sets[k % 3]
+            return ops.v2_qdq_bwd_params(x, gr, c, npc, scale, offset, -128, 127)
+
+        def torch_ops(k):
+            x, gr = sets[k % 3]
+            s, o = scale.view(-1, 1), offset.view(-1, 1)
+            q = x / s
+            r = torch.round(q)
+            mask = (-128 <= r - o) & (r - o <= 127)
+            return (gr * mask, (gr * (r.clamp(o - 128, o + 127) - q * mask)).sum(dim=1),
+                    (gr * (~mask * s)).sum(dim=1))
+
+        def timed(fn):
+            for k in range(5):
+                fn(k)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for k in range(steps):
+                fn(k)
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / steps
+
+        t_fused, t_torch = timed(fused), timed(torch_ops)
+        out[name] = {"elements": n, "one_pass_ms": t_fused, "torch_ops_ms": t_torch,
+                     "one_pass_GBps": 12.0 * n / t_fused / 1e6, "frac_hbm": 12.0 * n / t_fused / 1e6 / HBM_PEAK_GBPS,
+                     "speedup_vs_torch_ops": t_torch / t_fused}
+    return out
+
+
 def cpu_baseline_qdq(seconds=10.0):
     """Single-threaded oracle (C restatement of the reference CPU loops) on a [1024, 4096] slice of the workload."""
     import numpy as np
@@ -503,7 +552,7 @@ def main():
     ap.add_argument("--full", action="store_true", help="also measure every shape x dtype x bit-width cell")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run a subset of the legs, comma separated (main|pt|calib|sqnr|quantsim|adaround|copyref), for profiling")
+                    help="run a subset of the legs, comma separated (main|pt|calib|sqnr|learn|quantsim|adaround|copyref), for profiling")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
@@ -542,6 +591,8 @@ def main():
         extra["tf_enhanced_calibration"] = bench_calibration(torch, ops, 5)
     if want("sqnr"):
         extra["v2_sqnr_calibration"] = bench_sqnr(torch, ops)
+    if want("learn"):
+        extra["v2_range_learning_backward"] = bench_v2_range_learning(torch, ops)
     if want("quantsim"):
         extra["quantsim_resnet50_shaped"] = bench_quantsim(torch)
     if want("adaround"):

@@ -151,6 +151,26 @@ int miq_v2_qdq_bwd_f32(const float* x, const float* grad_out, float* grad_in, in
 int miq_v2_qdq_bwd_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* grad_in, int64_t num_channel,
                         int64_t num_element, int64_t num_element_per_channel, const float* scale,
                         const float* offset, int qmin, int qmax, void* stream);
+/* Backward w.r.t. the input, scale and offset in one pass (torch_builtins.py:329-344):
+ *   q = x / scale; r = round(q); mask = qmin <= r - offset <= qmax
+ *   grad_in     = grad * mask                                                    (may be NULL: not written)
+ *   scale_grad  = sum over the channel of grad * (clamp(r, offset+qmin, offset+qmax) - q * mask)
+ *   offset_grad = sum over the channel of grad * (~mask * scale)
+ * where the reference leaves the two sums to autograd's reduction to the parameter shape.  The tensor is laid out
+ * [outer][num_channel][num_element_per_channel] (outer = num_element / (num_channel * num_element_per_channel)).
+ * scale_grad / offset_grad: device float[num_channel], either may be NULL.  Element terms are float32; they are
+ * added per workgroup in float32 and across workgroups in double, in a fixed order.  workspace: device memory of
+ * miq_v2_qdq_bwd_params_workspace_bytes() bytes, overwritten by each call. */
+int64_t miq_v2_qdq_bwd_params_workspace_bytes(int64_t num_channel, int64_t num_element,
+                                              int64_t num_element_per_channel);
+int miq_v2_qdq_bwd_params_f32(const float* x, const float* grad_out, float* grad_in, int64_t num_channel,
+                              int64_t num_element, int64_t num_element_per_channel, const float* scale,
+                              const float* offset, int qmin, int qmax, float* scale_grad, float* offset_grad,
+                              void* workspace, void* stream);
+int miq_v2_qdq_bwd_params_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* grad_in, int64_t num_channel,
+                               int64_t num_element, int64_t num_element_per_channel, const float* scale,
+                               const float* offset, int qmin, int qmax, float* scale_grad, float* offset_grad,
+                               void* workspace, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
  * Calibration statistics

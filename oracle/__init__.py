@@ -84,6 +84,8 @@ class _Oracle:
                                      C.c_int, C.c_int]
         L.orc_v2_qdq_bf16.argtypes = [_u16p, _i64, _i64, _i64, _u16p, C.c_void_p, _f32p, _f32p, C.c_int, C.c_int]
         L.orc_v2_qdq_bwd_f32.argtypes = [_f32p, _f32p, _i64, _i64, _i64, _f32p, _f32p, _f32p, C.c_int, C.c_int]
+        L.orc_v2_qdq_bwd_params_f32.argtypes = [_f32p, _f32p, _i64, _i64, _i64, _f32p, _f32p, _f32p, C.c_int, C.c_int,
+                                                _f64p, _f64p]
         L.orc_bf16_to_f32.argtypes = [C.c_uint16]
         L.orc_bf16_to_f32.restype = C.c_float
         L.orc_f32_to_bf16.argtypes = [C.c_float]
@@ -210,6 +212,15 @@ class _Oracle:
         self.L.orc_v2_qdq_bwd_f32(x.reshape(-1), g.reshape(-1), num_channel, x.size, n_per_channel,
                                   out.reshape(-1), _f32(scale), _f32(offset), qmin, qmax)
         return out
+
+    def v2_qdq_bwd_params(self, x, g, num_channel, n_per_channel, scale, offset, qmin, qmax):
+        """(grad_in float32, scale_grad float64[C], offset_grad float64[C])."""
+        x, g = _f32(x), _f32(g)
+        gin = np.empty_like(x)
+        sg, og = np.zeros(num_channel, np.float64), np.zeros(num_channel, np.float64)
+        self.L.orc_v2_qdq_bwd_params_f32(x.reshape(-1), g.reshape(-1), num_channel, x.size, n_per_channel,
+                                         gin.reshape(-1), _f32(scale), _f32(offset), qmin, qmax, sg, og)
+        return gin, sg, og
 
     # -- bf16 helpers ------------------------------------------------------------------------------------------
     def f32_to_bf16_bits(self, x):

@@ -712,3 +712,39 @@ void orc_v2_qdq_bwd_f32(const float* in, const float* gout, int64_t numChannel, 
         gin[i]     = gout[i] * (float) inside;
     }
 }
+
+/* torch_builtins.py:329-344, all three gradients of QuantDequantFunc:
+ *   scale_grad  = grad * (clamp(round(x/s), o+qmin, o+qmax) - (x/s) * mask)
+ *   offset_grad = grad * (~mask * s)
+ * each element term in float32 as the reference forms it; the reduction to the parameter shape, which the reference
+ * leaves to autograd's float32 sum (order unspecified), is done here in double.  gin may be NULL. */
+void orc_v2_qdq_bwd_params_f32(const float* in, const float* gout, int64_t numChannel, int64_t numElement,
+                               int64_t numElementPerChannel, float* gin, const float* scale, const float* offset,
+                               int qmin, int qmax, double* scaleGrad, double* offsetGrad)
+{
+    for (int64_t c = 0; c < numChannel; ++c)
+        scaleGrad[c] = offsetGrad[c] = 0.0;
+    for (int64_t i = 0; i < numElement; ++i)
+    {
+        int64_t c  = (i / numElementPerChannel) % numChannel;
+        float q    = in[i] / scale[c];
+        float r    = rintf(q);
+        float rm   = r - offset[c];
+        int inside = ((float) qmin <= rm) && (rm <= (float) qmax);
+        float lo   = offset[c] + (float) qmin;
+        float hi   = offset[c] + (float) qmax;
+        float cl   = r;
+        if (cl < lo)
+            cl = lo;
+        if (cl > hi)
+            cl = hi;
+        float masked = q * (float) inside;
+        float ts     = gout[i] * (cl - masked);
+        float notm   = (float) (!inside) * scale[c];
+        float to     = gout[i] * notm;
+        scaleGrad[c] += (double) ts;
+        offsetGrad[c] += (double) to;
+        if (gin)
+            gin[i] = gout[i] * (float) inside;
+    }
+}
