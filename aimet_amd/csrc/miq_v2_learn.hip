@@ -30,6 +30,8 @@ struct LearnGeom
     int64_t npc;            // elements per row
     int64_t span;           // elements per workgroup (multiple of the vector width)
     int64_t rows;           // outer * num_channel
+    uint32_t outer;
+    bool direct;            // one workgroup per channel in total: its sums are the result, no second kernel
 };
 
 struct LearnParams
@@ -100,7 +102,9 @@ template <typename IO, bool VECTOR, bool WRITE_GX>
 __global__ __launch_bounds__(kBlock) void learn_bwd_kernel(const IO* __restrict__ x, const IO* __restrict__ g,
                                                            IO* __restrict__ gx, const float* __restrict__ scale,
                                                            const float* __restrict__ offset, int qmin, int qmax,
-                                                           LearnGeom geo, float2* __restrict__ partial)
+                                                           LearnGeom geo, float2* __restrict__ partial,
+                                                           float* __restrict__ scale_grad,
+                                                           float* __restrict__ offset_grad)
 {
     using T              = IOTraits<IO>;
     const uint32_t row   = fastdiv(blockIdx.x, geo.chunks_div);
@@ -182,21 +186,30 @@ __global__ __launch_bounds__(kBlock) void learn_bwd_kernel(const IO* __restrict_
             a += wave_sum[w].x;
             b += wave_sum[w].y;
         }
-        partial[blockIdx.x] = make_float2(a, b);
+        if (geo.direct)
+        {
+            if (scale_grad)
+                scale_grad[blockIdx.x] = a;
+            if (offset_grad)
+                offset_grad[blockIdx.x] = b;
+        }
+        else
+            partial[blockIdx.x] = make_float2(a, b);
     }
 }
 
-// One wavefront per channel: adds the channel's partials (outer x chunks of them) in double.
-__global__ __launch_bounds__(64) void learn_reduce_kernel(const float2* __restrict__ partial, LearnGeom geo,
-                                                          uint32_t outer, float* __restrict__ scale_grad,
-                                                          float* __restrict__ offset_grad)
+// One workgroup per channel: adds the channel's partials (outer x chunks of them) in double, each lane a strided
+// share in index order, then a fixed tree over the lanes.
+__global__ __launch_bounds__(kBlock) void learn_reduce_kernel(const float2* __restrict__ partial, LearnGeom geo,
+                                                              float* __restrict__ scale_grad,
+                                                              float* __restrict__ offset_grad)
 {
     const uint32_t ch = blockIdx.x;
     double a = 0.0, b = 0.0;
-    for (uint32_t o = 0; o < outer; ++o)
+    for (uint32_t o = 0; o < geo.outer; ++o)
     {
         const float2* row = partial + ((int64_t) o * geo.num_channel + ch) * geo.chunks;
-        for (uint32_t k = threadIdx.x; k < geo.chunks; k += 64)
+        for (uint32_t k = threadIdx.x; k < geo.chunks; k += kBlock)
         {
             const float2 v = row[k];
             a += (double) v.x;
@@ -209,8 +222,22 @@ __global__ __launch_bounds__(64) void learn_reduce_kernel(const float2* __restri
         a += __shfl_xor(a, o);
         b += __shfl_xor(b, o);
     }
+    __shared__ double wave_sum[2][kBlock / 64];
+    if ((threadIdx.x & 63) == 0)
+    {
+        wave_sum[0][threadIdx.x >> 6] = a;
+        wave_sum[1][threadIdx.x >> 6] = b;
+    }
+    __syncthreads();
     if (threadIdx.x == 0)
     {
+        a = b = 0.0;
+#pragma unroll
+        for (int w = 0; w < kBlock / 64; ++w)
+        {
+            a += wave_sum[0][w];
+            b += wave_sum[1][w];
+        }
         if (scale_grad)
             scale_grad[ch] = (float) a;
         if (offset_grad)
@@ -237,6 +264,8 @@ int make_learn_geom(int64_t num_channel, int64_t n, int64_t npc, LearnGeom& geo,
     geo.span       = span;
     geo.chunks     = (uint32_t) chunks;
     geo.chunks_div = make_fastdiv((uint32_t) chunks);
+    geo.outer      = (uint32_t) outer;
+    geo.direct     = outer == 1 && chunks == 1;
     return MIQ_OK;
 }
 
@@ -260,7 +289,8 @@ int launch_learn(const IO* x, const IO* g, IO* gx, int64_t num_channel, int64_t 
     {
         const dim3 grid((uint32_t) (geo.rows * geo.chunks));
 #define MIQ_LEARN(V, W)                                                                                                \
-    learn_bwd_kernel<IO, V, W><<<grid, kBlock, 0, stream>>>(x, g, gx, scale, offset, qmin, qmax, geo, partial)
+    learn_bwd_kernel<IO, V, W><<<grid, kBlock, 0, stream>>>(x, g, gx, scale, offset, qmin, qmax, geo, partial,         \
+                                                            scale_grad, offset_grad)
         if (vector && gx)
             MIQ_LEARN(true, true);
         else if (vector)
@@ -272,9 +302,11 @@ int launch_learn(const IO* x, const IO* g, IO* gx, int64_t num_channel, int64_t 
 #undef MIQ_LEARN
         MIQ_CHECK_LAUNCH();
     }
-    learn_reduce_kernel<<<dim3(geo.num_channel), 64, 0, stream>>>(partial, geo, (uint32_t) outer, scale_grad,
-                                                                  offset_grad);
-    MIQ_CHECK_LAUNCH();
+    if (!geo.direct)
+    {
+        learn_reduce_kernel<<<dim3(geo.num_channel), kBlock, 0, stream>>>(partial, geo, scale_grad, offset_grad);
+        MIQ_CHECK_LAUNCH();
+    }
     return MIQ_OK;
 }
 }   // namespace
