@@ -10,18 +10,24 @@ Same functions, argument meaning and error behaviour as the reference's torch_bu
 The forward of quantize / quantize_dequantize is one fused kernel (the reference runs about seven elementwise ATen
 kernels and saves a bool mask); the input gradient is one fused kernel that recomputes the mask from the saved
 input.  float32 and bfloat16 tensors are computed in float32, as the reference does for 4- and 8-bit grids; other
-float types are upcast to float32.  Scale / offset must be per-tensor or per-channel along one axis (numpy-style
-broadcast); block quantization (`block_size`) and multi-axis scales are not implemented.
+float types are upcast to float32.
 
-Gradients w.r.t. scale and offset (range learning) are formed with tensor ops from the same formulas
-(torch_builtins.py:329-344); they are not on the measured hot path.
+Scale / offset may be per-tensor, per-channel, vary along several axes, or be blockwise (`block_size`, reference
+:347-399).  The kernels index parameters as channel(i) = (i / n_per_channel) % num_channel over the flat tensor, which
+covers every layout whose varying axes are adjacent in memory (per-channel along any one axis; blocks cutting the
+last varying axis, e.g. weight [out, in] with scale [out, in / block]) without a copy; other layouts take one permuted
+copy each way.
+
+Gradients w.r.t. scale and offset (range learning, :329-344) come from one fused pass over the input and the
+incoming gradient when a channel's elements form runs of at least 256; shorter runs use tensor ops.
 """
 from typing import List, Optional
 
 import torch
 
 from ..... import ops
-from ....utils import _is_expandable
+from ....utils import (_is_expandable, channel_view, channel_view_restore, get_encoding_shape_with_blocks,
+                       reshape_tensor_for_blocks)
 
 
 def _is_value_representable(dtype: torch.dtype, value: int) -> bool:
@@ -35,8 +41,21 @@ def _is_grid_representable(dtype: torch.dtype, qmin: int, qmax: int) -> bool:
 
 def _validate_arguments(tensor, scale, offset, qmin=None, qmax=None, block_size=None):
     if block_size is not None:
-        raise RuntimeError("block_size is not implemented by the hip_gfx950 backend")
-    if not _is_expandable(scale.shape, tensor.shape):
+        if len(scale.shape) != len(block_size):
+            raise RuntimeError(f'Length of scale shape {scale.shape} must equal length of block size {block_size}')
+        if len(block_size) > tensor.dim():
+            raise RuntimeError(f'Block size {block_size} has more dimensions than the tensor of shape {tensor.shape}')
+        for i in range(1, len(block_size) + 1):
+            if block_size[-i] == -1:
+                if tensor.shape[-i] % scale.shape[-i] != 0:
+                    raise RuntimeError(f'Each tensor dimension size for tensor shape {tensor.shape} must divide '
+                                       f'evenly with corresponding scale dimension value for scale shape '
+                                       f'{scale.shape}')
+            elif block_size[-i] * scale.shape[-i] != tensor.shape[-i]:
+                raise RuntimeError(f'Each tensor dimension size for tensor shape {tensor.shape} must equal the '
+                                   f'corresponding scale dimension size * block size for scale shape {scale.shape} '
+                                   f'and block size {block_size}')
+    elif not _is_expandable(scale.shape, tensor.shape):
         raise RuntimeError(f"Scale of shape {scale.shape} cannot be expanded like input tensor of shape "
                            f"{tensor.shape}")
     if tensor.device != scale.device or tensor.device != offset.device:
@@ -47,22 +66,22 @@ def _validate_arguments(tensor, scale, offset, qmin=None, qmax=None, block_size=
 
 
 def _channel_geometry(tensor_shape, scale_shape):
-    """(num_channel, n_per_channel) of a scale that is per-tensor or varies along exactly one axis."""
-    padded = (1,) * (len(tensor_shape) - len(scale_shape)) + tuple(scale_shape)
-    axes = [a for a, d in enumerate(padded) if d != 1]
-    if not axes:
-        n = 1
-        for d in tensor_shape:
-            n *= d
-        return 1, max(n, 1)
-    if len(axes) > 1:
-        raise RuntimeError(f"scale of shape {tuple(scale_shape)} varies along more than one axis: not implemented by "
-                           "the hip_gfx950 backend")
-    axis = axes[0]
-    npc = 1
-    for d in tensor_shape[axis + 1:]:
-        npc *= d
-    return tensor_shape[axis], npc
+    """(num_channel, n_per_channel) of a tensor laid out [outer, num_channel, n_per_channel] by channel_view."""
+    assert len(tensor_shape) == 3 and tuple(scale_shape) == (tensor_shape[1], 1)
+    return tensor_shape[1], max(tensor_shape[2], 1)
+
+
+def _apply_per_channel(func, tensor, scale, offset, qmin, qmax, block_size):
+    """Runs an autograd function of (tensor3, scale[C, 1], offset[C, 1]) on the channel layout of the tensor.  The
+    re-layout is made of differentiable views / copies, so gradients flow back in the callers' shapes."""
+    shape = tensor.shape
+    if scale.shape != offset.shape:
+        scale, offset = torch.broadcast_tensors(scale, offset)
+    expanded = reshape_tensor_for_blocks(tensor, scale.shape, block_size)
+    tensor3, perm = channel_view(expanded, get_encoding_shape_with_blocks(scale.shape, block_size))
+    c = tensor3.shape[1]
+    out = func.apply(tensor3, scale.reshape(c, 1), offset.reshape(c, 1), qmin, qmax)
+    return channel_view_restore(out, expanded.shape, perm).reshape(shape)
 
 
 # The one-pass backward gives each contiguous channel row to its own workgroups; below this row length that is
@@ -155,7 +174,7 @@ def quantize(tensor: torch.Tensor, scale: torch.Tensor, offset: torch.Tensor, qm
     if not _is_grid_representable(tensor.dtype, qmin, qmax):
         raise RuntimeError(f"{tensor.dtype} is unable to represent quantized output of range [{qmin}, {qmax}].")
     x, orig = _prepare(tensor, scale, offset)
-    out = _QuantizeFunc.apply(x, scale, offset, qmin, qmax)
+    out = _apply_per_channel(_QuantizeFunc, x, scale, offset, qmin, qmax, block_size)
     return out.to(orig) if orig is not None else out
 
 
@@ -166,7 +185,7 @@ def quantize_dequantize(tensor: torch.Tensor, scale: torch.Tensor, offset: torch
     if not _is_grid_representable(torch.float32, qmin, qmax):
         raise RuntimeError(f"{torch.float32} is unable to represent quantized output of range [{qmin}, {qmax}].")
     x, orig = _prepare(tensor, scale, offset)
-    out = _QuantDequantFunc.apply(x, scale, offset, qmin, qmax)
+    out = _apply_per_channel(_QuantDequantFunc, x, scale, offset, qmin, qmax, block_size)
     return out.to(orig) if orig is not None else out
 
 
@@ -174,4 +193,8 @@ def dequantize(tensor: torch.Tensor, scale: torch.Tensor, offset: torch.Tensor,
                block_size: Optional[List] = None) -> torch.Tensor:
     """(x + offset) * scale on an already quantized tensor; not a hot op (two elementwise tensor ops)."""
     _validate_arguments(tensor, scale, offset, block_size=block_size)
-    return (tensor + offset.to(tensor.dtype)) * scale.to(tensor.dtype)
+    shape = tensor.shape
+    expanded = reshape_tensor_for_blocks(tensor, scale.shape, block_size)
+    pshape = get_encoding_shape_with_blocks(scale.shape, block_size)
+    out = (expanded + offset.to(tensor.dtype).reshape(pshape)) * scale.to(tensor.dtype).reshape(pshape)
+    return out.reshape(shape)

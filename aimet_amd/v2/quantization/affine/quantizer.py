@@ -12,7 +12,8 @@ from typing import Optional
 import torch
 from torch import nn
 
-from ...utils import StatisticsNotFoundError, _is_expandable, patch_attr, ste_round
+from ...utils import (StatisticsNotFoundError, _is_expandable, get_encoding_shape_with_blocks, patch_attr,
+                      reshape_tensor_for_blocks, ste_round)
 from ..encoding_analyzer import EncodingAnalyzer, MinMaxEncodingAnalyzer
 from .backends import _derive_qmin_qmax, quantize, quantize_dequantize
 
@@ -73,13 +74,14 @@ class MinMaxQuantizer(nn.Module):
                             f"{', '.join(kwargs)}")
         if qmin >= qmax:
             raise ValueError(f"qmax should be strictly larger than qmin. Got qmax={qmax}, qmin={qmin}")
-        if block_size is not None:
-            raise NotImplementedError("block_size is not implemented")
         self.qmin, self.qmax = qmin, qmax
         self._symmetric = symmetric
-        self.block_size = None
-        self.encoding_analyzer: EncodingAnalyzer = encoding_analyzer or MinMaxEncodingAnalyzer(self.shape)
-        if not _is_expandable(self.encoding_analyzer.observer.shape, self.shape):
+        self.block_size = tuple(block_size) if block_size is not None else None
+        # with blocks, statistics are gathered on the tensor split into (blocks, block length) per axis, by an
+        # analyzer whose shape has a 1 after every axis (reference :140-148)
+        self.encoding_analyzer: EncodingAnalyzer = encoding_analyzer or MinMaxEncodingAnalyzer(
+            get_encoding_shape_with_blocks(self.shape, self.block_size))
+        if self.block_size is None and not _is_expandable(self.encoding_analyzer.observer.shape, self.shape):
             raise RuntimeError(f'Encoding analyzer of shape {self.encoding_analyzer.observer.shape} '
                                f'is incompatible with quantizer of shape {self.shape}.')
         self.min = nn.Parameter(-torch.ones(self.shape))
@@ -131,10 +133,13 @@ class MinMaxQuantizer(nn.Module):
 
         @functools.wraps(original_forward)
         def forward_wrapper(input):  # pylint: disable=redefined-builtin
-            batch_statistics = self.encoding_analyzer.update_stats(input)
+            expanded = reshape_tensor_for_blocks(input, self.shape, self.block_size)
+            batch_statistics = self.encoding_analyzer.update_stats(expanded)
             num_steps = self.qmax - self.qmin
             dyn_min, dyn_max = self.encoding_analyzer.compute_encodings_from_stats(batch_statistics, num_steps,
                                                                                    self.symmetric)
+            if self.block_size is not None:
+                dyn_min, dyn_max = dyn_min.view(self.min.shape), dyn_max.view(self.max.shape)
             dyn_min = dyn_min.to(dtype=self.min.dtype, device=self.min.device).expand_as(self.min)
             dyn_max = dyn_max.to(dtype=self.max.dtype, device=self.max.device).expand_as(self.max)
             with patch_attr(self, 'min', dyn_min), patch_attr(self, 'max', dyn_max), \
@@ -151,6 +156,8 @@ class MinMaxQuantizer(nn.Module):
             return
         if enc_min is None or enc_max is None:
             return
+        if self.block_size is not None:
+            enc_min, enc_max = enc_min.view(self.min.shape), enc_max.view(self.max.shape)
         self.set_range(enc_min, enc_max)
 
     def set_range(self, min: torch.Tensor, max: torch.Tensor):  # pylint: disable=redefined-builtin
@@ -219,7 +226,8 @@ class Quantize(MinMaxQuantizer):
             raise RuntimeError('Failed to run Quantize since quantization parameters are not initialized.'
                                ' Please initialize the quantization parameters using `compute_encodings()`.')
         encoding = self.get_encoding()
-        return quantize(input, encoding.scale, encoding.offset, encoding.qmin, encoding.qmax)
+        return quantize(input, encoding.scale, encoding.offset, encoding.qmin, encoding.qmax,
+                        block_size=self.block_size)
 
 
 class QuantizeDequantize(MinMaxQuantizer):
@@ -230,4 +238,5 @@ class QuantizeDequantize(MinMaxQuantizer):
             raise RuntimeError('Failed to run QuantizeDequantize since quantization parameters are not initialized.'
                                ' Please initialize the quantization parameters using `compute_encodings()`.')
         encoding = self.get_encoding()
-        return quantize_dequantize(input, encoding.scale, encoding.offset, encoding.qmin, encoding.qmax)
+        return quantize_dequantize(input, encoding.scale, encoding.offset, encoding.qmin, encoding.qmax,
+                                   block_size=self.block_size)

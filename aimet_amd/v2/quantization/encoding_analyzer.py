@@ -10,7 +10,7 @@ _HistogramObserver (:131-270) and SqnrEncodingAnalyzer (:522-725): the running h
 search live on the GPU.  One update is five kernels and reads the batch twice (finite min/max; one binning pass that
 fills the batch's histogram and the merged-range histogram together); the reference reads it about eight times and
 re-bins with per-element Python loops.  Nothing synchronises until an encoding or a statistic is read.  Differences:
-observer shapes must be per-tensor or vary along the leading axis of the input only (contiguous slabs); an input
+an observer shape that does not split the input into contiguous slabs costs one re-laid-out copy per update; an input
 without any finite value is reported (ValueError) when results are next read, not at update time; candidate scores are
 accumulated in double, so near-ties between candidates may resolve differently from torch.sum's float32 order.
 """
@@ -21,7 +21,7 @@ from typing import Optional, Tuple
 import torch
 
 from ... import ops
-from ..utils import StatisticsNotFoundError, _is_expandable
+from ..utils import StatisticsNotFoundError, _is_expandable, channel_view
 
 
 @dataclass
@@ -45,17 +45,13 @@ class _MinMaxObserver:
         if not _is_expandable(self.shape, input_tensor.shape):
             raise RuntimeError(f"Input of shape {list(input_tensor.shape)} can't be reduced to shape "
                                f"{list(self.shape)}")
-        padded = (1,) * (input_tensor.dim() - len(self.shape)) + self.shape
-        axes = [a for a, d in enumerate(padded) if d != 1]
-        if not axes:
+        if math.prod(self.shape) == 1:
             mm = ops.minmax(input_tensor)
-            return _MinMaxRange(mm[0].reshape(self.shape).to(input_tensor.dtype),
-                                mm[1].reshape(self.shape).to(input_tensor.dtype))
-        if len(axes) > 1:
-            raise RuntimeError(f"observer shape {self.shape} varies along more than one axis: not implemented")
-        axis = axes[0]
-        n_per_channel = math.prod(input_tensor.shape[axis + 1:])
-        mm = ops.minmax_per_channel(input_tensor, input_tensor.shape[axis], n_per_channel)
+        else:
+            # [outer, channel, run]: one launch for every channel; axes that are not adjacent in memory cost one
+            # permuted copy
+            tensor3, _ = channel_view(input_tensor, self.shape)
+            mm = ops.minmax_per_channel(tensor3, tensor3.shape[1], tensor3.shape[2])
         return _MinMaxRange(mm[0].reshape(self.shape).to(input_tensor.dtype),
                             mm[1].reshape(self.shape).to(input_tensor.dtype))
 
@@ -224,12 +220,11 @@ class _HistogramObserver:
             raise RuntimeError(f"Shape {self.shape} is incompatible with input of shape {input_tensor.shape}")
         if not input_tensor.is_cuda:
             raise RuntimeError("the histogram observer (aimet_amd) computes on the GPU only")
-        padded = (1,) * (input_tensor.dim() - len(self.shape)) + self.shape
-        axes = [a for a, d in enumerate(padded) if d != 1]
-        if axes and (len(axes) > 1 or any(d != 1 for d in input_tensor.shape[:axes[0]])):
-            raise RuntimeError(f"observer shape {self.shape} does not split the input of shape "
-                               f"{tuple(input_tensor.shape)} into contiguous slabs: not implemented")
-        return input_tensor.detach().to(torch.float32).contiguous()
+        # one contiguous slab per histogram; layouts that are not already slabs take one copy
+        tensor3, _ = channel_view(input_tensor.detach().to(torch.float32), self.shape)
+        if tensor3.shape[0] != 1:
+            tensor3 = tensor3.transpose(0, 1)
+        return tensor3.reshape(self.num_histograms, -1).contiguous()
 
     @torch.no_grad()
     def _update(self, input_tensor: torch.Tensor, merge: bool, want_batch: bool = True):

@@ -1,6 +1,7 @@
 """Small helpers shared by the v2 modules (TrainingExtensions/torch/src/python/aimet_torch/v2/utils.py:46-204)."""
 import contextlib
 import functools
+import math
 from typing import Any, Callable, Tuple
 
 import torch
@@ -14,6 +15,63 @@ def _is_expandable(src_shape: Tuple[int, ...], target_shape: Tuple[int, ...]) ->
         if src_dim not in (1, dst_dim):
             return False
     return True
+
+
+def channel_view(tensor: torch.Tensor, param_shape: Tuple[int, ...]):
+    """Lays `tensor` out as [outer, num_channel, n_per_channel] so that every [n_per_channel] run shares the element
+    of a parameter of shape `param_shape` (numpy-style broadcastable to the tensor) it is quantized with, channels in
+    the parameter's row-major order.
+
+    Returns (tensor3, perm).  When the axes along which the parameter varies are adjacent in memory this is a plain
+    reshape (perm None): per-tensor, per-channel along one axis, and blocks that cut only the last varying axis
+    (e.g. a Linear weight [out, in] with scale [out, in / block]).  Otherwise the varying axes are moved to the front
+    with one permuted copy; `perm` is then the permutation that channel_view_restore undoes."""
+    shape = tuple(tensor.shape)
+    padded = (1,) * (len(shape) - len(param_shape)) + tuple(param_shape)
+    varying = [a for a, p in enumerate(padded) if p != 1]
+    if not varying:
+        return tensor.reshape(1, 1, tensor.numel()), None
+    first, last = varying[0], varying[-1]
+    num_channel = math.prod(padded)
+    if all(padded[a] == shape[a] for a in range(first, last + 1)):
+        return tensor.reshape(math.prod(shape[:first]), num_channel, math.prod(shape[last + 1:])), None
+    shared = [a for a in range(len(shape)) if a not in varying]
+    perm = varying + shared
+    return tensor.permute(perm).reshape(1, num_channel, math.prod(shape[a] for a in shared)), perm
+
+
+def channel_view_restore(tensor3: torch.Tensor, shape: Tuple[int, ...], perm) -> torch.Tensor:
+    """Inverse of channel_view for a result of the same layout."""
+    if perm is None:
+        return tensor3.reshape(shape)
+    inverse = [0] * len(perm)
+    for i, a in enumerate(perm):
+        inverse[a] = i
+    return tensor3.reshape([shape[a] for a in perm]).permute(inverse).contiguous()
+
+
+def reshape_tensor_for_blocks(tensor: torch.Tensor, encoding_shape, block_size) -> torch.Tensor:
+    """Splits each of the last len(block_size) axes into (number of blocks, block length); -1 means "derive the
+    block length from the shapes" (reference torch_builtins.py:364-399)."""
+    if block_size is None:
+        return tensor
+    nb = len(block_size)
+    split = []
+    for axis in range(nb):
+        dim, blocks = tensor.shape[tensor.dim() - nb + axis], encoding_shape[axis]
+        split += [blocks, dim // blocks if block_size[axis] == -1 else block_size[axis]]
+    return tensor.reshape(list(tensor.shape[:tensor.dim() - nb]) + split)
+
+
+def get_encoding_shape_with_blocks(encoding_shape, block_size):
+    """Parameter shape that broadcasts against reshape_tensor_for_blocks' result: a 1 after every axis (reference
+    torch_builtins.py:347-362)."""
+    if block_size is None:
+        return tuple(encoding_shape)
+    out = []
+    for d in encoding_shape:
+        out += [d, 1]
+    return tuple(out)
 
 
 class StatisticsNotFoundError(RuntimeError):

@@ -121,7 +121,7 @@ def test_per_channel(ea):
     assert qmin.shape == shape and qmax.shape == shape
     assert torch.equal(qmin.cpu().view(-1), rmin) and torch.equal(qmax.cpu().view(-1), rmax)
     with pytest.raises(RuntimeError):
-        ea.SqnrEncodingAnalyzer((1, 3, 1, 1)).update_stats(x.cuda())     # slabs not contiguous: not implemented
+        ea.SqnrEncodingAnalyzer((1, 4, 1, 1)).update_stats(x.cuda())     # shape does not broadcast to the input
 
 
 def test_reference_cases_through_the_analyzer(ea):

@@ -190,3 +190,50 @@ def test_cpu_tensors_are_rejected_everywhere():
                  lambda: ops.Analyzer(1, torch.device("cpu")).update_stats(x)):
         with pytest.raises((RuntimeError, AssertionError)):
             call()
+
+
+# ---------------------------------------------------------------------------------- v2 channel layouts and blocks
+@pytest.mark.parametrize("shape,param_shape,copies", [
+    ((6, 5, 4), (), False), ((6, 5, 4), (6, 1, 1), False), ((6, 5, 4), (5, 1), False), ((6, 5, 4), (4,), False),
+    ((6, 5, 4), (6, 5, 1), False), ((6, 5, 4), (6, 1, 4), True), ((2, 6, 1, 4), (6, 1, 4), False),
+    ((4, 1, 3, 2), (4, 1, 3, 1), False),          # Linear weight [4, 6] split into blocks of 2 along the input axis
+    ((2, 2, 3, 2), (2, 1, 3, 1), True),           # blocks along both axes
+])
+def test_channel_view_groups_elements_by_parameter(shape, param_shape, copies):
+    from aimet_amd.v2.utils import channel_view, channel_view_restore
+    n_param = int(math.prod(param_shape))
+    which = torch.arange(n_param, dtype=torch.float32).reshape(param_shape).expand(shape)
+    values = torch.arange(math.prod(shape), dtype=torch.float32).reshape(shape)
+    t3, perm = channel_view(which, param_shape)
+    v3, perm_v = channel_view(values, param_shape)
+    assert (perm is not None) == copies and perm == perm_v
+    assert t3.dim() == 3 and t3.shape[1] == n_param
+    # every run of channel c holds elements that broadcast against parameter element c
+    assert torch.equal(t3, torch.arange(n_param, dtype=torch.float32).view(1, -1, 1).expand_as(t3))
+    assert torch.equal(channel_view_restore(v3, shape, perm), values)
+    if not copies:
+        # no copy: the flat order is untouched, which is what the kernels' (i / run) % channels indexing assumes
+        assert torch.equal(v3.reshape(-1), values.reshape(-1))
+
+
+def test_block_reshape_helpers_follow_the_reference_shapes():
+    # test_backend.py:627-639 of the reference
+    from aimet_amd.v2.utils import get_encoding_shape_with_blocks, reshape_tensor_for_blocks
+    inp = torch.randn(8, 6, 8, 3)
+    assert reshape_tensor_for_blocks(inp, (4, 3, 8, 1), [-1, 2, 1, 3]).shape == (4, 2, 3, 2, 8, 1, 1, 3)
+    assert get_encoding_shape_with_blocks((4, 3, 8, 1), [-1, 2, 1, 3]) == (4, 1, 3, 1, 8, 1, 1, 1)
+    assert reshape_tensor_for_blocks(inp, (4, 3, 8, 1), None) is inp
+    assert get_encoding_shape_with_blocks((4, 3), None) == (4, 3)
+    # leading axes beyond the block specification stay as they are
+    assert reshape_tensor_for_blocks(torch.randn(3, 5, 4, 6), (2, 3), [2, 2]).shape == (3, 5, 2, 2, 3, 2)
+
+
+def test_affine_call_forms():
+    # reference backends/__init__.py:334-356
+    from aimet_amd.v2.quantization.affine.backends import _parse_args
+    assert _parse_args((8,), {}) == (0, 255, None)
+    assert _parse_args((8, True), {}) == (-128, 127, None)
+    assert _parse_args((4, True, (1, 2)), {}) == (-8, 7, (1, 2))
+    assert _parse_args((-7, 7), {"block_size": [2, 1]}) == (-7, 7, [2, 1])
+    assert _parse_args((), {"num_steps": 254, "signed": True}) == (-127, 127, None)
+    assert _parse_args((), {"qmin": 0, "qmax": 15}) == (0, 15, None)
