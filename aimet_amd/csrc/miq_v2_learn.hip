@@ -10,12 +10,17 @@
 // two sums in registers, and stores one (scale, offset) partial per workgroup.  A second small kernel adds the
 // partials of each channel in double precision in a fixed order, so results do not depend on scheduling.
 //
+// Rows of at most kShortRow elements (blockwise scales, small convolution kernels) are given to groups of 1..64 lanes
+// instead of whole workgroups: a group streams its row, the sums are combined with lane shuffles inside the group, and
+// the group's first lane stores the row's pair.
+//
 // Layout: the tensor is [outer][channel][elements-per-channel] in memory (outer = 1 for weights quantized along
 // axis 0, channel = 1 for per-tensor), so a "row" is one contiguous run that shares its parameters.
 #include "miq_common.h"
 #include "miq_fastmath.h"
 #include "miq_io.h"
 
+#include <algorithm>
 #include <cmath>
 
 namespace miq
@@ -32,7 +37,14 @@ struct LearnGeom
     int64_t rows;           // outer * num_channel
     uint32_t outer;
     bool direct;            // one workgroup per channel in total: its sums are the result, no second kernel
+    // short rows: lane groups instead of workgroups
+    bool short_rows;
+    uint32_t lanes;             // lanes per row, a power of two in 1..64
+    uint32_t lanes_log2;
+    uint32_t rows_per_block;
 };
+
+constexpr int64_t kShortRow = 2048;
 
 struct LearnParams
 {
@@ -70,6 +82,29 @@ __device__ __forceinline__ float learn_elem(const LearnParams& p, float x, float
     return g * m;
 }
 
+// one vector already in registers: the exact-division fast path is decided once for the vector
+template <int V>
+__device__ __forceinline__ void learn_vec_regs(const LearnParams& p, const float* xf, const float* gf, float* of,
+                                               float& sg, float& og)
+{
+    float m = 0.0f;
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+        m = fmaxf(m, fabsf(xf[j]));
+    if (p.rcp != 0.0f && m <= kFastDivMaxDividend)
+    {
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+            of[j] = learn_elem<true>(p, xf[j], gf[j], sg, og);
+    }
+    else
+    {
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+            of[j] = learn_elem<false>(p, xf[j], gf[j], sg, og);
+    }
+}
+
 template <typename IO, bool WRITE_GX>
 __device__ __forceinline__ void learn_vec(const LearnParams& p, const IO* x, const IO* g, IO* gx, int64_t at,
                                           float& sg, float& og)
@@ -78,22 +113,7 @@ __device__ __forceinline__ void learn_vec(const LearnParams& p, const IO* x, con
     float xf[T::VEC], gf[T::VEC], of[T::VEC];
     T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(x + at)), xf);
     T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(g + at)), gf);
-    float m = 0.0f;
-#pragma unroll
-    for (int j = 0; j < T::VEC; ++j)
-        m = fmaxf(m, fabsf(xf[j]));
-    if (p.rcp != 0.0f && m <= kFastDivMaxDividend)
-    {
-#pragma unroll
-        for (int j = 0; j < T::VEC; ++j)
-            of[j] = learn_elem<true>(p, xf[j], gf[j], sg, og);
-    }
-    else
-    {
-#pragma unroll
-        for (int j = 0; j < T::VEC; ++j)
-            of[j] = learn_elem<false>(p, xf[j], gf[j], sg, og);
-    }
+    learn_vec_regs<T::VEC>(p, xf, gf, of, sg, og);
     if (WRITE_GX)
         stream_store(reinterpret_cast<typename T::Vec*>(gx + at), T::pack(of));
 }
@@ -245,8 +265,125 @@ __global__ __launch_bounds__(kBlock) void learn_reduce_kernel(const float2* __re
     }
 }
 
+// Short rows.  A group of geo.lanes lanes owns a row at a time; a workgroup owns rows_per_block consecutive rows, so
+// what it reads and writes is one contiguous stretch.  Two rows are in flight per group.  partial has one pair per
+// row (chunks == 1), or, when outer == 1, the sums go straight to scale_grad / offset_grad.
+template <typename IO, bool VECTOR, bool WRITE_GX>
+__global__ __launch_bounds__(kBlock) void learn_rows_kernel(const IO* __restrict__ x, const IO* __restrict__ g,
+                                                            IO* __restrict__ gx, const float* __restrict__ scale,
+                                                            const float* __restrict__ offset, int qmin, int qmax,
+                                                            LearnGeom geo, float2* __restrict__ partial,
+                                                            float* __restrict__ scale_grad,
+                                                            float* __restrict__ offset_grad)
+{
+    using T                 = IOTraits<IO>;
+    constexpr int V         = VECTOR ? T::VEC : 1;
+    const uint32_t lane     = threadIdx.x & (geo.lanes - 1);
+    const uint32_t group    = threadIdx.x >> geo.lanes_log2;
+    const uint32_t groups   = kBlock >> geo.lanes_log2;
+    const int64_t row_begin = (int64_t) blockIdx.x * geo.rows_per_block;
+    const int64_t row_end   = min(row_begin + (int64_t) geo.rows_per_block, geo.rows);
+    const int64_t stride    = (int64_t) geo.lanes * V;
+    for (int64_t row0 = row_begin + group; row0 < row_end; row0 += 2 * groups)
+    {
+        float sg[2] = {0.0f, 0.0f}, og[2] = {0.0f, 0.0f};
+        const int64_t row1 = row0 + groups;
+        const bool two     = row1 < row_end;   // uniform over the group
+        const LearnParams p0 = load_params(scale, offset, (uint32_t) (row0 % geo.num_channel), qmin, qmax);
+        const LearnParams p1 =
+            load_params(scale, offset, (uint32_t) ((two ? row1 : row0) % geo.num_channel), qmin, qmax);
+        for (int64_t i = (int64_t) lane * V; i < geo.npc; i += stride)
+        {
+            if (VECTOR)
+            {
+                float xa[V], ga[V], xb[V], gb[V], oa[V], ob[V];
+                const int64_t at0 = row0 * geo.npc + i, at1 = row1 * geo.npc + i;
+                T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(x + at0)), xa);
+                T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(g + at0)), ga);
+                if (two)
+                {
+                    T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(x + at1)), xb);
+                    T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(g + at1)), gb);
+                }
+                learn_vec_regs<V>(p0, xa, ga, oa, sg[0], og[0]);
+                if (WRITE_GX)
+                    stream_store(reinterpret_cast<typename T::Vec*>(gx + at0), T::pack(oa));
+                if (two)
+                {
+                    learn_vec_regs<V>(p1, xb, gb, ob, sg[1], og[1]);
+                    if (WRITE_GX)
+                        stream_store(reinterpret_cast<typename T::Vec*>(gx + at1), T::pack(ob));
+                }
+            }
+            else
+            {
+                const int64_t at0 = row0 * geo.npc + i, at1 = row1 * geo.npc + i;
+                const float xa = T::load1(x + at0), ga = T::load1(g + at0);
+                const float xb = two ? T::load1(x + at1) : 0.0f, gb = two ? T::load1(g + at1) : 0.0f;
+                const float oa = learn_elem<false>(p0, xa, ga, sg[0], og[0]);
+                if (WRITE_GX)
+                    T::store1(gx + at0, oa);
+                if (two)
+                {
+                    const float ob = learn_elem<false>(p1, xb, gb, sg[1], og[1]);
+                    if (WRITE_GX)
+                        T::store1(gx + at1, ob);
+                }
+            }
+        }
+        // every lane of the group is here (lanes past the end of a short row hold zeros)
+        for (uint32_t o = geo.lanes >> 1; o > 0; o >>= 1)
+        {
+            sg[0] += __shfl_xor(sg[0], o);
+            og[0] += __shfl_xor(og[0], o);
+            sg[1] += __shfl_xor(sg[1], o);
+            og[1] += __shfl_xor(og[1], o);
+        }
+        if (lane == 0)
+        {
+#pragma unroll
+            for (int k = 0; k < 2; ++k)
+            {
+                if (k == 1 && !two)
+                    break;
+                const int64_t row = k ? row1 : row0;
+                if (geo.direct)
+                {
+                    if (scale_grad)
+                        scale_grad[row] = sg[k];
+                    if (offset_grad)
+                        offset_grad[row] = og[k];
+                }
+                else
+                    partial[row] = make_float2(sg[k], og[k]);
+            }
+        }
+    }
+}
+
+// Short rows with outer > 1: one lane per channel adds its `outer` row pairs in double, in index order.
+__global__ __launch_bounds__(kBlock) void learn_reduce_rows_kernel(const float2* __restrict__ partial, LearnGeom geo,
+                                                                   float* __restrict__ scale_grad,
+                                                                   float* __restrict__ offset_grad)
+{
+    const uint32_t ch = blockIdx.x * kBlock + threadIdx.x;
+    if (ch >= geo.num_channel)
+        return;
+    double a = 0.0, b = 0.0;
+    for (uint32_t o = 0; o < geo.outer; ++o)
+    {
+        const float2 v = partial[(int64_t) o * geo.num_channel + ch];
+        a += (double) v.x;
+        b += (double) v.y;
+    }
+    if (scale_grad)
+        scale_grad[ch] = (float) a;
+    if (offset_grad)
+        offset_grad[ch] = (float) b;
+}
+
 // rows, chunks and span for a tensor of num_channel x npc rows repeated `outer` times
-int make_learn_geom(int64_t num_channel, int64_t n, int64_t npc, LearnGeom& geo, int64_t& outer)
+int make_learn_geom(int64_t num_channel, int64_t n, int64_t npc, int vec, LearnGeom& geo, int64_t& outer)
 {
     MIQ_CHECK_ARG(num_channel >= 1 && npc >= 1 && n >= 0, "non-positive channel geometry");
     MIQ_CHECK_ARG(num_channel <= 0x7fffffff, "too many channels");
@@ -255,6 +392,33 @@ int make_learn_geom(int64_t num_channel, int64_t n, int64_t npc, LearnGeom& geo,
     geo.rows = outer * num_channel;
     geo.npc  = npc;
     geo.num_channel = (uint32_t) num_channel;
+    geo.outer      = (uint32_t) outer;
+    geo.short_rows = npc <= kShortRow;
+    if (geo.short_rows)
+    {
+        // lanes per row: enough to cover the row with one vector (or element) each, at most a wavefront
+        const int64_t per_lane = (npc % vec == 0) ? vec : 1;
+        uint32_t lanes = 1, log2 = 0;
+        while (lanes < 64 && (int64_t) lanes * per_lane < npc)
+        {
+            lanes <<= 1;
+            ++log2;
+        }
+        geo.lanes      = lanes;
+        geo.lanes_log2 = log2;
+        // about 8192 elements per workgroup, in whole passes of two rows per group; fewer when the tensor is small
+        const int64_t groups = kBlock / lanes;
+        int64_t rows_pb      = 2 * groups * std::max<int64_t>(1, 8192 / (2 * groups * npc));
+        while (rows_pb > 2 * groups && (geo.rows + rows_pb - 1) / rows_pb < 2048)
+            rows_pb -= 2 * groups;
+        geo.rows_per_block = (uint32_t) rows_pb;
+        geo.span           = npc;
+        geo.chunks         = 1;
+        geo.chunks_div     = make_fastdiv(1);
+        geo.direct         = outer == 1;
+        MIQ_CHECK_ARG((geo.rows + rows_pb - 1) / rows_pb < 0x7fffffff, "tensor too large for one launch");
+        return MIQ_OK;
+    }
     // Spans of 8192 elements keep partials few; shorter ones when that would leave compute units idle.
     int64_t span = 8192;
     while (span > 2048 && geo.rows * ((npc + span - 1) / span) < 2048)
@@ -264,7 +428,6 @@ int make_learn_geom(int64_t num_channel, int64_t n, int64_t npc, LearnGeom& geo,
     geo.span       = span;
     geo.chunks     = (uint32_t) chunks;
     geo.chunks_div = make_fastdiv((uint32_t) chunks);
-    geo.outer      = (uint32_t) outer;
     geo.direct     = outer == 1 && chunks == 1;
     return MIQ_OK;
 }
@@ -277,34 +440,49 @@ int launch_learn(const IO* x, const IO* g, IO* gx, int64_t num_channel, int64_t 
     MIQ_CHECK_ARG(scale && offset, "null parameter pointer");
     MIQ_CHECK_ARG(qmin <= qmax, "qmin must not exceed qmax");
     MIQ_CHECK_ARG(scale_grad || offset_grad, "neither scale_grad nor offset_grad requested");
+    const bool vector = npc % IOTraits<IO>::VEC == 0 && aligned16(x) && aligned16(g) && (!gx || aligned16(gx));
     LearnGeom geo{};
     int64_t outer = 0;
-    if (int rc = make_learn_geom(num_channel, n, npc, geo, outer))
+    if (int rc = make_learn_geom(num_channel, n, npc, vector ? IOTraits<IO>::VEC : 1, geo, outer))
         return rc;
     MIQ_CHECK_ARG(n == 0 || (x && g && workspace), "null pointer");
-    const bool vector = npc % IOTraits<IO>::VEC == 0 && aligned16(x) && aligned16(g) && (!gx || aligned16(gx));
-    float2* partial   = static_cast<float2*>(workspace);
+    float2* partial = static_cast<float2*>(workspace);
     // an empty tensor launches only the reduction, which then writes the zero sums
     if (n > 0)
     {
-        const dim3 grid((uint32_t) (geo.rows * geo.chunks));
-#define MIQ_LEARN(V, W)                                                                                                \
-    learn_bwd_kernel<IO, V, W><<<grid, kBlock, 0, stream>>>(x, g, gx, scale, offset, qmin, qmax, geo, partial,         \
-                                                            scale_grad, offset_grad)
-        if (vector && gx)
-            MIQ_LEARN(true, true);
-        else if (vector)
-            MIQ_LEARN(true, false);
-        else if (gx)
-            MIQ_LEARN(false, true);
+#define MIQ_LEARN(KERNEL, V, W)                                                                                        \
+    KERNEL<IO, V, W><<<grid, kBlock, 0, stream>>>(x, g, gx, scale, offset, qmin, qmax, geo, partial, scale_grad,       \
+                                                  offset_grad)
+#define MIQ_LEARN_VARIANTS(KERNEL)                                                                                     \
+    if (vector && gx)                                                                                                  \
+        MIQ_LEARN(KERNEL, true, true);                                                                                 \
+    else if (vector)                                                                                                   \
+        MIQ_LEARN(KERNEL, true, false);                                                                                \
+    else if (gx)                                                                                                       \
+        MIQ_LEARN(KERNEL, false, true);                                                                                \
+    else                                                                                                               \
+        MIQ_LEARN(KERNEL, false, false)
+        if (geo.short_rows)
+        {
+            const dim3 grid((uint32_t) ((geo.rows + geo.rows_per_block - 1) / geo.rows_per_block));
+            MIQ_LEARN_VARIANTS(learn_rows_kernel);
+        }
         else
-            MIQ_LEARN(false, false);
+        {
+            const dim3 grid((uint32_t) (geo.rows * geo.chunks));
+            MIQ_LEARN_VARIANTS(learn_bwd_kernel);
+        }
+#undef MIQ_LEARN_VARIANTS
 #undef MIQ_LEARN
         MIQ_CHECK_LAUNCH();
     }
     if (!geo.direct)
     {
-        learn_reduce_kernel<<<dim3(geo.num_channel), kBlock, 0, stream>>>(partial, geo, scale_grad, offset_grad);
+        if (geo.short_rows)
+            learn_reduce_rows_kernel<<<dim3((geo.num_channel + kBlock - 1) / kBlock), kBlock, 0, stream>>>(
+                partial, geo, scale_grad, offset_grad);
+        else
+            learn_reduce_kernel<<<dim3(geo.num_channel), kBlock, 0, stream>>>(partial, geo, scale_grad, offset_grad);
         MIQ_CHECK_LAUNCH();
     }
     return MIQ_OK;
@@ -321,7 +499,7 @@ int64_t miq_v2_qdq_bwd_params_workspace_bytes(int64_t num_channel, int64_t num_e
 {
     LearnGeom geo{};
     int64_t outer = 0;
-    if (make_learn_geom(num_channel, num_element, num_element_per_channel, geo, outer) != MIQ_OK)
+    if (make_learn_geom(num_channel, num_element, num_element_per_channel, 1, geo, outer) != MIQ_OK)
         return 0;
     const int64_t blocks = geo.rows * geo.chunks;
     return (int64_t) sizeof(float2) * (blocks > 0 ? blocks : 1);

@@ -19,7 +19,7 @@ last varying axis, e.g. weight [out, in] with scale [out, in / block]) without a
 copy each way.
 
 Gradients w.r.t. scale and offset (range learning, :329-344) come from one fused pass over the input and the
-incoming gradient when a channel's elements form runs of at least 256; shorter runs use tensor ops.
+incoming gradient, together with the input gradient.
 """
 from typing import List, Optional
 
@@ -84,11 +84,6 @@ def _apply_per_channel(func, tensor, scale, offset, qmin, qmax, block_size):
     return channel_view_restore(out, expanded.shape, perm).reshape(shape)
 
 
-# The one-pass backward gives each contiguous channel row to its own workgroups; below this row length that is
-# slower than torch's elementwise ops plus a reduction.
-_MIN_ROW_FOR_FUSED_PARAM_GRADS = 256
-
-
 def _reduce_like(grad: torch.Tensor, shape) -> torch.Tensor:
     return grad.sum_to_size(shape) if tuple(grad.shape) != tuple(shape) else grad
 
@@ -108,26 +103,12 @@ class _QuantDequantFunc(torch.autograd.Function):
         c, npc, qmin, qmax = ctx.geom
         tensor_grad = scale_grad = offset_grad = None
         if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-            if c == 1 or npc >= _MIN_ROW_FOR_FUSED_PARAM_GRADS:
-                # x and grad are read once: tensor_grad and both parameter sums come out of the same pass
-                tensor_grad, sg, og = ops.v2_qdq_bwd_params(tensor, grad, c, npc, scale, offset, qmin, qmax,
-                                                            want_grad_in=ctx.needs_input_grad[0])
-                scale_grad = sg.reshape(scale.shape).to(scale.dtype) if ctx.needs_input_grad[1] else None
-                offset_grad = og.reshape(offset.shape).to(offset.dtype) if ctx.needs_input_grad[2] else None
-                return tensor_grad, scale_grad, offset_grad, None, None
-            # short channel rows (a scale that varies along one of the innermost axes): elementwise terms from
-            # torch, reduced to the parameter shape as autograd would
-            s, o = scale.to(torch.float32), offset.to(torch.float32)
-            x = tensor.to(torch.float32) / s
-            x_round = torch.round(x) - o
-            mask = (qmin <= x_round) & (x_round <= qmax)
-            g = grad.to(torch.float32)
-            if ctx.needs_input_grad[1]:
-                scale_grad = _reduce_like(g * (torch.round(x).clamp(o + qmin, o + qmax) - x * mask),
-                                          scale.shape).to(scale.dtype)
-            if ctx.needs_input_grad[2]:
-                offset_grad = _reduce_like(g * (~mask * s), offset.shape).to(offset.dtype)
-        if ctx.needs_input_grad[0]:
+            # x and grad are read once: tensor_grad and both parameter sums come out of the same pass
+            tensor_grad, sg, og = ops.v2_qdq_bwd_params(tensor, grad, c, npc, scale, offset, qmin, qmax,
+                                                        want_grad_in=ctx.needs_input_grad[0])
+            scale_grad = sg.reshape(scale.shape).to(scale.dtype) if ctx.needs_input_grad[1] else None
+            offset_grad = og.reshape(offset.shape).to(offset.dtype) if ctx.needs_input_grad[2] else None
+        elif ctx.needs_input_grad[0]:
             tensor_grad = ops.v2_qdq_bwd(tensor, grad, c, npc, scale, offset, qmin, qmax)
         return tensor_grad, scale_grad, offset_grad, None, None
 

@@ -429,10 +429,11 @@ def bench_sqnr(torch, ops, reps=5):
 def bench_v2_range_learning(torch, ops, steps=50):
     """v2 quantize-dequantize backward with learnable scale and offset: the one-pass kernel (tensor_grad + both
     parameter sums; 12 B per element) against the torch elementwise ops + reductions of the same expressions, on the
-    main weight shape (per channel) and the activation shape (per tensor)."""
+    main weight shape (per channel), the activation shape (per tensor) and a blockwise weight (blocks of 128)."""
     dev = torch.device("cuda", 0)
     out = {}
-    for name, shape, c in (("per_channel_11008x4096", (11008, 4096), 11008), ("per_tensor_32x64x56x56", (32, 64, 56, 56), 1)):
+    for name, shape, c in (("per_channel_11008x4096", (11008, 4096), 11008), ("per_tensor_32x64x56x56", (32, 64, 56, 56), 1),
+                           ("blockwise_4096x4096_block128", (4096, 4096), 4096 * 32)):
         g = torch.Generator(device=dev).manual_seed(1006)
         n = 1
         for d in shape:

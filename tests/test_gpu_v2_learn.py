@@ -32,9 +32,17 @@ def _case(seed, outer, c, npc, qmin, qmax):
 
 
 def _check_sums(got, want, x, g, c, npc, scale, offset, qmin, qmax, oracle):
-    # magnitude of what was summed: the same terms with |grad|
-    _, mag_s, mag_o = oracle.v2_qdq_bwd_params(x, np.abs(g), c, npc, scale, offset, qmin, qmax)
-    for k, (a, b, m) in enumerate(zip(got, want, (np.abs(mag_s) + 1.0, np.abs(mag_o) + 1e-3))):
+    # the yardstick of the tolerance: per channel, the sum of the magnitudes of the terms that were added
+    xs = x.astype(np.float64).reshape(-1, c, npc)
+    ga = np.abs(g.astype(np.float64)).reshape(-1, c, npc)
+    s, o = scale.astype(np.float64).reshape(1, c, 1), offset.astype(np.float64).reshape(1, c, 1)
+    with np.errstate(all="ignore"):
+        q = xs / s
+        r = np.rint(q)
+        mask = (qmin <= r - o) & (r - o <= qmax)
+        mag_s = np.nansum(ga * np.abs(np.clip(r, o + qmin, o + qmax) - np.where(mask, q, 0.0)), axis=(0, 2))
+        mag_o = np.nansum(ga * np.where(mask, 0.0, s), axis=(0, 2))
+    for k, (a, b, m) in enumerate(zip(got, want, (mag_s + 1e-3, mag_o + 1e-6))):
         assert np.all(np.abs(a.astype(np.float64) - b) <= 2e-5 * m), (k, np.abs(a - b).max(), m.min())
 
 
@@ -47,6 +55,13 @@ def _check_sums(got, want, x, g, c, npc, scale, offset, qmin, qmax, oracle):
     (1, 64, 1030),         # rows that are no multiple of the vector width
     (8, 32, 784),          # activations per channel: the sums run over the outer dimension
     (3, 7, 5),             # tiny rows
+    (1, 4096, 128),        # blockwise weight: 32 lanes per row, sums stored directly
+    (1, 8192, 64),         # 16 lanes per row
+    (1, 1000, 16),         # 4 lanes per row, row count no multiple of the rows per workgroup
+    (5, 300, 36),          # 3x3 kernels of 4 input channels, activations-style outer dimension
+    (1, 333, 9),           # odd rows: one element per lane
+    (2, 40, 2048),         # the longest row the lane-group kernel takes
+    (2, 40, 2052),         # the shortest row the workgroup kernel takes
     (1, 3, 8192 + 2048 + 4),   # last span of a row much shorter than the others
 ])
 def test_bwd_params_matches_oracle(ops, oracle, qmin, qmax, outer, c, npc):
@@ -72,8 +87,8 @@ def test_bwd_params_is_deterministic(ops):
     assert all(torch.equal(u, v) for u, v in zip(a, b))
 
 
-def test_bwd_params_bf16(ops, oracle):
-    c, npc = 48, 2048
+@pytest.mark.parametrize("c,npc", [(48, 2048), (24, 4096), (512, 64), (100, 24)])
+def test_bwd_params_bf16(ops, oracle, c, npc):
     x, g, scale, offset = _case(11, 1, c, npc, -128, 127)
     xb, gb = torch.from_numpy(x).to(torch.bfloat16), torch.from_numpy(g).to(torch.bfloat16)
     gin, sg, og = ops.v2_qdq_bwd_params(xb.cuda(), gb.cuda(), c, npc, _gpu(scale), _gpu(offset), -128, 127)
