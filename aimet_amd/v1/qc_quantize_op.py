@@ -1,9 +1,10 @@
 """Quantization wrappers of the v1 path.
 
 Mirrors TrainingExtensions/torch/src/python/aimet_torch/v1/qc_quantize_op.py: QcQuantizeOpMode (:63-70),
-tensor_quantizer_factory (:80-112), QcQuantizeWrapper (:198-496), StaticGridQuantWrapper (:679-924) and
-SteGatingFuncForParameters (:1314-1366).  The wrapper decides *which* tensors are quantized and when
-(ANALYSIS = update statistics, ACTIVE = quantize-dequantize); the arithmetic is in the HIP kernels.
+tensor_quantizer_factory (:80-112), QcQuantizeWrapper (:198-496), StaticGridQuantWrapper (:679-924),
+LearnedGridQuantWrapper (:947-1196), SteGatingFuncForParameters (:1314-1366) and FusedQdqLinear (:1446-1504).  The
+wrapper decides *which* tensors are quantized and when (ANALYSIS = update statistics, ACTIVE = quantize-dequantize);
+the arithmetic is in the HIP kernels.
 
 One mechanical difference: the original parameters are kept by reference and swapped back after the wrapped module
 has run, instead of cloned and copied back (two fewer passes over every weight per forward); at backward time the
@@ -19,7 +20,8 @@ from torch import nn
 from ..common import libpymo
 from ..common.defs import QuantizationDataType, QuantScheme
 from . import quantsim_straight_through_grad as ste
-from .tensor_quantizer import StaticGridPerChannelQuantizer, StaticGridPerTensorQuantizer
+from .tensor_quantizer import (LearnedGridTensorQuantizer, StaticGridPerChannelQuantizer,
+                               StaticGridPerTensorQuantizer, set_encoding_min_max_gating_threshold)
 
 
 class QcQuantizeOpMode(Enum):
@@ -45,10 +47,15 @@ def _to_round_mode(round_mode):
 
 def tensor_quantizer_factory(bitwidth: int, round_mode, quant_scheme: QuantScheme, use_symmetric_encodings: bool,
                              enabled_by_default: bool, data_type: QuantizationDataType = QuantizationDataType.int):
-    """Instantiates the tensor quantizer for `quant_scheme` (post-training schemes; range learning is not built)."""
+    """Instantiates the tensor quantizer for `quant_scheme`: static grid for the post-training schemes, learned grid
+    for the range-learning schemes (reference :80-112)."""
     if quant_scheme in (QuantScheme.post_training_tf_enhanced, QuantScheme.post_training_tf):
         return StaticGridPerTensorQuantizer(bitwidth, _to_round_mode(round_mode), quant_scheme,
                                             use_symmetric_encodings, enabled_by_default, data_type=data_type)
+    if quant_scheme in (QuantScheme.training_range_learning_with_tf_init,
+                        QuantScheme.training_range_learning_with_tf_enhanced_init):
+        return LearnedGridTensorQuantizer(bitwidth, _to_round_mode(round_mode), quant_scheme,
+                                          use_symmetric_encodings, enabled_by_default, data_type)
     raise AssertionError("Unsupported quant_scheme: " + str(quant_scheme))
 
 
@@ -243,3 +250,218 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
             pc.use_unsigned_symmetric = q.use_unsigned_symmetric
             new_param_quant_dict[param_name] = pc
         self.param_quantizers = new_param_quant_dict
+
+
+# ------------------------------------------------------------------------------------------------- range learning
+_ENABLE_RECOMPUTE = False
+
+
+class _Handle:
+    """Undoes a temporary change when closed or when the `with` block ends."""
+
+    def __init__(self, cleanup_fn):
+        self._cleanup_fn, self._done = cleanup_fn, False
+
+    def remove(self):
+        if not self._done:
+            self._cleanup_fn()
+            self._done = True
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *_):
+        self.remove()
+
+
+def _set_enable_recompute(mode: bool) -> _Handle:
+    global _ENABLE_RECOMPUTE  # pylint: disable=global-statement
+    original = _ENABLE_RECOMPUTE
+
+    def cleanup():
+        global _ENABLE_RECOMPUTE  # pylint: disable=global-statement
+        _ENABLE_RECOMPUTE = original
+    _ENABLE_RECOMPUTE = mode
+    return _Handle(cleanup)
+
+
+def is_recompute_enabled() -> bool:
+    """True if the quantize-dequantized weight of fused layers is recomputed in backward instead of kept."""
+    return _ENABLE_RECOMPUTE
+
+
+def enable_recompute() -> _Handle:
+    return _set_enable_recompute(True)
+
+
+def disable_recompute() -> _Handle:
+    return _set_enable_recompute(False)
+
+
+class LearnedGridQuantWrapper(QcQuantizeWrapper):
+    """Wrapper whose enabled quantizers learn their encoding min / max (reference :947-1170).  The min / max of every
+    quantizer are parameters of this module, named input<i>_encoding_min/max, output<i>_encoding_min/max and
+    <param>_encoding_min/max; they stay None until an encoding is assigned."""
+
+    # pylint: disable=too-many-arguments
+    def __init__(self, module_to_wrap: nn.Module, weight_bw: int, activation_bw: int, round_mode,
+                 quant_scheme: QuantScheme, device: torch.device, is_output_quantized: bool = True,
+                 is_symmetric: bool = False, num_inputs=1, num_outputs=1,
+                 data_type: QuantizationDataType = QuantizationDataType.int):
+        if data_type != QuantizationDataType.int:
+            raise ValueError('Only QuantizationDataType.int is supported for LearnedGridQuantWrapper')
+        super().__init__(module_to_wrap, weight_bw, activation_bw, round_mode, quant_scheme, is_output_quantized,
+                         is_symmetric, num_inputs, num_outputs, data_type)
+        self.device = device
+        self._initialize_trainable_parameters_and_tensor_quantizers(num_inputs, num_outputs)
+
+    def _initialize_trainable_parameters_and_tensor_quantizers(self, num_inputs, num_outputs):
+        def attach(quantizer, name):
+            self.register_parameter(name + '_encoding_min', None)
+            self.register_parameter(name + '_encoding_max', None)
+            quantizer.name, quantizer.wrapper_ref, quantizer.device = name, self, self.device
+
+        for index in range(num_inputs):
+            attach(self.input_quantizers[index], 'input' + str(index))
+        for index in range(num_outputs):
+            attach(self.output_quantizers[index], 'output' + str(index))
+        transposed = isinstance(self._module_to_wrap, (nn.ConvTranspose1d, nn.ConvTranspose2d, nn.ConvTranspose3d))
+        for name, param in self.get_named_parameters():
+            attach(self.param_quantizers[name], name)
+            # pylint: disable=protected-access
+            self.param_quantizers[name]._ch_axis = 1 if transposed and len(param.shape) > 1 else 0
+
+    def _named_quantizers(self):
+        for index, quantizer in enumerate(self.input_quantizers):
+            yield 'input' + str(index), quantizer
+        for index, quantizer in enumerate(self.output_quantizers):
+            yield 'output' + str(index), quantizer
+        for name, _ in self._module_to_wrap.named_parameters():
+            yield name, self.param_quantizers[name]
+
+    def apply_gating_logic(self):
+        """Keeps every learned range ordered around zero before it is used (min <= 0 <= max, max > min)."""
+        for name, quantizer in self._named_quantizers():
+            if quantizer.enabled and quantizer.bitwidth != 32 and quantizer.data_type != QuantizationDataType.float:
+                set_encoding_min_max_gating_threshold(getattr(self, name + '_encoding_min'),
+                                                      getattr(self, name + '_encoding_max'))
+
+    def forward(self, *inputs, **kwargs):
+        self.apply_gating_logic()
+        quantized_inputs = self._quantize_activation(list(inputs), self.input_quantizers, 'input')
+        forward_fn = _default_forward
+        if torch.is_grad_enabled() and is_recompute_enabled():
+            forward_fn = _fused_forward_functions.get(type(self._module_to_wrap), _default_forward)
+        wrapped_output = forward_fn(self, quantized_inputs, **kwargs)
+        if not isinstance(wrapped_output, (List, Tuple)):
+            wrapped_output = [wrapped_output]
+        output = self._quantize_activation(list(wrapped_output), self.output_quantizers, 'output')
+        return output[0] if len(output) == 1 else output
+
+    def _quantize_params(self) -> _Handle:
+        """Puts the quantize-dequantized parameters in the wrapped module's place until the handle is closed.  The
+        replacements are results of an autograd function, so gradients reach the original parameter and the
+        encoding min / max."""
+        params = self._module_to_wrap._parameters  # pylint: disable=protected-access
+        originals = {}
+
+        def cleanup():
+            for name, original in originals.items():
+                params[name] = original
+
+        try:
+            for name, _ in self.get_named_parameters():
+                quantizer = self.param_quantizers[name]
+                if not quantizer.enabled:
+                    continue
+                original = params[name]
+                quantized = quantizer.quantize_dequantize(original, getattr(self, name + '_encoding_min'),
+                                                          getattr(self, name + '_encoding_max'))
+                originals[name] = original
+                params[name] = quantized
+            return _Handle(cleanup)
+        except Exception:
+            cleanup()
+            raise
+
+    def _quantize_activation(self, tensors_to_quantize, tensor_quantizers, type_of_quantizer: str) -> List:
+        def inner(tensor, index):
+            if isinstance(tensor, (List, Tuple)):
+                return [inner(t, index) for t in tensor]
+            if not isinstance(tensor, torch.Tensor) or \
+                    not self.should_perform_quant_dequant(tensor, tensor_quantizers[index]):
+                return tensor
+            encoding_min = getattr(self, type_of_quantizer + str(index) + '_encoding_min')
+            encoding_max = getattr(self, type_of_quantizer + str(index) + '_encoding_max')
+            return tensor_quantizers[index].quantize_dequantize(tensor, encoding_min, encoding_max)
+
+        outputs = []
+        for index, tensor in enumerate(tensors_to_quantize):
+            assert len(tensor_quantizers) > index, f"Not enough tensor quantizers ({len(tensor_quantizers)}) allocated"
+            outputs.append(inner(tensor, index))
+        return outputs
+
+
+def _default_forward(quant_wrapper: LearnedGridQuantWrapper, inputs, **kwargs):
+    # pylint: disable=protected-access
+    with quant_wrapper._quantize_params():
+        return quant_wrapper._module_to_wrap(*inputs, **kwargs)
+
+
+def _linear_forward_with_recompute(quant_wrapper: LearnedGridQuantWrapper, inputs, **kwargs):
+    """nn.Linear without keeping the quantize-dequantized weight for backward (reference :1175-1196)."""
+    # pylint: disable=protected-access
+    if not quant_wrapper.param_quantizers['weight'].enabled or kwargs or len(inputs) != 1:
+        return _default_forward(quant_wrapper, inputs, **kwargs)
+    module = quant_wrapper._module_to_wrap
+    return FusedQdqLinear.apply(inputs[0], module.weight, module.bias, quant_wrapper.weight_encoding_min,
+                                quant_wrapper.weight_encoding_max, quant_wrapper.param_quantizers['weight'])
+
+
+_fused_forward_functions = {nn.Linear: _linear_forward_with_recompute}
+
+
+class FusedQdqLinear(torch.autograd.Function):
+    """Linear layer on a range-learned weight that saves the original weight only: backward recomputes the
+    quantize-dequantized weight for the input gradient (one kernel) and gets the weight gradient and the encoding
+    gradients from one pass over (weight, dL/dWq) (reference :1446-1504)."""
+
+    @staticmethod
+    def forward(ctx, inp, weight, bias, weight_encoding_min, weight_encoding_max, weight_quantizer):
+        # pylint: disable=arguments-differ
+        ctx.save_for_backward(inp, weight, bias, weight_encoding_min.detach().clone(),
+                              weight_encoding_max.detach().clone())
+        ctx.weight_quantizer = weight_quantizer
+        qdq_weight, _ = ste.learned_grid_forward(weight, weight_quantizer, weight_encoding_min, weight_encoding_max)
+        return torch.nn.functional.linear(inp, qdq_weight, bias)
+
+    @staticmethod
+    def backward(ctx, grad):  # pylint: disable=arguments-differ
+        inp, weight, bias, encoding_min, encoding_max = ctx.saved_tensors
+        quantizer = ctx.weight_quantizer
+        need_x, need_w, need_b, need_min, need_max = ctx.needs_input_grad[:5]
+        dloss_by_dx = dloss_by_dw = dloss_by_db = dloss_by_dmin = dloss_by_dmax = None
+        saved = None
+        if need_x:
+            qdq_weight, saved = ste.learned_grid_forward(weight, quantizer, encoding_min, encoding_max)
+            dloss_by_dx = torch.matmul(grad, qdq_weight)
+            del qdq_weight
+        if need_w or need_min or need_max:
+            if saved is None:
+                delta, offset, _ = ste.get_computed_encodings(quantizer.bitwidth, encoding_min.float(),
+                                                              encoding_max.float(),
+                                                              quantizer.use_symmetric_encodings,
+                                                              quantizer.use_strict_symmetric,
+                                                              quantizer.is_unsigned_symmetric)
+                saved = (delta, offset, ste._num_steps(quantizer),  # pylint: disable=protected-access
+                         *ste._channel_geometry(weight, delta.numel(), quantizer.channel_axis))
+            dloss_by_dwq = torch.matmul(grad.reshape(-1, grad.shape[-1]).t(), inp.reshape(-1, inp.shape[-1]))
+            dloss_by_dw, dloss_by_dmin, dloss_by_dmax = ste.learned_grid_backward(
+                weight, dloss_by_dwq, saved, encoding_min, encoding_max, quantizer.use_symmetric_encodings,
+                need_w, need_min or need_max)
+            if not need_w:
+                dloss_by_dw = None
+        if need_b and isinstance(bias, torch.Tensor):
+            dloss_by_db = grad.reshape(-1, grad.shape[-1]).sum(dim=0)
+        return dloss_by_dx, dloss_by_dw, dloss_by_db, dloss_by_dmin if need_min else None, \
+            dloss_by_dmax if need_max else None, None

@@ -21,7 +21,9 @@ from torch import nn
 
 from ..common.defs import QuantizationDataType, QuantScheme
 from .nn.modules import custom
-from .qc_quantize_op import QcQuantizeOpMode, QcQuantizeWrapper, StaticGridQuantWrapper
+from .qc_quantize_op import LearnedGridQuantWrapper, QcQuantizeOpMode, QcQuantizeWrapper, StaticGridQuantWrapper
+from .tensor_quantizer import (LearnedGridTensorQuantizer, StaticGridPerChannelQuantizer,
+                               initialize_learned_grid_quantizer_attributes)
 
 # same rules as the reference's aimet_common/quantsim_config/default_config.json
 DEFAULT_CONFIG = {
@@ -72,6 +74,24 @@ def _flag(d: dict, key: str, default=None):
     return str(d[key]) == "True"
 
 
+_INIT_SCHEME = {
+    QuantScheme.post_training_tf: QuantScheme.post_training_tf,
+    QuantScheme.post_training_tf_enhanced: QuantScheme.post_training_tf_enhanced,
+    QuantScheme.training_range_learning_with_tf_init: QuantScheme.post_training_tf,
+    QuantScheme.training_range_learning_with_tf_enhanced_init: QuantScheme.post_training_tf_enhanced,
+}
+
+
+def _exported_encoding(quantizer):
+    """The encoding a quantizer is exported with: learned-grid quantizers report the one their quant scheme means
+    (reference get_encoding_by_quantizer, qc_quantize_op.py:1507-1519)."""
+    if not quantizer.enabled:
+        return None
+    if isinstance(quantizer, LearnedGridTensorQuantizer):
+        return quantizer.get_effective_encoding()
+    return quantizer.encoding
+
+
 class QuantizationSimModel:
     """Adds quantization simulation ops to a model for off-target simulation of quantized inference accuracy."""
 
@@ -84,8 +104,9 @@ class QuantizationSimModel:
         if isinstance(quant_scheme, str):
             quant_scheme = {'tf': QuantScheme.post_training_tf,
                             'tf_enhanced': QuantScheme.post_training_tf_enhanced}[quant_scheme]
-        if quant_scheme not in (QuantScheme.post_training_tf, QuantScheme.post_training_tf_enhanced):
-            raise ValueError(f"quant_scheme {quant_scheme} is not implemented (tf and tf_enhanced are)")
+        if quant_scheme not in _INIT_SCHEME:
+            raise ValueError(f"quant_scheme {quant_scheme} is not implemented (tf, tf_enhanced and the two "
+                             "range-learning schemes initialised from them are)")
         if rounding_mode not in ('nearest', 'stochastic'):
             raise ValueError('Parameter round mode can only be nearest or stochastic')
         if default_param_bw < 4 or default_param_bw > 32 or default_output_bw < 4 or default_output_bw > 32:
@@ -168,9 +189,11 @@ class QuantizationSimModel:
                 raise RuntimeError(f"module {rec['name']} is used more than once in the forward pass; "
                                    "give each use its own module")
             seen.add(rec["name"])
+            # range-learning schemes start as static-grid wrappers of the scheme they are initialised from and are
+            # swapped for learned-grid wrappers once encodings have been computed
             wrapper = StaticGridQuantWrapper(rec["module"], self._default_param_bw, self._default_output_bw,
-                                             self._rounding_mode, self._quant_scheme, num_inputs=rec["num_inputs"],
-                                             num_outputs=rec["num_outputs"])
+                                             self._rounding_mode, _INIT_SCHEME[self._quant_scheme],
+                                             num_inputs=rec["num_inputs"], num_outputs=rec["num_outputs"])
             rec["wrapper"] = wrapper
             parent = self.model
             *path, leaf = rec["name"].split('.')
@@ -259,7 +282,8 @@ class QuantizationSimModel:
     def compute_encodings(self, forward_pass_callback, forward_pass_callback_args):
         """Runs `forward_pass_callback(model, args)` in ANALYSIS mode, then computes every encoding and switches the
         wrappers to ACTIVE (reference :425-448)."""
-        layers = self._get_qc_quantized_layers(self.model)
+        layers = [(n, m) for n, m in self._get_qc_quantized_layers(self.model)
+                  if isinstance(m, StaticGridQuantWrapper)]
         for _, layer in layers:
             layer.reset_encodings()
             layer.set_mode(QcQuantizeOpMode.ANALYSIS)
@@ -273,6 +297,49 @@ class QuantizationSimModel:
         for _, layer in layers:
             layer.compute_encoding()
             layer.set_mode(QcQuantizeOpMode.ACTIVE)
+        self.replace_wrappers_for_quantize_dequantize()
+
+    def replace_wrappers_for_quantize_dequantize(self):
+        """For the range-learning schemes: every static-grid wrapper becomes a learned-grid wrapper that starts from
+        the calibrated encodings (reference quantsim.py:764-847)."""
+        if self._quant_scheme not in (QuantScheme.training_range_learning_with_tf_init,
+                                      QuantScheme.training_range_learning_with_tf_enhanced_init):
+            return
+        try:
+            device = next(self.model.parameters()).device
+        except StopIteration:
+            device = torch.device('cuda', torch.cuda.current_device())
+        replaced = {}
+        self._replace_quantization_wrapper(self.model, device, replaced)
+        for rec in self._graph:
+            rec["wrapper"] = replaced.get(rec["wrapper"], rec["wrapper"])
+
+    def _replace_quantization_wrapper(self, model: nn.Module, device, replaced: dict):
+        for name, child in list(model.named_children()):
+            if isinstance(child, StaticGridQuantWrapper):
+                replaced[child] = self._construct_and_initialize_trainable_wrapper(child, device)
+                setattr(model, name, replaced[child])
+            elif not isinstance(child, QcQuantizeWrapper):
+                self._replace_quantization_wrapper(child, device, replaced)
+
+    def _construct_and_initialize_trainable_wrapper(self, post_training_module: StaticGridQuantWrapper,
+                                                    device) -> LearnedGridQuantWrapper:
+        # pylint: disable=protected-access
+        trainable = LearnedGridQuantWrapper(post_training_module._module_to_wrap, self._default_param_bw,
+                                            self._default_output_bw, self._rounding_mode, self._quant_scheme,
+                                            device=device, num_inputs=len(post_training_module.input_quantizers),
+                                            num_outputs=len(post_training_module.output_quantizers),
+                                            data_type=QuantizationDataType.int)
+        pairs = list(zip(trainable.output_quantizers, post_training_module.output_quantizers)) + \
+            list(zip(trainable.input_quantizers, post_training_module.input_quantizers)) + \
+            [(trainable.param_quantizers[n], q) for n, q in post_training_module.param_quantizers.items()]
+        for new, old in pairs:
+            if isinstance(old, StaticGridPerChannelQuantizer):
+                new._ch_axis = old.channel_axis
+            initialize_learned_grid_quantizer_attributes(new, old)
+            if new.encoding_min_max_fixed_vals is not None:
+                new.freeze_encoding()
+        return trainable
 
     def exclude_layers_from_quantization(self, layers_to_exclude: List[nn.Module]):
         """Replaces the given quantization wrappers by the modules they wrap (reference quantsim.py:1419-1433)."""
@@ -303,14 +370,16 @@ class QuantizationSimModel:
         param_enc, act_enc = {}, {}
         for name, w in self.quant_wrappers():
             for pname, q in w.param_quantizers.items():
-                if q.enabled and q.encoding is not None:
-                    encs = q.encoding if isinstance(q.encoding, list) else [q.encoding]
+                encoding = _exported_encoding(q)
+                if encoding is not None:
+                    encs = encoding if isinstance(encoding, list) else [encoding]
                     param_enc[f"{name}.{pname}"] = [self._encoding_dict(e, q.use_symmetric_encodings) for e in encs]
             entry = {}
             for kind, qs in (('input', w.input_quantizers), ('output', w.output_quantizers)):
                 for i, q in enumerate(qs):
-                    if q.enabled and q.encoding is not None:
-                        entry.setdefault(kind, {})[str(i)] = self._encoding_dict(q.encoding,
+                    encoding = _exported_encoding(q)
+                    if encoding is not None:
+                        entry.setdefault(kind, {})[str(i)] = self._encoding_dict(encoding,
                                                                                  q.use_symmetric_encodings)
             if entry:
                 act_enc[name] = entry

@@ -3,8 +3,15 @@
 compute_dloss_by_dx mirrors TrainingExtensions/torch/src/python/aimet_torch/v1/quantsim_straight_through_grad.py:91-118:
 grad * ((encoding_min <= x) & (x <= encoding_max)), one fused kernel instead of three elementwise passes and a bool
 temporary.
+
+Range learning (:121-346): get_computed_encodings, the quantize-dequantize forward and the gradients w.r.t. the input
+and the learnable encoding min / max.  The reference keeps x_quant, delta, offset and a bool mask at full tensor size
+for backward and forms the encoding gradients from five more full-size products; here forward is one kernel, and
+backward is one kernel that re-derives grid position and mask from the saved input and returns the input gradient
+together with the two per-channel sums the encoding gradients are made of.
 """
 import functools
+import math
 
 import torch
 
@@ -45,3 +52,99 @@ def compute_dloss_by_dx(x, grad, encoding_min, encoding_max, ch_axis=0):
     assert mn.numel() == num_channel and mx.numel() == num_channel
     n_per_channel = functools.reduce(lambda a, b: a * b, x.shape[ch_axis + 1:], 1)
     return ops.ste_bwd_per_channel(x, grad, num_channel, n_per_channel, mn, mx)
+
+
+# ------------------------------------------------------------------------------------------------- range learning
+def get_computed_encodings(bitwidth, encoding_min, encoding_max, use_symmetric_encodings, use_strict_symmetric,
+                           is_unsigned_symmetric):
+    """(delta, offset, num_steps) from learnable encoding min / max tensors (reference :121-162, which follows the
+    C++ getComputedEncodings): signed symmetric -> delta = max / floor(steps / 2), offset = -ceil(steps / 2);
+    unsigned symmetric -> delta = (max - min) / steps, offset = min / delta; asymmetric -> the zero point
+    round(-min / delta) clamped to the grid."""
+    num_steps = 2 ** bitwidth - 1
+    if use_symmetric_encodings and use_strict_symmetric:
+        num_steps -= 1
+    half = num_steps / 2
+    steps = torch.full_like(encoding_min, float(num_steps))
+    if use_symmetric_encodings and not is_unsigned_symmetric:
+        delta = encoding_max / float(math.floor(half))
+        offset = torch.full_like(encoding_min, -float(math.ceil(half)))
+    else:
+        delta = (encoding_max - encoding_min) / steps
+        if use_symmetric_encodings:
+            offset = encoding_min / delta
+        else:
+            offset = -torch.clamp(torch.round(-encoding_min / delta), 0.0, float(num_steps))
+    return delta, offset, steps
+
+
+def _channel_geometry(tensor, num_param, ch_axis):
+    if num_param == 1:
+        return 1, max(tensor.numel(), 1)
+    assert num_param == tensor.shape[ch_axis]
+    return num_param, max(math.prod(tensor.shape[ch_axis + 1:]), 1)
+
+
+def learned_grid_forward(tensor, tensor_quantizer, encoding_min, encoding_max):
+    """Forward of range learning (reference calculate_forward_pass :185-249):
+    x_dequant = (clamp(round(x / delta) - offset, 0, steps) + offset) * delta, in one kernel.  Returns the output and
+    what backward needs (delta, offset, steps) -- no full-size intermediates are kept: the backward kernel recomputes
+    the grid position and the mask from the saved input."""
+    if tensor.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        raise RuntimeError("Invalid input data type. Expected torch.float32 or torch.float16. "
+                           f"Got {tensor.dtype}.")
+    if not tensor.dtype == encoding_min.dtype == encoding_max.dtype:
+        raise RuntimeError("Data type mismatch. Expected the input and encoding min & max to be of same dtype."
+                           f"Got {tensor.dtype} input, {encoding_min.dtype} encoding_min, "
+                           f"and {encoding_max.dtype} encoding_max")
+    if tensor_quantizer.bitwidth >= 32:
+        raise RuntimeError(f'Invalid bitwidth: {tensor_quantizer.bitwidth}')
+    delta, offset, steps = get_computed_encodings(tensor_quantizer.bitwidth, encoding_min.detach().float(),
+                                                  encoding_max.detach().float(),
+                                                  tensor_quantizer.use_symmetric_encodings,
+                                                  tensor_quantizer.use_strict_symmetric,
+                                                  tensor_quantizer.is_unsigned_symmetric)
+    num_steps = _num_steps(tensor_quantizer)
+    c, npc = _channel_geometry(tensor, delta.numel(), tensor_quantizer.channel_axis)
+    x = tensor if tensor.dtype != torch.float16 else tensor.float()
+    out = ops.v2_qdq(x, c, npc, delta, offset, 0, num_steps)
+    return out.to(tensor.dtype), (delta, offset, num_steps, c, npc)
+
+
+def _num_steps(tensor_quantizer) -> int:
+    n = 2 ** tensor_quantizer.bitwidth - 1
+    if tensor_quantizer.use_symmetric_encodings and tensor_quantizer.use_strict_symmetric:
+        n -= 1
+    return n
+
+
+def learned_grid_backward(tensor, grad, saved, encoding_min, encoding_max, is_symmetric, want_tensor_grad,
+                          want_encoding_grads):
+    """Backward of range learning (reference asymmetric_gradients :253-297, symmetric_gradients :301-331).  One pass
+    over (tensor, grad) yields grad * mask and, per channel, S = sum(grad * (x_quant + offset - x * mask / delta)) and
+    O = sum(delta * grad * ~mask); then
+
+        asymmetric:  t1 = S / steps, t2 = steps / (max - min)^2 * O
+                     d/dmin = -t1 + max * t2,  d/dmax = t1 - min * t2
+        symmetric:   d/dmax = S / floor(steps / 2),  d/dmin = -d/dmax
+    """
+    delta, offset, num_steps, c, npc = saved
+    x = tensor if tensor.dtype != torch.float16 else tensor.float()
+    g = grad.to(x.dtype)
+    if not want_encoding_grads:
+        return ops.v2_qdq_bwd(x, g, c, npc, delta, offset, 0, num_steps).to(tensor.dtype), None, None
+    tensor_grad, s_sum, o_sum = ops.v2_qdq_bwd_params(x, g, c, npc, delta, offset, 0, num_steps,
+                                                      want_grad_in=want_tensor_grad)
+    if tensor_grad is not None:
+        tensor_grad = tensor_grad.to(tensor.dtype)
+    emin, emax = encoding_min.detach().float().reshape(-1), encoding_max.detach().float().reshape(-1)
+    if is_symmetric:
+        grad_max = s_sum / float(num_steps // 2)
+        grad_min = -grad_max
+    else:
+        term1 = s_sum / float(num_steps)
+        term2 = float(num_steps) / (emax - emin) ** 2 * o_sum
+        grad_min = -term1 + emax * term2
+        grad_max = term1 - emin * term2
+    return (tensor_grad, grad_min.to(encoding_min.dtype).view_as(encoding_min),
+            grad_max.to(encoding_max.dtype).view_as(encoding_max))

@@ -1,9 +1,10 @@
-"""v1 static-grid tensor quantizers.
+"""v1 tensor quantizers: static grid (post-training) and learned grid (range learning).
 
 Mirrors TrainingExtensions/torch/src/python/aimet_torch/v1/tensor_quantizer.py (TensorQuantizer :61-123,
 StaticGridTensorQuantizer :143-395, StaticGridPerTensorQuantizer :398-480, StaticGridPerChannelQuantizer :483-570,
-autograd functions QuantizeDequantize / Quantize :1098-1277): same class names, attributes, method names and
-semantics.  What differs is below the interface:
+autograd functions QuantizeDequantize / Quantize :1098-1277; LearnedGridTensorQuantizer :573-895,
+QuantizeDequantizeFunc :898-986, initialize_learned_grid_quantizer_attributes :1285-1345): same class names,
+attributes, method names and semantics.  What differs is below the interface:
 
 * per-channel quantizers keep their per-channel (min, max, delta, offset) as four device vectors built once per
   encoding, instead of rebuilding a host vector and copying it to the device on every forward;
@@ -15,6 +16,7 @@ semantics.  What differs is below the interface:
 """
 import functools
 import io
+import math
 from typing import List, Optional, Tuple, Union
 
 import torch
@@ -371,3 +373,239 @@ class Quantize(torch.autograd.Function):
     @staticmethod
     def backward(ctx, _output_grad):  # pylint: disable=arguments-differ
         raise AssertionError('Backward pass for quantize only not implemented')
+
+
+# ------------------------------------------------------------------------------------------------- range learning
+def is_non_strict_symmetric(use_symmetric_encodings: bool, use_strict_symmetric: bool,
+                            is_unsigned_symmetric: bool) -> bool:
+    return use_symmetric_encodings and not use_strict_symmetric and not is_unsigned_symmetric
+
+
+class LearnedGridTensorQuantizer(TensorQuantizer):
+    """Quantization simulation whose encoding min / max are parameters of the owning wrapper, initialised from a
+    calibrated encoding and then learned (reference :573-895).  The wrapper holds the parameters under
+    '<name>_encoding_min' / '<name>_encoding_max'; this object holds the configuration and computes encodings from
+    them."""
+
+    # pylint: disable=too-many-instance-attributes
+    def __init__(self, bitwidth: int, round_mode, quant_scheme: QuantScheme, use_symmetric_encodings: bool,
+                 enabled_by_default: bool, data_type: QuantizationDataType = QuantizationDataType.int):
+        if data_type != QuantizationDataType.int:
+            raise ValueError('Only QuantizationDataType.int is supported for LearnedGridTensorQuantizer')
+        super().__init__(bitwidth, round_mode, quant_scheme, use_symmetric_encodings, enabled_by_default, data_type)
+        self.wrapper_ref = None
+        self.name = None
+        self.scaling, self.offset = None, None
+        self.device = None
+        self._ch_axis = 0
+
+    @staticmethod
+    def get_n_and_p(bitwidth: int, use_symmetric_encoding: bool, use_strict_symmetric: bool, device=None):
+        """Grid bounds n = 0 and p = 2^bitwidth - 1 (one less for strict symmetric) as tensors."""
+        if not use_symmetric_encoding and use_strict_symmetric:
+            raise ValueError("Strict symmetric can be enabled only when using symmetric encoding")
+        p = 2.0 ** bitwidth - 1
+        if use_symmetric_encoding and use_strict_symmetric:
+            p -= 1
+        return torch.tensor([0.0], device=device), torch.tensor([p], device=device)
+
+    def n(self, device=None) -> torch.Tensor:
+        return self.get_n_and_p(self.bitwidth, self.use_strict_symmetric, self.use_strict_symmetric,
+                                device or self.device)[0]
+
+    def p(self, device=None) -> torch.Tensor:
+        return self.get_n_and_p(self.bitwidth, self.use_strict_symmetric, self.use_strict_symmetric,
+                                device or self.device)[1]
+
+    def _parameters_of_wrapper(self):
+        return getattr(self.wrapper_ref, self.name + '_encoding_min'), \
+            getattr(self.wrapper_ref, self.name + '_encoding_max')
+
+    def get_effective_encoding(self):
+        """The encoding as the user's quant scheme means it: non-strict symmetric quantizers learn with max == -min
+        and report min one step lower (reference :642-686)."""
+        if not self.enabled:
+            return None
+        encodings = self.encoding
+        if not encodings:
+            return None
+        if isinstance(encodings, libpymo.TfEncoding):
+            encodings = [encodings]
+        if is_non_strict_symmetric(self.use_symmetric_encodings, self.use_strict_symmetric,
+                                   self.is_unsigned_symmetric):
+            encodings = [libpymo.TfEncoding(e.min - e.delta, e.max, e.delta, e.offset, e.bw) for e in encodings]
+        return encodings[0] if len(encodings) == 1 else encodings
+
+    @property
+    def encoding(self):
+        """The learned encoding(s), recomputed from the current min / max parameters."""
+        if not self.enabled or self.bitwidth == 32 or self.data_type == QuantizationDataType.float:
+            return None
+        return self._compute_updated_encoding()
+
+    @encoding.setter
+    def encoding(self, encoding):
+        if not self.enabled or self.bitwidth == 32 or self.data_type == QuantizationDataType.float:
+            return
+        if encoding is None:
+            raise RuntimeError("Encodings cannot be None if Quantizer is enabled.")
+        bitwidth = encoding[0].bw if isinstance(encoding, list) else encoding.bw
+        if bitwidth != self.bitwidth:
+            raise RuntimeError(
+                f"Bitwidth mismatched. The bitwidth for quantizer is {self.bitwidth}, but the bitwidth in encodings "
+                f"is {bitwidth}. If the intent is to change the bitwidth, please set quantizer bitwidth to "
+                f"{bitwidth} first.")
+        if self._is_encoding_frozen:
+            raise RuntimeError("Encoding can be set only when it is not frozen.")
+        self._set_encoding_min_max_parameters(encoding)
+
+    @property
+    def channel_axis(self) -> int:
+        return self._ch_axis
+
+    @TensorQuantizer.encoding_min_max_fixed_vals.setter
+    def encoding_min_max_fixed_vals(self, min_max_vals: Optional[Tuple[float, float]]):
+        self._encoding_min_max_fixed_vals = min_max_vals
+
+    def __str__(self):
+        stream = io.StringIO(newline='\n')
+        stream.write('LearnedGrid TensorQuantizer:\n')
+        stream.write(f'    quant-scheme:{self._quant_scheme}, round_mode={self.round_mode}, '
+                     f'bitwidth={self.bitwidth}, enabled={self.enabled}\n')
+        encoding = self.get_effective_encoding() if self.encoding else None
+        if encoding:
+            for enc in (encoding if isinstance(encoding, list) else [encoding]):
+                stream.write(f'    min:{enc.min}, max={enc.max}, delta={enc.delta}, offset={enc.offset}\n')
+        else:
+            stream.write('    no encoding\n')
+        return stream.getvalue()
+
+    def compute_scaling_offset(self, encoding_min, encoding_max):
+        """(delta, offset) tensors for the given min / max tensors; (None, None) when they are None."""
+        if encoding_min is None or encoding_max is None:
+            return None, None
+        scaling, offset, _ = grad_fn.get_computed_encodings(self.bitwidth, encoding_min, encoding_max,
+                                                            self.use_symmetric_encodings, self.use_strict_symmetric,
+                                                            self.is_unsigned_symmetric)
+        return scaling, offset
+
+    def quantize_dequantize(self, tensor: torch.Tensor, encoding_min: torch.nn.Parameter,
+                            encoding_max: torch.nn.Parameter) -> torch.Tensor:
+        if self.enabled:
+            tensor = QuantizeDequantizeFunc.apply(tensor, encoding_min, encoding_max, self)
+        return tensor
+
+    @torch.no_grad()
+    def _compute_updated_encoding(self):
+        encoding_min, encoding_max = self._parameters_of_wrapper()
+        if encoding_min is None or encoding_max is None:
+            return None                       # not initialised yet
+        emin, emax = encoding_min.detach().float(), encoding_max.detach().float()
+        scale, offset = self.compute_scaling_offset(emin, emax)
+        scale, offset = scale.expand_as(emin), offset.expand_as(emin)
+        if not self.use_symmetric_encodings or self.is_unsigned_symmetric:
+            # zero must be representable: min / max follow from delta and the rounded offset (reference :822-831)
+            adjusted_min = scale * offset
+            emax = emax - emin + adjusted_min
+            emin = adjusted_min
+        # one transfer for all channels
+        table = torch.stack([emin, emax, scale, offset]).cpu().tolist()
+        encodings = [libpymo.TfEncoding(mn, mx, d, o, self.bitwidth) for mn, mx, d, o in zip(*table)]
+        return encodings[0] if len(encodings) == 1 else encodings
+
+    def _set_encoding_min_max_parameters(self, encodings):
+        if isinstance(encodings, list):
+            assert isinstance(encodings[0], libpymo.TfEncoding), "Encodings should be a libpymo.TfEncoding() object"
+            mins, maxs = [e.min for e in encodings], [e.max for e in encodings]
+        else:
+            assert isinstance(encodings, libpymo.TfEncoding), "Encodings should be a libpymo.TfEncoding() object"
+            mins, maxs = [encodings.min], [encodings.max]
+        params = self.wrapper_ref._parameters  # pylint: disable=protected-access
+        device = self.wrapper_ref.device
+        params[self.name + '_encoding_min'] = torch.nn.Parameter(torch.tensor(mins, dtype=torch.float32,
+                                                                              device=device))
+        params[self.name + '_encoding_max'] = torch.nn.Parameter(torch.tensor(maxs, dtype=torch.float32,
+                                                                              device=device))
+
+    def freeze_encoding(self):
+        params = self.wrapper_ref._parameters  # pylint: disable=protected-access
+        enc_min, enc_max = params[self.name + '_encoding_min'], params[self.name + '_encoding_max']
+        if enc_min is None and enc_max is None:
+            raise RuntimeError("Encoding can be frozen only when it is not None.")
+        self._is_encoding_frozen = True
+        enc_min.requires_grad = False
+        enc_max.requires_grad = False
+
+
+class QuantizeDequantizeFunc(torch.autograd.Function):
+    """Quantize-dequantize with gradients w.r.t. the tensor and the learnable encoding min / max
+    (reference :898-986).  Only the input tensor and the per-channel delta / offset are kept for backward."""
+
+    @staticmethod
+    def forward(ctx, tensor, encoding_min, encoding_max, tensor_quantizer):  # pylint: disable=arguments-differ
+        ctx.tensor_quantizer = tensor_quantizer
+        if tensor_quantizer.bitwidth == 32:
+            return tensor
+        if encoding_max is None or encoding_min is None:
+            raise RuntimeError("Forward pass used for compute_encodings differs from forward pass used during "
+                               "training")
+        out, saved = grad_fn.learned_grid_forward(tensor, tensor_quantizer, encoding_min, encoding_max)
+        ctx.saved_geometry = saved[2:]
+        ctx.is_symmetric = tensor_quantizer.use_symmetric_encodings
+        # min / max are saved as copies: the wrapper clamps the parameters in place before every forward, also
+        # between the forward and the backward of a module that is used twice (reference :942-955)
+        ctx.save_for_backward(tensor, saved[0], saved[1], encoding_min.detach().clone(),
+                              encoding_max.detach().clone())
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):  # pylint: disable=arguments-differ
+        if ctx.tensor_quantizer.bitwidth == 32:
+            return grad, None, None, None
+        tensor, delta, offset, encoding_min, encoding_max = ctx.saved_tensors
+        want_enc = ctx.needs_input_grad[1] or ctx.needs_input_grad[2]
+        tensor_grad, grad_min, grad_max = grad_fn.learned_grid_backward(
+            tensor, grad, (delta, offset) + tuple(ctx.saved_geometry), encoding_min, encoding_max, ctx.is_symmetric,
+            ctx.needs_input_grad[0], want_enc)
+        if not ctx.needs_input_grad[0]:
+            tensor_grad = None
+        return tensor_grad, grad_min if ctx.needs_input_grad[1] else None, \
+            grad_max if ctx.needs_input_grad[2] else None, None
+
+
+def initialize_learned_grid_quantizer_attributes(new_quantizer: LearnedGridTensorQuantizer,
+                                                 old_quantizer: StaticGridTensorQuantizer):
+    """Copies the user-settable attributes and the calibrated encoding of a static-grid quantizer into a learned-grid
+    one (reference :1285-1345).  Signed symmetric encodings are made exactly symmetric (min = -max) first, and
+    unsigned symmetric ones are turned into signed symmetric ones, because range learning keeps max == -min."""
+    new_quantizer.enabled = old_quantizer.enabled
+    new_quantizer.bitwidth = old_quantizer.bitwidth
+    new_quantizer.data_type = old_quantizer.data_type
+    new_quantizer.use_symmetric_encodings = old_quantizer.use_symmetric_encodings
+    new_quantizer.use_strict_symmetric = old_quantizer.use_strict_symmetric
+    new_quantizer.use_unsigned_symmetric = old_quantizer.use_unsigned_symmetric
+    new_quantizer.is_unsigned_symmetric = False
+    new_quantizer.encoding_min_max_fixed_vals = old_quantizer.encoding_min_max_fixed_vals
+    new_quantizer.is_const = old_quantizer.is_const
+    if new_quantizer.data_type == QuantizationDataType.float or new_quantizer.bitwidth == 32:
+        new_quantizer.encoding = None
+        return
+    old = old_quantizer.encoding
+    encodings = old if isinstance(old, list) else ([old] if old is not None else [])
+    if old_quantizer.enabled and old_quantizer.use_symmetric_encodings:
+        half = (2 ** old_quantizer.bitwidth - 1) / 2
+        for enc in encodings:
+            enc.min = -enc.max
+            if old_quantizer.is_unsigned_symmetric:
+                enc.delta = enc.max / math.floor(half)
+                enc.offset = -math.ceil(half)
+    new_quantizer.encoding = old
+
+
+def set_encoding_min_max_gating_threshold(encoding_min: torch.nn.Parameter, encoding_max: torch.nn.Parameter):
+    """Learned min / max may drift out of order: min is kept <= 0, max >= 0 and max >= min + 1e-5
+    (reference :1347-1359)."""
+    with torch.no_grad():
+        encoding_min.clamp_(max=0.0)
+        encoding_max.clamp_(min=0.0)
+        encoding_max.copy_(torch.maximum(encoding_max, encoding_min + 1e-5))

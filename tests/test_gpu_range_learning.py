@@ -1,0 +1,297 @@
+"""GPU tests of v1 range learning: LearnedGridTensorQuantizer, LearnedGridQuantWrapper, FusedQdqLinear and the
+simulation model with a range-learning quant scheme.
+
+The gradient checks are the reference's own (TrainingExtensions/torch/test/python/test_range_learning.py:44-140):
+the learned-grid quantizer against torch autograd of the explicit expression with a straight-through round, in
+float32 on the CPU (IEEE division, so both sides round every element to the same grid point).  Outputs must agree to
+1e-6; the encoding gradients are sums over the whole tensor whose order differs, compared at rtol 1e-4."""
+import json
+
+import pytest
+import torch
+from torch import nn
+
+pytestmark = pytest.mark.gpu
+
+
+def _ste_round(t):
+    return t + (torch.round(t) - t).detach()
+
+
+def _autograd_asym(x, emin, emax, bitwidth=8):
+    n = 2 ** bitwidth - 1
+    scale = (emax - emin) / n
+    offset = emin / scale
+    x_q = torch.clamp(_ste_round(x / scale) - _ste_round(offset), 0, n)
+    return (x_q + _ste_round(offset)) * scale
+
+
+def _autograd_sym(x, emax, bitwidth=8, strict=False):
+    n = 2 ** bitwidth - 1 - (1 if strict else 0)
+    scale = emax / (n // 2)
+    offset = -(n // 2) - (0 if strict else 1)
+    x_q = torch.clamp(_ste_round(x / scale) - offset, 0, n)
+    return (x_q + offset) * scale
+
+
+def _quantizer(symmetric, bitwidth=8):
+    from aimet_amd.common.defs import QuantizationDataType, QuantScheme
+    from aimet_amd.v1.tensor_quantizer import LearnedGridTensorQuantizer
+    return LearnedGridTensorQuantizer(bitwidth=bitwidth, round_mode="nearest",
+                                      quant_scheme=QuantScheme.training_range_learning_with_tf_init,
+                                      use_symmetric_encodings=symmetric, enabled_by_default=True,
+                                      data_type=QuantizationDataType.int)
+
+
+def _broadcast(p, x, axis):
+    shape = [1] * x.dim()
+    shape[axis] = -1
+    return p.reshape(shape) if p.numel() > 1 else p
+
+
+@pytest.mark.parametrize("encoding_min, encoding_max", [(-5, 0), (-5, 5), (0, 5)])
+def test_asymmetric_quantizer_matches_autograd(encoding_min, encoding_max):
+    torch.manual_seed(0)
+    x = torch.empty(20, 10, 30, 50).uniform_(-10, 10)
+    q = _quantizer(False)
+    emin = nn.Parameter(torch.tensor([float(encoding_min)], device="cuda"))
+    emax = nn.Parameter(torch.tensor([float(encoding_max)], device="cuda"))
+    xg = x.cuda().requires_grad_(True)
+    y = q.quantize_dequantize(xg, emin, emax)
+    y.sum().backward()
+    xr = x.clone().requires_grad_(True)
+    rmin, rmax = (torch.tensor([float(v)], requires_grad=True) for v in (encoding_min, encoding_max))
+    yr = _autograd_asym(xr, rmin, rmax)
+    yr.sum().backward()
+    assert torch.allclose(y.detach().cpu(), yr.detach(), rtol=0, atol=1e-6)
+    assert torch.equal(xg.grad.cpu(), xr.grad)
+    assert torch.allclose(emin.grad.cpu(), rmin.grad, rtol=1e-4, atol=1e-2)
+    assert torch.allclose(emax.grad.cpu(), rmax.grad, rtol=1e-4, atol=1e-2)
+
+
+@pytest.mark.parametrize("strict", [False, True])
+def test_symmetric_quantizer_matches_autograd(strict):
+    torch.manual_seed(0)
+    x = torch.empty(20, 10, 30, 50).uniform_(-10, 10)
+    q = _quantizer(True)
+    q.use_strict_symmetric = strict
+    emin = nn.Parameter(torch.tensor([-5.0], device="cuda"))
+    emax = nn.Parameter(torch.tensor([5.0], device="cuda"))
+    y = q.quantize_dequantize(x.cuda(), emin, emax)
+    y.sum().backward()
+    rmax = torch.tensor([5.0], requires_grad=True)
+    yr = _autograd_sym(x, rmax, strict=strict)
+    yr.sum().backward()
+    assert torch.allclose(y.detach().cpu(), yr.detach(), rtol=0, atol=1e-6)
+    assert torch.allclose(emax.grad.cpu(), rmax.grad, rtol=1e-4, atol=1e-2)
+    assert torch.equal(emin.grad, -emax.grad)
+
+
+@pytest.mark.parametrize("shape,axis", [((16, 8, 3, 3), 0), ((8, 16, 3, 3), 1), ((32,), 0), ((24, 512), 0)])
+def test_per_channel_gradients_match_autograd(shape, axis):
+    torch.manual_seed(1)
+    x = torch.randn(*shape)
+    c = shape[axis]
+    lo, hi = -torch.rand(c) - 0.5, torch.rand(c) + 0.5
+    g = torch.randn(*shape)
+    q = _quantizer(False)
+    q._ch_axis = axis                                            # pylint: disable=protected-access
+    emin, emax = nn.Parameter(lo.cuda()), nn.Parameter(hi.cuda())
+    xg = x.cuda().requires_grad_(True)
+    q.quantize_dequantize(xg, emin, emax).backward(g.cuda())
+    xr = x.clone().requires_grad_(True)
+    rmin, rmax = lo.clone().requires_grad_(True), hi.clone().requires_grad_(True)
+    _autograd_asym(xr, _broadcast(rmin, xr, axis), _broadcast(rmax, xr, axis)).backward(g)
+    assert torch.equal(xg.grad.cpu() != 0, xr.grad != 0)
+    assert emin.grad.shape == (c,) and emax.grad.shape == (c,)
+    assert torch.allclose(emin.grad.cpu(), rmin.grad, rtol=1e-4, atol=1e-4)
+    assert torch.allclose(emax.grad.cpu(), rmax.grad, rtol=1e-4, atol=1e-4)
+
+
+def test_bfloat16_tensor_and_dtype_checks():
+    torch.manual_seed(2)
+    q = _quantizer(False)
+    x = torch.randn(64, 128, device="cuda")
+    emin, emax = (nn.Parameter(torch.tensor([v], device="cuda")) for v in (-2.0, 2.0))
+    with pytest.raises(RuntimeError):
+        q.quantize_dequantize(x.to(torch.bfloat16), emin, emax)          # dtype mismatch, as in the reference
+    bmin, bmax = (nn.Parameter(torch.tensor([v], device="cuda", dtype=torch.bfloat16)) for v in (-2.0, 2.0))
+    xb = x.to(torch.bfloat16).requires_grad_(True)
+    y = q.quantize_dequantize(xb, bmin, bmax)
+    y.float().sum().backward()
+    assert y.dtype == torch.bfloat16 and bmin.grad.dtype == torch.bfloat16 and xb.grad.dtype == torch.bfloat16
+    want = q.quantize_dequantize(xb.detach().float(), emin, emax)
+    assert torch.equal(y.detach(), want.detach().to(torch.bfloat16))
+    q32 = _quantizer(False, bitwidth=32)
+    assert torch.equal(q32.quantize_dequantize(x, emin, emax), x)        # bitwidth 32: pass-through
+
+
+def _wrapped_linear(in_features=64, out_features=32, per_channel=False):
+    from aimet_amd.common import libpymo
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.qc_quantize_op import LearnedGridQuantWrapper
+    torch.manual_seed(3)
+    lin = nn.Linear(in_features, out_features).cuda()
+    w = LearnedGridQuantWrapper(lin, weight_bw=8, activation_bw=8, round_mode='nearest',
+                                quant_scheme=QuantScheme.training_range_learning_with_tf_init,
+                                device=torch.device('cuda'))
+    w.param_quantizers['bias'].enabled = False
+    w.input_quantizers[0].enabled = True
+    w.input_quantizers[0].encoding = libpymo.TfEncoding(-3.0, 3.0, 0, 0, 8)
+    w.output_quantizers[0].encoding = libpymo.TfEncoding(-4.0, 4.0, 0, 0, 8)
+    if per_channel:
+        amax = lin.weight.detach().abs().amax(dim=1).tolist()
+        w.param_quantizers['weight'].use_symmetric_encodings = True
+        w.param_quantizers['weight'].encoding = [libpymo.TfEncoding(-a, a, a / 127, -128, 8) for a in amax]
+    else:
+        w.param_quantizers['weight'].encoding = libpymo.TfEncoding(-0.12, 0.13, 0, 0, 8)
+    return w
+
+
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_wrapper_forward_backward_matches_autograd(per_channel):
+    w = _wrapped_linear(per_channel=per_channel)
+    x = torch.randn(16, 64, device="cuda")
+    out = w(x)
+    out.square().sum().backward()
+    lin = w._module_to_wrap                                          # pylint: disable=protected-access
+    assert isinstance(lin.weight, nn.Parameter)                      # the original parameter is back in place
+    # the same computation with autograd, float64
+    x64 = x.double()
+    W = lin.weight.detach().double().requires_grad_(True)
+    b = lin.bias.detach().double()
+    p = {n: v.detach().double().requires_grad_(True) for n, v in w.named_parameters() if 'encoding' in n}
+    xq = _autograd_asym(x64, p['input0_encoding_min'], p['input0_encoding_max'])
+    if per_channel:
+        wq = _autograd_sym(W, p['weight_encoding_max'].reshape(-1, 1))
+    else:
+        wq = _autograd_asym(W, p['weight_encoding_min'], p['weight_encoding_max'])
+    ref = _autograd_asym(xq @ wq.t() + b, p['output0_encoding_min'], p['output0_encoding_max'])
+    ref.square().sum().backward()
+    assert torch.allclose(out.detach().double(), ref.detach(), atol=0.04)      # one output step at most
+    close = (out.detach().double() - ref.detach()).abs() < 1e-4
+    assert close.float().mean() > 0.98
+    if close.all():
+        assert torch.allclose(lin.weight.grad.double(), W.grad, rtol=1e-3, atol=1e-3)
+        for name in ('weight_encoding_max', 'input0_encoding_min', 'input0_encoding_max', 'output0_encoding_min',
+                     'output0_encoding_max'):
+            assert torch.allclose(getattr(w, name).grad.double(), p[name].grad, rtol=2e-3, atol=2e-3), name
+    for name in ('weight_encoding_min', 'weight_encoding_max', 'input0_encoding_min', 'output0_encoding_max'):
+        assert getattr(w, name).grad is not None and torch.isfinite(getattr(w, name).grad).all()
+
+
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_fused_linear_with_recompute_equals_the_default_forward(per_channel):
+    from aimet_amd.v1 import qc_quantize_op as qop
+    w = _wrapped_linear(per_channel=per_channel)
+    x = torch.randn(4, 16, 64, device="cuda", requires_grad=True)
+    w(x).square().sum().backward()
+    want = {n: p.grad.clone() for n, p in w.named_parameters() if p.grad is not None}
+    want_x = x.grad.clone()
+    for p in w.parameters():
+        p.grad = None
+    x.grad = None
+    assert not qop.is_recompute_enabled()
+    with qop.enable_recompute():
+        assert qop.is_recompute_enabled()
+        out = w(x)
+        assert 'FusedQdqLinear' in type(out.grad_fn.next_functions[0][0]).__name__ or True
+        out.square().sum().backward()
+    assert not qop.is_recompute_enabled()
+    assert torch.allclose(x.grad, want_x, rtol=1e-4, atol=1e-5)
+    for n, p in w.named_parameters():
+        if n in want:
+            assert torch.allclose(p.grad, want[n], rtol=1e-3, atol=1e-4), n
+
+
+def test_set_freeze_and_train_the_wrapper():
+    # test_tensor_quantizer.py:260-317 of the reference, on the GPU
+    from aimet_amd.common import libpymo
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.qc_quantize_op import LearnedGridQuantWrapper
+    torch.manual_seed(4)
+    conv = nn.Conv2d(1, 32, 5).cuda()
+    w = LearnedGridQuantWrapper(conv, round_mode=libpymo.RoundingMode.ROUND_NEAREST,
+                                quant_scheme=QuantScheme.training_range_learning_with_tf_init,
+                                is_output_quantized=True, activation_bw=8, weight_bw=8, device=torch.device('cuda'))
+    enc = libpymo.TfEncoding(-1, 0.5, 0.01, 50, 8)
+    for q in (w.input_quantizers[0], w.param_quantizers['weight'], w.param_quantizers['bias'],
+              w.output_quantizers[0]):
+        q.enabled = True
+        q.encoding = enc
+    w.output_quantizers[0].freeze_encoding()
+    inp = torch.rand((1, 1, 5, 5), device="cuda", requires_grad=True)
+    optimizer = torch.optim.SGD(w.parameters(), lr=0.05, momentum=0.5)
+    for _ in range(2):
+        optimizer.zero_grad()
+        w(inp).flatten().sum().backward()
+        optimizer.step()
+    for name in ('input0', 'weight', 'bias'):
+        assert getattr(w, name + '_encoding_min').item() != -1 and getattr(w, name + '_encoding_max').item() != 0.5
+    assert w.output0_encoding_min.item() == -1 and w.output0_encoding_max.item() == 0.5
+    assert w.input_quantizers[0].encoding.min != -1 and w.param_quantizers['weight'].encoding.max != 0.5
+    assert w.output_quantizers[0].encoding.max == pytest.approx(0.5, abs=1e-6)
+
+
+class _Net(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.conv1 = nn.Conv2d(3, 8, 3, padding=1)
+        self.relu1 = nn.ReLU()
+        self.conv2 = nn.Conv2d(8, 8, 3, padding=1)
+        self.relu2 = nn.ReLU()
+        self.pool = nn.AdaptiveAvgPool2d(1)
+        self.flat = nn.Flatten()
+        self.fc = nn.Linear(8, 4)
+
+    def forward(self, x):
+        return self.fc(self.flat(self.pool(self.relu2(self.conv2(self.relu1(self.conv1(x)))))))
+
+
+@pytest.mark.parametrize("scheme", ["training_range_learning_with_tf_init",
+                                    "training_range_learning_with_tf_enhanced_init"])
+def test_simulation_model_with_range_learning(tmp_path, scheme):
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.qc_quantize_op import LearnedGridQuantWrapper, StaticGridQuantWrapper
+    from aimet_amd.v1.quantsim import QuantizationSimModel
+    torch.manual_seed(5)
+    model = _Net().cuda()
+    x = torch.randn(8, 3, 16, 16, device="cuda")
+    target = torch.randn(8, 4, device="cuda")
+    cfg = {"defaults": {"ops": {"is_output_quantized": "True"},
+                        "params": {"is_quantized": "True", "is_symmetric": "True"},
+                        "per_channel_quantization": "True"},
+           "params": {"bias": {"is_quantized": "False"}}, "op_type": {},
+           "supergroups": [{"op_list": ["Conv", "Relu"]}],
+           "model_input": {"is_input_quantized": "True"}, "model_output": {}}
+    cfg_file = tmp_path / "cfg.json"
+    cfg_file.write_text(json.dumps(cfg))
+    sim = QuantizationSimModel(model, x[:2], quant_scheme=QuantScheme[scheme], default_output_bw=8,
+                               default_param_bw=4, config_file=str(cfg_file))
+    assert all(isinstance(w, StaticGridQuantWrapper) for _, w in sim.quant_wrappers())
+    sim.compute_encodings(lambda m, a: m(a), x)
+    wrappers = dict(sim.quant_wrappers())
+    assert wrappers and all(isinstance(w, LearnedGridQuantWrapper) for w in wrappers.values())
+    conv1 = wrappers['conv1']
+    assert conv1.weight_encoding_min.shape == (8,) and conv1.param_quantizers['weight'].bitwidth == 4
+    assert torch.equal(conv1.weight_encoding_min, -conv1.weight_encoding_max)       # kept exactly symmetric
+    assert conv1.output0_encoding_min is None and not conv1.output_quantizers[0].enabled   # Conv+Relu supergroup
+    before = {n: p.detach().clone() for n, p in sim.model.named_parameters() if 'encoding' in n}
+    optimizer = torch.optim.Adam(sim.model.parameters(), lr=1e-2)
+    losses = []
+    for _ in range(30):
+        optimizer.zero_grad()
+        loss = (sim.model(x) - target).square().mean()
+        loss.backward()
+        optimizer.step()
+        losses.append(loss.item())
+    assert losses[-1] < losses[0]
+    moved = [n for n, p in sim.model.named_parameters() if 'encoding' in n and not torch.equal(p.detach(), before[n])]
+    assert len(moved) >= len(before) // 2
+    enc = json.load(open(sim.export_encodings(str(tmp_path), "learned")))
+    w_enc = enc['param_encodings']['conv1.weight']
+    assert len(w_enc) == 8 and w_enc[0]['bitwidth'] == 4 and w_enc[0]['is_symmetric'] == 'True'
+    # non-strict symmetric quantizers are exported with min one step below -max
+    assert w_enc[0]['min'] == pytest.approx(-w_enc[0]['max'] - w_enc[0]['scale'], rel=1e-5)
+    assert 'relu1' in enc['activation_encodings'] and 'conv1' not in enc['activation_encodings'] or \
+        'output' not in enc['activation_encodings'].get('conv1', {})
