@@ -14,7 +14,8 @@ import torch
 from .. import ops
 from .libpymo import QuantizationMode, RoundingMode, TfEncoding
 
-_MODE_TO_MIQ = {QuantizationMode.QUANTIZATION_TF: 0, QuantizationMode.QUANTIZATION_TF_ENHANCED: 1}
+_MODE_TO_MIQ = {QuantizationMode.QUANTIZATION_TF: 0, QuantizationMode.QUANTIZATION_TF_ENHANCED: 1,
+                QuantizationMode.QUANTIZATION_PERCENTILE: 2}
 
 
 def _round_mode(round_mode) -> int:
@@ -32,9 +33,10 @@ class AimetTensorQuantizer:
 
     def __init__(self, quantizationScheme: QuantizationMode):
         if quantizationScheme not in _MODE_TO_MIQ:
-            raise RuntimeError(f"{quantizationScheme} is not implemented: only QUANTIZATION_TF and "
-                               "QUANTIZATION_TF_ENHANCED are")
+            raise RuntimeError(f"{quantizationScheme} is not implemented: QUANTIZATION_TF, "
+                               "QUANTIZATION_TF_ENHANCED and QUANTIZATION_PERCENTILE are")
         self._scheme = quantizationScheme
+        self._percentile = 100.0
         self._analyzer = None          # created on the first updateStats, on that tensor's device
         self._is_encoding_valid = False
 
@@ -48,6 +50,7 @@ class AimetTensorQuantizer:
         self._check_gpu(input, use_cuda)
         if self._analyzer is None or self._analyzer.device != input.device:
             self._analyzer = ops.Analyzer(_MODE_TO_MIQ[self._scheme], input.device)
+            self._analyzer.set_percentile(self._percentile)
         self._is_encoding_valid = True
         self._analyzer.update_stats(input)
 
@@ -60,7 +63,7 @@ class AimetTensorQuantizer:
         return _to_tf_encoding(enc), bool(valid)
 
     def getStatsHistogram(self) -> List[Tuple[float, float]]:
-        if self._scheme != QuantizationMode.QUANTIZATION_TF_ENHANCED:
+        if self._scheme == QuantizationMode.QUANTIZATION_TF:
             raise RuntimeError("no histogram is kept by the TF (min/max) analyzer")
         if self._analyzer is None:
             return []
@@ -68,8 +71,12 @@ class AimetTensorQuantizer:
         return list(zip(x_left.tolist(), pdf.tolist()))
 
     def setPercentileValue(self, percentile: float):
-        """Only meaningful for the percentile scheme, which is not implemented; a no-op for TF / TF-Enhanced, as in
-        the reference."""
+        """Used by the percentile scheme only; a no-op for TF / TF-Enhanced, as in the reference
+        (AimetTensorQuantizer.cpp:200-207)."""
+        if self._scheme == QuantizationMode.QUANTIZATION_PERCENTILE:
+            self._percentile = float(percentile)
+            if self._analyzer is not None:
+                self._analyzer.set_percentile(self._percentile)
 
     # ----------------------------------------------------------------------------------------- quantize-dequantize
     @staticmethod

@@ -17,11 +17,13 @@
 // meet on an address.
 #include "miq_common.h"
 
+#include <algorithm>
 #include <cfloat>
 #include <cstddef>
 #include <cmath>
 #include <cstring>
 #include <new>
+#include <vector>
 
 namespace miq
 {
@@ -821,6 +823,7 @@ using namespace miq;
 struct miq_analyzer
 {
     int mode;
+    float percentile;    // percentile analyzer only
     int device;
     DevState* st;        // device
     void* pinned;        // host staging (pinned) for read-backs
@@ -882,17 +885,87 @@ int miq_minmax_per_channel_f32(const float* in, int64_t num_channel, int64_t num
                               reinterpret_cast<uint32_t*>(out_min_max), (hipStream_t) stream);
 }
 
+// PercentileEncodingAnalyzer<float>::computeEncoding on the PDF read back from the device
+// (DLQ/src/PercentileEncodingAnalyzer.cpp:78-198; findOriginalRange: DLQ/src/math_functions.cpp:400-433).
+// 512 buckets of host arithmetic, in the reference's types: float range values, double cdf.
+static int percentile_encoding(const DevState* h, float percentile, int bw, int sym, int strict, int uns,
+                               miq_encoding* out)
+{
+    float num_steps = (float) (std::pow(2, bw) - 1);
+    if (sym && strict)
+        num_steps -= 1;
+    if (!h->initialized)
+    {
+        // only zeros were seen: an encoding that covers float 0
+        out->min    = -1;
+        out->max    = 1;
+        out->delta  = (out->max - out->min) / (int) num_steps;
+        out->offset = std::floor(out->min / out->delta);
+        out->min    = out->offset * out->delta;
+        out->max    = out->min + (int) num_steps * out->delta;
+        out->bw     = bw;
+        return MIQ_OK;
+    }
+    float min_val = (float) h->xLeft[0], max_val = (float) h->xLeft[kPdf - 1];
+    for (int i = 0; i < kPdf; ++i)
+        if (h->pdf[i] > 0)
+        {
+            min_val = (float) h->xLeft[i];
+            break;
+        }
+    for (int i = kPdf - 1; i > 0; --i)
+        if (h->pdf[i] > 0)
+        {
+            max_val = (float) h->xLeft[i];
+            break;
+        }
+    min_val = std::min(min_val, 0.0f);
+    max_val = std::max(max_val, 0.0f);
+    max_val = std::max(max_val, min_val + (float) 0.01);
+    float a_min = min_val, a_max = max_val;
+    if (percentile != 100.0f)
+    {
+        const float width = (float) (h->xLeft[1] - h->xLeft[0]);
+        a_min             = (float) h->xLeft[0];
+        a_max             = (float) (h->xLeft[kPdf - 1] + width);
+        std::vector<double> cdf(h->pdf, h->pdf + kPdf);
+        for (int i = 1; i < kPdf; ++i)
+            cdf[i] += cdf[i - 1];
+        const float left = 1 - percentile / 100;
+        for (int i = 0; i < kPdf; ++i)
+            if (cdf[i] >= left)
+            {
+                a_min = (float) h->xLeft[i];
+                break;
+            }
+        const float right = percentile / 100;
+        for (int i = kPdf - 1; i >= 0; --i)
+            if (cdf[i] < right && h->xLeft[i] < max_val)
+            {
+                a_max = (float) (h->xLeft[i] + width);
+                break;
+            }
+        if (a_min == a_max)
+            a_max += width;
+    }
+    a_min = std::min(a_min, 0.0f);
+    a_max = std::max(a_max, 0.0f);
+    return miq_get_computed_encodings(bw, a_min, a_max, sym, strict, uns, out);
+}
+
 int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
 {
     MIQ_CHECK_ARG(out != nullptr, "null output handle");
-    if (quantization_mode != MIQ_QUANTIZATION_TF && quantization_mode != MIQ_QUANTIZATION_TF_ENHANCED)
+    if (quantization_mode != MIQ_QUANTIZATION_TF && quantization_mode != MIQ_QUANTIZATION_TF_ENHANCED &&
+        quantization_mode != MIQ_QUANTIZATION_PERCENTILE)
     {
-        set_error("quantization mode %d is not implemented (only TF and TF_ENHANCED are)", quantization_mode);
+        set_error("quantization mode %d is not implemented (TF, TF_ENHANCED and PERCENTILE are)", quantization_mode);
         return MIQ_ERR_UNSUPPORTED;
     }
     miq_analyzer* a = new (std::nothrow) miq_analyzer();
     MIQ_CHECK_ARG(a != nullptr, "out of host memory");
     a->mode          = quantization_mode;
+    a->percentile    = 100.0f;   // PercentileEncodingAnalyzer.h: the default clips nothing
     a->st            = nullptr;
     a->pinned        = nullptr;
     a->stats_updated = false;
@@ -934,6 +1007,15 @@ int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
         return MIQ_ERR_HIP;
     }
     *out = a;
+    return MIQ_OK;
+}
+
+int miq_analyzer_set_percentile(miq_analyzer* a, float percentile)
+{
+    MIQ_CHECK_ARG(a != nullptr, "null analyzer");
+    MIQ_CHECK_ARG(percentile >= 0.0f && percentile <= 100.0f, "percentile must be in [0, 100] (got %g)",
+                  (double) percentile);
+    a->percentile = percentile;
     return MIQ_OK;
 }
 
@@ -1029,7 +1111,7 @@ int miq_analyzer_update_stats_f32(miq_analyzer* a, const float* data, int64_t n,
 
 static int flush_pending(miq_analyzer* a, hipStream_t s)
 {
-    if (a->mode == MIQ_QUANTIZATION_TF_ENHANCED && a->seq != 0)
+    if (a->mode != MIQ_QUANTIZATION_TF && a->seq != 0)
     {
         hipLaunchKernelGGL(hist_flush_kernel, dim3(1), dim3(kBlock), 0, s, a->st, a->seq);
         MIQ_CHECK_LAUNCH();
@@ -1071,6 +1153,15 @@ int miq_analyzer_compute_encoding(miq_analyzer* a, int bw, int use_symmetric, in
         double hi = std::max(0.0, h->acc_max);
         hi        = std::max(hi, lo + 0.01);
         return miq_get_computed_encodings(bw, lo, hi, use_symmetric, use_strict_symmetric, use_unsigned_symmetric, out);
+    }
+    if (a->mode == MIQ_QUANTIZATION_PERCENTILE)
+    {
+        if (int rc = flush_pending(a, s))
+            return rc;
+        if (int rc = read_state(a, s))
+            return rc;
+        return percentile_encoding(static_cast<const DevState*>(a->pinned), a->percentile, bw, use_symmetric,
+                                   use_strict_symmetric, use_unsigned_symmetric, out);
     }
     SearchArgs sa{};
     sa.bw             = bw;
@@ -1120,7 +1211,7 @@ int miq_analyzer_compute_encoding(miq_analyzer* a, int bw, int use_symmetric, in
 int miq_analyzer_get_stats_histogram(miq_analyzer* a, double* x_left, double* pdf, int* num_buckets, void* stream)
 {
     MIQ_CHECK_ARG(a && x_left && pdf && num_buckets, "null argument");
-    if (a->mode != MIQ_QUANTIZATION_TF_ENHANCED)
+    if (a->mode == MIQ_QUANTIZATION_TF)
     {
         set_error("no histogram is kept by the TF (min/max) analyzer");
         return MIQ_ERR_UNSUPPORTED;

@@ -415,7 +415,8 @@ def adaround_linear_bwd_adam(weight_floor, grad_out, x, row_index, alpha, exp_av
 
 
 class Analyzer:
-    """Device-resident encoding analyzer (TF min/max or TF-Enhanced 512-bucket PDF + SQNR search)."""
+    """Device-resident encoding analyzer: mode 0 = TF min/max, 1 = TF-Enhanced (512-bucket PDF + SQNR search),
+    2 = percentile on the same PDF."""
 
     def __init__(self, mode, device=None):
         self.mode = int(mode)
@@ -440,6 +441,9 @@ class Analyzer:
     def reset(self):
         with torch.cuda.device(self.device):
             check(lib.miq_analyzer_reset(self._h, self._s()))
+
+    def set_percentile(self, percentile: float):
+        check(lib.miq_analyzer_set_percentile(self._h, float(percentile)))
 
     def update_stats(self, x):
         """Queue one batch.  Lean on purpose: a batch of a few MB takes microseconds on the device, so the Python

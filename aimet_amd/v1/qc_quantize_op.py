@@ -49,7 +49,8 @@ def tensor_quantizer_factory(bitwidth: int, round_mode, quant_scheme: QuantSchem
                              enabled_by_default: bool, data_type: QuantizationDataType = QuantizationDataType.int):
     """Instantiates the tensor quantizer for `quant_scheme`: static grid for the post-training schemes, learned grid
     for the range-learning schemes (reference :80-112)."""
-    if quant_scheme in (QuantScheme.post_training_tf_enhanced, QuantScheme.post_training_tf):
+    if quant_scheme in (QuantScheme.post_training_tf_enhanced, QuantScheme.post_training_tf,
+                        QuantScheme.post_training_percentile):
         return StaticGridPerTensorQuantizer(bitwidth, _to_round_mode(round_mode), quant_scheme,
                                             use_symmetric_encodings, enabled_by_default, data_type=data_type)
     if quant_scheme in (QuantScheme.training_range_learning_with_tf_init,
@@ -189,6 +190,8 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
                 if self._module_to_wrap.training or quantizer.encoding is None:
                     quantizer.reset_encoding_stats()
                     quantizer.update_encoding_stats(param.data)
+                    if quantizer.quant_scheme == QuantScheme.post_training_percentile:
+                        quantizer.set_percentile_value(100)
                     quantizer.compute_encoding()
                 round_mode = quantizer.round_mode if self.training else libpymo.RoundingMode.ROUND_NEAREST
                 param.data = quantizer.quantize_dequantize(param.data, round_mode)
@@ -204,6 +207,12 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
             quantizer.compute_encoding()
         for quantizer in self.output_quantizers:
             quantizer.compute_encoding()
+
+    def set_percentile_value(self, percentile_value: float):
+        """Percentile of the activation quantizers of this wrapper (reference :827-835); parameters are always
+        calibrated at 100 (:775-776)."""
+        for quantizer in list(self.input_quantizers) + list(self.output_quantizers):
+            quantizer.set_percentile_value(percentile_value)
 
     def _quantize_activation(self, tensor_quantizers, tensors_to_quantize):
         def inner(tensor, index):

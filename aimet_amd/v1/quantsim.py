@@ -77,6 +77,7 @@ def _flag(d: dict, key: str, default=None):
 _INIT_SCHEME = {
     QuantScheme.post_training_tf: QuantScheme.post_training_tf,
     QuantScheme.post_training_tf_enhanced: QuantScheme.post_training_tf_enhanced,
+    QuantScheme.post_training_percentile: QuantScheme.post_training_percentile,
     QuantScheme.training_range_learning_with_tf_init: QuantScheme.post_training_tf,
     QuantScheme.training_range_learning_with_tf_enhanced_init: QuantScheme.post_training_tf_enhanced,
 }
@@ -103,10 +104,11 @@ class QuantizationSimModel:
                  default_data_type: QuantizationDataType = QuantizationDataType.int):
         if isinstance(quant_scheme, str):
             quant_scheme = {'tf': QuantScheme.post_training_tf,
-                            'tf_enhanced': QuantScheme.post_training_tf_enhanced}[quant_scheme]
+                            'tf_enhanced': QuantScheme.post_training_tf_enhanced,
+                            'percentile': QuantScheme.post_training_percentile}[quant_scheme]
         if quant_scheme not in _INIT_SCHEME:
-            raise ValueError(f"quant_scheme {quant_scheme} is not implemented (tf, tf_enhanced and the two "
-                             "range-learning schemes initialised from them are)")
+            raise ValueError(f"quant_scheme {quant_scheme} is not implemented (tf, tf_enhanced, percentile and the "
+                             "two range-learning schemes are)")
         if rounding_mode not in ('nearest', 'stochastic'):
             raise ValueError('Parameter round mode can only be nearest or stochastic')
         if default_param_bw < 4 or default_param_bw > 32 or default_output_bw < 4 or default_output_bw > 32:
@@ -115,6 +117,7 @@ class QuantizationSimModel:
             raise ValueError('only QuantizationDataType.int is implemented')
         self.model = model if in_place else copy.deepcopy(model)
         self._quant_scheme = quant_scheme
+        self._percentile_value = 100                 # default of the reference (:278)
         self._rounding_mode = rounding_mode
         self._default_output_bw = default_output_bw
         self._default_param_bw = default_param_bw
@@ -287,6 +290,8 @@ class QuantizationSimModel:
         for _, layer in layers:
             layer.reset_encodings()
             layer.set_mode(QcQuantizeOpMode.ANALYSIS)
+            if self._quant_scheme == QuantScheme.post_training_percentile:
+                layer.set_percentile_value(self._percentile_value)     # reference :395-400
         was_training = self.model.training
         self.model.eval()
         try:
@@ -340,6 +345,13 @@ class QuantizationSimModel:
             if new.encoding_min_max_fixed_vals is not None:
                 new.freeze_encoding()
         return trainable
+
+    def set_percentile_value(self, percentile_value: float):
+        """Percentile used by the quantizers of the percentile scheme at the next compute_encodings
+        (reference quantsim.py:478-484)."""
+        if percentile_value < 90 or percentile_value > 100:
+            raise ValueError("Percentile value must be in range [90, 100]")
+        self._percentile_value = percentile_value
 
     def exclude_layers_from_quantization(self, layers_to_exclude: List[nn.Module]):
         """Replaces the given quantization wrappers by the modules they wrap (reference quantsim.py:1419-1433)."""

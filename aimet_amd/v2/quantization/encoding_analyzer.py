@@ -6,7 +6,7 @@ _MinMaxObserver (:91-129), EncodingAnalyzer (:272-319) and MinMaxEncodingAnalyze
 ``observer.shape``.  Statistics are collected by the fused min/max kernels (one pass for min and max together;
 per-channel shapes in one launch) instead of two torch reductions over a permuted copy.
 
-_HistogramObserver (:131-270) and SqnrEncodingAnalyzer (:522-725): the running histogram, its range and the candidate
+_HistogramObserver (:131-270), PercentileEncodingAnalyzer (:428-519) and SqnrEncodingAnalyzer (:522-725): the running histogram, its range and the candidate
 search live on the GPU.  One update is five kernels and reads the batch twice (finite min/max; one binning pass that
 fills the batch's histogram and the merged-range histogram together); the reference reads it about eight times and
 re-bins with per-element Python loops.  Nothing synchronises until an encoding or a statistic is read.  Differences:
@@ -275,6 +275,74 @@ class _HistogramObserver:
         if self._state is None:
             return [_Histogram() for _ in range(self.num_histograms)]
         return self._state
+
+
+def adjust_min_max(curr_min: torch.Tensor, curr_max: torch.Tensor, num_steps, is_symmetric: bool):
+    """Widens a range to contain zero, keeps it finite and at least _MINIMUM_SCALE * num_steps wide; a symmetric grid
+    takes the larger of its two half ranges (reference :397-425).  Works on tensors of any shape."""
+    curr_min = torch.clamp(curr_min, min=torch.finfo(curr_min.dtype).min, max=0)
+    curr_max = torch.clamp(curr_max, min=0, max=torch.finfo(curr_max.dtype).max)
+    too_close = (curr_max - curr_min) / num_steps < _MINIMUM_SCALE
+    if is_symmetric:
+        num_pos_steps, num_neg_steps = math.floor(num_steps / 2), math.ceil(num_steps / 2)
+        curr_min = torch.where(too_close, curr_min - _MINIMUM_SCALE * num_neg_steps, curr_min)
+        curr_max = torch.where(too_close, curr_max + _MINIMUM_SCALE * num_pos_steps, curr_max)
+        delta = torch.maximum(curr_max / num_pos_steps, -curr_min / num_neg_steps)
+        return -num_neg_steps * delta, num_pos_steps * delta
+    return curr_min, torch.where(too_close, curr_max + _MINIMUM_SCALE * num_steps, curr_max)
+
+
+class PercentileEncodingAnalyzer(EncodingAnalyzer):
+    """Percentile calibration: values are recorded in a histogram and the range is cut where the cumulative count
+    reaches (100 - p) % and p % of the total (reference :428-519).  All histograms are searched at once on the
+    device."""
+
+    def __init__(self, shape: tuple, num_bins: int = 2048, percentile: float = 100):
+        if num_bins <= 0:
+            raise ValueError('Number of bins cannot be less than or equal to 0.')
+        super().__init__(_HistogramObserver(shape=shape, num_bins=num_bins))
+        self.set_percentile(percentile)
+
+    def set_percentile(self, percentile):
+        if percentile < 50 or percentile > 100:
+            raise ValueError('Percentile value must be within 50-100 range')
+        self.percentile = percentile
+
+    @torch.no_grad()
+    def update_stats(self, input_tensor: torch.Tensor):
+        return self.observer.collect_and_merge_stats(input_tensor)
+
+    @torch.no_grad()
+    def compute_encodings_from_stats(self, stats, num_steps: int, is_symmetric: bool) \
+            -> Tuple[torch.Tensor, torch.Tensor]:
+        if num_steps <= 0:
+            raise ValueError('The number of quantization bins cannot be less than or equal to 0.')
+        if isinstance(stats, (list, tuple)):
+            if stats[0].histogram is None:
+                raise StatisticsNotFoundError('No statistics present to compute encodings.')
+            hist = torch.stack([s.histogram for s in stats])
+            minmax = torch.stack([torch.stack((s.min, s.max)) for s in stats]).to(torch.float32)
+        else:
+            stats.check()
+            hist, minmax = stats.hist, stats.minmax
+        num_bins = hist.shape[1]
+        if self.percentile == 100:
+            min_index = torch.zeros(hist.shape[0], 1, dtype=torch.long, device=hist.device)
+            max_index = torch.full_like(min_index, num_bins)
+        else:
+            cum_sum = torch.cumsum(hist, dim=1)
+            total = cum_sum[:, -1:]
+            hundred = torch.tensor(100.0, device=hist.device)
+            max_index = torch.searchsorted(cum_sum, total * self.percentile / hundred)
+            min_index = torch.searchsorted(cum_sum, total * (1 - self.percentile / 100))
+        # bin_edges[index] of every histogram: index * bin width + min, the arithmetic of _bin_edges
+        mn, mx = minmax[:, 0:1], minmax[:, 1:2]
+        same = mx == mn
+        mn, mx = torch.where(same, mn - 0.5, mn), torch.where(same, mx + 0.5, mx)
+        step = (mx - mn) / torch.tensor(float(num_bins), device=hist.device)
+        curr_min, curr_max = min_index * step + mn, max_index * step + mn
+        enc_min, enc_max = adjust_min_max(curr_min, curr_max, num_steps, is_symmetric)
+        return enc_min.view(self.observer.shape), enc_max.view(self.observer.shape)
 
 
 class SqnrEncodingAnalyzer(EncodingAnalyzer):

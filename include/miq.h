@@ -34,6 +34,7 @@ extern "C" {
 /* DLQ/include/DlQuantization/Quantization.hpp:83-105 (QuantizationMode) */
 #define MIQ_QUANTIZATION_TF 0
 #define MIQ_QUANTIZATION_TF_ENHANCED 1
+#define MIQ_QUANTIZATION_PERCENTILE 2
 
 #define MIQ_PDF_SIZE 512 /* DLQ/src/math_functions.hpp:80 */
 
@@ -188,13 +189,18 @@ int miq_minmax_per_channel_f32(const float* in, int64_t num_channel, int64_t num
  * (DLQ/include/DlQuantization/IQuantizationEncodingAnalyzer.hpp:48-126) as instantiated by
  * getEncodingAnalyzerInstance<float>(mode) (DLQ/src/QuantizerFactory.cpp:74-97) for QUANTIZATION_TF
  * (TfEncodingAnalyzer, DLQ/src/TfEncodingAnalyzer.cpp:59-101) and QUANTIZATION_TF_ENHANCED
- * (TfEnhancedEncodingAnalyzer, DLQ/src/TfEnhancedEncodingAnalyzer.cpp:68-397).  All statistics (running min/max,
+ * (TfEnhancedEncodingAnalyzer, DLQ/src/TfEnhancedEncodingAnalyzer.cpp:68-397) and QUANTIZATION_PERCENTILE
+ * (PercentileEncodingAnalyzer, DLQ/src/PercentileEncodingAnalyzer.cpp:54-215: the same PDF, cut where its cumulative
+ * sum reaches 100 - p and p percent).  All statistics (running min/max,
  * the 512-bucket PDF, its range and iteration count) live in device memory owned by the object on the device that
  * was current at creation; update_stats enqueues work and never synchronises.  compute_encoding synchronises
  * `stream` once to read the result back.  An object must not be used from two threads at once. */
 typedef struct miq_analyzer miq_analyzer;
 int miq_analyzer_create(int quantization_mode, miq_analyzer** out);
 int miq_analyzer_destroy(miq_analyzer* a);
+/* setPercentileValue (IQuantizationEncodingAnalyzer.hpp:104-112; PercentileEncodingAnalyzer.cpp:203-207), 0..100,
+ * default 100.  Stored by every analyzer, used by the percentile one. */
+int miq_analyzer_set_percentile(miq_analyzer* a, float percentile);
 /* resetEncodingStats (TSRC/AimetTensorQuantizer.cpp:85-92) */
 int miq_analyzer_reset(miq_analyzer* a, void* stream);
 /* updateStats(tensor, tensorSize, mode, allocator) (IQuantizationEncodingAnalyzer.hpp:59-69) */

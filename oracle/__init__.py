@@ -287,6 +287,18 @@ class OraclePdf:
                                           costs.ctypes.data, C.byref(best))
         return e, costs, best.value
 
+    def percentile_range(self, percentile):
+        a, b = C.c_float(), C.c_float()
+        self.o.L.orc_percentile_range(C.byref(self.s), C.c_float(percentile), C.byref(a), C.byref(b))
+        return np.float32(a.value), np.float32(b.value)
+
+    def compute_percentile_encoding(self, bw, percentile, sym=False, strict=False, unsigned_sym=False):
+        """PercentileEncodingAnalyzer<float>::computeEncoding on the same PDF."""
+        e = Encoding()
+        self.o.L.orc_percentile_compute_encoding(C.byref(self.s), C.c_float(percentile), bw, int(sym), int(strict),
+                                                 int(unsigned_sym), C.byref(e))
+        return e
+
 
 class _Ref:
     """The reference's own CPU classes, compiled in place (present only where oracle/_ref was built)."""
@@ -361,6 +373,9 @@ class _Ref:
     def new_tfe(self):
         return _RefAnalyzer(self, enhanced=True)
 
+    def new_percentile(self, percentile):
+        return _RefPercentile(self, percentile)
+
 
 class _RefAnalyzer:
     def __init__(self, ref, enhanced):
@@ -400,6 +415,33 @@ class _RefAnalyzer:
         costs = np.empty(512, np.float64)
         n = self.r.L.ref_tfe_candidates(self.h, bw, int(sym), int(strict), int(unsigned_sym), 512, d, off, costs)
         return d[:n].copy(), off[:n].copy(), costs[:n].copy()
+
+
+class _RefPercentile:
+    """The reference's PercentileEncodingAnalyzer<float>, compiled in place."""
+
+    def __init__(self, ref, percentile):
+        L = self.L = ref.L
+        L.ref_pct_create.restype = C.c_void_p
+        L.ref_pct_create.argtypes = [C.c_float]
+        L.ref_pct_destroy.argtypes = [C.c_void_p]
+        L.ref_pct_update.argtypes = [C.c_void_p, _f32p, _i64]
+        L.ref_pct_compute.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _f64p]
+        self.h = C.c_void_p(L.ref_pct_create(percentile))
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            self.L.ref_pct_destroy(self.h)
+            self.h = None
+
+    def update(self, x):
+        x = _f32(x)
+        self.L.ref_pct_update(self.h, x.reshape(-1), x.size)
+
+    def compute_encoding(self, bw, sym=False, strict=False, unsigned_sym=False):
+        o = np.empty(5)
+        self.L.ref_pct_compute(self.h, bw, int(sym), int(strict), int(unsigned_sym), o)
+        return _Ref._enc(o)
 
 
 def _load():

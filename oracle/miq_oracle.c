@@ -652,6 +652,81 @@ void orc_tfe_compute_encoding(const orc_pdf* p, int bw, int sym, int strict, int
 }
 
 /* ------------------------------------------------------------------------------------------------------------
+ * Percentile calibration on the same 512-bucket PDF (PercentileEncodingAnalyzer<float>;
+ * DLQ/src/PercentileEncodingAnalyzer.cpp:78-198).  Statistics are gathered by UpdatePdf with signed_vals = true,
+ * i.e. by orc_pdf_update_f32 above.
+ * ---------------------------------------------------------------------------------------------------------- */
+
+/* _computePercentileRange, :133-198 */
+void orc_percentile_range(const orc_pdf* p, float percentile, float* minOut, float* maxOut)
+{
+    float minVal, maxVal;
+    orc_tfe_find_range(p, &minVal, &maxVal); /* findOriginalRange<float>: the same steps (math_functions.cpp:400-433) */
+    if (percentile == 100.0f)
+    {
+        *minOut = minVal;
+        *maxOut = maxVal;
+        return;
+    }
+    const float histBinWidth = (float) (p->xLeft[1] - p->xLeft[0]);
+    float histMin            = (float) p->xLeft[0];
+    float histMax            = (float) (p->xLeft[ORC_PDF_SIZE - 1] + histBinWidth);
+    float percentileMin      = histMin;
+    float percentileMax      = histMax;
+    double cdf[ORC_PDF_SIZE];
+    cdf[0] = p->pdf[0];
+    for (int i = 1; i < ORC_PDF_SIZE; ++i)
+        cdf[i] = p->pdf[i] + cdf[i - 1];
+    float leftPercentile = 1 - percentile / 100;
+    for (int i = 0; i < ORC_PDF_SIZE; ++i)
+        if (cdf[i] >= leftPercentile)
+        {
+            percentileMin = (float) p->xLeft[i];
+            break;
+        }
+    float rightPercentile = percentile / 100;
+    for (int i = ORC_PDF_SIZE - 1; i >= 0; --i)
+        if (cdf[i] < rightPercentile && p->xLeft[i] < maxVal)
+        {
+            percentileMax = (float) (p->xLeft[i] + histBinWidth);
+            break;
+        }
+    if (percentileMin == percentileMax)
+        percentileMax += histBinWidth;
+    *minOut = percentileMin;
+    *maxOut = percentileMax;
+}
+
+/* computeEncoding, :78-130 */
+void orc_percentile_compute_encoding(const orc_pdf* p, float percentile, int bw, int sym, int strict, int unsignedSym,
+                                     orc_encoding* e)
+{
+    memset(e, 0, sizeof(*e));
+    float numSteps = (float) (pow(2, bw) - 1);
+    if (sym && strict)
+        numSteps -= 1;
+    if (!p->initialized)
+    {
+        if (p->stats_updated)
+        {
+            e->min    = -1;
+            e->max    = 1;
+            e->delta  = (e->max - e->min) / (int) numSteps;
+            e->offset = floor(e->min / e->delta);
+            e->min    = e->offset * e->delta;
+            e->max    = e->min + (int) numSteps * e->delta;
+            e->bw     = bw;
+        }
+        return;
+    }
+    float aMin, aMax;
+    orc_percentile_range(p, percentile, &aMin, &aMax);
+    aMin = STD_MIN(aMin, 0.0f);
+    aMax = STD_MAX(aMax, 0.0f);
+    orc_get_computed_encodings(bw, aMin, aMax, sym, strict, unsignedSym, e);
+}
+
+/* ------------------------------------------------------------------------------------------------------------
  * a7  v2 quantize-dequantize (TORCH/v2/quantization/affine/backends/torch_builtins.py:303-344), float32 internal
  * dtype.  scale/offset are per "channel" with channel = (i / numElementPerChannel) % numChannel, which covers the
  * per-tensor ([1]) and per-output-channel ([C,1,...]) broadcast shapes.  torch.round is half-to-even (rintf under

@@ -9,6 +9,7 @@
 //   TensorQuantizationSim<float>      ModelOptimizations/DlQuantization/src/TensorQuantizationSim.cpp:62-126, 300-317
 //   TfEncodingAnalyzer<float>         ModelOptimizations/DlQuantization/src/TfEncodingAnalyzer.cpp:59-101
 //   TfEnhancedEncodingAnalyzer<float> ModelOptimizations/DlQuantization/src/TfEnhancedEncodingAnalyzer.cpp:68-397
+//   PercentileEncodingAnalyzer<float> ModelOptimizations/DlQuantization/src/PercentileEncodingAnalyzer.cpp:54-215
 //   getComputedEncodings              ModelOptimizations/DlQuantization/src/quantization_utils.cpp:58-143
 //   quantizeDequantizeBroadcastCpu    ModelOptimizations/DlQuantization/src/trim_functions.cpp:634-660
 
@@ -30,6 +31,7 @@
 #include "TfEnhancedEncodingAnalyzer.h"
 #undef private
 #include "TensorQuantizationSim.h"
+#include "PercentileEncodingAnalyzer.h"
 #include "TfEncodingAnalyzer.h"
 #include "quantization_utils.hpp"
 #include "trim_functions.hpp"
@@ -181,5 +183,26 @@ void ref_tfe_range(void* h, float* minVal, float* maxVal)
 {
     auto* a                    = static_cast<TfEnhancedEncodingAnalyzer<float>*>(h);
     std::tie(*minVal, *maxVal) = a->_findRangeOfAggregateStats();
+}
+// ---- PercentileEncodingAnalyzer<float> -----------------------------------------------------------
+void* ref_pct_create(float percentile)
+{
+    auto* a = new PercentileEncodingAnalyzer<float>();
+    a->setPercentileValue(percentile);
+    return a;
+}
+void ref_pct_destroy(void* h)
+{
+    delete static_cast<PercentileEncodingAnalyzer<float>*>(h);
+}
+void ref_pct_update(void* h, const float* data, int64_t n)
+{
+    static_cast<PercentileEncodingAnalyzer<float>*>(h)->updateStats(data, (size_t) n, COMP_MODE_CPU);
+}
+void ref_pct_compute(void* h, int bw, int sym, int strict, int unsignedSym, double* out5)
+{
+    TfEncoding e = static_cast<PercentileEncodingAnalyzer<float>*>(h)->computeEncoding((uint8_t) bw, sym != 0,
+                                                                                       strict != 0, unsignedSym != 0);
+    putEncoding(e, out5);
 }
 }   // extern "C"

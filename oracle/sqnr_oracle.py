@@ -10,10 +10,12 @@ EA = TrainingExtensions/torch/src/python/aimet_torch/v2/quantization/encoding_an
   pick_test_candidates[_asymmetric|_symmetric], clamp_delta_offset_values     EA:594-660
   estimate_clip_and_quant_noise           EA:675-725
   select_best_candidates, compute_encodings_from_stats                        EA:566-592, 662-673
+  adjust_min_max, percentile_encodings_from_stats                             EA:397-425, 486-519
 
 Pinned by the reference's own tests (TrainingExtensions/torch/test/python/v2/quantization/test_encoding_analyzer.py:
 657-881, restated in tests/test_oracle_sqnr.py): exact encodings of a uniform grid, the outlier construction, candidate
-grids, clamping, estimated-vs-measured noise, best-candidate selection.
+grids, clamping, estimated-vs-measured noise, best-candidate selection; the percentile part by :544-655 (sequential
+data with known percentiles, 100 % = observed range, non-strict symmetric grid, outliers).
 """
 import math
 from typing import List, NamedTuple, Optional
@@ -202,3 +204,48 @@ class SqnrAnalyzer:
 
     def compute_encodings(self, num_steps, is_symmetric):
         return compute_encodings_from_stats(self.stats, num_steps, is_symmetric, self.gamma)
+
+
+# ------------------------------------------------------------------------------------------ percentile calibration
+def adjust_min_max(curr_min, curr_max, num_steps, is_symmetric):
+    """EA:397-425: the range is widened to contain zero, kept finite and at least MINIMUM_SCALE * num_steps wide; a
+    symmetric grid takes the larger of the two half ranges."""
+    curr_min = torch.minimum(curr_min, torch.zeros_like(curr_min)).clone()
+    curr_max = torch.maximum(curr_max, torch.zeros_like(curr_max)).clone()
+    curr_min = curr_min.clamp(min=torch.finfo(curr_max.dtype).min, max=0)
+    curr_max = curr_max.clamp(min=0, max=torch.finfo(curr_max.dtype).max)
+    too_close = (curr_max - curr_min) / num_steps < MINIMUM_SCALE
+    if is_symmetric:
+        curr_min = torch.where(too_close, curr_min - MINIMUM_SCALE * math.ceil(num_steps / 2), curr_min)
+        curr_max = torch.where(too_close, curr_max + MINIMUM_SCALE * math.floor(num_steps / 2), curr_max)
+        num_pos_steps, num_neg_steps = math.floor(num_steps / 2), math.ceil(num_steps / 2)
+        delta = torch.maximum(curr_max / num_pos_steps, -curr_min / num_neg_steps)
+        curr_min, curr_max = -num_neg_steps * delta, num_pos_steps * delta
+    else:
+        curr_max = torch.where(too_close, curr_max + MINIMUM_SCALE * num_steps, curr_max)
+    return curr_min, curr_max
+
+
+def percentile_encodings_from_stats(stats: List[Histogram], percentile: float, num_steps, is_symmetric):
+    """EA:486-519 (PercentileEncodingAnalyzer.compute_encodings_from_stats): per histogram, the bin edges at which the
+    cumulative count reaches (100 - p) % and p % of the total, then adjust_min_max."""
+    mins, maxs = [], []
+    for h in stats:
+        cum_sum = torch.cumsum(h.histogram, dim=0)
+        max_index = torch.searchsorted(cum_sum, cum_sum[-1] * percentile / 100)
+        min_index = torch.searchsorted(cum_sum, cum_sum[-1] * (1 - percentile / 100))
+        if percentile == 100:
+            min_index, max_index = 0, -1
+        lo, hi = adjust_min_max(h.bin_edges[min_index], h.bin_edges[max_index], num_steps, is_symmetric)
+        mins.append(lo)
+        maxs.append(hi)
+    return torch.stack(mins), torch.stack(maxs)
+
+
+class PercentileAnalyzer(SqnrAnalyzer):
+    def __init__(self, num_histograms=1, num_bins=2048, percentile=100.0):
+        super().__init__(num_histograms, num_bins)
+        self.percentile = percentile
+
+    def compute_encodings(self, num_steps, is_symmetric):
+        return percentile_encodings_from_stats(self.stats, self.percentile, num_steps, is_symmetric)

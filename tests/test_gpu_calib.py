@@ -193,3 +193,91 @@ def test_cfg3_full_size_properties(ops, oracle):
     assert 0.99 < p.sum() <= 1.0 + 1e-12
     enc, valid = an.compute_encoding(8)
     assert valid and enc.delta > 0 and enc.min <= 0 <= enc.max
+
+
+# ------------------------------------------------------------------------------------------ percentile analyzer
+PERCENTILE = 2
+
+
+@pytest.mark.parametrize("percentile", [100.0, 99.9999, 99.9, 99.0, 90.0, 50.0])
+def test_percentile_analyzer_matches_the_oracle(ops, oracle, percentile):
+    """PercentileEncodingAnalyzer<float>: the PDF is the TF-Enhanced one; every field of the encoding is identical."""
+    rng = np.random.default_rng(int(percentile * 10))
+    cases = {
+        "normal": [(rng.standard_normal(30000) * (1 + b) + 0.5).astype(np.float32) for b in range(3)],
+        "relu-pareto": [_relu_pareto(20 + b, 50000) for b in range(2)],
+        "negative": [(-np.abs(rng.standard_normal(10000)) - 0.25).astype(np.float32)],
+        "constant": [np.full(6000, 4, np.float32)],
+        "zeros": [np.zeros(6000, np.float32)],
+        "zeros-then-data": [np.zeros(100, np.float32), rng.standard_normal(9999).astype(np.float32)],
+    }
+    for kind, batches in cases.items():
+        an, pdf = ops.Analyzer(PERCENTILE), oracle.new_pdf()
+        an.set_percentile(percentile)
+        for b in batches:
+            an.update_stats(_gpu(b))
+            pdf.update(b)
+        for bw, sym, strict, uns in ((8, 0, 0, 0), (8, 1, 0, 0), (8, 1, 1, 0), (8, 1, 0, 1), (4, 0, 0, 0),
+                                     (16, 0, 0, 0)):
+            e, valid = an.compute_encoding(bw, sym, strict, uns)
+            want = pdf.compute_percentile_encoding(bw, percentile, sym, strict, uns)
+            assert valid and (e.min, e.max, e.delta, e.offset, e.bw) == want.astuple(), (kind, bw, sym, strict, uns)
+
+
+def test_percentile_analyzer_edge_behaviour(ops):
+    from aimet_amd._lib import MiqError
+    an = ops.Analyzer(PERCENTILE)
+    e, valid = an.compute_encoding(8)
+    assert not valid and (e.min, e.max, e.delta, e.offset) == (0, 0, 0, 0)        # nothing seen
+    with pytest.raises(MiqError):
+        an.set_percentile(101.0)
+    x = torch.randn(5000, device="cuda")
+    an.update_stats(x)
+    xl, p = an.get_stats_histogram()                                              # the PDF is inspectable
+    assert len(xl) == 512 and abs(p.sum() - 1.0) < 1e-9
+    e100, _ = an.compute_encoding(8)
+    an.set_percentile(95.0)
+    e95, _ = an.compute_encoding(8)
+    assert e95.max < e100.max and e95.min > e100.min
+    an.reset()
+    assert not an.compute_encoding(8)[1]
+
+
+def test_percentile_scheme_through_the_v1_quantizers():
+    """test_tensor_quantizer / quantsim flow of the reference with quant_scheme = post_training_percentile."""
+    from aimet_amd.common import libpymo
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.quantsim import QuantizationSimModel
+    from aimet_amd.v1.tensor_quantizer import StaticGridPerTensorQuantizer
+    torch.manual_seed(0)
+    x = torch.randn(40000, device="cuda")
+    x[:4] = 500.0
+    q = StaticGridPerTensorQuantizer(8, libpymo.RoundingMode.ROUND_NEAREST, QuantScheme.post_training_percentile,
+                                     use_symmetric_encodings=False, enabled_by_default=True)
+    q.set_percentile_value(99.9)
+    q.update_encoding_stats(x)
+    q.compute_encoding()
+    assert q.encoding.max < 10 and q.encoding.min > -10                   # the outliers are cut off
+    q.reset_encoding_stats()
+    q.set_percentile_value(100)
+    q.update_encoding_stats(x)
+    q.compute_encoding()
+    assert q.encoding.max > 490
+
+    model = torch.nn.Sequential(torch.nn.Conv2d(3, 8, 3), torch.nn.ReLU(), torch.nn.Conv2d(8, 4, 3)).cuda()
+    data = torch.randn(8, 3, 12, 12, device="cuda")
+    data[0, 0, 0, 0] = 1000.0
+    sim = QuantizationSimModel(model, data[:1], quant_scheme=QuantScheme.post_training_percentile)
+    with pytest.raises(ValueError):
+        sim.set_percentile_value(80)
+    sim.set_percentile_value(99)
+    sim.compute_encodings(lambda m, a: m(a), data)
+    wrappers = dict(sim.quant_wrappers())
+    first = wrappers['0']
+    out_enc = wrappers['1'].output_quantizers[0].encoding                  # Conv + ReLU: quantized after the ReLU
+    full = model[1](model[0](data))
+    assert out_enc.max < full.max().item() * 0.5                           # activations: clipped at 99 %
+    w_enc = first.param_quantizers['weight'].encoding
+    w_abs = model[0].weight.abs().max().item()
+    assert max(abs(w_enc.min), w_enc.max) >= w_abs * 0.99                  # parameters: always 100 %
+    assert torch.isfinite(sim.model(data)).all()

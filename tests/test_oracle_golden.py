@@ -388,3 +388,39 @@ def test_bf16_roundtrip_matches_torch(oracle):
     assert np.array_equal(bits, tb)
     for v in x[:200].numpy():
         assert oracle.L.orc_f32_to_bf16(float(v)) == int(oracle.f32_to_bf16_bits(np.array([v]))[0])
+
+
+# ------------------------------------------------------------------------------- percentile analyzer (v1, C++)
+def test_percentile_cases_of_the_reference_unit_tests(oracle):
+    """ModelOptimizations/DlQuantization/test/TestPercentileEncodingAnalyzer.cpp:56-370: the assertions of its cases
+    on data of the same distribution (the reference draws from std::normal_distribution; the bounds it asserts hold
+    for any sample of that size)."""
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal(100000) * 2 + 2).astype(np.float32)
+    pdf = oracle.new_pdf()
+    pdf.update(x)
+    e = pdf.compute_percentile_encoding(8, 99.9999)                      # Asymmetric, :56-109
+    assert 2 - 12 < e.min < 2 - 4 and 2 + 4 < e.max < 2 + 12
+    e = pdf.compute_percentile_encoding(8, 99.9999, sym=True)            # Symmetric, :111-159
+    assert e.min > -np.abs(x).max() - e.delta and e.max < np.abs(x).max() and e.offset == -128 and e.bw == 8
+    assert e.delta == pytest.approx((e.max - e.min) / 255, rel=1e-6)
+    e = pdf.compute_percentile_encoding(8, 99.9999, sym=True, strict=True)   # StrictSymmetric, :161-210
+    assert e.offset == -127 and e.min == -e.max and e.delta == pytest.approx((e.max - e.min) / 254, rel=1e-6)
+    pos = np.abs(x)
+    pdf = oracle.new_pdf()
+    pdf.update(pos)
+    e = pdf.compute_percentile_encoding(8, 99.9999, sym=True, unsigned_sym=True)   # SymmetricUnsigned, :212-260
+    assert e.min == 0 and e.max == pytest.approx(pos.max(), abs=0.05) and e.offset == 0
+    pdf = oracle.new_pdf()                                                # AllSameValuesAsymmetric, :311-346
+    pdf.update(np.full(6000, 4, np.float32))
+    e = pdf.compute_percentile_encoding(8, 99.9999)
+    assert e.min <= 0 and e.max >= 3.99006
+    pdf = oracle.new_pdf()
+    pdf.update(np.full(6000, -5, np.float32))
+    e = pdf.compute_percentile_encoding(8, 99.9999)
+    assert e.min <= -4.99992 and e.max >= 0
+    pdf = oracle.new_pdf()                                                # AllZeroesAsymmetric, :348-370
+    pdf.update(np.zeros(6000, np.float32))
+    e = pdf.compute_percentile_encoding(8, 99.9999)
+    assert e.min == pytest.approx(-1.00392, abs=1e-4) and e.max == pytest.approx(0.996078, abs=1e-4)
+    assert e.offset == -128 and e.bw == 8

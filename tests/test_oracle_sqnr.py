@@ -126,3 +126,59 @@ def test_merge_keeps_mass_and_range():
     assert abs(st.histogram.sum().item() - 10000) <= 2048 * 0.5
     an.update_stats(a * 0.1)                       # inside the range: histogram simply accumulates
     assert an.stats[0].min == st.min and abs(an.stats[0].histogram.sum().item() - 14000) <= 1024
+
+
+# ------------------------------------------------------------------------------------------ percentile calibration
+def test_percentile_known_answers():
+    # test_encoding_analyzer.py:562-595: 0..1000 in 500 bins, 99 % -> [0, 990]; symmetric with 254 steps -> +-990
+    x = torch.arange(start=0, end=1001, step=1, dtype=torch.float)
+    an = sq.PercentileAnalyzer(1, 500, 99)
+    an.update_stats(x)
+    lo, hi = an.compute_encodings(math.pow(2, 8) - 1, False)
+    assert lo.item() == 0 and hi.item() == 990.0
+    lo, hi = an.compute_encodings(math.pow(2, 8) - 2, True)
+    assert lo.item() == -990.0 and hi.item() == 990.0
+
+
+def test_percentile_100_is_the_observed_range_and_non_strict_symmetric_grid():
+    # test_encoding_analyzer.py:596-622
+    an = sq.PercentileAnalyzer(1, 1, 100)
+    an.update_stats(torch.arange(start=-2, end=10, step=1, dtype=torch.float))
+    lo, hi = an.compute_encodings(pow(2, 3) - 1, True)
+    assert torch.isclose(lo, torch.tensor([-12.0])).all() and torch.isclose(hi, torch.tensor([9.0])).all()
+    torch.manual_seed(0)
+    x = torch.randn(10000) * 2 + 2
+    an = sq.PercentileAnalyzer(1, 3, 100)
+    an.update_stats(x)
+    lo, hi = an.compute_encodings(254, True)
+    assert torch.allclose(lo, -x.abs().max()) and torch.allclose(hi, x.abs().max())
+    lo, hi = an.compute_encodings(255, False)
+    assert torch.allclose(lo, x.min()) and torch.allclose(hi, x.max())
+
+
+def test_percentile_50_and_outliers():
+    # test_encoding_analyzer.py:624-655
+    x = torch.arange(start=0, end=1001, step=1, dtype=torch.float)
+    an = sq.PercentileAnalyzer(1, 3, 50)
+    an.update_stats(x)
+    st = an.stats[0]
+    cum = torch.cumsum(st.histogram, dim=0)
+    mid = st.bin_edges[torch.searchsorted(cum, torch.quantile(cum, 0.5))]
+    lo, hi = an.compute_encodings(254, True)
+    assert lo.item() == -mid.item() and hi.item() == mid.item()
+    lo, hi = an.compute_encodings(255, False)
+    assert lo.item() == 0 and hi.item() == mid.item()
+    x = torch.arange(start=0, end=101, step=1, dtype=torch.float)
+    x[-1], x[-2] = 1000, 800
+    an = sq.PercentileAnalyzer(1, 2048, 90.0)
+    an.update_stats(x)
+    lo, hi = an.compute_encodings(255, False)
+    assert 89 < hi.item() < 91
+
+
+def test_adjust_min_max_widens_degenerate_ranges():
+    eps = sq.MINIMUM_SCALE
+    lo, hi = sq.adjust_min_max(torch.tensor([0.5, 0.0]), torch.tensor([2.0, 0.0]), 255, False)
+    assert lo.tolist() == [0.0, 0.0] and hi[0] == 2.0 and hi[1].item() == pytest.approx(eps * 255)
+    lo, hi = sq.adjust_min_max(torch.tensor([0.0]), torch.tensor([0.0]), 255, True)
+    assert hi.item() == pytest.approx(127 * eps, rel=1e-6) and lo.item() == pytest.approx(-128 * eps, rel=1e-6)

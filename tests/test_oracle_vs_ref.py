@@ -171,3 +171,44 @@ def test_tf_enhanced_empty_states(oracle, ref):
     r.update(z)
     for bw in (4, 8, 16):
         assert pdf.compute_encoding(bw)[0].astuple() == r.compute_encoding(bw)
+
+
+@pytest.mark.parametrize("percentile", [100.0, 99.9999, 99.9, 99.0, 90.0, 50.0])
+def test_percentile_analyzer(oracle, ref, percentile):
+    """PercentileEncodingAnalyzer<float>: same PDF accumulation as TF-Enhanced, different computeEncoding."""
+    rng = np.random.default_rng(int(percentile * 100))
+    for kind in ("normal", "relu", "negative", "outliers", "constant", "zeros-then-data"):
+        pdf, an = oracle.new_pdf(), ref.new_percentile(percentile)
+        batches = []
+        for b in range(3):
+            x = (rng.standard_normal(20000) * (1 + b) + 0.5).astype(np.float32)
+            if kind == "relu":
+                x = np.maximum(x, 0)
+            elif kind == "negative":
+                x = -np.abs(x) - 0.25
+            elif kind == "outliers":
+                x[:5] = 300.0
+            elif kind == "constant":
+                x[:] = 4.0
+            elif kind == "zeros-then-data" and b == 0:
+                x[:] = 0.0
+            batches.append(x)
+        for x in batches:
+            pdf.update(x)
+            an.update(x)
+        for bw in (4, 8, 16):
+            for sym, strict, uns in ((False, False, False), (True, False, False), (True, True, False),
+                                     (True, False, True)):
+                got = pdf.compute_percentile_encoding(bw, percentile, sym, strict, uns)
+                want = an.compute_encoding(bw, sym, strict, uns)
+                assert got.astuple() == want, (kind, bw, sym, strict, uns)
+
+
+def test_percentile_analyzer_without_usable_statistics(oracle, ref):
+    pdf, an = oracle.new_pdf(), ref.new_percentile(99.0)
+    assert pdf.compute_percentile_encoding(8, 99.0).astuple() == an.compute_encoding(8)     # nothing seen: zeros
+    z = np.zeros(100, np.float32)
+    pdf.update(z)
+    an.update(z)
+    for bw, sym, strict in ((8, False, False), (8, True, True), (4, False, False)):
+        assert pdf.compute_percentile_encoding(bw, 99.0, sym, strict).astuple() == an.compute_encoding(bw, sym, strict)
