@@ -56,8 +56,9 @@ _SIGNATURES = {
     "miq_v2_qdq_bwd_params_workspace_bytes": ([_i64, _i64, _i64], _i64),
     "miq_v2_qdq_bwd_params_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p, _p, _p, _p], _int),
     "miq_v2_qdq_bwd_params_bf16": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p, _p, _p, _p], _int),
-    "miq_minmax_f32": ([_p, _i64, _p, _p], _int),
-    "miq_minmax_per_channel_f32": ([_p, _i64, _i64, _i64, _p, _p], _int),
+    "miq_minmax_workspace_bytes": ([_i64, _i64, _i64], _i64),
+    "miq_minmax_f32": ([_p, _i64, _p, _p, _p], _int),
+    "miq_minmax_per_channel_f32": ([_p, _i64, _i64, _i64, _p, _p, _p], _int),
     "miq_analyzer_create": ([_int, C.POINTER(_p)], _int),
     "miq_analyzer_set_percentile": ([_p, C.c_float], _int),
     "miq_analyzer_destroy": ([_p], _int),

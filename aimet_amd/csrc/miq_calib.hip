@@ -334,6 +334,113 @@ __global__ __launch_bounds__(kBlock) void minmax_rows_kernel(const float* __rest
     }
 }
 
+// The same reduction without atomics: every (row, chunk) workgroup stores its pair, 16-byte loads where the row
+// layout allows; a second kernel folds the pairs of a channel.  With one workgroup per channel (direct) the pair is
+// the result.
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void minmax_rows_partial_kernel(const float* __restrict__ in,
+                                                                     int64_t n_per_channel, int64_t chunk,
+                                                                     uint32_t chunks_per_row, float2* partial,
+                                                                     float* direct_out, int64_t num_channel)
+{
+    const int64_t row   = blockIdx.x / chunks_per_row;
+    const int64_t begin = (int64_t) (blockIdx.x % chunks_per_row) * chunk;
+    int64_t end         = begin + chunk;
+    if (end > n_per_channel)
+        end = n_per_channel;
+    const float* p = in + row * n_per_channel;
+    float mn = INFINITY, mx = -INFINITY;
+    if (VEC)
+    {
+        // the base address and chunk are multiples of 16 bytes / 4 elements on this path, and so is the row
+        // length unless there is only one row
+        const float4* v   = reinterpret_cast<const float4*>(p + begin);
+        const int64_t cnt = (end - begin) / 4;
+        int64_t i         = threadIdx.x;
+        for (; i + kBlock < cnt; i += 2 * kBlock)
+        {
+            const float4 a = v[i], b = v[i + kBlock];
+            mn = fminf(fminf(fminf(mn, a.x), fminf(a.y, a.z)), fminf(fminf(a.w, b.x), fminf(b.y, fminf(b.z, b.w))));
+            mx = fmaxf(fmaxf(fmaxf(mx, a.x), fmaxf(a.y, a.z)), fmaxf(fmaxf(a.w, b.x), fmaxf(b.y, fmaxf(b.z, b.w))));
+        }
+        if (i < cnt)
+        {
+            const float4 a = v[i];
+            mn             = fminf(fminf(mn, a.x), fminf(fminf(a.y, a.z), a.w));
+            mx             = fmaxf(fmaxf(mx, a.x), fmaxf(fmaxf(a.y, a.z), a.w));
+        }
+        // up to three trailing elements of a single row whose length is no multiple of 4
+        const int64_t tail = begin + cnt * 4 + threadIdx.x;
+        if (tail < end)
+        {
+            mn = fminf(mn, p[tail]);
+            mx = fmaxf(mx, p[tail]);
+        }
+    }
+    else
+    {
+        for (int64_t i = begin + threadIdx.x; i < end; i += kBlock)
+        {
+            const float a = p[i];
+            mn            = fminf(mn, a);
+            mx            = fmaxf(mx, a);
+        }
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    __shared__ float smn[kBlock / 64], smx[kBlock / 64];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0)
+    {
+        smn[wave] = mn;
+        smx[wave] = mx;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        for (int w = 1; w < kBlock / 64; ++w)
+        {
+            mn = fminf(mn, smn[w]);
+            mx = fmaxf(mx, smx[w]);
+        }
+        if (direct_out)
+        {
+            direct_out[blockIdx.x]               = mn;
+            direct_out[num_channel + blockIdx.x] = mx;
+        }
+        else
+            partial[blockIdx.x] = make_float2(mn, mx);
+    }
+}
+
+// One wavefront per channel folds its outer x chunks pairs.
+__global__ __launch_bounds__(kBlock) void minmax_rows_fold_kernel(const float2* __restrict__ partial,
+                                                                  int64_t num_channel, int64_t outer,
+                                                                  uint32_t chunks_per_row, float* out)
+{
+    const int64_t c = (int64_t) blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (c >= num_channel)
+        return;
+    const int lane = threadIdx.x & 63;
+    float mn = INFINITY, mx = -INFINITY;
+    for (int64_t o = 0; o < outer; ++o)
+    {
+        const float2* row = partial + (o * num_channel + c) * chunks_per_row;
+        for (uint32_t k = lane; k < chunks_per_row; k += 64)
+        {
+            mn = fminf(mn, row[k].x);
+            mx = fmaxf(mx, row[k].y);
+        }
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    if (lane == 0)
+    {
+        out[c]               = mn;
+        out[num_channel + c] = mx;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------- histogram
 // Adds one sample to the workgroup's LDS histogram.  Row kPdf is a sink for dropped samples, so the add is
 // unconditional (no divergent branch per element).
@@ -839,9 +946,42 @@ struct miq_analyzer
 
 extern "C" {
 
-static int launch_minmax_rows(const float* in, int64_t num_channel, int64_t rows, int64_t n_per_channel,
-                              uint32_t* keys, hipStream_t s)
+// chunk length and chunks per row of the workspace path: about 16 K elements per workgroup, shorter when that would
+// leave compute units idle
+static void minmax_geometry(int64_t rows, int64_t n_per_channel, int64_t& chunk, int64_t& bx)
 {
+    chunk = 16384;
+    while (chunk > 2048 && rows * ((n_per_channel + chunk - 1) / chunk) < 2048)
+        chunk /= 2;
+    bx = (n_per_channel + chunk - 1) / chunk;
+}
+
+static int launch_minmax_rows(const float* in, int64_t num_channel, int64_t rows, int64_t n_per_channel,
+                              uint32_t* keys, void* workspace, hipStream_t s)
+{
+    if (workspace && rows > 0)
+    {
+        int64_t chunk, bx;
+        minmax_geometry(rows, n_per_channel, chunk, bx);
+        MIQ_CHECK_ARG(rows * bx < (1ll << 31), "too many rows for one launch");
+        float* out        = reinterpret_cast<float*>(keys);
+        const bool direct = rows == num_channel && bx == 1;
+        const bool vec    = (n_per_channel % 4 == 0 || rows == 1) && aligned16(in);
+        float2* partial   = static_cast<float2*>(workspace);
+        const dim3 grid((unsigned) (rows * bx));
+        if (vec)
+            hipLaunchKernelGGL(minmax_rows_partial_kernel<true>, grid, dim3(kBlock), 0, s, in, n_per_channel, chunk,
+                               (uint32_t) bx, partial, direct ? out : nullptr, num_channel);
+        else
+            hipLaunchKernelGGL(minmax_rows_partial_kernel<false>, grid, dim3(kBlock), 0, s, in, n_per_channel, chunk,
+                               (uint32_t) bx, partial, direct ? out : nullptr, num_channel);
+        if (!direct)
+            hipLaunchKernelGGL(minmax_rows_fold_kernel, dim3((unsigned) ((num_channel + kBlock / 64 - 1) / (kBlock / 64))),
+                               dim3(kBlock), 0, s, partial, num_channel, rows / num_channel, (uint32_t) bx, out);
+        MIQ_CHECK_LAUNCH();
+        return MIQ_OK;
+    }
+    // without a workspace: partial results meet in the output through atomics on order-preserving integer keys
     // keys: uint32[2C] ordered keys (min block then max block); decoded in place to float at the end
     hipLaunchKernelGGL(fill_keys_kernel, dim3((unsigned) ((num_channel + kBlock - 1) / kBlock)), dim3(kBlock), 0, s,
                        keys, num_channel);
@@ -866,23 +1006,35 @@ static int launch_minmax_rows(const float* in, int64_t num_channel, int64_t rows
     return MIQ_OK;
 }
 
-int miq_minmax_f32(const float* in, int64_t n, float* out_min_max, void* stream)
+int64_t miq_minmax_workspace_bytes(int64_t num_channel, int64_t num_element, int64_t num_element_per_channel)
+{
+    if (num_channel <= 0 || num_element_per_channel <= 0 || num_element <= 0)
+        return 8;
+    int64_t chunk, bx;
+    const int64_t rows = num_element / num_element_per_channel;
+    minmax_geometry(rows, num_element_per_channel, chunk, bx);
+    return (int64_t) sizeof(float2) * std::max<int64_t>(rows * bx, 1);
+}
+
+int miq_minmax_f32(const float* in, int64_t n, float* out_min_max, void* workspace, void* stream)
 {
     MIQ_CHECK_ARG(n >= 0 && out_min_max && (n == 0 || in), "null pointer or negative count");
     return launch_minmax_rows(in, 1, n > 0 ? 1 : 0, n > 0 ? n : 1, reinterpret_cast<uint32_t*>(out_min_max),
-                              (hipStream_t) stream);
+                              workspace, (hipStream_t) stream);
 }
 
 int miq_minmax_per_channel_f32(const float* in, int64_t num_channel, int64_t num_element,
-                               int64_t num_element_per_channel, float* out_min_max, void* stream)
+                               int64_t num_element_per_channel, float* out_min_max, void* workspace, void* stream)
 {
     MIQ_CHECK_ARG(num_channel > 0 && num_element_per_channel > 0 && num_element >= 0 && out_min_max,
                   "bad channel geometry or null output");
     MIQ_CHECK_ARG(num_element == 0 || in, "null input");
     MIQ_CHECK_ARG(num_element % num_element_per_channel == 0,
                   "num_element must be a multiple of num_element_per_channel");
+    MIQ_CHECK_ARG((num_element / num_element_per_channel) % num_channel == 0,
+                  "num_element must be a multiple of num_channel * num_element_per_channel");
     return launch_minmax_rows(in, num_channel, num_element / num_element_per_channel, num_element_per_channel,
-                              reinterpret_cast<uint32_t*>(out_min_max), (hipStream_t) stream);
+                              reinterpret_cast<uint32_t*>(out_min_max), workspace, (hipStream_t) stream);
 }
 
 // PercentileEncodingAnalyzer<float>::computeEncoding on the PDF read back from the device

@@ -218,13 +218,19 @@ def v2_qdq_bwd_params(x, grad_out, num_channel, n_per_channel, scale, offset, qm
 
 
 # -------------------------------------------------------------------------------------------------------- statistics
+def _minmax_workspace(num_channel, n, n_per_channel, device):
+    nbytes = int(lib.miq_minmax_workspace_bytes(int(num_channel), int(n), int(n_per_channel)))
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
 def minmax(x):
     """float32 device tensor [min, max] of x (NaN ignored); asynchronous."""
     _require_gpu(x)
     x = x.to(_F32).contiguous()
     out = torch.empty(2, dtype=_F32, device=x.device)
+    ws = _minmax_workspace(1, x.numel(), max(x.numel(), 1), x.device)
     with torch.cuda.device(x.device):
-        check(lib.miq_minmax_f32(_ptr(x), x.numel(), _ptr(out), _stream(x)))
+        check(lib.miq_minmax_f32(_ptr(x), x.numel(), _ptr(out), _ptr(ws), _stream(x)))
     return out
 
 
@@ -233,9 +239,10 @@ def minmax_per_channel(x, num_channel, n_per_channel):
     _require_gpu(x)
     x = x.to(_F32).contiguous()
     out = torch.empty(2, num_channel, dtype=_F32, device=x.device)
+    ws = _minmax_workspace(num_channel, x.numel(), n_per_channel, x.device)
     with torch.cuda.device(x.device):
         check(lib.miq_minmax_per_channel_f32(_ptr(x), int(num_channel), x.numel(), int(n_per_channel), _ptr(out),
-                                             _stream(x)))
+                                             _ptr(ws), _stream(x)))
     return out
 
 

@@ -178,12 +178,16 @@ int miq_v2_qdq_bwd_params_bf16(const uint16_t* x, const uint16_t* grad_out, uint
  * ------------------------------------------------------------------------------------------------------------- */
 
 /* GetMin + GetMax (DLQ/src/math_functions.cpp:328-347; GPU twins math_functions.cu:52-64) fused into one pass.
- * out_min_max: device float[2] = {min, max}; NaN elements are ignored, an empty input yields {+inf, -inf}. */
-int miq_minmax_f32(const float* in, int64_t n, float* out_min_max, void* stream);
+ * out_min_max: device float[2] = {min, max}; NaN elements are ignored, an empty input yields {+inf, -inf}.
+ * workspace: device memory of miq_minmax_workspace_bytes(1, n, n) bytes, or NULL.  With a workspace the partial
+ * results of the workgroups are stored and folded by a second kernel; without one they meet in the output through
+ * atomics, which is several times slower on large tensors. */
+int64_t miq_minmax_workspace_bytes(int64_t num_channel, int64_t num_element, int64_t num_element_per_channel);
+int miq_minmax_f32(const float* in, int64_t n, float* out_min_max, void* workspace, void* stream);
 /* Per-channel form used for per-channel min/max (TF) encodings: out is device float[2*num_channel] laid out
  * {min_0..min_{C-1}, max_0..max_{C-1}}; channel(i) = (i / num_element_per_channel) % num_channel. */
 int miq_minmax_per_channel_f32(const float* in, int64_t num_channel, int64_t num_element,
-                               int64_t num_element_per_channel, float* out_min_max, void* stream);
+                               int64_t num_element_per_channel, float* out_min_max, void* workspace, void* stream);
 
 /* Encoding analyzer object = IQuantizationEncodingAnalyzer<float>
  * (DLQ/include/DlQuantization/IQuantizationEncodingAnalyzer.hpp:48-126) as instantiated by

@@ -195,6 +195,32 @@ def test_cfg3_full_size_properties(ops, oracle):
     assert valid and enc.delta > 0 and enc.min <= 0 <= enc.max
 
 
+@pytest.mark.parametrize("outer,c,npc", [(1, 1, 100003), (1, 1, 3), (1, 1, 1 << 22), (1, 300, 4096), (1, 7, 70001),
+                                         (6, 32, 784), (3, 5, 40000), (4, 1000, 9), (2, 3, 1 << 18)])
+def test_minmax_with_and_without_workspace(ops, outer, c, npc):
+    """Both reductions (stored partials folded by a second kernel; atomics on ordered keys) give the exact values."""
+    import ctypes
+    from aimet_amd._lib import check, lib
+    torch.manual_seed(outer * 1000 + c + npc)
+    x = torch.randn(outer, c, npc)
+    x.view(-1)[::97] = float("nan")                                  # NaN is ignored
+    x.view(-1)[5 % x.numel()] = -0.0
+    xg = x.cuda()
+    want_min = torch.nan_to_num(x, nan=float("inf")).amin(dim=(0, 2))
+    want_max = torch.nan_to_num(x, nan=float("-inf")).amax(dim=(0, 2))
+    got = ops.minmax_per_channel(xg, c, npc).cpu()
+    assert torch.equal(got[0], want_min) and torch.equal(got[1], want_max)
+    out = torch.empty(2, c, device="cuda")
+    check(lib.miq_minmax_per_channel_f32(xg.data_ptr(), c, xg.numel(), npc, out.data_ptr(), None,
+                                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    assert torch.equal(out.cpu(), got)
+    if c == 1:
+        flat = ops.minmax(xg.reshape(-1)[1:])                        # misaligned base: scalar loads
+        rest = x.reshape(-1)[1:]
+        assert flat[0].item() == torch.nan_to_num(rest, nan=float("inf")).min().item()
+        assert flat[1].item() == torch.nan_to_num(rest, nan=float("-inf")).max().item()
+
+
 # ------------------------------------------------------------------------------------------ percentile analyzer
 PERCENTILE = 2
 
