@@ -413,28 +413,45 @@ __global__ __launch_bounds__(kBlock) void minmax_rows_partial_kernel(const float
     }
 }
 
-// One wavefront per channel folds its outer x chunks pairs.
+// LANES lanes per channel (a wavefront, or the workgroup when a channel has many pairs) fold its outer x chunks
+// pairs.
+template <int LANES>
 __global__ __launch_bounds__(kBlock) void minmax_rows_fold_kernel(const float2* __restrict__ partial,
                                                                   int64_t num_channel, int64_t outer,
                                                                   uint32_t chunks_per_row, float* out)
 {
-    const int64_t c = (int64_t) blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
-    if (c >= num_channel)
-        return;
-    const int lane = threadIdx.x & 63;
+    const int64_t c = (int64_t) blockIdx.x * (kBlock / LANES) + threadIdx.x / LANES;
+    const int lane  = threadIdx.x % LANES;
     float mn = INFINITY, mx = -INFINITY;
-    for (int64_t o = 0; o < outer; ++o)
+    if (c < num_channel)
     {
-        const float2* row = partial + (o * num_channel + c) * chunks_per_row;
-        for (uint32_t k = lane; k < chunks_per_row; k += 64)
+        const int64_t items = outer * chunks_per_row;
+        for (int64_t j = lane; j < items; j += LANES)
         {
-            mn = fminf(mn, row[k].x);
-            mx = fmaxf(mx, row[k].y);
+            const int64_t o = j / chunks_per_row, k = j % chunks_per_row;
+            const float2 v  = partial[(o * num_channel + c) * chunks_per_row + k];
+            mn              = fminf(mn, v.x);
+            mx              = fmaxf(mx, v.y);
         }
     }
     mn = wave_min(mn);
     mx = wave_max(mx);
-    if (lane == 0)
+    if (LANES > 64)
+    {
+        __shared__ float smn[kBlock / 64], smx[kBlock / 64];
+        if ((threadIdx.x & 63) == 0)
+        {
+            smn[threadIdx.x >> 6] = mn;
+            smx[threadIdx.x >> 6] = mx;
+        }
+        __syncthreads();
+        for (int w = 0; w < kBlock / 64; ++w)
+        {
+            mn = fminf(mn, smn[w]);
+            mx = fmaxf(mx, smx[w]);
+        }
+    }
+    if (lane == 0 && c < num_channel)
     {
         out[c]               = mn;
         out[num_channel + c] = mx;
@@ -975,9 +992,12 @@ static int launch_minmax_rows(const float* in, int64_t num_channel, int64_t rows
         else
             hipLaunchKernelGGL(minmax_rows_partial_kernel<false>, grid, dim3(kBlock), 0, s, in, n_per_channel, chunk,
                                (uint32_t) bx, partial, direct ? out : nullptr, num_channel);
-        if (!direct)
-            hipLaunchKernelGGL(minmax_rows_fold_kernel, dim3((unsigned) ((num_channel + kBlock / 64 - 1) / (kBlock / 64))),
-                               dim3(kBlock), 0, s, partial, num_channel, rows / num_channel, (uint32_t) bx, out);
+        if (!direct && (rows / num_channel) * bx >= 1024)
+            hipLaunchKernelGGL(minmax_rows_fold_kernel<kBlock>, dim3((unsigned) num_channel), dim3(kBlock), 0, s, partial,
+                               num_channel, rows / num_channel, (uint32_t) bx, out);
+        else if (!direct)
+            hipLaunchKernelGGL(minmax_rows_fold_kernel<64>, dim3((unsigned) ((num_channel + 3) / 4)), dim3(kBlock), 0, s,
+                               partial, num_channel, rows / num_channel, (uint32_t) bx, out);
         MIQ_CHECK_LAUNCH();
         return MIQ_OK;
     }

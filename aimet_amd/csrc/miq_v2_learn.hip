@@ -218,20 +218,26 @@ __global__ __launch_bounds__(kBlock) void learn_bwd_kernel(const IO* __restrict_
     }
 }
 
-// One workgroup per channel: adds the channel's partials (outer x chunks of them) in double, each lane a strided
-// share in index order, then a fixed tree over the lanes.
+// Adds the partial pairs of each channel (outer x chunks of them) in double: LANES lanes per channel (a wavefront,
+// or the whole workgroup when a channel has many pairs), each lane a strided share in index order, then a fixed
+// tree over the lanes -- the result does not depend on scheduling.
+template <int LANES>
 __global__ __launch_bounds__(kBlock) void learn_reduce_kernel(const float2* __restrict__ partial, LearnGeom geo,
                                                               float* __restrict__ scale_grad,
                                                               float* __restrict__ offset_grad)
 {
-    const uint32_t ch = blockIdx.x;
+    constexpr int kPerBlock = kBlock / LANES;
+    const uint32_t ch       = blockIdx.x * kPerBlock + threadIdx.x / LANES;
+    const uint32_t lane     = threadIdx.x % LANES;
     double a = 0.0, b = 0.0;
-    for (uint32_t o = 0; o < geo.outer; ++o)
+    if (ch < geo.num_channel)
     {
-        const float2* row = partial + ((int64_t) o * geo.num_channel + ch) * geo.chunks;
-        for (uint32_t k = threadIdx.x; k < geo.chunks; k += kBlock)
+        const uint32_t items = geo.outer * geo.chunks;
+        for (uint32_t j = lane; j < items; j += LANES)
         {
-            const float2 v = row[k];
+            const uint32_t o = fastdiv(j, geo.chunks_div);
+            const uint32_t k = j - o * geo.chunks;
+            const float2 v   = partial[((int64_t) o * geo.num_channel + ch) * geo.chunks + k];
             a += (double) v.x;
             b += (double) v.y;
         }
@@ -242,15 +248,15 @@ __global__ __launch_bounds__(kBlock) void learn_reduce_kernel(const float2* __re
         a += __shfl_xor(a, o);
         b += __shfl_xor(b, o);
     }
-    __shared__ double wave_sum[2][kBlock / 64];
-    if ((threadIdx.x & 63) == 0)
+    if (LANES > 64)
     {
-        wave_sum[0][threadIdx.x >> 6] = a;
-        wave_sum[1][threadIdx.x >> 6] = b;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0)
-    {
+        __shared__ double wave_sum[2][kBlock / 64];
+        if ((threadIdx.x & 63) == 0)
+        {
+            wave_sum[0][threadIdx.x >> 6] = a;
+            wave_sum[1][threadIdx.x >> 6] = b;
+        }
+        __syncthreads();
         a = b = 0.0;
 #pragma unroll
         for (int w = 0; w < kBlock / 64; ++w)
@@ -258,6 +264,9 @@ __global__ __launch_bounds__(kBlock) void learn_reduce_kernel(const float2* __re
             a += wave_sum[0][w];
             b += wave_sum[1][w];
         }
+    }
+    if (lane == 0 && ch < geo.num_channel)
+    {
         if (scale_grad)
             scale_grad[ch] = (float) a;
         if (offset_grad)
@@ -361,27 +370,6 @@ __global__ __launch_bounds__(kBlock) void learn_rows_kernel(const IO* __restrict
     }
 }
 
-// Short rows with outer > 1: one lane per channel adds its `outer` row pairs in double, in index order.
-__global__ __launch_bounds__(kBlock) void learn_reduce_rows_kernel(const float2* __restrict__ partial, LearnGeom geo,
-                                                                   float* __restrict__ scale_grad,
-                                                                   float* __restrict__ offset_grad)
-{
-    const uint32_t ch = blockIdx.x * kBlock + threadIdx.x;
-    if (ch >= geo.num_channel)
-        return;
-    double a = 0.0, b = 0.0;
-    for (uint32_t o = 0; o < geo.outer; ++o)
-    {
-        const float2 v = partial[(int64_t) o * geo.num_channel + ch];
-        a += (double) v.x;
-        b += (double) v.y;
-    }
-    if (scale_grad)
-        scale_grad[ch] = (float) a;
-    if (offset_grad)
-        offset_grad[ch] = (float) b;
-}
-
 // rows, chunks and span for a tensor of num_channel x npc rows repeated `outer` times
 int make_learn_geom(int64_t num_channel, int64_t n, int64_t npc, int vec, LearnGeom& geo, int64_t& outer)
 {
@@ -478,11 +466,12 @@ int launch_learn(const IO* x, const IO* g, IO* gx, int64_t num_channel, int64_t 
     }
     if (!geo.direct)
     {
-        if (geo.short_rows)
-            learn_reduce_rows_kernel<<<dim3((geo.num_channel + kBlock - 1) / kBlock), kBlock, 0, stream>>>(
-                partial, geo, scale_grad, offset_grad);
+        if ((int64_t) geo.outer * geo.chunks >= 1024)
+            learn_reduce_kernel<kBlock><<<dim3(geo.num_channel), kBlock, 0, stream>>>(partial, geo, scale_grad,
+                                                                                      offset_grad);
         else
-            learn_reduce_kernel<<<dim3(geo.num_channel), kBlock, 0, stream>>>(partial, geo, scale_grad, offset_grad);
+            learn_reduce_kernel<64><<<dim3((geo.num_channel + 3) / 4), kBlock, 0, stream>>>(partial, geo, scale_grad,
+                                                                                            offset_grad);
         MIQ_CHECK_LAUNCH();
     }
     return MIQ_OK;
