@@ -7,6 +7,9 @@ context, get_min / get_max / get_scale / get_offset / set_range), Quantize (:448
 """
 import contextlib
 import functools
+import math
+import warnings
+import weakref
 from typing import Optional
 
 import torch
@@ -16,6 +19,17 @@ from ...utils import (StatisticsNotFoundError, _is_expandable, get_encoding_shap
                       reshape_tensor_for_blocks, ste_round)
 from ..encoding_analyzer import EncodingAnalyzer, MinMaxEncodingAnalyzer
 from .backends import _derive_qmin_qmax, quantize, quantize_dequantize
+
+
+def _flag_extreme_min_max(curr_min: torch.Tensor, curr_max: torch.Tensor):
+    """Warns about ranges that are not finite or sit at the edge of the dtype (reference
+    encoding_analyzer.py:388-395)."""
+    if not (torch.all(torch.isfinite(curr_min)) and torch.all(torch.isfinite(curr_max))):
+        warnings.warn('Infinite or NaN values detected within input! This may skew the associated encodings')
+    extreme = torch.full_like(curr_min, torch.finfo(curr_min.dtype).max)
+    if torch.any(torch.isclose(torch.abs(curr_min), extreme, rtol=0.05)) or \
+            torch.any(torch.isclose(torch.abs(curr_max), extreme, rtol=0.05)):
+        warnings.warn('Extreme values detected within input! This may skew the associated encodings')
 
 
 class _AffineEncoding:
@@ -84,9 +98,11 @@ class MinMaxQuantizer(nn.Module):
         if self.block_size is None and not _is_expandable(self.encoding_analyzer.observer.shape, self.shape):
             raise RuntimeError(f'Encoding analyzer of shape {self.encoding_analyzer.observer.shape} '
                                f'is incompatible with quantizer of shape {self.shape}.')
+        self._initial_parameters = {}
         self.min = nn.Parameter(-torch.ones(self.shape))
         self.max = nn.Parameter(torch.ones(self.shape))
-        self._initialized = False
+        self._remember_initial('min', self.min)
+        self._remember_initial('max', self.max)
         self._allow_overwrite = True
 
     # ---------------------------------------------------------------------------------------------- properties
@@ -98,25 +114,95 @@ class MinMaxQuantizer(nn.Module):
     def symmetric(self, symmetric: bool):
         self._symmetric = symmetric
 
+    def _grid_is_regular(self) -> bool:
+        return self.qmin + self.qmax == -1 or self.qmin == 0
+
     @property
     def bitwidth(self) -> int:
-        return (self.qmax - self.qmin).bit_length()
+        """B such that the grid is [0, 2^B - 1] or [-2^(B-1), 2^(B-1) - 1]; undefined for other grids
+        (reference affine/_utils.py:89-144)."""
+        if self._grid_is_regular():
+            bitwidth = math.log2(self.qmax - self.qmin + 1)
+            if bitwidth == int(bitwidth):
+                return int(bitwidth)
+        raise RuntimeError(f"bitwidth is undefined for a quantization grid of [{self.qmin}, {self.qmax}]")
+
+    @bitwidth.setter
+    def bitwidth(self, bitwidth: int):
+        if bitwidth == int(bitwidth):
+            bitwidth = int(bitwidth)
+        if not isinstance(bitwidth, int):
+            raise TypeError(f"Setting bitwidth to a non-integer value {bitwidth:.3f} is not supported; set "
+                            f"{type(self).__qualname__}.qmin and .qmax instead.")
+        if bitwidth < 1:
+            raise ValueError(f"Bitwidth can't be smaller than 1. Got {bitwidth}")
+        if self.qmin + self.qmax == -1:
+            self.qmin, self.qmax = -2 ** (bitwidth - 1), 2 ** (bitwidth - 1) - 1
+        elif self.qmin == 0:
+            self.qmin, self.qmax = 0, 2 ** bitwidth - 1
+        else:
+            raise RuntimeError(f"bitwidth is undefined for a quantization grid of [{self.qmin}, {self.qmax}]")
 
     @property
     def signed(self) -> bool:
-        return self.qmin < 0
+        if self._grid_is_regular():
+            return self.qmin < 0 <= self.qmax
+        raise RuntimeError(f"signed is undefined for a quantization grid of [{self.qmin}, {self.qmax}]")
+
+    @signed.setter
+    def signed(self, signed: bool):
+        """Shifts the grid between [0, 2^B - 1] and [-2^(B-1), 2^(B-1) - 1] (reference affine/_utils.py:170-188)."""
+        bitwidth = self.bitwidth
+        if signed:
+            self.qmin, self.qmax = -2 ** (bitwidth - 1), 2 ** (bitwidth - 1) - 1
+        else:
+            self.qmin, self.qmax = 0, 2 ** bitwidth - 1
+
+    # A parameter counts as initialised once it is no longer the untouched object it was created as: it has been
+    # assigned anew, or modified in place (its version counter moved) -- reference base/quantizer.py:100-140.
+    def _remember_initial(self, name: str, param: nn.Parameter):
+        self._initial_parameters[name] = (weakref.ref(param), param._version)  # pylint: disable=protected-access
+
+    def _is_initialized(self, name: str) -> bool:
+        initial_ref, initial_version = self._initial_parameters[name]
+        initial = initial_ref() if initial_ref is not None else None
+        if initial is None:
+            return True
+        current = getattr(self, name)
+        return not (current is initial and current._version == initial_version)  # pylint: disable=protected-access
 
     def is_initialized(self) -> bool:
-        return self._initialized
+        return all(self._is_initialized(name) for name in ('min', 'max'))
 
-    def __setattr__(self, name, value):
-        # assigning new min and max parameters by hand initialises the quantizer, as in the reference
-        if name in ('min', 'max') and '_initialized' in self.__dict__ and isinstance(value, nn.Parameter):
-            assigned = self.__dict__.setdefault('_assigned', set())
-            assigned.add(name)
-            if assigned >= {'min', 'max'}:
-                self.__dict__['_initialized'] = True
-        super().__setattr__(name, value)
+    def allow_overwrite(self, mode: bool):
+        """With False, compute_encodings() leaves the current parameters alone."""
+        self._allow_overwrite = mode
+
+    def get_extra_state(self):
+        return {name: torch.tensor(self._is_initialized(name)) for name in ('min', 'max')}
+
+    @torch.no_grad()
+    def set_extra_state(self, state):
+        for name in ('min', 'max'):
+            if bool(state.get(name, False)):
+                self._initial_parameters[name] = (None, -1)
+            else:
+                self._remember_initial(name, getattr(self, name))
+
+    def __getstate__(self):
+        state = self.__dict__.copy()
+        state['_initial_parameters'] = {name: self._is_initialized(name) for name in ('min', 'max')}
+        return state
+
+    def __setstate__(self, state):
+        flags = state.pop('_initial_parameters')
+        super().__setstate__(state)
+        self._initial_parameters = {}
+        for name, initialized in flags.items():
+            if initialized:
+                self._initial_parameters[name] = (None, -1)
+            else:
+                self._remember_initial(name, getattr(self, name))
 
     def extra_repr(self) -> str:
         return f'shape={self.shape}, qmin={self.qmin}, qmax={self.qmax}, symmetric={self.symmetric}'
@@ -142,8 +228,7 @@ class MinMaxQuantizer(nn.Module):
                 dyn_min, dyn_max = dyn_min.view(self.min.shape), dyn_max.view(self.max.shape)
             dyn_min = dyn_min.to(dtype=self.min.dtype, device=self.min.device).expand_as(self.min)
             dyn_max = dyn_max.to(dtype=self.max.dtype, device=self.max.device).expand_as(self.max)
-            with patch_attr(self, 'min', dyn_min), patch_attr(self, 'max', dyn_max), \
-                    patch_attr(self, '_initialized', True):
+            with patch_attr(self, 'min', dyn_min), patch_attr(self, 'max', dyn_max):
                 return original_forward(input)
 
         self.encoding_analyzer.reset_stats()
@@ -158,13 +243,13 @@ class MinMaxQuantizer(nn.Module):
             return
         if self.block_size is not None:
             enc_min, enc_max = enc_min.view(self.min.shape), enc_max.view(self.max.shape)
+        _flag_extreme_min_max(enc_min, enc_max)
         self.set_range(enc_min, enc_max)
 
     def set_range(self, min: torch.Tensor, max: torch.Tensor):  # pylint: disable=redefined-builtin
         with torch.no_grad():
             self.min.copy_(min)
             self.max.copy_(max)
-        self._initialized = True
 
     def get_scale(self, dtype=None) -> Optional[torch.Tensor]:
         if not self.is_initialized():
