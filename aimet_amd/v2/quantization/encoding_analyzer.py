@@ -276,6 +276,8 @@ class _HistogramObserver:
             return [_Histogram() for _ in range(self.num_histograms)]
         return self._state
 
+    stats = property(get_stats)          # the reference exposes the running statistics as an attribute
+
 
 def adjust_min_max(curr_min: torch.Tensor, curr_max: torch.Tensor, num_steps, is_symmetric: bool):
     """Widens a range to contain zero, keeps it finite and at least _MINIMUM_SCALE * num_steps wide; a symmetric grid

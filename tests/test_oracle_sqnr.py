@@ -182,3 +182,36 @@ def test_adjust_min_max_widens_degenerate_ranges():
     assert lo.tolist() == [0.0, 0.0] and hi[0] == 2.0 and hi[1].item() == pytest.approx(eps * 255)
     lo, hi = sq.adjust_min_max(torch.tensor([0.0]), torch.tensor([0.0]), 255, True)
     assert hi.item() == pytest.approx(127 * eps, rel=1e-6) and lo.item() == pytest.approx(-128 * eps, rel=1e-6)
+
+
+# ------------------------------------------------------------- the reference's histogram-observer cases (golden)
+def _run(an, batch):
+    an.update_stats(torch.tensor(batch, dtype=torch.float32))
+    return an.stats[0]
+
+
+@pytest.mark.parametrize("name,num_bins,steps", __import__("_hist_cases").MERGE_CASES)
+def test_histogram_merge_cases_of_the_reference(name, num_bins, steps):
+    an = sq.SqnrAnalyzer(1, num_bins)
+    for batch, mn, mx, hist, edges in steps:
+        st = _run(an, batch)
+        assert st.min.item() == pytest.approx(mn) and st.max.item() == pytest.approx(mx), name
+        if hist is not None:
+            assert st.histogram.tolist() == hist, name
+            assert torch.allclose(st.bin_edges, torch.tensor(edges, dtype=torch.float32)), name
+
+
+def test_infinite_inputs_are_clipped_to_the_finite_range():
+    import _hist_cases as hc
+    an = sq.SqnrAnalyzer(1, 10)
+    for batch, mn, mx, bins, edges in hc.INF_CASE:
+        st = _run(an, batch)
+        assert st.min.item() == mn and st.max.item() == mx
+        for b, count in bins.items():
+            assert st.histogram[b].item() == count
+        assert torch.allclose(st.bin_edges, torch.tensor(edges))
+    old = an.stats[0].histogram.clone()
+    st = _run(an, hc.INF_THIRD_BATCH)
+    assert st.histogram[0] == old[0] + 2 and st.histogram[-1] == old[-1] + 1
+    with pytest.raises(ValueError):
+        sq.SqnrAnalyzer(1, 10).update_stats(torch.tensor([hc.INF, -hc.INF, -hc.INF, hc.INF, hc.INF]))
