@@ -1,8 +1,10 @@
 """Model-walking helpers the AdaRound flow needs (the counterparts of the few functions of
 TrainingExtensions/torch/src/python/aimet_torch/utils.py that ADA/adaround_weight.py and ADA/activation_sampler.py
 call: get_device, get_named_module, get_ordered_list_of_modules, CachedDataset, ModuleData, get_all_quantizers,
-change_tensor_device_placement, in_eval_mode).  Graph questions are answered with forward hooks on one pass of the
-model instead of the reference's traced ConnectedGraph.
+change_tensor_device_placement, in_eval_mode), and the helpers of the encodings file format
+(create_encoding_dict / create_encoding_from_dict, partial encodings, per-tensor <-> per-channel quantizer swaps).
+Graph questions are answered with forward hooks on one pass of the model instead of the reference's traced
+ConnectedGraph.
 """
 import contextlib
 from typing import Any, Callable, Dict, List, Tuple, Union
@@ -188,3 +190,117 @@ def get_all_quantizers(model: nn.Module):
             input_quantizers.extend(module.input_quantizers)
             output_quantizers.extend(module.output_quantizers)
     return param_quantizers, input_quantizers, output_quantizers
+
+
+# ------------------------------------------------------------------------------------ encodings on disk (v1 format)
+# The JSON entry of one encoding is {'min', 'max', 'scale', 'offset', 'bitwidth', 'is_symmetric', 'dtype'}
+# (reference aimet_torch/utils.py:785-800, 1140-1170).
+def create_encoding_dict(encoding, quantizer, propagate_encodings: bool = False):
+    """Exportable dictionary of one TfEncoding of `quantizer`; None when there is no encoding."""
+    from .common.defs import QuantizationDataType  # pylint: disable=import-outside-toplevel
+    if quantizer.data_type == QuantizationDataType.float:
+        return {'bitwidth': quantizer.bitwidth, 'dtype': 'float'}
+    if not encoding:
+        return None
+    if propagate_encodings:
+        return {'bitwidth': encoding.bw, 'dtype': 'int'}
+    return {'min': encoding.min, 'max': encoding.max, 'scale': encoding.delta, 'offset': int(encoding.offset),
+            'bitwidth': encoding.bw, 'is_symmetric': str(quantizer.use_symmetric_encodings), 'dtype': 'int'}
+
+
+def create_encoding_from_dict(encoding_dict: dict):
+    """TfEncoding from its dictionary form."""
+    from .common import libpymo  # pylint: disable=import-outside-toplevel
+    if encoding_dict.get('is_symmetric') not in ('True', 'False'):
+        raise AssertionError(f"Unexpected value for is_symmetric: {encoding_dict.get('is_symmetric')}")
+    return libpymo.TfEncoding(encoding_dict.get('min'), encoding_dict.get('max'), encoding_dict.get('scale'),
+                              encoding_dict.get('offset'), encoding_dict.get('bitwidth'))
+
+
+def _check_is_symmetric_flag(quantizer, encoding_dict: Dict, strict: bool):
+    if 'is_symmetric' not in encoding_dict:
+        raise AttributeError("Provided encoding doesn't have 'is_symmetric' flag")
+    is_symmetric = encoding_dict['is_symmetric'] == 'True'
+    if quantizer.use_symmetric_encodings != is_symmetric and strict:
+        raise AssertionError(f"Provided 'is_symmetric' flag in encodings (set to {is_symmetric}) doesn't match with "
+                             f"quantizer setting (set to {quantizer.use_symmetric_encodings})")
+
+
+def validate_is_symmetric_flag(quantizer, encoding_dict: Dict, strict: bool = True):
+    """The 'is_symmetric' flag of an imported encoding must agree with the quantizer: always for a full encoding,
+    and for a partial one when `strict` (reference aimet_torch/utils.py:1199-1270)."""
+    if not (encoding_dict.get('max', 0) == 0 and encoding_dict.get('min', 0) == 0) and \
+            encoding_dict.get('delta', 0) != 0:
+        _check_is_symmetric_flag(quantizer, encoding_dict, strict=True)
+    _check_is_symmetric_flag(quantizer, encoding_dict, strict=strict)
+
+
+def compute_partial_encoding(quantizer, encoding_dict: Dict) -> Dict:
+    """Completes an encoding given only as (min, max) or only as (scale, offset)
+    (reference aimet_torch/utils.py:1273-1302; the arithmetic is DlQuantization's computePartialEncoding,
+    ModelOptimizations/DlQuantization/src/TensorQuantizer.cpp:327-343 and quantization_utils.cpp:158-238)."""
+    from . import ops  # pylint: disable=import-outside-toplevel
+    bw = encoding_dict.get('bitwidth')
+    e_max, e_min = encoding_dict.get('max', 0), encoding_dict.get('min', 0)
+    delta, offset = encoding_dict.get('scale', 0), encoding_dict.get('offset', 0)
+    if not (e_max == 0 and e_min == 0) and delta != 0:
+        return encoding_dict                                   # already complete
+    sym, uns, strict = quantizer.use_symmetric_encodings, quantizer.use_unsigned_symmetric, \
+        quantizer.use_strict_symmetric
+    if not bw:
+        raise ValueError("Encodings must have a valid non-zero bitwidth")
+    if e_min == 0 and e_max == 0:
+        # min / max from delta / offset
+        if delta == 0 and offset > 0:
+            raise ValueError("Encoding must have a valid non-zero delta/offset if min and max are zero")
+        num_steps = 2.0 ** bw - 1
+        if sym and strict:
+            num_steps -= 1
+        e_min = offset * delta
+        if sym and (e_min < 0.0 or not uns):
+            e_max = delta * (num_steps // 2)
+        else:
+            e_max = delta * num_steps + e_min
+        if e_max - e_min < 1e-5:                               # gateMinMax: zero inside, a real range
+            e_min, e_max = min(e_min, 0.0), max(e_max, 0.0)
+            e_max = max(e_max, e_min + 1e-5)
+    elif delta == 0:
+        # delta / offset from min / max, which are kept as given
+        if offset != 0:
+            raise ValueError("Encoding delta and offset must be zero to use this function")
+        computed = ops.get_computed_encodings(bw, e_min, e_max, sym, strict, uns)
+        delta, offset = computed.delta, computed.offset
+    else:
+        raise RuntimeError("Cannot determine how to compute partial encoding")
+    encoding_dict['max'], encoding_dict['min'] = e_max, e_min
+    encoding_dict['scale'], encoding_dict['offset'] = delta, offset
+    encoding_dict['is_symmetric'] = 'True' if quantizer.use_symmetric_encodings else 'False'
+    return encoding_dict
+
+
+def get_per_channel_quantizer_from_per_tensor(quantizer, original_module: nn.Module):
+    """Per-channel quantizer with the settings of a per-tensor one (axis 0; axis 1 for transposed convolutions)."""
+    from .v1.tensor_quantizer import StaticGridPerChannelQuantizer  # pylint: disable=import-outside-toplevel
+    channel_axis = 0
+    if isinstance(original_module, (nn.ConvTranspose1d, nn.ConvTranspose2d, nn.ConvTranspose3d)) and \
+            len(original_module.weight.shape) > 1:
+        channel_axis = 1
+    new = StaticGridPerChannelQuantizer(quantizer.bitwidth, quantizer.round_mode, quantizer.quant_scheme,
+                                        quantizer.use_symmetric_encodings,
+                                        num_channels=original_module.weight.shape[channel_axis],
+                                        enabled_by_default=quantizer.enabled, ch_axis=channel_axis,
+                                        data_type=quantizer.data_type)
+    new.use_strict_symmetric, new.use_unsigned_symmetric = quantizer.use_strict_symmetric, \
+        quantizer.use_unsigned_symmetric
+    return new
+
+
+def get_per_tensor_quantizer_from_per_channel(quantizer):
+    """Per-tensor quantizer with the settings of a per-channel one."""
+    from .v1.tensor_quantizer import StaticGridPerTensorQuantizer  # pylint: disable=import-outside-toplevel
+    new = StaticGridPerTensorQuantizer(quantizer.bitwidth, quantizer.round_mode, quantizer.quant_scheme,
+                                       quantizer.use_symmetric_encodings, enabled_by_default=quantizer.enabled,
+                                       data_type=quantizer.data_type)
+    new.use_strict_symmetric, new.use_unsigned_symmetric = quantizer.use_strict_symmetric, \
+        quantizer.use_unsigned_symmetric
+    return new

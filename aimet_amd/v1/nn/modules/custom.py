@@ -29,3 +29,23 @@ class Concat(nn.Module):
 
     def forward(self, *x):
         return torch.cat(x, dim=self._axis)
+
+
+class Divide(nn.Module):
+    @staticmethod
+    def forward(x, y):
+        return x / y
+
+
+class MatMul(nn.Module):
+    @staticmethod
+    def forward(x, y):
+        return torch.matmul(x, y)
+
+
+class Addmm(nn.Module):
+    """beta * input + alpha * (mat1 @ mat2), with the scaling factors as keyword arguments."""
+
+    @staticmethod
+    def forward(input, mat1, mat2, **kwargs):  # pylint: disable=redefined-builtin
+        return torch.addmm(input, mat1, mat2, **kwargs)

@@ -19,6 +19,9 @@ from torch import nn
 
 from ..common import libpymo
 from ..common.defs import QuantizationDataType, QuantScheme
+from ..utils import (compute_partial_encoding, create_encoding_dict, create_encoding_from_dict,
+                     get_per_channel_quantizer_from_per_tensor, get_per_tensor_quantizer_from_per_channel,
+                     validate_is_symmetric_flag)
 from . import quantsim_straight_through_grad as ste
 from .tensor_quantizer import (LearnedGridTensorQuantizer, StaticGridPerChannelQuantizer,
                                StaticGridPerTensorQuantizer, set_encoding_min_max_gating_threshold)
@@ -58,6 +61,25 @@ def tensor_quantizer_factory(bitwidth: int, round_mode, quant_scheme: QuantSchem
         return LearnedGridTensorQuantizer(bitwidth, _to_round_mode(round_mode), quant_scheme,
                                           use_symmetric_encodings, enabled_by_default, data_type)
     raise AssertionError("Unsupported quant_scheme: " + str(quant_scheme))
+
+
+def get_encoding_by_quantizer(quantizer):
+    """The encoding a quantizer is exported with: learned-grid quantizers report the one their quant scheme means
+    (reference :1507-1519)."""
+    if isinstance(quantizer, LearnedGridTensorQuantizer):
+        return quantizer.get_effective_encoding()
+    return quantizer.encoding
+
+
+def export_quantizer_encoding(quantizer):
+    """List of encoding dictionaries of an enabled quantizer, else None (reference :1522-1538)."""
+    if not quantizer.enabled:
+        return None
+    encoding = get_encoding_by_quantizer(quantizer)
+    if isinstance(encoding, list):
+        return [create_encoding_dict(enc, quantizer, False) for enc in encoding]
+    entry = create_encoding_dict(encoding, quantizer, False)
+    return [entry] if entry else None
 
 
 class QcQuantizeWrapper(nn.Module):
@@ -125,6 +147,147 @@ class QcQuantizeWrapper(nn.Module):
             quantizer.reset_encoding_stats()
         for quantizer in self.input_quantizers:
             quantizer.reset_encoding_stats()
+
+    # ------------------------------------------------------------------------------- encodings in / out
+    def export_param_encodings(self):
+        """{parameter name: list of encoding dictionaries, or None} (reference :481-485)."""
+        return {name: export_quantizer_encoding(q) for name, q in self.param_quantizers.items()}
+
+    def export_output_encodings(self):
+        return [export_quantizer_encoding(q) for q in self.output_quantizers]
+
+    def export_input_encodings(self):
+        return [export_quantizer_encoding(q) for q in self.input_quantizers]
+
+    def set_param_encoding(self, module_name: str, param_encodings: dict, ignore_when_quantizer_disabled: bool = False,
+                           disable_quantizer_without_encoding: bool = True):
+        """Sets the parameter encodings found under '<module_name>.<parameter>' (reference :399-420)."""
+        mine = {name: param_encodings[f'{module_name}.{name}'] for name in self.param_quantizers
+                if f'{module_name}.{name}' in param_encodings}
+        self.import_param_encodings(mine, strict=not ignore_when_quantizer_disabled,
+                                    partial=not disable_quantizer_without_encoding, requires_grad=None,
+                                    allow_overwrite=None)
+
+    def set_activation_encoding(self, module_name: str, activation_encodings: dict,
+                                ignore_when_quantizer_disabled: bool = False,
+                                disable_quantizer_without_encoding: bool = True):
+        """Sets input / output encodings found under activation_encodings[module_name] (reference :363-397)."""
+        entry = activation_encodings.get(module_name, {})
+        for kind, fn in (('input', self.import_input_encodings), ('output', self.import_output_encodings)):
+            fn(entry.get(kind, {}), strict=not ignore_when_quantizer_disabled,
+               partial=not disable_quantizer_without_encoding, requires_grad=None, allow_overwrite=None)
+
+    def freeze_param_encoding(self, module_name: str, param_encodings: dict):
+        for name, quantizer in self.param_quantizers.items():
+            if f'{module_name}.{name}' in param_encodings and quantizer.enabled:
+                quantizer.freeze_encoding()
+
+    def freeze_activation_encoding(self, name: str, activation_encoding: dict):
+        for input_quantizer, output_quantizer in zip(self.input_quantizers, self.output_quantizers):
+            if name in activation_encoding:
+                if QUANTIZER_TYPE_INPUT in activation_encoding[name] and input_quantizer.enabled:
+                    input_quantizer.freeze_encoding()
+                if QUANTIZER_TYPE_OUTPUT in activation_encoding[name] and output_quantizer.enabled:
+                    output_quantizer.freeze_encoding()
+
+    @staticmethod
+    def _apply_int_encoding(quantizer, dicts, strict: bool):
+        """Symmetry flags, bitwidth and the (completed) encodings of an 'int' entry onto one quantizer."""
+        validate_is_symmetric_flag(quantizer, dicts[0], strict)
+        is_symmetric = dicts[0]['is_symmetric'] == 'True'
+        quantizer.use_symmetric_encodings = is_symmetric
+        quantizer.use_unsigned_symmetric = quantizer.use_unsigned_symmetric if is_symmetric else False
+        quantizer.use_strict_symmetric = quantizer.use_strict_symmetric if is_symmetric else False
+        dicts = [compute_partial_encoding(quantizer, dict(d)) for d in dicts]
+        quantizer.bitwidth = dicts[0]['bitwidth']
+        encodings = [create_encoding_from_dict(d) for d in dicts]
+        per_channel = isinstance(quantizer, StaticGridPerChannelQuantizer) or \
+            (isinstance(quantizer, LearnedGridTensorQuantizer) and len(encodings) > 1)
+        quantizer.encoding = encodings if per_channel else encodings[0]
+        quantizer.data_type = QuantizationDataType.int
+
+    @staticmethod
+    def _finish_import(quantizer, requires_grad, allow_overwrite):
+        if requires_grad is not None and isinstance(quantizer, LearnedGridTensorQuantizer) and quantizer.wrapper_ref:
+            getattr(quantizer.wrapper_ref, quantizer.name + '_encoding_min').requires_grad_(requires_grad)
+            getattr(quantizer.wrapper_ref, quantizer.name + '_encoding_max').requires_grad_(requires_grad)
+        if allow_overwrite is not None and not allow_overwrite and quantizer.encoding is not None:
+            quantizer.freeze_encoding()
+
+    def import_param_encodings(self, encodings, strict: bool, partial: bool, requires_grad, allow_overwrite):
+        """Imports {'parameter name': [dict, ...]} (reference :499-585).  strict: raise on a mismatch between the
+        encodings and the quantizers instead of adapting; partial: leave quantizers without an entry alone instead
+        of disabling them; allow_overwrite False freezes what was imported."""
+        # pylint: disable=protected-access
+        for name, quantizer in list(self.param_quantizers.items()):
+            if quantizer._is_encoding_frozen:
+                continue
+            encoding = encodings.get(name, None)
+            if not encoding:
+                if not partial:
+                    quantizer.enabled = False
+                continue
+            if not quantizer.enabled:
+                if strict:
+                    raise RuntimeError("The quantsim passed for loading encodings does not have the same "
+                                       "configuration as the quantsim which was used to export the encodings")
+                continue
+            if isinstance(quantizer, StaticGridPerChannelQuantizer) and len(quantizer._cppOp) != len(encoding):
+                assert len(encoding) == 1, (f'Number of Per Channel encodings provided ({len(encoding)}) is not same '
+                                            f'as number of channels ({len(quantizer._cppOp)})')
+                if strict:
+                    raise ValueError(f"Invalid PerChannel encodings for {name}, the quantizer is a "
+                                     f"PerChannelQuantizer. To avoid this, disable per_channel_quantization")
+                quantizer = get_per_tensor_quantizer_from_per_channel(quantizer)
+                self.param_quantizers[name] = quantizer
+            elif isinstance(quantizer, StaticGridPerTensorQuantizer) and len(encoding) != 1:
+                if strict:
+                    raise ValueError(f"Invalid PerTensor encodings for {name}, the quantizer is a "
+                                     f"PerTensorQuantizer. To avoid this, enable per_channel_quantization")
+                quantizer = get_per_channel_quantizer_from_per_tensor(quantizer, self.get_original_module())
+                assert len(quantizer._cppOp) == len(encoding), \
+                    f'Number of per channel encodings ({len(encoding)}) should match the number of output channels'
+                self.param_quantizers[name] = quantizer
+            if encoding[0]['dtype'] == 'int':
+                self._apply_int_encoding(quantizer, encoding, strict)
+            elif encoding[0]['dtype'] == 'float':
+                raise RuntimeError("float encodings are not implemented")
+            else:
+                raise RuntimeError("Data type does not match int or float in encodings file")
+            self._finish_import(quantizer, requires_grad, allow_overwrite)
+
+    def import_output_encodings(self, encodings, strict: bool, partial: bool, requires_grad, allow_overwrite):
+        """Imports {'0': dict, '1': dict, ...} for the output quantizers (reference :588-676)."""
+        self._import_encoding(encodings, self.output_quantizers, strict, partial, requires_grad, allow_overwrite)
+
+    def import_input_encodings(self, encodings, strict: bool, partial: bool, requires_grad, allow_overwrite):
+        self._import_encoding(encodings, self.input_quantizers, strict, partial, requires_grad, allow_overwrite)
+
+    def _import_encoding(self, encodings, quantizers, strict, partial, requires_grad, allow_overwrite):
+        for i, quantizer in enumerate(quantizers):
+            if quantizer._is_encoding_frozen:  # pylint: disable=protected-access
+                continue
+            encoding = encodings.get(str(i), None)
+            if not encoding:
+                if not partial:
+                    quantizer.enabled = False
+                continue
+            if not quantizer.enabled:
+                if not strict:
+                    continue
+                raise RuntimeError("The quantsim passed for loading encodings does not have the same "
+                                   "configuration as the quantsim which was used to export the encodings")
+            if encoding['dtype'] == 'int':
+                self._apply_int_encoding(quantizer, [encoding], strict)
+            elif encoding['dtype'] == 'float':
+                raise RuntimeError("float encodings are not implemented")
+            else:
+                raise RuntimeError("Unrecognized encodings datatype")
+            self._finish_import(quantizer, requires_grad, allow_overwrite)
+
+    def enable_per_channel_quantization(self):
+        """Changes the parameter quantizers to per-channel mode where the wrapper type supports it (static grid);
+        a no-op otherwise (reference :355-361)."""
 
     def should_perform_quant_dequant(self, tensor: torch.Tensor, tensor_quantizer) -> bool:
         """Only floating point tensors with an enabled quantizer are quantized (reference :452-468)."""

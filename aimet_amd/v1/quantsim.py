@@ -407,21 +407,58 @@ class QuantizationSimModel:
             json.dump(self.get_encodings_dict(), f, sort_keys=True, indent=4)
         return file
 
+    def load_encodings(self, encodings, strict: bool = True, partial: bool = True, requires_grad=None,
+                       allow_overwrite: bool = True):
+        """Imports parameter and activation encodings from a dictionary or a JSON file
+        (reference quantsim.py:1695-1836).
+
+        strict: raise when the file names modules / parameters the model does not have, or when an encoding cannot
+        be set as the quantizers are configured.  partial: quantizers without an entry are left alone (otherwise
+        they are disabled).  requires_grad: for learned-grid quantizers, whether the imported min / max train.
+        allow_overwrite: False freezes every imported encoding."""
+        if isinstance(encodings, (str, os.PathLike)):
+            with open(encodings) as f:
+                encodings = json.load(f)
+        if 'param_encodings' not in encodings:
+            param_encodings, activation_encodings = encodings, {}      # the older AdaRound export: parameters only
+        else:
+            param_encodings = encodings.get('param_encodings', {})
+            activation_encodings = encodings.get('activation_encodings', {})
+        if not param_encodings and not activation_encodings:
+            raise RuntimeError("the encodings hold neither parameter nor activation entries")
+        if strict:
+            model_keys = set()
+            for name, module in self.model.named_modules():
+                model_keys.add(name.replace("._module_to_wrap", ""))
+                for pname, _ in module.named_parameters(recurse=False):
+                    model_keys.add(f"{name}.{pname}".replace("._module_to_wrap", ""))
+            missing = (set(param_encodings) | set(activation_encodings)) - model_keys
+            if missing:
+                raise RuntimeError("Encoding dictionary contains modules/parameters that doesn't exist in the "
+                                   f"model: {', '.join(sorted(missing))}")
+        for name, wrapper in self.quant_wrappers():
+            try:
+                mine = {pname: param_encodings[f'{name}.{pname}'] for pname in wrapper.param_quantizers
+                        if f'{name}.{pname}' in param_encodings}
+                wrapper.import_param_encodings(mine, strict, partial, requires_grad, allow_overwrite)
+                entry = activation_encodings.get(name, {})
+                wrapper.import_input_encodings(entry.get('input', {}), strict, partial, requires_grad,
+                                               allow_overwrite)
+                wrapper.import_output_encodings(entry.get('output', {}), strict, partial, requires_grad,
+                                                allow_overwrite)
+            except RuntimeError as e:
+                raise RuntimeError(f"Encoding import failed for module: {name}.\n{e}") from e
+
+    def load_and_freeze_encodings(self, encoding_path: str, ignore_when_quantizer_disabled: bool = False):
+        """Sets parameter and activation encodings from a file exported by this class and freezes them
+        (reference :1758-1773)."""
+        self.load_encodings(encoding_path, strict=not ignore_when_quantizer_disabled, partial=True,
+                            requires_grad=False, allow_overwrite=False)
+
     def set_and_freeze_param_encodings(self, encoding_path: str):
-        """Loads parameter encodings written by export_encodings / Adaround and freezes them
-        (reference quantsim.py:1695-1756, qc_quantize_op.py:499-560)."""
-        from ..common import libpymo
+        """Sets and freezes the parameter encodings of a file written by export_encodings / Adaround
+        (reference :1838-1854)."""
         with open(encoding_path) as f:
-            data = json.load(f)
-        param_encodings = data.get('param_encodings', data)
-        for name, w in self.quant_wrappers():
-            for pname, q in w.param_quantizers.items():
-                key = f"{name}.{pname}"
-                if key in param_encodings:
-                    encs = [libpymo.TfEncoding(e['min'], e['max'], e['scale'], e['offset'], e['bitwidth'])
-                            for e in param_encodings[key]]
-                    q.enabled = True
-                    q.bitwidth = encs[0].bw
-                    q.use_symmetric_encodings = param_encodings[key][0]['is_symmetric'] == 'True'
-                    q.encoding = encs if isinstance(q.encoding, list) or len(encs) > 1 else encs[0]
-                    q.freeze_encoding()
+            encodings = json.load(f)
+        encodings.pop('activation_encodings', None)
+        self.load_encodings(encodings, strict=True, partial=True, requires_grad=False, allow_overwrite=False)

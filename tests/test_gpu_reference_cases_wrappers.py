@@ -1,0 +1,406 @@
+"""The cases of the reference's own wrapper tests (TrainingExtensions/torch/test/python/test_qc_quantize_op.py) on the
+GPU path: static-grid and learned-grid wrappers, gradient gating, quantize-only known answers, frozen encodings,
+encodings import / export, pickling, dtype preservation."""
+import copy
+import pickle
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = torch.device("cuda")
+
+
+@pytest.fixture(scope="module")
+def api():
+    from aimet_amd.common import libpymo
+    from aimet_amd.common.defs import QuantizationDataType, QuantScheme
+    from aimet_amd.v1 import qc_quantize_op as qop
+    from aimet_amd.v1 import tensor_quantizer as tq
+    from aimet_amd.v1.nn.modules import custom
+
+    class Api:
+        pass
+    a = Api()
+    a.libpymo, a.QuantScheme, a.QuantizationDataType, a.qop, a.tq, a.custom = libpymo, QuantScheme, \
+        QuantizationDataType, qop, tq, custom
+    a.nearest = libpymo.RoundingMode.ROUND_NEAREST
+    return a
+
+
+def _enc(api, bw, mx, mn, delta, offset):
+    return api.libpymo.TfEncoding(mn, mx, delta, offset, bw)
+
+
+def _static(api, module, **kw):
+    return api.qop.StaticGridQuantWrapper(module, weight_bw=8, activation_bw=8, round_mode='nearest',
+                                          quant_scheme=kw.pop("scheme", api.QuantScheme.post_training_tf_enhanced),
+                                          **kw)
+
+
+def _learned(api, module, **kw):
+    return api.qop.LearnedGridQuantWrapper(module, weight_bw=kw.pop("weight_bw", 8),
+                                           activation_bw=kw.pop("activation_bw", 8), round_mode='nearest',
+                                           quant_scheme=api.QuantScheme.training_range_learning_with_tf_init,
+                                           device=DEV, **kw)
+
+
+# ------------------------------------------------------------------------------------------------ static grid
+def test_update_stats_and_quantize_dequantize(api):
+    # :59-100
+    conv = torch.nn.Conv2d(4, 4, 1).cuda()
+    wrapper = _static(api, conv)
+    x = torch.randn(4, 4, 2, 2, device=DEV, requires_grad=True)
+    wrapper.set_mode(api.qop.QcQuantizeOpMode.ANALYSIS)
+    wrapper(x)
+    wrapper.compute_encoding()
+    enc = wrapper.output_quantizers[0].encoding
+    assert enc.bw == 8 and enc.min <= 0 <= enc.max and enc.delta > 0
+    wrapper.set_mode(api.qop.QcQuantizeOpMode.ACTIVE)
+    out = wrapper(x)
+    assert out.min().item() >= enc.min - 1e-6 and out.max().item() <= enc.max + 1e-6
+
+
+def test_qc_post_training_wrapper_gates_gradients(api):
+    # :102-159: gradients outside the (new) encoding range are cut for input, output and weight
+    torch.manual_seed(0)
+    encodings = _enc(api, 8, 0.5, -1, 1, 0.2)
+    encodings_new = _enc(api, 8, 0.4, -0.98, 1, 0.2)
+    output_grad = []
+    conv1 = torch.nn.Conv2d(1, 2, 1).cuda()
+    wrapper = _static(api, conv1)
+    wrapper.train()
+    conv1.register_full_backward_hook(lambda m, grad_in, grad_out: output_grad.append(grad_out[0]))
+    wrapper.input_quantizers[0].enabled = True
+    wrapper.output_quantizers[0].enabled = True
+    wrapper.input_quantizers[0].encoding = encodings
+    wrapper.output_quantizers[0].encoding = encodings
+    new_input = torch.tensor([[[[0.6469]]], [[[-0.9]]]], device=DEV, requires_grad=True)
+    wrapper.set_mode(api.qop.QcQuantizeOpMode.ACTIVE)
+    out = wrapper(new_input)
+    wrapper.input_quantizers[0].encoding = encodings_new
+    wrapper.output_quantizers[0].encoding = encodings_new
+    wrapper.param_quantizers['weight'].encoding = encodings_new
+    out.flatten().sum().backward()
+    for i, val in enumerate(new_input.flatten()):
+        if encodings_new.min > val or val > encodings_new.max:
+            assert new_input.grad.flatten()[i] == 0.0
+    raw = conv1(wrapper.input_quantizers[0].quantize_dequantize(new_input.detach(), api.nearest)).flatten()
+    gated = output_grad[0].flatten()
+    for i, val in enumerate(raw):
+        assert gated[i] == (1.0 if encodings_new.min <= val <= encodings_new.max else 0.0)
+    for i, val in enumerate(conv1.weight.flatten()):
+        if encodings_new.min > val or val > encodings_new.max:
+            assert conv1.weight.grad.flatten()[i] == 0.0
+
+
+@pytest.mark.parametrize("symmetric,unsigned,mx,mn,offset,inp,expected", [
+    (False, False, 2.23, -5.19, -178, [-7, -5, -3, 0, .1, 2.5], [-128., -122., -53., 50., 53., 127.]),    # :304-326
+    (True, False, 5.19, -5.20, -128, [-7, -5, -3, 0, .1, 2.5], [-128, -123, -74, 0, 2, 61]),               # :328-350
+    (True, True, 5.19, 0.0, 0, [0, 1.2, 1.5, 4.0, 4.9, 5.3], [0., 59., 74., 197., 241., 255.]),            # :352-379
+])
+def test_quantize_only_known_answers(api, symmetric, unsigned, mx, mn, offset, inp, expected):
+    quantizer = api.tq.StaticGridPerTensorQuantizer(8, api.nearest, api.QuantScheme.post_training_tf,
+                                                    use_symmetric_encodings=symmetric, enabled_by_default=True)
+    quantizer.use_unsigned_symmetric = unsigned
+    quantizer.is_unsigned_symmetric = unsigned
+    e = api.libpymo.TfEncoding()
+    e.bw, e.max, e.min, e.offset = 8, mx, mn, offset
+    quantizer.encoding = e
+    out = quantizer.quantize(torch.tensor(inp, device=DEV), api.nearest)
+    assert torch.equal(out, torch.tensor(expected, dtype=torch.float32, device=DEV))
+
+
+def test_compute_encoding_with_no_stats_and_ste_function(api):
+    # :405-425
+    quantizer = api.tq.StaticGridPerTensorQuantizer(8, api.nearest, api.QuantScheme.post_training_tf_enhanced,
+                                                    use_symmetric_encodings=False, enabled_by_default=True)
+    quantizer.compute_encoding()
+    assert quantizer._encoding == []                               # pylint: disable=protected-access
+    inputs = torch.randn(3, requires_grad=True, device=DEV)
+    outputs = api.qop.SteGatingFuncForParameters.apply(None, inputs)
+    outputs = [out.clone() for out in outputs]
+    outputs = [out.copy_(torch.randn(3, device=DEV)) for out in outputs]          # must not raise
+    assert len(outputs) == 1
+
+
+def test_prefreezed_encodings(api):
+    # :427-474
+    torch.manual_seed(2023)
+    x = torch.randn((4, 200), device=DEV)
+    linear = torch.nn.Linear(200, 100, bias=False).cuda()
+    with torch.no_grad():
+        linear.weight.copy_(torch.randn((100, 200)).clamp(-1, 1))
+    wrapper = _static(api, linear, scheme=api.QuantScheme.post_training_tf)
+    for kind in ("input_quantizers", "output_quantizers"):
+        getattr(wrapper, kind)[0].enabled = True
+    gated_wrapper = copy.deepcopy(wrapper)
+    assert torch.allclose(wrapper(x), gated_wrapper(x), rtol=0.1)
+    enc = _enc(api, 8, 0.5, -0.5, 1, 0.2)
+    for kind in ("input_quantizers", "output_quantizers"):
+        quantizers = getattr(gated_wrapper, kind)
+        quantizers[0].encoding = enc
+        quantizers[0]._is_encoding_frozen = True                   # pylint: disable=protected-access
+        assert not torch.allclose(wrapper(x), gated_wrapper(x), rtol=0.1)
+        quantizers[0]._is_encoding_frozen = False                  # pylint: disable=protected-access
+        quantizers[0].encoding = None
+        assert torch.allclose(wrapper(x), gated_wrapper(x), rtol=0.1)
+
+
+def test_wrapper_for_in_place_operation_and_param_switches(api):
+    # :803-842
+    wrapper = _static(api, torch.nn.Conv2d(3, 4, 2).cuda())
+    x = torch.randn(1, 3, 8, 8, device=DEV, requires_grad=True)
+    wrapper.set_mode(api.qop.QcQuantizeOpMode.ANALYSIS)
+    output = wrapper(x)
+    output += output
+    wrapper.compute_encoding()
+    wrapper.set_mode(api.qop.QcQuantizeOpMode.ACTIVE)
+    output = wrapper(x)
+    output += output
+    wrapper.param_quantizers['bias'].enabled = False
+    wrapper.enable_param_quantizers(enabled=True)
+    assert wrapper.param_quantizers['weight'].enabled and not wrapper.param_quantizers['bias'].enabled
+    wrapper.enable_param_quantizers(enabled=False, param_name_to_exclude=("weight",))
+    assert wrapper.param_quantizers['weight'].enabled and not wrapper.param_quantizers['bias'].enabled
+    wrapper.param_quantizers['bias'].enabled = True
+    wrapper.enable_param_quantizers(enabled=False, param_name_to_exclude=None)
+    assert not wrapper.param_quantizers['weight'].enabled and not wrapper.param_quantizers['bias'].enabled
+
+
+PARAM_ENCODINGS = {'conv1.weight': [{'bitwidth': 4, 'is_symmetric': 'False', 'max': 0.3, 'min': -0.2,
+                                     'offset': -7.0, 'scale': 0.038, 'dtype': 'int'}]}
+
+
+def test_set_and_freeze_param_encoding_static(api):
+    # :844-866
+    wrapper = _static(api, torch.nn.Conv2d(4, 4, 1).cuda())
+    wrapper.set_param_encoding('conv1', PARAM_ENCODINGS)
+    wrapper.freeze_param_encoding('conv1', PARAM_ENCODINGS)
+    q = wrapper.param_quantizers['weight']
+    assert q.encoding.bw == 4 and q.encoding.offset == -7.0 and q.encoding.delta == 0.038
+    assert not q.use_symmetric_encodings and q.bitwidth == 4
+    wrapper.reset_encodings()
+    assert wrapper.param_quantizers['weight'].encoding                 # frozen: survives a reset
+    # the frozen encoding is what the forward pass uses
+    out = wrapper(torch.randn(1, 4, 3, 3, device=DEV))
+    assert torch.isfinite(out).all()
+
+
+def test_set_and_freeze_param_encoding_learned(api):
+    # :868-901
+    wrapper = _learned(api, torch.nn.Conv2d(4, 4, 1).cuda())
+    wrapper.param_quantizers['weight'].encoding = _enc(api, 8, 0.5, -1, 1, 0.2)
+    wrapper.param_quantizers['weight'].bitwidth = 4
+    wrapper.set_param_encoding('conv1', PARAM_ENCODINGS)
+    wrapper.freeze_param_encoding('conv1', PARAM_ENCODINGS)
+    for _ in range(2):
+        q = wrapper.param_quantizers['weight']
+        assert q.encoding.bw == 4 and np.isclose(q.encoding.min, -0.2, atol=0.02) and np.isclose(q.encoding.max, 0.3)
+        assert not q.use_symmetric_encodings
+        with pytest.raises(RuntimeError):
+            wrapper.param_quantizers['weight'].encoding = _enc(api, 8, 0.4, -0.98, 1, 0.2)
+
+
+@pytest.mark.parametrize("kind", ["static", "learned"])
+def test_wrapper_pickle_unpickle(api, kind):
+    # :903-1003
+    conv = torch.nn.Conv2d(1, 32, 5).cuda()
+    wrapper = _static(api, conv) if kind == "static" else _learned(api, conv)
+    enc = _enc(api, 8, 0.5, -1, 0.01, 50)
+    for q in (wrapper.input_quantizers[0], wrapper.param_quantizers['weight'], wrapper.param_quantizers['bias'],
+              wrapper.output_quantizers[0]):
+        q.enabled = True
+        q.encoding = enc
+    assert wrapper.output_quantizers[0].encoding.min == pytest.approx(enc.min, abs=1e-6)
+    wrapper.output_quantizers[0].freeze_encoding()
+    loaded = pickle.loads(pickle.dumps(wrapper))
+    # pylint: disable=protected-access
+    assert loaded.output_quantizers[0]._is_encoding_frozen
+    assert not loaded.input_quantizers[0]._is_encoding_frozen
+    assert not loaded.param_quantizers['weight']._is_encoding_frozen
+    assert not loaded.param_quantizers['bias']._is_encoding_frozen
+    for q in (loaded.param_quantizers['weight'], loaded.param_quantizers['bias'], loaded.output_quantizers[0],
+              loaded.input_quantizers[0]):
+        assert q.encoding.max == pytest.approx(0.5, abs=1e-6)
+    enc_new = _enc(api, 8, 0.4, -0.98, 1, 0.2)
+    loaded.param_quantizers['weight'].encoding = enc_new
+    loaded.param_quantizers['bias'].encoding = enc_new
+    loaded.input_quantizers[0].encoding = enc_new
+    with pytest.raises(RuntimeError):
+        loaded.output_quantizers[0].encoding = enc_new
+    assert torch.isfinite(loaded(torch.rand(1, 1, 8, 8, device=DEV))).all()
+
+
+@pytest.mark.parametrize("kind", ["static", "learned"])
+def test_wrapper_with_kwargs(api, kind):
+    # :1067-1088
+    make = _static if kind == "static" else _learned
+    wrapper = make(api, api.custom.Addmm(), num_inputs=3, num_outputs=1)
+    for q in wrapper.input_quantizers + wrapper.output_quantizers:
+        q.enabled = False
+    a, b, c = (torch.randn(s, device=DEV) for s in ((2, 3), (2, 3), (3, 3)))
+    out1 = wrapper(a, b, c, beta=1, alpha=1)
+    out2 = wrapper(a, b, c, beta=1)
+    out3 = wrapper(a, b, c)
+    assert out1.shape == out2.shape == out3.shape and torch.equal(out1, out3)
+
+
+@pytest.mark.parametrize("kind", ["static", "learned"])
+def test_export_quantizer_encodings(api, kind):
+    # :1090-1130
+    make = _static if kind == "static" else _learned
+    wrapper = make(api, torch.nn.Linear(10, 10).cuda(), num_inputs=2, num_outputs=2)
+    wrapper.input_quantizers[0].enabled, wrapper.input_quantizers[1].enabled = True, False
+    wrapper.output_quantizers[0].enabled, wrapper.output_quantizers[1].enabled = False, True
+    wrapper.param_quantizers["weight"].enabled, wrapper.param_quantizers["bias"].enabled = True, False
+    encoding = api.libpymo.TfEncoding(-128.0, 127.0, 1.0, -128, 8)
+    as_dict = {"min": -128.0, "max": 127.0, "scale": 1.0, "offset": -128, "bitwidth": 8, "is_symmetric": "False",
+               "dtype": "int"}
+    wrapper.enable_per_channel_quantization()
+    wrapper.param_quantizers["weight"].encoding = [encoding] * 10
+    wrapper.input_quantizers[0].encoding = encoding
+    wrapper.output_quantizers[1].encoding = encoding
+    input_encodings = wrapper.export_input_encodings()
+    output_encodings = wrapper.export_output_encodings()
+    param_encodings = wrapper.export_param_encodings()
+
+    def same(got, want):
+        return all(g[k] == pytest.approx(want[k]) if isinstance(want[k], float) else g[k] == want[k]
+                   for g in got for k in want)
+    assert len(input_encodings) == 2 and same(input_encodings[0], as_dict) and input_encodings[1] is None
+    assert len(output_encodings) == 2 and output_encodings[0] is None and same(output_encodings[1], as_dict)
+    assert set(param_encodings) == {"weight", "bias"} and param_encodings["bias"] is None
+    assert len(param_encodings["weight"]) == 10 and same(param_encodings["weight"], as_dict)
+
+
+# ----------------------------------------------------------------------------------------------- learned grid
+def test_trainable_tensor_quantizer_forward(api):
+    # :487-530: outputs stay inside the grid implied by min / max
+    q = api.tq.LearnedGridTensorQuantizer(8, 'nearest', api.QuantScheme.training_range_learning_with_tf_init,
+                                          use_symmetric_encodings=True, enabled_by_default=True,
+                                          data_type=api.QuantizationDataType.int)
+    for is_unsigned, emin in ((True, -5.0), (True, 0.0), (False, -5.0), (False, -1.0)):
+        q.is_unsigned_symmetric = is_unsigned
+        encoding_min = torch.nn.Parameter(torch.tensor([emin], device=DEV))
+        encoding_max = torch.nn.Parameter(torch.tensor([5.0], device=DEV))
+        tensor = torch.empty(2, 1, 3, 5, device=DEV).uniform_(-10, 10)
+        out = q.quantize_dequantize(tensor, encoding_min, encoding_max)
+        if is_unsigned:
+            min_val, grid_length = emin, (5 - emin) / (2 ** 8 - 1)
+        else:
+            min_val = -5.0
+            grid_length = (5 - min_val) / (2 ** 8 - 2)
+        assert out.max().item() <= 5 + grid_length and out.min().item() >= min_val - grid_length
+
+
+def test_custom_gradient_math_for_range_learning(api):
+    # :532-622: against autograd of the explicit expression with a straight-through round
+    torch.manual_seed(0)
+    custom_input = torch.rand((100, 100), requires_grad=True)
+    _min, _max = -0.5, 0.9
+
+    class Ste(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x):                                       # pylint: disable=arguments-differ
+            return torch.round(x)
+
+        @staticmethod
+        def backward(ctx, g):                                      # pylint: disable=arguments-differ
+            return g
+    a_input = custom_input.detach().clone().requires_grad_(True)
+    a_min, a_max = torch.nn.Parameter(torch.tensor([_min])), torch.nn.Parameter(torch.tensor([_max]))
+    delta = (a_max - a_min) / 255.0
+    offset = Ste.apply(a_min / delta)
+    y = (torch.clamp(Ste.apply(a_input / delta) - offset, 0.0, 255.0) + offset) * delta
+    y.flatten().sum().backward()
+    oc_input = custom_input.detach().clone().cuda().requires_grad_(True)
+    oc_min, oc_max = torch.nn.Parameter(torch.tensor([_min], device=DEV)), \
+        torch.nn.Parameter(torch.tensor([_max], device=DEV))
+    q = api.tq.LearnedGridTensorQuantizer(8, "nearest", api.QuantScheme.training_range_learning_with_tf_init,
+                                          use_symmetric_encodings=False, enabled_by_default=True,
+                                          data_type=api.QuantizationDataType.int)
+    api.tq.QuantizeDequantizeFunc.apply(oc_input, oc_min, oc_max, q).flatten().sum().backward()
+    assert torch.allclose(a_input.grad, oc_input.grad.cpu())
+    assert torch.isclose(a_min.grad, oc_min.grad.cpu(), atol=1e-3)
+    assert torch.isclose(a_max.grad, oc_max.grad.cpu(), atol=1e-3)
+
+
+def test_quantizer_ignores_non_float_tensors(api):
+    # :220-236, 557-566
+    for wrapper in (_static(api, torch.nn.ReLU()), _learned(api, torch.nn.ReLU())):
+        inputs = torch.tensor([[True, True, False, False]], device=DEV)
+        if isinstance(wrapper, api.qop.LearnedGridQuantWrapper):
+            out = wrapper._quantize_activation([inputs], wrapper.output_quantizers, 'output')[0]  # pylint: disable=protected-access
+        else:
+            wrapper.set_mode(api.qop.QcQuantizeOpMode.ACTIVE)
+            out = wrapper._quantize_activation(wrapper.output_quantizers, [inputs])[0]             # pylint: disable=protected-access
+        assert torch.equal(out, inputs)
+
+
+def test_ste_gating_for_learnable_grid_wrapper(api):
+    # :744-801
+    torch.manual_seed(0)
+    encodings = _enc(api, 8, 0.5, -1, 1, 0.2)
+    encodings_new = _enc(api, 8, 0.4, -0.98, 1, 0.2)
+    output_grad = []
+    conv1 = torch.nn.Conv2d(1, 2, 1).cuda()
+    conv1.weight.data = torch.tensor([[[[-0.8]]], [[[0.9]]]], device=DEV)
+    wrapper = _learned(api, conv1)
+    wrapper.train()
+    conv1.register_full_backward_hook(lambda m, grad_in, grad_out: output_grad.append(grad_out[0]))
+    wrapper.input_quantizers[0].enabled = True
+    wrapper.output_quantizers[0].enabled = True
+    wrapper.input_quantizers[0].encoding = encodings
+    wrapper.output_quantizers[0].encoding = encodings
+    wrapper.param_quantizers['weight'].encoding = encodings
+    wrapper.param_quantizers['bias'].enabled = False
+    new_input = torch.tensor([[[[-0.8469]]], [[[0.9]]]], device=DEV, requires_grad=True)
+    out = wrapper(new_input)
+    # in the learned-grid wrapper the gate uses the encodings of the forward pass: what was saved, not what is
+    # assigned afterwards
+    wrapper.input_quantizers[0].encoding = encodings_new
+    wrapper.output_quantizers[0].encoding = encodings_new
+    wrapper.param_quantizers['weight'].encoding = encodings_new
+    out.flatten().sum().backward()
+    assert new_input.grad.flatten()[1] == 0.0                      # 0.9 is above max = 0.5
+    assert conv1.weight.grad.flatten()[1] == 0.0                   # so is the weight 0.9
+    raw = torch.nn.functional.conv2d(torch.tensor([[[[-0.8469]]], [[[0.5]]]], device=DEV).clamp(-1, 0.5),
+                                     conv1.weight.detach().clamp(-1, 0.5), conv1.bias.detach()).flatten()
+    gated = output_grad[0].flatten()
+    for i, val in enumerate(raw):
+        if val < -1.01 or val > 0.51:
+            assert gated[i] == 0.0
+
+
+@pytest.mark.parametrize('act_bw', [8, 16])
+def test_learned_grid_preserves_fp16(api, act_bw):
+    # :1005-1065
+    torch.manual_seed(2023)
+    x = torch.randn((4, 200)).cuda().half()
+    linear = torch.nn.Linear(200, 100).cuda()
+    with torch.no_grad():
+        linear.weight.copy_(torch.randn((100, 200)).clamp(-1, 1))
+        linear.bias.copy_(torch.randn(100))
+    wrapper = _learned(api, linear, weight_bw=4, activation_bw=act_bw)
+    for q in list(wrapper.param_quantizers.values()) + wrapper.input_quantizers + wrapper.output_quantizers:
+        q.enabled = False
+    wrapper.param_quantizers['weight'].enabled = True
+    wrapper.weight_encoding_min = torch.nn.Parameter(torch.full((100,), -1.0))
+    wrapper.weight_encoding_max = torch.nn.Parameter(torch.full((100,), 1.0))
+    wrapper.input_quantizers[0].enabled = True
+    wrapper.input0_encoding_min = torch.nn.Parameter(torch.tensor([-3.5]))
+    wrapper.input0_encoding_max = torch.nn.Parameter(torch.tensor([3.5]))
+    wrapper.output_quantizers[0].enabled = True
+    wrapper.output0_encoding_min = torch.nn.Parameter(torch.tensor([-30.]))
+    wrapper.output0_encoding_max = torch.nn.Parameter(torch.tensor([30.]))
+    wrapper.cuda().train().half()
+    out_16 = wrapper(x.half())
+    assert out_16.dtype == torch.float16
+    out_16.sum().backward()
+    grads = [linear.weight.grad] + [getattr(wrapper, n + s).grad for n in ('weight', 'input0', 'output0')
+                                    for s in ('_encoding_min', '_encoding_max')]
+    for g in grads:
+        assert g.dtype == torch.float16 and torch.isfinite(g).all()
