@@ -295,3 +295,133 @@ def test_simulation_model_with_range_learning(tmp_path, scheme):
     assert w_enc[0]['min'] == pytest.approx(-w_enc[0]['max'] - w_enc[0]['scale'], rel=1e-5)
     assert 'relu1' in enc['activation_encodings'] and 'conv1' not in enc['activation_encodings'] or \
         'output' not in enc['activation_encodings'].get('conv1', {})
+
+
+# ---------------------------------- per-channel learned-grid cases of the reference's test_per_channel_quantization.py
+def _per_channel_learned_wrapper():
+    # create_learned_grid_wrapper of the reference: Conv2d(2, 3, 5), per-channel weight
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.qc_quantize_op import LearnedGridQuantWrapper
+    torch.manual_seed(0)
+    conv1 = nn.Conv2d(2, 3, kernel_size=5).cuda()
+    return LearnedGridQuantWrapper(conv1, round_mode='nearest',
+                                   quant_scheme=QuantScheme.training_range_learning_with_tf_init,
+                                   is_output_quantized=True, activation_bw=8, weight_bw=8,
+                                   device=torch.device('cuda'))
+
+
+def _three_encodings(mx=3, mn=-2):
+    from aimet_amd.common import libpymo
+    return [libpymo.TfEncoding(mn, mx, 1, 0.2, 8) for _ in range(3)]
+
+
+def test_per_channel_learned_tensor_quantizer_encodings():
+    # :438-462
+    wrapper = _per_channel_learned_wrapper()
+    q = wrapper.param_quantizers['weight']
+    encodings = _three_encodings()
+    q.encoding = encodings
+    new = q.encoding
+    assert isinstance(new, list) and len(new) == 3
+    for a, b in zip(encodings, new):
+        assert b.min == pytest.approx(a.min, abs=2e-2) and b.max == pytest.approx(a.max, abs=2e-2)
+        assert b.delta == new[0].delta and b.offset == new[0].offset
+    assert "LearnedGrid TensorQuantizer" in str(q)
+
+
+def test_per_channel_quantize_dequantize_known_answer():
+    # :464-492
+    q = _quantizer(False)
+    q._ch_axis = 0                                               # pylint: disable=protected-access
+    encoding_min = nn.Parameter(torch.tensor([0.0, 0.0, 0.0], device="cuda"))
+    encoding_max = nn.Parameter(torch.tensor([1.0, 2.5, 3.5], device="cuda"))
+    tensor = torch.ones((3, 1, 1, 2), device="cuda")
+    tensor[0] *= 1.5
+    tensor[2] *= 4
+    out = q.quantize_dequantize(tensor, encoding_min, encoding_max)
+    expected = torch.ones((3, 1, 1, 2), device="cuda")
+    expected[2] *= 3.5
+    assert torch.all(expected.eq(out))
+    assert encoding_min.grad is None and encoding_max.grad is None
+    optimizer = torch.optim.SGD([encoding_min, encoding_max], lr=0.05, momentum=0.5)
+    out.sum().backward()
+    optimizer.step()
+    assert encoding_min.grad is not None and len(encoding_max) == len(encoding_max.grad)
+
+
+def test_replacement_of_wrapper():
+    # :495-524: what the simulation model copies when it swaps a static-grid wrapper for a learned-grid one
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.qc_quantize_op import StaticGridQuantWrapper
+    from aimet_amd.v1.quantsim import QuantizationSimModel
+    torch.manual_seed(0)
+    conv1 = nn.Conv2d(3, 3, kernel_size=5).cuda()
+    post = StaticGridQuantWrapper(conv1, round_mode='nearest', quant_scheme=QuantScheme.post_training_tf,
+                                  is_symmetric=False, is_output_quantized=False, activation_bw=8, weight_bw=8)
+    post.enable_per_channel_quantization()
+    encodings = _three_encodings()
+    post.input_quantizers[0].enabled = True
+    post.input_quantizers[0].encoding = encodings[0]
+    post.param_quantizers['weight'].enabled = True
+    post.param_quantizers['weight'].encoding = encodings
+    post.param_quantizers['bias'].enabled = False
+    sim = QuantizationSimModel(conv1, quant_scheme=QuantScheme.training_range_learning_with_tf_init,
+                               dummy_input=torch.randn(1, 3, 12, 12, device="cuda"))
+    trainable = sim._construct_and_initialize_trainable_wrapper(post, device=torch.device('cuda'))  # pylint: disable=protected-access
+    assert trainable.output_quantizers[0].use_symmetric_encodings is False
+    assert trainable.output_quantizers[0].enabled is False
+    assert trainable.input0_encoding_min.item() == -2.0
+    assert isinstance(trainable.param_quantizers['weight'].encoding, list)
+    assert trainable.weight_encoding_max.tolist() == [3.0, 3.0, 3.0]
+
+
+def test_apply_gating_logic_on_the_wrapper():
+    # :527-546: min above max is pulled to [0, 1e-5]
+    wrapper = _per_channel_learned_wrapper()
+    encodings = _three_encodings(mx=-3, mn=2)
+    wrapper.output_quantizers[0].encoding = encodings[0]
+    wrapper.input_quantizers[0].enabled = False
+    wrapper.param_quantizers['weight'].encoding = encodings
+    wrapper.param_quantizers['bias'].enabled = False
+    wrapper.apply_gating_logic()
+    assert wrapper.output_quantizers[0].encoding.min == 0.0
+    assert abs(wrapper.output_quantizers[0].encoding.max - 1e-5) < 1e-6
+    for enc in wrapper.param_quantizers['weight'].encoding:
+        assert enc.min == 0.0 and abs(enc.max - 1e-5) < 1e-6
+
+
+@pytest.mark.parametrize('dtype', (torch.float32, torch.float16, torch.bfloat16))
+@pytest.mark.parametrize('shape', [(3, 1, 1, 2), (3,)])
+def test_per_channel_encoding_gradients_are_opposite_when_nothing_is_clipped_low(dtype, shape):
+    # :549-594: with every value at or above zero = min, d/dmax == -d/dmin for every channel, weights and biases
+    from aimet_amd.v1 import quantsim_straight_through_grad as grad_fn
+    q = _quantizer(False)
+    q._ch_axis = 0                                               # pylint: disable=protected-access
+    encoding_min = nn.Parameter(torch.tensor([0.0, 0.0, 0.0]).to('cuda', dtype))
+    encoding_max = nn.Parameter(torch.tensor([1.0, 2.5, 3.5]).to('cuda', dtype))
+    tensor = torch.ones(shape).to('cuda', dtype)
+    grad = torch.randn(shape).to('cuda', dtype)
+    _, saved = grad_fn.learned_grid_forward(tensor, q, encoding_min, encoding_max)
+    _, g_min, g_max = grad_fn.learned_grid_backward(tensor, grad, saved, encoding_min, encoding_max, False, True, True)
+    assert len(g_min) == len(g_max) == 3 and g_min.dtype == dtype
+    assert torch.all(torch.eq(g_max, -g_min))
+
+
+def test_qc_trainable_wrapper_per_channel():
+    # :597-635
+    wrapper = _per_channel_learned_wrapper()
+    encodings = _three_encodings()
+    wrapper.input_quantizers[0].enabled = False
+    for name in ('weight', 'bias'):
+        wrapper.param_quantizers[name].enabled = True
+        wrapper.param_quantizers[name].encoding = encodings
+    wrapper.output_quantizers[0].enabled = True
+    wrapper.output_quantizers[0].encoding = encodings[0]
+    inp = torch.rand((1, 2, 5, 5), device="cuda", requires_grad=True)
+    optimizer = torch.optim.SGD(wrapper.parameters(), lr=0.05, momentum=0.5)
+    wrapper(inp).flatten().sum().backward()
+    optimizer.step()
+    assert wrapper.output0_encoding_min.item() != -2.0 and wrapper.output0_encoding_max.item() != 3.0
+    for name in ('weight', 'bias'):
+        assert all(v.item() != -2.0 for v in getattr(wrapper, name + '_encoding_min'))
+        assert all(v.item() != 3.0 for v in getattr(wrapper, name + '_encoding_max'))
