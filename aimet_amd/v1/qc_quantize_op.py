@@ -332,12 +332,35 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
             # cannot corrupt the gradient bookkeeping of that view.  Without autograd there is nothing to gate and
             # nothing to protect: no extra pass over the activations.
             quantized_inputs = [inp.clone() if isinstance(inp, torch.Tensor) else inp for inp in quantized_inputs]
-        wrapped_output = self._module_to_wrap(*quantized_inputs, **kwargs)
+        if self._relu_is_absorbed(quantized_inputs, kwargs):
+            wrapped_output = quantized_inputs[0]
+        else:
+            wrapped_output = self._module_to_wrap(*quantized_inputs, **kwargs)
         self._restore_shadow_params(shadow_params)
         if not isinstance(wrapped_output, (List, Tuple)):
             wrapped_output = [wrapped_output]
         output = self._quantize_activation(self.output_quantizers, list(wrapped_output))
         return output[0] if len(output) == 1 else output
+
+    def _relu_is_absorbed(self, inputs, kwargs) -> bool:
+        """True when running the wrapped nn.ReLU would not change the wrapper's result, so its pass over the
+        activations (one read and one write of the whole tensor, as much traffic as the quantizer itself) can be left
+        out.  Quantize-dequantize first clamps to [encoding.min, encoding.max]; with encoding.min == 0 that clamp
+        already maps every negative input to 0, NaN to encoding.max and leaves the rest alone, exactly as
+        clamp(relu(x)) does, so QDQ(x) == QDQ(relu(x)) element for element.  Only taken without autograd (the
+        straight-through mask of the pre-activation differs at x == 0) and for a ReLU that is not in-place (an
+        in-place ReLU also rewrites its input, which other readers of that tensor may rely on)."""
+        module = self._module_to_wrap
+        if type(module) is not nn.ReLU or module.inplace or kwargs or torch.is_grad_enabled():  # pylint: disable=unidiomatic-typecheck
+            return False
+        if self._mode is not QcQuantizeOpMode.ACTIVE or len(inputs) != 1 or len(self.output_quantizers) != 1:
+            return False
+        tensor, quantizer = inputs[0], self.output_quantizers[0]
+        if not isinstance(tensor, torch.Tensor) or not self.should_perform_quant_dequant(tensor, quantizer):
+            return False
+        encoding = getattr(quantizer, 'encoding', None)
+        return quantizer.bitwidth < 32 and quantizer.data_type == QuantizationDataType.int and \
+            encoding is not None and not isinstance(encoding, (list, tuple)) and encoding.min == 0.0
 
     def _restore_shadow_params(self, shadow_params):
         for name, param in self.get_named_parameters():

@@ -236,3 +236,79 @@ def test_quantsim_per_channel_config(api, tmp_path):
     with torch.no_grad():
         y = sim.model(dummy)
     assert torch.isfinite(y).all()
+
+
+class _ReluNet(nn.Module):
+    def __init__(self, inplace=False):
+        super().__init__()
+        self.conv1, self.relu1 = nn.Conv2d(3, 8, 3, padding=1), nn.ReLU(inplace=inplace)
+        self.conv2, self.relu2 = nn.Conv2d(8, 8, 3, padding=1), nn.ReLU(inplace=inplace)
+
+    def forward(self, x):
+        return self.relu2(self.conv2(self.relu1(self.conv1(x))))
+
+
+def test_relu_absorbed_by_output_quantizer(api, monkeypatch):
+    """A ReLU whose output quantizer has encoding.min == 0 is not executed in inference (the quantizer's clamp does
+    its work): results must be identical, element for element, to those with the ReLU executed, for negative, huge,
+    infinite and NaN pre-activations alike; and the ReLU must run whenever that identity does not hold."""
+    torch.manual_seed(3)
+    model = _ReluNet().eval().cuda()
+    dummy = torch.randn(2, 3, 6, 6).cuda()
+    sim = api.quantsim.QuantizationSimModel(model, dummy_input=dummy, quant_scheme='tf')
+    sim.compute_encodings(_calibrate, [torch.randn(8, 3, 6, 6).cuda() for _ in range(2)])
+    w = dict(sim.quant_wrappers())
+    assert w["relu1"].output_quantizers[0].encoding.min == 0.0
+    calls = []
+    for name in ("relu1", "relu2"):
+        w[name]._module_to_wrap.register_forward_hook(lambda m, i, o, name=name: calls.append(name))
+
+    x = torch.randn(8, 3, 6, 6).cuda() * 3
+    with torch.no_grad():
+        y_absorbed = sim.model(x)
+    assert calls == []
+    with monkeypatch.context() as mp:
+        mp.setattr(api.qc.StaticGridQuantWrapper, "_relu_is_absorbed", lambda self, inputs, kwargs: False)
+        with torch.no_grad():
+            y_executed = sim.model(x)
+    assert calls == ["relu1", "relu2"]
+    assert torch.equal(y_absorbed, y_executed)
+
+    # the wrapper alone, on special values
+    special = torch.tensor([-float('inf'), -3e38, -1.0, -1e-30, -0.0, 0.0, 1e-30, 0.3, 1e30, float('inf'),
+                            float('nan')], device='cuda')
+    calls.clear()
+    with torch.no_grad():
+        got = w["relu1"](special)
+    assert calls == []
+    enc = w["relu1"].output_quantizers[0].encoding
+    want = w["relu1"].output_quantizers[0].quantize_dequantize(torch.relu(special), api.nearest)
+    assert torch.equal(got, want) and got[-1].item() == pytest.approx(enc.max)
+
+    # with autograd the ReLU runs (its gradient at 0 differs from the quantizer's mask)
+    calls.clear()
+    sim.model(x.clone().requires_grad_(True)).sum().backward()
+    assert calls == ["relu1", "relu2"]
+    # a symmetric (signed) output grid does not clamp at zero: the ReLU runs
+    calls.clear()
+    q = w["relu1"].output_quantizers[0]
+    q.use_symmetric_encodings = True
+    q.reset_encoding_stats()
+    q.update_encoding_stats(torch.randn(1000, device='cuda'))
+    q.compute_encoding()
+    assert q.encoding.min < 0
+    with torch.no_grad():
+        sim.model(x)
+    assert calls == ["relu1"]
+
+    # an in-place ReLU also rewrites its input: it always runs
+    model = _ReluNet(inplace=True).eval().cuda()
+    sim = api.quantsim.QuantizationSimModel(model, dummy_input=dummy, quant_scheme='tf')
+    sim.compute_encodings(_calibrate, [torch.randn(8, 3, 6, 6).cuda()])
+    calls.clear()
+    for name, wrapper in sim.quant_wrappers():
+        if name.startswith("relu"):
+            wrapper._module_to_wrap.register_forward_hook(lambda m, i, o, name=name: calls.append(name))
+    with torch.no_grad():
+        sim.model(x)
+    assert calls == ["relu1", "relu2"]
