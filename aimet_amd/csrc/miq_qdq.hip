@@ -15,6 +15,7 @@
 #include "miq_common.h"
 #include "miq_fastmath.h"
 #include "miq_io.h"
+#include "miq_stochastic.h"
 
 #include <cmath>
 
@@ -455,10 +456,7 @@ int check_round(int rounding_mode)
     if (rounding_mode == MIQ_ROUND_NEAREST)
         return MIQ_OK;
     if (rounding_mode == MIQ_ROUND_STOCHASTIC)
-    {
-        set_error("stochastic rounding is not implemented (the reference's is not reproducible by design)");
-        return MIQ_ERR_UNSUPPORTED;
-    }
+        return MIQ_OK;
     set_error("unknown rounding mode %d", rounding_mode);
     return MIQ_ERR_INVALID_ARG;
 }
@@ -586,6 +584,8 @@ int miq_qdq_per_tensor_f32(const float* in, float* out, int64_t n, double enc_mi
     miq_encoding e;
     if (int rc = miq_fill_encoding_info(bw, enc_min, enc_max, &e))
         return rc;
+    if (rounding_mode == MIQ_ROUND_STOCHASTIC)
+        return stochastic_qdq_per_tensor<float>(in, out, n, e, (hipStream_t) stream);
     EwPtrs<float, uint8_t> p{in, nullptr, out, nullptr};
     return launch_ew<float, OpV1Qdq, false>(p, per_tensor_src(e), n, 1, 1, (hipStream_t) stream);
 }
@@ -599,6 +599,8 @@ int miq_qdq_per_tensor_bf16(const uint16_t* in, uint16_t* out, int64_t n, double
     miq_encoding e;
     if (int rc = miq_fill_encoding_info(bw, enc_min, enc_max, &e))
         return rc;
+    if (rounding_mode == MIQ_ROUND_STOCHASTIC)
+        return stochastic_qdq_per_tensor<uint16_t>(in, out, n, e, (hipStream_t) stream);
     EwPtrs<uint16_t, uint8_t> p{in, nullptr, out, nullptr};
     return launch_ew<uint16_t, OpV1Qdq, false>(p, per_tensor_src(e), n, 1, 1, (hipStream_t) stream);
 }
@@ -616,6 +618,8 @@ int miq_quantize_per_tensor_f32(const float* in, float* out, int64_t n, double e
     // DlQuantization/src/trim_functions.cpp:207-216: shift = 2^(bw-1) held in an unsigned int, subtracted in float
     unsigned int shift = shift_to_signed ? (unsigned int) std::pow(2, bw - 1) : 0u;
     s.shift            = (float) shift;
+    if (rounding_mode == MIQ_ROUND_STOCHASTIC)
+        return stochastic_quantize_per_tensor(in, out, n, e, s.shift, (hipStream_t) stream);
     EwPtrs<float, uint8_t> p{in, nullptr, out, nullptr};
     return launch_ew<float, OpV1Quantize, false>(p, s, n, 1, 1, (hipStream_t) stream);
 }
@@ -657,6 +661,9 @@ int miq_qdq_per_channel_f32(const float* in, float* out, int64_t num_channel, in
     MIQ_CHECK_ARG(num_element == 0 || (in && out && enc_min && enc_max && enc_delta && enc_offset), "null pointer");
     if (int rc = check_round(rounding_mode))
         return rc;
+    if (rounding_mode == MIQ_ROUND_STOCHASTIC)
+        return stochastic_qdq_per_channel<float>(in, out, num_channel, num_element, num_element_per_channel, enc_min,
+                                                 enc_max, enc_delta, enc_offset, (hipStream_t) stream);
     EwPtrs<float, uint8_t> p{in, nullptr, out, nullptr};
     return launch_ew<float, OpV1Qdq, true>(p, v1_channel_src(enc_min, enc_max, enc_delta, enc_offset), num_element,
                                            num_channel, num_element_per_channel, (hipStream_t) stream);
@@ -671,6 +678,9 @@ int miq_qdq_per_channel_bf16(const uint16_t* in, uint16_t* out, int64_t num_chan
     MIQ_CHECK_ARG(num_element == 0 || (in && out && enc_min && enc_max && enc_delta && enc_offset), "null pointer");
     if (int rc = check_round(rounding_mode))
         return rc;
+    if (rounding_mode == MIQ_ROUND_STOCHASTIC)
+        return stochastic_qdq_per_channel<uint16_t>(in, out, num_channel, num_element, num_element_per_channel,
+                                                    enc_min, enc_max, enc_delta, enc_offset, (hipStream_t) stream);
     EwPtrs<uint16_t, uint8_t> p{in, nullptr, out, nullptr};
     return launch_ew<uint16_t, OpV1Qdq, true>(p, v1_channel_src(enc_min, enc_max, enc_delta, enc_offset), num_element,
                                               num_channel, num_element_per_channel, (hipStream_t) stream);

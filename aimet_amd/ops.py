@@ -59,6 +59,19 @@ def get_computed_encodings(bw, mn, mx, symmetric, strict_symmetric, unsigned_sym
 
 
 # ------------------------------------------------------------------------------------------------------------ v1 QDQ
+def set_stochastic_seed(seed: int):
+    """Seed of the stochastic rounding mode (the counterpart of srand for the reference's CPU path); restarts the
+    library's count of stochastic launches."""
+    check(lib.miq_set_stochastic_seed(int(seed) & 0xFFFFFFFFFFFFFFFF))
+
+
+def stochastic_state():
+    """(seed, number of stochastic launches since the seed was set)."""
+    seed, calls = C.c_uint64(), C.c_uint64()
+    check(lib.miq_get_stochastic_state(C.byref(seed), C.byref(calls)))
+    return seed.value, calls.value
+
+
 def qdq_per_tensor(x, enc_min, enc_max, bw, rounding_mode=_lib.ROUND_NEAREST, out=None):
     """DlQuantization per-tensor quantize-dequantize; float32 or bfloat16 storage, float32 arithmetic."""
     _require_gpu(x, out)

@@ -26,10 +26,21 @@ extern "C" {
 #define MIQ_ERR_HIP (-2)
 #define MIQ_ERR_UNSUPPORTED (-3)
 
-/* DLQ/include/DlQuantization/Quantization.hpp:145-149 (RoundingMode).  Only nearest is implemented: the
- * reference's stochastic mode seeds from clock() per element and is not reproducible by design. */
+/* DLQ/include/DlQuantization/Quantization.hpp:145-149 (RoundingMode).
+ * Stochastic: q = floor(t + u), u uniform in [0,1) (DLQ/src/trim_functions.cpp:155-158), accepted by the per-tensor
+ * and per-channel quantize-dequantize entry points and by miq_quantize_per_tensor_f32.  The reference draws u from
+ * libc rand() (CPU) or a clock-seeded generator per element (GPU); here u is a function of (seed, call, element index):
+ *     key = splitmix64(seed + 0x9E3779B97F4A7C15 * (call + 1)), k0 = low word, k1 = high word
+ *     r   = mix32((uint32) i + k0) ^ k1 ^ (uint32)(i >> 32),  u = (r >> 8) * 2^-24
+ *     mix32(x): x ^= x >> 16; x *= 0x7feb352d; x ^= x >> 15; x *= 0x846ca68b; x ^= x >> 16
+ * with `call` the number of stochastic launches on non-empty tensors since the seed was set. */
 #define MIQ_ROUND_NEAREST 0
 #define MIQ_ROUND_STOCHASTIC 1
+
+/* Counterpart of srand() for the stochastic rounding mode: sets the seed (0 at load) and restarts the call count. */
+int miq_set_stochastic_seed(uint64_t seed);
+/* Current seed and number of stochastic launches since it was set. */
+int miq_get_stochastic_state(uint64_t* seed /* host */, uint64_t* calls /* host */);
 
 /* DLQ/include/DlQuantization/Quantization.hpp:83-105 (QuantizationMode) */
 #define MIQ_QUANTIZATION_TF 0

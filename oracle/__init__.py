@@ -60,6 +60,9 @@ class _Oracle:
         L.orc_per_channel_params_f32.argtypes = [_f64p, _f64p, _i64, C.c_int, _f32p, _f32p, _f32p, _f32p]
         L.orc_qdq_per_channel_f32.argtypes = [_f32p, _i64, _i64, _i64, _f32p, _f32p, _f32p, _f32p, _f32p]
         L.orc_quantize_per_channel_f32.argtypes = L.orc_qdq_per_channel_f32.argtypes
+        L.orc_stochastic_f32.argtypes = [_f32p, _i64, _i64, _i64, _f32p, _f32p, _f32p, _f32p, _f32p, _f64p, C.c_int,
+                                         C.c_float]
+        L.orc_stochastic_uniforms.argtypes = [C.c_uint64, C.c_uint64, _i64, _i64, _f64p]
         L.orc_qdq_per_channel_bf16.argtypes = [_u16p, _i64, _i64, _i64, _u16p, _f32p, _f32p, _f32p, _f32p]
         L.orc_qdq_broadcast_f32.argtypes = [_f32p, _f32p, _i64, _i64, _i64p, _i64p, _f32p, _f32p, _f32p, _f32p]
         L.orc_ste_bwd_per_tensor_f32.argtypes = [_f32p, _f32p, _f32p, _i64, C.c_float, C.c_float]
@@ -125,6 +128,31 @@ class _Oracle:
         out = np.empty_like(x_bits)
         self.L.orc_qdq_per_tensor_bf16(x_bits.reshape(-1), x_bits.size, out.reshape(-1), mn, mx, bw)
         return out
+
+    # -- stochastic rounding -----------------------------------------------------------------------------------
+    def stochastic_uniforms(self, seed, call, n, first=0):
+        """The product's documented generator: u(i) for i in [first, first + n)."""
+        u = np.empty(n, np.float64)
+        self.L.orc_stochastic_uniforms(seed, call, first, n, u)
+        return u
+
+    def stochastic(self, x, num_channel, n_per_channel, params, u, dequant=True, shift=0.0):
+        """floor(t + u) quantize(-dequantize) with explicit uniform numbers; params = (min, max, delta, offset) float32
+        vectors of length num_channel."""
+        x = _f32(x)
+        out = np.empty_like(x)
+        mn, mx, d, o = (_f32(p).reshape(-1) for p in params)
+        u = np.ascontiguousarray(u, dtype=np.float64).reshape(-1)
+        assert u.size == x.size and mn.size == num_channel
+        self.L.orc_stochastic_f32(x.reshape(-1), num_channel, x.size, n_per_channel, out.reshape(-1), mn, mx, d, o, u,
+                                  int(dequant), float(shift))
+        return out
+
+    def stochastic_per_tensor(self, x, mn, mx, bw, u, dequant=True, shift_to_signed=False):
+        e = self.fill_encoding_info(bw, mn, mx)
+        params = tuple(np.array([v], np.float32) for v in (e.min, e.max, e.delta, e.offset))
+        shift = float(2 ** (bw - 1)) if (shift_to_signed and not dequant) else 0.0
+        return self.stochastic(x, 1, max(np.asarray(x).size, 1), params, u, dequant, shift)
 
     # -- per-channel -------------------------------------------------------------------------------------------
     def per_channel_params(self, enc_min, enc_max, bw):
@@ -310,6 +338,12 @@ class _Ref:
         L.ref_quantize_per_tensor.argtypes = [_f32p, _i64, _f32p, C.c_double, C.c_double, C.c_int, C.c_int]
         L.ref_qdq_per_channel.argtypes = [_f32p, _i64, _i64, _i64, _f32p, _f32p, _f32p, _f32p, _f32p]
         L.ref_qdq_broadcast.argtypes = [_f32p, _f32p, _i64, _i64, _i64p, _i64p, _f32p, _f32p, _f32p, _f32p]
+        L.ref_qdq_per_tensor_stochastic.argtypes = [_f32p, _i64, _f32p, C.c_double, C.c_double, C.c_int, C.c_uint]
+        L.ref_quantize_per_tensor_stochastic.argtypes = [_f32p, _i64, _f32p, C.c_double, C.c_double, C.c_int, C.c_int,
+                                                         C.c_uint]
+        L.ref_qdq_per_channel_stochastic.argtypes = [_f32p, _i64, _i64, _i64, _f32p, _f32p, _f32p, _f32p, _f32p,
+                                                     C.c_uint]
+        L.ref_libc_uniforms.argtypes = [C.c_uint, _i64, _f64p]
         L.ref_get_computed_encodings.argtypes = [C.c_int, C.c_double, C.c_double, C.c_int, C.c_int, C.c_int, _f64p]
         for name in ("ref_tf_create", "ref_tfe_create"):
             getattr(L, name).restype = C.c_void_p
@@ -349,6 +383,33 @@ class _Ref:
         x = _f32(x)
         out = np.empty_like(x)
         self.L.ref_quantize_per_tensor(x.reshape(-1), x.size, out.reshape(-1), mn, mx, bw, int(shift_to_signed))
+        return out
+
+    # ROUND_STOCHASTIC: srand(seed), then the reference's CPU loop; libc_uniforms replays the same rand() sequence
+    def libc_uniforms(self, seed, n):
+        u = np.empty(n, np.float64)
+        self.L.ref_libc_uniforms(seed, n, u)
+        return u
+
+    def qdq_per_tensor_stochastic(self, x, mn, mx, bw, seed):
+        x = _f32(x)
+        out = np.empty_like(x)
+        self.L.ref_qdq_per_tensor_stochastic(x.reshape(-1), x.size, out.reshape(-1), mn, mx, bw, seed)
+        return out
+
+    def quantize_per_tensor_stochastic(self, x, mn, mx, bw, shift_to_signed, seed):
+        x = _f32(x)
+        out = np.empty_like(x)
+        self.L.ref_quantize_per_tensor_stochastic(x.reshape(-1), x.size, out.reshape(-1), mn, mx, bw,
+                                                  int(shift_to_signed), seed)
+        return out
+
+    def qdq_per_channel_stochastic(self, x, num_channel, n_per_channel, params, seed):
+        x = _f32(x)
+        out = np.empty_like(x)
+        mn, mx, d, o = (_f32(p).copy() for p in params)
+        self.L.ref_qdq_per_channel_stochastic(x.reshape(-1), num_channel, x.size, n_per_channel, out.reshape(-1), mn,
+                                              mx, d, o, seed)
         return out
 
     def qdq_per_channel(self, x, num_channel, n_per_channel, params):

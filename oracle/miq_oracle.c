@@ -202,6 +202,59 @@ void orc_qdq_per_channel_f32(const float* in, int64_t numChannel, int64_t numEle
     }
 }
 
+/* ------------------------------------------------------------------------------------------------------------
+ * a3 with ROUND_STOCHASTIC (DLQ/src/trim_functions.cpp:141-166): *out = floor(*out + randUniformCpu()) -- the float
+ * grid position is widened to double, the uniform number added, the floor stored back as float.  The uniform numbers
+ * are an argument here so that the formula can be pinned against the reference fed from libc rand() and the product
+ * kernel against its own documented generator (orc_stochastic_uniforms).
+ * ---------------------------------------------------------------------------------------------------------- */
+static inline float orc_quantize_value_stochastic(float x, float mn, float mx, float delta, float offset, double u)
+{
+    float t = fmaxf(fminf(x, mx), mn);
+    t       = t / delta - offset;
+    return (float) floor((double) t + u);
+}
+
+/* dequant != 0: quantize-dequantize; dequant == 0: grid index minus `shift` (quantizeToFxp, trim_functions.cpp:203-218).
+ * numChannel == 1 with parameter vectors of length 1 is the per-tensor case. */
+void orc_stochastic_f32(const float* in, int64_t numChannel, int64_t numElement, int64_t numElementPerChannel,
+                        float* out, const float* mn, const float* mx, const float* delta, const float* offset,
+                        const double* u, int dequant, float shift)
+{
+    for (int64_t i = 0; i < numElement; ++i)
+    {
+        int64_t c = (i / numElementPerChannel) % numChannel;
+        float q   = orc_quantize_value_stochastic(in[i], mn[c], mx[c], delta[c], offset[c], u[i]);
+        out[i]    = dequant ? orc_dequantize_value(q, delta[c], offset[c]) : q - shift;
+    }
+}
+
+/* The product's generator (include/miq.h, MIQ_ROUND_STOCHASTIC): u is a function of (seed, call, element index). */
+static inline uint32_t orc_mix32(uint32_t x)
+{
+    x ^= x >> 16;
+    x *= 0x7feb352du;
+    x ^= x >> 15;
+    x *= 0x846ca68bu;
+    x ^= x >> 16;
+    return x;
+}
+
+void orc_stochastic_uniforms(uint64_t seed, uint64_t call, int64_t first, int64_t n, double* u)
+{
+    uint64_t z = seed + 0x9E3779B97F4A7C15ull * (call + 1);
+    z          = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z          = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z          = z ^ (z >> 31);
+    uint32_t k0 = (uint32_t) z, k1 = (uint32_t) (z >> 32);
+    for (int64_t j = 0; j < n; ++j)
+    {
+        uint64_t i = (uint64_t) (first + j);
+        uint32_t r = orc_mix32((uint32_t) i + k0) ^ k1 ^ (uint32_t) (i >> 32);
+        u[j]       = (double) (r >> 8) * 0x1p-24;
+    }
+}
+
 /* quantize only (the float-valued grid index), per channel; used to pin integer codes */
 void orc_quantize_per_channel_f32(const float* in, int64_t numChannel, int64_t numElement,
                                   int64_t numElementPerChannel, float* out, const float* mn, const float* mx,

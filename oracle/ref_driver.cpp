@@ -17,6 +17,7 @@
 #include <cmath>
 #include <cstddef>
 #include <cstdint>
+#include <cstdlib>
 #include <cstring>
 #include <limits>
 #include <memory>
@@ -65,6 +66,43 @@ void ref_qdq_per_tensor(const float* in, int64_t n, float* out, double encMin, d
 {
     TensorQuantizationSim<float> sim;
     sim.quantizeDequantizeTensor(in, (size_t) n, out, encMin, encMax, (uint8_t) bw, ROUND_NEAREST, false);
+}
+
+// ROUND_STOCHASTIC on the CPU path draws from libc rand() (trim_functions.cpp:56-59); srand(seed) first, and
+// ref_libc_uniforms replays the same sequence: rand() / (RAND_MAX + 1.0).
+void ref_qdq_per_tensor_stochastic(const float* in, int64_t n, float* out, double encMin, double encMax, int bw,
+                                   unsigned int seed)
+{
+    TensorQuantizationSim<float> sim;
+    srand(seed);
+    sim.quantizeDequantizeTensor(in, (size_t) n, out, encMin, encMax, (uint8_t) bw, ROUND_STOCHASTIC, false);
+}
+
+void ref_quantize_per_tensor_stochastic(const float* in, int64_t n, float* out, double encMin, double encMax, int bw,
+                                        int shiftToSigned, unsigned int seed)
+{
+    TensorQuantizationSim<float> sim;
+    srand(seed);
+    sim.quantizeTensor(in, (size_t) n, out, encMin, encMax, (uint8_t) bw, ROUND_STOCHASTIC, false,
+                       shiftToSigned != 0);
+}
+
+void ref_qdq_per_channel_stochastic(const float* in, int64_t numChannel, int64_t numElement,
+                                    int64_t numElementPerChannel, float* out, float* encMin, float* encMax,
+                                    float* encDelta, float* encOffset, unsigned int seed)
+{
+    TensorQuantizationSim<float> sim;
+    srand(seed);
+    sim.quantizeDequantizeTensorPerChannel(in, (size_t) numChannel, (size_t) numElement,
+                                           (size_t) numElementPerChannel, out, encMin, encMax, encDelta, encOffset,
+                                           ROUND_STOCHASTIC, false);
+}
+
+void ref_libc_uniforms(unsigned int seed, int64_t n, double* u)
+{
+    srand(seed);
+    for (int64_t i = 0; i < n; ++i)
+        u[i] = rand() / (RAND_MAX + 1.0);
 }
 
 void ref_quantize_per_tensor(const float* in, int64_t n, float* out, double encMin, double encMax, int bw,

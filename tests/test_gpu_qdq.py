@@ -135,10 +135,9 @@ def test_per_tensor_bf16(ops, oracle):
     assert np.array_equal(gin.float().numpy(), expect)
 
 
-def test_stochastic_rounding_is_refused(ops):
-    from aimet_amd import _lib
-    with pytest.raises(RuntimeError, match="stochastic"):
-        ops.qdq_per_tensor(torch.zeros(16, device="cuda"), -1, 1, 8, rounding_mode=_lib.ROUND_STOCHASTIC)
+def test_unknown_rounding_mode_is_refused(ops):
+    with pytest.raises(RuntimeError, match="rounding mode"):
+        ops.qdq_per_tensor(torch.zeros(16, device="cuda"), -1, 1, 8, rounding_mode=2)
 
 
 # --------------------------------------------------------------------------------------------------- per-channel
