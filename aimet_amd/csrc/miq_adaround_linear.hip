@@ -64,7 +64,8 @@ constexpr int kLdsRow = kTileK + 4;   // floats per LDS tile row; the pad spread
 // row segment: fully coalesced) while the MFMAs see their own operand / accumulator layout.
 // (Measured alternative: wavefront-private [16 o] x [128 k] tiles without workgroup barriers were 10-20 % slower.)
 
-// grid (O / 32, K / 256), 256 threads.
+// grid (K / 256, O / 32), 256 threads: consecutive workgroups walk along the rows, so the workgroups that run together
+// cover contiguous memory (with the row blocks as the fast index the same tile reads measured 25 % slower).
 __global__ __launch_bounds__(256) void lin_fwd_kernel(const float* __restrict__ F, const float* __restrict__ alpha,
                                                       const float* __restrict__ X, const int* __restrict__ row_index,
                                                       int64_t x_row_stride, float* __restrict__ partial, LinGeom g)
@@ -72,11 +73,20 @@ __global__ __launch_bounds__(256) void lin_fwd_kernel(const float* __restrict__ 
     __shared__ __attribute__((aligned(16))) float tile[kTileO * kLdsRow];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int n = lane & 15, s = lane >> 4;
-    const int o_blk = blockIdx.x * kTileO;
-    const int k_blk = blockIdx.y * kTileK;
+    const int o_blk = blockIdx.y * kTileO;
+    const int k_blk = blockIdx.x * kTileK;
     const int K     = g.in_features;
 
     // phase 1: adarounded weight tile, streaming layout: wavefront w forms rows 8w .. 8w+7
+    // the rows' delta / offset are requested first: a load issued where it is used makes that row wait for a round trip
+    float dl[8], of[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+    {
+        const int c = (o_blk + wave * 8 + j) * g.chan_stride;
+        dl[j]       = g.delta[c];
+        of[j]       = g.offset[c];
+    }
     v4f f[8], al[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j)
@@ -102,13 +112,11 @@ __global__ __launch_bounds__(256) void lin_fwd_kernel(const float* __restrict__ 
 #pragma unroll
     for (int j = 0; j < 8; ++j)
     {
-        const int r   = wave * 8 + j;
-        const int c   = (o_blk + r) * g.chan_stride;
-        const float d = g.delta[c], off = g.offset[c];
+        const int r = wave * 8 + j;
         v4f wq;
 #pragma unroll
         for (int t = 0; t < 4; ++t)
-            wq[t] = adarounded_f<true>(f[j][t], al[j][t], d, off, g.clip_min, g.clip_max);
+            wq[t] = adarounded_f<true>(f[j][t], al[j][t], dl[j], of[j], g.clip_min, g.clip_max);
         *reinterpret_cast<v4f*>(&tile[r * kLdsRow + 4 * lane]) = wq;
     }
     __syncthreads();
@@ -153,7 +161,7 @@ __global__ __launch_bounds__(256) void lin_fwd_kernel(const float* __restrict__ 
         const int mt = t4 >> 1, nt = t4 & 1;
         const int o  = o_blk + nt * 16 + (ln & 15);
         const int b0 = mt * 16 + 4 * (ln >> 4);
-        float* dst   = partial + ((int64_t) blockIdx.y * kBatch + b0) * g.out_features + o;
+        float* dst   = partial + ((int64_t) blockIdx.x * kBatch + b0) * g.out_features + o;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             dst[(int64_t) i * g.out_features] = sum[i];
@@ -199,7 +207,7 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
     }
 }
 
-// grid (O / 32, K / 256), 256 threads.  Phase 1: wavefront w forms dLoss/dW' for k in [64w, 64w + 64) as four 16-wide k
+// grid (K / 256, O / 32), 256 threads.  Phase 1: wavefront w forms dLoss/dW' for k in [64w, 64w + 64) as four 16-wide k
 // tiles (the M dimension of the MFMA) by two 16-wide o tiles (N), the batch being the MFMA's K dimension (8 steps of
 // 4), and parks it in the LDS tile.  Phase 2: the alpha-gradient + regulariser + Adam epilogue in the streaming layout.
 template <int PF>
@@ -213,8 +221,8 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const float* __restrict__ 
     __shared__ __attribute__((aligned(16))) float tile[kTileO * kLdsRow];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int n = lane & 15, s = lane >> 4;
-    const int o_blk = blockIdx.x * kTileO;
-    const int k_blk = blockIdx.y * kTileK;
+    const int o_blk = blockIdx.y * kTileO;
+    const int k_blk = blockIdx.x * kTileK;
     const int K = g.in_features, O = g.out_features;
 
     // the epilogue's first rows are requested before the MFMA phase so that they arrive while it runs
@@ -227,6 +235,15 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const float* __restrict__ 
         av[j]           = ldg4(alpha + e);
         mv[j]           = ldg4(m + e);
         vv[j]           = ldg4(v + e);
+    }
+
+    float dl[8], of[8];   // per-row delta / offset, requested here and not where they are used (see lin_fwd_kernel)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+    {
+        const int c = (o_blk + wave * 8 + j) * g.chan_stride;
+        dl[j]       = g.delta[c];
+        of[j]       = g.offset[c];
     }
 
     v4f acc[4][2];
@@ -278,8 +295,7 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const float* __restrict__ 
             mv[slot]         = ldg4(m + e2);
             vv[slot]         = ldg4(v + e2);
         }
-        const int c   = (o_blk + r) * g.chan_stride;
-        const float d = g.delta[c], off = g.offset[c];
+        const float d = dl[j], off = of[j];
         const v4f gw  = *reinterpret_cast<const v4f*>(&tile[r * kLdsRow + 4 * lane]);
         float as[4] = {a4[0], a4[1], a4[2], a4[3]}, ms[4] = {m4[0], m4[1], m4[2], m4[3]};
         float vs[4] = {v4[0], v4[1], v4[2], v4[3]};
@@ -364,7 +380,7 @@ int miq_adaround_linear_fwd_f32(const float* weight, const float* alpha, const f
     MIQ_CHECK_ARG(x_row_stride >= in_features && target_row_stride >= out_features, "row stride shorter than a row");
     MIQ_CHECK_ARG(activation == 0 || activation == 1, "activation must be 0 (none) or 1 (ReLU)");
     const int splits = (int) (in_features / kTileK);
-    hipLaunchKernelGGL(lin_fwd_kernel, dim3((unsigned) (out_features / kTileO), (unsigned) splits), dim3(256), 0,
+    hipLaunchKernelGGL(lin_fwd_kernel, dim3((unsigned) splits, (unsigned) (out_features / kTileO)), dim3(256), 0,
                        (hipStream_t) stream, weight, alpha, x, row_index, x_row_stride, workspace, g);
     MIQ_CHECK_LAUNCH();
     const unsigned blocks = (unsigned) ((kBatch * out_features + 255) / 256);
@@ -393,7 +409,7 @@ int miq_adaround_linear_bwd_adam_f32(const float* weight, const float* grad_out,
     if (int rc = make_adam(a, reg_param, beta, lr, beta1, beta2, eps, step))
         return rc;
     // two rows of the epilogue in flight per lane: deeper prefetch (4, 8) costs occupancy and measured 5 % slower
-    hipLaunchKernelGGL(lin_bwd_kernel<2>, dim3((unsigned) (out_features / kTileO), (unsigned) (in_features / kTileK)),
+    hipLaunchKernelGGL(lin_bwd_kernel<2>, dim3((unsigned) (in_features / kTileK), (unsigned) (out_features / kTileO)),
                        dim3(256), 0, (hipStream_t) stream, weight, grad_out, x, row_index, x_row_stride, alpha, exp_avg,
                        exp_avg_sq, grad_alpha, g, a, reg_partial);
     MIQ_CHECK_LAUNCH();

@@ -16,9 +16,11 @@
 // l mod 16, so that even when every sample of a wavefront falls into one bin (post-ReLU data) at most two lanes
 // meet on an address.
 #include "miq_common.h"
+#include "miq_fastmath.h"
 
 #include <algorithm>
 #include <cfloat>
+#include <climits>
 #include <cstddef>
 #include <cmath>
 #include <cstring>
@@ -461,11 +463,14 @@ __global__ __launch_bounds__(kBlock) void minmax_rows_fold_kernel(const float2* 
 // ---------------------------------------------------------------------------------------------------- histogram
 // Adds one sample to the workgroup's LDS histogram.  Row kPdf is a sink for dropped samples, so the add is
 // unconditional (no divergent branch per element).
-__device__ __forceinline__ void hist_add(uint32_t* lds, float x, float bucket, float off, int copy)
+// `rcp` is the correctly rounded 1 / bucket when the five-operation exact division applies to this bucket width (else 0);
+// it then gives the IEEE quotient bit for bit wherever the quotient can decide a bucket (miq_fastmath.h).
+__device__ __forceinline__ void hist_add(uint32_t* lds, float x, float bucket, float rcp, float off, int copy)
 {
     // DLQ/src/math_functions.cpp:375-382; the range test is done on the rounded float so that NaN and values
     // beyond the int range are dropped, as they are on the reference's CPU path
-    const float r  = roundf(x / bucket - off);
+    const float q  = (rcp != 0.0f && fabsf(x) <= kFastDivMaxDividend) ? div_by_invariant(x, bucket, rcp) : x / bucket;
+    const float r  = roundf(q - off);
     const bool ok  = (r >= 0.0f && r < (float) kPdf);
     const int row  = ok ? (int) r : kPdf;
     atomicAdd(&lds[row * kCopies + copy], 1u);
@@ -553,6 +558,7 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
         bucket = st->bucket_f;
         off    = st->pdf_offset_f;
     }
+    const float rcp = fastdiv_divisor_ok(bucket) ? 1.0f / bucket : 0.0f;
     for (int i = threadIdx.x; i < (kPdf + 1) * kCopies; i += kBlock)
         lds[i] = 0;
     __syncthreads();
@@ -564,10 +570,10 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
             {
-                hist_add(lds, a[u].x, bucket, off, copy);
-                hist_add(lds, a[u].y, bucket, off, copy);
-                hist_add(lds, a[u].z, bucket, off, copy);
-                hist_add(lds, a[u].w, bucket, off, copy);
+                hist_add(lds, a[u].x, bucket, rcp, off, copy);
+                hist_add(lds, a[u].y, bucket, rcp, off, copy);
+                hist_add(lds, a[u].z, bucket, rcp, off, copy);
+                hist_add(lds, a[u].w, bucket, rcp, off, copy);
             }
             base += stride;
             if (base >= nvec)
@@ -580,12 +586,12 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
             }
         }
         if (group == 0 && threadIdx.x < (uint32_t) (n - nvec * 4))
-            hist_add(lds, in[nvec * 4 + threadIdx.x], bucket, off, copy);
+            hist_add(lds, in[nvec * 4 + threadIdx.x], bucket, rcp, off, copy);
     }
     else
     {
         for (int64_t i = (int64_t) group * kBlock + threadIdx.x; i < n; i += (int64_t) data_groups * kBlock)
-            hist_add(lds, in[i], bucket, off, copy);
+            hist_add(lds, in[i], bucket, rcp, off, copy);
     }
     __syncthreads();
     uint32_t* dst = st->counts[buf][group % kReplicas];
@@ -612,6 +618,15 @@ __global__ __launch_bounds__(kBlock) void hist_flush_kernel(DevState* st, uint32
 }
 
 // ------------------------------------------------------------------------------------------------ SQNR search
+// (int) of a floating-point value as the reference's x86-64 build performs it (cvttsd2si / cvttss2si): truncation
+// inside the int range, INT_MIN for everything else, NaN included.  The C++ cast is undefined there and this GPU's
+// conversion saturates instead; the difference decides a cost when a candidate range is more than 2^31 PDF buckets wide
+// (data spanning less than about 1e-12 against the 1e-5 minimum encoding range).
+__device__ __forceinline__ int cvtt_x86(double v)
+{
+    return (v >= -2147483648.0 && v < 2147483648.0) ? (int) v : INT_MIN;
+}
+
 struct SearchArgs
 {
     int bw;
@@ -761,9 +776,9 @@ __global__ __launch_bounds__(kBlock) void tfe_search_kernel(DevState* st, Search
             const float cMax      = delta * ((float) offset + stepSize);
             const float pdfStart  = (float) st->xLeft[0];
             const double pdfStep  = st->xLeft[1] - st->xLeft[0];
-            int minInd            = (int) floor((cMin - pdfStart) / pdfStep);
+            int minInd            = cvtt_x86(floor((cMin - pdfStart) / pdfStep));
             minInd                = minInd < 0 ? 0 : (minInd > kPdf - 1 ? kPdf - 1 : minInd);
-            int maxInd            = (int) floor((cMax - pdfStart) / pdfStep);
+            int maxInd            = cvtt_x86(floor((cMax - pdfStart) / pdfStep));
             maxInd                = maxInd < 0 ? 0 : (maxInd > kPdf - 1 ? kPdf - 1 : maxInd);
             const float minMid    = (float) (pdfStart + (minInd * pdfStep) + pdfStep / 2);
             const float maxMid    = (float) (pdfStart + (maxInd * pdfStep) + pdfStep / 2);
@@ -787,7 +802,7 @@ __global__ __launch_bounds__(kBlock) void tfe_search_kernel(DevState* st, Search
                 else
                 {
                     const float fv   = (float) mid;
-                    const int q      = (int) roundf(fv / delta - (float) offset);
+                    const int q      = cvtt_x86((double) roundf(fv / delta - (float) offset));
                     const float dq   = delta * (float) (q + offset);
                     const double d   = (double) (fv - dq);
                     t                = p * (d * d);
@@ -799,8 +814,26 @@ __global__ __launch_bounds__(kBlock) void tfe_search_kernel(DevState* st, Search
             // The three sums are accumulated in ascending bucket order, the order of the reference's loops.  Every
             // lane runs the same chain (uniform bounds, LDS broadcast reads), so no cross-lane traffic is needed.
             const double satBottom = ordered_sum(term, 0, minInd);
-            const double satTop    = ordered_sum(term, maxInd, kPdf);
+            double satTop          = ordered_sum(term, maxInd, kPdf);
             const double quant     = ordered_sum(term, minInd, maxInd);
+            if (maxInd < minInd)
+            {
+                // Only after an index conversion left the int range (cvtt_x86).  The reference's three loops then
+                // overlap: buckets [maxInd, minInd) are saturation at the bottom AND at the top, and no bucket is
+                // quantization noise.  Redo the top sum with every bucket's distance to the top mid-point.
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int k = 0; k < kPdf / 64; ++k)
+                {
+                    const int i      = k * 64 + lane;
+                    const double mid = pdfStart + i * pdfStep + pdfStep / 2;
+                    const double d   = mid - maxMid;
+                    term[i]          = st->pdf[i] * (d * d);
+                }
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_s_waitcnt(0xc07f);
+                satTop = ordered_sum(term, maxInd, kPdf);
+            }
             cost = 3.0 * (satBottom + satTop) + quant;
             cost                   = (cost < DBL_MAX) ? cost : DBL_MAX;   // std::min(sqnr, max())
         }

@@ -21,6 +21,7 @@
  *   (oracle/_ref), except where its comment says "parity unpinned".
  */
 #include <float.h>
+#include <limits.h>
 #include <math.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -604,6 +605,14 @@ int orc_tfe_candidates(const orc_pdf* p, int bw, int sym, int strict, int unsign
 }
 
 /* DLQ/src/TfEnhancedEncodingAnalyzer.cpp:293-355, GAMMA = 3.0 (.h:102).  pow(v, 2) of the reference is v*v. */
+/* The reference casts with (int); outside the int range that is undefined in C++, and its x86-64 build (cvttsd2si /
+ * cvttss2si) yields INT_MIN, which then clamps to bucket 0.  Written out so that the restatement does not depend on
+ * what this compiler makes of the undefined cast. */
+static inline int orc_cvtt_x86(double v)
+{
+    return (v >= -2147483648.0 && v < 2147483648.0) ? (int) v : INT_MIN;
+}
+
 double orc_tfe_cost(const orc_pdf* p, int bw, float delta, int offset)
 {
     float minVal   = delta * (float) offset;
@@ -611,10 +620,10 @@ double orc_tfe_cost(const orc_pdf* p, int bw, float delta, int offset)
     float maxVal   = delta * ((float) offset + stepSize);
     float pdfStart = (float) p->xLeft[0];
     double pdfStep = p->xLeft[1] - p->xLeft[0];
-    int minInd     = (int) floor((minVal - pdfStart) / pdfStep);
+    int minInd     = orc_cvtt_x86(floor((minVal - pdfStart) / pdfStep));
     minInd         = (minInd < 0) ? 0 : minInd;
     minInd         = (minInd > ORC_PDF_SIZE - 1) ? ORC_PDF_SIZE - 1 : minInd;
-    int maxInd     = (int) floor((maxVal - pdfStart) / pdfStep);
+    int maxInd     = orc_cvtt_x86(floor((maxVal - pdfStart) / pdfStep));
     maxInd         = (maxInd < 0) ? 0 : maxInd;
     maxInd         = (maxInd > ORC_PDF_SIZE - 1) ? ORC_PDF_SIZE - 1 : maxInd;
 
@@ -638,7 +647,7 @@ double orc_tfe_cost(const orc_pdf* p, int bw, float delta, int offset)
     for (int i = minInd; i < maxInd; ++i)
     {
         float fv    = (float) (pdfStart + i * pdfStep + pdfStep / 2);
-        int q       = (int) roundf(fv / delta - (float) offset);
+        int q       = orc_cvtt_x86((double) roundf(fv / delta - (float) offset));
         float dq    = delta * (float) (q + offset);
         double diff = (double) (fv - dq);
         quant += p->pdf[i] * (diff * diff);

@@ -143,6 +143,19 @@ def test_tfe_constant_and_tiny(ops, oracle):
     _check_tfe(ops, oracle, [np.array([0.25], np.float32), np.array([0.25, 0.3, -0.1], np.float32)])
 
 
+@pytest.mark.parametrize("scale", [1e-30, 1e-22, 1e-12, 1.0, 1e12, 1e22, 1e30])
+def test_tfe_bucket_index_at_extreme_scales(ops, oracle, scale):
+    """The bucket index is round(x / bucket - offset) with an IEEE division.  The kernel divides through a reciprocal
+    plus residual corrections where that is exact (bucket width in [2^-64, 2^64], |x| <= 2^60) and with a true
+    division elsewhere; both sides of each limit, and a second batch with values far outside the first one's range."""
+    rng = np.random.default_rng(77)
+    b0 = (rng.standard_normal(150001) * scale).astype(np.float32)
+    b1 = (rng.standard_normal(150001) * scale).astype(np.float32)
+    b1[::97] *= np.float32(1e6)                       # outside the PDF range: dropped
+    b1[5:9] = [3e38, -3e38, np.inf, np.nan]
+    _check_tfe(ops, oracle, [b0, b1], modes=((8, 0, 0, 0), (8, 1, 0, 0)))
+
+
 def test_tfe_reset_and_unaligned(ops, oracle):
     an = ops.Analyzer(TFE)
     x = _relu_pareto(8, 50001)

@@ -127,11 +127,19 @@ def _relu_pareto(rng, n):
     return x
 
 
-@pytest.mark.parametrize("kind", ["n22", "relu_pareto", "gauss_outliers", "tiny", "zeros_then_data"])
+@pytest.mark.parametrize("kind", ["n22", "relu_pareto", "gauss_outliers", "tiny", "zeros_then_data", "scale_1e-30",
+                                  "scale_1e-22", "scale_1e-12", "scale_1e12", "scale_1e22", "scale_1e30"])
 def test_tf_enhanced_pdf_candidates_costs(oracle, ref, n22, kind):
     rng = np.random.default_rng(16)
     if kind == "n22":
         batches = [n22]
+    elif kind.startswith("scale_"):
+        # extreme magnitudes: at the small end a candidate range is more than 2^31 PDF buckets wide and the reference's
+        # (int) cast leaves the int range (its x86-64 build yields INT_MIN there, which the restatement spells out)
+        scale = float(kind[6:])
+        batches = [(rng.standard_normal(30000) * scale).astype(np.float32) for _ in range(2)]
+        batches[1][::97] *= np.float32(1e6)
+        batches[1][5:9] = [3e38, -3e38, np.inf, np.nan]
     elif kind == "relu_pareto":
         batches = [_relu_pareto(rng, 50000) for _ in range(4)]
     elif kind == "gauss_outliers":
