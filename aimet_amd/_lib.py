@@ -72,6 +72,7 @@ _SIGNATURES = {
     "miq_analyzer_last_search": ([_p, _p, _p, _p, _int, C.POINTER(_int), C.POINTER(_int), _p], _int),
     "miq_adaround_soft_round_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int, _p], _int),
     "miq_adaround_floor_f32": ([_p, _p, _i64, _i64, _i64, _p, _p], _int),
+    "miq_adaround_floor_i8": ([_p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _p, _p], _int),
     "miq_adaround_init_alpha_f32": ([_p, _p, _i64, _i64, _i64, _p, _p], _int),
     "miq_adaround_bwd_adam_f32": ([_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _flt, _flt, _flt,
                                    _flt, _flt, _flt, _int, _p, _p], _int),
@@ -87,6 +88,10 @@ _SIGNATURES = {
                                      _p, _p, _p, _p, _p], _int),
     "miq_adaround_linear_bwd_adam_f32": ([_p, _p, _p, _p, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
                                           _flt, _flt, _flt, _flt, _flt, _flt, _int, _p, _p], _int),
+    "miq_adaround_linear_fwd_i8": ([_p, _p, _p, _p, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
+                                    _p, _p, _p, _p, _p], _int),
+    "miq_adaround_linear_bwd_adam_i8": ([_p, _p, _p, _p, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
+                                         _flt, _flt, _flt, _flt, _flt, _flt, _int, _p, _p], _int),
 }
 
 # Entry points declared in include/miq.h; the loader insists on every one of them.

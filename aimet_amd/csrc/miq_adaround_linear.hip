@@ -57,6 +57,23 @@ __device__ __forceinline__ v4f ldg4_stream(const float* p)
     return __builtin_nontemporal_load(reinterpret_cast<const v4f*>(p));
 }
 
+// Four consecutive values of floor(W / delta), stored as float32 or, where every channel's window of useful values fits,
+// as int8 (miq_adaround_floor_i8): a quarter of the bytes of the operand that never changes during the optimisation.
+template <typename FT>
+__device__ __forceinline__ v4f load_floor4(const FT* p);
+template <>
+__device__ __forceinline__ v4f load_floor4<float>(const float* p)
+{
+    return ldg4_stream(p);
+}
+template <>
+__device__ __forceinline__ v4f load_floor4<int8_t>(const int8_t* p)
+{
+    const int32_t w = __builtin_nontemporal_load(reinterpret_cast<const int32_t*>(p));
+    return (v4f) {(float) (int8_t) (w & 0xff), (float) (int8_t) ((w >> 8) & 0xff), (float) (int8_t) ((w >> 16) & 0xff),
+                  (float) (w >> 24)};
+}
+
 constexpr int kLdsRow = kTileK + 4;   // floats per LDS tile row; the pad spreads the MFMA-layout accesses over banks
 
 // Both kernels work on a [32 o] x [256 k] tile of the weight-shaped tensors per workgroup and move it through LDS, so
@@ -66,7 +83,8 @@ constexpr int kLdsRow = kTileK + 4;   // floats per LDS tile row; the pad spread
 
 // grid (K / 256, O / 32), 256 threads: consecutive workgroups walk along the rows, so the workgroups that run together
 // cover contiguous memory (with the row blocks as the fast index the same tile reads measured 25 % slower).
-__global__ __launch_bounds__(256) void lin_fwd_kernel(const float* __restrict__ F, const float* __restrict__ alpha,
+template <typename FT>
+__global__ __launch_bounds__(256) void lin_fwd_kernel(const FT* __restrict__ F, const float* __restrict__ alpha,
                                                       const float* __restrict__ X, const int* __restrict__ row_index,
                                                       int64_t x_row_stride, float* __restrict__ partial, LinGeom g)
 {
@@ -92,7 +110,7 @@ __global__ __launch_bounds__(256) void lin_fwd_kernel(const float* __restrict__ 
     for (int j = 0; j < 8; ++j)
     {
         const int64_t e = (int64_t) (o_blk + wave * 8 + j) * K + k_blk + 4 * lane;
-        f[j]            = ldg4_stream(F + e);
+        f[j]            = load_floor4<FT>(F + e);
         al[j]           = ldg4_stream(alpha + e);
     }
     // the activations of this wavefront's MFMA k-range [64w, 64w + 64), fetched while the weights are in flight
@@ -210,8 +228,8 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
 // grid (K / 256, O / 32), 256 threads.  Phase 1: wavefront w forms dLoss/dW' for k in [64w, 64w + 64) as four 16-wide k
 // tiles (the M dimension of the MFMA) by two 16-wide o tiles (N), the batch being the MFMA's K dimension (8 steps of
 // 4), and parks it in the LDS tile.  Phase 2: the alpha-gradient + regulariser + Adam epilogue in the streaming layout.
-template <int PF>
-__global__ __launch_bounds__(256) void lin_bwd_kernel(const float* __restrict__ F, const float* __restrict__ G,
+template <int PF, typename FT>
+__global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, const float* __restrict__ G,
                                                       const float* __restrict__ X, const int* __restrict__ row_index,
                                                       int64_t x_row_stride, float* __restrict__ alpha,
                                                       float* __restrict__ m, float* __restrict__ v,
@@ -231,7 +249,7 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const float* __restrict__ 
     for (int j = 0; j < PF; ++j)
     {
         const int64_t e = (int64_t) (o_blk + wave * 8 + j) * K + k_blk + 4 * lane;
-        fv[j]           = ldg4_stream(F + e);
+        fv[j]           = load_floor4<FT>(F + e);
         av[j]           = ldg4(alpha + e);
         mv[j]           = ldg4(m + e);
         vv[j]           = ldg4(v + e);
@@ -290,7 +308,7 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const float* __restrict__ 
         if (j + PF < 8)
         {
             const int64_t e2 = e + PF * (int64_t) K;
-            fv[slot]         = ldg4_stream(F + e2);
+            fv[slot]         = load_floor4<FT>(F + e2);
             av[slot]         = ldg4(alpha + e2);
             mv[slot]         = ldg4(m + e2);
             vv[slot]         = ldg4(v + e2);
@@ -349,6 +367,58 @@ int make_lin_geom(LinGeom& g, int64_t out_features, int64_t in_features, int64_t
 
 using namespace miq;
 
+template <typename FT>
+static int linear_fwd(const FT* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
+                      int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+                      int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
+                      const float* offset, float clip_min, float clip_max, int activation, float* workspace, float* out,
+                      float* grad_out, float* loss_partial, void* stream)
+{
+    LinGeom g;
+    if (int rc = make_lin_geom(g, out_features, in_features, num_channel, delta, offset, clip_min, clip_max))
+        return rc;
+    MIQ_CHECK_ARG(weight_floor && alpha && x && target && workspace && grad_out, "null tensor pointer");
+    MIQ_CHECK_ARG(aligned16(weight_floor) && aligned16(alpha) && aligned16(x) && (x_row_stride % 4) == 0,
+                  "weight_floor, alpha and the rows of x must be 16-byte aligned");
+    MIQ_CHECK_ARG(x_row_stride >= in_features && target_row_stride >= out_features, "row stride shorter than a row");
+    MIQ_CHECK_ARG(activation == 0 || activation == 1, "activation must be 0 (none) or 1 (ReLU)");
+    const int splits = (int) (in_features / kTileK);
+    hipLaunchKernelGGL((lin_fwd_kernel<FT>), dim3((unsigned) splits, (unsigned) (out_features / kTileO)), dim3(256), 0,
+                       (hipStream_t) stream, weight_floor, alpha, x, row_index, x_row_stride, workspace, g);
+    MIQ_CHECK_LAUNCH();
+    const unsigned blocks = (unsigned) ((kBatch * out_features + 255) / 256);
+    hipLaunchKernelGGL(lin_loss_kernel, dim3(blocks), dim3(256), 0, (hipStream_t) stream, workspace, splits, bias, target,
+                       row_index, target_row_stride, (int) out_features, activation, out, grad_out, loss_partial);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+template <typename FT>
+static int linear_bwd_adam(const FT* weight_floor, const float* grad_out, const float* x, const int32_t* row_index,
+                           int64_t x_row_stride, float* alpha, float* exp_avg, float* exp_avg_sq, float* grad_alpha,
+                           int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
+                           const float* offset, float clip_min, float clip_max, float reg_param, float beta, float lr,
+                           float beta1, float beta2, float eps, int step, float* reg_partial, void* stream)
+{
+    LinGeom g;
+    if (int rc = make_lin_geom(g, out_features, in_features, num_channel, delta, offset, clip_min, clip_max))
+        return rc;
+    MIQ_CHECK_ARG(weight_floor && grad_out && x && alpha && exp_avg && exp_avg_sq, "null tensor pointer");
+    MIQ_CHECK_ARG(aligned16(weight_floor) && aligned16(alpha) && aligned16(exp_avg) && aligned16(exp_avg_sq) &&
+                      aligned16(grad_alpha),
+                  "tensors must be 16-byte aligned");
+    MIQ_CHECK_ARG(x_row_stride >= in_features, "row stride shorter than a row");
+    AdamArgs a;
+    if (int rc = make_adam(a, reg_param, beta, lr, beta1, beta2, eps, step))
+        return rc;
+    // two rows of the epilogue in flight per lane: deeper prefetch (3, 4) costs registers and measured no faster
+    hipLaunchKernelGGL((lin_bwd_kernel<2, FT>), dim3((unsigned) (in_features / kTileK), (unsigned) (out_features / kTileO)),
+                       dim3(256), 0, (hipStream_t) stream, weight_floor, grad_out, x, row_index, x_row_stride, alpha,
+                       exp_avg, exp_avg_sq, grad_alpha, g, a, reg_partial);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
 extern "C" {
 
 int64_t miq_adaround_linear_workspace_bytes(int64_t out_features, int64_t in_features)
@@ -364,56 +434,51 @@ int miq_adaround_linear_blocks(int64_t out_features, int64_t in_features)
     return (int) ((out_features / kTileO) * (in_features / kTileK));
 }
 
-int miq_adaround_linear_fwd_f32(const float* weight, const float* alpha, const float* x, const int32_t* row_index,
+int miq_adaround_linear_fwd_f32(const float* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
                                 int64_t x_row_stride, const float* target, int64_t target_row_stride,
                                 const float* bias, int64_t out_features, int64_t in_features, int64_t num_channel,
                                 const float* delta, const float* offset, float clip_min, float clip_max,
                                 int activation, float* workspace, float* out, float* grad_out, float* loss_partial,
                                 void* stream)
 {
-    LinGeom g;
-    if (int rc = make_lin_geom(g, out_features, in_features, num_channel, delta, offset, clip_min, clip_max))
-        return rc;
-    MIQ_CHECK_ARG(weight && alpha && x && target && workspace && grad_out, "null tensor pointer");
-    MIQ_CHECK_ARG(aligned16(weight) && aligned16(alpha) && aligned16(x) && (x_row_stride % 4) == 0,
-                  "weight, alpha and the rows of x must be 16-byte aligned");
-    MIQ_CHECK_ARG(x_row_stride >= in_features && target_row_stride >= out_features, "row stride shorter than a row");
-    MIQ_CHECK_ARG(activation == 0 || activation == 1, "activation must be 0 (none) or 1 (ReLU)");
-    const int splits = (int) (in_features / kTileK);
-    hipLaunchKernelGGL(lin_fwd_kernel, dim3((unsigned) splits, (unsigned) (out_features / kTileO)), dim3(256), 0,
-                       (hipStream_t) stream, weight, alpha, x, row_index, x_row_stride, workspace, g);
-    MIQ_CHECK_LAUNCH();
-    const unsigned blocks = (unsigned) ((kBatch * out_features + 255) / 256);
-    hipLaunchKernelGGL(lin_loss_kernel, dim3(blocks), dim3(256), 0, (hipStream_t) stream, workspace, splits, bias, target,
-                       row_index, target_row_stride, (int) out_features, activation, out, grad_out, loss_partial);
-    MIQ_CHECK_LAUNCH();
-    return MIQ_OK;
+    return linear_fwd<float>(weight_floor, alpha, x, row_index, x_row_stride, target, target_row_stride, bias,
+                             out_features, in_features, num_channel, delta, offset, clip_min, clip_max, activation,
+                             workspace, out, grad_out, loss_partial, stream);
 }
 
-int miq_adaround_linear_bwd_adam_f32(const float* weight, const float* grad_out, const float* x,
+int miq_adaround_linear_fwd_i8(const int8_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
+                               int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+                               int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
+                               const float* offset, float clip_min, float clip_max, int activation, float* workspace,
+                               float* out, float* grad_out, float* loss_partial, void* stream)
+{
+    return linear_fwd<int8_t>(weight_floor, alpha, x, row_index, x_row_stride, target, target_row_stride, bias,
+                              out_features, in_features, num_channel, delta, offset, clip_min, clip_max, activation,
+                              workspace, out, grad_out, loss_partial, stream);
+}
+
+int miq_adaround_linear_bwd_adam_f32(const float* weight_floor, const float* grad_out, const float* x,
                                      const int32_t* row_index, int64_t x_row_stride, float* alpha, float* exp_avg,
                                      float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                      int64_t num_channel, const float* delta, const float* offset, float clip_min,
                                      float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
                                      float eps, int step, float* reg_partial, void* stream)
 {
-    LinGeom g;
-    if (int rc = make_lin_geom(g, out_features, in_features, num_channel, delta, offset, clip_min, clip_max))
-        return rc;
-    MIQ_CHECK_ARG(weight && grad_out && x && alpha && exp_avg && exp_avg_sq, "null tensor pointer");
-    MIQ_CHECK_ARG(aligned16(weight) && aligned16(alpha) && aligned16(exp_avg) && aligned16(exp_avg_sq) &&
-                      aligned16(grad_alpha),
-                  "tensors must be 16-byte aligned");
-    MIQ_CHECK_ARG(x_row_stride >= in_features, "row stride shorter than a row");
-    AdamArgs a;
-    if (int rc = make_adam(a, reg_param, beta, lr, beta1, beta2, eps, step))
-        return rc;
-    // two rows of the epilogue in flight per lane: deeper prefetch (4, 8) costs occupancy and measured 5 % slower
-    hipLaunchKernelGGL(lin_bwd_kernel<2>, dim3((unsigned) (in_features / kTileK), (unsigned) (out_features / kTileO)),
-                       dim3(256), 0, (hipStream_t) stream, weight, grad_out, x, row_index, x_row_stride, alpha, exp_avg,
-                       exp_avg_sq, grad_alpha, g, a, reg_partial);
-    MIQ_CHECK_LAUNCH();
-    return MIQ_OK;
+    return linear_bwd_adam<float>(weight_floor, grad_out, x, row_index, x_row_stride, alpha, exp_avg, exp_avg_sq,
+                                  grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min, clip_max,
+                                  reg_param, beta, lr, beta1, beta2, eps, step, reg_partial, stream);
+}
+
+int miq_adaround_linear_bwd_adam_i8(const int8_t* weight_floor, const float* grad_out, const float* x,
+                                    const int32_t* row_index, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                    float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
+                                    int64_t num_channel, const float* delta, const float* offset, float clip_min,
+                                    float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
+                                    float eps, int step, float* reg_partial, void* stream)
+{
+    return linear_bwd_adam<int8_t>(weight_floor, grad_out, x, row_index, x_row_stride, alpha, exp_avg, exp_avg_sq,
+                                   grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min,
+                                   clip_max, reg_param, beta, lr, beta1, beta2, eps, step, reg_partial, stream);
 }
 
 }   // extern "C"

@@ -343,6 +343,20 @@ def adaround_floor(weight, num_channel, n_per_channel, delta):
     return out
 
 
+def adaround_floor_i8(weight, num_channel, n_per_channel, delta, offset, clip_min, clip_max):
+    """floor(w / delta) as int8, saturated per channel to the window outside which its value cannot matter
+    (offset + clip_min - 2 .. offset + clip_max + 1), or None when some channel's window does not fit int8.
+    Reads one flag back from the device (once per layer)."""
+    _ada_check(weight)
+    out = torch.empty(weight.shape, dtype=torch.int8, device=weight.device)
+    unfit = torch.zeros(1, dtype=torch.int32, device=weight.device)
+    with torch.cuda.device(weight.device):
+        check(lib.miq_adaround_floor_i8(_ptr(weight), _ptr(out), int(num_channel), weight.numel(), int(n_per_channel),
+                                        _ptr(delta), _ptr(offset), float(clip_min), float(clip_max), _ptr(unfit),
+                                        _stream(weight)))
+    return None if int(unfit.item()) else out
+
+
 def adaround_init_alpha(weight, num_channel, n_per_channel, delta):
     """alpha such that h(alpha) equals the fractional part of w / delta."""
     _ada_check(weight)
@@ -400,10 +414,19 @@ def adaround_linear_blocks(out_features, in_features):
     return int(lib.miq_adaround_linear_blocks(int(out_features), int(in_features)))
 
 
+def _floor_variant(weight_floor, alpha, prefix):
+    """Entry point for the storage type of floor(W / delta): float32 or int8 (adaround_floor_i8)."""
+    if weight_floor.dtype not in (_F32, torch.int8) or not weight_floor.is_contiguous() or \
+            weight_floor.shape != alpha.shape or not weight_floor.is_cuda:
+        raise RuntimeError("weight_floor must be a contiguous float32 or int8 GPU tensor of alpha's shape")
+    return getattr(lib, prefix + ("f32" if weight_floor.dtype == _F32 else "i8"))
+
+
 def adaround_linear_fwd(weight_floor, alpha, x, row_index, target, bias, num_channel, delta, offset, clip_min, clip_max,
                         activation, workspace, grad_out, out=None, loss_partial=None):
     """Fused apply_adaround + Linear forward + reconstruction-loss gradient for 32 rows of x / target."""
-    _ada_check(weight_floor, alpha, workspace, grad_out, out)
+    _ada_check(alpha, workspace, grad_out, out)
+    fn = _floor_variant(weight_floor, alpha, "miq_adaround_linear_fwd_")
     _require_gpu(weight_floor, x, target, bias, row_index)
     if x.dtype != _F32 or target.dtype != _F32 or x.stride(-1) != 1 or target.stride(-1) != 1:
         raise RuntimeError("x and target must be float32 with contiguous rows")
@@ -411,27 +434,24 @@ def adaround_linear_fwd(weight_floor, alpha, x, row_index, target, bias, num_cha
         raise RuntimeError("row_index must hold 32 int32 row numbers")
     o, k = weight_floor.shape
     with torch.cuda.device(weight_floor.device):
-        check(lib.miq_adaround_linear_fwd_f32(_ptr(weight_floor), _ptr(alpha), _ptr(x), _ptr(row_index), x.stride(0),
-                                              _ptr(target), target.stride(0), _ptr(bias), o, k, int(num_channel),
-                                              _ptr(delta), _ptr(offset), float(clip_min), float(clip_max),
-                                              int(activation), _ptr(workspace), _ptr(out), _ptr(grad_out),
-                                              _ptr(loss_partial), _stream(weight_floor)))
+        check(fn(_ptr(weight_floor), _ptr(alpha), _ptr(x), _ptr(row_index), x.stride(0), _ptr(target), target.stride(0),
+                 _ptr(bias), o, k, int(num_channel), _ptr(delta), _ptr(offset), float(clip_min), float(clip_max),
+                 int(activation), _ptr(workspace), _ptr(out), _ptr(grad_out), _ptr(loss_partial), _stream(weight_floor)))
 
 
 def adaround_linear_bwd_adam(weight_floor, grad_out, x, row_index, alpha, exp_avg, exp_avg_sq, num_channel, delta, offset,
                              clip_min, clip_max, reg_param, beta, lr, beta1, beta2, eps, step, reg_partial=None,
                              grad_alpha=None):
     """Fused dLoss/dW' = grad_out^T x (MFMA) + alpha gradient + regulariser + Adam update (alpha, moments in place)."""
-    _ada_check(weight_floor, grad_out, alpha, exp_avg, exp_avg_sq, grad_alpha)
+    _ada_check(grad_out, alpha, exp_avg, exp_avg_sq, grad_alpha)
+    fn = _floor_variant(weight_floor, alpha, "miq_adaround_linear_bwd_adam_")
     _require_gpu(weight_floor, x, row_index)
     o, k = weight_floor.shape
     with torch.cuda.device(weight_floor.device):
-        check(lib.miq_adaround_linear_bwd_adam_f32(_ptr(weight_floor), _ptr(grad_out), _ptr(x), _ptr(row_index),
-                                                   x.stride(0), _ptr(alpha), _ptr(exp_avg), _ptr(exp_avg_sq),
-                                                   _ptr(grad_alpha), o, k, int(num_channel), _ptr(delta),
-                                                   _ptr(offset), float(clip_min), float(clip_max), float(reg_param),
-                                                   float(beta), float(lr), float(beta1), float(beta2), float(eps),
-                                                   int(step), _ptr(reg_partial), _stream(weight_floor)))
+        check(fn(_ptr(weight_floor), _ptr(grad_out), _ptr(x), _ptr(row_index), x.stride(0), _ptr(alpha), _ptr(exp_avg),
+                 _ptr(exp_avg_sq), _ptr(grad_alpha), o, k, int(num_channel), _ptr(delta), _ptr(offset), float(clip_min),
+                 float(clip_max), float(reg_param), float(beta), float(lr), float(beta1), float(beta2), float(eps),
+                 int(step), _ptr(reg_partial), _stream(weight_floor)))
 
 
 class Analyzer:

@@ -182,7 +182,27 @@ def bench_calibration(torch, ops, reps):
     acc = sum(acc_ms) / len(acc_ms)
     tot = sum(total_ms) / len(total_ms)
     elems = 16 * n
+    # the same accumulation when the calibration batches are larger (one update call = one launch: the launch's fixed
+    # cost is what keeps the 25.7 MB batches of the configuration below the kernel's streaming rate)
+    by_size = {}
+    for mult in (1, 4, 8):
+        big = torch.cat(batches[:mult]) if mult > 1 else batches[0]
+        an.reset()
+        an.update_stats(big)
+        an.update_stats(big)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(8):
+            an.update_stats(big)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / 8
+        by_size[f"{mult}x[32,256,28,28]"] = {"update_us": ms * 1e3, "GBps": 4 * n * mult / ms / 1e6,
+                                             "frac_hbm": 4 * n * mult / ms / 1e6 / HBM_PEAK_GBPS}
+        del big
     return {"elements": elems, "accumulate_ms": acc, "search_ms_wall": sum(search_ms) / len(search_ms),
+            "update_by_batch_size": by_size,
             "total_ms_wall": tot, "elements_per_s": elems / (tot / 1e3),
             "accumulate_GBps": 17 * 4 * n / acc / 1e6, "accumulate_frac_hbm": 17 * 4 * n / acc / 1e6 / HBM_PEAK_GBPS,
             "encoding": [enc.min, enc.max, enc.delta, enc.offset]}
@@ -236,8 +256,14 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
             wrapper.alpha.data.copy_(alpha0)
     AdaroundOptimizer.use_fused_linear = True
 
-    # per-kernel times of the fused iteration
-    w = ops.adaround_floor(wrapper.weight.detach(), wrapper.num_channel, wrapper.n_per_channel, wrapper.delta)
+    # per-kernel times of the fused iteration (floor(W / delta) as the optimizer stores it: int8 for this 4-bit grid;
+    # the algorithmic bytes below stay those of the float32 formulation, 8 and 28 B/element)
+    w = ops.adaround_floor_i8(wrapper.weight.detach(), wrapper.num_channel, wrapper.n_per_channel, wrapper.delta,
+                              wrapper.offset, wrapper.clip_min, wrapper.clip_max)
+    floor_storage = "int8"
+    if w is None:
+        w = ops.adaround_floor(wrapper.weight.detach(), wrapper.num_channel, wrapper.n_per_channel, wrapper.delta)
+        floor_storage = "float32"
     alpha = wrapper.alpha.data
     m, v = torch.zeros_like(alpha), torch.zeros_like(alpha)
     ws = ops.adaround_linear_workspace(o, k, w.device)
@@ -258,7 +284,7 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
     f = sum(e[0].elapsed_time(e[1]) for e in ev) / timed_kernel_iters
     b = sum(e[1].elapsed_time(e[2]) for e in ev) / timed_kernel_iters
     res["fused_kernels"] = {
-        "fwd_ms": f, "bwd_ms": b,
+        "fwd_ms": f, "bwd_ms": b, "floor_storage": floor_storage,
         "fwd_algorithmic_bytes": 8 * n, "fwd_GBps": 8 * n / f / 1e6, "fwd_frac_hbm": 8 * n / f / 1e6 / HBM_PEAK_GBPS,
         "fwd_mfma_TFLOPs": 2.0 * 32 * n / f / 1e9,
         "bwd_algorithmic_bytes": 28 * n, "bwd_GBps": 28 * n / b / 1e6, "bwd_frac_hbm": 28 * n / b / 1e6 / HBM_PEAK_GBPS,

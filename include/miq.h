@@ -260,6 +260,14 @@ int miq_adaround_soft_round_f32(const float* weight, const float* alpha, float* 
  * on alpha; the fused Linear entry points below take it in place of the weight. */
 int miq_adaround_floor_f32(const float* weight, float* weight_floor, int64_t num_channel, int64_t num_element,
                            int64_t num_element_per_channel, const float* delta, void* stream);
+/* floor(weight / delta) saturated per channel to [offset + clip_min - 2, offset + clip_max + 1] and stored as int8.
+ * h(alpha) lies in [0, 1], so outside that window clamp(floor + h - offset, clip_min, clip_max) and its gradient mask
+ * no longer depend on the exact value: the fused Linear kernels give the same results from this form as from the
+ * float32 one.  *unfit (device int32, zero on entry) is set to 1 when some channel's window leaves the int8 range
+ * (grids wider than 7 bits, or offsets far from zero): the output is then unusable and the caller keeps float32. */
+int miq_adaround_floor_i8(const float* weight, int8_t* weight_floor, int64_t num_channel, int64_t num_element,
+                          int64_t num_element_per_channel, const float* delta, const float* offset, float clip_min,
+                          float clip_max, int32_t* unfit, void* stream);
 /* AdaroundWrapper._generate_alpha_parameter (ADA/adaround_wrapper.py:211-224):
  *   alpha = -log((zeta - gamma) / (w / delta - floor(w / delta) - gamma) - 1) */
 int miq_adaround_init_alpha_f32(const float* weight, float* alpha, int64_t num_channel, int64_t num_element,
@@ -303,6 +311,10 @@ int miq_adaround_blocks(int64_t num_element);
  * activation: 0 none, 1 ReLU (the act_func the reference applies to both outputs, ADA/adaround_optimizer.py:192-194).
  * ------------------------------------------------------------------------------------------------------------- */
 
+/* The same two entry points with weight_floor stored as int8 (miq_adaround_floor_i8): a quarter of the bytes of the one
+ * weight-shaped operand that never changes during the optimisation.  No counterpart in the reference; results are
+ * identical to the float32 form, element for element. */
+
 /* Bytes of device workspace the forward needs (partial products of the split K dimension). */
 int64_t miq_adaround_linear_workspace_bytes(int64_t out_features, int64_t in_features);
 /* Number of regulariser partial sums miq_adaround_linear_bwd_adam_f32 writes. */
@@ -323,6 +335,18 @@ int miq_adaround_linear_bwd_adam_f32(const float* weight_floor, const float* gra
                                      int64_t num_channel, const float* delta, const float* offset, float clip_min,
                                      float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
                                      float eps, int step, float* reg_partial, void* stream);
+
+int miq_adaround_linear_fwd_i8(const int8_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
+                               int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+                               int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
+                               const float* offset, float clip_min, float clip_max, int activation, float* workspace,
+                               float* out, float* grad_out, float* loss_partial, void* stream);
+int miq_adaround_linear_bwd_adam_i8(const int8_t* weight_floor, const float* grad_out, const float* x,
+                                    const int32_t* row_index, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                    float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
+                                    int64_t num_channel, const float* delta, const float* offset, float clip_min,
+                                    float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
+                                    float eps, int step, float* reg_partial, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
  * v2 histogram observer + SQNR encoding analyzer

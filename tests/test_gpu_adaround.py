@@ -173,6 +173,9 @@ def test_fused_linear_forward_and_backward(ops, shape, per_channel, act):
     per-element arithmetic, different summation order in the GEMMs) and against the CPU restatement."""
     O, K = shape
     weight, delta, offset, C, npc, cmin, cmax = _case(31, shape, 0, per_channel)
+    weight[1, 5] *= 6.0                                 # far outside the grid on both sides
+    weight[2, 7] = -weight[2].abs().max() * 5.0
+    weight[3, 9] = weight[3].abs().max() * 5.0
     torch.manual_seed(32)
     X, bias = torch.randn(100, K), torch.randn(O) * 0.1
     Y = torch.nn.functional.linear(X, weight, bias) + torch.randn(100, O) * 0.01
@@ -223,6 +226,26 @@ def test_fused_linear_forward_and_backward(ops, shape, per_channel, act):
     assert torch.allclose(m1, m2, atol=2e-5 * m2.abs().max().item(), rtol=1e-4)
     assert torch.allclose(v1, v2, atol=2e-5 * v2.abs().max().item(), rtol=1e-4)
     assert rp1.sum().item() == pytest.approx(rp2.sum().item(), rel=1e-5)
+    # floor(W / delta) stored as int8: saturated to the window outside which its value cannot matter; everything the
+    # two kernels produce from it is identical, bit for bit, to what they produce from the float32 form
+    f8 = ops.adaround_floor_i8(wg, C, npc, dg, og, cmin, cmax)
+    assert f8 is not None and f8.dtype == torch.int8
+    lo, hi = o + cmin - 2, o + cmax + 1
+    assert torch.equal(f8.cpu().float(), torch.minimum(torch.maximum(torch.floor(weight / d), lo), hi))
+    assert (torch.floor(weight / d) < lo).any() and (torch.floor(weight / d) > hi).any()   # saturation happens
+    G8, out8, lp8 = torch.empty_like(G), torch.empty_like(out), torch.zeros_like(lp)
+    ops.adaround_linear_fwd(f8, ag, Xg, ig, Yg, bg, C, dg, og, cmin, cmax, act, ws, G8, out=out8, loss_partial=lp8)
+    assert torch.equal(out8, out) and torch.equal(G8, G) and torch.equal(lp8, lp)
+    a8, m8, v8 = ag.clone(), m0.cuda(), v0.cuda()
+    g8, rp8 = torch.empty_like(a8), torch.zeros_like(rp1)
+    ops.adaround_linear_bwd_adam(f8, G, Xg, ig, a8, m8, v8, C, dg, og, cmin, cmax, reg_partial=rp8, grad_alpha=g8,
+                                 **hyper)
+    assert torch.equal(a8, a1) and torch.equal(m8, m1) and torch.equal(v8, v1) and torch.equal(g8, g1)
+    assert torch.equal(rp8, rp1)
+    # a grid of 8 bits does not fit: the window is 259 values wide
+    assert ops.adaround_floor_i8(wg, C, npc, dg, og, 0, 255) is None
+    assert ops.adaround_floor_i8(wg, C, npc, dg, og + 200, cmin, cmax) is None
+
     # CPU gradient of the full loss (reconstruction + regulariser) w.r.t. alpha
     h = ada.rectified_sigmoid(a_ref)
     reg = hyper["reg_param"] * torch.add(1, -(torch.add(2 * h, -1).abs()).pow(hyper["beta"])).sum()
@@ -267,6 +290,13 @@ def test_fused_optimisation_trajectory(ops, act, per_channel, monkeypatch):
     a, m, v, g = _run_product_loop("linear", weight, alpha0, delta, offset, C, npc, cmin, cmax, all_inp, all_out,
                                    batches, hyper, act, {})
     assert len(calls) == iters                          # the fused path ran
+    from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
+    assert AdaroundOptimizer.use_int8_floor
+    monkeypatch.setattr(AdaroundOptimizer, "use_int8_floor", False)
+    a32, m32, v32, g32 = _run_product_loop("linear", weight, alpha0, delta, offset, C, npc, cmin, cmax, all_inp,
+                                           all_out, batches, hyper, act, {})
+    for got, want in ((a, a32), (m, m32), (v, v32), (g, g32)):
+        assert torch.equal(got, want)                   # int8 and float32 storage of floor(W / delta): same trajectory
     assert (a_ref - alpha0).abs().max() > 5e-3
     assert _close_except_few(a, a_ref, atol=5e-5)
     assert (a - a_ref).abs().max() < 5e-3               # and nowhere by more than a few steps of lr = 1e-3
