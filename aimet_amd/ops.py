@@ -14,8 +14,20 @@ from ._lib import Encoding, check, lib
 _F32, _BF16 = torch.float32, torch.bfloat16
 
 
+# torch.cuda.current_stream() builds a Stream object (about 3 us per call, as much as queueing a kernel); the raw
+# handle of the same stream is available without it
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)  # pylint: disable=protected-access
+
+
+def _stream_of(device):
+    """HIP stream handle (an integer) of torch's current stream on `device`."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
+
+
 def _stream(t):
-    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+    return C.c_void_p(_stream_of(t.device))
 
 
 def _ptr(t):
@@ -476,7 +488,7 @@ class Analyzer:
             lib.miq_analyzer_destroy(h)
 
     def _s(self):
-        return C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+        return C.c_void_p(_stream_of(self.device))
 
     def reset(self):
         with torch.cuda.device(self.device):
@@ -496,7 +508,7 @@ class Analyzer:
         # the caching allocator cannot hand its memory to anyone else before they have run
         if torch.cuda.current_device() == self.device.index:
             check(lib.miq_analyzer_update_stats_f32(self._h, x.data_ptr(), x.numel(),
-                                                    torch.cuda.current_stream().cuda_stream))
+                                                    _stream_of(self.device)))
         else:
             with torch.cuda.device(self.device):
                 check(lib.miq_analyzer_update_stats_f32(self._h, x.data_ptr(), x.numel(), self._s()))

@@ -320,3 +320,29 @@ def test_more_than_2_31_elements(ops, oracle):
         xs = x[a0:b].cpu().numpy()
         want = oracle.qdq_per_channel(xs, C, npc, params)
         assert np.array_equal(yc[a0:b].cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_kernels_run_on_torch_current_stream(ops, oracle):
+    """The entry points take a stream; the Python layer passes torch's current one.  On a side stream the input is
+    written after a long sleep kernel: a launch on any other stream would read the tensor before that write."""
+    n = 1 << 20
+    side = torch.cuda.Stream()
+    x = torch.zeros(n, device="cuda")
+    g = torch.ones(n, device="cuda")
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        torch.cuda._sleep(100_000_000)                   # tens of milliseconds on this stream only
+        x.fill_(0.7)
+        y = ops.qdq_per_tensor(x, -1.0, 1.0, 8)
+        gin = ops.ste_bwd_per_tensor(x * 2, g, -1.0, 1.0)
+        an = ops.Analyzer(1)
+        an.update_stats(x)
+        mm = ops.minmax(x)
+    assert not side.query()                              # nothing above waited for the device
+    side.synchronize()
+    want = oracle.qdq_per_tensor(np.full(4, 0.7, np.float32), -1.0, 1.0, 8)[0]
+    assert torch.equal(y, torch.full_like(y, float(want)))
+    assert gin.sum().item() == 0                         # 1.4 lies outside [-1, 1]
+    assert mm.tolist() == [pytest.approx(0.7), pytest.approx(0.7)]
+    xl, pdf = an.get_stats_histogram()
+    assert pdf.sum() == pytest.approx(1.0) and (pdf > 0).sum() == 1
