@@ -129,7 +129,10 @@ class QuantizationSimModel:
 
     # ------------------------------------------------------------------------------------------------ construction
     @staticmethod
-    def _load_config(config_file: str) -> dict:
+    def _load_config(config_file) -> dict:
+        """`config_file`: path of a JSON configuration, or the configuration itself as a dictionary."""
+        if isinstance(config_file, dict):
+            return config_file
         with open(config_file) as f:
             return json.load(f)
 

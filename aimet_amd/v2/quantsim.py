@@ -1,82 +1,144 @@
-"""Minimal v2 QuantizationSimModel: every supported leaf module becomes a quantized module with QuantizeDequantize
-quantizers (reference: TrainingExtensions/torch/src/python/aimet_torch/v2/quantsim/quantsim.py, which builds on the v1
-configurator; here only the defaults are implemented: symmetric parameter quantizers for weights, asymmetric output
-quantizers for every layer, an input quantizer for the model inputs, per-tensor or per-output-channel weights).
+"""v2 QuantizationSimModel: the model's leaf modules become quantized modules (aimet_amd.v2.nn) whose quantizers are the
+HIP-backed QuantizeDequantize modules.
+
+As in the reference (TrainingExtensions/torch/src/python/aimet_torch/v2/quantsim/quantsim.py:94-205, which derives from
+the v1 class), which quantizers exist and how they are set up is decided by the v1 configurator -- defaults, params,
+op_type, supergroups, model_input / model_output of the JSON configuration -- and every enabled v1 quantizer is then
+realised as its v2 counterpart (aimet_torch/quantsim_config/builder.py:204-357): QuantizeDequantize(shape, bitwidth,
+symmetric, encoding analyzer of the quant scheme), shape () per tensor or [C, 1, ...] per channel.  Strict-symmetric and
+unsigned-symmetric grids are refused for symmetric quantizers, as the reference's builder does.
 """
-import copy
+import contextlib
+import json
+import os
 from typing import Tuple, Union
 
 import torch
 from torch import nn
 
-from ..common.defs import QuantScheme
+from ..common.defs import QuantizationDataType, QuantScheme
+from ..v1.qc_quantize_op import StaticGridQuantWrapper
+from ..v1.quantsim import QuantizationSimModel as _V1QuantizationSimModel
+from ..v1.tensor_quantizer import StaticGridPerChannelQuantizer
 from .nn import BaseQuantizationMixin, QuantizationMixin
 from .quantization.affine import QuantizeDequantize
-from .quantization.encoding_analyzer import MinMaxEncodingAnalyzer, SqnrEncodingAnalyzer
+from .quantization.encoding_analyzer import MinMaxEncodingAnalyzer, PercentileEncodingAnalyzer, SqnrEncodingAnalyzer
+
+_RANGE_LEARNING = (QuantScheme.training_range_learning_with_tf_init,
+                   QuantScheme.training_range_learning_with_tf_enhanced_init)
 
 
 def _analyzer(quant_scheme: QuantScheme, shape):
-    if quant_scheme == QuantScheme.post_training_tf:
+    """Encoding analyzer of a v1 quant scheme (builder.py:290-305)."""
+    if quant_scheme in (QuantScheme.post_training_tf, QuantScheme.training_range_learning_with_tf_init):
         return MinMaxEncodingAnalyzer(shape)
-    if quant_scheme == QuantScheme.post_training_tf_enhanced:
+    if quant_scheme == QuantScheme.post_training_percentile:
+        return PercentileEncodingAnalyzer(shape)
+    if quant_scheme in (QuantScheme.post_training_tf_enhanced,
+                        QuantScheme.training_range_learning_with_tf_enhanced_init):
         return SqnrEncodingAnalyzer(shape)
-    raise ValueError(f"quant_scheme {quant_scheme} is not implemented (tf and tf_enhanced are)")
+    raise NotImplementedError(f"quant scheme {quant_scheme} is not supported")
 
 
 class QuantizationSimModel:
-    """Replaces the supported leaf modules of a copy of `model` by their quantized counterparts."""
+    """Replaces the leaf modules of (a copy of) `model` by quantized modules configured like the v1 simulation."""
 
+    # pylint: disable=too-many-arguments
     def __init__(self, model: nn.Module, dummy_input: Union[torch.Tensor, Tuple] = None,
                  quant_scheme: Union[str, QuantScheme] = QuantScheme.post_training_tf_enhanced,
-                 default_output_bw: int = 8, default_param_bw: int = 8, in_place: bool = False,
-                 per_channel_quantization: bool = False, config_file: str = None):
-        if config_file is not None:
-            raise NotImplementedError("configuration files are implemented by the v1 QuantizationSimModel only")
-        if isinstance(quant_scheme, str):
-            quant_scheme = {'tf': QuantScheme.post_training_tf,
-                            'tf_enhanced': QuantScheme.post_training_tf_enhanced}[quant_scheme]
-        self._quant_scheme = quant_scheme
-        self.model = model if in_place else copy.deepcopy(model)
+                 rounding_mode: str = 'nearest', default_output_bw: int = 8, default_param_bw: int = 8,
+                 in_place: bool = False, config_file: Union[str, dict] = None,
+                 default_data_type: QuantizationDataType = QuantizationDataType.int,
+                 per_channel_quantization: bool = None):
+        if dummy_input is None:
+            raise ValueError("dummy_input is needed: the configuration follows the order in which modules run")
+        if rounding_mode != 'nearest':
+            raise ValueError("v2 quantizers round to nearest")
+        if per_channel_quantization is not None:
+            # shorthand for the one default most callers change
+            if isinstance(config_file, (str, os.PathLike)):
+                with open(config_file) as f:
+                    config_file = json.load(f)
+            elif config_file is None:
+                from ..v1.quantsim import DEFAULT_CONFIG  # pylint: disable=import-outside-toplevel
+                config_file = DEFAULT_CONFIG
+            config_file = json.loads(json.dumps(config_file))
+            config_file.setdefault("defaults", {})["per_channel_quantization"] = str(bool(per_channel_quantization))
+        v1 = _V1QuantizationSimModel(model, dummy_input, quant_scheme, rounding_mode, default_output_bw,
+                                     default_param_bw, in_place, config_file, default_data_type)
+        self._quant_scheme = v1._quant_scheme                          # pylint: disable=protected-access
+        self._percentile_value = 100
+        self.model = v1.model
         first_param = next(self.model.parameters(), None)
-        self._device = first_param.device if first_param is not None else torch.device("cuda")
-        self._convert(self.model, default_output_bw, default_param_bw, per_channel_quantization)
-        first = next((m for m in self.model.modules() if isinstance(m, BaseQuantizationMixin)), None)
-        if first is not None:
-            first.input_quantizers[0] = self._make((), default_output_bw, False, first)
+        self._device = first_param.device if first_param is not None else torch.device("cuda",
+                                                                                       torch.cuda.current_device())
+        self._realize(self.model)
 
-    def _make(self, shape, bitwidth, symmetric, like: nn.Module):
-        q = QuantizeDequantize(shape, bitwidth=bitwidth, symmetric=symmetric,
-                               encoding_analyzer=_analyzer(self._quant_scheme, shape))
-        param = next(like.parameters(), None)
-        return q.to(param.device if param is not None else self._device)
-
-    def _convert(self, module: nn.Module, output_bw: int, param_bw: int, per_channel: bool):
+    # ------------------------------------------------------------------------------------------------ construction
+    def _realize(self, module: nn.Module):
         for name, child in list(module.named_children()):
-            if type(child) in QuantizationMixin.cls_to_qcls and not list(child.children()):
-                q = QuantizationMixin.from_module(child)
-                for pname, param in child.named_parameters(recurse=False):
-                    if pname != 'weight':
-                        continue            # biases are not quantized by default
-                    shape = ()
-                    if per_channel and param.dim() > 1:
-                        axis = 1 if isinstance(child, (nn.ConvTranspose1d, nn.ConvTranspose2d,
-                                                       nn.ConvTranspose3d)) else 0
-                        shape = tuple(d if a == axis else 1 for a, d in enumerate(param.shape))
-                    q.param_quantizers[pname] = self._make(shape, param_bw, True, child)
-                if not isinstance(child, (nn.Flatten, nn.Dropout)):
-                    q.output_quantizers[0] = self._make((), output_bw, False, child)
-                setattr(module, name, q)
+            if isinstance(child, StaticGridQuantWrapper):
+                setattr(module, name, self._realize_wrapper(child))
             else:
-                self._convert(child, output_bw, param_bw, per_channel)
+                self._realize(child)
 
+    def _realize_wrapper(self, wrapper: StaticGridQuantWrapper) -> nn.Module:
+        original = wrapper._module_to_wrap                             # pylint: disable=protected-access
+        if type(original) not in QuantizationMixin.cls_to_qcls:
+            QuantizationMixin.wrap(type(original))
+        quantized = QuantizationMixin.from_module(original)
+        param = next(original.parameters(), None)
+        device = param.device if param is not None else self._device
+        quantized.input_quantizers = nn.ModuleList([self._realize_quantizer(q, (), device)
+                                                    for q in wrapper.input_quantizers])
+        quantized.output_quantizers = nn.ModuleList([self._realize_quantizer(q, (), device)
+                                                     for q in wrapper.output_quantizers])
+        for pname, q in wrapper.param_quantizers.items():
+            shape = ()
+            if isinstance(q, StaticGridPerChannelQuantizer):
+                p = getattr(original, pname)
+                axis = q._ch_axis                                      # pylint: disable=protected-access
+                shape = tuple(d if a == axis else 1 for a, d in enumerate(p.shape))
+            quantized.param_quantizers[pname] = self._realize_quantizer(q, shape, device)
+        return quantized
+
+    def _realize_quantizer(self, q, shape, device):
+        if not q.enabled or q.bitwidth == 32:
+            return None
+        if q.use_symmetric_encodings and (q.use_strict_symmetric or q.use_unsigned_symmetric):
+            raise NotImplementedError("strict-symmetric and unsigned-symmetric grids are not available in the v2 "
+                                      "simulation (the reference's builder asserts the same)")
+        if q.data_type != QuantizationDataType.int:
+            raise NotImplementedError("only integer grids are implemented")
+        quantizer = QuantizeDequantize(shape, q.bitwidth, q.use_symmetric_encodings,
+                                       _analyzer(self._quant_scheme, shape)).to(device)
+        if self._quant_scheme not in _RANGE_LEARNING:
+            for param in quantizer.parameters():
+                param.requires_grad = False                            # builder.py:187-202
+        return quantizer
+
+    # --------------------------------------------------------------------------------------------------- usage
     def qmodules(self):
         for name, module in self.model.named_modules():
             if isinstance(module, BaseQuantizationMixin):
                 yield name, module
 
+    named_qmodules = qmodules
+
+    def set_percentile_value(self, percentile_value: float):
+        """Percentile of every percentile analyzer (reference v2 quantsim.py:270-278)."""
+        if percentile_value < 90 or percentile_value > 100:
+            raise ValueError("Percentile value must be in range [90, 100]")
+        self._percentile_value = percentile_value
+        for _, module in self.qmodules():
+            for quantizer in list(module.input_quantizers) + list(module.output_quantizers) + \
+                    list(module.param_quantizers.values()):
+                analyzer = getattr(quantizer, 'encoding_analyzer', None)
+                if isinstance(analyzer, PercentileEncodingAnalyzer):
+                    analyzer.set_percentile(percentile_value)
+
     def compute_encodings(self, forward_pass_callback, forward_pass_callback_args):
-        """Runs the callback with every quantizer observing, then fixes the encodings."""
-        import contextlib
+        """Runs the callback with every quantizer observing, then fixes the encodings (v2 quantsim.py:205-224)."""
         with contextlib.ExitStack() as stack:
             for _, module in self.qmodules():
                 stack.enter_context(module.compute_encodings())
@@ -87,3 +149,29 @@ class QuantizationSimModel:
                     forward_pass_callback(self.model, forward_pass_callback_args)
             finally:
                 self.model.train(was_training)
+
+    def get_encodings_dict(self) -> dict:
+        """The exported dictionary, laid out as the v1 simulation's: parameters by '<module>.<parameter>', activations
+        by module with 'input' / 'output' entries per tensor index."""
+        param_encodings, activation_encodings = {}, {}
+        for name, module in self.qmodules():
+            for pname, quantizer in module.param_quantizers.items():
+                if quantizer is not None and quantizer.is_initialized():
+                    param_encodings[f"{name}.{pname}"] = quantizer.get_legacy_encodings()
+            entry = {}
+            for kind, quantizers in (("input", module.input_quantizers), ("output", module.output_quantizers)):
+                found = {str(i): q.get_legacy_encodings()[0] for i, q in enumerate(quantizers)
+                         if q is not None and q.is_initialized()}
+                if found:
+                    entry[kind] = found
+            if entry:
+                activation_encodings[name] = entry
+        return {"version": "0.6.1", "activation_encodings": activation_encodings, "param_encodings": param_encodings,
+                "excluded_layers": []}
+
+    def export_encodings(self, path: str, filename_prefix: str) -> str:
+        os.makedirs(path, exist_ok=True)
+        file = os.path.join(path, filename_prefix + '.encodings')
+        with open(file, 'w') as f:
+            json.dump(self.get_encodings_dict(), f, sort_keys=True, indent=4)
+        return file

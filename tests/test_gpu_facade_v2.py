@@ -8,6 +8,7 @@ w.r.t. input / scale / offset (min / max), dynamic quantization inside compute_e
 import numpy as np
 import pytest
 import torch
+from torch import nn
 
 pytestmark = pytest.mark.gpu
 
@@ -136,3 +137,154 @@ def test_per_channel_module(v2, oracle):
     assert np.array_equal(y.detach().cpu().numpy().reshape(-1), want)
     # every row uses its own grid
     assert torch.unique(scale).numel() == 12
+
+
+# ------------------------------------------------------------------------------------------ v2 simulation model
+class _ResBlockNet(nn.Module):
+    """conv-relu, a residual block with a functional-free Add module, pooling, flatten, linear."""
+
+    def __init__(self):
+        super().__init__()
+        from aimet_amd.v1.nn.modules.custom import Add
+        self.conv1, self.relu1 = nn.Conv2d(3, 8, 3, padding=1), nn.ReLU()
+        self.conv2, self.bn2, self.relu2 = nn.Conv2d(8, 8, 3, padding=1, bias=False), nn.BatchNorm2d(8), nn.ReLU()
+        self.conv3 = nn.Conv2d(8, 8, 3, padding=1)
+        self.add, self.relu3 = Add(), nn.ReLU()
+        self.pool, self.flatten, self.drop = nn.AdaptiveAvgPool2d(2), nn.Flatten(), nn.Dropout(0.1)
+        self.fc = nn.Linear(32, 5)
+
+    def forward(self, x):
+        x = self.relu1(self.conv1(x))
+        y = self.relu2(self.bn2(self.conv2(x)))
+        y = self.conv3(y)
+        x = self.relu3(self.add(x, y))
+        return self.fc(self.drop(self.flatten(self.pool(x))))
+
+
+def _placement_v1(sim):
+    out = {}
+    for name, w in sim.quant_wrappers():
+        out[name] = ([q.enabled for q in w.input_quantizers], [q.enabled for q in w.output_quantizers],
+                     {p: q.enabled for p, q in w.param_quantizers.items()})
+    return out
+
+
+def _placement_v2(sim):
+    out = {}
+    for name, m in sim.qmodules():
+        out[name] = ([q is not None for q in m.input_quantizers], [q is not None for q in m.output_quantizers],
+                     {p: q is not None for p, q in m.param_quantizers.items()})
+    return out
+
+
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_v2_sim_follows_the_configuration(tmp_path, per_channel):
+    """The v2 simulation places and shapes its quantizers as the v1 configurator decides (defaults, params, op_type,
+    supergroups, model input / output), for the default configuration and for a configuration file; with min-max
+    calibration both simulations then describe the same grids and give the same outputs."""
+    import json
+    from aimet_amd.v1.quantsim import QuantizationSimModel as V1Sim, DEFAULT_CONFIG
+    from aimet_amd.v2.quantsim import QuantizationSimModel as V2Sim
+    from aimet_amd.v2.quantization.affine import QuantizeDequantize
+    torch.manual_seed(5)
+    model = _ResBlockNet().eval().cuda()
+    dummy = torch.randn(2, 3, 8, 8).cuda()
+    cfg = json.loads(json.dumps(DEFAULT_CONFIG))
+    cfg["defaults"]["per_channel_quantization"] = str(per_channel)
+    cfg["model_output"] = {"is_output_quantized": "True"}
+    cfg["op_type"]["AveragePool"] = {"is_output_quantized": "False"}
+    path = str(tmp_path / "cfg.json")
+    with open(path, "w") as f:
+        json.dump(cfg, f)
+    v1 = V1Sim(model, dummy, quant_scheme='tf', default_output_bw=8, default_param_bw=4, config_file=path)
+    v2 = V2Sim(model, dummy, quant_scheme='tf', default_output_bw=8, default_param_bw=4, config_file=path)
+    place = _placement_v2(v2)
+    assert place == _placement_v1(v1)
+    # what the configuration means for this graph
+    assert place["conv1"] == ([True], [False], {"weight": True, "bias": False})        # model input; Conv+Relu
+    assert place["relu1"][1] == [True] and place["bn2"][2] == {"weight": False, "bias": False}
+    assert place["add"] == ([False, False], [False], {}) and place["relu3"][1] == [True]   # Add+Relu
+    assert place["flatten"][1] == [False] and place["drop"][1] == [False] and place["fc"][1] == [True]
+    qm = dict(v2.qmodules())
+    wq = qm["conv2"].param_quantizers["weight"]
+    assert isinstance(wq, QuantizeDequantize) and wq.bitwidth == 4 and wq.symmetric
+    assert tuple(wq.shape) == ((8, 1, 1, 1) if per_channel else ())
+    assert not any(p.requires_grad for p in wq.parameters())
+    oq = qm["relu1"].output_quantizers[0]
+    assert oq.bitwidth == 8 and not oq.symmetric and tuple(oq.shape) == ()
+
+    batches = [torch.randn(16, 3, 8, 8).cuda() for _ in range(3)]
+
+    def calibrate(m, _):
+        for b in batches:
+            m(b)
+    v1.compute_encodings(calibrate, None)
+    v2.compute_encodings(calibrate, None)
+    e1, e2 = v1.get_encodings_dict(), v2.get_encodings_dict()
+    assert set(e1["param_encodings"]) == set(e2["param_encodings"])
+    assert set(e1["activation_encodings"]) == set(e2["activation_encodings"])
+    # symmetric grids differ between the two generations by design (v1: absmax / floor(steps / 2); v2: the larger of
+    # max / floor(steps / 2) and -min / ceil(steps / 2)), so parameters -- and everything downstream of them -- agree
+    # only approximately; the model-input quantizer sees the same data and must agree exactly
+    for key, encs in e1["param_encodings"].items():
+        assert len(encs) == len(e2["param_encodings"][key])
+        for a, b in zip(encs, e2["param_encodings"][key]):
+            assert a["bitwidth"] == b["bitwidth"] == 4 and a["is_symmetric"] == b["is_symmetric"] == "True"
+            assert b["scale"] == pytest.approx(a["scale"], rel=0.15)
+    a, b = e1["activation_encodings"]["conv1"]["input"]["0"], e2["activation_encodings"]["conv1"]["input"]["0"]
+    assert b["scale"] == pytest.approx(a["scale"], rel=1e-6) and b["offset"] == a["offset"] and b["bitwidth"] == 8
+    for name, entry in e1["activation_encodings"].items():
+        for kind, encs in entry.items():
+            for idx, a in encs.items():
+                assert e2["activation_encodings"][name][kind][idx]["scale"] == pytest.approx(a["scale"], rel=0.2)
+    x = torch.randn(8, 3, 8, 8).cuda()
+    with torch.no_grad():
+        y0, y1, y2 = model(x), v1.model(x), v2.model(x)
+    cos = torch.nn.functional.cosine_similarity
+    assert cos(y1.flatten(), y2.flatten(), dim=0).item() > 0.97
+    assert cos(y0.flatten(), y2.flatten(), dim=0).item() > 0.9        # 4-bit weights: close to fp32, not equal
+    e = e2["activation_encodings"]["fc"]["output"]["0"]
+    steps = (y2.double() / e["scale"]).cpu().numpy()
+    assert np.abs(steps - np.round(steps)).max() < 1e-3             # the model output lies on its quantizer's grid
+    file = v2.export_encodings(str(tmp_path), "v2net")
+    with open(file) as f:
+        assert json.load(f)["param_encodings"].keys() == e2["param_encodings"].keys()
+
+
+def test_v2_sim_schemes_and_refusals():
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.quantsim import DEFAULT_CONFIG
+    from aimet_amd.v2.quantsim import QuantizationSimModel as V2Sim
+    from aimet_amd.v2.quantization.encoding_analyzer import (MinMaxEncodingAnalyzer, PercentileEncodingAnalyzer,
+                                                             SqnrEncodingAnalyzer)
+    import json
+    torch.manual_seed(6)
+    model = _ResBlockNet().eval().cuda()
+    dummy = torch.randn(2, 3, 8, 8).cuda()
+    for scheme, analyzer, trainable in ((QuantScheme.post_training_tf, MinMaxEncodingAnalyzer, False),
+                                        (QuantScheme.post_training_tf_enhanced, SqnrEncodingAnalyzer, False),
+                                        (QuantScheme.post_training_percentile, PercentileEncodingAnalyzer, False),
+                                        (QuantScheme.training_range_learning_with_tf_init, MinMaxEncodingAnalyzer,
+                                         True)):
+        sim = V2Sim(model, dummy, quant_scheme=scheme)
+        q = dict(sim.qmodules())["relu1"].output_quantizers[0]
+        assert isinstance(q.encoding_analyzer, analyzer)
+        assert all(p.requires_grad == trainable for p in q.parameters())
+        if scheme == QuantScheme.post_training_percentile:
+            sim.set_percentile_value(99.0)
+            assert q.encoding_analyzer.percentile == 99.0
+            with pytest.raises(ValueError):
+                sim.set_percentile_value(50.0)
+        sim.compute_encodings(lambda m, _: m(torch.randn(16, 3, 8, 8).cuda()), None)
+        with torch.no_grad():
+            y = sim.model(dummy)
+        assert torch.isfinite(y).all()
+        if trainable:
+            sim.model(dummy).sum().backward()
+            assert q.min.grad is not None and q.max.grad is not None
+    cfg = json.loads(json.dumps(DEFAULT_CONFIG))
+    cfg["defaults"]["strict_symmetric"] = "True"
+    with pytest.raises(NotImplementedError):
+        V2Sim(model, dummy, config_file=cfg)
+    with pytest.raises(ValueError):
+        V2Sim(model, None)
