@@ -12,6 +12,8 @@
 //       ModelOptimizations/DlQuantization/src/trim_functions.cpp:141-182, 698-709
 //   v2  (aimet_torch.v2): r = rint(x / scale) - offset; y = (clamp(r, qmin, qmax) + offset) * scale
 //       TrainingExtensions/torch/src/python/aimet_torch/v2/quantization/affine/backends/torch_builtins.py:303-344
+#include <hip/hip_fp16.h>
+
 #include "miq_common.h"
 #include "miq_fastmath.h"
 #include "miq_io.h"
@@ -100,6 +102,29 @@ struct OpV1Quantize : OpV1
         float q = quant<FAST>(p, x);
         code    = 0;
         return q - s.shift;
+    }
+};
+
+// y = float(half(x)): the simulation of a float16 tensor (TORCH/v1/tensor_quantizer.py:1104-1107, tensor.half().float()),
+// round to nearest even, overflow to infinity, as the conversion instruction does
+struct OpFp16
+{
+    using P                  = int;   // no parameters
+    static constexpr int NIN = 1;
+    using Code               = uint8_t;
+    __device__ static P load(const ParamSrc&, uint32_t)
+    {
+        return 0;
+    }
+    __device__ static bool fast_ok(const P&, const float*, int)
+    {
+        return true;
+    }
+    template <bool FAST>
+    __device__ static float apply(const ParamSrc&, const P&, float x, float, int& code)
+    {
+        code = 0;
+        return __half2float(__float2half_rn(x));
     }
 };
 
@@ -196,6 +221,11 @@ template <>
 __device__ V1P scalar_params<OpV1Quantize>(const ParamSrc& s)
 {
     return V1P{s.scalar.x, s.scalar.y, s.scalar.z, s.scalar.w, s.scalar_rcp};
+}
+template <>
+__device__ int scalar_params<OpFp16>(const ParamSrc&)
+{
+    return 0;
 }
 template <>
 __device__ float2 scalar_params<OpV1Ste>(const ParamSrc& s)
@@ -603,6 +633,13 @@ int miq_qdq_per_tensor_bf16(const uint16_t* in, uint16_t* out, int64_t n, double
         return stochastic_qdq_per_tensor<uint16_t>(in, out, n, e, (hipStream_t) stream);
     EwPtrs<uint16_t, uint8_t> p{in, nullptr, out, nullptr};
     return launch_ew<uint16_t, OpV1Qdq, false>(p, per_tensor_src(e), n, 1, 1, (hipStream_t) stream);
+}
+
+int miq_fp16_round_trip_f32(const float* in, float* out, int64_t n, void* stream)
+{
+    MIQ_CHECK_ARG(n >= 0 && (n == 0 || (in && out)), "null tensor pointer or negative count");
+    EwPtrs<float, uint8_t> p{in, nullptr, out, nullptr};
+    return launch_ew<float, OpFp16, false>(p, ParamSrc{}, n, 1, 1, (hipStream_t) stream);
 }
 
 int miq_quantize_per_tensor_f32(const float* in, float* out, int64_t n, double enc_min, double enc_max, int bw,

@@ -96,6 +96,18 @@ def qdq_per_tensor(x, enc_min, enc_max, bw, rounding_mode=_lib.ROUND_NEAREST, ou
     return out
 
 
+def fp16_round_trip(x, out=None):
+    """float(half(x)) in one pass over a float32 tensor: the float16 data type of the simulation."""
+    _require_gpu(x, out)
+    if x.dtype != _F32:
+        raise RuntimeError("fp16_round_trip takes float32 tensors")
+    x = x.contiguous()
+    out = torch.empty_like(x) if out is None else out
+    with torch.cuda.device(x.device):
+        check(lib.miq_fp16_round_trip_f32(_ptr(x), _ptr(out), x.numel(), _stream(x)))
+    return out
+
+
 def quantize_per_tensor(x, enc_min, enc_max, bw, shift_to_signed, rounding_mode=_lib.ROUND_NEAREST):
     """Float-valued grid indices (minus 2^(bw-1) when shift_to_signed)."""
     _require_gpu(x)

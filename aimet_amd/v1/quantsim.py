@@ -83,11 +83,16 @@ _INIT_SCHEME = {
 }
 
 
+_FLOAT16_ENTRY = object()     # marks a float16 quantizer in the export: it has no encoding, only a type
+
+
 def _exported_encoding(quantizer):
     """The encoding a quantizer is exported with: learned-grid quantizers report the one their quant scheme means
     (reference get_encoding_by_quantizer, qc_quantize_op.py:1507-1519)."""
     if not quantizer.enabled:
         return None
+    if quantizer.data_type == QuantizationDataType.float:
+        return _FLOAT16_ENTRY if quantizer.bitwidth != 32 else None      # reference quantsim.py:2320
     if isinstance(quantizer, LearnedGridTensorQuantizer):
         return quantizer.get_effective_encoding()
     return quantizer.encoding
@@ -113,8 +118,14 @@ class QuantizationSimModel:
             raise ValueError('Parameter round mode can only be nearest or stochastic')
         if default_param_bw < 4 or default_param_bw > 32 or default_output_bw < 4 or default_output_bw > 32:
             raise ValueError('Default bitwidth for parameters and activations must be between 4 and 32')
-        if default_data_type != QuantizationDataType.int:
-            raise ValueError('only QuantizationDataType.int is implemented')
+        if default_data_type == QuantizationDataType.float and (default_output_bw != 16 or default_param_bw != 16):
+            # the reference also takes 8 (an 8-bit float grid, aimet_torch/fp_quantization.py); not built here
+            raise ValueError('float data_type can only be used when default_output_bw and default_param_bw are 16')
+        if default_data_type == QuantizationDataType.float and quant_scheme not in (
+                QuantScheme.post_training_tf, QuantScheme.post_training_tf_enhanced,
+                QuantScheme.post_training_percentile):
+            raise NotImplementedError('range learning on float16 quantizers is not implemented')
+        self._default_data_type = default_data_type
         self.model = model if in_place else copy.deepcopy(model)
         self._quant_scheme = quant_scheme
         self._percentile_value = 100                 # default of the reference (:278)
@@ -199,7 +210,8 @@ class QuantizationSimModel:
             # swapped for learned-grid wrappers once encodings have been computed
             wrapper = StaticGridQuantWrapper(rec["module"], self._default_param_bw, self._default_output_bw,
                                              self._rounding_mode, _INIT_SCHEME[self._quant_scheme],
-                                             num_inputs=rec["num_inputs"], num_outputs=rec["num_outputs"])
+                                             num_inputs=rec["num_inputs"], num_outputs=rec["num_outputs"],
+                                             data_type=self._default_data_type)
             rec["wrapper"] = wrapper
             parent = self.model
             *path, leaf = rec["name"].split('.')
@@ -386,21 +398,27 @@ class QuantizationSimModel:
         for name, w in self.quant_wrappers():
             for pname, q in w.param_quantizers.items():
                 encoding = _exported_encoding(q)
-                if encoding is not None:
+                if encoding is _FLOAT16_ENTRY:
+                    param_enc[f"{name}.{pname}"] = [{'bitwidth': q.bitwidth, 'dtype': 'float'}]
+                elif encoding is not None:
                     encs = encoding if isinstance(encoding, list) else [encoding]
                     param_enc[f"{name}.{pname}"] = [self._encoding_dict(e, q.use_symmetric_encodings) for e in encs]
             entry = {}
             for kind, qs in (('input', w.input_quantizers), ('output', w.output_quantizers)):
                 for i, q in enumerate(qs):
                     encoding = _exported_encoding(q)
-                    if encoding is not None:
+                    if encoding is _FLOAT16_ENTRY:
+                        entry.setdefault(kind, {})[str(i)] = {'bitwidth': q.bitwidth, 'dtype': 'float'}
+                    elif encoding is not None:
                         entry.setdefault(kind, {})[str(i)] = self._encoding_dict(encoding,
                                                                                  q.use_symmetric_encodings)
             if entry:
                 act_enc[name] = entry
         return {'version': '0.6.1', 'activation_encodings': act_enc, 'param_encodings': param_enc,
                 'quantizer_args': {'activation_bitwidth': self._default_output_bw,
-                                   'param_bitwidth': self._default_param_bw, 'dtype': 'int',
+                                   'param_bitwidth': self._default_param_bw,
+                                   'dtype': 'float' if self._default_data_type == QuantizationDataType.float
+                                   else 'int',
                                    'quant_scheme': self._quant_scheme.name}}
 
     def export_encodings(self, path: str, filename_prefix: str) -> str:

@@ -70,8 +70,9 @@ class StaticGridTensorQuantizer(TensorQuantizer):
 
     def __init__(self, bitwidth, round_mode, quant_scheme, use_symmetric_encodings, enabled_by_default,
                  data_type=QuantizationDataType.int):
-        if data_type != QuantizationDataType.int:
-            raise ValueError("only QuantizationDataType.int is implemented for the static-grid quantizers")
+        if data_type == QuantizationDataType.float and bitwidth not in (16, 32):
+            # the reference also has an 8-bit float grid (aimet_torch/fp_quantization.py); not built here
+            raise NotImplementedError("the float data type is implemented for bitwidth 16 (float16) only")
         super().__init__(bitwidth, round_mode, quant_scheme, use_symmetric_encodings, enabled_by_default, data_type)
         self._cppOp = None
         self._encoding = None
@@ -147,8 +148,8 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         if self.enabled and not self._is_encoding_frozen:
             self._encoding = []
             self._dev_params = None
-            if self.bitwidth == 32:
-                self._encoding = None
+            if self.bitwidth == 32 or self.data_type == QuantizationDataType.float:
+                self._encoding = None                   # float16 has no encoding (reference :286-290)
                 return
             for encoding, valid in self._compute_op_encodings():
                 if not valid:
@@ -215,7 +216,7 @@ class StaticGridPerTensorQuantizer(StaticGridTensorQuantizer):
 
     def update_encoding_stats(self, tensor: torch.Tensor):
         if self.enabled and not self._is_encoding_frozen:
-            if self.bitwidth == 32:
+            if self.bitwidth == 32 or self.data_type == QuantizationDataType.float:
                 return
             self._cppOp[0].updateStats(self._stats_tensor(tensor), tensor.is_cuda)
 
@@ -242,7 +243,7 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
 
     def update_encoding_stats(self, tensor: torch.Tensor):
         if self.enabled and not self._is_encoding_frozen:
-            if self.bitwidth == 32:
+            if self.bitwidth == 32 or self.data_type == QuantizationDataType.float:
                 return
             if self.encoding_min_max_fixed_vals is not None:
                 fixed = self._stats_tensor(tensor)
@@ -320,9 +321,20 @@ class QuantizeDequantize(torch.autograd.Function):
         return out.to(dtype)
 
     @staticmethod
+    def _quantize_float(tensor, tensor_quantizer):
+        """float16 simulation: tensor.half().float() (reference :1104-1113), one fused pass for float32 tensors."""
+        if tensor_quantizer.bitwidth != 16:
+            raise ValueError('float data_type only supports bitwidth 16 here')
+        if tensor.dtype == torch.float32 and tensor.is_cuda:
+            return ops.fp16_round_trip(tensor)
+        return tensor.half().float()
+
+    @staticmethod
     def forward(ctx, tensor, tensor_quantizer, round_mode):  # pylint: disable=arguments-differ
         if tensor_quantizer.enabled and tensor_quantizer.bitwidth != 32:
-            if isinstance(tensor_quantizer, StaticGridPerChannelQuantizer):
+            if tensor_quantizer.data_type == QuantizationDataType.float:
+                quantized = QuantizeDequantize._quantize_float(tensor, tensor_quantizer)
+            elif isinstance(tensor_quantizer, StaticGridPerChannelQuantizer):
                 quantized = QuantizeDequantize._per_channel_quantize_dequantize(tensor, tensor_quantizer, round_mode)
             else:
                 dtype = tensor.dtype

@@ -90,6 +90,10 @@ int miq_qdq_per_tensor_f32(const float* in, float* out, int64_t n, double enc_mi
 int miq_qdq_per_tensor_bf16(const uint16_t* in, uint16_t* out, int64_t n, double enc_min, double enc_max, int bw,
                             int rounding_mode, void* stream);
 
+/* out = float(half(in)): quantize-dequantize of the float16 data type (QuantizationDataType.float, bitwidth 16), which
+ * the reference forms as tensor.half().float() (TORCH/v1/tensor_quantizer.py:1104-1107), in one pass. */
+int miq_fp16_round_trip_f32(const float* in, float* out, int64_t n, void* stream);
+
 /* ITensorQuantizationSim<float>::quantizeTensor(..., shiftToSigned) (ITensorQuantizationSim.h:57-59,
  * DLQ/src/TensorQuantizationSim.cpp:116-126; kernel DLQ/src/trim_functions.cu:62-76): float-valued grid indices. */
 int miq_quantize_per_tensor_f32(const float* in, float* out, int64_t n, double enc_min, double enc_max, int bw,

@@ -312,3 +312,72 @@ def test_relu_absorbed_by_output_quantizer(api, monkeypatch):
     with torch.no_grad():
         sim.model(x)
     assert calls == ["relu1", "relu2"]
+
+
+def test_float16_data_type(api, tmp_path):
+    """QuantizationDataType.float with bitwidth 16: quantize-dequantize is tensor.half().float() (reference
+    tensor_quantizer.py:1104-1107), there are no statistics and no encoding, the gradient passes through, and the
+    export names only the type.  Values, special ones included, must equal torch's own conversion bit for bit."""
+    from aimet_amd.common.defs import QuantizationDataType
+    from aimet_amd import ops
+    x = torch.randn(100_003, device="cuda") * 100
+    x[:12] = torch.tensor([0.0, -0.0, 65504.0, 65519.9, 65520.0, -70000.0, 1e-8, 5.96e-8, 2.98e-8, 6.1e-5,
+                           float("inf"), float("nan")], device="cuda")
+    want = x.half().float()
+    got = ops.fp16_round_trip(x)
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    got = ops.fp16_round_trip(x[1:])                      # 4-byte aligned only: the element-wise kernel
+    assert torch.equal(got.view(torch.int32), want[1:].view(torch.int32))
+
+    q = api.tq.StaticGridPerTensorQuantizer(16, api.nearest, api.QuantScheme.post_training_tf_enhanced, False,
+                                            enabled_by_default=True, data_type=QuantizationDataType.float)
+    q.update_encoding_stats(x)
+    q.compute_encoding()
+    assert q.encoding is None and q.enabled
+    xr = x[12:].clone().requires_grad_(True)
+    y = q.quantize_dequantize(xr, api.nearest)
+    assert torch.equal(y.detach(), want[12:])
+    y.backward(torch.full_like(y, 2.0))
+    assert torch.equal(xr.grad, torch.full_like(xr, 2.0))
+    xb = x[12:1000].bfloat16()
+    assert torch.equal(q.quantize_dequantize(xb, api.nearest), xb.half().float())
+    with pytest.raises(NotImplementedError):
+        api.tq.StaticGridPerTensorQuantizer(8, api.nearest, api.QuantScheme.post_training_tf, False, True,
+                                            data_type=QuantizationDataType.float)
+
+    # a wrapper: parameters and output pass through float16
+    torch.manual_seed(2)
+    lin = nn.Linear(32, 16).cuda()
+    w = api.qc.StaticGridQuantWrapper(lin, 16, 16, 'nearest', api.QuantScheme.post_training_tf,
+                                      data_type=QuantizationDataType.float)
+    inp = torch.randn(8, 32, device="cuda")
+    w.set_mode(api.qc.QcQuantizeOpMode.ANALYSIS)
+    w(inp)
+    w.compute_encoding()
+    w.set_mode(api.qc.QcQuantizeOpMode.ACTIVE)
+    with torch.no_grad():
+        out = w(inp)
+    ref = torch.nn.functional.linear(inp, lin.weight.half().float(), lin.bias.half().float()).half().float()
+    assert torch.equal(out, ref)
+    assert torch.equal(w._module_to_wrap.weight, lin.weight)
+
+    # the simulation model
+    model = _Net().eval().cuda()
+    dummy = torch.randn(2, 3, 6, 6).cuda()
+    with pytest.raises(ValueError):
+        api.quantsim.QuantizationSimModel(model, dummy_input=dummy, default_data_type=QuantizationDataType.float)
+    sim = api.quantsim.QuantizationSimModel(model, dummy_input=dummy, quant_scheme='tf', default_output_bw=16,
+                                            default_param_bw=16, default_data_type=QuantizationDataType.float)
+    sim.compute_encodings(_calibrate, [torch.randn(4, 3, 6, 6).cuda()])
+    with torch.no_grad():
+        y = sim.model(dummy)
+        h = torch.relu(torch.nn.functional.conv2d(dummy.half().float(), model.conv1.weight.half().float(),
+                                                  model.conv1.bias, padding=1)).half().float()
+        h = torch.nn.functional.conv2d(h, model.conv2.weight.half().float(), padding=1).half().float()
+        h = model.bn(h).half().float()
+        want_y = torch.nn.functional.linear(h.flatten(1), model.fc.weight.half().float(), model.fc.bias).half().float()
+    assert torch.allclose(y, want_y, rtol=1e-3, atol=1e-3)      # same casts; convolution algorithms may differ
+    data = sim.get_encodings_dict()
+    assert data["param_encodings"]["conv2.weight"] == [{"bitwidth": 16, "dtype": "float"}]
+    assert data["activation_encodings"]["relu1"]["output"]["0"] == {"bitwidth": 16, "dtype": "float"}
+    assert data["quantizer_args"]["dtype"] == "float"
