@@ -25,6 +25,7 @@ namespace
 {
 constexpr int kMaxBins    = 4096;
 constexpr int kHistBlock  = 256;
+constexpr int kMaxReplicas = 32;   // global copies of a histogram's counts that the workgroups of one update add into
 constexpr float kMinScale = 1.1920928955078125e-07f;   // torch.finfo(torch.float32).eps (EA:322)
 
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -37,7 +38,7 @@ __global__ __launch_bounds__(kHistBlock) void finite_minmax_kernel(const float* 
                                                                    int vec)
 {
     const int h = blockIdx.y;
-    // this launch also clears the count sums that the later kernels of the same update accumulate into
+    // this launch also clears the count replicas that the binning kernel of the same update accumulates into
     for (int i = blockIdx.x * kHistBlock + threadIdx.x; i < sums_per_hist; i += gridDim.x * kHistBlock)
         sums[(int64_t) h * sums_per_hist + i] = 0;
     const float* row = x + (int64_t) h * n_per_hist;
@@ -206,22 +207,39 @@ struct Binner
 
 // grid (blocks, H).  Each workgroup first derives the binning ranges of histogram h from the (min, max) partials of the
 // previous launch (every workgroup repeats this small reduction: cheaper than a launch of its own), then bins its
-// share of row h into LDS -- the batch's own range and / or the merged range, in one pass over the data -- and stores
-// its counts to its own slice of `partial` (plain stores: no atomics on global memory).
+// share of row h into LDS -- the batch's own range and / or the merged range, in one pass over the data -- and adds
+// its non-zero counts to one of `replicas` global copies (workgroup b -> copy b % replicas, so at most
+// blocks / replicas atomics ever meet on one address; same-address device atomics cost about 15 ns each here).
 // LDS: [kinds][num_bins][copies] uint32, copy = lane % copies (lanes of a wavefront that hit the same bin spread out).
-// partial layout: [h][block][kinds][num_bins] uint32
+// global layout: [h][replica][kinds][num_bins] uint32, cleared by the min/max kernel of the same update
 __global__ __launch_bounds__(kHistBlock) void hist_kernel(const float* __restrict__ x, int64_t n_per_hist, int num_bins,
                                                           int has_stats, int count_batch, int count_merged,
                                                           int copies, const float* __restrict__ mm_partial,
                                                           const float* __restrict__ state_minmax,
                                                           Ranges* __restrict__ ranges, float* __restrict__ batch_minmax,
                                                           int* __restrict__ bad_flag, uint32_t* __restrict__ partial,
-                                                          int vec)
+                                                          int replicas, int vec)
 {
     extern __shared__ uint32_t lds[];
     __shared__ float s_mm[2][kHistBlock / 64];
     const int h = blockIdx.y;
     const int kinds = count_batch + count_merged;
+    // the first tile's loads go out before anything else: they are in flight while the ranges are derived
+    const float* row     = x + (int64_t) h * n_per_hist;
+    const v4f* rv        = reinterpret_cast<const v4f*>(row);
+    const int64_t nvec   = n_per_hist / 4;
+    const int64_t stride = (int64_t) gridDim.x * kHistBlock * 2;
+    int64_t base         = (int64_t) blockIdx.x * kHistBlock * 2;
+    v4f a[2];
+    if (vec)
+    {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+        {
+            const int64_t i = base + u * kHistBlock + threadIdx.x;
+            a[u]            = i < nvec ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
+        }
+    }
     for (int i = threadIdx.x; i < kinds * num_bins * copies; i += kHistBlock)
         lds[i] = 0;
     float lo = INFINITY, hi = -INFINITY;
@@ -266,7 +284,6 @@ __global__ __launch_bounds__(kHistBlock) void hist_kernel(const float* __restric
     const int copy = threadIdx.x & (copies - 1);
     uint32_t* lb   = lds + copy;                                        // batch-range counts
     uint32_t* lm   = lds + (count_batch ? num_bins * copies : 0) + copy;   // merged-range counts
-    const float* row = x + (int64_t) h * n_per_hist;
     auto count = [&](float v) {
         if (v != v)
             return;
@@ -277,18 +294,8 @@ __global__ __launch_bounds__(kHistBlock) void hist_kernel(const float* __restric
     };
     if (vec)
     {
-        const v4f* rv        = reinterpret_cast<const v4f*>(row);
-        const int64_t nvec   = n_per_hist / 4;
-        const int64_t stride = (int64_t) gridDim.x * kHistBlock * 2;
-        for (int64_t base = (int64_t) blockIdx.x * kHistBlock * 2; base < nvec; base += stride)
+        while (base < nvec)
         {
-            v4f a[2];
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-            {
-                const int64_t i = base + u * kHistBlock + threadIdx.x;
-                a[u]            = i < nvec ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
-            }
 #pragma unroll
             for (int u = 0; u < 2; ++u)
             {
@@ -296,6 +303,15 @@ __global__ __launch_bounds__(kHistBlock) void hist_kernel(const float* __restric
                 count(a[u][1]);
                 count(a[u][2]);
                 count(a[u][3]);
+            }
+            base += stride;
+            if (base >= nvec)
+                break;
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+            {
+                const int64_t i = base + u * kHistBlock + threadIdx.x;
+                a[u]            = i < nvec ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
             }
         }
     }
@@ -306,51 +322,22 @@ __global__ __launch_bounds__(kHistBlock) void hist_kernel(const float* __restric
             count(row[i]);
     }
     __syncthreads();
-    uint32_t* dst = partial + ((int64_t) h * gridDim.x + blockIdx.x) * kinds * num_bins;
+    uint32_t* dst = partial + ((int64_t) h * replicas + blockIdx.x % replicas) * kinds * num_bins;
     for (int i = threadIdx.x; i < kinds * num_bins; i += kHistBlock)
     {
         uint32_t sum = 0;
         for (int c = 0; c < copies; ++c)
             sum += lds[i * copies + c];
-        dst[i] = sum;
+        if (sum)
+            atomicAdd(&dst[i], sum);
     }
 }
 
-// grid (ceil(width / 256), slices, H), width = kinds * bins: adds a slice of the workgroups' counts into sums[h][width]
-__global__ __launch_bounds__(kHistBlock) void reduce_counts_kernel(const uint32_t* __restrict__ partial, int blocks,
-                                                                   int width, uint32_t* __restrict__ sums)
-{
-    const int i = blockIdx.x * kHistBlock + threadIdx.x;
-    const int h = blockIdx.z;
-    if (i >= width)
-        return;
-    const int per   = (blocks + gridDim.y - 1) / gridDim.y;
-    const int b0    = blockIdx.y * per;
-    const int b1    = min(blocks, b0 + per);
-    const uint32_t* p = partial + (int64_t) h * blocks * width + i;
-    // independent loads, eight in flight per lane
-    uint32_t acc = 0;
-    int b        = b0;
-    for (; b + 8 <= b1; b += 8)
-    {
-        uint32_t t[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-            t[u] = p[(int64_t) (b + u) * width];
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-            acc += t[u];
-    }
-    for (; b < b1; ++b)
-        acc += p[(int64_t) b * width];
-    if (acc)
-        atomicAdd(&sums[(int64_t) h * width + i], acc);
-}
-
-// grid H, 256 threads: writes the batch histogram, re-bins the running histogram when the
+// grid (H, ceil(bins / 256)), 256 threads: writes the batch histogram, re-bins the running histogram when the
 // range grew (merge_stats, EA:222-251) and adds the batch's counts over the merged range.
-__global__ __launch_bounds__(kHistBlock) void merge_kernel(const uint32_t* __restrict__ sums, int num_bins,
-                                                           int has_stats, int count_batch, int count_merged,
+__global__ __launch_bounds__(kHistBlock) void merge_kernel(const uint32_t* __restrict__ sums, int replicas,
+                                                           int num_bins, int has_stats, int count_batch,
+                                                           int count_merged,
                                                            const Ranges* __restrict__ ranges,
                                                            float* __restrict__ state_hist,
                                                            float* __restrict__ state_minmax,
@@ -359,15 +346,38 @@ __global__ __launch_bounds__(kHistBlock) void merge_kernel(const uint32_t* __res
     __shared__ float upd[kMaxBins];
     const int h    = blockIdx.x;
     const Ranges r = ranges[h];
+    // gridDim.y workgroups share a histogram's bins when the running histogram keeps its range (the usual case: every
+    // bin is then updated on its own).  Re-binning scatters every old bin into the new range, so one workgroup does
+    // all of it and the others leave.
+    const bool rebinning = has_stats && r.rebin;
+    if (rebinning && blockIdx.y != 0)
+        return;
+    const int slice   = rebinning ? num_bins : (num_bins + (int) gridDim.y - 1) / (int) gridDim.y;
+    const int bin_lo  = rebinning ? 0 : (int) blockIdx.y * slice;
+    const int bin_hi  = min(num_bins, bin_lo + slice);
     float* sh      = state_hist + (int64_t) h * num_bins;
     float* bh      = batch_hist ? batch_hist + (int64_t) h * num_bins : nullptr;
-    const uint32_t* p  = sums + (int64_t) h * (count_batch + count_merged) * num_bins;
-    const uint32_t* pm = p + (count_batch ? num_bins : 0);
-    for (int i = threadIdx.x; i < num_bins; i += kHistBlock)
-        upd[i] = 0.f;
-    __syncthreads();
-    if (has_stats && r.rebin)
+    const int width      = (count_batch + count_merged) * num_bins;
+    const uint32_t* rep  = sums + (int64_t) h * replicas * width;
+    const int merged_off = count_batch ? num_bins : 0;
+    // counts of bin i over all replicas (integers: the order of the additions does not matter)
+    // (all loads of a bin are issued before the first addition: one round trip per bin, not one per replica)
+    auto total = [&](int i) {
+        uint32_t t[kMaxReplicas];
+#pragma unroll
+        for (int r = 0; r < kMaxReplicas; ++r)
+            t[r] = r < replicas ? rep[(int64_t) r * width + i] : 0u;
+        uint32_t sum = 0;
+#pragma unroll
+        for (int r = 0; r < kMaxReplicas; ++r)
+            sum += t[r];
+        return sum;
+    };
+    if (rebinning)
     {
+        for (int i = threadIdx.x; i < num_bins; i += kHistBlock)
+            upd[i] = 0.f;
+        __syncthreads();
         const float nbf            = (float) num_bins;
         const float dest_bin_width = (r.new_max - r.new_min) / nbf;
         const float src_bin_width  = (r.old_max - r.old_min) / nbf;
@@ -391,16 +401,20 @@ __global__ __launch_bounds__(kHistBlock) void merge_kernel(const uint32_t* __res
         }
         __syncthreads();
     }
-    for (int i = threadIdx.x; i < num_bins; i += kHistBlock)
+    for (int i = bin_lo + threadIdx.x; i < bin_hi; i += kHistBlock)
     {
-        if (count_batch && batch_hist)
-            bh[i] = (float) p[i];
-        if (!has_stats)
-            sh[i] = (float) p[i];
-        else if (count_merged)
-            sh[i] = (float) pm[i] + (r.rebin ? upd[i] : sh[i]);
+        if (count_batch && (batch_hist || !has_stats))
+        {
+            const float c = (float) total(i);
+            if (batch_hist)
+                bh[i] = c;
+            if (!has_stats)
+                sh[i] = c;
+        }
+        if (has_stats && count_merged)
+            sh[i] = (float) total(merged_off + i) + (r.rebin ? upd[i] : sh[i]);
     }
-    if (threadIdx.x == 0)
+    if (threadIdx.x == 0 && blockIdx.y == 0)
     {
         state_minmax[2 * h]     = r.new_min;
         state_minmax[2 * h + 1] = r.new_max;
@@ -562,8 +576,8 @@ __global__ __launch_bounds__(64) void sqnr_pick_kernel(const double* __restrict_
 int hist_blocks(int64_t num_hist, int64_t n_per_hist)
 {
     // enough workgroups to fill 256 CUs three times over, at least ~8K elements each
-    int64_t per_row = (n_per_hist + 8191) / 8192;
-    int64_t want    = (768 + num_hist - 1) / num_hist;
+    int64_t per_row = (n_per_hist + 6143) / 6144;
+    int64_t want    = (1024 + num_hist - 1) / num_hist;
     int64_t b       = per_row < want ? per_row : want;
     return (int) (b < 1 ? 1 : b);
 }
@@ -612,10 +626,11 @@ int64_t miq_v2_hist_workspace_bytes(int64_t num_hist, int64_t n_per_hist, int nu
 {
     if (num_hist <= 0 || n_per_hist <= 0 || num_bins <= 0)
         return 0;
-    const int64_t blocks = hist_blocks(num_hist, n_per_hist);
-    // per-workgroup counts + their sums + per-workgroup (min, max) + the per-histogram ranges
-    return num_hist * blocks * 2 * (int64_t) num_bins * 4 + num_hist * 2 * (int64_t) num_bins * 4 +
-           num_hist * blocks * 2 * 4 + num_hist * (int64_t) sizeof(Ranges) + 256;
+    const int64_t blocks   = hist_blocks(num_hist, n_per_hist);
+    const int64_t replicas = blocks < kMaxReplicas ? blocks : kMaxReplicas;
+    // count replicas (two kinds of histogram) + per-workgroup (min, max) + the per-histogram ranges
+    return num_hist * replicas * 2 * (int64_t) num_bins * 4 + num_hist * blocks * 2 * 4 +
+           num_hist * (int64_t) sizeof(Ranges) + 256;
 }
 
 int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hist, int num_bins, int has_stats,
@@ -632,12 +647,11 @@ int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hi
     const int count_merged = has_stats != 0;
     const int kinds        = count_batch + count_merged;
     const int copies       = kinds == 1 ? 4 : 2;   // LDS: kinds * bins * copies * 4 B <= 64 KiB at 4096 bins
-    const int blocks = hist_blocks(num_hist, n_per_hist);
-    char* ws         = (char*) workspace;
-    uint32_t* counts = (uint32_t*) ws;
-    ws += num_hist * blocks * 2 * (int64_t) num_bins * 4;
-    uint32_t* sums = (uint32_t*) ws;
-    ws += num_hist * 2 * (int64_t) num_bins * 4;
+    const int blocks   = hist_blocks(num_hist, n_per_hist);
+    const int replicas = blocks < kMaxReplicas ? blocks : kMaxReplicas;
+    char* ws           = (char*) workspace;
+    uint32_t* counts   = (uint32_t*) ws;
+    ws += num_hist * replicas * 2 * (int64_t) num_bins * 4;
     float* mm_part = (float*) ws;
     ws += num_hist * blocks * 2 * 4;
     ws             = (char*) (((uintptr_t) ws + 15) & ~(uintptr_t) 15);
@@ -646,18 +660,17 @@ int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hi
     const int vec  = (n_per_hist % 4 == 0) && aligned16(data);
     const int width = kinds * num_bins;
     hipLaunchKernelGGL(finite_minmax_kernel, dim3(blocks, (unsigned) num_hist), dim3(kHistBlock), 0, s, data, n_per_hist,
-                       mm_part, sums, width, vec);
+                       mm_part, counts, replicas * width, vec);
     MIQ_CHECK_LAUNCH();
     hipLaunchKernelGGL(hist_kernel, dim3(blocks, (unsigned) num_hist), dim3(kHistBlock),
                        (size_t) width * copies * sizeof(uint32_t), s, data, n_per_hist, num_bins, has_stats, count_batch,
-                       count_merged, copies, mm_part, state_minmax, ranges, batch_minmax, bad_flag, counts, vec);
+                       count_merged, copies, mm_part, state_minmax, ranges, batch_minmax, bad_flag, counts, replicas,
+                       vec);
     MIQ_CHECK_LAUNCH();
-    const int slices = blocks < 32 ? blocks : 32;
-    hipLaunchKernelGGL(reduce_counts_kernel, dim3((width + kHistBlock - 1) / kHistBlock, slices, (unsigned) num_hist),
-                       dim3(kHistBlock), 0, s, counts, blocks, width, sums);
-    MIQ_CHECK_LAUNCH();
-    hipLaunchKernelGGL(merge_kernel, dim3((unsigned) num_hist), dim3(kHistBlock), 0, s, sums, num_bins, has_stats,
-                       count_batch, count_merged, ranges, state_hist, state_minmax, want_batch_hist ? batch_hist : nullptr);
+    hipLaunchKernelGGL(merge_kernel, dim3((unsigned) num_hist, (unsigned) ((num_bins + kHistBlock - 1) / kHistBlock)),
+                       dim3(kHistBlock), 0, s, counts, replicas, num_bins,
+                       has_stats, count_batch, count_merged, ranges, state_hist, state_minmax,
+                       want_batch_hist ? batch_hist : nullptr);
     MIQ_CHECK_LAUNCH();
     return MIQ_OK;
 }
