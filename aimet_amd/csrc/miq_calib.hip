@@ -33,9 +33,12 @@ namespace
 {
 constexpr int kPdf      = MIQ_PDF_SIZE;
 constexpr int kMaxCand  = 512;
-constexpr int kCopies   = 16;
-constexpr int kMaxGrid  = 1024;   // upper bound on streaming workgroups (4 per CU): each lane keeps several 16-byte
-                                  // loads in flight, so this many waves already cover the HBM latency
+// LDS copies of the histogram per workgroup (lane l counts into copy l % kCopies) and the upper bound on streaming
+// workgroups.  8 copies are 16 KB, so 8 workgroups fit a compute unit and 2048 run in a single round: 7.3 us for a 25.7 MB
+// batch against 9.3 us with 16 copies / 1024 workgroups.  4 and 2 copies are faster still on spread-out data (6.9 / 6.7 us)
+// but collapse when the values share a bucket (constant tensor: 8.8 / 14.0 us against 6.9 us here).
+constexpr int kCopies   = 8;
+constexpr int kMaxGrid  = 2048;
 constexpr int kReplicas = 32;     // global count replicas: workgroup b merges into replica b % kReplicas, so at most
                                   // kMaxGrid / kReplicas atomics ever meet on one address
 
