@@ -74,6 +74,7 @@ _SIGNATURES = {
     "miq_adaround_soft_round_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int, _p], _int),
     "miq_adaround_floor_f32": ([_p, _p, _i64, _i64, _i64, _p, _p], _int),
     "miq_adaround_floor_i8": ([_p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _p, _p], _int),
+    "miq_adaround_floor_i16": ([_p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _p, _p], _int),
     "miq_adaround_init_alpha_f32": ([_p, _p, _i64, _i64, _i64, _p, _p], _int),
     "miq_adaround_bwd_adam_f32": ([_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _flt, _flt, _flt,
                                    _flt, _flt, _flt, _int, _p, _p], _int),
@@ -93,6 +94,10 @@ _SIGNATURES = {
                                     _p, _p, _p, _p, _p], _int),
     "miq_adaround_linear_bwd_adam_i8": ([_p, _p, _p, _p, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
                                          _flt, _flt, _flt, _flt, _flt, _flt, _int, _p, _p], _int),
+    "miq_adaround_linear_fwd_i16": ([_p, _p, _p, _p, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
+                                     _p, _p, _p, _p, _p], _int),
+    "miq_adaround_linear_bwd_adam_i16": ([_p, _p, _p, _p, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
+                                          _flt, _flt, _flt, _flt, _flt, _flt, _int, _p, _p], _int),
 }
 
 # Entry points declared in include/miq.h; the loader insists on every one of them.

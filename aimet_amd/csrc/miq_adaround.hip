@@ -93,26 +93,27 @@ __global__ __launch_bounds__(kBlock) void floor_kernel(const float* __restrict__
         out[e] = floorf(w[e] / g.delta[channel_of(e, g)]);
 }
 
-// floor(w / delta) saturated to [offset + clip_min - 2, offset + clip_max + 1] and stored as int8.  Outside that window
+// floor(w / delta) saturated to [offset + clip_min - 2, offset + clip_max + 1] and stored as int8 or int16.  Outside that window
 // the value no longer matters: h(alpha) lies in [0, 1], so floor + h - offset stays below clip_min (resp. above
 // clip_max) whatever alpha is, the clamp returns the same grid end and its gradient mask stays closed.  A channel whose
-// window does not fit int8 raises *unfit (the caller then keeps the float32 form).
-__global__ __launch_bounds__(kBlock) void floor_i8_kernel(const float* __restrict__ w, int8_t* __restrict__ out, AdaGeom g,
-                                                          int* __restrict__ unfit)
+// window does not fit the integer type raises *unfit (the caller then takes the next wider form).
+template <typename T, int LO, int HI>
+__global__ __launch_bounds__(kBlock) void floor_int_kernel(const float* __restrict__ w, T* __restrict__ out, AdaGeom g,
+                                                           int* __restrict__ unfit)
 {
     for (int64_t e = (int64_t) blockIdx.x * kBlock + threadIdx.x; e < g.n; e += (int64_t) gridDim.x * kBlock)
     {
         const uint32_t c = channel_of(e, g);
         const float lo   = g.offset[c] + g.clip_min - 2.0f;
         const float hi   = g.offset[c] + g.clip_max + 1.0f;
-        if (!(lo >= -128.0f && hi <= 127.0f))   // also true for NaN parameters
+        if (!(lo >= (float) LO && hi <= (float) HI))   // also true for NaN parameters
         {
             *unfit = 1;
             out[e] = 0;
             continue;
         }
         const float f = floorf(w[e] / g.delta[c]);
-        out[e]        = (int8_t) (int) fminf(fmaxf(f, lo), hi);   // NaN -> lo, as fmaxf drops it
+        out[e]        = (T) (int) fminf(fmaxf(f, lo), hi);   // NaN -> lo, as fmaxf drops it
     }
 }
 
@@ -286,7 +287,27 @@ int miq_adaround_floor_i8(const float* weight, int8_t* weight_floor, int64_t num
     int64_t blocks = (num_element + kBlock - 1) / kBlock;
     if (blocks > 65536)
         blocks = 65536;
-    hipLaunchKernelGGL(floor_i8_kernel, dim3((unsigned) blocks), dim3(kBlock), 0, (hipStream_t) stream, weight,
+    hipLaunchKernelGGL((floor_int_kernel<int8_t, -128, 127>), dim3((unsigned) blocks), dim3(kBlock), 0, (hipStream_t) stream, weight,
+                       weight_floor, g, unfit);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int miq_adaround_floor_i16(const float* weight, int16_t* weight_floor, int64_t num_channel, int64_t num_element,
+                          int64_t num_element_per_channel, const float* delta, const float* offset, float clip_min,
+                          float clip_max, int32_t* unfit, void* stream)
+{
+    AdaGeom g;
+    if (int rc = make_geom(g, num_channel, num_element, num_element_per_channel, delta, offset, clip_min, clip_max))
+        return rc;
+    MIQ_CHECK_ARG(unfit, "null flag pointer");
+    if (num_element == 0)
+        return MIQ_OK;
+    MIQ_CHECK_ARG(weight && weight_floor, "null tensor pointer");
+    int64_t blocks = (num_element + kBlock - 1) / kBlock;
+    if (blocks > 65536)
+        blocks = 65536;
+    hipLaunchKernelGGL((floor_int_kernel<int16_t, -32768, 32767>), dim3((unsigned) blocks), dim3(kBlock), 0, (hipStream_t) stream, weight,
                        weight_floor, g, unfit);
     MIQ_CHECK_LAUNCH();
     return MIQ_OK;

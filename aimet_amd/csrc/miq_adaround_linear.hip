@@ -58,7 +58,8 @@ __device__ __forceinline__ v4f ldg4_stream(const float* p)
 }
 
 // Four consecutive values of floor(W / delta), stored as float32 or, where every channel's window of useful values fits,
-// as int8 (miq_adaround_floor_i8): a quarter of the bytes of the operand that never changes during the optimisation.
+// as int8 or int16 (miq_adaround_floor_i8 / _i16): a quarter or half of the bytes of the operand that never changes
+// during the optimisation.
 template <typename FT>
 __device__ __forceinline__ v4f load_floor4(const FT* p);
 template <>
@@ -72,6 +73,15 @@ __device__ __forceinline__ v4f load_floor4<int8_t>(const int8_t* p)
     const int32_t w = __builtin_nontemporal_load(reinterpret_cast<const int32_t*>(p));
     return (v4f) {(float) (int8_t) (w & 0xff), (float) (int8_t) ((w >> 8) & 0xff), (float) (int8_t) ((w >> 16) & 0xff),
                   (float) (w >> 24)};
+}
+
+template <>
+__device__ __forceinline__ v4f load_floor4<int16_t>(const int16_t* p)
+{
+    typedef int v2i __attribute__((ext_vector_type(2)));
+    const v2i w = __builtin_nontemporal_load(reinterpret_cast<const v2i*>(p));
+    return (v4f) {(float) (int16_t) (w[0] & 0xffff), (float) (w[0] >> 16), (float) (int16_t) (w[1] & 0xffff),
+                  (float) (w[1] >> 16)};
 }
 
 constexpr int kLdsRow = kTileK + 4;   // floats per LDS tile row; the pad spreads the MFMA-layout accesses over banks
@@ -477,6 +487,29 @@ int miq_adaround_linear_bwd_adam_i8(const int8_t* weight_floor, const float* gra
                                     float eps, int step, float* reg_partial, void* stream)
 {
     return linear_bwd_adam<int8_t>(weight_floor, grad_out, x, row_index, x_row_stride, alpha, exp_avg, exp_avg_sq,
+                                   grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min,
+                                   clip_max, reg_param, beta, lr, beta1, beta2, eps, step, reg_partial, stream);
+}
+
+int miq_adaround_linear_fwd_i16(const int16_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
+                               int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+                               int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
+                               const float* offset, float clip_min, float clip_max, int activation, float* workspace,
+                               float* out, float* grad_out, float* loss_partial, void* stream)
+{
+    return linear_fwd<int16_t>(weight_floor, alpha, x, row_index, x_row_stride, target, target_row_stride, bias,
+                              out_features, in_features, num_channel, delta, offset, clip_min, clip_max, activation,
+                              workspace, out, grad_out, loss_partial, stream);
+}
+
+int miq_adaround_linear_bwd_adam_i16(const int16_t* weight_floor, const float* grad_out, const float* x,
+                                    const int32_t* row_index, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                    float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
+                                    int64_t num_channel, const float* delta, const float* offset, float clip_min,
+                                    float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
+                                    float eps, int step, float* reg_partial, void* stream)
+{
+    return linear_bwd_adam<int16_t>(weight_floor, grad_out, x, row_index, x_row_stride, alpha, exp_avg, exp_avg_sq,
                                    grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min,
                                    clip_max, reg_param, beta, lr, beta1, beta2, eps, step, reg_partial, stream);
 }

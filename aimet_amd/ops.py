@@ -367,18 +367,31 @@ def adaround_floor(weight, num_channel, n_per_channel, delta):
     return out
 
 
-def adaround_floor_i8(weight, num_channel, n_per_channel, delta, offset, clip_min, clip_max):
-    """floor(w / delta) as int8, saturated per channel to the window outside which its value cannot matter
-    (offset + clip_min - 2 .. offset + clip_max + 1), or None when some channel's window does not fit int8.
+def adaround_floor_int(weight, num_channel, n_per_channel, delta, offset, clip_min, clip_max, dtype=torch.int8):
+    """floor(w / delta) as int8 or int16, saturated per channel to the window outside which its value cannot matter
+    (offset + clip_min - 2 .. offset + clip_max + 1), or None when some channel's window does not fit the type.
     Reads one flag back from the device (once per layer)."""
     _ada_check(weight)
-    out = torch.empty(weight.shape, dtype=torch.int8, device=weight.device)
+    fn = {torch.int8: lib.miq_adaround_floor_i8, torch.int16: lib.miq_adaround_floor_i16}[dtype]
+    out = torch.empty(weight.shape, dtype=dtype, device=weight.device)
     unfit = torch.zeros(1, dtype=torch.int32, device=weight.device)
     with torch.cuda.device(weight.device):
-        check(lib.miq_adaround_floor_i8(_ptr(weight), _ptr(out), int(num_channel), weight.numel(), int(n_per_channel),
-                                        _ptr(delta), _ptr(offset), float(clip_min), float(clip_max), _ptr(unfit),
-                                        _stream(weight)))
+        check(fn(_ptr(weight), _ptr(out), int(num_channel), weight.numel(), int(n_per_channel), _ptr(delta),
+                 _ptr(offset), float(clip_min), float(clip_max), _ptr(unfit), _stream(weight)))
     return None if int(unfit.item()) else out
+
+
+def adaround_floor_i8(weight, num_channel, n_per_channel, delta, offset, clip_min, clip_max):
+    return adaround_floor_int(weight, num_channel, n_per_channel, delta, offset, clip_min, clip_max, torch.int8)
+
+
+def adaround_floor_packed(weight, num_channel, n_per_channel, delta, offset, clip_min, clip_max):
+    """The narrowest integer form of floor(w / delta) that fits (int8, then int16), or None."""
+    for dtype in (torch.int8, torch.int16):
+        out = adaround_floor_int(weight, num_channel, n_per_channel, delta, offset, clip_min, clip_max, dtype)
+        if out is not None:
+            return out
+    return None
 
 
 def adaround_init_alpha(weight, num_channel, n_per_channel, delta):
@@ -439,11 +452,12 @@ def adaround_linear_blocks(out_features, in_features):
 
 
 def _floor_variant(weight_floor, alpha, prefix):
-    """Entry point for the storage type of floor(W / delta): float32 or int8 (adaround_floor_i8)."""
-    if weight_floor.dtype not in (_F32, torch.int8) or not weight_floor.is_contiguous() or \
-            weight_floor.shape != alpha.shape or not weight_floor.is_cuda:
-        raise RuntimeError("weight_floor must be a contiguous float32 or int8 GPU tensor of alpha's shape")
-    return getattr(lib, prefix + ("f32" if weight_floor.dtype == _F32 else "i8"))
+    """Entry point for the storage type of floor(W / delta): float32, int8 or int16 (adaround_floor_int)."""
+    suffix = {_F32: "f32", torch.int8: "i8", torch.int16: "i16"}.get(weight_floor.dtype)
+    if suffix is None or not weight_floor.is_contiguous() or weight_floor.shape != alpha.shape or \
+            not weight_floor.is_cuda:
+        raise RuntimeError("weight_floor must be a contiguous float32, int8 or int16 GPU tensor of alpha's shape")
+    return getattr(lib, prefix + suffix)
 
 
 def adaround_linear_fwd(weight_floor, alpha, x, row_index, target, bias, num_channel, delta, offset, clip_min, clip_max,

@@ -29,7 +29,7 @@ class AdaroundOptimizer:
     # Linear layers whose shape the MFMA-fused kernels take (out % 32 == 0, in % 256 == 0, batch 32, no activation or
     # ReLU) use them; everything else runs soft-round kernel + torch layer + fused backward/Adam kernel
     use_fused_linear = True
-    use_int8_floor = True    # store floor(W / delta) as int8 for the fused Linear path when the grid allows it
+    use_int8_floor = True    # store floor(W / delta) as int8 / int16 for the fused Linear path when the grid allows it
 
     @classmethod
     def adaround_module(cls, module: torch.nn.Module, quant_module: AdaroundWrapper, orig_model: torch.nn.Module,
@@ -95,10 +95,10 @@ class AdaroundOptimizer:
                 cls._fused_linear_applies(module, weight, qm, all_inp_data, all_orig_out_data, batches):
             # soft rounding fused into the MFMA GEMMs: three launches per iteration, nothing weight-shaped is
             # written except alpha and the Adam moments
-            # floor(W / delta) never changes during the optimisation: int8 where the grid allows it (a quarter of the
-            # bytes, identical results), float32 otherwise (grids wider than 7 bits)
-            weight_floor = ops.adaround_floor_i8(weight, qm.num_channel, qm.n_per_channel, qm.delta, qm.offset,
-                                                 qm.clip_min, qm.clip_max) if cls.use_int8_floor else None
+            # floor(W / delta) never changes during the optimisation: int8 where the grid allows it (up to 7 bits; a
+            # quarter of the bytes), else int16, else float32 -- identical results in every form
+            weight_floor = ops.adaround_floor_packed(weight, qm.num_channel, qm.n_per_channel, qm.delta, qm.offset,
+                                                     qm.clip_min, qm.clip_max) if cls.use_int8_floor else None
             if weight_floor is None:
                 weight_floor = ops.adaround_floor(weight, qm.num_channel, qm.n_per_channel, qm.delta)
             index = torch.stack(batches).to(dtype=torch.int32, device=device).contiguous()

@@ -272,6 +272,10 @@ int miq_adaround_floor_f32(const float* weight, float* weight_floor, int64_t num
 int miq_adaround_floor_i8(const float* weight, int8_t* weight_floor, int64_t num_channel, int64_t num_element,
                           int64_t num_element_per_channel, const float* delta, const float* offset, float clip_min,
                           float clip_max, int32_t* unfit, void* stream);
+/* The same with int16 storage (grids of 8 to 14 bits). */
+int miq_adaround_floor_i16(const float* weight, int16_t* weight_floor, int64_t num_channel, int64_t num_element,
+                          int64_t num_element_per_channel, const float* delta, const float* offset, float clip_min,
+                          float clip_max, int32_t* unfit, void* stream);
 /* AdaroundWrapper._generate_alpha_parameter (ADA/adaround_wrapper.py:211-224):
  *   alpha = -log((zeta - gamma) / (w / delta - floor(w / delta) - gamma) - 1) */
 int miq_adaround_init_alpha_f32(const float* weight, float* alpha, int64_t num_channel, int64_t num_element,
@@ -315,8 +319,8 @@ int miq_adaround_blocks(int64_t num_element);
  * activation: 0 none, 1 ReLU (the act_func the reference applies to both outputs, ADA/adaround_optimizer.py:192-194).
  * ------------------------------------------------------------------------------------------------------------- */
 
-/* The same two entry points with weight_floor stored as int8 (miq_adaround_floor_i8): a quarter of the bytes of the one
- * weight-shaped operand that never changes during the optimisation.  No counterpart in the reference; results are
+/* The same two entry points with weight_floor stored as int8 or int16 (miq_adaround_floor_i8 / _i16): a quarter or half of
+ * the bytes of the one weight-shaped operand that never changes during the optimisation.  No counterpart in the reference; results are
  * identical to the float32 form, element for element. */
 
 /* Bytes of device workspace the forward needs (partial products of the split K dimension). */
@@ -346,6 +350,17 @@ int miq_adaround_linear_fwd_i8(const int8_t* weight_floor, const float* alpha, c
                                const float* offset, float clip_min, float clip_max, int activation, float* workspace,
                                float* out, float* grad_out, float* loss_partial, void* stream);
 int miq_adaround_linear_bwd_adam_i8(const int8_t* weight_floor, const float* grad_out, const float* x,
+                                    const int32_t* row_index, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                    float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
+                                    int64_t num_channel, const float* delta, const float* offset, float clip_min,
+                                    float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
+                                    float eps, int step, float* reg_partial, void* stream);
+int miq_adaround_linear_fwd_i16(const int16_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
+                               int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+                               int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
+                               const float* offset, float clip_min, float clip_max, int activation, float* workspace,
+                               float* out, float* grad_out, float* loss_partial, void* stream);
+int miq_adaround_linear_bwd_adam_i16(const int16_t* weight_floor, const float* grad_out, const float* x,
                                     const int32_t* row_index, int64_t x_row_stride, float* alpha, float* exp_avg,
                                     float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                     int64_t num_channel, const float* delta, const float* offset, float clip_min,

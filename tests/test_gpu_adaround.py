@@ -242,9 +242,26 @@ def test_fused_linear_forward_and_backward(ops, shape, per_channel, act):
                                  **hyper)
     assert torch.equal(a8, a1) and torch.equal(m8, m1) and torch.equal(v8, v1) and torch.equal(g8, g1)
     assert torch.equal(rp8, rp1)
-    # a grid of 8 bits does not fit: the window is 259 values wide
+    # a grid of 8 bits does not fit int8 (the window is 259 values wide) and goes to int16: same results again
     assert ops.adaround_floor_i8(wg, C, npc, dg, og, 0, 255) is None
     assert ops.adaround_floor_i8(wg, C, npc, dg, og + 200, cmin, cmax) is None
+    assert ops.adaround_floor_packed(wg, C, npc, dg, og, cmin, cmax).dtype == torch.int8
+    d8, o8 = dg / 16, og * 16                            # the 8-bit grid over the same range
+    f16 = ops.adaround_floor_packed(wg, C, npc, d8, o8, 0, 255)
+    assert f16.dtype == torch.int16
+    f32 = ops.adaround_floor(wg, C, npc, d8)
+    lo16 = ada.broadcast(o8.cpu(), weight, 0) - 2
+    hi16 = ada.broadcast(o8.cpu(), weight, 0) + 256
+    assert torch.equal(f16.cpu().float(), torch.minimum(torch.maximum(f32.cpu(), lo16), hi16))
+    res = []
+    for fl in (f32, f16):
+        Gx, ax, mx_, vx, gx = torch.empty_like(G), ag.clone(), m0.cuda(), v0.cuda(), torch.empty_like(ag)
+        ops.adaround_linear_fwd(fl, ag, Xg, ig, Yg, bg, C, d8, o8, 0, 255, act, ws, Gx)
+        ops.adaround_linear_bwd_adam(fl, Gx, Xg, ig, ax, mx_, vx, C, d8, o8, 0, 255, grad_alpha=gx, **hyper)
+        res.append((Gx, ax, mx_, vx, gx))
+    for t32, t16 in zip(*res):
+        assert torch.equal(t32, t16)
+    assert ops.adaround_floor_int(wg, C, npc, dg / 4096, og * 4096, 0, 65535, torch.int16) is None   # 16-bit grid
 
     # CPU gradient of the full loss (reconstruction + regulariser) w.r.t. alpha
     h = ada.rectified_sigmoid(a_ref)
