@@ -75,6 +75,29 @@ def test_large_batch_counts(ea):
     _same_hist(new[0], sq.collect_histogram(x, 2048))
 
 
+def test_very_large_and_concentrated_inputs(ea):
+    """Everything in one bin is the worst case for the per-workgroup counters and the replica merge: a constant tensor of
+    more than 130 M elements, first as the batch histogram, then merged a second time; and concentrated data next to
+    a few other values."""
+    n = 2048 * 63488 + 4099
+    x = torch.full((n,), 0.75, device="cuda")
+    obs = ea._HistogramObserver((1,), 2048)
+    for rep in (1, 2):
+        obs.collect_and_merge_stats(x)
+        hist = obs.get_stats()[0].histogram
+        want = float(np.float32(rep * n))             # the histogram is float32, as torch.histc's is
+        assert hist.max().item() == want and (hist > 0).sum().item() == 1
+    del x
+    y = torch.zeros(40_000_000, device="cuda")
+    y[::1000] = 1.0
+    y[1::1000] = 1.0 / 2048          # the bin next to the zeros'
+    obs = ea._HistogramObserver((1,), 2048)
+    new = obs.collect_and_merge_stats(y)
+    hist = new[0].histogram
+    assert hist[0].item() == 40_000_000 - 80_000 and hist[1].item() == 40_000 and hist[-1].item() == 40_000
+    assert hist.sum().item() == 40_000_000
+
+
 @pytest.mark.parametrize("symmetric", [False, True])
 @pytest.mark.parametrize("num_steps,gamma", [(255.0, 3.0), (255.0, 1.0), (15.0, 3.0), (65535.0, 3.0)])
 def test_search_matches_restatement(ea, symmetric, num_steps, gamma):
