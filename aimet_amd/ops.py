@@ -30,6 +30,26 @@ def _stream(t):
     return C.c_void_p(_stream_of(t.device))
 
 
+class _OnDevice:
+    """`with torch.cuda.device(d)` only when d is not already the current device: the context manager costs several
+    microseconds per call, as much as queueing the kernel, and the devices nearly always agree."""
+    __slots__ = ("_guard",)
+
+    def __init__(self, device):
+        self._guard = None
+        if device.index is not None and device.index != torch.cuda.current_device():
+            self._guard = torch.cuda.device(device)
+
+    def __enter__(self):
+        if self._guard is not None:
+            self._guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self._guard is not None:
+            self._guard.__exit__(*exc)
+        return False
+
+
 def _ptr(t):
     return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
 
@@ -90,7 +110,7 @@ def qdq_per_tensor(x, enc_min, enc_max, bw, rounding_mode=_lib.ROUND_NEAREST, ou
     x = x.contiguous()
     out = torch.empty_like(x) if out is None else out
     fn = getattr(lib, "miq_qdq_per_tensor_" + _suffix(x))
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(fn(_ptr(x), _ptr(out), x.numel(), float(enc_min), float(enc_max), int(bw), int(rounding_mode),
                  _stream(x)))
     return out
@@ -103,7 +123,7 @@ def fp16_round_trip(x, out=None):
         raise RuntimeError("fp16_round_trip takes float32 tensors")
     x = x.contiguous()
     out = torch.empty_like(x) if out is None else out
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(lib.miq_fp16_round_trip_f32(_ptr(x), _ptr(out), x.numel(), _stream(x)))
     return out
 
@@ -113,7 +133,7 @@ def quantize_per_tensor(x, enc_min, enc_max, bw, shift_to_signed, rounding_mode=
     _require_gpu(x)
     x = x.to(_F32).contiguous()
     out = torch.empty_like(x)
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(lib.miq_quantize_per_tensor_f32(_ptr(x), _ptr(out), x.numel(), float(enc_min), float(enc_max), int(bw),
                                               int(rounding_mode), int(bool(shift_to_signed)), _stream(x)))
     return out
@@ -125,7 +145,7 @@ def qdq_codes_per_tensor(x, enc_min, enc_max, bw, shift_to_signed=False, want_de
     x = x.to(_F32).contiguous()
     out = torch.empty_like(x) if want_dequant else None
     codes = torch.empty(x.shape, dtype=torch.int8 if shift_to_signed else torch.uint8, device=x.device)
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(lib.miq_qdq_codes_per_tensor_f32(_ptr(x), _ptr(out), _ptr(codes), x.numel(), float(enc_min),
                                                float(enc_max), int(bw), int(bool(shift_to_signed)), _stream(x)))
     return out, codes
@@ -137,7 +157,7 @@ def per_channel_params(enc_min, enc_max, num_steps):
     enc_min, enc_max = enc_min.to(_F32).contiguous(), enc_max.to(_F32).contiguous()
     c = enc_min.numel()
     outs = torch.empty(4, c, dtype=_F32, device=enc_min.device)
-    with torch.cuda.device(enc_min.device):
+    with _OnDevice(enc_min.device):
         check(lib.miq_per_channel_params_f32(_ptr(enc_min), _ptr(enc_max), c, float(num_steps), _ptr(outs[0]),
                                              _ptr(outs[1]), _ptr(outs[2]), _ptr(outs[3]), _stream(enc_min)))
     return outs[0], outs[1], outs[2], outs[3]
@@ -150,7 +170,7 @@ def qdq_per_channel(x, num_channel, n_per_channel, mn, mx, delta, offset, roundi
     out = torch.empty_like(x) if out is None else out
     fn = getattr(lib, "miq_qdq_per_channel_" + _suffix(x))
     mn, mx, delta, offset = (_params_f32(p, x) for p in (mn, mx, delta, offset))
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(fn(_ptr(x), _ptr(out), int(num_channel), x.numel(), int(n_per_channel), _ptr(mn), _ptr(mx),
                  _ptr(delta), _ptr(offset), int(rounding_mode), _stream(x)))
     return out
@@ -163,7 +183,7 @@ def qdq_codes_per_channel(x, num_channel, n_per_channel, mn, mx, delta, offset, 
     out = torch.empty_like(x) if want_dequant else None
     codes = torch.empty(x.shape, dtype=torch.int8 if shift_to_signed else torch.uint8, device=x.device)
     mn, mx, delta, offset = (_params_f32(p, x) for p in (mn, mx, delta, offset))
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(lib.miq_qdq_codes_per_channel_f32(_ptr(x), _ptr(out), _ptr(codes), int(num_channel), x.numel(),
                                                 int(n_per_channel), _ptr(mn), _ptr(mx), _ptr(delta), _ptr(offset),
                                                 int(bool(shift_to_signed)), int(bw), _stream(x)))
@@ -178,7 +198,7 @@ def qdq_broadcast(x, input_strides, encoding_strides, mn, mx, delta, offset):
     ist = (C.c_int64 * nd)(*[int(v) for v in input_strides])
     est = (C.c_int64 * nd)(*[int(v) for v in encoding_strides])
     mn, mx, delta, offset = (_params_f32(p, x) for p in (mn, mx, delta, offset))
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(lib.miq_qdq_broadcast_f32(_ptr(x), _ptr(out), x.numel(), nd, ist, est, _ptr(mn), _ptr(mx), _ptr(delta),
                                         _ptr(offset), _stream(x)))
     return out
@@ -189,7 +209,7 @@ def ste_bwd_per_tensor(x, grad_out, enc_min, enc_max, out=None):
     x, grad_out = x.contiguous(), grad_out.to(x.dtype).contiguous()
     gin = torch.empty_like(x) if out is None else out
     fn = getattr(lib, "miq_ste_bwd_per_tensor_" + _suffix(x))
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(fn(_ptr(x), _ptr(grad_out), _ptr(gin), x.numel(), float(enc_min), float(enc_max), _stream(x)))
     return gin
 
@@ -200,7 +220,7 @@ def ste_bwd_per_channel(x, grad_out, num_channel, n_per_channel, enc_min, enc_ma
     gin = torch.empty_like(x) if out is None else out
     fn = getattr(lib, "miq_ste_bwd_per_channel_" + _suffix(x))
     enc_min, enc_max = _params_f32(enc_min, x), _params_f32(enc_max, x)
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(fn(_ptr(x), _ptr(grad_out), _ptr(gin), int(num_channel), x.numel(), int(n_per_channel), _ptr(enc_min),
                  _ptr(enc_max), _stream(x)))
     return gin
@@ -212,7 +232,7 @@ def v2_qdq(x, num_channel, n_per_channel, scale, offset, qmin, qmax, want_codes=
     x = x.contiguous()
     scale, offset = _params_f32(scale, x).reshape(-1), _params_f32(offset, x).reshape(-1)
     out = torch.empty_like(x)
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         if x.dtype == _F32:
             codes = torch.empty(x.shape, dtype=torch.int32, device=x.device) if want_codes else None
             check(lib.miq_v2_qdq_f32(_ptr(x), _ptr(out), _ptr(codes), int(num_channel), x.numel(), int(n_per_channel),
@@ -231,7 +251,7 @@ def v2_qdq_bwd(x, grad_out, num_channel, n_per_channel, scale, offset, qmin, qma
     scale, offset = _params_f32(scale, x).reshape(-1), _params_f32(offset, x).reshape(-1)
     gin = torch.empty_like(x)
     fn = getattr(lib, "miq_v2_qdq_bwd_" + _suffix(x))
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(fn(_ptr(x), _ptr(grad_out), _ptr(gin), int(num_channel), x.numel(), int(n_per_channel), _ptr(scale),
                  _ptr(offset), int(qmin), int(qmax), _stream(x)))
     return gin
@@ -248,7 +268,7 @@ def v2_qdq_bwd_params(x, grad_out, num_channel, n_per_channel, scale, offset, qm
     ws = torch.empty(int(lib.miq_v2_qdq_bwd_params_workspace_bytes(c, x.numel(), npc)), dtype=torch.uint8,
                      device=x.device)
     fn = getattr(lib, "miq_v2_qdq_bwd_params_" + _suffix(x))
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(fn(_ptr(x), _ptr(grad_out), _ptr(gin) if want_grad_in else None, c, x.numel(), npc, _ptr(scale),
                  _ptr(offset), int(qmin), int(qmax), _ptr(grads[0]), _ptr(grads[1]), _ptr(ws), _stream(x)))
     return gin, grads[0], grads[1]
@@ -266,7 +286,7 @@ def minmax(x):
     x = x.to(_F32).contiguous()
     out = torch.empty(2, dtype=_F32, device=x.device)
     ws = _minmax_workspace(1, x.numel(), max(x.numel(), 1), x.device)
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(lib.miq_minmax_f32(_ptr(x), x.numel(), _ptr(out), _ptr(ws), _stream(x)))
     return out
 
@@ -277,7 +297,7 @@ def minmax_per_channel(x, num_channel, n_per_channel):
     x = x.to(_F32).contiguous()
     out = torch.empty(2, num_channel, dtype=_F32, device=x.device)
     ws = _minmax_workspace(num_channel, x.numel(), n_per_channel, x.device)
-    with torch.cuda.device(x.device):
+    with _OnDevice(x.device):
         check(lib.miq_minmax_per_channel_f32(_ptr(x), int(num_channel), x.numel(), int(n_per_channel), _ptr(out),
                                              _ptr(ws), _stream(x)))
     return out
@@ -299,7 +319,7 @@ def v2_hist_update(data, num_hist, num_bins, has_stats, state_hist, state_minmax
     n_per_hist = data.numel() // num_hist
     batch_hist = torch.empty(num_hist, num_bins, dtype=_F32, device=data.device) if want_batch_hist else None
     batch_minmax = torch.empty(num_hist, 2, dtype=_F32, device=data.device)
-    with torch.cuda.device(data.device):
+    with _OnDevice(data.device):
         check(lib.miq_v2_hist_update_f32(_ptr(data), int(num_hist), int(n_per_hist), int(num_bins), int(has_stats),
                                          int(bool(want_batch_hist)), _ptr(state_hist), _ptr(state_minmax),
                                          _ptr(batch_hist), _ptr(batch_minmax), _ptr(bad_flag), _ptr(workspace),
@@ -325,7 +345,7 @@ def v2_sqnr_search(hist, minmax, num_steps, symmetric, gamma, asym_deltas, sym_d
     out = torch.empty(2, num_hist, dtype=_F32, device=hist.device)
     noise = torch.empty(num_hist, ncand, dtype=torch.float64, device=hist.device)
     best = torch.empty(num_hist, dtype=torch.int32, device=hist.device) if want_details else None
-    with torch.cuda.device(hist.device):
+    with _OnDevice(hist.device):
         check(lib.miq_v2_sqnr_search_f32(_ptr(hist), _ptr(minmax), num_hist, num_bins, float(num_steps),
                                          int(symmetric), float(gamma), int(asym_deltas), int(sym_deltas),
                                          int(offset_candidates), _ptr(out[0]), _ptr(out[1]), _ptr(noise), _ptr(best),
@@ -350,7 +370,7 @@ def adaround_soft_round(weight, alpha, num_channel, n_per_channel, delta, offset
     """(clamp(floor(w / delta) + h(alpha) - offset, clip_min, clip_max) + offset) * delta."""
     _ada_check(weight, alpha, out)
     out = torch.empty_like(weight) if out is None else out
-    with torch.cuda.device(weight.device):
+    with _OnDevice(weight.device):
         check(lib.miq_adaround_soft_round_f32(_ptr(weight), _ptr(alpha), _ptr(out), int(num_channel), weight.numel(),
                                               int(n_per_channel), _ptr(delta), _ptr(offset), float(clip_min),
                                               float(clip_max), int(bool(use_soft_rounding)), _stream(weight)))
@@ -361,7 +381,7 @@ def adaround_floor(weight, num_channel, n_per_channel, delta):
     """floor(w / delta): the alpha-independent part of apply_adaround, input of the fused Linear kernels."""
     _ada_check(weight)
     out = torch.empty_like(weight)
-    with torch.cuda.device(weight.device):
+    with _OnDevice(weight.device):
         check(lib.miq_adaround_floor_f32(_ptr(weight), _ptr(out), int(num_channel), weight.numel(),
                                          int(n_per_channel), _ptr(delta), _stream(weight)))
     return out
@@ -375,7 +395,7 @@ def adaround_floor_int(weight, num_channel, n_per_channel, delta, offset, clip_m
     fn = {torch.int8: lib.miq_adaround_floor_i8, torch.int16: lib.miq_adaround_floor_i16}[dtype]
     out = torch.empty(weight.shape, dtype=dtype, device=weight.device)
     unfit = torch.zeros(1, dtype=torch.int32, device=weight.device)
-    with torch.cuda.device(weight.device):
+    with _OnDevice(weight.device):
         check(fn(_ptr(weight), _ptr(out), int(num_channel), weight.numel(), int(n_per_channel), _ptr(delta),
                  _ptr(offset), float(clip_min), float(clip_max), _ptr(unfit), _stream(weight)))
     return None if int(unfit.item()) else out
@@ -398,7 +418,7 @@ def adaround_init_alpha(weight, num_channel, n_per_channel, delta):
     """alpha such that h(alpha) equals the fractional part of w / delta."""
     _ada_check(weight)
     alpha = torch.empty_like(weight)
-    with torch.cuda.device(weight.device):
+    with _OnDevice(weight.device):
         check(lib.miq_adaround_init_alpha_f32(_ptr(weight), _ptr(alpha), int(num_channel), weight.numel(),
                                               int(n_per_channel), _ptr(delta), _stream(weight)))
     return alpha
@@ -413,7 +433,7 @@ def adaround_bwd(weight, grad_weight, alpha, num_channel, n_per_channel, delta, 
     """dLoss/dW' -> dLoss/dalpha (rounding regulariser included when beta >= 0); returns the gradient."""
     _ada_check(weight, grad_weight, alpha)
     grad_alpha = torch.empty_like(alpha)
-    with torch.cuda.device(weight.device):
+    with _OnDevice(weight.device):
         check(lib.miq_adaround_bwd_f32(_ptr(weight), _ptr(grad_weight), _ptr(alpha), _ptr(grad_alpha),
                                        int(num_channel), weight.numel(), int(n_per_channel), _ptr(delta),
                                        _ptr(offset), float(clip_min), float(clip_max), float(reg_param), float(beta),
@@ -428,7 +448,7 @@ def adaround_bwd_adam(weight, grad_weight, alpha, exp_avg, exp_avg_sq, num_chann
     _ada_check(weight, grad_weight, alpha, exp_avg, exp_avg_sq)
     if reg_partial is not None and reg_partial.numel() < adaround_blocks(weight.numel()):
         raise RuntimeError("reg_partial is too small")
-    with torch.cuda.device(weight.device):
+    with _OnDevice(weight.device):
         check(lib.miq_adaround_bwd_adam_f32(_ptr(weight), _ptr(grad_weight), _ptr(alpha), _ptr(exp_avg),
                                             _ptr(exp_avg_sq), _ptr(grad_alpha), int(num_channel), weight.numel(), int(n_per_channel),
                                             _ptr(delta), _ptr(offset), float(clip_min), float(clip_max),
@@ -471,7 +491,7 @@ def adaround_linear_fwd(weight_floor, alpha, x, row_index, target, bias, num_cha
     if row_index is not None and (row_index.dtype != torch.int32 or row_index.numel() != 32):
         raise RuntimeError("row_index must hold 32 int32 row numbers")
     o, k = weight_floor.shape
-    with torch.cuda.device(weight_floor.device):
+    with _OnDevice(weight_floor.device):
         check(fn(_ptr(weight_floor), _ptr(alpha), _ptr(x), _ptr(row_index), x.stride(0), _ptr(target), target.stride(0),
                  _ptr(bias), o, k, int(num_channel), _ptr(delta), _ptr(offset), float(clip_min), float(clip_max),
                  int(activation), _ptr(workspace), _ptr(out), _ptr(grad_out), _ptr(loss_partial), _stream(weight_floor)))
@@ -485,7 +505,7 @@ def adaround_linear_bwd_adam(weight_floor, grad_out, x, row_index, alpha, exp_av
     fn = _floor_variant(weight_floor, alpha, "miq_adaround_linear_bwd_adam_")
     _require_gpu(weight_floor, x, row_index)
     o, k = weight_floor.shape
-    with torch.cuda.device(weight_floor.device):
+    with _OnDevice(weight_floor.device):
         check(fn(_ptr(weight_floor), _ptr(grad_out), _ptr(x), _ptr(row_index), x.stride(0), _ptr(alpha), _ptr(exp_avg),
                  _ptr(exp_avg_sq), _ptr(grad_alpha), o, k, int(num_channel), _ptr(delta), _ptr(offset), float(clip_min),
                  float(clip_max), float(reg_param), float(beta), float(lr), float(beta1), float(beta2), float(eps),
@@ -510,7 +530,7 @@ class Analyzer:
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
-        if h:
+        if h and lib is not None:                 # at interpreter shutdown the module's globals may already be gone
             lib.miq_analyzer_destroy(h)
 
     def _s(self):

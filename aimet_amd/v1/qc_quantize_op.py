@@ -105,7 +105,12 @@ class QcQuantizeWrapper(nn.Module):
         self.supported_kernels = {}
 
     def get_named_parameters(self):
-        yield from self._module_to_wrap.named_parameters()
+        module = self._module_to_wrap
+        if not module._modules:                     # pylint: disable=protected-access
+            # a leaf module: its own parameter table, without named_parameters' walk over the module tree (this runs
+            # several times per forward pass of every wrapper)
+            return [(name, p) for name, p in module._parameters.items() if p is not None]  # pylint: disable=protected-access
+        return list(module.named_parameters())
 
     def __getattr__(self, name):
         try:
@@ -337,7 +342,7 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
         else:
             wrapped_output = self._module_to_wrap(*quantized_inputs, **kwargs)
         self._restore_shadow_params(shadow_params)
-        if not isinstance(wrapped_output, (List, Tuple)):
+        if not isinstance(wrapped_output, (list, tuple)):
             wrapped_output = [wrapped_output]
         output = self._quantize_activation(self.output_quantizers, list(wrapped_output))
         return output[0] if len(output) == 1 else output
@@ -402,7 +407,7 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
 
     def _quantize_activation(self, tensor_quantizers, tensors_to_quantize):
         def inner(tensor, index):
-            if isinstance(tensor, (List, Tuple)):
+            if isinstance(tensor, (list, tuple)):
                 return [inner(t, index) for t in tensor]
             if not isinstance(tensor, torch.Tensor):
                 return tensor
@@ -548,7 +553,7 @@ class LearnedGridQuantWrapper(QcQuantizeWrapper):
         if torch.is_grad_enabled() and is_recompute_enabled():
             forward_fn = _fused_forward_functions.get(type(self._module_to_wrap), _default_forward)
         wrapped_output = forward_fn(self, quantized_inputs, **kwargs)
-        if not isinstance(wrapped_output, (List, Tuple)):
+        if not isinstance(wrapped_output, (list, tuple)):
             wrapped_output = [wrapped_output]
         output = self._quantize_activation(list(wrapped_output), self.output_quantizers, 'output')
         return output[0] if len(output) == 1 else output
@@ -581,7 +586,7 @@ class LearnedGridQuantWrapper(QcQuantizeWrapper):
 
     def _quantize_activation(self, tensors_to_quantize, tensor_quantizers, type_of_quantizer: str) -> List:
         def inner(tensor, index):
-            if isinstance(tensor, (List, Tuple)):
+            if isinstance(tensor, (list, tuple)):
                 return [inner(t, index) for t in tensor]
             if not isinstance(tensor, torch.Tensor) or \
                     not self.should_perform_quant_dequant(tensor, tensor_quantizers[index]):

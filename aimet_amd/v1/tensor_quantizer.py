@@ -166,6 +166,9 @@ class StaticGridTensorQuantizer(TensorQuantizer):
                                self.use_unsigned_symmetric) for op in self._cppOp]
 
     def quantize_dequantize(self, tensor: torch.Tensor, round_mode: libpymo.RoundingMode) -> torch.Tensor:
+        if not torch.is_grad_enabled():
+            # inference: the same forward without the autograd.Function machinery (about 10 us per call)
+            return QuantizeDequantize.forward(_NoContext(), tensor, self, round_mode)
         return QuantizeDequantize.apply(tensor, self, round_mode)
 
     def quantize(self, tensor: torch.Tensor, round_mode: libpymo.RoundingMode) -> torch.Tensor:
@@ -298,6 +301,14 @@ def _channel_geometry(tensor, ch_axis):
     num_channel = sizes[ch_axis]
     n_per_channel = functools.reduce(lambda x, y: x * y, sizes[ch_axis + 1:])
     return num_channel, n_per_channel
+
+
+class _NoContext:
+    """Stands in for the autograd context when QuantizeDequantize.forward is called directly (no gradient)."""
+    __slots__ = ("tensor_quantizer",)
+
+    def save_for_backward(self, *_):
+        pass
 
 
 class QuantizeDequantize(torch.autograd.Function):

@@ -402,6 +402,26 @@ def bench_quantsim(torch, steps=10, batch=64):
 
     fp32_ms = timed(lambda: model(x))
     sim_ms = timed(lambda: sim.model(x))
+    # Latency at batch 1: launch- and Python-bound when run eagerly, so the simulated forward is also captured in a HIP
+    # graph (nothing on the path waits for the device) and replayed.
+    x1 = x[:1].clone()
+    lat = {"fp32_eager_ms": timed(lambda: model(x1)), "sim_eager_ms": timed(lambda: sim.model(x1))}
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                sim.model(x1)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y1 = sim.model(x1)
+    lat["sim_hip_graph_replay_ms"] = timed(graph.replay)
+    with torch.no_grad():
+        ref1 = sim.model(x1)
+    # (the convolutions of this model are not run-to-run deterministic, so two eager passes differ as much)
+    lat["graph_vs_eager_max_abs_diff"] = float((y1 - ref1).abs().max())
+    del graph
     wrappers = list(sim.quant_wrappers())
     n_act = sum(q.enabled for _, w in wrappers for q in w.input_quantizers + w.output_quantizers)
     n_par = sum(q.enabled for _, w in wrappers for q in w.param_quantizers.values())
@@ -409,7 +429,8 @@ def bench_quantsim(torch, steps=10, batch=64):
             "activation_quantizers": int(n_act), "param_quantizers": int(n_par),
             "fp32_forward_ms": fp32_ms, "quantsim_forward_ms": sim_ms,
             "qdq_overhead_ms": sim_ms - fp32_ms, "qdq_overhead_pct_of_fp32": 100.0 * (sim_ms - fp32_ms) / fp32_ms,
-            "images_per_s": batch / (sim_ms / 1e3), "fp32_images_per_s": batch / (fp32_ms / 1e3)}
+            "images_per_s": batch / (sim_ms / 1e3), "fp32_images_per_s": batch / (fp32_ms / 1e3),
+            "latency_batch1": lat}
 
 
 def bench_sqnr(torch, ops, reps=5):

@@ -381,3 +381,50 @@ def test_float16_data_type(api, tmp_path):
     assert data["param_encodings"]["conv2.weight"] == [{"bitwidth": 16, "dtype": "float"}]
     assert data["activation_encodings"]["relu1"]["output"]["0"] == {"bitwidth": 16, "dtype": "float"}
     assert data["quantizer_args"]["dtype"] == "float"
+
+
+class _LinearNet(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.fc1, self.relu1 = nn.Linear(64, 128), nn.ReLU()
+        self.fc2, self.relu2 = nn.Linear(128, 128), nn.ReLU()
+        self.fc3 = nn.Linear(128, 10)
+
+    def forward(self, x):
+        return self.fc3(self.relu2(self.fc2(self.relu1(self.fc1(x)))))
+
+
+def test_simulation_forward_in_a_hip_graph(api):
+    """Inference through the simulation model queues kernels on torch's current stream and never waits for the device,
+    so it can be captured once and replayed (a small-batch forward is bound by launch and Python overhead otherwise).
+    Replays are interleaved with eager work and synchronisations and each one is checked against the eager result."""
+    torch.manual_seed(11)
+    model = _LinearNet().eval().cuda()
+    dummy = torch.randn(4, 64).cuda()
+    cfg = {"defaults": {"ops": {"is_output_quantized": "True"},
+                        "params": {"is_quantized": "True", "is_symmetric": "True"},
+                        "per_channel_quantization": "True"},
+           "params": {"bias": {"is_quantized": "False"}}, "op_type": {},
+           "supergroups": [{"op_list": ["Gemm", "Relu"]}], "model_input": {"is_input_quantized": "True"},
+           "model_output": {}}
+    sim = api.quantsim.QuantizationSimModel(model, dummy_input=dummy, quant_scheme='tf_enhanced', config_file=cfg)
+    sim.compute_encodings(_calibrate, [torch.randn(32, 64).cuda() for _ in range(2)])
+    static_x = torch.randn(16, 64).cuda()
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                sim.model(static_x)                         # warm-up outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_y = sim.model(static_x)
+        for rep in range(5):
+            x = torch.randn(16, 64).cuda() * (rep + 1)
+            static_x.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            eager = sim.model(x)                            # eager work between the replays
+            assert torch.equal(static_y, eager), rep
+            torch.cuda.synchronize()
