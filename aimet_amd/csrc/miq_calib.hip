@@ -473,7 +473,7 @@ __device__ __forceinline__ void hist_add(uint32_t* lds, float x, float bucket, f
     // DLQ/src/math_functions.cpp:375-382; the range test is done on the rounded float so that NaN and values
     // beyond the int range are dropped, as they are on the reference's CPU path
     const float q  = (rcp != 0.0f && fabsf(x) <= kFastDivMaxDividend) ? div_by_invariant(x, bucket, rcp) : x / bucket;
-    const float r  = roundf(q - off);
+    const float r  = round_half_away(q - off);   // == roundf
     const bool ok  = (r >= 0.0f && r < (float) kPdf);
     const int row  = ok ? (int) r : kPdf;
     atomicAdd(&lds[row * kCopies + copy], 1u);

@@ -42,5 +42,14 @@ MIQ_HD inline float div_by_invariant(float a, float b, float y)
     q       = __builtin_fmaf(r, y, q);
     return __builtin_copysignf(q, a);
 }
+// roundf (halves away from zero) in three operations: add the largest float below one half with the sign of x, then
+// truncate.  Equal to roundf(x) for every binary32 value (tests/test_fastmath.py walks through all of them below 2^24 in
+// both signs; from 2^23 on every float is an integer and comes back unchanged): x + 0.49999997 crosses the next integer
+// exactly when the fraction of |x| is at least one half, and the one case where the sum itself rounds (fraction exactly
+// one half: 0.5 + 0.49999997 rounds to 1.0) rounds the way roundf does.  The compiler's own expansion of roundf takes six.
+MIQ_HD inline float round_half_away(float x)
+{
+    return __builtin_truncf(x + __builtin_copysignf(0.49999997f, x));
+}
 }   // namespace miq
 #endif

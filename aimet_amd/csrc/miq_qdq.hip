@@ -73,7 +73,7 @@ struct OpV1
         float t = fmaxf(fminf(x, p.mx), p.mn);
         t       = FAST ? div_by_invariant(t, p.delta, p.rcp) : t / p.delta;
         t       = t - p.offset;
-        return roundf(t);
+        return round_half_away(t);   // == roundf(t), three operations instead of six
     }
 };
 

@@ -3,6 +3,7 @@
 * div_by_invariant (aimet_amd/csrc/miq_fastmath.h) must equal IEEE binary32 division bit for bit inside its
   contract: the header is compiled for the host and compared with `/` on hundreds of millions of operand pairs.
 * the multiply-high division by a launch-invariant 31-bit divisor (miq_common.h) must equal integer division.
+* round_half_away (miq_fastmath.h), the three-operation roundf, must equal roundf for every float.
 """
 import os
 import subprocess
@@ -20,6 +21,17 @@ def test_div_by_invariant_equals_ieee_division(tmp_path):
         flags.append("-mfma")          # hardware fused multiply-add; otherwise libm's (slower, equally exact)
     subprocess.run(["g++", *flags, "-o", str(exe), src], check=True)
     out = subprocess.run([str(exe), "20"], capture_output=True, text=True, timeout=600)
+    assert out.returncode == 0, out.stdout[-2000:]
+    assert out.stdout.startswith("OK")
+
+
+def test_round_half_away_equals_roundf(tmp_path):
+    exe = tmp_path / "round_check"
+    src = os.path.join(ROOT, "tests", "host", "round_check.cpp")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-o", str(exe), src], check=True)
+    # every 5th bit pattern up to 2^24 in both signs + a dense sweep around the half-integers (about 10 s; stride 1
+    # is the exhaustive walk)
+    out = subprocess.run([str(exe), "5"], capture_output=True, text=True, timeout=600)
     assert out.returncode == 0, out.stdout[-2000:]
     assert out.stdout.startswith("OK")
 
