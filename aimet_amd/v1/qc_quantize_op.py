@@ -295,8 +295,15 @@ class QcQuantizeWrapper(nn.Module):
         a no-op otherwise (reference :355-361)."""
 
     def should_perform_quant_dequant(self, tensor: torch.Tensor, tensor_quantizer) -> bool:
-        """Only floating point tensors with an enabled quantizer are quantized (reference :452-468)."""
-        return tensor_quantizer.enabled and tensor.dtype in (torch.float32, torch.float16, torch.bfloat16)
+        """Only floating point tensors with an enabled quantizer are quantized.  A quantizer that meets anything else,
+        or a constant of one element, is switched off for good (reference :452-472)."""
+        if not tensor_quantizer.enabled:
+            return False
+        if tensor.dtype not in (torch.float32, torch.float16, torch.bfloat16) or \
+                (tensor_quantizer.is_const and tensor.numel() == 1):
+            tensor_quantizer.enabled = False
+            return False
+        return True
 
 
 class SteGatingFuncForParameters(torch.autograd.Function):

@@ -83,6 +83,7 @@ _INIT_SCHEME = {
 }
 
 
+_CONSTANT = "__constant__"     # source of a module input that does not depend on the model's inputs
 _FLOAT16_ENTRY = object()     # marks a float16 quantizer in the export: it has no encoding, only a type
 
 
@@ -152,15 +153,52 @@ class QuantizationSimModel:
         return len(list(module.children())) == 0
 
     def _trace(self, model: nn.Module, dummy_input: Tuple):
-        """One hooked forward pass: execution order of the leaf modules and tensor producers / consumers."""
+        """One hooked forward pass: execution order of the leaf modules and tensor producers / consumers.
+
+        Every positional input of a module is classified: produced by a module, a model input, an intermediate value
+        that a functional op computed from the model's inputs (producer unknown: None), or a constant -- a tensor
+        that does not depend on the model's inputs (a buffer, a tensor created in forward) or a python number.
+        Constants are told from intermediates by following, through every torch function called during the pass,
+        which tensors derive from the model's inputs.
+        """
         records, handles = [], []
         producer: Dict[int, str] = {}
         consumers: Dict[str, List[str]] = {}      # producing module -> consuming modules
         keep_alive = []
+        derived = set()                           # ids of tensors computed from the model's inputs
         names = {m: n for n, m in model.named_modules()}
-        for t in dummy_input:
-            if isinstance(t, torch.Tensor):
-                producer[id(t)] = "__model_input__"
+
+        def tensors_in(obj):
+            if isinstance(obj, torch.Tensor):
+                yield obj
+            elif isinstance(obj, (list, tuple)):
+                for item in obj:
+                    yield from tensors_in(item)
+            elif isinstance(obj, dict):
+                for item in obj.values():
+                    yield from tensors_in(item)
+
+        for t in tensors_in(dummy_input):
+            producer[id(t)] = "__model_input__"
+            derived.add(id(t))
+
+        class Follow(torch.overrides.TorchFunctionMode):
+            def __torch_function__(self, func, types, args=(), kwargs=None):
+                out = func(*args, **(kwargs or {}))
+                if any(id(t) in derived for t in tensors_in((args, kwargs or {}))):
+                    for t in tensors_in(out):
+                        keep_alive.append(t)
+                        derived.add(id(t))
+                return out
+
+        def classify(value):
+            if isinstance(value, torch.Tensor):
+                if id(value) in producer:
+                    return producer[id(value)]
+                return None if id(value) in derived else _CONSTANT
+            if isinstance(value, (int, float)) and not isinstance(value, bool):
+                return _CONSTANT
+            return None
 
         def hook(module, inputs, output):
             name = names[module]
@@ -168,35 +206,44 @@ class QuantizationSimModel:
             outs = [t for t in (output if isinstance(output, (tuple, list)) else (output,))
                     if isinstance(t, torch.Tensor)]
             keep_alive.extend(ins + outs)            # ids stay unique while the pass runs
-            for t in ins:
+            sources = [classify(value) for value in inputs]
+            for src in sources:
                 # resolved now, not afterwards: an in-place op returns the tensor it was given, so the tensor's id
                 # says nothing about who produced the value a later module reads
-                if id(t) in producer:
-                    consumers.setdefault(producer[id(t)], []).append(name)
-            records.append({"name": name, "module": module, "type": _op_type(module),
-                            "inputs": [producer.get(id(t)) for t in ins], "in_ids": [id(t) for t in ins],
-                            "out_ids": [id(t) for t in outs], "num_inputs": max(1, len(ins)),
-                            "num_outputs": max(1, len(outs))})
+                if src is not None and src is not _CONSTANT:
+                    consumers.setdefault(src, []).append(name)
+            records.append({"name": name, "module": module, "type": _op_type(module), "inputs": sources,
+                            "num_inputs": max(1, len(inputs)), "num_outputs": max(1, len(outs))})
             for t in outs:
                 producer[id(t)] = name
+                derived.add(id(t))
 
         for module in model.modules():
-            if self._is_leaf(module) and module is not model:
+            # nn.Identity is never wrapped (reference :205-207, :1430-1434); unhooked, the tensor it passes through
+            # keeps its producer
+            if self._is_leaf(module) and module is not model and not isinstance(module, nn.Identity):
                 handles.append(module.register_forward_hook(hook))
         was_training = model.training
         model.eval()
         try:
-            with torch.no_grad():
+            with torch.no_grad(), Follow():
                 out = model(*dummy_input)
         finally:
             for h in handles:
                 h.remove()
             model.train(was_training)
-        outs = out if isinstance(out, (tuple, list)) else (out,)
-        model_outputs = {producer.get(id(t)) for t in outs if isinstance(t, torch.Tensor)}
+        model_outputs = {producer.get(id(t)) for t in tensors_in(out)}
         for r in records:
             r["consumers"] = list(consumers.get(r["name"], []))
             r["is_model_output"] = r["name"] in model_outputs
+        # leaf modules that the forward pass never reached are wrapped too, with the default configuration
+        # (the reference wraps every quantizable leaf, :1440-1454)
+        reached = {r["name"] for r in records}
+        for name, module in model.named_modules():
+            if self._is_leaf(module) and module is not model and not isinstance(module, nn.Identity) \
+                    and name not in reached and not isinstance(module, QcQuantizeWrapper):
+                records.append({"name": name, "module": module, "type": _op_type(module), "inputs": [],
+                                "num_inputs": 1, "num_outputs": 1, "consumers": [], "is_model_output": False})
         return records
 
     def _add_quantization_wrappers(self):
@@ -213,6 +260,8 @@ class QuantizationSimModel:
                                              num_inputs=rec["num_inputs"], num_outputs=rec["num_outputs"],
                                              data_type=self._default_data_type)
             rec["wrapper"] = wrapper
+            for idx, src in enumerate(rec["inputs"]):
+                wrapper.input_quantizers[idx].is_const = src is _CONSTANT     # reference :1456-1471
             parent = self.model
             *path, leaf = rec["name"].split('.')
             for p in path:
@@ -270,8 +319,9 @@ class QuantizationSimModel:
                     member["wrapper"].enable_input_quantizers(False)
         if _flag(cfg.get("model_input", {}), "is_input_quantized", False):
             for rec in self._graph:
+                # model inputs and constant inputs alike (reference quantsim_config.py:560-581)
                 for idx, src in enumerate(rec["inputs"]):
-                    if src == "__model_input__" and idx < len(rec["wrapper"].input_quantizers):
+                    if (src == "__model_input__" or src is _CONSTANT) and idx < len(rec["wrapper"].input_quantizers):
                         rec["wrapper"].input_quantizers[idx].enabled = True
         if _flag(cfg.get("model_output", {}), "is_output_quantized", False):
             for rec in self._graph:
@@ -300,13 +350,7 @@ class QuantizationSimModel:
     def compute_encodings(self, forward_pass_callback, forward_pass_callback_args):
         """Runs `forward_pass_callback(model, args)` in ANALYSIS mode, then computes every encoding and switches the
         wrappers to ACTIVE (reference :425-448)."""
-        layers = [(n, m) for n, m in self._get_qc_quantized_layers(self.model)
-                  if isinstance(m, StaticGridQuantWrapper)]
-        for _, layer in layers:
-            layer.reset_encodings()
-            layer.set_mode(QcQuantizeOpMode.ANALYSIS)
-            if self._quant_scheme == QuantScheme.post_training_percentile:
-                layer.set_percentile_value(self._percentile_value)     # reference :395-400
+        self.prepare_sim_for_compute_encodings()
         was_training = self.model.training
         self.model.eval()
         try:
@@ -314,7 +358,23 @@ class QuantizationSimModel:
                 forward_pass_callback(self.model, forward_pass_callback_args)
         finally:
             self.model.train(was_training)
-        for _, layer in layers:
+        self.compute_layer_encodings_for_sim()
+
+    def _static_grid_layers(self):
+        return [m for _, m in self._get_qc_quantized_layers(self.model) if isinstance(m, StaticGridQuantWrapper)]
+
+    def prepare_sim_for_compute_encodings(self):
+        """Statistics cleared, wrappers in ANALYSIS mode (reference :384-403)."""
+        for layer in self._static_grid_layers():
+            layer.reset_encodings()
+            layer.set_mode(QcQuantizeOpMode.ANALYSIS)
+            if self._quant_scheme == QuantScheme.post_training_percentile:
+                layer.set_percentile_value(self._percentile_value)     # reference :395-400
+
+    def compute_layer_encodings_for_sim(self):
+        """Encodings from the gathered statistics, wrappers back to ACTIVE; a quantizer that saw no data is switched
+        off (reference :405-423)."""
+        for layer in self._static_grid_layers():
             layer.compute_encoding()
             layer.set_mode(QcQuantizeOpMode.ACTIVE)
         self.replace_wrappers_for_quantize_dequantize()
@@ -483,3 +543,32 @@ class QuantizationSimModel:
             encodings = json.load(f)
         encodings.pop('activation_encodings', None)
         self.load_encodings(encodings, strict=True, partial=True, requires_grad=False, allow_overwrite=False)
+
+
+def has_valid_encodings(qc_quantize_op: QcQuantizeWrapper) -> bool:
+    """True if any enabled input, parameter or output quantizer of the wrapper holds an encoding (or simulates
+    float16, which needs none) -- reference quantsim.py:2301-2323."""
+    if not isinstance(qc_quantize_op, QcQuantizeWrapper):
+        raise AssertionError("has_valid_encodings is only supported for quantization wrappers")
+    quantizers = list(qc_quantize_op.input_quantizers) + list(qc_quantize_op.output_quantizers) + \
+        list(qc_quantize_op.param_quantizers.values())
+    return any(_exported_encoding(q) is not None for q in quantizers)
+
+
+def compute_encodings_for_sims(sim_list: List[QuantizationSimModel], forward_pass_callback,
+                               forward_pass_callback_args):
+    """Calibrates several simulation models with one callback, which receives the list of their models in the order
+    of `sim_list` (reference quantsim.py:2326-2356).  All models run in eval mode and without autograd during the
+    callback and get their own mode back afterwards."""
+    modes = [sim.model.training for sim in sim_list]
+    for sim in sim_list:
+        sim.prepare_sim_for_compute_encodings()
+        sim.model.eval()
+    try:
+        with torch.no_grad():
+            forward_pass_callback([sim.model for sim in sim_list], forward_pass_callback_args)
+    finally:
+        for sim, mode in zip(sim_list, modes):
+            sim.model.train(mode)
+    for sim in sim_list:
+        sim.compute_layer_encodings_for_sim()

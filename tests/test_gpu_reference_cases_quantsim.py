@@ -1,0 +1,489 @@
+"""Cases of the reference's simulation-model tests (TrainingExtensions/torch/test/python/test_quantizer.py and
+test_percentile_quantization_scheme.py) that exercise the quantize-dequantize / calibration path, with the same models,
+inputs and assertions, on GPU tensors.  Cases about ONNX / TorchScript export, recurrent layers and the model preparer
+belong to parts of the reference that are not rebuilt and are left out.
+"""
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+pytestmark = pytest.mark.gpu
+
+from aimet_amd.common import libpymo                                                        # noqa: E402
+from aimet_amd.common.defs import QuantizationDataType, QuantScheme                         # noqa: E402
+from aimet_amd.v1.nn.modules import custom as aimet_modules                                 # noqa: E402
+from aimet_amd.v1.qc_quantize_op import (LearnedGridQuantWrapper, QcQuantizeOpMode, QcQuantizeWrapper,  # noqa: E402
+                                         StaticGridQuantWrapper)
+from aimet_amd.v1.quantsim import QuantizationSimModel, compute_encodings_for_sims, has_valid_encodings  # noqa: E402
+from aimet_amd.v1.quantsim_straight_through_grad import compute_dloss_by_dx                 # noqa: E402
+
+
+def evaluate(model, dummy_input):
+    model.eval()
+    if isinstance(dummy_input, torch.Tensor):
+        dummy_input = [dummy_input]
+    with torch.no_grad():
+        model(*dummy_input)
+
+
+def dummy_forward_pass(model, _):
+    model.eval()
+    with torch.no_grad():
+        return model(torch.randn((32, 1, 28, 28)).cuda())
+
+
+class SmallMnist(nn.Module):                        # test_quantizer.py:136-158
+    def __init__(self):
+        super().__init__()
+        self.conv1, self.relu1 = nn.Conv2d(1, 10, kernel_size=5), nn.ReLU()
+        self.conv2, self.conv2_drop, self.relu2 = nn.Conv2d(10, 20, kernel_size=5), nn.Dropout2d(), nn.ReLU()
+        self.fc1, self.relu3, self.dropout = nn.Linear(320, 50), nn.ReLU(), nn.Dropout()
+        self.fc2, self.log_softmax = nn.Linear(50, 10), nn.LogSoftmax(dim=1)
+
+    def forward(self, x):
+        x = self.relu1(self.conv1(x))
+        x = self.relu2(self.conv2_drop(self.conv2(x)))
+        x = self.relu3(self.fc1(x.view(-1, 320)))
+        return self.log_softmax(self.fc2(self.dropout(x)))
+
+
+class ModelWithTwoInputsOneToAdd(nn.Module):        # test_quantizer.py:225-261
+    def __init__(self):
+        super().__init__()
+        self.conv1_a, self.maxpool1_a, self.relu1_a = nn.Conv2d(1, 10, kernel_size=5), nn.MaxPool2d(2), nn.ReLU()
+        self.conv1_b, self.maxpool1_b, self.relu1_b = nn.Conv2d(10, 10, kernel_size=5), nn.MaxPool2d(2), nn.ReLU()
+        self.add = aimet_modules.Add()
+        self.conv2, self.maxpool2, self.relu2 = nn.Conv2d(10, 20, kernel_size=5), nn.MaxPool2d(2), nn.ReLU()
+        self.fc1, self.relu3, self.dropout = nn.Linear(320, 50), nn.ReLU(), nn.Dropout()
+        self.fc2, self.softmax = nn.Linear(50, 10), nn.LogSoftmax(dim=1)
+
+    def forward(self, x1, x2):
+        x1 = self.relu1_a(self.maxpool1_a(self.conv1_a(x1)))
+        x1 = self.relu1_b(self.maxpool1_b(self.conv1_b(x1)))
+        x = self.add(x1, x2)
+        x = self.relu2(self.maxpool2(self.conv2(x)))
+        x = self.relu3(self.fc1(x.view(-1, 320)))
+        return self.softmax(self.fc2(self.dropout(x)))
+
+
+class ConvReluModel(nn.Module):                     # test_quantizer.py:335-342
+    def __init__(self):
+        super().__init__()
+        self.conv, self.relu = nn.Conv2d(3, 5, kernel_size=2, bias=False), nn.ReLU()
+
+    def forward(self, inputs):
+        return self.relu(self.conv(inputs))
+
+
+class _TwoConvs(nn.Module):
+    def __init__(self, c_in, c_mid, c_out, k, **kw):
+        super().__init__()
+        self.conv1, self.conv2 = nn.Conv2d(c_in, c_mid, k, **kw), nn.Conv2d(c_mid, c_out, k, **kw)
+
+    def forward(self, *inputs):
+        return self.conv2(self.conv1(inputs[0]))
+
+
+# ------------------------------------------------------------------------------------- straight-through gradient
+@pytest.mark.parametrize("per_channel", [True, False])
+def test_ste_gradient_math(per_channel):            # :1693-1777
+    c_enc_min, c_enc_max = ([-0.25, -0.25], [1.0, 1.0]) if per_channel else (-0.25, 1.0)
+    grad = torch.Tensor([[1.0, 1.0], [1.0, 1.0]]).cuda()
+    cases = [([[1.0, 1.5], [0.125, -0.12]], [[1.0, 0.0], [1.0, 1.0]]),         # input > max
+             ([[1.0, 0.5], [0.125, -0.30]], [[1.0, 1.0], [1.0, 0.0]]),         # input < min
+             ([[1.0, 0.5], [0.125, -0.25]], [[1.0, 1.0], [1.0, 1.0]])]         # valid input range
+    for custom_input, expected in cases:
+        out = compute_dloss_by_dx(torch.Tensor(custom_input).cuda(), grad, c_enc_min, c_enc_max)
+        assert torch.allclose(torch.Tensor(expected).cuda(), out)
+
+
+# ----------------------------------------------------------------------------------------------- static grid sim
+@pytest.mark.parametrize("scheme, shape", [(QuantScheme.post_training_tf_enhanced, (1, 1, 12, 12)),
+                                           (QuantScheme.post_training_tf, (1, 1, 28, 28))])
+def test_no_fine_tuning(scheme, shape):             # :1072-1085, :1567-1576
+    # the reference traces with a 12x12 input although the model needs 28x28 (its tracer tolerates the failure);
+    # the wrappers only depend on the module list, so the 28x28 input is used for both
+    sim = QuantizationSimModel(SmallMnist().cuda(), quant_scheme=scheme, dummy_input=torch.rand(1, 1, 28, 28).cuda())
+    assert isinstance(sim.model.conv1, QcQuantizeWrapper)
+    sim.compute_encodings(dummy_forward_pass, None)
+    dummy_forward_pass(sim.model, None)
+
+
+def test_input_quantization():                      # :1141-1163
+    sim = QuantizationSimModel(SmallMnist().cuda(), quant_scheme=QuantScheme.post_training_tf,
+                               dummy_input=torch.rand(1, 1, 28, 28).cuda())
+    for module in sim.model.modules():
+        if isinstance(module, QcQuantizeWrapper):
+            module.output_quantizers[0].enabled = False
+            module.input_quantizers[0].enabled = True
+    sim.compute_encodings(dummy_forward_pass, None)
+    dummy_forward_pass(sim.model, None)
+    assert not sim.model.conv1.output_quantizers[0].encoding
+    assert sim.model.conv1.input_quantizers[0].encoding
+    assert str(sim.model.conv1.input_quantizers[0]) and str(sim.model.conv1.output_quantizers[0])
+
+
+def test_per_layer_bitwidths():                     # :1578-1594
+    sim = QuantizationSimModel(SmallMnist().cuda(), quant_scheme=QuantScheme.post_training_tf,
+                               dummy_input=torch.rand(1, 1, 28, 28).cuda())
+    sim.model.conv1.set_output_bw(16)
+    sim.compute_encodings(dummy_forward_pass, None)
+    dummy_forward_pass(sim.model, None)
+    assert sim.model.conv1.output_quantizers[0].bitwidth == 16
+    assert sim.model.conv2.output_quantizers[0].bitwidth == 8
+
+
+def test_changing_param_quantizer_settings():       # :1779-1815
+    torch.random.manual_seed(10)
+    model = SmallMnist().cuda()
+    old_weight = model.conv1.weight.detach().clone()                # skew the weights of conv1
+    model.conv1.weight = nn.Parameter(old_weight + .5 * torch.abs(torch.min(old_weight)), requires_grad=False)
+    sim = QuantizationSimModel(model, dummy_input=torch.rand(1, 1, 28, 28).cuda())
+    weight_quantizer = sim.model.conv1.param_quantizers['weight']
+    assert not weight_quantizer.encoding
+    sim.compute_encodings(dummy_forward_pass, None)
+    asym_min, asym_max = weight_quantizer.encoding.min, weight_quantizer.encoding.max
+    assert weight_quantizer.encoding.bw == 8
+    assert weight_quantizer.encoding.offset == -128.0               # symmetric by default
+    weight_quantizer.use_symmetric_encodings = False
+    weight_quantizer.bitwidth = 4
+    sim.compute_encodings(dummy_forward_pass, None)
+    sym_min, sym_max = weight_quantizer.encoding.min, weight_quantizer.encoding.max
+    assert weight_quantizer.encoding.bw == 4
+    assert weight_quantizer.encoding.offset not in [-127, -128]
+    assert not np.allclose(asym_min, sym_min)
+    assert not np.allclose(asym_max, sym_max)
+
+
+def test_compute_encodings_on_subset_of_modules():  # :1817-1835
+    def forward_pass(model, _):
+        model.relu1(model.conv1(torch.randn((1, 1, 28, 28)).cuda()))
+
+    sim = QuantizationSimModel(SmallMnist().cuda().eval(), dummy_input=torch.rand(1, 1, 28, 28).cuda())
+    sim.compute_encodings(forward_pass, None)
+    for name, module in sim.model.named_modules():
+        if isinstance(module, StaticGridQuantWrapper):
+            assert module._mode == QcQuantizeOpMode.ACTIVE
+            if name == 'relu1':
+                assert module.output_quantizers[0].enabled
+            elif name in ['conv2', 'conv2_drop', 'relu2', 'relu3', 'dropout', 'fc2', 'log_softmax']:
+                assert not module.output_quantizers[0].enabled
+
+
+def test_change_quant_scheme_tf_enhanced_to_tf():   # :2146-2185
+    dummy_input = torch.rand(1, 10, 24, 24).cuda()
+    sim = QuantizationSimModel(_TwoConvs(10, 10, 20, 5).cuda(), dummy_input)
+    sim.compute_encodings(evaluate, dummy_input)
+    quantizer = sim.model.conv2.output_quantizers[0]
+    assert quantizer.quant_scheme == QuantScheme.post_training_tf_enhanced
+
+    def calibrate_with_outlier():
+        tensor = torch.rand(1, 10, 24, 24).cuda()
+        quantizer.reset_encoding_stats()
+        quantizer.update_encoding_stats(tensor)
+        tensor[0, 0, 0, 0] = 1000
+        quantizer.update_encoding_stats(tensor)
+        quantizer.compute_encoding()
+
+    calibrate_with_outlier()
+    assert quantizer.encoding.max < 1.0
+    quantizer.quant_scheme = QuantScheme.post_training_tf
+    calibrate_with_outlier()
+    assert quantizer.encoding.max == pytest.approx(1000.0, rel=0.1)
+
+
+def test_change_quant_scheme_tf_enhanced_to_tf_per_channel():       # :2187-2237
+    dummy_input = torch.rand(1, 10, 24, 24).cuda()
+    model = _TwoConvs(10, 10, 20, 5).cuda()
+    sim1 = QuantizationSimModel(model, dummy_input)
+    sim1.model.conv2.enable_per_channel_quantization()
+    sim1.compute_encodings(evaluate, dummy_input)
+    quantizer = sim1.model.conv2.param_quantizers['weight']
+    assert quantizer.quant_scheme == QuantScheme.post_training_tf_enhanced
+
+    def calibrate_with_outlier():
+        tensor = torch.rand(20, 10, 5, 5).cuda()
+        quantizer.reset_encoding_stats()
+        quantizer.update_encoding_stats(tensor)
+        tensor[0, 0, 0, 0] = 100
+        quantizer.update_encoding_stats(tensor)
+        quantizer.compute_encoding()
+
+    calibrate_with_outlier()
+    quantizer.quant_scheme = QuantScheme.post_training_tf
+    calibrate_with_outlier()
+    assert quantizer.encoding[0].max == pytest.approx(100.0, rel=0.1)
+
+    # the scheme is set before compute_encodings
+    sim2 = QuantizationSimModel(model, dummy_input)
+    sim2.model.conv2.enable_per_channel_quantization()
+    sim2.model.conv2.param_quantizers['weight'].quant_scheme = QuantScheme.post_training_tf
+    tensor = torch.rand(20, 10, 5, 5).cuda()
+    tensor[0, 0, 0, 0] = 100
+    sim2.model.conv2._module_to_wrap.weight.data = tensor
+    sim2.compute_encodings(evaluate, dummy_input)
+    assert sim2.model.conv2.param_quantizers['weight'].encoding[0].max == pytest.approx(100.0, rel=0.1)
+
+
+def test_has_valid_encodings():                     # :2358-2384
+    class Model(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.relu1, self.conv, self.relu2 = nn.ReLU(), nn.Conv2d(3, 8, (2, 2)), nn.ReLU()
+            self.unused_module = nn.PReLU()
+
+        def forward(self, *inputs):
+            return self.relu2(self.conv(self.relu1(inputs[0])))
+
+    qsim = QuantizationSimModel(Model().cuda().eval(), dummy_input=torch.randn(1, 3, 8, 8).cuda())
+    modules = [qsim.model.relu1, qsim.model.conv, qsim.model.relu2, qsim.model.unused_module]
+    for m in modules:
+        assert not has_valid_encodings(m)
+    qsim.compute_encodings(lambda m, _: m(torch.randn(1, 3, 8, 8).cuda()), None)
+    for m in modules:
+        assert has_valid_encodings(m) == (m is not qsim.model.unused_module)
+
+
+def test_compute_encodings_for_multiple_sims():     # :2651-2691
+    class SecondModel(nn.Module):
+        def __init__(self, const_inp_shape):
+            super().__init__()
+            self.add, self.sub = aimet_modules.Add(), aimet_modules.Subtract()
+            self.batchnorm = nn.BatchNorm1d(10)
+            self.const_tensor = torch.randn(const_inp_shape).cuda()
+
+        def forward(self, inp, inp2):
+            return self.sub(self.batchnorm(self.add(inp, self.const_tensor)), inp2)
+
+    model = ModelWithTwoInputsOneToAdd().cuda().eval()
+    dummy_input = (torch.rand(32, 1, 100, 100).cuda(), torch.rand(32, 10, 22, 22).cuda())
+    model_1_out = model(*dummy_input)
+    model_2 = SecondModel(model_1_out.shape).cuda().eval()
+    dummy_input_2 = torch.randn(model_1_out.shape).cuda()
+    sim1 = QuantizationSimModel(model, dummy_input)
+    sim2 = QuantizationSimModel(model_2, (dummy_input_2, dummy_input_2))
+
+    def forward_pass_callback(model_list, _):
+        return model_list[1](model_list[0](*dummy_input), dummy_input_2)
+
+    sim2.model.train()
+    running_mean = sim2.model.batchnorm.running_mean.clone().detach()
+    compute_encodings_for_sims([sim1, sim2], forward_pass_callback, None)
+    # sim2 ran in eval mode during the calibration and is back in training mode afterwards
+    assert sim2.model.training
+    assert torch.equal(running_mean, sim2.model.batchnorm.running_mean)
+    assert sim1.model.conv1_a.output_quantizers[0].encoding is not None
+    assert sim2.model.add.input_quantizers[0].encoding is not None
+    assert sim2.model.add.input_quantizers[1].encoding is not None
+
+
+def test_model_with_percentile_scheme():            # test_percentile_quantization_scheme.py:45-95
+    model = _TwoConvs(3, 16, 16, 3, padding="same").cuda()
+    dummy_input = torch.rand(1, 3, 224, 224).cuda()
+    sim = QuantizationSimModel(model, dummy_input, quant_scheme="percentile")
+    sim.set_percentile_value(99.99)
+    sim.compute_encodings(evaluate, dummy_input)
+    tensor = torch.rand(1, 3, 224, 224).cuda()
+
+    def recalibrate(layer, percentile):
+        layer.output_quantizers[0].reset_encoding_stats()
+        layer.output_quantizers[0].update_encoding_stats(tensor)
+        layer.set_percentile_value(percentile)
+        layer.output_quantizers[0].compute_encoding()
+        return layer.output_quantizers[0].encoding
+
+    enc1, enc2 = recalibrate(sim.model.conv1, 99.999), recalibrate(sim.model.conv2, 99.999)
+    assert enc1.max == enc2.max and enc1.delta == enc2.delta
+    enc1, enc2 = recalibrate(sim.model.conv1, 99), recalibrate(sim.model.conv2, 99.999)
+    assert enc1.max != enc2.max and enc1.delta != enc2.delta
+
+
+# ---------------------------------------------------------------------------------------------- learned grid sim
+def test_set_and_get_encoding_properties():         # :3429-3454
+    torch.manual_seed(0)
+    conv1 = nn.Conv2d(1, 32, kernel_size=5).cuda()
+    trainable_module = LearnedGridQuantWrapper(conv1, round_mode='nearest',
+                                               quant_scheme=QuantScheme.training_range_learning_with_tf_init,
+                                               is_symmetric=False, is_output_quantized=True, activation_bw=8,
+                                               weight_bw=8, device='cuda', data_type=QuantizationDataType.int)
+    trainable_module.input_quantizers[0].enabled = True
+    encodings = libpymo.TfEncoding()
+    encodings.bw, encodings.max, encodings.min, encodings.delta, encodings.offset = 8, 5, -5, 1, 0.2
+    with pytest.raises(RuntimeError):               # an enabled quantizer cannot lose its encoding
+        trainable_module.input_quantizers[0].encoding = None
+    trainable_module.input_quantizers[0].encoding = encodings
+    assert trainable_module.input_quantizers[0].encoding is not None
+    assert np.allclose(trainable_module.input0_encoding_min.detach().cpu().numpy(), encodings.min)
+
+
+def test_get_effective_encoding():                  # :3314-3366
+    torch.manual_seed(42)
+    model = ModelWithTwoInputsOneToAdd().cuda()
+    dummy_input = (torch.rand(32, 1, 100, 100).cuda(), torch.rand(32, 10, 22, 22).cuda())
+    sim = QuantizationSimModel(model, dummy_input=dummy_input,
+                               quant_scheme=QuantScheme.training_range_learning_with_tf_init)
+    sim.compute_encodings(evaluate, dummy_input)
+    optimizer = torch.optim.SGD(sim.model.parameters(), lr=0.005, momentum=0.5)
+    for _ in range(20):
+        inputs = (torch.rand(32, 1, 100, 100).cuda(), torch.rand(32, 10, 22, 22).cuda())
+        sim.model(*inputs).flatten().sum().backward()
+        optimizer.step()
+        optimizer.zero_grad()
+    for module_name in ["conv1_a", "maxpool1_a", "relu1_a", "conv1_b", "maxpool1_b", "relu1_b", "add", "conv2",
+                        "maxpool2", "relu2", "fc1", "relu3", "dropout", "fc2"]:
+        wrapper = getattr(sim.model, module_name)
+        for quantizer in list(wrapper.output_quantizers) + list(wrapper.param_quantizers.values()):
+            if not quantizer.enabled:
+                continue
+            encoding = quantizer.get_effective_encoding()
+            assert np.isclose(encoding.min, encoding.delta * encoding.offset, atol=1e-5)
+            assert np.isclose(encoding.max, encoding.min + encoding.delta * 255, atol=1e-5)
+
+
+@pytest.mark.parametrize("quant_scheme", [QuantScheme.post_training_tf_enhanced,
+                                          QuantScheme.training_range_learning_with_tf_enhanced_init])
+@pytest.mark.parametrize("inplace_op", ["relu", "add"])
+def test_inplace_modification(quant_scheme, inplace_op):            # :3954-4031
+    class ModelWithInPlaceOp(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv1 = nn.Conv2d(3, 4, kernel_size=2, stride=2, padding=2, bias=False)
+            if inplace_op == "relu":
+                self.relu = nn.ReLU(inplace=True)
+
+        def forward(self, *inputs):
+            x = self.conv1(inputs[0])
+            if inplace_op == "relu":
+                return self.relu(x)
+            x += 1
+            return x
+
+    dummy_input = torch.randn(1, 3, 8, 8).cuda()
+    model = ModelWithInPlaceOp().cuda().train()     # in-place ops are problematic only during training
+    quant_sim = QuantizationSimModel(model, dummy_input, quant_scheme=quant_scheme, default_param_bw=4,
+                                     default_output_bw=4)
+    quant_sim.compute_encodings(evaluate, dummy_input)
+    optimizer = torch.optim.SGD(quant_sim.model.parameters(), lr=0.001, momentum=0.5)
+    quant_sim.model.train()
+    quant_sim.model(dummy_input).flatten().sum().backward()         # must not raise
+    optimizer.step()
+    optimizer.zero_grad()
+
+
+def test_gradient_accumulation():                   # :4599-4646
+    quantsim_config = {
+        "defaults": {"ops": {"is_output_quantized": "True", "is_symmetric": "True"},
+                     "params": {"is_quantized": "True", "is_symmetric": "True"},
+                     "strict_symmetric": "False", "unsigned_symmetric": "True", "per_channel_quantization": "True"},
+        "params": {}, "op_type": {}, "supergroups": [], "model_input": {}, "model_output": {}}
+    dummy_input = torch.rand(16, 3, 28, 28).cuda()
+    sim = QuantizationSimModel(ConvReluModel().cuda(), dummy_input=dummy_input,
+                               quant_scheme=QuantScheme.training_range_learning_with_tf_init,
+                               config_file=quantsim_config)
+    sim.compute_encodings(evaluate, dummy_input)
+    inputs = torch.rand(32, 3, 28, 28).cuda()
+    grads = None
+    for i in range(20):
+        sim.model(inputs).flatten().sum().backward()
+        if grads is None:
+            grads = {name: param.grad.clone() for name, param in sim.model.named_parameters()}
+        for name, param in sim.model.named_parameters():
+            assert torch.allclose(param.grad, grads[name] * (i + 1)), name
+
+
+# ------------------------------------------------------------------------- constants, pass-through, unused modules
+def test_inputs_shared_constant_intermediate_quantization():        # :1165-1196 (model :424-444)
+    class Model(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.add1, self.add2, self.mul = aimet_modules.Add(), aimet_modules.Add(), aimet_modules.Multiply()
+            self.register_buffer('tensor1', torch.tensor([2.0]))
+            self.relu1, self.relu2, self.relu3 = nn.ReLU(), nn.ReLU(), nn.ReLU()
+
+        def forward(self, a, b, c):
+            x = self.add1(a, torch.tensor([2.0], device=a.device))
+            y = self.add2(self.tensor1, b)
+            z = self.mul(c, x)
+            return self.relu1(x), self.relu2(y), self.relu3(z)
+
+    dummy_input = tuple(torch.randn(1, 10, 10, 10).cuda() for _ in range(3))
+    sim = QuantizationSimModel(Model().cuda(), dummy_input=dummy_input)
+    sim.compute_encodings(lambda m, _: m(*dummy_input), None)
+    # mul's first input is a model input (quantized), its second an intermediate value (not quantized)
+    assert sim.model.mul.input_quantizers[0].enabled
+    assert not sim.model.mul.input_quantizers[1].enabled
+    assert not sim.model.add1.input_quantizers[0].is_const
+    assert sim.model.add1.input_quantizers[1].is_const
+    assert sim.model.add2.input_quantizers[0].is_const
+    assert not sim.model.add2.input_quantizers[1].is_const
+    activation_encodings = sim.get_encodings_dict()['activation_encodings']
+    assert 'input' in activation_encodings['add1'] and 'input' in activation_encodings['add2']
+    assert 'input' in activation_encodings['mul']
+
+
+def test_constant_quantization():                   # :1198-1220 (model :464-479)
+    class Model(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.relu = nn.ReLU()
+            self.add, self.add2, self.add3 = aimet_modules.Add(), aimet_modules.Add(), aimet_modules.Add()
+            self.tensor1 = 1.0
+            self.register_buffer('tensor2', torch.tensor([2.0]))
+
+        def forward(self, inp):
+            x = self.relu(inp)
+            x = self.add(x, self.tensor1)
+            x = self.add2(self.tensor2, x)
+            return self.add3(x, torch.tensor([1.0, 2.0], device=inp.device))
+
+    dummy_input = torch.rand(1, 2).cuda()
+    sim = QuantizationSimModel(Model().cuda(), dummy_input)
+    assert not sim.model.add.input_quantizers[0].enabled
+    assert sim.model.add.input_quantizers[1].enabled
+    assert sim.model.add2.input_quantizers[0].enabled
+    assert not sim.model.add2.input_quantizers[1].enabled
+    assert not sim.model.add3.input_quantizers[0].enabled
+    assert sim.model.add3.input_quantizers[1].enabled
+    sim.compute_encodings(lambda m, _: m(dummy_input), None)
+    # add and add2 take constants of one element: no statistics, so those quantizers are switched off
+    assert not sim.model.add.input_quantizers[1].enabled
+    assert not sim.model.add2.input_quantizers[0].enabled
+    assert sim.model.add3.input_quantizers[1].enabled
+    encodings = sim.get_encodings_dict()['activation_encodings']
+    # relu: input and output; add, add2: output; add3: constant input and output
+    assert sum(len(tensors) for entry in encodings.values() for tensors in entry.values()) == 6
+
+
+def test_pass_through_modules_are_transparent():    # model :112-133, supergroups of the default configuration
+    class Model(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv1, self.pt1, self.relu1 = nn.Conv2d(1, 10, kernel_size=5), nn.Identity(), nn.ReLU()
+
+        def forward(self, x):
+            return self.relu1(self.pt1(self.conv1(x)))
+
+    sim = QuantizationSimModel(Model().cuda(), dummy_input=torch.rand(1, 1, 28, 28).cuda())
+    assert isinstance(sim.model.pt1, nn.Identity)                   # never wrapped (reference :205-207)
+    assert not sim.model.conv1.output_quantizers[0].enabled         # conv + relu is still one supergroup
+    assert sim.model.relu1.output_quantizers[0].enabled
+
+
+@pytest.mark.parametrize("quant_scheme", [QuantScheme.post_training_tf_enhanced,
+                                          QuantScheme.training_range_learning_with_tf_init])
+def test_unused_module_handling(quant_scheme):      # :4186-4210
+    class SimpleModel(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv1 = nn.Conv2d(3, 3, kernel_size=2, stride=2, padding=2, bias=False)
+            self.conv2 = nn.Conv2d(3, 3, kernel_size=2, stride=2, padding=2, bias=False)      # never called
+
+        def forward(self, inputs):
+            return self.conv1(inputs)
+
+    dummy_input = torch.randn(1, 3, 10, 10).cuda()
+    quant_sim = QuantizationSimModel(SimpleModel().cuda().eval(), dummy_input=dummy_input, quant_scheme=quant_scheme)
+    assert isinstance(quant_sim.model.conv2, QcQuantizeWrapper)
+    quant_sim.compute_encodings(evaluate, dummy_input)
+    quant_sim.model(dummy_input).sum().backward()                   # forward and backward finish without error
