@@ -84,6 +84,14 @@ _INIT_SCHEME = {
 
 
 _CONSTANT = "__constant__"     # source of a module input that does not depend on the model's inputs
+# torch functions, tensor methods and operators that the reference's connected graph lists as Add / Mul / Div / Concat
+_ELEMENTWISE_FUNCTIONS = {
+    **dict.fromkeys(('add', 'add_', '__add__', '__radd__', '__iadd__'), 'Add'),
+    **dict.fromkeys(('mul', 'mul_', 'multiply', 'multiply_', '__mul__', '__rmul__', '__imul__'), 'Mul'),
+    **dict.fromkeys(('div', 'div_', 'divide', 'divide_', 'true_divide', 'true_divide_', '__truediv__',
+                     '__rtruediv__', '__itruediv__'), 'Div'),
+    **dict.fromkeys(('cat', 'concat', 'concatenate'), 'Concat'),
+}
 _FLOAT16_ENTRY = object()     # marks a float16 quantizer in the export: it has no encoding, only a type
 
 
@@ -159,7 +167,10 @@ class QuantizationSimModel:
         that a functional op computed from the model's inputs (producer unknown: None), or a constant -- a tensor
         that does not depend on the model's inputs (a buffer, a tensor created in forward) or a python number.
         Constants are told from intermediates by following, through every torch function called during the pass,
-        which tensors derive from the model's inputs.
+        which tensors derive from the model's inputs.  The same watch names the results of the element-wise
+        operations that the reference's configurator treats as ops of their own although no module stands for them
+        (Add, Mul, Div, Concat written as functions or operators; quantsim_config.py:879-885): a module that reads
+        such a result directly gets the source ("__functional__", type).
         """
         records, handles = [], []
         producer: Dict[int, str] = {}
@@ -182,19 +193,33 @@ class QuantizationSimModel:
             producer[id(t)] = "__model_input__"
             derived.add(id(t))
 
+        functional: Dict[int, str] = {}           # id of a derived tensor -> type of the functional op it came from
+
         class Follow(torch.overrides.TorchFunctionMode):
             def __torch_function__(self, func, types, args=(), kwargs=None):
                 out = func(*args, **(kwargs or {}))
                 if any(id(t) in derived for t in tensors_in((args, kwargs or {}))):
+                    fname = getattr(func, '__name__', None) or ''
+                    op_type = _ELEMENTWISE_FUNCTIONS.get(fname)
+                    in_place = (fname.endswith('_') and not fname.endswith('__')) or fname.startswith('__i')
                     for t in tensors_in(out):
                         keep_alive.append(t)
                         derived.add(id(t))
+                        if in_place or op_type is not None:
+                            # an in-place operation hands back the tensor it was given: from here on the value is
+                            # this operation's, no longer that of the module which made the tensor
+                            producer.pop(id(t), None)
+                            functional.pop(id(t), None)
+                        if op_type is not None:
+                            functional[id(t)] = op_type
                 return out
 
         def classify(value):
             if isinstance(value, torch.Tensor):
                 if id(value) in producer:
                     return producer[id(value)]
+                if id(value) in functional:
+                    return ("__functional__", functional[id(value)])
                 return None if id(value) in derived else _CONSTANT
             if isinstance(value, (int, float)) and not isinstance(value, bool):
                 return _CONSTANT
@@ -210,12 +235,13 @@ class QuantizationSimModel:
             for src in sources:
                 # resolved now, not afterwards: an in-place op returns the tensor it was given, so the tensor's id
                 # says nothing about who produced the value a later module reads
-                if src is not None and src is not _CONSTANT:
+                if isinstance(src, str) and src is not _CONSTANT:
                     consumers.setdefault(src, []).append(name)
             records.append({"name": name, "module": module, "type": _op_type(module), "inputs": sources,
                             "num_inputs": max(1, len(inputs)), "num_outputs": max(1, len(outs))})
             for t in outs:
                 producer[id(t)] = name
+                functional.pop(id(t), None)
                 derived.add(id(t))
 
         for module in model.modules():
@@ -299,6 +325,16 @@ class QuantizationSimModel:
                 w.enable_param_quantizers(False, None)        # BN statistics are never quantized
             if _flag(op_cfg, "per_channel_quantization", per_channel) and w.param_quantizers:
                 w.enable_per_channel_quantization()
+        # results of functional Add / Mul / Div / Concat: their "output quantizer" is the input quantizer of the
+        # modules that read them (reference quantsim_config.py:211-237)
+        for rec in self._graph:
+            for idx, src in enumerate(rec["inputs"]):
+                if isinstance(src, tuple):
+                    setting = _flag(cfg.get("op_type", {}).get(src[1], {}), "is_output_quantized", None)
+                    if setting is not None:
+                        rec["wrapper"].input_quantizers[idx].enabled = setting
+                    elif out_q:
+                        rec["wrapper"].input_quantizers[idx].enabled = True
         # supergroups: inside a matched chain only the last op keeps its output quantizer
         for group in cfg.get("supergroups", []):
             ops_list = group["op_list"]

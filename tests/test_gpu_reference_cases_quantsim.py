@@ -487,3 +487,55 @@ def test_unused_module_handling(quant_scheme):      # :4186-4210
     assert isinstance(quant_sim.model.conv2, QcQuantizeWrapper)
     quant_sim.compute_encodings(evaluate, dummy_input)
     quant_sim.model(dummy_input).sum().backward()                   # forward and backward finish without error
+
+
+# ----------------------------------------------------------------- element-wise operations written as functions
+class _BranchNet(nn.Module):
+    """Net of :1246-1287 (combine='add') and :1523-1564 (combine='cat'), also with mul and div (:1437-1521)."""
+
+    def __init__(self, combine):
+        super().__init__()
+        wide = 10 if combine == 'cat' else 20
+        self.combine = combine
+        self.conv1 = nn.Conv2d(3, 10, kernel_size=5)
+        self.conv2a, self.conv2b = nn.Conv2d(10, wide, kernel_size=5), nn.Conv2d(10, wide, kernel_size=5)
+        self.conv3 = nn.Conv2d(20, 20, kernel_size=5)
+        self.conv4a, self.conv4b = nn.Conv2d(20, wide, kernel_size=5), nn.Conv2d(20, wide, kernel_size=5)
+        self.conv5 = nn.Conv2d(20, 20, kernel_size=5)
+
+    def _join(self, ya, yb):
+        return {'add': lambda: ya + yb, 'mul': lambda: ya * yb, 'div': lambda: ya / yb,
+                'cat': lambda: torch.cat((ya, yb), 1), 'iadd': lambda: ya.add_(yb)}[self.combine]()
+
+    def forward(self, inp):
+        x = self.conv1(inp)
+        x = self.conv3(self._join(self.conv2a(x), self.conv2b(x)))
+        return self.conv5(self._join(self.conv4a(x), self.conv4b(x)))
+
+
+@pytest.mark.parametrize("combine", ['add', 'mul', 'div', 'cat', 'iadd'])
+def test_quantizing_models_with_functional_ops(combine):
+    sim = QuantizationSimModel(_BranchNet(combine).cuda(), quant_scheme=QuantScheme.post_training_tf,
+                               dummy_input=torch.rand(1, 3, 28, 28).cuda())
+    assert sim.model.conv3.input_quantizers[0].enabled
+    assert sim.model.conv5.input_quantizers[0].enabled
+    assert not sim.model.conv2a.input_quantizers[0].enabled         # fed by a module: no input quantizer
+    assert str(sim)
+    sim.compute_encodings(lambda m, _: m(torch.rand(2, 3, 28, 28).cuda()), None)
+    assert sim.model.conv3.input_quantizers[0].encoding is not None
+
+
+def test_functional_op_setting_of_the_configuration():
+    config = {"defaults": {"ops": {"is_output_quantized": "True"}, "params": {"is_quantized": "True"}},
+              "params": {}, "op_type": {"Add": {"is_output_quantized": "False"}}, "supergroups": [],
+              "model_input": {"is_input_quantized": "True"}, "model_output": {}}
+    sim = QuantizationSimModel(_BranchNet('add').cuda(), dummy_input=torch.rand(1, 3, 28, 28).cuda(),
+                               config_file=config)
+    assert not sim.model.conv3.input_quantizers[0].enabled
+    assert sim.model.conv1.input_quantizers[0].enabled
+
+
+def test_reshape_between_modules_is_no_constant():
+    sim = QuantizationSimModel(SmallMnist().cuda(), dummy_input=torch.rand(1, 1, 28, 28).cuda())
+    assert not sim.model.fc1.input_quantizers[0].enabled            # x.view(-1, 320) derives from the input
+    assert not sim.model.fc1.input_quantizers[0].is_const
