@@ -581,6 +581,17 @@ class QuantizationSimModel:
         self.load_encodings(encodings, strict=True, partial=True, requires_grad=False, allow_overwrite=False)
 
 
+def load_encodings_to_sim(quant_sim_model: QuantizationSimModel, pytorch_encoding_path: str):
+    """Loads an exported encodings file into a simulation model configured like the one that wrote it: wrappers go to
+    ACTIVE mode, every quantizer the file has no entry for is switched off, and range-learning models get their
+    learned-grid wrappers (reference quantsim.py:2277-2298)."""
+    for _, wrapper in quant_sim_model.quant_wrappers():
+        wrapper.set_mode(QcQuantizeOpMode.ACTIVE)
+    quant_sim_model.load_encodings(pytorch_encoding_path, strict=True, partial=False, requires_grad=None,
+                                   allow_overwrite=None)
+    quant_sim_model.replace_wrappers_for_quantize_dequantize()
+
+
 def has_valid_encodings(qc_quantize_op: QcQuantizeWrapper) -> bool:
     """True if any enabled input, parameter or output quantizer of the wrapper holds an encoding (or simulates
     float16, which needs none) -- reference quantsim.py:2301-2323."""
