@@ -170,7 +170,7 @@ class QuantizationSimModel:
         which tensors derive from the model's inputs.  The same watch names the results of the element-wise
         operations that the reference's configurator treats as ops of their own although no module stands for them
         (Add, Mul, Div, Concat written as functions or operators; quantsim_config.py:879-885): a module that reads
-        such a result directly gets the source ("__functional__", type).
+        such a result directly gets the source ("__functional__", type, index into self._functional_ops).
         """
         records, handles = [], []
         producer: Dict[int, str] = {}
@@ -193,15 +193,21 @@ class QuantizationSimModel:
             producer[id(t)] = "__model_input__"
             derived.add(id(t))
 
-        functional: Dict[int, str] = {}           # id of a derived tensor -> type of the functional op it came from
+        functional: Dict[int, tuple] = {}         # id of a derived tensor -> source tuple of the functional op
+        functional_ops = self._functional_ops = []    # per functional op: type, modules that made its operands
 
         class Follow(torch.overrides.TorchFunctionMode):
             def __torch_function__(self, func, types, args=(), kwargs=None):
                 out = func(*args, **(kwargs or {}))
                 if any(id(t) in derived for t in tensors_in((args, kwargs or {}))):
                     fname = getattr(func, '__name__', None) or ''
-                    op_type = _ELEMENTWISE_FUNCTIONS.get(fname)
+                    # what a leaf module computes inside belongs to that module
+                    op_type = _ELEMENTWISE_FUNCTIONS.get(fname) if not inside_leaf[0] else None
                     in_place = (fname.endswith('_') and not fname.endswith('__')) or fname.startswith('__i')
+                    if op_type is not None:
+                        operands = [producer.get(id(t)) for t in tensors_in((args, kwargs or {}))]
+                        functional_ops.append({"type": op_type, "producers": [
+                            p for p in operands if p is not None and p != "__model_input__"]})
                     for t in tensors_in(out):
                         keep_alive.append(t)
                         derived.add(id(t))
@@ -211,7 +217,7 @@ class QuantizationSimModel:
                             producer.pop(id(t), None)
                             functional.pop(id(t), None)
                         if op_type is not None:
-                            functional[id(t)] = op_type
+                            functional[id(t)] = ("__functional__", op_type, len(functional_ops) - 1)
                 return out
 
         def classify(value):
@@ -219,13 +225,19 @@ class QuantizationSimModel:
                 if id(value) in producer:
                     return producer[id(value)]
                 if id(value) in functional:
-                    return ("__functional__", functional[id(value)])
+                    return functional[id(value)]
                 return None if id(value) in derived else _CONSTANT
             if isinstance(value, (int, float)) and not isinstance(value, bool):
                 return _CONSTANT
             return None
 
+        inside_leaf = [0]
+
+        def pre_hook(module, inputs):
+            inside_leaf[0] += 1
+
         def hook(module, inputs, output):
+            inside_leaf[0] -= 1
             name = names[module]
             ins = [t for t in inputs if isinstance(t, torch.Tensor)]
             outs = [t for t in (output if isinstance(output, (tuple, list)) else (output,))
@@ -248,6 +260,7 @@ class QuantizationSimModel:
             # nn.Identity is never wrapped (reference :205-207, :1430-1434); unhooked, the tensor it passes through
             # keeps its producer
             if self._is_leaf(module) and module is not model and not isinstance(module, nn.Identity):
+                handles.append(module.register_forward_pre_hook(pre_hook))
                 handles.append(module.register_forward_hook(hook))
         was_training = model.training
         model.eval()
@@ -325,34 +338,93 @@ class QuantizationSimModel:
                 w.enable_param_quantizers(False, None)        # BN statistics are never quantized
             if _flag(op_cfg, "per_channel_quantization", per_channel) and w.param_quantizers:
                 w.enable_per_channel_quantization()
-        # results of functional Add / Mul / Div / Concat: their "output quantizer" is the input quantizer of the
-        # modules that read them (reference quantsim_config.py:211-237)
+        # functional Add / Mul / Div / Concat have no wrapper: their "output quantizer" is the input quantizer of the
+        # modules that read the result, their "input quantizers" are the output quantizers of the modules that made
+        # the operands (reference quantsim_config.py:183-237)
+        functional_readers: Dict[int, list] = {}
         for rec in self._graph:
             for idx, src in enumerate(rec["inputs"]):
                 if isinstance(src, tuple):
+                    functional_readers.setdefault(src[2], []).append(rec)
                     setting = _flag(cfg.get("op_type", {}).get(src[1], {}), "is_output_quantized", None)
                     if setting is not None:
                         rec["wrapper"].input_quantizers[idx].enabled = setting
                     elif out_q:
                         rec["wrapper"].input_quantizers[idx].enabled = True
+        for op in self._functional_ops:
+            setting = _flag(cfg.get("op_type", {}).get(op["type"], {}), "is_input_quantized", None)
+            if setting is None and not in_q:
+                continue
+            for name in op["producers"]:
+                by_name[name]["wrapper"].output_quantizers[0].enabled = True if setting is None else setting
+        # a batch norm that is the only reader of a convolution / linear layer can be folded into it: such batch
+        # norms are skipped when supergroups are matched, and afterwards take over the layer's output quantizer
+        # (reference quantsim_config.py:486-560)
+        def only_consumer(rec):
+            readers = set(rec["consumers"])
+            return by_name[next(iter(readers))] if len(readers) == 1 and not rec["is_model_output"] else None
+
+        foldable = {}                             # batch norm name -> record of the layer it folds into
+        for rec in self._graph:
+            if rec["type"] in ("Conv", "ConvTranspose", "Gemm"):
+                module = rec["module"]
+                if isinstance(module, nn.ConvTranspose2d) and module.groups != 1:
+                    continue
+                reader = only_consumer(rec)
+                if reader is not None and reader["type"] == "BatchNormalization":
+                    foldable[reader["name"]] = rec
+
+        def next_in_chain(rec):
+            reader = only_consumer(rec)
+            while reader is not None and reader["name"] in foldable:
+                reader = only_consumer(reader)
+            return reader
+
         # supergroups: inside a matched chain only the last op keeps its output quantizer
         for group in cfg.get("supergroups", []):
             ops_list = group["op_list"]
             for rec in self._graph:
+                if rec["type"] != ops_list[0] or rec["name"] in foldable:
+                    continue
                 chain, cur = [rec], rec
                 for want in ops_list[1:]:
-                    nxt = [by_name[c] for c in set(cur["consumers"])]
-                    if len(nxt) != 1 or nxt[0]["type"] != want or cur["is_model_output"]:
+                    cur = next_in_chain(cur)
+                    if cur is None or cur["type"] != want:
                         chain = None
                         break
-                    cur = nxt[0]
                     chain.append(cur)
-                if chain is None or rec["type"] != ops_list[0]:
+                if chain is None:
                     continue
                 for member in chain[:-1]:
                     member["wrapper"].enable_output_quantizers(False)
                 for member in chain[1:]:
                     member["wrapper"].enable_input_quantizers(False)
+            # a chain that starts at a functional op: the op itself has nothing to switch off, the modules after it
+            # are treated as inside the chain (reference SupergroupConfigCallback, quantsim_config.py:80-104)
+            for index, readers in functional_readers.items():
+                if self._functional_ops[index]["type"] != ops_list[0] or len(readers) != 1 or len(ops_list) < 2:
+                    continue
+                chain, cur = [], readers[0]
+                for position, want in enumerate(ops_list[1:]):
+                    if position:
+                        cur = next_in_chain(cur)
+                    if cur is None or cur["type"] != want:
+                        chain = None
+                        break
+                    chain.append(cur)
+                if chain is None:
+                    continue
+                for member in chain[:-1]:
+                    member["wrapper"].enable_output_quantizers(False)
+                for member in chain:
+                    member["wrapper"].enable_input_quantizers(False)
+        for bn_name, layer in foldable.items():
+            bn_wrapper, layer_wrapper = by_name[bn_name]["wrapper"], layer["wrapper"]
+            bn_wrapper.enable_input_quantizers(False)
+            bn_wrapper.enable_param_quantizers(False, None)
+            for layer_q, bn_q in zip(layer_wrapper.output_quantizers, bn_wrapper.output_quantizers):
+                bn_q.enabled = layer_q.enabled
+                layer_q.enabled = False
         if _flag(cfg.get("model_input", {}), "is_input_quantized", False):
             for rec in self._graph:
                 # model inputs and constant inputs alike (reference quantsim_config.py:560-581)
