@@ -40,7 +40,9 @@ def test_quantsim_default_configuration():
     assert all(isinstance(x, StaticGridQuantWrapper) for x in w.values())
     assert w["conv1"].input_quantizers[0].enabled and not w["conv2"].input_quantizers[0].enabled
     assert not w["conv1"].output_quantizers[0].enabled and w["relu1"].output_quantizers[0].enabled   # Conv+Relu
-    assert w["conv2"].output_quantizers[0].enabled
+    # conv2 hands its output quantizer to the batch norm that can be folded into it
+    assert not w["conv2"].output_quantizers[0].enabled and w["bn"].output_quantizers[0].enabled
+    assert not w["bn"].input_quantizers[0].enabled
     assert not w["fc"].output_quantizers[0].enabled and w["act"].output_quantizers[0].enabled        # Gemm+Relu
     assert not w["drop"].output_quantizers[0].enabled and not w["flatten"].output_quantizers[0].enabled
     assert w["conv1"].param_quantizers["weight"].enabled and not w["conv1"].param_quantizers["bias"].enabled
