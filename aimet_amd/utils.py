@@ -208,6 +208,23 @@ def create_encoding_dict(encoding, quantizer, propagate_encodings: bool = False)
             'bitwidth': encoding.bw, 'is_symmetric': str(quantizer.use_symmetric_encodings), 'dtype': 'int'}
 
 
+def compute_encoding_for_given_bitwidth(data, bitwidth: int, quant_scheme, is_symmetric: bool, data_type) -> Dict:
+    """Encoding dictionary of `data` (numpy array or tensor; it is analysed on the current GPU) for the given bitwidth,
+    scheme and symmetry; {} when no valid encoding exists (reference aimet_torch/utils.py:803-829)."""
+    # pylint: disable=import-outside-toplevel
+    from .common.AimetTensorQuantizer import AimetTensorQuantizer
+    from .common.defs import MAP_QUANT_SCHEME_TO_PYMO, QuantizationDataType
+    tensor = torch.as_tensor(data, dtype=torch.float32).cuda()
+    analyzer = AimetTensorQuantizer(MAP_QUANT_SCHEME_TO_PYMO[quant_scheme])
+    analyzer.updateStats(tensor, True)
+    encoding, is_encoding_valid = analyzer.getEncoding(bitwidth, is_symmetric, False, False)
+    if not is_encoding_valid:
+        return {}
+    return {'min': encoding.min, 'max': encoding.max, 'scale': encoding.delta, 'offset': encoding.offset,
+            'bitwidth': encoding.bw, 'is_symmetric': str(is_symmetric),
+            'dtype': 'int' if data_type == QuantizationDataType.int else 'float'}
+
+
 def create_encoding_from_dict(encoding_dict: dict):
     """TfEncoding from its dictionary form."""
     from .common import libpymo  # pylint: disable=import-outside-toplevel

@@ -1,5 +1,6 @@
 """The end-to-end cases of the reference's AdaRound tests (TrainingExtensions/torch/test/python/
-test_adaround_weight.py:295-1045) on the GPU path, with the reference's test models."""
+test_adaround_weight.py:295-1045) on the GPU path, with the reference's test models, and the cases of
+test_adaround_optimizer.py / test_adaround_loss.py with the expected numbers those files hold."""
 import json
 import os
 from unittest.mock import patch
@@ -133,6 +134,7 @@ def _params(ada, loader, iterations=5):
 
 def _delta(weight, bw=4):
     from aimet_amd import ops
+    weight = weight.detach()
     return ops.get_computed_encodings(bw, float(weight.min()), float(weight.max()), False, False, False).delta
 
 
@@ -301,3 +303,96 @@ def test_adaround_default_values(ada, tmp_path):
         assert opt_params.num_iterations == want
     with pytest.raises(ValueError):
         ada.AdaroundParameters(data_loader=_loader(), num_batches=5)          # the loader holds 4 batches
+
+
+# ---------------------------------------------------- golden values of the reference's optimizer and loss tests
+def _golden_layer(seed_order):
+    """Weights and data of test_adaround_optimizer.py:122-199, drawn in the same order from numpy's seeded legacy
+    generator, so that the reference's expected numbers apply."""
+    import numpy as np
+    np.random.seed(0)
+    torch.manual_seed(0)
+    weight_data = np.random.rand(4, 4, 1, 1).astype(dtype='float32')
+    conv1 = nn.Conv2d(4, 4, 1, bias=False).cuda()
+    conv1.weight.data = torch.from_numpy(weight_data).cuda()
+    inp_data = torch.from_numpy(np.random.rand(1, 4, 10, 10).astype(dtype='float32')).cuda()
+    out_data = torch.from_numpy(np.random.rand(1, 4, 10, 10).astype(dtype='float32')).cuda()
+    return weight_data, conv1, inp_data, out_data
+
+
+def test_compute_recons_metrics():                  # test_adaround_optimizer.py:122-155
+    from aimet_amd.common.defs import QuantizationDataType, QuantScheme
+    from aimet_amd.utils import compute_encoding_for_given_bitwidth, create_encoding_from_dict
+    from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
+    from aimet_amd.v1.adaround.adaround_wrapper import AdaroundWrapper
+    from aimet_amd.v1.qc_quantize_op import StaticGridQuantWrapper
+    weight_data, conv1, inp_data, out_data = _golden_layer(0)
+    encoding_dict = compute_encoding_for_given_bitwidth(weight_data, 8, QuantScheme.post_training_tf_enhanced, False,
+                                                        QuantizationDataType.int)
+    assert encoding_dict['scale'] == pytest.approx(0.003772232448682189, abs=5e-4)
+    quant_module = StaticGridQuantWrapper(conv1, 8, 8, round_mode='nearest',
+                                          quant_scheme=QuantScheme.post_training_tf_enhanced)
+    quant_module.param_quantizers['weight'].encoding = create_encoding_from_dict(encoding_dict)
+    quant_module = AdaroundWrapper(quant_module)
+    recons_err_hard, recons_err_soft = AdaroundOptimizer._compute_recons_metrics(quant_module, None, inp_data,
+                                                                                 out_data)
+    assert recons_err_hard == pytest.approx(0.610206663608551, abs=5e-4)
+    assert recons_err_soft == pytest.approx(0.6107949018478394, abs=5e-4)
+
+
+def test_compute_output_with_adarounded_weights():  # test_adaround_optimizer.py:157-199
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.adaround.adaround_loss import AdaroundLoss
+    from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
+    from aimet_amd.v1.adaround.adaround_wrapper import AdaroundWrapper
+    from aimet_amd.v1.qc_quantize_op import StaticGridQuantWrapper
+    _, conv1, inp_data, out_tensor = _golden_layer(0)
+    quant_module = StaticGridQuantWrapper(conv1, 8, 8, round_mode='nearest',
+                                          quant_scheme=QuantScheme.post_training_tf_enhanced)
+    quant_module.param_quantizers['weight'].update_encoding_stats(conv1.weight.data)
+    quant_module.param_quantizers['weight'].compute_encoding()
+    quant_module = AdaroundWrapper(quant_module)
+    adaround_out_tensor = AdaroundOptimizer._compute_output_with_adarounded_weights(quant_module, inp_data)
+    mse_loss = torch.nn.functional.mse_loss(adaround_out_tensor, out_tensor)
+    assert float(mse_loss) == pytest.approx(0.6107949, abs=5e-3)
+    recon_loss = AdaroundLoss.compute_recon_loss(adaround_out_tensor, out_tensor)     # squared Frobenius norm
+    assert float(recon_loss) == pytest.approx(2.4431798, abs=5e-3)
+
+
+def test_compute_recon_loss():                      # test_adaround_loss.py:50-74
+    import numpy as np
+    from aimet_amd.v1.adaround.adaround_loss import AdaroundLoss
+    np.random.seed(0)
+    for shape in [(32, 3, 12, 12), (32, 10)]:
+        inp_tensor = torch.from_numpy(np.random.rand(*shape)).cuda()
+        target_tensor = torch.from_numpy(np.random.rand(*shape)).cuda()
+        recons_loss = AdaroundLoss.compute_recon_loss(inp_tensor, target_tensor)
+        expected = torch.nn.functional.mse_loss(inp_tensor, target_tensor, reduction='none').sum(1).mean()
+        assert recons_loss.item() == pytest.approx(expected.item(), abs=1e-5)
+
+
+@pytest.mark.parametrize("warm_start", [1.0, 0.2])  # test_adaround_optimizer.py:62-120
+def test_optimize_layer_rounding(ada, warm_start, tmp_path):
+    from aimet_amd.common import libpymo
+    from aimet_amd.utils import CachedDataset
+    from aimet_amd.v1.adaround.adaround_loss import AdaroundHyperParameters
+    from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
+    from aimet_amd.v1.quantsim import QuantizationSimModel
+    torch.manual_seed(0)
+    model = TinyModel().cuda().eval()
+    sim = QuantizationSimModel(model, dummy_input=torch.randn(1, 3, 32, 32).cuda(), quant_scheme='tf_enhanced',
+                               default_param_bw=4)
+    quantizer = sim.model.conv1.param_quantizers['weight']
+    quantizer.encoding = libpymo.TfEncoding(-127.0 * 0.001551126479, (15 - 127.0) * 0.001551126479, 0.001551126479,
+                                            -127.0, 4)
+    with ada.Adaround._replace_quantization_layer(sim.model, "conv1") as adaround_wrapper:
+        alpha = torch.randn(adaround_wrapper.weight.shape, requires_grad=True, device='cuda')
+        adaround_wrapper.alpha = nn.Parameter(alpha)
+        before_opt = alpha.detach().clone()
+        cached_dataset = CachedDataset(_loader(dataset_size=50, batch_size=10), 5, str(tmp_path))
+        opt_params = AdaroundHyperParameters(num_iterations=10, reg_param=0.01, beta_range=(20, 2),
+                                             warm_start=warm_start)
+        AdaroundOptimizer.adaround_module(model.conv1, adaround_wrapper, model, sim.model, None, cached_dataset,
+                                          _forward_fn, opt_params)
+        # the rounding parameter has moved
+        assert not torch.equal(before_opt, adaround_wrapper.alpha.detach())
