@@ -249,7 +249,10 @@ class QuantizationSimModel:
                 # says nothing about who produced the value a later module reads
                 if isinstance(src, str) and src is not _CONSTANT:
                     consumers.setdefault(src, []).append(name)
+            singleton = [value.numel() == 1 if isinstance(value, torch.Tensor) else src is _CONSTANT
+                         for value, src in zip(inputs, sources)]
             records.append({"name": name, "module": module, "type": _op_type(module), "inputs": sources,
+                            "singleton": singleton,
                             "num_inputs": max(1, len(inputs)), "num_outputs": max(1, len(outs))})
             for t in outs:
                 producer[id(t)] = name
@@ -301,6 +304,7 @@ class QuantizationSimModel:
             rec["wrapper"] = wrapper
             for idx, src in enumerate(rec["inputs"]):
                 wrapper.input_quantizers[idx].is_const = src is _CONSTANT     # reference :1456-1471
+                wrapper.input_quantizers[idx].is_singleton = rec["singleton"][idx]
             parent = self.model
             *path, leaf = rec["name"].split('.')
             for p in path:

@@ -45,6 +45,7 @@ class TensorQuantizer:
         self.enabled = enabled_by_default
         self.data_type = data_type
         self.is_const = False
+        self.is_singleton = False
         self._encoding_min_max_fixed_vals = None
         self._is_encoding_frozen = False
 
@@ -610,6 +611,7 @@ def initialize_learned_grid_quantizer_attributes(new_quantizer: LearnedGridTenso
     new_quantizer.is_unsigned_symmetric = False
     new_quantizer.encoding_min_max_fixed_vals = old_quantizer.encoding_min_max_fixed_vals
     new_quantizer.is_const = old_quantizer.is_const
+    new_quantizer.is_singleton = old_quantizer.is_singleton
     if new_quantizer.data_type == QuantizationDataType.float or new_quantizer.bitwidth == 32:
         new_quantizer.encoding = None
         return

@@ -105,6 +105,8 @@ class QuantizationSimModel:
     def _realize_quantizer(self, q, shape, device):
         if not q.enabled or q.bitwidth == 32:
             return None
+        if q.is_const and q.is_singleton:
+            return None                                                # a constant of one element (builder.py:332)
         if q.use_symmetric_encodings and (q.use_strict_symmetric or q.use_unsigned_symmetric):
             raise NotImplementedError("strict-symmetric and unsigned-symmetric grids are not available in the v2 "
                                       "simulation (the reference's builder asserts the same)")
