@@ -1,0 +1,91 @@
+// Simulation of an 8-bit float grid: every element is rounded to the grid of a float format with `mantissa_bits`
+// mantissa and 7 - mantissa_bits exponent bits whose largest value is the tensor's (or the channel's) maxval
+// (TORCH/fp_quantization.py:133-209, quantize_to_fp8 / fake_cast_to_ieee_float).  A float grid is an integer grid whose
+// step depends on the element's own exponent:
+//   x_c   = clamp(x, -maxval, maxval)
+//   e     = max(floor(log2|x_c| + bias), 1)                    bias = 2^E - log2(maxval) + log2(2 - 2^-M) - 1
+//   step  = 2^(e - M - bias)
+//   y     = round_half_even(x_c / step) * step
+// in float32, one operation at a time and in this order, with the same library log2 / pow as torch's elementwise
+// kernels, so that the result follows the reference's torch expression.  maxval and bias are per channel, on the
+// device; the caller computes bias once per call with the formula above.
+//
+// HBM-bound by design (4 B read + 4 B written per element), but log2f and powf cost about a hundred VALU operations
+// per element, which is what limits the kernel today.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "miq_common.h"
+
+namespace miq
+{
+namespace
+{
+__device__ __forceinline__ float fp8_elem(float x, float mx, float bias, float mant)
+{
+    float xc = x != x ? x : fminf(fmaxf(x, -mx), mx);   // clamp that lets NaN through, as torch.clamp does
+    float e  = fmaxf(floorf(log2f(fabsf(xc)) + bias), 1.0f);
+    float st = powf(2.0f, (e - mant) - bias);
+    return rintf(xc / st) * st;
+}
+
+// Elements are [outer][channels][inner]; a vector of four never straddles a channel when inner % 4 == 0.
+template <bool VEC>
+__global__ void __launch_bounds__(256) fp8_kernel(const float* __restrict__ in, float* __restrict__ out, int64_t n,
+                                                   int64_t channels, int64_t inner, const float* __restrict__ maxval,
+                                                   const float* __restrict__ bias, float mant)
+{
+    const int64_t stride = (int64_t) gridDim.x * blockDim.x;
+    int64_t i            = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (VEC)
+    {
+        const int64_t nv = n >> 2;
+        for (; i < nv; i += stride)
+        {
+            const int64_t c = channels == 1 ? 0 : ((i << 2) / inner) % channels;
+            const float mx = maxval[c], b = bias[c];
+            float4 v = reinterpret_cast<const float4*>(in)[i];
+            v.x      = fp8_elem(v.x, mx, b, mant);
+            v.y      = fp8_elem(v.y, mx, b, mant);
+            v.z      = fp8_elem(v.z, mx, b, mant);
+            v.w      = fp8_elem(v.w, mx, b, mant);
+            reinterpret_cast<float4*>(out)[i] = v;
+        }
+    }
+    else
+    {
+        for (; i < n; i += stride)
+        {
+            const int64_t c = channels == 1 ? 0 : (i / inner) % channels;
+            out[i]          = fp8_elem(in[i], maxval[c], bias[c], mant);
+        }
+    }
+}
+}   // namespace
+}   // namespace miq
+
+extern "C" int miq_fp8_fake_cast_f32(const float* in, float* out, int64_t n, int64_t num_channels, int64_t inner,
+                                     const float* maxval, const float* bias, int mantissa_bits, void* stream)
+{
+    using namespace miq;
+    MIQ_CHECK_ARG(n >= 0 && (n == 0 || (in && out && maxval && bias)), "null tensor pointer or negative count");
+    MIQ_CHECK_ARG(num_channels >= 1 && inner >= 1, "num_channels and inner must be positive");
+    MIQ_CHECK_ARG(n % (num_channels * inner) == 0, "element count is not a multiple of num_channels * inner");
+    MIQ_CHECK_ARG(mantissa_bits >= 1 && mantissa_bits <= 6, "mantissa_bits must be in [1, 6]");
+    if (n == 0)
+        return MIQ_OK;
+    const bool vec = (n % 4 == 0) && (num_channels == 1 || inner % 4 == 0) &&
+                     ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) % 16 == 0);
+    const int64_t work   = vec ? n / 4 : n;
+    const int64_t blocks = (work + 255) / 256;
+    const unsigned grid  = (unsigned) (blocks < 8192 ? blocks : 8192);
+    if (vec)
+        hipLaunchKernelGGL(fp8_kernel<true>, dim3(grid), dim3(256), 0, (hipStream_t) stream, in, out, n, num_channels,
+                           inner, maxval, bias, (float) mantissa_bits);
+    else
+        hipLaunchKernelGGL(fp8_kernel<false>, dim3(grid), dim3(256), 0, (hipStream_t) stream, in, out, n,
+                           num_channels, inner, maxval, bias, (float) mantissa_bits);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}

@@ -6,6 +6,7 @@ only; there is no torch-op fallback: tensors that are not on a GPU are rejected.
 """
 import ctypes as C
 
+
 import torch
 
 from . import _lib
@@ -125,6 +126,42 @@ def fp16_round_trip(x, out=None):
     out = torch.empty_like(x) if out is None else out
     with _OnDevice(x.device):
         check(lib.miq_fp16_round_trip_f32(_ptr(x), _ptr(out), x.numel(), _stream(x)))
+    return out
+
+
+_FP8_LOG2_TOP = {}
+
+
+def fp8_fake_cast(x, maxval, mantissa_bits: int = 3, ch_axis: int = 0, out=None):
+    """Rounds a float32 tensor to the 8-bit float grid (mantissa_bits mantissa, 7 - mantissa_bits exponent bits) whose
+    largest value is `maxval`: a 0-dim / one-element tensor or float for the whole tensor, or a 1-d tensor with one
+    value per channel along `ch_axis` (reference aimet_torch/fp_quantization.py:133-209)."""
+    _require_gpu(x, out)
+    if x.dtype != _F32:
+        raise RuntimeError("fp8_fake_cast takes float32 tensors")
+    x = x.contiguous()
+    maxval = torch.as_tensor(maxval, dtype=_F32, device=x.device).reshape(-1).contiguous()
+    channels = maxval.numel()
+    inner = x.numel()
+    if channels > 1:
+        if x.dim() <= ch_axis or x.shape[ch_axis] != channels:
+            raise RuntimeError(f"maxval has {channels} entries but dimension {ch_axis} of the tensor has "
+                               f"{x.shape[ch_axis] if x.dim() > ch_axis else 'no'} channels")
+        inner = 1
+        for d in x.shape[ch_axis + 1:]:
+            inner *= d
+    # the bias of the format follows from its largest value: maxval = (2 - 2^-M) * 2^(2^E - 1 - bias)
+    exponent_bits = 7 - mantissa_bits
+    key = (x.device, mantissa_bits)
+    if key not in _FP8_LOG2_TOP:
+        # log2(2 - 2^-M) as torch's float32 kernel on this device gives it (read back once)
+        _FP8_LOG2_TOP[key] = float(torch.log2(torch.tensor(2.0 - 2.0 ** (-mantissa_bits), dtype=_F32,
+                                                           device=x.device)))
+    bias = (2.0 ** exponent_bits - torch.log2(maxval) + _FP8_LOG2_TOP[key] - 1.0).contiguous()
+    out = torch.empty_like(x) if out is None else out
+    with _OnDevice(x.device):
+        check(lib.miq_fp8_fake_cast_f32(_ptr(x), _ptr(out), x.numel(), channels, max(inner, 1), _ptr(maxval),
+                                        _ptr(bias), mantissa_bits, _stream(x)))
     return out
 
 

@@ -94,6 +94,15 @@ int miq_qdq_per_tensor_bf16(const uint16_t* in, uint16_t* out, int64_t n, double
  * the reference forms as tensor.half().float() (TORCH/v1/tensor_quantizer.py:1104-1107), in one pass. */
 int miq_fp16_round_trip_f32(const float* in, float* out, int64_t n, void* stream);
 
+/* Quantize-dequantize of the 8-bit float data type (QuantizationDataType.float, bitwidth 8): quantize_to_fp8 /
+ * fake_cast_to_ieee_float (TORCH/fp_quantization.py:133-209, called from TORCH/v1/tensor_quantizer.py:1108-1109).
+ * Elements are laid out [outer][num_channels][inner]; channel c has the largest representable value maxval[c] and
+ * bias[c] = 2^(7-M) - log2(maxval[c]) + log2(2 - 2^-M) - 1 (both device arrays of num_channels floats; per tensor:
+ * num_channels = 1, inner = n).  Per element, in float32 and in this order: x_c = clamp(x, -maxval, maxval);
+ * e = max(floor(log2|x_c| + bias), 1); step = 2^((e - M) - bias); out = rint(x_c / step) * step. */
+int miq_fp8_fake_cast_f32(const float* in, float* out, int64_t n, int64_t num_channels, int64_t inner,
+                          const float* maxval, const float* bias, int mantissa_bits, void* stream);
+
 /* ITensorQuantizationSim<float>::quantizeTensor(..., shiftToSigned) (ITensorQuantizationSim.h:57-59,
  * DLQ/src/TensorQuantizationSim.cpp:116-126; kernel DLQ/src/trim_functions.cu:62-76): float-valued grid indices. */
 int miq_quantize_per_tensor_f32(const float* in, float* out, int64_t n, double enc_min, double enc_max, int bw,

@@ -1,0 +1,89 @@
+"""8-bit float simulation: the HIP kernel against the reference's torch expression (aimet_torch/fp_quantization.py:
+133-209), evaluated by torch in float32 on the same GPU.  Both sides use the device's library log2 / pow, but torch and
+this library are built with different releases of it, so single results may differ in the last bit: the bar is a
+relative error of 1e-6, and the share of bit-identical elements is checked to be overwhelming.
+"""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _reference(x_float, maxval, mantissa_bits, ch_axis=0):
+    """torch float32 statement of the fake cast, op for op."""
+    m = torch.tensor([float(mantissa_bits)], device=x_float.device)
+    exponent_bits = 7 - m
+    if maxval.dim() and maxval.shape[0] != 1:
+        shape = [1] * x_float.dim()
+        shape[ch_axis] = -1
+        maxval = maxval.view(shape)
+    bias = 2 ** exponent_bits - torch.log2(maxval) + torch.log2(2 - 2 ** (-m)) - 1
+    x_clipped = x_float.clamp(-maxval, maxval)
+    log_scales = torch.clamp(torch.floor(torch.log2(torch.abs(x_clipped)) + bias), 1.)
+    scales = 2. ** (log_scales - m - bias)
+    return torch.round(x_clipped / scales) * scales
+
+
+def _check(got, want):
+    assert got.shape == want.shape
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(got), nan)
+    torch.testing.assert_close(got[~nan], want[~nan], rtol=1e-6, atol=0.0)
+    assert (got[~nan] == want[~nan]).float().mean().item() > 0.999
+
+
+@pytest.mark.parametrize("mantissa_bits", [3, 2, 4])
+@pytest.mark.parametrize("shape", [(4096, 1024), (3, 7, 5), (1,), (64, 3, 3, 3)])
+def test_per_tensor(shape, mantissa_bits):
+    from aimet_amd import ops
+    g = torch.Generator(device='cuda').manual_seed(5)
+    x = torch.randn(shape, device='cuda', generator=g) * 3
+    maxval = x.abs().max() * 0.7                      # part of the tensor clips
+    _check(ops.fp8_fake_cast(x, maxval, mantissa_bits), _reference(x, maxval, mantissa_bits))
+
+
+def test_grid_properties():
+    """What the format fixes: at most 2^8 distinct values, symmetric, idempotent, maxval itself representable, zero
+    and the subnormal range on a uniform grid."""
+    from aimet_amd import ops
+    g = torch.Generator(device='cuda').manual_seed(6)
+    x = torch.randn(1 << 20, device='cuda', generator=g) * torch.logspace(-6, 1, 1 << 20, device='cuda')
+    maxval = torch.tensor(7.5, device='cuda')         # 1.875 * 2^2: the grid is the unscaled E4M3-shaped one
+    y = ops.fp8_fake_cast(x, maxval)
+    assert torch.unique(y).numel() <= 256
+    assert torch.equal(ops.fp8_fake_cast(-x, maxval), -y)
+    torch.testing.assert_close(ops.fp8_fake_cast(y, maxval), y, rtol=1e-6, atol=0.0)
+    assert y.abs().max().item() == pytest.approx(7.5, rel=1e-6)
+    assert ops.fp8_fake_cast(torch.zeros(8, device='cuda'), maxval).abs().sum().item() == 0
+    # steps of 2^-1 in [4, 8), 2^-2 in [2, 4), ...; the step itself comes out of pow() and is exact to a few ulp
+    probe = torch.tensor([4.3, 7.4, 2.1, 100.0, -100.0, 1.06], device='cuda')
+    assert ops.fp8_fake_cast(probe, maxval).tolist() == pytest.approx([4.5, 7.5, 2.0, 7.5, -7.5, 1.0], rel=1e-6)
+    small = ops.fp8_fake_cast(torch.linspace(0, 2.0 ** -11, 4097, device='cuda'), maxval)
+    steps = torch.unique(small)
+    assert steps.numel() > 2
+    assert torch.allclose(steps[1:] - steps[:-1], (steps[1] - steps[0]).expand(steps.numel() - 1))
+
+
+@pytest.mark.parametrize("shape, axis", [((16, 8, 3, 3), 0), ((8, 16, 3, 3), 1), ((32, 100), 0), ((5, 7), 1),
+                                         ((6, 4, 8), 1)])
+def test_per_channel(shape, axis):
+    from aimet_amd import ops
+    g = torch.Generator(device='cuda').manual_seed(7)
+    x = torch.randn(shape, device='cuda', generator=g)
+    x = x * torch.logspace(-2, 2, shape[axis], device='cuda').view([-1 if a == axis else 1 for a in range(len(shape))])
+    reduce_dims = [a for a in range(len(shape)) if a != axis]
+    maxval = x.abs().amax(dim=reduce_dims) * 0.9
+    _check(ops.fp8_fake_cast(x, maxval, 3, axis), _reference(x, maxval, 3, axis))
+
+
+def test_special_values_and_errors():
+    from aimet_amd import ops
+    x = torch.tensor([float('nan'), float('inf'), -float('inf'), 0.0, -0.0, 1e-30, -1e-30, 3.0], device='cuda')
+    maxval = torch.tensor(2.0, device='cuda')
+    _check(ops.fp8_fake_cast(x, maxval), _reference(x, maxval, 3))
+    with pytest.raises(RuntimeError):
+        ops.fp8_fake_cast(torch.zeros(4, 4, device='cuda'), torch.ones(3, device='cuda'))
+    with pytest.raises(RuntimeError):
+        ops.fp8_fake_cast(torch.zeros(4), torch.tensor(1.0))
+    with pytest.raises(RuntimeError):
+        ops.fp8_fake_cast(torch.zeros(4, device='cuda'), torch.tensor(1.0, device='cuda'), mantissa_bits=0)
