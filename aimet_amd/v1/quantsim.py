@@ -127,9 +127,10 @@ class QuantizationSimModel:
             raise ValueError('Parameter round mode can only be nearest or stochastic')
         if default_param_bw < 4 or default_param_bw > 32 or default_output_bw < 4 or default_output_bw > 32:
             raise ValueError('Default bitwidth for parameters and activations must be between 4 and 32')
-        if default_data_type == QuantizationDataType.float and (default_output_bw != 16 or default_param_bw != 16):
-            # the reference also takes 8 (an 8-bit float grid, aimet_torch/fp_quantization.py); not built here
-            raise ValueError('float data_type can only be used when default_output_bw and default_param_bw are 16')
+        if default_data_type == QuantizationDataType.float and \
+                (default_output_bw not in (8, 16) or default_param_bw not in (8, 16)):
+            raise ValueError('float data_type can only be used when default_output_bw and default_param_bw are '
+                             '16 (float16) or 8 (8-bit float grid)')
         if default_data_type == QuantizationDataType.float and quant_scheme not in (
                 QuantScheme.post_training_tf, QuantScheme.post_training_tf_enhanced,
                 QuantScheme.post_training_percentile):

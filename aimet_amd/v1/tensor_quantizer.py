@@ -71,12 +71,49 @@ class StaticGridTensorQuantizer(TensorQuantizer):
 
     def __init__(self, bitwidth, round_mode, quant_scheme, use_symmetric_encodings, enabled_by_default,
                  data_type=QuantizationDataType.int):
-        if data_type == QuantizationDataType.float and bitwidth not in (16, 32):
-            # the reference also has an 8-bit float grid (aimet_torch/fp_quantization.py); not built here
-            raise NotImplementedError("the float data type is implemented for bitwidth 16 (float16) only")
+        if data_type == QuantizationDataType.float and bitwidth not in (8, 16, 32):
+            raise ValueError("float data_type only supports bitwidth in {16, 8}")
         super().__init__(bitwidth, round_mode, quant_scheme, use_symmetric_encodings, enabled_by_default, data_type)
         self._cppOp = None
         self._encoding = None
+        self.fp8_maxval = None        # largest value of the 8-bit float grid: 0-dim tensor, or one entry per channel
+
+    # ---- 8-bit float grid (reference tensor_quantizer.py:393-400, :461-468, :544-552; fp_quantization.py:45-122)
+    @property
+    def _is_fp8(self) -> bool:
+        return self.data_type == QuantizationDataType.float and self.bitwidth == 8
+
+    def update_maxval(self, maxval: torch.Tensor):
+        """Running estimate of the grid's largest value: the first observation, then 0.9 old + 0.1 new."""
+        self.fp8_maxval = maxval if self.fp8_maxval is None else 0.9 * self.fp8_maxval + 0.1 * maxval
+
+    def _fp8_observe(self, tensor: torch.Tensor, per_channel: bool):
+        """One calibration step of the 8-bit float grid: the batch's maxval by the rule of the quant scheme (largest
+        magnitude for TF; for TF-Enhanced the candidate among 111 between 0.1 and 1.2 times the largest magnitude
+        with the smallest mean squared error), folded into fp8_maxval, which also becomes the encoding's max."""
+        if self._quant_scheme == QuantScheme.post_training_percentile:
+            raise NotImplementedError("Percentile scheme is not supported for FP8")
+        tensor = tensor.detach().to(torch.float32)
+        axis = self.channel_axis if per_channel else None
+        if per_channel:
+            other = [d for d in range(tensor.dim()) if d != axis]
+            largest = tensor.abs().amax(dim=other) if other else tensor.abs()
+        else:
+            largest = tensor.abs().max()
+        if self._quant_scheme == QuantScheme.post_training_tf:
+            maxval = largest
+        else:
+            fractions = torch.linspace(0.1, 1.2, 111, device=tensor.device)
+            errors = []
+            for fraction in fractions:
+                cast = ops.fp8_fake_cast(tensor, largest * fraction, 3, axis or 0)
+                squared = (tensor - cast) ** 2
+                errors.append(squared.mean(dim=other) if per_channel and other else squared.mean())
+            best = torch.stack(errors).argmin(0)
+            maxval = largest * fractions[best]
+        self.update_maxval(maxval)
+        self._encoding = [libpymo.TfEncoding(-float(m), float(m), 0.0, 0.0, 8)
+                          for m in self.fp8_maxval.reshape(-1).tolist()]
 
     def __str__(self):
         stream = io.StringIO(newline='\n')
@@ -150,7 +187,12 @@ class StaticGridTensorQuantizer(TensorQuantizer):
             self._encoding = []
             self._dev_params = None
             if self.bitwidth == 32 or self.data_type == QuantizationDataType.float:
-                self._encoding = None                   # float16 has no encoding (reference :286-290)
+                # float16 has no encoding (reference :286-290).  The 8-bit float grid is described by fp8_maxval
+                # alone; the encoding keeps [-maxval, maxval] for display (the reference leaves an empty one here)
+                self._encoding = None
+                if self._is_fp8 and self.fp8_maxval is not None:
+                    self._encoding = [libpymo.TfEncoding(-float(m), float(m), 0.0, 0.0, 8)
+                                      for m in self.fp8_maxval.reshape(-1).tolist()]
                 return
             for encoding, valid in self._compute_op_encodings():
                 if not valid:
@@ -220,6 +262,9 @@ class StaticGridPerTensorQuantizer(StaticGridTensorQuantizer):
 
     def update_encoding_stats(self, tensor: torch.Tensor):
         if self.enabled and not self._is_encoding_frozen:
+            if self._is_fp8:
+                self._fp8_observe(tensor, per_channel=False)
+                return
             if self.bitwidth == 32 or self.data_type == QuantizationDataType.float:
                 return
             self._cppOp[0].updateStats(self._stats_tensor(tensor), tensor.is_cuda)
@@ -247,6 +292,9 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
 
     def update_encoding_stats(self, tensor: torch.Tensor):
         if self.enabled and not self._is_encoding_frozen:
+            if self._is_fp8:
+                self._fp8_observe(tensor, per_channel=True)
+                return
             if self.bitwidth == 32 or self.data_type == QuantizationDataType.float:
                 return
             if self.encoding_min_max_fixed_vals is not None:
@@ -334,9 +382,16 @@ class QuantizeDequantize(torch.autograd.Function):
 
     @staticmethod
     def _quantize_float(tensor, tensor_quantizer):
-        """float16 simulation: tensor.half().float() (reference :1104-1113), one fused pass for float32 tensors."""
+        """float16 simulation: tensor.half().float(); 8-bit float simulation: the fake cast to the grid that ends at
+        the quantizer's fp8_maxval (reference :1100-1113), each one fused pass for float32 tensors."""
+        if tensor_quantizer.bitwidth == 8:
+            if tensor_quantizer.fp8_maxval is None:
+                raise ValueError('tensor_quantizer.fp8_maxval not present or not initialized!')
+            out = ops.fp8_fake_cast(tensor.to(torch.float32), tensor_quantizer.fp8_maxval, 3,
+                                    tensor_quantizer.channel_axis or 0)
+            return out.to(tensor.dtype)
         if tensor_quantizer.bitwidth != 16:
-            raise ValueError('float data_type only supports bitwidth 16 here')
+            raise ValueError('float data_type only supports bitwidth in {16, 8}')
         if tensor.dtype == torch.float32 and tensor.is_cuda:
             return ops.fp16_round_trip(tensor)
         return tensor.half().float()

@@ -341,8 +341,8 @@ def test_float16_data_type(api, tmp_path):
     assert torch.equal(xr.grad, torch.full_like(xr, 2.0))
     xb = x[12:1000].bfloat16()
     assert torch.equal(q.quantize_dequantize(xb, api.nearest), xb.half().float())
-    with pytest.raises(NotImplementedError):
-        api.tq.StaticGridPerTensorQuantizer(8, api.nearest, api.QuantScheme.post_training_tf, False, True,
+    with pytest.raises(ValueError):                       # float grids exist for 16 and 8 bits
+        api.tq.StaticGridPerTensorQuantizer(4, api.nearest, api.QuantScheme.post_training_tf, False, True,
                                             data_type=QuantizationDataType.float)
 
     # a wrapper: parameters and output pass through float16
@@ -364,8 +364,9 @@ def test_float16_data_type(api, tmp_path):
     # the simulation model
     model = _Net().eval().cuda()
     dummy = torch.randn(2, 3, 6, 6).cuda()
-    with pytest.raises(ValueError):
-        api.quantsim.QuantizationSimModel(model, dummy_input=dummy, default_data_type=QuantizationDataType.float)
+    with pytest.raises(ValueError):                       # float needs bitwidths 16 or 8
+        api.quantsim.QuantizationSimModel(model, dummy_input=dummy, default_output_bw=4,
+                                          default_data_type=QuantizationDataType.float)
     sim = api.quantsim.QuantizationSimModel(model, dummy_input=dummy, quant_scheme='tf', default_output_bw=16,
                                             default_param_bw=16, default_data_type=QuantizationDataType.float)
     sim.compute_encodings(_calibrate, [torch.randn(4, 3, 6, 6).cuda()])
