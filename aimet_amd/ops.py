@@ -129,18 +129,44 @@ def fp16_round_trip(x, out=None):
     return out
 
 
-_FP8_LOG2_TOP = {}
+def fp8_grid(maxval, mantissa_bits: int = 3):
+    """(maxval, bias, steps) device tensors that describe the 8-bit float grid ending at `maxval` (a float, a one-element
+    tensor, or one value per channel): bias of the format, and for every channel the step 2^((e - M) - bias) of each
+    exponent e = 0 .. 2^E, all in float32 as the reference's expression evaluates them
+    (aimet_torch/fp_quantization.py:171-209).  Reusable for as long as maxval does not change."""
+    if not isinstance(maxval, torch.Tensor) or not maxval.is_cuda:
+        raise RuntimeError("maxval must be a tensor on the GPU")
+    maxval = maxval.detach().to(_F32).reshape(-1).contiguous()
+    key = (maxval.device, mantissa_bits)
+    if key not in _FP8_CONSTANTS:
+        m = torch.tensor([float(mantissa_bits)], dtype=_F32, device=maxval.device)
+        exponents = torch.arange((1 << (7 - mantissa_bits)) + 1, dtype=_F32, device=maxval.device)
+        # 2^E, log2(2 - 2^-M) and e - M, each as torch's float32 kernels on this device give them
+        _FP8_CONSTANTS[key] = (2 ** (7 - m), torch.log2(2 - 2 ** (-m)), exponents - m)
+    two_to_e, log2_top, e_minus_m = _FP8_CONSTANTS[key]
+    # the bias of the format follows from its largest value: maxval = (2 - 2^-M) * 2^(2^E - 1 - bias)
+    bias = (two_to_e - torch.log2(maxval) + log2_top - 1).contiguous()
+    steps = (2. ** (e_minus_m.unsqueeze(0) - bias.unsqueeze(1))).contiguous()
+    return maxval, bias, steps
 
 
-def fp8_fake_cast(x, maxval, mantissa_bits: int = 3, ch_axis: int = 0, out=None):
+_FP8_CONSTANTS = {}
+
+
+def fp8_fake_cast(x, maxval, mantissa_bits: int = 3, ch_axis: int = 0, out=None, grid=None):
     """Rounds a float32 tensor to the 8-bit float grid (mantissa_bits mantissa, 7 - mantissa_bits exponent bits) whose
-    largest value is `maxval`: a 0-dim / one-element tensor or float for the whole tensor, or a 1-d tensor with one
-    value per channel along `ch_axis` (reference aimet_torch/fp_quantization.py:133-209)."""
+    largest value is `maxval`: a one-element tensor or float for the whole tensor, or a 1-d tensor with one value per
+    channel along `ch_axis` (reference aimet_torch/fp_quantization.py:133-209).  `grid` = fp8_grid(maxval,
+    mantissa_bits) computed earlier saves recomputing it."""
     _require_gpu(x, out)
     if x.dtype != _F32:
         raise RuntimeError("fp8_fake_cast takes float32 tensors")
+    if not 1 <= mantissa_bits <= 6:
+        raise RuntimeError("mantissa_bits must be in [1, 6]")
     x = x.contiguous()
-    maxval = torch.as_tensor(maxval, dtype=_F32, device=x.device).reshape(-1).contiguous()
+    if grid is None:
+        grid = fp8_grid(torch.as_tensor(maxval, dtype=_F32, device=x.device), mantissa_bits)
+    maxval, bias, steps = grid
     channels = maxval.numel()
     inner = x.numel()
     if channels > 1:
@@ -150,18 +176,10 @@ def fp8_fake_cast(x, maxval, mantissa_bits: int = 3, ch_axis: int = 0, out=None)
         inner = 1
         for d in x.shape[ch_axis + 1:]:
             inner *= d
-    # the bias of the format follows from its largest value: maxval = (2 - 2^-M) * 2^(2^E - 1 - bias)
-    exponent_bits = 7 - mantissa_bits
-    key = (x.device, mantissa_bits)
-    if key not in _FP8_LOG2_TOP:
-        # log2(2 - 2^-M) as torch's float32 kernel on this device gives it (read back once)
-        _FP8_LOG2_TOP[key] = float(torch.log2(torch.tensor(2.0 - 2.0 ** (-mantissa_bits), dtype=_F32,
-                                                           device=x.device)))
-    bias = (2.0 ** exponent_bits - torch.log2(maxval) + _FP8_LOG2_TOP[key] - 1.0).contiguous()
     out = torch.empty_like(x) if out is None else out
     with _OnDevice(x.device):
         check(lib.miq_fp8_fake_cast_f32(_ptr(x), _ptr(out), x.numel(), channels, max(inner, 1), _ptr(maxval),
-                                        _ptr(bias), mantissa_bits, _stream(x)))
+                                        _ptr(bias), _ptr(steps), mantissa_bits, _stream(x)))
     return out
 
 

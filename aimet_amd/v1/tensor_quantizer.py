@@ -77,6 +77,7 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         self._cppOp = None
         self._encoding = None
         self.fp8_maxval = None        # largest value of the 8-bit float grid: 0-dim tensor, or one entry per channel
+        self._fp8_grid = None         # (maxval, bias, steps) device tensors of that grid, and the maxval they are for
 
     # ---- 8-bit float grid (reference tensor_quantizer.py:393-400, :461-468, :544-552; fp_quantization.py:45-122)
     @property
@@ -133,7 +134,7 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         state['_num_ops'] = len(self._cppOp)
         state['_encoding'] = None if self._encoding is None else \
             [(e.min, e.max, e.delta, e.offset, e.bw) for e in self._encoding]
-        for key in ('_cppOp', '_dev_params'):
+        for key in ('_cppOp', '_dev_params', '_fp8_grid'):
             state.pop(key, None)
         return state
 
@@ -144,6 +145,7 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         self._cppOp = [AimetTensorQuantizer(MAP_QUANT_SCHEME_TO_PYMO[self._quant_scheme]) for _ in range(num_ops)]
         self._encoding = None if encoding is None else [libpymo.TfEncoding(*e) for e in encoding]
         self._dev_params = None
+        self._fp8_grid = None
 
     @property
     def quant_scheme(self) -> QuantScheme:
@@ -387,8 +389,13 @@ class QuantizeDequantize(torch.autograd.Function):
         if tensor_quantizer.bitwidth == 8:
             if tensor_quantizer.fp8_maxval is None:
                 raise ValueError('tensor_quantizer.fp8_maxval not present or not initialized!')
-            out = ops.fp8_fake_cast(tensor.to(torch.float32), tensor_quantizer.fp8_maxval, 3,
-                                    tensor_quantizer.channel_axis or 0)
+            maxval = tensor_quantizer.fp8_maxval
+            cached = tensor_quantizer._fp8_grid               # pylint: disable=protected-access
+            if cached is None or cached[0] is not maxval or cached[1] != maxval._version:
+                cached = (maxval, maxval._version, ops.fp8_grid(maxval.to(tensor.device), 3))
+                tensor_quantizer._fp8_grid = cached           # pylint: disable=protected-access
+            out = ops.fp8_fake_cast(tensor.to(torch.float32), None, 3, tensor_quantizer.channel_axis or 0,
+                                    grid=cached[2])
             return out.to(tensor.dtype)
         if tensor_quantizer.bitwidth != 16:
             raise ValueError('float data_type only supports bitwidth in {16, 8}')

@@ -122,6 +122,38 @@ def bench_per_channel(torch, ops, shape, dtype, bw, steps, warmup, seed, nsets=3
             "fwd_bwd_GBps": 5 * esz * n / wall / 1e6, "buffer_sets": nsets}
 
 
+def bench_fp8(torch, ops, steps, warmup):
+    """8-bit float simulation (fake cast to the E4M3-shaped grid scaled to maxval) of the main weight shape, per
+    output channel, and of the activation shape, per tensor: forward only (its gradient is a pass-through)."""
+    dev = torch.device("cuda", 0)
+    out = {}
+    for name, shape, per_channel in (("per_channel_11008x4096", (11008, 4096), True),
+                                     ("per_tensor_32x64x56x56", (32, 64, 56, 56), False)):
+        n = 1
+        for d in shape:
+            n *= d
+        nsets = max(3, int(1.2e9 // (8 * n)))
+        sets = []
+        for k in range(nsets):
+            x = torch.randn(shape, device=dev, generator=torch.Generator(device=dev).manual_seed(1201 + k))
+            sets.append((x, torch.empty_like(x)))
+        maxval = sets[0][0].abs().amax(dim=1) if per_channel else sets[0][0].abs().max()
+        grid = ops.fp8_grid(maxval)                 # as the tensor quantizer holds it between calls
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        for i in range(warmup):
+            ops.fp8_fake_cast(sets[i % nsets][0], None, out=sets[i % nsets][1], grid=grid)
+        torch.cuda.synchronize()
+        ev[0].record()
+        for i in range(steps):
+            ops.fp8_fake_cast(sets[i % nsets][0], None, out=sets[i % nsets][1], grid=grid)
+        ev[1].record()
+        torch.cuda.synchronize()
+        ms = ev[0].elapsed_time(ev[1]) / steps
+        out[name] = {"elements": n, "ms_per_call": ms, "GBps": 8 * n / ms / 1e6,
+                     "frac_hbm": 8 * n / ms / 1e6 / HBM_PEAK_GBPS, "buffer_sets": nsets}
+    return out
+
+
 def bench_per_tensor(torch, ops, steps, warmup):
     dev = torch.device("cuda", 0)
     shape = (32, 64, 56, 56)
@@ -600,7 +632,7 @@ def main():
     ap.add_argument("--full", action="store_true", help="also measure every shape x dtype x bit-width cell")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run a subset of the legs, comma separated (main|pt|calib|sqnr|learn|quantsim|adaround|copyref), for profiling")
+                    help="run a subset of the legs, comma separated (main|pt|fp8|calib|sqnr|learn|quantsim|adaround|copyref), for profiling")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
@@ -635,6 +667,8 @@ def main():
         res = bench_per_channel(torch, ops, main_shape, torch.float32, 8, args.steps, args.warmup, 1004)
     if want("pt"):
         extra["per_tensor_act_int8"] = bench_per_tensor(torch, ops, max(20, args.steps), args.warmup)
+    if want("fp8"):
+        extra["fp8_simulation"] = bench_fp8(torch, ops, max(20, args.steps), args.warmup)
     if want("calib"):
         extra["tf_enhanced_calibration"] = bench_calibration(torch, ops, 5)
     if want("sqnr"):

@@ -99,9 +99,11 @@ int miq_fp16_round_trip_f32(const float* in, float* out, int64_t n, void* stream
  * Elements are laid out [outer][num_channels][inner]; channel c has the largest representable value maxval[c] and
  * bias[c] = 2^(7-M) - log2(maxval[c]) + log2(2 - 2^-M) - 1 (both device arrays of num_channels floats; per tensor:
  * num_channels = 1, inner = n).  Per element, in float32 and in this order: x_c = clamp(x, -maxval, maxval);
- * e = max(floor(log2|x_c| + bias), 1); step = 2^((e - M) - bias); out = rint(x_c / step) * step. */
+ * e = max(floor(log2|x_c| + bias), 1); step = 2^((e - M) - bias); out = rint(x_c / step) * step.  e is an integer in
+ * [1, 2^(7-M)], so the caller passes the steps as a table: steps[c * T + e] = 2^((e - M) - bias[c]) for e = 0 .. T-1,
+ * T = 2^(7-M) + 1 (a device array of num_channels * T floats). */
 int miq_fp8_fake_cast_f32(const float* in, float* out, int64_t n, int64_t num_channels, int64_t inner,
-                          const float* maxval, const float* bias, int mantissa_bits, void* stream);
+                          const float* maxval, const float* bias, const float* steps, int mantissa_bits, void* stream);
 
 /* ITensorQuantizationSim<float>::quantizeTensor(..., shiftToSigned) (ITensorQuantizationSim.h:57-59,
  * DLQ/src/TensorQuantizationSim.cpp:116-126; kernel DLQ/src/trim_functions.cu:62-76): float-valued grid indices. */
