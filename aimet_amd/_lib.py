@@ -87,17 +87,17 @@ _SIGNATURES = {
     "miq_v2_sqnr_search_f32": ([_p, _p, _i64, _int, _dbl, _int, _dbl, _int, _int, _int, _p, _p, _p, _p, _p], _int),
     "miq_adaround_linear_workspace_bytes": ([_i64, _i64], _i64),
     "miq_adaround_linear_blocks": ([_i64, _i64], _int),
-    "miq_adaround_linear_fwd_f32": ([_p, _p, _p, _p, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
+    "miq_adaround_linear_fwd_f32": ([_p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
                                      _p, _p, _p, _p, _p], _int),
-    "miq_adaround_linear_bwd_adam_f32": ([_p, _p, _p, _p, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
+    "miq_adaround_linear_bwd_adam_f32": ([_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
                                           _flt, _flt, _flt, _flt, _flt, _flt, _int, _p, _p], _int),
-    "miq_adaround_linear_fwd_i8": ([_p, _p, _p, _p, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
+    "miq_adaround_linear_fwd_i8": ([_p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
                                     _p, _p, _p, _p, _p], _int),
-    "miq_adaround_linear_bwd_adam_i8": ([_p, _p, _p, _p, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
+    "miq_adaround_linear_bwd_adam_i8": ([_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
                                          _flt, _flt, _flt, _flt, _flt, _flt, _int, _p, _p], _int),
-    "miq_adaround_linear_fwd_i16": ([_p, _p, _p, _p, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
+    "miq_adaround_linear_fwd_i16": ([_p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
                                      _p, _p, _p, _p, _p], _int),
-    "miq_adaround_linear_bwd_adam_i16": ([_p, _p, _p, _p, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
+    "miq_adaround_linear_bwd_adam_i16": ([_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
                                           _flt, _flt, _flt, _flt, _flt, _flt, _int, _p, _p], _int),
 }
 

@@ -47,6 +47,14 @@ __device__ __forceinline__ v4f mfma16(float a, float b, v4f c)
     return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
 
+// Row of x / target for batch entry b.  An index outside [0, num_rows) is clamped so that the read stays inside the
+// buffer; lin_loss_kernel marks such a row's results NaN.
+__device__ __forceinline__ int64_t gather_row(const int* row_index, int b, int num_rows)
+{
+    const int r = row_index ? row_index[b] : b;
+    return (int64_t) min(max(r, 0), num_rows - 1);
+}
+
 __device__ __forceinline__ v4f ldg4(const float* p)
 {
     return *reinterpret_cast<const v4f*>(p);
@@ -96,7 +104,8 @@ constexpr int kLdsRow = kTileK + 4;   // floats per LDS tile row; the pad spread
 template <typename FT>
 __global__ __launch_bounds__(256) void lin_fwd_kernel(const FT* __restrict__ F, const float* __restrict__ alpha,
                                                       const float* __restrict__ X, const int* __restrict__ row_index,
-                                                      int64_t x_row_stride, float* __restrict__ partial, LinGeom g)
+                                                      int num_rows, int64_t x_row_stride, float* __restrict__ partial,
+                                                      LinGeom g)
 {
     __shared__ __attribute__((aligned(16))) float tile[kTileO * kLdsRow];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -129,7 +138,7 @@ __global__ __launch_bounds__(256) void lin_fwd_kernel(const FT* __restrict__ F, 
     for (int mt = 0; mt < 2; ++mt)
     {
         const int b = mt * 16 + n;
-        xrow[mt]    = X + (int64_t) (row_index ? row_index[b] : b) * x_row_stride + k_blk + wave * 64 + 4 * s;
+        xrow[mt]    = X + gather_row(row_index, b, num_rows) * x_row_stride + k_blk + wave * 64 + 4 * s;
     }
     v4f a[4][2];
 #pragma unroll
@@ -199,8 +208,8 @@ __global__ __launch_bounds__(256) void lin_fwd_kernel(const FT* __restrict__ F, 
 // one thread per (b, o): out = sum_s partial[s][b][o] + bias[o]; G = 2 (act(out) - act(y)) act'(out) / batch
 __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__ partial, int num_split,
                                                        const float* __restrict__ bias, const float* __restrict__ Y,
-                                                       const int* __restrict__ row_index, int64_t y_row_stride,
-                                                       int out_features, int act, float* __restrict__ out,
+                                                       const int* __restrict__ row_index, int num_rows,
+                                                       int64_t y_row_stride, int out_features, int act, float* __restrict__ out,
                                                        float* __restrict__ G, float* __restrict__ loss_partial)
 {
     const int idx = blockIdx.x * 256 + threadIdx.x;
@@ -213,7 +222,10 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
             acc += partial[((int64_t) s * kBatch + b) * out_features + o];
         if (bias)
             acc += bias[o];
-        float y = Y[(int64_t) (row_index ? row_index[b] : b) * y_row_stride + o];
+        const int r = row_index ? row_index[b] : b;
+        float y     = Y[gather_row(row_index, b, num_rows) * y_row_stride + o];
+        if (r < 0 || r >= num_rows)
+            acc = NAN;   // no such row: poison everything derived from it
         if (out)
             out[idx] = acc;
         float pass = 1.f, ao = acc;
@@ -225,7 +237,7 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
         }
         const float diff = ao - y;
         sq               = diff * diff;
-        G[idx]           = 2.0f * diff * pass * (1.0f / kBatch);
+        G[idx]           = (acc != acc) ? acc : 2.0f * diff * pass * (1.0f / kBatch);
     }
     if (loss_partial)
     {
@@ -241,7 +253,7 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
 template <int PF, typename FT>
 __global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, const float* __restrict__ G,
                                                       const float* __restrict__ X, const int* __restrict__ row_index,
-                                                      int64_t x_row_stride, float* __restrict__ alpha,
+                                                      int num_rows, int64_t x_row_stride, float* __restrict__ alpha,
                                                       float* __restrict__ m, float* __restrict__ v,
                                                       float* __restrict__ grad_out, LinGeom g, AdamArgs a,
                                                       float* __restrict__ reg_partial)
@@ -284,7 +296,7 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, 
     for (int step = 0; step < 8; ++step)
     {
         const int b       = 4 * step + s;
-        const float* xrow = X + (int64_t) (row_index ? row_index[b] : b) * x_row_stride + k_blk + wave * 64 + n;
+        const float* xrow = X + gather_row(row_index, b, num_rows) * x_row_stride + k_blk + wave * 64 + n;
         const float* grow = G + (int64_t) b * O + o_blk + n;
         float xa[4], gb[2];
 #pragma unroll
@@ -379,7 +391,7 @@ using namespace miq;
 
 template <typename FT>
 static int linear_fwd(const FT* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
-                      int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+                      int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
                       int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
                       const float* offset, float clip_min, float clip_max, int activation, float* workspace, float* out,
                       float* grad_out, float* loss_partial, void* stream)
@@ -392,20 +404,24 @@ static int linear_fwd(const FT* weight_floor, const float* alpha, const float* x
                   "weight_floor, alpha and the rows of x must be 16-byte aligned");
     MIQ_CHECK_ARG(x_row_stride >= in_features && target_row_stride >= out_features, "row stride shorter than a row");
     MIQ_CHECK_ARG(activation == 0 || activation == 1, "activation must be 0 (none) or 1 (ReLU)");
+    MIQ_CHECK_ARG(num_rows >= 1 && num_rows < (1ll << 31) && (row_index || num_rows >= kBatch),
+                  "num_rows (%lld) must be positive, and at least 32 without a row index", (long long) num_rows);
     const int splits = (int) (in_features / kTileK);
     hipLaunchKernelGGL((lin_fwd_kernel<FT>), dim3((unsigned) splits, (unsigned) (out_features / kTileO)), dim3(256), 0,
-                       (hipStream_t) stream, weight_floor, alpha, x, row_index, x_row_stride, workspace, g);
+                       (hipStream_t) stream, weight_floor, alpha, x, row_index, (int) num_rows, x_row_stride, workspace,
+                       g);
     MIQ_CHECK_LAUNCH();
     const unsigned blocks = (unsigned) ((kBatch * out_features + 255) / 256);
     hipLaunchKernelGGL(lin_loss_kernel, dim3(blocks), dim3(256), 0, (hipStream_t) stream, workspace, splits, bias, target,
-                       row_index, target_row_stride, (int) out_features, activation, out, grad_out, loss_partial);
+                       row_index, (int) num_rows, target_row_stride, (int) out_features, activation, out, grad_out,
+                       loss_partial);
     MIQ_CHECK_LAUNCH();
     return MIQ_OK;
 }
 
 template <typename FT>
 static int linear_bwd_adam(const FT* weight_floor, const float* grad_out, const float* x, const int32_t* row_index,
-                           int64_t x_row_stride, float* alpha, float* exp_avg, float* exp_avg_sq, float* grad_alpha,
+                           int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg, float* exp_avg_sq, float* grad_alpha,
                            int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
                            const float* offset, float clip_min, float clip_max, float reg_param, float beta, float lr,
                            float beta1, float beta2, float eps, int step, float* reg_partial, void* stream)
@@ -418,12 +434,14 @@ static int linear_bwd_adam(const FT* weight_floor, const float* grad_out, const 
                       aligned16(grad_alpha),
                   "tensors must be 16-byte aligned");
     MIQ_CHECK_ARG(x_row_stride >= in_features, "row stride shorter than a row");
+    MIQ_CHECK_ARG(num_rows >= 1 && num_rows < (1ll << 31) && (row_index || num_rows >= kBatch),
+                  "num_rows (%lld) must be positive, and at least 32 without a row index", (long long) num_rows);
     AdamArgs a;
     if (int rc = make_adam(a, reg_param, beta, lr, beta1, beta2, eps, step))
         return rc;
     // two rows of the epilogue in flight per lane: deeper prefetch (3, 4) costs registers and measured no faster
     hipLaunchKernelGGL((lin_bwd_kernel<2, FT>), dim3((unsigned) (in_features / kTileK), (unsigned) (out_features / kTileO)),
-                       dim3(256), 0, (hipStream_t) stream, weight_floor, grad_out, x, row_index, x_row_stride, alpha,
+                       dim3(256), 0, (hipStream_t) stream, weight_floor, grad_out, x, row_index, (int) num_rows, x_row_stride, alpha,
                        exp_avg, exp_avg_sq, grad_alpha, g, a, reg_partial);
     MIQ_CHECK_LAUNCH();
     return MIQ_OK;
@@ -445,71 +463,71 @@ int miq_adaround_linear_blocks(int64_t out_features, int64_t in_features)
 }
 
 int miq_adaround_linear_fwd_f32(const float* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
-                                int64_t x_row_stride, const float* target, int64_t target_row_stride,
+                                int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride,
                                 const float* bias, int64_t out_features, int64_t in_features, int64_t num_channel,
                                 const float* delta, const float* offset, float clip_min, float clip_max,
                                 int activation, float* workspace, float* out, float* grad_out, float* loss_partial,
                                 void* stream)
 {
-    return linear_fwd<float>(weight_floor, alpha, x, row_index, x_row_stride, target, target_row_stride, bias,
+    return linear_fwd<float>(weight_floor, alpha, x, row_index, num_rows, x_row_stride, target, target_row_stride, bias,
                              out_features, in_features, num_channel, delta, offset, clip_min, clip_max, activation,
                              workspace, out, grad_out, loss_partial, stream);
 }
 
 int miq_adaround_linear_fwd_i8(const int8_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
-                               int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+                               int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
                                int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
                                const float* offset, float clip_min, float clip_max, int activation, float* workspace,
                                float* out, float* grad_out, float* loss_partial, void* stream)
 {
-    return linear_fwd<int8_t>(weight_floor, alpha, x, row_index, x_row_stride, target, target_row_stride, bias,
+    return linear_fwd<int8_t>(weight_floor, alpha, x, row_index, num_rows, x_row_stride, target, target_row_stride, bias,
                               out_features, in_features, num_channel, delta, offset, clip_min, clip_max, activation,
                               workspace, out, grad_out, loss_partial, stream);
 }
 
 int miq_adaround_linear_bwd_adam_f32(const float* weight_floor, const float* grad_out, const float* x,
-                                     const int32_t* row_index, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                     const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                      float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                      int64_t num_channel, const float* delta, const float* offset, float clip_min,
                                      float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
                                      float eps, int step, float* reg_partial, void* stream)
 {
-    return linear_bwd_adam<float>(weight_floor, grad_out, x, row_index, x_row_stride, alpha, exp_avg, exp_avg_sq,
+    return linear_bwd_adam<float>(weight_floor, grad_out, x, row_index, num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq,
                                   grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min, clip_max,
                                   reg_param, beta, lr, beta1, beta2, eps, step, reg_partial, stream);
 }
 
 int miq_adaround_linear_bwd_adam_i8(const int8_t* weight_floor, const float* grad_out, const float* x,
-                                    const int32_t* row_index, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                    const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                     float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                     int64_t num_channel, const float* delta, const float* offset, float clip_min,
                                     float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
                                     float eps, int step, float* reg_partial, void* stream)
 {
-    return linear_bwd_adam<int8_t>(weight_floor, grad_out, x, row_index, x_row_stride, alpha, exp_avg, exp_avg_sq,
+    return linear_bwd_adam<int8_t>(weight_floor, grad_out, x, row_index, num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq,
                                    grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min,
                                    clip_max, reg_param, beta, lr, beta1, beta2, eps, step, reg_partial, stream);
 }
 
 int miq_adaround_linear_fwd_i16(const int16_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
-                               int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+                               int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
                                int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
                                const float* offset, float clip_min, float clip_max, int activation, float* workspace,
                                float* out, float* grad_out, float* loss_partial, void* stream)
 {
-    return linear_fwd<int16_t>(weight_floor, alpha, x, row_index, x_row_stride, target, target_row_stride, bias,
+    return linear_fwd<int16_t>(weight_floor, alpha, x, row_index, num_rows, x_row_stride, target, target_row_stride, bias,
                               out_features, in_features, num_channel, delta, offset, clip_min, clip_max, activation,
                               workspace, out, grad_out, loss_partial, stream);
 }
 
 int miq_adaround_linear_bwd_adam_i16(const int16_t* weight_floor, const float* grad_out, const float* x,
-                                    const int32_t* row_index, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                    const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                     float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                     int64_t num_channel, const float* delta, const float* offset, float clip_min,
                                     float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
                                     float eps, int step, float* reg_partial, void* stream)
 {
-    return linear_bwd_adam<int16_t>(weight_floor, grad_out, x, row_index, x_row_stride, alpha, exp_avg, exp_avg_sq,
+    return linear_bwd_adam<int16_t>(weight_floor, grad_out, x, row_index, num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq,
                                    grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min,
                                    clip_max, reg_param, beta, lr, beta1, beta2, eps, step, reg_partial, stream);
 }

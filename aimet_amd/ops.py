@@ -547,7 +547,8 @@ def adaround_linear_fwd(weight_floor, alpha, x, row_index, target, bias, num_cha
         raise RuntimeError("row_index must hold 32 int32 row numbers")
     o, k = weight_floor.shape
     with _OnDevice(weight_floor.device):
-        check(fn(_ptr(weight_floor), _ptr(alpha), _ptr(x), _ptr(row_index), x.stride(0), _ptr(target), target.stride(0),
+        check(fn(_ptr(weight_floor), _ptr(alpha), _ptr(x), _ptr(row_index), min(x.size(0), target.size(0)), x.stride(0),
+                 _ptr(target), target.stride(0),
                  _ptr(bias), o, k, int(num_channel), _ptr(delta), _ptr(offset), float(clip_min), float(clip_max),
                  int(activation), _ptr(workspace), _ptr(out), _ptr(grad_out), _ptr(loss_partial), _stream(weight_floor)))
 
@@ -561,7 +562,8 @@ def adaround_linear_bwd_adam(weight_floor, grad_out, x, row_index, alpha, exp_av
     _require_gpu(weight_floor, x, row_index)
     o, k = weight_floor.shape
     with _OnDevice(weight_floor.device):
-        check(fn(_ptr(weight_floor), _ptr(grad_out), _ptr(x), _ptr(row_index), x.stride(0), _ptr(alpha), _ptr(exp_avg),
+        check(fn(_ptr(weight_floor), _ptr(grad_out), _ptr(x), _ptr(row_index), x.size(0), x.stride(0), _ptr(alpha),
+                 _ptr(exp_avg),
                  _ptr(exp_avg_sq), _ptr(grad_alpha), o, k, int(num_channel), _ptr(delta), _ptr(offset), float(clip_min),
                  float(clip_max), float(reg_param), float(beta), float(lr), float(beta1), float(beta2), float(eps),
                  int(step), _ptr(reg_partial), _stream(weight_floor)))

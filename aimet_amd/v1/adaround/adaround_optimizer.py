@@ -101,7 +101,13 @@ class AdaroundOptimizer:
                                                      qm.clip_min, qm.clip_max) if cls.use_int8_floor else None
             if weight_floor is None:
                 weight_floor = ops.adaround_floor(weight, qm.num_channel, qm.n_per_channel, qm.delta)
-            index = torch.stack(batches).to(dtype=torch.int32, device=device).contiguous()
+            index = torch.stack(batches)
+            # the kernels gather rows by these numbers; the reference's all_inp_data[indices] raises on a bad one
+            num_rows = min(all_inp_data.size(0), all_orig_out_data.size(0))
+            if index.numel() and (int(index.min()) < -num_rows or int(index.max()) >= num_rows):
+                raise IndexError(f"batch index out of range for {num_rows} cached rows")
+            index = torch.where(index < 0, index + num_rows, index)      # negative numbers count from the end
+            index = index.to(dtype=torch.int32, device=device).contiguous()
             bias = None if module.bias is None else module.bias.detach().to(torch.float32).contiguous()
             out_features, in_features = weight.shape
             workspace = ops.adaround_linear_workspace(out_features, in_features, device)

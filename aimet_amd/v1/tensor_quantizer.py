@@ -157,6 +157,7 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         self._quant_scheme = quant_scheme
         assert self._cppOp
         self._cppOp = [AimetTensorQuantizer(MAP_QUANT_SCHEME_TO_PYMO[quant_scheme]) for _ in self._cppOp]
+        self._drop_fused_stats()
 
     @property
     def encoding(self):
@@ -177,6 +178,10 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         if self.quant_scheme != QuantScheme.post_training_tf:
             self.quant_scheme = QuantScheme.post_training_tf
         self._encoding_min_max_fixed_vals = min_max_vals
+        self._drop_fused_stats()
+
+    def _drop_fused_stats(self):
+        """Statistics a subclass keeps outside the analyzer objects go with them."""
 
     def _stats_tensor(self, tensor: torch.Tensor) -> torch.Tensor:
         if self.encoding_min_max_fixed_vals is not None:
@@ -291,6 +296,9 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
         super().reset_encoding_stats()
         if not self._is_encoding_frozen:
             self._tf_minmax = None
+
+    def _drop_fused_stats(self):
+        self._tf_minmax = None
 
     def update_encoding_stats(self, tensor: torch.Tensor):
         if self.enabled and not self._is_encoding_frozen:

@@ -397,9 +397,11 @@ def _resnet50_shaped(torch):
     return Net().eval()
 
 
-def bench_quantsim(torch, steps=10, batch=64):
-    """cfg4: QuantizationSimModel forward on a random-init ResNet-50-shaped net, batch 64, int8 per-channel weight
-    quantizers and int8 per-tensor activation quantizers; QDQ overhead against the plain fp32 forward."""
+def quantsim_resnet50_shaped(torch, batch=64):
+    """The simulation-model workload: the ResNet-50-shaped net on the GPU, a QuantizationSimModel around it with int8
+    per-channel symmetric weight quantizers and int8 per-tensor activation quantizers (Conv+ReLU and Add+ReLU
+    supergroups, model input quantized), calibrated on 16 of the `batch` seeded N(0,1) images.
+    Returns (model, sim, images)."""
     import tempfile
     from aimet_amd.v1.quantsim import QuantizationSimModel
     dev = torch.device("cuda", 0)
@@ -420,6 +422,13 @@ def bench_quantsim(torch, steps=10, batch=64):
     os.unlink(f.name)
     with torch.no_grad():
         sim.compute_encodings(lambda m, a: m(a), x[:16])
+    return model, sim, x
+
+
+def bench_quantsim(torch, steps=10, batch=64):
+    """cfg4: QuantizationSimModel forward on a random-init ResNet-50-shaped net, batch 64, int8 per-channel weight
+    quantizers and int8 per-tensor activation quantizers; QDQ overhead against the plain fp32 forward."""
+    model, sim, x = quantsim_resnet50_shaped(torch, batch)
 
     def timed(fn):
         with torch.no_grad():

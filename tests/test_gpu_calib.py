@@ -171,41 +171,83 @@ def test_tfe_reset_and_unaligned(ops, oracle):
     assert (enc.min, enc.max, enc.delta, enc.offset, enc.bw) == pdf.compute_encoding(8)[0].astuple()
 
 
-def test_cfg3_full_size_properties(ops, oracle):
-    """16 batches of [32,256,28,28] on the GPU: counts of every batch sum to the batch size minus the dropped samples,
-    the PDF sums to the kept fraction, and a sub-sampled oracle run agrees on the first batch bit for bit."""
-    n = 32 * 256 * 28 * 28
-    an = ops.Analyzer(TFE)
+def _cfg3_batch(b, n):
     g = torch.Generator(device="cuda")
-    first = None
-    kept = []
-    for b in range(16):
-        g.manual_seed(1003 + b)
-        x = torch.randn(n, device="cuda", generator=g).abs_()
-        u = torch.rand(n, device="cuda", generator=g)
-        t = torch.rand(n, device="cuda", generator=g)
-        x = torch.where(u < 0.005, (1 - t).rsqrt(), x)
-        an.update_stats(x)
-        if b == 0:
-            first = x.cpu().numpy()
-            counts0 = an.last_batch_counts()
-        if b in (0, 7, 15):
-            c = an.last_batch_counts()
-            xl, _ = an.get_stats_histogram()
-            bucket = np.float32(xl[1] - xl[0])
-            off = np.float32(xl[0]) / bucket
-            r = torch.round(x / float(bucket) - float(off))   # not bit-exact near ties; used only for the drop count
-            kept.append((int(c.sum()), int(((r >= 0) & (r < 512)).sum())))
-    for got, approx in kept:
-        assert abs(got - approx) <= 64                 # samples within rounding distance of the range ends
+    g.manual_seed(1003 + b)
+    x = torch.randn(n, device="cuda", generator=g).abs_()
+    u = torch.rand(n, device="cuda", generator=g)
+    t = torch.rand(n, device="cuda", generator=g)
+    return torch.where(u < 0.005, (1 - t).rsqrt(), x)
+
+
+def _same_search(an, pdf, modes=((8, 0, 0, 0), (8, 1, 0, 0), (4, 0, 0, 0))):
+    for bw, sym, strict, uns in modes:
+        enc, valid = an.compute_encoding(bw, sym, strict, uns)
+        oenc, ocosts, obest = pdf.compute_encoding(bw, sym, strict, uns)
+        assert valid and (enc.min, enc.max, enc.delta, enc.offset, enc.bw) == oenc.astuple(), (bw, sym, strict, uns)
+        d, o, c, best = an.last_search()
+        od, oo = pdf.candidates(bw, sym, strict, uns)
+        assert np.array_equal(d.view(np.uint32), od.view(np.uint32)) and np.array_equal(o, oo)
+        assert np.array_equal(c.view(np.uint64), ocosts[:len(od)].view(np.uint64))
+        assert best == obest
+
+
+def test_cfg3_full_size_bit_exact(ops, oracle):
+    """The calibration configuration at its size: 16 batches of [32,256,28,28].  One analyzer is fed back to back with
+    nothing read in between (the path a calibration loop takes: counts folded by the following launch, bucket
+    parameters learnt asynchronously), a second one is read after every batch.  Per-batch counts, the final PDF
+    (as bits), every candidate cost and the chosen encodings equal the oracle's."""
+    n = 32 * 256 * 28 * 28
+    stream_an, step_an = ops.Analyzer(TFE), ops.Analyzer(TFE)
     pdf = oracle.new_pdf()
-    hist = pdf.update(first)
-    assert np.array_equal(counts0, hist)               # first batch: bit-exact against the oracle at full size
+    for b in range(16):
+        x = _cfg3_batch(b, n)
+        stream_an.update_stats(x)
+        step_an.update_stats(x)
+        hist = pdf.update(x.cpu().numpy())
+        got = step_an.last_batch_counts()
+        assert np.array_equal(got, hist), b
+        assert int(got.sum()) <= n
+    for an in (stream_an, step_an):
+        xl, p = an.get_stats_histogram()
+        assert np.array_equal(xl.view(np.uint64), pdf.x_left().view(np.uint64))
+        assert np.array_equal(p.view(np.uint64), pdf.pdf().view(np.uint64))
+        assert np.array_equal(an.last_batch_counts(), hist)
+        _same_search(an, pdf)
+
+
+def test_tfe_back_to_back_without_reads(ops, oracle):
+    """update_stats calls queued with no read-back between them: a leading all-zero batch (no range yet), ragged batch
+    sizes, a reset in the middle; only the final state is read and compared with the oracle fed the same batches."""
+    rng = np.random.default_rng(31)
+    first = [np.zeros(4096, np.float32)] + [_relu_pareto(40 + b, 300000 + 17 * b) for b in range(9)]
+    second = [(rng.standard_normal(250001 + 5 * b) * (1 + 0.1 * b)).astype(np.float32) for b in range(12)]
+    an = ops.Analyzer(TFE)
+    dev = [[_gpu(b) for b in first], [_gpu(b) for b in second]]
+    torch.cuda.synchronize()
+    for b in dev[0]:
+        an.update_stats(b)
+    an.reset()
+    for b in dev[1]:
+        an.update_stats(b)
+    pdf = oracle.new_pdf()
+    for b in second:
+        hist = pdf.update(b)
     xl, p = an.get_stats_histogram()
-    assert np.array_equal(xl, pdf.x_left())
-    assert 0.99 < p.sum() <= 1.0 + 1e-12
-    enc, valid = an.compute_encoding(8)
-    assert valid and enc.delta > 0 and enc.min <= 0 <= enc.max
+    assert np.array_equal(xl.view(np.uint64), pdf.x_left().view(np.uint64))
+    assert np.array_equal(p.view(np.uint64), pdf.pdf().view(np.uint64))
+    assert np.array_equal(an.last_batch_counts(), hist)
+    _same_search(an, pdf)
+    # the same without the reset, zero batch first
+    an2, pdf2 = ops.Analyzer(TFE), oracle.new_pdf()
+    for b in dev[0]:
+        an2.update_stats(b)
+    for b in first:
+        pdf2.update(b)
+    xl, p = an2.get_stats_histogram()
+    assert np.array_equal(xl.view(np.uint64), pdf2.x_left().view(np.uint64))
+    assert np.array_equal(p.view(np.uint64), pdf2.pdf().view(np.uint64))
+    _same_search(an2, pdf2, modes=((8, 0, 0, 0),))
 
 
 @pytest.mark.parametrize("outer,c,npc", [(1, 1, 100003), (1, 1, 3), (1, 1, 1 << 22), (1, 300, 4096), (1, 7, 70001),

@@ -180,6 +180,21 @@ def test_cfg2_weight_shapes(ops, oracle, shape, axis_c, bw):
     yb = ops.qdq_per_channel(wb.cuda(), c, npc, *gp).cpu()
     assert np.array_equal(yb.view(torch.int16).numpy().view(np.uint16),
                           oracle.qdq_per_channel_bf16(bits, c, npc, params))
+    _check_bf16_channel_backward(ops, oracle, wb, grad, c, npc, emn, emx)
+
+
+def _bf16_bits(t):
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _check_bf16_channel_backward(ops, oracle, xb, grad, c, npc, emn, emx):
+    """STE backward with bf16 storage: both inputs widen exactly to float32, grad * {0, 1} is exact, so the expected
+    bf16 words are the oracle's float32 result on the widened inputs, narrowed (sign of zero included)."""
+    gb = torch.from_numpy(np.ascontiguousarray(grad)).to(torch.bfloat16).reshape(xb.shape)
+    gin = ops.ste_bwd_per_channel(xb.cuda(), gb.cuda(), c, npc, _gpu(emn), _gpu(emx)).cpu()
+    want = oracle.ste_bwd_per_channel(xb.float().numpy(), gb.float().numpy(), c, npc, emn, emx)
+    want_b = torch.from_numpy(np.ascontiguousarray(want)).to(torch.bfloat16).reshape(xb.shape)
+    assert np.array_equal(_bf16_bits(gin), _bf16_bits(want_b))
 
 
 @pytest.mark.parametrize("c,npc,outer", [(4, 6, 1), (7, 1, 3), (5, 9, 4), (3, 17, 5), (16, 20, 2), (33, 4100, 2),
@@ -203,6 +218,7 @@ def test_per_channel_ragged(ops, oracle, c, npc, outer):
     yb = ops.qdq_per_channel(xb.cuda(), c, npc, *gp).cpu()
     assert np.array_equal(yb.view(torch.int16).numpy().view(np.uint16),
                           oracle.qdq_per_channel_bf16(xb.view(torch.int16).numpy().view(np.uint16), c, npc, params))
+    _check_bf16_channel_backward(ops, oracle, xb, grad, c, npc, params[0], params[1])
 
 
 def test_reference_per_channel_vectors(ops, oracle, vectors):

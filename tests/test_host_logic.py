@@ -334,3 +334,25 @@ def test_gating_keeps_learned_ranges_ordered():
     mx = nn.Parameter(torch.tensor([0.5, -0.2, 0.0]))
     set_encoding_min_max_gating_threshold(mn, mx)
     assert mn.tolist() == pytest.approx([0.0, -1.0, -1e-7]) and mx.tolist() == pytest.approx([0.5, 0.0, 1e-5 - 1e-7])
+
+
+def test_per_channel_fused_statistics_go_with_the_scheme():
+    """The per-channel quantizer keeps TF statistics outside its analyzer objects (one fused min/max pass).  A change of
+    scheme or fixed min/max values re-instantiates the analyzers (reference tensor_quantizer.py:222-247) and must
+    drop those statistics with them; reset does the same."""
+    from aimet_amd.common import libpymo
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.tensor_quantizer import StaticGridPerChannelQuantizer
+    q = StaticGridPerChannelQuantizer(8, libpymo.RoundingMode.ROUND_NEAREST, QuantScheme.post_training_tf,
+                                      use_symmetric_encodings=True, num_channels=4, enabled_by_default=True)
+    stale = torch.tensor([[-1.0] * 4, [1.0] * 4])
+    q._tf_minmax = stale                                    # pylint: disable=protected-access
+    q.quant_scheme = QuantScheme.post_training_tf_enhanced
+    assert q._tf_minmax is None                             # pylint: disable=protected-access
+    q.quant_scheme = QuantScheme.post_training_tf
+    q._tf_minmax = stale                                    # pylint: disable=protected-access
+    q.encoding_min_max_fixed_vals = (-0.5, 0.5)
+    assert q._tf_minmax is None and q.quant_scheme == QuantScheme.post_training_tf  # pylint: disable=protected-access
+    q._tf_minmax = stale                                    # pylint: disable=protected-access
+    q.reset_encoding_stats()
+    assert q._tf_minmax is None                             # pylint: disable=protected-access
