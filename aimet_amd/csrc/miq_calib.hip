@@ -24,6 +24,7 @@
 #include <cstddef>
 #include <cmath>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -966,6 +967,34 @@ __global__ void reset_state_kernel(DevState* st)
     }
 }
 
+// Partial (min, max) pairs of miq_minmax_per_channel_static_f32: device memory that belongs to the loaded library, one
+// copy per GPU, held until the process ends.  In host code this name is only a handle for hipGetSymbolAddress; the
+// address kernels receive is the one that call returns for the current device (static_scratch below).
+constexpr int64_t kStaticPairs = 32768;   // 256 KiB
+static __device__ __align__(256) float2 scratch[kStaticPairs];
+
+constexpr int kMaxDevices = 64;
+float2* g_scratch_ptr[kMaxDevices];   // per device: address of that GPU's copy of `scratch`; null until first use
+std::mutex g_scratch_mutex;
+
+// Address of the current device's copy of `scratch`, looked up once per device.
+int static_scratch(float2** out)
+{
+    int dev = 0;
+    MIQ_CHECK_HIP(hipGetDevice(&dev));
+    MIQ_CHECK_ARG(dev >= 0 && dev < kMaxDevices, "device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev])
+    {
+        float2* ptr = nullptr;
+        MIQ_CHECK_HIP(hipGetSymbolAddress((void**) &ptr, HIP_SYMBOL(scratch)));
+        MIQ_CHECK_ARG(ptr != nullptr, "no device address for the library's scratch array");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return MIQ_OK;
+}
+
 int stream_grid(int64_t n)
 {
     int64_t blocks = (n / 4 + (int64_t) kBlock * kUnroll - 1) / ((int64_t) kBlock * kUnroll);
@@ -1091,6 +1120,29 @@ int miq_minmax_per_channel_f32(const float* in, int64_t num_channel, int64_t num
                   "num_element must be a multiple of num_channel * num_element_per_channel");
     return launch_minmax_rows(in, num_channel, num_element / num_element_per_channel, num_element_per_channel,
                               reinterpret_cast<uint32_t*>(out_min_max), workspace, (hipStream_t) stream);
+}
+
+int miq_minmax_per_channel_static_f32(const float* in, int64_t num_channel, int64_t num_element,
+                                      int64_t num_element_per_channel, float* out_min_max, void* stream)
+{
+    MIQ_CHECK_ARG(num_channel > 0 && num_element_per_channel > 0 && num_element >= 0 && out_min_max,
+                  "bad channel geometry or null output");
+    MIQ_CHECK_ARG(num_element == 0 || in, "null input");
+    MIQ_CHECK_ARG(num_element % num_element_per_channel == 0,
+                  "num_element must be a multiple of num_element_per_channel");
+    MIQ_CHECK_ARG((num_element / num_element_per_channel) % num_channel == 0,
+                  "num_element must be a multiple of num_channel * num_element_per_channel");
+    const int64_t need = miq_minmax_workspace_bytes(num_channel, num_element, num_element_per_channel);
+    MIQ_CHECK_ARG(need <= kStaticPairs * (int64_t) sizeof(float2),
+                  "tensor too large for the allocation-free min/max: it needs %lld bytes of partial results, the "
+                  "library's static scratch holds %lld; use miq_minmax_per_channel_f32 with a workspace",
+                  (long long) need, (long long) (kStaticPairs * (int64_t) sizeof(float2)));
+    float2* ws = nullptr;
+    if (int rc = static_scratch(&ws))
+        return rc;
+    // every partial pair the fold kernel reads is written by the kernel before it in this call: nothing to clear
+    return launch_minmax_rows(in, num_channel, num_element / num_element_per_channel, num_element_per_channel,
+                              reinterpret_cast<uint32_t*>(out_min_max), ws, (hipStream_t) stream);
 }
 
 // PercentileEncodingAnalyzer<float>::computeEncoding on the PDF read back from the device

@@ -215,6 +215,17 @@ int miq_minmax_f32(const float* in, int64_t n, float* out_min_max, void* workspa
 int miq_minmax_per_channel_f32(const float* in, int64_t num_channel, int64_t num_element,
                                int64_t num_element_per_channel, float* out_min_max, void* workspace, void* stream);
 
+/* miq_minmax_per_channel_f32 for callers that cannot allocate device memory (code under HIP graph capture, serving
+ * loops, harnesses that forbid hipMalloc): the workgroups' partial results go to a 256 KiB array inside the loaded
+ * library (one copy per GPU, held until the process ends) instead of a caller workspace, and the call allocates and
+ * frees nothing.  No counterpart in the reference.  Same arguments and results as miq_minmax_per_channel_f32
+ * (num_channel = 1, num_element_per_channel = num_element gives the per-tensor form).  Limit: tensors whose
+ * miq_minmax_workspace_bytes() exceeds 256 KiB (32768 partial pairs: about 5.4e8 elements per tensor) are refused with
+ * MIQ_ERR_INVALID_ARG.  All calls on one GPU share the array: calls that overlap in time on one GPU (two streams,
+ * two threads) race and must be serialised by the caller. */
+int miq_minmax_per_channel_static_f32(const float* in, int64_t num_channel, int64_t num_element,
+                                      int64_t num_element_per_channel, float* out_min_max, void* stream);
+
 /* Encoding analyzer object = IQuantizationEncodingAnalyzer<float>
  * (DLQ/include/DlQuantization/IQuantizationEncodingAnalyzer.hpp:48-126) as instantiated by
  * getEncodingAnalyzerInstance<float>(mode) (DLQ/src/QuantizerFactory.cpp:74-97) for QUANTIZATION_TF
