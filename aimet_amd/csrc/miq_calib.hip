@@ -9,12 +9,11 @@
 //   TfEnhancedEncodingAnalyzer       DLQ/src/TfEnhancedEncodingAnalyzer.cpp:78-397
 //
 // Design: every statistic lives in one device-resident state block per analyzer.  update_stats is one streaming
-// kernel per batch in steady state (the first batch adds a min/max pass); the workgroup that finishes last folds
-// the batch's integer bin counts into the running PDF, so nothing is copied to the host and nothing synchronises
-// until an encoding is asked for.  Bin counts are integers, hence independent of the order in which lanes add them.
-// The histogram is privatised in LDS: 16 interleaved copies of the 512 bins per workgroup, lane l using copy
-// l mod 16, so that even when every sample of a wavefront falls into one bin (post-ReLU data) at most two lanes
-// meet on an address.
+// kernel per batch in steady state (the first batch adds a min/max pass); each launch also folds the previous
+// batch's integer bin counts into the running PDF, so nothing is copied to the host and nothing synchronises until
+// an encoding is asked for.  Bin counts are integers, hence independent of the order in which lanes add them.
+// The histogram is privatised in LDS: 8 interleaved copies of the 512 bins per workgroup, lane l using copy
+// l mod 8, and merged into one of 32 global replicas per batch.
 #include "miq_common.h"
 #include "miq_fastmath.h"
 
@@ -35,9 +34,11 @@ namespace
 constexpr int kPdf      = MIQ_PDF_SIZE;
 constexpr int kMaxCand  = 512;
 // LDS copies of the histogram per workgroup (lane l counts into copy l % kCopies) and the upper bound on streaming
-// workgroups.  8 copies are 16 KB, so 8 workgroups fit a compute unit and 2048 run in a single round: 7.3 us for a 25.7 MB
-// batch against 9.3 us with 16 copies / 1024 workgroups.  4 and 2 copies are faster still on spread-out data (6.9 / 6.7 us)
-// but collapse when the values share a bucket (constant tensor: 8.8 / 14.0 us against 6.9 us here).
+// workgroups.  8 copies are 16 KB, so 8 workgroups fit a compute unit and 2048 are resident at once: the streaming
+// workgroups plus the one that folds the previous batch must not exceed that, or the last one is dispatched only when
+// another has retired and lengthens the launch (measured: 0.5 us of 7).  4 and 2 copies are faster on spread-out data but
+// collapse when the values share a bucket (constant tensor: 8.8 / 14.0 us against 6.9 us with 8).
+typedef float vf4 __attribute__((ext_vector_type(4)));
 constexpr int kCopies   = 8;
 constexpr int kMaxGrid  = 2048;
 constexpr int kReplicas = 32;     // global count replicas: workgroup b merges into replica b % kReplicas, so at most
@@ -75,13 +76,15 @@ struct DevState
     // ---- head
     uint32_t ticket_search;
     int stats_updated;   // _statsUpdated
-    int minmax_valid;    // the min/max pass of this batch ran (it returns at once when the PDF range is fixed)
+    uint32_t minmax_seq; // number of the update call whose (min, max) partials wait in `partial`; 0 = none
     int initialized;     // PDF range fixed (xLeft.size() != 0 in the reference)
-    int iterations;
+    int iterations;      // batches folded into the PDF so far (mirror of iters[] for inspection)
     float bucket_f, pdf_offset_f;
     int n_cand;
     int best_index;
     int enc_bw;
+    int iters[2];            // the same count, written alternately: the launch of update call k reads iters[(k - 1) & 1]
+                             // and writes iters[k & 1], so that workgroups of one launch never read what it writes
     uint32_t batch_seq[2];   // update-call number whose counts sit in counts[i]; 0 = none pending
     int64_t batch_n[2];      // element count of that batch
     double acc_min, acc_max; // TF analyzer: accumulated range in double (TfEncodingAnalyzer.h:84-90)
@@ -106,6 +109,13 @@ template <typename T>
 __device__ __forceinline__ T agent_load(const T* p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// relaxed agent-scope store: written through, so that the launch leaves no modified lines behind in a cache for its
+// end-of-kernel release to write back
+template <typename T>
+__device__ __forceinline__ void agent_store(T* p, T v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ float wave_min(float v)
@@ -132,9 +142,16 @@ enum
     kMinMaxTfe = 2
 };
 
-__device__ void initialize_pdf(DevState* st, float min_val, float max_val)
+// Range of the PDF from the extremes of the first batch that is not all zeros: DLQ/src/math_functions.cpp:208-241 with
+// signed_vals = true, DTYPE = float.  bucket_f and offset_f are the two floats every later bucket index is formed from.
+struct PdfRange
 {
-    // DLQ/src/math_functions.cpp:208-241 with signed_vals = true, DTYPE = float
+    float min_val;
+    double bucket;
+    float bucket_f, offset_f;
+};
+__device__ __forceinline__ PdfRange pdf_range(float min_val, float max_val)
+{
     if (min_val == max_val)
     {
         const float t = min_val + (float) 0.01;
@@ -145,30 +162,70 @@ __device__ void initialize_pdf(DevState* st, float min_val, float max_val)
     const float hi     = center + 3 * (max_val - center);
     min_val            = (-FLT_MAX < lo) ? lo : -FLT_MAX;
     max_val            = (hi < FLT_MAX) ? hi : FLT_MAX;
-    const double bucket = ((double) max_val - (double) min_val) / kPdf;
+    PdfRange r;
+    r.min_val = min_val;
+    r.bucket  = ((double) max_val - (double) min_val) / kPdf;
+    // x_left[1] - x_left[0] and x_left[0], rounded to float, drive the bucket index of every later batch
+    const double x0 = min_val + 0 * r.bucket;
+    const double x1 = min_val + 1 * r.bucket;
+    r.bucket_f      = (float) (x1 - x0);
+    r.offset_f      = (float) x0 / r.bucket_f;
+    return r;
+}
+
+__device__ void initialize_pdf(DevState* st, const PdfRange& r)
+{
     for (int i = threadIdx.x; i < kPdf; i += blockDim.x)
     {
-        st->xLeft[i] = min_val + i * bucket;
+        st->xLeft[i] = r.min_val + i * r.bucket;
         st->pdf[i]   = 0.0;
     }
     if (threadIdx.x == 0)
     {
-        // x_left[1] - x_left[0] and x_left[0], rounded to float, drive the bucket index of every later batch
-        const double x0   = min_val + 0 * bucket;
-        const double x1   = min_val + 1 * bucket;
-        const float bf    = (float) (x1 - x0);
-        st->bucket_f      = bf;
-        st->pdf_offset_f  = (float) x0 / bf;
-        st->iterations    = 0;
-        st->initialized   = 1;
+        st->bucket_f     = r.bucket_f;
+        st->pdf_offset_f = r.offset_f;
+        st->initialized  = 1;
     }
 }
 
+// Folds `count` per-workgroup (min, max) pairs; every thread of the workgroup (kBlock threads) gets the result.
+__device__ __forceinline__ float2 fold_partials(const float2* partial, int count)
+{
+    float mn = INFINITY, mx = -INFINITY;
+    for (int i = threadIdx.x; i < count; i += kBlock)
+    {
+        const float2 p = partial[i];
+        mn             = fminf(mn, p.x);
+        mx             = fmaxf(mx, p.y);
+    }
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    __shared__ float smn[kBlock / 64], smx[kBlock / 64];
+    if ((threadIdx.x & 63) == 0)
+    {
+        smn[threadIdx.x >> 6] = mn;
+        smx[threadIdx.x >> 6] = mx;
+    }
+    __syncthreads();
+    float gmn = smn[0], gmx = smx[0];
+    for (int w = 1; w < kBlock / 64; ++w)
+    {
+        gmn = fminf(gmn, smn[w]);
+        gmx = fmaxf(gmx, smx[w]);
+    }
+    return make_float2(gmn, gmx);
+}
+
 // Pass 1: every workgroup reduces its share and stores one (min, max) pair -- plain stores, no atomics, because
-// same-address device atomics from a thousand workgroups serialise at roughly 15 ns each on this part.
+// same-address device atomics from a thousand workgroups serialise at roughly 15 ns each on this part.  Wide workgroups
+// (1024 lanes, four 16-byte loads in flight per lane, one workgroup per compute unit for a 25 MB batch) measured
+// fastest for a read-only pass and leave few pairs for the consumer to fold.
+constexpr int kMmBlock  = 1024;
+constexpr int kMmUnroll = 4;
+constexpr int kMmGrid   = 256;
 template <bool VEC>
-__global__ __launch_bounds__(kBlock) void minmax_kernel(const float* __restrict__ in, int64_t n, DevState* st,
-                                                        int mode)
+__global__ __launch_bounds__(kMmBlock) void minmax_kernel(const float* __restrict__ in, int64_t n, DevState* st, int mode,
+                                                          uint32_t seq)
 {
     if (mode == kMinMaxTfe && st->initialized)
         return;   // range already fixed: later batches need no min/max pass
@@ -176,22 +233,25 @@ __global__ __launch_bounds__(kBlock) void minmax_kernel(const float* __restrict_
     if (VEC)
     {
         const int64_t nvec   = n / 4;
-        const float4* v      = reinterpret_cast<const float4*>(in);
-        const int64_t stride = (int64_t) gridDim.x * kBlock * kUnroll;
-        for (int64_t base = (int64_t) blockIdx.x * kBlock * kUnroll; base < nvec; base += stride)
+        const vf4* v         = reinterpret_cast<const vf4*>(in);
+        const int64_t stride = (int64_t) gridDim.x * kMmBlock * kMmUnroll;
+        const vf4 nan4       = {NAN, NAN, NAN, NAN};   // fminf/fmaxf skip NaN
+        for (int64_t base = (int64_t) blockIdx.x * kMmBlock * kMmUnroll; base < nvec; base += stride)
         {
-            float4 a[kUnroll];
+            vf4 a[kMmUnroll];
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
+            for (int u = 0; u < kMmUnroll; ++u)
             {
-                const int64_t i = base + u * kBlock + threadIdx.x;
-                a[u] = (i < nvec) ? v[i] : make_float4(NAN, NAN, NAN, NAN);   // fminf/fmaxf skip NaN
+                const int64_t i = base + u * kMmBlock + threadIdx.x;
+                a[u]            = nan4;
+                if (i < nvec)
+                    a[u] = __builtin_nontemporal_load(v + i);
             }
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
+            for (int u = 0; u < kMmUnroll; ++u)
             {
-                mn = fminf(fminf(mn, a[u].x), fminf(a[u].y, fminf(a[u].z, a[u].w)));
-                mx = fmaxf(fmaxf(mx, a[u].x), fmaxf(a[u].y, fmaxf(a[u].z, a[u].w)));
+                mn = fminf(fminf(mn, a[u][0]), fminf(a[u][1], fminf(a[u][2], a[u][3])));
+                mx = fmaxf(fmaxf(mx, a[u][0]), fmaxf(a[u][1], fmaxf(a[u][2], a[u][3])));
             }
         }
         if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * 4))
@@ -203,7 +263,7 @@ __global__ __launch_bounds__(kBlock) void minmax_kernel(const float* __restrict_
     }
     else
     {
-        for (int64_t i = (int64_t) blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t) gridDim.x * kBlock)
+        for (int64_t i = (int64_t) blockIdx.x * kMmBlock + threadIdx.x; i < n; i += (int64_t) gridDim.x * kMmBlock)
         {
             const float a = in[i];
             mn            = fminf(mn, a);
@@ -212,7 +272,7 @@ __global__ __launch_bounds__(kBlock) void minmax_kernel(const float* __restrict_
     }
     mn = wave_min(mn);
     mx = wave_max(mx);
-    __shared__ float smn[kBlock / 64], smx[kBlock / 64];
+    __shared__ float smn[kMmBlock / 64], smx[kMmBlock / 64];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     if (lane == 0)
     {
@@ -222,65 +282,33 @@ __global__ __launch_bounds__(kBlock) void minmax_kernel(const float* __restrict_
     __syncthreads();
     if (threadIdx.x == 0)
     {
-        for (int w = 1; w < kBlock / 64; ++w)
+        for (int w = 1; w < kMmBlock / 64; ++w)
         {
             mn = fminf(mn, smn[w]);
             mx = fmaxf(mx, smx[w]);
         }
         st->partial[blockIdx.x] = make_float2(mn, mx);
         if (blockIdx.x == 0)
-            st->minmax_valid = 1;
+            st->minmax_seq = seq;
     }
 }
 
-// Pass 2 (one workgroup of kBlock lanes): fold the per-workgroup pairs and apply the analyzer's rule.
-__global__ __launch_bounds__(kBlock) void minmax_finalize_kernel(DevState* st, int grid, int mode)
+// Pass 2 of the TF (min/max) analyzer, one workgroup: fold the pairs into the accumulated range.  (The TF-Enhanced
+// analyzer has no second launch: the histogram kernel of the same update call folds the pairs in its prologue.)
+__global__ __launch_bounds__(kBlock) void minmax_finalize_kernel(DevState* st, int grid)
 {
-    if (!st->minmax_valid)
+    if (st->minmax_seq == 0)
         return;
-    float mn = INFINITY, mx = -INFINITY;
-    for (int i = threadIdx.x; i < grid; i += kBlock)
-    {
-        const float2 p = st->partial[i];
-        mn             = fminf(mn, p.x);
-        mx             = fmaxf(mx, p.y);
-    }
-    mn = wave_min(mn);
-    mx = wave_max(mx);
-    __shared__ float smn[kBlock / 64], smx[kBlock / 64];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    if (lane == 0)
-    {
-        smn[wave] = mn;
-        smx[wave] = mx;
-    }
-    __syncthreads();
-    float gmn = smn[0], gmx = smx[0];
-    for (int w = 1; w < kBlock / 64; ++w)
-    {
-        gmn = fminf(gmn, smn[w]);
-        gmx = fmaxf(gmx, smx[w]);
-    }
+    const float2 g = fold_partials(st->partial, grid);
     if (threadIdx.x == 0)
     {
-        st->minmax_valid  = 0;
+        st->minmax_seq    = 0;
         st->stats_updated = 1;
+        // DLQ/src/TfEncodingAnalyzer.cpp:59-71
+        const double cmn = (double) g.x, cmx = (double) g.y;
+        st->acc_min = (cmn < st->acc_min) ? cmn : st->acc_min;
+        st->acc_max = (st->acc_max < cmx) ? cmx : st->acc_max;
     }
-    if (mode == kMinMaxTf)
-    {
-        if (threadIdx.x == 0)
-        {
-            // DLQ/src/TfEncodingAnalyzer.cpp:59-71
-            const double cmn = (double) gmn, cmx = (double) gmx;
-            st->acc_min = (cmn < st->acc_min) ? cmn : st->acc_min;
-            st->acc_max = (st->acc_max < cmx) ? cmx : st->acc_max;
-        }
-        return;
-    }
-    // TF-Enhanced: DLQ/src/math_functions.cpp:248-262
-    if (gmn == 0 && gmx == 0)
-        return;   // an all-zero batch cannot fix a range; the PDF stays uninitialised and this batch is not counted
-    initialize_pdf(st, gmn, gmx);
 }
 
 // per-channel min/max: partial reductions meet in `keys` (uint32[2C], ordered keys) through atomics
@@ -465,105 +493,180 @@ __global__ __launch_bounds__(kBlock) void minmax_rows_fold_kernel(const float2* 
 }
 
 // ---------------------------------------------------------------------------------------------------- histogram
-// Adds one sample to the workgroup's LDS histogram.  Row kPdf is a sink for dropped samples, so the add is
-// unconditional (no divergent branch per element).
-// `rcp` is the correctly rounded 1 / bucket when the five-operation exact division applies to this bucket width (else 0);
-// it then gives the IEEE quotient bit for bit wherever the quotient can decide a bucket (miq_fastmath.h).
-__device__ __forceinline__ void hist_add(uint32_t* lds, float x, float bucket, float rcp, float off, int copy)
+// Adds one sample to the workgroup's LDS histogram: row 1 + bucket, rows 0 and kPdf + 1 collect dropped samples (out of
+// range, NaN), so the add is unconditional.  bucket_row (miq_fastmath.h) decides most samples with one fused
+// multiply-add and evaluates the reference's divide / subtract / round sequence (DLQ/src/math_functions.cpp:375-382)
+// only within a hair of a bucket edge; the bucket is the reference's for every sample.
+constexpr int kRows = kPdf + 2;
+template <int COPIES>
+__device__ __forceinline__ void hist_add(uint32_t* lds, float x, const BucketMap& m, int copy)
 {
-    // DLQ/src/math_functions.cpp:375-382; the range test is done on the rounded float so that NaN and values
-    // beyond the int range are dropped, as they are on the reference's CPU path
-    const float q  = (rcp != 0.0f && fabsf(x) <= kFastDivMaxDividend) ? div_by_invariant(x, bucket, rcp) : x / bucket;
-    const float r  = round_half_away(q - off);   // == roundf
-    const bool ok  = (r >= 0.0f && r < (float) kPdf);
-    const int row  = ok ? (int) r : kPdf;
-    atomicAdd(&lds[row * kCopies + copy], 1u);
+    atomicAdd(&lds[bucket_row<kPdf>(x, m) * COPIES + copy], 1u);
 }
 
 // Folds the counts of one finished batch into the running PDF (DLQ/src/math_functions.cpp:279-287; the element
-// count is an int in the reference) and clears them.  Run by one workgroup.
-__device__ void fold_batch(DevState* st, int buf)
+// count is an int in the reference) and clears them.  The work is cut into kFoldSlices slices of kFoldBins buckets;
+// a slice is folded by kFoldBins x kReplicas lanes, one replica count per lane (a single round trip to memory: load,
+// clear, add up across the 32 lanes of a bucket, one lane updates the running value).  In a histogram launch the
+// first kFoldSlices streaming workgroups fold one slice each while their first tile is on its way, so folding the
+// previous batch adds no workgroup and no latency to the launch.
+constexpr int kFoldBins   = kBlock / kReplicas;   // 8 buckets per slice
+constexpr int kFoldSlices = kPdf / kFoldBins;     // 64 slices
+static_assert(kReplicas == 32 && kFoldBins * kReplicas == kBlock && kFoldSlices * kFoldBins == kPdf, "fold layout");
+
+// One slice in two steps so that a caller can keep the loads in flight under other work.
+struct FoldLoad
 {
-    const int it     = st->iterations;
-    const double cnt = (double) (int) st->batch_n[buf];
-    for (int b = threadIdx.x; b < kPdf; b += blockDim.x)
+    uint32_t count;   // this lane's replica count
+    double running;   // leader lanes (replica 0): the bucket's running PDF value
+    int it;           // leader lanes: batches folded so far.  A per-lane (vector) load on purpose: a scalar load shares
+                      // its wait counter with the LDS operations and would hold up the histogram's LDS clear
+};
+// `lane_id` in [0, kBlock): lanes [32 j, 32 j + 32) share bucket slice * kFoldBins + j.
+__device__ __forceinline__ FoldLoad fold_load(const DevState* st, int buf, int it_slot, int slice, int lane_id)
+{
+    const int b = slice * kFoldBins + lane_id / kReplicas;
+    const int r = lane_id % kReplicas;
+    FoldLoad f;
+    f.running = 0.0;
+    f.it      = 0;
+    if (r == 0)
     {
-        // all replica loads in flight together, then the clears
-        uint32_t t[kReplicas];
-#pragma unroll
-        for (int r = 0; r < kReplicas; ++r)
-            t[r] = st->counts[buf][r][b];
-        uint32_t c = 0;
-#pragma unroll
-        for (int r = 0; r < kReplicas; ++r)
-        {
-            c += t[r];
-            st->counts[buf][r][b] = 0;
-        }
-        st->last_counts[b] = c;
-        const double prob  = (double) c / cnt;
-        st->pdf[b]         = (st->pdf[b] * it + prob) / (it + 1);
+        f.running = st->pdf[b];
+        f.it      = st->iters[it_slot];
     }
-    __syncthreads();
-    if (threadIdx.x == 0)
+    f.count = st->counts[buf][r][b];
+    return f;
+}
+// Plain loads and stores, not an atomic exchange: an atomic in flight would have to complete before the workgroup's
+// next barrier (its release fence), a load need not.
+__device__ __forceinline__ void fold_store(DevState* st, int buf, int64_t batch_n, int slice, int lane_id, FoldLoad f)
+{
+    const int b           = slice * kFoldBins + lane_id / kReplicas;
+    const int r           = lane_id % kReplicas;
+    agent_store(&st->counts[buf][r][b], 0u);
+    uint32_t c = f.count;
+#pragma unroll
+    for (int o = kReplicas / 2; o > 0; o >>= 1)
+        c += __shfl_xor(c, o);   // stays inside the 32 lanes of this bucket
+    if (r == 0)
     {
-        st->iterations     = it + 1;
-        st->batch_seq[buf] = 0;
+        agent_store(&st->last_counts[b], c);
+        const double prob = (double) c / (double) (int) batch_n;
+        agent_store(&st->pdf[b], (f.running * f.it + prob) / (f.it + 1));
     }
 }
 
-// One launch per batch.  Workgroups 0 .. gridDim.x-2 stream the tensor into counts[buf]; the extra last workgroup
-// meanwhile folds the previous batch (counts[1-buf], if that batch was accumulated) into the PDF and stamps this
-// batch as pending, so no second launch and no cross-workgroup hand-shake is needed.  `seq` numbers the update
-// calls of this analyzer; a buffer is pending iff its stamp equals the sequence number of the call that filled it.
-// With from_args the bucket width and offset arrive as kernel arguments (the host has learnt them); otherwise
-// they are read from the device state, which also says whether a range exists at all.
-template <bool VEC>
+// One launch per batch, every workgroup streams its share of the tensor into counts[buf]; while the first tile is in
+// flight kFoldSlices of the workgroups fold a slice each of the previous batch (counts[1 - buf], if that batch was
+// accumulated) into the PDF, and the first of them keeps the books (iteration count, stamp of this batch): no second
+// launch and no cross-workgroup hand-shake is needed.  (A dedicated folding workgroup was the longest-running one of
+// the launch: with the memory system saturated every dependent round trip costs microseconds.)  `seq` numbers the update calls of this analyzer; a buffer is pending
+// iff its stamp equals the sequence number of the call that filled it.
+// Where the bucket width and offset come from:
+//   KNOWN            kernel arguments (the host has learnt them; the steady state, compiled without the other two);
+//   else, when the min/max pass of this same update call ran (st->minmax_seq == seq): every workgroup folds that pass's
+//                    mm_grid (min, max) pairs itself and derives the range with the reference's arithmetic -- the first
+//                    batch that is not all zeros costs two launches, not three -- and workgroup 0 writes the range into
+//                    the state and, through `probe`, into host memory, so that the host can stop queuing min/max passes
+//                    without ever waiting for the device;
+//   else             the device state, which also says whether a range exists at all.
+// prev_n (KNOWN only): element count of the previous update call when the host knows that call was counted, else 0
+// (then the stamp decides).
+// probe: device-visible pinned host words {generation, -, bucket_f, pdf_offset_f}; the generation word is written last.
+template <bool VEC, bool KNOWN>
 __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ in, int64_t n, DevState* st, int buf,
-                                                      uint32_t seq, int from_args, float bucket_arg, float off_arg)
+                                                      uint32_t seq, float bucket_arg, float off_arg, int mm_grid,
+                                                      int* probe, int generation, int64_t prev_n, int fold_first)
 {
-    // workgroup 0 folds: it is dispatched first and runs beside the data workgroups (as the last one it would start only
-    // after a data workgroup had retired and would lengthen the launch by its own duration)
-    const bool fold_group = (blockIdx.x == 0);
-    const int data_groups = gridDim.x - 1;
-    const int group       = (int) blockIdx.x - 1;
-    if (fold_group)
-    {
-        if (st->batch_seq[1 - buf] != 0 && st->batch_seq[1 - buf] == seq - 1)
-            fold_batch(st, 1 - buf);
-        if (threadIdx.x == 0 && st->initialized)
-        {
-            st->batch_seq[buf] = seq;
-            st->batch_n[buf]   = n;
-        }
-        return;
-    }
-    __shared__ uint32_t lds[(kPdf + 1) * kCopies];
+    const int groups     = gridDim.x;
+    const int group      = (int) blockIdx.x;
+    const vf4* v         = reinterpret_cast<const vf4*>(in);
+    const vf4 nan4       = {NAN, NAN, NAN, NAN};   // dropped by hist_add
     const int64_t nvec   = n / 4;
-    const float4* v      = reinterpret_cast<const float4*>(in);
-    const int64_t stride = (int64_t) data_groups * kBlock * kUnroll;
+    const int64_t stride = (int64_t) groups * kBlock * kUnroll;
     int64_t base         = (int64_t) group * kBlock * kUnroll;
-    float4 a[kUnroll];
-    // first tile's loads go out before anything else: they overlap the state read and the LDS clear
+    // ---- the previous batch, step 1: kFoldSlices workgroups from fold_first on (the first of those with the smallest
+    // share of the tensor: they retire earliest) request their slice of its counts before anything else, so that this
+    // round trip runs under the first tile's
+    int64_t pending_n = 0;
+    const int slice   = group - fold_first;   // host: 0 <= fold_first <= groups - kFoldSlices
+    const bool folds  = slice >= 0 && slice < kFoldSlices;
+    FoldLoad fl{};
+    if (folds)
+    {
+        pending_n = KNOWN ? prev_n : 0;
+        if (pending_n == 0 && st->batch_seq[1 - buf] != 0 && st->batch_seq[1 - buf] == seq - 1)
+            pending_n = st->batch_n[1 - buf];
+        // (lane 0 of the last workgroup needs the iteration count even when nothing is pending: slice 0 loads it)
+        if (pending_n > 0 || slice == 0)
+            fl = fold_load(st, 1 - buf, 1 - buf, slice, threadIdx.x);
+    }
+    vf4 a[kUnroll];
+    // first tile's loads go out next: they overlap the state reads, the fold and the LDS clear
     if (VEC)
     {
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u)
         {
             const int64_t i = base + u * kBlock + threadIdx.x;
-            a[u] = (i < nvec) ? v[i] : make_float4(NAN, NAN, NAN, NAN);   // NaN is dropped by hist_add
+            a[u]            = nan4;
+            if (i < nvec)
+                a[u] = __builtin_nontemporal_load(v + i);   // read once: no reason to keep the line in the caches
         }
     }
+    // ---- the range
     float bucket = bucket_arg, off = off_arg;
-    if (!from_args)
+    bool have_range = true, fresh = false;
+    PdfRange range{};
+    if (!KNOWN)
     {
-        if (!st->initialized)
-            return;   // only all-zero batches so far: the reference returns without touching the PDF
-        bucket = st->bucket_f;
-        off    = st->pdf_offset_f;
+        fresh = (st->minmax_seq == seq);
+        if (fresh)
+        {
+            const float2 g = fold_partials(st->partial, mm_grid);
+            // DLQ/src/math_functions.cpp:248-262: an all-zero batch cannot fix a range; the PDF stays uninitialised and
+            // this batch is not counted
+            have_range = !(g.x == 0 && g.y == 0);
+            range      = pdf_range(g.x, g.y);
+            bucket     = range.bucket_f;
+            off        = range.offset_f;
+        }
+        else
+        {
+            have_range = st->initialized != 0;
+            bucket     = st->bucket_f;
+            off        = st->pdf_offset_f;
+        }
     }
-    const float rcp = fastdiv_divisor_ok(bucket) ? 1.0f / bucket : 0.0f;
-    for (int i = threadIdx.x; i < (kPdf + 1) * kCopies; i += kBlock)
+    if (slice == 0)
+    {
+        if (fresh && have_range)
+            initialize_pdf(st, range);
+        if (threadIdx.x == 0)
+        {
+            if (fresh)
+                st->stats_updated = 1;
+            if (have_range)
+            {
+                agent_store(&st->batch_seq[buf], seq);
+                agent_store(&st->batch_n[buf], n);
+                if (!KNOWN && probe)
+                {
+                    probe[2] = __float_as_int(bucket);
+                    probe[3] = __float_as_int(off);
+                    __threadfence_system();
+                    __hip_atomic_store(&probe[0], generation, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+                }
+            }
+        }
+    }
+    if (!have_range)
+        return;   // only all-zero batches so far: the reference returns without touching the PDF (and nothing can be
+                  // pending, both iteration slots are still 0: step 2 below has nothing to do)
+    __shared__ uint32_t lds[kRows * kCopies];
+    const BucketMap map = make_bucket_map(bucket, off, kPdf);
+    for (int i = threadIdx.x; i < kRows * kCopies; i += kBlock)
         lds[i] = 0;
     __syncthreads();
     const int copy = threadIdx.x & (kCopies - 1);
@@ -574,10 +677,9 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
 #pragma unroll
             for (int u = 0; u < kUnroll; ++u)
             {
-                hist_add(lds, a[u].x, bucket, rcp, off, copy);
-                hist_add(lds, a[u].y, bucket, rcp, off, copy);
-                hist_add(lds, a[u].z, bucket, rcp, off, copy);
-                hist_add(lds, a[u].w, bucket, rcp, off, copy);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    hist_add<kCopies>(lds, a[u][e], map, copy);
             }
             base += stride;
             if (base >= nvec)
@@ -586,16 +688,18 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
             for (int u = 0; u < kUnroll; ++u)
             {
                 const int64_t i = base + u * kBlock + threadIdx.x;
-                a[u] = (i < nvec) ? v[i] : make_float4(NAN, NAN, NAN, NAN);
+                a[u]            = nan4;
+                if (i < nvec)
+                    a[u] = __builtin_nontemporal_load(v + i);
             }
         }
         if (group == 0 && threadIdx.x < (uint32_t) (n - nvec * 4))
-            hist_add(lds, in[nvec * 4 + threadIdx.x], bucket, rcp, off, copy);
+            hist_add<kCopies>(lds, in[nvec * 4 + threadIdx.x], map, copy);
     }
     else
     {
-        for (int64_t i = (int64_t) group * kBlock + threadIdx.x; i < n; i += (int64_t) data_groups * kBlock)
-            hist_add(lds, in[i], bucket, rcp, off, copy);
+        for (int64_t i = (int64_t) group * kBlock + threadIdx.x; i < n; i += (int64_t) groups * kBlock)
+            hist_add<kCopies>(lds, in[i], map, copy);
     }
     __syncthreads();
     uint32_t* dst = st->counts[buf][group % kReplicas];
@@ -604,20 +708,50 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
         uint32_t s = 0;
 #pragma unroll
         for (int c = 0; c < kCopies; ++c)
-            s += lds[b * kCopies + c];
+            s += lds[(b + 1) * kCopies + c];
         if (s)
             atomicAdd(&dst[b], s);
     }
+    // ---- the previous batch, step 2: fold the slice requested at the top (its loads landed long ago; doing this last
+    // keeps every wait of the streaming part free of them); the workgroup of slice 0 keeps the books
+    if (folds)
+    {
+        if (pending_n > 0)
+            fold_store(st, 1 - buf, pending_n, slice, threadIdx.x, fl);
+        if (slice == 0 && threadIdx.x == 0)
+        {
+            // (the stamp of the folded batch stays: the other folding workgroups may not have read it yet, and no
+            // later launch can take it for pending because it compares with its own seq - 1)
+            const int now = fl.it + (pending_n > 0 ? 1 : 0);
+            agent_store(&st->iters[buf], now);
+            agent_store(&st->iterations, now);
+        }
+    }
 }
 
-// Folds whichever batch is still pending (at most one).  Queued before anything reads the PDF.
-__global__ __launch_bounds__(kBlock) void hist_flush_kernel(DevState* st, uint32_t seq)
+// Folds whichever batch is still pending (at most one).  Queued before anything reads the PDF.  One workgroup of
+// 1024 lanes: four slices per round, the loads of all sixteen rounds independent of each other.
+constexpr int kFlushBlock = 1024;
+__global__ __launch_bounds__(kFlushBlock) void hist_flush_kernel(DevState* st, uint32_t seq)
 {
-    for (int buf = 0; buf < 2; ++buf)
+    const int buf = (int) (seq & 1u);
+    if (st->batch_seq[buf] == 0 || st->batch_seq[buf] != seq)
+        return;
+    const int64_t batch_n  = st->batch_n[buf];
+    constexpr int kPerRound = kFlushBlock / kBlock, kRounds = kFoldSlices / kPerRound;
+    FoldLoad f[kRounds];
+#pragma unroll
+    for (int round = 0; round < kRounds; ++round)
+        f[round] = fold_load(st, buf, buf, round * kPerRound + threadIdx.x / kBlock, threadIdx.x % kBlock);
+#pragma unroll
+    for (int round = 0; round < kRounds; ++round)
+        fold_store(st, buf, batch_n, round * kPerRound + threadIdx.x / kBlock, threadIdx.x % kBlock, f[round]);
+    __syncthreads();   // every leader has read iters[buf]
+    if (threadIdx.x == 0)
     {
-        if (st->batch_seq[buf] != 0 && st->batch_seq[buf] == seq)
-            fold_batch(st, buf);
-        __syncthreads();
+        st->iters[buf]     = f[0].it + 1;   // what the next update call's launch reads
+        st->iterations     = f[0].it + 1;
+        st->batch_seq[buf] = 0;
     }
 }
 
@@ -945,10 +1079,11 @@ __global__ void reset_state_kernel(DevState* st)
     {
         st->ticket_search = 0;
         st->stats_updated = 0;
-        st->minmax_valid  = 0;
+        st->minmax_seq    = 0;
         st->acc_min       = DBL_MAX;
         st->acc_max       = -DBL_MAX;
         st->initialized = st->iterations = 0;
+        st->iters[0] = st->iters[1] = 0;
         st->bucket_f = st->pdf_offset_f = 0.f;
         st->n_cand                      = 0;
         st->best_index                  = -1;
@@ -1018,9 +1153,11 @@ struct miq_analyzer
     void* pinned;        // host staging (pinned) for read-backs
     bool stats_updated;  // host mirror of _isEncodingValid / _statsUpdated
     bool range_known;    // host knows the PDF range has been fixed, so no further min/max pass is queued
-    hipEvent_t probe;    // marks the completion of an asynchronous read of DevState::initialized
-    bool probe_pending;
-    int* probe_flag;     // pinned host words receiving that read: {initialized, iterations, bucket_f, pdf_offset_f}
+    int* probe_flag;     // pinned host words the histogram kernel writes once the range is fixed:
+                         // {generation, -, bucket_f, pdf_offset_f}; the host only ever polls them
+    int* probe_dev;      // the same words as the device addresses them
+    int64_t counted_n;   // element count of the last update call if the range was already known to the host then, else 0
+    int generation;      // bumped by reset, so that a launch queued before the reset cannot be believed after it
     float bucket_f, pdf_offset_f;   // valid once range_known
     uint32_t seq;        // number of TF-Enhanced update calls since the last reset
     int last_bw;
@@ -1230,9 +1367,10 @@ int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
     a->pinned        = nullptr;
     a->stats_updated = false;
     a->range_known   = false;
-    a->probe         = nullptr;
-    a->probe_pending = false;
     a->probe_flag    = nullptr;
+    a->probe_dev     = nullptr;
+    a->generation    = 1;
+    a->counted_n     = 0;
     a->bucket_f = a->pdf_offset_f = 0.f;
     a->seq           = 0;
     a->last_bw       = 0;
@@ -1242,7 +1380,11 @@ int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
     if (e == hipSuccess)
         e = hipHostMalloc(&a->pinned, kInspectBytes + 64, hipHostMallocDefault);   // + 4 probe words
     if (e == hipSuccess)
-        e = hipEventCreateWithFlags(&a->probe, hipEventDisableTiming);
+    {
+        a->probe_flag = reinterpret_cast<int*>(static_cast<char*>(a->pinned) + kInspectBytes);
+        memset(a->probe_flag, 0, 4 * sizeof(int));
+        e = hipHostGetDevicePointer(reinterpret_cast<void**>(&a->probe_dev), a->probe_flag, 0);
+    }
     if (e != hipSuccess)
     {
         set_error("analyzer allocation failed: %s", hipGetErrorString(e));
@@ -1253,8 +1395,6 @@ int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
         delete a;
         return MIQ_ERR_HIP;
     }
-    a->probe_flag  = reinterpret_cast<int*>(static_cast<char*>(a->pinned) + kInspectBytes);
-    *a->probe_flag = 0;
     hipLaunchKernelGGL(reset_state_kernel, dim3(1), dim3(kPdf), 0, (hipStream_t) nullptr, a->st);
     e = hipStreamSynchronize(nullptr);
     if (e != hipSuccess)
@@ -1262,7 +1402,6 @@ int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
         set_error("analyzer initialisation failed: %s", hipGetErrorString(e));
         (void) hipFree(a->st);
         (void) hipHostFree(a->pinned);
-        (void) hipEventDestroy(a->probe);
         delete a;
         return MIQ_ERR_HIP;
     }
@@ -1283,9 +1422,6 @@ int miq_analyzer_destroy(miq_analyzer* a)
 {
     if (!a)
         return MIQ_OK;
-    if (a->probe_pending)
-        (void) hipEventSynchronize(a->probe);
-    (void) hipEventDestroy(a->probe);
     (void) hipFree(a->st);
     (void) hipHostFree(a->pinned);
     delete a;
@@ -1300,13 +1436,9 @@ int miq_analyzer_reset(miq_analyzer* a, void* stream)
     a->stats_updated = false;
     a->range_known   = false;
     a->seq           = 0;
-    if (a->probe_pending)
-    {
-        // a read of the pre-reset state may still be in flight; its answer must not be believed afterwards
-        MIQ_CHECK_HIP(hipEventSynchronize(a->probe));
-        a->probe_pending = false;
-    }
-    *a->probe_flag = 0;
+    // a histogram launch queued before this reset may still publish its range: it carries the old generation
+    a->generation = (a->generation == INT_MAX) ? 1 : a->generation + 1;
+    a->counted_n  = 0;
     return MIQ_OK;
 }
 
@@ -1317,55 +1449,64 @@ int miq_analyzer_update_stats_f32(miq_analyzer* a, const float* data, int64_t n,
     hipStream_t s  = (hipStream_t) stream;
     const bool vec = aligned16(data);
     a->stats_updated = true;
-    const int grid = stream_grid(n);
+    const int grid    = stream_grid(n);
+    const int mm_grid = (int) std::max<int64_t>(
+        1, std::min<int64_t>(kMmGrid, (n / 4 + (int64_t) kMmBlock * kMmUnroll - 1) / ((int64_t) kMmBlock * kMmUnroll)));
     if (a->mode == MIQ_QUANTIZATION_TF)
     {
         if (vec)
-            hipLaunchKernelGGL(minmax_kernel<true>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st, kMinMaxTf);
+            hipLaunchKernelGGL(minmax_kernel<true>, dim3(mm_grid), dim3(kMmBlock), 0, s, data, n, a->st, kMinMaxTf, 1u);
         else
-            hipLaunchKernelGGL(minmax_kernel<false>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st, kMinMaxTf);
-        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(1), dim3(kBlock), 0, s, a->st, grid, kMinMaxTf);
+            hipLaunchKernelGGL(minmax_kernel<false>, dim3(mm_grid), dim3(kMmBlock), 0, s, data, n, a->st, kMinMaxTf, 1u);
+        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(1), dim3(kBlock), 0, s, a->st, mm_grid);
         MIQ_CHECK_LAUNCH();
         return MIQ_OK;
     }
-    if (!a->range_known && a->probe_pending && hipEventQuery(a->probe) == hipSuccess)
+    if (!a->range_known && __atomic_load_n(&a->probe_flag[0], __ATOMIC_ACQUIRE) == a->generation)
     {
-        a->probe_pending = false;
-        if (a->probe_flag[0] != 0)
-        {
-            a->range_known = true;
-            memcpy(&a->bucket_f, &a->probe_flag[2], sizeof(float));
-            memcpy(&a->pdf_offset_f, &a->probe_flag[3], sizeof(float));
-        }
-    }
-    if (!a->range_known)
-    {
-        // The range is fixed by the first batch that is not all zeros.  Whether that has happened is device state;
-        // the pass below returns at once when it has, and the host stops queuing it once an asynchronous read of
-        // that flag (queued after each batch until it answers yes) has landed.  Nothing here blocks.
-        if (vec)
-            hipLaunchKernelGGL(minmax_kernel<true>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st, kMinMaxTfe);
-        else
-            hipLaunchKernelGGL(minmax_kernel<false>, dim3(grid), dim3(kBlock), 0, s, data, n, a->st, kMinMaxTfe);
-        hipLaunchKernelGGL(minmax_finalize_kernel, dim3(1), dim3(kBlock), 0, s, a->st, grid, kMinMaxTfe);
+        // a histogram launch of this generation has fixed the range and written it into these pinned words
+        a->range_known = true;
+        memcpy(&a->bucket_f, &a->probe_flag[2], sizeof(float));
+        memcpy(&a->pdf_offset_f, &a->probe_flag[3], sizeof(float));
     }
     a->seq += 1;
-    const int buf       = (int) (a->seq & 1u);
-    const int from_args = a->range_known ? 1 : 0;
-    if (vec)
-        hipLaunchKernelGGL(hist_kernel<true>, dim3(grid + 1), dim3(kBlock), 0, s, data, n, a->st, buf, a->seq, from_args,
-                           a->bucket_f, a->pdf_offset_f);
-    else
-        hipLaunchKernelGGL(hist_kernel<false>, dim3(grid + 1), dim3(kBlock), 0, s, data, n, a->st, buf, a->seq,
-                           from_args, a->bucket_f, a->pdf_offset_f);
-    MIQ_CHECK_LAUNCH();
-    if (!a->range_known && !a->probe_pending)
+    if (!a->range_known)
     {
-        // {initialized, iterations, bucket_f, pdf_offset_f} are adjacent in DevState
-        MIQ_CHECK_HIP(hipMemcpyAsync(a->probe_flag, &a->st->initialized, 4 * sizeof(int), hipMemcpyDeviceToHost, s));
-        MIQ_CHECK_HIP(hipEventRecord(a->probe, s));
-        a->probe_pending = true;
+        // The range is fixed by the first batch that is not all zeros.  Whether that has happened is device state:
+        // the pass below returns at once when it has, and the host stops queuing it as soon as it sees the words a
+        // histogram launch writes into pinned memory when it fixes the range.  Nothing here blocks or copies.
+        if (vec)
+            hipLaunchKernelGGL(minmax_kernel<true>, dim3(mm_grid), dim3(kMmBlock), 0, s, data, n, a->st, kMinMaxTfe,
+                               a->seq);
+        else
+            hipLaunchKernelGGL(minmax_kernel<false>, dim3(mm_grid), dim3(kMmBlock), 0, s, data, n, a->st, kMinMaxTfe,
+                               a->seq);
     }
+    const int buf = (int) (a->seq & 1u);
+    // at least one workgroup per fold slice (those beyond the data only fold)
+    const int hist_groups = std::max(grid, kFoldSlices);
+    const dim3 hgrid((unsigned) hist_groups), hblock(kBlock);
+    // workgroups [rem, groups) stream one tile fewer than the others (none at all when there are fewer tiles than
+    // workgroups): the previous batch is folded by the first kFoldSlices of them
+    const int64_t tiles  = (n / 4 + (int64_t) kBlock * kUnroll - 1) / ((int64_t) kBlock * kUnroll);
+    const int fold_first = (int) std::min<int64_t>(tiles % hist_groups, hist_groups - kFoldSlices);
+    if (a->range_known)
+    {
+        if (vec)
+            hipLaunchKernelGGL((hist_kernel<true, true>), hgrid, hblock, 0, s, data, n, a->st, buf, a->seq, a->bucket_f,
+                               a->pdf_offset_f, mm_grid, a->probe_dev, a->generation, a->counted_n, fold_first);
+        else
+            hipLaunchKernelGGL((hist_kernel<false, true>), hgrid, hblock, 0, s, data, n, a->st, buf, a->seq, a->bucket_f,
+                               a->pdf_offset_f, mm_grid, a->probe_dev, a->generation, a->counted_n, fold_first);
+        a->counted_n = n;
+    }
+    else if (vec)
+        hipLaunchKernelGGL((hist_kernel<true, false>), hgrid, hblock, 0, s, data, n, a->st, buf, a->seq, 0.f, 0.f, mm_grid,
+                           a->probe_dev, a->generation, (int64_t) 0, fold_first);
+    else
+        hipLaunchKernelGGL((hist_kernel<false, false>), hgrid, hblock, 0, s, data, n, a->st, buf, a->seq, 0.f, 0.f,
+                           mm_grid, a->probe_dev, a->generation, (int64_t) 0, fold_first);
+    MIQ_CHECK_LAUNCH();
     return MIQ_OK;
 }
 
@@ -1373,8 +1514,9 @@ static int flush_pending(miq_analyzer* a, hipStream_t s)
 {
     if (a->mode != MIQ_QUANTIZATION_TF && a->seq != 0)
     {
-        hipLaunchKernelGGL(hist_flush_kernel, dim3(1), dim3(kBlock), 0, s, a->st, a->seq);
+        hipLaunchKernelGGL(hist_flush_kernel, dim3(1), dim3(kFlushBlock), 0, s, a->st, a->seq);
         MIQ_CHECK_LAUNCH();
+        a->counted_n = 0;   // nothing is pending any more: the next launch must not fold on the host's word
     }
     return MIQ_OK;
 }

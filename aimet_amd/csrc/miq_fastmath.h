@@ -51,5 +51,59 @@ MIQ_HD inline float round_half_away(float x)
 {
     return __builtin_truncf(x + __builtin_copysignf(0.49999997f, x));
 }
+
+// ---- bucket index of the 512-bucket PDF --------------------------------------------------------------------
+// Reference arithmetic (DlQuantization/src/math_functions.cpp:375-382), all binary32:
+//     q = x / bucket;  t = q - off;  r = roundf(t);  counted in bucket (int) r  iff  0 <= r < buckets
+// Three roundings separate t from the real number x / bucket - off, and one fused multiply-add
+//     u = fma(x, RN(1 / bucket), RN(1.5 - off))
+// lands within  (3 |off| + 2 buckets + 4) 2^-24  of t + 1.5 for every x whose t lies in [-1, buckets + 1]:
+//     |q - x/bucket| <= |x/bucket| 2^-24,  |t - (q - off)| <= |t| 2^-24,
+//     |x RN(1/bucket) - x/bucket| <= |x/bucket| 2^-24,  |RN(1.5 - off) - (1.5 - off)| <= (|off| + 1.5) 2^-24,
+//     |u - (x RN(1/bucket) + RN(1.5 - off))| <= |u| 2^-24,  and |x/bucket| <= |off| + buckets + 1.
+// roundf(t) changes only where t + 0.5 crosses an integer, so whenever the fraction of u stays at least
+// eps = (|off| + 2 buckets) 2^-21 (more than twice the bound above) away from 0 and 1, floor(u) - 1 is the reference's
+// bucket.  Otherwise (a sample within eps of a bucket edge, NaN, infinities, |u| >= 2^23, or a bucket width outside
+// the contract of div_by_invariant) the reference sequence itself is evaluated.  Rows: 1 .. buckets are the
+// buckets, 0 and buckets + 1 collect what the reference drops.
+struct BucketMap
+{
+    float bucket, rcp, off;   // reference sequence; rcp = RN(1 / bucket) or 0 when div_by_invariant does not apply
+    float fast_scale;         // RN(1 / bucket), only read when thr > 0
+    float fast_shift;         // RN(1.5 - off)
+    float thr;                // 0.5 - eps; not positive: the one-operation path is never taken
+};
+
+MIQ_HD inline BucketMap make_bucket_map(float bucket, float off, int buckets)
+{
+    BucketMap m;
+    m.bucket        = bucket;
+    m.off           = off;
+    const bool ok   = fastdiv_divisor_ok(bucket);
+    m.rcp           = ok ? 1.0f / bucket : 0.0f;
+    m.fast_scale    = m.rcp;
+    m.fast_shift    = 1.5f - off;
+    const float eps = (__builtin_fabsf(off) + 2.0f * (float) buckets) * 4.76837158203125e-07f;   // 2^-21
+    m.thr           = (ok && eps < 0.25f) ? 0.5f - eps : -1.0f;   // false for a NaN offset
+    return m;
+}
+
+template <int BUCKETS>
+MIQ_HD inline int bucket_row(float x, const BucketMap& m)
+{
+    const float u  = __builtin_fmaf(x, m.fast_scale, m.fast_shift);
+    const float fl = __builtin_floorf(u);
+    const float f  = u - fl;   // exact
+    if (__builtin_fabsf(f - 0.5f) < m.thr)
+    {
+        // fl is an integer below 2^23 here (larger floats have no fraction: f == 0 fails the test)
+        const int k = (int) fl;
+        return k < 0 ? 0 : (k > BUCKETS + 1 ? BUCKETS + 1 : k);
+    }
+    const float q = (m.rcp != 0.0f && __builtin_fabsf(x) <= kFastDivMaxDividend) ? div_by_invariant(x, m.bucket, m.rcp)
+                                                                                 : x / m.bucket;
+    const float r = round_half_away(q - m.off);
+    return (r >= 0.0f && r < (float) BUCKETS) ? (int) r + 1 : 0;
+}
 }   // namespace miq
 #endif

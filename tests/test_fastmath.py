@@ -57,3 +57,20 @@ def test_multiply_high_division():
         n = n[n < (1 << 31)]             # the dividend has at most 31 bits (the launcher guarantees it)
         q = ((n * np.uint64(magic)) >> np.uint64(32)) >> np.uint64(shift)
         assert np.array_equal(q, n // np.uint64(d)), d
+
+
+def test_bucket_row_equals_the_reference_sequence(tmp_path):
+    """bucket_row (miq_fastmath.h) answers most samples with one fused multiply-add and falls back to the reference's
+    divide / subtract / round sequence near bucket edges; it must select the reference's bucket for every sample:
+    thousands of PDF ranges over 60 decades, the floats around every bucket edge, random samples, arbitrary bit
+    patterns."""
+    exe = tmp_path / "bucket_check"
+    src = os.path.join(ROOT, "tests", "host", "bucket_check.cpp")
+    flags = ["-O2", "-std=c++17", "-ffp-contract=off"]
+    if "fma" in open("/proc/cpuinfo").read():
+        flags.append("-mfma")
+    subprocess.run(["g++", *flags, "-o", str(exe), src], check=True)
+    out = subprocess.run([str(exe), "3000"], capture_output=True, text=True, timeout=600)
+    assert out.returncode == 0, out.stdout[-2000:]
+    assert out.stdout.startswith("OK")
+    assert float(out.stdout.split()[2]) > 0.2          # the one-operation path did answer a good share
