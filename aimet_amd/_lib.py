@@ -86,6 +86,15 @@ _SIGNATURES = {
     "miq_v2_hist_update_f32": ([_p, _i64, _i64, _int, _int, _int, _p, _p, _p, _p, _p, _p, _p], _int),
     "miq_v2_sqnr_num_candidates": ([_dbl, _int, _int, _int, _int], _int),
     "miq_v2_sqnr_search_f32": ([_p, _p, _i64, _int, _dbl, _int, _dbl, _int, _int, _int, _p, _p, _p, _p, _p], _int),
+    "miq_channel_analyzer_state_bytes": ([_i64], _i64),
+    "miq_channel_analyzer_workspace_bytes": ([_i64, _i64, _i64], _i64),
+    "miq_channel_analyzer_create": ([_int, _i64, _p, _p, C.POINTER(_p)], _int),
+    "miq_channel_analyzer_destroy": ([_p], _int),
+    "miq_channel_analyzer_reset": ([_p, _p], _int),
+    "miq_channel_analyzer_set_percentile": ([_p, _flt], _int),
+    "miq_channel_analyzer_update_stats_f32": ([_p, _p, _i64, _i64, _p, _p], _int),
+    "miq_channel_analyzer_compute_encodings": ([_p, _int, _int, _int, _int, _p, C.POINTER(_int), _p], _int),
+    "miq_channel_analyzer_get_stats_histogram": ([_p, _i64, _p, _p, C.POINTER(_int), _p], _int),
     "miq_adaround_linear_workspace_bytes": ([_i64, _i64], _i64),
     "miq_adaround_linear_blocks": ([_i64, _i64], _int),
     "miq_adaround_linear_fwd_f32": ([_p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,

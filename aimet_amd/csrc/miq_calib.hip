@@ -16,6 +16,7 @@
 // l mod 8, and merged into one of 32 global replicas per batch.
 #include "miq_common.h"
 #include "miq_fastmath.h"
+#include "miq_tfe_search.h"
 
 #include <algorithm>
 #include <cfloat>
@@ -80,6 +81,7 @@ struct DevState
     int initialized;     // PDF range fixed (xLeft.size() != 0 in the reference)
     int iterations;      // batches folded into the PDF so far (mirror of iters[] for inspection)
     float bucket_f, pdf_offset_f;
+    float range_min;         // x_left[i] = range_min + i * range_bucket
     int n_cand;
     int best_index;
     int enc_bw;
@@ -87,6 +89,7 @@ struct DevState
                              // and writes iters[k & 1], so that workgroups of one launch never read what it writes
     uint32_t batch_seq[2];   // update-call number whose counts sit in counts[i]; 0 = none pending
     int64_t batch_n[2];      // element count of that batch
+    double range_bucket;
     double acc_min, acc_max; // TF analyzer: accumulated range in double (TfEncodingAnalyzer.h:84-90)
     double enc_min, enc_max, enc_delta, enc_offset;
     // ---- inspection block
@@ -184,6 +187,8 @@ __device__ void initialize_pdf(DevState* st, const PdfRange& r)
     {
         st->bucket_f     = r.bucket_f;
         st->pdf_offset_f = r.offset_f;
+        st->range_min    = r.min_val;
+        st->range_bucket = r.bucket;
         st->initialized  = 1;
     }
 }
@@ -756,57 +761,8 @@ __global__ __launch_bounds__(kFlushBlock) void hist_flush_kernel(DevState* st, u
 }
 
 // ------------------------------------------------------------------------------------------------ SQNR search
-// (int) of a floating-point value as the reference's x86-64 build performs it (cvttsd2si / cvttss2si): truncation
-// inside the int range, INT_MIN for everything else, NaN included.  The C++ cast is undefined there and this GPU's
-// conversion saturates instead; the difference decides a cost when a candidate range is more than 2^31 PDF buckets wide
-// (data spanning less than about 1e-12 against the 1e-5 minimum encoding range).
-__device__ __forceinline__ int cvtt_x86(double v)
-{
-    return (v >= -2147483648.0 && v < 2147483648.0) ? (int) v : INT_MIN;
-}
-
-struct SearchArgs
-{
-    int bw;
-    int sym, strict, uns;
-    float num_steps_cand;   // 2^bw - 1, minus 1 for strict symmetric (candidate generation and final min/max)
-    float step_size_cost;   // 2^bw - 1 (the cost function never reduces it)
-    int n_cand;             // grid size: 17*21 + 1 asymmetric, number of float steps of 0.01 symmetric
-    int n_delta;            // 17 or the symmetric count
-};
-
-__device__ __forceinline__ float std_max(float a, float b)
-{
-    return (a < b) ? b : a;   // std::max(a, b)
-}
-__device__ __forceinline__ float std_min(float a, float b)
-{
-    return (b < a) ? b : a;   // std::min(a, b)
-}
-
-// Sum of term[lo..hi) in ascending index order.  Eight loads are issued ahead of the eight dependent adds.
-__device__ __forceinline__ double ordered_sum(const double* term, int lo, int hi)
-{
-    double acc = 0;
-    int i      = lo;
-    for (; i + 8 <= hi; i += 8)
-    {
-        double t[8];
-#pragma unroll
-        for (int k = 0; k < 8; ++k)
-            t[k] = term[i + k];
-#pragma unroll
-        for (int k = 0; k < 8; ++k)
-            acc += t[k];
-    }
-    for (; i < hi; ++i)
-        acc += term[i];
-    return acc;
-}
-
-// One wavefront per candidate.  Lanes evaluate the per-bucket error terms in parallel; the three sums of the
-// cost are then accumulated by one lane in bucket order, the order the reference's loops use, so that costs are
-// bit-identical to the CPU result and ties between candidates resolve identically.
+// One wavefront per candidate (miq_tfe_search.h); the workgroup that finishes last picks the winner.
+using tfe::SearchArgs;
 __global__ __launch_bounds__(kBlock) void tfe_search_kernel(DevState* st, SearchArgs a)
 {
     constexpr int kWaves = kBlock / 64;
@@ -815,166 +771,16 @@ __global__ __launch_bounds__(kBlock) void tfe_search_kernel(DevState* st, Search
     const int lane       = threadIdx.x & 63;
     __shared__ double term_all[kWaves][kPdf];
     __shared__ bool is_last;
-    double* term = term_all[wave];
 
     if (st->initialized && cand < a.n_cand)
     {
-        // ---- range of the aggregate stats: DLQ/src/TfEnhancedEncodingAnalyzer.cpp:255-291
-        int first = -1, last = -1;
-#pragma unroll
-        for (int k = 0; k < kPdf / 64; ++k)
-        {
-            const uint64_t m = __ballot(st->pdf[k * 64 + lane] > 0);
-            if (m)
-            {
-                if (first < 0)
-                    first = k * 64 + __builtin_ctzll(m);
-                const uint64_t m1 = (k == 0) ? (m & ~1ull) : m;   // the downward scan stops above bucket 0
-                if (m1)
-                    last = k * 64 + 63 - __builtin_clzll(m1);
-            }
-        }
-        float minVal = (float) st->xLeft[first < 0 ? 0 : first];
-        float maxVal = (float) st->xLeft[last < 0 ? kPdf - 1 : last];
-        minVal       = std_min(minVal, 0.0f);
-        maxVal       = std_max(maxVal, 0.0f);
-        maxVal       = std_max(maxVal, minVal + (float) 0.01);
-
-        // ---- this wavefront's candidate
-        float delta = 0.f;
-        int offset  = 0;
-        bool valid  = true;
-        const float numSteps = a.num_steps_cand;
-        if (a.sym)
-        {
-            // DLQ/src/TfEnhancedEncodingAnalyzer.cpp:216-253
-            float deltaMax;
-            if ((minVal == 0.0) && a.uns)
-            {
-                deltaMax = maxVal / numSteps;
-                offset   = 0;
-            }
-            else
-            {
-                const float absMax = std_max(fabsf(maxVal), fabsf(minVal));
-                deltaMax           = (float) (absMax / (numSteps / 2.0));
-                offset             = (int) floorf(-numSteps / 2);
-            }
-            float f = (float) (1.0 / 100);
-            for (int k = 0; k < cand; ++k)
-                f = (float) ((double) f + 1.0 / 100);
-            delta = f * deltaMax;
-        }
-        else
-        {
-            // DLQ/src/TfEnhancedEncodingAnalyzer.cpp:177-214
-            const float obsDelta = (float) (((double) maxVal - (double) minVal) / numSteps);
-            const int obsOffset  = (int) roundf(minVal / obsDelta);
-            const float obsMin   = std_max(obsDelta * (float) obsOffset, -FLT_MAX);
-            const float obsMax   = std_min(obsDelta * ((float) obsOffset + numSteps), FLT_MAX);
-            if (cand == a.n_cand - 1)
-            {
-                delta  = obsDelta;
-                offset = obsOffset;
-            }
-            else
-            {
-                const int fi = cand / 21, oi = cand % 21;
-                float f = (float) (1.0 / 16);
-                for (int k = 0; k < fi; ++k)
-                    f = (float) ((double) f + 1.0 / 16);
-                delta  = f * obsDelta;
-                offset = (int) ((double) (-numSteps) + (double) numSteps / 20.0 * oi);
-                // clamp to the observed range: DLQ/src/TfEnhancedEncodingAnalyzer.cpp:149-175
-                float tMin = std_max(delta * (float) offset, -FLT_MAX);
-                float tMax = std_min(delta * ((float) offset + numSteps), FLT_MAX);
-                if ((tMin < obsMin) && (tMax > obsMax))
-                    valid = false;
-                else
-                {
-                    tMin = std_max(obsMin, tMin);
-                    tMax = std_min(obsMax, tMax);
-                    if (tMin == tMax)
-                        valid = false;
-                    else
-                    {
-                        delta  = (float) (((double) tMax - tMin) / numSteps);
-                        offset = (int) roundf(tMin / delta);
-                    }
-                }
-            }
-        }
-
-        // ---- cost: DLQ/src/TfEnhancedEncodingAnalyzer.cpp:293-355
-        double cost = 0;
-        if (valid)
-        {
-            const float cMin      = delta * (float) offset;
-            const float stepSize  = a.step_size_cost;
-            const float cMax      = delta * ((float) offset + stepSize);
-            const float pdfStart  = (float) st->xLeft[0];
-            const double pdfStep  = st->xLeft[1] - st->xLeft[0];
-            int minInd            = cvtt_x86(floor((cMin - pdfStart) / pdfStep));
-            minInd                = minInd < 0 ? 0 : (minInd > kPdf - 1 ? kPdf - 1 : minInd);
-            int maxInd            = cvtt_x86(floor((cMax - pdfStart) / pdfStep));
-            maxInd                = maxInd < 0 ? 0 : (maxInd > kPdf - 1 ? kPdf - 1 : maxInd);
-            const float minMid    = (float) (pdfStart + (minInd * pdfStep) + pdfStep / 2);
-            const float maxMid    = (float) (pdfStart + (maxInd * pdfStep) + pdfStep / 2);
-#pragma unroll
-            for (int k = 0; k < kPdf / 64; ++k)
-            {
-                const int i      = k * 64 + lane;
-                const double p   = st->pdf[i];
-                const double mid = pdfStart + i * pdfStep + pdfStep / 2;
-                double t;
-                if (i < minInd)
-                {
-                    const double d = mid - minMid;
-                    t              = p * (d * d);
-                }
-                else if (i >= maxInd)
-                {
-                    const double d = mid - maxMid;
-                    t              = p * (d * d);
-                }
-                else
-                {
-                    const float fv   = (float) mid;
-                    const int q      = cvtt_x86((double) roundf(fv / delta - (float) offset));
-                    const float dq   = delta * (float) (q + offset);
-                    const double d   = (double) (fv - dq);
-                    t                = p * (d * d);
-                }
-                term[i] = t;
-            }
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_s_waitcnt(0xc07f);   // LDS writes of this wavefront have landed (lgkmcnt = 0)
-            // The three sums are accumulated in ascending bucket order, the order of the reference's loops.  Every
-            // lane runs the same chain (uniform bounds, LDS broadcast reads), so no cross-lane traffic is needed.
-            const double satBottom = ordered_sum(term, 0, minInd);
-            double satTop          = ordered_sum(term, maxInd, kPdf);
-            const double quant     = ordered_sum(term, minInd, maxInd);
-            if (maxInd < minInd)
-            {
-                // Only after an index conversion left the int range (cvtt_x86).  The reference's three loops then
-                // overlap: buckets [maxInd, minInd) are saturation at the bottom AND at the top, and no bucket is
-                // quantization noise.  Redo the top sum with every bucket's distance to the top mid-point.
-                __builtin_amdgcn_wave_barrier();
-#pragma unroll
-                for (int k = 0; k < kPdf / 64; ++k)
-                {
-                    const int i      = k * 64 + lane;
-                    const double mid = pdfStart + i * pdfStep + pdfStep / 2;
-                    const double d   = mid - maxMid;
-                    term[i]          = st->pdf[i] * (d * d);
-                }
-                __builtin_amdgcn_wave_barrier();
-                __builtin_amdgcn_s_waitcnt(0xc07f);
-                satTop = ordered_sum(term, maxInd, kPdf);
-            }
-            cost = 3.0 * (satBottom + satTop) + quant;
-            cost                   = (cost < DBL_MAX) ? cost : DBL_MAX;   // std::min(sqnr, max())
-        }
+        // x_left[i] of the state is min_val + i * bucket with these two values (initialize_pdf)
+        const tfe::PdfView view{st->pdf, st->range_min, st->range_bucket};
+        float minVal, maxVal, delta;
+        int offset;
+        tfe::wave_range(view, lane, minVal, maxVal);
+        const bool valid  = tfe::candidate(a, minVal, maxVal, cand, delta, offset);
+        const double cost = valid ? tfe::wave_cost(view, a, delta, offset, lane, term_all[wave]) : 0.0;
         if (lane == 0)
         {
             st->cand_delta[cand]  = delta;
@@ -1001,28 +807,16 @@ __global__ __launch_bounds__(kBlock) void tfe_search_kernel(DevState* st, Search
         st->ticket_search = 0;
         st->n_cand        = st->initialized ? a.n_cand : 0;
     }
+    double enc[4] = {0, 0, 0, 0};
     if (!st->initialized)
     {
         if (lane == 0)
         {
             st->best_index = -1;
             if (st->stats_updated)
-            {
-                // only zeros were seen: DLQ/src/TfEnhancedEncodingAnalyzer.cpp:85-100
-                const float ns    = a.step_size_cost;
-                double mn = -1, mx = 1;
-                const double d = (mx - mn) / (int) ns;
-                const double o = floor(mn / d);
-                mn             = o * d;
-                mx             = mn + (int) ns * d;
-                st->enc_min = mn, st->enc_max = mx, st->enc_delta = d, st->enc_offset = o;
-                st->enc_bw = a.bw;
-            }
-            else
-            {
-                st->enc_min = st->enc_max = st->enc_delta = st->enc_offset = 0;
-                st->enc_bw                                                = 0;
-            }
+                tfe::encoding_of_zeros(a, enc);
+            st->enc_min = enc[0], st->enc_max = enc[1], st->enc_delta = enc[2], st->enc_offset = enc[3];
+            st->enc_bw = st->stats_updated ? a.bw : 0;
         }
         return;
     }
@@ -1060,15 +854,10 @@ __global__ __launch_bounds__(kBlock) void tfe_search_kernel(DevState* st, Search
         }
         else
             bidx = -1;
-        // DLQ/src/TfEnhancedEncodingAnalyzer.cpp:383-396
-        const float bMin = std_max(bestDelta * (float) bestOffset, -FLT_MAX);
-        const float bMax = std_min(bestDelta * ((float) bestOffset + a.num_steps_cand), FLT_MAX);
-        st->enc_delta    = bestDelta;
-        st->enc_offset   = bestOffset;
-        st->enc_bw       = a.bw;
-        st->enc_min      = bMin;
-        st->enc_max      = bMax;
-        st->best_index   = bidx;
+        tfe::encoding_of(a, bestDelta, bestOffset, enc);
+        st->enc_min = enc[0], st->enc_max = enc[1], st->enc_delta = enc[2], st->enc_offset = enc[3];
+        st->enc_bw     = a.bw;
+        st->best_index = bidx;
     }
 }
 
@@ -1084,7 +873,8 @@ __global__ void reset_state_kernel(DevState* st)
         st->acc_max       = -DBL_MAX;
         st->initialized = st->iterations = 0;
         st->iters[0] = st->iters[1] = 0;
-        st->bucket_f = st->pdf_offset_f = 0.f;
+        st->bucket_f = st->pdf_offset_f = st->range_min = 0.f;
+        st->range_bucket                = 0;
         st->n_cand                      = 0;
         st->best_index                  = -1;
         st->enc_min = st->enc_max = st->enc_delta = st->enc_offset = 0;
@@ -1140,6 +930,75 @@ int stream_grid(int64_t n)
     return (int) blocks;
 }
 }   // namespace
+
+// PercentileEncodingAnalyzer<float>::computeEncoding on the PDF read back from the device
+// (DLQ/src/PercentileEncodingAnalyzer.cpp:78-198; findOriginalRange: DLQ/src/math_functions.cpp:400-433).
+// 512 buckets of host arithmetic, in the reference's types: float range values, double cdf.
+int percentile_encoding_host(bool initialized, const double* x_left, const double* pdf, float percentile, int bw, int sym,
+                             int strict, int uns, miq_encoding* out)
+{
+    float num_steps = (float) (std::pow(2, bw) - 1);
+    if (sym && strict)
+        num_steps -= 1;
+    if (!initialized)
+    {
+        // only zeros were seen: an encoding that covers float 0
+        out->min    = -1;
+        out->max    = 1;
+        out->delta  = (out->max - out->min) / (int) num_steps;
+        out->offset = std::floor(out->min / out->delta);
+        out->min    = out->offset * out->delta;
+        out->max    = out->min + (int) num_steps * out->delta;
+        out->bw     = bw;
+        return MIQ_OK;
+    }
+    float min_val = (float) x_left[0], max_val = (float) x_left[kPdf - 1];
+    for (int i = 0; i < kPdf; ++i)
+        if (pdf[i] > 0)
+        {
+            min_val = (float) x_left[i];
+            break;
+        }
+    for (int i = kPdf - 1; i > 0; --i)
+        if (pdf[i] > 0)
+        {
+            max_val = (float) x_left[i];
+            break;
+        }
+    min_val = std::min(min_val, 0.0f);
+    max_val = std::max(max_val, 0.0f);
+    max_val = std::max(max_val, min_val + (float) 0.01);
+    float a_min = min_val, a_max = max_val;
+    if (percentile != 100.0f)
+    {
+        const float width = (float) (x_left[1] - x_left[0]);
+        a_min             = (float) x_left[0];
+        a_max             = (float) (x_left[kPdf - 1] + width);
+        std::vector<double> cdf(pdf, pdf + kPdf);
+        for (int i = 1; i < kPdf; ++i)
+            cdf[i] += cdf[i - 1];
+        const float left = 1 - percentile / 100;
+        for (int i = 0; i < kPdf; ++i)
+            if (cdf[i] >= left)
+            {
+                a_min = (float) x_left[i];
+                break;
+            }
+        const float right = percentile / 100;
+        for (int i = kPdf - 1; i >= 0; --i)
+            if (cdf[i] < right && x_left[i] < max_val)
+            {
+                a_max = (float) (x_left[i] + width);
+                break;
+            }
+        if (a_min == a_max)
+            a_max += width;
+    }
+    a_min = std::min(a_min, 0.0f);
+    a_max = std::max(a_max, 0.0f);
+    return miq_get_computed_encodings(bw, a_min, a_max, sym, strict, uns, out);
+}
+
 }   // namespace miq
 
 using namespace miq;
@@ -1282,72 +1141,10 @@ int miq_minmax_per_channel_static_f32(const float* in, int64_t num_channel, int6
                               reinterpret_cast<uint32_t*>(out_min_max), ws, (hipStream_t) stream);
 }
 
-// PercentileEncodingAnalyzer<float>::computeEncoding on the PDF read back from the device
-// (DLQ/src/PercentileEncodingAnalyzer.cpp:78-198; findOriginalRange: DLQ/src/math_functions.cpp:400-433).
-// 512 buckets of host arithmetic, in the reference's types: float range values, double cdf.
 static int percentile_encoding(const DevState* h, float percentile, int bw, int sym, int strict, int uns,
                                miq_encoding* out)
 {
-    float num_steps = (float) (std::pow(2, bw) - 1);
-    if (sym && strict)
-        num_steps -= 1;
-    if (!h->initialized)
-    {
-        // only zeros were seen: an encoding that covers float 0
-        out->min    = -1;
-        out->max    = 1;
-        out->delta  = (out->max - out->min) / (int) num_steps;
-        out->offset = std::floor(out->min / out->delta);
-        out->min    = out->offset * out->delta;
-        out->max    = out->min + (int) num_steps * out->delta;
-        out->bw     = bw;
-        return MIQ_OK;
-    }
-    float min_val = (float) h->xLeft[0], max_val = (float) h->xLeft[kPdf - 1];
-    for (int i = 0; i < kPdf; ++i)
-        if (h->pdf[i] > 0)
-        {
-            min_val = (float) h->xLeft[i];
-            break;
-        }
-    for (int i = kPdf - 1; i > 0; --i)
-        if (h->pdf[i] > 0)
-        {
-            max_val = (float) h->xLeft[i];
-            break;
-        }
-    min_val = std::min(min_val, 0.0f);
-    max_val = std::max(max_val, 0.0f);
-    max_val = std::max(max_val, min_val + (float) 0.01);
-    float a_min = min_val, a_max = max_val;
-    if (percentile != 100.0f)
-    {
-        const float width = (float) (h->xLeft[1] - h->xLeft[0]);
-        a_min             = (float) h->xLeft[0];
-        a_max             = (float) (h->xLeft[kPdf - 1] + width);
-        std::vector<double> cdf(h->pdf, h->pdf + kPdf);
-        for (int i = 1; i < kPdf; ++i)
-            cdf[i] += cdf[i - 1];
-        const float left = 1 - percentile / 100;
-        for (int i = 0; i < kPdf; ++i)
-            if (cdf[i] >= left)
-            {
-                a_min = (float) h->xLeft[i];
-                break;
-            }
-        const float right = percentile / 100;
-        for (int i = kPdf - 1; i >= 0; --i)
-            if (cdf[i] < right && h->xLeft[i] < max_val)
-            {
-                a_max = (float) (h->xLeft[i] + width);
-                break;
-            }
-        if (a_min == a_max)
-            a_max += width;
-    }
-    a_min = std::min(a_min, 0.0f);
-    a_max = std::max(a_max, 0.0f);
-    return miq_get_computed_encodings(bw, a_min, a_max, sym, strict, uns, out);
+    return percentile_encoding_host(h->initialized != 0, h->xLeft, h->pdf, percentile, bw, sym, strict, uns, out);
 }
 
 int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
@@ -1565,33 +1362,7 @@ int miq_analyzer_compute_encoding(miq_analyzer* a, int bw, int use_symmetric, in
         return percentile_encoding(static_cast<const DevState*>(a->pinned), a->percentile, bw, use_symmetric,
                                    use_strict_symmetric, use_unsigned_symmetric, out);
     }
-    SearchArgs sa{};
-    sa.bw             = bw;
-    sa.sym            = use_symmetric ? 1 : 0;
-    sa.strict         = use_strict_symmetric ? 1 : 0;
-    sa.uns            = use_unsigned_symmetric ? 1 : 0;
-    sa.step_size_cost = (float) (std::pow(2, bw) - 1);
-    sa.num_steps_cand = sa.step_size_cost;
-    if (sa.sym && sa.strict)
-        sa.num_steps_cand -= 1;
-    if (sa.sym)
-    {
-        // the delta factor advances by adding the double 0.01 to a float; how many steps fit below 1.01 is decided
-        // by that float arithmetic (DLQ/src/TfEnhancedEncodingAnalyzer.cpp:248)
-        int cnt = 0;
-        for (float f = (float) (1.0 / 100); (double) f <= 1 + 1.0 / 100; f = (float) ((double) f + 1.0 / 100))
-            ++cnt;
-        sa.n_delta = cnt;
-        sa.n_cand  = cnt;
-    }
-    else
-    {
-        int cnt = 0;
-        for (float f = (float) (1.0 / 16); (double) f <= 1 + 1.0 / 16; f = (float) ((double) f + 1.0 / 16))
-            ++cnt;
-        sa.n_delta = cnt;
-        sa.n_cand  = cnt * 21 + 1;
-    }
+    const SearchArgs sa = tfe::make_search_args(bw, use_symmetric, use_strict_symmetric, use_unsigned_symmetric);
     MIQ_CHECK_ARG(sa.n_cand <= kMaxCand, "internal: candidate grid too large");
     if (int rc = flush_pending(a, s))
         return rc;

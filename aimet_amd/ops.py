@@ -650,3 +650,71 @@ class Analyzer:
             check(lib.miq_analyzer_last_search(self._h, d.ctypes.data, o.ctypes.data, c.ctypes.data, cap, C.byref(n),
                                                C.byref(best), self._s()))
         return d[:n.value], o[:n.value], c[:n.value], best.value
+
+
+class ChannelAnalyzer:
+    """Device-resident per-channel TF-Enhanced (mode 1) / percentile (mode 2) analyzer: one 512-bucket PDF per channel of
+    a tensor laid out [outer][channels][n_per_channel], one launch sequence per update, one search launch for all
+    channels.  Channel c behaves like an `Analyzer` fed ``tensor.select(axis, c)``.  The state is a torch tensor
+    (torch's caching allocator); nothing is allocated per channel."""
+
+    def __init__(self, mode, num_channel, device=None):
+        self.mode, self.num_channel = int(mode), int(num_channel)
+        self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        if self.device.type != "cuda":
+            raise RuntimeError("a ChannelAnalyzer lives on a GPU")
+        if self.device.index is None:
+            self.device = torch.device("cuda", torch.cuda.current_device())
+        nbytes = int(lib.miq_channel_analyzer_state_bytes(self.num_channel))
+        self._state = torch.empty(nbytes // 8 + 1, dtype=torch.float64, device=self.device)
+        h = C.c_void_p()
+        with torch.cuda.device(self.device):
+            check(lib.miq_channel_analyzer_create(self.mode, self.num_channel, _ptr(self._state), self._s(),
+                                                  C.byref(h)))
+        self._h = h
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h and lib is not None:
+            lib.miq_channel_analyzer_destroy(h)
+
+    def _s(self):
+        return C.c_void_p(_stream_of(self.device))
+
+    def reset(self):
+        with torch.cuda.device(self.device):
+            check(lib.miq_channel_analyzer_reset(self._h, self._s()))
+
+    def set_percentile(self, percentile: float):
+        check(lib.miq_channel_analyzer_set_percentile(self._h, float(percentile)))
+
+    def update_stats(self, x, n_per_channel):
+        """x: float32 GPU tensor whose flat layout is [outer][num_channel][n_per_channel]."""
+        if not x.is_cuda or x.device != self.device:
+            raise RuntimeError(f"analyzer lives on {self.device}, tensor on {x.device}")
+        if x.dtype != _F32 or not x.is_contiguous():
+            x = x.to(_F32).contiguous()
+        ws = _minmax_workspace(self.num_channel, x.numel(), int(n_per_channel), x.device)
+        with torch.cuda.device(self.device):
+            check(lib.miq_channel_analyzer_update_stats_f32(self._h, _ptr(x), x.numel(), int(n_per_channel), _ptr(ws),
+                                                            self._s()))
+
+    def compute_encodings(self, bw, symmetric=False, strict_symmetric=False, unsigned_symmetric=False):
+        """returns (list of Encoding, one per channel; is_valid)"""
+        encs = (Encoding * self.num_channel)()
+        valid = C.c_int(0)
+        with torch.cuda.device(self.device):
+            check(lib.miq_channel_analyzer_compute_encodings(self._h, int(bw), int(bool(symmetric)),
+                                                             int(bool(strict_symmetric)),
+                                                             int(bool(unsigned_symmetric)), encs, C.byref(valid),
+                                                             self._s()))
+        return list(encs), bool(valid.value)
+
+    def get_stats_histogram(self, channel):
+        import numpy as np
+        xl, pdf = np.zeros(_lib.PDF_SIZE), np.zeros(_lib.PDF_SIZE)
+        n = C.c_int(0)
+        with torch.cuda.device(self.device):
+            check(lib.miq_channel_analyzer_get_stats_histogram(self._h, int(channel), xl.ctypes.data, pdf.ctypes.data,
+                                                               C.byref(n), self._s()))
+        return xl[:n.value], pdf[:n.value]

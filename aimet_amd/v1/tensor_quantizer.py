@@ -134,7 +134,7 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         state['_num_ops'] = len(self._cppOp)
         state['_encoding'] = None if self._encoding is None else \
             [(e.min, e.max, e.delta, e.offset, e.bw) for e in self._encoding]
-        for key in ('_cppOp', '_dev_params', '_fp8_grid'):
+        for key in ('_cppOp', '_dev_params', '_fp8_grid', '_channel_analyzer'):
             state.pop(key, None)
         return state
 
@@ -146,6 +146,8 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         self._encoding = None if encoding is None else [libpymo.TfEncoding(*e) for e in encoding]
         self._dev_params = None
         self._fp8_grid = None
+        if '_tf_minmax' in state:
+            self._channel_analyzer = None
 
     @property
     def quant_scheme(self) -> QuantScheme:
@@ -287,6 +289,8 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
         self._ch_axis = ch_axis
         self._dev_params = None      # (min, max, delta, offset, raw_min, raw_max) device vectors of the encoding
         self._tf_minmax = None       # fused per-channel running min/max for the TF scheme: device tensor [2, C]
+        self._channel_analyzer = None   # TF-Enhanced / percentile: every channel's PDF in one device object
+        self._percentile_value = 100.0
 
     @property
     def channel_axis(self) -> int:
@@ -296,9 +300,32 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
         super().reset_encoding_stats()
         if not self._is_encoding_frozen:
             self._tf_minmax = None
+            if self._channel_analyzer is not None:
+                self._channel_analyzer.reset()
 
     def _drop_fused_stats(self):
         self._tf_minmax = None
+        self._channel_analyzer = None
+
+    def set_percentile_value(self, percentile_value: float):
+        super().set_percentile_value(percentile_value)
+        if self._quant_scheme == QuantScheme.post_training_percentile:
+            self._percentile_value = float(percentile_value)
+            if self._channel_analyzer is not None:
+                self._channel_analyzer.set_percentile(self._percentile_value)
+
+    def get_stats_histogram(self) -> List[List]:
+        if self._channel_analyzer is None:
+            return super().get_stats_histogram()
+        if self._quant_scheme != QuantScheme.post_training_tf_enhanced:
+            raise RuntimeError("get_stats_histogram() can be invoked only when quantization scheme is TF-Enhanced.")
+        if not self._encoding:
+            raise RuntimeError("get_stats_histogram() can be invoked only when encoding is computed.")
+        out = []
+        for channel in range(self._channel_analyzer.num_channel):
+            x_left, pdf = self._channel_analyzer.get_stats_histogram(channel)
+            out.append(list(zip(x_left.tolist(), pdf.tolist())))
+        return out
 
     def update_encoding_stats(self, tensor: torch.Tensor):
         if self.enabled and not self._is_encoding_frozen:
@@ -325,12 +352,26 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
                     self._tf_minmax = torch.stack((torch.minimum(self._tf_minmax[0], mm[0]),
                                                    torch.maximum(self._tf_minmax[1], mm[1])))
                 return
-            for channel_idx, op in enumerate(self._cppOp):
-                tensor_slice = tensor.select(self._ch_axis, channel_idx).contiguous(
-                    memory_format=torch.contiguous_format)
-                op.updateStats(tensor_slice, tensor.is_cuda)
+            # TF-Enhanced / percentile: the reference feeds one analyzer object per channel with
+            # tensor.select(ch_axis, c).contiguous() (:567-570); here one device object holds every channel's PDF and
+            # one launch sequence updates them all -- channel c sees exactly the samples of that slice
+            if not tensor.is_cuda:
+                raise RuntimeError("aimet_amd computes on the GPU only: pass a GPU tensor")
+            num_channel = tensor.shape[self._ch_axis]
+            n_per_channel = functools.reduce(lambda a, b: a * b, tensor.shape[self._ch_axis + 1:], 1)
+            analyzer = self._channel_analyzer
+            if analyzer is None or analyzer.device != tensor.device or analyzer.num_channel != num_channel:
+                mode = 1 if self._quant_scheme == QuantScheme.post_training_tf_enhanced else 2
+                analyzer = ops.ChannelAnalyzer(mode, num_channel, tensor.device)
+                analyzer.set_percentile(self._percentile_value)
+                self._channel_analyzer = analyzer
+            analyzer.update_stats(tensor, n_per_channel)
 
     def _compute_op_encodings(self):
+        if self._channel_analyzer is not None:
+            encodings, valid = self._channel_analyzer.compute_encodings(
+                self.bitwidth, self.use_symmetric_encodings, self.use_strict_symmetric, self.use_unsigned_symmetric)
+            return [(libpymo.TfEncoding(e.min, e.max, e.delta, e.offset, e.bw), valid) for e in encodings]
         if self._tf_minmax is None:
             return super()._compute_op_encodings()
         # TfEncodingAnalyzer::computeEncoding per channel (DlQuantization/src/TfEncodingAnalyzer.cpp:80-101) on the

@@ -265,6 +265,36 @@ int miq_analyzer_last_search(miq_analyzer* a, float* deltas /* host */, int32_t*
                              double* costs /* host */, int cap, int* count /* host */, int* best_index /* host */,
                              void* stream);
 
+/* Per-channel TF-Enhanced / percentile analyzer: C independent 512-bucket PDFs over the channels of one tensor,
+ * channel(i) = (i / num_element_per_channel) % num_channel, updated by one launch sequence per batch and searched by
+ * one launch.  It replaces the reference's list of per-channel analyzer objects fed slice by slice
+ * (TrainingExtensions/torch/src/python/aimet_torch/v1/tensor_quantizer.py:535-570, each an
+ * IQuantizationEncodingAnalyzer<float> behind TrainingExtensions/torch/src/AimetTensorQuantizer.cpp:85-126, 180-192):
+ * channel c's PDF and encoding are those a miq_analyzer fed `tensor.select(axis, c).contiguous()` produces.
+ * quantization_mode: MIQ_QUANTIZATION_TF_ENHANCED or MIQ_QUANTIZATION_PERCENTILE.
+ * device_state: device memory of miq_channel_analyzer_state_bytes(num_channel) bytes, 16-byte aligned, owned by the
+ * caller and alive as long as the object (so that it can come from the caller's own allocator), or NULL to let the
+ * library allocate it.  workspace (update_stats): device memory of miq_channel_analyzer_workspace_bytes(...) bytes, or
+ * NULL (slower min/max pass).  update_stats enqueues work and never synchronises; compute_encodings and
+ * get_stats_histogram synchronise `stream` once.  out (compute_encodings): host miq_encoding[num_channel]. */
+typedef struct miq_channel_analyzer miq_channel_analyzer;
+int64_t miq_channel_analyzer_state_bytes(int64_t num_channel);
+int64_t miq_channel_analyzer_workspace_bytes(int64_t num_channel, int64_t num_element,
+                                             int64_t num_element_per_channel);
+int miq_channel_analyzer_create(int quantization_mode, int64_t num_channel, void* device_state, void* stream,
+                                miq_channel_analyzer** out);
+int miq_channel_analyzer_destroy(miq_channel_analyzer* a);
+int miq_channel_analyzer_reset(miq_channel_analyzer* a, void* stream);
+int miq_channel_analyzer_set_percentile(miq_channel_analyzer* a, float percentile);
+int miq_channel_analyzer_update_stats_f32(miq_channel_analyzer* a, const float* data, int64_t num_element,
+                                          int64_t num_element_per_channel, void* workspace, void* stream);
+int miq_channel_analyzer_compute_encodings(miq_channel_analyzer* a, int bw, int use_symmetric,
+                                           int use_strict_symmetric, int use_unsigned_symmetric,
+                                           miq_encoding* out /* host[num_channel] */, int* is_valid /* host */,
+                                           void* stream);
+int miq_channel_analyzer_get_stats_histogram(miq_channel_analyzer* a, int64_t channel, double* x_left /* host[512] */,
+                                             double* pdf /* host[512] */, int* num_buckets /* host */, void* stream);
+
 /* ---------------------------------------------------------------------------------------------------------------
  * AdaRound (ADA = TrainingExtensions/torch/src/python/aimet_torch/v1/adaround)
  *

@@ -1,0 +1,166 @@
+"""The per-channel TF-Enhanced / percentile analyzer (one device object for all channels of a tensor) against the CPU
+oracle fed channel by channel, through the C ABI: channel c must see exactly the samples of tensor.select(axis, c)
+-- the reference's per-channel flow (TrainingExtensions/torch/src/python/aimet_torch/v1/tensor_quantizer.py:535-570)
+-- and produce that slice's PDF (bit for bit) and encoding (every field)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TFE, PERCENTILE = 1, 2
+MODES = ((8, 0, 0, 0), (8, 1, 0, 0), (8, 1, 1, 0), (8, 1, 0, 1), (4, 1, 0, 0), (4, 0, 0, 0))
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from aimet_amd import ops as o
+    return o
+
+
+def _laplace(rng, shape):
+    u = rng.random(shape) - 0.5
+    w = (-0.02 * np.sign(u) * np.log(1 - 2 * np.abs(u))).astype(np.float32)
+    w[rng.random(shape) < 0.001] *= 20
+    return w
+
+
+def _check(ops, oracle, batches, c, npc, mode=TFE, percentile=99.9, modes=MODES, channels=None):
+    """batches: arrays of shape [outer, c, npc]"""
+    an = ops.ChannelAnalyzer(mode, c)
+    if mode == PERCENTILE:
+        an.set_percentile(percentile)
+    pdfs = [oracle.new_pdf() for _ in range(c)]
+    for b in batches:
+        an.update_stats(torch.from_numpy(np.ascontiguousarray(b)).cuda(), npc)
+        for ch in range(c):
+            pdfs[ch].update(np.ascontiguousarray(b[:, ch, :]).reshape(-1))
+    for ch in (range(c) if channels is None else channels):
+        xl, p = an.get_stats_histogram(ch)
+        if pdfs[ch].initialized:
+            assert np.array_equal(xl.view(np.uint64), pdfs[ch].x_left().view(np.uint64)), ch
+            assert np.array_equal(p.view(np.uint64), pdfs[ch].pdf().view(np.uint64)), ch
+        else:
+            assert xl.size == 0
+    for bw, sym, strict, uns in modes:
+        encs, valid = an.compute_encodings(bw, sym, strict, uns)
+        assert valid and len(encs) == c
+        for ch in (range(c) if channels is None else channels):
+            if mode == TFE:
+                want = pdfs[ch].compute_encoding(bw, sym, strict, uns)[0]
+            else:
+                want = pdfs[ch].compute_percentile_encoding(bw, percentile, sym, strict, uns)
+            e = encs[ch]
+            assert (e.min, e.max, e.delta, e.offset, e.bw) == want.astuple(), (ch, bw, sym, strict, uns)
+    return an
+
+
+@pytest.mark.parametrize("outer,c,npc", [(1, 48, 1024), (1, 16, 4608), (3, 5, 300), (2, 7, 9), (1, 3, 40000),
+                                         (1, 1, 5000), (4, 6, 1030), (1, 33, 2)])
+def test_channel_analyzer_matches_per_slice_oracle(ops, oracle, outer, c, npc):
+    """Every layout: one workgroup per channel (weights), an outer dimension in front of the channel axis (transposed
+    convolutions, activations), rows that are not a multiple of the vector width, rows longer than one workgroup's
+    share, tiny rows; two batches, the second with values outside the first one's range."""
+    rng = np.random.default_rng(outer * 100 + c + npc)
+    b0 = _laplace(rng, (outer, c, npc))
+    b1 = _laplace(rng, (outer, c, npc)) * 1.5
+    b1.reshape(-1)[::53] = np.nan
+    _check(ops, oracle, [b0, b1], c, npc)
+
+
+def test_channel_analyzer_special_channels(ops, oracle):
+    """Channels that are all zero (no range: the reference's -1 .. 1 encoding), constant, all zero first and data
+    later, next to ordinary ones; post-ReLU-like data with a heavy tail."""
+    rng = np.random.default_rng(3)
+    c, npc = 8, 2048
+    b0 = np.abs(rng.standard_normal((1, c, npc))).astype(np.float32)
+    b1 = np.abs(rng.standard_normal((1, c, npc))).astype(np.float32)
+    b0[0, 0] = 0
+    b1[0, 0] = 0                      # never anything but zeros
+    b0[0, 1] = 4.0
+    b1[0, 1] = 4.0                    # constant
+    b0[0, 2] = 0                      # zeros first, data in the second batch
+    b0[0, 3, ::7] *= 40               # outliers
+    b1[0, 4] = -b1[0, 4] - 0.25       # negative only
+    an = _check(ops, oracle, [b0, b1], c, npc)
+    xl, p = an.get_stats_histogram(0)
+    assert xl.size == 0
+    an.reset()
+    encs, valid = an.compute_encodings(8)
+    assert not valid
+
+
+@pytest.mark.parametrize("percentile", [100.0, 99.9, 90.0])
+def test_channel_analyzer_percentile(ops, oracle, percentile):
+    rng = np.random.default_rng(int(percentile))
+    c, npc = 12, 3000
+    batches = [(rng.standard_normal((2, c, npc)) * (1 + b)).astype(np.float32) for b in range(2)]
+    _check(ops, oracle, batches, c, npc, mode=PERCENTILE, percentile=percentile,
+           modes=((8, 0, 0, 0), (8, 1, 0, 0), (4, 1, 1, 0)))
+
+
+def test_cfg2_largest_weight_per_channel_tf_enhanced(ops, oracle):
+    """[11008, 4096] Laplace(0, 0.02) weights with 0.1 % outliers x20, TF-Enhanced per output channel in one update and
+    one search: every channel's PDF equals the oracle's for that row, and the symmetric 8-bit and 4-bit encodings of
+    every 16th channel (688 searches on the CPU) equal the oracle's field for field."""
+    c, npc = 11008, 4096
+    rng = np.random.default_rng(1004)
+    w = _laplace(rng, (c, npc))
+    an = ops.ChannelAnalyzer(TFE, c)
+    an.update_stats(torch.from_numpy(w).cuda(), npc)
+    enc8, valid = an.compute_encodings(8, True, False, False)
+    enc4, _ = an.compute_encodings(4, True, False, False)
+    assert valid
+    state_pdf = None
+    for ch in range(c):
+        pdf = oracle.new_pdf()
+        pdf.update(w[ch])
+        if ch % 16 == 0:
+            xl, p = an.get_stats_histogram(ch)
+            assert np.array_equal(xl.view(np.uint64), pdf.x_left().view(np.uint64)), ch
+            assert np.array_equal(p.view(np.uint64), pdf.pdf().view(np.uint64)), ch
+            for encs, bw in ((enc8, 8), (enc4, 4)):
+                want = pdf.compute_encoding(bw, True, False, False)[0]
+                e = encs[ch]
+                assert (e.min, e.max, e.delta, e.offset, e.bw) == want.astuple(), (ch, bw)
+    # every channel: a symmetric encoding around zero inside the row's 3x-widened range
+    amax = np.abs(w).max(axis=1)
+    for ch in range(c):
+        e = enc8[ch]
+        assert e.delta > 0 and e.min < 0 < e.max and e.max <= 3.1 * amax[ch]
+
+
+def test_per_channel_quantizer_uses_one_device_object(ops):
+    """StaticGridPerChannelQuantizer with the TF-Enhanced scheme: same encodings as one single-tensor analyzer per
+    channel slice (the reference's flow), histograms per channel, scheme switch drops the statistics."""
+    from aimet_amd.common import libpymo
+    from aimet_amd.common.AimetTensorQuantizer import AimetTensorQuantizer
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.tensor_quantizer import StaticGridPerChannelQuantizer
+    torch.manual_seed(4)
+    for shape, axis in (((24, 40, 3, 3), 0), ((10, 16, 3, 3), 1)):
+        w = (torch.randn(shape) * 0.05).cuda()
+        q = StaticGridPerChannelQuantizer(8, libpymo.RoundingMode.ROUND_NEAREST, QuantScheme.post_training_tf_enhanced,
+                                          use_symmetric_encodings=True, num_channels=shape[axis],
+                                          enabled_by_default=True, ch_axis=axis)
+        q.update_encoding_stats(w)
+        q.compute_encoding()
+        assert len(q.encoding) == shape[axis] and q._channel_analyzer is not None     # pylint: disable=protected-access
+        hist = q.get_stats_histogram()
+        assert len(hist) == shape[axis] and len(hist[0]) == 512
+        for ch in range(shape[axis]):
+            single = AimetTensorQuantizer(libpymo.QuantizationMode.QUANTIZATION_TF_ENHANCED)
+            single.updateStats(w.select(axis, ch).contiguous(), True)
+            want, valid = single.getEncoding(8, True, False, False)
+            got = q.encoding[ch]
+            assert valid and (got.min, got.max, got.delta, got.offset) == (want.min, want.max, want.delta, want.offset)
+            assert hist[ch] == single.getStatsHistogram()
+        y = q.quantize_dequantize(w, libpymo.RoundingMode.ROUND_NEAREST)
+        assert torch.isfinite(y).all() and (y - w).abs().max() < 0.05
+        q.reset_encoding_stats()
+        q.quant_scheme = QuantScheme.post_training_percentile
+        assert q._channel_analyzer is None                                            # pylint: disable=protected-access
+        q.set_percentile_value(99.0)
+        q.update_encoding_stats(w)
+        q.compute_encoding()
+        assert max(e.max for e in q.encoding) < float(w.abs().max())                  # the tails are cut
