@@ -65,6 +65,8 @@ _SIGNATURES = {
     "miq_minmax_per_channel_f32": ([_p, _i64, _i64, _i64, _p, _p, _p], _int),
     "miq_minmax_per_channel_static_f32": ([_p, _i64, _i64, _i64, _p, _p], _int),
     "miq_analyzer_create": ([_int, C.POINTER(_p)], _int),
+    "miq_analyzer_state_bytes": ([], _i64),
+    "miq_analyzer_create_in": ([_int, _p, C.POINTER(_p)], _int),
     "miq_analyzer_set_percentile": ([_p, C.c_float], _int),
     "miq_analyzer_destroy": ([_p], _int),
     "miq_analyzer_reset": ([_p, _p], _int),

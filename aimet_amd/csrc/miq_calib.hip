@@ -1010,6 +1010,8 @@ struct miq_analyzer
     int device;
     DevState* st;        // device
     void* pinned;        // host staging (pinned) for read-backs
+    bool owns_state;     // st was allocated here (no caller memory given)
+    bool needs_reset;    // st has not been cleared yet: the first call that queues work does it
     bool stats_updated;  // host mirror of _isEncodingValid / _statsUpdated
     bool range_known;    // host knows the PDF range has been fixed, so no further min/max pass is queued
     int* probe_flag;     // pinned host words the histogram kernel writes once the range is fixed:
@@ -1147,9 +1149,33 @@ static int percentile_encoding(const DevState* h, float percentile, int bw, int 
     return percentile_encoding_host(h->initialized != 0, h->xLeft, h->pdf, percentile, bw, sym, strict, uns, out);
 }
 
+int64_t miq_analyzer_state_bytes(void)
+{
+    return (int64_t) sizeof(DevState);
+}
+
+// The state is cleared by the first call that queues work (on that call's stream): creation itself queues nothing and
+// waits for nothing.
+static int ensure_reset(miq_analyzer* a, hipStream_t s)
+{
+    if (a->needs_reset)
+    {
+        hipLaunchKernelGGL(reset_state_kernel, dim3(1), dim3(kPdf), 0, s, a->st);
+        MIQ_CHECK_LAUNCH();
+        a->needs_reset = false;
+    }
+    return MIQ_OK;
+}
+
 int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
 {
+    return miq_analyzer_create_in(quantization_mode, nullptr, out);
+}
+
+int miq_analyzer_create_in(int quantization_mode, void* device_state, miq_analyzer** out)
+{
     MIQ_CHECK_ARG(out != nullptr, "null output handle");
+    MIQ_CHECK_ARG(device_state == nullptr || aligned16(device_state), "device_state must be 16-byte aligned");
     if (quantization_mode != MIQ_QUANTIZATION_TF && quantization_mode != MIQ_QUANTIZATION_TF_ENHANCED &&
         quantization_mode != MIQ_QUANTIZATION_PERCENTILE)
     {
@@ -1160,7 +1186,9 @@ int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
     MIQ_CHECK_ARG(a != nullptr, "out of host memory");
     a->mode          = quantization_mode;
     a->percentile    = 100.0f;   // PercentileEncodingAnalyzer.h: the default clips nothing
-    a->st            = nullptr;
+    a->st            = static_cast<DevState*>(device_state);
+    a->owns_state    = (device_state == nullptr);
+    a->needs_reset   = true;
     a->pinned        = nullptr;
     a->stats_updated = false;
     a->range_known   = false;
@@ -1172,7 +1200,7 @@ int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
     a->seq           = 0;
     a->last_bw       = 0;
     hipError_t e     = hipGetDevice(&a->device);
-    if (e == hipSuccess)
+    if (e == hipSuccess && a->owns_state)
         e = hipMalloc((void**) &a->st, sizeof(DevState));
     if (e == hipSuccess)
         e = hipHostMalloc(&a->pinned, kInspectBytes + 64, hipHostMallocDefault);   // + 4 probe words
@@ -1185,20 +1213,10 @@ int miq_analyzer_create(int quantization_mode, miq_analyzer** out)
     if (e != hipSuccess)
     {
         set_error("analyzer allocation failed: %s", hipGetErrorString(e));
-        if (a->st)
+        if (a->st && a->owns_state)
             (void) hipFree(a->st);
         if (a->pinned)
             (void) hipHostFree(a->pinned);
-        delete a;
-        return MIQ_ERR_HIP;
-    }
-    hipLaunchKernelGGL(reset_state_kernel, dim3(1), dim3(kPdf), 0, (hipStream_t) nullptr, a->st);
-    e = hipStreamSynchronize(nullptr);
-    if (e != hipSuccess)
-    {
-        set_error("analyzer initialisation failed: %s", hipGetErrorString(e));
-        (void) hipFree(a->st);
-        (void) hipHostFree(a->pinned);
         delete a;
         return MIQ_ERR_HIP;
     }
@@ -1219,7 +1237,8 @@ int miq_analyzer_destroy(miq_analyzer* a)
 {
     if (!a)
         return MIQ_OK;
-    (void) hipFree(a->st);
+    if (a->owns_state)
+        (void) hipFree(a->st);
     (void) hipHostFree(a->pinned);
     delete a;
     return MIQ_OK;
@@ -1230,6 +1249,7 @@ int miq_analyzer_reset(miq_analyzer* a, void* stream)
     MIQ_CHECK_ARG(a != nullptr, "null analyzer");
     hipLaunchKernelGGL(reset_state_kernel, dim3(1), dim3(kPdf), 0, (hipStream_t) stream, a->st);
     MIQ_CHECK_LAUNCH();
+    a->needs_reset = false;
     a->stats_updated = false;
     a->range_known   = false;
     a->seq           = 0;
@@ -1245,6 +1265,8 @@ int miq_analyzer_update_stats_f32(miq_analyzer* a, const float* data, int64_t n,
     MIQ_CHECK_ARG(n > 0 && data, "update_stats needs a non-empty tensor");
     hipStream_t s  = (hipStream_t) stream;
     const bool vec = aligned16(data);
+    if (int rc = ensure_reset(a, s))
+        return rc;
     a->stats_updated = true;
     const int grid    = stream_grid(n);
     const int mm_grid = (int) std::max<int64_t>(
@@ -1320,6 +1342,8 @@ static int flush_pending(miq_analyzer* a, hipStream_t s)
 
 static int read_state(miq_analyzer* a, hipStream_t s, size_t bytes = kInspectBytes)
 {
+    if (int rc = ensure_reset(a, s))
+        return rc;
     MIQ_CHECK_HIP(hipMemcpyAsync(a->pinned, a->st, bytes, hipMemcpyDeviceToHost, s));
     MIQ_CHECK_HIP(hipStreamSynchronize(s));
     const DevState* h = static_cast<const DevState*>(a->pinned);

@@ -569,7 +569,21 @@ def adaround_linear_bwd_adam(weight_floor, grad_out, x, row_index, alpha, exp_av
                  int(step), _ptr(reg_partial), _stream(weight_floor)))
 
 
-class Analyzer:
+class _StateOwner:
+    """Keeps a device-state tensor (torch's caching allocator) safe when the object is used on several streams: the
+    allocator may hand the block to someone else as soon as the tensor dies, unless it knows which streams used it."""
+
+    def _init_state(self, nbytes):
+        self._state = torch.empty(int(nbytes) // 8 + 1, dtype=torch.float64, device=self.device)
+        self._streams_seen = {_stream_of(self.device)}
+
+    def _note_stream(self, handle):
+        if handle not in self._streams_seen:
+            self._streams_seen.add(handle)
+            self._state.record_stream(torch.cuda.current_stream(self.device))
+
+
+class Analyzer(_StateOwner):
     """Device-resident encoding analyzer: mode 0 = TF min/max, 1 = TF-Enhanced (512-bucket PDF + SQNR search),
     2 = percentile on the same PDF."""
 
@@ -581,8 +595,10 @@ class Analyzer:
         if self.device.index is None:
             self.device = torch.device("cuda", torch.cuda.current_device())
         h = C.c_void_p()
+        # the device state comes from torch's caching allocator
+        self._init_state(lib.miq_analyzer_state_bytes())
         with torch.cuda.device(self.device):
-            check(lib.miq_analyzer_create(self.mode, C.byref(h)))
+            check(lib.miq_analyzer_create_in(self.mode, _ptr(self._state), C.byref(h)))
         self._h = h
 
     def __del__(self):
@@ -610,8 +626,10 @@ class Analyzer:
         # x was produced on (or converted on) the current stream and the kernels are queued on the same stream, so
         # the caching allocator cannot hand its memory to anyone else before they have run
         if torch.cuda.current_device() == self.device.index:
-            check(lib.miq_analyzer_update_stats_f32(self._h, x.data_ptr(), x.numel(),
-                                                    _stream_of(self.device)))
+            stream = _stream_of(self.device)
+            if stream not in self._streams_seen:
+                self._note_stream(stream)
+            check(lib.miq_analyzer_update_stats_f32(self._h, x.data_ptr(), x.numel(), stream))
         else:
             with torch.cuda.device(self.device):
                 check(lib.miq_analyzer_update_stats_f32(self._h, x.data_ptr(), x.numel(), self._s()))
@@ -652,7 +670,7 @@ class Analyzer:
         return d[:n.value], o[:n.value], c[:n.value], best.value
 
 
-class ChannelAnalyzer:
+class ChannelAnalyzer(_StateOwner):
     """Device-resident per-channel TF-Enhanced (mode 1) / percentile (mode 2) analyzer: one 512-bucket PDF per channel of
     a tensor laid out [outer][channels][n_per_channel], one launch sequence per update, one search launch for all
     channels.  Channel c behaves like an `Analyzer` fed ``tensor.select(axis, c)``.  The state is a torch tensor
@@ -665,8 +683,7 @@ class ChannelAnalyzer:
             raise RuntimeError("a ChannelAnalyzer lives on a GPU")
         if self.device.index is None:
             self.device = torch.device("cuda", torch.cuda.current_device())
-        nbytes = int(lib.miq_channel_analyzer_state_bytes(self.num_channel))
-        self._state = torch.empty(nbytes // 8 + 1, dtype=torch.float64, device=self.device)
+        self._init_state(lib.miq_channel_analyzer_state_bytes(self.num_channel))
         h = C.c_void_p()
         with torch.cuda.device(self.device):
             check(lib.miq_channel_analyzer_create(self.mode, self.num_channel, _ptr(self._state), self._s(),
@@ -696,6 +713,7 @@ class ChannelAnalyzer:
             x = x.to(_F32).contiguous()
         ws = _minmax_workspace(self.num_channel, x.numel(), int(n_per_channel), x.device)
         with torch.cuda.device(self.device):
+            self._note_stream(_stream_of(self.device))
             check(lib.miq_channel_analyzer_update_stats_f32(self._h, _ptr(x), x.numel(), int(n_per_channel), _ptr(ws),
                                                             self._s()))
 

@@ -238,6 +238,12 @@ int miq_minmax_per_channel_static_f32(const float* in, int64_t num_channel, int6
  * `stream` once to read the result back.  An object must not be used from two threads at once. */
 typedef struct miq_analyzer miq_analyzer;
 int miq_analyzer_create(int quantization_mode, miq_analyzer** out);
+/* The same with the object's device state in caller memory (miq_analyzer_state_bytes() bytes, 16-byte aligned, alive as
+ * long as the object): the reference routes its scratch memory through the caller's allocator too (IAllocator,
+ * DLQ/include/DlQuantization/Quantization.hpp:62-76, TrainingExtensions/torch/src/AimetTensorQuantizer.cpp:56-71).
+ * Neither form queues or waits for device work. */
+int64_t miq_analyzer_state_bytes(void);
+int miq_analyzer_create_in(int quantization_mode, void* device_state, miq_analyzer** out);
 int miq_analyzer_destroy(miq_analyzer* a);
 /* setPercentileValue (IQuantizationEncodingAnalyzer.hpp:104-112; PercentileEncodingAnalyzer.cpp:203-207), 0..100,
  * default 100.  Stored by every analyzer, used by the percentile one. */
