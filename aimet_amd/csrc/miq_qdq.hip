@@ -304,7 +304,7 @@ __device__ __forceinline__ void store_codes<int32_t, 8>(int32_t* dst, const int*
 }
 
 // Vectorised tile kernel.  Requires 16-byte aligned pointers; n < 2^31 when PER_CHANNEL.
-template <typename IO, typename OP, bool PER_CHANNEL>
+template <typename IO, typename OP, bool PER_CHANNEL, int kUnroll>
 __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::Code> ptr, ParamSrc src, int64_t n,
                                                         uint32_t num_channel, FastDiv fd)
 {
@@ -456,7 +456,11 @@ int launch_ew(EwPtrs<IO, typename OP::Code> ptr, const ParamSrc& src, int64_t n,
     if (n == 0)
         return MIQ_OK;
     using T                = IOTraits<IO>;
-    constexpr int64_t TILE = (int64_t) kBlock * kUnroll * T::VEC;
+    // 16-byte vectors in flight per lane.  Measured on [32,64,56,56], [4096,4096] and [11008,4096], one and two
+    // inputs, float32 and bfloat16: 1, 4 and 8 are never faster than 2 by more than the run-to-run spread and are
+    // slower on the bfloat16 forward (+7 %) and on two-input kernels (+5 %)
+    constexpr int U        = kUnroll;
+    constexpr int64_t TILE = (int64_t) kBlock * U * T::VEC;
     bool vec_ok = aligned16(ptr.x) && (OP::NIN == 1 || aligned16(ptr.g)) && (!ptr.y || aligned16(ptr.y)) &&
                   (!ptr.codes || aligned16(ptr.codes));
     if (PER_CHANNEL)
@@ -466,7 +470,7 @@ int launch_ew(EwPtrs<IO, typename OP::Code> ptr, const ParamSrc& src, int64_t n,
     {
         const int64_t blocks = (n + TILE - 1) / TILE;
         FastDiv fd           = make_fastdiv(PER_CHANNEL ? (uint32_t) n_per_channel : 1u);
-        hipLaunchKernelGGL((ew_vec_kernel<IO, OP, PER_CHANNEL>), dim3((unsigned) blocks), dim3(kBlock), 0, stream, ptr,
+        hipLaunchKernelGGL((ew_vec_kernel<IO, OP, PER_CHANNEL, U>), dim3((unsigned) blocks), dim3(kBlock), 0, stream, ptr,
                            src, n, (uint32_t) num_channel, fd);
     }
     else

@@ -28,7 +28,7 @@ def _stream_of(device):
 
 
 def _stream(t):
-    return C.c_void_p(_stream_of(t.device))
+    return _stream_of(t.device)
 
 
 class _OnDevice:
@@ -52,16 +52,20 @@ class _OnDevice:
 
 
 def _ptr(t):
-    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+    # (a plain integer converts to a void* argument without building a ctypes object)
+    return t.data_ptr() if t is not None else None
 
 
 def _require_gpu(*tensors):
+    """Every tensor given lives on one GPU (Tensor.get_device() is an int, -1 off the GPU: no device objects built)."""
+    index = tensors[0].get_device()
     for t in tensors:
         if t is None:
             continue
-        if not t.is_cuda:
-            raise RuntimeError("aimet_amd kernels run on the GPU only; got a tensor on " + str(t.device))
-        if t.device != tensors[0].device:
+        i = t.get_device()
+        if i != index or i < 0:
+            if not t.is_cuda:
+                raise RuntimeError("aimet_amd kernels run on the GPU only; got a tensor on " + str(t.device))
             raise RuntimeError(f"tensors are on different devices: {t.device} vs {tensors[0].device}")
 
 
@@ -74,6 +78,8 @@ def _suffix(t):
 
 
 def _params_f32(t, like):
+    if t.dtype is _F32 and t.is_contiguous() and t.get_device() == like.get_device():
+        return t
     return t.to(device=like.device, dtype=_F32).contiguous()
 
 
