@@ -91,6 +91,35 @@ def _time_fwd_bwd(torch, fwd, bwd, sets, steps, warmup):
     return wall_ms, e[2].elapsed_time(e[3]) / steps, e[4].elapsed_time(e[5]) / steps
 
 
+def _graph_replay_ms(torch, fn, sets, launches):
+    """Mean duration of `launches` back-to-back launches of fn (rotating the buffer sets) replayed from a HIP graph:
+    the kernels as the GPU runs them when the host is not what paces them.  For tensors of a few MB the Python and
+    launch cost of a call (6 to 8 us) exceeds the kernel's duration, and the eager figures measure the host."""
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(3):
+                fn(sets[i % len(sets)])
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(launches):
+                fn(sets[i % len(sets)])
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / launches
+        del graph
+        return ms
+    except RuntimeError:
+        return None
+
+
 def bench_per_channel(torch, ops, shape, dtype, bw, steps, warmup, seed, nsets=3):
     dev = torch.device("cuda", 0)
     c, npc = shape[0], 1
@@ -115,11 +144,23 @@ def bench_per_channel(torch, ops, shape, dtype, bw, steps, warmup, seed, nsets=3
     def bwd(s):
         ops.ste_bwd_per_channel(s[0], s[1], c, npc, emin, emax, out=s[3])
 
+    if n < 8e6:
+        steps = max(steps, 100)                 # microsecond kernels: more launches per region
     wall, f, b = _time_fwd_bwd(torch, fwd, bwd, sets, steps, warmup)
-    return {"shape": list(shape), "dtype": "fp32" if esz == 4 else "bf16", "bw": bw, "elements": n,
-            "ms_per_step": wall, "fwd_ms": f, "bwd_ms": b,
-            "fwd_GBps": 2 * esz * n / f / 1e6, "bwd_GBps": 3 * esz * n / b / 1e6,
-            "fwd_bwd_GBps": 5 * esz * n / wall / 1e6, "buffer_sets": nsets}
+    out = {"shape": list(shape), "dtype": "fp32" if esz == 4 else "bf16", "bw": bw, "elements": n,
+           "ms_per_step": wall, "fwd_ms": f, "bwd_ms": b,
+           "fwd_GBps": 2 * esz * n / f / 1e6, "bwd_GBps": 3 * esz * n / b / 1e6,
+           "fwd_bwd_GBps": 5 * esz * n / wall / 1e6, "buffer_sets": nsets}
+    if n < 2e7:
+        # host-paced above; the same launches replayed from a HIP graph
+        gf = _graph_replay_ms(torch, fwd, sets, min(64, 4 * nsets))
+        gb = _graph_replay_ms(torch, bwd, sets, min(64, 4 * nsets))
+        if gf and gb:
+            out["graph_replay"] = {"fwd_ms": gf, "bwd_ms": gb, "fwd_GBps": 2 * esz * n / gf / 1e6,
+                                   "bwd_GBps": 3 * esz * n / gb / 1e6,
+                                   "fwd_bwd_GBps": 5 * esz * n / (gf + gb) / 1e6,
+                                   "frac_hbm": 5 * esz * n / (gf + gb) / 1e6 / HBM_PEAK_GBPS}
+    return out
 
 
 def bench_fp8(torch, ops, steps, warmup):
@@ -174,10 +215,20 @@ def bench_per_tensor(torch, ops, steps, warmup):
     def bwd(s):
         ops.ste_bwd_per_tensor(s[0], s[1], e.min, e.max, out=s[3])
 
-    wall, f, b = _time_fwd_bwd(torch, fwd, bwd, sets, steps, warmup)
-    return {"shape": list(shape), "dtype": "fp32", "bw": 8, "elements": n, "ms_per_step": wall, "fwd_ms": f,
-            "bwd_ms": b, "fwd_GBps": 8 * n / f / 1e6, "bwd_GBps": 12 * n / b / 1e6,
-            "fwd_bwd_GBps": 20 * n / wall / 1e6, "buffer_sets": nsets}
+    wall, f, b = _time_fwd_bwd(torch, fwd, bwd, sets, max(steps, 100), warmup)
+    out = {"shape": list(shape), "dtype": "fp32", "bw": 8, "elements": n, "ms_per_step": wall, "fwd_ms": f,
+           "bwd_ms": b, "fwd_GBps": 8 * n / f / 1e6, "bwd_GBps": 12 * n / b / 1e6,
+           "fwd_bwd_GBps": 20 * n / wall / 1e6, "frac_hbm": 20 * n / wall / 1e6 / HBM_PEAK_GBPS, "buffer_sets": nsets}
+    gf, gb = _graph_replay_ms(torch, fwd, sets, 64), _graph_replay_ms(torch, bwd, sets, 64)
+    if gf and gb:
+        out["graph_replay"] = {"fwd_ms": gf, "bwd_ms": gb, "fwd_bwd_GBps": 20 * n / (gf + gb) / 1e6,
+                               "frac_hbm": 20 * n / (gf + gb) / 1e6 / HBM_PEAK_GBPS}
+    # the same region with one buffer set: 103 MB of operands, served by the 256 MB last-level cache
+    one = sets[:1]
+    wall1, f1, b1 = _time_fwd_bwd(torch, fwd, bwd, one, max(steps, 100), warmup)
+    out["same_buffer_cache_resident"] = {"ms_per_step": wall1, "fwd_ms": f1, "bwd_ms": b1,
+                                         "fwd_bwd_GBps": 20 * n / wall1 / 1e6}
+    return out
 
 
 def bench_calibration(torch, ops, reps):
@@ -215,24 +266,30 @@ def bench_calibration(torch, ops, reps):
     tot = sum(total_ms) / len(total_ms)
     elems = 16 * n
     # the same accumulation when the calibration batches are larger (one update call = one launch: the launch's fixed
-    # cost is what keeps the 25.7 MB batches of the configuration below the kernel's streaming rate)
+    # cost is what keeps the 25.7 MB batches of the configuration below the kernel's streaming rate).  Two rows per
+    # size: distinct buffers rotated so that every read comes from HBM, and one buffer read over and over, which at
+    # 25.7 and 103 MB is served by the 256 MB last-level cache and is labelled so.
     by_size = {}
     for mult in (1, 4, 8):
-        big = torch.cat(batches[:mult]) if mult > 1 else batches[0]
-        an.reset()
-        an.update_stats(big)
-        an.update_stats(big)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(8):
-            an.update_stats(big)
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / 8
-        by_size[f"{mult}x[32,256,28,28]"] = {"update_us": ms * 1e3, "GBps": 4 * n * mult / ms / 1e6,
-                                             "frac_hbm": 4 * n * mult / ms / 1e6 / HBM_PEAK_GBPS}
-        del big
+        nrot = max(2, 16 // mult)
+        bigs = [torch.cat(batches[k * mult:(k + 1) * mult]) if mult > 1 else batches[k] for k in range(nrot)]
+        for label, pick in (("rotated_hbm", lambda i: bigs[i % nrot]), ("same_buffer_cache_resident", lambda i: bigs[0])):
+            an.reset()
+            an.update_stats(pick(0))
+            an.update_stats(pick(1))
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            reps = 16
+            e0.record()
+            for i in range(reps):
+                an.update_stats(pick(i))
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / reps
+            by_size.setdefault(f"{mult}x[32,256,28,28]", {})[label] = {
+                "update_us": ms * 1e3, "GBps": 4 * n * mult / ms / 1e6,
+                "frac_hbm": 4 * n * mult / ms / 1e6 / HBM_PEAK_GBPS}
+        del bigs
     return {"elements": elems, "accumulate_ms": acc, "search_ms_wall": sum(search_ms) / len(search_ms),
             "update_by_batch_size": by_size,
             "total_ms_wall": tot, "elements_per_s": elems / (tot / 1e3),
@@ -289,7 +346,10 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
     AdaroundOptimizer.use_fused_linear = True
 
     # per-kernel times of the fused iteration (floor(W / delta) as the optimizer stores it: int8 for this 4-bit grid;
-    # the algorithmic bytes below stay those of the float32 formulation, 8 and 28 B/element)
+    # the algorithmic bytes below stay those of the float32 formulation, 8 and 28 B/element).  Each kernel is timed over
+    # a region of back-to-back launches of that kernel alone between one event pair (events between single launches
+    # would put a bubble after every kernel); the forward region is the pair of launches the forward entry point makes
+    # (split-K GEMM + loss/gradient kernel).
     w = ops.adaround_floor_i8(wrapper.weight.detach(), wrapper.num_channel, wrapper.n_per_channel, wrapper.delta,
                               wrapper.offset, wrapper.clip_min, wrapper.clip_max)
     floor_storage = "int8"
@@ -301,26 +361,68 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
     ws = ops.adaround_linear_workspace(o, k, w.device)
     gout = torch.empty(32, o, device=w.device)
     idx = torch.stack(batches[:timed_kernel_iters]).to(torch.int32).to(w.device)
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(timed_kernel_iters)]
-    torch.cuda.synchronize()
-    for i in range(timed_kernel_iters):
-        ev[i][0].record()
+
+    def fwd(i):
         ops.adaround_linear_fwd(w, alpha, x, idx[i], y, None, wrapper.num_channel, wrapper.delta, wrapper.offset,
                                 wrapper.clip_min, wrapper.clip_max, 0, ws, gout)
-        ev[i][1].record()
+
+    def bwd(i):
         ops.adaround_linear_bwd_adam(w, gout, x, idx[i], alpha, m, v, wrapper.num_channel, wrapper.delta,
                                      wrapper.offset, wrapper.clip_min, wrapper.clip_max, 0.01, 10.0, 1e-3, 0.9, 0.999,
                                      1e-8, i + 1)
-        ev[i][2].record()
-    torch.cuda.synchronize()
-    f = sum(e[0].elapsed_time(e[1]) for e in ev) / timed_kernel_iters
-    b = sum(e[1].elapsed_time(e[2]) for e in ev) / timed_kernel_iters
+
+    def region(fn):
+        for i in range(3):
+            fn(i)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(timed_kernel_iters):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / timed_kernel_iters
+
+    f, b = region(fwd), region(bwd)
     res["fused_kernels"] = {
+        "timing": "mean over back-to-back launches of one kernel between one event pair",
         "fwd_ms": f, "bwd_ms": b, "floor_storage": floor_storage,
         "fwd_algorithmic_bytes": 8 * n, "fwd_GBps": 8 * n / f / 1e6, "fwd_frac_hbm": 8 * n / f / 1e6 / HBM_PEAK_GBPS,
         "fwd_mfma_TFLOPs": 2.0 * 32 * n / f / 1e9,
         "bwd_algorithmic_bytes": 28 * n, "bwd_GBps": 28 * n / b / 1e6, "bwd_frac_hbm": 28 * n / b / 1e6 / HBM_PEAK_GBPS,
         "bwd_mfma_TFLOPs": 2.0 * 32 * n / b / 1e9}
+
+    # the GEMM-bound variant: every iteration uses all 2048 cached rows.  The fused kernels are built for the
+    # reference's batch of 32 (the weight-shaped traffic dominates there); a batch of 2048 goes through the general
+    # path: soft-rounding kernel, torch's GEMMs (hipBLASLt) for the layer and its weight gradient, fused
+    # backward/regulariser/Adam kernel.  The two GEMMs are also timed alone.
+    rows = x.size(0)
+    full = [torch.arange(rows) for _ in range(12)]
+    alpha0 = wrapper.alpha.data.clone()
+    AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, x, y, params, batches=full[:2])
+    wrapper.alpha.data.copy_(alpha0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, x, y, params, batches=full[2:])
+    torch.cuda.synchronize()
+    it_ms = (time.perf_counter() - t0) * 1e3 / 10
+    wrapper.alpha.data.copy_(alpha0)
+    wq = torch.randn(o, k, device=x.device) * 0.02
+    go = torch.randn(rows, o, device=x.device)
+
+    def gemms(i):
+        torch.nn.functional.linear(x, wq)
+        torch.mm(go.t(), x)
+
+    g_ms = region(gemms)
+    flops = 2 * 2.0 * rows * o * k
+    res["batch_2048_gemm_bound"] = {
+        "path": "soft-round kernel + torch GEMMs (hipBLASLt) + fused backward/Adam kernel; the MFMA-fused kernels "
+                "take batches of 32 only",
+        "ms_per_iteration": it_ms, "gflop_per_iteration": flops / 1e9,
+        "iteration_TFLOPs": flops / it_ms / 1e9,
+        "gemms_alone_ms": g_ms, "gemms_alone_TFLOPs": flops / g_ms / 1e9,
+        "gemms_alone_frac_fp32_mfma_peak": flops / g_ms / 1e9 / 157.3}
     return res
 
 
@@ -633,15 +735,231 @@ def cpu_baseline_calibration(seconds=5.0):
             "sample": f"{reps} histogram updates of a quarter batch ({x.size} elements), {dt:.1f} s"}
 
 
+def bench_per_channel_calibration(torch, ops):
+    """Per-output-channel TF-Enhanced calibration of the [11008, 4096] weight: every channel's PDF and symmetric 8-bit
+    encoding from one device object (one update, one search), beside the reference's flow of one analyzer object per
+    channel fed slice by slice -- that one measured on 128 channels and scaled."""
+    dev = torch.device("cuda", 0)
+    c, npc = 11008, 4096
+    w = _laplace_weights(torch, (c, npc), 1004, dev)
+    an = ops.ChannelAnalyzer(1, c, dev)
+    an.update_stats(w, npc)
+    an.compute_encodings(8, True)
+    upd, srch = [], []
+    for _ in range(3):
+        an.reset()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        an.update_stats(w, npc)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        encs, valid = an.compute_encodings(8, True)
+        t2 = time.perf_counter()
+        upd.append((t1 - t0) * 1e3)
+        srch.append((t2 - t1) * 1e3)
+    sub = 128
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for ch in range(sub):
+        a1 = ops.Analyzer(1, dev)
+        a1.update_stats(w[ch].contiguous())
+        a1.compute_encoding(8, True)
+    t_loop = (time.perf_counter() - t0) * 1e3 / sub
+    return {"shape": [c, npc], "channels": c, "update_ms": min(upd), "search_and_readback_ms": min(srch),
+            "update_GBps": 4.0 * c * npc / min(upd) / 1e6,
+            "one_object_per_channel_ms_per_channel": t_loop, "one_object_per_channel_ms_scaled": t_loop * c,
+            "speedup_vs_one_object_per_channel": t_loop * c / (min(upd) + min(srch)),
+            "first_encoding": [encs[0].min, encs[0].max, encs[0].delta, encs[0].offset]}
+
+
+def parity_checks(torch, ops):
+    """One cheap comparison per leg against the CPU oracle, outside every timed region: the checker confirms that the
+    kernels being timed produce the reference's results on this machine (the full comparisons are the GPU tests).
+    Returns {leg: bool}."""
+    import numpy as np
+    import oracle
+    from oracle import adaround_oracle as ada
+    from oracle import sqnr_oracle as sq
+    o = oracle.lib
+    dev = torch.device("cuda", 0)
+    out = {}
+    rng = np.random.default_rng(7)
+    # per-tensor QDQ forward + STE backward (cfg1 arithmetic, 1 M samples)
+    x = rng.standard_normal(1 << 20).astype(np.float32)
+    g = rng.standard_normal(1 << 20).astype(np.float32)
+    enc = o.tf_compute_encoding(float(x.min()), float(x.max()), 8)
+    y = ops.qdq_per_tensor(torch.from_numpy(x).to(dev), enc.min, enc.max, 8).cpu().numpy()
+    gin = ops.ste_bwd_per_tensor(torch.from_numpy(x).to(dev), torch.from_numpy(g).to(dev), enc.min, enc.max).cpu().numpy()
+    out["per_tensor_act_int8"] = bool(
+        np.array_equal(y.view(np.uint32), o.qdq_per_tensor(x, enc.min, enc.max, 8).view(np.uint32)) and
+        np.array_equal(gin, o.ste_bwd_per_tensor(x, g, np.float32(enc.min), np.float32(enc.max))))
+    # per-channel symmetric int8 / int4, fp32 and bf16 storage ([256, 4096] rows of the main workload's distribution)
+    c, npc = 256, 4096
+    u = rng.random((c, npc)) - 0.5
+    w = (-0.02 * np.sign(u) * np.log1p(-2 * np.abs(u))).astype(np.float32)
+    ok = True
+    for bw in (8, 4):
+        amax = np.abs(w).max(axis=1).astype(np.float64)
+        encs = [o.tf_compute_encoding(-a, a, bw, sym=True) for a in amax]
+        emin, emax = np.array([e.min for e in encs]), np.array([e.max for e in encs])
+        params = o.per_channel_params(emin, emax, bw)
+        steps = 2 ** bw - 1 - (1 if emin[0] == -emax[0] else 0)
+        gp = ops.per_channel_params(torch.from_numpy(emin.astype(np.float32)).to(dev),
+                                    torch.from_numpy(emax.astype(np.float32)).to(dev), steps)
+        wg = torch.from_numpy(w).to(dev)
+        ok &= np.array_equal(ops.qdq_per_channel(wg, c, npc, *gp).cpu().numpy().view(np.uint32),
+                             o.qdq_per_channel(w, c, npc, params).view(np.uint32))
+        wb = torch.from_numpy(w).to(torch.bfloat16)
+        got = ops.qdq_per_channel(wb.to(dev), c, npc, *gp).cpu().view(torch.int16).numpy().view(np.uint16)
+        ok &= np.array_equal(got, o.qdq_per_channel_bf16(wb.view(torch.int16).numpy().view(np.uint16), c, npc, params))
+        gr = rng.standard_normal((c, npc)).astype(np.float32)
+        emn32, emx32 = emin.astype(np.float32), emax.astype(np.float32)
+        gin = ops.ste_bwd_per_channel(wg, torch.from_numpy(gr).to(dev), c, npc, torch.from_numpy(emn32).to(dev),
+                                      torch.from_numpy(emx32).to(dev)).cpu().numpy()
+        ok &= np.array_equal(gin, o.ste_bwd_per_channel(w, gr, c, npc, emn32, emx32))
+    out["per_channel_cells"] = bool(ok)
+    # TF-Enhanced calibration: two batches of the calibration distribution, PDF bits and the chosen encoding
+    an, pdf = ops.Analyzer(1, dev), o.new_pdf()
+    for seed in (1, 2):
+        a = np.abs(np.random.default_rng(seed).standard_normal(1 << 20)).astype(np.float32)
+        a[::200] = (1.0 / np.sqrt(1.0 - np.random.default_rng(seed + 9).random(a[::200].size))).astype(np.float32)
+        an.update_stats(torch.from_numpy(a).to(dev))
+        pdf.update(a)
+    xl, p = an.get_stats_histogram()
+    e, _ = an.compute_encoding(8)
+    out["tf_enhanced_calibration"] = bool(np.array_equal(p.view(np.uint64), pdf.pdf().view(np.uint64)) and
+                                          (e.min, e.max, e.delta, e.offset, e.bw) == pdf.compute_encoding(8)[0].astuple())
+    # per-channel TF-Enhanced: 64 rows
+    ca = ops.ChannelAnalyzer(1, 64, dev)
+    ca.update_stats(torch.from_numpy(w[:64]).to(dev), npc)
+    encs, _ = ca.compute_encodings(8, True)
+    ok = True
+    for ch in (0, 17, 63):
+        pc = o.new_pdf()
+        pc.update(w[ch])
+        ok &= (encs[ch].min, encs[ch].max, encs[ch].delta, encs[ch].offset, encs[ch].bw) == \
+            pc.compute_encoding(8, True)[0].astuple()
+    out["per_channel_tf_enhanced"] = bool(ok)
+    # v2 SQNR observer: histogram of one batch and the chosen range
+    from aimet_amd.v2.quantization.encoding_analyzer import SqnrEncodingAnalyzer
+    xs = torch.randn(1 << 20) * 1.5 + 0.2
+    an2, ref2 = SqnrEncodingAnalyzer((1,)), sq.SqnrAnalyzer()
+    an2.update_stats(xs.to(dev))
+    ref2.update_stats(xs)
+    qmin, qmax = an2.compute_encodings(255.0, False)
+    rmin, rmax, _ = ref2.compute_encodings(255.0, False)
+    out["v2_sqnr_calibration"] = bool(torch.equal(an2.observer.get_stats()[0].histogram.cpu(), ref2.stats[0].histogram) and
+                                      torch.allclose(qmin.cpu(), rmin, rtol=1e-6) and torch.allclose(qmax.cpu(), rmax, rtol=1e-6))
+    # v2 backward with learnable scale / offset: input gradient bit for bit, parameter sums to 2e-5
+    xw = (rng.standard_normal((64, 1024)) * 0.5).astype(np.float32)
+    gw = rng.standard_normal((64, 1024)).astype(np.float32)
+    sc = (np.abs(xw).max(axis=1) / 127).astype(np.float32)
+    of = np.zeros(64, np.float32)
+    gi, gs, go = ops.v2_qdq_bwd_params(torch.from_numpy(xw).to(dev), torch.from_numpy(gw).to(dev), 64, 1024,
+                                       torch.from_numpy(sc).to(dev), torch.from_numpy(of).to(dev), -128, 127)
+    want_gi = o.v2_qdq_bwd(xw, gw, 64, 1024, sc, of, -128, 127)
+    xt = torch.from_numpy(xw)
+    s_, o_ = torch.from_numpy(sc).view(-1, 1), torch.from_numpy(of).view(-1, 1)
+    q = xt / s_
+    r = torch.round(q)
+    mask = (-128 <= r - o_) & (r - o_ <= 127)
+    want_gs = (torch.from_numpy(gw) * (r.clamp(o_ - 128, o_ + 127) - q * mask)).double().sum(dim=1)
+    out["v2_range_learning_backward"] = bool(np.array_equal(gi.cpu().numpy().view(np.uint32), want_gi.view(np.uint32)) and
+                                             torch.allclose(gs.double().cpu(), want_gs, rtol=2e-5, atol=1e-4))
+    # AdaRound fused Linear path: three iterations on a [64, 256] layer against the torch-CPU restatement
+    torch.manual_seed(0)
+    wt = torch.randn(64, 256) * 0.05
+    delta = (wt.abs().amax(dim=1) * 2 / 15).float()
+    offset = torch.full((64,), -8.0)
+    alpha0 = ada.generate_alpha(wt, ada.broadcast(delta, wt, 0))
+    xs_, ys_ = torch.randn(96, 256), None
+    ys_ = ada.layer_output("linear", xs_, wt) + 0.02 * torch.randn(96, 64)
+    bts = [torch.randperm(96)[:32] for _ in range(3)]
+    a_ref, _, _, _ = ada.optimize_rounding("linear", wt, alpha0, delta, offset, 0, 15, xs_, ys_, bts, 3, 0.01, (20, 2), 0.2)
+    wg_, dg, og, xg, yg = (t.to(dev) for t in (wt, delta, offset, xs_, ys_))
+    alpha = ops.adaround_init_alpha(wg_, 64, 256, dg)
+    fl = ops.adaround_floor(wg_, 64, 256, dg)
+    m_, v_ = torch.zeros_like(alpha), torch.zeros_like(alpha)
+    ws = ops.adaround_linear_workspace(64, 256, dev)
+    gout = torch.empty(32, 64, device=dev)
+    for k_, idx in enumerate(bts):
+        beta = -1.0 if k_ < 0.2 * 3 else ada.compute_beta(3, k_, (20, 2), 0.2)
+        ig = idx.to(torch.int32).to(dev)
+        ops.adaround_linear_fwd(fl, alpha, xg, ig, yg, None, 64, dg, og, 0, 15, 0, ws, gout)
+        ops.adaround_linear_bwd_adam(fl, gout, xg, ig, alpha, m_, v_, 64, dg, og, 0, 15, 0.01, beta, 1e-3, 0.9, 0.999,
+                                     1e-8, k_ + 1)
+    out["adaround_linear_4096"] = bool(torch.allclose(alpha.cpu(), a_ref, atol=5e-5))
+    return out
+
+
+def cpu_baseline_adaround(iterations=3):
+    """The AdaRound iteration of the configuration ([4096,4096], 32 of 2048 cached rows, 4-bit) as the reference runs it
+    on the CPU: torch ops + autograd + torch.optim.Adam (oracle/adaround_oracle.py), all host threads."""
+    import torch
+    from oracle import adaround_oracle as ada
+    g = torch.Generator().manual_seed(1005)
+    wt = torch.randn(4096, 4096, generator=g) * 0.02
+    xs = torch.randn(2048, 4096, generator=g)
+    ys = torch.nn.functional.linear(xs, wt)
+    delta = (wt.abs().amax(dim=1) / 7.0).float()
+    offset = torch.full((4096,), -8.0)
+    alpha0 = ada.generate_alpha(wt, ada.broadcast(delta, wt, 0))
+    bts = [torch.randperm(2048, generator=g)[:32] for _ in range(iterations + 1)]
+    ada.optimize_rounding("linear", wt, alpha0, delta, offset, 0, 15, xs, ys, bts[:1], 1000, 0.01, (20, 2), 0.2,
+                          first_iteration=300)
+    t0 = time.perf_counter()
+    ada.optimize_rounding("linear", wt, alpha0, delta, offset, 0, 15, xs, ys, bts[1:], 1000, 0.01, (20, 2), 0.2,
+                          first_iteration=300)
+    dt = time.perf_counter() - t0
+    return {"value": dt * 1e3 / iterations, "unit": "ms/iteration", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{iterations} iterations of the [4096,4096] layer, batch 32, torch CPU ops + autograd + Adam"}
+
+
+def cpu_baseline_v2(passes=3):
+    """The v2 formulas as torch CPU ops with all host threads: quantize-dequantize forward + backward of the
+    [11008,4096] weight (per channel), and one update of the 2048-bin histogram observer on a calibration batch."""
+    import torch
+    from oracle import sqnr_oracle as sq
+    g = torch.Generator().manual_seed(1006)
+    x = torch.randn(11008, 4096, generator=g) * 0.05
+    gr = torch.randn(11008, 4096, generator=g)
+    s = (x.abs().amax(dim=1, keepdim=True) / 127).clamp_min(1e-6)
+
+    def one():
+        q = x / s
+        r = torch.round(q)
+        mask = (-128 <= r) & (r <= 127)
+        y = r.clamp(-128, 127) * s
+        return y, gr * mask
+
+    one()
+    t0 = time.perf_counter()
+    for _ in range(passes):
+        one()
+    dt = (time.perf_counter() - t0) / passes
+    batch = torch.randn(32 * 256 * 28 * 28, generator=g).abs_()
+    obs = sq.SqnrAnalyzer()
+    obs.update_stats(batch)
+    t0 = time.perf_counter()
+    obs.update_stats(batch)
+    t_obs = time.perf_counter() - t0
+    n = x.numel()
+    return {"qdq_fwd_bwd": {"value": 20.0 * n / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                            "kind": "port", "sample": f"{passes} fwd+bwd passes over [11008,4096] fp32, torch CPU ops"},
+            "histogram_observer_update": {"value": batch.numel() / t_obs, "unit": "elements/s",
+                                          "cores": torch.get_num_threads(), "kind": "port",
+                                          "sample": "one update of a [32,256,28,28] batch, torch.histc on the CPU"}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--full", action="store_true", help="also measure every shape x dtype x bit-width cell")
+    ap.add_argument("--full", action="store_true", help="(kept for old command lines: every cell is measured anyway)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run a subset of the legs, comma separated (main|pt|fp8|calib|sqnr|learn|quantsim|adaround|copyref), for profiling")
+                    help="run a subset of the legs, comma separated (main|pt|fp8|calib|chcalib|sqnr|learn|quantsim|adaround|copyref), for profiling")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
@@ -680,6 +998,8 @@ def main():
         extra["fp8_simulation"] = bench_fp8(torch, ops, max(20, args.steps), args.warmup)
     if want("calib"):
         extra["tf_enhanced_calibration"] = bench_calibration(torch, ops, 5)
+    if want("chcalib"):
+        extra["per_channel_tf_enhanced"] = bench_per_channel_calibration(torch, ops)
     if want("sqnr"):
         extra["v2_sqnr_calibration"] = bench_sqnr(torch, ops)
     if want("learn"):
@@ -690,13 +1010,15 @@ def main():
         extra["adaround_linear_4096"] = bench_adaround(torch, ops, 1000 if args.only is None else args.steps)
         extra["adaround_linear_4096"]["torch_ops_same_gpu"] = torch_ops_adaround_baseline(torch)
     if args.only is None:
-        cells = [((11008, 4096), torch.bfloat16, 8), ((11008, 4096), torch.float32, 4)]
-        if args.full:
-            cells = [(s, d, b) for s in ((512, 512, 3, 3), (4096, 4096), (11008, 4096))
-                     for d in (torch.float32, torch.bfloat16) for b in (8, 4)]
+        # every shape x dtype x bit-width cell of the weight configuration (the main cell is the headline above)
+        cells = [(s, d, b) for s in ((512, 512, 3, 3), (4096, 4096), (11008, 4096))
+                 for d in (torch.float32, torch.bfloat16) for b in (8, 4)]
         extra["per_channel_cells"] = [
             bench_per_channel(torch, ops, s, d, b, max(20, args.steps // 2), 5, 1002 + {512: 0, 4096: 1, 11008: 2}[s[0]])
             for (s, d, b) in cells if not (s == main_shape and d == torch.float32 and b == 8)]
+        for cell in extra["per_channel_cells"]:
+            cell["frac_hbm"] = cell["fwd_bwd_GBps"] / HBM_PEAK_GBPS
+        extra["parity_checked"] = parity_checks(torch, ops)
     if res is None:
         print(json.dumps({"extra": extra}))
         return
@@ -728,6 +1050,9 @@ def main():
         ref_fwd = cpu_reference_qdq_forward()
         if ref_fwd is not None:
             extra["cpu_reference_qdq_forward"] = ref_fwd
+        if args.only is None:
+            extra["cpu_baseline_adaround"] = cpu_baseline_adaround()
+            extra["cpu_baseline_v2"] = cpu_baseline_v2()
     line["extra"] = extra
     print(json.dumps(line))
 
