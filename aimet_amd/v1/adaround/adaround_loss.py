@@ -1,10 +1,12 @@
 """Hyper-parameters and loss terms of AdaRound.
 
-Mirrors TrainingExtensions/torch/src/python/aimet_torch/v1/adaround/adaround_loss.py: AdaroundHyperParameters
-(:48-62), AdaroundLoss.compute_recon_loss (:70-80), compute_round_loss (:82-111), _compute_beta (:113-135).
-The optimisation loop does not call compute_round_loss per iteration -- its gradient is fused into the backward
-kernel -- but the function is kept for callers that want the value.
+Same names and values as TrainingExtensions/torch/src/python/aimet_torch/v1/adaround/adaround_loss.py
+(AdaroundHyperParameters :48-62, AdaroundLoss.compute_recon_loss :70-80, compute_round_loss :82-111, _compute_beta
+:113-135).  The optimisation loop itself never evaluates the rounding loss: its gradient is part of the fused backward
+kernel (aimet_amd/csrc/miq_adaround_math.h), which also returns the sum this module's compute_round_loss forms.
 """
+import math
+from dataclasses import dataclass
 from typing import Tuple
 
 import numpy as np
@@ -13,14 +15,24 @@ import torch
 from ...common.defs import AdaroundConstants
 
 
+@dataclass
 class AdaroundHyperParameters:
     """Hyper parameters of the per-layer optimisation."""
+    num_iterations: int
+    reg_param: float
+    beta_range: Tuple
+    warm_start: float
 
-    def __init__(self, num_iterations: int, reg_param: float, beta_range: Tuple, warm_start: float):
-        self.num_iterations = num_iterations
-        self.reg_param = reg_param
-        self.beta_range = beta_range
-        self.warm_start = warm_start
+    @property
+    def warm_start_iterations(self) -> float:
+        """Iterations (a real number) during which only the reconstruction loss is optimised."""
+        return self.num_iterations * self.warm_start
+
+
+def _soft_rounding(alpha: torch.Tensor) -> torch.Tensor:
+    """h(alpha): the sigmoid stretched to [GAMMA, ZETA] and cut to [0, 1]."""
+    stretch = AdaroundConstants.ZETA - AdaroundConstants.GAMMA
+    return torch.sigmoid(alpha).mul(stretch).add(AdaroundConstants.GAMMA).clamp(0, 1)
 
 
 class AdaroundLoss:
@@ -28,29 +40,32 @@ class AdaroundLoss:
 
     @staticmethod
     def compute_recon_loss(ada_quantized_output: torch.Tensor, orig_output: torch.Tensor) -> torch.Tensor:
-        """Squared Frobenius norm over dim 1, averaged over the remaining dims."""
-        return (torch.norm(ada_quantized_output - orig_output, p="fro", dim=1) ** 2).mean()
+        """Squared error summed along dim 1 (output channels), averaged over everything else -- what the squared
+        Frobenius norm over dim 1 followed by a mean amounts to."""
+        error = ada_quantized_output - orig_output
+        return error.square().sum(dim=1).mean()
 
     @classmethod
     def in_warm_start(cls, opt_params: AdaroundHyperParameters, cur_iter: int) -> bool:
-        return cur_iter < opt_params.num_iterations * opt_params.warm_start
+        return cur_iter < opt_params.warm_start_iterations
 
     @classmethod
     def compute_round_loss(cls, alpha: torch.Tensor, opt_params: AdaroundHyperParameters, cur_iter: int):
-        """reg_param * sum(1 - |2 h(alpha) - 1|^beta); 0 during the warm-start period."""
+        """reg_param * sum(1 - |2 h(alpha) - 1|^beta): zero where the soft rounding has decided (h = 0 or 1), largest
+        at h = 1/2; 0 during the warm-start period."""
         if cls.in_warm_start(opt_params, cur_iter):
             return 0
-        h_alpha = torch.clamp(torch.sigmoid(alpha) * (AdaroundConstants.ZETA - AdaroundConstants.GAMMA) +
-                              AdaroundConstants.GAMMA, 0, 1)
         beta = cls._compute_beta(opt_params.num_iterations, cur_iter, opt_params.beta_range, opt_params.warm_start)
-        reg_term = torch.add(1, -(torch.add(2 * h_alpha, -1).abs()).pow(beta)).sum()
-        return opt_params.reg_param * reg_term
+        undecided = 1 - (2 * _soft_rounding(alpha) - 1).abs().pow(beta)
+        return opt_params.reg_param * undecided.sum()
 
     @staticmethod
     def _compute_beta(max_iter: int, cur_iter: int, beta_range: Tuple, warm_start: float) -> float:
-        """Cosine decay of beta from beta_range[0] to beta_range[1] after the warm-start period."""
-        assert cur_iter < max_iter, 'Current iteration should be less than total maximum number of iterations.'
-        start_beta, end_beta = beta_range
-        warm_start_end_iter = warm_start * max_iter
-        rel_iter = (cur_iter - warm_start_end_iter) / (max_iter - warm_start_end_iter)
-        return end_beta + 0.5 * (start_beta - end_beta) * (1 + np.cos(rel_iter * np.pi))
+        """Half a cosine period from beta_range[0] (at the end of the warm start) down to beta_range[1] (last iteration)."""
+        if not cur_iter < max_iter:
+            raise AssertionError('Current iteration should be less than total maximum number of iterations.')
+        high, low = beta_range
+        first = warm_start * max_iter
+        phase = (cur_iter - first) / (max_iter - first) * np.pi
+        # (this order of operations reproduces the reference's value to the last bit)
+        return low + 0.5 * (high - low) * (1 + np.cos(phase))

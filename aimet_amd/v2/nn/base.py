@@ -74,6 +74,60 @@ class BaseQuantizationMixin:
                 stack.enter_context(quantizer.compute_encodings())
             yield
 
+    # ------------------------------------------------------------------------------- encodings in the exported format
+    def export_param_encodings(self):
+        """{parameter name: list of encoding dicts, or None without an initialised quantizer}"""
+        return {name: (q.get_legacy_encodings() if q is not None else None)
+                for name, q in self.param_quantizers.items()}
+
+    def export_input_encodings(self):
+        return [q.get_legacy_encodings() if q is not None else None for q in self.input_quantizers]
+
+    def export_output_encodings(self):
+        return [q.get_legacy_encodings() if q is not None else None for q in self.output_quantizers]
+
+    @staticmethod
+    def _import_into(slots, keys, what, encodings, strict, partial, requires_grad, allow_overwrite):
+        """Common part of the three imports (reference aimet_torch/v2/nn/base.py:282-330, :332-380, :395-470 without
+        vector encodings).  `slots` is the ModuleList / ModuleDict of quantizers and `keys` its (slot key, key in
+        `encodings`) pairs.  A frozen quantizer is skipped; a slot without an entry is left alone when `partial`, else
+        emptied; an entry for an empty slot raises when `strict`."""
+        for slot, key in keys:
+            quantizer = slots[slot]
+            if quantizer is not None and not quantizer._allow_overwrite:              # pylint: disable=protected-access
+                continue
+            entry = encodings.get(key)
+            if not entry:
+                if not partial:
+                    slots[slot] = None
+                continue
+            if quantizer is None:
+                if strict:
+                    raise RuntimeError(f"Failed to import {what} {key}: no quantizer present.")
+                continue
+            quantizer.set_legacy_encodings([entry] if isinstance(entry, dict) else entry)
+            if requires_grad is not None:
+                quantizer.requires_grad_(requires_grad)
+            quantizer.allow_overwrite(allow_overwrite)
+
+    def import_param_encodings(self, encodings, strict: bool, partial: bool, requires_grad, allow_overwrite: bool):
+        """encodings: {parameter name: [dict per channel]}"""
+        keys = [(name, name) for name in self.param_quantizers]
+        self._import_into(self.param_quantizers, keys, "encoding for parameter", encodings, strict, partial,
+                          requires_grad, allow_overwrite)
+
+    def import_input_encodings(self, encodings, strict: bool, partial: bool, requires_grad, allow_overwrite: bool):
+        """encodings: {'0': dict, '1': dict, ...} by input index"""
+        keys = [(i, str(i)) for i in range(len(self.input_quantizers))]
+        self._import_into(self.input_quantizers, keys, "input encoding at index", encodings, strict, partial,
+                          requires_grad, allow_overwrite)
+
+    def import_output_encodings(self, encodings, strict: bool, partial: bool, requires_grad, allow_overwrite: bool):
+        """encodings: {'0': dict, '1': dict, ...} by output index"""
+        keys = [(i, str(i)) for i in range(len(self.output_quantizers))]
+        self._import_into(self.output_quantizers, keys, "output encoding at index", encodings, strict, partial,
+                          requires_grad, allow_overwrite)
+
     def get_original_module(self) -> nn.Module:
         """A plain module of the base class sharing this module's parameters and buffers."""
         base_cls = type(self).qcls_to_cls[type(self)]

@@ -177,3 +177,56 @@ class QuantizationSimModel:
         with open(file, 'w') as f:
             json.dump(self.get_encodings_dict(), f, sort_keys=True, indent=4)
         return file
+
+    def load_encodings(self, encodings, strict: bool = True, partial: bool = True, requires_grad=None,
+                       allow_overwrite: bool = True):
+        """Sets quantizer ranges from an exported dictionary or its JSON file (the v2 class inherits this from the v1
+        one: aimet_torch/v1/quantsim.py:1695-1756, acting through the quantized modules' import_* methods,
+        aimet_torch/v2/nn/base.py:282-470).
+
+        strict: a name in the file that is neither a module nor a parameter of the model, or an encoding for a
+        quantizer that does not exist, raises RuntimeError.  partial=False removes every quantizer the file has no
+        entry for.  requires_grad, if given, is applied to the imported quantizers' min / max.  allow_overwrite=False
+        freezes them against later compute_encodings() / load_encodings()."""
+        if isinstance(encodings, (str, os.PathLike)):
+            with open(encodings) as f:
+                encodings = json.load(f)
+        if 'param_encodings' in encodings:
+            for_params = encodings.get('param_encodings') or {}
+            for_activations = encodings.get('activation_encodings') or {}
+        else:
+            for_params, for_activations = encodings, {}                 # parameters only: the older AdaRound export
+        if not for_params and not for_activations:
+            raise RuntimeError("the encodings hold neither parameter nor activation entries")
+        if strict:
+            known = {name for name, _ in self.model.named_modules()} | {name for name, _ in
+                                                                         self.model.named_parameters()}
+            unknown = sorted((for_params.keys() | for_activations.keys()) - known)
+            if unknown:
+                raise RuntimeError("Encoding dictionary contains modules/parameters that doesn't exist in the "
+                                   f"model: {', '.join(unknown)}")
+        args = (strict, partial, requires_grad, allow_overwrite)
+        for name, module in self.qmodules():
+            prefix = f'{name}.'
+            own = {key[len(prefix):]: value for key, value in for_params.items()
+                   if key.startswith(prefix) and key[len(prefix):] in module.param_quantizers}
+            on_tensors = for_activations.get(name, {})
+            try:
+                module.import_param_encodings(own, *args)
+                module.import_input_encodings(on_tensors.get('input', {}), *args)
+                module.import_output_encodings(on_tensors.get('output', {}), *args)
+            except RuntimeError as e:
+                raise RuntimeError(f"Encoding import failed for module: {name}.\n{e}") from e
+
+    def load_and_freeze_encodings(self, encoding_path: str, ignore_when_quantizer_disabled: bool = False):
+        """Parameter and activation encodings of a file, frozen (aimet_torch/v1/quantsim.py:1758-1773)."""
+        self.load_encodings(encoding_path, strict=not ignore_when_quantizer_disabled, partial=True,
+                            requires_grad=False, allow_overwrite=False)
+
+    def set_and_freeze_param_encodings(self, encoding_path: str):
+        """Only the parameter encodings of a file (e.g. the one AdaRound writes), frozen
+        (aimet_torch/v1/quantsim.py:1838-1854)."""
+        with open(encoding_path) as f:
+            content = json.load(f)
+        params_only = {'param_encodings': content['param_encodings']} if 'param_encodings' in content else content
+        self.load_encodings(params_only, strict=True, partial=True, requires_grad=False, allow_overwrite=False)

@@ -318,3 +318,126 @@ def test_v2_sim_constants_and_functional_ops():
     sim.compute_encodings(lambda m, _: m(x), None)
     assert sim.model.add_vector.input_quantizers[1].is_initialized()
     assert torch.isfinite(sim.model(x)).all()
+
+
+def test_v2_load_encodings_after_adaround(tmp_path):
+    """The documented AdaRound flow on the v2 classes: apply_adaround writes '<prefix>.encodings'; a new simulation of
+    the returned model loads them with load_encodings(allow_overwrite=False) (the v2 class inherits it from v1:
+    aimet_torch/v1/quantsim.py:1695-1756) -- the weight quantizers then sit exactly on the grid the weights were rounded
+    on, quantize-dequantizing those weights changes nothing, and calibration afterwards leaves them alone."""
+    import json
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v2.adaround import Adaround, AdaroundParameters
+    from aimet_amd.v2.quantsim import QuantizationSimModel as V2Sim
+    torch.manual_seed(11)
+    model = _ResBlockNet().eval().cuda()
+    dummy = torch.randn(2, 3, 8, 8).cuda()
+    g = torch.Generator().manual_seed(3)
+    loader = [(torch.randn(8, 3, 8, 8, generator=g).cuda(), torch.zeros(8)) for _ in range(3)]
+    params = AdaroundParameters(loader, num_batches=3, default_num_iterations=40,
+                                forward_fn=lambda m, batch: m(batch[0]))
+    rounded = Adaround.apply_adaround(model, dummy, params, str(tmp_path), "net", default_param_bw=4,
+                                      default_quant_scheme=QuantScheme.post_training_tf)
+    file = str(tmp_path / "net.encodings")
+    with open(file) as f:
+        exported = json.load(f)["param_encodings"]
+    assert set(exported) == {"conv1.weight", "conv2.weight", "conv3.weight", "fc.weight"}
+
+    sim = V2Sim(rounded, dummy, quant_scheme='tf', default_param_bw=4)
+    sim.load_encodings(file, allow_overwrite=False)
+    qm = dict(sim.qmodules())
+    for key, (entry,) in exported.items():
+        layer = key.rsplit(".", 1)[0]
+        q = qm[layer].param_quantizers["weight"]
+        assert not q._allow_overwrite and q.is_initialized()                       # pylint: disable=protected-access
+        got, = q.get_legacy_encodings()
+        assert got["bitwidth"] == 4 and got["is_symmetric"] == "True" and got["offset"] == entry["offset"]
+        assert got["scale"] == pytest.approx(entry["scale"], rel=1e-6)
+        w = qm[layer].weight.detach()
+        steps = w.double() / entry["scale"]
+        assert (steps - steps.round()).abs().max().item() < 2e-3                 # adarounded weights lie on the grid
+        assert torch.allclose(q(w), w, atol=entry["scale"] * 2e-3, rtol=0)        # ... so the quantizer keeps them
+
+    def calibrate(m, _):
+        for x, _y in loader:
+            m(x)
+    before = {k: qm[k.rsplit(".", 1)[0]].param_quantizers["weight"].get_legacy_encodings() for k in exported}
+    sim.compute_encodings(calibrate, None)
+    after = {k: qm[k.rsplit(".", 1)[0]].param_quantizers["weight"].get_legacy_encodings() for k in exported}
+    assert before == after                                                        # frozen
+    assert qm["relu1"].output_quantizers[0].is_initialized()                      # the rest was calibrated
+    with torch.no_grad():
+        y = sim.model(loader[0][0])
+    assert torch.isfinite(y).all()
+
+    # set_and_freeze_param_encodings is the same import under its older name
+    sim2 = V2Sim(rounded, dummy, quant_scheme='tf', default_param_bw=4)
+    sim2.set_and_freeze_param_encodings(file)
+    assert {k: dict(sim2.qmodules())[k.rsplit(".", 1)[0]].param_quantizers["weight"].get_legacy_encodings()
+            for k in exported} == before
+
+
+def test_v2_load_encodings_options(tmp_path):
+    """strict / partial / requires_grad / allow_overwrite as in aimet_torch/v2/nn/base.py:282-470: unknown names raise
+    under strict, an entry for a slot without a quantizer raises under strict and is skipped otherwise, partial=False
+    removes the quantizers the dictionary does not mention, a full export -> load round trip reproduces the export,
+    per-channel lists are taken channel by channel, frozen quantizers ignore a later load."""
+    from aimet_amd.v2.quantsim import QuantizationSimModel as V2Sim
+    torch.manual_seed(12)
+    model = _ResBlockNet().eval().cuda()
+    dummy = torch.randn(2, 3, 8, 8).cuda()
+    batches = [torch.randn(8, 3, 8, 8).cuda() for _ in range(2)]
+
+    def calibrate(m, _):
+        for b in batches:
+            m(b)
+    src = V2Sim(model, dummy, quant_scheme='tf', default_param_bw=8, per_channel_quantization=True)
+    src.compute_encodings(calibrate, None)
+    full = src.get_encodings_dict()
+    assert len(full["param_encodings"]["conv2.weight"]) == 8
+
+    dst = V2Sim(model, dummy, quant_scheme='tf', default_param_bw=8, per_channel_quantization=True)
+    dst.load_encodings(full, partial=False)
+    again = dst.get_encodings_dict()
+    for kind in ("param_encodings", "activation_encodings"):
+        assert again[kind].keys() == full[kind].keys()
+    for key, encs in full["param_encodings"].items():
+        for a, b in zip(encs, again["param_encodings"][key]):
+            assert b["scale"] == pytest.approx(a["scale"], rel=1e-6) and b["offset"] == a["offset"]
+    x = batches[0]
+    with torch.no_grad():
+        assert torch.equal(src.model(x), dst.model(x))
+
+    # unknown names
+    bad = {"param_encodings": {"nope.weight": full["param_encodings"]["fc.weight"]}, "activation_encodings": {}}
+    with pytest.raises(RuntimeError, match="nope.weight"):
+        dst.load_encodings(bad)
+    with pytest.raises(RuntimeError):
+        dst.load_encodings({"param_encodings": {}, "activation_encodings": {}})
+    # bn2 has no output quantizer (Conv+BN+Relu supergroup): an entry for it raises under strict only
+    stray = {"param_encodings": {}, "activation_encodings": {"bn2": {"output": {"0": full["activation_encodings"]
+                                                                                   ["relu1"]["output"]["0"]}}}}
+    with pytest.raises(RuntimeError, match="bn2"):
+        dst.load_encodings(stray)
+    dst.load_encodings(stray, strict=False)
+    assert dict(dst.qmodules())["bn2"].output_quantizers[0] is None
+
+    # partial=False: only fc keeps quantizers; requires_grad reaches the imported min / max
+    only_fc = {"param_encodings": {"fc.weight": full["param_encodings"]["fc.weight"]},
+               "activation_encodings": {"fc": full["activation_encodings"]["fc"]}}
+    part = V2Sim(model, dummy, quant_scheme='tf', default_param_bw=8, per_channel_quantization=True)
+    part.load_encodings(only_fc, partial=False, requires_grad=True)
+    qm = dict(part.qmodules())
+    assert qm["conv1"].param_quantizers["weight"] is None and qm["relu1"].output_quantizers[0] is None
+    fcq = qm["fc"].param_quantizers["weight"]
+    assert fcq is not None and all(p.requires_grad for p in fcq.parameters())
+    assert qm["fc"].output_quantizers[0] is not None
+
+    # frozen quantizers ignore a later import
+    frozen = V2Sim(model, dummy, quant_scheme='tf', default_param_bw=8, per_channel_quantization=True)
+    frozen.load_encodings(only_fc, allow_overwrite=False)
+    changed = {"param_encodings": {"fc.weight": [dict(e, min=2 * e["min"], max=2 * e["max"], scale=2 * e["scale"])
+                                                 for e in full["param_encodings"]["fc.weight"]]}}
+    frozen.load_encodings(changed)
+    got = dict(frozen.qmodules())["fc"].param_quantizers["weight"].get_legacy_encodings()
+    assert got[0]["scale"] == pytest.approx(full["param_encodings"]["fc.weight"][0]["scale"], rel=1e-6)
