@@ -31,7 +31,9 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kBatch  = 32;    // rows per iteration (BATCH_SIZE of ADA/adaround_optimizer.py:58)
 constexpr int kTileO  = 32;    // output channels per workgroup
-constexpr int kTileK  = 256;   // K extent per workgroup: one 1 KiB row segment per wavefront-wide 16-byte access
+constexpr int kTileK  = 256;   // K extent of a tile: one 1 KiB row segment per wavefront-wide 16-byte access
+constexpr int kFwdTileK = 128;        // k extent of a forward tile
+constexpr int kFwdGroupsWanted = 512; // forward workgroups: two of them fit on each of the 256 CUs
 
 struct LinGeom
 {
@@ -67,132 +69,259 @@ __device__ __forceinline__ v4f ldg4_stream(const float* p)
 
 // Four consecutive values of floor(W / delta), stored as float32 or, where every channel's window of useful values fits,
 // as int8 or int16 (miq_adaround_floor_i8 / _i16): a quarter or half of the bytes of the operand that never changes
-// during the optimisation.
+// during the optimisation.  `type` is the raw form in which they travel from memory (one register for int8): the
+// forward kernel keeps them like that while the loads are in flight.
 template <typename FT>
-__device__ __forceinline__ v4f load_floor4(const FT* p);
+struct FloorRaw;
 template <>
-__device__ __forceinline__ v4f load_floor4<float>(const float* p)
+struct FloorRaw<float>
 {
-    return ldg4_stream(p);
-}
+    typedef v4f type;
+    static __device__ __forceinline__ type load(const float* p) { return ldg4_stream(p); }
+    static __device__ __forceinline__ v4f widen(type w) { return w; }
+};
 template <>
-__device__ __forceinline__ v4f load_floor4<int8_t>(const int8_t* p)
+struct FloorRaw<int8_t>
 {
-    const int32_t w = __builtin_nontemporal_load(reinterpret_cast<const int32_t*>(p));
-    return (v4f) {(float) (int8_t) (w & 0xff), (float) (int8_t) ((w >> 8) & 0xff), (float) (int8_t) ((w >> 16) & 0xff),
-                  (float) (w >> 24)};
-}
+    typedef int32_t type;
+    static __device__ __forceinline__ type load(const int8_t* p)
+    {
+        return __builtin_nontemporal_load(reinterpret_cast<const int32_t*>(p));
+    }
+    static __device__ __forceinline__ v4f widen(type w)
+    {
+        return (v4f) {(float) (int8_t) (w & 0xff), (float) (int8_t) ((w >> 8) & 0xff), (float) (int8_t) ((w >> 16) & 0xff),
+                      (float) (w >> 24)};
+    }
+};
+template <>
+struct FloorRaw<int16_t>
+{
+    typedef int type __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ type load(const int16_t* p)
+    {
+        return __builtin_nontemporal_load(reinterpret_cast<const type*>(p));
+    }
+    static __device__ __forceinline__ v4f widen(type w)
+    {
+        return (v4f) {(float) (int16_t) (w[0] & 0xffff), (float) (w[0] >> 16), (float) (int16_t) (w[1] & 0xffff),
+                      (float) (w[1] >> 16)};
+    }
+};
 
-template <>
-__device__ __forceinline__ v4f load_floor4<int16_t>(const int16_t* p)
+template <typename FT>
+__device__ __forceinline__ v4f load_floor4(const FT* p)
 {
-    typedef int v2i __attribute__((ext_vector_type(2)));
-    const v2i w = __builtin_nontemporal_load(reinterpret_cast<const v2i*>(p));
-    return (v4f) {(float) (int16_t) (w[0] & 0xffff), (float) (w[0] >> 16), (float) (int16_t) (w[1] & 0xffff),
-                  (float) (w[1] >> 16)};
+    return FloorRaw<FT>::widen(FloorRaw<FT>::load(p));
 }
 
 constexpr int kLdsRow = kTileK + 4;   // floats per LDS tile row; the pad spreads the MFMA-layout accesses over banks
 
-// Both kernels work on a [32 o] x [256 k] tile of the weight-shaped tensors per workgroup and move it through LDS, so
-// that global memory is always touched in the streaming layout (lane l of a wavefront owns floats 4l..4l+3 of a 1 KiB
-// row segment: fully coalesced) while the MFMAs see their own operand / accumulator layout.
+// Both kernels move [32 o] x [256 k] (backward) or [32 o] x [128 k] (forward) tiles of the weight-shaped tensors
+// through LDS, so that global memory is always touched in the streaming layout (a lane owns 16 consecutive bytes of a
+// row segment that its wavefront covers without gaps) while the MFMAs see their own operand / accumulator layout.
 // (Measured alternative: wavefront-private [16 o] x [128 k] tiles without workgroup barriers were 10-20 % slower.)
 
-// grid (K / 256, O / 32), 256 threads: consecutive workgroups walk along the rows, so the workgroups that run together
-// cover contiguous memory (with the row blocks as the fast index the same tile reads measured 25 % slower).
-template <typename FT>
-__global__ __launch_bounds__(256) void lin_fwd_kernel(const FT* __restrict__ F, const float* __restrict__ alpha,
-                                                      const float* __restrict__ X, const int* __restrict__ row_index,
-                                                      int num_rows, int64_t x_row_stride, float* __restrict__ partial,
-                                                      LinGeom g)
+// Workgroup barrier that waits for this wavefront's LDS traffic only.  __syncthreads() would also wait for every
+// global load in flight, and the point of the loop below is to keep the next tile's loads in flight across it.
+__device__ __forceinline__ void lds_barrier()
 {
-    __shared__ __attribute__((aligned(16))) float tile[kTileO * kLdsRow];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int n = lane & 15, s = lane >> 4;
-    const int o_blk = blockIdx.y * kTileO;
-    const int k_blk = blockIdx.x * kTileK;
-    const int K     = g.in_features;
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
 
-    // phase 1: adarounded weight tile, streaming layout: wavefront w forms rows 8w .. 8w+7
-    // the rows' delta / offset are requested first: a load issued where it is used makes that row wait for a round trip
-    float dl[8], of[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
+// Forward tiles ([32 o] x [TK k]) are stored without a row pad, 16-byte chunk q of row r at chunk q ^ (r & 15): a
+// wavefront's streaming store (consecutive chunks of a row) and its MFMA-layout load (16 rows x one chunk, four chunk
+// columns) both touch every bank group once (SQ_LDS_BANK_CONFLICT reads 0).
+template <int TK>
+__device__ __forceinline__ int fwd_slot(int r, int chunk)
+{
+    return r * TK + 4 * (chunk ^ (r & 15));
+}
+
+// grid (ceil(K / TK / tiles_per_group), O / 32), 512 threads.  A workgroup owns 32 output channels and walks
+// `tiles_per_group` consecutive TK-wide k tiles of them with its eight wavefronts in two roles:
+//   wavefronts 4..7 (producers) stream floor(W / delta) and alpha, form W' and store it to one of two LDS tiles;
+//   wavefronts 0..3 (consumers) multiply the other LDS tile with the 32 activation rows on the MFMA.
+// One barrier per tile hands a finished tile over.  Every SIMD so holds wavefronts that issue the conversion's vector
+// arithmetic and wavefronts that issue MFMAs -- the two run in different pipes -- and a producer requests its next tile
+// as soon as it has converted one, before it waits at the barrier.
+// Consumer w multiplies k in [TK/4 w, TK/4 (w + 1)) of every tile and keeps its [32 b] x [32 o] partial product in
+// registers; the four are added once, at the end: K / TK / tiles_per_group partial products per output in the workspace.
+// Consecutive workgroups walk along the rows, so the workgroups that run together cover contiguous memory.
+//
+// Measured on the [4096, 4096] layer with int8 floor values (84 MB moved; the same loads and barriers without the
+// conversion and the MFMAs take 20 us):
+//   one tile per 256-thread workgroup, every wavefront converts, then multiplies (2048 workgroups)       28.8 us
+//   the same wavefronts walking 4 tiles with the next tile's loads in flight                              27.7 us
+//   producer / consumer roles, TK 256, producers two tiles ahead                                          27.0 us
+//   roles, TK 128: producers four / two / one tile ahead                                    26.0 / 23.4 / 22.9 us
+//   roles, TK 64, one tile ahead, two / four workgroups per CU                                     25.3 / 24.3 us
+// What a workgroup still has to compute when its last bytes arrive (a conversion, then a multiplication) is exposed at
+// the end of the kernel, and loads requested further ahead arrive in larger bunches: small tiles, one tile ahead.
+// Raising the producers' or the consumers' wavefront priority changed nothing or lost 1.5 us.
+template <typename FT, int TK>
+__global__ __launch_bounds__(512, 4) void lin_fwd_kernel(const FT* __restrict__ F, const float* __restrict__ alpha,
+                                                         const float* __restrict__ X, const int* __restrict__ row_index,
+                                                         int num_rows, int64_t x_row_stride, float* __restrict__ partial,
+                                                         LinGeom g, int tiles_per_group)
+{
+    static_assert(TK == 64 || TK == 128 || TK == 256, "a wavefront-wide 16-byte access covers one, two or four rows of a tile");
+    constexpr int kLoads  = 8 * TK / 256;   // 16-byte accesses per lane and tile: 8 rows of TK floats per wavefront
+    constexpr int kRowsPerLoad = 256 / TK;  // rows one wavefront-wide access covers
+    constexpr int kSteps  = TK / 64;        // MFMA k steps of 16 per consumer and tile
+    typedef FloorRaw<FT> Raw;
+    __shared__ __attribute__((aligned(16))) float tile[2 * kTileO * TK];
+    // the wavefront number as a scalar: the role branch below is then a scalar branch, and a wavefront executes the
+    // barriers of its own role only
+    const int wave = __builtin_amdgcn_readfirstlane((int) (threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63;
+    const int w4   = wave & 3;
+    const int o_blk   = blockIdx.y * kTileO;
+    const int K       = g.in_features;
+    const int t_first = blockIdx.x * tiles_per_group;
+    const int T       = min(tiles_per_group, K / TK - t_first);   // tiles of this workgroup (>= 1)
+    float* const buf0 = tile;
+    float* const buf1 = tile + kTileO * TK;
+    v4f* const red    = reinterpret_cast<v4f*>(tile);   // after the last tile: [4 consumers][4 blocks][64 lanes]
+    static_assert(2 * kTileO * TK >= 4 * 4 * 64 * 4, "the partial products reuse the tiles' memory");
+
+    if (wave >= 4)
     {
-        const int c = (o_blk + wave * 8 + j) * g.chan_stride;
-        dl[j]       = g.delta[c];
-        of[j]       = g.offset[c];
-    }
-    v4f f[8], al[8];
+        // ---- producer: rows 8 w4 .. 8 w4 + 7 of every tile, streaming layout: access j of lane l is row
+        // kRowsPerLoad j + l / (TK / 4), floats 4 (l % (TK / 4)) .. + 3
+        const int sub_row = lane / (TK / 4), col4 = lane % (TK / 4);
+        float dl[kLoads], of[kLoads];
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < kLoads; ++j)
+        {
+            const int c = (o_blk + w4 * 8 + kRowsPerLoad * j + sub_row) * g.chan_stride;
+            dl[j]       = g.delta[c];
+            of[j]       = g.offset[c];
+        }
+        // everything but the lane's own offset is the same for the whole wavefront: scalar address arithmetic
+        const int64_t w_base      = (int64_t) (o_blk + w4 * 8) * K + (int64_t) t_first * TK;
+        const FT* const f_base    = F + w_base;
+        const float* const a_base = alpha + w_base;
+        const int64_t lane_off    = (int64_t) sub_row * K + 4 * col4;
+        typename Raw::type f[kLoads];
+        v4f al[kLoads];
+        auto request = [&](int i) {
+#pragma unroll
+            for (int j = 0; j < kLoads; ++j)
+            {
+                const int64_t row = (int64_t) (kRowsPerLoad * j) * K + i * TK;
+                f[j]  = Raw::load(f_base + row + lane_off);
+                al[j] = ldg4_stream(a_base + row + lane_off);
+            }
+        };
+        auto convert = [&](float* buf) {
+#pragma unroll
+            for (int j = 0; j < kLoads; ++j)
+            {
+                const v4f f4 = Raw::widen(f[j]);
+                v4f wq;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    wq[i] = adarounded_f<true>(f4[i], al[j][i], dl[j], of[j], g.clip_min, g.clip_max);
+                *reinterpret_cast<v4f*>(&buf[fwd_slot<TK>(w4 * 8 + kRowsPerLoad * j + sub_row, col4)]) = wq;
+            }
+        };
+        request(0);
+        convert(buf0);
+        if (1 < T)
+            request(1);
+        lds_barrier();
+        // phase i: tile i + 1 is converted while the consumers multiply tile i
+        for (int i0 = 0; i0 < T; i0 += 2)
+        {
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+            {
+                const int i = i0 + u;
+                if (i >= T)
+                    break;
+                if (i + 1 < T)
+                {
+                    convert(u == 0 ? buf1 : buf0);
+                    if (i + 2 < T)
+                        request(i + 2);
+                }
+                lds_barrier();
+            }
+        }
+    }
+    else
     {
-        const int64_t e = (int64_t) (o_blk + wave * 8 + j) * K + k_blk + 4 * lane;
-        f[j]            = load_floor4<FT>(F + e);
-        al[j]           = ldg4_stream(alpha + e);
-    }
-    // the activations of this wavefront's MFMA k-range [64w, 64w + 64), fetched while the weights are in flight
-    const float* xrow[2];
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-    {
-        const int b = mt * 16 + n;
-        xrow[mt]    = X + gather_row(row_index, b, num_rows) * x_row_stride + k_blk + wave * 64 + 4 * s;
-    }
-    v4f a[4][2];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
+        // ---- consumer: MFMA layout, lane (n, s) supplies batch rows n and 16 + n, k = TK/4 w4 + 16 kk + 4 s + i
+        const int n = lane & 15, s = lane >> 4;
+        const float* xrow[2];
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
-            a[kk][mt] = ldg4(xrow[mt] + kk * 16);
+            xrow[mt] = X + gather_row(row_index, mt * 16 + n, num_rows) * x_row_stride + (int64_t) t_first * TK +
+                       w4 * (TK / 4) + 4 * s;
+        v4f acc[2][2];
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-    {
-        const int r = wave * 8 + j;
-        v4f wq;
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-            wq[t] = adarounded_f<true>(f[j][t], al[j][t], dl[j], of[j], g.clip_min, g.clip_max);
-        *reinterpret_cast<v4f*>(&tile[r * kLdsRow + 4 * lane]) = wq;
-    }
-    __syncthreads();
-
-    // phase 2: out[b][o] += x[b][k] W'[o][k] over this wavefront's 64 k
-    v4f acc[2][2];
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
-            acc[mt][nt] = (v4f) {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk)
-    {
-        const int col = wave * 64 + kk * 16 + 4 * s;
-        v4f wq[2];
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
-            wq[nt] = *reinterpret_cast<const v4f*>(&tile[(nt * 16 + n) * kLdsRow + col]);
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
             for (int nt = 0; nt < 2; ++nt)
+                acc[mt][nt] = (v4f) {0.f, 0.f, 0.f, 0.f};
+        v4f x[2][kSteps][2];
+        auto request_x = [&](v4f(&xr)[kSteps][2], int i) {
+#pragma unroll
+            for (int kk = 0; kk < kSteps; ++kk)
 #pragma unroll
                 for (int mt = 0; mt < 2; ++mt)
-                    acc[mt][nt] = mfma16(a[kk][mt][t], wq[nt][t], acc[mt][nt]);
+                    xr[kk][mt] = ldg4(xrow[mt] + i * TK + kk * 16);
+        };
+        auto multiply = [&](const v4f(&xr)[kSteps][2], const float* buf) {
+            v4f wq[kSteps][2];
+#pragma unroll
+            for (int kk = 0; kk < kSteps; ++kk)
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt)
+                    wq[kk][nt] =
+                        *reinterpret_cast<const v4f*>(&buf[fwd_slot<TK>(nt * 16 + n, w4 * (TK / 16) + kk * 4 + s)]);
+#pragma unroll
+            for (int kk = 0; kk < kSteps; ++kk)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                        for (int mt = 0; mt < 2; ++mt)
+                            acc[mt][nt] = mfma16(xr[kk][mt][i], wq[kk][nt][i], acc[mt][nt]);
+        };
+        request_x(x[0], 0);
+        if (1 < T)
+            request_x(x[1], 1);
+        lds_barrier();
+        for (int i0 = 0; i0 < T; i0 += 2)
+        {
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+            {
+                const int i = i0 + u;
+                if (i >= T)
+                    break;
+                multiply(x[u], u == 0 ? buf0 : buf1);
+                if (i + 2 < T)
+                    request_x(x[u], i + 2);
+                lds_barrier();
+            }
+        }
+        // the barrier above followed every consumer's last multiplication: the tiles' memory is free
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+                red[(wave * 4 + mt * 2 + nt) * 64 + lane] = acc[mt][nt];
     }
-    __syncthreads();   // every wavefront is done reading the weight tile: its memory now holds the partial products
-
-    // add the four wavefronts' products in wavefront order, then one partial [32, 32] tile per workgroup
-    v4f* red = reinterpret_cast<v4f*>(tile);   // [4 waves][4 tiles][64 lanes]
-#pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
-            red[(wave * 4 + mt * 2 + nt) * 64 + lane] = acc[mt][nt];
+    // Both roles have passed T + 1 barriers.  Add the four consumers' products in wavefront order, then one partial
+    // [32, 32] block per workgroup.
     __syncthreads();
+    if (wave < 4)
     {
-        const int t4 = threadIdx.x >> 6, ln = threadIdx.x & 63;   // tile index, lane within the tile
+        const int t4 = wave, ln = lane;   // block index, lane within the block
         const v4f sum = ((red[(0 * 4 + t4) * 64 + ln] + red[(1 * 4 + t4) * 64 + ln]) + red[(2 * 4 + t4) * 64 + ln]) +
                         red[(3 * 4 + t4) * 64 + ln];
         const int mt = t4 >> 1, nt = t4 & 1;
@@ -217,9 +346,18 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
     if (idx < kBatch * out_features)
     {
         const int b = idx / out_features, o = idx - b * out_features;
-        float acc = 0.f;
-        for (int s = 0; s < num_split; ++s)
-            acc += partial[((int64_t) s * kBatch + b) * out_features + o];
+        // the partial products are added in split order; four of them are requested at a time
+        const float* p      = partial + (int64_t) b * out_features + o;
+        const int64_t pitch = (int64_t) kBatch * out_features;
+        float acc           = 0.f;
+        int s               = 0;
+        for (; s + 4 <= num_split; s += 4)
+        {
+            const float p0 = p[s * pitch], p1 = p[(s + 1) * pitch], p2 = p[(s + 2) * pitch], p3 = p[(s + 3) * pitch];
+            acc            = (((acc + p0) + p1) + p2) + p3;
+        }
+        for (; s < num_split; ++s)
+            acc += p[s * pitch];
         if (bias)
             acc += bias[o];
         const int r = row_index ? row_index[b] : b;
@@ -389,6 +527,17 @@ int make_lin_geom(LinGeom& g, int64_t out_features, int64_t in_features, int64_t
 
 using namespace miq;
 
+// Consecutive k tiles per forward workgroup: as many as still leave one workgroup for each of the 512 places the chip
+// has for this kernel (two per CU, 256 CUs), at most 16.
+static int fwd_tiles_per_group(int64_t out_features, int64_t in_features)
+{
+    const int64_t along = in_features / kFwdTileK;
+    const int64_t tiles = (out_features / kTileO) * along;
+    int64_t per_group   = tiles / kFwdGroupsWanted;
+    per_group           = per_group < 1 ? 1 : (per_group > 16 ? 16 : per_group);
+    return (int) (per_group > along ? along : per_group);
+}
+
 template <typename FT>
 static int linear_fwd(const FT* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
                       int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
@@ -406,10 +555,11 @@ static int linear_fwd(const FT* weight_floor, const float* alpha, const float* x
     MIQ_CHECK_ARG(activation == 0 || activation == 1, "activation must be 0 (none) or 1 (ReLU)");
     MIQ_CHECK_ARG(num_rows >= 1 && num_rows < (1ll << 31) && (row_index || num_rows >= kBatch),
                   "num_rows (%lld) must be positive, and at least 32 without a row index", (long long) num_rows);
-    const int splits = (int) (in_features / kTileK);
-    hipLaunchKernelGGL((lin_fwd_kernel<FT>), dim3((unsigned) splits, (unsigned) (out_features / kTileO)), dim3(256), 0,
-                       (hipStream_t) stream, weight_floor, alpha, x, row_index, (int) num_rows, x_row_stride, workspace,
-                       g);
+    const int tiles_per_group = fwd_tiles_per_group(out_features, in_features);
+    const int splits          = (int) ((in_features / kFwdTileK + tiles_per_group - 1) / tiles_per_group);
+    hipLaunchKernelGGL((lin_fwd_kernel<FT, kFwdTileK>),
+                       dim3((unsigned) splits, (unsigned) (out_features / kTileO)), dim3(512), 0, (hipStream_t) stream,
+                       weight_floor, alpha, x, row_index, (int) num_rows, x_row_stride, workspace, g, tiles_per_group);
     MIQ_CHECK_LAUNCH();
     const unsigned blocks = (unsigned) ((kBatch * out_features + 255) / 256);
     hipLaunchKernelGGL(lin_loss_kernel, dim3(blocks), dim3(256), 0, (hipStream_t) stream, workspace, splits, bias, target,
@@ -453,7 +603,11 @@ int64_t miq_adaround_linear_workspace_bytes(int64_t out_features, int64_t in_fea
 {
     if (out_features <= 0 || in_features <= 0)
         return 0;
-    const int64_t splits = (in_features + kTileK - 1) / kTileK;
+    if (out_features % kTileO != 0 || in_features % kTileK != 0)
+        return 0;   // not a shape the fused path takes
+    const int64_t along  = in_features / kFwdTileK;
+    const int64_t per    = fwd_tiles_per_group(out_features, in_features);
+    const int64_t splits = (along + per - 1) / per;
     return splits * kBatch * out_features * (int64_t) sizeof(float);
 }
 
