@@ -105,5 +105,73 @@ MIQ_HD inline int bucket_row(float x, const BucketMap& m)
     const float r = round_half_away(q - m.off);
     return (r >= 0.0f && r < (float) BUCKETS) ? (int) r + 1 : 0;
 }
+
+// ---- bin of torch.histc --------------------------------------------------------------------------------------
+// torch.histc(x, bins, lo, hi) counts x in bin (int) ((x - lo) * bins / (hi - lo)), all binary32, x == hi in the last
+// bin (ATen/native/cuda/SummaryOps.cu getBin; the CPU kernel agrees).  The histogram observer adds: below lo -> first
+// bin, above hi -> last bin.  bin() evaluates exactly that sequence (the division through div_by_invariant where its
+// contract holds).  Most samples are answered by one fused multiply-add instead,
+//     u = fma(x, RN(bins / width), RN(-lo * RN(bins / width))):
+// with K = max(|lo|, |hi|) / width, u lies within bins (K + 2) 2^-24 of the real number (x - lo) bins / width (one
+// rounding each in the scale, the shift and the result), and the three roundings of the sequence keep it within
+// 3 bins 2^-24 of the same number, so the truncated sequence and floor(u) agree whenever the fraction of u stays
+// eps = bins (K + 1) 2^-21 (more than 1.6 times the sum of the bounds) away from 0 and 1; u below 0 or from bins on is
+// what the observer's rule for outside values maps to the end bins.  Samples
+// within eps of a bin edge, infinities, NaN (bin -1) and ranges for which eps reaches 1/4 take the sequence.
+// tests/test_fastmath.py checks bin() against the plain sequence on ranges over many decades, the floats around every
+// bin edge and random samples.
+struct HistcBinner
+{
+    float lo, hi, width, recip, nbf;
+    int nb;
+    bool divisor_ok;
+    float fast_scale, fast_shift, thr;   // thr <= 0: the one-operation path is never taken
+
+    MIQ_HD void init(float lo_, float hi_, int nb_)
+    {
+        lo         = lo_;
+        hi         = hi_;
+        nb         = nb_;
+        nbf        = (float) nb_;
+        width      = hi_ - lo_;
+        divisor_ok = fastdiv_divisor_ok(width);
+        recip      = divisor_ok ? 1.0f / width : 0.f;
+        fast_scale = nbf / width;
+        fast_shift = -lo_ * fast_scale;
+        const float k   = __builtin_fmaxf(__builtin_fabsf(lo_), __builtin_fabsf(hi_)) / width;
+        const float eps = nbf * (k + 1.0f) * 4.76837158203125e-07f;   // 2^-21
+        // (comparisons are false for NaN: a range that is not finite never takes the short path)
+        thr = (divisor_ok && eps < 0.25f && __builtin_fabsf(fast_shift) < 1e30f && fast_scale < 1e30f) ? 0.5f - eps
+                                                                                                     : -1.0f;
+    }
+
+    MIQ_HD int bin_by_sequence(float x) const
+    {
+        if (x != x)
+            return -1;
+        if (x < lo)
+            return 0;
+        if (x > hi)
+            return nb - 1;
+        const float a = (x - lo) * nbf;
+        const float q = (divisor_ok && a <= kFastDivMaxDividend) ? div_by_invariant(a, width, recip) : a / width;
+        const int pos = (int) q;
+        return pos >= nb ? nb - 1 : pos;
+    }
+
+    MIQ_HD int bin(float x) const
+    {
+        const float u  = __builtin_fmaf(x, fast_scale, fast_shift);
+        const float fl = __builtin_floorf(u);
+        const float f  = u - fl;   // exact; NaN for infinite u
+        if (__builtin_fabsf(f - 0.5f) < thr)
+        {
+            // |fl| < 2^23 here (larger floats have no fraction: f == 0 fails the test)
+            const int k = (int) fl;
+            return k < 0 ? 0 : (k >= nb ? nb - 1 : k);
+        }
+        return bin_by_sequence(x);
+    }
+};
 }   // namespace miq
 #endif

@@ -367,7 +367,8 @@ def minmax_per_channel(x, num_channel, n_per_channel):
 # ------------------------------------------------------------------------------------- v2 histogram observer / SQNR
 def v2_hist_workspace(num_hist, n_per_hist, num_bins, device):
     nbytes = int(lib.miq_v2_hist_workspace_bytes(int(num_hist), int(n_per_hist), int(num_bins)))
-    return torch.empty((nbytes + 3) // 4, dtype=torch.int32, device=device)
+    # zero-filled: the library keeps counters in it that are zero between updates
+    return torch.zeros((nbytes + 3) // 4, dtype=torch.int32, device=device)
 
 
 def v2_hist_update(data, num_hist, num_bins, has_stats, state_hist, state_minmax, bad_flag, workspace,

@@ -442,9 +442,13 @@ int64_t miq_v2_hist_workspace_bytes(int64_t num_hist, int64_t n_per_hist, int nu
  * (what collect_stats returns) to batch_hist / batch_minmax and merges them into state_* (has_stats = 0: the state is
  * empty and becomes the batch's statistics).  bad_flag: device int32, set to 1 when a slab holds no finite value (the
  * reference raises ValueError there; the caller checks the flag when it next reads results).  workspace: device
- * buffer of miq_v2_hist_workspace_bytes.  want_batch_hist = 0 skips the batch's own histogram (batch_hist may then be
- * NULL; batch_minmax, optional, is still written): only callers that quantize dynamically with the batch's statistics
- * read it.  Enqueues four kernels; never synchronises. */
+ * buffer of miq_v2_hist_workspace_bytes, zero-filled by the caller before its first use and not written by anyone
+ * else afterwards (it holds counters that every update leaves at zero); updates that share a workspace must not
+ * overlap.  want_batch_hist = 0 skips the batch's own histogram (batch_hist may then be NULL; batch_minmax, optional,
+ * is still written): only callers that quantize dynamically with the batch's statistics read it.
+ * has_stats = 1, want_batch_hist = 0 (the calibration loop) enqueues two kernels and reads the batch once as long as
+ * the batch stays inside the statistics' range (twice when it does not); the other modes enqueue three kernels and
+ * read it twice.  Never synchronises. */
 int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hist, int num_bins, int has_stats,
                            int want_batch_hist, float* state_hist, float* state_minmax, float* batch_hist,
                            float* batch_minmax, int32_t* bad_flag, void* workspace, void* stream);

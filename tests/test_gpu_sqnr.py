@@ -98,6 +98,54 @@ def test_very_large_and_concentrated_inputs(ea):
     assert hist.sum().item() == 40_000_000
 
 
+def test_updates_inside_and_outside_the_running_range(ea):
+    """An update of running statistics bins the batch over the statistics' range while it looks for the batch's own
+    range, and redoes the binning only when the range grew.  Long runs of batches that stay inside, batches that grow
+    the range on one side or both, a batch that repeats the extremes exactly, non-finite values in either kind of
+    batch, sizes that are not a multiple of the vector width: the running histogram equals torch.histc + merge_stats
+    of the restatement after every update, and the counters the library keeps in its workspace are back at zero."""
+    g = torch.Generator().manual_seed(21)
+    obs = ea._HistogramObserver((1,), 2048)
+    ref = sq.SqnrAnalyzer(1, 2048)
+    first = torch.randn(70001, generator=g) * 2
+    plan = [first]
+    plan += [torch.randn(50000 + 7 * k, generator=g) * 0.5 for k in range(6)]            # inside
+    plan += [torch.cat([torch.randn(1000, generator=g), first.max().view(1), first.min().view(1)])]   # touches both ends
+    plan += [torch.randn(30000, generator=g) * 4]                                          # grows on both sides
+    plan += [torch.randn(30000, generator=g) for _ in range(3)]                            # inside the new range
+    plan += [torch.rand(999, generator=g) * 40]                                            # grows on the right
+    inside_bad = torch.randn(20000, generator=g)
+    inside_bad[:3] = torch.tensor([float('nan'), float('inf'), -float('inf')])
+    plan += [inside_bad]                                                                   # inside, non-finite values
+    grow_bad = torch.randn(20000, generator=g) * 30
+    grow_bad[5:8] = torch.tensor([float('nan'), float('inf'), -float('inf')])
+    plan += [grow_bad, torch.randn(4096 * 64, generator=g)]
+    for x in plan:
+        obs.merge_stats(None, x.cuda())
+        ref.update_stats(x)
+        _same_hist(obs.get_stats()[0], ref.stats[0])
+        assert int(obs._workspace[:2 * 2048].abs().sum()) == 0                    # pylint: disable=protected-access
+
+
+def test_per_channel_updates_where_some_ranges_grow(ea):
+    """Per-channel statistics, one update in which some channels stay inside their range and others grow: each
+    histogram takes its own path."""
+    torch.manual_seed(22)
+    shape = (5, 1, 1)
+    obs = ea._HistogramObserver(shape, 512)
+    ref = sq.SqnrAnalyzer(5, 512)
+    base = torch.randn(5, 40, 1000)
+    scales = [torch.tensor(v).view(5, 1, 1) for v in ([1.0] * 5, [0.5, 2.0, 0.5, 3.0, 0.9], [0.1] * 5,
+                                                       [4.0, 0.2, 0.2, 0.2, 5.0], [1.0] * 5)]
+    for k, sc in enumerate(scales):
+        x = torch.randn(5, 40, 1000) * sc if k else base
+        obs.merge_stats(None, x.cuda())
+        ref.update_stats(x)
+        st = obs.get_stats()
+        for i in range(5):
+            _same_hist(st[i], ref.stats[i])
+
+
 @pytest.mark.parametrize("symmetric", [False, True])
 @pytest.mark.parametrize("num_steps,gamma", [(255.0, 3.0), (255.0, 1.0), (15.0, 3.0), (65535.0, 3.0)])
 def test_search_matches_restatement(ea, symmetric, num_steps, gamma):
