@@ -104,14 +104,17 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         if self._quant_scheme == QuantScheme.post_training_tf:
             maxval = largest
         else:
-            fractions = torch.linspace(0.1, 1.2, 111, device=tensor.device)
+            # candidates as aimet_torch/fp_quantization.py:78-110 forms them: per channel, 111 float32 values from
+            # torch.linspace(0.1 * largest, 1.2 * largest) with Python-float end points
+            ends = largest.reshape(-1).cpu().tolist()
+            candidates = torch.stack([torch.linspace(0.1 * mx, 1.2 * mx, 111) for mx in ends]).to(tensor.device).t()
             errors = []
-            for fraction in fractions:
-                cast = ops.fp8_fake_cast(tensor, largest * fraction, 3, axis or 0)
+            for candidate in candidates:                              # [111, channels]
+                cast = ops.fp8_fake_cast(tensor, candidate if per_channel else candidate[0], 3, axis or 0)
                 squared = (tensor - cast) ** 2
-                errors.append(squared.mean(dim=other) if per_channel and other else squared.mean())
+                errors.append((squared.mean(dim=other) if per_channel and other else squared.mean()).reshape(-1))
             best = torch.stack(errors).argmin(0)
-            maxval = largest * fractions[best]
+            maxval = candidates.gather(0, best.view(1, -1)).view(largest.shape)
         self.update_maxval(maxval)
         self._encoding = [libpymo.TfEncoding(-float(m), float(m), 0.0, 0.0, 8)
                           for m in self.fp8_maxval.reshape(-1).tolist()]
