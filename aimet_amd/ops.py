@@ -380,13 +380,34 @@ def v2_hist_update(data, num_hist, num_bins, has_stats, state_hist, state_minmax
         raise RuntimeError("the histogram observer takes contiguous float32 data")
     n_per_hist = data.numel() // num_hist
     batch_hist = torch.empty(num_hist, num_bins, dtype=_F32, device=data.device) if want_batch_hist else None
-    batch_minmax = torch.empty(num_hist, 2, dtype=_F32, device=data.device)
+    batch_minmax = torch.empty(num_hist, 2, dtype=_F32, device=data.device) if want_batch_hist else None
     with _OnDevice(data.device):
         check(lib.miq_v2_hist_update_f32(_ptr(data), int(num_hist), int(n_per_hist), int(num_bins), int(has_stats),
                                          int(bool(want_batch_hist)), _ptr(state_hist), _ptr(state_minmax),
                                          _ptr(batch_hist), _ptr(batch_minmax), _ptr(bad_flag), _ptr(workspace),
                                          _stream(data)))
     return batch_hist, batch_minmax
+
+
+class V2HistRepeat:
+    """A prepared v2_hist_update for running per-tensor statistics (one histogram, has_stats, no batch histogram):
+    everything but the data pointer and the stream is fixed, so the calibration loop's call costs one check and one
+    foreign call.  Holds the state tensors it points into."""
+    __slots__ = ("_device", "_numel", "_args", "_keep")
+
+    def __init__(self, like, num_bins, state_hist, state_minmax, bad_flag, workspace):
+        self._device = like.get_device()
+        self._numel = like.numel()
+        self._keep = (state_hist, state_minmax, bad_flag, workspace)
+        self._args = (1, self._numel, int(num_bins), 1, 0, state_hist.data_ptr(), state_minmax.data_ptr(), None, None,
+                      bad_flag.data_ptr(), workspace.data_ptr())
+
+    def matches(self, data):
+        return (data.get_device() == self._device and data.numel() == self._numel and data.dtype == _F32
+                and data.is_contiguous() and torch.cuda.current_device() == self._device)
+
+    def __call__(self, data):
+        check(lib.miq_v2_hist_update_f32(data.data_ptr(), *self._args, _stream_of(data.device)))
 
 
 def v2_sqnr_num_candidates(num_steps, symmetric, asym_deltas, sym_deltas, offset_candidates):

@@ -212,6 +212,7 @@ class _HistogramObserver:
 
     def reset_stats(self):
         self._state = None          # _DeviceHistograms once the first batch has been seen
+        self._repeat = None         # prepared call for the next update of the same kind (per-tensor statistics)
         self._workspace = None
         self._bad_flag = None
 
@@ -220,6 +221,8 @@ class _HistogramObserver:
             raise RuntimeError(f"Shape {self.shape} is incompatible with input of shape {input_tensor.shape}")
         if not input_tensor.is_cuda:
             raise RuntimeError("the histogram observer (aimet_amd) computes on the GPU only")
+        if self.num_histograms == 1 and input_tensor.dtype == torch.float32 and input_tensor.is_contiguous():
+            return input_tensor.detach().view(1, -1)                  # the common case, without the general reshuffle
         # one contiguous slab per histogram; layouts that are not already slabs take one copy
         tensor3, _ = channel_view(input_tensor.detach().to(torch.float32), self.shape)
         if tensor3.shape[0] != 1:
@@ -228,6 +231,7 @@ class _HistogramObserver:
 
     @torch.no_grad()
     def _update(self, input_tensor: torch.Tensor, merge: bool, want_batch: bool = True):
+        self._repeat = None         # (state tensors and workspace may be replaced below)
         data = self._slabs(input_tensor)
         n_per_hist = data.numel() // self.num_histograms
         device = data.device
@@ -263,7 +267,14 @@ class _HistogramObserver:
         """collect_stats followed by merge_stats.  The batch's own histogram is what only dynamic quantization inside
         compute_encodings() reads, so it is formed when first looked at, from the tensor handed in here (which the
         caller therefore must not modify in place before looking)."""
-        self._update(input_tensor, merge=True, want_batch=False)
+        repeat = self._repeat
+        if repeat is not None and repeat.matches(input_tensor):
+            repeat(input_tensor)          # same device, size and layout as the update before: nothing to set up
+        else:
+            self._update(input_tensor, merge=True, want_batch=False)
+            if self.num_histograms == 1 and input_tensor.dtype == torch.float32 and input_tensor.is_contiguous():
+                self._repeat = ops.V2HistRepeat(input_tensor, self.num_bins, self._state.hist, self._state.minmax,
+                                                self._bad_flag, self._workspace)
         return _LazyBatchHistograms(self, input_tensor)
 
     def merge_stats(self, new_stats_list, input_tensor: torch.Tensor):
