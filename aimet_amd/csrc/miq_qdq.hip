@@ -561,6 +561,45 @@ __global__ __launch_bounds__(kBlock) void qdq_broadcast_kernel(const float* in, 
         out[e]        = p.delta * (q + p.offset);
     }
 }
+// True when the broadcast is "encoding (e / run) % channels for element e" of a dense row-major tensor; see the caller.
+static bool broadcast_as_channels(const BcastArgs& b, int64_t n, int64_t& channels, int64_t& run)
+{
+    int64_t size[8];
+    for (int d = 0; d < b.ndims; ++d)
+    {
+        const int64_t outer = d == 0 ? n : b.istride[d - 1];
+        if (outer % b.istride[d] != 0)
+            return false;
+        size[d] = outer / b.istride[d];
+    }
+    if (b.istride[b.ndims - 1] != 1)
+        return false;   // not densely laid out
+    int first = -1, last = -1;
+    for (int d = 0; d < b.ndims; ++d)
+        if (b.estride[d] != 0 && size[d] != 1)
+        {
+            if (first < 0)
+                first = d;
+            last = d;
+        }
+    if (first < 0)
+    {
+        channels = 1;
+        run      = n;
+        return true;
+    }
+    int64_t expect = 1;
+    for (int d = last; d >= first; --d)
+    {
+        if (size[d] != 1 && b.estride[d] != expect)
+            return false;   // a broadcast axis inside the run, or an encoding that is not dense over it
+        expect *= size[d];
+    }
+    channels = expect;
+    run      = b.istride[last];
+    return true;
+}
+
 static ParamSrc v1_channel_src(const float* mn, const float* mx, const float* d, const float* o)
 {
     ParamSrc s{};
@@ -760,6 +799,19 @@ int miq_qdq_broadcast_f32(const float* in, float* out, int64_t num_element, int6
         MIQ_CHECK_ARG(input_strides[d] > 0, "input strides must be positive");
         b.istride[d] = input_strides[d];
         b.estride[d] = encoding_strides[d];
+    }
+    // The usual broadcasts -- one encoding for the tensor, or encodings that vary along one run of adjacent axes of a
+    // densely laid out tensor, themselves densely laid out (per channel on any axis, blocks that cut the last varying
+    // axis) -- are the [outer, channel, run] layout of the vector kernel: element e uses encoding (e / run) % channels.
+    int64_t channels = 0, run = 0;
+    if (broadcast_as_channels(b, num_element, channels, run))
+    {
+        EwPtrs<float, uint8_t> p{in, nullptr, out, nullptr};
+        if (channels == 1)
+            return launch_ew<float, OpV1Qdq, true>(p, v1_channel_src(enc_min, enc_max, enc_delta, enc_offset), num_element, 1,
+                                                   num_element, (hipStream_t) stream);
+        return launch_ew<float, OpV1Qdq, true>(p, v1_channel_src(enc_min, enc_max, enc_delta, enc_offset), num_element,
+                                               channels, run, (hipStream_t) stream);
     }
     int64_t blocks = (num_element + kBlock - 1) / kBlock;
     if (blocks > 65536)

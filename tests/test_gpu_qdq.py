@@ -248,6 +248,37 @@ def test_broadcast(ops, oracle):
         assert np.array_equal(_bits(y), _bits(oracle.qdq_broadcast(x, strides, est, params)))
 
 
+@pytest.mark.parametrize("shape,enc_shape", [
+    ((6, 64, 7, 9), (1, 64, 1, 1)),        # per channel on axis 1 with an outer axis: (e / run) % channels
+    ((96, 33, 3, 3), (96, 1, 1, 1)),       # per output channel
+    ((48, 4, 128), (48, 4, 1)),            # blocks of 128 along the last axis of a [48, 512] tensor
+    ((5, 12, 10, 6), (1, 12, 10, 1)),      # two adjacent varying axes
+    ((4, 6, 10, 8), (4, 1, 10, 1)),        # varying axes that are not adjacent: the general kernel
+    ((7, 1, 5, 3), (1, 1, 5, 3)),          # the encoding covers the trailing axes
+    ((1000,), (1,)),
+])
+def test_broadcast_layouts(ops, oracle, shape, enc_shape):
+    """Broadcast layouts that the library maps onto its [outer, channel, run] vector kernel, and one that it cannot:
+    the result is the restatement's, bit for bit, either way (reference DlQuantization/src/trim_functions.cpp:634-660)."""
+    rng = np.random.default_rng(len(shape) * 100 + shape[0])
+    x = (rng.standard_normal(int(np.prod(shape))) * 1.5).astype(np.float32)
+    strides, acc = [], 1
+    for d in reversed(shape):
+        strides.append(acc)
+        acc *= d
+    strides = strides[::-1]
+    est, acc = [], 1
+    for d in reversed(enc_shape):
+        est.append(acc if d > 1 else 0)
+        acc *= d
+    est = est[::-1]
+    n_enc = int(np.prod(enc_shape))
+    params = oracle.per_channel_params(-np.abs(rng.standard_normal(n_enc)) - 0.1, np.abs(rng.standard_normal(n_enc)) + 0.1,
+                                       8)
+    y = ops.qdq_broadcast(_gpu(x), strides, est, *[_gpu(p) for p in params]).cpu().numpy()
+    assert np.array_equal(_bits(y), _bits(oracle.qdq_broadcast(x, strides, est, params)))
+
+
 # ------------------------------------------------------------------------------------------------------------ v2
 @pytest.mark.parametrize("qmin,qmax", [(0, 255), (-128, 127), (-8, 7), (0, 15)])
 @pytest.mark.parametrize("c,npc,outer", [(1, 100003, 1), (512, 4608, 1), (64, 1030, 1), (7, 5, 3)])
