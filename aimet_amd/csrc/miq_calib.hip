@@ -734,28 +734,28 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
     }
 }
 
-// Folds whichever batch is still pending (at most one).  Queued before anything reads the PDF.  One workgroup of
-// 1024 lanes: four slices per round, the loads of all sixteen rounds independent of each other.
-constexpr int kFlushBlock = 1024;
-__global__ __launch_bounds__(kFlushBlock) void hist_flush_kernel(DevState* st, uint32_t seq)
+// Folds whichever batch is still pending (at most one).  Queued before anything reads the PDF.  kFoldSlices workgroups,
+// a slice each, as in hist_kernel (one workgroup doing all of it took 28 us: its write-through stores go out one after
+// the other).  Every workgroup reads the iteration count before it draws its ticket, so the workgroup that draws the
+// last one may overwrite it.  (The ticket counter is the search kernel's: the two never run at the same time.)
+__global__ __launch_bounds__(kBlock) void hist_flush_kernel(DevState* st, uint32_t seq)
 {
     const int buf = (int) (seq & 1u);
     if (st->batch_seq[buf] == 0 || st->batch_seq[buf] != seq)
         return;
-    const int64_t batch_n  = st->batch_n[buf];
-    constexpr int kPerRound = kFlushBlock / kBlock, kRounds = kFoldSlices / kPerRound;
-    FoldLoad f[kRounds];
-#pragma unroll
-    for (int round = 0; round < kRounds; ++round)
-        f[round] = fold_load(st, buf, buf, round * kPerRound + threadIdx.x / kBlock, threadIdx.x % kBlock);
-#pragma unroll
-    for (int round = 0; round < kRounds; ++round)
-        fold_store(st, buf, batch_n, round * kPerRound + threadIdx.x / kBlock, threadIdx.x % kBlock, f[round]);
-    __syncthreads();   // every leader has read iters[buf]
+    const int64_t batch_n = st->batch_n[buf];
+    const FoldLoad f      = fold_load(st, buf, buf, blockIdx.x, threadIdx.x);
+    fold_store(st, buf, batch_n, blockIdx.x, threadIdx.x, f);
+    __shared__ int it_seen;
     if (threadIdx.x == 0)
+        it_seen = f.it;   // lane 0 leads a bucket: it has read the count
+    __syncthreads();      // every leader of this workgroup has read iters[buf] and batch_seq[buf]
+    if (threadIdx.x == 0 &&
+        __hip_atomic_fetch_add(&st->ticket_search, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1)
     {
-        st->iters[buf]     = f[0].it + 1;   // what the next update call's launch reads
-        st->iterations     = f[0].it + 1;
+        st->ticket_search  = 0;
+        st->iters[buf]     = it_seen + 1;   // what the next update call's launch reads
+        st->iterations     = it_seen + 1;
         st->batch_seq[buf] = 0;
     }
 }
@@ -1333,7 +1333,7 @@ static int flush_pending(miq_analyzer* a, hipStream_t s)
 {
     if (a->mode != MIQ_QUANTIZATION_TF && a->seq != 0)
     {
-        hipLaunchKernelGGL(hist_flush_kernel, dim3(1), dim3(kFlushBlock), 0, s, a->st, a->seq);
+        hipLaunchKernelGGL(hist_flush_kernel, dim3(kFoldSlices), dim3(kBlock), 0, s, a->st, a->seq);
         MIQ_CHECK_LAUNCH();
         a->counted_n = 0;   // nothing is pending any more: the next launch must not fold on the host's word
     }

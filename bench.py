@@ -399,11 +399,12 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
     rows = x.size(0)
     full = [torch.arange(rows) for _ in range(12)]
     alpha0 = wrapper.alpha.data.clone()
-    AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, x, y, params, batches=full[:2])
+    full_params = AdaroundHyperParameters(max(iterations, len(full)), 0.01, (20, 2), 0.2)
+    AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, x, y, full_params, batches=full[:2])
     wrapper.alpha.data.copy_(alpha0)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, x, y, params, batches=full[2:])
+    AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, x, y, full_params, batches=full[2:])
     torch.cuda.synchronize()
     it_ms = (time.perf_counter() - t0) * 1e3 / 10
     wrapper.alpha.data.copy_(alpha0)
