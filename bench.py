@@ -317,6 +317,43 @@ def _adaround_layer(torch, seed=1005, out_features=4096, in_features=4096, rows=
     return AdaroundWrapper(qw), x, y
 
 
+def bench_launch_floors(torch, ops, launches=200):
+    """What launches of the benchmark's tensor sizes cost on this GPU whatever the kernel computes: back-to-back launches
+    of the simplest kernels of the same traffic (torch's elementwise add with a scalar for 1-read-1-write, with a tensor
+    for 2-read-1-write), rotated over several buffer sets, one event pair around the region.  The fractions
+    of HBM peak that the per-tensor cell and the calibration loop are held against come from here."""
+    dev = torch.device("cuda", 0)
+    out = {}
+    for name, n in (("32x64x56x56", 32 * 64 * 56 * 56), ("11008x4096", 11008 * 4096)):
+        sets = 16 if n < (1 << 24) else 3
+        a = [torch.randn(n, device=dev) for _ in range(sets)]
+        b = [torch.randn(n, device=dev) for _ in range(sets)]
+        c = [torch.empty(n, device=dev) for _ in range(sets)]
+        kinds = {
+            "one_read_one_write": (8, lambda i: torch.add(a[i % sets], 1.0, out=c[i % sets])),
+            "two_reads_one_write": (12, lambda i: torch.add(a[i % sets], b[i % sets], out=c[i % sets])),
+        }
+        row = {}
+        for kind, (bytes_per_elem, fn) in kinds.items():
+            for i in range(5):
+                fn(i)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for i in range(launches):
+                fn(i)
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / launches * 1e3
+            row[kind] = {"us_per_launch": us, "GBps": bytes_per_elem * n / us / 1e3,
+                         "frac_hbm": bytes_per_elem * n / us / 1e3 / HBM_PEAK_GBPS}
+        row["fwd_plus_bwd_floor_us"] = row["one_read_one_write"]["us_per_launch"] + row["two_reads_one_write"]["us_per_launch"]
+        row["fwd_plus_bwd_floor_frac_hbm"] = 20 * n / row["fwd_plus_bwd_floor_us"] / 1e3 / HBM_PEAK_GBPS
+        out[name] = row
+        del a, b, c
+    return out
+
+
 def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
     """AdaRound inner loop of one Linear [4096,4096] layer (cfg5): whole loop wall-clock through AdaroundOptimizer, then
     the three kernels of one iteration timed with events."""
@@ -960,7 +997,7 @@ def main():
     ap.add_argument("--full", action="store_true", help="(kept for old command lines: every cell is measured anyway)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run a subset of the legs, comma separated (main|pt|fp8|calib|chcalib|sqnr|learn|quantsim|adaround|copyref), for profiling")
+                    help="run a subset of the legs, comma separated (main|pt|fp8|calib|chcalib|sqnr|learn|quantsim|adaround|floors|copyref), for profiling")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
@@ -991,6 +1028,8 @@ def main():
             torch.add(a, 1.0, out=b)
         torch.cuda.synchronize()
         extra["copyref"] = {"elements": a.numel(), "bytes_read": 4 * a.numel(), "bytes_written": 4 * a.numel()}
+    if want("floors"):
+        extra["launch_floors"] = bench_launch_floors(torch, ops)
     if want("main"):
         res = bench_per_channel(torch, ops, main_shape, torch.float32, 8, args.steps, args.warmup, 1004)
     if want("pt"):
