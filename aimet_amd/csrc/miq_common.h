@@ -108,5 +108,14 @@ __device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi)
     return w;
 }
 
+// the same conversion for values known not to be NaN (nothing to canonicalise)
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_no_nan(float lo, float hi)
+{
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    const f2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2));
+}
+
 }   // namespace miq
 #endif

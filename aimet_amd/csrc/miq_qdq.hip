@@ -210,6 +210,26 @@ struct OpV2Bwd : OpV2
     }
 };
 
+// Whether a vector's results are known not to be NaN from its parameters alone.  The v1 forward clamps its input with
+// fminf / fmaxf (a NaN input comes out as a bound) and then only rounds, adds the offset and multiplies by delta: with
+// finite min, max, delta (what a non-zero rcp says) and offset every result is finite.
+template <typename OP>
+struct NoNanOut
+{
+    __device__ static bool get(const typename OP::P&)
+    {
+        return false;
+    }
+};
+template <>
+struct NoNanOut<OpV1Qdq>
+{
+    __device__ static bool get(const V1P& p)
+    {
+        return p.rcp != 0.0f && fabsf(p.offset) < INFINITY;
+    }
+};
+
 template <typename OP>
 __device__ typename OP::P scalar_params(const ParamSrc& s);
 template <>
@@ -303,8 +323,9 @@ __device__ __forceinline__ void store_codes<int32_t, 8>(int32_t* dst, const int*
     store_codes<int32_t, 4>(dst + 4, c + 4);
 }
 
-// Vectorised tile kernel.  Requires 16-byte aligned pointers; n < 2^31 when PER_CHANNEL.
-template <typename IO, typename OP, bool PER_CHANNEL, int kUnroll>
+// Vectorised tile kernel.  Requires 16-byte aligned pointers; n < 2^31 when PER_CHANNEL.  CODES: the integer codes are
+// stored too (ptr.codes is not null); without it their arithmetic (two operations per element) is not compiled in.
+template <typename IO, typename OP, bool PER_CHANNEL, int kUnroll, bool CODES>
 __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::Code> ptr, ParamSrc src, int64_t n,
                                                         uint32_t num_channel, FastDiv fd)
 {
@@ -375,9 +396,11 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
         T::unpack(vx[u], fx);
         if constexpr (OP::NIN == 2)
             T::unpack(vg[u], fg);
+        bool no_nan = false;
         if (one_row)
         {
             apply_n<OP, VEC, OP::NIN == 2>(src, pt, fx, fg, fy, code);
+            no_nan = NoNanOut<OP>::get(pt);
         }
         else
         {
@@ -388,6 +411,7 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
             {
                 const P p = win[lr];
                 apply_n<OP, VEC, OP::NIN == 2>(src, p, fx, fg, fy, code);
+                no_nan = NoNanOut<OP>::get(p);
             }
             else
             {
@@ -401,8 +425,8 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
             }
         }
         if (ptr.y)
-            stream_store(reinterpret_cast<Vec*>(ptr.y) + v, T::pack(fy));
-        if (ptr.codes)
+            stream_store(reinterpret_cast<Vec*>(ptr.y) + v, no_nan ? T::pack_no_nan(fy) : T::pack(fy));
+        if constexpr (CODES)
             store_codes<typename OP::Code, VEC>(ptr.codes + v * VEC, code);
     }
     // the n % VEC trailing elements
@@ -470,8 +494,12 @@ int launch_ew(EwPtrs<IO, typename OP::Code> ptr, const ParamSrc& src, int64_t n,
     {
         const int64_t blocks = (n + TILE - 1) / TILE;
         FastDiv fd           = make_fastdiv(PER_CHANNEL ? (uint32_t) n_per_channel : 1u);
-        hipLaunchKernelGGL((ew_vec_kernel<IO, OP, PER_CHANNEL, U>), dim3((unsigned) blocks), dim3(kBlock), 0, stream, ptr,
-                           src, n, (uint32_t) num_channel, fd);
+        if (ptr.codes)
+            hipLaunchKernelGGL((ew_vec_kernel<IO, OP, PER_CHANNEL, U, true>), dim3((unsigned) blocks), dim3(kBlock), 0,
+                               stream, ptr, src, n, (uint32_t) num_channel, fd);
+        else
+            hipLaunchKernelGGL((ew_vec_kernel<IO, OP, PER_CHANNEL, U, false>), dim3((unsigned) blocks), dim3(kBlock), 0,
+                               stream, ptr, src, n, (uint32_t) num_channel, fd);
     }
     else
     {
