@@ -614,6 +614,30 @@ __global__ __launch_bounds__(kHistBlock) void settle_kernel(const float* __restr
     __shared__ float s_mm[2][kHistBlock / 64];
     __shared__ int s_last;
     const int h = blockIdx.y;
+    float* sh             = state_hist + (int64_t) h * num_bins;
+    const int slot_stride = 2 * num_bins;
+    uint32_t* rep         = counts + (int64_t) h * replicas * slot_stride;
+    // The workgroups that would add the first launch's counts request their first bins' counts and running values
+    // now, before it is known that they will be used: they arrive together with the partials.
+    const int settlers = min((int) gridDim.x, kSettlers);
+    const bool settler = (int) blockIdx.x < settlers;
+    const int slice    = (num_bins + settlers - 1) / settlers;
+    const int first = blockIdx.x * slice, last = min(num_bins, first + slice);
+    constexpr int kEarly = 2;
+    uint32_t early[kEarly][kSpecReplicas];
+    float before[kEarly];
+    if (settler)
+    {
+#pragma unroll
+        for (int j = 0; j < kEarly; ++j)
+        {
+            const int i = first + j * kHistBlock + threadIdx.x;
+#pragma unroll
+            for (int k = 0; k < kSpecReplicas; ++k)
+                early[j][k] = (i < last && k < replicas) ? rep[(int64_t) k * slot_stride + i] : 0u;
+            before[j] = i < last ? sh[i] : 0.f;
+        }
+    }
     float lo = INFINITY, hi = -INFINITY;
     {
         const float* p = mm_partial + (int64_t) h * num_partials * 2;
@@ -654,9 +678,6 @@ __global__ __launch_bounds__(kHistBlock) void settle_kernel(const float* __restr
     }
     bool ok;
     const Ranges r = compute_ranges(lo, hi, num_bins, 1, state_minmax, h, ok);
-    float* sh              = state_hist + (int64_t) h * num_bins;
-    const int slot_stride  = 2 * num_bins;
-    uint32_t* rep          = counts + (int64_t) h * replicas * slot_stride;
     auto publish = [&]() {
         ranges[h] = r;
         if (batch_minmax)
@@ -669,20 +690,34 @@ __global__ __launch_bounds__(kHistBlock) void settle_kernel(const float* __restr
     };
     if (!r.rebin)
     {
-        const int settlers = min((int) gridDim.x, kSettlers);
-        if ((int) blockIdx.x >= settlers)
+        if (!settler)
             return;
-        const int slice = (num_bins + settlers - 1) / settlers;
-        const int first = blockIdx.x * slice, last = min(num_bins, first + slice);
-        for (int i = first + threadIdx.x; i < last; i += kHistBlock)
+#pragma unroll
+        for (int j = 0; j < kEarly; ++j)
+        {
+            const int i = first + j * kHistBlock + threadIdx.x;
+            if (i < last)
+            {
+                uint32_t total = 0;
+#pragma unroll
+                for (int k = 0; k < kSpecReplicas; ++k)
+                {
+                    total += early[j][k];
+                    if (k < replicas)
+                        rep[(int64_t) k * slot_stride + i] = 0u;
+                }
+                sh[i] = (float) total + before[j];
+            }
+        }
+        for (int i = first + kEarly * kHistBlock + threadIdx.x; i < last; i += kHistBlock)
         {
             // all loads of a bin are issued before the first addition: one round trip per bin, not one per replica
             uint32_t t[kSpecReplicas];
 #pragma unroll
             for (int k = 0; k < kSpecReplicas; ++k)
                 t[k] = k < replicas ? rep[(int64_t) k * slot_stride + i] : 0u;
-            const float before = sh[i];
-            uint32_t total     = 0;
+            const float was = sh[i];
+            uint32_t total  = 0;
 #pragma unroll
             for (int k = 0; k < kSpecReplicas; ++k)
             {
@@ -690,7 +725,7 @@ __global__ __launch_bounds__(kHistBlock) void settle_kernel(const float* __restr
                 if (k < replicas)
                     rep[(int64_t) k * slot_stride + i] = 0u;
             }
-            sh[i] = (float) total + before;
+            sh[i] = (float) total + was;
         }
         if (blockIdx.x == 0 && threadIdx.x == 0)
             publish();   // (state_minmax keeps its values)
@@ -1102,6 +1137,7 @@ int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hi
                                lds_bytes, s, data, n_per_hist, num_bins, 4, state_minmax, mm_part, counts, spec_replicas,
                                vec);
         MIQ_CHECK_LAUNCH();
+        // (a smaller grid for this launch -- all but eight workgroups per histogram leave at once -- measured the same)
         hipLaunchKernelGGL(settle_kernel, dim3(blocks, (unsigned) num_hist), dim3(kHistBlock), lds_bytes, s, data,
                            n_per_hist, num_bins, 4, mm_part, sblocks, state_hist, state_minmax, ranges, batch_minmax,
                            bad_flag, counts, spec_replicas, tickets, vec);
