@@ -115,8 +115,9 @@ MIQ_HD inline int bucket_row(float x, const BucketMap& m)
 // with K = max(|lo|, |hi|) / width, u lies within bins (K + 2) 2^-24 of the real number (x - lo) bins / width (one
 // rounding each in the scale, the shift and the result), and the three roundings of the sequence keep it within
 // 3 bins 2^-24 of the same number, so the truncated sequence and floor(u) agree whenever the fraction of u stays
-// eps = bins (K + 1) 2^-21 (more than 1.6 times the sum of the bounds) away from 0 and 1; u below 0 or from bins on is
-// what the observer's rule for outside values maps to the end bins.  Samples
+// eps = 2 bins (K + 5) 2^-24 (twice the sum of the bounds; in the host check mismatches first appear at three eighths
+// of it) away from 0 and 1; u below 0 or from bins on is what the observer's rule for outside values
+// maps to the end bins.  A wavefront takes the sequence as soon as one of its lanes does, so eps is kept small.  Samples
 // within eps of a bin edge, infinities, NaN (bin -1) and ranges for which eps reaches 1/4 take the sequence.
 // tests/test_fastmath.py checks bin() against the plain sequence on ranges over many decades, the floats around every
 // bin edge and random samples.
@@ -139,7 +140,7 @@ struct HistcBinner
         fast_scale = nbf / width;
         fast_shift = -lo_ * fast_scale;
         const float k   = __builtin_fmaxf(__builtin_fabsf(lo_), __builtin_fabsf(hi_)) / width;
-        const float eps = nbf * (k + 1.0f) * 4.76837158203125e-07f;   // 2^-21
+        const float eps = nbf * (k + 5.0f) * 1.1920928955078125e-07f;   // 2^-23
         // (comparisons are false for NaN: a range that is not finite never takes the short path)
         thr = (divisor_ok && eps < 0.25f && __builtin_fabsf(fast_shift) < 1e30f && fast_scale < 1e30f) ? 0.5f - eps
                                                                                                      : -1.0f;
