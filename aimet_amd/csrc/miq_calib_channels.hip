@@ -222,19 +222,24 @@ __global__ __launch_bounds__(256) void chan_count_batch_kernel(ChanState s, int6
         s.head[i].iterations += 1;
 }
 
-// One workgroup per channel: its four wavefronts walk the candidate grid (one candidate per wavefront at a time,
-// miq_tfe_search.h), each keeping the first strict minimum it has seen; the lowest-numbered candidate among equal
-// costs wins, as in the reference's single loop.
-__global__ __launch_bounds__(256) void chan_search_kernel(ChanState s, tfe::SearchArgs a)
+// One workgroup per channel, one candidate of the grid per lane (tfe::lane_cost): every wavefront walks the channel's
+// PDF once for its 64 candidates.  The lowest-numbered candidate among equal costs wins, as in the reference's single
+// loop with its strict comparison.  Launched with 64 * ceil(n_cand / 64) threads (kSearchBlockMax at most; candidates
+// beyond that take further walks).
+constexpr int kSearchBlockMax = 512;
+__global__ __launch_bounds__(kSearchBlockMax) void chan_search_kernel(ChanState s, tfe::SearchArgs a)
 {
-    constexpr int kWaves = 4;
-    const int64_t c      = blockIdx.x;
+    constexpr int kWavesMax = kSearchBlockMax / 64;
+    const int64_t c         = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    __shared__ double term_all[kWaves][kPdf];
-    __shared__ double best_cost[kWaves];
-    __shared__ int best_index[kWaves];
-    __shared__ float best_delta[kWaves];
-    __shared__ int best_offset[kWaves];
+    const int waves = (int) blockDim.x >> 6;
+    __shared__ double pdf_s[kPdf];
+    __shared__ double mid_s[kPdf];
+    __shared__ float fmid_s[kPdf];
+    __shared__ double best_cost[kWavesMax];
+    __shared__ int best_index[kWavesMax];
+    __shared__ float best_delta[kWavesMax];
+    __shared__ int best_offset[kWavesMax];
     ChanHead& h = s.head[c];
     if (!h.initialized)
     {
@@ -249,22 +254,37 @@ __global__ __launch_bounds__(256) void chan_search_kernel(ChanState s, tfe::Sear
         return;
     }
     const tfe::PdfView view{s.pdf + c * kPdf, h.min_val, h.bucket};
+    tfe::stage_pdf(view, pdf_s, mid_s, fmid_s, threadIdx.x, blockDim.x);
     float minVal, maxVal;
     tfe::wave_range(view, lane, minVal, maxVal);
+    __syncthreads();
     double best = DBL_MAX;
     int bidx    = 0x7fffffff;
     float bdelta = -1;
     int boffset  = -1;
-    for (int cand = wave; cand < a.n_cand; cand += kWaves)
+    for (int first = 0; first < a.n_cand; first += blockDim.x)
     {
-        float delta;
-        int offset;
-        if (!tfe::candidate(a, minVal, maxVal, cand, delta, offset))
-            continue;
-        const double cost = tfe::wave_cost(view, a, delta, offset, lane, term_all[wave]);
-        if (cost < best)
+        const int cand = first + threadIdx.x;
+        float delta    = 1.f;
+        int offset     = 0;
+        const bool active = cand < a.n_cand && tfe::candidate(a, minVal, maxVal, cand, delta, offset);
+        const double cost = tfe::lane_cost(view, pdf_s, mid_s, fmid_s, a, active, delta, offset);
+        if (active && cost < best)
         {
             best = cost, bidx = cand, bdelta = delta, boffset = offset;
+        }
+    }
+    // lowest (cost, candidate number) of the wavefront, then of the workgroup
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1)
+    {
+        const double oc = __shfl_xor(best, m);
+        const int oi    = __shfl_xor(bidx, m);
+        const float od  = __shfl_xor(bdelta, m);
+        const int oo    = __shfl_xor(boffset, m);
+        if (oc < best || (oc == best && oi < bidx))
+        {
+            best = oc, bidx = oi, bdelta = od, boffset = oo;
         }
     }
     if (lane == 0)
@@ -277,7 +297,7 @@ __global__ __launch_bounds__(256) void chan_search_kernel(ChanState s, tfe::Sear
     __syncthreads();
     if (threadIdx.x == 0)
     {
-        for (int w = 1; w < kWaves; ++w)
+        for (int w = 1; w < waves; ++w)
             if (best_cost[w] < best || (best_cost[w] == best && best_index[w] < bidx))
             {
                 best = best_cost[w], bidx = best_index[w], bdelta = best_delta[w], boffset = best_offset[w];
@@ -473,7 +493,8 @@ int miq_channel_analyzer_compute_encodings(miq_channel_analyzer* a, int bw, int 
     }
     const tfe::SearchArgs sa =
         tfe::make_search_args(bw, use_symmetric, use_strict_symmetric, use_unsigned_symmetric);
-    hipLaunchKernelGGL(chan_search_kernel, dim3((unsigned) c), dim3(256), 0, s, a->st, sa);
+    const int search_block = std::min(kSearchBlockMax, 64 * ((sa.n_cand + 63) / 64));
+    hipLaunchKernelGGL(chan_search_kernel, dim3((unsigned) c), dim3(search_block), 0, s, a->st, sa);
     MIQ_CHECK_LAUNCH();
     MIQ_CHECK_HIP(hipMemcpyAsync(heads.data(), a->st.head, sizeof(ChanHead) * c, hipMemcpyDeviceToHost, s));
     MIQ_CHECK_HIP(hipStreamSynchronize(s));

@@ -13,6 +13,7 @@
 #include <cmath>
 
 #include "../../include/miq.h"
+#include "miq_fastmath.h"
 
 namespace miq
 {
@@ -278,6 +279,125 @@ __device__ __forceinline__ double wave_cost(const PdfView& v, const SearchArgs& 
     __builtin_amdgcn_wave_barrier();   // the next candidate of this wavefront overwrites `term`
     double cost = 3.0 * (satBottom + satTop) + quant;
     return (cost < DBL_MAX) ? cost : DBL_MAX;   // std::min(sqnr, max())
+}
+
+// The same cost with one candidate per LANE: a lane walks the buckets in ascending order and keeps the three running
+// sums itself, so a wavefront prices 64 candidates at once and nothing is exchanged between lanes.  Each sum receives
+// the terms wave_cost() adds, in the same order, so the two functions agree bit for bit (wave_cost()'s overlap case
+// included: a bucket below minInd and at or above maxInd enters both saturation sums, none enters the noise sum).
+// The three sums are three loops, each over the buckets that at least one lane of the wavefront needs (the bounds are
+// reduced over the wavefront, so they are uniform), with the lanes outside their own range masked off.
+// pdf_s / mid_s / fmid_s: the PDF, the bucket mid-points and their binary32 values (stage_pdf()), read as LDS
+// broadcasts.  Every lane of the wavefront must call lane_cost(); lanes without a candidate pass active = false.
+//
+// Three steps of the noise term have cheaper sequences with the same result: the division through
+// div_by_invariant() where its contract holds (a quotient below its 2^-36 limit vanishes in the subtraction of the
+// integer offset, or rounds to zero without one), roundf through round_half_away(), and the x86 conversion of the
+// rounded value straight from binary32 (it is an integer, an infinity or NaN there, so the detour through double
+// changes nothing; where |mid / delta| + |offset| stays below 2^30 for every bucket the range test is dropped too).
+// A wavefront uses them when all its lanes can.
+__device__ __forceinline__ void stage_pdf(const PdfView& v, double* pdf_s, double* mid_s, float* fmid_s, int tid,
+                                          int nthreads)
+{
+    const float pdfStart = (float) v.x_left(0);
+    const double pdfStep = v.x_left(1) - v.x_left(0);
+    for (int i = tid; i < kBuckets; i += nthreads)
+    {
+        const double mid = pdfStart + i * pdfStep + pdfStep / 2;
+        pdf_s[i]         = v.pdf[i];
+        mid_s[i]         = mid;
+        fmid_s[i]        = (float) mid;
+    }
+}
+__device__ __forceinline__ int cvtt_x86_of_rounded(float r)
+{
+    return (r >= -2147483648.0f && r < 2147483648.0f) ? (int) r : INT_MIN;
+}
+__device__ __forceinline__ int wave_min_int(int v)
+{
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1)
+    {
+        const int o = __shfl_xor(v, m);
+        v           = o < v ? o : v;
+    }
+    return __builtin_amdgcn_readfirstlane(v);
+}
+// Sum of p * d^2 over the buckets [from, to) of this lane, d = mid - ref, inside the wavefront's loop [begin, end).
+__device__ __forceinline__ double saturation_sum(const double* pdf_s, const double* mid_s, int begin, int end, int from,
+                                                 int to, float ref)
+{
+    double acc = 0;
+#pragma unroll 4
+    for (int i = begin; i < end; ++i)
+        if (i >= from && i < to)
+        {
+            const double d = mid_s[i] - ref;
+            acc += pdf_s[i] * (d * d);
+        }
+    return acc;
+}
+template <bool SHORT>
+__device__ __forceinline__ double noise_sum(const double* pdf_s, const float* fmid_s, int begin, int end, int from,
+                                            int to, float delta, float rcp, int offset)
+{
+    const float foffset = (float) offset;
+    double acc          = 0;
+#pragma unroll 4
+    for (int i = begin; i < end; ++i)
+        if (i >= from && i < to)
+        {
+            const float fv = fmid_s[i];
+            int q;
+            if (SHORT)
+                q = (int) round_half_away(div_by_invariant(fv, delta, rcp) - foffset);
+            else
+                q = cvtt_x86_of_rounded(round_half_away(fv / delta - foffset));
+            const float dq = delta * (float) (q + offset);
+            const double d = (double) (fv - dq);
+            acc += pdf_s[i] * (d * d);
+        }
+    return acc;
+}
+__device__ __forceinline__ double lane_cost(const PdfView& v, const double* pdf_s, const double* mid_s,
+                                            const float* fmid_s, const SearchArgs& a, bool active, float delta,
+                                            int offset)
+{
+    const float foffset   = (float) offset;
+    const float cMin      = delta * foffset;
+    const float stepSize  = a.step_size_cost;
+    const float cMax      = delta * (foffset + stepSize);
+    const float pdfStart  = (float) v.x_left(0);
+    const double pdfStep  = v.x_left(1) - v.x_left(0);
+    int minInd            = cvtt_x86(floor((cMin - pdfStart) / pdfStep));
+    minInd                = minInd < 0 ? 0 : (minInd > kBuckets - 1 ? kBuckets - 1 : minInd);
+    int maxInd            = cvtt_x86(floor((cMax - pdfStart) / pdfStep));
+    maxInd                = maxInd < 0 ? 0 : (maxInd > kBuckets - 1 ? kBuckets - 1 : maxInd);
+    const float minMid    = (float) (pdfStart + (minInd * pdfStep) + pdfStep / 2);
+    const float maxMid    = (float) (pdfStart + (maxInd * pdfStep) + pdfStep / 2);
+    // this lane's three ranges (empty without a candidate) and the wavefront's
+    const int bottom_to  = active ? minInd : 0;
+    const int top_from   = active ? maxInd : kBuckets;
+    const int noise_from = active ? minInd : kBuckets;
+    const int noise_to   = active ? maxInd : 0;
+    const int w_bottom_to  = -wave_min_int(-bottom_to);
+    const int w_top_from   = wave_min_int(top_from);
+    const int w_noise_from = wave_min_int(noise_from);
+    const int w_noise_to   = -wave_min_int(-noise_to);
+    // the mid-points grow with the bucket number: the end ones bound the dividends
+    const float far      = fmaxf(fabsf(fmid_s[0]), fabsf(fmid_s[kBuckets - 1]));
+    const bool can_short = fastdiv_divisor_ok(delta) && far <= kFastDivMaxDividend &&
+                           far / delta + fabsf(foffset) < 1073741824.0f;
+    const bool all_short = wave_min_int((can_short || !active) ? 1 : 0) != 0;
+    const float rcp      = 1.0f / delta;
+
+    const double satBottom = saturation_sum(pdf_s, mid_s, 0, w_bottom_to, 0, bottom_to, minMid);
+    const double satTop    = saturation_sum(pdf_s, mid_s, w_top_from, kBuckets, top_from, kBuckets, maxMid);
+    const double quant =
+        all_short ? noise_sum<true>(pdf_s, fmid_s, w_noise_from, w_noise_to, noise_from, noise_to, delta, rcp, offset)
+                  : noise_sum<false>(pdf_s, fmid_s, w_noise_from, w_noise_to, noise_from, noise_to, delta, rcp, offset);
+    double cost = 3.0 * (satBottom + satTop) + quant;
+    return (cost < DBL_MAX) ? cost : DBL_MAX;
 }
 
 // {min, max, delta, offset} of the winning candidate, DLQ/src/TfEnhancedEncodingAnalyzer.cpp:383-396

@@ -746,7 +746,7 @@ class ChannelAnalyzer(_StateOwner):
                                                             self._s()))
 
     def compute_encodings(self, bw, symmetric=False, strict_symmetric=False, unsigned_symmetric=False):
-        """returns (list of Encoding, one per channel; is_valid)"""
+        """returns (ctypes array of Encoding, one per channel: indexable and iterable; is_valid)"""
         encs = (Encoding * self.num_channel)()
         valid = C.c_int(0)
         with torch.cuda.device(self.device):
@@ -754,7 +754,7 @@ class ChannelAnalyzer(_StateOwner):
                                                              int(bool(strict_symmetric)),
                                                              int(bool(unsigned_symmetric)), encs, C.byref(valid),
                                                              self._s()))
-        return list(encs), bool(valid.value)
+        return encs, bool(valid.value)
 
     def get_stats_histogram(self, channel):
         import numpy as np
