@@ -952,11 +952,18 @@ __global__ __launch_bounds__(256) void sqnr_noise_kernel(const float* __restrict
     {
         float delta, offset;
         candidate(a, mn, mx, c, delta, offset);
-        double acc = 0.0;
+        // mid / delta through div_by_invariant where its contract holds for every bin of this histogram (the end
+        // mid-points bound the dividends; a quotient below its 2^-36 limit vanishes in the subtraction of the integer
+        // offset, or rounds to zero without one); delta is the wavefront's, so the choice is uniform
+        const bool short_div =
+            __builtin_amdgcn_readfirstlane((int) (fastdiv_divisor_ok(delta) &&
+                                                  fmaxf(fabsf(s_mid[0]), fabsf(s_mid[nb - 1])) <= kFastDivMaxDividend)) != 0;
+        const float rcp = 1.0f / delta;
+        double acc      = 0.0;
         for (int i = lane; i < nb; i += 64)
         {
             const float mid = s_mid[i];
-            float q         = rintf(mid / delta - offset);
+            float q         = rintf((short_div ? div_by_invariant(mid, delta, rcp) : mid / delta) - offset);
             const bool clip = q < 0.0f || q > a.num_steps;
             q               = fminf(fmaxf(q, 0.0f), a.num_steps);
             const float d   = (q + offset) * delta - mid;
