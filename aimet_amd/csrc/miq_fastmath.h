@@ -169,7 +169,8 @@ struct HistcBinner
         {
             // |fl| < 2^23 here (larger floats have no fraction: f == 0 fails the test)
             const int k = (int) fl;
-            return k < 0 ? 0 : (k >= nb ? nb - 1 : k);
+            const int below = k < nb - 1 ? k : nb - 1;
+            return below > 0 ? below : 0;
         }
         return bin_by_sequence(x);
     }

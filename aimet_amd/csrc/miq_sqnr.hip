@@ -35,6 +35,7 @@ constexpr int kMaxReplicas = 32;   // global copies of a histogram's counts that
 // (8 K / 16 K / 50 K: +2.5 / +0.8 / +4 us), two 16-byte loads of a lane in flight (4 / 8: +0.8 / +1.1 us).
 constexpr int kSpecReplicas     = 8;
 constexpr int kSpecLoads        = 2;
+constexpr int kSpecCopies       = 4;
 constexpr int64_t kSpecElems    = 32768;
 constexpr int64_t kSpecWideFrom = 65536;
 constexpr float kMinScale = 1.1920928955078125e-07f;   // torch.finfo(torch.float32).eps (EA:322)
@@ -465,6 +466,22 @@ __device__ void rebin_running_histogram(float* __restrict__ upd, const float* __
     __syncthreads();
 }
 
+// min / max of a number and a value that is a number or a quiet NaN: the number when the other is NaN.  One
+// instruction each; fminf / fmaxf first pass both operands through a canonicalising max, which triples the count in
+// a loop that is short on issue slots.
+__device__ __forceinline__ float min_of_number_and_maybe_nan(float number, float other)
+{
+    float r;
+    asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(number), "v"(other));
+    return r;
+}
+__device__ __forceinline__ float max_of_number_and_maybe_nan(float number, float other)
+{
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(number), "v"(other));
+    return r;
+}
+
 // ---- speculative update (running statistics exist, the batch's own histogram is not wanted) -----------------
 // First launch.  grid (blocks, H).  One pass over row h: finite min / max (one partial per workgroup, as
 // finite_minmax_kernel writes them) and, in the same pass, the counts of the row over the range the running statistics
@@ -474,10 +491,12 @@ __device__ void rebin_running_histogram(float* __restrict__ upd, const float* __
 // rows go to few workgroups of 1024 threads.
 template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void spec_bin_kernel(const float* __restrict__ x, int64_t n_per_hist, int num_bins,
-                                                         int copies, const float* __restrict__ state_minmax,
+                                                         const float* __restrict__ state_minmax,
                                                          float* __restrict__ mm_partial, uint32_t* __restrict__ counts,
                                                          int replicas, int vec)
 {
+    constexpr int copies = kSpecCopies;   // LDS copies of the histogram, interleaved (a constant: the bin index is
+                                          // scaled by it per element, and a 32-bit multiply runs at quarter rate)
     extern __shared__ uint32_t lds[];
     __shared__ float s_mm[2][BLOCK / 64];
     constexpr int kInFlight = kSpecLoads;   // 16-byte loads of a lane in flight
@@ -485,8 +504,12 @@ __global__ __launch_bounds__(BLOCK) void spec_bin_kernel(const float* __restrict
     const float* row     = x + (int64_t) h * n_per_hist;
     const v4f* rv        = reinterpret_cast<const v4f*>(row);
     const int64_t nvec   = n_per_hist / 4;
-    const int64_t stride = (int64_t) gridDim.x * BLOCK * kInFlight;
-    int64_t base         = (int64_t) blockIdx.x * BLOCK * kInFlight;
+    // workgroup b counts the 16-byte groups [b * share, (b + 1) * share) of the row: equal shares (a multiple of a
+    // wavefront's 64 loads) whatever the grid, so that a grid of one workgroup per compute unit splits the row evenly
+    const int64_t share  = (((nvec + gridDim.x - 1) / gridDim.x) + 63) & ~(int64_t) 63;
+    const int64_t stride = (int64_t) BLOCK * kInFlight;
+    int64_t base         = (int64_t) blockIdx.x * share;
+    const int64_t end    = base + share < nvec ? base + share : nvec;
     v4f a[kInFlight];
     if (vec)
     {
@@ -494,7 +517,7 @@ __global__ __launch_bounds__(BLOCK) void spec_bin_kernel(const float* __restrict
         for (int u = 0; u < kInFlight; ++u)
         {
             const int64_t i = base + u * BLOCK + threadIdx.x;
-            a[u]            = i < nvec ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
+            a[u]            = i < end ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
         }
     }
     for (int i = threadIdx.x; i < num_bins * copies; i += BLOCK)
@@ -513,28 +536,27 @@ __global__ __launch_bounds__(BLOCK) void spec_bin_kernel(const float* __restrict
     auto take = [&](float v) {
         if (v != v)
             return;
-        if (fabsf(v) < INFINITY)
-        {
-            lo = fminf(lo, v);
-            hi = fmaxf(hi, v);
-        }
+        // infinities enter the minimum and maximum as a quiet NaN, which the hardware's min / max drop
+        const float finite = fabsf(v) < INFINITY ? v : NAN;
+        lo                 = min_of_number_and_maybe_nan(lo, finite);
+        hi                 = max_of_number_and_maybe_nan(hi, finite);
         atomicAdd(&lm[mb.bin(v) * copies], 1u);
     };
     __syncthreads();
     if (vec)
     {
         // the next tile is requested before this one is counted
-        while (base < nvec)
+        while (base < end)
         {
             const int64_t next = base + stride;
             v4f nx[kInFlight];
-            if (next < nvec)
+            if (next < end)
             {
 #pragma unroll
                 for (int u = 0; u < kInFlight; ++u)
                 {
                     const int64_t i = next + u * BLOCK + threadIdx.x;
-                    nx[u]           = i < nvec ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
+                    nx[u]           = i < end ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
                 }
             }
 #pragma unroll
@@ -545,7 +567,7 @@ __global__ __launch_bounds__(BLOCK) void spec_bin_kernel(const float* __restrict
                 take(a[u][2]);
                 take(a[u][3]);
             }
-            if (next >= nvec)
+            if (next >= end)
                 break;
 #pragma unroll
             for (int u = 0; u < kInFlight; ++u)
@@ -1034,13 +1056,29 @@ int hist_blocks(int64_t num_hist, int64_t n_per_hist)
     return (int) (b < 1 ? 1 : b);
 }
 
-// workgroups of 1024 threads per row in a speculative update of long rows: kSpecElems elements each, at most
-// hist_blocks() of them (the workspace is sized for that many partials)
+// workgroups of 1024 threads per row in a speculative update of long rows: about kSpecElems elements each, at most
+// hist_blocks() of them (the workspace is sized for that many partials).  A compute unit runs one such workgroup after
+// the other, so among the counts near that size the one is taken for which the busiest of the 256 compute units has
+// the least to do: rounds * (elements of a workgroup + what clearing and flushing its LDS histogram is worth).
 int spec_blocks(int64_t num_hist, int64_t n_per_hist)
 {
-    const int64_t b   = (n_per_hist + kSpecElems - 1) / kSpecElems;
-    const int64_t cap = hist_blocks(num_hist, n_per_hist);
-    return (int) (b < 1 ? 1 : (b > cap ? cap : b));
+    constexpr int64_t kComputeUnits = 256, kFixedCost = 6144;
+    const int64_t cap  = hist_blocks(num_hist, n_per_hist);
+    const int64_t near = (n_per_hist + kSpecElems - 1) / kSpecElems;
+    int64_t best = 1, best_cost = INT64_MAX;
+    int64_t first = near / 2 > 1 ? near / 2 : 1;
+    first         = first < cap ? first : cap;
+    for (int64_t b = first; b <= 2 * near && b <= cap; ++b)
+    {
+        const int64_t rounds = (b * num_hist + kComputeUnits - 1) / kComputeUnits;
+        const int64_t cost   = rounds * ((n_per_hist + b - 1) / b + kFixedCost);
+        if (cost < best_cost)
+        {
+            best_cost = cost;
+            best      = b;
+        }
+    }
+    return (int) best;
 }
 
 int make_search(SearchArgs& a, int64_t num_hist, int num_bins, double num_steps, int symmetric, double gamma,
@@ -1135,13 +1173,13 @@ int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hi
         const bool wide         = n_per_hist >= kSpecWideFrom;
         const int sblocks       = wide ? spec_blocks(num_hist, n_per_hist) : blocks;
         const int spec_replicas = sblocks < kSpecReplicas ? sblocks : kSpecReplicas;
-        const size_t lds_bytes  = (size_t) num_bins * 4 * sizeof(uint32_t);
+        const size_t lds_bytes  = (size_t) num_bins * kSpecCopies * sizeof(uint32_t);
         if (wide)
             hipLaunchKernelGGL(spec_bin_kernel<1024>, dim3(sblocks, (unsigned) num_hist), dim3(1024), lds_bytes, s, data,
-                               n_per_hist, num_bins, 4, state_minmax, mm_part, counts, spec_replicas, vec);
+                               n_per_hist, num_bins, state_minmax, mm_part, counts, spec_replicas, vec);
         else
             hipLaunchKernelGGL(spec_bin_kernel<kHistBlock>, dim3(sblocks, (unsigned) num_hist), dim3(kHistBlock),
-                               lds_bytes, s, data, n_per_hist, num_bins, 4, state_minmax, mm_part, counts, spec_replicas,
+                               lds_bytes, s, data, n_per_hist, num_bins, state_minmax, mm_part, counts, spec_replicas,
                                vec);
         MIQ_CHECK_LAUNCH();
         // (a smaller grid for this launch -- all but eight workgroups per histogram leave at once -- measured the same)
