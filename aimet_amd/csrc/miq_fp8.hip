@@ -18,6 +18,7 @@
 #include <cstdint>
 
 #include "miq_common.h"
+#include "miq_fastmath.h"
 
 namespace miq
 {
@@ -30,6 +31,72 @@ __device__ __forceinline__ float fp8_elem(float x, float mx, float bias, const f
     int idx  = (int) fminf(e, (float) last);
     float st = steps[idx];
     return rintf(xc / st) * st;
+}
+
+// Rows of `inner4` 16-byte groups, row r belonging to channel r % channels: workgroup b takes piece b % pieces of row
+// b / pieces, so the channel is found once per workgroup (the element-indexed kernel below divides twice in 64 bits
+// per group of four, which made it ALU-bound at 56 % of HBM peak on [11008, 4096]).  The channel's steps go to LDS next
+// to their reciprocals, and the division runs through div_by_invariant() when every step and maxval are inside its
+// contract (a quotient below its 2^-36 limit rounds to zero either way).
+constexpr int kFp8TableMax = 65;   // 2^6 + 1 steps at one mantissa bit
+__global__ void __launch_bounds__(256) fp8_rows_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                        int64_t inner4, int64_t channels, int pieces,
+                                                        const float* __restrict__ maxval,
+                                                        const float* __restrict__ bias,
+                                                        const float* __restrict__ steps, int table)
+{
+    typedef float vec4 __attribute__((ext_vector_type(4)));
+    constexpr int kInFlight = 4;   // loads of a lane in flight before the first is used
+    __shared__ float2 s_step[kFp8TableMax];
+    const int64_t row  = blockIdx.x / (unsigned) pieces;
+    const int piece    = (int) (blockIdx.x - row * pieces);
+    const int64_t c    = row % channels;
+    const vec4* src    = reinterpret_cast<const vec4*>(in) + row * inner4;
+    vec4* dst          = reinterpret_cast<vec4*>(out) + row * inner4;
+    const int64_t step = (int64_t) pieces * 256;
+    int64_t j          = (int64_t) piece * 256 + threadIdx.x;
+    vec4 v[kInFlight];
+    auto request = [&]() {
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u)
+            if (j + u * step < inner4)
+                v[u] = __builtin_nontemporal_load(src + j + u * step);
+    };
+    request();   // the first loads travel while the channel's table is set up
+    const float mx = maxval[c], b = bias[c];
+    bool in_contract = true;
+    if ((int) threadIdx.x < table)
+    {
+        const float st      = steps[c * table + threadIdx.x];
+        s_step[threadIdx.x] = make_float2(st, 1.0f / st);
+        in_contract         = fastdiv_divisor_ok(st);
+    }
+    const bool short_div = __syncthreads_and(in_contract) && mx <= kFastDivMaxDividend;
+    const float last     = (float) (table - 1);
+    auto elem = [&](float x) {
+        const float xc = x != x ? x : fminf(fmaxf(x, -mx), mx);
+        const float e  = fmaxf(floorf(log2f(fabsf(xc)) + b), 1.0f);
+        const float2 s = s_step[(int) fminf(e, last)];
+        const float q  = short_div ? div_by_invariant(xc, s.x, s.y) : xc / s.x;
+        return rintf(q) * s.x;
+    };
+    while (true)
+    {
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u)
+            if (j + u * step < inner4)
+            {
+                v[u][0] = elem(v[u][0]);
+                v[u][1] = elem(v[u][1]);
+                v[u][2] = elem(v[u][2]);
+                v[u][3] = elem(v[u][3]);
+                __builtin_nontemporal_store(v[u], dst + j + u * step);
+            }
+        j += kInFlight * step;
+        if (j >= inner4)
+            break;
+        request();
+    }
 }
 
 // Elements are [outer][channels][inner]; a vector of four never straddles a channel when inner % 4 == 0.
@@ -86,7 +153,21 @@ extern "C" int miq_fp8_fake_cast_f32(const float* in, float* out, int64_t n, int
     const int64_t work   = vec ? n / 4 : n;
     const int64_t blocks = (work + 255) / 256;
     const unsigned grid  = (unsigned) (blocks < 8192 ? blocks : 8192);
-    if (vec)
+    // rows long enough to give every wavefront of a workgroup its own loads go by rows
+    const int64_t row_len = num_channels == 1 ? n : inner;
+    const int64_t rows    = n / row_len;
+    if (vec && row_len >= 1024 && table <= kFp8TableMax)
+    {
+        // four 16-byte groups per lane, and no more pieces than keep the grid near 16K workgroups
+        const int64_t inner4 = row_len / 4;
+        int64_t pieces       = (inner4 + 1023) / 1024;
+        const int64_t most   = rows >= 16384 ? 1 : 16384 / rows;
+        pieces               = pieces < most ? pieces : most;
+        MIQ_CHECK_ARG(rows * pieces < (int64_t) 1 << 31, "too many rows");
+        hipLaunchKernelGGL(fp8_rows_kernel, dim3((unsigned) (rows * pieces)), dim3(256), 0, (hipStream_t) stream, in, out,
+                           inner4, num_channels, (int) pieces, maxval, bias, steps, table);
+    }
+    else if (vec)
         hipLaunchKernelGGL(fp8_kernel<true>, dim3(grid), dim3(256), 0, (hipStream_t) stream, in, out, n, num_channels,
                            inner, maxval, bias, steps, table);
     else
