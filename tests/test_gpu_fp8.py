@@ -113,7 +113,11 @@ def test_nearest_point_of_the_enumerated_grid(mantissa_bits, k):
 
 
 @pytest.mark.parametrize("shape, axis", [((16, 8, 3, 3), 0), ((8, 16, 3, 3), 1), ((32, 100), 0), ((5, 7), 1),
-                                         ((6, 4, 8), 1)])
+                                         ((6, 4, 8), 1),
+                                         # rows of 1024 elements and more take the row-wise kernel: a ragged row, rows
+                                         # inside an outer dimension, several workgroups per row, the shortest such row
+                                         ((12, 4100), 0), ((3, 5, 2048), 1), ((64, 8192), 0), ((2, 3, 1024), 1),
+                                         ((3, 20000), 0)])
 def test_per_channel(shape, axis):
     from aimet_amd import ops
     g = torch.Generator(device='cuda').manual_seed(7)
