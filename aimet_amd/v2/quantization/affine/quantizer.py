@@ -90,7 +90,7 @@ class MinMaxQuantizer(nn.Module):
             raise ValueError(f"qmax should be strictly larger than qmin. Got qmax={qmax}, qmin={qmin}")
         self.qmin, self.qmax = qmin, qmax
         self._symmetric = symmetric
-        self.block_size = tuple(block_size) if block_size is not None else None
+        self.block_size = block_size   # kept as given (list or tuple), as the reference does
         # with blocks, statistics are gathered on the tensor split into (blocks, block length) per axis, by an
         # analyzer whose shape has a 1 after every axis (reference :140-148)
         self.encoding_analyzer: EncodingAnalyzer = encoding_analyzer or MinMaxEncodingAnalyzer(
@@ -325,3 +325,73 @@ class QuantizeDequantize(MinMaxQuantizer):
         encoding = self.get_encoding()
         return quantize_dequantize(input, encoding.scale, encoding.offset, encoding.qmin, encoding.qmax,
                                    block_size=self.block_size)
+
+
+class GroupedBlockQuantizeDequantize(QuantizeDequantize):
+    """Blockwise quantize-dequantize whose block scales are small integers times one scale per group of blocks
+    (reference :700-822).
+
+    The block scales that min / max define are themselves put on a grid: within a group of ``block_grouping`` blocks
+    per axis, gamma = (largest block scale) / 2^(decompressed_bw - bitwidth), and every block of the group uses
+    clamp(round(scale / gamma), 1, 2^(decompressed_bw - bitwidth)) * gamma.  A weight quantized this way expands to
+    ``decompressed_bw``-bit integers times one floating-point scale per group.  -1 in ``block_grouping`` groups all
+    blocks of that axis; the default groups nothing (every block is its own group, so its scale is kept).
+    """
+
+    def __init__(self, shape, bitwidth: int, symmetric: bool, decompressed_bw: int,
+                 encoding_analyzer: EncodingAnalyzer = None, block_size=None, block_grouping=None):
+        super().__init__(shape, bitwidth, symmetric, encoding_analyzer, block_size)
+        self.decompressed_bw = decompressed_bw
+        if block_grouping is None:
+            self.block_grouping = tuple(1 for _ in self.shape)
+        else:
+            self.block_grouping = block_grouping   # kept as given
+            if len(self.block_grouping) != len(self.shape):
+                raise RuntimeError(f'Length of block grouping {block_grouping} must equal length of shape {shape}.')
+            for size, group in zip(self.shape, self.block_grouping):
+                if group != -1 and size % group != 0:
+                    raise RuntimeError(f'Quantizer shape dimensions must divide evenly with corresponding block '
+                                       f'grouping values for shapes {shape} and block grouping {block_grouping}.')
+        if self.decompressed_bw < self.bitwidth:
+            raise RuntimeError(f'Decompressed bitwidth {decompressed_bw} cannot be smaller than self.bitwidth '
+                               f'{bitwidth}')
+        if not symmetric:
+            raise RuntimeError('GroupedBlockQuantizeDequantize only supports symmetric quantization.')
+
+    def get_expanded_scale_shape(self):
+        """The scale's shape with every axis split into (groups, blocks per group)."""
+        expanded = []
+        for size, group in zip(self.shape, self.block_grouping):
+            per_group = size if group == -1 else group
+            expanded += [size // per_group, per_group]
+        return expanded
+
+    def _block_scales_by_group(self, dtype):
+        """(block scales viewed as [groups, blocks per group] per axis, gamma of every group)"""
+        grouped = super().get_scale(dtype).view(self.get_expanded_scale_shape())
+        within_group = list(range(1, grouped.dim(), 2))
+        gamma = torch.amax(grouped, within_group, keepdim=True) / 2 ** (self.decompressed_bw - self.bitwidth)
+        return grouped, gamma
+
+    def get_per_channel_scale(self, dtype=None) -> Optional[torch.Tensor]:
+        """gamma: the floating-point scale every block of a group shares."""
+        if not self.is_initialized():
+            return None
+        return self._block_scales_by_group(dtype)[1]
+
+    def get_scale(self, dtype=None) -> Optional[torch.Tensor]:
+        """The block scales after rounding to integer multiples of their group's gamma."""
+        if not self.is_initialized():
+            return None
+        grouped, gamma = self._block_scales_by_group(dtype)
+        on_grid = quantize_dequantize(grouped, gamma, torch.zeros_like(gamma), 1,
+                                      2 ** (self.decompressed_bw - self.bitwidth))
+        return on_grid.view(self.shape)
+
+    def get_per_block_integer_scale(self) -> Optional[torch.Tensor]:
+        """The integer of every block: its scale divided by its group's gamma."""
+        if not self.is_initialized():
+            return None
+        gamma = self.get_per_channel_scale()
+        grouped = self.get_scale().view(self.get_expanded_scale_shape())
+        return torch.round(grouped / gamma).int().view(self.shape)

@@ -16,13 +16,13 @@ from typing import Tuple, Union
 import torch
 from torch import nn
 
-from ..common.defs import QuantizationDataType, QuantScheme
-from ..v1.qc_quantize_op import StaticGridQuantWrapper
-from ..v1.quantsim import QuantizationSimModel as _V1QuantizationSimModel
-from ..v1.tensor_quantizer import StaticGridPerChannelQuantizer
-from .nn import BaseQuantizationMixin, QuantizationMixin
-from .quantization.affine import QuantizeDequantize
-from .quantization.encoding_analyzer import MinMaxEncodingAnalyzer, PercentileEncodingAnalyzer, SqnrEncodingAnalyzer
+from ...common.defs import QuantizationDataType, QuantScheme
+from ...v1.qc_quantize_op import StaticGridQuantWrapper
+from ...v1.quantsim import QuantizationSimModel as _V1QuantizationSimModel
+from ...v1.tensor_quantizer import StaticGridPerChannelQuantizer
+from ..nn import BaseQuantizationMixin, QuantizationMixin
+from ..quantization.affine import QuantizeDequantize
+from ..quantization.encoding_analyzer import MinMaxEncodingAnalyzer, PercentileEncodingAnalyzer, SqnrEncodingAnalyzer
 
 _RANGE_LEARNING = (QuantScheme.training_range_learning_with_tf_init,
                    QuantScheme.training_range_learning_with_tf_enhanced_init)
@@ -60,7 +60,7 @@ class QuantizationSimModel:
                 with open(config_file) as f:
                     config_file = json.load(f)
             elif config_file is None:
-                from ..v1.quantsim import DEFAULT_CONFIG  # pylint: disable=import-outside-toplevel
+                from ...v1.quantsim import DEFAULT_CONFIG  # pylint: disable=import-outside-toplevel
                 config_file = DEFAULT_CONFIG
             config_file = json.loads(json.dumps(config_file))
             config_file.setdefault("defaults", {})["per_channel_quantization"] = str(bool(per_channel_quantization))

@@ -1,0 +1,166 @@
+"""GPU tests of the helpers that switch weight quantizers of a v2 simulation model to blockwise / grouped blockwise.
+
+Cases follow TrainingExtensions/torch/test/python/v2/quantsim/test_config_utils.py:116-320: selection by layer list,
+predicate and module type, the quantizer shapes and settings that result, the error for a weight the block size does
+not divide, single-value block size / grouping on Conv2d, Linear and ConvTranspose2d, and the error for a layer type
+without input / output channels."""
+import pytest
+import torch
+from torch import nn
+
+pytestmark = pytest.mark.gpu
+
+
+class _Net(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.conv1, self.relu1 = nn.Conv2d(3, 8, 3, padding=1), nn.ReLU()
+        self.conv2, self.relu2 = nn.Conv2d(8, 16, 3, padding=1), nn.ReLU()
+        self.conv3, self.relu3 = nn.Conv2d(16, 8, 3, padding=1), nn.ReLU()
+        self.conv4 = nn.Conv2d(8, 8, 1)
+        self.pool, self.flatten = nn.AdaptiveAvgPool2d(2), nn.Flatten()
+        self.fc = nn.Linear(32, 12)
+
+    def forward(self, x):
+        x = self.relu1(self.conv1(x))
+        x = self.relu3(self.conv3(self.relu2(self.conv2(x))))
+        return self.fc(self.flatten(self.pool(self.conv4(x))))
+
+
+def _sim(model, dummy):
+    from aimet_amd.v2.quantsim import QuantizationSimModel
+    return QuantizationSimModel(model.eval().cuda(), dummy)
+
+
+def _per_tensor_8bit(q):
+    return q.is_initialized() and len(q.shape) == 0 and q.bitwidth == 8
+
+
+def test_blockwise_by_layer_list_predicate_and_type():
+    from aimet_amd.v2.quantization.affine import QuantizeDequantize
+    from aimet_amd.v2.quantsim.config_utils import set_blockwise_quantization_for_weights
+    torch.manual_seed(0)
+    dummy = torch.randn(1, 3, 16, 16).cuda()
+    sim = _sim(_Net(), dummy)
+    sim.compute_encodings(lambda m, _: m(dummy), None)
+    convs = [sim.model.conv2, sim.model.conv3, sim.model.conv4]   # not conv1: 3 input channels
+    assert all(_per_tensor_8bit(c.param_quantizers['weight']) for c in convs)
+
+    def blockwise(c):
+        q = c.param_quantizers['weight']
+        return (isinstance(q, QuantizeDequantize) and not q.is_initialized() and q.bitwidth == 4 and
+                q.min.device == c.weight.device and
+                tuple(q.shape) == (c.weight.shape[0], c.weight.shape[1] // 4, 1, 1))
+
+    set_blockwise_quantization_for_weights(sim, [convs[0]], 4, True, [1, 4, -1, -1])
+    assert blockwise(convs[0])
+    assert all(_per_tensor_8bit(c.param_quantizers['weight']) for c in convs[1:])
+    set_blockwise_quantization_for_weights(sim, lambda m: m is convs[1], 4, True, [1, 4, -1, -1])
+    assert blockwise(convs[0]) and blockwise(convs[1])
+    assert _per_tensor_8bit(convs[2].param_quantizers['weight'])
+    assert _per_tensor_8bit(sim.model.fc.param_quantizers['weight'])
+    with pytest.raises(RuntimeError, match='do not align with block size'):
+        set_blockwise_quantization_for_weights(sim, [type(sim.model.conv1)], 4, True, [1, 4, -1, -1])
+    set_blockwise_quantization_for_weights(sim, [type(sim.model.fc)], 4, True, [1, 4])
+    fc = sim.model.fc.param_quantizers['weight']
+    assert not fc.is_initialized() and fc.bitwidth == 4 and tuple(fc.shape) == (12, 8)
+    # the reconfigured model calibrates and runs
+    sim.compute_encodings(lambda m, _: m(dummy), None)
+    assert fc.is_initialized() and torch.isfinite(sim.model(dummy)).all()
+
+
+def test_grouped_blockwise_by_layer_list_predicate_and_type():
+    from aimet_amd.v2.quantization.affine import GroupedBlockQuantizeDequantize, QuantizeDequantize
+    from aimet_amd.v2.quantsim.config_utils import set_grouped_blockwise_quantization_for_weights
+    torch.manual_seed(0)
+    dummy = torch.randn(1, 3, 16, 16).cuda()
+    sim = _sim(_Net(), dummy)
+    sim.compute_encodings(lambda m, _: m(dummy), None)
+    convs = [sim.model.conv2, sim.model.conv3, sim.model.conv4]
+
+    def grouped(c):
+        q = c.param_quantizers['weight']
+        return (isinstance(q, GroupedBlockQuantizeDequantize) and not q.is_initialized() and q.bitwidth == 4 and
+                q.decompressed_bw == 8 and tuple(q.block_grouping) == (1, -1, 1, 1) and
+                q.min.device == c.weight.device and
+                tuple(q.shape) == (c.weight.shape[0], c.weight.shape[1] // 4, 1, 1))
+
+    set_grouped_blockwise_quantization_for_weights(sim, [convs[0]], 4, True, 8, [1, 4, -1, -1], [1, -1, 1, 1])
+    assert grouped(convs[0])
+    for c in convs[1:]:
+        assert type(c.param_quantizers['weight']) is QuantizeDequantize and _per_tensor_8bit(c.param_quantizers['weight'])
+    set_grouped_blockwise_quantization_for_weights(sim, lambda m: m is convs[1], 4, True, 8, [1, 4, -1, -1],
+                                                   [1, -1, 1, 1])
+    assert grouped(convs[0]) and grouped(convs[1])
+    assert _per_tensor_8bit(convs[2].param_quantizers['weight'])
+    with pytest.raises(RuntimeError):
+        set_grouped_blockwise_quantization_for_weights(sim, [type(sim.model.conv1)], 4, True, 8, [1, 4, -1, -1],
+                                                       [1, -1, -1, -1])
+    set_grouped_blockwise_quantization_for_weights(sim, [type(sim.model.fc)], 4, True, 8, [1, 4], [1, -1])
+    fc = sim.model.fc.param_quantizers['weight']
+    assert isinstance(fc, GroupedBlockQuantizeDequantize) and not fc.is_initialized() and fc.bitwidth == 4
+    assert tuple(fc.shape) == (12, 8) and fc.decompressed_bw == 8 and tuple(fc.block_grouping) == (1, -1)
+
+
+def test_single_value_block_size_and_grouping():
+    from aimet_amd.v2.quantsim.config_utils import set_grouped_blockwise_quantization_for_weights
+    torch.manual_seed(0)
+    dummy = torch.randn(1, 3, 16, 16).cuda()
+    sim = _sim(_Net(), dummy)
+    layers = [m for m in sim.model.modules() if isinstance(m, (nn.Conv2d, nn.Linear)) and m.weight.shape[1] != 3]
+    assert len(layers) == 4
+    set_grouped_blockwise_quantization_for_weights(sim, lambda m: any(m is x for x in layers), 4, True, 8, 4, -1)
+    sim.compute_encodings(lambda m, _: m(dummy), None)
+    assert torch.isfinite(sim.model(dummy)).all()
+    for m in layers:
+        q = m.param_quantizers['weight']
+        if isinstance(m, nn.Conv2d):
+            assert q.block_size == [1, 4, -1, -1] and q.block_grouping == [1, -1, 1, 1]
+        else:
+            assert q.block_size == [1, 4] and q.block_grouping == [1, -1]
+        # one gamma per output channel: the integers of a row reach 16 and its scales are integers times gamma
+        integers = q.get_per_block_integer_scale()
+        assert int(integers.min()) >= 1 and int(integers.amax()) == 16
+
+    class Transposed(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up1, self.relu, self.up2 = nn.ConvTranspose2d(10, 10, 3), nn.ReLU(), nn.ConvTranspose2d(10, 4, 3)
+
+        def forward(self, x):
+            return self.up2(self.relu(self.up1(x)))
+
+    dummy = torch.randn(2, 10, 3, 4).cuda()
+    sim = _sim(Transposed(), dummy)
+    layers = [m for m in sim.model.modules() if isinstance(m, nn.ConvTranspose2d)]
+    assert len(layers) == 2
+    set_grouped_blockwise_quantization_for_weights(sim, lambda m: any(m is x for x in layers), 4, True, 8, 2, -1)
+    sim.compute_encodings(lambda m, _: m(dummy), None)
+    assert torch.isfinite(sim.model(dummy)).all()
+    for m in layers:
+        q = m.param_quantizers['weight']
+        # input channels are axis 0 of a transposed convolution's weight
+        assert q.block_size == [2, 1, -1, -1] and q.block_grouping == [-1, 1, 1, 1]
+        assert tuple(q.shape) == (5, m.weight.shape[1], 1, 1)
+
+
+def test_single_value_needs_a_layer_with_channels():
+    from aimet_amd.v2.quantization.affine import QuantizeDequantize
+    from aimet_amd.v2.quantsim.config_utils import set_blockwise_quantization_for_weights
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc, self.norm = nn.Linear(10, 10), nn.LayerNorm(10)
+
+        def forward(self, x):
+            return self.norm(self.fc(x))
+
+    dummy = torch.randn(1, 10).cuda()
+    sim = _sim(Net(), dummy)
+    if sim.model.norm.param_quantizers['weight'] is None:
+        sim.model.norm.param_quantizers['weight'] = QuantizeDequantize((), 8, True).cuda()
+    with pytest.raises(RuntimeError, match='modules_with_in_out_channels'):
+        set_blockwise_quantization_for_weights(sim, lambda m: isinstance(m, nn.LayerNorm), 4, True, 2)
+    with pytest.raises(RuntimeError, match='must contain either'):
+        set_blockwise_quantization_for_weights(sim, ['fc'], 4, True, 2)
