@@ -57,7 +57,9 @@ _SIGNATURES = {
     "miq_v2_qdq_bwd_params_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p, _p, _p, _p], _int),
     "miq_v2_qdq_bwd_params_bf16": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p, _p, _p, _p], _int),
     "miq_fp16_round_trip_f32": ([_p, _p, _i64, _p], _int),
+    "miq_bf16_round_trip_f32": ([_p, _p, _i64, _p], _int),
     "miq_fp8_fake_cast_f32": ([_p, _p, _i64, _i64, _i64, _p, _p, _p, _int, _p], _int),
+    "miq_float_fake_cast_f32": ([_p, _p, _i64, _i64, _i64, _p, _p, _p, _int, _p], _int),
     "miq_set_stochastic_seed": ([C.c_uint64], _int),
     "miq_get_stochastic_state": ([C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)], _int),
     "miq_minmax_workspace_bytes": ([_i64, _i64, _i64], _i64),

@@ -1,6 +1,7 @@
-// Simulation of an 8-bit float grid: every element is rounded to the grid of a float format with `mantissa_bits`
-// mantissa and 7 - mantissa_bits exponent bits whose largest value is the tensor's (or the channel's) maxval
-// (TORCH/fp_quantization.py:133-209, quantize_to_fp8 / fake_cast_to_ieee_float).  A float grid is an integer grid whose
+// Simulation of a narrow float grid: every element is rounded to the grid of a float format with M mantissa and E
+// exponent bits (the 8-bit formats have E = 7 - M) whose largest value is the tensor's (or the channel's) maxval
+// (TORCH/fp_quantization.py:133-209, quantize_to_fp8 / fake_cast_to_ieee_float; the v2 float quantizer calls the latter
+// with any E and M: TORCH/v2/quantization/float/quantizer.py:302-322).  A float grid is an integer grid whose
 // step depends on the element's own exponent:
 //   x_c   = clamp(x, -maxval, maxval)
 //   e     = max(floor(log2|x_c| + bias), 1)                    bias = 2^E - log2(maxval) + log2(2 - 2^-M) - 1
@@ -38,7 +39,7 @@ __device__ __forceinline__ float fp8_elem(float x, float mx, float bias, const f
 // per group of four, which made it ALU-bound at 56 % of HBM peak on [11008, 4096]).  The channel's steps go to LDS next
 // to their reciprocals, and the division runs through div_by_invariant() when every step and maxval are inside its
 // contract (a quotient below its 2^-36 limit rounds to zero either way).
-constexpr int kFp8TableMax = 65;   // 2^6 + 1 steps at one mantissa bit
+constexpr int kFp8TableMax = 257;   // 2^8 + 1 steps: eight exponent bits (bfloat16's)
 __global__ void __launch_bounds__(256) fp8_rows_kernel(const float* __restrict__ in, float* __restrict__ out,
                                                         int64_t inner4, int64_t channels, int pieces,
                                                         const float* __restrict__ maxval,
@@ -65,11 +66,11 @@ __global__ void __launch_bounds__(256) fp8_rows_kernel(const float* __restrict__
     request();   // the first loads travel while the channel's table is set up
     const float mx = maxval[c], b = bias[c];
     bool in_contract = true;
-    if ((int) threadIdx.x < table)
+    for (int t = threadIdx.x; t < table; t += 256)
     {
-        const float st      = steps[c * table + threadIdx.x];
-        s_step[threadIdx.x] = make_float2(st, 1.0f / st);
-        in_contract         = fastdiv_divisor_ok(st);
+        const float st = steps[c * table + t];
+        s_step[t]      = make_float2(st, 1.0f / st);
+        in_contract    = in_contract && fastdiv_divisor_ok(st);
     }
     const bool short_div = __syncthreads_and(in_contract) && mx <= kFastDivMaxDividend;
     const float last     = (float) (table - 1);
@@ -136,19 +137,20 @@ __global__ void __launch_bounds__(256) fp8_kernel(const float* __restrict__ in, 
 }   // namespace
 }   // namespace miq
 
-extern "C" int miq_fp8_fake_cast_f32(const float* in, float* out, int64_t n, int64_t num_channels, int64_t inner,
-                                     const float* maxval, const float* bias, const float* steps, int mantissa_bits,
-                                     void* stream)
+extern "C" {
+
+int miq_float_fake_cast_f32(const float* in, float* out, int64_t n, int64_t num_channels, int64_t inner,
+                            const float* maxval, const float* bias, const float* steps, int table, void* stream)
 {
     using namespace miq;
     MIQ_CHECK_ARG(n >= 0 && (n == 0 || (in && out && maxval && bias && steps)), "null tensor pointer or negative count");
     MIQ_CHECK_ARG(num_channels >= 1 && inner >= 1, "num_channels and inner must be positive");
     MIQ_CHECK_ARG(n % (num_channels * inner) == 0, "element count is not a multiple of num_channels * inner");
-    MIQ_CHECK_ARG(mantissa_bits >= 1 && mantissa_bits <= 6, "mantissa_bits must be in [1, 6]");
+    MIQ_CHECK_ARG(table >= 3 && table <= kFp8TableMax, "the step table must hold 2^E + 1 entries, E in [1, 8] (got %d)",
+                  table);
     if (n == 0)
         return MIQ_OK;
-    const int table = (1 << (7 - mantissa_bits)) + 1;   // step of every exponent e = 0 .. 2^E
-    const bool vec  = (n % 4 == 0) && (num_channels == 1 || inner % 4 == 0) &&
+    const bool vec = (n % 4 == 0) && (num_channels == 1 || inner % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) % 16 == 0);
     const int64_t work   = vec ? n / 4 : n;
     const int64_t blocks = (work + 255) / 256;
@@ -156,7 +158,7 @@ extern "C" int miq_fp8_fake_cast_f32(const float* in, float* out, int64_t n, int
     // rows long enough to give every wavefront of a workgroup its own loads go by rows
     const int64_t row_len = num_channels == 1 ? n : inner;
     const int64_t rows    = n / row_len;
-    if (vec && row_len >= 1024 && table <= kFp8TableMax)
+    if (vec && row_len >= 1024)
     {
         // four 16-byte groups per lane, and no more pieces than keep the grid near 16K workgroups
         const int64_t inner4 = row_len / 4;
@@ -176,3 +178,13 @@ extern "C" int miq_fp8_fake_cast_f32(const float* in, float* out, int64_t n, int
     MIQ_CHECK_LAUNCH();
     return MIQ_OK;
 }
+
+int miq_fp8_fake_cast_f32(const float* in, float* out, int64_t n, int64_t num_channels, int64_t inner,
+                          const float* maxval, const float* bias, const float* steps, int mantissa_bits, void* stream)
+{
+    MIQ_CHECK_ARG(mantissa_bits >= 1 && mantissa_bits <= 6, "mantissa_bits must be in [1, 6]");
+    return miq_float_fake_cast_f32(in, out, n, num_channels, inner, maxval, bias, steps,
+                                   (1 << (7 - mantissa_bits)) + 1, stream);
+}
+
+}   // extern "C"

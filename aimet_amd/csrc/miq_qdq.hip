@@ -128,6 +128,29 @@ struct OpFp16
     }
 };
 
+// y = float(bfloat16(x)): the v2 float quantizer's bfloat16 case (TORCH/v2/quantization/float/quantizer.py:309-314,
+// input.to(torch.bfloat16).to(input.dtype)), round to nearest even
+struct OpBf16
+{
+    using P                  = int;   // no parameters
+    static constexpr int NIN = 1;
+    using Code               = uint8_t;
+    __device__ static P load(const ParamSrc&, uint32_t)
+    {
+        return 0;
+    }
+    __device__ static bool fast_ok(const P&, const float*, int)
+    {
+        return true;
+    }
+    template <bool FAST>
+    __device__ static float apply(const ParamSrc&, const P&, float x, float, int& code)
+    {
+        code = 0;
+        return bf16_to_f32(f32_to_bf16(x));
+    }
+};
+
 // gin = g * (min <= x <= max)
 struct OpV1Ste
 {
@@ -244,6 +267,11 @@ __device__ V1P scalar_params<OpV1Quantize>(const ParamSrc& s)
 }
 template <>
 __device__ int scalar_params<OpFp16>(const ParamSrc&)
+{
+    return 0;
+}
+template <>
+__device__ int scalar_params<OpBf16>(const ParamSrc&)
 {
     return 0;
 }
@@ -711,6 +739,13 @@ int miq_fp16_round_trip_f32(const float* in, float* out, int64_t n, void* stream
     MIQ_CHECK_ARG(n >= 0 && (n == 0 || (in && out)), "null tensor pointer or negative count");
     EwPtrs<float, uint8_t> p{in, nullptr, out, nullptr};
     return launch_ew<float, OpFp16, false>(p, ParamSrc{}, n, 1, 1, (hipStream_t) stream);
+}
+
+int miq_bf16_round_trip_f32(const float* in, float* out, int64_t n, void* stream)
+{
+    MIQ_CHECK_ARG(n >= 0 && (n == 0 || (in && out)), "null tensor pointer or negative count");
+    EwPtrs<float, uint8_t> p{in, nullptr, out, nullptr};
+    return launch_ew<float, OpBf16, false>(p, ParamSrc{}, n, 1, 1, (hipStream_t) stream);
 }
 
 int miq_quantize_per_tensor_f32(const float* in, float* out, int64_t n, double enc_min, double enc_max, int bw,

@@ -6,7 +6,7 @@ only; there is no torch-op fallback: tensors that are not on a GPU are rejected.
 """
 import ctypes as C
 
-
+import numpy as np
 import torch
 
 from . import _lib
@@ -135,43 +135,60 @@ def fp16_round_trip(x, out=None):
     return out
 
 
-def fp8_grid(maxval, mantissa_bits: int = 3):
-    """(maxval, bias, steps) device tensors that describe the 8-bit float grid ending at `maxval` (a float, a one-element
-    tensor, or one value per channel): bias of the format, and for every channel the step 2^((e - M) - bias) of each
-    exponent e = 0 .. 2^E, all in float32 as the reference's expression evaluates them
-    (aimet_torch/fp_quantization.py:171-209).  Reusable for as long as maxval does not change."""
+def float_grid(maxval, exponent_bits: int, mantissa_bits: int, host_constants: bool = False, host_bias=None):
+    """(maxval, bias, steps) device tensors that describe the float grid of `exponent_bits` and `mantissa_bits` ending at
+    `maxval` (a one-element tensor, or one value per channel): bias of the format, and for every channel the step
+    2^((e - M) - bias) of each exponent e = 0 .. 2^E, all in float32 as the reference's expression evaluates them
+    (aimet_torch/fp_quantization.py:171-209).  Reusable for as long as maxval does not change.
+
+    The expression meets its constants in two ways.  The v1 path passes the mantissa bits as a device tensor, so
+    2^E and log2(2 - 2^-M) are torch float32 results (the default here).  The v2 float quantizer passes Python
+    numbers: log2(2 - 2^-M) is then numpy's float64 value, rounded to float32 where it meets the tensor
+    (`host_constants`), and when maxval too is a Python number the whole bias is a float64 that is rounded once
+    (`host_bias` = that number)."""
     if not isinstance(maxval, torch.Tensor) or not maxval.is_cuda:
         raise RuntimeError("maxval must be a tensor on the GPU")
+    if not 1 <= exponent_bits <= 8 or mantissa_bits < 1:
+        raise RuntimeError("float grids take 1 to 8 exponent bits and at least one mantissa bit")
     maxval = maxval.detach().to(_F32).reshape(-1).contiguous()
-    key = (maxval.device, mantissa_bits)
-    if key not in _FP8_CONSTANTS:
+    key = (maxval.device, exponent_bits, mantissa_bits)
+    if key not in _FLOAT_GRID_CONSTANTS:
         m = torch.tensor([float(mantissa_bits)], dtype=_F32, device=maxval.device)
-        exponents = torch.arange((1 << (7 - mantissa_bits)) + 1, dtype=_F32, device=maxval.device)
+        e = torch.tensor([float(exponent_bits)], dtype=_F32, device=maxval.device)
+        exponents = torch.arange((1 << exponent_bits) + 1, dtype=_F32, device=maxval.device)
         # 2^E, log2(2 - 2^-M) and e - M, each as torch's float32 kernels on this device give them
-        _FP8_CONSTANTS[key] = (2 ** (7 - m), torch.log2(2 - 2 ** (-m)), exponents - m)
-    two_to_e, log2_top, e_minus_m = _FP8_CONSTANTS[key]
+        _FLOAT_GRID_CONSTANTS[key] = (2 ** e, torch.log2(2 - 2 ** (-m)), exponents - m)
+    two_to_e, log2_top, e_minus_m = _FLOAT_GRID_CONSTANTS[key]
     # the bias of the format follows from its largest value: maxval = (2 - 2^-M) * 2^(2^E - 1 - bias)
-    bias = (two_to_e - torch.log2(maxval) + log2_top - 1).contiguous()
+    if host_bias is not None:
+        bias = torch.full_like(maxval, float(host_bias))
+    elif host_constants:
+        bias = (2 ** exponent_bits - torch.log2(maxval) + float(np.log2(2 - 2 ** (-mantissa_bits))) - 1).contiguous()
+    else:
+        bias = (two_to_e - torch.log2(maxval) + log2_top - 1).contiguous()
     steps = (2. ** (e_minus_m.unsqueeze(0) - bias.unsqueeze(1))).contiguous()
     return maxval, bias, steps
 
 
-_FP8_CONSTANTS = {}
+def fp8_grid(maxval, mantissa_bits: int = 3):
+    """float_grid() of the 8-bit format with `mantissa_bits` mantissa and 7 - mantissa_bits exponent bits."""
+    return float_grid(maxval, 7 - mantissa_bits, mantissa_bits)
 
 
-def fp8_fake_cast(x, maxval, mantissa_bits: int = 3, ch_axis: int = 0, out=None, grid=None):
-    """Rounds a float32 tensor to the 8-bit float grid (mantissa_bits mantissa, 7 - mantissa_bits exponent bits) whose
-    largest value is `maxval`: a one-element tensor or float for the whole tensor, or a 1-d tensor with one value per
-    channel along `ch_axis` (reference aimet_torch/fp_quantization.py:133-209).  `grid` = fp8_grid(maxval,
-    mantissa_bits) computed earlier saves recomputing it."""
+_FLOAT_GRID_CONSTANTS = {}
+
+
+def float_fake_cast(x, maxval, exponent_bits: int, mantissa_bits: int, ch_axis: int = 0, out=None, grid=None):
+    """Rounds a float32 tensor to the float grid of `exponent_bits` (1 to 8) and `mantissa_bits` whose largest value is
+    `maxval`: a one-element tensor for the whole tensor, or a 1-d tensor with one value per channel along `ch_axis`
+    (reference aimet_torch/fp_quantization.py:171-209, fake_cast_to_ieee_float).  `grid` = float_grid(maxval,
+    exponent_bits, mantissa_bits) computed earlier saves recomputing it."""
     _require_gpu(x, out)
     if x.dtype != _F32:
-        raise RuntimeError("fp8_fake_cast takes float32 tensors")
-    if not 1 <= mantissa_bits <= 6:
-        raise RuntimeError("mantissa_bits must be in [1, 6]")
+        raise RuntimeError("float_fake_cast takes float32 tensors")
     x = x.contiguous()
     if grid is None:
-        grid = fp8_grid(torch.as_tensor(maxval, dtype=_F32, device=x.device), mantissa_bits)
+        grid = float_grid(torch.as_tensor(maxval, dtype=_F32, device=x.device), exponent_bits, mantissa_bits)
     maxval, bias, steps = grid
     channels = maxval.numel()
     inner = x.numel()
@@ -184,8 +201,28 @@ def fp8_fake_cast(x, maxval, mantissa_bits: int = 3, ch_axis: int = 0, out=None,
             inner *= d
     out = torch.empty_like(x) if out is None else out
     with _OnDevice(x.device):
-        check(lib.miq_fp8_fake_cast_f32(_ptr(x), _ptr(out), x.numel(), channels, max(inner, 1), _ptr(maxval),
-                                        _ptr(bias), _ptr(steps), mantissa_bits, _stream(x)))
+        check(lib.miq_float_fake_cast_f32(_ptr(x), _ptr(out), x.numel(), channels, max(inner, 1), _ptr(maxval),
+                                          _ptr(bias), _ptr(steps), steps.shape[1], _stream(x)))
+    return out
+
+
+def fp8_fake_cast(x, maxval, mantissa_bits: int = 3, ch_axis: int = 0, out=None, grid=None):
+    """float_fake_cast() on the 8-bit grid with `mantissa_bits` mantissa and 7 - mantissa_bits exponent bits
+    (reference aimet_torch/fp_quantization.py:133-169, quantize_to_fp8)."""
+    if not 1 <= mantissa_bits <= 6:
+        raise RuntimeError("mantissa_bits must be in [1, 6]")
+    return float_fake_cast(x, maxval, 7 - mantissa_bits, mantissa_bits, ch_axis, out, grid)
+
+
+def bf16_round_trip(x, out=None):
+    """float(bfloat16(x)) for a float32 tensor, in one pass."""
+    _require_gpu(x, out)
+    if x.dtype != _F32:
+        raise RuntimeError("bf16_round_trip takes float32 tensors")
+    x = x.contiguous()
+    out = torch.empty_like(x) if out is None else out
+    with _OnDevice(x.device):
+        check(lib.miq_bf16_round_trip_f32(_ptr(x), _ptr(out), x.numel(), _stream(x)))
     return out
 
 

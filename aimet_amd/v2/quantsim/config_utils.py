@@ -1,5 +1,5 @@
 """Helpers that swap the weight quantizers of chosen layers of a v2 simulation model for blockwise or grouped blockwise
-ones, and put activation quantizers on a float grid.
+ones, and the activation quantizers for float quantizers.
 
 Mirrors TrainingExtensions/torch/src/python/aimet_torch/v2/quantsim/config_utils.py: which layers are meant is given as
 a list of module types, a list of the simulation model's own layers, or a predicate (:134-147); a single block size
@@ -7,11 +7,13 @@ applies to the weight's input-channel axis with one scale per output channel (:8
 input-channel axis (:110-131); -1 spans the axis; a weight whose shape a block size does not divide is an error that
 names the layer (:312-331).
 """
-from typing import Callable, List, Optional, Tuple, Type, Union
+import itertools
+from typing import Callable, List, Optional, Tuple, Union
 
 import torch
 
 from ..quantization.affine import GroupedBlockQuantizeDequantize, QuantizeDequantize
+from ..quantization.float import FloatQuantizeDequantize
 
 _TRANSPOSED = (torch.nn.ConvTranspose1d, torch.nn.ConvTranspose2d, torch.nn.ConvTranspose3d)
 modules_with_in_out_channels = (torch.nn.Linear, torch.nn.Conv1d, torch.nn.Conv2d, torch.nn.Conv3d) + _TRANSPOSED
@@ -88,7 +90,7 @@ def _layers_and_shapes(sim, condition, block_size):
 
 
 def _device_of(quantizer: torch.nn.Module, default):
-    for tensor in quantizer.parameters():
+    for tensor in itertools.chain(quantizer.parameters(), quantizer.buffers()):
         return tensor.device
     return default
 
@@ -119,3 +121,19 @@ def set_grouped_blockwise_quantization_for_weights(sim, arg, bitwidth: int, symm
         device = _device_of(layer.param_quantizers['weight'], model_device)
         layer.param_quantizers['weight'] = GroupedBlockQuantizeDequantize(shape, bitwidth, symmetric, decompressed_bw,
                                                                           None, per_axis, grouping).to(device)
+
+
+def set_activation_quantizers_to_float(sim, arg, exponent_bits: int = None, mantissa_bits: int = None,
+                                       dtype: torch.dtype = None):
+    """Input and output quantizers of the layers `arg` selects become float quantizers of the given format (a torch
+    dtype, or exponent and mantissa bits); slots without a quantizer stay empty (reference :187-242)."""
+    condition = _as_condition(arg)
+    model_device = next(sim.model.parameters()).device
+    for _, layer in sim.named_qmodules():
+        if not condition(layer):
+            continue
+        for slots in (layer.input_quantizers, layer.output_quantizers):
+            for index, quantizer in enumerate(slots):
+                if quantizer is not None:
+                    device = _device_of(quantizer, model_device)
+                    slots[index] = FloatQuantizeDequantize(exponent_bits, mantissa_bits, dtype).to(device)

@@ -22,6 +22,7 @@ from ...v1.quantsim import QuantizationSimModel as _V1QuantizationSimModel
 from ...v1.tensor_quantizer import StaticGridPerChannelQuantizer
 from ..nn import BaseQuantizationMixin, QuantizationMixin
 from ..quantization.affine import QuantizeDequantize
+from ..quantization.float import FloatQuantizeDequantize
 from ..quantization.encoding_analyzer import MinMaxEncodingAnalyzer, PercentileEncodingAnalyzer, SqnrEncodingAnalyzer
 
 _RANGE_LEARNING = (QuantScheme.training_range_learning_with_tf_init,
@@ -111,7 +112,13 @@ class QuantizationSimModel:
             raise NotImplementedError("strict-symmetric and unsigned-symmetric grids are not available in the v2 "
                                       "simulation (the reference's builder asserts the same)")
         if q.data_type != QuantizationDataType.int:
-            raise NotImplementedError("only integer grids are implemented")
+            # builder.py:343-355: float16 is a cast there and back; the 8-bit float has 3 mantissa and 4 exponent bits
+            # and takes its largest value from the statistics of the quant scheme's analyzer
+            if q.bitwidth == 16:
+                return FloatQuantizeDequantize(dtype=torch.float16).to(device)
+            if q.bitwidth != 8:
+                raise NotImplementedError(f"float quantizers have 16 or 8 bits (got {q.bitwidth})")
+            return FloatQuantizeDequantize(4, 3, encoding_analyzer=_analyzer(self._quant_scheme, shape)).to(device)
         quantizer = QuantizeDequantize(shape, q.bitwidth, q.use_symmetric_encodings,
                                        _analyzer(self._quant_scheme, shape)).to(device)
         if self._quant_scheme not in _RANGE_LEARNING:

@@ -105,6 +105,17 @@ int miq_fp16_round_trip_f32(const float* in, float* out, int64_t n, void* stream
 int miq_fp8_fake_cast_f32(const float* in, float* out, int64_t n, int64_t num_channels, int64_t inner,
                           const float* maxval, const float* bias, const float* steps, int mantissa_bits, void* stream);
 
+/* The same for a float format of E exponent and M mantissa bits, E in [1, 8]: fake_cast_to_ieee_float as the v2 float
+ * quantizer calls it (TORCH/v2/quantization/float/quantizer.py:302-322; TORCH/fp_quantization.py:171-209) with
+ * bias[c] = 2^E - log2(maxval[c]) + log2(2 - 2^-M) - 1.  M enters only through the steps, so the entry point takes the
+ * table and its length: steps[c * table + e] = 2^((e - M) - bias[c]) for e = 0 .. table - 1, table = 2^E + 1. */
+int miq_float_fake_cast_f32(const float* in, float* out, int64_t n, int64_t num_channels, int64_t inner,
+                            const float* maxval, const float* bias, const float* steps, int table, void* stream);
+
+/* out = float(bfloat16(in)), round to nearest even, NaN stays NaN: the v2 float quantizer's bfloat16 case,
+ * input.to(torch.bfloat16).to(input.dtype) (TORCH/v2/quantization/float/quantizer.py:309-314), in one pass. */
+int miq_bf16_round_trip_f32(const float* in, float* out, int64_t n, void* stream);
+
 /* ITensorQuantizationSim<float>::quantizeTensor(..., shiftToSigned) (ITensorQuantizationSim.h:57-59,
  * DLQ/src/TensorQuantizationSim.cpp:116-126; kernel DLQ/src/trim_functions.cu:62-76): float-valued grid indices. */
 int miq_quantize_per_tensor_f32(const float* in, float* out, int64_t n, double enc_min, double enc_max, int bw,

@@ -164,3 +164,76 @@ def test_single_value_needs_a_layer_with_channels():
         set_blockwise_quantization_for_weights(sim, lambda m: isinstance(m, nn.LayerNorm), 4, True, 2)
     with pytest.raises(RuntimeError, match='must contain either'):
         set_blockwise_quantization_for_weights(sim, ['fc'], 4, True, 2)
+
+
+def test_activation_quantizers_to_float():
+    # test_config_utils.py:55-113
+    from aimet_amd.v2.quantization.affine import QuantizeDequantize
+    from aimet_amd.v2.quantization.float import FloatQuantizeDequantize
+    from aimet_amd.v2.quantsim.config_utils import set_activation_quantizers_to_float
+    torch.manual_seed(0)
+    dummy = torch.randn(1, 3, 16, 16).cuda()
+    sim = _sim(_Net(), dummy)
+    sim.compute_encodings(lambda m, _: m(dummy), None)
+
+    def count():
+        return sum(isinstance(m, (QuantizeDequantize, FloatQuantizeDequantize)) for m in sim.model.modules())
+    before = count()
+    relus = [sim.model.relu1, sim.model.relu2, sim.model.relu3]
+    others = [m for _, m in sim.named_qmodules() if not isinstance(m, nn.ReLU) and len(m.output_quantizers) > 0 and
+              m.output_quantizers[0] is not None]
+    assert others and all(r.output_quantizers[0] is not None for r in relus)
+    for layer in relus + others:
+        assert layer.output_quantizers[0].is_initialized() and isinstance(layer.output_quantizers[0], QuantizeDequantize)
+    with pytest.raises(RuntimeError):
+        set_activation_quantizers_to_float(sim, [1], dtype=torch.float16)
+    set_activation_quantizers_to_float(sim, [relus[0]], dtype=torch.float16)
+    assert isinstance(relus[0].output_quantizers[0], FloatQuantizeDequantize)
+    assert all(isinstance(r.output_quantizers[0], QuantizeDequantize) for r in relus[1:])
+    set_activation_quantizers_to_float(sim, lambda m: m is relus[1], dtype=torch.float16)
+    assert all(isinstance(r.output_quantizers[0], FloatQuantizeDequantize) for r in relus[:2])
+    assert isinstance(relus[2].output_quantizers[0], QuantizeDequantize)
+    set_activation_quantizers_to_float(sim, [type(relus[0])], dtype=torch.float16)
+    assert all(isinstance(r.output_quantizers[0], FloatQuantizeDequantize) for r in relus)
+    assert all(r.output_quantizers[0].is_float16() for r in relus)
+    assert all(isinstance(o.output_quantizers[0], QuantizeDequantize) for o in others)
+    assert count() == before
+    assert torch.isfinite(sim.model(dummy)).all()
+    # exponent / mantissa bits instead of a dtype
+    set_activation_quantizers_to_float(sim, [relus[2]], exponent_bits=4, mantissa_bits=3)
+    assert relus[2].output_quantizers[0].bitwidth == 8
+    assert torch.isfinite(sim.model(dummy)).all()
+
+
+@pytest.mark.parametrize('bitwidth', [16, 8])
+def test_simulation_model_with_float_data_type(bitwidth, tmp_path):
+    """default_data_type=float: 16 bits become float16 casts, 8 bits the 4-exponent-3-mantissa format whose largest
+    value follows the statistics (aimet_torch/quantsim_config/builder.py:343-355)."""
+    from aimet_amd.common.defs import QuantizationDataType
+    from aimet_amd.v2.quantization.float import FloatQuantizeDequantize
+    from aimet_amd.v2.quantsim import QuantizationSimModel
+    torch.manual_seed(0)
+    model = _Net().eval().cuda()
+    dummy = torch.randn(2, 3, 16, 16).cuda()
+    sim = QuantizationSimModel(model, dummy, quant_scheme='tf', default_output_bw=bitwidth, default_param_bw=bitwidth,
+                               default_data_type=QuantizationDataType.float)
+    quantizers = [m for m in sim.model.modules() if isinstance(m, FloatQuantizeDequantize)]
+    assert quantizers and all(q.bitwidth == bitwidth for q in quantizers)
+    sim.compute_encodings(lambda m, _: m(dummy), None)
+    with torch.no_grad():
+        out, plain = sim.model(dummy), model(dummy)
+    assert torch.isfinite(out).all()
+    if bitwidth == 16:
+        assert all(q.is_float16() and q.maxval is None for q in quantizers)
+        assert torch.allclose(out, plain, rtol=5e-3, atol=5e-3) and not torch.equal(out, plain)
+        w = sim.model.fc.param_quantizers['weight']
+        assert torch.equal(w(model.fc.weight), model.fc.weight.half().float())
+    else:
+        assert all((q.exponent_bits, q.mantissa_bits) == (4, 3) for q in quantizers)
+        w = sim.model.fc.param_quantizers['weight']
+        # largest value of the grid = largest weight magnitude; at most 2^8 distinct outputs
+        assert torch.equal(w.maxval.view(()), model.fc.weight.abs().max())
+        assert w(model.fc.weight).unique().numel() <= 256
+        assert (out - plain).abs().max() < 0.5 * plain.abs().max()
+    exported = sim.get_encodings_dict()
+    assert exported['param_encodings']['fc.weight'] == [{'bitwidth': bitwidth, 'dtype': 'float'}]
