@@ -42,6 +42,13 @@ constexpr int kMaxCand  = 512;
 typedef float vf4 __attribute__((ext_vector_type(4)));
 constexpr int kCopies   = 8;
 constexpr int kMaxGrid  = 2048;
+// The histogram launch: four 16-byte loads of a lane in flight and at most 1024 workgroups.  Every workgroup clears an
+// LDS histogram and flushes it with up to 512 global atomics, so fewer, longer workgroups pay less of that (the flush
+// alone is 0.8 us of a 7.5 us launch at 2048 workgroups); with two loads in flight 1024 workgroups keep too few bytes
+// on their way.  Measured per [32,256,28,28] batch, back to back: 2 loads x 2048 workgroups 7.4 us, 4 x 1024 7.1 us,
+// 4 x 1568 7.6 us, 4 x 512 9.2 us, 8 x 784 8.7 us.
+constexpr int kHistUnroll  = 4;
+constexpr int kHistMaxGrid = 1024;
 constexpr int kReplicas = 32;     // global count replicas: workgroup b merges into replica b % kReplicas, so at most
                                   // kMaxGrid / kReplicas atomics ever meet on one address
 
@@ -589,8 +596,8 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
     const vf4* v         = reinterpret_cast<const vf4*>(in);
     const vf4 nan4       = {NAN, NAN, NAN, NAN};   // dropped by hist_add
     const int64_t nvec   = n / 4;
-    const int64_t stride = (int64_t) groups * kBlock * kUnroll;
-    int64_t base         = (int64_t) group * kBlock * kUnroll;
+    const int64_t stride = (int64_t) groups * kBlock * kHistUnroll;
+    int64_t base         = (int64_t) group * kBlock * kHistUnroll;
     // ---- the previous batch, step 1: kFoldSlices workgroups from fold_first on (the first of those with the smallest
     // share of the tensor: they retire earliest) request their slice of its counts before anything else, so that this
     // round trip runs under the first tile's
@@ -607,12 +614,12 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
         if (pending_n > 0 || slice == 0)
             fl = fold_load(st, 1 - buf, 1 - buf, slice, threadIdx.x);
     }
-    vf4 a[kUnroll];
+    vf4 a[kHistUnroll];
     // first tile's loads go out next: they overlap the state reads, the fold and the LDS clear
     if (VEC)
     {
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
+        for (int u = 0; u < kHistUnroll; ++u)
         {
             const int64_t i = base + u * kBlock + threadIdx.x;
             a[u]            = nan4;
@@ -680,7 +687,7 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
         while (true)
         {
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
+            for (int u = 0; u < kHistUnroll; ++u)
             {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
@@ -690,7 +697,7 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
             if (base >= nvec)
                 break;
 #pragma unroll
-            for (int u = 0; u < kUnroll; ++u)
+            for (int u = 0; u < kHistUnroll; ++u)
             {
                 const int64_t i = base + u * kBlock + threadIdx.x;
                 a[u]            = nan4;
@@ -920,13 +927,13 @@ int static_scratch(float2** out)
     return MIQ_OK;
 }
 
-int stream_grid(int64_t n)
+int hist_grid(int64_t n)
 {
-    int64_t blocks = (n / 4 + (int64_t) kBlock * kUnroll - 1) / ((int64_t) kBlock * kUnroll);
+    int64_t blocks = (n / 4 + (int64_t) kBlock * kHistUnroll - 1) / ((int64_t) kBlock * kHistUnroll);
     if (blocks < 1)
         blocks = 1;
-    if (blocks > kMaxGrid)
-        blocks = kMaxGrid;
+    if (blocks > kHistMaxGrid)
+        blocks = kHistMaxGrid;
     return (int) blocks;
 }
 }   // namespace
@@ -1268,7 +1275,7 @@ int miq_analyzer_update_stats_f32(miq_analyzer* a, const float* data, int64_t n,
     if (int rc = ensure_reset(a, s))
         return rc;
     a->stats_updated = true;
-    const int grid    = stream_grid(n);
+    const int grid    = hist_grid(n);
     const int mm_grid = (int) std::max<int64_t>(
         1, std::min<int64_t>(kMmGrid, (n / 4 + (int64_t) kMmBlock * kMmUnroll - 1) / ((int64_t) kMmBlock * kMmUnroll)));
     if (a->mode == MIQ_QUANTIZATION_TF)
@@ -1307,7 +1314,7 @@ int miq_analyzer_update_stats_f32(miq_analyzer* a, const float* data, int64_t n,
     const dim3 hgrid((unsigned) hist_groups), hblock(kBlock);
     // workgroups [rem, groups) stream one tile fewer than the others (none at all when there are fewer tiles than
     // workgroups): the previous batch is folded by the first kFoldSlices of them
-    const int64_t tiles  = (n / 4 + (int64_t) kBlock * kUnroll - 1) / ((int64_t) kBlock * kUnroll);
+    const int64_t tiles  = (n / 4 + (int64_t) kBlock * kHistUnroll - 1) / ((int64_t) kBlock * kHistUnroll);
     const int fold_first = (int) std::min<int64_t>(tiles % hist_groups, hist_groups - kFoldSlices);
     if (a->range_known)
     {
