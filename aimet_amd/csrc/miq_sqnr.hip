@@ -36,6 +36,7 @@ constexpr int kMaxReplicas = 32;   // global copies of a histogram's counts that
 constexpr int kSpecReplicas     = 8;
 constexpr int kSpecLoads        = 2;
 constexpr int kSpecCopies       = 4;
+constexpr int kCompactFrom      = 64;   // histograms per search from which empty bins are skipped
 constexpr int64_t kSpecElems    = 32768;
 constexpr int64_t kSpecWideFrom = 65536;
 constexpr float kMinScale = 1.1920928955078125e-07f;   // torch.finfo(torch.float32).eps (EA:322)
@@ -965,10 +966,46 @@ __global__ __launch_bounds__(256) void sqnr_noise_kernel(const float* __restrict
         s_cnt[i] = hist[(int64_t) h * nb + i];
     }
     __syncthreads();
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // An empty bin adds an exact zero to every candidate's sum, so the bins that hold something are moved to the front
+    // and only those are walked (a channel of a weight leaves a third or more of 2048 bins empty: 11008 channels of
+    // 4096 samples search in 1.02 ms instead of 1.39 ms).  One wavefront does the moving, 5 us that a search over one
+    // or a few histograms does not get back, so those walk all bins.  Nor is it done for ranges so wide that a squared
+    // distance could overflow: there an empty bin contributes NaN, not zero, as in the tensor expression.
+    __shared__ int s_used;
+    if (a.num_hist < kCompactFrom)
+    {
+        if (threadIdx.x == 0)
+            s_used = nb;
+    }
+    else if (wave == 0)
+    {
+        const bool keep_all = !(fmaxf(fabsf(lo), fabsf(hi)) < 1e18f);
+        int used            = 0;
+        for (int first = 0; first < nb; first += 64)
+        {
+            const int i      = first + lane;
+            const float mid  = i < nb ? s_mid[i] : 0.0f;
+            const float cnt  = i < nb ? s_cnt[i] : 0.0f;
+            const bool keep  = i < nb && (keep_all || cnt != 0.0f);
+            const uint64_t m = __ballot(keep);
+            if (keep)
+            {
+                // (writes land at or below the lowest index this pass has read)
+                const int at = used + __popcll(m & ((1ull << lane) - 1ull));
+                s_mid[at]    = mid;
+                s_cnt[at]    = cnt;
+            }
+            used += __popcll(m);
+        }
+        if (lane == 0)
+            s_used = used;
+    }
+    __syncthreads();
+    const int used = s_used;
     float mn, mx;
     gated_minmax(minmax, h, a.num_steps, eps_steps, mn, mx);
     const int ncand = a.n_delta * a.n_offset;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int c_end = min(ncand, (int) (blockIdx.x + 1) * cand_per_block);
     for (int c = blockIdx.x * cand_per_block + wave; c < c_end; c += 4)
     {
@@ -979,10 +1016,10 @@ __global__ __launch_bounds__(256) void sqnr_noise_kernel(const float* __restrict
         // offset, or rounds to zero without one); delta is the wavefront's, so the choice is uniform
         const bool short_div =
             __builtin_amdgcn_readfirstlane((int) (fastdiv_divisor_ok(delta) &&
-                                                  fmaxf(fabsf(s_mid[0]), fabsf(s_mid[nb - 1])) <= kFastDivMaxDividend)) != 0;
+                                                  fmaxf(fabsf(lo), fabsf(hi)) <= kFastDivMaxDividend)) != 0;
         const float rcp = 1.0f / delta;
         double acc      = 0.0;
-        for (int i = lane; i < nb; i += 64)
+        for (int i = lane; i < used; i += 64)
         {
             const float mid = s_mid[i];
             float q         = rintf((short_div ? div_by_invariant(mid, delta, rcp) : mid / delta) - offset);

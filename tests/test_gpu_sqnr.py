@@ -195,6 +195,34 @@ def test_per_channel(ea):
         ea.SqnrEncodingAnalyzer((1, 4, 1, 1)).update_stats(x.cuda())     # shape does not broadcast to the input
 
 
+@pytest.mark.parametrize("symmetric", [False, True])
+def test_many_sparse_channels(ea, symmetric):
+    """96 channels of 300 samples: most of the 2048 bins of a channel are empty, and a search over this many histograms
+    walks only the bins that hold something.  Scores and choices against the restatement, which walks all bins."""
+    torch.manual_seed(11)
+    channels = 96
+    x = torch.randn(channels, 300) * torch.logspace(-2, 2, channels).view(-1, 1) + torch.linspace(-1, 1, channels).view(-1, 1)
+    x[5] = 0.0                                             # one histogram with a single occupied bin
+    an = ea.SqnrEncodingAnalyzer((channels, 1))
+    ref = sq.SqnrAnalyzer(channels, 2048)
+    an.update_stats(x.cuda())
+    ref.update_stats(x)
+    rmin, rmax, rnoise = ref.compute_encodings(255.0, symmetric)
+    st = an.observer.get_stats()
+    from aimet_amd import ops
+    gmin, gmax, gnoise, best = ops.v2_sqnr_search(st.hist, st.minmax, 255.0, symmetric, 3.0, 17, 101, 21,
+                                                  want_details=True)
+    assert (st.hist == 0).float().mean().item() > 0.8
+    assert torch.allclose(gnoise.cpu().float(), rnoise, rtol=1e-5, atol=0)
+    ref_best = torch.argmin(rnoise, dim=1)
+    agree = best.cpu().long() == ref_best
+    assert agree.float().mean().item() > 0.9
+    assert torch.equal(gmin.cpu()[agree], rmin[agree]) and torch.equal(gmax.cpu()[agree], rmax[agree])
+    for c in torch.nonzero(~agree).flatten().tolist():
+        # a near-tie resolved differently by the two summation orders: the scores must be indistinguishable
+        assert abs(rnoise[c, int(best[c])] - rnoise[c, int(ref_best[c])]) <= 2e-6 * rnoise[c, int(ref_best[c])]
+
+
 def test_reference_cases_through_the_analyzer(ea):
     # test_encoding_analyzer.py:659-674: equally spaced input, gamma = 1 -> the observed range exactly
     x = torch.arange(-100, 101) / 100
