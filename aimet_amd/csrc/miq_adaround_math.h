@@ -92,9 +92,11 @@ __device__ __forceinline__ float alpha_grad_f(float f, float gw, float alpha, fl
     {
         const float x   = 2.0f * h - 1.0f;
         const float ax  = fabsf(x);
-        reg             = 1.0f - pow01(ax, a.beta);
+        // one power for both: |x|^beta = |x|^(beta - 1) * |x| (a logarithm and an exponential less per element)
+        const float pm1 = (ax > 0.0f) ? pow01(ax, a.beta - 1.0f) : 0.0f;
+        reg             = 1.0f - pm1 * ax;
         const float sgn = (x > 0.0f) ? 1.0f : ((x < 0.0f) ? -1.0f : 0.0f);
-        const float dp  = (ax > 0.0f) ? a.beta * pow01(ax, a.beta - 1.0f) : 0.0f;
+        const float dp  = a.beta * pm1;
         grad += -a.reg_param * dp * sgn * 2.0f * dh;
     }
     return grad;
