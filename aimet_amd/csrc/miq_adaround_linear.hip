@@ -156,6 +156,8 @@ __device__ __forceinline__ int fwd_slot(int r, int chunk)
 //   producer / consumer roles, TK 256, producers two tiles ahead                                          27.0 us
 //   roles, TK 128: producers four / two / one tile ahead                                    26.0 / 23.4 / 22.9 us
 //   roles, TK 64, one tile ahead, two / four workgroups per CU                                     25.3 / 24.3 us
+//   roles, TK 128, two tiles ahead as straight-line code for exactly 8 tiles (the waits then count loads) 22.5 us,
+//       and 2 us slower than one ahead with float32 floor values: not kept
 // What a workgroup still has to compute when its last bytes arrive (a conversion, then a multiplication) is exposed at
 // the end of the kernel, and loads requested further ahead arrive in larger bunches: small tiles, one tile ahead.
 // Raising the producers' or the consumers' wavefront priority changed nothing or lost 1.5 us.
