@@ -1263,12 +1263,15 @@ int miq_v2_sqnr_search_f32(const float* hist, const float* minmax, int64_t num_h
     const int ncand = a.n_delta * a.n_offset;
     // MINIMUM_SCALE * num_steps is a Python float product, cast to float32 when added to the tensor
     const float eps_steps = (float) ((double) kMinScale * num_steps);
-    // few histograms: spread one histogram's candidates over many workgroups
-    int cand_per_block = num_hist >= 256 ? ncand : 8;
-    const int groups   = (ncand + cand_per_block - 1) / cand_per_block;
+    // few histograms: spread one histogram's candidates over many workgroups -- one candidate per wavefront while that
+    // keeps the grid within about a thousand workgroups
+    int64_t cand_per_block = (ncand * num_hist + 1023) / 1024;
+    cand_per_block         = (cand_per_block + 3) / 4 * 4;
+    cand_per_block         = cand_per_block > ncand ? ncand : cand_per_block;
+    const int groups   = (int) ((ncand + cand_per_block - 1) / cand_per_block);
     hipStream_t s      = (hipStream_t) stream;
     hipLaunchKernelGGL(sqnr_noise_kernel, dim3(groups, (unsigned) num_hist), dim3(256), 0, s, hist, minmax, a, eps_steps,
-                       cand_per_block, noise);
+                       (int) cand_per_block, noise);
     MIQ_CHECK_LAUNCH();
     hipLaunchKernelGGL(sqnr_pick_kernel, dim3((unsigned) num_hist), dim3(64), 0, s, noise, minmax, a, eps_steps, out_min,
                        out_max, best_index);
