@@ -144,6 +144,17 @@ def test_per_channel_updates_where_some_ranges_grow(ea):
         st = obs.get_stats()
         for i in range(5):
             _same_hist(st[i], ref.stats[i])
+    # rows long enough for the wide workgroups, a length that is and one that is not a multiple of the vector width
+    for length in (262144, 200003):
+        obs = ea._HistogramObserver((3, 1), 2048)
+        ref = sq.SqnrAnalyzer(3, 2048)
+        for sc in ([1.0, 1.0, 1.0], [0.5, 2.0, 0.7], [0.3, 0.3, 3.0], [1.0, 1.0, 1.0]):
+            x = torch.randn(3, length) * torch.tensor(sc).view(3, 1)
+            obs.merge_stats(None, x.cuda())
+            ref.update_stats(x)
+            st = obs.get_stats()
+            for i in range(3):
+                _same_hist(st[i], ref.stats[i])
 
 
 @pytest.mark.parametrize("symmetric", [False, True])
