@@ -1,43 +1,32 @@
-"""What a float quantizer's get_encoding() returns (aimet_torch/v2/quantization/float/encoding.py:48-125)."""
+"""What a float quantizer's get_encoding() returns: the format and, when statistics set it, the largest representable
+value (interface of aimet_torch/v2/quantization/float/encoding.py:48-125)."""
+import dataclasses
 from typing import Optional
 
 import torch
 
 
+@dataclasses.dataclass(frozen=True)
 class FloatEncoding:
-    """Mantissa bits, exponent bits and the largest representable value (None: the format's own)."""
-
-    def __init__(self, mantissa_bits: int, exponent_bits: int, maxval: Optional[torch.Tensor]):
-        self._mantissa_bits = mantissa_bits
-        self._exponent_bits = exponent_bits
-        self._maxval = maxval
-
-    mapping = "float"
-
-    @property
-    def mantissa_bits(self) -> int:
-        return self._mantissa_bits
-
-    @property
-    def exponent_bits(self) -> int:
-        return self._exponent_bits
-
-    @property
-    def maxval(self) -> Optional[torch.Tensor]:
-        return self._maxval
+    """Immutable record; `maxval` is None when the format's own largest value applies."""
+    mantissa_bits: int
+    exponent_bits: int
+    maxval: Optional[torch.Tensor] = None
+    mapping: str = dataclasses.field(default="float", init=False)
 
     @property
     def bitwidth(self) -> int:
-        return self._mantissa_bits + self._exponent_bits + 1
+        """sign + exponent + mantissa"""
+        return 1 + self.exponent_bits + self.mantissa_bits
 
     @property
     def granularity(self) -> str:
-        if self._maxval is None or self._maxval.numel() == 1:
-            return "pertensor"
-        if sum(1 for d in self._maxval.shape if d > 1) == 1:
-            return "perchannel"
-        return "unknown"
+        """'pertensor', 'perchannel' (maxval varies along exactly one axis) or 'unknown'"""
+        varying = 0 if self.maxval is None else sum(size > 1 for size in self.maxval.shape)
+        return ("pertensor", "perchannel")[varying] if varying < 2 else "unknown"
 
-    def to(self, *args, **kwargs):
-        maxval = None if self._maxval is None else self._maxval.to(*args, **kwargs)
-        return type(self)(self._mantissa_bits, self._exponent_bits, maxval)
+    def to(self, *args, **kwargs) -> "FloatEncoding":
+        """The same encoding with maxval moved / cast as torch.Tensor.to would."""
+        if self.maxval is None:
+            return self
+        return dataclasses.replace(self, maxval=self.maxval.to(*args, **kwargs))
