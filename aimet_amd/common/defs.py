@@ -1,25 +1,18 @@
 """Quantization scheme / data type enums and the scheme->analyzer maps
 (TrainingExtensions/common/src/python/aimet_common/defs.py:47-84, 302-315)."""
-from enum import Enum
+import enum
 
 from . import libpymo
 
+# Same member names and values as the reference's enumerations (members are numbered in the order listed).
+QuantScheme = enum.Enum('QuantScheme', ['post_training_tf', 'post_training_tf_enhanced',
+                                        'training_range_learning_with_tf_init',
+                                        'training_range_learning_with_tf_enhanced_init', 'training_range_learning',
+                                        'post_training_percentile'], start=1, module=__name__)
+QuantScheme.__doc__ = "How encodings are found: post-training calibration schemes and range-learning initialisations."
 
-class QuantScheme(Enum):
-    """Enumeration of quant schemes (same names and values as the reference)."""
-    post_training_tf = 1
-    post_training_tf_enhanced = 2
-    training_range_learning_with_tf_init = 3
-    training_range_learning_with_tf_enhanced_init = 4
-    training_range_learning = 5
-    post_training_percentile = 6
-
-
-class QuantizationDataType(Enum):
-    """Tensor quantizer data types."""
-    undefined = 0
-    int = 1
-    float = 2
+QuantizationDataType = enum.Enum('QuantizationDataType', ['undefined', 'int', 'float'], start=0, module=__name__)
+QuantizationDataType.__doc__ = "Grid of a tensor quantizer: integer (affine) or float."
 
 
 MAP_QUANT_SCHEME_TO_PYMO = {
@@ -35,6 +28,5 @@ MAP_ROUND_MODE_TO_PYMO = {'nearest': libpymo.RoundingMode.ROUND_NEAREST,
 
 
 class AdaroundConstants:
-    """Constants of the rectified sigmoid used by AdaRound."""
-    GAMMA = -0.1
-    ZETA = 1.1
+    """Stretch of AdaRound's rectified sigmoid: h = clamp(sigmoid(alpha) * (ZETA - GAMMA) + GAMMA, 0, 1)."""
+    GAMMA, ZETA = -0.1, 1.1

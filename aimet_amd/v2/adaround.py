@@ -9,6 +9,8 @@ delta / offset come from the weight quantizer's scale / offset and a signed quan
 """
 import contextlib
 import itertools
+import json
+import os
 from typing import Tuple, Union
 
 import torch
@@ -23,14 +25,24 @@ from .quantization.affine.quantizer import MinMaxQuantizer
 from .quantsim import QuantizationSimModel
 
 
+def _quantized_modules(root: nn.Module):
+    """Every v2 quantized module below (and including) `root`."""
+    return (m for m in root.modules() if isinstance(m, BaseQuantizationMixin))
+
+
 class AdaroundWrapper(V1AdaroundWrapper):
-    """AdaRound wrapper of a v2 quantized module."""
+    """AdaRound wrapper of a v2 quantized module: the grid comes from the weight quantizer's scale / offset."""
 
     def __init__(self, module: BaseQuantizationMixin):  # pylint: disable=super-init-not-called
         torch.nn.Module.__init__(self)
         assert self.weight_name in module.param_quantizers
         self.module_to_wrap = module
         self._init_param()
+
+    # the weight quantizer of the wrapped module, wherever a hook below needs it
+    @property
+    def _weight_quantizer(self):
+        return self.module_to_wrap.param_quantizers[self.weight_name]
 
     def forward(self, *args, **kwargs):
         """Runs the quantized module with its weight replaced by the adarounded weight."""
@@ -47,44 +59,41 @@ class AdaroundWrapper(V1AdaroundWrapper):
 
     @contextlib.contextmanager
     def _disable_weight_quantizer(self):
-        weight_quantizer = self.module_to_wrap.param_quantizers[self.weight_name]
-        self.module_to_wrap.param_quantizers[self.weight_name] = None
+        slots, parked = self.module_to_wrap.param_quantizers, self._weight_quantizer
+        slots[self.weight_name] = None
         try:
             yield
         finally:
-            self.module_to_wrap.param_quantizers[self.weight_name] = weight_quantizer
+            slots[self.weight_name] = parked
 
     def _is_weight_quantizer_enabled(self) -> bool:
-        return bool(self.module_to_wrap.param_quantizers[self.weight_name])
+        return self._weight_quantizer is not None
 
     def get_original_module(self) -> torch.nn.Module:
+        """The quantized module itself: there is no separate wrapped module in v2."""
         return self.module_to_wrap
 
     def _get_weight_quantizer_channel_axis(self) -> int:
-        quantizer = self.module_to_wrap.param_quantizers[self.weight_name]
-        shape = quantizer.shape
-        padded = (1,) * (self.weight.dim() - len(shape)) + tuple(shape)
-        for idx, dim in enumerate(padded):
-            if dim != 1:
-                return idx
-        return 0
+        # the quantizer's shape broadcasts against the weight from the right; the first axis along which it has more
+        # than one entry is the channel axis (0 for a per-tensor quantizer)
+        lead = self.weight.dim() - len(self._weight_quantizer.shape)
+        return next((lead + axis for axis, size in enumerate(self._weight_quantizer.shape) if size != 1), 0)
 
     def _get_weight_quantizer_delta_and_offset(self) -> Tuple[torch.Tensor, torch.Tensor]:
-        quantizer = self.module_to_wrap.param_quantizers[self.weight_name]
         with torch.no_grad():
-            scale = quantizer.get_scale().detach().to(torch.float32).reshape(-1)
-            offset = quantizer.get_offset().detach().to(torch.float32).reshape(-1)
-        return scale, offset
+            flat = [t.detach().to(torch.float32).reshape(-1)
+                    for t in (self._weight_quantizer.get_scale(), self._weight_quantizer.get_offset())]
+        return flat[0], flat[1]
 
     def _get_weight_quantizer_bitwidth(self) -> int:
-        return self.module_to_wrap.param_quantizers[self.weight_name].bitwidth
+        return self._weight_quantizer.bitwidth
 
     def _init_param(self):
         super()._init_param()
-        quantizer = self.module_to_wrap.param_quantizers[self.weight_name]
-        if quantizer.signed:
-            self.clip_max = 2 ** (self.bitwidth - 1) - 1
-            self.clip_min = - 2 ** (self.bitwidth - 1)
+        if self._weight_quantizer.signed:
+            # signed integer grid [-2^(bw-1), 2^(bw-1) - 1] instead of v1's [0, 2^bw - 1]
+            half = 2 ** (self.bitwidth - 1)
+            self.clip_min, self.clip_max = -half, half - 1
 
 
 class AdaroundParameters(V1AdaroundParameters):
@@ -97,8 +106,8 @@ class Adaround(V1Adaround):
     @staticmethod
     def _get_quantsim(model: nn.Module, dummy_input, quant_scheme: QuantScheme, default_param_bw: int,
                       config_file: str):
-        return QuantizationSimModel(model, dummy_input=dummy_input, quant_scheme=quant_scheme,
-                                    default_param_bw=default_param_bw, config_file=config_file)
+        return QuantizationSimModel(model, dummy_input, quant_scheme, default_param_bw=default_param_bw,
+                                    config_file=config_file)
 
     @staticmethod
     def _get_adaround_wrapper(quant_module: BaseQuantizationMixin):
@@ -106,53 +115,47 @@ class Adaround(V1Adaround):
 
     @classmethod
     def _remove_quantization_wrappers(cls, module: nn.Module):
-        for module_name, module_ref in module.named_children():
-            if isinstance(module_ref, BaseQuantizationMixin):
-                setattr(module, module_name, module_ref.get_original_module())
-            else:
-                cls._remove_quantization_wrappers(module_ref)
+        for child_name, child in list(module.named_children()):
+            if not isinstance(child, BaseQuantizationMixin):
+                cls._remove_quantization_wrappers(child)
+                continue
+            setattr(module, child_name, child.get_original_module())
 
     @staticmethod
     def _get_quant_wrapper(quant_sim_model: nn.Module, module_name: str) -> Union[BaseQuantizationMixin, None]:
-        for name, module in quant_sim_model.named_modules():
-            if name == module_name and isinstance(module, BaseQuantizationMixin):
-                return module
-        return None
+        found = dict(quant_sim_model.named_modules()).get(module_name)
+        return found if isinstance(found, BaseQuantizationMixin) else None
 
     @staticmethod
     def _compute_param_encodings(quant_sim: QuantizationSimModel):
-        for quant_module in quant_sim.model.modules():
-            if isinstance(quant_module, BaseQuantizationMixin):
-                # AdaRound requires input and output quantizers to be disabled
-                quant_module.input_quantizers = nn.ModuleList([None for _ in quant_module.input_quantizers])
-                quant_module.output_quantizers = nn.ModuleList([None for _ in quant_module.output_quantizers])
-                for name, param_quantizer in quant_module.param_quantizers.items():
-                    if not param_quantizer:
-                        continue
-                    with param_quantizer.compute_encodings():
-                        _ = param_quantizer(getattr(quant_module, name))
+        for quantized in _quantized_modules(quant_sim.model):
+            # only parameters are quantized while AdaRound runs: activation quantizers are taken out
+            quantized.input_quantizers = nn.ModuleList([None] * len(quantized.input_quantizers))
+            quantized.output_quantizers = nn.ModuleList([None] * len(quantized.output_quantizers))
+            for param_name, quantizer in quantized.param_quantizers.items():
+                if quantizer is not None:
+                    with quantizer.compute_encodings():
+                        quantizer(getattr(quantized, param_name))
 
     @staticmethod
     def _validate_quant_module_for_adaround(quant_module: BaseQuantizationMixin):
-        assert quant_module.param_quantizers['weight'], '%s does not have weight parameter.' % quant_module
-        assert quant_module.param_quantizers['weight'].is_initialized(), '%s encoding needs to be set.' % quant_module
+        weight_quantizer = quant_module.param_quantizers['weight']
+        assert weight_quantizer, f'{quant_module} does not have weight parameter.'
+        assert weight_quantizer.is_initialized(), f'{quant_module} encoding needs to be set.'
 
     @staticmethod
     def _check_input_output_quantizers_for_adaround(quant_model: nn.Module):
-        for module in quant_model.modules():
-            if isinstance(module, BaseQuantizationMixin):
-                for quantizer in itertools.chain(module.input_quantizers, module.output_quantizers):
-                    assert quantizer is None
+        leftover = [q for m in _quantized_modules(quant_model)
+                    for q in itertools.chain(m.input_quantizers, m.output_quantizers) if q is not None]
+        assert not leftover
 
     @staticmethod
     def _get_lowest_weight_bw(quant_model: nn.Module):
-        return min(quantizer.bitwidth for module in quant_model.modules() if isinstance(module, BaseQuantizationMixin)
+        return min(quantizer.bitwidth for module in _quantized_modules(quant_model)
                    for quantizer in module.param_quantizers.values() if isinstance(quantizer, MinMaxQuantizer))
 
     @classmethod
     def _export_encodings_to_json(cls, path: str, filename_prefix: str, quant_sim: QuantizationSimModel):
-        import json
-        import os
         param_encodings = {}
         for name, quant_module in quant_sim.model.named_modules():
             if isinstance(quant_module, BaseQuantizationMixin) and isinstance(quant_module, AdaroundSupportedModules):
