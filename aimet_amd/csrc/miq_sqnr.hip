@@ -467,6 +467,183 @@ __device__ void rebin_running_histogram(float* __restrict__ upd, const float* __
     __syncthreads();
 }
 
+// ---- one workgroup per histogram ------------------------------------------------------------------------------
+// grid (H), 256 threads.  When a row goes to a single workgroup (many histograms, or short rows: the weight of a layer
+// with one histogram per output channel) the whole update is one launch and touches no workspace: the workgroup finds
+// the row's finite min / max, derives the ranges, bins the row over the merged range into LDS, re-bins the running
+// histogram if the range grew and writes the new running histogram.  Rows of up to 6144 elements stay in registers
+// between the two passes; longer ones are read again (from the L2).  Serves the first batch (has_stats = 0) as well.
+// BATCH: the batch's own histogram (over the batch's range) is written as well; with running statistics that is a
+// second LDS histogram, counted in the same pass.
+constexpr int kRowKeep = 6;   // 16-byte groups a lane keeps
+template <bool BATCH>
+__global__ __launch_bounds__(kHistBlock) void row_update_kernel(const float* __restrict__ x, int64_t n_per_hist,
+                                                                int num_bins, int has_stats,
+                                                                float* __restrict__ state_hist,
+                                                                float* __restrict__ state_minmax,
+                                                                float* __restrict__ batch_hist,
+                                                                float* __restrict__ batch_minmax,
+                                                                int* __restrict__ bad_flag, int vec)
+{
+    constexpr int kRowCopies = BATCH ? 2 : 4;   // [kinds][num_bins][copies] words stay within 32 KiB at 2048 bins
+    extern __shared__ uint32_t lds[];
+    __shared__ float upd[kMaxBins];
+    __shared__ float s_mm[2][kHistBlock / 64];
+    const int h        = blockIdx.x;
+    const float* row   = x + (int64_t) h * n_per_hist;
+    const v4f* rv      = reinterpret_cast<const v4f*>(row);
+    const int64_t nvec = n_per_hist / 4;
+    const bool kept    = vec && nvec <= (int64_t) kRowKeep * kHistBlock;
+    v4f keep[kRowKeep];
+    float lo = INFINITY, hi = -INFINITY;
+    auto look = [&](float v) {
+        if (fabsf(v) < INFINITY)   // false for NaN and +-inf
+        {
+            lo = fminf(lo, v);
+            hi = fmaxf(hi, v);
+        }
+    };
+    if (kept)
+    {
+#pragma unroll
+        for (int u = 0; u < kRowKeep; ++u)
+        {
+            const int64_t i = u * kHistBlock + threadIdx.x;
+            keep[u]         = i < nvec ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
+        }
+    }
+    const bool two = BATCH && has_stats;   // two histograms: batch range and merged range
+    for (int i = threadIdx.x; i < (two ? 2 : 1) * num_bins * kRowCopies; i += kHistBlock)
+        lds[i] = 0;
+    if (kept)
+    {
+#pragma unroll
+        for (int u = 0; u < kRowKeep; ++u)
+        {
+            look(keep[u][0]);
+            look(keep[u][1]);
+            look(keep[u][2]);
+            look(keep[u][3]);
+        }
+    }
+    else if (vec)
+    {
+        for (int64_t i = threadIdx.x; i < nvec; i += kHistBlock)
+        {
+            const v4f a = rv[i];
+            look(a[0]);
+            look(a[1]);
+            look(a[2]);
+            look(a[3]);
+        }
+    }
+    else
+    {
+        for (int64_t i = threadIdx.x; i < n_per_hist; i += kHistBlock)
+            look(row[i]);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        lo = fminf(lo, __shfl_xor(lo, o));
+        hi = fmaxf(hi, __shfl_xor(hi, o));
+    }
+    if ((threadIdx.x & 63) == 0)
+    {
+        s_mm[0][threadIdx.x >> 6] = lo;
+        s_mm[1][threadIdx.x >> 6] = hi;
+    }
+    __syncthreads();   // also: the LDS histogram is clear
+    for (int k = 0; k < kHistBlock / 64; ++k)
+    {
+        lo = fminf(lo, s_mm[0][k]);
+        hi = fmaxf(hi, s_mm[1][k]);
+    }
+    bool ok;
+    const Ranges r = compute_ranges(lo, hi, num_bins, has_stats, state_minmax, h, ok);
+    if (threadIdx.x == 0)
+    {
+        if (batch_minmax)
+        {
+            batch_minmax[2 * h]     = r.batch_min;
+            batch_minmax[2 * h + 1] = r.batch_max;
+        }
+        if (!ok)
+            atomicOr(bad_flag, 1);
+    }
+    Binner mb, bb;
+    mb.init(r.m_lo, r.m_hi, num_bins);
+    bb.init(r.b_lo, r.b_hi, num_bins);
+    uint32_t* lm = lds + (threadIdx.x & (kRowCopies - 1));   // merged range (= batch range without statistics)
+    uint32_t* lb = lm + num_bins * kRowCopies;               // batch range, when both are counted
+    auto count = [&](float v) {
+        if (v == v)
+        {
+            atomicAdd(&lm[mb.bin(v) * kRowCopies], 1u);
+            if (two)
+                atomicAdd(&lb[bb.bin(v) * kRowCopies], 1u);
+        }
+    };
+    if (kept)
+    {
+#pragma unroll
+        for (int u = 0; u < kRowKeep; ++u)
+        {
+            count(keep[u][0]);
+            count(keep[u][1]);
+            count(keep[u][2]);
+            count(keep[u][3]);
+        }
+    }
+    else if (vec)
+    {
+        for (int64_t i = threadIdx.x; i < nvec; i += kHistBlock)
+        {
+            const v4f a = rv[i];
+            count(a[0]);
+            count(a[1]);
+            count(a[2]);
+            count(a[3]);
+        }
+    }
+    else
+    {
+        for (int64_t i = threadIdx.x; i < n_per_hist; i += kHistBlock)
+            count(row[i]);
+    }
+    __syncthreads();
+    float* sh          = state_hist + (int64_t) h * num_bins;
+    const bool rebins  = has_stats && r.rebin;
+    if (rebins)
+        rebin_running_histogram(upd, sh, r, num_bins);   // ends with a barrier
+    for (int i = threadIdx.x; i < num_bins; i += kHistBlock)
+    {
+        uint32_t total = 0;
+#pragma unroll
+        for (int c = 0; c < kRowCopies; ++c)
+            total += lds[i * kRowCopies + c];
+        const float before = !has_stats ? 0.0f : (rebins ? upd[i] : sh[i]);
+        sh[i]              = (float) total + before;
+        if (BATCH)
+        {
+            uint32_t own = total;
+            if (two)
+            {
+                own = 0;
+#pragma unroll
+                for (int c = 0; c < kRowCopies; ++c)
+                    own += lds[(num_bins + i) * kRowCopies + c];
+            }
+            batch_hist[(int64_t) h * num_bins + i] = (float) own;
+        }
+    }
+    if (threadIdx.x == 0)
+    {
+        state_minmax[2 * h]     = r.new_min;
+        state_minmax[2 * h + 1] = r.new_max;
+    }
+}
+
 // min / max of a number and a value that is a number or a quiet NaN: the number when the other is NaN.  One
 // instruction each; fminf / fmaxf first pass both operands through a canonicalising max, which triples the count in
 // a loop that is short on issue slots.
@@ -1167,6 +1344,8 @@ int64_t miq_v2_hist_workspace_bytes(int64_t num_hist, int64_t n_per_hist, int nu
     // count replicas (two histograms each) + per-workgroup (min, max) + the per-histogram ranges + the ticket counters of
     // the speculative update's second launch
     const int64_t groups = (blocks + kTicketGroup - 1) / kTicketGroup;
+    if (blocks == 1)   // a row per workgroup: nothing is kept outside LDS
+        return 512;
     return num_hist * replicas * 2 * (int64_t) num_bins * 4 + num_hist * blocks * 2 * 4 +
            num_hist * (int64_t) sizeof(Ranges) + num_hist * 4 +
            (groups > 1 ? num_hist * groups * kTicketStride * 4 : 0) + 512;
@@ -1204,6 +1383,21 @@ int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hi
     const int64_t groups  = (blocks + kTicketGroup - 1) / kTicketGroup;
     uint32_t* group_words = (uint32_t*) (((uintptr_t) (words + num_hist) + 127) & ~(uintptr_t) 127);
     const Tickets tickets = {words, groups > 1 ? group_words : nullptr};
+    if (blocks == 1)
+    {
+        // a row per workgroup: the whole update in one launch ([kinds][bins][copies] LDS words, kinds * copies = 4)
+        const size_t lds_bytes = (size_t) num_bins * 4 * sizeof(uint32_t);
+        if (want_batch_hist)
+            hipLaunchKernelGGL(row_update_kernel<true>, dim3((unsigned) num_hist), dim3(kHistBlock), lds_bytes, s, data,
+                               n_per_hist, num_bins, has_stats, state_hist, state_minmax, batch_hist, batch_minmax,
+                               bad_flag, vec);
+        else
+            hipLaunchKernelGGL(row_update_kernel<false>, dim3((unsigned) num_hist), dim3(kHistBlock), lds_bytes, s, data,
+                               n_per_hist, num_bins, has_stats, state_hist, state_minmax, batch_hist, batch_minmax,
+                               bad_flag, vec);
+        MIQ_CHECK_LAUNCH();
+        return MIQ_OK;
+    }
     if (has_stats && !want_batch_hist)
     {
         // speculative update: one pass when the statistics' range holds

@@ -647,11 +647,27 @@ def bench_sqnr(torch, ops, reps=5):
     acc = sum(acc_ms) / len(acc_ms)
     srch = sum(search_ms) / len(search_ms)
     elems = 16 * n
+    # per output channel of the [11008, 4096] weight: one 2048-bin histogram per row, then the symmetric 8-bit search
+    w = _laplace_weights(torch, (11008, 4096), 1004, dev)
+    first, later, search = [], [], []
+    for r in range(3):
+        chan = SqnrEncodingAnalyzer((11008, 1))
+        t = []
+        for step in (lambda: chan.update_stats(w), lambda: chan.update_stats(w),
+                     lambda: chan.compute_encodings(255.0, True)):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            step()
+            torch.cuda.synchronize()
+            t.append((time.perf_counter() - t0) * 1e3)
+        first.append(t[0]), later.append(t[1]), search.append(t[2])
     # two passes over each batch: 8 B/element
     return {"elements": elems, "num_bins": 2048, "accumulate_ms": acc, "search_ms": srch,
             "elements_per_s": elems / ((acc + srch) / 1e3), "accumulate_GBps": 8.0 * elems / acc / 1e6,
             "accumulate_frac_hbm": 8.0 * elems / acc / 1e6 / HBM_PEAK_GBPS,
-            "encoding": [float(mn), float(mx)]}
+            "encoding": [float(mn), float(mx)],
+            "per_channel_11008x4096": {"first_update_ms": min(first), "later_update_ms": min(later),
+                                       "search_ms": min(search), "timing": "wall clock around one call"}}
 
 
 def bench_v2_range_learning(torch, ops, steps=50):

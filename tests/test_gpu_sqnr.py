@@ -206,6 +206,29 @@ def test_per_channel(ea):
         ea.SqnrEncodingAnalyzer((1, 4, 1, 1)).update_stats(x.cuda())     # shape does not broadcast to the input
 
 
+@pytest.mark.parametrize("length", [1500, 6144, 7004, 7001])
+def test_many_rows_one_workgroup_each(ea, length):
+    """More than a thousand histograms per update: each row goes to one workgroup that does the whole update (rows that
+    fit its registers, rows it reads twice, a length that is not a multiple of the vector width), first batch, batches
+    inside the range and batches that grow some rows' ranges, rows with non-finite values."""
+    torch.manual_seed(23)
+    rows = 1100
+    obs = ea._HistogramObserver((rows, 1), 2048)
+    grow = torch.ones(rows, 1)
+    grow[::7] = 3.0
+    sample = sorted(set(list(range(0, rows, 97)) + [3, 7, rows - 1]))   # the restatement follows these rows only
+    ref = sq.SqnrAnalyzer(len(sample), 2048)
+    for k, sc in enumerate((1.0, 0.5, grow, 0.8)):
+        x = torch.randn(rows, length) * sc
+        if k == 1:
+            x[3, :3] = torch.tensor([float('nan'), float('inf'), -float('inf')])
+        obs.merge_stats(None, x.cuda())
+        ref.update_stats(x[sample])
+        st = obs.get_stats()
+        for at, i in enumerate(sample):
+            _same_hist(st[i], ref.stats[at])
+
+
 @pytest.mark.parametrize("symmetric", [False, True])
 def test_many_sparse_channels(ea, symmetric):
     """96 channels of 300 samples: most of the 2048 bins of a channel are empty, and a search over this many histograms
