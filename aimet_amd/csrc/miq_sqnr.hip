@@ -475,7 +475,8 @@ __device__ void rebin_running_histogram(float* __restrict__ upd, const float* __
 // between the two passes; longer ones are read again (from the L2).  Serves the first batch (has_stats = 0) as well.
 // BATCH: the batch's own histogram (over the batch's range) is written as well; with running statistics that is a
 // second LDS histogram, counted in the same pass.
-constexpr int kRowKeep = 6;   // 16-byte groups a lane keeps
+constexpr int kRowKeep    = 6;      // 16-byte groups a lane keeps
+constexpr int kRowBinsMax = 2048;   // 32 KiB of counts + 16 KiB for re-binning: within the 64 KiB of LDS a launch may ask for
 template <bool BATCH>
 __global__ __launch_bounds__(kHistBlock) void row_update_kernel(const float* __restrict__ x, int64_t n_per_hist,
                                                                 int num_bins, int has_stats,
@@ -1344,7 +1345,7 @@ int64_t miq_v2_hist_workspace_bytes(int64_t num_hist, int64_t n_per_hist, int nu
     // count replicas (two histograms each) + per-workgroup (min, max) + the per-histogram ranges + the ticket counters of
     // the speculative update's second launch
     const int64_t groups = (blocks + kTicketGroup - 1) / kTicketGroup;
-    if (blocks == 1)   // a row per workgroup: nothing is kept outside LDS
+    if (blocks == 1 && num_bins <= kRowBinsMax)   // a row per workgroup: nothing is kept outside LDS
         return 512;
     return num_hist * replicas * 2 * (int64_t) num_bins * 4 + num_hist * blocks * 2 * 4 +
            num_hist * (int64_t) sizeof(Ranges) + num_hist * 4 +
@@ -1383,7 +1384,7 @@ int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hi
     const int64_t groups  = (blocks + kTicketGroup - 1) / kTicketGroup;
     uint32_t* group_words = (uint32_t*) (((uintptr_t) (words + num_hist) + 127) & ~(uintptr_t) 127);
     const Tickets tickets = {words, groups > 1 ? group_words : nullptr};
-    if (blocks == 1)
+    if (blocks == 1 && num_bins <= kRowBinsMax)
     {
         // a row per workgroup: the whole update in one launch ([kinds][bins][copies] LDS words, kinds * copies = 4)
         const size_t lds_bytes = (size_t) num_bins * 4 * sizeof(uint32_t);

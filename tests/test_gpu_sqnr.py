@@ -206,6 +206,22 @@ def test_per_channel(ea):
         ea.SqnrEncodingAnalyzer((1, 4, 1, 1)).update_stats(x.cuda())     # shape does not broadcast to the input
 
 
+@pytest.mark.parametrize("num_bins", [4096, 2048, 64])
+def test_short_rows_at_several_bin_counts(ea, num_bins):
+    """Six short rows per update at the largest bin count the library takes (the general kernels), the default one
+    and a small one (one launch per update)."""
+    torch.manual_seed(24)
+    obs = ea._HistogramObserver((6, 1), num_bins)
+    ref = sq.SqnrAnalyzer(6, num_bins)
+    for sc in (1.0, 0.4, 2.5, 1.0):
+        x = torch.randn(6, 1500) * sc
+        obs.merge_stats(None, x.cuda())
+        ref.update_stats(x)
+        st = obs.get_stats()
+        for i in range(6):
+            _same_hist(st[i], ref.stats[i])
+
+
 @pytest.mark.parametrize("length", [1500, 6144, 7004, 7001])
 def test_many_rows_one_workgroup_each(ea, length):
     """More than a thousand histograms per update: each row goes to one workgroup that does the whole update (rows that
