@@ -459,7 +459,9 @@ int64_t miq_v2_hist_workspace_bytes(int64_t num_hist, int64_t n_per_hist, int nu
  * is still written): only callers that quantize dynamically with the batch's statistics read it.
  * has_stats = 1, want_batch_hist = 0 (the calibration loop) enqueues two kernels and reads the batch once as long as
  * the batch stays inside the statistics' range (twice when it does not); the other modes enqueue three kernels and
- * read it twice.  Never synchronises. */
+ * read it twice.  Shapes that give every histogram to one workgroup (a thousand histograms or more, or slabs of up
+ * to 6144 elements, at up to 2048 bins) take one kernel in every mode and leave the workspace untouched.
+ * Never synchronises. */
 int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hist, int num_bins, int has_stats,
                            int want_batch_hist, float* state_hist, float* state_minmax, float* batch_hist,
                            float* batch_minmax, int32_t* bad_flag, void* workspace, void* stream);
