@@ -58,6 +58,7 @@ struct ChanState
     double* pdf;        // [C][512]
     uint32_t* counts;   // [C][512]   counts of the batch in flight (multi-workgroup channels only); zero when idle
     float* minmax;      // [2 C]      per-channel (min, max) of the batch in flight
+    miq_encoding* enc;  // [C]        what the last search found, in the layout the caller's array has
 };
 
 size_t align_up(size_t v)
@@ -67,7 +68,7 @@ size_t align_up(size_t v)
 size_t state_bytes(int64_t c)
 {
     return align_up(sizeof(ChanHead) * c) + align_up(sizeof(double) * kPdf * c) + align_up(sizeof(uint32_t) * kPdf * c) +
-           align_up(sizeof(float) * 2 * c);
+           align_up(sizeof(float) * 2 * c) + align_up(sizeof(miq_encoding) * c);
 }
 ChanState carve(void* base, int64_t c)
 {
@@ -80,6 +81,8 @@ ChanState carve(void* base, int64_t c)
     s.counts = reinterpret_cast<uint32_t*>(p);
     p += align_up(sizeof(uint32_t) * kPdf * c);
     s.minmax = reinterpret_cast<float*>(p);
+    p += align_up(sizeof(float) * 2 * c);
+    s.enc = reinterpret_cast<miq_encoding*>(p);
     return s;
 }
 
@@ -250,6 +253,7 @@ __global__ __launch_bounds__(kSearchBlockMax) void chan_search_kernel(ChanState 
                 tfe::encoding_of_zeros(a, enc);
             h.enc_min = enc[0], h.enc_max = enc[1], h.enc_delta = enc[2], h.enc_offset = enc[3];
             h.enc_bw = h.stats_updated ? a.bw : 0;
+            s.enc[c] = miq_encoding{enc[0], enc[1], enc[2], enc[3], h.enc_bw};
         }
         return;
     }
@@ -311,6 +315,7 @@ __global__ __launch_bounds__(kSearchBlockMax) void chan_search_kernel(ChanState 
         tfe::encoding_of(a, bdelta, boffset, enc);
         h.enc_min = enc[0], h.enc_max = enc[1], h.enc_delta = enc[2], h.enc_offset = enc[3];
         h.enc_bw = a.bw;
+        s.enc[c] = miq_encoding{enc[0], enc[1], enc[2], enc[3], a.bw};
     }
 }
 }   // namespace
@@ -467,13 +472,16 @@ int miq_channel_analyzer_compute_encodings(miq_channel_analyzer* a, int bw, int 
     MIQ_CHECK_ARG(bw >= 1 && bw <= 32, "bitwidth must be in [1, 32] (got %d)", bw);
     hipStream_t s   = (hipStream_t) stream;
     const int64_t c = a->num_channel;
-    memset(out, 0, sizeof(miq_encoding) * c);
     *is_valid = a->stats_updated ? 1 : 0;
     if (!a->stats_updated)
+    {
+        memset(out, 0, sizeof(miq_encoding) * c);
         return MIQ_OK;
-    std::vector<ChanHead> heads(c);
+    }
     if (a->mode == MIQ_QUANTIZATION_PERCENTILE)
     {
+        memset(out, 0, sizeof(miq_encoding) * c);
+        std::vector<ChanHead> heads(c);
         // PercentileEncodingAnalyzer::computeEncoding is 512 buckets of host arithmetic per channel: read the PDFs back
         std::vector<double> pdf((size_t) c * kPdf), x_left(kPdf);
         MIQ_CHECK_HIP(hipMemcpyAsync(heads.data(), a->st.head, sizeof(ChanHead) * c, hipMemcpyDeviceToHost, s));
@@ -496,16 +504,9 @@ int miq_channel_analyzer_compute_encodings(miq_channel_analyzer* a, int bw, int 
     const int search_block = std::min(kSearchBlockMax, 64 * ((sa.n_cand + 63) / 64));
     hipLaunchKernelGGL(chan_search_kernel, dim3((unsigned) c), dim3(search_block), 0, s, a->st, sa);
     MIQ_CHECK_LAUNCH();
-    MIQ_CHECK_HIP(hipMemcpyAsync(heads.data(), a->st.head, sizeof(ChanHead) * c, hipMemcpyDeviceToHost, s));
+    // the kernel leaves the encodings in the caller's layout: one copy straight into `out`
+    MIQ_CHECK_HIP(hipMemcpyAsync(out, a->st.enc, sizeof(miq_encoding) * c, hipMemcpyDeviceToHost, s));
     MIQ_CHECK_HIP(hipStreamSynchronize(s));
-    for (int64_t ch = 0; ch < c; ++ch)
-    {
-        out[ch].min    = heads[ch].enc_min;
-        out[ch].max    = heads[ch].enc_max;
-        out[ch].delta  = heads[ch].enc_delta;
-        out[ch].offset = heads[ch].enc_offset;
-        out[ch].bw     = heads[ch].enc_bw;
-    }
     return MIQ_OK;
 }
 
