@@ -256,10 +256,13 @@ __global__ __launch_bounds__(512, 4) void lin_fwd_kernel(const FT* __restrict__ 
     {
         // ---- consumer: MFMA layout, lane (n, s) supplies batch rows n and 16 + n, k = TK/4 w4 + 16 kk + 4 s + i
         const int n = lane & 15, s = lane >> 4;
+        // the row numbers in one load (lane l: batch entry l % 32), passed on by shuffles: a load per use is a chain of
+        // round trips before the first activation can be requested
+        const int row_of_lane = (int) gather_row(row_index, lane & 31, num_rows);
         const float* xrow[2];
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
-            xrow[mt] = X + gather_row(row_index, mt * 16 + n, num_rows) * x_row_stride + (int64_t) t_first * TK +
+            xrow[mt] = X + (int64_t) __shfl(row_of_lane, mt * 16 + n) * x_row_stride + (int64_t) t_first * TK +
                        w4 * (TK / 4) + 4 * s;
         v4f acc[2][2];
 #pragma unroll
@@ -390,11 +393,12 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
 // grid (K / 256, O / 32), 256 threads.  Phase 1: wavefront w forms dLoss/dW' for k in [64w, 64w + 64) as four 16-wide k
 // tiles (the M dimension of the MFMA) by two 16-wide o tiles (N), the batch being the MFMA's K dimension (8 steps of
 // 4), and parks it in the LDS tile.  Phase 2: the alpha-gradient + regulariser + Adam epilogue in the streaming layout.
-// (At most 128 registers, four wavefronts per SIMD: the LDS tile allows four workgroups per CU as well.  The cap only
-// holds without spills because the per-row parameters below travel through scalar registers.)
 //
-// Measured on the [4096, 4096] layer with int8 floor values (432 MB moved): 82.5 us; without phase 1, 73.6 us; without
-// phase 1 and with the epilogue's arithmetic replaced by additions, 70.9 us.  Ways of hiding phase 1 that were tried:
+// Measured on the [4096, 4096] layer with int8 floor values (432 MB moved): 78 us; without phase 1, 73.6 us; without
+// phase 1 and with the epilogue's arithmetic replaced by additions, 70.9 us.  Phase 1 as a loop of "row number,
+// activations, multiply" per step compiles into sixteen dependent round trips (a wait for every outstanding load
+// before each of them, the epilogue's first rows included) and took 82.5 us: its operands are requested up front,
+// ahead of the epilogue's rows, with the row numbers from one load.  Other ways of hiding phase 1 that were tried:
 //   one 16-byte activation load per lane and step feeding four MFMAs (k interleaved instead of blocked)    no change
 //   the register cap alone, eight registers spilled                                                         89 us
 //   workgroups of two roles as in lin_fwd_kernel walking 4 tiles, two LDS tiles, two workgroups per CU:
@@ -402,7 +406,7 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
 //       4 epilogue + 1 MFMA wavefront, two or four rows ahead                                         125 / 121 us
 // Eight streaming wavefronts per CU do not keep enough bytes in flight; sixteen with the multiplication in between do.
 template <int PF, typename FT>
-__global__ __launch_bounds__(256, 4) void lin_bwd_kernel(const FT* __restrict__ F, const float* __restrict__ G,
+__global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, const float* __restrict__ G,
                                                       const float* __restrict__ X, const int* __restrict__ row_index,
                                                       int num_rows, int64_t x_row_stride, float* __restrict__ alpha,
                                                       float* __restrict__ m, float* __restrict__ v,
@@ -416,18 +420,6 @@ __global__ __launch_bounds__(256, 4) void lin_bwd_kernel(const FT* __restrict__ 
     const int k_blk = blockIdx.x * kTileK;
     const int K = g.in_features, O = g.out_features;
 
-    // the epilogue's first rows are requested before the MFMA phase so that they arrive while it runs
-    v4f fv[PF], av[PF], mv[PF], vv[PF];
-#pragma unroll
-    for (int j = 0; j < PF; ++j)
-    {
-        const int64_t e = (int64_t) (o_blk + wave * 8 + j) * K + k_blk + 4 * lane;
-        fv[j]           = load_floor4<FT>(F + e);
-        av[j]           = ldg4(alpha + e);
-        mv[j]           = ldg4(m + e);
-        vv[j]           = ldg4(v + e);
-    }
-
     // per-row delta / offset, requested here and not where they are used (see lin_fwd_kernel); a row belongs to one
     // wavefront, so with the wavefront number as a scalar these are scalar loads
     float dl[8], of[8];
@@ -439,6 +431,39 @@ __global__ __launch_bounds__(256, 4) void lin_bwd_kernel(const FT* __restrict__ 
         of[j]       = g.offset[c];
     }
 
+    // phase 1's operands are requested first: loads return in the order of their requests, so the multiplication
+    // starts once these (cache hits) are back and does not wait for the epilogue's rows requested after them
+    float xa[8][4], gb[8][2];
+    // the 32 row numbers in one load (lane l holds that of batch entry l % 32), handed to the lanes that need them by
+    // shuffles: a load per step is a chain of eight round trips.  (Scalar loads of the 32 numbers measured the same.)
+    const int row_of_lane = (int) gather_row(row_index, lane & 31, num_rows);
+#pragma unroll
+    for (int step = 0; step < 8; ++step)
+    {
+        const int b       = 4 * step + s;
+        const float* xrow = X + (int64_t) __shfl(row_of_lane, b) * x_row_stride + k_blk + wave * 64 + n;
+        const float* grow = G + (int64_t) b * O + o_blk + n;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+            xa[step][mt] = xrow[mt * 16];
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+            gb[step][nt] = grow[nt * 16];
+    }
+    __builtin_amdgcn_sched_barrier(0);   // the requests above stay above: nothing below is scheduled between them
+    // the epilogue's first rows: they arrive while phase 1 runs
+    v4f fv[PF], av[PF], mv[PF], vv[PF];
+#pragma unroll
+    for (int j = 0; j < PF; ++j)
+    {
+        const int64_t e = (int64_t) (o_blk + wave * 8 + j) * K + k_blk + 4 * lane;
+        fv[j]           = load_floor4<FT>(F + e);
+        av[j]           = ldg4(alpha + e);
+        mv[j]           = ldg4(m + e);
+        vv[j]           = ldg4(v + e);
+    }
+
+    __builtin_amdgcn_sched_barrier(0);   // the requests above stay above: nothing below is scheduled between them
     v4f acc[4][2];
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt)
@@ -447,23 +472,11 @@ __global__ __launch_bounds__(256, 4) void lin_bwd_kernel(const FT* __restrict__ 
             acc[mt][nt] = (v4f) {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int step = 0; step < 8; ++step)
-    {
-        const int b       = 4 * step + s;
-        const float* xrow = X + gather_row(row_index, b, num_rows) * x_row_stride + k_blk + wave * 64 + n;
-        const float* grow = G + (int64_t) b * O + o_blk + n;
-        float xa[4], gb[2];
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-            xa[mt] = xrow[mt * 16];
-#pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
-            gb[nt] = grow[nt * 16];
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
             for (int nt = 0; nt < 2; ++nt)
-                acc[mt][nt] = mfma16(xa[mt], gb[nt], acc[mt][nt]);
-    }
+                acc[mt][nt] = mfma16(xa[step][mt], gb[step][nt], acc[mt][nt]);
     // lane holds dW'[o = 16 nt + n][k = 64 w + 16 mt + 4 s + i], i = 0..3
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt)
