@@ -351,11 +351,27 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
     if (idx < kBatch * out_features)
     {
         const int b = idx / out_features, o = idx - b * out_features;
+        // the row number and the bias are requested before the partial products, and the target as soon as the row
+        // number is back: two dependent round trips in all (requested where they are used, the four kinds of load
+        // form a chain of four)
+        const int r         = row_index ? row_index[b] : b;
+        const float bias_o  = bias ? bias[o] : 0.f;
         // the partial products are added in split order; four of them are requested at a time
         const float* p      = partial + (int64_t) b * out_features + o;
         const int64_t pitch = (int64_t) kBatch * out_features;
         float acc           = 0.f;
         int s               = 0;
+        float first[4]      = {0.f, 0.f, 0.f, 0.f};
+        if (num_split >= 4)
+        {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                first[q] = p[q * pitch];
+            s = 4;
+        }
+        float y = Y[(int64_t) min(max(r, 0), num_rows - 1) * y_row_stride + o];   // as gather_row
+        if (num_split >= 4)
+            acc = (((acc + first[0]) + first[1]) + first[2]) + first[3];
         for (; s + 4 <= num_split; s += 4)
         {
             const float p0 = p[s * pitch], p1 = p[(s + 1) * pitch], p2 = p[(s + 2) * pitch], p3 = p[(s + 3) * pitch];
@@ -364,9 +380,7 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
         for (; s < num_split; ++s)
             acc += p[s * pitch];
         if (bias)
-            acc += bias[o];
-        const int r = row_index ? row_index[b] : b;
-        float y     = Y[gather_row(row_index, b, num_rows) * y_row_stride + o];
+            acc += bias_o;
         if (r < 0 || r >= num_rows)
             acc = NAN;   // no such row: poison everything derived from it
         if (out)
