@@ -365,19 +365,38 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
     const int64_t e_base    = (int64_t) blockIdx.x * TILE;
     const int64_t nvec      = n / VEC;
 
-    // 1. the tile's loads go out first; everything below overlaps their latency
+    // 1. the tile's loads go out first; everything below overlaps their latency.  A workgroup whose whole tile exists
+    //    (all but the last) requests them without a condition per lane: under a per-lane condition the compiler moves
+    //    the first arithmetic on a vector into the conditional block, waits for that vector there, and only then
+    //    requests the next one.
     Vec vx[kUnroll], vg[kUnroll];
     bool live[kUnroll];
-#pragma unroll
-    for (int u = 0; u < kUnroll; ++u)
+    const bool whole_tile = e_base / VEC + (int64_t) kUnroll * kBlock <= nvec;   // workgroup-uniform
+    if (whole_tile)
     {
-        const int64_t v = e_base / VEC + (int64_t) u * kBlock + threadIdx.x;
-        live[u]         = v < nvec;
-        if (live[u])
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
         {
-            vx[u] = stream_load(reinterpret_cast<const Vec*>(ptr.x) + v);
+            const int64_t v = e_base / VEC + (int64_t) u * kBlock + threadIdx.x;
+            live[u]         = true;
+            vx[u]           = stream_load(reinterpret_cast<const Vec*>(ptr.x) + v);
             if constexpr (OP::NIN == 2)
                 vg[u] = stream_load(reinterpret_cast<const Vec*>(ptr.g) + v);
+        }
+    }
+    else
+    {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+        {
+            const int64_t v = e_base / VEC + (int64_t) u * kBlock + threadIdx.x;
+            live[u]         = v < nvec;
+            if (live[u])
+            {
+                vx[u] = stream_load(reinterpret_cast<const Vec*>(ptr.x) + v);
+                if constexpr (OP::NIN == 2)
+                    vg[u] = stream_load(reinterpret_cast<const Vec*>(ptr.g) + v);
+            }
         }
     }
 
@@ -411,24 +430,26 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
         pt = scalar_params<OP>(src);
     }
 
-    // 3. compute and store
+    // 3. compute every vector, then store them: with a store between two vectors' arithmetic the wait for the second
+    //    vector would also wait for that store (loads and stores complete in one order, and the store is conditional)
+    float fy[kUnroll][VEC];
+    int code[kUnroll][VEC];
+    bool no_nan[kUnroll];
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u)
     {
+        no_nan[u] = false;
         if (!live[u])
             continue;
         const uint32_t le = ((uint32_t) u * kBlock + threadIdx.x) * VEC;
-        const int64_t v   = e_base / VEC + (int64_t) u * kBlock + threadIdx.x;
-        float fx[VEC], fg[VEC], fy[VEC];
-        int code[VEC];
+        float fx[VEC], fg[VEC];
         T::unpack(vx[u], fx);
         if constexpr (OP::NIN == 2)
             T::unpack(vg[u], fg);
-        bool no_nan = false;
         if (one_row)
         {
-            apply_n<OP, VEC, OP::NIN == 2>(src, pt, fx, fg, fy, code);
-            no_nan = NoNanOut<OP>::get(pt);
+            apply_n<OP, VEC, OP::NIN == 2>(src, pt, fx, fg, fy[u], code[u]);
+            no_nan[u] = NoNanOut<OP>::get(pt);
         }
         else
         {
@@ -438,8 +459,8 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
             if (rem + VEC <= fd.d)
             {
                 const P p = win[lr];
-                apply_n<OP, VEC, OP::NIN == 2>(src, p, fx, fg, fy, code);
-                no_nan = NoNanOut<OP>::get(p);
+                apply_n<OP, VEC, OP::NIN == 2>(src, p, fx, fg, fy[u], code[u]);
+                no_nan[u] = NoNanOut<OP>::get(p);
             }
             else
             {
@@ -448,14 +469,21 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
                 for (int j = 0; j < VEC; ++j)
                 {
                     const P p = win[lr + ((rem + j >= fd.d) ? 1u : 0u)];
-                    fy[j]     = OP::template apply<false>(src, p, fx[j], OP::NIN == 2 ? fg[j] : 0.f, code[j]);
+                    fy[u][j]  = OP::template apply<false>(src, p, fx[j], OP::NIN == 2 ? fg[j] : 0.f, code[u][j]);
                 }
             }
         }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+    {
+        if (!live[u])
+            continue;
+        const int64_t v = e_base / VEC + (int64_t) u * kBlock + threadIdx.x;
         if (ptr.y)
-            stream_store(reinterpret_cast<Vec*>(ptr.y) + v, no_nan ? T::pack_no_nan(fy) : T::pack(fy));
+            stream_store(reinterpret_cast<Vec*>(ptr.y) + v, no_nan[u] ? T::pack_no_nan(fy[u]) : T::pack(fy[u]));
         if constexpr (CODES)
-            store_codes<typename OP::Code, VEC>(ptr.codes + v * VEC, code);
+            store_codes<typename OP::Code, VEC>(ptr.codes + v * VEC, code[u]);
     }
     // the n % VEC trailing elements
     if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * VEC))
