@@ -139,14 +139,43 @@ __global__ __launch_bounds__(kBlock) void learn_bwd_kernel(const IO* __restrict_
         // len and base are multiples of the vector width on this path (checked by the host)
         constexpr int64_t kStep = (int64_t) kBlock * T::VEC;
         int64_t i               = (int64_t) threadIdx.x * T::VEC;
-        for (; i + kStep < len; i += 2 * kStep)
+        // two vectors per array in flight before the arithmetic starts, and the next pair of each array requested
+        // before this pair's results are stored: loads and stores complete in one order, so a load requested after a
+        // store cannot be used before that store has finished its trip to memory
+        typedef typename T::Vec Vec;
+        Vec nxa, nxb, nga, ngb;
+        auto request = [&](int64_t at) {
+            nxa = stream_load(reinterpret_cast<const Vec*>(x + base + at));
+            nxb = stream_load(reinterpret_cast<const Vec*>(x + base + at + kStep));
+            nga = stream_load(reinterpret_cast<const Vec*>(g + base + at));
+            ngb = stream_load(reinterpret_cast<const Vec*>(g + base + at + kStep));
+        };
+        // The wait for a requested pair is placed by hand, where the number of younger stores is known (none before
+        // the loop, this iteration's two at its end): left to the first use at the top of the loop, it would have to
+        // cover both ways into the loop and would wait for the stores as well.
+        auto arrived = [&]() {
+            asm volatile("" : "+v"(nxa.x), "+v"(nxa.y), "+v"(nxa.z), "+v"(nxa.w), "+v"(nxb.x), "+v"(nxb.y), "+v"(nxb.z),
+                         "+v"(nxb.w));
+            asm volatile("" : "+v"(nga.x), "+v"(nga.y), "+v"(nga.z), "+v"(nga.w), "+v"(ngb.x), "+v"(ngb.y), "+v"(ngb.z),
+                         "+v"(ngb.w));
+        };
+        bool have = i + kStep < len;
+        if (have)
         {
-            // two vectors per array in flight before the arithmetic starts
+            request(i);
+            arrived();
+        }
+        while (have)
+        {
             float xa[T::VEC], ga[T::VEC], xb[T::VEC], gb[T::VEC], oa[T::VEC], ob[T::VEC];
-            T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(x + base + i)), xa);
-            T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(x + base + i + kStep)), xb);
-            T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(g + base + i)), ga);
-            T::unpack(stream_load(reinterpret_cast<const typename T::Vec*>(g + base + i + kStep)), gb);
+            T::unpack(nxa, xa);
+            T::unpack(nxb, xb);
+            T::unpack(nga, ga);
+            T::unpack(ngb, gb);
+            const int64_t i_next = i + 2 * kStep;
+            have                 = i_next + kStep < len;
+            if (have)
+                request(i_next);
             float m = 0.0f;
 #pragma unroll
             for (int j = 0; j < T::VEC; ++j)
@@ -171,9 +200,12 @@ __global__ __launch_bounds__(kBlock) void learn_bwd_kernel(const IO* __restrict_
             }
             if (WRITE_GX)
             {
-                stream_store(reinterpret_cast<typename T::Vec*>(gx + base + i), T::pack(oa));
-                stream_store(reinterpret_cast<typename T::Vec*>(gx + base + i + kStep), T::pack(ob));
+                stream_store(reinterpret_cast<Vec*>(gx + base + i), T::pack(oa));
+                stream_store(reinterpret_cast<Vec*>(gx + base + i + kStep), T::pack(ob));
             }
+            if (have)
+                arrived();
+            i = i_next;
         }
         if (i < len)
             learn_vec<IO, WRITE_GX>(p, x, g, gx, base + i, sg, og);
