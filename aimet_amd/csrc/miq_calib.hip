@@ -616,17 +616,29 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
     }
     vf4 a[kHistUnroll];
     // first tile's loads go out next: they overlap the state reads, the fold and the LDS clear
-    if (VEC)
-    {
-#pragma unroll
-        for (int u = 0; u < kHistUnroll; ++u)
+    // (a tile that exists as a whole is requested without a condition per lane: the compiler then waits for each
+    // vector where it is first used instead of for all four before the first)
+    auto request = [&](vf4(&to)[kHistUnroll], int64_t at) {
+        if (at + kHistUnroll * kBlock <= nvec)   // workgroup-uniform
         {
-            const int64_t i = base + u * kBlock + threadIdx.x;
-            a[u]            = nan4;
-            if (i < nvec)
-                a[u] = __builtin_nontemporal_load(v + i);   // read once: no reason to keep the line in the caches
+#pragma unroll
+            for (int u = 0; u < kHistUnroll; ++u)
+                to[u] = __builtin_nontemporal_load(v + at + u * kBlock + threadIdx.x);   // read once: not kept in the caches
         }
-    }
+        else
+        {
+#pragma unroll
+            for (int u = 0; u < kHistUnroll; ++u)
+            {
+                const int64_t i = at + u * kBlock + threadIdx.x;
+                to[u]           = nan4;
+                if (i < nvec)
+                    to[u] = __builtin_nontemporal_load(v + i);
+            }
+        }
+    };
+    if (VEC)
+        request(a, base);
     // ---- the range
     float bucket = bucket_arg, off = off_arg;
     bool have_range = true, fresh = false;
@@ -696,14 +708,7 @@ __global__ __launch_bounds__(kBlock) void hist_kernel(const float* __restrict__ 
             base += stride;
             if (base >= nvec)
                 break;
-#pragma unroll
-            for (int u = 0; u < kHistUnroll; ++u)
-            {
-                const int64_t i = base + u * kBlock + threadIdx.x;
-                a[u]            = nan4;
-                if (i < nvec)
-                    a[u] = __builtin_nontemporal_load(v + i);
-            }
+            request(a, base);   // (requested before the first tile is counted, into a second register set: 8.4 us per batch against 7.0)
         }
         if (group == 0 && threadIdx.x < (uint32_t) (n - nvec * 4))
             hist_add<kCopies>(lds, in[nvec * 4 + threadIdx.x], map, copy);
