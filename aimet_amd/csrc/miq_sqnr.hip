@@ -690,15 +690,28 @@ __global__ __launch_bounds__(BLOCK) void spec_bin_kernel(const float* __restrict
     int64_t base         = (int64_t) blockIdx.x * share;
     const int64_t end    = base + share < nvec ? base + share : nvec;
     v4f a[kInFlight];
-    if (vec)
-    {
-#pragma unroll
-        for (int u = 0; u < kInFlight; ++u)
+    // A tile that lies inside the share as a whole is requested without a condition per lane.  With one, the loaded
+    // value passes through a select, the compiler waits for it there, and a tile requested "ahead" is waited for
+    // before the current one is counted.
+    auto request = [&](v4f(&to)[kInFlight], int64_t at) {
+        if (at + (int64_t) kInFlight * BLOCK <= end)   // workgroup-uniform
         {
-            const int64_t i = base + u * BLOCK + threadIdx.x;
-            a[u]            = i < end ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u)
+                to[u] = __builtin_nontemporal_load(rv + at + u * BLOCK + threadIdx.x);
         }
-    }
+        else
+        {
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u)
+            {
+                const int64_t i = at + u * BLOCK + threadIdx.x;
+                to[u]           = i < end ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
+            }
+        }
+    };
+    if (vec)
+        request(a, base);
     for (int i = threadIdx.x; i < num_bins * copies; i += BLOCK)
         lds[i] = 0;
     // torch.histc(min, max) over the statistics' range: equal bounds are widened by one each way
@@ -730,14 +743,7 @@ __global__ __launch_bounds__(BLOCK) void spec_bin_kernel(const float* __restrict
             const int64_t next = base + stride;
             v4f nx[kInFlight];
             if (next < end)
-            {
-#pragma unroll
-                for (int u = 0; u < kInFlight; ++u)
-                {
-                    const int64_t i = next + u * BLOCK + threadIdx.x;
-                    nx[u]           = i < end ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
-                }
-            }
+                request(nx, next);
 #pragma unroll
             for (int u = 0; u < kInFlight; ++u)
             {
