@@ -513,6 +513,23 @@ __global__ __launch_bounds__(kHistBlock) void row_update_kernel(const float* __r
             keep[u]         = i < nvec ? __builtin_nontemporal_load(rv + i) : (v4f) {NAN, NAN, NAN, NAN};
         }
     }
+    // the running statistics are requested with the row: asked for where they are used, the range and the running
+    // counts are two more round trips in a workgroup whose whole life is a handful of them
+    float* sh = state_hist + (int64_t) h * num_bins;
+    constexpr int kBinsPerLane = kRowBinsMax / kHistBlock;
+    float old_mm[2]            = {0.f, 0.f};
+    float old_count[kBinsPerLane];
+    if (has_stats)
+    {
+        old_mm[0] = state_minmax[2 * h];
+        old_mm[1] = state_minmax[2 * h + 1];
+#pragma unroll
+        for (int k = 0; k < kBinsPerLane; ++k)
+        {
+            const int i  = k * kHistBlock + threadIdx.x;
+            old_count[k] = i < num_bins ? sh[i] : 0.f;
+        }
+    }
     const bool two = BATCH && has_stats;   // two histograms: batch range and merged range
     for (int i = threadIdx.x; i < (two ? 2 : 1) * num_bins * kRowCopies; i += kHistBlock)
         lds[i] = 0;
@@ -561,7 +578,7 @@ __global__ __launch_bounds__(kHistBlock) void row_update_kernel(const float* __r
         hi = fmaxf(hi, s_mm[1][k]);
     }
     bool ok;
-    const Ranges r = compute_ranges(lo, hi, num_bins, has_stats, state_minmax, h, ok);
+    const Ranges r = compute_ranges(lo, hi, num_bins, has_stats, old_mm, 0, ok);
     if (threadIdx.x == 0)
     {
         if (batch_minmax)
@@ -613,17 +630,20 @@ __global__ __launch_bounds__(kHistBlock) void row_update_kernel(const float* __r
             count(row[i]);
     }
     __syncthreads();
-    float* sh          = state_hist + (int64_t) h * num_bins;
     const bool rebins  = has_stats && r.rebin;
     if (rebins)
         rebin_running_histogram(upd, sh, r, num_bins);   // ends with a barrier
-    for (int i = threadIdx.x; i < num_bins; i += kHistBlock)
+#pragma unroll
+    for (int k = 0; k < kBinsPerLane; ++k)
     {
+        const int i = k * kHistBlock + threadIdx.x;
+        if (i >= num_bins)
+            break;
         uint32_t total = 0;
 #pragma unroll
         for (int c = 0; c < kRowCopies; ++c)
             total += lds[i * kRowCopies + c];
-        const float before = !has_stats ? 0.0f : (rebins ? upd[i] : sh[i]);
+        const float before = !has_stats ? 0.0f : (rebins ? upd[i] : old_count[k]);
         sh[i]              = (float) total + before;
         if (BATCH)
         {
