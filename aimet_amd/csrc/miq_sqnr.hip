@@ -476,7 +476,7 @@ __device__ void rebin_running_histogram(float* __restrict__ upd, const float* __
 // BATCH: the batch's own histogram (over the batch's range) is written as well; with running statistics that is a
 // second LDS histogram, counted in the same pass.
 constexpr int kRowKeep    = 6;      // 16-byte groups a lane keeps
-constexpr int kRowBinsMax = 2048;   // 32 KiB of counts + 16 KiB for re-binning: within the 64 KiB of LDS a launch may ask for
+constexpr int kRowBinsMax = 2048;   // 16 KiB of counts + 8 KiB for re-binning per workgroup: six of them fit a compute unit
 template <bool BATCH>
 __global__ __launch_bounds__(kHistBlock) void row_update_kernel(const float* __restrict__ x, int64_t n_per_hist,
                                                                 int num_bins, int has_stats,
@@ -486,9 +486,12 @@ __global__ __launch_bounds__(kHistBlock) void row_update_kernel(const float* __r
                                                                 float* __restrict__ batch_minmax,
                                                                 int* __restrict__ bad_flag, int vec)
 {
-    constexpr int kRowCopies = BATCH ? 2 : 4;   // [kinds][num_bins][copies] words stay within 32 KiB at 2048 bins
+    // [kinds][num_bins][copies] words: 16 KiB at 2048 bins.  The workgroup's life is a chain of round trips, so what
+    // counts is how many of them a compute unit holds: with twice the copies (three workgroups per unit instead of six)
+    // the launch over [11008, 4096] took 94 us instead of 61.
+    constexpr int kRowCopies = BATCH ? 1 : 2;
     extern __shared__ uint32_t lds[];
-    __shared__ float upd[kMaxBins];
+    __shared__ float upd[kRowBinsMax];
     __shared__ float s_mm[2][kHistBlock / 64];
     const int h        = blockIdx.x;
     const float* row   = x + (int64_t) h * n_per_hist;
@@ -1412,8 +1415,8 @@ int miq_v2_hist_update_f32(const float* data, int64_t num_hist, int64_t n_per_hi
     const Tickets tickets = {words, groups > 1 ? group_words : nullptr};
     if (blocks == 1 && num_bins <= kRowBinsMax)
     {
-        // a row per workgroup: the whole update in one launch ([kinds][bins][copies] LDS words, kinds * copies = 4)
-        const size_t lds_bytes = (size_t) num_bins * 4 * sizeof(uint32_t);
+        // a row per workgroup: the whole update in one launch ([kinds][bins][copies] LDS words, kinds * copies = 2)
+        const size_t lds_bytes = (size_t) num_bins * 2 * sizeof(uint32_t);   // row_update_kernel's [kinds][bins][copies]
         if (want_batch_hist)
             hipLaunchKernelGGL(row_update_kernel<true>, dim3((unsigned) num_hist), dim3(kHistBlock), lds_bytes, s, data,
                                n_per_hist, num_bins, has_stats, state_hist, state_minmax, batch_hist, batch_minmax,
