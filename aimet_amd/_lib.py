@@ -82,10 +82,11 @@ _SIGNATURES = {
     "miq_adaround_floor_i8": ([_p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _p, _p], _int),
     "miq_adaround_floor_i16": ([_p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _p, _p], _int),
     "miq_adaround_init_alpha_f32": ([_p, _p, _i64, _i64, _i64, _p, _p], _int),
-    "miq_adaround_bwd_adam_f32": ([_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _flt, _flt, _flt,
-                                   _flt, _flt, _flt, _int, _p, _p], _int),
-    "miq_adaround_bwd_f32": ([_p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _flt, _flt, _p, _p], _int),
+    "miq_adaround_bwd_adam_f32": ([_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _dbl, _dbl, _dbl,
+                                   _dbl, _dbl, _dbl, _int, _p, _p], _int),
+    "miq_adaround_bwd_f32": ([_p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _dbl, _dbl, _p, _p], _int),
     "miq_adaround_blocks": ([_i64], _int),
+    "miq_adaround_eval_terms_f32": ([_p, _p, _i64, _int, _dbl, _p], _int),
     "miq_v2_hist_workspace_bytes": ([_i64, _i64, _int], _i64),
     "miq_v2_hist_update_f32": ([_p, _i64, _i64, _int, _int, _int, _p, _p, _p, _p, _p, _p, _p], _int),
     "miq_v2_sqnr_num_candidates": ([_dbl, _int, _int, _int, _int], _int),
@@ -104,15 +105,15 @@ _SIGNATURES = {
     "miq_adaround_linear_fwd_f32": ([_p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
                                      _p, _p, _p, _p, _p], _int),
     "miq_adaround_linear_bwd_adam_f32": ([_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
-                                          _flt, _flt, _flt, _flt, _flt, _flt, _int, _p, _p], _int),
+                                          _dbl, _dbl, _dbl, _dbl, _dbl, _dbl, _int, _p, _p], _int),
     "miq_adaround_linear_fwd_i8": ([_p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
                                     _p, _p, _p, _p, _p], _int),
     "miq_adaround_linear_bwd_adam_i8": ([_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
-                                         _flt, _flt, _flt, _flt, _flt, _flt, _int, _p, _p], _int),
+                                         _dbl, _dbl, _dbl, _dbl, _dbl, _dbl, _int, _p, _p], _int),
     "miq_adaround_linear_fwd_i16": ([_p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
                                      _p, _p, _p, _p, _p], _int),
     "miq_adaround_linear_bwd_adam_i16": ([_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
-                                          _flt, _flt, _flt, _flt, _flt, _flt, _int, _p, _p], _int),
+                                          _dbl, _dbl, _dbl, _dbl, _dbl, _dbl, _int, _p, _p], _int),
 }
 
 # Entry points declared in include/miq.h; the loader insists on every one of them.

@@ -20,19 +20,25 @@ namespace miq
 {
 namespace ada
 {
-int make_adam(AdamArgs& a, float reg_param, float beta, float lr, float beta1, float beta2, float eps, int step)
+int make_adam(AdamArgs& a, double reg_param, double beta, double lr, double beta1, double beta2, double eps, int step)
 {
-    MIQ_CHECK_ARG(step >= 1, "Adam step count starts at 1");
-    MIQ_CHECK_ARG(beta1 >= 0.f && beta1 < 1.f && beta2 >= 0.f && beta2 < 1.f, "Adam betas must lie in [0, 1)");
-    a.reg_param = reg_param;
-    a.beta      = beta;
-    const double bc1 = 1.0 - std::pow((double) beta1, (double) step);
-    const double bc2 = 1.0 - std::pow((double) beta2, (double) step);
-    a.lr_over_bc1    = (float) ((double) lr / bc1);
-    a.inv_bc2_sqrt   = (float) (1.0 / std::sqrt(bc2));
-    a.beta1          = beta1;
-    a.beta2          = beta2;
-    a.eps            = eps;
+    a           = {};
+    a.reg_param = (float) reg_param;
+    a.beta      = (float) beta;
+    a.pow_exp   = (double) (float) (beta - 1.0);
+    if (step < 1)
+        return MIQ_OK;
+    MIQ_CHECK_ARG(beta1 >= 0.0 && beta1 < 1.0 && beta2 >= 0.0 && beta2 < 1.0, "Adam betas must lie in [0, 1)");
+    MIQ_CHECK_ARG((float) (1.0 - beta1) < 0.5f, "beta1 must exceed 0.5 (the update uses lerp's small-weight form)");
+    // Python-float arithmetic of torch/optim/adam.py, then the casts of the kernels that receive the scalars
+    const double bc1 = 1.0 - std::pow(beta1, (double) step);
+    const double bc2 = 1.0 - std::pow(beta2, (double) step);
+    a.w1             = (float) (1.0 - beta1);
+    a.beta2          = (float) beta2;
+    a.c2             = (float) (1.0 - beta2);
+    a.bc2_sqrt_rcp   = 1.0f / (float) std::pow(bc2, 0.5);
+    a.eps            = (float) eps;
+    a.neg_step       = (float) (-(lr / bc1));
     return MIQ_OK;
 }
 }   // namespace ada
@@ -138,6 +144,11 @@ __global__ __launch_bounds__(kBlock) void bwd_kernel(const float* __restrict__ w
                                                      float* __restrict__ v, float* __restrict__ grad_out, AdaGeom g,
                                                      AdamArgs a, float* __restrict__ reg_partial)
 {
+    __shared__ PowEntry tab[128];
+    PowTableLoad tl;
+    tl.request();
+    tl.store(tab);
+    __syncthreads();
     const int64_t nvec = g.n / 4;
     const int64_t i    = (int64_t) blockIdx.x * kBlock + threadIdx.x;
     float reg          = 0.0f;
@@ -162,7 +173,7 @@ __global__ __launch_bounds__(kBlock) void bwd_kernel(const float* __restrict__ w
         {
             const uint32_t c = (c0 == c3) ? c0 : channel_of(i * 4 + j, g);
             float r;
-            gr[j] = alpha_grad(ws[j], gs[j], as[j], g.delta[c], g.offset[c], g.clip_min, g.clip_max, a, r);
+            gr[j] = alpha_grad(ws[j], gs[j], as[j], g.delta[c], g.offset[c], g.clip_min, g.clip_max, a, tab, r);
             reg += r;
             if (ADAM)
                 adam_update(gr[j], as[j], ms[j], vs[j], a);
@@ -181,7 +192,7 @@ __global__ __launch_bounds__(kBlock) void bwd_kernel(const float* __restrict__ w
         const int64_t e  = nvec * 4 + threadIdx.x;
         const uint32_t c = channel_of(e, g);
         float r;
-        const float gr = alpha_grad(w[e], gw[e], alpha[e], g.delta[c], g.offset[c], g.clip_min, g.clip_max, a, r);
+        const float gr = alpha_grad(w[e], gw[e], alpha[e], g.delta[c], g.offset[c], g.clip_min, g.clip_max, a, tab, r);
         reg += r;
         if (ADAM)
             adam_update(gr, alpha[e], m[e], v[e], a);
@@ -194,6 +205,36 @@ __global__ __launch_bounds__(kBlock) void bwd_kernel(const float* __restrict__ w
         const float t = block_sum_256(reg);
         if (threadIdx.x == 0)
             reg_partial[blockIdx.x] = t;
+    }
+}
+
+// The kernels' own per-element terms for arrays of alpha (what = 0: sigmoid, h, dh/dalpha) or of h (what = 1:
+// 1 - |2h - 1|^beta and its derivative with respect to h), for accuracy measurements against float64.
+__global__ __launch_bounds__(kBlock) void eval_terms_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                            int64_t n, int what, AdamArgs a)
+{
+    __shared__ PowEntry tab[128];
+    PowTableLoad tl;
+    tl.request();
+    tl.store(tab);
+    __syncthreads();
+    for (int64_t e = (int64_t) blockIdx.x * kBlock + threadIdx.x; e < n; e += (int64_t) gridDim.x * kBlock)
+    {
+        if (what == 0)
+        {
+            float sig, inner, ee, dh;
+            soft_h(in[e], sig, inner, ee);
+            const float h  = soft_h_grad(in[e], dh);
+            out[e]         = sig;
+            out[n + e]     = h;
+            out[2 * n + e] = dh;
+        }
+        else
+        {
+            float dreg;
+            out[e]     = reg_terms(in[e], a, tab, dreg);
+            out[n + e] = dreg;
+        }
     }
 }
 
@@ -333,8 +374,8 @@ int miq_adaround_init_alpha_f32(const float* weight, float* alpha, int64_t num_c
 
 int miq_adaround_bwd_f32(const float* weight, const float* grad_weight, const float* alpha, float* grad_alpha,
                          int64_t num_channel, int64_t num_element, int64_t num_element_per_channel,
-                         const float* delta, const float* offset, float clip_min, float clip_max, float reg_param,
-                         float beta, float* reg_partial, void* stream)
+                         const float* delta, const float* offset, float clip_min, float clip_max, double reg_param,
+                         double beta, float* reg_partial, void* stream)
 {
     AdaGeom g;
     if (int rc = make_geom(g, num_channel, num_element, num_element_per_channel, delta, offset, clip_min, clip_max))
@@ -344,9 +385,9 @@ int miq_adaround_bwd_f32(const float* weight, const float* grad_weight, const fl
     MIQ_CHECK_ARG(weight && grad_weight && alpha && grad_alpha, "null tensor pointer");
     MIQ_CHECK_ARG(aligned16(weight) && aligned16(grad_weight) && aligned16(alpha) && aligned16(grad_alpha),
                   "tensors must be 16-byte aligned");
-    AdamArgs a    = {};
-    a.reg_param   = reg_param;
-    a.beta        = beta;
+    AdamArgs a;
+    if (int rc = make_adam(a, reg_param, beta, 0.0, 0.0, 0.0, 0.0, 0))
+        return rc;
     hipLaunchKernelGGL(bwd_kernel<false>, dim3(vec_blocks(num_element)), dim3(kBlock), 0, (hipStream_t) stream, weight,
                        grad_weight, const_cast<float*>(alpha), (float*) nullptr, (float*) nullptr, grad_alpha, g, a,
                        reg_partial);
@@ -357,8 +398,8 @@ int miq_adaround_bwd_f32(const float* weight, const float* grad_weight, const fl
 int miq_adaround_bwd_adam_f32(const float* weight, const float* grad_weight, float* alpha, float* exp_avg,
                               float* exp_avg_sq, float* grad_alpha, int64_t num_channel, int64_t num_element,
                               int64_t num_element_per_channel, const float* delta, const float* offset, float clip_min,
-                              float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
-                              float eps, int step, float* reg_partial, void* stream)
+                              float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
+                              double eps, int step, float* reg_partial, void* stream)
 {
     AdaGeom g;
     if (int rc = make_geom(g, num_channel, num_element, num_element_per_channel, delta, offset, clip_min, clip_max))
@@ -369,11 +410,31 @@ int miq_adaround_bwd_adam_f32(const float* weight, const float* grad_weight, flo
     MIQ_CHECK_ARG(aligned16(weight) && aligned16(grad_weight) && aligned16(alpha) && aligned16(exp_avg) &&
                       aligned16(exp_avg_sq) && aligned16(grad_alpha),
                   "tensors must be 16-byte aligned");
+    MIQ_CHECK_ARG(step >= 1, "Adam step count starts at 1");
     AdamArgs a;
     if (int rc = make_adam(a, reg_param, beta, lr, beta1, beta2, eps, step))
         return rc;
     hipLaunchKernelGGL(bwd_kernel<true>, dim3(vec_blocks(num_element)), dim3(kBlock), 0, (hipStream_t) stream, weight,
                        grad_weight, alpha, exp_avg, exp_avg_sq, grad_alpha, g, a, reg_partial);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int miq_adaround_eval_terms_f32(const float* in, float* out, int64_t num_element, int what, double beta, void* stream)
+{
+    MIQ_CHECK_ARG(num_element >= 0 && (what == 0 || what == 1), "what must be 0 (terms of alpha) or 1 (terms of h)");
+    MIQ_CHECK_ARG(what == 0 || beta >= 1.0, "the regulariser's exponent must be at least 1");
+    if (num_element == 0)
+        return MIQ_OK;
+    MIQ_CHECK_ARG(in && out, "null tensor pointer");
+    AdamArgs a;
+    if (int rc = make_adam(a, 1.0, beta, 0.0, 0.0, 0.0, 0.0, 0))
+        return rc;
+    int64_t blocks = (num_element + kBlock - 1) / kBlock;
+    if (blocks > 4096)
+        blocks = 4096;
+    hipLaunchKernelGGL(eval_terms_kernel, dim3((unsigned) blocks), dim3(kBlock), 0, (hipStream_t) stream, in, out,
+                       num_element, what, a);
     MIQ_CHECK_LAUNCH();
     return MIQ_OK;
 }

@@ -428,10 +428,13 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, 
                                                       float* __restrict__ reg_partial)
 {
     __shared__ __attribute__((aligned(16))) float tile[kTileO * kLdsRow];
+    __shared__ PowEntry tab[128];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int n = lane & 15, s = lane >> 4;
     const int o_blk = blockIdx.y * kTileO;
     const int k_blk = blockIdx.x * kTileK;
+    PowTableLoad tl;
+    tl.request();
     const int K = g.in_features, O = g.out_features;
 
     // per-row delta / offset, requested here and not where they are used (see lin_fwd_kernel); a row belongs to one
@@ -497,6 +500,7 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, 
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
             *reinterpret_cast<v4f*>(&tile[(nt * 16 + n) * kLdsRow + wave * 64 + mt * 16 + 4 * s]) = acc[mt][nt];
+    tl.store(tab);
     __syncthreads();
 
     float reg = 0.f;
@@ -524,7 +528,7 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, 
         for (int i = 0; i < 4; ++i)
         {
             float rr;
-            const float gi = alpha_grad_f(f4[i], gw[i], as[i], d, off, g.clip_min, g.clip_max, a, rr);
+            const float gi = alpha_grad_f(f4[i], gw[i], as[i], d, off, g.clip_min, g.clip_max, a, tab, rr);
             reg += rr;
             adam_update(gi, as[i], ms[i], vs[i], a);
             gr[i] = gi;
@@ -615,8 +619,8 @@ template <typename FT>
 static int linear_bwd_adam(const FT* weight_floor, const float* grad_out, const float* x, const int32_t* row_index,
                            int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg, float* exp_avg_sq, float* grad_alpha,
                            int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
-                           const float* offset, float clip_min, float clip_max, float reg_param, float beta, float lr,
-                           float beta1, float beta2, float eps, int step, float* reg_partial, void* stream)
+                           const float* offset, float clip_min, float clip_max, double reg_param, double beta, double lr,
+                           double beta1, double beta2, double eps, int step, float* reg_partial, void* stream)
 {
     LinGeom g;
     if (int rc = make_lin_geom(g, out_features, in_features, num_channel, delta, offset, clip_min, clip_max))
@@ -628,6 +632,7 @@ static int linear_bwd_adam(const FT* weight_floor, const float* grad_out, const 
     MIQ_CHECK_ARG(x_row_stride >= in_features, "row stride shorter than a row");
     MIQ_CHECK_ARG(num_rows >= 1 && num_rows < (1ll << 31) && (row_index || num_rows >= kBatch),
                   "num_rows (%lld) must be positive, and at least 32 without a row index", (long long) num_rows);
+    MIQ_CHECK_ARG(step >= 1, "Adam step count starts at 1");
     AdamArgs a;
     if (int rc = make_adam(a, reg_param, beta, lr, beta1, beta2, eps, step))
         return rc;
@@ -685,8 +690,8 @@ int miq_adaround_linear_bwd_adam_f32(const float* weight_floor, const float* gra
                                      const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                      float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                      int64_t num_channel, const float* delta, const float* offset, float clip_min,
-                                     float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
-                                     float eps, int step, float* reg_partial, void* stream)
+                                     float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
+                                     double eps, int step, float* reg_partial, void* stream)
 {
     return linear_bwd_adam<float>(weight_floor, grad_out, x, row_index, num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq,
                                   grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min, clip_max,
@@ -697,8 +702,8 @@ int miq_adaround_linear_bwd_adam_i8(const int8_t* weight_floor, const float* gra
                                     const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                     float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                     int64_t num_channel, const float* delta, const float* offset, float clip_min,
-                                    float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
-                                    float eps, int step, float* reg_partial, void* stream)
+                                    float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
+                                    double eps, int step, float* reg_partial, void* stream)
 {
     return linear_bwd_adam<int8_t>(weight_floor, grad_out, x, row_index, num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq,
                                    grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min,
@@ -720,8 +725,8 @@ int miq_adaround_linear_bwd_adam_i16(const int16_t* weight_floor, const float* g
                                     const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                     float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                     int64_t num_channel, const float* delta, const float* offset, float clip_min,
-                                    float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
-                                    float eps, int step, float* reg_partial, void* stream)
+                                    float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
+                                    double eps, int step, float* reg_partial, void* stream)
 {
     return linear_bwd_adam<int16_t>(weight_floor, grad_out, x, row_index, num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq,
                                    grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min,

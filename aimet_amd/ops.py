@@ -548,6 +548,19 @@ def adaround_blocks(num_element):
     return int(lib.miq_adaround_blocks(int(num_element)))
 
 
+def adaround_eval_terms(values, what, beta=2.0):
+    """The kernels' own per-element AdaRound terms, for accuracy measurements.
+
+    what = 0: `values` is alpha; returns (sigmoid(alpha), h(alpha), dh/dalpha).
+    what = 1: `values` is h; returns (1 - |2h - 1|^beta, its derivative with respect to h)."""
+    _ada_check(values)
+    n = values.numel()
+    out = torch.empty((3 if what == 0 else 2, n), dtype=_F32, device=values.device)
+    with _OnDevice(values.device):
+        check(lib.miq_adaround_eval_terms_f32(_ptr(values), _ptr(out), n, int(what), float(beta), _stream(values)))
+    return tuple(out[i] for i in range(out.size(0)))
+
+
 def adaround_bwd(weight, grad_weight, alpha, num_channel, n_per_channel, delta, offset, clip_min, clip_max,
                  reg_param=0.0, beta=-1.0, reg_partial=None):
     """dLoss/dW' -> dLoss/dalpha (rounding regulariser included when beta >= 0); returns the gradient."""

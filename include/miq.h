@@ -356,22 +356,31 @@ int miq_adaround_init_alpha_f32(const float* weight, float* alpha, int64_t num_c
  * reg_param * sum(1 - |2h - 1|^beta) (AdaroundLoss.compute_round_loss, ADA/adaround_loss.py:82-111) when beta >= 0
  * (beta < 0 = warm-start period, regulariser off), and applies torch.optim.Adam's update (no weight decay, no
  * amsgrad) to alpha with moments exp_avg / exp_avg_sq; `step` is the 1-based count of this update.
+ * The hyper-parameters are doubles because the reference's are Python floats: 1 - beta1, 1 - beta2, the bias
+ * corrections and lr / (1 - beta1^step) are formed in double and cast to float32 where torch's kernels cast them
+ * (1 - float32(0.999) differs from float32(1 - 0.999) by 1.3e-5 of its value).  beta1 must exceed 0.5.
  * grad_alpha: optional (may be null) device tensor receiving dLoss/dalpha, what alpha.grad holds in the reference.
  * reg_partial: optional device float[miq_adaround_blocks(num_element)] receiving per-workgroup partial sums of
  * (1 - |2h - 1|^beta) evaluated at the alpha *before* the update (summed and scaled by reg_param by the caller). */
 int miq_adaround_bwd_adam_f32(const float* weight, const float* grad_weight, float* alpha, float* exp_avg,
                               float* exp_avg_sq, float* grad_alpha, int64_t num_channel, int64_t num_element,
                               int64_t num_element_per_channel, const float* delta, const float* offset, float clip_min,
-                              float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
-                              float eps, int step, float* reg_partial, void* stream);
+                              float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
+                              double eps, int step, float* reg_partial, void* stream);
 /* The gradient alone (autograd of apply_adaround + compute_round_loss w.r.t. alpha), nothing updated: for callers
  * that keep their own optimiser. */
 int miq_adaround_bwd_f32(const float* weight, const float* grad_weight, const float* alpha, float* grad_alpha,
                          int64_t num_channel, int64_t num_element, int64_t num_element_per_channel,
-                         const float* delta, const float* offset, float clip_min, float clip_max, float reg_param,
-                         float beta, float* reg_partial, void* stream);
+                         const float* delta, const float* offset, float clip_min, float clip_max, double reg_param,
+                         double beta, float* reg_partial, void* stream);
 /* Number of workgroups (= partial sums) miq_adaround_bwd_adam_f32 / miq_adaround_bwd_f32 use for num_element elements. */
 int miq_adaround_blocks(int64_t num_element);
+/* The per-element terms exactly as the kernels above evaluate them, for accuracy measurements (no counterpart in the
+ * reference, whose terms are separate torch ops: ADA/adaround_wrapper.py:136-139, ADA/adaround_loss.py:100-106).
+ *   what = 0: in = alpha[n]; out = float[3 n]: sigmoid(alpha), h(alpha), dh/dalpha
+ *   what = 1: in = h[n];     out = float[2 n]: 1 - |2h - 1|^beta, and its derivative with respect to h,
+ *             -beta |2h - 1|^(beta - 1) sgn(2h - 1) 2, with the exponent float32(beta - 1) as torch's pow backward takes it */
+int miq_adaround_eval_terms_f32(const float* in, float* out, int64_t num_element, int what, double beta, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
  * AdaRound iteration of a Linear layer, soft rounding fused into MFMA GEMMs (the adarounded weight and its gradient
@@ -413,8 +422,8 @@ int miq_adaround_linear_bwd_adam_f32(const float* weight_floor, const float* gra
                                      const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                      float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                      int64_t num_channel, const float* delta, const float* offset, float clip_min,
-                                     float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
-                                     float eps, int step, float* reg_partial, void* stream);
+                                     float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
+                                     double eps, int step, float* reg_partial, void* stream);
 
 int miq_adaround_linear_fwd_i8(const int8_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
                                int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
@@ -425,8 +434,8 @@ int miq_adaround_linear_bwd_adam_i8(const int8_t* weight_floor, const float* gra
                                     const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                     float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                     int64_t num_channel, const float* delta, const float* offset, float clip_min,
-                                    float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
-                                    float eps, int step, float* reg_partial, void* stream);
+                                    float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
+                                    double eps, int step, float* reg_partial, void* stream);
 int miq_adaround_linear_fwd_i16(const int16_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
                                int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
                                int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
@@ -436,8 +445,8 @@ int miq_adaround_linear_bwd_adam_i16(const int16_t* weight_floor, const float* g
                                     const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                     float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                     int64_t num_channel, const float* delta, const float* offset, float clip_min,
-                                    float clip_max, float reg_param, float beta, float lr, float beta1, float beta2,
-                                    float eps, int step, float* reg_partial, void* stream);
+                                    float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
+                                    double eps, int step, float* reg_partial, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
  * v2 histogram observer + SQNR encoding analyzer

@@ -116,7 +116,7 @@ def optimize_rounding(kind, weight, alpha0, delta, offset, clip_min, clip_max, a
         rnd = compute_round_loss(alpha, num_iterations, reg_param, beta_range, warm_start, iteration)
         (recon + rnd).backward()
         if trace is not None:
-            trace.append((float(recon), float(rnd)))
+            trace.append((float(recon.detach()), float(rnd.detach()) if torch.is_tensor(rnd) else float(rnd)))
         optimizer.step()
     state = optimizer.state[alpha]
     return alpha.detach(), state["exp_avg"], state["exp_avg_sq"], alpha.grad

@@ -1,14 +1,23 @@
 """GPU parity of the AdaRound kernels and of the AdaRound flow against the CPU restatement of the reference
 (oracle/adaround_oracle.py: torch CPU ops, torch autograd and torch.optim.Adam), through the C ABI.
 
-Tolerances (float32 path, transcendental functions differ by an ulp or two between the GPU and the host libm):
-  adarounded weights   hard rounding: identical; soft rounding: |diff| <= 4 ulp(2^bw) * delta
-  alpha initialisation |diff| <= 2e-6 (alpha lies in [-2.4, 2.4])
-  gradients            1e-4 relative to the largest gradient magnitude
+Accuracy of the per-element terms is measured in ulp against float64 evaluated on the same float32 inputs
+(test_term_accuracy_in_ulp), next to what torch's float32 CPU ops reach on the same inputs:
+  h(alpha)             |error| <= 2 ulp(1)                      (torch CPU: 1.4)
+  dh/dalpha            <= 8 ulp                                  (torch CPU: 11.4, from the cancellation in 1 - sigmoid)
+  1 - |2h - 1|^beta    |error| <= 1.25 ulp(1)                    (torch CPU: 0.5)
+  its derivative in h  <= 2.5 ulp                                (torch CPU: 1.3 ... 8.3)
+The alpha gradient is the float32 combination of those terms, bit for bit (test_alpha_gradient).  Against the CPU
+restatement's autograd it can only be compared up to the conditioning both sides share: a last-bit difference in h
+moves |2h - 1|^(beta - 1) by (beta - 1) / |2h - 1| last bits, which is where the 2e-5 of the largest gradient comes from.
+Adam: both moments equal torch.optim.Adam's on the CPU bit for bit given the same gradients; alpha in all but about one
+element in a thousand per step, those by one ulp (test_adam_update_against_torch_cpu).
+Trajectories over N iterations (GEMMs with different summation orders on the two sides):
   alpha after N Adam iterations  5e-5 absolute (lr = 1e-3, so this is 5 % of one step) for 99.9 % of the elements;
                        elements that crossed a clamp boundary may differ by a few steps (see _close_except_few)
 """
 import json
+import math
 import os
 
 import numpy as np
@@ -67,6 +76,101 @@ def test_init_alpha_and_soft_round(ops, shape, ch_axis, per_channel):
     assert torch.allclose(soft, soft_ref, atol=float(4 * 2.0 ** -23 * 16 * delta.max()), rtol=0)
 
 
+def _ulps(got, want64):
+    """|got - want| in units of the float32 spacing at |want|."""
+    want64 = np.asarray(want64, np.float64)
+    spacing = np.maximum(np.spacing(np.abs(want64).astype(np.float32)).astype(np.float64), 2.0 ** -149)
+    return np.abs(got.astype(np.float64) - want64) / spacing
+
+
+def test_term_accuracy_in_ulp(ops):
+    """The kernels' own sigmoid / h / dh and regulariser terms against float64 on the same float32 inputs, alpha over
+    [-12, 12] and beta over the schedule's range; torch's float32 CPU ops on the same inputs for comparison."""
+    g = torch.Generator().manual_seed(0)
+    edge = math.log(11.0)                                # h leaves / reaches the clamp at sigmoid = 1/12 and 11/12
+    alpha = torch.cat([torch.linspace(-12, 12, 2_000_001), torch.randn(1_000_000, generator=g) * 2.5,
+                       edge + (torch.rand(200_000, generator=g) - 0.5) * 1e-3,
+                       -edge + (torch.rand(200_000, generator=g) - 0.5) * 1e-3,
+                       torch.tensor([0.0, -0.0, 30.0, -30.0, 88.0, -88.0, 100.0, -100.0, float("inf"), -float("inf")])])
+    a64 = alpha.numpy().astype(np.float64)
+    with np.errstate(over="ignore"):
+        sig64 = 1.0 / (1.0 + np.exp(-a64))
+    zeta_gamma, gamma = np.float64(np.float32(ada.ZETA - ada.GAMMA)), np.float64(np.float32(ada.GAMMA))
+    inner64 = sig64 * zeta_gamma + gamma
+    h64 = np.clip(inner64, 0, 1)
+    dh64 = np.where((inner64 >= 0) & (inner64 <= 1), zeta_gamma * sig64 * (1 - sig64), 0.0)
+    sig, h, dh = (t.cpu().numpy() for t in ops.adaround_eval_terms(alpha.cuda(), 0))
+    at = alpha.clone().requires_grad_(True)
+    ht = ada.rectified_sigmoid(at)
+    ht.sum().backward()
+    sig_t, h_t, dh_t = torch.sigmoid(alpha).numpy(), ht.detach().numpy(), at.grad.numpy()
+    assert np.isfinite(sig).all() and np.isfinite(h).all() and np.isfinite(dh).all()
+    assert np.array_equal(sig[-2:], [1.0, 0.0]) and np.array_equal(dh[-6:], np.zeros(6))
+    open_range = np.abs(a64) <= 2.5                      # where the clamp is open and sigmoid's value matters
+    inside = (inner64 > 1e-3) & (inner64 < 1 - 1e-3)
+    decided = inside | (inner64 < -1e-6) | (inner64 > 1 + 1e-6)
+    report = {
+        "sigmoid, |alpha| <= 2.5 [ulp]": (_ulps(sig, sig64)[open_range].max(), _ulps(sig_t, sig64)[open_range].max(), 4.0),
+        "sigmoid, |alpha| <= 12 [ulp]": (_ulps(sig, sig64)[np.abs(a64) <= 12].max(),
+                                         _ulps(sig_t, sig64)[np.abs(a64) <= 12].max(), 16.0),
+        "h [ulp(1)]": (np.abs(h - h64).max() / 2.0 ** -23, np.abs(h_t - h64).max() / 2.0 ** -23, 2.0),
+        "dh/dalpha [ulp]": (_ulps(dh, dh64)[inside].max(), _ulps(dh_t, dh64)[inside].max(), 8.0),
+    }
+    assert np.array_equal((dh == 0)[decided], (dh64 == 0)[decided])
+    # the regulariser's terms as functions of a float32 h
+    hh = torch.cat([torch.rand(2_000_000, generator=g), 0.5 + (torch.rand(300_000, generator=g) - 0.5) * 1e-3,
+                    torch.rand(200_000, generator=g) * 1e-3, 1 - torch.rand(200_000, generator=g) * 1e-3,
+                    torch.tensor([0.0, 1.0, 0.5, 0.25, 0.75, 2.0 ** -25, 0.5 + 2.0 ** -25])])
+    x32 = (2 * hh.numpy() - 1).astype(np.float32)       # the float32 2h - 1 every float32 implementation forms
+    x64 = np.abs(x32).astype(np.float64)
+    for beta in (2.0, 2.000492, 4.636038969321072, 11.0, 20.0):
+        b32, bm1 = np.float64(np.float32(beta)), np.float64(np.float32(beta - 1.0))   # torch's pow takes float32
+        reg64 = 1 - x64 ** b32
+        dreg64 = -b32 * x64 ** bm1 * np.sign(x32) * 2
+        reg, dreg = (t.cpu().numpy() for t in ops.adaround_eval_terms(hh.cuda(), 1, beta))
+        hv = hh.clone().requires_grad_(True)
+        rt = torch.add(1, -(torch.add(2 * hv, -1).abs()).pow(beta))
+        rt.sum().backward()
+        normal = np.abs(dreg64) > 1e-30
+        report[f"1 - |2h-1|^beta, beta {beta:g} [ulp(1)]"] = (np.abs(reg - reg64).max() / 2.0 ** -23,
+                                                             np.abs(rt.detach().numpy() - reg64).max() / 2.0 ** -23, 1.25)
+        report[f"d/dh of it, beta {beta:g} [ulp]"] = (_ulps(dreg, dreg64)[normal].max(),
+                                                      _ulps(hv.grad.numpy(), dreg64)[normal].max(), 2.5)
+        assert reg[-7] == 0 and reg[-6] == 0 and abs(dreg[-7]) == abs(dreg[-6]) == np.float32(2 * beta)   # h = 0, 1: |2h - 1| = 1
+    for name, (gpu, cpu, bound) in report.items():
+        print(f"{name:42s} gpu {gpu:7.2f}   torch cpu {cpu:7.2f}   bound {bound}")
+    for name, (gpu, cpu, bound) in report.items():
+        assert gpu <= bound, name
+
+
+def test_adam_update_against_torch_cpu(ops):
+    """30 updates with the kernel's own gradient output replayed through torch.optim.Adam on the CPU."""
+    torch.manual_seed(5)
+    O, K = 64, 512
+    w = torch.randn(O, K) * 0.05
+    delta, offset = (w.abs().amax(dim=1) * 1.7 / 15).float(), torch.full((O,), -8.0)
+    alpha = torch.randn(O, K) * 2
+    ag, mg, vg = alpha.cuda(), torch.zeros(O, K).cuda(), torch.zeros(O, K).cuda()
+    p = torch.nn.Parameter(alpha.clone())
+    opt = torch.optim.Adam([p])
+    for step in range(1, 31):
+        gw = torch.randn(O, K) * 10 ** float(torch.randn(1))
+        gout = torch.empty(O, K, device="cuda")
+        ops.adaround_bwd_adam(w.cuda(), gw.cuda(), ag, mg, vg, O, K, delta.cuda(), offset.cuda(), 0.0, 15.0, 0.01,
+                              20 - step * 0.5, 1e-3, 0.9, 0.999, 1e-8, step, grad_alpha=gout)
+        p.grad = gout.cpu()
+        opt.step()
+    state = opt.state[p]
+    assert torch.equal(mg.cpu(), state["exp_avg"]) and torch.equal(vg.cpu(), state["exp_avg_sq"])
+    diff = (ag.cpu() - p.detach()).numpy().astype(np.float64)
+    same = (diff == 0).mean()
+    # a differing update moves alpha by one ulp of alpha, or (alpha near zero) by the few 1e-7 of the lr-sized step that
+    # the one-ulp square root and reciprocal leave
+    allowed = np.maximum(2 * np.spacing(np.abs(p.detach().numpy())), 30 * 1e-3 * 1e-6)
+    print(f"alpha after 30 updates: identical {same:.5f}, largest difference {np.abs(diff).max():.3g}")
+    assert same > 0.97 and (np.abs(diff) <= allowed).all()
+
+
 @pytest.mark.parametrize("shape,ch_axis,per_channel", CASES[:4])
 @pytest.mark.parametrize("beta", [-1.0, 20.0, 4.636038969321072, 2.0])
 def test_alpha_gradient(ops, shape, ch_axis, per_channel, beta):
@@ -86,8 +190,20 @@ def test_alpha_gradient(ops, shape, ch_axis, per_channel, beta):
     partial = torch.zeros(ops.adaround_blocks(weight.numel()), device="cuda")
     got = ops.adaround_bwd(weight.cuda(), grad_w.cuda(), alpha.detach().cuda(), C, npc, delta.cuda(), offset.cuda(),
                            cmin, cmax, reg_param, beta, partial).cpu()
+    # the gradient is the float32 combination of the terms whose accuracy test_term_accuracy_in_ulp bounds:
+    #   (clip_min <= floor(w / delta) + h - offset <= clip_max ? grad_w delta dh : 0) + reg_param dreg dh
+    f32 = np.float32
+    _, h_g, dh_g = (t.cpu().numpy().reshape(weight.shape) for t in ops.adaround_eval_terms(alpha.detach().cuda(), 0))
+    dn, on = np.broadcast_to(d.numpy(), weight.shape), np.broadcast_to(o.numpy(), weight.shape)
+    t = np.floor(weight.numpy() / dn) + h_g - on
+    want = np.where((t >= f32(cmin)) & (t <= f32(cmax)), grad_w.numpy() * dn * dh_g, f32(0))
+    if beta >= 0:
+        _, dreg_g = ops.adaround_eval_terms(torch.from_numpy(h_g).cuda(), 1, beta)
+        want = want + f32(reg_param) * dreg_g.cpu().numpy().reshape(weight.shape) * dh_g
+    assert np.array_equal(got.numpy().view(np.uint32), want.astype(f32).view(np.uint32))
+    # against the restatement's autograd: up to the conditioning of |2h - 1|^(beta - 1) in h (see the module docstring)
     scale = alpha.grad.abs().max().item()
-    assert torch.allclose(got, alpha.grad, atol=1e-4 * scale, rtol=1e-4)
+    assert torch.allclose(got, alpha.grad, atol=2e-5 * scale, rtol=2e-5)
     # same zero pattern: the clamp masks are decided identically
     assert torch.equal(got == 0, alpha.grad == 0)
     if beta >= 0:
@@ -435,6 +551,82 @@ def test_cfg5_fused_linear_at_configured_size(ops):
     hard = ops.adaround_soft_round(wg, a.cuda(), O, K, dg, og, cmin, cmax, False).cpu()
     hard_ref = ada.apply_adaround(weight, a_ref, d, ada.broadcast(offset, weight, 0), cmin, cmax, False)
     assert ((hard == hard_ref).double().mean().item()) >= same - 1e-12
+
+
+@pytest.mark.parametrize("target_noise", [0.02, 0.0])
+def test_cfg5_whole_schedule(ops, target_noise, monkeypatch):
+    """All 1000 iterations of the AdaRound configuration (Linear [4096,4096], 2048 cached rows, 4-bit per-channel
+    symmetric min/max encodings, seed 1005, warm start 0.2, beta 20 -> 2) through the fused kernels, from the initial
+    alpha, against the restatement's torch ops, autograd and torch.optim.Adam on the same GPU and the same batches:
+    loss curves and the fraction of identical hard-rounding decisions at the end.
+
+    target_noise = 0.02: the target is the layer's output plus noise, so every iteration has a gradient that means
+    something: curves agree to 1e-5 and the decisions to 0.9999.
+    target_noise = 0: the configuration as written, the target is exactly what alpha's initial value reproduces (the
+    symmetric grid clips no weight), so for the 200 warm-start iterations the reconstruction gradient is the summation
+    noise of the GEMMs, which Adam normalises into full-size steps of random sign.  Any two summation orders then walk
+    apart: the yardstick is the restatement against itself with the layer's GEMM accumulated in float64 (the same sums,
+    rounded once instead of at every step)."""
+    O = K = 4096
+    rows, iters = 2048, 1000
+    hyper = (iters, 0.01, (20, 2), 0.2)
+    g = torch.Generator().manual_seed(1005)
+    weight = torch.randn(O, K, generator=g) * 0.02
+    X = torch.randn(rows, K, generator=g)
+    Y = torch.nn.functional.linear(X, weight)
+    if target_noise:
+        Y = Y + target_noise * torch.randn(rows, O, generator=g)
+    delta, offset = (weight.abs().amax(dim=1) / 7.0).float(), torch.full((O,), -8.0)
+    cmin, cmax = 0.0, 15.0
+    alpha0 = ada.generate_alpha(weight, ada.broadcast(delta, weight, 0))
+    batches = [torch.randperm(rows, generator=g)[:32] for _ in range(iters)]
+    wg, dg, og, Xg, Yg, a0g = (t.cuda() for t in (weight, delta, offset, X, Y, alpha0))
+
+    def restatement(batch_list):
+        trace = []
+        a, _, _, _ = ada.optimize_rounding("linear", wg, a0g, dg, og, cmin, cmax, Xg, Yg, batch_list, *hyper,
+                                           trace=trace)
+        return a, np.array(trace)
+
+    a_ref, curve_ref = restatement([b.cuda() for b in batches])
+    index = torch.stack(batches).to(torch.int32).cuda()
+    ws = ops.adaround_linear_workspace(O, K, "cuda")
+    f8 = ops.adaround_floor_i8(wg, O, K, dg, og, cmin, cmax)
+    alpha, m, v = a0g.clone(), torch.zeros(O, K, device="cuda"), torch.zeros(O, K, device="cuda")
+    gout = torch.empty(32, O, device="cuda")
+    recon = torch.zeros(iters, (32 * O + 255) // 256, device="cuda")
+    reg = torch.zeros(iters, ops.adaround_linear_blocks(O, K), device="cuda")
+    for k in range(iters):
+        beta = -1.0 if k < hyper[3] * iters else ada.compute_beta(iters, k, hyper[2], hyper[3])
+        ops.adaround_linear_fwd(f8, alpha, Xg, index[k], Yg, None, O, dg, og, cmin, cmax, 0, ws, gout,
+                                loss_partial=recon[k])
+        ops.adaround_linear_bwd_adam(f8, gout, Xg, index[k], alpha, m, v, O, dg, og, cmin, cmax, hyper[1], beta, 1e-3,
+                                     0.9, 0.999, 1e-8, k + 1, reg_partial=reg[k])
+    curve = np.stack([recon.double().sum(dim=1).cpu().numpy(), hyper[1] * reg.double().sum(dim=1).cpu().numpy()], 1)
+    same = ((alpha >= 0) == (a_ref >= 0)).double().mean().item()
+    late = slice(200, iters)
+    dev_recon = (np.abs(curve[late, 0] - curve_ref[late, 0]) / curve_ref[late, 0]).max()
+    dev_round = (np.abs(curve[late, 1] - curve_ref[late, 1]) / curve_ref[late, 1]).max()
+    print(f"cfg5 x 1000, target noise {target_noise}: identical hard-rounding decisions {same:.8f}; largest relative "
+          f"deviation of the loss curves after the warm start: reconstruction {dev_recon:.3g}, rounding {dev_round:.3g}; "
+          f"final losses {curve[-1, 0]:.6g} / {curve[-1, 1]:.6g} against {curve_ref[-1, 0]:.6g} / {curve_ref[-1, 1]:.6g}")
+    assert (a_ref - a0g).abs().mean() > 0.5              # the schedule did its work
+    assert curve[:200, 1].max() == 0 and curve_ref[:200, 1].max() == 0
+    if target_noise:
+        assert same >= 0.9999
+        assert dev_recon < 1e-5 and dev_round < 1e-5
+        assert np.abs(curve[:200, 0] - curve_ref[:200, 0]).max() < 1e-5 * curve_ref[:200, 0].max()
+    else:
+        monkeypatch.setattr(ada, "layer_output",
+                            lambda kind, inp, w, bias=None: (inp.double() @ w.double().t()).float())
+        a_f64, curve_f64 = restatement([b.cuda() for b in batches])
+        yardstick = ((a_f64 >= 0) == (a_ref >= 0)).double().mean().item()
+        dev_f64 = (np.abs(curve_f64[late, 0] - curve_ref[late, 0]) / curve_ref[late, 0]).max()
+        dev_round_f64 = (np.abs(curve_f64[late, 1] - curve_ref[late, 1]) / curve_ref[late, 1]).max()
+        print(f"   the restatement against itself with the GEMM accumulated in float64: {yardstick:.8f}, curves "
+              f"{dev_f64:.3g} / {dev_round_f64:.3g}")
+        assert same > 0.999 and same >= yardstick - 3e-4
+        assert dev_recon < max(2 * dev_f64, 5e-3) and dev_round < max(2 * dev_round_f64, 1e-4)
 
 
 class _TinyNet(torch.nn.Module):
