@@ -49,6 +49,15 @@ _SIGNATURES = {
     "miq_ste_bwd_per_tensor_bf16": ([_p, _p, _p, _i64, _flt, _flt, _p], _int),
     "miq_ste_bwd_per_channel_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _p], _int),
     "miq_ste_bwd_per_channel_bf16": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _p], _int),
+    "miq_ste_mask_bytes": ([_i64, _int], _i64),
+    "miq_qdq_mask_per_tensor_f32": ([_p, _p, _p, _i64, _dbl, _dbl, _int, _flt, _flt, _p], _int),
+    "miq_qdq_mask_per_tensor_bf16": ([_p, _p, _p, _i64, _dbl, _dbl, _int, _flt, _flt, _p], _int),
+    "miq_qdq_mask_per_channel_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _p], _int),
+    "miq_qdq_mask_per_channel_bf16": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _p, _p, _p, _p, _p], _int),
+    "miq_v2_qdq_mask_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p], _int),
+    "miq_v2_qdq_mask_bf16": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p], _int),
+    "miq_ste_bwd_mask_f32": ([_p, _p, _p, _i64, _p], _int),
+    "miq_ste_bwd_mask_bf16": ([_p, _p, _p, _i64, _p], _int),
     "miq_v2_qdq_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p], _int),
     "miq_v2_qdq_bf16": ([_p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p], _int),
     "miq_v2_qdq_bwd_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p], _int),

@@ -33,6 +33,9 @@ struct ParamSrc
     const float* b;   // v1: max      v2: offset
     const float* c;   // v1: delta
     const float* d;   // v1: offset
+    const float* e;   // v1 with a saved mask: the stored encoding's min (the straight-through bounds)
+    const float* f;   // v1 with a saved mask: the stored encoding's max
+    float2 raw;       // per-tensor: the same two values
     float4 scalar;    // per-tensor: the same four values
     float scalar_rcp; // per-tensor: RN(1/delta), or 0 when delta is outside the fast-division contract
     int qmin, qmax;   // v2 grid
@@ -87,6 +90,37 @@ struct OpV1Qdq : OpV1
     {
         float q = quant<FAST>(p, x);
         code    = (int) q - s.ishift;
+        return p.delta * (q + p.offset);
+    }
+};
+
+// y = QDQ(x) and, as the "code", whether x lies inside the stored encoding's [min, max]: the factor the straight-through
+// backward multiplies the gradient with (TORCH/v1/quantsim_straight_through_grad.py:100-118).  The kernel packs these
+// flags into the saved mask (one bit per element) instead of integer codes.
+struct V1PM
+{
+    float mn, mx, delta, offset, rcp, raw_min, raw_max;
+};
+struct OpV1QdqMask
+{
+    static constexpr bool kMask = true;
+    using P                  = V1PM;
+    static constexpr int NIN = 1;
+    using Code               = uint8_t;
+    __device__ static P load(const ParamSrc& s, uint32_t ch)
+    {
+        const V1P q = OpV1::load(s, ch);
+        return P{q.mn, q.mx, q.delta, q.offset, q.rcp, s.e[ch], s.f[ch]};
+    }
+    __device__ static bool fast_ok(const P& p, const float*, int)
+    {
+        return p.rcp != 0.0f;
+    }
+    template <bool FAST>
+    __device__ static float apply(const ParamSrc&, const P& p, float x, float, int& code)
+    {
+        const float q = OpV1::quant<FAST>(V1P{p.mn, p.mx, p.delta, p.offset, p.rcp}, x);
+        code          = (p.raw_min <= x) && (x <= p.raw_max);
         return p.delta * (q + p.offset);
     }
 };
@@ -220,6 +254,25 @@ struct OpV2Qdq : OpV2
     }
 };
 
+// The v2 forward with the mask its backward multiplies the gradient with (torch_builtins.py:303-327 saves exactly
+// this mask) as the "code"
+struct OpV2QdqMask : OpV2
+{
+    static constexpr bool kMask = true;
+    static constexpr int NIN = 1;
+    using Code               = int32_t;
+    template <bool FAST>
+    __device__ static float apply(const ParamSrc& s, const P& p, float x, float, int& code)
+    {
+        const float r = grid<FAST>(p, x);
+        code          = ((float) s.qmin <= r) && (r <= (float) s.qmax);
+        float q       = r;
+        q             = (q < (float) s.qmin) ? (float) s.qmin : q;
+        q             = (q > (float) s.qmax) ? (float) s.qmax : q;
+        return (q + p.offset) * p.scale;
+    }
+};
+
 struct OpV2Bwd : OpV2
 {
     static constexpr int NIN = 2;
@@ -253,8 +306,27 @@ struct NoNanOut<OpV1Qdq>
     }
 };
 
+template <>
+struct NoNanOut<OpV1QdqMask>
+{
+    __device__ static bool get(const V1PM& p)
+    {
+        return p.rcp != 0.0f && fabsf(p.offset) < INFINITY;
+    }
+};
+
 template <typename OP>
 __device__ typename OP::P scalar_params(const ParamSrc& s);
+template <>
+__device__ V1PM scalar_params<OpV1QdqMask>(const ParamSrc& s)
+{
+    return V1PM{s.scalar.x, s.scalar.y, s.scalar.z, s.scalar.w, s.scalar_rcp, s.raw.x, s.raw.y};
+}
+template <>
+__device__ V2P scalar_params<OpV2QdqMask>(const ParamSrc& s)
+{
+    return OpV2::load(s, 0);
+}
 template <>
 __device__ V1P scalar_params<OpV1Qdq>(const ParamSrc& s)
 {
@@ -319,7 +391,41 @@ struct EwPtrs
     const IO* g;    // second input (backward), else unused
     IO* y;          // may be null when only codes are wanted
     CodeT* codes;   // may be null
+    uint64_t* mask; // saved straight-through mask (mask ops only), else null
 };
+
+// ---- the saved straight-through mask ---------------------------------------------------------------------------
+// One bit per element, laid out for wavefront-wide compares: with V = the elements of a 16-byte vector (4 for
+// float32, 8 for bfloat16 storage) the elements are taken in groups of 64 V; group g owns the V consecutive 64-bit
+// words g V .. g V + V - 1, and bit t of word j is the flag of element 64 V g + V t + j -- element j of the vector
+// lane t of a wavefront holds, i.e. exactly what a compare over the wavefront leaves in a scalar register pair.  The
+// n % V elements after the last whole vector have their flags in bits 0 .. of one more word after the last group.
+template <int VEC>
+__host__ __device__ inline int64_t mask_groups(int64_t n)
+{
+    return (n / VEC + 63) / 64;
+}
+template <int VEC>
+__host__ __device__ inline int64_t mask_words(int64_t n)
+{
+    return mask_groups<VEC>(n) * VEC + 1;
+}
+
+// One group's V words from V wavefront-wide compares: lane j < V keeps word j and stores it.  (Written without an
+// array of words: the compiler moved such an array to LDS.)
+template <int VEC, typename FLAG>
+__device__ __forceinline__ void store_mask_group(uint64_t* dst, int lane, bool store, FLAG flag)
+{
+    uint64_t mine = 0;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+    {
+        const uint64_t w = __builtin_amdgcn_ballot_w64(flag(j));
+        mine             = (lane == j) ? w : mine;
+    }
+    if (store && lane < VEC)
+        __builtin_nontemporal_store(mine, dst + lane);
+}
 
 constexpr int kWin = 264;   // LDS window rows; host guarantees tile / elements-per-channel + 2 <= kWin
 
@@ -353,7 +459,8 @@ __device__ __forceinline__ void store_codes<int32_t, 8>(int32_t* dst, const int*
 
 // Vectorised tile kernel.  Requires 16-byte aligned pointers; n < 2^31 when PER_CHANNEL.  CODES: the integer codes are
 // stored too (ptr.codes is not null); without it their arithmetic (two operations per element) is not compiled in.
-template <typename IO, typename OP, bool PER_CHANNEL, int kUnroll, bool CODES>
+// MASK: the ops' "codes" are in-range flags, packed into ptr.mask (see above) instead of being stored as integers.
+template <typename IO, typename OP, bool PER_CHANNEL, int kUnroll, bool CODES, bool MASK = false>
 __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::Code> ptr, ParamSrc src, int64_t n,
                                                         uint32_t num_channel, FastDiv fd)
 {
@@ -485,6 +592,19 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
         if constexpr (CODES)
             store_codes<typename OP::Code, VEC>(ptr.codes + v * VEC, code[u]);
     }
+    if constexpr (MASK)
+    {
+        // every lane of the wavefront takes part in the compares; a wavefront whose first lane has no vector has none
+        const int wave = __builtin_amdgcn_readfirstlane((int) (threadIdx.x >> 6));
+        const int lane = threadIdx.x & 63;
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+        {
+            const int64_t v0 = e_base / VEC + (int64_t) u * kBlock + wave * 64;   // wavefront-uniform
+            store_mask_group<VEC>(ptr.mask + (v0 / 64) * VEC, lane, v0 < nvec,
+                                  [&](int j) { return live[u] && code[u][j] != 0; });
+        }
+    }
     // the n % VEC trailing elements
     if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * VEC))
     {
@@ -499,9 +619,18 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
             OP::template apply<false>(src, p, T::load1(ptr.x + e), OP::NIN == 2 ? T::load1(ptr.g + e) : 0.f, code);
         if (ptr.y)
             T::store1(ptr.y + e, y);
-        if (ptr.codes)
+        if constexpr (MASK)
+        {
+            const uint64_t w = __builtin_amdgcn_ballot_w64(code != 0);   // the active lanes are 0 .. n % VEC - 1
+            if (threadIdx.x == 0)
+                ptr.mask[mask_words<VEC>(n) - 1] = w;
+        }
+        else if (ptr.codes)
             ptr.codes[e] = (typename OP::Code) code;
     }
+    if constexpr (MASK)
+        if (blockIdx.x == 0 && threadIdx.x == 0 && n == nvec * VEC)
+            ptr.mask[mask_words<VEC>(n) - 1] = 0;   // no trailing elements: the word is still defined
 }
 
 // Fallback for unaligned pointers, tiny channels (elements-per-channel < 16) and n >= 2^31: one element per lane,
@@ -529,6 +658,191 @@ __global__ __launch_bounds__(kBlock) void ew_scalar_kernel(EwPtrs<IO, typename O
     }
 }
 
+// Mask-writing forward for what the tile kernel does not take (unaligned pointers, tiny channels, n >= 2^31): a
+// wavefront per mask group, lane t handling elements V t .. V t + V - 1 of the group one at a time, 64-bit indexing,
+// parameters read through the cache.  Same mask layout as the tile kernel.
+template <typename IO, typename OP, bool PER_CHANNEL>
+__global__ __launch_bounds__(kBlock) void ew_mask_group_kernel(EwPtrs<IO, typename OP::Code> ptr, ParamSrc src,
+                                                               int64_t n, int64_t num_channel, int64_t n_per_channel)
+{
+    using T           = IOTraits<IO>;
+    using P           = typename OP::P;
+    constexpr int VEC = T::VEC;
+    const int lane    = threadIdx.x & 63;
+    const int64_t nvec = n / VEC, groups = mask_groups<VEC>(n);
+    const int64_t wave0 = (int64_t) blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    for (int64_t grp = wave0; grp < groups; grp += (int64_t) gridDim.x * (kBlock / 64))
+    {
+        const int64_t v = grp * 64 + lane;
+        store_mask_group<VEC>(ptr.mask + grp * VEC, lane, true, [&](int j) {
+            int code = 0;
+            if (v < nvec)
+            {
+                const int64_t e = v * VEC + j;
+                P p;
+                if constexpr (PER_CHANNEL)
+                    p = OP::load(src, (uint32_t) ((e / n_per_channel) % num_channel));
+                else
+                    p = scalar_params<OP>(src);
+                T::store1(ptr.y + e, OP::template apply<false>(src, p, T::load1(ptr.x + e), 0.f, code));
+            }
+            return code != 0;
+        });
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * VEC))
+    {
+        const int64_t e = nvec * VEC + threadIdx.x;
+        P p;
+        if constexpr (PER_CHANNEL)
+            p = OP::load(src, (uint32_t) ((e / n_per_channel) % num_channel));
+        else
+            p = scalar_params<OP>(src);
+        int code;
+        T::store1(ptr.y + e, OP::template apply<false>(src, p, T::load1(ptr.x + e), 0.f, code));
+        const uint64_t w = __builtin_amdgcn_ballot_w64(code != 0);
+        if (threadIdx.x == 0)
+            ptr.mask[mask_words<VEC>(n) - 1] = w;
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0 && n == nvec * VEC)
+        ptr.mask[mask_words<VEC>(n) - 1] = 0;
+}
+
+// ---- straight-through backward from the saved mask: grad_in = grad_out * bit -------------------------------------
+// No parameters and no x: 4 bytes read + 1/8 byte of mask + 4 bytes written per float32 element (8.125 instead of the
+// 12 of the backward that recomputes the mask from x).  A wavefront's V mask words are one scalar load, and each word
+// is used as the lane mask of a select as it stands.
+template <typename IO, int kUnroll>
+__global__ __launch_bounds__(kBlock) void ste_mask_bwd_kernel(const uint64_t* __restrict__ mask,
+                                                              const IO* __restrict__ g, IO* __restrict__ gin, int64_t n)
+{
+    using T                 = IOTraits<IO>;
+    using Vec               = typename T::Vec;
+    constexpr int VEC       = T::VEC;
+    constexpr uint32_t TILE = kBlock * kUnroll * VEC;
+    const int64_t e_base    = (int64_t) blockIdx.x * TILE;
+    const int64_t nvec      = n / VEC;
+    const int wave          = __builtin_amdgcn_readfirstlane((int) (threadIdx.x >> 6));
+    Vec vg[kUnroll];
+    bool live[kUnroll];
+    const bool whole_tile = e_base / VEC + (int64_t) kUnroll * kBlock <= nvec;   // workgroup-uniform
+    if (whole_tile)
+    {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+        {
+            live[u] = true;
+            vg[u]   = stream_load(reinterpret_cast<const Vec*>(g) + e_base / VEC + (int64_t) u * kBlock + threadIdx.x);
+        }
+    }
+    else
+    {
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u)
+        {
+            const int64_t v = e_base / VEC + (int64_t) u * kBlock + threadIdx.x;
+            live[u]         = v < nvec;
+            if (live[u])
+                vg[u] = stream_load(reinterpret_cast<const Vec*>(g) + v);
+        }
+    }
+    uint64_t w[kUnroll][VEC];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+    {
+        const int64_t v0 = e_base / VEC + (int64_t) u * kBlock + wave * 64;   // wavefront-uniform
+        const uint64_t* mw = mask + (v0 / 64) * VEC;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            w[u][j] = (v0 < nvec) ? mw[j] : 0;
+    }
+    Vec out[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+    {
+        float fg[VEC], fy[VEC];
+        T::unpack(vg[u], fg);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+            fy[j] = fg[j] * (__builtin_amdgcn_inverse_ballot_w64(w[u][j]) ? 1.0f : 0.0f);
+        out[u] = T::pack(fy);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+        if (live[u])
+            stream_store(reinterpret_cast<Vec*>(gin) + e_base / VEC + (int64_t) u * kBlock + threadIdx.x, out[u]);
+    if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * VEC))
+    {
+        const int64_t e  = nvec * VEC + threadIdx.x;
+        const uint64_t t = mask[mask_words<VEC>(n) - 1];
+        T::store1(gin + e, T::load1(g + e) * (float) ((t >> threadIdx.x) & 1));
+    }
+}
+
+// the same for unaligned pointers: a wavefront per mask group, one element at a time
+template <typename IO>
+__global__ __launch_bounds__(kBlock) void ste_mask_bwd_group_kernel(const uint64_t* __restrict__ mask,
+                                                                    const IO* __restrict__ g, IO* __restrict__ gin,
+                                                                    int64_t n)
+{
+    using T           = IOTraits<IO>;
+    constexpr int VEC = T::VEC;
+    const int lane    = threadIdx.x & 63;
+    const int64_t nvec = n / VEC, groups = mask_groups<VEC>(n);
+    const int64_t wave0 = (int64_t) blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    for (int64_t grp = wave0; grp < groups; grp += (int64_t) gridDim.x * (kBlock / 64))
+    {
+        const int64_t v = grp * 64 + lane;
+        if (v < nvec)
+#pragma unroll
+            for (int j = 0; j < VEC; ++j)
+            {
+                const int64_t e = v * VEC + j;
+                T::store1(gin + e, T::load1(g + e) * (float) ((mask[grp * VEC + j] >> lane) & 1));
+            }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * VEC))
+    {
+        const int64_t e  = nvec * VEC + threadIdx.x;
+        const uint64_t t = mask[mask_words<VEC>(n) - 1];
+        T::store1(gin + e, T::load1(g + e) * (float) ((t >> threadIdx.x) & 1));
+    }
+}
+
+template <typename IO>
+int launch_ste_mask_bwd(const uint64_t* mask, const IO* g, IO* gin, int64_t n, hipStream_t stream)
+{
+    if (n == 0)
+        return MIQ_OK;
+    using T                = IOTraits<IO>;
+    constexpr int64_t TILE = (int64_t) kBlock * kUnroll * T::VEC;
+    if (aligned16(g) && aligned16(gin))
+    {
+        hipLaunchKernelGGL((ste_mask_bwd_kernel<IO, kUnroll>), dim3((unsigned) ((n + TILE - 1) / TILE)), dim3(kBlock), 0,
+                           stream, mask, g, gin, n);
+    }
+    else
+    {
+        int64_t blocks = (mask_groups<T::VEC>(n) + kBlock / 64 - 1) / (kBlock / 64);
+        blocks         = blocks < 1 ? 1 : (blocks > 65536 ? 65536 : blocks);
+        hipLaunchKernelGGL((ste_mask_bwd_group_kernel<IO>), dim3((unsigned) blocks), dim3(kBlock), 0, stream, mask, g, gin,
+                           n);
+    }
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+// whether OP's codes are straight-through flags (the mask-writing kernels are compiled for these only)
+template <typename OP, typename = void>
+struct WritesMask
+{
+    static constexpr bool value = false;
+};
+template <typename OP>
+struct WritesMask<OP, decltype((void) OP::kMask)>
+{
+    static constexpr bool value = true;
+};
+
 template <typename IO, typename OP, bool PER_CHANNEL>
 int launch_ew(EwPtrs<IO, typename OP::Code> ptr, const ParamSrc& src, int64_t n, int64_t num_channel,
               int64_t n_per_channel, hipStream_t stream)
@@ -550,12 +864,22 @@ int launch_ew(EwPtrs<IO, typename OP::Code> ptr, const ParamSrc& src, int64_t n,
     {
         const int64_t blocks = (n + TILE - 1) / TILE;
         FastDiv fd           = make_fastdiv(PER_CHANNEL ? (uint32_t) n_per_channel : 1u);
-        if (ptr.codes)
+        if constexpr (WritesMask<OP>::value)
+            hipLaunchKernelGGL((ew_vec_kernel<IO, OP, PER_CHANNEL, U, false, true>), dim3((unsigned) blocks),
+                               dim3(kBlock), 0, stream, ptr, src, n, (uint32_t) num_channel, fd);
+        else if (ptr.codes)
             hipLaunchKernelGGL((ew_vec_kernel<IO, OP, PER_CHANNEL, U, true>), dim3((unsigned) blocks), dim3(kBlock), 0,
                                stream, ptr, src, n, (uint32_t) num_channel, fd);
         else
             hipLaunchKernelGGL((ew_vec_kernel<IO, OP, PER_CHANNEL, U, false>), dim3((unsigned) blocks), dim3(kBlock), 0,
                                stream, ptr, src, n, (uint32_t) num_channel, fd);
+    }
+    else if constexpr (WritesMask<OP>::value)
+    {
+        int64_t blocks = (mask_groups<T::VEC>(n) + kBlock / 64 - 1) / (kBlock / 64);
+        blocks         = blocks < 1 ? 1 : (blocks > 65536 ? 65536 : blocks);
+        hipLaunchKernelGGL((ew_mask_group_kernel<IO, OP, PER_CHANNEL>), dim3((unsigned) blocks), dim3(kBlock), 0, stream,
+                           ptr, src, n, num_channel, n_per_channel);
     }
     else
     {
@@ -729,6 +1053,52 @@ static ParamSrc v2_src(const float* scale, const float* offset, int qmin, int qm
 }   // namespace miq
 
 using namespace miq;
+
+template <typename IO>
+static int qdq_mask_per_tensor(const IO* in, IO* out, uint64_t* mask, int64_t n, double enc_min, double enc_max, int bw,
+                               float mask_min, float mask_max, void* stream)
+{
+    MIQ_CHECK_ARG(n >= 0 && (n == 0 || (in && out && mask)), "null tensor pointer or negative count");
+    MIQ_CHECK_ARG((reinterpret_cast<uintptr_t>(mask) & 7u) == 0, "the mask must be 8-byte aligned");
+    miq_encoding e;
+    if (int rc = miq_fill_encoding_info(bw, enc_min, enc_max, &e))
+        return rc;
+    ParamSrc s = per_tensor_src(e);
+    s.raw      = make_float2(mask_min, mask_max);
+    EwPtrs<IO, uint8_t> p{in, nullptr, out, nullptr, mask};
+    return launch_ew<IO, OpV1QdqMask, false>(p, s, n, 1, 1, (hipStream_t) stream);
+}
+
+template <typename IO>
+static int qdq_mask_per_channel(const IO* in, IO* out, uint64_t* mask, int64_t num_channel, int64_t num_element,
+                                int64_t npc, const float* enc_min, const float* enc_max, const float* enc_delta,
+                                const float* enc_offset, const float* raw_min, const float* raw_max, void* stream)
+{
+    if (int rc = check_channels(num_channel, num_element, npc))
+        return rc;
+    MIQ_CHECK_ARG(num_element == 0 || (in && out && mask && enc_min && enc_max && enc_delta && enc_offset && raw_min &&
+                                       raw_max),
+                  "null pointer");
+    MIQ_CHECK_ARG((reinterpret_cast<uintptr_t>(mask) & 7u) == 0, "the mask must be 8-byte aligned");
+    ParamSrc s = v1_channel_src(enc_min, enc_max, enc_delta, enc_offset);
+    s.e        = raw_min;
+    s.f        = raw_max;
+    EwPtrs<IO, uint8_t> p{in, nullptr, out, nullptr, mask};
+    return launch_ew<IO, OpV1QdqMask, true>(p, s, num_element, num_channel, npc, (hipStream_t) stream);
+}
+
+template <typename IO>
+static int v2_qdq_mask(const IO* in, IO* out, uint64_t* mask, int64_t num_channel, int64_t num_element, int64_t npc,
+                       const float* scale, const float* offset, int qmin, int qmax, void* stream)
+{
+    if (int rc = check_v2(num_channel, num_element, npc, scale, offset, qmin, qmax))
+        return rc;
+    MIQ_CHECK_ARG(num_element == 0 || (in && out && mask), "null pointer");
+    MIQ_CHECK_ARG((reinterpret_cast<uintptr_t>(mask) & 7u) == 0, "the mask must be 8-byte aligned");
+    EwPtrs<IO, int32_t> p{in, nullptr, out, nullptr, mask};
+    return launch_v2<IO, OpV2QdqMask>(p, v2_src(scale, offset, qmin, qmax), num_element, num_channel, npc,
+                                      (hipStream_t) stream);
+}
 
 extern "C" {
 
@@ -1012,6 +1382,75 @@ int miq_v2_qdq_bwd_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* g
     EwPtrs<uint16_t, int32_t> p{x, grad_out, grad_in, nullptr};
     return launch_v2<uint16_t, OpV2Bwd>(p, v2_src(scale, offset, qmin, qmax), num_element, num_channel,
                                         num_element_per_channel, (hipStream_t) stream);
+}
+
+/* ---- forward with the saved straight-through mask, backward from the mask ----------------------------------- */
+
+int64_t miq_ste_mask_bytes(int64_t num_element, int elem_bytes)
+{
+    if (num_element < 0 || (elem_bytes != 4 && elem_bytes != 2))
+        return -1;
+    return 8 * (elem_bytes == 4 ? mask_words<4>(num_element) : mask_words<8>(num_element));
+}
+
+int miq_qdq_mask_per_tensor_f32(const float* in, float* out, uint64_t* mask, int64_t n, double enc_min, double enc_max,
+                                int bw, float mask_min, float mask_max, void* stream)
+{
+    return qdq_mask_per_tensor<float>(in, out, mask, n, enc_min, enc_max, bw, mask_min, mask_max, stream);
+}
+
+int miq_qdq_mask_per_tensor_bf16(const uint16_t* in, uint16_t* out, uint64_t* mask, int64_t n, double enc_min,
+                                 double enc_max, int bw, float mask_min, float mask_max, void* stream)
+{
+    return qdq_mask_per_tensor<uint16_t>(in, out, mask, n, enc_min, enc_max, bw, mask_min, mask_max, stream);
+}
+
+int miq_qdq_mask_per_channel_f32(const float* in, float* out, uint64_t* mask, int64_t num_channel, int64_t num_element,
+                                 int64_t num_element_per_channel, const float* enc_min, const float* enc_max,
+                                 const float* enc_delta, const float* enc_offset, const float* raw_min,
+                                 const float* raw_max, void* stream)
+{
+    return qdq_mask_per_channel<float>(in, out, mask, num_channel, num_element, num_element_per_channel, enc_min,
+                                       enc_max, enc_delta, enc_offset, raw_min, raw_max, stream);
+}
+
+int miq_qdq_mask_per_channel_bf16(const uint16_t* in, uint16_t* out, uint64_t* mask, int64_t num_channel,
+                                  int64_t num_element, int64_t num_element_per_channel, const float* enc_min,
+                                  const float* enc_max, const float* enc_delta, const float* enc_offset,
+                                  const float* raw_min, const float* raw_max, void* stream)
+{
+    return qdq_mask_per_channel<uint16_t>(in, out, mask, num_channel, num_element, num_element_per_channel, enc_min,
+                                          enc_max, enc_delta, enc_offset, raw_min, raw_max, stream);
+}
+
+int miq_v2_qdq_mask_f32(const float* in, float* out, uint64_t* mask, int64_t num_channel, int64_t num_element,
+                        int64_t num_element_per_channel, const float* scale, const float* offset, int qmin, int qmax,
+                        void* stream)
+{
+    return v2_qdq_mask<float>(in, out, mask, num_channel, num_element, num_element_per_channel, scale, offset, qmin,
+                              qmax, stream);
+}
+
+int miq_v2_qdq_mask_bf16(const uint16_t* in, uint16_t* out, uint64_t* mask, int64_t num_channel, int64_t num_element,
+                         int64_t num_element_per_channel, const float* scale, const float* offset, int qmin, int qmax,
+                         void* stream)
+{
+    return v2_qdq_mask<uint16_t>(in, out, mask, num_channel, num_element, num_element_per_channel, scale, offset, qmin,
+                                 qmax, stream);
+}
+
+int miq_ste_bwd_mask_f32(const uint64_t* mask, const float* grad_out, float* grad_in, int64_t n, void* stream)
+{
+    MIQ_CHECK_ARG(n >= 0 && (n == 0 || (mask && grad_out && grad_in)), "null tensor pointer or negative count");
+    MIQ_CHECK_ARG((reinterpret_cast<uintptr_t>(mask) & 7u) == 0, "the mask must be 8-byte aligned");
+    return launch_ste_mask_bwd<float>(mask, grad_out, grad_in, n, (hipStream_t) stream);
+}
+
+int miq_ste_bwd_mask_bf16(const uint64_t* mask, const uint16_t* grad_out, uint16_t* grad_in, int64_t n, void* stream)
+{
+    MIQ_CHECK_ARG(n >= 0 && (n == 0 || (mask && grad_out && grad_in)), "null tensor pointer or negative count");
+    MIQ_CHECK_ARG((reinterpret_cast<uintptr_t>(mask) & 7u) == 0, "the mask must be 8-byte aligned");
+    return launch_ste_mask_bwd<uint16_t>(mask, grad_out, grad_in, n, (hipStream_t) stream);
 }
 
 }   // extern "C"

@@ -324,6 +324,77 @@ def ste_bwd_per_channel(x, grad_out, num_channel, n_per_channel, enc_min, enc_ma
     return gin
 
 
+# ------------------------------------------------------------------------------------- saved straight-through mask
+def _new_mask(x):
+    """Device buffer for the one-bit-per-element straight-through mask of `x` (int64 words, never initialised: the
+    forward writes every word the backward reads)."""
+    nbytes = int(lib.miq_ste_mask_bytes(x.numel(), x.element_size()))
+    return torch.empty(nbytes // 8, dtype=torch.int64, device=x.device)
+
+
+def _out_and_mask(x, out, mask):
+    if mask is not None and (mask.dtype != torch.int64 or
+                             mask.numel() * 8 != int(lib.miq_ste_mask_bytes(x.numel(), x.element_size()))):
+        raise RuntimeError("the mask buffer does not fit a tensor of this size and dtype")
+    return (torch.empty_like(x) if out is None else out), (_new_mask(x) if mask is None else mask)
+
+
+def qdq_mask_per_tensor(x, enc_min, enc_max, bw, mask_min=None, mask_max=None, out=None, mask=None):
+    """qdq_per_tensor (nearest rounding) that also returns the mask ste_bwd_mask multiplies the gradient with:
+    mask_min <= x <= mask_max, by default the encoding's bounds as ste_bwd_per_tensor would take them."""
+    _require_gpu(x, out, mask)
+    x = x.contiguous()
+    out, mask = _out_and_mask(x, out, mask)
+    fn = getattr(lib, "miq_qdq_mask_per_tensor_" + _suffix(x))
+    mask_min = float(enc_min) if mask_min is None else float(mask_min)
+    mask_max = float(enc_max) if mask_max is None else float(mask_max)
+    with _OnDevice(x.device):
+        check(fn(_ptr(x), _ptr(out), _ptr(mask), x.numel(), float(enc_min), float(enc_max), int(bw), mask_min,
+                 mask_max, _stream(x)))
+    return out, mask
+
+
+def qdq_mask_per_channel(x, num_channel, n_per_channel, mn, mx, delta, offset, raw_min, raw_max, out=None, mask=None):
+    """qdq_per_channel (nearest rounding) + mask; raw_min / raw_max are the stored encodings' bounds, the ones
+    ste_bwd_per_channel compares with."""
+    _require_gpu(x, mn, mx, delta, offset, raw_min, raw_max, out, mask)
+    x = x.contiguous()
+    out, mask = _out_and_mask(x, out, mask)
+    fn = getattr(lib, "miq_qdq_mask_per_channel_" + _suffix(x))
+    raw_min, raw_max = _params_f32(raw_min, x), _params_f32(raw_max, x)
+    with _OnDevice(x.device):
+        check(fn(_ptr(x), _ptr(out), _ptr(mask), int(num_channel), x.numel(), int(n_per_channel), _ptr(mn), _ptr(mx),
+                 _ptr(delta), _ptr(offset), _ptr(raw_min), _ptr(raw_max), _stream(x)))
+    return out, mask
+
+
+def v2_qdq_mask(x, num_channel, n_per_channel, scale, offset, qmin, qmax, out=None, mask=None):
+    """v2_qdq + the mask of its backward (qmin <= round(x / scale) - offset <= qmax)."""
+    _require_gpu(x, scale, offset)
+    x = x.contiguous()
+    scale, offset = _params_f32(scale, x).reshape(-1), _params_f32(offset, x).reshape(-1)
+    out, mask = _out_and_mask(x, out, mask)
+    fn = getattr(lib, "miq_v2_qdq_mask_" + _suffix(x))
+    with _OnDevice(x.device):
+        check(fn(_ptr(x), _ptr(out), _ptr(mask), int(num_channel), x.numel(), int(n_per_channel), _ptr(scale),
+                 _ptr(offset), int(qmin), int(qmax), _stream(x)))
+    return out, mask
+
+
+def ste_bwd_mask(mask, grad_out, out=None):
+    """grad_out * bit, from the mask a *_mask forward wrote for a tensor of grad_out's dtype and element count."""
+    _require_gpu(grad_out, mask, out)
+    grad_out = grad_out.contiguous()
+    if mask.dtype != torch.int64 or mask.numel() * 8 != int(lib.miq_ste_mask_bytes(grad_out.numel(),
+                                                                                   grad_out.element_size())):
+        raise RuntimeError("the mask does not belong to a tensor of this size and dtype")
+    gin = torch.empty_like(grad_out) if out is None else out
+    fn = getattr(lib, "miq_ste_bwd_mask_" + _suffix(grad_out))
+    with _OnDevice(grad_out.device):
+        check(fn(_ptr(mask), _ptr(grad_out), _ptr(gin), grad_out.numel(), _stream(grad_out)))
+    return gin
+
+
 # ------------------------------------------------------------------------------------------------------------ v2 QDQ
 def v2_qdq(x, num_channel, n_per_channel, scale, offset, qmin, qmax, want_codes=False):
     _require_gpu(x, scale, offset)

@@ -406,9 +406,14 @@ def _channel_geometry(tensor, ch_axis):
     return num_channel, n_per_channel
 
 
+def _is_nearest(round_mode) -> bool:
+    value = round_mode.value if isinstance(round_mode, libpymo.RoundingMode) else round_mode
+    return int(value) == int(libpymo.RoundingMode.ROUND_NEAREST.value)
+
+
 class _NoContext:
     """Stands in for the autograd context when QuantizeDequantize.forward is called directly (no gradient)."""
-    __slots__ = ("tensor_quantizer",)
+    __slots__ = ("tensor_quantizer", "masked")
 
     def save_for_backward(self, *_):
         pass
@@ -455,18 +460,54 @@ class QuantizeDequantize(torch.autograd.Function):
             return ops.fp16_round_trip(tensor)
         return tensor.half().float()
 
+    # The backward needs one bit per element: whether the input lay inside the stored encoding's range.  When the
+    # input wants a gradient the forward writes those bits itself (ops.qdq_mask_*) and keeps them instead of the
+    # input -- 1/8 byte per element instead of 4, and the backward reads 1/8 byte instead of the input again.  The
+    # reference keeps the input and compares in backward (reference :1186-1212); the results are the same bit for bit
+    # as long as the encoding is not changed between the two passes.  False: keep the input, as the reference does.
+    save_mask = True
+
+    @staticmethod
+    def _masked_forward(tensor, tensor_quantizer):
+        """(quantized, mask) through the mask-writing forward, or None where it does not apply."""
+        if not (tensor.is_cuda and tensor.dtype in (torch.float32, torch.bfloat16) and tensor.is_contiguous()):
+            return None
+        if isinstance(tensor_quantizer, StaticGridPerChannelQuantizer):
+            num_channel, n_per_channel = _channel_geometry(tensor, tensor_quantizer.channel_axis)
+            mn, mx, delta, offset, raw_min, raw_max = tensor_quantizer.device_params(tensor.device)
+            return ops.qdq_mask_per_channel(tensor, num_channel, n_per_channel, mn, mx, delta, offset, raw_min,
+                                            raw_max)
+        enc = tensor_quantizer.encoding
+        mask_min, mask_max = enc.min, enc.max
+        if tensor.dtype != torch.float32:
+            # the reference compares against a 0-dim tensor, which torch's type promotion casts to x's dtype
+            mask_min = float(torch.tensor(mask_min, dtype=torch.float32).to(tensor.dtype))
+            mask_max = float(torch.tensor(mask_max, dtype=torch.float32).to(tensor.dtype))
+        return ops.qdq_mask_per_tensor(tensor, enc.min, enc.max, enc.bw, mask_min, mask_max)
+
     @staticmethod
     def forward(ctx, tensor, tensor_quantizer, round_mode):  # pylint: disable=arguments-differ
+        ctx.masked = False
         if tensor_quantizer.enabled and tensor_quantizer.bitwidth != 32:
-            if tensor_quantizer.data_type == QuantizationDataType.float:
-                quantized = QuantizeDequantize._quantize_float(tensor, tensor_quantizer)
-            elif isinstance(tensor_quantizer, StaticGridPerChannelQuantizer):
-                quantized = QuantizeDequantize._per_channel_quantize_dequantize(tensor, tensor_quantizer, round_mode)
+            masked = None
+            if QuantizeDequantize.save_mask and tensor_quantizer.data_type == QuantizationDataType.int and \
+                    getattr(ctx, "needs_input_grad", (False,))[0] and _is_nearest(round_mode):
+                masked = QuantizeDequantize._masked_forward(tensor, tensor_quantizer)
+            if masked is not None:
+                quantized, mask = masked
+                ctx.masked = True
+                ctx.save_for_backward(mask)
             else:
-                dtype = tensor.dtype
-                quantized = QuantizeDequantize._per_tensor_quantize_dequantize(tensor, tensor_quantizer,
-                                                                               round_mode).to(dtype)
-            ctx.save_for_backward(tensor)
+                if tensor_quantizer.data_type == QuantizationDataType.float:
+                    quantized = QuantizeDequantize._quantize_float(tensor, tensor_quantizer)
+                elif isinstance(tensor_quantizer, StaticGridPerChannelQuantizer):
+                    quantized = QuantizeDequantize._per_channel_quantize_dequantize(tensor, tensor_quantizer,
+                                                                                    round_mode)
+                else:
+                    dtype = tensor.dtype
+                    quantized = QuantizeDequantize._per_tensor_quantize_dequantize(tensor, tensor_quantizer,
+                                                                                   round_mode).to(dtype)
+                ctx.save_for_backward(tensor)
         else:
             quantized = tensor
         ctx.tensor_quantizer = tensor_quantizer
@@ -475,7 +516,10 @@ class QuantizeDequantize(torch.autograd.Function):
     @staticmethod
     def backward(ctx, output_grad):  # pylint: disable=arguments-differ
         q = ctx.tensor_quantizer
-        if q.enabled and q.data_type == QuantizationDataType.int and q.bitwidth != 32:
+        if ctx.masked:
+            mask, = ctx.saved_tensors
+            grad = ops.ste_bwd_mask(mask, output_grad)
+        elif q.enabled and q.data_type == QuantizationDataType.int and q.bitwidth != 32:
             tensor, = ctx.saved_tensors
             if isinstance(q, StaticGridPerChannelQuantizer):
                 _, _, _, _, raw_min, raw_max = q.device_params(tensor.device)

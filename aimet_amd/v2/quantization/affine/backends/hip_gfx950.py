@@ -8,8 +8,8 @@ Same functions, argument meaning and error behaviour as the reference's torch_bu
     quantize_dequantize out = (clamp(round_half_even(x / scale) - offset, qmin, qmax) + offset) * scale
 
 The forward of quantize / quantize_dequantize is one fused kernel (the reference runs about seven elementwise ATen
-kernels and saves a bool mask); the input gradient is one fused kernel that recomputes the mask from the saved
-input.  float32 and bfloat16 tensors are computed in float32, as the reference does for 4- and 8-bit grids; other
+kernels and saves a bool mask); the input gradient is one fused kernel: from a one-bit-per-element mask the forward
+wrote when only the input wants a gradient, else recomputing the mask from the saved input.  float32 and bfloat16 tensors are computed in float32, as the reference does for 4- and 8-bit grids; other
 float types are upcast to float32.
 
 Scale / offset may be per-tensor, per-channel, vary along several axes, or be blockwise (`block_size`, reference
@@ -89,16 +89,30 @@ def _reduce_like(grad: torch.Tensor, shape) -> torch.Tensor:
 
 
 class _QuantDequantFunc(torch.autograd.Function):
+    # When only the input wants a gradient (static scale / offset) the forward writes the backward's mask itself, one
+    # bit per element, and keeps that instead of the input; the reference keeps the same mask as a bool tensor, one
+    # byte per element (torch_builtins.py:303-327).  False: keep the input and recompute the mask in backward.
+    save_mask = True
+
     @staticmethod
     def forward(ctx, tensor, scale, offset, qmin, qmax):  # pylint: disable=arguments-differ
         c, npc = _channel_geometry(tensor.shape, scale.shape)
-        out = ops.v2_qdq(tensor, c, npc, scale, offset, qmin, qmax)
         ctx.geom = (c, npc, qmin, qmax)
+        ctx.masked = _QuantDequantFunc.save_mask and ctx.needs_input_grad[0] and \
+            not (ctx.needs_input_grad[1] or ctx.needs_input_grad[2])
+        if ctx.masked:
+            out, mask = ops.v2_qdq_mask(tensor, c, npc, scale, offset, qmin, qmax)
+            ctx.save_for_backward(mask)
+            return out
+        out = ops.v2_qdq(tensor, c, npc, scale, offset, qmin, qmax)
         ctx.save_for_backward(tensor, scale, offset)
         return out
 
     @staticmethod
     def backward(ctx, grad):  # pylint: disable=arguments-differ
+        if ctx.masked:
+            mask, = ctx.saved_tensors
+            return ops.ste_bwd_mask(mask, grad), None, None, None, None
         tensor, scale, offset = ctx.saved_tensors
         c, npc, qmin, qmax = ctx.geom
         tensor_grad = scale_grad = offset_grad = None

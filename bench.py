@@ -120,6 +120,18 @@ def _graph_replay_ms(torch, fn, sets, launches):
         return None
 
 
+def _saved_mask_figures(wall, f, b, n, esz):
+    """Bytes the saved-mask step moves: forward reads x, writes y and n / 8 bytes of mask; backward reads the
+    gradient and the mask, writes the input gradient.  GB/s on those bytes; and what the same time would be worth on
+    the 5-accesses-per-element formulation the other figures use."""
+    fwd_bytes, bwd_bytes = 2 * esz * n + n / 8, 2 * esz * n + n / 8
+    return {"ms_per_step": wall, "fwd_ms": f, "bwd_ms": b, "bytes_moved_per_step": fwd_bytes + bwd_bytes,
+            "fwd_GBps_moved": fwd_bytes / f / 1e6, "bwd_GBps_moved": bwd_bytes / b / 1e6,
+            "fwd_bwd_GBps_moved": (fwd_bytes + bwd_bytes) / wall / 1e6,
+            "frac_hbm_moved": (fwd_bytes + bwd_bytes) / wall / 1e6 / HBM_PEAK_GBPS,
+            "fwd_bwd_GBps_on_recompute_formulation": 5 * esz * n / wall / 1e6}
+
+
 def bench_per_channel(torch, ops, shape, dtype, bw, steps, warmup, seed, nsets=3):
     dev = torch.device("cuda", 0)
     c, npc = shape[0], 1
@@ -151,6 +163,18 @@ def bench_per_channel(torch, ops, shape, dtype, bw, steps, warmup, seed, nsets=3
            "ms_per_step": wall, "fwd_ms": f, "bwd_ms": b,
            "fwd_GBps": 2 * esz * n / f / 1e6, "bwd_GBps": 3 * esz * n / b / 1e6,
            "fwd_bwd_GBps": 5 * esz * n / wall / 1e6, "buffer_sets": nsets}
+    # the same step with the straight-through mask saved by the forward, one bit per element, and read by the
+    # backward instead of x
+    masks = [ops._new_mask(s[0]) for s in sets]                      # pylint: disable=protected-access
+
+    def fwd_m(s):
+        ops.qdq_mask_per_channel(s[0], c, npc, mn, mx, delta, offset, emin, emax, out=s[2], mask=s[4])
+
+    def bwd_m(s):
+        ops.ste_bwd_mask(s[4], s[1], out=s[3])
+
+    msets = [s + (m,) for s, m in zip(sets, masks)]
+    out["saved_mask"] = _saved_mask_figures(*_time_fwd_bwd(torch, fwd_m, bwd_m, msets, steps, warmup), n, esz)
     if n < 2e7:
         # host-paced above; the same launches replayed from a HIP graph
         gf = _graph_replay_ms(torch, fwd, sets, min(64, 4 * nsets))
@@ -223,6 +247,19 @@ def bench_per_tensor(torch, ops, steps, warmup):
     if gf and gb:
         out["graph_replay"] = {"fwd_ms": gf, "bwd_ms": gb, "fwd_bwd_GBps": 20 * n / (gf + gb) / 1e6,
                                "frac_hbm": 20 * n / (gf + gb) / 1e6 / HBM_PEAK_GBPS}
+    # the same step with the straight-through mask saved by the forward (one bit per element)
+    msets = [s + (ops._new_mask(s[0]),) for s in sets]              # pylint: disable=protected-access
+
+    def fwd_m(s):
+        ops.qdq_mask_per_tensor(s[0], e.min, e.max, 8, out=s[2], mask=s[4])
+
+    def bwd_m(s):
+        ops.ste_bwd_mask(s[4], s[1], out=s[3])
+
+    out["saved_mask"] = _saved_mask_figures(*_time_fwd_bwd(torch, fwd_m, bwd_m, msets, max(steps, 100), warmup), n, 4)
+    gf, gb = _graph_replay_ms(torch, fwd_m, msets, 64), _graph_replay_ms(torch, bwd_m, msets, 64)
+    if gf and gb:
+        out["saved_mask"]["graph_replay"] = {"fwd_ms": gf, "bwd_ms": gb, "ms_per_step": gf + gb}
     # the same region with one buffer set: 103 MB of operands, served by the 256 MB last-level cache
     one = sets[:1]
     wall1, f1, b1 = _time_fwd_bwd(torch, fwd, bwd, one, max(steps, 100), warmup)
@@ -1098,6 +1135,8 @@ def main():
                                         "avg_launch_ms": res["fwd_ms"], "algorithmic_bytes_per_launch": 8 * n,
                                         "traffic": MEASURED_TRAFFIC_BYTES["qdq_fwd_per_channel_f32"]}},
     }
+    line["saved_mask_step"] = dict(res["saved_mask"], note="the same fwd+bwd step with the forward writing the "
+                                   "straight-through mask (1 bit per element) and the backward reading it instead of x")
     if "tf_enhanced_calibration" in extra:
         line["calib_elements_per_s"] = extra["tf_enhanced_calibration"]["elements_per_s"]
     if not args.no_cpu:

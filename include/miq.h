@@ -171,6 +171,54 @@ int miq_ste_bwd_per_channel_bf16(const uint16_t* x, const uint16_t* grad_out, ui
                                  const float* enc_min, const float* enc_max, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
+ * Straight-through estimator through a saved one-bit mask.
+ * The reference's v2 QuantDequantFunc saves the mask of its backward as a bool tensor, one byte per element
+ * (TORCH/v2/quantization/affine/backends/torch_builtins.py:303-327); its v1 QuantizeDequantize keeps the input alive
+ * and recomputes the comparison (TORCH/v1/tensor_quantizer.py:1098-1212, quantsim_straight_through_grad.py:100-118).
+ * Here the forward can write the mask with one BIT per element and the backward reads it instead of x: per float32
+ * element 8.125 + 8.125 bytes instead of 8 + 12, and 1/8 byte kept between the passes instead of 4.
+ * The miq_*_mask_* forwards compute exactly what their counterparts without "mask" compute, and mask bit = the factor
+ * the matching backward would multiply the gradient with: (min <= x && x <= max) on the float32 casts of the stored
+ * encoding's min / max for v1 (what miq_ste_bwd_per_*_* is given), qmin <= round(x / scale) - offset <= qmax for v2.
+ * miq_ste_bwd_mask_* then gives grad_in = grad_out * bit, bit for bit what miq_ste_bwd_per_*_* / miq_v2_qdq_bwd_* give.
+ * Mask layout (the same for every entry point of one storage type): with V = 4 (float32) or 8 (bfloat16) the elements
+ * are taken in groups of 64 V; group g owns the 64-bit words g V .. g V + V - 1, and bit t of word j belongs to element
+ * 64 V g + V t + j; the num_element % V elements after the last whole 16-byte vector have their bits in bits 0.. of
+ * one more word after the last group.  mask: device memory of miq_ste_mask_bytes() bytes, 8-byte aligned.
+ * Nearest rounding only (the stochastic mode keeps the recomputing backward).
+ * ------------------------------------------------------------------------------------------------------------- */
+/* Bytes of the mask for num_element elements stored in elem_bytes bytes each (4: float32, 2: bfloat16); -1 on
+ * invalid arguments. */
+int64_t miq_ste_mask_bytes(int64_t num_element, int elem_bytes);
+/* miq_qdq_per_tensor_* + mask; mask_min / mask_max: the bounds the matching miq_ste_bwd_per_tensor_* call would be
+ * given (the stored encoding's min / max as float32; for a bfloat16 tensor the reference's comparison casts them to
+ * bfloat16, quantsim_straight_through_grad.py:115 with torch's promotion of a 0-dim tensor). */
+int miq_qdq_mask_per_tensor_f32(const float* in, float* out, uint64_t* mask, int64_t n, double enc_min, double enc_max,
+                                int bw, float mask_min, float mask_max, void* stream);
+int miq_qdq_mask_per_tensor_bf16(const uint16_t* in, uint16_t* out, uint64_t* mask, int64_t n, double enc_min,
+                                 double enc_max, int bw, float mask_min, float mask_max, void* stream);
+/* miq_qdq_per_channel_* + mask; raw_min / raw_max: device float[num_channel], the stored encodings' min / max (the
+ * vectors miq_ste_bwd_per_channel_* is given), as opposed to enc_min / enc_max, the gated ones of the forward. */
+int miq_qdq_mask_per_channel_f32(const float* in, float* out, uint64_t* mask, int64_t num_channel, int64_t num_element,
+                                 int64_t num_element_per_channel, const float* enc_min, const float* enc_max,
+                                 const float* enc_delta, const float* enc_offset, const float* raw_min,
+                                 const float* raw_max, void* stream);
+int miq_qdq_mask_per_channel_bf16(const uint16_t* in, uint16_t* out, uint64_t* mask, int64_t num_channel,
+                                  int64_t num_element, int64_t num_element_per_channel, const float* enc_min,
+                                  const float* enc_max, const float* enc_delta, const float* enc_offset,
+                                  const float* raw_min, const float* raw_max, void* stream);
+/* miq_v2_qdq_* + mask */
+int miq_v2_qdq_mask_f32(const float* in, float* out, uint64_t* mask, int64_t num_channel, int64_t num_element,
+                        int64_t num_element_per_channel, const float* scale, const float* offset, int qmin, int qmax,
+                        void* stream);
+int miq_v2_qdq_mask_bf16(const uint16_t* in, uint16_t* out, uint64_t* mask, int64_t num_channel, int64_t num_element,
+                         int64_t num_element_per_channel, const float* scale, const float* offset, int qmin, int qmax,
+                         void* stream);
+/* grad_in = grad_out * bit (grad_in may alias grad_out) */
+int miq_ste_bwd_mask_f32(const uint64_t* mask, const float* grad_out, float* grad_in, int64_t n, void* stream);
+int miq_ste_bwd_mask_bf16(const uint64_t* mask, const uint16_t* grad_out, uint16_t* grad_in, int64_t n, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
  * v2 quantize-dequantize (TORCH/v2/quantization/affine/backends/torch_builtins.py:290-344, QuantDequantFunc):
  * r = round-half-even(x/scale) - offset; mask = qmin <= r <= qmax; y = (clamp(r,qmin,qmax) + offset) * scale,
  * computed in float32.  scale/offset: device float[num_channel], channel(i) = (i / num_element_per_channel) %
