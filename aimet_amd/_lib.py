@@ -33,6 +33,7 @@ _flt = C.c_float
 
 _SIGNATURES = {
     "miq_version": ([], _int),
+    "miq_init": ([], _int),
     "miq_last_error": ([], C.c_char_p),
     "miq_fill_encoding_info": ([_int, _dbl, _dbl, C.POINTER(Encoding)], _int),
     "miq_get_computed_encodings": ([_int, _dbl, _dbl, _int, _int, _int, C.POINTER(Encoding)], _int),

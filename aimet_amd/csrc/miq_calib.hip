@@ -15,6 +15,7 @@
 // The histogram is privatised in LDS: 8 interleaved copies of the 512 bins per workgroup, lane l using copy
 // l mod 8, and merged into one of 32 global replicas per batch.
 #include "miq_common.h"
+#include "miq_agent.h"
 #include "miq_fastmath.h"
 #include "miq_tfe_search.h"
 
@@ -113,20 +114,6 @@ struct DevState
 };
 constexpr size_t kHeadBytes    = offsetof(DevState, xLeft);
 constexpr size_t kInspectBytes = offsetof(DevState, counts);
-
-// relaxed agent-scope loads: used by the workgroup that finishes last to read what the others published
-template <typename T>
-__device__ __forceinline__ T agent_load(const T* p)
-{
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// relaxed agent-scope store: written through, so that the launch leaves no modified lines behind in a cache for its
-// end-of-kernel release to write back
-template <typename T>
-__device__ __forceinline__ void agent_store(T* p, T v)
-{
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
 __device__ __forceinline__ float wave_min(float v)
 {
@@ -802,9 +789,8 @@ __global__ __launch_bounds__(kBlock) void tfe_search_kernel(DevState* st, Search
             agent_store(&st->cand_cost[cand], cost);
         }
     }
-    // Every wavefront waits for the acknowledgement of its stores, then the workgroup draws its ticket: the ticket is
-    // performed after all of them.  (A device-scope release fence per wavefront instead writes the L2 back each time.)
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // the ticket is drawn after every wavefront's stores have been acknowledged (miq_agent.h)
+    publications_acknowledged();
     __syncthreads();
     if (threadIdx.x == 0)
     {
@@ -814,6 +800,7 @@ __global__ __launch_bounds__(kBlock) void tfe_search_kernel(DevState* st, Search
     __syncthreads();
     if (!is_last || wave != 0)
         return;
+    last_ticket_acquire();
 
     // ---- last wavefront: pick the winner (first strict minimum) and form the encoding
     if (lane == 0)
@@ -1148,6 +1135,12 @@ int miq_minmax_per_channel_f32(const float* in, int64_t num_channel, int64_t num
                   "num_element must be a multiple of num_channel * num_element_per_channel");
     return launch_minmax_rows(in, num_channel, num_element / num_element_per_channel, num_element_per_channel,
                               reinterpret_cast<uint32_t*>(out_min_max), workspace, (hipStream_t) stream);
+}
+
+int miq_init(void)
+{
+    float2* unused = nullptr;
+    return static_scratch(&unused);
 }
 
 int miq_minmax_per_channel_static_f32(const float* in, int64_t num_channel, int64_t num_element,

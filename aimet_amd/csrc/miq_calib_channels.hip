@@ -430,6 +430,10 @@ int miq_channel_analyzer_update_stats_f32(miq_channel_analyzer* a, const float* 
                   "num_element (%lld) must be a multiple of num_channel * num_element_per_channel (%lld x %lld)",
                   (long long) num_element, (long long) a->num_channel, (long long) num_element_per_channel);
     MIQ_CHECK_ARG(num_element_per_channel < (1ll << 31), "rows of 2^31 elements or more are not handled");
+    // a channel's element count per batch is an int in the reference (UpdatePdf's `cnt`) and in the fold kernels
+    MIQ_CHECK_ARG(num_element / a->num_channel < (1ll << 31),
+                  "a channel holds %lld elements in this batch; the per-channel statistics take fewer than 2^31",
+                  (long long) (num_element / a->num_channel));
     hipStream_t s      = (hipStream_t) stream;
     const int64_t c    = a->num_channel;
     const int64_t npc  = num_element_per_channel;

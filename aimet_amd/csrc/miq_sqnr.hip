@@ -18,6 +18,7 @@
 // histogram.  The first batch, and updates that also want the batch's own
 // histogram, read the batch twice (finite min/max, then one binning pass for both histograms).  The reference reads a
 // batch about eight times (isfinite x4, histc x2, comparisons x4) and re-bins with per-element Python loops.
+#include "miq_agent.h"
 #include "miq_common.h"
 #include "miq_fastmath.h"
 
@@ -43,19 +44,6 @@ constexpr float kMinScale = 1.1920928955078125e-07f;   // torch.finfo(torch.floa
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-// relaxed agent-scope accesses: how the workgroup that finishes last reads what the others published (their atomics and
-// their stores, released by a fence before they took their ticket), and how it leaves results and cleared memory behind
-template <typename T>
-__device__ __forceinline__ T agent_load(const T* p)
-{
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-template <typename T>
-__device__ __forceinline__ void agent_store(T* p, T v)
-{
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // Ticket counters of one launch: `last[h]` and, for grids of more than 32 workgroups per histogram, one counter per
 // group of 32 workgroups, 128 bytes apart (tickets drawn from one address are served one after the other, about 25 ns
 // each: 1024 workgroups that finish together would wait 25 us for theirs).
@@ -67,15 +55,13 @@ struct Tickets
 constexpr int kTicketGroup  = 32;
 constexpr int kTicketStride = 32;   // words
 
-// Ticket of a workgroup that has finished its share of histogram h; true for the one that finishes last.  What the
-// workgroup published before -- device-scope atomic adds and agent_store()s, which are performed at the device's
-// point of coherence, not in a cache of their own -- has been acknowledged to every wavefront when it passes its
-// "s_waitcnt vmcnt(0)", so the ticket, taken after the barrier, is performed after all of it, and the workgroup that
-// draws the last ticket reads all of it with agent_load().  (A device-scope release fence per wavefront instead costs a
-// write-back of the L2 each: measured 65 us for 1024 workgroups.)  All counters are back at zero afterwards.
+// Ticket of a workgroup that has finished its share of histogram h; true for the one that finishes last, which has
+// then passed last_ticket_acquire() and reads what the others published (device-scope atomic adds and agent_store()s)
+// with agent_load() -- the pattern and its invariant are stated in miq_agent.h.  All counters are back at zero
+// afterwards.
 __device__ __forceinline__ bool last_ticket(const Tickets& t, int h, int* s_flag)
 {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    publications_acknowledged();
     __syncthreads();
     if (threadIdx.x == 0)
     {
@@ -101,7 +87,10 @@ __device__ __forceinline__ bool last_ticket(const Tickets& t, int h, int* s_flag
         *s_flag = last;
     }
     __syncthreads();
-    return *s_flag != 0;
+    const bool last = *s_flag != 0;
+    if (last)
+        last_ticket_acquire();
+    return last;
 }
 
 // The last workgroup's reads are agent-scope loads that travel to the device's point of coherence (1-2 us each way):

@@ -724,12 +724,22 @@ class _StateOwner:
 
     def _init_state(self, nbytes):
         self._state = torch.empty(int(nbytes) // 8 + 1, dtype=torch.float64, device=self.device)
-        self._streams_seen = {_stream_of(self.device)}
+        self._last_stream = torch.cuda.current_stream(self.device)
+        self._last_handle = self._last_stream.cuda_stream
+        self._streams_seen = {self._last_handle}
 
     def _note_stream(self, handle):
-        if handle not in self._streams_seen:
-            self._streams_seen.add(handle)
-            self._state.record_stream(torch.cuda.current_stream(self.device))
+        """Called with the stream handle of every call that queues work on the state.  The object's host-side
+        bookkeeping (pending batch, sequence numbers, whether the range is known) assumes that its launches run in the
+        order they were queued; when the caller moves to another stream, that stream is made to wait for everything
+        queued on the previous one."""
+        if handle != self._last_handle:
+            current = torch.cuda.current_stream(self.device)
+            current.wait_event(self._last_stream.record_event())
+            self._last_stream, self._last_handle = current, handle
+            if handle not in self._streams_seen:
+                self._streams_seen.add(handle)
+                self._state.record_stream(current)
 
 
 class Analyzer(_StateOwner):
@@ -756,7 +766,10 @@ class Analyzer(_StateOwner):
             lib.miq_analyzer_destroy(h)
 
     def _s(self):
-        return C.c_void_p(_stream_of(self.device))
+        handle = _stream_of(self.device)
+        if handle != self._last_handle:
+            self._note_stream(handle)
+        return C.c_void_p(handle)
 
     def reset(self):
         with torch.cuda.device(self.device):
@@ -776,7 +789,7 @@ class Analyzer(_StateOwner):
         # the caching allocator cannot hand its memory to anyone else before they have run
         if torch.cuda.current_device() == self.device.index:
             stream = _stream_of(self.device)
-            if stream not in self._streams_seen:
+            if stream != self._last_handle:
                 self._note_stream(stream)
             check(lib.miq_analyzer_update_stats_f32(self._h, x.data_ptr(), x.numel(), stream))
         else:
@@ -845,7 +858,10 @@ class ChannelAnalyzer(_StateOwner):
             lib.miq_channel_analyzer_destroy(h)
 
     def _s(self):
-        return C.c_void_p(_stream_of(self.device))
+        handle = _stream_of(self.device)
+        if handle != self._last_handle:
+            self._note_stream(handle)
+        return C.c_void_p(handle)
 
     def reset(self):
         with torch.cuda.device(self.device):

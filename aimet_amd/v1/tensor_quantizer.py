@@ -344,6 +344,11 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
                 return
             if tensor.dtype == torch.float16:
                 tensor = tensor.to(torch.float32)
+            # the reference walks its fixed list of per-channel analyzers (:567-570): a tensor with another number of
+            # channels along ch_axis fails there, and statistics gathered so far are never dropped
+            if tensor.shape[self._ch_axis] != len(self._cppOp):
+                raise RuntimeError(f"the tensor has {tensor.shape[self._ch_axis]} channels along axis {self._ch_axis}; "
+                                   f"this quantizer was created for {len(self._cppOp)}")
             if self._quant_scheme == QuantScheme.post_training_tf:
                 # one fused pass: per-channel min and max of the whole tensor
                 num_channel = tensor.shape[self._ch_axis]
@@ -363,7 +368,9 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
             num_channel = tensor.shape[self._ch_axis]
             n_per_channel = functools.reduce(lambda a, b: a * b, tensor.shape[self._ch_axis + 1:], 1)
             analyzer = self._channel_analyzer
-            if analyzer is None or analyzer.device != tensor.device or analyzer.num_channel != num_channel:
+            if analyzer is not None and analyzer.device != tensor.device:
+                raise RuntimeError(f"statistics were gathered on {analyzer.device}; this batch is on {tensor.device}")
+            if analyzer is None:
                 mode = 1 if self._quant_scheme == QuantScheme.post_training_tf_enhanced else 2
                 analyzer = ops.ChannelAnalyzer(mode, num_channel, tensor.device)
                 analyzer.set_percentile(self._percentile_value)

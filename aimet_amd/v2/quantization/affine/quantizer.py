@@ -56,6 +56,31 @@ class _AffineEncoding:
         return self.scale * (self.offset + self.qmax)
 
 
+def _grid_arguments(owner: str, args, kwargs):
+    """(qmin, qmax, symmetric, encoding_analyzer, block_size) from either call form of the constructor
+    (reference affine/quantizer.py:91-140):
+
+        (shape, qmin, qmax, symmetric, encoding_analyzer=None, block_size=None)
+        (shape, bitwidth, symmetric, encoding_analyzer=None, block_size=None)
+
+    The two forms are told apart by what follows the first number: another number (or a `qmax` keyword) means a
+    grid, a bool means `symmetric` and the first number was a bit-width.  Python's own argument binding then reports
+    what is missing or unknown."""
+    def from_grid(qmin, qmax, symmetric, encoding_analyzer=None, block_size=None):
+        return qmin, qmax, symmetric, encoding_analyzer, block_size
+
+    def from_bitwidth(bitwidth, symmetric, encoding_analyzer=None, block_size=None):
+        return (*_derive_qmin_qmax(bitwidth=bitwidth, signed=symmetric), symmetric, encoding_analyzer, block_size)
+
+    second = args[1] if len(args) > 1 else None
+    grid_form = 'qmax' in kwargs or 'qmin' in kwargs or (second is not None and not isinstance(second, bool))
+    try:
+        return (from_grid if grid_form else from_bitwidth)(*args, **kwargs)
+    except TypeError as error:
+        raise TypeError(f"{owner}.__init__ expects (shape, qmin, qmax, symmetric) or (shape, bitwidth, symmetric), each "
+                        f"optionally followed by encoding_analyzer and block_size: {error}") from None
+
+
 class MinMaxQuantizer(nn.Module):
     """Affine quantizer with min / max as trainable parameters."""
 
@@ -64,28 +89,7 @@ class MinMaxQuantizer(nn.Module):
         if isinstance(shape, int):
             shape = (shape,)
         self.shape = tuple(shape)
-        # (qmin, qmax, symmetric[, encoding_analyzer[, block_size]]) or (bitwidth, symmetric[, encoding_analyzer[, block_size]])
-        args = list(args) + [None] * (5 - len(args))
-        arg0 = kwargs.pop('qmin', kwargs.pop('bitwidth', args[0]))
-        arg1 = kwargs.pop('qmax', args[1])
-        if arg1 is not None and not isinstance(arg1, bool):
-            qmin, qmax = arg0, arg1
-            symmetric = kwargs.pop('symmetric', args[2])
-            encoding_analyzer = kwargs.pop('encoding_analyzer', args[3])
-            block_size = kwargs.pop('block_size', args[4])
-            if qmin is None or qmax is None or symmetric is None:
-                raise TypeError("expected (shape, qmin, qmax, symmetric) or (shape, bitwidth, symmetric)")
-        else:
-            bitwidth = arg0
-            symmetric = kwargs.pop('symmetric', args[1])
-            if bitwidth is None or symmetric is None:
-                raise TypeError("expected (shape, qmin, qmax, symmetric) or (shape, bitwidth, symmetric)")
-            qmin, qmax = _derive_qmin_qmax(bitwidth=bitwidth, signed=symmetric)
-            encoding_analyzer = kwargs.pop('encoding_analyzer', args[2])
-            block_size = kwargs.pop('block_size', args[3])
-        if kwargs:
-            raise TypeError(f"{type(self).__qualname__}.__init__ got unexpected keyword argument: "
-                            f"{', '.join(kwargs)}")
+        qmin, qmax, symmetric, encoding_analyzer, block_size = _grid_arguments(type(self).__qualname__, args, kwargs)
         if qmin >= qmax:
             raise ValueError(f"qmax should be strictly larger than qmin. Got qmax={qmax}, qmin={qmin}")
         self.qmin, self.qmax = qmin, qmax
@@ -215,36 +219,42 @@ class MinMaxQuantizer(nn.Module):
         if not self._allow_overwrite:
             yield
             return
-        original_forward = self.forward
-
-        @functools.wraps(original_forward)
-        def forward_wrapper(input):  # pylint: disable=redefined-builtin
-            expanded = reshape_tensor_for_blocks(input, self.shape, self.block_size)
-            batch_statistics = self.encoding_analyzer.update_stats(expanded)
-            num_steps = self.qmax - self.qmin
-            dyn_min, dyn_max = self.encoding_analyzer.compute_encodings_from_stats(batch_statistics, num_steps,
-                                                                                   self.symmetric)
-            if self.block_size is not None:
-                dyn_min, dyn_max = dyn_min.view(self.min.shape), dyn_max.view(self.max.shape)
-            dyn_min = dyn_min.to(dtype=self.min.dtype, device=self.min.device).expand_as(self.min)
-            dyn_max = dyn_max.to(dtype=self.max.dtype, device=self.max.device).expand_as(self.max)
-            with patch_attr(self, 'min', dyn_min), patch_attr(self, 'max', dyn_max):
-                return original_forward(input)
-
-        self.encoding_analyzer.reset_stats()
-        with patch_attr(self, 'forward', forward_wrapper):
+        analyzer = self.encoding_analyzer
+        analyzer.reset_stats()
+        plain_forward = self.forward
+        with patch_attr(self, 'forward', functools.wraps(plain_forward)(
+                lambda tensor: self._forward_on_batch_statistics(plain_forward, tensor))):
             yield
+        # on exit: the statistics gathered inside become the parameters, if there are any
         try:
-            num_steps = self.qmax - self.qmin
-            enc_min, enc_max = self.encoding_analyzer.compute_encodings(num_steps, self.symmetric)
+            found = analyzer.compute_encodings(self.qmax - self.qmin, self.symmetric)
         except StatisticsNotFoundError:
             return
-        if enc_min is None or enc_max is None:
+        if any(bound is None for bound in found):
             return
-        if self.block_size is not None:
-            enc_min, enc_max = enc_min.view(self.min.shape), enc_max.view(self.max.shape)
-        _flag_extreme_min_max(enc_min, enc_max)
-        self.set_range(enc_min, enc_max)
+        new_min, new_max = (self._in_parameter_shape(bound) for bound in found)
+        _flag_extreme_min_max(new_min, new_max)
+        self.set_range(new_min, new_max)
+
+    def _in_parameter_shape(self, bound: torch.Tensor) -> torch.Tensor:
+        """Blockwise statistics come with a singleton axis after every axis; the parameters do not have them."""
+        return bound if self.block_size is None else bound.view(self.min.shape)
+
+    def _forward_on_batch_statistics(self, plain_forward, tensor):
+        """One forward inside compute_encodings(): the batch enters the running statistics, and the output is
+        quantized with the range of this batch alone (reference :330-352)."""
+        per_block = reshape_tensor_for_blocks(tensor, self.shape, self.block_size)
+        batch = self.encoding_analyzer.update_stats(per_block)
+        bounds = self.encoding_analyzer.compute_encodings_from_stats(batch, self.qmax - self.qmin, self.symmetric)
+        stand_ins = {}
+        for name, bound in zip(('min', 'max'), bounds):
+            param = getattr(self, name)
+            stand_ins[name] = self._in_parameter_shape(bound).to(dtype=param.dtype, device=param.device) \
+                .expand_as(param)
+        with contextlib.ExitStack() as stack:
+            for name, value in stand_ins.items():
+                stack.enter_context(patch_attr(self, name, value))
+            return plain_forward(tensor)
 
     def set_range(self, min: torch.Tensor, max: torch.Tensor):  # pylint: disable=redefined-builtin
         with torch.no_grad():

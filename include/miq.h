@@ -62,6 +62,11 @@ typedef struct miq_encoding
 const char* miq_last_error(void);
 /* Library/ABI version, bumped when a signature changes. */
 int miq_version(void);
+/* One-time, per-GPU set-up of the library for the current device (today: the device address of the static scratch
+ * array behind miq_minmax_per_channel_static_f32).  Optional -- everything it prepares is also prepared on first use --
+ * but callers that capture HIP graphs should call it before the first capture on each GPU.  Allocates nothing.
+ * No counterpart in the reference. */
+int miq_init(void);
 
 /* ---------------------------------------------------------------------------------------------------------------
  * Host-side encoding arithmetic (double precision, no device work)
@@ -281,7 +286,10 @@ int miq_minmax_per_channel_f32(const float* in, int64_t num_channel, int64_t num
  * (num_channel = 1, num_element_per_channel = num_element gives the per-tensor form).  Limit: tensors whose
  * miq_minmax_workspace_bytes() exceeds 256 KiB (32768 partial pairs: about 5.4e8 elements per tensor) are refused with
  * MIQ_ERR_INVALID_ARG.  All calls on one GPU share the array: calls that overlap in time on one GPU (two streams,
- * two threads) race and must be serialised by the caller. */
+ * two threads) race and must be serialised by the caller.  The array's device address is looked up once per GPU
+ * (hipGetSymbolAddress, under a mutex): by miq_init(), or else by the first call on that GPU -- call miq_init() with
+ * the GPU current before a stream capture that contains this entry point, since the lookup is not a capturable
+ * operation. */
 int miq_minmax_per_channel_static_f32(const float* in, int64_t num_channel, int64_t num_element,
                                       int64_t num_element_per_channel, float* out_min_max, void* stream);
 

@@ -216,6 +216,27 @@ def test_cfg3_full_size_bit_exact(ops, oracle):
         _same_search(an, pdf)
 
 
+def test_tfe_updates_across_streams(ops, oracle):
+    """Batches queued on alternating torch streams: the analyzer orders each stream after the previous one, so the
+    result is that of the same batches queued on one stream."""
+    batches = [_relu_pareto(70 + b, 400000 + 13 * b) for b in range(8)]
+    dev = [_gpu(b) for b in batches]
+    torch.cuda.synchronize()
+    an = ops.Analyzer(TFE)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for k, b in enumerate(dev):
+        with torch.cuda.stream(streams[k % 2]):
+            an.update_stats(b)
+    pdf = oracle.new_pdf()
+    for b in batches:
+        pdf.update(b)
+    xl, p = an.get_stats_histogram()          # on the default stream: ordered after both
+    torch.cuda.synchronize()
+    assert np.array_equal(xl.view(np.uint64), pdf.x_left().view(np.uint64))
+    assert np.array_equal(p.view(np.uint64), pdf.pdf().view(np.uint64))
+    _same_search(an, pdf, modes=((8, 0, 0, 0),))
+
+
 def test_tfe_back_to_back_without_reads(ops, oracle):
     """update_stats calls queued with no read-back between them: a leading all-zero batch (no range yet), ragged batch
     sizes, a reset in the middle; only the final state is read and compared with the oracle fed the same batches."""

@@ -164,3 +164,19 @@ def test_per_channel_quantizer_uses_one_device_object(ops):
         q.update_encoding_stats(w)
         q.compute_encoding()
         assert max(e.max for e in q.encoding) < float(w.abs().max())                  # the tails are cut
+
+
+def test_per_channel_quantizer_refuses_another_channel_count():
+    """A batch with another number of channels along ch_axis raises instead of silently dropping the statistics
+    gathered so far (the reference walks its fixed list of per-channel analyzers)."""
+    from aimet_amd.common import libpymo
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.tensor_quantizer import StaticGridPerChannelQuantizer
+    for scheme in (QuantScheme.post_training_tf_enhanced, QuantScheme.post_training_tf):
+        q = StaticGridPerChannelQuantizer(8, libpymo.RoundingMode.ROUND_NEAREST, scheme, True, 6, True, ch_axis=0)
+        q.update_encoding_stats(torch.randn(6, 40, device="cuda"))
+        with pytest.raises(RuntimeError, match="channels"):
+            q.update_encoding_stats(torch.randn(5, 40, device="cuda"))
+        q.update_encoding_stats(torch.randn(6, 40, device="cuda"))
+        q.compute_encoding()
+        assert len(q.encoding) == 6

@@ -41,3 +41,10 @@ def test_static_scratch_minmax_refuses_what_does_not_fit():
     assert lib.miq_minmax_workspace_bytes(1, n, n) > 32768 * 8
     with pytest.raises(MiqError, match="too large"):
         check(lib.miq_minmax_per_channel_static_f32(x.data_ptr(), 1, n, n, out.data_ptr(), None))
+
+
+def test_init_is_idempotent():
+    """miq_init prepares the static scratch's device address ahead of the first use (for callers that capture)."""
+    from aimet_amd._lib import check, lib
+    for _ in range(2):
+        check(lib.miq_init())
