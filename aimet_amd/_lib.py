@@ -25,6 +25,14 @@ class Encoding(C.Structure):
                 ("bw", C.c_int)]
 
 
+class QdqSegment(C.Structure):
+    """struct miq_qdq_segment: one tensor of a multi-tensor quantize-dequantize launch"""
+    _fields_ = [("in_", C.c_void_p), ("out", C.c_void_p), ("num_element", C.c_int64), ("num_channel", C.c_int64),
+                ("num_element_per_channel", C.c_int64), ("enc_min", C.c_void_p), ("enc_max", C.c_void_p),
+                ("enc_delta", C.c_void_p), ("enc_offset", C.c_void_p), ("fd_magic", C.c_uint32),
+                ("fd_shift", C.c_uint32), ("first_tile", C.c_int32), ("reserved", C.c_int32)]
+
+
 _p = C.c_void_p
 _i64 = C.c_int64
 _int = C.c_int
@@ -50,6 +58,9 @@ _SIGNATURES = {
     "miq_ste_bwd_per_tensor_bf16": ([_p, _p, _p, _i64, _flt, _flt, _p], _int),
     "miq_ste_bwd_per_channel_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _p], _int),
     "miq_ste_bwd_per_channel_bf16": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _p], _int),
+    "miq_qdq_multi_plan": ([C.POINTER(QdqSegment), _int, _int], _i64),
+    "miq_qdq_per_channel_multi_f32": ([_p, _int, _i64, _p], _int),
+    "miq_qdq_per_channel_multi_bf16": ([_p, _int, _i64, _p], _int),
     "miq_ste_mask_bytes": ([_i64, _int], _i64),
     "miq_qdq_mask_per_tensor_f32": ([_p, _p, _p, _i64, _dbl, _dbl, _int, _flt, _flt, _p], _int),
     "miq_qdq_mask_per_tensor_bf16": ([_p, _p, _p, _i64, _dbl, _dbl, _int, _flt, _flt, _p], _int),

@@ -460,16 +460,17 @@ __device__ __forceinline__ void store_codes<int32_t, 8>(int32_t* dst, const int*
 // Vectorised tile kernel.  Requires 16-byte aligned pointers; n < 2^31 when PER_CHANNEL.  CODES: the integer codes are
 // stored too (ptr.codes is not null); without it their arithmetic (two operations per element) is not compiled in.
 // MASK: the ops' "codes" are in-range flags, packed into ptr.mask (see above) instead of being stored as integers.
+// `tile`: which tile of the tensor this workgroup takes (the workgroup's index for a launch over one tensor).
 template <typename IO, typename OP, bool PER_CHANNEL, int kUnroll, bool CODES, bool MASK = false>
-__global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::Code> ptr, ParamSrc src, int64_t n,
-                                                        uint32_t num_channel, FastDiv fd)
+__device__ __forceinline__ void ew_vec_tile(const EwPtrs<IO, typename OP::Code>& ptr, const ParamSrc& src, int64_t n,
+                                            uint32_t num_channel, const FastDiv& fd, uint32_t tile)
 {
     using T                 = IOTraits<IO>;
     using Vec               = typename T::Vec;
     using P                 = typename OP::P;
     constexpr int VEC       = T::VEC;
     constexpr uint32_t TILE = kBlock * kUnroll * VEC;
-    const int64_t e_base    = (int64_t) blockIdx.x * TILE;
+    const int64_t e_base    = (int64_t) tile * TILE;
     const int64_t nvec      = n / VEC;
 
     // 1. the tile's loads go out first; everything below overlaps their latency.  A workgroup whose whole tile exists
@@ -606,7 +607,7 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
         }
     }
     // the n % VEC trailing elements
-    if (blockIdx.x == 0 && threadIdx.x < (uint32_t) (n - nvec * VEC))
+    if (tile == 0 && threadIdx.x < (uint32_t) (n - nvec * VEC))
     {
         const int64_t e = nvec * VEC + threadIdx.x;
         P p;
@@ -629,8 +630,52 @@ __global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::
             ptr.codes[e] = (typename OP::Code) code;
     }
     if constexpr (MASK)
-        if (blockIdx.x == 0 && threadIdx.x == 0 && n == nvec * VEC)
+        if (tile == 0 && threadIdx.x == 0 && n == nvec * VEC)
             ptr.mask[mask_words<VEC>(n) - 1] = 0;   // no trailing elements: the word is still defined
+}
+
+template <typename IO, typename OP, bool PER_CHANNEL, int kUnroll, bool CODES, bool MASK = false>
+__global__ __launch_bounds__(kBlock) void ew_vec_kernel(EwPtrs<IO, typename OP::Code> ptr, ParamSrc src, int64_t n,
+                                                        uint32_t num_channel, FastDiv fd)
+{
+    ew_vec_tile<IO, OP, PER_CHANNEL, kUnroll, CODES, MASK>(ptr, src, n, num_channel, fd, blockIdx.x);
+}
+
+// ---- several tensors in one launch --------------------------------------------------------------------------------
+// The workgroups of one launch are dealt out over the tiles of all segments (miq_qdq_segment, a table in device
+// memory): a workgroup finds its segment by counting the segments that start at or before its tile -- every lane reads
+// one segment's first tile, one round trip -- reads that segment's record and runs the per-channel tile code on it.
+// For the dozens of small weight tensors of a convolutional network, each a few microseconds of traffic, this removes
+// the launches' fixed cost and lets the tensors' ramps overlap.
+constexpr int kMaxSegments = kBlock;
+template <typename IO>
+__global__ __launch_bounds__(kBlock) void ew_multi_kernel(const miq_qdq_segment* __restrict__ segs, int num_segments)
+{
+    __shared__ int s_count[kBlock / 64];
+    const uint32_t tile = blockIdx.x;
+    const bool before   = (int) threadIdx.x < num_segments && (uint32_t) segs[threadIdx.x].first_tile <= tile;
+    const int in_wave   = __popcll(__builtin_amdgcn_ballot_w64(before));
+    if ((threadIdx.x & 63) == 0)
+        s_count[threadIdx.x >> 6] = in_wave;
+    __syncthreads();
+    int count = 0;
+#pragma unroll
+    for (int k = 0; k < kBlock / 64; ++k)
+        count += s_count[k];
+    const int seg             = __builtin_amdgcn_readfirstlane(count - 1);   // first_tile of segment 0 is 0
+    const miq_qdq_segment sg  = segs[seg];
+    EwPtrs<IO, uint8_t> ptr{static_cast<const IO*>(sg.in), nullptr, static_cast<IO*>(sg.out), nullptr, nullptr};
+    ParamSrc src{};
+    src.a = sg.enc_min;
+    src.b = sg.enc_max;
+    src.c = sg.enc_delta;
+    src.d = sg.enc_offset;
+    FastDiv fd;
+    fd.d     = (uint32_t) sg.num_element_per_channel;
+    fd.magic = sg.fd_magic;
+    fd.shift = sg.fd_shift;
+    ew_vec_tile<IO, OpV1Qdq, true, kUnroll, false, false>(ptr, src, sg.num_element, (uint32_t) sg.num_channel, fd,
+                                                         tile - (uint32_t) sg.first_tile);
 }
 
 // Fallback for unaligned pointers, tiny channels (elements-per-channel < 16) and n >= 2^31: one element per lane,
@@ -1100,6 +1145,18 @@ static int v2_qdq_mask(const IO* in, IO* out, uint64_t* mask, int64_t num_channe
                                       (hipStream_t) stream);
 }
 
+template <typename IO>
+static int qdq_multi(const miq_qdq_segment* segments, int num_segments, int64_t total_tiles, void* stream)
+{
+    MIQ_CHECK_ARG(segments && num_segments >= 1 && num_segments <= kMaxSegments, "1..%d segments per launch",
+                  kMaxSegments);
+    MIQ_CHECK_ARG(total_tiles >= 1 && total_tiles < (1ll << 31), "total_tiles must be what miq_qdq_multi_plan returned");
+    hipLaunchKernelGGL((ew_multi_kernel<IO>), dim3((unsigned) total_tiles), dim3(kBlock), 0, (hipStream_t) stream,
+                       segments, num_segments);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
 extern "C" {
 
 int miq_qdq_per_tensor_f32(const float* in, float* out, int64_t n, double enc_min, double enc_max, int bw,
@@ -1382,6 +1439,55 @@ int miq_v2_qdq_bwd_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* g
     EwPtrs<uint16_t, int32_t> p{x, grad_out, grad_in, nullptr};
     return launch_v2<uint16_t, OpV2Bwd>(p, v2_src(scale, offset, qmin, qmax), num_element, num_channel,
                                         num_element_per_channel, (hipStream_t) stream);
+}
+
+/* ---- several tensors in one launch ------------------------------------------------------------------------- */
+
+int64_t miq_qdq_multi_plan(miq_qdq_segment* segments, int num_segments, int elem_bytes)
+{
+    if (!segments || num_segments < 1 || num_segments > kMaxSegments || (elem_bytes != 4 && elem_bytes != 2))
+    {
+        set_error("miq_qdq_multi_plan takes 1..%d segments of float32 (4) or bfloat16 (2) elements", kMaxSegments);
+        return -1;
+    }
+    const int64_t tile = (int64_t) kBlock * kUnroll * (elem_bytes == 4 ? 4 : 8);
+    int64_t tiles      = 0;
+    for (int i = 0; i < num_segments; ++i)
+    {
+        miq_qdq_segment& g = segments[i];
+        const bool ok = g.in && g.out && g.enc_min && g.enc_max && g.enc_delta && g.enc_offset && g.num_element > 0 &&
+                        g.num_channel > 0 && g.num_element_per_channel > 0 && g.num_element < (1ll << 31) &&
+                        g.num_channel < (1ll << 31) && aligned16(g.in) && aligned16(g.out) &&
+                        tile / g.num_element_per_channel + 2 <= kWin;
+        if (!ok)
+        {
+            set_error("segment %d cannot go into a multi-tensor launch (null or unaligned pointer, empty, 2^31 elements "
+                      "or more, or fewer than %lld elements per channel): quantize it on its own", i,
+                      (long long) (tile / (kWin - 2) + 1));
+            return -1;
+        }
+        const FastDiv fd = make_fastdiv((uint32_t) g.num_element_per_channel);
+        g.fd_magic       = fd.magic;
+        g.fd_shift       = fd.shift;
+        if (tiles >= (1ll << 31) - (g.num_element + tile - 1) / tile)
+        {
+            set_error("too many tiles for one launch");
+            return -1;
+        }
+        g.first_tile = (int32_t) tiles;
+        tiles += (g.num_element + tile - 1) / tile;
+    }
+    return tiles;
+}
+
+int miq_qdq_per_channel_multi_f32(const miq_qdq_segment* segments, int num_segments, int64_t total_tiles, void* stream)
+{
+    return qdq_multi<float>(segments, num_segments, total_tiles, stream);
+}
+
+int miq_qdq_per_channel_multi_bf16(const miq_qdq_segment* segments, int num_segments, int64_t total_tiles, void* stream)
+{
+    return qdq_multi<uint16_t>(segments, num_segments, total_tiles, stream);
 }
 
 /* ---- forward with the saved straight-through mask, backward from the mask ----------------------------------- */

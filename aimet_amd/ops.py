@@ -324,6 +324,53 @@ def ste_bwd_per_channel(x, grad_out, num_channel, n_per_channel, enc_min, enc_ma
     return gin
 
 
+# ---------------------------------------------------------------------------------------- several tensors, one launch
+class QdqMulti:
+    """A prepared quantize-dequantize of several tensors in one launch (nearest rounding, v1 arithmetic).
+
+    entries: (x, num_channel, n_per_channel, enc_min, enc_max, enc_delta, enc_offset) with x a contiguous float32 (or
+    all bfloat16) GPU tensor and the four parameter vectors as qdq_per_channel takes them (one-element vectors for a
+    per-tensor encoding).  Outputs are allocated once (`outputs`, same order) and rewritten by every call.  Raises
+    RuntimeError when an entry cannot take part (tiny channels, unaligned data): quantize that one by itself."""
+    MAX_SEGMENTS = 256
+
+    def __init__(self, entries, outputs=None):
+        entries = list(entries)
+        if not 1 <= len(entries) <= self.MAX_SEGMENTS:
+            raise RuntimeError(f"1 .. {self.MAX_SEGMENTS} tensors per launch")
+        first = entries[0][0]
+        _require_gpu(*[t for e in entries for t in (e[0],) + tuple(e[3:7])])
+        self.device = first.device
+        self._suffix = _suffix(first)
+        self.outputs = [torch.empty_like(e[0]) for e in entries] if outputs is None else list(outputs)
+        self._keep = []
+        table = (_lib.QdqSegment * len(entries))()
+        for seg, entry, out in zip(table, entries, self.outputs):
+            x, c, npc = entry[0], int(entry[1]), int(entry[2])
+            if x.dtype != first.dtype or not x.is_contiguous() or out.shape != x.shape or out.dtype != x.dtype:
+                raise RuntimeError("the tensors of one launch share a dtype and are contiguous")
+            params = [_params_f32(p, x).reshape(-1) for p in entry[3:7]]
+            if any(p.numel() != c for p in params):
+                raise RuntimeError("parameter vectors must hold one value per channel")
+            self._keep.append((x, out, params))
+            seg.in_, seg.out, seg.num_element, seg.num_channel, seg.num_element_per_channel = \
+                x.data_ptr(), out.data_ptr(), x.numel(), c, npc
+            seg.enc_min, seg.enc_max, seg.enc_delta, seg.enc_offset = (p.data_ptr() for p in params)
+        self._tiles = int(lib.miq_qdq_multi_plan(table, len(entries), first.element_size()))
+        if self._tiles < 0:
+            raise _lib.MiqError(lib.miq_last_error().decode())
+        self._count = len(entries)
+        self.elements = sum(e[0].numel() for e in entries)
+        host = torch.frombuffer(bytearray(bytes(table)), dtype=torch.uint8)
+        self._table = host.to(self.device)
+        self._fn = getattr(lib, "miq_qdq_per_channel_multi_" + self._suffix)
+
+    def __call__(self):
+        with _OnDevice(self.device):
+            check(self._fn(self._table.data_ptr(), self._count, self._tiles, _stream_of(self.device)))
+        return self.outputs
+
+
 # ------------------------------------------------------------------------------------- saved straight-through mask
 def _new_mask(x):
     """Device buffer for the one-bit-per-element straight-through mask of `x` (int64 words, never initialised: the

@@ -378,8 +378,37 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
         for name, param in self.get_named_parameters():
             param.data = shadow_params[name]
 
+    # Quantized parameters are kept between forwards while nothing they depend on has changed: the reference
+    # quantize-dequantizes every parameter in every forward (reference :747-763), which for a model in evaluation mode
+    # is the same computation on the same numbers every time.  A kept tensor is used again only for the same storage
+    # (data pointer), the same version of the parameter (in-place operations on the parameter count it up), shape and
+    # dtype, and the same encoding object with the same bounds.  Not seen: an in-place edit through a `param.data`
+    # alias (`w.data.mul_(2)` leaves pointer and version alone) -- call invalidate_param_cache() after one, or set
+    # StaticGridQuantWrapper.cache_quantized_params = False.
+    cache_quantized_params = True
+
+    @staticmethod
+    def _encoding_stamp(quantizer):
+        enc = quantizer.encoding
+        if isinstance(enc, (list, tuple)):
+            return (id(enc), len(enc), enc[0].min, enc[0].max, enc[-1].min, enc[-1].max, enc[0].bw)
+        return (id(enc), enc.min, enc.max, enc.bw)
+
+    def _param_cache_key(self, param, quantizer):
+        return (param.data_ptr(), param._version, param.dtype, tuple(param.shape), quantizer.bitwidth,  # pylint: disable=protected-access
+                quantizer.data_type, self._encoding_stamp(quantizer))
+
+    def _params_may_be_kept(self) -> bool:
+        return StaticGridQuantWrapper.cache_quantized_params and not self.training and \
+            not self._module_to_wrap.training
+
+    def invalidate_param_cache(self):
+        self.__dict__['_param_cache'] = {}
+
     def _quantize_dequantize_params(self):
         shadow_params = {}
+        keep = self._params_may_be_kept()
+        cache = self.__dict__.setdefault('_param_cache', {})
         for name, param in self.get_named_parameters():
             shadow_params[name] = param.data
             quantizer = self.param_quantizers[name]
@@ -391,6 +420,14 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
                     if quantizer.quant_scheme == QuantScheme.post_training_percentile:
                         quantizer.set_percentile_value(100)
                     quantizer.compute_encoding()
+                if keep and quantizer.encoding is not None:
+                    key = self._param_cache_key(param, quantizer)
+                    kept = cache.get(name)
+                    if kept is None or kept[0] != key:
+                        kept = (key, quantizer.quantize_dequantize(param.data, libpymo.RoundingMode.ROUND_NEAREST))
+                        cache[name] = kept
+                    param.data = kept[1]
+                    continue
                 round_mode = quantizer.round_mode if self.training else libpymo.RoundingMode.ROUND_NEAREST
                 param.data = quantizer.quantize_dequantize(param.data, round_mode)
         return shadow_params

@@ -13,12 +13,14 @@ aimet_amd.v1.nn.modules.custom, as in the reference).
 """
 import copy
 import json
+import math
 import os
 from typing import Dict, List, Tuple, Union
 
 import torch
 from torch import nn
 
+from .. import ops
 from ..common.defs import QuantizationDataType, QuantScheme
 from .nn.modules import custom
 from .qc_quantize_op import LearnedGridQuantWrapper, QcQuantizeOpMode, QcQuantizeWrapper, StaticGridQuantWrapper
@@ -472,6 +474,61 @@ class QuantizationSimModel:
         finally:
             self.model.train(was_training)
         self.compute_layer_encodings_for_sim()
+        if not self.model.training:
+            self.quantize_params_together()
+
+    def quantize_params_together(self) -> int:
+        """Quantize-dequantizes the parameters of every static-grid wrapper in evaluation mode with ONE launch over
+        all of them (aimet_amd.ops.QdqMulti) and leaves the results where the wrappers keep quantized parameters
+        between forwards.  Called at the end of compute_encodings(); call it again after the weights have changed
+        when the next forwards should not re-quantize tensor by tensor.  Returns the number of tensors it took;
+        tensors that cannot go into such a launch (tiny channels, other data types, disabled quantizers) are left
+        to their wrappers.  The reference has no counterpart: it quantizes each parameter in each forward
+        (qc_quantize_op.py:747-763)."""
+        groups = {}
+        for layer in self._static_grid_layers():
+            if not layer._params_may_be_kept():                      # pylint: disable=protected-access
+                continue
+            for name, param in layer.get_named_parameters():
+                quantizer = layer.param_quantizers[name]
+                if not (quantizer.enabled and quantizer.bitwidth != 32 and quantizer.encoding is not None and
+                        quantizer.data_type == QuantizationDataType.int and param.is_cuda and
+                        param.dtype in (torch.float32, torch.bfloat16) and param.data.is_contiguous()):
+                    continue
+                data = param.data
+                if isinstance(quantizer, StaticGridPerChannelQuantizer):
+                    sizes = [*data.shape, 1]
+                    num_channel = sizes[quantizer.channel_axis]
+                    n_per_channel = math.prod(sizes[quantizer.channel_axis + 1:])
+                    params = quantizer.device_params(data.device)[:4]
+                else:
+                    enc = ops.fill_encoding_info(quantizer.encoding.bw, quantizer.encoding.min, quantizer.encoding.max)
+                    num_channel, n_per_channel = 1, data.numel()
+                    params = (enc.min, enc.max, enc.delta, enc.offset)       # uploaded below, all at once
+                if n_per_channel < 16 or data.numel() >= 2 ** 31:
+                    continue
+                groups.setdefault((data.device, data.dtype), []).append(
+                    (layer, name, param, quantizer, data, num_channel, n_per_channel, params))
+        taken = 0
+        for (device, _), items in groups.items():
+            scalars = [it[7] for it in items if not isinstance(it[7][0], torch.Tensor)]
+            uploaded = torch.tensor(scalars, dtype=torch.float64).to(torch.float32).to(device) if scalars else None
+            k = 0
+            entries = []
+            for it in items:
+                params = it[7]
+                if not isinstance(params[0], torch.Tensor):
+                    params = tuple(uploaded[k, j:j + 1] for j in range(4))
+                    k += 1
+                entries.append((it[4], it[5], it[6], *params))
+            for first in range(0, len(entries), ops.QdqMulti.MAX_SEGMENTS):
+                chunk = entries[first:first + ops.QdqMulti.MAX_SEGMENTS]
+                outputs = ops.QdqMulti(chunk)()
+                for it, out in zip(items[first:first + len(chunk)], outputs):
+                    layer, name, param, quantizer = it[:4]
+                    layer.__dict__.setdefault('_param_cache', {})[name] = (layer._param_cache_key(param, quantizer), out)  # pylint: disable=protected-access
+                    taken += 1
+        return taken
 
     def _static_grid_layers(self):
         return [m for _, m in self._get_qc_quantized_layers(self.model) if isinstance(m, StaticGridQuantWrapper)]

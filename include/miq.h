@@ -176,6 +176,40 @@ int miq_ste_bwd_per_channel_bf16(const uint16_t* x, const uint16_t* grad_out, ui
                                  const float* enc_min, const float* enc_max, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
+ * Several tensors in one launch.  A simulation model quantizes every parameter tensor in every forward
+ * (StaticGridQuantWrapper._quantize_dequantize_params, TORCH/v1/qc_quantize_op.py:705-763, one
+ * quantizeDequantizePerChannel call per tensor); for the dozens of small tensors of a convolutional network the
+ * launches' fixed cost exceeds their traffic.  One launch takes a table of segments instead; each segment is
+ * miq_qdq_per_channel_* on its own tensor (nearest rounding), results identical.  No counterpart in the reference.
+ * A per-tensor encoding is a segment with num_channel = 1 and one-element parameter vectors (the values
+ * miq_fill_encoding_info gives, as float32).
+ * ------------------------------------------------------------------------------------------------------------- */
+typedef struct miq_qdq_segment
+{
+    const void* in;                    /* device: float32 or bfloat16 elements, 16-byte aligned */
+    void* out;                         /* device, 16-byte aligned; may be `in` */
+    int64_t num_element;               /* 1 .. 2^31 - 1 */
+    int64_t num_channel;
+    int64_t num_element_per_channel;   /* at least 8 (float32) / 16 (bfloat16) */
+    const float* enc_min;              /* device float[num_channel]: as miq_qdq_per_channel_* takes them */
+    const float* enc_max;
+    const float* enc_delta;
+    const float* enc_offset;
+    uint32_t fd_magic, fd_shift;       /* filled by miq_qdq_multi_plan */
+    int32_t first_tile;                /* filled by miq_qdq_multi_plan */
+    int32_t reserved;
+} miq_qdq_segment;
+/* Host side, once per table: checks every segment, fills the fields marked above and returns the number of tiles of
+ * the launch (-1 with miq_last_error() set when a segment cannot take part: the caller quantizes that one by itself).
+ * segments: HOST array of 1 .. 256 records; the caller then copies it to device memory. */
+int64_t miq_qdq_multi_plan(miq_qdq_segment* segments /* host, in/out */, int num_segments, int elem_bytes);
+/* segments: the planned table in DEVICE memory; total_tiles: what miq_qdq_multi_plan returned for it. */
+int miq_qdq_per_channel_multi_f32(const miq_qdq_segment* segments /* device */, int num_segments, int64_t total_tiles,
+                                  void* stream);
+int miq_qdq_per_channel_multi_bf16(const miq_qdq_segment* segments /* device */, int num_segments, int64_t total_tiles,
+                                   void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
  * Straight-through estimator through a saved one-bit mask.
  * The reference's v2 QuantDequantFunc saves the mask of its backward as a bool tensor, one byte per element
  * (TORCH/v2/quantization/affine/backends/torch_builtins.py:303-327); its v1 QuantizeDequantize keeps the input alive

@@ -26,6 +26,15 @@ def test_cfg4_every_quantizer_matches_the_oracle(oracle):
     with torch.no_grad():
         plain = sim.model(x).cpu()
 
+    # compute_encodings() left every weight quantized by ONE multi-tensor launch; those tensors are checked against the
+    # oracle below, then dropped so that the checked pass sees every quantizer at work
+    from_multi_launch = {}
+    for _, w in wrappers:
+        for name, (_, kept) in w.__dict__.get('_param_cache', {}).items():
+            from_multi_launch[dict(w.get_named_parameters())[name].data_ptr()] = kept
+        w.invalidate_param_cache()
+    assert len(from_multi_launch) == enabled_par
+
     seen = {"per_tensor": 0, "per_channel": 0, "elements": 0}
     real = tq.StaticGridTensorQuantizer.quantize_dequantize
 
@@ -43,6 +52,8 @@ def test_cfg4_every_quantizer_matches_the_oracle(oracle):
                                                self.bitwidth)
             want = oracle.qdq_per_channel(host, c, npc, params)
             seen["per_channel"] += 1
+            kept = from_multi_launch[tensor.data_ptr()]
+            assert np.array_equal(kept.cpu().numpy().view(np.uint32), want.view(np.uint32)), "multi-tensor launch"
         else:
             enc = self.encoding
             want = oracle.qdq_per_tensor(host, enc.min, enc.max, self.bitwidth)
@@ -70,3 +81,54 @@ def test_cfg4_every_quantizer_matches_the_oracle(oracle):
     diff = (plain - through_oracle).abs()
     assert diff.max().item() <= 0.05 * scale
     assert diff.mean().item() <= 0.005 * scale
+
+
+def test_quantized_parameters_are_kept_between_forwards():
+    """In evaluation mode a wrapper keeps its quantized parameters while parameter and encoding stay the same, and
+    compute_encodings() fills every wrapper from one multi-tensor launch: same outputs as quantizing in every forward,
+    and every change that the key sees (in-place update of the parameter, a new encoding, training mode) is seen."""
+    from aimet_amd.v1.qc_quantize_op import StaticGridQuantWrapper
+    from aimet_amd.v1.quantsim import QuantizationSimModel
+    torch.manual_seed(0)
+    model = torch.nn.Sequential(torch.nn.Conv2d(3, 16, 3, padding=1), torch.nn.ReLU(), torch.nn.Conv2d(16, 32, 1),
+                                torch.nn.ReLU(), torch.nn.AdaptiveAvgPool2d(1), torch.nn.Flatten(),
+                                torch.nn.Linear(32, 10)).eval().cuda()
+    x = torch.randn(4, 3, 16, 16).cuda()
+    sim = QuantizationSimModel(model, dummy_input=x, quant_scheme='tf', default_param_bw=4)
+    sim.compute_encodings(lambda m, a: m(a), x)
+    layers = [w for _, w in sim.quant_wrappers() if w.param_quantizers]
+    assert all('weight' in w.__dict__['_param_cache'] for w in layers)       # filled by compute_encodings
+    assert sim.quantize_params_together() >= 3
+
+    def forward(cached):
+        StaticGridQuantWrapper.cache_quantized_params = cached
+        try:
+            with torch.no_grad():
+                return sim.model(x)
+        finally:
+            StaticGridQuantWrapper.cache_quantized_params = True
+
+    assert torch.equal(forward(True), forward(False))
+    conv = layers[0]
+    kept = conv.__dict__['_param_cache']['weight'][1]
+    forward(True)
+    assert conv.__dict__['_param_cache']['weight'][1] is kept               # used again, not recomputed
+    with torch.no_grad():
+        conv._module_to_wrap.weight.mul_(1.5)                                # in place on the parameter: version moves
+    assert torch.equal(forward(True), forward(False))
+    assert conv.__dict__['_param_cache']['weight'][1] is not kept
+    q = conv.param_quantizers['weight']
+    from aimet_amd.common import libpymo
+    old = q.encoding if isinstance(q.encoding, list) else [q.encoding]
+    new = [libpymo.TfEncoding(e.min * 0.5, e.max * 0.5, e.delta * 0.5, e.offset, e.bw) for e in old]
+    q.encoding = new if isinstance(q.encoding, list) else new[0]             # a new encoding
+    assert torch.equal(forward(True), forward(False))
+    sim.model.train()
+    out_train = sim.model(x)
+    sim.model.eval()
+    assert torch.isfinite(out_train).all() and torch.equal(forward(True), forward(False))
+    # through a .data alias nothing moves: the documented way out
+    conv._module_to_wrap.weight.data.mul_(2.0)
+    for w in layers:
+        w.invalidate_param_cache()
+    assert torch.equal(forward(True), forward(False))

@@ -393,3 +393,43 @@ def test_kernels_run_on_torch_current_stream(ops, oracle):
     assert mm.tolist() == [pytest.approx(0.7), pytest.approx(0.7)]
     xl, pdf = an.get_stats_histogram()
     assert pdf.sum() == pytest.approx(1.0) and (pdf > 0).sum() == 1
+
+
+# ------------------------------------------------------------------------------------- several tensors in one launch
+def test_multi_tensor_launch(ops, oracle):
+    """One launch over a table of tensors: every tensor's result is that of its own per-channel call (and the
+    oracle's), for ragged shapes, a per-tensor encoding (one channel), an outer axis, bf16; what cannot take part is
+    refused."""
+    rng = np.random.default_rng(77)
+    shapes = [((64, 3, 7, 7), 64, 147), ((256, 64, 1, 1), 256, 64), ((96, 33, 3, 3), 96, 297), ((1000, 2048), 1000, 2048),
+              ((5, 4099), 5, 4099), ((3, 8, 50), 8, 50), ((7, 6001), 1, 42007), ((16, 9), 16, 9)]
+    entries, want = [], []
+    for k, (shape, c, npc) in enumerate(shapes):
+        x = _normal(300 + k, shape, 0.3)
+        enc_min = -np.abs(rng.standard_normal(c)) * 0.4
+        enc_max = np.abs(rng.standard_normal(c)) * 0.4
+        params = oracle.per_channel_params(enc_min, enc_max, 8 if k % 2 else 4)
+        entries.append((_gpu(x), c, npc, *[_gpu(p) for p in params]))
+        want.append(oracle.qdq_per_channel(x, c, npc, params))
+    multi = ops.QdqMulti(entries)
+    for _ in range(2):                       # the prepared launch is reusable
+        outs = multi()
+        for e, out, w in zip(entries, outs, want):
+            assert np.array_equal(_bits(out.cpu().numpy()), _bits(w))
+            assert torch.equal(out, ops.qdq_per_channel(e[0], e[1], e[2], *e[3:7]))
+        for out in outs:
+            out.zero_()
+    # bf16 storage
+    bentries = [(e[0].to(torch.bfloat16), *e[1:]) for e in entries[:-1]]    # 9 elements per channel: too few for bf16
+    bouts = ops.QdqMulti(bentries)()
+    for e, out in zip(bentries, bouts):
+        assert torch.equal(out.view(torch.int16), ops.qdq_per_channel(e[0], e[1], e[2], *e[3:7]).view(torch.int16))
+    # tiny channels / unaligned data cannot take part
+    x = _gpu(_normal(1, (40, 4), 1.0))
+    p4 = [_gpu(p) for p in oracle.per_channel_params(-np.ones(40), np.ones(40), 8)]
+    with pytest.raises(RuntimeError, match="multi-tensor"):
+        ops.QdqMulti([(x, 40, 4, *p4)])
+    base = _gpu(_normal(2, 4097, 1.0))
+    p1 = [_gpu(p) for p in oracle.per_channel_params(-np.ones(1), np.ones(1), 8)]
+    with pytest.raises(RuntimeError, match="multi-tensor"):
+        ops.QdqMulti([(base[1:], 1, 4096, *p1)])
