@@ -62,6 +62,12 @@ class AimetTensorQuantizer:
                                                      useUnsignedSymmetric)
         return _to_tf_encoding(enc), bool(valid)
 
+    def queueEncoding(self, bitwidth: int, useSymmetricEncodings: bool, useStrictSymmetric: bool,
+                      useUnsignedSymmetric: bool) -> None:
+        """Start the device work of the next getEncoding call with the same arguments; does not wait."""
+        if self._is_encoding_valid and self._analyzer is not None:
+            self._analyzer.queue_encoding(bitwidth, useSymmetricEncodings, useStrictSymmetric, useUnsignedSymmetric)
+
     def getStatsHistogram(self) -> List[Tuple[float, float]]:
         if self._scheme == QuantizationMode.QUANTIZATION_TF:
             raise RuntimeError("no histogram is kept by the TF (min/max) analyzer")

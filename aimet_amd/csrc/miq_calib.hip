@@ -1039,6 +1039,11 @@ struct miq_analyzer
     float bucket_f, pdf_offset_f;   // valid once range_known
     uint32_t seq;        // number of TF-Enhanced update calls since the last reset
     int last_bw;
+    // an encoding request queued ahead of its read-back (miq_analyzer_queue_encoding): valid while nothing else has
+    // been asked of the object since
+    bool queued;
+    int queued_args[4];
+    hipStream_t queued_stream;
 };
 
 extern "C" {
@@ -1253,6 +1258,7 @@ int miq_analyzer_set_percentile(miq_analyzer* a, float percentile)
     MIQ_CHECK_ARG(percentile >= 0.0f && percentile <= 100.0f, "percentile must be in [0, 100] (got %g)",
                   (double) percentile);
     a->percentile = percentile;
+    a->queued     = false;
     return MIQ_OK;
 }
 
@@ -1273,6 +1279,7 @@ int miq_analyzer_reset(miq_analyzer* a, void* stream)
     hipLaunchKernelGGL(reset_state_kernel, dim3(1), dim3(kPdf), 0, (hipStream_t) stream, a->st);
     MIQ_CHECK_LAUNCH();
     a->needs_reset = false;
+    a->queued      = false;
     a->stats_updated = false;
     a->range_known   = false;
     a->seq           = 0;
@@ -1291,6 +1298,7 @@ int miq_analyzer_update_stats_f32(miq_analyzer* a, const float* data, int64_t n,
     if (int rc = ensure_reset(a, s))
         return rc;
     a->stats_updated = true;
+    a->queued        = false;
     const int grid    = hist_grid(n);
     const int mm_grid = (int) std::max<int64_t>(
         1, std::min<int64_t>(kMmGrid, (n / 4 + (int64_t) kMmBlock * kMmUnroll - 1) / ((int64_t) kMmBlock * kMmUnroll)));
@@ -1363,11 +1371,20 @@ static int flush_pending(miq_analyzer* a, hipStream_t s)
     return MIQ_OK;
 }
 
-static int read_state(miq_analyzer* a, hipStream_t s, size_t bytes = kInspectBytes)
+static int finish_read(miq_analyzer* a, hipStream_t s);
+static int read_state(miq_analyzer* a, hipStream_t s, size_t bytes = kInspectBytes, bool wait = true)
 {
+    a->queued = false;   // the staging buffer is about to be overwritten
     if (int rc = ensure_reset(a, s))
         return rc;
     MIQ_CHECK_HIP(hipMemcpyAsync(a->pinned, a->st, bytes, hipMemcpyDeviceToHost, s));
+    if (!wait)
+        return MIQ_OK;
+    return finish_read(a, s);
+}
+
+static int finish_read(miq_analyzer* a, hipStream_t s)
+{
     MIQ_CHECK_HIP(hipStreamSynchronize(s));
     const DevState* h = static_cast<const DevState*>(a->pinned);
     if (h->initialized)
@@ -1376,6 +1393,43 @@ static int read_state(miq_analyzer* a, hipStream_t s, size_t bytes = kInspectByt
         a->bucket_f     = h->bucket_f;
         a->pdf_offset_f = h->pdf_offset_f;
     }
+    return MIQ_OK;
+}
+
+// Everything of compute_encoding that can be queued: the pending batch folded, the search launched, the copy of the
+// results into the staging buffer requested.  Nothing waits.
+static int queue_encoding(miq_analyzer* a, int bw, int use_symmetric, int use_strict_symmetric,
+                          int use_unsigned_symmetric, hipStream_t s)
+{
+    if (a->mode == MIQ_QUANTIZATION_TF)
+        return read_state(a, s, kHeadBytes, false);
+    if (int rc = flush_pending(a, s))
+        return rc;
+    if (a->mode == MIQ_QUANTIZATION_PERCENTILE)
+        return read_state(a, s, kInspectBytes, false);
+    const SearchArgs sa = tfe::make_search_args(bw, use_symmetric, use_strict_symmetric, use_unsigned_symmetric);
+    MIQ_CHECK_ARG(sa.n_cand <= kMaxCand, "internal: candidate grid too large");
+    hipLaunchKernelGGL(tfe_search_kernel, dim3((sa.n_cand + kBlock / 64 - 1) / (kBlock / 64)), dim3(kBlock), 0, s, a->st,
+                       sa);
+    MIQ_CHECK_LAUNCH();
+    return read_state(a, s, kHeadBytes, false);
+}
+
+int miq_analyzer_queue_encoding(miq_analyzer* a, int bw, int use_symmetric, int use_strict_symmetric,
+                                int use_unsigned_symmetric, void* stream)
+{
+    MIQ_CHECK_ARG(a != nullptr, "null argument");
+    MIQ_CHECK_ARG(bw >= 1 && bw <= 32, "bitwidth must be in [1, 32] (got %d)", bw);
+    if (!a->stats_updated)
+        return MIQ_OK;
+    if (int rc = queue_encoding(a, bw, use_symmetric, use_strict_symmetric, use_unsigned_symmetric, (hipStream_t) stream))
+        return rc;
+    a->queued         = true;
+    a->queued_args[0] = bw;
+    a->queued_args[1] = use_symmetric != 0;
+    a->queued_args[2] = use_strict_symmetric != 0;
+    a->queued_args[3] = use_unsigned_symmetric != 0;
+    a->queued_stream  = (hipStream_t) stream;
     return MIQ_OK;
 }
 
@@ -1389,11 +1443,18 @@ int miq_analyzer_compute_encoding(miq_analyzer* a, int bw, int use_symmetric, in
     *is_valid = a->stats_updated ? 1 : 0;
     if (!a->stats_updated)
         return MIQ_OK;   // AimetTensorQuantizer::getEncoding returns a default encoding and valid = false
+    const bool ahead = a->queued && a->queued_stream == s && a->queued_args[0] == bw &&
+                       a->queued_args[1] == (use_symmetric != 0) && a->queued_args[2] == (use_strict_symmetric != 0) &&
+                       a->queued_args[3] == (use_unsigned_symmetric != 0);
+    if (!ahead)
+        if (int rc = queue_encoding(a, bw, use_symmetric, use_strict_symmetric, use_unsigned_symmetric, s))
+            return rc;
+    a->queued = false;
+    if (int rc = finish_read(a, s))
+        return rc;
+    const DevState* h = static_cast<const DevState*>(a->pinned);
     if (a->mode == MIQ_QUANTIZATION_TF)
     {
-        if (int rc = read_state(a, s, kHeadBytes))
-            return rc;
-        const DevState* h = static_cast<const DevState*>(a->pinned);
         // DLQ/src/TfEncodingAnalyzer.cpp:80-101 (MIN_RANGE = 0.01)
         double lo = std::min(0.0, h->acc_min);
         double hi = std::max(0.0, h->acc_max);
@@ -1401,24 +1462,8 @@ int miq_analyzer_compute_encoding(miq_analyzer* a, int bw, int use_symmetric, in
         return miq_get_computed_encodings(bw, lo, hi, use_symmetric, use_strict_symmetric, use_unsigned_symmetric, out);
     }
     if (a->mode == MIQ_QUANTIZATION_PERCENTILE)
-    {
-        if (int rc = flush_pending(a, s))
-            return rc;
-        if (int rc = read_state(a, s))
-            return rc;
-        return percentile_encoding(static_cast<const DevState*>(a->pinned), a->percentile, bw, use_symmetric,
-                                   use_strict_symmetric, use_unsigned_symmetric, out);
-    }
-    const SearchArgs sa = tfe::make_search_args(bw, use_symmetric, use_strict_symmetric, use_unsigned_symmetric);
-    MIQ_CHECK_ARG(sa.n_cand <= kMaxCand, "internal: candidate grid too large");
-    if (int rc = flush_pending(a, s))
-        return rc;
-    hipLaunchKernelGGL(tfe_search_kernel, dim3((sa.n_cand + kBlock / 64 - 1) / (kBlock / 64)), dim3(kBlock), 0, s, a->st,
-                       sa);
-    MIQ_CHECK_LAUNCH();
-    if (int rc = read_state(a, s, kHeadBytes))
-        return rc;
-    const DevState* h = static_cast<const DevState*>(a->pinned);
+        return percentile_encoding(h, a->percentile, bw, use_symmetric, use_strict_symmetric, use_unsigned_symmetric,
+                                   out);
     out->min    = h->enc_min;
     out->max    = h->enc_max;
     out->delta  = h->enc_delta;

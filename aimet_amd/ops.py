@@ -843,6 +843,12 @@ class Analyzer(_StateOwner):
             with torch.cuda.device(self.device):
                 check(lib.miq_analyzer_update_stats_f32(self._h, x.data_ptr(), x.numel(), self._s()))
 
+    def queue_encoding(self, bw, symmetric=False, strict_symmetric=False, unsigned_symmetric=False):
+        """Queue the device work of the next compute_encoding call with these arguments without waiting for it."""
+        with torch.cuda.device(self.device):
+            check(lib.miq_analyzer_queue_encoding(self._h, int(bw), int(bool(symmetric)), int(bool(strict_symmetric)),
+                                                  int(bool(unsigned_symmetric)), self._s()))
+
     def compute_encoding(self, bw, symmetric=False, strict_symmetric=False, unsigned_symmetric=False):
         """returns (Encoding, is_valid)"""
         e, valid = Encoding(), C.c_int(0)

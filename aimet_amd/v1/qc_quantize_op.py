@@ -405,6 +405,43 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
     def invalidate_param_cache(self):
         self.__dict__['_param_cache'] = {}
 
+    @staticmethod
+    def _observe_param(quantizer, param):
+        """The statistics of a parameter quantizer are those of the parameter as it is now (reference :769-777)."""
+        quantizer.reset_encoding_stats()
+        quantizer.update_encoding_stats(param.data)
+        if quantizer.quant_scheme == QuantScheme.post_training_percentile:
+            quantizer.set_percentile_value(100)
+
+    @staticmethod
+    def _param_identity(param):
+        return (param.data_ptr(), param._version, tuple(param.shape), param.dtype)  # pylint: disable=protected-access
+
+    def observe_params_ahead(self):
+        """What the first forward after a reset does for every parameter that has no encoding yet (reference
+        :769-777), taken out of that forward: the statistics of all parameters of a model are queued here, and the
+        encodings are read back by compute_param_encodings_ahead() before the calibration batches occupy the device,
+        instead of one wait per parameter in the middle of the first batch.  A parameter that is replaced or changed in
+        place before its wrapper's next forward is observed again there, as the reference would see it.  Returns the
+        quantizers that were fed."""
+        fed = []
+        if self._module_to_wrap.training:
+            return fed                      # recomputed in every pass anyway
+        ahead = self.__dict__.setdefault('_param_encodings_ahead', {})
+        for name, param in self.get_named_parameters():
+            quantizer = self.param_quantizers[name]
+            if quantizer.enabled and quantizer.bitwidth != 32 and quantizer.encoding is None and param.is_cuda:
+                self._observe_param(quantizer, param)
+                ahead[name] = self._param_identity(param)
+                fed.append(quantizer)
+        return fed
+
+    def drop_params_observed_in_vain(self):
+        """A wrapper whose forward never ran since observe_params_ahead() would not have fed its parameter quantizers
+        in the reference: their statistics go, so that compute_encoding() switches them off as it does there."""
+        for name in self.__dict__.pop('_param_encodings_ahead', {}):
+            self.param_quantizers[name].reset_encoding_stats()
+
     def _quantize_dequantize_params(self):
         shadow_params = {}
         keep = self._params_may_be_kept()
@@ -414,11 +451,10 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
             quantizer = self.param_quantizers[name]
             if quantizer.enabled and quantizer.bitwidth != 32:
                 # in training mode the parameter encodings are recomputed in every pass
-                if self._module_to_wrap.training or quantizer.encoding is None:
-                    quantizer.reset_encoding_stats()
-                    quantizer.update_encoding_stats(param.data)
-                    if quantizer.quant_scheme == QuantScheme.post_training_percentile:
-                        quantizer.set_percentile_value(100)
+                ahead = self.__dict__.get('_param_encodings_ahead')
+                stale = ahead is not None and ahead.pop(name, None) not in (None, self._param_identity(param))
+                if self._module_to_wrap.training or quantizer.encoding is None or stale:
+                    self._observe_param(quantizer, param)
                     quantizer.compute_encoding()
                 if keep and quantizer.encoding is not None:
                     key = self._param_cache_key(param, quantizer)

@@ -469,10 +469,16 @@ class QuantizationSimModel:
         was_training = self.model.training
         self.model.eval()
         try:
+            # parameter encodings do not depend on the batches: observed and read back while the device is idle
+            fed = [q for layer in self._static_grid_layers() for q in layer.observe_params_ahead()]
+            for quantizer in fed:
+                quantizer.compute_encoding()
             with torch.no_grad():
                 forward_pass_callback(self.model, forward_pass_callback_args)
         finally:
             self.model.train(was_training)
+            for layer in self._static_grid_layers():
+                layer.drop_params_observed_in_vain()
         self.compute_layer_encodings_for_sim()
         if not self.model.training:
             self.quantize_params_together()
@@ -544,7 +550,13 @@ class QuantizationSimModel:
     def compute_layer_encodings_for_sim(self):
         """Encodings from the gathered statistics, wrappers back to ACTIVE; a quantizer that saw no data is switched
         off (reference :405-423)."""
-        for layer in self._static_grid_layers():
+        layers = self._static_grid_layers()
+        # every per-tensor search is started before the first result is waited for: one round trip to the device for
+        # the whole model instead of one per quantizer
+        for layer in layers:
+            for quantizer in list(layer.input_quantizers) + list(layer.output_quantizers):
+                quantizer.queue_encoding()
+        for layer in layers:
             layer.compute_encoding()
             layer.set_mode(QcQuantizeOpMode.ACTIVE)
         self.replace_wrappers_for_quantize_dequantize()

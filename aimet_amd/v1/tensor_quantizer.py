@@ -137,7 +137,7 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         state['_num_ops'] = len(self._cppOp)
         state['_encoding'] = None if self._encoding is None else \
             [(e.min, e.max, e.delta, e.offset, e.bw) for e in self._encoding]
-        for key in ('_cppOp', '_dev_params', '_fp8_grid', '_channel_analyzer'):
+        for key in ('_cppOp', '_dev_params', '_fp8_grid', '_channel_analyzer', '_computed_from'):
             state.pop(key, None)
         return state
 
@@ -162,6 +162,7 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         self._quant_scheme = quant_scheme
         assert self._cppOp
         self._cppOp = [AimetTensorQuantizer(MAP_QUANT_SCHEME_TO_PYMO[quant_scheme]) for _ in self._cppOp]
+        self._stats_changed()
         self._drop_fused_stats()
 
     @property
@@ -193,9 +194,24 @@ class StaticGridTensorQuantizer(TensorQuantizer):
             return torch.tensor(list(self.encoding_min_max_fixed_vals), dtype=torch.float32, device=tensor.device)
         return tensor
 
+    def _stats_changed(self):
+        """Every update / reset of the statistics (and of what turns them into encodings) counts up."""
+        self.__dict__['_stats_version'] = self.__dict__.get('_stats_version', 0) + 1
+
+    def _encoding_recipe(self):
+        return (self.__dict__.get('_stats_version', 0), self.bitwidth, self.data_type, self.use_symmetric_encodings,
+                self.use_strict_symmetric, self.use_unsigned_symmetric, self._quant_scheme,
+                self.encoding_min_max_fixed_vals, getattr(self, '_percentile_value', None))
+
     def compute_encoding(self):
         """Compute the encoding(s) from the accumulated statistics; skipped for bitwidth 32 (reference :280-321)."""
         if self.enabled and not self._is_encoding_frozen:
+            # The same statistics and settings give the same encodings: the simulation model asks twice for every
+            # parameter (once when the first forward needs the encoding, once at the end of compute_encodings), and
+            # a per-channel answer costs a search launch, a read-back and thousands of encoding objects
+            recipe, result = self.__dict__.get('_computed_from') or (None, None)
+            if self._encoding and result is self._encoding and recipe == self._encoding_recipe():
+                return
             self._encoding = []
             self._dev_params = None
             if self.bitwidth == 32 or self.data_type == QuantizationDataType.float:
@@ -215,10 +231,19 @@ class StaticGridTensorQuantizer(TensorQuantizer):
                 all(enc.min >= 0 and enc.max >= 0 for enc in self._encoding)
             assert not (not self.enabled and self._encoding), \
                 'At least one encoding for a multi-encoding quantizer is invalid.'
+            self.__dict__['_computed_from'] = (self._encoding_recipe(), self._encoding) if self.enabled else None
 
     def _compute_op_encodings(self):
         return [op.getEncoding(self.bitwidth, self.use_symmetric_encodings, self.use_strict_symmetric,
                                self.use_unsigned_symmetric) for op in self._cppOp]
+
+    def queue_encoding(self):
+        """Queue the device work of the next compute_encoding() call without waiting for it.  An owner of many
+        quantizers calls this on all of them first: the read-backs that follow then share one wait for the device."""
+        if self.enabled and not self._is_encoding_frozen and self.bitwidth != 32 and \
+                self.data_type != QuantizationDataType.float and len(self._cppOp) == 1:
+            self._cppOp[0].queueEncoding(self.bitwidth, self.use_symmetric_encodings, self.use_strict_symmetric,
+                                         self.use_unsigned_symmetric)
 
     def quantize_dequantize(self, tensor: torch.Tensor, round_mode: libpymo.RoundingMode) -> torch.Tensor:
         if not torch.is_grad_enabled():
@@ -231,6 +256,7 @@ class StaticGridTensorQuantizer(TensorQuantizer):
 
     def reset_encoding_stats(self):
         if not self._is_encoding_frozen:
+            self._stats_changed()
             for op in self._cppOp:
                 op.resetEncodingStats()
             self._encoding = None
@@ -249,6 +275,7 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         self._is_encoding_frozen = True
 
     def set_percentile_value(self, percentile_value: float):
+        self._stats_changed()
         for op in self._cppOp:
             op.setPercentileValue(percentile_value)
 
@@ -274,6 +301,7 @@ class StaticGridPerTensorQuantizer(StaticGridTensorQuantizer):
 
     def update_encoding_stats(self, tensor: torch.Tensor):
         if self.enabled and not self._is_encoding_frozen:
+            self._stats_changed()
             if self._is_fp8:
                 self._fp8_observe(tensor, per_channel=False)
                 return
@@ -300,7 +328,14 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
         return self._ch_axis
 
     def reset_encoding_stats(self):
-        super().reset_encoding_stats()
+        if self.__dict__.get('_ops_hold_stats', True):
+            super().reset_encoding_stats()           # walks the per-channel objects (thousands of calls)
+            self.__dict__['_ops_hold_stats'] = False
+        elif not self._is_encoding_frozen:
+            # the per-channel objects never saw a tensor: the statistics live in the fused objects below
+            self._stats_changed()
+            self._encoding = None
+            self._dev_params = None
         if not self._is_encoding_frozen:
             self._tf_minmax = None
             if self._channel_analyzer is not None:
@@ -332,6 +367,7 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
 
     def update_encoding_stats(self, tensor: torch.Tensor):
         if self.enabled and not self._is_encoding_frozen:
+            self._stats_changed()
             if self._is_fp8:
                 self._fp8_observe(tensor, per_channel=True)
                 return
@@ -339,6 +375,7 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
                 return
             if self.encoding_min_max_fixed_vals is not None:
                 fixed = self._stats_tensor(tensor)
+                self.__dict__['_ops_hold_stats'] = True
                 for op in self._cppOp:
                     op.updateStats(fixed, fixed.is_cuda)
                 return

@@ -712,6 +712,123 @@ def bench_quantsim(torch, steps=10, batch=64):
             "latency_batch1": lat}
 
 
+def bench_end_to_end(torch, ops):
+    """The two entry points a user calls, timed whole: QuantizationSimModel.compute_encodings on the ResNet-50-shaped
+    net (TF-Enhanced analyzers on every activation, per-channel on every weight) against the plain forward over the
+    same batches, and Adaround.apply_adaround on a small multi-layer model against the isolated iteration loop.
+    "host" is the time until the Python call has queued everything (the device may still be working), "wall" the time
+    until the device is done as well: where the two agree, the host paces the run."""
+    import tempfile
+    from aimet_amd.v1.quantsim import QuantizationSimModel
+    dev = torch.device("cuda", 0)
+    out = {}
+    # ---- compute_encodings
+    model = _resnet50_shaped(torch).to(dev)
+    g = torch.Generator(device=dev).manual_seed(1004)
+    num_batches, batch = 4, 64
+    data = [torch.randn(batch, 3, 224, 224, device=dev, generator=g) for _ in range(num_batches)]
+    cfg = {"defaults": {"ops": {"is_output_quantized": "True"},
+                        "params": {"is_quantized": "True", "is_symmetric": "True"},
+                        "strict_symmetric": "False", "per_channel_quantization": "True"},
+           "params": {"bias": {"is_quantized": "False"}},
+           "op_type": {"Flatten": {"is_output_quantized": "False"}},
+           "supergroups": [{"op_list": ["Conv", "Relu"]}, {"op_list": ["Add", "Relu"]}],
+           "model_input": {"is_input_quantized": "True"}, "model_output": {}}
+    with tempfile.NamedTemporaryFile("w", suffix=".json", delete=False) as f:
+        json.dump(cfg, f)
+    sim = QuantizationSimModel(model, dummy_input=data[0][:2], quant_scheme='tf_enhanced', default_output_bw=8,
+                               default_param_bw=8, config_file=f.name)
+    os.unlink(f.name)
+
+    def passes(m, batches):
+        for xb in batches:
+            m(xb)
+
+    seen = {"elements": 0, "updates": 0}
+    real_update = ops.Analyzer.update_stats
+
+    def counting(self, x):
+        seen["elements"] += x.numel()
+        seen["updates"] += 1
+        return real_update(self, x)
+
+    with torch.no_grad():
+        for _ in range(2):
+            passes(model, data)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        passes(model, data)
+        host_fp32 = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        wall_fp32 = time.perf_counter() - t0
+    sim.compute_encodings(passes, data[:1])                     # warm-up (kernels, allocator)
+    ops.Analyzer.update_stats = counting
+    try:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        sim.compute_encodings(passes, data)
+        host_cal = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        wall_cal = time.perf_counter() - t0
+    finally:
+        ops.Analyzer.update_stats = real_update
+    n_act = sum(q.enabled for _, w in sim.quant_wrappers() for q in w.input_quantizers + w.output_quantizers)
+    n_par = sum(q.enabled for _, w in sim.quant_wrappers() for q in w.param_quantizers.values())
+    out["compute_encodings_resnet50_shaped"] = {
+        "scheme": "tf_enhanced", "batches": num_batches, "batch": batch, "activation_analyzers": int(n_act),
+        "param_quantizers_per_channel": int(n_par), "activation_updates": seen["updates"],
+        "activation_elements_observed": seen["elements"],
+        "plain_forward_wall_ms": wall_fp32 * 1e3, "plain_forward_host_ms": host_fp32 * 1e3,
+        "compute_encodings_wall_ms": wall_cal * 1e3, "compute_encodings_host_ms": host_cal * 1e3,
+        "calibration_overhead_pct_of_forward": 100.0 * (wall_cal - wall_fp32) / wall_fp32,
+        "observed_elements_per_s": seen["elements"] / wall_cal,
+        "note": "compute_encodings reads every encoding back at its end, so its host time includes the device's"}
+    del sim, model, data
+    import gc
+    gc.collect()          # the simulation model is a web of reference cycles: collected here, not inside a timed region
+
+    # ---- apply_adaround
+    from aimet_amd.v1.adaround.adaround_weight import Adaround, AdaroundParameters
+    width, layers, iters = 2048, 3, 500
+    torch.manual_seed(1005)
+    mods = []
+    for k in range(layers):
+        mods += [torch.nn.Linear(width, width), torch.nn.ReLU()]
+    net = torch.nn.Sequential(*mods[:-1]).eval().to(dev)
+    loader = [(torch.randn(256, width, device=dev), torch.zeros(256)) for _ in range(4)]
+    params = AdaroundParameters(loader, num_batches=4, default_num_iterations=iters,
+                                forward_fn=lambda m, b: m(b[0]))
+    with tempfile.TemporaryDirectory() as tmp:
+        Adaround.apply_adaround(net, loader[0][0][:2], AdaroundParameters(loader, 4, 20, forward_fn=lambda m, b: m(b[0])),
+                                tmp, "warm", default_param_bw=4)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        Adaround.apply_adaround(net, loader[0][0][:2], params, tmp, "bench", default_param_bw=4)
+        torch.cuda.synchronize()
+        total = time.perf_counter() - t0
+    # the isolated loop on one layer of this size (activations cached, nothing else)
+    from aimet_amd.v1.adaround.adaround_loss import AdaroundHyperParameters
+    from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
+    wrapper, xs, ys = _adaround_layer(torch, out_features=width, in_features=width, rows=1024)
+    hp = AdaroundHyperParameters(iters, 0.01, (20, 2), 0.2)
+    AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, xs, ys, AdaroundHyperParameters(20, 0.01, (20, 2), 0.2))
+    gc.collect()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, xs, ys, hp)
+    torch.cuda.synchronize()
+    loop = time.perf_counter() - t0
+    out["apply_adaround_3x_linear_2048"] = {
+        "layers": layers, "layer": [width, width], "samples": 1024, "iterations_per_layer": iters, "bitwidth": 4,
+        "apply_adaround_s": total, "s_per_layer": total / layers,
+        "ms_per_iteration_end_to_end": total / layers / iters * 1e3,
+        "isolated_loop_s_per_layer": loop, "isolated_ms_per_iteration": loop / iters * 1e3,
+        "outside_the_loop_s_per_layer": total / layers - loop,
+        "note": "outside the loop: building the simulation model, weight encodings, sampling the layer's input and "
+                "output activations through both models, writing the encodings file"}
+    return out
+
+
 def bench_sqnr(torch, ops, reps=5):
     """v2 SQNR analyzer on the calibration workload: 16 batches of [32,256,28,28] through the 2048-bin histogram
     observer (finite min/max + one dual-range binning pass per batch), then the 8-bit asymmetric search."""
@@ -1113,7 +1230,7 @@ def main():
     ap.add_argument("--full", action="store_true", help="(kept for old command lines: every cell is measured anyway)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run a subset of the legs, comma separated (main|pt|fp8|calib|chcalib|sqnr|learn|quantsim|adaround|floors|copyref), for profiling")
+                    help="run a subset of the legs, comma separated (main|pt|fp8|calib|chcalib|sqnr|learn|quantsim|e2e|adaround|floors|copyref), for profiling")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
@@ -1162,6 +1279,8 @@ def main():
         extra["v2_range_learning_backward"] = bench_v2_range_learning(torch, ops)
     if want("quantsim"):
         extra["quantsim_resnet50_shaped"] = bench_quantsim(torch)
+    if want("e2e"):
+        extra["end_to_end"] = bench_end_to_end(torch, ops)
     if want("adaround"):
         extra["adaround_linear_4096"] = bench_adaround(torch, ops, 1000 if args.only is None else args.steps)
         extra["adaround_linear_4096"]["torch_ops_same_gpu"] = torch_ops_adaround_baseline(torch)

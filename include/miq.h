@@ -359,6 +359,16 @@ int miq_analyzer_update_stats_f32(miq_analyzer* a, const float* data, int64_t n,
 int miq_analyzer_compute_encoding(miq_analyzer* a, int bw, int use_symmetric, int use_strict_symmetric,
                                   int use_unsigned_symmetric, miq_encoding* out /* host */, int* is_valid /* host */,
                                   void* stream);
+/* The part of compute_encoding that needs no waiting, queued ahead: the pending batch is folded, the TF-Enhanced search
+ * launched and the copy of its result requested on `stream`.  A compute_encoding call with the same arguments and
+ * stream that follows with no other call on the object in between only waits for that copy, so a caller that owns many
+ * analyzers (one per activation of a model: QuantizationSimModel.compute_encodings,
+ * TrainingExtensions/torch/src/python/aimet_torch/v1/quantsim.py:435-470) queues all of them first and pays for one
+ * round trip to the device instead of one per analyzer.  Any other call on the object drops the request, and
+ * compute_encoding then does all of its work as usual; without statistics the call does nothing.  No counterpart in
+ * the reference, whose analyzers compute on the host. */
+int miq_analyzer_queue_encoding(miq_analyzer* a, int bw, int use_symmetric, int use_strict_symmetric,
+                                int use_unsigned_symmetric, void* stream);
 /* getStatsHistogram() (IQuantizationEncodingAnalyzer.hpp:95-102): 512 (xLeft, pdf) pairs into host arrays.
  * Returns MIQ_ERR_UNSUPPORTED for a TF analyzer (the reference asserts) and writes *num_buckets = 0 while the PDF
  * has not been initialised. */

@@ -237,6 +237,50 @@ def test_tfe_updates_across_streams(ops, oracle):
     _same_search(an, pdf, modes=((8, 0, 0, 0),))
 
 
+@pytest.mark.parametrize("mode", [TF, TFE, 2])
+def test_encodings_queued_ahead(ops, oracle, mode):
+    """Several analyzers whose searches are queued before the first result is read: every answer is the one an
+    analyzer gives that was asked directly.  A request is dropped by any call in between (another batch, other
+    arguments) and the answer is then that of the new state."""
+    def enc_tuple(e):
+        return (e.min, e.max, e.delta, e.offset, e.bw)
+
+    data = [[_gpu(_relu_pareto(900 + 10 * k + b, 120000 + 7 * k)) for b in range(3)] for k in range(6)]
+    queued, direct = [ops.Analyzer(mode) for _ in data], [ops.Analyzer(mode) for _ in data]
+    for group in (queued, direct):
+        for an, batches in zip(group, data):
+            if mode == 2:
+                an.set_percentile(99.9)
+            for b in batches:
+                an.update_stats(b)
+    for an in queued:
+        an.queue_encoding(8, True, False, False)
+    want = [enc_tuple(an.compute_encoding(8, True, False, False)[0]) for an in direct]
+    got = [enc_tuple(an.compute_encoding(8, True, False, False)[0]) for an in queued]
+    assert got == want
+    # other arguments than the queued ones
+    queued[0].queue_encoding(8, True, False, False)
+    assert enc_tuple(queued[0].compute_encoding(4, False, False, False)[0]) == \
+        enc_tuple(direct[0].compute_encoding(4, False, False, False)[0])
+    # another batch after the request
+    extra = _gpu(_relu_pareto(77, 50000) * 3)
+    queued[1].queue_encoding(8, False, False, False)
+    queued[1].update_stats(extra)
+    direct[1].update_stats(extra)
+    assert enc_tuple(queued[1].compute_encoding(8, False, False, False)[0]) == \
+        enc_tuple(direct[1].compute_encoding(8, False, False, False)[0])
+    # a histogram read between request and answer uses the same staging memory
+    if mode != TF:
+        queued[2].queue_encoding(8, False, False, False)
+        queued[2].get_stats_histogram()
+        assert enc_tuple(queued[2].compute_encoding(8, False, False, False)[0]) == \
+            enc_tuple(direct[2].compute_encoding(8, False, False, False)[0])
+    # nothing to queue without statistics
+    fresh = ops.Analyzer(mode)
+    fresh.queue_encoding(8, False, False, False)
+    assert fresh.compute_encoding(8, False, False, False)[1] is False
+
+
 def test_tfe_back_to_back_without_reads(ops, oracle):
     """update_stats calls queued with no read-back between them: a leading all-zero batch (no range yet), ragged batch
     sizes, a reset in the middle; only the final state is read and compared with the oracle fed the same batches."""

@@ -132,3 +132,63 @@ def test_quantized_parameters_are_kept_between_forwards():
     for w in layers:
         w.invalidate_param_cache()
     assert torch.equal(forward(True), forward(False))
+
+
+@pytest.mark.parametrize("scheme", ["tf", "tf_enhanced"])
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_parameter_encodings_taken_ahead_of_the_batches(scheme, per_channel):
+    """compute_encodings() observes the parameters before the calibration batches run.  The encodings are those of a
+    quantizer fed with the parameter as the wrapper's first forward sees it: a weight changed by the callback before
+    that forward is observed again, and a wrapper that never runs loses what was observed for it."""
+    from aimet_amd.v1.quantsim import QuantizationSimModel
+    from aimet_amd.v1.tensor_quantizer import StaticGridPerChannelQuantizer, StaticGridPerTensorQuantizer
+    from aimet_amd.common import libpymo
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = torch.nn.Conv2d(3, 8, 3, padding=1)
+            self.b = torch.nn.Conv2d(8, 8, 1)
+            self.spare = torch.nn.Conv2d(8, 8, 1)
+
+        def forward(self, x):
+            return self.b(torch.relu(self.a(x)))
+
+    torch.manual_seed(3)
+    model = Net().eval().cuda()
+    x = torch.randn(2, 3, 12, 12).cuda()
+    sim = QuantizationSimModel(model, dummy_input=x, quant_scheme=scheme, default_param_bw=8)
+    if per_channel:
+        for _, w in sim.quant_wrappers():
+            if 'weight' in w.param_quantizers:
+                w.enable_per_channel_quantization()
+
+    def callback(m, _):
+        with torch.no_grad():
+            m.b._module_to_wrap.weight.mul_(3.0)          # after the parameters were observed, before b's forward
+        m(x)
+
+    sim.compute_encodings(callback, None)
+
+    def fresh_encoding(like, weight):
+        if isinstance(like, StaticGridPerChannelQuantizer):
+            q = StaticGridPerChannelQuantizer(like.bitwidth, like.round_mode, like.quant_scheme,
+                                              like.use_symmetric_encodings, weight.shape[0], True, ch_axis=0)
+        else:
+            q = StaticGridPerTensorQuantizer(like.bitwidth, like.round_mode, like.quant_scheme,
+                                             like.use_symmetric_encodings, True)
+        q.use_strict_symmetric, q.use_unsigned_symmetric = like.use_strict_symmetric, like.use_unsigned_symmetric
+        q.update_encoding_stats(weight)
+        q.compute_encoding()
+        enc = q.encoding if isinstance(q.encoding, list) else [q.encoding]
+        return [(e.min, e.max, e.delta, e.offset, e.bw) for e in enc]
+
+    for name in ('a', 'b'):
+        wrapper = getattr(sim.model, name)
+        q = wrapper.param_quantizers['weight']
+        assert q.enabled and not wrapper.__dict__.get('_param_encodings_ahead')
+        enc = q.encoding if isinstance(q.encoding, list) else [q.encoding]
+        assert [(e.min, e.max, e.delta, e.offset, e.bw) for e in enc] == \
+            fresh_encoding(q, wrapper._module_to_wrap.weight.data)
+    spare = sim.model.spare.param_quantizers['weight']
+    assert not spare.enabled and not spare.encoding
