@@ -122,19 +122,19 @@ _SIGNATURES = {
     "miq_channel_analyzer_update_stats_f32": ([_p, _p, _i64, _i64, _p, _p], _int),
     "miq_channel_analyzer_compute_encodings": ([_p, _int, _int, _int, _int, _p, C.POINTER(_int), _p], _int),
     "miq_channel_analyzer_get_stats_histogram": ([_p, _i64, _p, _p, C.POINTER(_int), _p], _int),
-    "miq_adaround_linear_workspace_bytes": ([_i64, _i64], _i64),
+    "miq_adaround_linear_workspace_bytes": ([_i64, _i64, _i64], _i64),
     "miq_adaround_linear_blocks": ([_i64, _i64], _int),
-    "miq_adaround_linear_fwd_f32": ([_p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
+    "miq_adaround_linear_fwd_f32": ([_p, _p, _p, _p, _i64, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
                                      _p, _p, _p, _p, _p], _int),
-    "miq_adaround_linear_bwd_adam_f32": ([_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
+    "miq_adaround_linear_bwd_adam_f32": ([_p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
                                           _dbl, _dbl, _dbl, _dbl, _dbl, _dbl, _int, _p, _p], _int),
-    "miq_adaround_linear_fwd_i8": ([_p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
+    "miq_adaround_linear_fwd_i8": ([_p, _p, _p, _p, _i64, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
                                     _p, _p, _p, _p, _p], _int),
-    "miq_adaround_linear_bwd_adam_i8": ([_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
+    "miq_adaround_linear_bwd_adam_i8": ([_p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
                                          _dbl, _dbl, _dbl, _dbl, _dbl, _dbl, _int, _p, _p], _int),
-    "miq_adaround_linear_fwd_i16": ([_p, _p, _p, _p, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
+    "miq_adaround_linear_fwd_i16": ([_p, _p, _p, _p, _i64, _i64, _i64, _p, _i64, _p, _i64, _i64, _i64, _p, _p, _flt, _flt, _int,
                                      _p, _p, _p, _p, _p], _int),
-    "miq_adaround_linear_bwd_adam_i16": ([_p, _p, _p, _p, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
+    "miq_adaround_linear_bwd_adam_i16": ([_p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _p, _p, _i64, _i64, _i64, _p, _p, _flt, _flt,
                                           _dbl, _dbl, _dbl, _dbl, _dbl, _dbl, _int, _p, _p], _int),
 }
 

@@ -7,8 +7,9 @@
 //   loss = recon_loss(act(out), act(y[batch])) + round_loss    ADA/adaround_loss.py:70-111
 //   loss.backward(); Adam step on alpha
 //
-// With 32 rows per iteration the GEMMs are bandwidth-bound on the weight-shaped operands, so the point of fusing is
-// that W' and dLoss/dW' never exist in memory:
+// With 32 rows per iteration (the reference's BATCH_SIZE; 64, 128 and 256 rows are taken as 2, 4 and 8 blocks of 32, which
+// is how a 1x1 convolution over a few pixels arrives here: its rows are the pixels of the 32 images) the GEMMs are
+// bandwidth-bound on the weight-shaped operands, so the point of fusing is that W' and dLoss/dW' never exist in memory:
 //   (W enters as F = floor(W / delta), computed once per layer: W and delta do not change during the optimisation)
 //   lin_fwd_kernel   reads F and alpha once, forms W' in registers and feeds it to 16x16x4 fp32 MFMAs as the B
 //                    operand; the K dimension is split over workgroups, partial [32, O] products go to a workspace
@@ -29,7 +30,8 @@ using namespace ada;
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kBatch  = 32;    // rows per iteration (BATCH_SIZE of ADA/adaround_optimizer.py:58)
+constexpr int kBatch  = 32;    // rows of a block: BATCH_SIZE of ADA/adaround_optimizer.py:58; an iteration has 1, 2, 4 or 8 blocks
+constexpr int kMaxRowBlocks = 8;
 constexpr int kTileO  = 32;    // output channels per workgroup
 constexpr int kTileK  = 256;   // K extent of a tile: one 1 KiB row segment per wavefront-wide 16-byte access
 constexpr int kFwdTileK = 128;        // k extent of a forward tile
@@ -161,11 +163,17 @@ __device__ __forceinline__ int fwd_slot(int r, int chunk)
 // What a workgroup still has to compute when its last bytes arrive (a conversion, then a multiplication) is exposed at
 // the end of the kernel, and loads requested further ahead arrive in larger bunches: small tiles, one tile ahead.
 // Raising the producers' or the consumers' wavefront priority changed nothing or lost 1.5 us.
-template <typename FT, int TK>
-__global__ __launch_bounds__(512, 4) void lin_fwd_kernel(const FT* __restrict__ F, const float* __restrict__ alpha,
-                                                         const float* __restrict__ X, const int* __restrict__ row_index,
-                                                         int num_rows, int64_t x_row_stride, float* __restrict__ partial,
-                                                         LinGeom g, int tiles_per_group)
+//
+// R blocks of 32 rows: the consumers multiply every tile with each block in turn (the tile's W' is read from LDS once
+// per tile, the blocks' activations come through the caches) and keep R partial products; more than two blocks need
+// more registers than four wavefronts per SIMD leave.
+template <typename FT, int TK, int R>
+__global__ __launch_bounds__(512, (R <= 2 ? 4 : 2)) void lin_fwd_kernel(const FT* __restrict__ F,
+                                                                       const float* __restrict__ alpha,
+                                                                       const float* __restrict__ X,
+                                                                       const int* __restrict__ row_index, int num_rows,
+                                                                       int64_t x_row_stride, float* __restrict__ partial,
+                                                                       LinGeom g, int tiles_per_group)
 {
     static_assert(TK == 64 || TK == 128 || TK == 256, "a wavefront-wide 16-byte access covers one, two or four rows of a tile");
     constexpr int kLoads  = 8 * TK / 256;   // 16-byte accesses per lane and tile: 8 rows of TK floats per wavefront
@@ -186,6 +194,7 @@ __global__ __launch_bounds__(512, 4) void lin_fwd_kernel(const FT* __restrict__ 
     float* const buf1 = tile + kTileO * TK;
     v4f* const red    = reinterpret_cast<v4f*>(tile);   // after the last tile: [4 consumers][4 blocks][64 lanes]
     static_assert(2 * kTileO * TK >= 4 * 4 * 64 * 4, "the partial products reuse the tiles' memory");
+    v4f acc[R][2][2];   // consumers only
 
     if (wave >= 4)
     {
@@ -254,38 +263,46 @@ __global__ __launch_bounds__(512, 4) void lin_fwd_kernel(const FT* __restrict__ 
     }
     else
     {
-        // ---- consumer: MFMA layout, lane (n, s) supplies batch rows n and 16 + n, k = TK/4 w4 + 16 kk + 4 s + i
+        // ---- consumer: MFMA layout, lane (n, s) supplies rows n and 16 + n of a block, k = TK/4 w4 + 16 kk + 4 s + i
         const int n = lane & 15, s = lane >> 4;
-        // the row numbers in one load (lane l: batch entry l % 32), passed on by shuffles: a load per use is a chain of
-        // round trips before the first activation can be requested
-        const int row_of_lane = (int) gather_row(row_index, lane & 31, num_rows);
-        const float* xrow[2];
+        // the row numbers of a block in one load (lane l: entry l % 32), passed on by shuffles: a load per use is a
+        // chain of round trips before the first activation can be requested
+        int rows[R][2];
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-            xrow[mt] = X + (int64_t) __shfl(row_of_lane, mt * 16 + n) * x_row_stride + (int64_t) t_first * TK +
-                       w4 * (TK / 4) + 4 * s;
-        v4f acc[2][2];
+        for (int rb = 0; rb < R; ++rb)
+        {
+            const int row_of_lane = (int) gather_row(row_index, rb * kBatch + (lane & 31), num_rows);
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
+            for (int mt = 0; mt < 2; ++mt)
+                rows[rb][mt] = __shfl(row_of_lane, mt * 16 + n);
+        }
+        const float* const xcol = X + (int64_t) t_first * TK + w4 * (TK / 4) + 4 * s;
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
-                acc[mt][nt] = (v4f) {0.f, 0.f, 0.f, 0.f};
+        for (int rb = 0; rb < R; ++rb)
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt)
+                    acc[rb][mt][nt] = (v4f) {0.f, 0.f, 0.f, 0.f};
+        // the activations of (tile, block) units, requested two units ahead of their use
         v4f x[2][kSteps][2];
-        auto request_x = [&](v4f(&xr)[kSteps][2], int i) {
+        auto request_x = [&](v4f(&xr)[kSteps][2], int i, const int(&row)[2]) {
 #pragma unroll
             for (int kk = 0; kk < kSteps; ++kk)
 #pragma unroll
                 for (int mt = 0; mt < 2; ++mt)
-                    xr[kk][mt] = ldg4(xrow[mt] + i * TK + kk * 16);
+                    xr[kk][mt] = ldg4(xcol + (int64_t) row[mt] * x_row_stride + i * TK + kk * 16);
         };
-        auto multiply = [&](const v4f(&xr)[kSteps][2], const float* buf) {
-            v4f wq[kSteps][2];
+        v4f wq[kSteps][2];
+        auto load_w = [&](const float* buf) {
 #pragma unroll
             for (int kk = 0; kk < kSteps; ++kk)
 #pragma unroll
                 for (int nt = 0; nt < 2; ++nt)
                     wq[kk][nt] =
                         *reinterpret_cast<const v4f*>(&buf[fwd_slot<TK>(nt * 16 + n, w4 * (TK / 16) + kk * 4 + s)]);
+        };
+        auto multiply = [&](const v4f(&xr)[kSteps][2], v4f(&ac)[2][2]) {
 #pragma unroll
             for (int kk = 0; kk < kSteps; ++kk)
 #pragma unroll
@@ -294,11 +311,13 @@ __global__ __launch_bounds__(512, 4) void lin_fwd_kernel(const FT* __restrict__ 
                     for (int nt = 0; nt < 2; ++nt)
 #pragma unroll
                         for (int mt = 0; mt < 2; ++mt)
-                            acc[mt][nt] = mfma16(xr[kk][mt][i], wq[kk][nt][i], acc[mt][nt]);
+                            ac[mt][nt] = mfma16(xr[kk][mt][i], wq[kk][nt][i], ac[mt][nt]);
         };
-        request_x(x[0], 0);
-        if (1 < T)
-            request_x(x[1], 1);
+        request_x(x[0], 0, rows[0]);
+        if constexpr (R > 1)
+            request_x(x[1], 0, rows[R > 1 ? 1 : 0]);
+        else if (1 < T)
+            request_x(x[1], 1, rows[0]);
         lds_barrier();
         for (int i0 = 0; i0 < T; i0 += 2)
         {
@@ -308,34 +327,51 @@ __global__ __launch_bounds__(512, 4) void lin_fwd_kernel(const FT* __restrict__ 
                 const int i = i0 + u;
                 if (i >= T)
                     break;
-                multiply(x[u], u == 0 ? buf0 : buf1);
-                if (i + 2 < T)
-                    request_x(x[u], i + 2);
+                load_w(u == 0 ? buf0 : buf1);
+#pragma unroll
+                for (int rb = 0; rb < R; ++rb)
+                {
+                    constexpr int kAhead = 2;                      // units between a request and its use
+                    const int b          = (u * R + rb) & 1;       // the unit's buffer (R is 1 or even)
+                    multiply(x[b], acc[rb]);
+                    const int next_rb = (rb + kAhead) % R, next_i = i + (rb + kAhead) / R;
+                    if (next_i < T)
+                        request_x(x[b], next_i, rows[next_rb]);
+                }
                 lds_barrier();
             }
         }
-        // the barrier above followed every consumer's last multiplication: the tiles' memory is free
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
-                red[(wave * 4 + mt * 2 + nt) * 64 + lane] = acc[mt][nt];
     }
-    // Both roles have passed T + 1 barriers.  Add the four consumers' products in wavefront order, then one partial
-    // [32, 32] block per workgroup.
-    __syncthreads();
-    if (wave < 4)
-    {
-        const int t4 = wave, ln = lane;   // block index, lane within the block
-        const v4f sum = ((red[(0 * 4 + t4) * 64 + ln] + red[(1 * 4 + t4) * 64 + ln]) + red[(2 * 4 + t4) * 64 + ln]) +
-                        red[(3 * 4 + t4) * 64 + ln];
-        const int mt = t4 >> 1, nt = t4 & 1;
-        const int o  = o_blk + nt * 16 + (ln & 15);
-        const int b0 = mt * 16 + 4 * (ln >> 4);
-        float* dst   = partial + ((int64_t) blockIdx.x * kBatch + b0) * g.out_features + o;
+    // Both roles have passed T + 1 barriers, the last of them after every consumer's last multiplication: the tiles'
+    // memory is free.  Block by block, the four consumers' products are added in wavefront order: one partial [32, 32]
+    // product per block and workgroup.
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            dst[(int64_t) i * g.out_features] = sum[i];
+    for (int rb = 0; rb < R; ++rb)
+    {
+        if (rb > 0)
+            __syncthreads();
+        if (wave < 4)
+        {
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < 2; ++nt)
+                    red[(wave * 4 + mt * 2 + nt) * 64 + lane] = acc[rb][mt][nt];
+        }
+        __syncthreads();
+        if (wave < 4)
+        {
+            const int t4 = wave, ln = lane;   // block index, lane within the block
+            const v4f sum = ((red[(0 * 4 + t4) * 64 + ln] + red[(1 * 4 + t4) * 64 + ln]) + red[(2 * 4 + t4) * 64 + ln]) +
+                            red[(3 * 4 + t4) * 64 + ln];
+            const int mt = t4 >> 1, nt = t4 & 1;
+            const int o  = o_blk + nt * 16 + (ln & 15);
+            const int b0 = rb * kBatch + mt * 16 + 4 * (ln >> 4);
+            float* dst   = partial + ((int64_t) blockIdx.x * (R * kBatch) + b0) * g.out_features + o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                dst[(int64_t) i * g.out_features] = sum[i];
+        }
     }
 }
 
@@ -343,12 +379,14 @@ __global__ __launch_bounds__(512, 4) void lin_fwd_kernel(const FT* __restrict__ 
 __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__ partial, int num_split,
                                                        const float* __restrict__ bias, const float* __restrict__ Y,
                                                        const int* __restrict__ row_index, int num_rows,
-                                                       int64_t y_row_stride, int out_features, int act, float* __restrict__ out,
-                                                       float* __restrict__ G, float* __restrict__ loss_partial)
+                                                       int64_t y_row_stride, int out_features, int batch, int act,
+                                                       float* __restrict__ out, float* __restrict__ G,
+                                                       float* __restrict__ loss_partial)
 {
-    const int idx = blockIdx.x * 256 + threadIdx.x;
-    float sq      = 0.f;
-    if (idx < kBatch * out_features)
+    const int idx         = blockIdx.x * 256 + threadIdx.x;
+    const float per_batch = 1.0f / (float) batch;   // a power of two: multiplying is dividing
+    float sq              = 0.f;
+    if (idx < batch * out_features)
     {
         const int b = idx / out_features, o = idx - b * out_features;
         // the row number and the bias are requested before the partial products, and the target as soon as the row
@@ -358,7 +396,7 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
         const float bias_o  = bias ? bias[o] : 0.f;
         // the partial products are added in split order; four of them are requested at a time
         const float* p      = partial + (int64_t) b * out_features + o;
-        const int64_t pitch = (int64_t) kBatch * out_features;
+        const int64_t pitch = (int64_t) batch * out_features;
         float acc           = 0.f;
         int s               = 0;
         float first[4]      = {0.f, 0.f, 0.f, 0.f};
@@ -394,13 +432,13 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
         }
         const float diff = ao - y;
         sq               = diff * diff;
-        G[idx]           = (acc != acc) ? acc : 2.0f * diff * pass * (1.0f / kBatch);
+        G[idx]           = (acc != acc) ? acc : 2.0f * diff * pass * per_batch;
     }
     if (loss_partial)
     {
         const float t = block_sum_256(sq);
         if (threadIdx.x == 0)
-            loss_partial[blockIdx.x] = t * (1.0f / kBatch);
+            loss_partial[blockIdx.x] = t * per_batch;
     }
 }
 
@@ -419,13 +457,18 @@ __global__ __launch_bounds__(256) void lin_loss_kernel(const float* __restrict__
 //       4 epilogue + 4 MFMA wavefronts                                                                      86.5 us
 //       4 epilogue + 1 MFMA wavefront, two or four rows ahead                                         125 / 121 us
 // Eight streaming wavefronts per CU do not keep enough bytes in flight; sixteen with the multiplication in between do.
-template <int PF, typename FT>
+//
+// More than 32 rows (MULTI): the rank-32 product is repeated for every block of 32 rows into the same accumulators, a
+// block's operands being requested when the previous block's multiplications have been issued.
+// in_features that are a multiple of 128 but not of 256: the last tile of a row has 128 columns.  Its workgroups read
+// the first half twice (every address stays inside the row) and the lanes of the missing half store nothing.
+template <int PF, typename FT, bool MULTI>
 __global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, const float* __restrict__ G,
                                                       const float* __restrict__ X, const int* __restrict__ row_index,
                                                       int num_rows, int64_t x_row_stride, float* __restrict__ alpha,
                                                       float* __restrict__ m, float* __restrict__ v,
                                                       float* __restrict__ grad_out, LinGeom g, AdamArgs a,
-                                                      float* __restrict__ reg_partial)
+                                                      float* __restrict__ reg_partial, int row_blocks)
 {
     __shared__ __attribute__((aligned(16))) float tile[kTileO * kLdsRow];
     __shared__ PowEntry tab[128];
@@ -436,6 +479,11 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, 
     PowTableLoad tl;
     tl.request();
     const int K = g.in_features, O = g.out_features;
+    const bool half_tile = k_blk + kTileK > K;          // the same for the whole workgroup
+    const bool live      = k_blk + 4 * lane < K;        // this lane's four columns exist
+    const int k_lane     = k_blk + 4 * lane - (live ? 0 : kTileK / 2);
+    // the 64 columns whose products this wavefront forms: those of wavefront w - 2 again where there are none
+    const int k_wave = k_blk + 64 * (half_tile && wave >= 2 ? wave - 2 : wave);
 
     // per-row delta / offset, requested here and not where they are used (see lin_fwd_kernel); a row belongs to one
     // wavefront, so with the wavefront number as a scalar these are scalar loads
@@ -451,29 +499,33 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, 
     // phase 1's operands are requested first: loads return in the order of their requests, so the multiplication
     // starts once these (cache hits) are back and does not wait for the epilogue's rows requested after them
     float xa[8][4], gb[8][2];
-    // the 32 row numbers in one load (lane l holds that of batch entry l % 32), handed to the lanes that need them by
-    // shuffles: a load per step is a chain of eight round trips.  (Scalar loads of the 32 numbers measured the same.)
-    const int row_of_lane = (int) gather_row(row_index, lane & 31, num_rows);
+    // the 32 row numbers of a block in one load (lane l holds that of entry l % 32), handed to the lanes that need
+    // them by shuffles: a load per step is a chain of eight round trips.  (Scalar loads of the 32 numbers measured
+    // the same.)
+    auto request_block = [&](int rb) {
+        const int row_of_lane = (int) gather_row(row_index, rb * kBatch + (lane & 31), num_rows);
 #pragma unroll
-    for (int step = 0; step < 8; ++step)
-    {
-        const int b       = 4 * step + s;
-        const float* xrow = X + (int64_t) __shfl(row_of_lane, b) * x_row_stride + k_blk + wave * 64 + n;
-        const float* grow = G + (int64_t) b * O + o_blk + n;
+        for (int step = 0; step < 8; ++step)
+        {
+            const int b       = 4 * step + s;
+            const float* xrow = X + (int64_t) __shfl(row_of_lane, b) * x_row_stride + k_wave + n;
+            const float* grow = G + (int64_t) (rb * kBatch + b) * O + o_blk + n;
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-            xa[step][mt] = xrow[mt * 16];
+            for (int mt = 0; mt < 4; ++mt)
+                xa[step][mt] = xrow[mt * 16];
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
-            gb[step][nt] = grow[nt * 16];
-    }
+            for (int nt = 0; nt < 2; ++nt)
+                gb[step][nt] = grow[nt * 16];
+        }
+    };
+    request_block(0);
     __builtin_amdgcn_sched_barrier(0);   // the requests above stay above: nothing below is scheduled between them
     // the epilogue's first rows: they arrive while phase 1 runs
     v4f fv[PF], av[PF], mv[PF], vv[PF];
 #pragma unroll
     for (int j = 0; j < PF; ++j)
     {
-        const int64_t e = (int64_t) (o_blk + wave * 8 + j) * K + k_blk + 4 * lane;
+        const int64_t e = (int64_t) (o_blk + wave * 8 + j) * K + k_lane;
         fv[j]           = load_floor4<FT>(F + e);
         av[j]           = ldg4(alpha + e);
         mv[j]           = ldg4(m + e);
@@ -487,13 +539,19 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, 
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
             acc[mt][nt] = (v4f) {0.f, 0.f, 0.f, 0.f};
+    const int blocks = MULTI ? row_blocks : 1;
+    for (int rb = 0; rb < blocks; ++rb)
+    {
+        if (MULTI && rb > 0)
+            request_block(rb);
 #pragma unroll
-    for (int step = 0; step < 8; ++step)
+        for (int step = 0; step < 8; ++step)
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
+            for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
-                acc[mt][nt] = mfma16(xa[step][mt], gb[step][nt], acc[mt][nt]);
+                for (int nt = 0; nt < 2; ++nt)
+                    acc[mt][nt] = mfma16(xa[step][mt], gb[step][nt], acc[mt][nt]);
+    }
     // lane holds dW'[o = 16 nt + n][k = 64 w + 16 mt + 4 s + i], i = 0..3
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt)
@@ -509,7 +567,7 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, 
     {
         const int r     = wave * 8 + j;
         const int slot  = j % PF;
-        const int64_t e = (int64_t) (o_blk + r) * K + k_blk + 4 * lane;
+        const int64_t e = (int64_t) (o_blk + r) * K + k_lane;
         const v4f f4 = fv[slot], a4 = av[slot], m4 = mv[slot], v4 = vv[slot];
         if (j + PF < 8)
         {
@@ -529,15 +587,18 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, 
         {
             float rr;
             const float gi = alpha_grad_f(f4[i], gw[i], as[i], d, off, g.clip_min, g.clip_max, a, tab, rr);
-            reg += rr;
+            reg += live ? rr : 0.f;
             adam_update(gi, as[i], ms[i], vs[i], a);
             gr[i] = gi;
         }
-        *reinterpret_cast<v4f*>(alpha + e) = (v4f) {as[0], as[1], as[2], as[3]};
-        *reinterpret_cast<v4f*>(m + e)     = (v4f) {ms[0], ms[1], ms[2], ms[3]};
-        *reinterpret_cast<v4f*>(v + e)     = (v4f) {vs[0], vs[1], vs[2], vs[3]};
-        if (grad_out)
-            *reinterpret_cast<v4f*>(grad_out + e) = gr;
+        if (live)
+        {
+            *reinterpret_cast<v4f*>(alpha + e) = (v4f) {as[0], as[1], as[2], as[3]};
+            *reinterpret_cast<v4f*>(m + e)     = (v4f) {ms[0], ms[1], ms[2], ms[3]};
+            *reinterpret_cast<v4f*>(v + e)     = (v4f) {vs[0], vs[1], vs[2], vs[3]};
+            if (grad_out)
+                *reinterpret_cast<v4f*>(grad_out + e) = gr;
+        }
     }
     if (reg_partial)
     {
@@ -547,13 +608,22 @@ __global__ __launch_bounds__(256) void lin_bwd_kernel(const FT* __restrict__ F, 
     }
 }
 
+// 1, 2, 4 or 8 blocks of 32 rows; 0 for a batch the fused path does not take
+int row_blocks_of(int64_t batch)
+{
+    for (int r = 1; r <= kMaxRowBlocks; r *= 2)
+        if (batch == (int64_t) r * kBatch)
+            return r;
+    return 0;
+}
+
 int make_lin_geom(LinGeom& g, int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
                   const float* offset, float clip_min, float clip_max)
 {
     MIQ_CHECK_ARG(out_features > 0 && in_features > 0, "bad layer shape");
-    MIQ_CHECK_ARG(out_features % kTileO == 0 && in_features % kTileK == 0,
+    MIQ_CHECK_ARG(out_features % kTileO == 0 && in_features % kFwdTileK == 0,
                   "the fused Linear path takes out_features that are a multiple of 32 and in_features that are a "
-                  "multiple of 256 (got %lld x %lld)", (long long) out_features, (long long) in_features);
+                  "multiple of 128 (got %lld x %lld)", (long long) out_features, (long long) in_features);
     MIQ_CHECK_ARG(out_features * in_features < (1ll << 31), "layer too large for the fused Linear path");
     MIQ_CHECK_ARG(num_channel == 1 || num_channel == out_features,
                   "delta/offset must have one entry, or one per output channel");
@@ -584,9 +654,18 @@ static int fwd_tiles_per_group(int64_t out_features, int64_t in_features)
     return (int) (per_group > along ? along : per_group);
 }
 
+template <typename FT, int R>
+static void launch_lin_fwd(dim3 grid, hipStream_t s, const FT* weight_floor, const float* alpha, const float* x,
+                           const int32_t* row_index, int num_rows, int64_t x_row_stride, float* workspace,
+                           const LinGeom& g, int tiles_per_group)
+{
+    hipLaunchKernelGGL((lin_fwd_kernel<FT, kFwdTileK, R>), grid, dim3(512), 0, s, weight_floor, alpha, x, row_index,
+                       num_rows, x_row_stride, workspace, g, tiles_per_group);
+}
+
 template <typename FT>
 static int linear_fwd(const FT* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
-                      int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+                      int64_t batch, int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
                       int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
                       const float* offset, float clip_min, float clip_max, int activation, float* workspace, float* out,
                       float* grad_out, float* loss_partial, void* stream)
@@ -599,17 +678,26 @@ static int linear_fwd(const FT* weight_floor, const float* alpha, const float* x
                   "weight_floor, alpha and the rows of x must be 16-byte aligned");
     MIQ_CHECK_ARG(x_row_stride >= in_features && target_row_stride >= out_features, "row stride shorter than a row");
     MIQ_CHECK_ARG(activation == 0 || activation == 1, "activation must be 0 (none) or 1 (ReLU)");
-    MIQ_CHECK_ARG(num_rows >= 1 && num_rows < (1ll << 31) && (row_index || num_rows >= kBatch),
-                  "num_rows (%lld) must be positive, and at least 32 without a row index", (long long) num_rows);
+    const int row_blocks = row_blocks_of(batch);
+    MIQ_CHECK_ARG(row_blocks != 0, "the fused Linear path takes 32, 64, 128 or 256 rows per iteration (got %lld)",
+                  (long long) batch);
+    MIQ_CHECK_ARG(num_rows >= 1 && num_rows < (1ll << 31) && (row_index || num_rows >= batch),
+                  "num_rows (%lld) must be positive, and at least the batch without a row index", (long long) num_rows);
     const int tiles_per_group = fwd_tiles_per_group(out_features, in_features);
     const int splits          = (int) ((in_features / kFwdTileK + tiles_per_group - 1) / tiles_per_group);
-    hipLaunchKernelGGL((lin_fwd_kernel<FT, kFwdTileK>),
-                       dim3((unsigned) splits, (unsigned) (out_features / kTileO)), dim3(512), 0, (hipStream_t) stream,
-                       weight_floor, alpha, x, row_index, (int) num_rows, x_row_stride, workspace, g, tiles_per_group);
+    const dim3 grid((unsigned) splits, (unsigned) (out_features / kTileO));
+    hipStream_t s = (hipStream_t) stream;
+    switch (row_blocks)
+    {
+    case 1: launch_lin_fwd<FT, 1>(grid, s, weight_floor, alpha, x, row_index, (int) num_rows, x_row_stride, workspace, g, tiles_per_group); break;
+    case 2: launch_lin_fwd<FT, 2>(grid, s, weight_floor, alpha, x, row_index, (int) num_rows, x_row_stride, workspace, g, tiles_per_group); break;
+    case 4: launch_lin_fwd<FT, 4>(grid, s, weight_floor, alpha, x, row_index, (int) num_rows, x_row_stride, workspace, g, tiles_per_group); break;
+    default: launch_lin_fwd<FT, 8>(grid, s, weight_floor, alpha, x, row_index, (int) num_rows, x_row_stride, workspace, g, tiles_per_group); break;
+    }
     MIQ_CHECK_LAUNCH();
-    const unsigned blocks = (unsigned) ((kBatch * out_features + 255) / 256);
-    hipLaunchKernelGGL(lin_loss_kernel, dim3(blocks), dim3(256), 0, (hipStream_t) stream, workspace, splits, bias, target,
-                       row_index, (int) num_rows, target_row_stride, (int) out_features, activation, out, grad_out,
+    const unsigned blocks = (unsigned) ((batch * out_features + 255) / 256);
+    hipLaunchKernelGGL(lin_loss_kernel, dim3(blocks), dim3(256), 0, s, workspace, splits, bias, target, row_index,
+                       (int) num_rows, target_row_stride, (int) out_features, (int) batch, activation, out, grad_out,
                        loss_partial);
     MIQ_CHECK_LAUNCH();
     return MIQ_OK;
@@ -617,7 +705,7 @@ static int linear_fwd(const FT* weight_floor, const float* alpha, const float* x
 
 template <typename FT>
 static int linear_bwd_adam(const FT* weight_floor, const float* grad_out, const float* x, const int32_t* row_index,
-                           int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg, float* exp_avg_sq, float* grad_alpha,
+                           int64_t batch, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg, float* exp_avg_sq, float* grad_alpha,
                            int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
                            const float* offset, float clip_min, float clip_max, double reg_param, double beta, double lr,
                            double beta1, double beta2, double eps, int step, float* reg_partial, void* stream)
@@ -630,105 +718,117 @@ static int linear_bwd_adam(const FT* weight_floor, const float* grad_out, const 
                       aligned16(grad_alpha),
                   "tensors must be 16-byte aligned");
     MIQ_CHECK_ARG(x_row_stride >= in_features, "row stride shorter than a row");
-    MIQ_CHECK_ARG(num_rows >= 1 && num_rows < (1ll << 31) && (row_index || num_rows >= kBatch),
-                  "num_rows (%lld) must be positive, and at least 32 without a row index", (long long) num_rows);
+    const int row_blocks = row_blocks_of(batch);
+    MIQ_CHECK_ARG(row_blocks != 0, "the fused Linear path takes 32, 64, 128 or 256 rows per iteration (got %lld)",
+                  (long long) batch);
+    MIQ_CHECK_ARG(num_rows >= 1 && num_rows < (1ll << 31) && (row_index || num_rows >= batch),
+                  "num_rows (%lld) must be positive, and at least the batch without a row index", (long long) num_rows);
     MIQ_CHECK_ARG(step >= 1, "Adam step count starts at 1");
     AdamArgs a;
     if (int rc = make_adam(a, reg_param, beta, lr, beta1, beta2, eps, step))
         return rc;
     // two rows of the epilogue in flight per lane: deeper prefetch (3, 4) costs registers and measured no faster
-    hipLaunchKernelGGL((lin_bwd_kernel<2, FT>), dim3((unsigned) (in_features / kTileK), (unsigned) (out_features / kTileO)),
-                       dim3(256), 0, (hipStream_t) stream, weight_floor, grad_out, x, row_index, (int) num_rows, x_row_stride, alpha,
-                       exp_avg, exp_avg_sq, grad_alpha, g, a, reg_partial);
+    const dim3 grid((unsigned) ((in_features + kTileK - 1) / kTileK), (unsigned) (out_features / kTileO));
+    if (row_blocks == 1)
+        hipLaunchKernelGGL((lin_bwd_kernel<2, FT, false>), grid, dim3(256), 0, (hipStream_t) stream, weight_floor, grad_out,
+                           x, row_index, (int) num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq, grad_alpha, g, a,
+                           reg_partial, 1);
+    else
+        hipLaunchKernelGGL((lin_bwd_kernel<2, FT, true>), grid, dim3(256), 0, (hipStream_t) stream, weight_floor, grad_out,
+                           x, row_index, (int) num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq, grad_alpha, g, a,
+                           reg_partial, row_blocks);
     MIQ_CHECK_LAUNCH();
     return MIQ_OK;
 }
 
 extern "C" {
 
-int64_t miq_adaround_linear_workspace_bytes(int64_t out_features, int64_t in_features)
+int64_t miq_adaround_linear_workspace_bytes(int64_t out_features, int64_t in_features, int64_t batch)
 {
     if (out_features <= 0 || in_features <= 0)
         return 0;
-    if (out_features % kTileO != 0 || in_features % kTileK != 0)
+    if (out_features % kTileO != 0 || in_features % kFwdTileK != 0 || row_blocks_of(batch) == 0)
         return 0;   // not a shape the fused path takes
     const int64_t along  = in_features / kFwdTileK;
     const int64_t per    = fwd_tiles_per_group(out_features, in_features);
     const int64_t splits = (along + per - 1) / per;
-    return splits * kBatch * out_features * (int64_t) sizeof(float);
+    return splits * batch * out_features * (int64_t) sizeof(float);
 }
 
 int miq_adaround_linear_blocks(int64_t out_features, int64_t in_features)
 {
-    return (int) ((out_features / kTileO) * (in_features / kTileK));
+    return (int) ((out_features / kTileO) * ((in_features + kTileK - 1) / kTileK));
 }
 
-int miq_adaround_linear_fwd_f32(const float* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
-                                int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride,
+int miq_adaround_linear_fwd_f32(const float* weight_floor, const float* alpha, const float* x, const int32_t* row_index, int64_t batch,
+        int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride,
                                 const float* bias, int64_t out_features, int64_t in_features, int64_t num_channel,
                                 const float* delta, const float* offset, float clip_min, float clip_max,
                                 int activation, float* workspace, float* out, float* grad_out, float* loss_partial,
                                 void* stream)
 {
-    return linear_fwd<float>(weight_floor, alpha, x, row_index, num_rows, x_row_stride, target, target_row_stride, bias,
+    return linear_fwd<float>(weight_floor, alpha, x, row_index, batch, num_rows, x_row_stride, target, target_row_stride, bias,
                              out_features, in_features, num_channel, delta, offset, clip_min, clip_max, activation,
                              workspace, out, grad_out, loss_partial, stream);
 }
 
-int miq_adaround_linear_fwd_i8(const int8_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
-                               int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+int miq_adaround_linear_fwd_i8(const int8_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index, int64_t batch,
+        int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
                                int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
                                const float* offset, float clip_min, float clip_max, int activation, float* workspace,
                                float* out, float* grad_out, float* loss_partial, void* stream)
 {
-    return linear_fwd<int8_t>(weight_floor, alpha, x, row_index, num_rows, x_row_stride, target, target_row_stride, bias,
+    return linear_fwd<int8_t>(weight_floor, alpha, x, row_index, batch, num_rows, x_row_stride, target, target_row_stride, bias,
                               out_features, in_features, num_channel, delta, offset, clip_min, clip_max, activation,
                               workspace, out, grad_out, loss_partial, stream);
 }
 
 int miq_adaround_linear_bwd_adam_f32(const float* weight_floor, const float* grad_out, const float* x,
-                                     const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                     const int32_t* row_index, int64_t batch,
+        int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                      float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                      int64_t num_channel, const float* delta, const float* offset, float clip_min,
                                      float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
                                      double eps, int step, float* reg_partial, void* stream)
 {
-    return linear_bwd_adam<float>(weight_floor, grad_out, x, row_index, num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq,
+    return linear_bwd_adam<float>(weight_floor, grad_out, x, row_index, batch, num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq,
                                   grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min, clip_max,
                                   reg_param, beta, lr, beta1, beta2, eps, step, reg_partial, stream);
 }
 
 int miq_adaround_linear_bwd_adam_i8(const int8_t* weight_floor, const float* grad_out, const float* x,
-                                    const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                    const int32_t* row_index, int64_t batch,
+        int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                     float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                     int64_t num_channel, const float* delta, const float* offset, float clip_min,
                                     float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
                                     double eps, int step, float* reg_partial, void* stream)
 {
-    return linear_bwd_adam<int8_t>(weight_floor, grad_out, x, row_index, num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq,
+    return linear_bwd_adam<int8_t>(weight_floor, grad_out, x, row_index, batch, num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq,
                                    grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min,
                                    clip_max, reg_param, beta, lr, beta1, beta2, eps, step, reg_partial, stream);
 }
 
-int miq_adaround_linear_fwd_i16(const int16_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
-                               int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+int miq_adaround_linear_fwd_i16(const int16_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index, int64_t batch,
+        int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
                                int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
                                const float* offset, float clip_min, float clip_max, int activation, float* workspace,
                                float* out, float* grad_out, float* loss_partial, void* stream)
 {
-    return linear_fwd<int16_t>(weight_floor, alpha, x, row_index, num_rows, x_row_stride, target, target_row_stride, bias,
+    return linear_fwd<int16_t>(weight_floor, alpha, x, row_index, batch, num_rows, x_row_stride, target, target_row_stride, bias,
                               out_features, in_features, num_channel, delta, offset, clip_min, clip_max, activation,
                               workspace, out, grad_out, loss_partial, stream);
 }
 
 int miq_adaround_linear_bwd_adam_i16(const int16_t* weight_floor, const float* grad_out, const float* x,
-                                    const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                    const int32_t* row_index, int64_t batch,
+        int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                     float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                     int64_t num_channel, const float* delta, const float* offset, float clip_min,
                                     float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
                                     double eps, int step, float* reg_partial, void* stream)
 {
-    return linear_bwd_adam<int16_t>(weight_floor, grad_out, x, row_index, num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq,
+    return linear_bwd_adam<int16_t>(weight_floor, grad_out, x, row_index, batch, num_rows, x_row_stride, alpha, exp_avg, exp_avg_sq,
                                    grad_alpha, out_features, in_features, num_channel, delta, offset, clip_min,
                                    clip_max, reg_param, beta, lr, beta1, beta2, eps, step, reg_partial, stream);
 }

@@ -709,12 +709,12 @@ def adaround_bwd_adam(weight, grad_weight, alpha, exp_avg, exp_avg_sq, num_chann
 
 def adaround_linear_supported(out_features, in_features, batch):
     """Shapes the MFMA-fused Linear path takes."""
-    return batch == 32 and out_features % 32 == 0 and in_features % 256 == 0 and \
+    return batch in (32, 64, 128, 256) and out_features % 32 == 0 and in_features % 128 == 0 and \
         out_features * in_features < 2 ** 31
 
 
-def adaround_linear_workspace(out_features, in_features, device):
-    nbytes = int(lib.miq_adaround_linear_workspace_bytes(int(out_features), int(in_features)))
+def adaround_linear_workspace(out_features, in_features, device, batch=32):
+    nbytes = int(lib.miq_adaround_linear_workspace_bytes(int(out_features), int(in_features), int(batch)))
     return torch.empty(nbytes // 4, dtype=_F32, device=device)
 
 
@@ -731,19 +731,34 @@ def _floor_variant(weight_floor, alpha, prefix):
     return getattr(lib, prefix + suffix)
 
 
+def _ada_batch(grad_out, out_features, row_index):
+    """Rows per iteration of the fused Linear path: grad_out is [batch, out_features]."""
+    if grad_out.dim() != 2 or grad_out.size(1) != out_features:
+        raise RuntimeError("grad_out must be [batch, out_features]")
+    batch = grad_out.size(0)
+    if row_index is not None and (row_index.dtype != torch.int32 or row_index.numel() != batch or
+                                  not row_index.is_contiguous()):
+        raise RuntimeError(f"row_index must hold {batch} int32 row numbers")
+    return batch
+
+
 def adaround_linear_fwd(weight_floor, alpha, x, row_index, target, bias, num_channel, delta, offset, clip_min, clip_max,
                         activation, workspace, grad_out, out=None, loss_partial=None):
-    """Fused apply_adaround + Linear forward + reconstruction-loss gradient for 32 rows of x / target."""
+    """Fused apply_adaround + Linear forward + reconstruction-loss gradient for the rows of x / target that row_index
+    names: as many as grad_out has rows (32, 64, 128 or 256)."""
     _ada_check(alpha, workspace, grad_out, out)
     fn = _floor_variant(weight_floor, alpha, "miq_adaround_linear_fwd_")
     _require_gpu(weight_floor, x, target, bias, row_index)
     if x.dtype != _F32 or target.dtype != _F32 or x.stride(-1) != 1 or target.stride(-1) != 1:
         raise RuntimeError("x and target must be float32 with contiguous rows")
-    if row_index is not None and (row_index.dtype != torch.int32 or row_index.numel() != 32):
-        raise RuntimeError("row_index must hold 32 int32 row numbers")
     o, k = weight_floor.shape
+    batch = _ada_batch(grad_out, o, row_index)
+    if workspace.numel() * 4 < lib.miq_adaround_linear_workspace_bytes(o, k, batch) or \
+            (out is not None and out.numel() < batch * o):
+        raise RuntimeError("workspace or out is too small for this batch")
     with _OnDevice(weight_floor.device):
-        check(fn(_ptr(weight_floor), _ptr(alpha), _ptr(x), _ptr(row_index), min(x.size(0), target.size(0)), x.stride(0),
+        check(fn(_ptr(weight_floor), _ptr(alpha), _ptr(x), _ptr(row_index), batch, min(x.size(0), target.size(0)),
+                 x.stride(0),
                  _ptr(target), target.stride(0),
                  _ptr(bias), o, k, int(num_channel), _ptr(delta), _ptr(offset), float(clip_min), float(clip_max),
                  int(activation), _ptr(workspace), _ptr(out), _ptr(grad_out), _ptr(loss_partial), _stream(weight_floor)))
@@ -757,8 +772,11 @@ def adaround_linear_bwd_adam(weight_floor, grad_out, x, row_index, alpha, exp_av
     fn = _floor_variant(weight_floor, alpha, "miq_adaround_linear_bwd_adam_")
     _require_gpu(weight_floor, x, row_index)
     o, k = weight_floor.shape
+    batch = _ada_batch(grad_out, o, row_index)
+    if x.dtype != _F32 or x.stride(-1) != 1:
+        raise RuntimeError("x must be float32 with contiguous rows")
     with _OnDevice(weight_floor.device):
-        check(fn(_ptr(weight_floor), _ptr(grad_out), _ptr(x), _ptr(row_index), x.size(0), x.stride(0), _ptr(alpha),
+        check(fn(_ptr(weight_floor), _ptr(grad_out), _ptr(x), _ptr(row_index), batch, x.size(0), x.stride(0), _ptr(alpha),
                  _ptr(exp_avg),
                  _ptr(exp_avg_sq), _ptr(grad_alpha), o, k, int(num_channel), _ptr(delta), _ptr(offset), float(clip_min),
                  float(clip_max), float(reg_param), float(beta), float(lr), float(beta1), float(beta2), float(eps),

@@ -26,8 +26,9 @@ ADAM_LR, ADAM_BETAS, ADAM_EPS = 1e-3, (0.9, 0.999), 1e-8      # torch.optim.Adam
 class AdaroundOptimizer:
     """Optimizes the weight rounding of a quantized wrapper module."""
 
-    # Linear layers whose shape the MFMA-fused kernels take (out % 32 == 0, in % 256 == 0, batch 32, no activation or
-    # ReLU) use them; everything else runs soft-round kernel + torch layer + fused backward/Adam kernel
+    # Linear layers and 1x1 convolutions whose shape the MFMA-fused kernels take (out % 32 == 0, in % 128 == 0,
+    # 32 / 64 / 128 / 256 rows per iteration, no activation or ReLU) use them; everything else runs soft-round kernel +
+    # torch layer + fused backward/Adam kernel
     use_fused_linear = True
     use_int8_floor = True    # store floor(W / delta) as int8 / int16 for the fused Linear path when the grid allows it
 
@@ -91,36 +92,45 @@ class AdaroundOptimizer:
 
         activation = cls._fused_activation_code(act_func)
         module = qm.get_original_module()
-        if cls.use_fused_linear and activation is not None and \
-                cls._fused_linear_applies(module, weight, qm, all_inp_data, all_orig_out_data, batches):
+        rows = cls._fused_rows(module, weight, qm, all_inp_data, all_orig_out_data, batches) \
+            if cls.use_fused_linear and activation is not None else None
+        if rows is not None:
             # soft rounding fused into the MFMA GEMMs: three launches per iteration, nothing weight-shaped is
             # written except alpha and the Adam moments
+            x_rows, y_rows, pixels = rows
+            out_features, in_features = weight.shape[:2]
+            as_matrix = lambda t: t.view(out_features, in_features)     # a 1x1 kernel is the same memory
+            weight2, alpha2 = as_matrix(weight), as_matrix(alpha)
             # floor(W / delta) never changes during the optimisation: int8 where the grid allows it (up to 7 bits; a
             # quarter of the bytes), else int16, else float32 -- identical results in every form
-            weight_floor = ops.adaround_floor_packed(weight, qm.num_channel, qm.n_per_channel, qm.delta, qm.offset,
+            weight_floor = ops.adaround_floor_packed(weight2, qm.num_channel, qm.n_per_channel, qm.delta, qm.offset,
                                                      qm.clip_min, qm.clip_max) if cls.use_int8_floor else None
             if weight_floor is None:
-                weight_floor = ops.adaround_floor(weight, qm.num_channel, qm.n_per_channel, qm.delta)
+                weight_floor = ops.adaround_floor(weight2, qm.num_channel, qm.n_per_channel, qm.delta)
             index = torch.stack(batches)
             # the kernels gather rows by these numbers; the reference's all_inp_data[indices] raises on a bad one
-            num_rows = min(all_inp_data.size(0), all_orig_out_data.size(0))
-            if index.numel() and (int(index.min()) < -num_rows or int(index.max()) >= num_rows):
-                raise IndexError(f"batch index out of range for {num_rows} cached rows")
-            index = torch.where(index < 0, index + num_rows, index)      # negative numbers count from the end
+            num_samples = min(all_inp_data.size(0), all_orig_out_data.size(0))
+            if index.numel() and (int(index.min()) < -num_samples or int(index.max()) >= num_samples):
+                raise IndexError(f"batch index out of range for {num_samples} cached rows")
+            index = torch.where(index < 0, index + num_samples, index)      # negative numbers count from the end
+            if pixels > 1:
+                # sample b owns rows b * pixels .. b * pixels + pixels - 1 of the channels-last copies
+                index = (index.unsqueeze(-1) * pixels + torch.arange(pixels)).flatten(1)
             index = index.to(dtype=torch.int32, device=device).contiguous()
+            batch_rows = index.size(1)
             bias = None if module.bias is None else module.bias.detach().to(torch.float32).contiguous()
-            out_features, in_features = weight.shape
-            workspace = ops.adaround_linear_workspace(out_features, in_features, device)
-            grad_out = torch.empty(BATCH_SIZE, out_features, dtype=torch.float32, device=device)
+            workspace = ops.adaround_linear_workspace(out_features, in_features, device, batch_rows)
+            grad_out = torch.empty(batch_rows, out_features, dtype=torch.float32, device=device)
+            moments = as_matrix(exp_avg), as_matrix(exp_avg_sq)
             for k in range(len(batches)):
-                ops.adaround_linear_fwd(weight_floor, alpha, all_inp_data, index[k], all_orig_out_data, bias,
+                ops.adaround_linear_fwd(weight_floor, alpha2, x_rows, index[k], y_rows, bias,
                                         qm.num_channel, qm.delta, qm.offset, qm.clip_min, qm.clip_max, activation,
                                         workspace, grad_out)
-                ops.adaround_linear_bwd_adam(weight_floor, grad_out, all_inp_data, index[k], alpha, exp_avg, exp_avg_sq,
+                ops.adaround_linear_bwd_adam(weight_floor, grad_out, x_rows, index[k], alpha2, *moments,
                                              qm.num_channel, qm.delta, qm.offset, qm.clip_min, qm.clip_max,
                                              opt_params.reg_param, beta_of(first_iteration + k), ADAM_LR,
                                              ADAM_BETAS[0], ADAM_BETAS[1], ADAM_EPS, k + 1,
-                                             grad_alpha=grad_alpha if k == len(batches) - 1 else None)
+                                             grad_alpha=as_matrix(grad_alpha) if k == len(batches) - 1 else None)
             qm.alpha.grad = grad_alpha
             return exp_avg, exp_avg_sq
 
@@ -156,15 +166,44 @@ class AdaroundOptimizer:
         return None
 
     @staticmethod
-    def _fused_linear_applies(module, weight, qm, all_inp_data, all_orig_out_data, batches) -> bool:
-        if not isinstance(module, torch.nn.Linear) or weight.dim() != 2:
-            return False
-        out_features, in_features = weight.shape
+    def _fused_rows(module, weight, qm, all_inp_data, all_orig_out_data, batches):
+        """(x rows, target rows, rows per sample) when the MFMA-fused kernels take this layer, else None.
+
+        They take a Linear layer on 2-D activations, and a Conv2d with a 1x1 kernel, unit stride, no padding and one
+        group, which is the same contraction over the channels for every pixel (the reference calls functional.conv2d
+        there, :268-272): its rows are the pixels, read from channels-last copies of the cached activations that are
+        made once per layer.  The rows of an iteration -- batch entries times pixels -- must be 32, 64, 128 or 256."""
+        if not batches or any(b.numel() != batches[0].numel() for b in batches):
+            return None
+        out_features, in_features = weight.shape[:2]
         per_channel_ok = qm.num_channel == 1 or (qm.num_channel == out_features and qm.n_per_channel == in_features)
-        data_ok = all(t.dim() == 2 and t.dtype == torch.float32 and t.stride(1) == 1 and t.stride(0) % 4 == 0 and
-                      t.data_ptr() % 16 == 0 for t in (all_inp_data, all_orig_out_data))
-        return per_channel_ok and data_ok and all(b.numel() == BATCH_SIZE for b in batches) and \
-            ops.adaround_linear_supported(out_features, in_features, BATCH_SIZE)
+        if not per_channel_ok or all_inp_data.dtype != torch.float32 or all_orig_out_data.dtype != torch.float32:
+            return None
+        if isinstance(module, torch.nn.Linear) and weight.dim() == 2:
+            pixels = 1
+            if all_inp_data.dim() != 2 or all_orig_out_data.dim() != 2:
+                return None
+            x_rows, y_rows = all_inp_data, all_orig_out_data
+        elif isinstance(module, torch.nn.Conv2d) and weight.dim() == 4:
+            one, zero = (1, 1), (0, 0)
+            if tuple(weight.shape[2:]) != one or tuple(module.stride) != one or tuple(module.dilation) != one or \
+                    module.groups != 1 or module.padding not in (zero, 0, 'valid') or \
+                    all_inp_data.dim() != 4 or all_orig_out_data.dim() != 4 or \
+                    all_inp_data.shape[2:] != all_orig_out_data.shape[2:]:
+                return None
+            pixels = all_inp_data.shape[2] * all_inp_data.shape[3]
+            if not ops.adaround_linear_supported(out_features, in_features, batches[0].numel() * pixels):
+                return None             # before anything is copied
+            x_rows = all_inp_data.permute(0, 2, 3, 1).reshape(-1, in_features).contiguous()
+            y_rows = all_orig_out_data.permute(0, 2, 3, 1).reshape(-1, out_features).contiguous()
+        else:
+            return None
+        if x_rows.size(1) != in_features or y_rows.size(1) != out_features:
+            return None
+        data_ok = all(t.stride(1) == 1 and t.stride(0) % 4 == 0 and t.data_ptr() % 16 == 0 for t in (x_rows, y_rows))
+        if data_ok and ops.adaround_linear_supported(out_features, in_features, batches[0].numel() * pixels):
+            return x_rows, y_rows, pixels
+        return None
 
     @classmethod
     def _compute_recons_metrics(cls, quant_module: AdaroundWrapper, act_func, inp_data: torch.Tensor,

@@ -475,6 +475,48 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
         "bwd_GBps_on_float32_formulation": 28 * n / b / 1e6,
         "bwd_mfma_TFLOPs": 2.0 * 32 * n / b / 1e9}
 
+    # the same layer with 64, 128 and 256 rows per iteration (2, 4, 8 blocks of 32 through the same kernels: the
+    # weight-shaped traffic stays, the MFMA work and the activation reads grow with the rows), each against the general
+    # path (soft-rounding kernel, torch GEMMs, fused backward kernel) on the same batches
+    per_rows = []
+    for rows_it in (32, 64, 128, 256):
+        gout_r = torch.empty(rows_it, o, device=w.device)
+        ws_r = ops.adaround_linear_workspace(o, k, w.device, rows_it)
+        torch.manual_seed(1005 + rows_it)
+        idx_r = torch.stack([torch.randperm(x.size(0))[:rows_it] for _ in range(timed_kernel_iters)])
+        idx_dev = idx_r.to(torch.int32).to(w.device)
+
+        def fwd_r(i):
+            ops.adaround_linear_fwd(w, alpha, x, idx_dev[i], y, None, wrapper.num_channel, wrapper.delta, wrapper.offset,
+                                    wrapper.clip_min, wrapper.clip_max, 0, ws_r, gout_r)
+
+        def bwd_r(i):
+            ops.adaround_linear_bwd_adam(w, gout_r, x, idx_dev[i], alpha, m, v, wrapper.num_channel, wrapper.delta,
+                                         wrapper.offset, wrapper.clip_min, wrapper.clip_max, 0.01, 10.0, 1e-3, 0.9,
+                                         0.999, 1e-8, i + 1)
+
+        f_r, b_r = region(fwd_r), region(bwd_r)
+        loops = {}
+        n_it = min(200, iterations)
+        for name, fused in (("fused", True), ("general", False)):
+            AdaroundOptimizer.use_fused_linear = fused
+            alpha0 = wrapper.alpha.data.clone()
+            bl = [idx_r[i % timed_kernel_iters] for i in range(n_it)]
+            AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, x, y, params, batches=bl[:10])
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, x, y, params, batches=bl)
+            torch.cuda.synchronize()
+            loops[name] = (time.perf_counter() - t0) * 1e3 / n_it
+            wrapper.alpha.data.copy_(alpha0)
+        AdaroundOptimizer.use_fused_linear = True
+        per_rows.append({"rows": rows_it, "fwd_ms": f_r, "bwd_ms": b_r,
+                         "fwd_GBps_moved": (fb + 4) * n / f_r / 1e6, "bwd_GBps_moved": (fb + 24) * n / b_r / 1e6,
+                         "fwd_mfma_TFLOPs": 2.0 * rows_it * n / f_r / 1e9, "bwd_mfma_TFLOPs": 2.0 * rows_it * n / b_r / 1e9,
+                         "loop_ms_per_iteration_fused": loops["fused"],
+                         "loop_ms_per_iteration_general": loops["general"]})
+    res["rows_per_iteration"] = per_rows
+
     # the GEMM-bound variant: every iteration uses all 2048 cached rows.  The fused kernels are built for the
     # reference's batch of 32 (the weight-shaped traffic dominates there); a batch of 2048 goes through the general
     # path: soft-rounding kernel, torch's GEMMs (hipBLASLt) for the layer and its weight gradient, fused
@@ -502,7 +544,7 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
     flops = 2 * 2.0 * rows * o * k
     res["batch_2048_gemm_bound"] = {
         "path": "soft-round kernel + torch GEMMs (hipBLASLt) + fused backward/Adam kernel; the MFMA-fused kernels "
-                "take batches of 32 only",
+                "take up to 256 rows",
         "ms_per_iteration": it_ms, "gflop_per_iteration": flops / 1e9,
         "iteration_TFLOPs": flops / it_ms / 1e9,
         "gemms_alone_ms": g_ms, "gemms_alone_TFLOPs": flops / g_ms / 1e9,

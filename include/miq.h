@@ -485,17 +485,19 @@ int miq_adaround_eval_terms_f32(const float* in, float* out, int64_t num_element
 /* ---------------------------------------------------------------------------------------------------------------
  * AdaRound iteration of a Linear layer, soft rounding fused into MFMA GEMMs (the adarounded weight and its gradient
  * never exist in memory).  One iteration of AdaroundOptimizer._optimize_rounding (ADA/adaround_optimizer.py:182-218)
- * for torch.nn.Linear with a batch of exactly 32 rows (BATCH_SIZE, ADA/adaround_optimizer.py:58):
+ * for torch.nn.Linear with a batch of 32 rows (BATCH_SIZE, ADA/adaround_optimizer.py:58), or of 64, 128 or 256 rows
+ * (a caller with another batch size; a 1x1 Conv2d over 2, 4 or 8 pixels, whose rows are the pixels of the 32 images
+ * in channels-last order: ADA/adaround_optimizer.py:268-272 runs the same contraction as functional.conv2d):
  *   fwd:  out = linear(x[rows], apply_adaround(W), bias);  grad_out = d recon_loss(act(out), act(target[rows])) / d out
  *   bwd:  dLoss/dW' = grad_out^T x[rows]  ->  alpha gradient + regulariser + Adam, as miq_adaround_bwd_adam_f32
  * weight_floor (= floor(W / delta), from miq_adaround_floor_f32), alpha, moments: [out_features, in_features] float32
  * row-major.  x: rows of in_features floats, row r at
- * x + r * x_row_stride; target likewise with out_features floats.  row_index: device int32[32] choosing the rows of x
- * and target (NULL = rows 0..31); num_rows: the number of rows x and target hold.  An index outside [0, num_rows) never
+ * x + r * x_row_stride; target likewise with out_features floats.  batch: 32, 64, 128 or 256.  row_index: device
+ * int32[batch] choosing the rows of x and target (NULL = rows 0..batch-1); num_rows: the number of rows x and target hold.  An index outside [0, num_rows) never
  * leaves the buffers: that row reads row 0 or num_rows - 1 and its grad_out / out entries are NaN, which the backward
  * spreads over alpha (the reference's indexing raises IndexError there; aimet_amd checks the indices on the host
  * before the first launch).  num_channel: 1 (per-tensor delta/offset) or out_features (per output channel).
- * Shapes: out_features % 32 == 0, in_features % 256 == 0, out_features * in_features < 2^31; other shapes return
+ * Shapes: out_features % 32 == 0, in_features % 128 == 0, out_features * in_features < 2^31; other shapes return
  * MIQ_ERR_INVALID_ARG and the caller uses the elementwise entry points around its own GEMM.
  * activation: 0 none, 1 ReLU (the act_func the reference applies to both outputs, ADA/adaround_optimizer.py:192-194).
  * ------------------------------------------------------------------------------------------------------------- */
@@ -505,44 +507,48 @@ int miq_adaround_eval_terms_f32(const float* in, float* out, int64_t num_element
  * identical to the float32 form, element for element. */
 
 /* Bytes of device workspace the forward needs (partial products of the split K dimension). */
-int64_t miq_adaround_linear_workspace_bytes(int64_t out_features, int64_t in_features);
+int64_t miq_adaround_linear_workspace_bytes(int64_t out_features, int64_t in_features, int64_t batch);
 /* Number of regulariser partial sums miq_adaround_linear_bwd_adam_f32 writes. */
 int miq_adaround_linear_blocks(int64_t out_features, int64_t in_features);
-/* out (optional, may be NULL): device float[32 * out_features], the layer output before the activation.
- * grad_out: device float[32 * out_features] = 2 (act(out) - act(target)) act'(out) / 32, the gradient of
- * AdaroundLoss.compute_recon_loss (ADA/adaround_loss.py:70-80) w.r.t. out.
- * loss_partial (optional): device float[ceil(32 * out_features / 256)] partial sums of the reconstruction loss. */
-int miq_adaround_linear_fwd_f32(const float* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
-                                int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride,
+/* out (optional, may be NULL): device float[batch * out_features], the layer output before the activation.
+ * grad_out: device float[batch * out_features] = 2 (act(out) - act(target)) act'(out) / batch, the gradient of
+ * AdaroundLoss.compute_recon_loss (ADA/adaround_loss.py:70-80: squared error summed over dimension 1, mean over the
+ * rest, which for rows that are pixels is the same number) w.r.t. out.
+ * loss_partial (optional): device float[ceil(batch * out_features / 256)] partial sums of the reconstruction loss. */
+int miq_adaround_linear_fwd_f32(const float* weight_floor, const float* alpha, const float* x, const int32_t* row_index, int64_t batch,
+        int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride,
                                 const float* bias, int64_t out_features, int64_t in_features, int64_t num_channel,
                                 const float* delta, const float* offset, float clip_min, float clip_max,
                                 int activation, float* workspace, float* out, float* grad_out, float* loss_partial,
                                 void* stream);
 int miq_adaround_linear_bwd_adam_f32(const float* weight_floor, const float* grad_out, const float* x,
-                                     const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                     const int32_t* row_index, int64_t batch,
+        int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                      float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                      int64_t num_channel, const float* delta, const float* offset, float clip_min,
                                      float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
                                      double eps, int step, float* reg_partial, void* stream);
 
-int miq_adaround_linear_fwd_i8(const int8_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
-                               int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+int miq_adaround_linear_fwd_i8(const int8_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index, int64_t batch,
+        int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
                                int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
                                const float* offset, float clip_min, float clip_max, int activation, float* workspace,
                                float* out, float* grad_out, float* loss_partial, void* stream);
 int miq_adaround_linear_bwd_adam_i8(const int8_t* weight_floor, const float* grad_out, const float* x,
-                                    const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                    const int32_t* row_index, int64_t batch,
+        int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                     float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                     int64_t num_channel, const float* delta, const float* offset, float clip_min,
                                     float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,
                                     double eps, int step, float* reg_partial, void* stream);
-int miq_adaround_linear_fwd_i16(const int16_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index,
-                               int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
+int miq_adaround_linear_fwd_i16(const int16_t* weight_floor, const float* alpha, const float* x, const int32_t* row_index, int64_t batch,
+        int64_t num_rows, int64_t x_row_stride, const float* target, int64_t target_row_stride, const float* bias,
                                int64_t out_features, int64_t in_features, int64_t num_channel, const float* delta,
                                const float* offset, float clip_min, float clip_max, int activation, float* workspace,
                                float* out, float* grad_out, float* loss_partial, void* stream);
 int miq_adaround_linear_bwd_adam_i16(const int16_t* weight_floor, const float* grad_out, const float* x,
-                                    const int32_t* row_index, int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
+                                    const int32_t* row_index, int64_t batch,
+        int64_t num_rows, int64_t x_row_stride, float* alpha, float* exp_avg,
                                     float* exp_avg_sq, float* grad_alpha, int64_t out_features, int64_t in_features,
                                     int64_t num_channel, const float* delta, const float* offset, float clip_min,
                                     float clip_max, double reg_param, double beta, double lr, double beta1, double beta2,

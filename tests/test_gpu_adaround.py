@@ -283,8 +283,12 @@ def test_optimisation_trajectory(ops, kind, act):
     assert _close_except_few(v, v_ref, atol=1e-4 * v_ref.abs().max().item(), rtol=1e-3)
 
 
-@pytest.mark.parametrize("shape,per_channel,act", [((128, 512), True, 0), ((64, 256), False, 1), ((192, 768), True, 1)])
-def test_fused_linear_forward_and_backward(ops, shape, per_channel, act):
+@pytest.mark.parametrize("shape,per_channel,act,batch", [
+    ((128, 512), True, 0, 32), ((64, 256), False, 1, 32), ((192, 768), True, 1, 32),
+    # in_features that end in half a backward tile, and 2 / 4 / 8 blocks of 32 rows
+    ((64, 128), True, 0, 32), ((96, 384), False, 1, 32), ((64, 384), True, 1, 64), ((96, 128), False, 0, 128),
+    ((128, 640), True, 1, 256), ((64, 512), True, 0, 256), ((160, 256), False, 1, 128)])
+def test_fused_linear_forward_and_backward(ops, shape, per_channel, act, batch):
     """The MFMA-fused Linear kernels against the elementwise kernels around torch's own GEMM on the GPU (same
     per-element arithmetic, different summation order in the GEMMs) and against the CPU restatement."""
     O, K = shape
@@ -293,17 +297,17 @@ def test_fused_linear_forward_and_backward(ops, shape, per_channel, act):
     weight[2, 7] = -weight[2].abs().max() * 5.0
     weight[3, 9] = weight[3].abs().max() * 5.0
     torch.manual_seed(32)
-    X, bias = torch.randn(100, K), torch.randn(O) * 0.1
-    Y = torch.nn.functional.linear(X, weight, bias) + torch.randn(100, O) * 0.01
-    idx = torch.randperm(100)[:32]
+    X, bias = torch.randn(300, K), torch.randn(O) * 0.1
+    Y = torch.nn.functional.linear(X, weight, bias) + torch.randn(300, O) * 0.01
+    idx = torch.randperm(300)[:batch]
     d, o = ada.broadcast(delta, weight, 0), ada.broadcast(offset, weight, 0)
     alpha = ada.generate_alpha(weight, d) + torch.randn_like(weight)
     wg, ag, dg, og, Xg, Yg, bg = (t.cuda() for t in (weight, alpha, delta, offset, X, Y, bias))
     ig = idx.to(torch.int32).cuda()
-    ws = ops.adaround_linear_workspace(O, K, "cuda")
-    G = torch.empty(32, O, device="cuda")
-    out = torch.empty(32, O, device="cuda")
-    lp = torch.zeros((32 * O + 255) // 256, device="cuda")
+    ws = ops.adaround_linear_workspace(O, K, "cuda", batch)
+    G = torch.empty(batch, O, device="cuda")
+    out = torch.empty(batch, O, device="cuda")
+    lp = torch.zeros((batch * O + 255) // 256, device="cuda")
     fg = ops.adaround_floor(wg, C, npc, dg)
     assert torch.equal(fg.cpu(), torch.floor(weight / d))
     ops.adaround_linear_fwd(fg, ag, Xg, ig, Yg, bg, C, dg, og, cmin, cmax, act, ws, G, out=out, loss_partial=lp)
@@ -395,6 +399,13 @@ def test_fused_linear_rejects_other_shapes(ops):
                                 None, 1, torch.ones(1, device="cuda"), torch.zeros(1, device="cuda"), 0, 15, 0,
                                 torch.zeros(32 * 48, device="cuda"), torch.zeros(32, 48, device="cuda"))
     assert not ops.adaround_linear_supported(48, 256, 32)
+    assert not ops.adaround_linear_supported(64, 192, 32) and ops.adaround_linear_supported(64, 128, 32)
+    assert not ops.adaround_linear_supported(64, 256, 96) and ops.adaround_linear_supported(64, 256, 256)
+    w = torch.zeros(64, 256, device="cuda")
+    with pytest.raises(MiqError, match="32, 64, 128 or 256"):
+        ops.adaround_linear_fwd(w, w, torch.zeros(96, 256, device="cuda"), None, torch.zeros(96, 64, device="cuda"),
+                                None, 1, torch.ones(1, device="cuda"), torch.zeros(1, device="cuda"), 0, 15, 0,
+                                torch.zeros(96 * 64 * 8, device="cuda"), torch.zeros(96, 64, device="cuda"))
     # fewer than 32 cached rows and no row index: refused before any launch
     w = torch.zeros(64, 256, device="cuda")
     with pytest.raises(MiqError, match="num_rows"):
@@ -477,6 +488,74 @@ def test_fused_optimisation_trajectory(ops, act, per_channel, monkeypatch):
     assert _close_except_few(g, g_ref, atol=1e-4 * g_ref.abs().max().item(), rtol=1e-3)
     assert _close_except_few(m, m_ref, atol=1e-4 * m_ref.abs().max().item(), rtol=1e-3)
     assert _close_except_few(v, v_ref, atol=1e-4 * v_ref.abs().max().item(), rtol=1e-3)
+
+
+@pytest.mark.parametrize("kind,shape,pixels,batch,per_channel", [
+    ("conv2d", (64, 128, 1, 1), (1, 1), 32, True),      # a 1x1 convolution on pooled features: 32 rows
+    ("conv2d", (32, 256, 1, 1), (2, 2), 32, True),      # 4 pixels: 128 rows
+    ("conv2d", (64, 384, 1, 1), (2, 4), 32, False),     # 8 pixels: 256 rows, half a backward tile at the end
+    ("conv2d", (32, 128, 1, 1), (1, 2), 32, True),      # 64 rows
+    ("linear", (64, 384), None, 64, True),
+    ("linear", (96, 256), None, 128, False)])
+def test_fused_path_for_more_rows_and_1x1_convolutions(ops, kind, shape, pixels, batch, per_channel, monkeypatch):
+    """30 iterations through AdaroundOptimizer on layers the widened fused path takes -- batches of 64 and 128 rows,
+    in_features that are a multiple of 128 only, 1x1 convolutions whose rows are the pixels of the 32 images -- against
+    the CPU restatement (functional.conv2d / functional.linear under autograd and torch.optim.Adam) on the same
+    batches, and against the unfused product path (soft-rounding kernel, torch's layer, fused backward kernel)."""
+    from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
+    iters = 30
+    hyper = (iters, 0.01, (20, 2), 0.2)
+    act = torch.relu
+    torch.manual_seed(61)
+    samples = 3 * batch
+    all_inp = torch.randn(samples, shape[1], *pixels) if kind == "conv2d" else torch.randn(samples, shape[1])
+    weight, delta, offset, C, npc, cmin, cmax = _case(63, shape, 0, per_channel)
+    alpha0 = ada.generate_alpha(weight, ada.broadcast(delta, weight, 0))
+    all_out = ada.layer_output(kind, all_inp, weight)
+    all_out = all_out + 0.02 * torch.randn_like(all_out)      # see test_fused_optimisation_trajectory
+    batches = [torch.randperm(samples)[:batch] for _ in range(iters)]
+    a_ref, m_ref, v_ref, g_ref = ada.optimize_rounding(kind, weight, alpha0, delta, offset, cmin, cmax, all_inp,
+                                                       all_out, batches, *hyper, act=act)
+    calls = []
+    real = ops.adaround_linear_fwd
+    monkeypatch.setattr(ops, "adaround_linear_fwd", lambda *a, **k: (calls.append(a[13].shape), real(*a, **k))[1])
+    a, m, v, g = _run_product_loop(kind, weight, alpha0, delta, offset, C, npc, cmin, cmax, all_inp, all_out,
+                                   batches, hyper, act, {})
+    rows = batch * (pixels[0] * pixels[1] if pixels else 1)
+    assert calls == [(rows, shape[0])] * iters            # the fused path ran, on that many rows
+    monkeypatch.setattr(AdaroundOptimizer, "use_fused_linear", False)
+    a_u, m_u, v_u, g_u = _run_product_loop(kind, weight, alpha0, delta, offset, C, npc, cmin, cmax, all_inp, all_out,
+                                           batches, hyper, act, {})
+    assert len(calls) == iters
+    assert a.shape == weight.shape and (a_ref - alpha0).abs().max() > 5e-3
+    for got, want, scale in ((a, a_ref, None), (a, a_u, None), (g, g_ref, g_ref), (g, g_u, g_ref), (m, m_ref, m_ref),
+                             (m, m_u, m_ref), (v, v_ref, v_ref), (v, v_u, v_ref)):
+        if scale is None:
+            assert _close_except_few(got, want, atol=5e-5) and (got - want).abs().max() < 5e-3
+        else:
+            assert _close_except_few(got, want, atol=1e-4 * scale.abs().max().item(), rtol=1e-3)
+
+
+def test_fused_path_leaves_other_convolutions_alone(ops, monkeypatch):
+    """A 3x3 kernel, a stride, a padding, groups, a row count that is not 32 / 64 / 128 / 256: the unfused path."""
+    from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
+    weight, delta, offset, C, npc, cmin, cmax = _case(65, (32, 128, 1, 1), 0, True)
+    qm = type("Q", (), dict(num_channel=C, n_per_channel=npc))()
+    batches = [torch.arange(32)]
+    x = torch.randn(64, 128, 2, 2).cuda()
+    y = torch.randn(64, 32, 2, 2).cuda()
+    ok = torch.nn.Conv2d(128, 32, 1)
+    assert AdaroundOptimizer._fused_rows(ok, weight.cuda(), qm, x, y, batches) is not None
+    for conv in (torch.nn.Conv2d(128, 32, 1, stride=2), torch.nn.Conv2d(128, 32, 1, padding=1),
+                 torch.nn.Conv2d(128, 32, 1, stride=(1, 2)), torch.nn.Conv2d(128, 32, 1, padding=(0, 1))):
+        assert AdaroundOptimizer._fused_rows(conv, weight.cuda(), qm, x, y, batches) is None
+    w3 = torch.randn(32, 128, 3, 3).cuda()
+    assert AdaroundOptimizer._fused_rows(torch.nn.Conv2d(128, 32, 3), w3, qm, x, y, batches) is None
+    x3 = torch.randn(64, 128, 1, 3).cuda()                 # 96 rows
+    assert AdaroundOptimizer._fused_rows(ok, weight.cuda(), qm, x3, torch.randn(64, 32, 1, 3).cuda(), batches) is None
+    assert AdaroundOptimizer._fused_rows(ok, weight.cuda(), qm, x, y, [torch.arange(16)]) is not None     # 64 rows
+    assert AdaroundOptimizer._fused_rows(ok, weight.cuda(), qm, x, y, [torch.arange(24)]) is None
+    assert AdaroundOptimizer._fused_rows(torch.nn.ConvTranspose2d(128, 32, 1), weight.cuda(), qm, x, y, batches) is None
 
 
 def test_cfg5_fused_linear_at_configured_size(ops):
