@@ -1281,9 +1281,11 @@ def main():
     if not os.path.exists(os.path.join(ROOT, "aimet_amd", "libmiq.so")):
         import __graft_entry__
         __graft_entry__.build()
+    import gc
     import torch
     from aimet_amd import ops
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    gc.disable()
     torch.cuda.set_device(0)
 
     main_shape = (11008, 4096)
@@ -1292,6 +1294,10 @@ def main():
     legs = None if args.only is None else set(args.only.split(","))
 
     def want(leg):
+        # Python's cycle collector is off while a leg runs (as timeit does) and is run between legs: a full collection
+        # walks every object the earlier legs left behind (a simulation model holds tens of thousands of encoding
+        # objects) and lands in whichever host-paced region happens to be timed then -- 6 ms on a 4 ms forward
+        gc.collect()
         return leg in legs if legs is not None else leg != "copyref"
 
     if want("copyref"):
