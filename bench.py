@@ -31,7 +31,8 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch at the main shape, from hardware counters (two rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE,
 # each scaled by what the same counter reads for a plain elementwise kernel of known traffic: x2.000 and x1.000).
 # The counter runs are separate from this program; these are their results for [11008,4096] fp32.
-MEASURED_TRAFFIC_BYTES = {"ste_bwd_per_channel_f32": 542.47e6, "qdq_fwd_per_channel_f32": 363.61e6}
+MEASURED_TRAFFIC_BYTES = {"ste_bwd_per_channel_f32": 542.47e6, "qdq_fwd_per_channel_f32": 363.65e6,
+                          "qdq_mask_fwd_per_channel_f32": 372.08e6, "ste_mask_bwd_f32": 372.07e6}
 
 
 def _laplace_weights(torch, shape, seed, device):
@@ -1369,7 +1370,8 @@ def main():
                                         "avg_launch_ms": res["fwd_ms"], "algorithmic_bytes_per_launch": 8 * n,
                                         "traffic": MEASURED_TRAFFIC_BYTES["qdq_fwd_per_channel_f32"]}},
     }
-    line["saved_mask_step"] = dict(res["saved_mask"], note="the same fwd+bwd step with the forward writing the "
+    line["saved_mask_step"] = dict(res["saved_mask"], fwd_traffic=MEASURED_TRAFFIC_BYTES["qdq_mask_fwd_per_channel_f32"],
+                                   bwd_traffic=MEASURED_TRAFFIC_BYTES["ste_mask_bwd_f32"], note="the same fwd+bwd step with the forward writing the "
                                    "straight-through mask (1 bit per element) and the backward reading it instead of x")
     if "tf_enhanced_calibration" in extra:
         # the metric's second half, as flat keys of the roofline object: hist_kernel over the 16 + 1 passes of the
