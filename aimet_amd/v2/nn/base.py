@@ -21,6 +21,9 @@ def _no_op(input):  # pylint: disable=redefined-builtin
     return input
 
 
+_no_op.is_pass_through = True      # a quantizer calibrating behind this forward need not quantize the batch
+
+
 class BaseQuantizationMixin:
     """Mixin that implements quantization on top of regular torch modules."""
 
@@ -41,11 +44,40 @@ class BaseQuantizationMixin:
         self._compute_param_encodings(overwrite=False)
         return super().__call__(*args, **kwargs)
 
+    # Quantized parameters are kept between forwards of a module in evaluation mode without autograd while nothing they
+    # depend on has changed (the reference quantizes every parameter in every forward, :205-213): the same parameter
+    # object at the same version and address, the same min / max parameter objects at the same versions, the same
+    # grid, and a quantizer whose forward is its class's own.  In-place edits through a `.data` alias move no version
+    # counter: set `keep_quantized_parameters = False` on the module (or the class) around them.
+    keep_quantized_parameters = True
+
+    def _kept_parameter_key(self, param, quantizer):
+        if not self.keep_quantized_parameters or self.training or torch.is_grad_enabled() or \
+                not isinstance(quantizer, MinMaxQuantizer) or 'forward' in quantizer.__dict__:
+            return None
+        mn, mx = quantizer.min, quantizer.max
+        # pylint: disable=protected-access
+        return (id(param), param._version, param.data_ptr(), param.dtype, tuple(param.shape), id(quantizer),
+                id(mn), mn._version, id(mx), mx._version, quantizer.qmin, quantizer.qmax, quantizer.symmetric,
+                quantizer.block_size)
+
     def _patch_quantized_parameters(self):
         stack = contextlib.ExitStack()
+        kept = self.__dict__.setdefault('_kept_quantized_parameters', {})
         for param_name, param_quantizer in self.param_quantizers.items():
             if param_quantizer and param_quantizer.is_initialized():
-                stack.enter_context(patch_attr(self, param_name, param_quantizer(getattr(self, param_name))))
+                param = getattr(self, param_name)
+                key = self._kept_parameter_key(param, param_quantizer)
+                entry = kept.get(param_name) if key is not None else None
+                if entry is not None and entry[0] == key and entry[1] is param:
+                    quantized = entry[2]
+                else:
+                    quantized = param_quantizer(param)
+                    if key is not None:
+                        kept[param_name] = (key, param, quantized)
+                    else:
+                        kept.pop(param_name, None)
+                stack.enter_context(patch_attr(self, param_name, quantized))
         return stack
 
     def _compute_param_encodings(self, overwrite: bool):
@@ -177,14 +209,33 @@ class QuantizationMixin(BaseQuantizationMixin):
         for i, quantizer in enumerate(self.input_quantizers):
             if quantizer and i < len(args) and isinstance(args[i], torch.Tensor) and args[i].is_floating_point():
                 args[i] = quantizer(args[i])
-        with self._patch_quantized_parameters():
-            output = super().forward(*args, **kwargs)
+        if self._relu_is_absorbed(args, kwargs):
+            output = args[0]
+        else:
+            with self._patch_quantized_parameters():
+                output = super().forward(*args, **kwargs)
         outputs = list(output) if isinstance(output, (tuple, list)) else [output]
         for i, quantizer in enumerate(self.output_quantizers):
             if quantizer and i < len(outputs) and isinstance(outputs[i], torch.Tensor) and \
                     outputs[i].is_floating_point():
                 outputs[i] = quantizer(outputs[i])
         return type(output)(outputs) if isinstance(output, (tuple, list)) else outputs[0]
+
+    def _relu_is_absorbed(self, args, kwargs) -> bool:
+        """True when running the ReLU would not change this module's result, so its pass over the activations (as
+        much traffic as the quantizer's) is left out: the output quantizer's grid starts exactly at zero, and
+        quantize-dequantize then maps every negative input to zero and leaves NaN a NaN, as it does after the ReLU --
+        identical element for element.  Only without autograd (the straight-through mask of the pre-activation
+        differs at zero) and for a ReLU that is not in-place (an in-place one also rewrites its input, which other
+        readers of that tensor may rely on)."""
+        if type(self).qcls_to_cls.get(type(self)) is not nn.ReLU or self.inplace or kwargs or \
+                torch.is_grad_enabled() or len(args) != 1 or len(self.output_quantizers) != 1:
+            return False
+        quantizer, tensor = self.output_quantizers[0], args[0]
+        if type(quantizer).__name__ != 'QuantizeDequantize' or 'forward' in quantizer.__dict__ or \
+                not isinstance(tensor, torch.Tensor) or not tensor.is_floating_point() or not tensor.is_cuda:
+            return False
+        return quantizer.is_initialized() and quantizer.lower_bound_is_zero()
 
     @classmethod
     def wrap(cls, module_cls: Type[nn.Module]):

@@ -21,6 +21,7 @@ copy each way.
 Gradients w.r.t. scale and offset (range learning, :329-344) come from one fused pass over the input and the
 incoming gradient, together with the input gradient.
 """
+import functools
 from typing import List, Optional
 
 import torch
@@ -35,6 +36,7 @@ def _is_value_representable(dtype: torch.dtype, value: int) -> bool:
     return bool(r.isfinite()) and int(r.long()) == value
 
 
+@functools.lru_cache(maxsize=256)
 def _is_grid_representable(dtype: torch.dtype, qmin: int, qmax: int) -> bool:
     return all(_is_value_representable(dtype, v) for v in (qmax, qmax - 1, qmin + 1, qmin))
 
@@ -80,7 +82,11 @@ def _apply_per_channel(func, tensor, scale, offset, qmin, qmax, block_size):
     expanded = reshape_tensor_for_blocks(tensor, scale.shape, block_size)
     tensor3, perm = channel_view(expanded, get_encoding_shape_with_blocks(scale.shape, block_size))
     c = tensor3.shape[1]
-    out = func.apply(tensor3, scale.reshape(c, 1), offset.reshape(c, 1), qmin, qmax)
+    if func is _QuantDequantFunc and not torch.is_grad_enabled():
+        # inference: the same kernel without the autograd.Function machinery around it
+        out = ops.v2_qdq(tensor3, c, max(tensor3.shape[2], 1), scale.reshape(c, 1), offset.reshape(c, 1), qmin, qmax)
+    else:
+        out = func.apply(tensor3, scale.reshape(c, 1), offset.reshape(c, 1), qmin, qmax)
     return channel_view_restore(out, expanded.shape, perm).reshape(shape)
 
 

@@ -21,15 +21,46 @@ from ..encoding_analyzer import EncodingAnalyzer, MinMaxEncodingAnalyzer
 from .backends import _derive_qmin_qmax, quantize, quantize_dequantize
 
 
+_pending_range_checks = None     # a list while batched_range_checks() is active
+
+
+def _examine_bounds(bounds: torch.Tensor, dtype: torch.dtype):
+    """bounds: float64 host tensor of range bounds that were computed in `dtype`."""
+    if not bool(torch.isfinite(bounds).all()):
+        warnings.warn('Infinite or NaN values detected within input! This may skew the associated encodings')
+    extreme = float(torch.finfo(dtype).max)
+    # torch.isclose(|x|, extreme, rtol=0.05) with its default atol of 1e-8
+    if bool(((bounds.abs() - extreme).abs() <= 1e-8 + 0.05 * extreme).any()):
+        warnings.warn('Extreme values detected within input! This may skew the associated encodings')
+
+
 def _flag_extreme_min_max(curr_min: torch.Tensor, curr_max: torch.Tensor):
     """Warns about ranges that are not finite or sit at the edge of the dtype (reference
-    encoding_analyzer.py:388-395)."""
-    if not (torch.all(torch.isfinite(curr_min)) and torch.all(torch.isfinite(curr_max))):
-        warnings.warn('Infinite or NaN values detected within input! This may skew the associated encodings')
-    extreme = torch.full_like(curr_min, torch.finfo(curr_min.dtype).max)
-    if torch.any(torch.isclose(torch.abs(curr_min), extreme, rtol=0.05)) or \
-            torch.any(torch.isclose(torch.abs(curr_max), extreme, rtol=0.05)):
-        warnings.warn('Extreme values detected within input! This may skew the associated encodings')
+    encoding_analyzer.py:388-395).  The bounds are parameter-sized: they are read back once and examined on the host,
+    instead of four reductions that each wait for the device; inside batched_range_checks() the read-back is shared
+    with every other quantizer's."""
+    bounds = torch.cat((curr_min.detach().reshape(-1), curr_max.detach().reshape(-1))).to(torch.float64)
+    if _pending_range_checks is not None:
+        _pending_range_checks.append((bounds, curr_min.dtype))
+        return
+    _examine_bounds(bounds.cpu(), curr_min.dtype)
+
+
+@contextlib.contextmanager
+def batched_range_checks():
+    """While active, the range warnings of every quantizer that leaves compute_encodings() are held back and issued
+    together at the end, from one device-to-host copy per device."""
+    global _pending_range_checks       # pylint: disable=global-statement
+    outer, _pending_range_checks = _pending_range_checks, []
+    try:
+        yield
+    finally:
+        pending, _pending_range_checks = _pending_range_checks, outer
+        groups = {}
+        for bounds, dtype in pending:
+            groups.setdefault((bounds.device, dtype), []).append(bounds)
+        for (_, dtype), tensors in groups.items():
+            _examine_bounds(torch.cat(tensors).cpu(), dtype)
 
 
 class _AffineEncoding:
@@ -245,6 +276,10 @@ class MinMaxQuantizer(nn.Module):
         quantized with the range of this batch alone (reference :330-352)."""
         per_block = reshape_tensor_for_blocks(tensor, self.shape, self.block_size)
         batch = self.encoding_analyzer.update_stats(per_block)
+        if getattr(plain_forward, 'is_pass_through', False):
+            # a quantized module calibrates with its activation quantizers switched to pass-through: the range of
+            # this batch alone would be computed (another pass over the batch, a search, a wait) and not used
+            return plain_forward(tensor)
         bounds = self.encoding_analyzer.compute_encodings_from_stats(batch, self.qmax - self.qmin, self.symmetric)
         stand_ins = {}
         for name, bound in zip(('min', 'max'), bounds):
@@ -289,8 +324,37 @@ class MinMaxQuantizer(nn.Module):
     def get_encoding(self) -> Optional[_AffineEncoding]:
         if not self.is_initialized():
             return None
-        return _AffineEncoding(self.get_scale(torch.float32), self.get_offset(torch.float32), self.qmin, self.qmax,
-                               self._symmetric, self.block_size)
+        # Scale and offset are a handful of parameter-sized tensor operations per call (the reference performs them in
+        # every forward).  When no gradient can flow into min / max they depend on nothing but the parameters' values:
+        # kept until a parameter object is replaced or modified in place (its version counter moves), or the grid
+        # changes.  An edit through a `.data` alias moves no counter: assign, or use set_range().
+        mn, mx = self.min, self.max
+        learning = torch.is_grad_enabled() and (mn.requires_grad or mx.requires_grad)
+        key = None if learning else (id(mn), mn._version, id(mx), mx._version, self.qmin, self.qmax,  # pylint: disable=protected-access
+                                     self._symmetric)
+        kept = self.__dict__.get('_kept_encoding')
+        if key is not None and kept is not None and kept[0] == key and kept[1] is mn and kept[2] is mx:
+            scale, offset = kept[3], kept[4]
+        else:
+            scale, offset = self.get_scale(torch.float32), self.get_offset(torch.float32)
+            if key is not None:
+                with torch.no_grad():
+                    scale, offset = scale.detach(), offset.detach()
+                self.__dict__['_kept_encoding'] = (key, mn, mx, scale, offset)
+        return _AffineEncoding(scale, offset, self.qmin, self.qmax, self._symmetric, self.block_size)
+
+    def lower_bound_is_zero(self) -> bool:
+        """True when the kept encoding's grid starts exactly at zero (offset == -qmin everywhere), known on the host:
+        one read-back per kept encoding, none when no encoding is being kept (then the answer is False)."""
+        if self.get_encoding() is None:
+            return False
+        kept = self.__dict__.get('_kept_encoding')
+        if kept is None or kept[1] is not self.min or kept[2] is not self.max:
+            return False
+        if len(kept) == 5:
+            kept = kept + (bool((kept[4] == -self.qmin).all()),)
+            self.__dict__['_kept_encoding'] = kept
+        return kept[5]
 
     @torch.no_grad()
     def get_legacy_encodings(self):

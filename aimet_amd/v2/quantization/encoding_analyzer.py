@@ -155,8 +155,13 @@ class _DeviceHistograms:
     def __init__(self, hist: torch.Tensor, minmax: torch.Tensor, bad_flag: torch.Tensor):
         self.hist, self.minmax, self._bad_flag = hist, minmax, bad_flag
 
+    known_bad = None     # the flag's value when an owner of many observers has read all of theirs in one copy
+
     def check(self):
-        if self._bad_flag is not None and int(self._bad_flag.item()) != 0:
+        bad, self.known_bad = self.known_bad, None
+        if bad is None and self._bad_flag is not None:
+            bad = int(self._bad_flag.item())
+        if bad:
             raise ValueError('Input tensor cannot contain only infinite or only NaN values')
 
     def __len__(self):
@@ -270,6 +275,7 @@ class _HistogramObserver:
         repeat = self._repeat
         if repeat is not None and repeat.matches(input_tensor):
             repeat(input_tensor)          # same device, size and layout as the update before: nothing to set up
+            self._state.known_bad = None  # (whatever was read of the flag before this batch is out of date)
         else:
             self._update(input_tensor, merge=True, want_batch=False)
             if self.num_histograms == 1 and input_tensor.dtype == torch.float32 and input_tensor.is_contiguous():
@@ -286,6 +292,21 @@ class _HistogramObserver:
         if self._state is None:
             return [_Histogram() for _ in range(self.num_histograms)]
         return self._state
+
+    @staticmethod
+    def read_flags_together(observers):
+        """One device-to-host copy for the "no finite value seen" flags of many observers instead of one wait per
+        observer when their statistics are read next (the owner of a model's quantizers calls this before it asks
+        each of them for its encoding)."""
+        by_device = {}
+        for observer in observers:
+            state, flag = observer._state, observer._bad_flag          # pylint: disable=protected-access
+            if state is not None and flag is not None and state._bad_flag is flag:   # pylint: disable=protected-access
+                by_device.setdefault(flag.device, []).append((state, flag))
+        for pairs in by_device.values():
+            values = torch.cat([flag for _, flag in pairs]).cpu().tolist()
+            for (state, _), value in zip(pairs, values):
+                state.known_bad = int(value)
 
     stats = property(get_stats)          # the reference exposes the running statistics as an attribute
 

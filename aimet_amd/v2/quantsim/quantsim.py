@@ -22,8 +22,10 @@ from ...v1.quantsim import QuantizationSimModel as _V1QuantizationSimModel
 from ...v1.tensor_quantizer import StaticGridPerChannelQuantizer
 from ..nn import BaseQuantizationMixin, QuantizationMixin
 from ..quantization.affine import QuantizeDequantize
+from ..quantization.affine.quantizer import batched_range_checks
 from ..quantization.float import FloatQuantizeDequantize
-from ..quantization.encoding_analyzer import MinMaxEncodingAnalyzer, PercentileEncodingAnalyzer, SqnrEncodingAnalyzer
+from ..quantization.encoding_analyzer import (MinMaxEncodingAnalyzer, PercentileEncodingAnalyzer,
+                                              SqnrEncodingAnalyzer, _HistogramObserver)
 
 _RANGE_LEARNING = (QuantScheme.training_range_learning_with_tf_init,
                    QuantScheme.training_range_learning_with_tf_enhanced_init)
@@ -148,7 +150,10 @@ class QuantizationSimModel:
 
     def compute_encodings(self, forward_pass_callback, forward_pass_callback_args):
         """Runs the callback with every quantizer observing, then fixes the encodings (v2 quantsim.py:205-224)."""
-        with contextlib.ExitStack() as stack:
+        # the quantizers fix their encodings as the stack unwinds, one after the other: what each of them would wait
+        # for the device for (has any observer seen only non-finite values, are the new ranges sane) is read for all
+        # of them together
+        with batched_range_checks(), contextlib.ExitStack() as stack:
             for _, module in self.qmodules():
                 stack.enter_context(module.compute_encodings())
             was_training = self.model.training
@@ -158,6 +163,10 @@ class QuantizationSimModel:
                     forward_pass_callback(self.model, forward_pass_callback_args)
             finally:
                 self.model.train(was_training)
+            observers = [getattr(getattr(q, 'encoding_analyzer', None), 'observer', None) for _, module in
+                         self.qmodules() for q in list(module.input_quantizers) + list(module.output_quantizers) +
+                         list(module.param_quantizers.values()) if q is not None]
+            _HistogramObserver.read_flags_together([o for o in observers if isinstance(o, _HistogramObserver)])
 
     def get_encodings_dict(self) -> dict:
         """The exported dictionary, laid out as the v1 simulation's: parameters by '<module>.<parameter>', activations

@@ -826,9 +826,45 @@ def bench_end_to_end(torch, ops):
         "calibration_overhead_pct_of_forward": 100.0 * (wall_cal - wall_fp32) / wall_fp32,
         "observed_elements_per_s": seen["elements"] / wall_cal,
         "note": "compute_encodings reads every encoding back at its end, so its host time includes the device's"}
-    del sim, model, data
+    del sim
     import gc
     gc.collect()          # the simulation model is a web of reference cycles: collected here, not inside a timed region
+
+    # ---- the same through the v2 classes (SQNR analyzers with 2048-bin observers on every activation and, per
+    # channel, on every weight), and its simulated forward afterwards
+    from aimet_amd.v2.quantsim import QuantizationSimModel as V2Sim
+    sim2 = V2Sim(model, dummy_input=data[0][:2], quant_scheme='tf_enhanced', default_output_bw=8, default_param_bw=8,
+                 config_file=cfg)
+    sim2.compute_encodings(passes, data[:1])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    sim2.compute_encodings(passes, data)
+    host_v2 = time.perf_counter() - t0
+    torch.cuda.synchronize()
+    wall_v2 = time.perf_counter() - t0
+
+    def per_forward(fn, steps=10):
+        with torch.no_grad():
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for _ in range(steps):
+                fn()
+            torch.cuda.synchronize()
+        return (time.perf_counter() - t1) * 1e3 / steps
+
+    x1 = data[0][:1].clone()
+    out["v2_resnet50_shaped"] = {
+        "scheme": "tf_enhanced (SqnrEncodingAnalyzer)", "batches": num_batches, "batch": batch,
+        "compute_encodings_wall_ms": wall_v2 * 1e3, "compute_encodings_host_ms": host_v2 * 1e3,
+        "plain_forward_wall_ms": wall_fp32 * 1e3,
+        "sim_forward_batch64_ms": per_forward(lambda: sim2.model(data[0])),
+        "fp32_forward_batch64_ms": per_forward(lambda: model(data[0])),
+        "sim_forward_batch1_ms": per_forward(lambda: sim2.model(x1)),
+        "fp32_forward_batch1_ms": per_forward(lambda: model(x1))}
+    del sim2, model, data
+    gc.collect()
 
     # ---- apply_adaround
     from aimet_amd.v1.adaround.adaround_weight import Adaround, AdaroundParameters
