@@ -49,6 +49,7 @@ _SIGNATURES = {
     "miq_qdq_per_tensor_bf16": ([_p, _p, _i64, _dbl, _dbl, _int, _int, _p], _int),
     "miq_quantize_per_tensor_f32": ([_p, _p, _i64, _dbl, _dbl, _int, _int, _int, _p], _int),
     "miq_qdq_codes_per_tensor_f32": ([_p, _p, _p, _i64, _dbl, _dbl, _int, _int, _p], _int),
+    "miq_tf_encodings_per_channel_f32": ([_p, _p, _i64, _int, _int, _int, _int, _p, _p, _p, _p, _p, _p, _p, _p], _int),
     "miq_per_channel_params_f32": ([_p, _p, _i64, _dbl, _p, _p, _p, _p, _p], _int),
     "miq_qdq_per_channel_f32": ([_p, _p, _i64, _i64, _i64, _p, _p, _p, _p, _int, _p], _int),
     "miq_qdq_per_channel_bf16": ([_p, _p, _i64, _i64, _i64, _p, _p, _p, _p, _int, _p], _int),

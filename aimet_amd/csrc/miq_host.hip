@@ -2,6 +2,7 @@
 // on the host (ModelOptimizations/DlQuantization/src/TensorQuantizationSim.cpp:62-92,
 // ModelOptimizations/DlQuantization/src/quantization_utils.cpp:58-156).
 #include "miq_common.h"
+#include "miq_encoding_math.h"
 
 #include <algorithm>
 #include <cmath>
@@ -59,46 +60,13 @@ int miq_get_computed_encodings(int bw, double mn, double mx, int use_symmetric, 
 {
     MIQ_CHECK_ARG(out != nullptr, "null output encoding");
     MIQ_CHECK_ARG(bw >= 1 && bw <= 32, "bitwidth must be in [1, 32] (got %d)", bw);
-    const double fmax = std::numeric_limits<float>::max();
-    double steps      = std::pow(2.0, bw) - 1;
-    if (use_symmetric && use_strict_symmetric)
-        steps -= 1;
-    out->bw = bw;
-    if (std::isinf(mn))
-        mn = -fmax;
-    if (std::isinf(mx))
-        mx = fmax;
-
-    if (use_symmetric && (mn < 0.0 || !use_unsigned_symmetric))
-    {
-        const double amax          = std::max(std::abs(mx), std::abs(mn));
-        const unsigned int n_pos   = (unsigned int) std::floor(steps / 2);
-        out->delta                 = amax / n_pos;
-        out->offset                = -std::ceil(steps / 2);
-        out->min                   = std::max(out->offset * out->delta, -fmax);
-        out->max                   = std::min(out->delta * n_pos, fmax);
-        return MIQ_OK;
-    }
-    out->delta = (mx - mn) / steps;
-    if (mn < 0 && mx > 0)
-    {
-        // zero must sit exactly on the grid
-        double z    = std::round(-mn / out->delta);
-        z           = std::min(steps, std::max(0.0, z));
-        out->offset = -z;
-    }
-    else
-    {
-        out->offset = std::round(mn / out->delta);
-        out->min    = mn;
-        out->max    = mx;
-        return MIQ_OK;
-    }
-    const double t = out->delta * out->offset;
-    out->min       = (t >= -fmax && t <= fmax) ? t : -fmax;
-    out->max       = mx - mn + out->min;
-    if (out->max > fmax)
-        out->max = fmax;
+    const miq::EncodingD e =
+        miq::computed_encodings(bw, mn, mx, use_symmetric != 0, use_strict_symmetric != 0, use_unsigned_symmetric != 0);
+    out->bw     = bw;
+    out->min    = e.min;
+    out->max    = e.max;
+    out->delta  = e.delta;
+    out->offset = e.offset;
     return MIQ_OK;
 }
 

@@ -15,6 +15,7 @@
 #include <hip/hip_fp16.h>
 
 #include "miq_common.h"
+#include "miq_encoding_math.h"
 #include "miq_fastmath.h"
 #include "miq_io.h"
 #include "miq_stochastic.h"
@@ -986,6 +987,48 @@ __global__ void per_channel_params_kernel(const float* enc_min, const float* enc
     ooffset[i] = rintf(lo / d);
 }
 
+// TF (min / max) encodings of every channel of a tensor and the kernel parameters that follow from them, without a
+// visit to the host: channel c's running (min, max) -> TfEncodingAnalyzer::computeEncoding
+// (DlQuantization/src/TfEncodingAnalyzer.cpp:80-101: zero inside the range, at least 0.01 wide) -> getComputedEncodings in
+// double -> the float32 recipe of per_channel_params_kernel on float32(min), float32(max).  The number of steps of that
+// recipe depends on channel 0's encoding (one step less iff its min == -max), which every thread derives for itself.
+__device__ __forceinline__ EncodingD tf_channel_encoding(float lo_f, float hi_f, int bw, bool sym, bool strict, bool uns)
+{
+    double lo = enc_min2(0.0, (double) lo_f);
+    double hi = enc_max2(0.0, (double) hi_f);
+    hi        = enc_max2(hi, lo + 0.01);
+    return computed_encodings(bw, lo, hi, sym, strict, uns);
+}
+
+__global__ void tf_channel_encodings_kernel(const float* ch_min, const float* ch_max, int64_t c, int bw, int sym, int strict,
+                                            int uns, double* enc, float* omin, float* omax, float* odelta, float* ooffset,
+                                            float* raw_min, float* raw_max)
+{
+    const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= c)
+        return;
+    const EncodingD first = tf_channel_encoding(ch_min[0], ch_max[0], bw, sym, strict, uns);
+    float num_steps       = (float) (ldexp(1.0, bw) - 1.0 - (first.min == -first.max ? 1.0 : 0.0));
+    const EncodingD e     = tf_channel_encoding(ch_min[i], ch_max[i], bw, sym, strict, uns);
+    enc[4 * i + 0]        = e.min;
+    enc[4 * i + 1]        = e.max;
+    enc[4 * i + 2]        = e.delta;
+    enc[4 * i + 3]        = e.offset;
+    float lo = (float) e.min, hi = (float) e.max;
+    raw_min[i] = lo;
+    raw_max[i] = hi;
+    // as per_channel_params_kernel
+    lo        = (lo != lo) ? lo : fminf(lo, 0.f);
+    hi        = (hi != hi) ? hi : fmaxf(hi, 0.f);
+    float eps = lo + 1e-5f;
+    hi        = (hi != hi || eps != eps) ? (hi + eps) : fmaxf(hi, eps);
+    float d   = (hi - lo) / num_steps;
+    omin[i]   = lo;
+    omax[i]   = hi;
+    odelta[i] = d;
+    ooffset[i] = rintf(lo / d);
+}
+
 struct BcastArgs
 {
     int64_t istride[8];
@@ -1249,6 +1292,23 @@ int miq_per_channel_params_f32(const float* enc_min, const float* enc_max, int64
     return MIQ_OK;
 }
 
+
+int miq_tf_encodings_per_channel_f32(const float* ch_min, const float* ch_max, int64_t num_channel, int bw,
+                                     int use_symmetric, int use_strict_symmetric, int use_unsigned_symmetric, double* enc,
+                                     float* out_min, float* out_max, float* out_delta, float* out_offset, float* raw_min,
+                                     float* raw_max, void* stream)
+{
+    MIQ_CHECK_ARG(ch_min && ch_max && enc && out_min && out_max && out_delta && out_offset && raw_min && raw_max &&
+                      num_channel > 0,
+                  "null pointer or non-positive channel count");
+    MIQ_CHECK_ARG(bw >= 1 && bw <= 31, "bitwidth must be in [1, 31] (got %d)", bw);
+    const int64_t blocks = (num_channel + kBlock - 1) / kBlock;
+    hipLaunchKernelGGL(tf_channel_encodings_kernel, dim3((unsigned) blocks), dim3(kBlock), 0, (hipStream_t) stream, ch_min,
+                       ch_max, num_channel, bw, use_symmetric, use_strict_symmetric, use_unsigned_symmetric, enc, out_min,
+                       out_max, out_delta, out_offset, raw_min, raw_max);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
 
 int miq_qdq_per_channel_f32(const float* in, float* out, int64_t num_channel, int64_t num_element,
                             int64_t num_element_per_channel, const float* enc_min, const float* enc_max,

@@ -249,6 +249,23 @@ def qdq_codes_per_tensor(x, enc_min, enc_max, bw, shift_to_signed=False, want_de
     return out, codes
 
 
+def tf_encodings_per_channel(minmax, bw, symmetric, strict_symmetric, unsigned_symmetric):
+    """minmax: float32 GPU tensor [2, C] of per-channel running minima and maxima.  Returns (enc, params): enc a
+    float64 GPU tensor [C, 4] = (min, max, delta, offset) of every channel's TF encoding, params the six float32
+    vectors (min, max, delta, offset, raw_min, raw_max) the per-channel kernels take.  Nothing waits for the device."""
+    _require_gpu(minmax)
+    if minmax.dtype != _F32 or minmax.dim() != 2 or minmax.size(0) != 2 or not minmax.is_contiguous():
+        raise RuntimeError("minmax must be a contiguous float32 tensor [2, C]")
+    c = minmax.size(1)
+    enc = torch.empty(c, 4, dtype=torch.float64, device=minmax.device)
+    outs = torch.empty(6, c, dtype=_F32, device=minmax.device)
+    with _OnDevice(minmax.device):
+        check(lib.miq_tf_encodings_per_channel_f32(_ptr(minmax[0]), _ptr(minmax[1]), c, int(bw), int(bool(symmetric)),
+                                                   int(bool(strict_symmetric)), int(bool(unsigned_symmetric)),
+                                                   _ptr(enc), *(_ptr(outs[k]) for k in range(6)), _stream(minmax)))
+    return enc, tuple(outs[k] for k in range(6))
+
+
 def per_channel_params(enc_min, enc_max, num_steps):
     """(min, max, delta, offset) float32 device vectors from raw per-channel min/max (float32 tensors on the GPU)."""
     _require_gpu(enc_min, enc_max)

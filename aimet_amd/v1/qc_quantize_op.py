@@ -322,7 +322,8 @@ class SteGatingFuncForParameters(torch.autograd.Function):
             if quantizer.bitwidth == 32 or quantizer.data_type == QuantizationDataType.float:
                 continue
             if quantizer.enabled and param.grad is not None:
-                if isinstance(quantizer.encoding, list):
+                if isinstance(quantizer, StaticGridPerChannelQuantizer):
+                    # (the bounds as device vectors: the per-channel encoding list is not needed on the host)
                     _, _, _, _, raw_min, raw_max = quantizer.device_params(param.device)
                     # pylint: disable=protected-access
                     param.grad = ste.compute_dloss_by_dx(param, param.grad, raw_min, raw_max, quantizer._ch_axis)

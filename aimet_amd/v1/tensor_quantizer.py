@@ -79,6 +79,26 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         self.fp8_maxval = None        # largest value of the 8-bit float grid: 0-dim tensor, or one entry per channel
         self._fp8_grid = None         # (maxval, bias, steps) device tensors of that grid, and the maxval they are for
 
+    # The list of TfEncoding objects.  A per-channel quantizer whose encodings were computed on the device keeps them
+    # there (`_pending_encoding`) and builds the list when somebody reads it: a wrapper in training mode recomputes its
+    # parameter encodings in every forward and only ever quantizes with them.
+    @property
+    def _encoding(self):
+        pending = self.__dict__.get('_pending_encoding')
+        if pending is not None:
+            self.__dict__['_pending_encoding'] = None
+            self.__dict__['_encoding_list'] = pending()
+        return self.__dict__.get('_encoding_list')
+
+    @_encoding.setter
+    def _encoding(self, value):
+        self.__dict__['_pending_encoding'] = None
+        self.__dict__['_encoding_list'] = value
+
+    def _has_encoding(self) -> bool:
+        """bool(self._encoding) without building the list."""
+        return self.__dict__.get('_pending_encoding') is not None or bool(self.__dict__.get('_encoding_list'))
+
     # ---- 8-bit float grid (reference tensor_quantizer.py:393-400, :461-468, :544-552; fp_quantization.py:45-122)
     @property
     def _is_fp8(self) -> bool:
@@ -137,7 +157,8 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         state['_num_ops'] = len(self._cppOp)
         state['_encoding'] = None if self._encoding is None else \
             [(e.min, e.max, e.delta, e.offset, e.bw) for e in self._encoding]
-        for key in ('_cppOp', '_dev_params', '_fp8_grid', '_channel_analyzer', '_computed_from'):
+        for key in ('_cppOp', '_dev_params', '_fp8_grid', '_channel_analyzer', '_computed_from', '_encoding_list',
+                    '_pending_encoding'):
             state.pop(key, None)
         return state
 
@@ -210,7 +231,8 @@ class StaticGridTensorQuantizer(TensorQuantizer):
             # parameter (once when the first forward needs the encoding, once at the end of compute_encodings), and
             # a per-channel answer costs a search launch, a read-back and thousands of encoding objects
             recipe, result = self.__dict__.get('_computed_from') or (None, None)
-            if self._encoding and result is self._encoding and recipe == self._encoding_recipe():
+            if result is not None and result is self.__dict__.get('_encoding_list') and result and \
+                    recipe == self._encoding_recipe():
                 return
             self._encoding = []
             self._dev_params = None
@@ -222,16 +244,24 @@ class StaticGridTensorQuantizer(TensorQuantizer):
                     self._encoding = [libpymo.TfEncoding(-float(m), float(m), 0.0, 0.0, 8)
                                       for m in self.fp8_maxval.reshape(-1).tolist()]
                 return
-            for encoding, valid in self._compute_op_encodings():
-                if not valid:
-                    self.enabled = False
-                else:
-                    self._encoding.append(encoding)
+            computed = self._compute_op_encodings()
+            if callable(computed):
+                # every channel's encoding exists, on the device: the list is built when it is first read
+                self.__dict__['_pending_encoding'] = computed
+            else:
+                for encoding, valid in computed:
+                    if not valid:
+                        self.enabled = False
+                    else:
+                        self._encoding.append(encoding)
             self.is_unsigned_symmetric = self.use_symmetric_encodings and self.use_unsigned_symmetric and \
                 all(enc.min >= 0 and enc.max >= 0 for enc in self._encoding)
-            assert not (not self.enabled and self._encoding), \
+            assert not (not self.enabled and self._has_encoding()), \
                 'At least one encoding for a multi-encoding quantizer is invalid.'
-            self.__dict__['_computed_from'] = (self._encoding_recipe(), self._encoding) if self.enabled else None
+            if self.__dict__.get('_pending_encoding') is None:
+                self.__dict__['_computed_from'] = (self._encoding_recipe(), self._encoding) if self.enabled else None
+            else:
+                self.__dict__['_computed_from'] = None
 
     def _compute_op_encodings(self):
         return [op.getEncoding(self.bitwidth, self.use_symmetric_encodings, self.use_strict_symmetric,
@@ -421,6 +451,8 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
             return [(libpymo.TfEncoding(e.min, e.max, e.delta, e.offset, e.bw), valid) for e in encodings]
         if self._tf_minmax is None:
             return super()._compute_op_encodings()
+        if self.compute_tf_encodings_on_device and self._tf_minmax.is_cuda:
+            return self._tf_encodings_on_device()
         # TfEncodingAnalyzer::computeEncoding per channel (DlQuantization/src/TfEncodingAnalyzer.cpp:80-101) on the
         # fused statistics: one small read-back, then the double-precision host recipe
         mm = self._tf_minmax.double().cpu()
@@ -432,6 +464,22 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
                                            self.use_strict_symmetric, self.use_unsigned_symmetric)
             out.append((libpymo.TfEncoding(e.min, e.max, e.delta, e.offset, e.bw), True))
         return out
+
+    # The TF (min / max) encodings of all channels from one launch, left on the device, instead of one read-back and
+    # one host computation per channel (thousands per layer, in every forward of a wrapper in training mode).  The
+    # numbers are the same: the kernel runs the host recipe's double arithmetic.  False: always the host path.
+    compute_tf_encodings_on_device = True
+
+    def _tf_encodings_on_device(self):
+        mm = self._tf_minmax.to(torch.float32).contiguous()
+        enc, params = ops.tf_encodings_per_channel(mm, self.bitwidth, self.use_symmetric_encodings,
+                                                   self.use_strict_symmetric, self.use_unsigned_symmetric)
+        self._dev_params = params
+        bitwidth = self.bitwidth
+
+        def build():
+            return [libpymo.TfEncoding(mn, mx, delta, offset, bitwidth) for mn, mx, delta, offset in enc.cpu().tolist()]
+        return build
 
     def device_params(self, device):
         """Per-channel kernel parameters on `device`, built once per encoding."""

@@ -863,7 +863,37 @@ def bench_end_to_end(torch, ops):
         "fp32_forward_batch64_ms": per_forward(lambda: model(data[0])),
         "sim_forward_batch1_ms": per_forward(lambda: sim2.model(x1)),
         "fp32_forward_batch1_ms": per_forward(lambda: model(x1))}
-    del sim2, model, data
+    # ---- a training step through the simulation (forward + backward at batch 32; quantization-aware training): in
+    # training mode a v1 wrapper recomputes its parameter encodings in every forward
+    xt = data[0][:32].clone()
+
+    def training_step(m):
+        def run():
+            m.zero_grad(set_to_none=True)
+            m(xt).float().pow(2).mean().backward()
+        for _ in range(3):
+            run()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(5):
+            run()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t1) * 1e3 / 5
+
+    _, sim_tf, _ = quantsim_resnet50_shaped(torch, 32)
+    steps = {"fp32_ms": training_step(model.train())}
+    steps["v1_sim_ms"] = training_step(sim_tf.model.train())
+    from aimet_amd.v1.tensor_quantizer import StaticGridPerChannelQuantizer
+    StaticGridPerChannelQuantizer.compute_tf_encodings_on_device = False
+    try:
+        steps["v1_sim_encodings_through_the_host_ms"] = training_step(sim_tf.model)
+    finally:
+        StaticGridPerChannelQuantizer.compute_tf_encodings_on_device = True
+    steps["v2_sim_ms"] = training_step(sim2.model.train())
+    steps["note"] = ("min/max per-channel weight encodings; a v1 wrapper in training mode recomputes them in every "
+                     "forward (as the reference does): one launch here, one host computation per channel there")
+    out["training_step_batch32_resnet50_shaped"] = steps
+    del sim2, sim_tf, model, data
     gc.collect()
 
     # ---- apply_adaround

@@ -138,6 +138,20 @@ int miq_qdq_codes_per_tensor_f32(const float* in, float* out, uint8_t* codes, in
 int miq_per_channel_params_f32(const float* enc_min, const float* enc_max, int64_t num_channel, double num_steps,
                                float* out_min, float* out_max, float* out_delta, float* out_offset, void* stream);
 
+/* The TF (min / max) encodings of all channels of a tensor, on the device: for channel c, TfEncodingAnalyzer::computeEncoding
+ * (DLQ/src/TfEncodingAnalyzer.cpp:80-101) on the running (ch_min[c], ch_max[c]) and getComputedEncodings in double, as
+ * miq_get_computed_encodings does on the host -- what StaticGridPerChannelQuantizer.compute_encoding
+ * (TrainingExtensions/torch/src/python/aimet_torch/v1/tensor_quantizer.py:280-321) obtains from one analyzer object per
+ * channel -- followed by miq_per_channel_params_f32 on the result.  enc: device double[num_channel][4] = (min, max,
+ * delta, offset) of every channel's TfEncoding; out_*: the four kernel parameter vectors; raw_min / raw_max: float32 of
+ * the encodings' min / max (the straight-through bounds).  All device float[num_channel].  Nothing waits: a wrapper in
+ * training mode recomputes its parameter encodings in every forward (qc_quantize_op.py:769-777), and a caller that only
+ * quantizes with them never needs them on the host. */
+int miq_tf_encodings_per_channel_f32(const float* ch_min, const float* ch_max, int64_t num_channel, int bw,
+                                     int use_symmetric, int use_strict_symmetric, int use_unsigned_symmetric,
+                                     double* enc, float* out_min, float* out_max, float* out_delta, float* out_offset,
+                                     float* raw_min, float* raw_max, void* stream);
+
 /* ITensorQuantizationSim<float>::quantizeDequantizeTensorPerChannel(in, numChannel, numElement, numElementPerChannel,
  * out, encMin*, encMax*, encDelta*, encOffset*, roundMode, useCuda, stream) (ITensorQuantizationSim.h:107-118,
  * DLQ/src/TensorQuantizationSim.cpp:300-317; kernel DLQ/src/trim_functions.cu:78-92):

@@ -429,3 +429,107 @@ def test_simulation_forward_in_a_hip_graph(api):
             eager = sim.model(x)                            # eager work between the replays
             assert torch.equal(static_y, eager), rep
             torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("bw,sym,strict,unsigned", [(8, True, False, False), (4, True, False, False), (8, False, False, False),
+                                                     (8, True, True, False), (8, True, False, True), (16, False, False, False)])
+def test_per_channel_tf_encodings_stay_on_the_device(api, oracle, bw, sym, strict, unsigned):
+    """The min / max encodings of a per-channel quantizer are computed by one launch and left on the device; the list of
+    TfEncoding objects is built when it is read.  Encodings, kernel parameters, quantized values and gradients are
+    those of the host path (one computation per channel), bit for bit, including channels that are all zero, all
+    positive, tiny and huge."""
+    import pickle
+    rng = np.random.default_rng(17)
+    w = (rng.laplace(0, 0.03, (48, 70))).astype(np.float32)
+    w[0] = 0.0                      # no range at all
+    w[1] = np.abs(w[1]) + 0.5       # strictly positive (the unsigned grid differs here)
+    w[2] = -np.abs(w[2]) - 0.5      # strictly negative
+    w[3] *= 1e-30
+    w[4] *= 1e30
+    w[5, 0] = np.float32(3e38)
+    wg = torch.from_numpy(w).cuda()
+
+    def make(on_device):
+        q = api.tq.StaticGridPerChannelQuantizer(bw, api.nearest, api.QuantScheme.post_training_tf, sym, 48,
+                                                 enabled_by_default=True, ch_axis=0)
+        q.use_strict_symmetric, q.use_unsigned_symmetric = strict, unsigned
+        q.compute_tf_encodings_on_device = on_device
+        q.update_encoding_stats(wg)
+        q.update_encoding_stats(wg * 0.5)
+        q.compute_encoding()
+        return q
+
+    dev, host = make(True), make(False)
+    # (the unsigned-symmetric flag of a quantizer is decided from every channel's encoding: that reads the list)
+    lazy = not (sym and unsigned)
+    pending = lambda q: q.__dict__.get('_pending_encoding') is not None
+    assert pending(dev) == lazy and not pending(host)
+    for a, b in zip(dev.device_params(wg.device), host.device_params(wg.device)):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))             # as bits: NaN included
+    assert pending(dev) == lazy                                                  # still not built
+    x = torch.from_numpy((rng.standard_normal(w.shape) * 0.1).astype(np.float32)).cuda()
+    outs = []
+    for q in (dev, host):
+        xg = x.clone().requires_grad_(True)
+        y = q.quantize_dequantize(xg, api.nearest)
+        y.backward(torch.ones_like(y))
+        outs.append((y.detach(), xg.grad))
+    assert torch.equal(outs[0][0].view(torch.int32), outs[1][0].view(torch.int32))
+    assert torch.equal(outs[0][1].view(torch.int32), outs[1][1].view(torch.int32))
+    assert pending(dev) == lazy                                                  # quantizing needs no list
+    got, want = dev.encoding, host.encoding                                      # now it is built
+    assert dev.__dict__.get('_pending_encoding') is None and isinstance(got, list) and len(got) == 48
+    assert [_enc_tuple(e) for e in got] == [_enc_tuple(e) for e in want]
+    mn, mx = np.minimum(w, w * 0.5).min(axis=1), np.maximum(w, w * 0.5).max(axis=1)
+    for c in (1, 2, 7):
+        lo, hi = min(0.0, float(mn[c])), max(0.0, float(mx[c]))
+        assert _enc_tuple(got[c]) == oracle.tf_compute_encoding(lo, max(hi, lo + 0.01), bw, sym, strict, unsigned).astuple()
+    assert dev.is_unsigned_symmetric == host.is_unsigned_symmetric
+    # a pending list travels through pickle as the list
+    again = make(True)
+    clone = pickle.loads(pickle.dumps(again))
+    assert [_enc_tuple(e) for e in clone.encoding] == [_enc_tuple(e) for e in want]
+
+
+def test_training_mode_wrapper_recomputes_parameter_encodings_on_the_device(api):
+    """A wrapper in training mode recomputes its parameter encodings in every forward (reference
+    qc_quantize_op.py:769-777).  With per-channel min / max encodings that is one launch and no wait; outputs, input
+    and weight gradients are those of the host computation."""
+    torch.manual_seed(9)
+    x = torch.randn(4, 8, 10, 10).cuda()
+
+    def run(on_device):
+        torch.manual_seed(10)
+        conv = nn.Conv2d(8, 16, 3, padding=1).cuda()
+        wrapper = api.qc.StaticGridQuantWrapper(conv, 8, 8, 'nearest', api.QuantScheme.post_training_tf)
+        wrapper.enable_per_channel_quantization()
+        q = wrapper.param_quantizers['weight']
+        q.compute_tf_encodings_on_device = on_device
+        q.use_symmetric_encodings = True
+        wrapper.set_mode(api.qc.QcQuantizeOpMode.ANALYSIS)
+        wrapper(x)
+        wrapper.compute_encoding()
+        wrapper.set_mode(api.qc.QcQuantizeOpMode.ACTIVE)
+        wrapper.train()
+        outs = []
+        for step in range(2):
+            xi = x.clone().requires_grad_(True)
+            conv.weight.grad = None
+            y = wrapper(xi)
+            y.pow(2).sum().backward()
+            outs.append((y.detach().clone(), xi.grad.clone(), conv.weight.grad.clone()))
+            with torch.no_grad():
+                conv.weight.mul_(1.1)                     # the next pass must see the new range
+        return outs, q
+
+    dev, qd = run(True)
+    host, qh = run(False)
+    assert qd.__dict__.get('_pending_encoding') is not None and qh.__dict__.get('_pending_encoding') is None
+    for a, b in zip(dev, host):
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+        # (the convolution's weight-gradient kernel adds in no fixed order: equal up to that, and zero in the same places,
+        # which is what the straight-through gate of the parameter decides)
+        assert torch.allclose(a[2], b[2], rtol=1e-4, atol=1e-4 * a[2].abs().max().item())
+        assert torch.equal(a[2] == 0, b[2] == 0)
+    assert not torch.equal(dev[0][0], dev[1][0])
+    assert [_enc_tuple(e) for e in qd.encoding] == [_enc_tuple(e) for e in qh.encoding]
