@@ -121,6 +121,8 @@ _SIGNATURES = {
     "miq_channel_analyzer_reset": ([_p, _p], _int),
     "miq_channel_analyzer_set_percentile": ([_p, _flt], _int),
     "miq_channel_analyzer_update_stats_f32": ([_p, _p, _i64, _i64, _p, _p], _int),
+    "miq_channel_analyzer_compute_encodings_device": ([_p, _int, _int, _int, _int, _p, _p, _p, _p, _p, _p, _p,
+                                                        C.POINTER(_int), _p], _int),
     "miq_channel_analyzer_compute_encodings": ([_p, _int, _int, _int, _int, _p, C.POINTER(_int), _p], _int),
     "miq_channel_analyzer_get_stats_histogram": ([_p, _i64, _p, _p, C.POINTER(_int), _p], _int),
     "miq_adaround_linear_workspace_bytes": ([_i64, _i64, _i64], _i64),

@@ -16,6 +16,7 @@
 // n_per_channel consecutive elements.  State (device memory handed in by the caller, or allocated here): one head
 // per channel, C x 512 running PDF values (double) and C x 512 counts of the batch in flight (uint32).
 #include "miq_common.h"
+#include "miq_encoding_math.h"
 #include "miq_fastmath.h"
 #include "miq_tfe_search.h"
 
@@ -335,6 +336,28 @@ struct miq_channel_analyzer
     bool stats_updated;
 };
 
+// Every channel's encoding as the search left it -> four doubles per channel for a later read-back, and the float32
+// parameters of the per-channel kernels (the number of steps follows channel 0's encoding).
+__global__ void chan_params_kernel(const miq_encoding* found, int64_t c, int bw, double* enc, float* omin, float* omax,
+                                   float* odelta, float* ooffset, float* raw_min, float* raw_max)
+{
+    const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= c)
+        return;
+    const miq_encoding e = found[i];
+    enc[4 * i + 0]       = e.min;
+    enc[4 * i + 1]       = e.max;
+    enc[4 * i + 2]       = e.delta;
+    enc[4 * i + 3]       = e.offset;
+    const ChannelKernelParams p = channel_kernel_params(e.min, e.max, found[0].min == -found[0].max, bw);
+    omin[i]    = p.min;
+    omax[i]    = p.max;
+    odelta[i]  = p.delta;
+    ooffset[i] = p.offset;
+    raw_min[i] = p.raw_min;
+    raw_max[i] = p.raw_max;
+}
+
 extern "C" {
 
 int64_t miq_channel_analyzer_state_bytes(int64_t num_channel)
@@ -511,6 +534,35 @@ int miq_channel_analyzer_compute_encodings(miq_channel_analyzer* a, int bw, int 
     // the kernel leaves the encodings in the caller's layout: one copy straight into `out`
     MIQ_CHECK_HIP(hipMemcpyAsync(out, a->st.enc, sizeof(miq_encoding) * c, hipMemcpyDeviceToHost, s));
     MIQ_CHECK_HIP(hipStreamSynchronize(s));
+    return MIQ_OK;
+}
+
+int miq_channel_analyzer_compute_encodings_device(miq_channel_analyzer* a, int bw, int use_symmetric,
+                                                  int use_strict_symmetric, int use_unsigned_symmetric, double* enc,
+                                                  float* out_min, float* out_max, float* out_delta, float* out_offset,
+                                                  float* raw_min, float* raw_max, int* is_valid, void* stream)
+{
+    MIQ_CHECK_ARG(a && enc && out_min && out_max && out_delta && out_offset && raw_min && raw_max && is_valid,
+                  "null argument");
+    MIQ_CHECK_ARG(bw >= 1 && bw <= 31, "bitwidth must be in [1, 31] (got %d)", bw);
+    if (a->mode == MIQ_QUANTIZATION_PERCENTILE)
+    {
+        set_error("the percentile analyzer computes its encodings on the host: use miq_channel_analyzer_compute_encodings");
+        return MIQ_ERR_UNSUPPORTED;
+    }
+    hipStream_t s   = (hipStream_t) stream;
+    const int64_t c = a->num_channel;
+    *is_valid       = a->stats_updated ? 1 : 0;
+    if (!a->stats_updated)
+        return MIQ_OK;
+    const tfe::SearchArgs sa =
+        tfe::make_search_args(bw, use_symmetric, use_strict_symmetric, use_unsigned_symmetric);
+    const int search_block = std::min(kSearchBlockMax, 64 * ((sa.n_cand + 63) / 64));
+    hipLaunchKernelGGL(chan_search_kernel, dim3((unsigned) c), dim3(search_block), 0, s, a->st, sa);
+    MIQ_CHECK_LAUNCH();
+    hipLaunchKernelGGL(chan_params_kernel, dim3((unsigned) ((c + 255) / 256)), dim3(256), 0, s, a->st.enc, c, bw, enc,
+                       out_min, out_max, out_delta, out_offset, raw_min, raw_max);
+    MIQ_CHECK_LAUNCH();
     return MIQ_OK;
 }
 

@@ -75,6 +75,36 @@ MIQ_ENC_HD inline EncodingD computed_encodings(int bw, double mn, double mx, boo
         e.max = fmax;
     return e;
 }
+#if defined(__HIPCC__)
+// The float32 parameters the per-channel kernels take, from a channel's encoding in double
+// (AimetTensorQuantizer::quantizeDequantizePerChannel, TrainingExtensions/torch/src/AimetTensorQuantizer.cpp:209-227,
+// 268-297, on float32(min), float32(max)): zero gated into the range, delta = (max - min) / steps, offset =
+// round-half-even(min / delta), with one step less iff channel 0's encoding has min == -max.
+struct ChannelKernelParams
+{
+    float min, max, delta, offset, raw_min, raw_max;
+};
+
+__device__ __forceinline__ ChannelKernelParams channel_kernel_params(double enc_min, double enc_max, bool first_is_symmetric,
+                                                                     int bw)
+{
+    ChannelKernelParams p;
+    const float num_steps = (float) (ldexp(1.0, bw) - 1.0 - (first_is_symmetric ? 1.0 : 0.0));
+    float lo = (float) enc_min, hi = (float) enc_max;
+    p.raw_min = lo;
+    p.raw_max = hi;
+    // torch.minimum / torch.maximum propagate NaN
+    lo        = (lo != lo) ? lo : fminf(lo, 0.f);
+    hi        = (hi != hi) ? hi : fmaxf(hi, 0.f);
+    float eps = lo + 1e-5f;
+    hi        = (hi != hi || eps != eps) ? (hi + eps) : fmaxf(hi, eps);
+    p.min     = lo;
+    p.max     = hi;
+    p.delta   = (hi - lo) / num_steps;
+    p.offset  = rintf(lo / p.delta);
+    return p;
+}
+#endif
 }   // namespace miq
 
 #endif

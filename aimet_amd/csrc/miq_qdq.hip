@@ -1008,25 +1008,18 @@ __global__ void tf_channel_encodings_kernel(const float* ch_min, const float* ch
     if (i >= c)
         return;
     const EncodingD first = tf_channel_encoding(ch_min[0], ch_max[0], bw, sym, strict, uns);
-    float num_steps       = (float) (ldexp(1.0, bw) - 1.0 - (first.min == -first.max ? 1.0 : 0.0));
     const EncodingD e     = tf_channel_encoding(ch_min[i], ch_max[i], bw, sym, strict, uns);
     enc[4 * i + 0]        = e.min;
     enc[4 * i + 1]        = e.max;
     enc[4 * i + 2]        = e.delta;
     enc[4 * i + 3]        = e.offset;
-    float lo = (float) e.min, hi = (float) e.max;
-    raw_min[i] = lo;
-    raw_max[i] = hi;
-    // as per_channel_params_kernel
-    lo        = (lo != lo) ? lo : fminf(lo, 0.f);
-    hi        = (hi != hi) ? hi : fmaxf(hi, 0.f);
-    float eps = lo + 1e-5f;
-    hi        = (hi != hi || eps != eps) ? (hi + eps) : fmaxf(hi, eps);
-    float d   = (hi - lo) / num_steps;
-    omin[i]   = lo;
-    omax[i]   = hi;
-    odelta[i] = d;
-    ooffset[i] = rintf(lo / d);
+    const ChannelKernelParams p = channel_kernel_params(e.min, e.max, first.min == -first.max, bw);
+    omin[i]    = p.min;
+    omax[i]    = p.max;
+    odelta[i]  = p.delta;
+    ooffset[i] = p.offset;
+    raw_min[i] = p.raw_min;
+    raw_max[i] = p.raw_max;
 }
 
 struct BcastArgs

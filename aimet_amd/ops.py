@@ -981,6 +981,21 @@ class ChannelAnalyzer(_StateOwner):
                                                              self._s()))
         return encs, bool(valid.value)
 
+    def compute_encodings_on_device(self, bw, symmetric=False, strict_symmetric=False, unsigned_symmetric=False):
+        """The search with its results left on the device: (enc, params) as tf_encodings_per_channel returns them, or
+        None when the analyzer has no statistics yet.  Nothing waits."""
+        c = self.num_channel
+        enc = torch.empty(c, 4, dtype=torch.float64, device=self.device)
+        outs = torch.empty(6, c, dtype=_F32, device=self.device)
+        valid = C.c_int(0)
+        with torch.cuda.device(self.device):
+            check(lib.miq_channel_analyzer_compute_encodings_device(
+                self._h, int(bw), int(bool(symmetric)), int(bool(strict_symmetric)), int(bool(unsigned_symmetric)),
+                _ptr(enc), *(_ptr(outs[k]) for k in range(6)), C.byref(valid), self._s()))
+        if not valid.value:
+            return None
+        return enc, tuple(outs[k] for k in range(6))
+
     def get_stats_histogram(self, channel):
         import numpy as np
         xl, pdf = np.zeros(_lib.PDF_SIZE), np.zeros(_lib.PDF_SIZE)

@@ -390,10 +390,7 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
 
     @staticmethod
     def _encoding_stamp(quantizer):
-        enc = quantizer.encoding
-        if isinstance(enc, (list, tuple)):
-            return (id(enc), len(enc), enc[0].min, enc[0].max, enc[-1].min, enc[-1].max, enc[0].bw)
-        return (id(enc), enc.min, enc.max, enc.bw)
+        return quantizer.encoding_stamp()
 
     def _param_cache_key(self, param, quantizer):
         return (param.data_ptr(), param._version, param.dtype, tuple(param.shape), quantizer.bitwidth,  # pylint: disable=protected-access
@@ -431,7 +428,7 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
         ahead = self.__dict__.setdefault('_param_encodings_ahead', {})
         for name, param in self.get_named_parameters():
             quantizer = self.param_quantizers[name]
-            if quantizer.enabled and quantizer.bitwidth != 32 and quantizer.encoding is None and param.is_cuda:
+            if quantizer.enabled and quantizer.bitwidth != 32 and not quantizer.has_encoding() and param.is_cuda:
                 self._observe_param(quantizer, param)
                 ahead[name] = self._param_identity(param)
                 fed.append(quantizer)
@@ -454,10 +451,10 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
                 # in training mode the parameter encodings are recomputed in every pass
                 ahead = self.__dict__.get('_param_encodings_ahead')
                 stale = ahead is not None and ahead.pop(name, None) not in (None, self._param_identity(param))
-                if self._module_to_wrap.training or quantizer.encoding is None or stale:
+                if self._module_to_wrap.training or not quantizer.has_encoding() or stale:
                     self._observe_param(quantizer, param)
                     quantizer.compute_encoding()
-                if keep and quantizer.encoding is not None:
+                if keep and quantizer.has_encoding():
                     key = self._param_cache_key(param, quantizer)
                     kept = cache.get(name)
                     if kept is None or kept[0] != key:

@@ -497,7 +497,7 @@ class QuantizationSimModel:
                 continue
             for name, param in layer.get_named_parameters():
                 quantizer = layer.param_quantizers[name]
-                if not (quantizer.enabled and quantizer.bitwidth != 32 and quantizer.encoding is not None and
+                if not (quantizer.enabled and quantizer.bitwidth != 32 and quantizer.has_encoding() and
                         quantizer.data_type == QuantizationDataType.int and param.is_cuda and
                         param.dtype in (torch.float32, torch.bfloat16) and param.data.is_contiguous()):
                     continue

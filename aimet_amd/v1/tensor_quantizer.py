@@ -88,16 +88,33 @@ class StaticGridTensorQuantizer(TensorQuantizer):
         if pending is not None:
             self.__dict__['_pending_encoding'] = None
             self.__dict__['_encoding_list'] = pending()
+            computed_from = self.__dict__.get('_computed_from')
+            if computed_from is not None and computed_from[1] is pending:
+                self.__dict__['_computed_from'] = (computed_from[0], self.__dict__['_encoding_list'])
         return self.__dict__.get('_encoding_list')
 
     @_encoding.setter
     def _encoding(self, value):
         self.__dict__['_pending_encoding'] = None
         self.__dict__['_encoding_list'] = value
+        self.__dict__['_encoding_serial'] = self.__dict__.get('_encoding_serial', 0) + 1
 
     def _has_encoding(self) -> bool:
         """bool(self._encoding) without building the list."""
         return self.__dict__.get('_pending_encoding') is not None or bool(self.__dict__.get('_encoding_list'))
+
+    has_encoding = _has_encoding
+
+    def encoding_stamp(self):
+        """Changes whenever the encoding does: a count of assignments, plus, where the list exists, the bounds at both
+        of its ends (an encoding object edited in place).  Does not build the list."""
+        serial = self.__dict__.get('_encoding_serial', 0)
+        if self.__dict__.get('_pending_encoding') is not None:
+            return ('on device', serial)
+        enc = self.__dict__.get('_encoding_list')
+        if not enc:
+            return (None, serial)
+        return (id(enc), serial, len(enc), enc[0].min, enc[0].max, enc[-1].min, enc[-1].max, enc[0].bw)
 
     # ---- 8-bit float grid (reference tensor_quantizer.py:393-400, :461-468, :544-552; fp_quantization.py:45-122)
     @property
@@ -231,8 +248,8 @@ class StaticGridTensorQuantizer(TensorQuantizer):
             # parameter (once when the first forward needs the encoding, once at the end of compute_encodings), and
             # a per-channel answer costs a search launch, a read-back and thousands of encoding objects
             recipe, result = self.__dict__.get('_computed_from') or (None, None)
-            if result is not None and result is self.__dict__.get('_encoding_list') and result and \
-                    recipe == self._encoding_recipe():
+            current = self.__dict__.get('_pending_encoding') or self.__dict__.get('_encoding_list')
+            if result is not None and result is current and recipe == self._encoding_recipe():
                 return
             self._encoding = []
             self._dev_params = None
@@ -248,6 +265,7 @@ class StaticGridTensorQuantizer(TensorQuantizer):
             if callable(computed):
                 # every channel's encoding exists, on the device: the list is built when it is first read
                 self.__dict__['_pending_encoding'] = computed
+                self.__dict__['_encoding_serial'] = self.__dict__.get('_encoding_serial', 0) + 1
             else:
                 for encoding, valid in computed:
                     if not valid:
@@ -258,10 +276,8 @@ class StaticGridTensorQuantizer(TensorQuantizer):
                 all(enc.min >= 0 and enc.max >= 0 for enc in self._encoding)
             assert not (not self.enabled and self._has_encoding()), \
                 'At least one encoding for a multi-encoding quantizer is invalid.'
-            if self.__dict__.get('_pending_encoding') is None:
-                self.__dict__['_computed_from'] = (self._encoding_recipe(), self._encoding) if self.enabled else None
-            else:
-                self.__dict__['_computed_from'] = None
+            current = self.__dict__.get('_pending_encoding') or self.__dict__.get('_encoding_list')
+            self.__dict__['_computed_from'] = (self._encoding_recipe(), current) if self.enabled and current else None
 
     def _compute_op_encodings(self):
         return [op.getEncoding(self.bitwidth, self.use_symmetric_encodings, self.use_strict_symmetric,
@@ -446,6 +462,11 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
 
     def _compute_op_encodings(self):
         if self._channel_analyzer is not None:
+            if self.compute_tf_encodings_on_device and self._quant_scheme == QuantScheme.post_training_tf_enhanced:
+                found = self._channel_analyzer.compute_encodings_on_device(
+                    self.bitwidth, self.use_symmetric_encodings, self.use_strict_symmetric, self.use_unsigned_symmetric)
+                if found is not None:
+                    return self._encodings_left_on_device(*found)
             encodings, valid = self._channel_analyzer.compute_encodings(
                 self.bitwidth, self.use_symmetric_encodings, self.use_strict_symmetric, self.use_unsigned_symmetric)
             return [(libpymo.TfEncoding(e.min, e.max, e.delta, e.offset, e.bw), valid) for e in encodings]
@@ -465,15 +486,20 @@ class StaticGridPerChannelQuantizer(StaticGridTensorQuantizer):
             out.append((libpymo.TfEncoding(e.min, e.max, e.delta, e.offset, e.bw), True))
         return out
 
-    # The TF (min / max) encodings of all channels from one launch, left on the device, instead of one read-back and
-    # one host computation per channel (thousands per layer, in every forward of a wrapper in training mode).  The
-    # numbers are the same: the kernel runs the host recipe's double arithmetic.  False: always the host path.
+    # The encodings of all channels (TF: min / max; TF-Enhanced: the per-channel search) from one launch, left on the
+    # device, instead of one read-back and one host computation or object per channel (thousands per layer, in every
+    # forward of a wrapper in training mode).  The numbers are the same: the min / max kernel runs the host recipe's
+    # double arithmetic, the search is the one the host path reads back.  False: always the host path.
     compute_tf_encodings_on_device = True
 
     def _tf_encodings_on_device(self):
         mm = self._tf_minmax.to(torch.float32).contiguous()
-        enc, params = ops.tf_encodings_per_channel(mm, self.bitwidth, self.use_symmetric_encodings,
-                                                   self.use_strict_symmetric, self.use_unsigned_symmetric)
+        return self._encodings_left_on_device(*ops.tf_encodings_per_channel(
+            mm, self.bitwidth, self.use_symmetric_encodings, self.use_strict_symmetric, self.use_unsigned_symmetric))
+
+    def _encodings_left_on_device(self, enc, params):
+        """Takes the kernel parameters as they are and returns the builder of the TfEncoding list for
+        compute_encoding(): one read-back of [C, 4] doubles when the list is first wanted."""
         self._dev_params = params
         bitwidth = self.bitwidth
 

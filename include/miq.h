@@ -423,6 +423,17 @@ int miq_channel_analyzer_compute_encodings(miq_channel_analyzer* a, int bw, int 
                                            int use_strict_symmetric, int use_unsigned_symmetric,
                                            miq_encoding* out /* host[num_channel] */, int* is_valid /* host */,
                                            void* stream);
+/* The same search with the results left on the device, for a caller that only quantizes with them: enc receives
+ * (min, max, delta, offset) of every channel's TfEncoding as device double[num_channel][4], the six device
+ * float[num_channel] vectors the kernel parameters of miq_per_channel_params_f32 and float32(min), float32(max) (the
+ * straight-through bounds).  Nothing waits.  *is_valid = 0 (and nothing is written) while no statistics were supplied.
+ * MIQ_ERR_UNSUPPORTED for the percentile analyzer, whose encodings are host arithmetic.  No counterpart in the
+ * reference. */
+int miq_channel_analyzer_compute_encodings_device(miq_channel_analyzer* a, int bw, int use_symmetric,
+                                                  int use_strict_symmetric, int use_unsigned_symmetric,
+                                                  double* enc, float* out_min, float* out_max, float* out_delta,
+                                                  float* out_offset, float* raw_min, float* raw_max,
+                                                  int* is_valid /* host */, void* stream);
 int miq_channel_analyzer_get_stats_histogram(miq_channel_analyzer* a, int64_t channel, double* x_left /* host[512] */,
                                              double* pdf /* host[512] */, int* num_buckets /* host */, void* stream);
 

@@ -533,3 +533,31 @@ def test_training_mode_wrapper_recomputes_parameter_encodings_on_the_device(api)
         assert torch.equal(a[2] == 0, b[2] == 0)
     assert not torch.equal(dev[0][0], dev[1][0])
     assert [_enc_tuple(e) for e in qd.encoding] == [_enc_tuple(e) for e in qh.encoding]
+
+
+@pytest.mark.parametrize("bw,sym", [(8, True), (4, True), (8, False)])
+def test_per_channel_tf_enhanced_encodings_stay_on_the_device(api, bw, sym):
+    """The per-channel TF-Enhanced search leaves its encodings on the device as well: same encodings, parameters and
+    quantized values as with the read-back per call; a quantizer without statistics still ends up disabled."""
+    rng = np.random.default_rng(23)
+    w = torch.from_numpy((rng.laplace(0, 0.03, (40, 300))).astype(np.float32)).cuda()
+
+    def make(on_device, feed=True):
+        q = api.tq.StaticGridPerChannelQuantizer(bw, api.nearest, api.QuantScheme.post_training_tf_enhanced, sym, 40,
+                                                 enabled_by_default=True, ch_axis=0)
+        q.compute_tf_encodings_on_device = on_device
+        if feed:
+            q.update_encoding_stats(w)
+            q.update_encoding_stats(w * 1.5)
+        q.compute_encoding()
+        return q
+
+    dev, host = make(True), make(False)
+    assert dev.__dict__.get('_pending_encoding') is not None and host.__dict__.get('_pending_encoding') is None
+    for a, b in zip(dev.device_params(w.device), host.device_params(w.device)):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    assert torch.equal(dev.quantize_dequantize(w, api.nearest), host.quantize_dequantize(w, api.nearest))
+    assert dev.__dict__.get('_pending_encoding') is not None
+    assert [_enc_tuple(e) for e in dev.encoding] == [_enc_tuple(e) for e in host.encoding]
+    empty = make(True, feed=False)
+    assert not empty.enabled and not empty.encoding
