@@ -356,3 +356,83 @@ def test_per_channel_fused_statistics_go_with_the_scheme():
     q._tf_minmax = stale                                    # pylint: disable=protected-access
     q.reset_encoding_stats()
     assert q._tf_minmax is None                             # pylint: disable=protected-access
+
+
+def test_encoding_list_built_on_first_read():
+    """A quantizer whose encodings were computed on the device holds a builder until the list is read: asking whether
+    an encoding exists, or for its stamp, does not run the builder; reading does, once; assigning drops it; pickling
+    carries the list."""
+    import pickle
+    from aimet_amd.common import libpymo
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.tensor_quantizer import StaticGridPerChannelQuantizer
+    q = StaticGridPerChannelQuantizer(8, libpymo.RoundingMode.ROUND_NEAREST, QuantScheme.post_training_tf, True, 3,
+                                      enabled_by_default=True)
+    assert not q.has_encoding() and q.encoding is None
+    built = []
+
+    def builder():
+        built.append(1)
+        return [libpymo.TfEncoding(-1.0 - c, 1.0 + c, 0.01, -128, 8) for c in range(3)]
+    q.__dict__['_pending_encoding'] = builder
+    stamp = q.encoding_stamp()
+    assert q.has_encoding() and stamp[0] == 'on device' and built == []
+    enc = q.encoding
+    assert built == [1] and len(enc) == 3 and q.encoding is enc and built == [1]
+    assert q.encoding_stamp() != stamp and q.encoding_stamp()[0] == id(enc)
+    serial = q.__dict__['_encoding_serial']
+    q.encoding = enc[:2]
+    assert q.__dict__['_encoding_serial'] == serial + 1 and len(q.encoding) == 2
+    q.__dict__['_pending_encoding'] = builder
+    clone = pickle.loads(pickle.dumps(q))
+    assert [e.max for e in clone.encoding] == [1.0, 2.0, 3.0] and clone.__dict__.get('_pending_encoding') is None
+    q.__dict__['_pending_encoding'] = builder
+    q.encoding = None                                              # an assignment wins over what was pending
+    assert not q.has_encoding() and q.encoding is None
+
+
+def test_v2_range_warnings_one_by_one_and_batched():
+    """The warnings about non-finite or extreme ranges (reference encoding_analyzer.py:388-395) are the same whether a
+    quantizer checks its own range at once or many of them are examined together at the end."""
+    import warnings
+    from aimet_amd.v2.quantization.affine import quantizer as qz
+    fine = (torch.tensor([-1.0, -2.0]), torch.tensor([1.0, 2.0]))
+    nan = (torch.tensor([float('nan')]), torch.tensor([1.0]))
+    huge = (torch.tensor([-1.0]), torch.tensor([torch.finfo(torch.float32).max * 0.97]))
+
+    def messages(fn):
+        with warnings.catch_warnings(record=True) as caught:
+            warnings.simplefilter("always")
+            fn()
+        return sorted(str(w.message)[:8] for w in caught)
+
+    assert messages(lambda: qz._flag_extreme_min_max(*fine)) == []
+    assert messages(lambda: qz._flag_extreme_min_max(*nan)) == ['Infinite']
+    assert messages(lambda: qz._flag_extreme_min_max(*huge)) == ['Extreme ']
+    # torch's own formulation of the same two tests
+    for mn, mx in (fine, nan, huge):
+        extreme = torch.full_like(mn, torch.finfo(mn.dtype).max)
+        want_extreme = bool(torch.any(torch.isclose(mn.abs(), extreme, rtol=0.05)) or
+                            torch.any(torch.isclose(mx.abs(), extreme, rtol=0.05)))
+        want_bad = not bool(torch.all(torch.isfinite(mn)) and torch.all(torch.isfinite(mx)))
+        got = messages(lambda: qz._flag_extreme_min_max(mn, mx))
+        assert ('Extreme ' in got) == want_extreme and ('Infinite' in got) == want_bad
+
+    def batched():
+        with qz.batched_range_checks():
+            for pair in (fine, nan, fine, huge):
+                qz._flag_extreme_min_max(*pair)
+            assert qz._pending_range_checks and len(qz._pending_range_checks) == 4      # held back
+    assert messages(batched) == ['Extreme ', 'Infinite']
+    assert qz._pending_range_checks is None
+
+
+def test_v2_grid_representability_is_memoised():
+    from aimet_amd.v2.quantization.affine.backends import hip_gfx950 as backend
+    backend._is_grid_representable.cache_clear()
+    assert backend._is_grid_representable(torch.float32, -128, 127)
+    assert backend._is_grid_representable(torch.float32, -128, 127)
+    assert backend._is_grid_representable.cache_info().hits == 1
+    assert not backend._is_grid_representable(torch.float16, 0, 2 ** 16 - 1)      # 65535 is not a float16
+    assert backend._is_grid_representable(torch.bfloat16, -128, 127)
+    assert not backend._is_grid_representable(torch.bfloat16, 0, 2 ** 9 - 1)       # 511 needs nine bits
