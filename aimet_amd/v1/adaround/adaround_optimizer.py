@@ -134,20 +134,28 @@ class AdaroundOptimizer:
             qm.alpha.grad = grad_alpha
             return exp_avg, exp_avg_sq
 
+        # the batch indices of all iterations in one host-to-device copy (one copy per iteration waits for the device
+        # every time); ragged batches (a caller's own) keep their own copies
+        same_size = all(b.numel() == batches[0].numel() for b in batches)
+        index_dev = torch.stack(batches).to(device) if same_size else None
+        explicit = cls.use_explicit_gradient and activation is not None and cls._explicit_gradient_applies(module)
         for k, indices in enumerate(batches):
-            indices = indices.to(device)
+            indices = index_dev[k] if index_dev is not None else indices.to(device)
             inp_data = all_inp_data[indices]
             orig_out_data = all_orig_out_data[indices]
 
             ada_weight = ops.adaround_soft_round(weight, alpha, qm.num_channel, qm.n_per_channel, qm.delta, qm.offset,
                                                  qm.clip_min, qm.clip_max, True)
-            ada_weight.requires_grad_(True)
-            quant_out_data = cls._layer_output(module, inp_data, ada_weight)
-            if act_func is not None:
-                orig_out_data = act_func(orig_out_data)
-                quant_out_data = act_func(quant_out_data)
-            recon_loss = AdaroundLoss.compute_recon_loss(quant_out_data, orig_out_data)
-            grad_weight, = torch.autograd.grad(recon_loss, ada_weight)
+            if explicit:
+                grad_weight = cls._recon_loss_weight_gradient(module, inp_data, orig_out_data, ada_weight, activation)
+            else:
+                ada_weight.requires_grad_(True)
+                quant_out_data = cls._layer_output(module, inp_data, ada_weight)
+                if act_func is not None:
+                    orig_out_data = act_func(orig_out_data)
+                    quant_out_data = act_func(quant_out_data)
+                recon_loss = AdaroundLoss.compute_recon_loss(quant_out_data, orig_out_data)
+                grad_weight, = torch.autograd.grad(recon_loss, ada_weight)
             ops.adaround_bwd_adam(weight, grad_weight.contiguous(), alpha, exp_avg, exp_avg_sq, qm.num_channel,
                                   qm.n_per_channel, qm.delta, qm.offset, qm.clip_min, qm.clip_max,
                                   opt_params.reg_param, beta_of(first_iteration + k), ADAM_LR, ADAM_BETAS[0],
@@ -155,6 +163,38 @@ class AdaroundOptimizer:
                                   grad_alpha=grad_alpha if k == len(batches) - 1 else None)
         qm.alpha.grad = grad_alpha
         return exp_avg, exp_avg_sq
+
+    # For Conv2d and Linear with no activation or ReLU the gradient of the reconstruction loss w.r.t. the soft-rounded
+    # weight is written out -- dLoss/dout = 2 (act(out) - act(target)) act'(out) / (elements per channel), then the
+    # layer's own weight-gradient routine -- instead of recorded and replayed by autograd: the same operations on the
+    # same numbers (torch's backward of square / sum / mean / relu / convolution performs exactly these), without the
+    # graph and the engine's hand-over, which at 32 samples per iteration cost more than the kernels.  False: autograd.
+    use_explicit_gradient = True
+
+    @staticmethod
+    def _explicit_gradient_applies(module) -> bool:
+        if isinstance(module, torch.nn.Linear):
+            return True
+        return isinstance(module, torch.nn.Conv2d) and isinstance(module.padding, tuple) and \
+            module.padding_mode == 'zeros'
+
+    @classmethod
+    @torch.no_grad()
+    def _recon_loss_weight_gradient(cls, module, inp_data, orig_out_data, ada_weight, activation):
+        out = cls._layer_output(module, inp_data, ada_weight)
+        if activation == 1:
+            quant_act, orig_act = torch.relu(out), torch.relu(orig_out_data)
+        else:
+            quant_act, orig_act = out, orig_out_data
+        # compute_recon_loss: squared error summed over dim 1, mean over the rest
+        grad_out = (quant_act - orig_act) * (2.0 / (out.numel() // out.shape[1]))
+        if activation == 1:
+            grad_out = grad_out * (quant_act > 0)              # relu's backward: the gradient where its result is positive
+        if isinstance(module, torch.nn.Linear):
+            return grad_out.reshape(-1, grad_out.shape[-1]).t().mm(inp_data.reshape(-1, inp_data.shape[-1]))
+        return torch.ops.aten.convolution_backward(
+            grad_out, inp_data, ada_weight, None, list(module.stride), list(module.padding), list(module.dilation),
+            False, [0, 0], module.groups, (False, True, False))[1]
 
     @staticmethod
     def _fused_activation_code(act_func):

@@ -518,6 +518,42 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
                          "loop_ms_per_iteration_general": loops["general"]})
     res["rows_per_iteration"] = per_rows
 
+    # convolution layers take the general path (soft-rounding kernel, torch's convolution and its weight gradient, fused
+    # backward / Adam kernel): the iteration with the loss gradient written out against autograd's recording of it
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.adaround.adaround_wrapper import AdaroundWrapper
+    from aimet_amd.v1.qc_quantize_op import StaticGridQuantWrapper
+    conv_rows = []
+    for cin, cout, ksize, hw in ((256, 256, 3, 14), (512, 512, 3, 7), (1024, 256, 1, 14), (64, 64, 3, 56)):
+        torch.manual_seed(1005)
+        conv = torch.nn.Conv2d(cin, cout, ksize, padding=ksize // 2, bias=False).to(w.device)
+        xc = torch.randn(256, cin, hw, hw, device=w.device)
+        with torch.no_grad():
+            yc = conv(xc)
+        qw = StaticGridQuantWrapper(conv, 4, 8, round_mode='nearest', quant_scheme=QuantScheme.post_training_tf,
+                                    is_symmetric=True)
+        qw.enable_per_channel_quantization()
+        qw.param_quantizers['weight'].update_encoding_stats(conv.weight.data)
+        qw.param_quantizers['weight'].compute_encoding()
+        layer = AdaroundWrapper(qw)
+        row = {"conv": [cout, cin, ksize, ksize], "input": [32, cin, hw, hw]}
+        n_it = min(200, iterations)
+        hp = AdaroundHyperParameters(n_it, 0.01, (20, 2), 0.2)
+        for name, explicit in (("ms_per_iteration", True), ("ms_per_iteration_through_autograd", False)):
+            AdaroundOptimizer.use_explicit_gradient = explicit
+            alpha0 = layer.alpha.data.clone()
+            AdaroundOptimizer.optimize_rounding_on_cached_acts(layer, torch.relu, xc, yc,
+                                                               AdaroundHyperParameters(10, 0.01, (20, 2), 0.2))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            AdaroundOptimizer.optimize_rounding_on_cached_acts(layer, torch.relu, xc, yc, hp)
+            torch.cuda.synchronize()
+            row[name] = (time.perf_counter() - t0) * 1e3 / n_it
+            layer.alpha.data.copy_(alpha0)
+        AdaroundOptimizer.use_explicit_gradient = True
+        conv_rows.append(row)
+    res["convolution_layers_general_path"] = conv_rows
+
     # the GEMM-bound variant: every iteration uses all 2048 cached rows.  The fused kernels are built for the
     # reference's batch of 32 (the weight-shaped traffic dominates there); a batch of 2048 goes through the general
     # path: soft-rounding kernel, torch's GEMMs (hipBLASLt) for the layer and its weight gradient, fused

@@ -536,6 +536,46 @@ def test_fused_path_for_more_rows_and_1x1_convolutions(ops, kind, shape, pixels,
             assert _close_except_few(got, want, atol=1e-4 * scale.abs().max().item(), rtol=1e-3)
 
 
+@pytest.mark.parametrize("kind,shape,conv_args,act", [
+    ("conv2d", (8, 6, 3, 3), {"padding": 1}, torch.relu), ("conv2d", (8, 6, 3, 3), {"padding": 1, "stride": 2}, None),
+    ("conv2d", (8, 4, 3, 3), {"padding": 2, "dilation": 2, "groups": 2}, torch.relu), ("linear", (48, 64), {}, torch.relu),
+    ("linear", (48, 64), {}, None)])
+def test_written_out_gradient_equals_autograd(ops, kind, shape, conv_args, act, monkeypatch):
+    """The general path forms dLoss/dW' of the reconstruction loss by hand for Conv2d / Linear with no activation or
+    ReLU.  Same trajectory as with autograd's recording of the same operations (to the summation order of the
+    convolution's weight-gradient kernel), and both against the CPU restatement."""
+    from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
+    iters = 25
+    hyper = (iters, 0.01, (20, 2), 0.2)
+    torch.manual_seed(71)
+    cin = shape[1] * conv_args.get("groups", 1)
+    all_inp = torch.randn(96, cin, 9, 9) if kind == "conv2d" else torch.randn(96, shape[1])
+    weight, delta, offset, C, npc, cmin, cmax = _case(73, shape, 0, True)
+    alpha0 = ada.generate_alpha(weight, ada.broadcast(delta, weight, 0))
+    all_out = ada.layer_output(kind, all_inp, weight, **conv_args)
+    all_out = all_out + 0.02 * torch.randn_like(all_out)
+    batches = [torch.randperm(96)[:32] for _ in range(iters)]
+    monkeypatch.setattr(AdaroundOptimizer, "use_fused_linear", False)
+    calls = []
+    real = AdaroundOptimizer._recon_loss_weight_gradient.__func__
+    monkeypatch.setattr(AdaroundOptimizer, "_recon_loss_weight_gradient",
+                        classmethod(lambda cls, *a: (calls.append(1), real(cls, *a))[1]))
+    run = lambda: _run_product_loop(kind, weight, alpha0, delta, offset, C, npc, cmin, cmax, all_inp, all_out, batches,
+                                    hyper, act, conv_args)
+    a, m, v, g = run()
+    assert len(calls) == iters
+    monkeypatch.setattr(AdaroundOptimizer, "use_explicit_gradient", False)
+    a2, m2, v2, g2 = run()
+    assert len(calls) == iters
+    assert _close_except_few(a, a2, atol=5e-5) and (a - a2).abs().max() < 5e-3
+    assert _close_except_few(g, g2, atol=1e-5 * g2.abs().max().item(), rtol=1e-4)
+    assert _close_except_few(m, m2, atol=1e-5 * m2.abs().max().item(), rtol=1e-4)
+    a_ref, m_ref, v_ref, g_ref = ada.optimize_rounding(kind, weight, alpha0, delta, offset, cmin, cmax, all_inp,
+                                                       all_out, batches, *hyper, act=act, conv_args=conv_args)
+    assert _close_except_few(a, a_ref, atol=5e-5) and (a - a_ref).abs().max() < 5e-3
+    assert _close_except_few(g, g_ref, atol=1e-4 * g_ref.abs().max().item(), rtol=1e-3)
+
+
 def test_fused_path_leaves_other_convolutions_alone(ops, monkeypatch):
     """A 3x3 kernel, a stride, a padding, groups, a row count that is not 32 / 64 / 128 / 256: the unfused path."""
     from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
