@@ -30,6 +30,10 @@ class AdaroundOptimizer:
     # 32 / 64 / 128 / 256 rows per iteration, no activation or ReLU) use them; everything else runs soft-round kernel +
     # torch layer + fused backward/Adam kernel
     use_fused_linear = True
+    # rows per iteration up to which the fused kernels are the faster path: on a [4096, 4096] layer they take 0.105 /
+    # 0.136 / 0.188 / 0.321 ms per iteration at 32 / 64 / 128 / 256 rows against 0.170 / 0.186 / 0.236 / 0.289 ms for
+    # the general path (the kernels themselves take up to 256)
+    fused_rows_limit = 128
     use_int8_floor = True    # store floor(W / delta) as int8 / int16 for the fused Linear path when the grid allows it
 
     @classmethod
@@ -212,9 +216,11 @@ class AdaroundOptimizer:
         They take a Linear layer on 2-D activations, and a Conv2d with a 1x1 kernel, unit stride, no padding and one
         group, which is the same contraction over the channels for every pixel (the reference calls functional.conv2d
         there, :268-272): its rows are the pixels, read from channels-last copies of the cached activations that are
-        made once per layer.  The rows of an iteration -- batch entries times pixels -- must be 32, 64, 128 or 256."""
+        made once per layer.  The rows of an iteration -- batch entries times pixels -- must be 32, 64 or 128 (256, which
+        the kernels also take, is faster through the general path: fused_rows_limit)."""
         if not batches or any(b.numel() != batches[0].numel() for b in batches):
             return None
+        limit = AdaroundOptimizer.fused_rows_limit
         out_features, in_features = weight.shape[:2]
         per_channel_ok = qm.num_channel == 1 or (qm.num_channel == out_features and qm.n_per_channel == in_features)
         if not per_channel_ok or all_inp_data.dtype != torch.float32 or all_orig_out_data.dtype != torch.float32:
@@ -232,7 +238,8 @@ class AdaroundOptimizer:
                     all_inp_data.shape[2:] != all_orig_out_data.shape[2:]:
                 return None
             pixels = all_inp_data.shape[2] * all_inp_data.shape[3]
-            if not ops.adaround_linear_supported(out_features, in_features, batches[0].numel() * pixels):
+            rows = batches[0].numel() * pixels
+            if rows > limit or not ops.adaround_linear_supported(out_features, in_features, rows):
                 return None             # before anything is copied
             x_rows = all_inp_data.permute(0, 2, 3, 1).reshape(-1, in_features).contiguous()
             y_rows = all_orig_out_data.permute(0, 2, 3, 1).reshape(-1, out_features).contiguous()
@@ -241,7 +248,8 @@ class AdaroundOptimizer:
         if x_rows.size(1) != in_features or y_rows.size(1) != out_features:
             return None
         data_ok = all(t.stride(1) == 1 and t.stride(0) % 4 == 0 and t.data_ptr() % 16 == 0 for t in (x_rows, y_rows))
-        if data_ok and ops.adaround_linear_supported(out_features, in_features, batches[0].numel() * pixels):
+        rows = batches[0].numel() * pixels
+        if data_ok and rows <= limit and ops.adaround_linear_supported(out_features, in_features, rows):
             return x_rows, y_rows, pixels
         return None
 

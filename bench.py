@@ -501,6 +501,7 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
         n_it = min(200, iterations)
         for name, fused in (("fused", True), ("general", False)):
             AdaroundOptimizer.use_fused_linear = fused
+            AdaroundOptimizer.fused_rows_limit = 256      # (the optimizer's own choice stops at 128 rows)
             alpha0 = wrapper.alpha.data.clone()
             bl = [idx_r[i % timed_kernel_iters] for i in range(n_it)]
             AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, x, y, params, batches=bl[:10])
@@ -511,6 +512,7 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
             loops[name] = (time.perf_counter() - t0) * 1e3 / n_it
             wrapper.alpha.data.copy_(alpha0)
         AdaroundOptimizer.use_fused_linear = True
+        AdaroundOptimizer.fused_rows_limit = 128
         per_rows.append({"rows": rows_it, "fwd_ms": f_r, "bwd_ms": b_r,
                          "fwd_GBps_moved": (fb + 4) * n / f_r / 1e6, "bwd_GBps_moved": (fb + 24) * n / b_r / 1e6,
                          "fwd_mfma_TFLOPs": 2.0 * rows_it * n / f_r / 1e9, "bwd_mfma_TFLOPs": 2.0 * rows_it * n / b_r / 1e9,

@@ -519,9 +519,15 @@ def test_fused_path_for_more_rows_and_1x1_convolutions(ops, kind, shape, pixels,
     calls = []
     real = ops.adaround_linear_fwd
     monkeypatch.setattr(ops, "adaround_linear_fwd", lambda *a, **k: (calls.append(a[13].shape), real(*a, **k))[1])
+    rows = batch * (pixels[0] * pixels[1] if pixels else 1)
+    if rows > AdaroundOptimizer.fused_rows_limit:
+        # 256 rows go through the general path by default (it is the faster one there); the kernels take them
+        a, _, _, _ = _run_product_loop(kind, weight, alpha0, delta, offset, C, npc, cmin, cmax, all_inp, all_out,
+                                       batches[:2], hyper, act, {})
+        assert calls == []
+        monkeypatch.setattr(AdaroundOptimizer, "fused_rows_limit", 256)
     a, m, v, g = _run_product_loop(kind, weight, alpha0, delta, offset, C, npc, cmin, cmax, all_inp, all_out,
                                    batches, hyper, act, {})
-    rows = batch * (pixels[0] * pixels[1] if pixels else 1)
     assert calls == [(rows, shape[0])] * iters            # the fused path ran, on that many rows
     monkeypatch.setattr(AdaroundOptimizer, "use_fused_linear", False)
     a_u, m_u, v_u, g_u = _run_product_loop(kind, weight, alpha0, delta, offset, C, npc, cmin, cmax, all_inp, all_out,
