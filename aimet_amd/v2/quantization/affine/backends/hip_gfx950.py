@@ -182,6 +182,13 @@ def quantize(tensor: torch.Tensor, scale: torch.Tensor, offset: torch.Tensor, qm
 def quantize_dequantize(tensor: torch.Tensor, scale: torch.Tensor, offset: torch.Tensor, qmin: int, qmax: int,
                         block_size: Optional[List] = None) -> torch.Tensor:
     """Differentiable quantize-dequantize (fake quantization)."""
+    if block_size is None and not torch.is_grad_enabled() and scale.numel() == 1 and offset.numel() == 1 and \
+            tensor.is_cuda and tensor.dtype in (torch.float32, torch.bfloat16) and tensor.is_contiguous() and \
+            tensor.numel() > 0 and scale.device == tensor.device and offset.device == tensor.device and qmin <= qmax and \
+            _is_grid_representable(torch.float32, qmin, qmax):
+        # inference with one scale for the whole tensor (every activation quantizer): none of the re-layout below has
+        # anything to do, and every check it makes has just been made
+        return ops.v2_qdq(tensor, 1, tensor.numel(), scale, offset, qmin, qmax)
     _validate_arguments(tensor, scale, offset, qmin, qmax, block_size)
     if not _is_grid_representable(torch.float32, qmin, qmax):
         raise RuntimeError(f"{torch.float32} is unable to represent quantized output of range [{qmin}, {qmax}].")
