@@ -403,6 +403,13 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
     def invalidate_param_cache(self):
         self.__dict__['_param_cache'] = {}
 
+    def __getstate__(self):
+        # what is kept between forwards is not part of a saved or copied wrapper
+        state = self.__dict__.copy()
+        state.pop('_param_cache', None)
+        state.pop('_param_encodings_ahead', None)
+        return state
+
     @staticmethod
     def _observe_param(quantizer, param):
         """The statistics of a parameter quantizer are those of the parameter as it is now (reference :769-777)."""

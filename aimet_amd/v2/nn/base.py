@@ -51,6 +51,12 @@ class BaseQuantizationMixin:
     # counter: set `keep_quantized_parameters = False` on the module (or the class) around them.
     keep_quantized_parameters = True
 
+    def __getstate__(self):
+        # what is kept between forwards is not part of a saved or copied module
+        state = self.__dict__.copy()
+        state.pop('_kept_quantized_parameters', None)
+        return state
+
     def _kept_parameter_key(self, param, quantizer):
         if not self.keep_quantized_parameters or self.training or torch.is_grad_enabled() or \
                 not isinstance(quantizer, MinMaxQuantizer) or 'forward' in quantizer.__dict__:

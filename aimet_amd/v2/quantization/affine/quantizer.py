@@ -227,6 +227,7 @@ class MinMaxQuantizer(nn.Module):
     def __getstate__(self):
         state = self.__dict__.copy()
         state['_initial_parameters'] = {name: self._is_initialized(name) for name in ('min', 'max')}
+        state.pop('_kept_encoding', None)
         return state
 
     def __setstate__(self, state):
