@@ -603,3 +603,34 @@ def test_copies_and_pickles_do_not_carry_what_is_kept_between_forwards():
                 assert module.__dict__.get('_kept_encoding') is None
             with torch.no_grad():
                 assert torch.equal(clone(x), want)
+
+
+def test_v2_simulation_forward_in_a_hip_graph():
+    """Inference through the v2 simulation model waits for nothing once scale / offset, the quantized parameters and
+    the "grid starts at zero" answers are kept (the warm-up passes fill them): it can be captured and replayed.
+    Replays are interleaved with eager work and synchronisations and each one is checked against the eager result."""
+    from aimet_amd.v2.quantsim import QuantizationSimModel
+    torch.manual_seed(12)
+    model = nn.Sequential(nn.Linear(64, 96), nn.ReLU(), nn.Linear(96, 32), nn.ReLU(), nn.Linear(32, 10)).eval().cuda()
+    dummy = torch.randn(4, 64).cuda()
+    sim = QuantizationSimModel(model, dummy, quant_scheme='tf_enhanced', per_channel_quantization=True)
+    sim.compute_encodings(lambda m, data: [m(b) for b in data], [torch.randn(32, 64).cuda() for _ in range(2)])
+    static_x = torch.randn(16, 64).cuda()
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                sim.model(static_x)                         # warm-up outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_y = sim.model(static_x)
+        for rep in range(5):
+            x = torch.randn(16, 64).cuda() * (rep + 1)
+            static_x.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            eager = sim.model(x)                            # eager work between the replays
+            assert torch.equal(static_y, eager), rep
+            torch.cuda.synchronize()
