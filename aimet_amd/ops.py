@@ -31,6 +31,9 @@ def _stream(t):
     return _stream_of(t.device)
 
 
+current_stream_handle = _stream_of
+
+
 class _OnDevice:
     """`with torch.cuda.device(d)` only when d is not already the current device: the context manager costs several
     microseconds per call, as much as queueing the kernel, and the devices nearly always agree."""

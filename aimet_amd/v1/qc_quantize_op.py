@@ -17,6 +17,7 @@ from typing import List, Tuple
 import torch
 from torch import nn
 
+from .. import ops
 from ..common import libpymo
 from ..common.defs import QuantizationDataType, QuantScheme
 from ..utils import (compute_partial_encoding, create_encoding_dict, create_encoding_from_dict,
@@ -393,8 +394,11 @@ class StaticGridQuantWrapper(QcQuantizeWrapper):
         return quantizer.encoding_stamp()
 
     def _param_cache_key(self, param, quantizer):
+        # (the stream is part of the key: a tensor kept by a forward on one stream is not handed to a forward on
+        # another, which nothing would order after the launch that wrote it)
+        stream = ops.current_stream_handle(param.device) if param.is_cuda else None
         return (param.data_ptr(), param._version, param.dtype, tuple(param.shape), quantizer.bitwidth,  # pylint: disable=protected-access
-                quantizer.data_type, self._encoding_stamp(quantizer))
+                quantizer.data_type, self._encoding_stamp(quantizer), stream)
 
     def _params_may_be_kept(self) -> bool:
         return StaticGridQuantWrapper.cache_quantized_params and not self.training and \

@@ -13,6 +13,7 @@ from typing import Type
 import torch
 from torch import nn
 
+from ... import ops
 from ..quantization.affine.quantizer import MinMaxQuantizer
 from ..utils import patch_attr
 
@@ -63,7 +64,9 @@ class BaseQuantizationMixin:
             return None
         mn, mx = quantizer.min, quantizer.max
         # pylint: disable=protected-access
-        return (id(param), param._version, param.data_ptr(), param.dtype, tuple(param.shape), id(quantizer),
+        # (the stream is part of the key: see StaticGridQuantWrapper._param_cache_key)
+        stream = ops.current_stream_handle(param.device) if param.is_cuda else None
+        return (stream, id(param), param._version, param.data_ptr(), param.dtype, tuple(param.shape), id(quantizer),
                 id(mn), mn._version, id(mx), mx._version, quantizer.qmin, quantizer.qmax, quantizer.symmetric,
                 quantizer.block_size)
 

@@ -15,6 +15,7 @@ from typing import Optional
 import torch
 from torch import nn
 
+from .... import ops
 from ...utils import (StatisticsNotFoundError, _is_expandable, get_encoding_shape_with_blocks, patch_attr,
                       reshape_tensor_for_blocks, ste_round)
 from ..encoding_analyzer import EncodingAnalyzer, MinMaxEncodingAnalyzer
@@ -331,8 +332,9 @@ class MinMaxQuantizer(nn.Module):
         # changes.  An edit through a `.data` alias moves no counter: assign, or use set_range().
         mn, mx = self.min, self.max
         learning = torch.is_grad_enabled() and (mn.requires_grad or mx.requires_grad)
+        stream = ops.current_stream_handle(mn.device) if mn.is_cuda else None    # (kept per stream, as the parameters)
         key = None if learning else (id(mn), mn._version, id(mx), mx._version, self.qmin, self.qmax,  # pylint: disable=protected-access
-                                     self._symmetric)
+                                     self._symmetric, stream)
         kept = self.__dict__.get('_kept_encoding')
         if key is not None and kept is not None and kept[0] == key and kept[1] is mn and kept[2] is mx:
             scale, offset = kept[3], kept[4]
@@ -353,6 +355,8 @@ class MinMaxQuantizer(nn.Module):
         if kept is None or kept[1] is not self.min or kept[2] is not self.max:
             return False
         if len(kept) == 5:
+            if kept[4].is_cuda and torch.cuda.is_current_stream_capturing():
+                return False             # would have to wait for the device: not while a graph is being captured
             kept = kept + (bool((kept[4] == -self.qmin).all()),)
             self.__dict__['_kept_encoding'] = kept
         return kept[5]

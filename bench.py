@@ -771,7 +771,8 @@ def bench_quantsim(torch, steps=10, batch=64):
                 sim.model(x1)
         torch.cuda.current_stream().wait_stream(side)
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        # captured on the stream the warm-up ran on: what the wrappers keep between forwards is kept per stream
+        with torch.cuda.graph(graph, stream=side):
             y1 = sim.model(x1)
     lat["sim_hip_graph_replay_ms"] = timed(graph.replay)
     with torch.no_grad():
