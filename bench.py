@@ -966,6 +966,29 @@ def bench_end_to_end(torch, ops):
     AdaroundOptimizer.optimize_rounding_on_cached_acts(wrapper, None, xs, ys, hp)
     torch.cuda.synchronize()
     loop = time.perf_counter() - t0
+    # a small convolutional model through the same entry point (its layers take the general path)
+    torch.manual_seed(1005)
+    cnet = torch.nn.Sequential(torch.nn.Conv2d(3, 64, 3, padding=1), torch.nn.ReLU(), torch.nn.Conv2d(64, 64, 3, padding=1),
+                               torch.nn.ReLU(), torch.nn.Conv2d(64, 128, 3, stride=2, padding=1), torch.nn.ReLU(),
+                               torch.nn.Conv2d(128, 128, 1), torch.nn.ReLU(), torch.nn.Conv2d(128, 256, 3, stride=2, padding=1),
+                               torch.nn.ReLU(), torch.nn.Conv2d(256, 256, 3, padding=1)).eval().to(dev)
+    cloader = [(torch.randn(64, 3, 32, 32, device=dev), torch.zeros(64)) for _ in range(4)]
+    conv_iters = 200
+    with tempfile.TemporaryDirectory() as tmp:
+        Adaround.apply_adaround(cnet, cloader[0][0][:2], AdaroundParameters(cloader, 4, 10, forward_fn=lambda m, b: m(b[0])),
+                                tmp, "warm", default_param_bw=4)
+        gc.collect()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        Adaround.apply_adaround(cnet, cloader[0][0][:2],
+                                AdaroundParameters(cloader, 4, conv_iters, forward_fn=lambda m, b: m(b[0])), tmp, "bench",
+                                default_param_bw=4)
+        torch.cuda.synchronize()
+        conv_total = time.perf_counter() - t0
+    out["apply_adaround_6_convolutions"] = {
+        "layers": 6, "input": [64, 3, 32, 32], "batches": 4, "iterations_per_layer": conv_iters, "bitwidth": 4,
+        "apply_adaround_s": conv_total, "s_per_layer": conv_total / 6,
+        "ms_per_iteration_end_to_end": conv_total / 6 / conv_iters * 1e3}
     out["apply_adaround_3x_linear_2048"] = {
         "layers": layers, "layer": [width, width], "samples": 1024, "iterations_per_layer": iters, "bitwidth": 4,
         "apply_adaround_s": total, "s_per_layer": total / layers,
