@@ -12,6 +12,7 @@ the supergroup and model-input rules to models built from modules (functional ``
 aimet_amd.v1.nn.modules.custom, as in the reference).
 """
 import copy
+import inspect
 import json
 import math
 import os
@@ -68,6 +69,17 @@ def _op_type(module: nn.Module) -> str:
         if isinstance(module, classes):
             return name
     return type(module).__name__
+
+
+def _declared_inputs(module: nn.Module) -> int:
+    """Number of tensors a module that was never called would take: the positional parameters of its forward() that
+    have no default (two for the elementwise modules), at least one."""
+    try:
+        params = inspect.signature(module.forward).parameters.values()
+    except (TypeError, ValueError):
+        return 1
+    required = [p for p in params if p.kind in (p.POSITIONAL_ONLY, p.POSITIONAL_OR_KEYWORD) and p.default is p.empty]
+    return max(1, len(required))
 
 
 def _flag(d: dict, key: str, default=None):
@@ -288,7 +300,8 @@ class QuantizationSimModel:
             if self._is_leaf(module) and module is not model and not isinstance(module, nn.Identity) \
                     and name not in reached and not isinstance(module, QcQuantizeWrapper):
                 records.append({"name": name, "module": module, "type": _op_type(module), "inputs": [],
-                                "num_inputs": 1, "num_outputs": 1, "consumers": [], "is_model_output": False})
+                                "num_inputs": _declared_inputs(module), "num_outputs": 1, "consumers": [],
+                                "is_model_output": False})
         return records
 
     def _add_quantization_wrappers(self):
@@ -335,6 +348,12 @@ class QuantizationSimModel:
             for q in w.input_quantizers + w.output_quantizers:
                 q.use_symmetric_encodings = _flag(op_cfg, "is_symmetric", act_sym)
                 q.use_strict_symmetric, q.use_unsigned_symmetric = strict, unsigned
+            fixed = op_cfg.get("encoding_constraints")
+            if fixed is not None:
+                # the op's outputs get this range whatever passes through them (reference quantsim_config.py:463-465,
+                # :806-808, :842-843)
+                for q in w.output_quantizers:
+                    q.encoding_min_max_fixed_vals = (fixed["min"], fixed["max"])
             for pname, q in w.param_quantizers.items():
                 pcfg = dict(cfg.get("params", {}).get(pname, {}))
                 pcfg.update(op_cfg.get("params", {}).get(pname, {}))
@@ -731,11 +750,13 @@ def load_encodings_to_sim(quant_sim_model: QuantizationSimModel, pytorch_encodin
     """Loads an exported encodings file into a simulation model configured like the one that wrote it: wrappers go to
     ACTIVE mode, every quantizer the file has no entry for is switched off, and range-learning models get their
     learned-grid wrappers (reference quantsim.py:2277-2298)."""
-    for _, wrapper in quant_sim_model.quant_wrappers():
-        wrapper.set_mode(QcQuantizeOpMode.ACTIVE)
+    for module in quant_sim_model.model.modules():
+        if isinstance(module, QcQuantizeWrapper):
+            module.set_mode(QcQuantizeOpMode.ACTIVE)
     quant_sim_model.load_encodings(pytorch_encoding_path, strict=True, partial=False, requires_grad=None,
                                    allow_overwrite=None)
-    quant_sim_model.replace_wrappers_for_quantize_dequantize()
+    if isinstance(quant_sim_model, QuantizationSimModel):
+        quant_sim_model.replace_wrappers_for_quantize_dequantize()          # a v2 simulation has no wrappers
 
 
 def has_valid_encodings(qc_quantize_op: QcQuantizeWrapper) -> bool:

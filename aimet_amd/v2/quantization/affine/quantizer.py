@@ -18,6 +18,7 @@ from torch import nn
 from .... import ops
 from ...utils import (StatisticsNotFoundError, _is_expandable, get_encoding_shape_with_blocks, patch_attr,
                       reshape_tensor_for_blocks, ste_round)
+from ..base import QuantizerBase
 from ..encoding_analyzer import EncodingAnalyzer, MinMaxEncodingAnalyzer
 from .backends import _derive_qmin_qmax, quantize, quantize_dequantize
 
@@ -113,7 +114,7 @@ def _grid_arguments(owner: str, args, kwargs):
                         f"optionally followed by encoding_analyzer and block_size: {error}") from None
 
 
-class MinMaxQuantizer(nn.Module):
+class MinMaxQuantizer(QuantizerBase):
     """Affine quantizer with min / max as trainable parameters."""
 
     def __init__(self, shape, *args, **kwargs):

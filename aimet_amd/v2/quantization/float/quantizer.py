@@ -19,6 +19,7 @@ from torch import nn
 from .... import ops
 from ...utils import StatisticsNotFoundError, patch_attr
 from ..affine.quantizer import _flag_extreme_min_max
+from ..base import QuantizerBase
 from ..encoding_analyzer import EncodingAnalyzer
 from .encoding import FloatEncoding
 
@@ -53,7 +54,7 @@ class _FakeCast(torch.autograd.Function):
         return (grad if ctx.passes_gradient else torch.zeros_like(grad)), None, None
 
 
-class FloatQuantizeDequantize(nn.Module):
+class FloatQuantizeDequantize(QuantizerBase):
     """out = input rounded to the nearest value of a float format with `exponent_bits` and `mantissa_bits`.
 
     Unlike the affine quantizers it needs no calibration: is_initialized() is always True.  With an

@@ -23,6 +23,7 @@ from ...v1.tensor_quantizer import StaticGridPerChannelQuantizer
 from ..nn import BaseQuantizationMixin, QuantizationMixin
 from ..quantization.affine import QuantizeDequantize
 from ..quantization.affine.quantizer import batched_range_checks
+from ..quantization.base import QuantizerBase
 from ..quantization.float import FloatQuantizeDequantize
 from ..quantization.encoding_analyzer import (MinMaxEncodingAnalyzer, PercentileEncodingAnalyzer,
                                               SqnrEncodingAnalyzer, _HistogramObserver)
@@ -43,6 +44,25 @@ def _analyzer(quant_scheme: QuantScheme, shape):
     raise NotImplementedError(f"quant scheme {quant_scheme} is not supported")
 
 
+def _refuse_quantized(model: nn.Module):
+    """Only models without quantized modules or quantizers can be simulated (reference v2 quantsim.py:126-150)."""
+    if isinstance(model, BaseQuantizationMixin):
+        found = f"the model itself is already a quantized module of type {type(model)}."
+    elif isinstance(model, QuantizerBase):
+        found = f"the model itself is already a quantizer object of type {type(model)}."
+    else:
+        qmodules = [name for name, m in model.named_modules() if isinstance(m, BaseQuantizationMixin)]
+        quantizers = [name for name, m in model.named_modules() if isinstance(m, QuantizerBase)]
+        if qmodules:
+            found = f"the model already contains quantized modules: {', '.join(qmodules)}."
+        elif quantizers:
+            found = f"the model already contains quantizers: {', '.join(quantizers)}."
+        else:
+            return
+    raise RuntimeError("QuantizationSimModel can only take base models WITHOUT quantized modules or quantizers, but "
+                       + found)
+
+
 class QuantizationSimModel:
     """Replaces the leaf modules of (a copy of) `model` by quantized modules configured like the v1 simulation."""
 
@@ -57,6 +77,7 @@ class QuantizationSimModel:
             raise ValueError("dummy_input is needed: the configuration follows the order in which modules run")
         if rounding_mode != 'nearest':
             raise ValueError("v2 quantizers round to nearest")
+        _refuse_quantized(model)
         if per_channel_quantization is not None:
             # shorthand for the one default most callers change
             if isinstance(config_file, (str, os.PathLike)):
@@ -126,6 +147,15 @@ class QuantizationSimModel:
         if self._quant_scheme not in _RANGE_LEARNING:
             for param in quantizer.parameters():
                 param.requires_grad = False                            # builder.py:187-202
+        fixed = q.encoding_min_max_fixed_vals
+        if fixed:
+            # a range the configuration prescribes ("encoding_constraints") is set once and never calibrated or
+            # trained (builder.py:173-181)
+            with torch.no_grad():
+                quantizer.min.fill_(fixed[0])
+                quantizer.max.fill_(fixed[1])
+            quantizer.allow_overwrite(False)
+            quantizer.requires_grad_(False)
         return quantizer
 
     # --------------------------------------------------------------------------------------------------- usage

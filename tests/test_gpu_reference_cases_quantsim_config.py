@@ -226,3 +226,46 @@ def test_parse_config_file_symmetric_modes():       # :1080-1120
                 list(module.param_quantizers.values()):
             assert q.use_strict_symmetric
             assert not q.use_unsigned_symmetric
+
+
+def test_encoding_constraints():                    # :2129-2183
+    """A range the configuration prescribes for an op type replaces what passes through the op's outputs: the quantizer
+    switches to the min/max scheme and its encoding covers exactly that range."""
+    import numpy as np
+    config = {"defaults": {"ops": {"is_output_quantized": "True", "is_symmetric": "False"},
+                           "params": {"is_quantized": "False", "is_symmetric": "True"}},
+              "params": {}, "op_type": {"Softmax": {"encoding_constraints": {"min": -5.0, "max": 5.0}}},
+              "supergroups": [], "model_input": {}, "model_output": {}}
+
+    class SoftmaxModel(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.softmax = nn.Softmax(dim=0)
+
+        def forward(self, inp):
+            return self.softmax(inp)
+
+    x = torch.tensor([0.5, 0.5]).cuda()
+    for config_file in (None, config):
+        sim = QuantizationSimModel(SoftmaxModel().cuda(), x, quant_scheme=QuantScheme.post_training_tf_enhanced,
+                                   config_file=config_file)
+        sim.compute_encodings(lambda m, _: m(x), None)
+        q = sim.model.softmax.output_quantizers[0]
+        if config_file is None:
+            assert q.quant_scheme == QuantScheme.post_training_tf_enhanced
+            assert q.encoding.min == 0.0
+            assert np.allclose(q.encoding.max, 0.5, atol=1e-2)
+        else:
+            assert q.quant_scheme == QuantScheme.post_training_tf
+            assert q.encoding_min_max_fixed_vals == (-5.0, 5.0)
+            assert np.allclose(q.encoding.min, -5.0, atol=1e-1)
+            assert np.allclose(q.encoding.max, 5.0, atol=1e-1)
+            # the grid is the 8-bit one over [-5, 5]: 0.5 lands on a multiple of its step
+            y = sim.model(x)
+            assert torch.allclose(y / q.encoding.delta, (y / q.encoding.delta).round(), atol=1e-3)
+            # range learning keeps such a quantizer frozen (reference v1/quantsim.py:817-829)
+            sim = QuantizationSimModel(SoftmaxModel().cuda(), x,
+                                       quant_scheme=QuantScheme.training_range_learning_with_tf_init,
+                                       config_file=config_file)
+            sim.compute_encodings(lambda m, _: m(x), None)
+            assert sim.model.softmax.output_quantizers[0].is_encoding_frozen

@@ -1,0 +1,404 @@
+"""GPU tests of the v2 simulation model along the cases of the reference's
+TrainingExtensions/torch/test/python/v2/quantsim/test_quantsim.py (class TestQuantsim): percentile value, the three ways
+of loading encodings with their freezing rules, strict / partial / requires_grad / allow_overwrite, legacy encoding
+files (partial, naming modules the model lacks, addressing a removed quantizer), unused and abstract modules, ranges
+prescribed by the configuration, and the refusal of models that are already quantized.
+
+The models are this file's own (small stand-ins for the reference's BasicConv2d, TinyModel and SmallMnist with the same
+module names where the cases use them); files are written with export_encodings(), which holds what the reference's
+export() writes into '<prefix>_torch.encodings'.  Everything the quantizers compute runs in the HIP kernels.
+"""
+import json
+
+import pytest
+import torch
+from torch import nn
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def _seed():
+    torch.manual_seed(0)
+
+
+def _sim(*args, **kwargs):
+    from aimet_amd.v2.quantsim import QuantizationSimModel
+    return QuantizationSimModel(*args, **kwargs)
+
+
+def _quantizers(sim):
+    from aimet_amd.v2.quantization.base import QuantizerBase
+    return [m for m in sim.model.modules() if isinstance(m, QuantizerBase)]
+
+
+class _ConvBnRelu(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.conv, self.bn, self.relu = nn.Conv2d(16, 16, 3), nn.BatchNorm2d(16), nn.ReLU()
+
+    def forward(self, x):
+        return self.relu(self.bn(self.conv(x)))
+
+
+class _TinyNet(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.conv1, self.bn1, self.relu1 = nn.Conv2d(3, 8, 3, padding=1), nn.BatchNorm2d(8), nn.ReLU()
+        self.pool = nn.MaxPool2d(2)
+        self.conv2, self.relu2 = nn.Conv2d(8, 8, 3), nn.ReLU()
+        self.avg, self.flat, self.fc = nn.AdaptiveAvgPool2d(1), nn.Flatten(), nn.Linear(8, 10)
+
+    def forward(self, x):
+        x = self.pool(self.relu1(self.bn1(self.conv1(x))))
+        return self.fc(self.flat(self.avg(self.relu2(self.conv2(x)))))
+
+
+class _DigitNet(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.conv1, self.relu1, self.pool1 = nn.Conv2d(1, 8, 5), nn.ReLU(), nn.MaxPool2d(2)
+        self.conv2, self.conv2_drop, self.relu2, self.pool2 = nn.Conv2d(8, 16, 5), nn.Dropout2d(), nn.ReLU(), \
+            nn.MaxPool2d(2)
+        self.flat, self.fc1, self.relu3, self.dropout = nn.Flatten(), nn.Linear(256, 32), nn.ReLU(), nn.Dropout()
+        self.fc2, self.log_softmax = nn.Linear(32, 10), nn.LogSoftmax(dim=1)
+
+    def forward(self, x):
+        x = self.pool1(self.relu1(self.conv1(x)))
+        x = self.pool2(self.relu2(self.conv2_drop(self.conv2(x))))
+        return self.log_softmax(self.fc2(self.dropout(self.relu3(self.fc1(self.flat(x))))))
+
+
+def _same_grid(a, b):
+    return torch.allclose(a.get_min(), b.get_min()) and torch.allclose(a.get_max(), b.get_max()) and \
+        a.bitwidth == b.bitwidth and a.symmetric == b.symmetric
+
+
+def _min_max(quantizer):
+    return quantizer.min.clone().detach(), quantizer.max.clone().detach()
+
+
+def _entry(lo, hi, scale, offset, bitwidth=8, symmetric="False"):
+    return {"min": lo, "max": hi, "scale": scale, "offset": offset, "bitwidth": bitwidth, "is_symmetric": symmetric,
+            "dtype": "int"}
+
+
+# ------------------------------------------------------------------------------------------------ percentile scheme
+def test_percentile_value_moves_the_parameter_range():
+    """test_set_percentile_value: a lower percentile gives a tighter weight range."""
+    from aimet_amd.v2.quantization.encoding_analyzer import PercentileEncodingAnalyzer
+    model = _ConvBnRelu().eval().cuda()
+    x = torch.rand(1, 16, 16, 16).cuda()
+    sim = _sim(model, x, quant_scheme="percentile")
+    weight_q = sim.model.conv.param_quantizers["weight"]
+    assert isinstance(weight_q.encoding_analyzer, PercentileEncodingAnalyzer)
+    largest = {}
+    for value in (99.9, 90.0):
+        sim.set_percentile_value(value)
+        assert weight_q.encoding_analyzer.percentile == value
+        sim.compute_encodings(lambda m, _: m(x), None)
+        largest[value] = weight_q.get_max().clone()
+    assert torch.all(largest[99.9] > largest[90.0])
+
+
+# ------------------------------------------------------------------------------------- loading and freezing encodings
+@pytest.mark.parametrize("per_channel", (False, True))
+def test_set_and_freeze_param_encodings(tmp_path, per_channel):
+    """Parameters come from the file and stay; activations keep following the data."""
+    model = _ConvBnRelu().eval().cuda()
+    x = torch.rand(1, 16, 16, 16).cuda()
+    sim = _sim(model, x, quant_scheme="tf", per_channel_quantization=per_channel)
+    sim.compute_encodings(lambda m, _: m(x), None)
+    file = sim.export_encodings(str(tmp_path), "conv")
+
+    other = _sim(model, x, quant_scheme="tf", per_channel_quantization=per_channel)
+    other.set_and_freeze_param_encodings(file)
+    weight_q = other.model.conv.param_quantizers["weight"]
+    assert weight_q.min.numel() == (16 if per_channel else 1)
+    assert _same_grid(sim.model.conv.param_quantizers["weight"], weight_q)
+
+    before = _min_max(weight_q)
+    with torch.no_grad():
+        other.model.conv.weight.mul_(10)
+    other.compute_encodings(lambda m, _: m(x), None)
+    assert torch.equal(before[0], weight_q.min) and torch.equal(before[1], weight_q.max)
+
+    input_q = other.model.conv.input_quantizers[0]
+    lo, hi = _min_max(input_q)
+    other.compute_encodings(lambda m, _: m(10 * x), None)
+    assert torch.allclose(10 * lo, input_q.min) and torch.allclose(10 * hi, input_q.max)
+
+
+@pytest.mark.parametrize("per_channel", (False, True))
+def test_load_and_freeze_encodings(tmp_path, per_channel):
+    """Parameters and activations both stay; no quantizer appears or disappears."""
+    x = torch.rand(1, 3, 32, 32).cuda()
+    sim = _sim(_TinyNet().eval().cuda(), x, quant_scheme="tf", per_channel_quantization=per_channel)
+    sim.compute_encodings(lambda m, _: m(x), None)
+    file = sim.export_encodings(str(tmp_path), "tiny")
+
+    other = _sim(_TinyNet().eval().cuda(), x, per_channel_quantization=per_channel)
+    present = _quantizers(other)
+    other.load_and_freeze_encodings(file)
+    assert len(present) == len(_quantizers(other)) and all(a is b for a, b in zip(present, _quantizers(other)))
+
+    weight_q, input_q = other.model.conv1.param_quantizers["weight"], other.model.conv1.input_quantizers[0]
+    weights, inputs = _min_max(weight_q), _min_max(input_q)
+    with torch.no_grad():
+        other.model.conv1.weight.mul_(10)
+    other.compute_encodings(lambda m, _: m(x), None)
+    assert torch.equal(weights[0], weight_q.min) and torch.equal(weights[1], weight_q.max)
+    other.compute_encodings(lambda m, _: m(10 * x), None)
+    assert torch.equal(inputs[0], input_q.min) and torch.equal(inputs[1], input_q.max)
+
+
+def test_load_and_freeze_part_of_the_encodings():
+    """Only what the dictionary names is frozen; everything else is calibrated as before."""
+    x = torch.randn(1, 3, 32, 32).cuda()
+    sample = _entry(-4, 4, 0.03, 8)
+    part = {"activation_encodings": {"conv1": {"input": {"0": sample}}}, "param_encodings": {"conv1.weight": [sample]}}
+    sim = _sim(_TinyNet().eval().cuda(), x, quant_scheme="tf")
+    present = _quantizers(sim)
+    sim.load_and_freeze_encodings(part)
+    assert all(a is b for a, b in zip(present, _quantizers(sim))) and len(present) == len(_quantizers(sim))
+
+    conv1_w, fc_w = sim.model.conv1.param_quantizers["weight"], sim.model.fc.param_quantizers["weight"]
+    conv1_in, fc_out = sim.model.conv1.input_quantizers[0], sim.model.fc.output_quantizers[0]
+    kept = _min_max(conv1_w)
+    with torch.no_grad():
+        sim.model.conv1.weight.mul_(10)
+    sim.compute_encodings(lambda m, _: m(x), None)
+    assert torch.equal(kept[0], conv1_w.min) and torch.equal(kept[1], conv1_w.max)
+
+    free = _min_max(fc_w)
+    with torch.no_grad():
+        sim.model.fc.weight.mul_(10)
+    sim.compute_encodings(lambda m, _: m(x), None)
+    assert torch.allclose(10 * free[0], fc_w.min) and torch.allclose(10 * free[1], fc_w.max)
+
+    kept, free = _min_max(conv1_in), _min_max(fc_out)
+    sim.compute_encodings(lambda m, _: m(10 * x), None)
+    assert torch.equal(kept[0], conv1_in.min) and torch.equal(kept[1], conv1_in.max)
+    assert not torch.isclose(free[0], fc_out.min) and not torch.isclose(free[1], fc_out.max)
+
+
+def test_load_encodings_options():
+    """test_load_encodings: strict, partial, requires_grad and allow_overwrite, one after the other."""
+    model = _TinyNet().eval().cuda()
+    x = torch.randn(1, 3, 32, 32).cuda()
+    first, second = _entry(-4, 4, 0.03, 8), _entry(-8, 8, 0.06, 8)
+    named = {"activation_encodings": {"conv1": {"input": {"0": first}}}, "param_encodings": {"conv1.weight": [first]}}
+    renamed = {"activation_encodings": {"conv1": {"input": {"0": second}}},
+               "param_encodings": {"conv1.weight": [second]}}
+    # conv1's output has no quantizer (conv1 + bn1 + relu1 share one at relu1's output)
+    stray = {"activation_encodings": {"conv1": {"input": {"0": first}, "output": {"0": first}}},
+             "param_encodings": {"conv1.weight": [first]}}
+
+    with pytest.raises(RuntimeError):
+        _sim(model, x).load_encodings(stray, strict=True)
+    sim = _sim(model, x)
+    sim.load_encodings(stray, strict=False)
+    assert sim.model.conv1.output_quantizers[0] is None
+
+    sim = _sim(model, x)
+    sim.load_encodings(named, partial=False)
+    left = _quantizers(sim)
+    assert len(left) == 2 and left[0] is sim.model.conv1.param_quantizers["weight"] and \
+        left[1] is sim.model.conv1.input_quantizers[0]
+
+    sim = _sim(model, x)
+    present = _quantizers(sim)
+    sim.load_encodings(named, partial=True)
+    assert len(present) == len(_quantizers(sim)) and all(a is b for a, b in zip(present, _quantizers(sim)))
+
+    for requires_grad in (True, False):
+        sim = _sim(model, x)
+        loaded = (sim.model.conv1.param_quantizers["weight"], sim.model.conv1.input_quantizers[0])
+        others = {q: (q.min.requires_grad, q.max.requires_grad) for q in _quantizers(sim) if q not in loaded}
+        for setting in (requires_grad, None):                       # None keeps what is there
+            sim.load_encodings(named, requires_grad=setting)
+            for q in loaded:
+                assert q.min.requires_grad == q.max.requires_grad == requires_grad
+            for q, (lo, hi) in others.items():
+                assert (q.min.requires_grad, q.max.requires_grad) == (lo, hi)
+
+    def ranges(s):
+        return [t for q in (s.model.conv1.param_quantizers["weight"], s.model.conv1.input_quantizers[0])
+                for t in _min_max(q)]
+
+    sim = _sim(model, x)
+    sim.load_encodings(named, allow_overwrite=True)
+    was = ranges(sim)
+    sim.compute_encodings(lambda m, _: m(x), None)
+    assert not any(torch.isclose(a, b) for a, b in zip(was, ranges(sim)))
+    was = ranges(sim)
+    sim.load_encodings(renamed)
+    assert not any(torch.isclose(a, b) for a, b in zip(was, ranges(sim)))
+
+    sim = _sim(model, x)
+    sim.load_encodings(named, allow_overwrite=False)
+    was = ranges(sim)
+    sim.compute_encodings(lambda m, _: m(x), None)
+    assert all(torch.equal(a, b) for a, b in zip(was, ranges(sim)))
+    sim.load_encodings(renamed)
+    assert all(torch.equal(a, b) for a, b in zip(was, ranges(sim)))
+    sim.load_encodings(named, allow_overwrite=None)                 # frozen quantizers stay frozen
+    assert all(torch.equal(a, b) for a, b in zip(was, ranges(sim)))
+
+
+# ------------------------------------------------------------------------------------------------ legacy files
+def _loaders():
+    from aimet_amd.v1.quantsim import load_encodings_to_sim
+    from aimet_amd.v2.quantsim import QuantizationSimModel
+    return {"load_encodings_to_sim": load_encodings_to_sim,
+            "load_and_freeze_encodings": QuantizationSimModel.load_and_freeze_encodings,
+            "set_and_freeze_param_encodings": QuantizationSimModel.set_and_freeze_param_encodings}
+
+
+_LOADER_NAMES = ("load_encodings_to_sim", "load_and_freeze_encodings", "set_and_freeze_param_encodings")
+
+
+def _legacy_file(tmp_path, activation_encodings, param_encodings):
+    content = {"activation_encodings": activation_encodings, "excluded_layers": [],
+               "param_encodings": param_encodings,
+               "quantizer_args": {"activation_bitwidth": 8, "dtype": "int", "is_symmetric": True, "param_bitwidth": 4,
+                                  "per_channel_quantization": False, "quant_scheme": "post_training_tf_enhanced"},
+               "version": "0.6.1"}
+    file = tmp_path / "legacy.encodings"
+    file.write_text(json.dumps(content))
+    return str(file)
+
+
+@pytest.mark.parametrize("loader", _LOADER_NAMES)
+def test_legacy_file_with_part_of_the_encodings(tmp_path, loader):
+    file = _legacy_file(tmp_path, {
+        "conv1": {"input": {"0": _entry(0.0, 0.9945, 0.0039, 0)}},
+        "conv2": {"output": {"0": _entry(-0.4335, 0.4896, 0.00362, -120)}},
+        "fc2": {"output": {"0": _entry(-0.1596, 0.1974, 0.0014, -114)}},
+        "relu1": {"output": {"0": _entry(0.0, 1.0455, 0.0041, 0)}},
+        "relu3": {"output": {"0": _entry(0.0, 0.5355, 0.0021, 0)}},
+    }, {
+        "conv1.weight": [_entry(-0.2144, 0.1876, 0.0268, -8, bitwidth=4, symmetric="True")],
+        "fc2.weight": [_entry(-0.1496, 0.1309, 0.0187, -8, bitwidth=4, symmetric="True")],
+    })
+    sim = _sim(_DigitNet().eval().cuda(), torch.rand(1, 1, 28, 28).cuda())
+    present = _quantizers(sim)
+    _loaders()[loader](sim, file)
+    if loader == "load_encodings_to_sim":
+        m = sim.model                                               # what the file does not name is gone
+        named = [m.conv1.input_quantizers[0], m.conv1.param_quantizers["weight"], m.conv2.output_quantizers[0],
+                 m.fc2.output_quantizers[0], m.fc2.param_quantizers["weight"], m.relu1.output_quantizers[0],
+                 m.relu3.output_quantizers[0]]
+        assert all(q is not None for q in named)
+        assert sorted(map(id, named)) == sorted(map(id, _quantizers(sim)))
+        assert m.conv1.param_quantizers["weight"].bitwidth == 4
+        assert torch.isfinite(m(torch.rand(2, 1, 28, 28).cuda())).all()
+    else:
+        assert len(present) == len(_quantizers(sim)) and all(a is b for a, b in zip(present, _quantizers(sim)))
+
+
+@pytest.mark.parametrize("loader", _LOADER_NAMES)
+def test_legacy_file_naming_what_the_model_lacks(tmp_path, loader):
+    file = _legacy_file(tmp_path, {"conv999": {"input": {"0": _entry(0.0, 0.9945, 0.0039, 0)}}},
+                        {"conv999.weight": [_entry(-0.2144, 0.1876, 0.0268, -8, bitwidth=4, symmetric="True")]})
+    sim = _sim(_DigitNet().eval().cuda(), torch.rand(1, 1, 28, 28).cuda())
+    with pytest.raises(RuntimeError):
+        _loaders()[loader](sim, file)
+
+
+@pytest.mark.parametrize("loader", _LOADER_NAMES)
+def test_legacy_file_for_removed_quantizers(tmp_path, loader):
+    file = _legacy_file(tmp_path, {"conv1": {"input": {"0": _entry(0.0, 0.9945, 0.0039, 0)}}},
+                        {"conv1.weight": [_entry(-0.2144, 0.1876, 0.0268, -8, bitwidth=4, symmetric="True")]})
+    sim = _sim(_DigitNet().eval().cuda(), torch.rand(1, 1, 28, 28).cuda())
+    sim.model.conv1.input_quantizers[0] = None
+    sim.model.conv1.param_quantizers["weight"] = None
+    with pytest.raises(RuntimeError):
+        _loaders()[loader](sim, file)
+
+
+# ------------------------------------------------------------------------------------------------ construction
+def test_modules_the_forward_pass_never_reaches():
+    """test_quantsim_with_unused_modules: they become quantized modules with all their quantizer slots."""
+    from aimet_amd.v1.nn.modules.custom import Add
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.identity, self.add = nn.Identity(), Add()
+
+        def forward(self, x):
+            return self.identity(x)
+
+    sim = _sim(Net().cuda(), torch.randn(10, 10).cuda())
+    assert len(sim.model.add.input_quantizers) == 2
+    assert type(sim.model.add.input_quantizers[0]) is type(sim.model.add.input_quantizers[1])
+    assert torch.isfinite(sim.model(torch.randn(10, 10).cuda())).all()
+
+
+def test_container_of_plain_module_type():
+    """test_quantsim_with_abstract_modules: a bare nn.Module that only holds children stays what it is."""
+    from aimet_amd.v2.nn import QuantizedConv2d
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.module = nn.Module()
+            self.module.conv = nn.Conv2d(3, 3, 3)
+
+        def forward(self, x):
+            return self.module.conv(x)
+
+    sim = _sim(Net().cuda(), torch.randn(1, 3, 10, 10).cuda())
+    assert type(sim.model.module) is nn.Module                      # pylint: disable=unidiomatic-typecheck
+    assert isinstance(sim.model.module.conv, QuantizedConv2d)
+
+
+def test_range_prescribed_by_the_configuration():
+    """test_encoding_min_max_fixed_vals: "encoding_constraints" of an op type fix its output range at construction;
+    calibration leaves it alone; float quantizers have no such range."""
+    from aimet_amd.common.defs import QuantizationDataType
+    config = {"defaults": {"ops": {"is_output_quantized": "True", "is_symmetric": "False"},
+                           "params": {"is_quantized": "False", "is_symmetric": "True"}},
+              "params": {"weight": {"is_quantized": "True"}},
+              "op_type": {"Softmax": {"encoding_constraints": {"min": 0.0, "max": 1.0}}},
+              "supergroups": [], "model_input": {}, "model_output": {}}
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.linear, self.softmax = nn.Linear(3, 8), nn.Softmax(dim=-1)
+
+        def forward(self, x):
+            return self.softmax(self.linear(x))
+
+    model, x = Net().cuda(), torch.randn(4, 3).cuda()
+    sim = _sim(model, x, config_file=config)
+    out_q = sim.model.softmax.output_quantizers[0]
+    assert torch.equal(out_q.min, torch.tensor(0., device="cuda")) and \
+        torch.equal(out_q.max, torch.tensor(1., device="cuda"))
+    assert not out_q.min.requires_grad and not out_q.max.requires_grad
+    sim.compute_encodings(lambda m, _: m(x), None)
+    assert out_q.min.item() == 0.0 and out_q.max.item() == 1.0
+    assert sim.model.linear.output_quantizers[0].max.item() != 1.0
+    y = sim.model(x)
+    steps = y * 255                                                 # the output lies on the 8-bit grid over [0, 1]
+    assert torch.allclose(steps, steps.round(), atol=1e-4)
+
+    sim = _sim(model, x, config_file=config, default_param_bw=16, default_output_bw=16,
+               default_data_type=QuantizationDataType.float)
+    assert not hasattr(sim.model.softmax.output_quantizers[0], "min")
+    assert not hasattr(sim.model.softmax.output_quantizers[0], "max")
+
+
+def test_models_that_are_quantized_already():
+    """test_already_quantized_model"""
+    from aimet_amd.v2.nn import QuantizedConv2d
+    from aimet_amd.v2.quantization.affine import QuantizeDequantize
+    x = torch.randn(1, 3, 24, 24).cuda()
+    for model in (nn.Sequential(QuantizedConv2d(3, 3, 3), nn.ReLU()),
+                  nn.Sequential(nn.Conv2d(3, 3, 3), QuantizeDequantize((), 0, 255, False)),
+                  QuantizedConv2d(3, 3, 3),
+                  QuantizeDequantize((), 0, 255, False)):
+        with pytest.raises(RuntimeError, match="WITHOUT quantized modules or quantizers"):
+            _sim(model.cuda(), x)
