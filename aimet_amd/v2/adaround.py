@@ -127,6 +127,11 @@ class Adaround(V1Adaround):
         return found if isinstance(found, BaseQuantizationMixin) else None
 
     @staticmethod
+    def _supported_wrappers(quant_sim_model: nn.Module):
+        return ((n, m) for n, m in quant_sim_model.named_modules()
+                if isinstance(m, BaseQuantizationMixin) and isinstance(m, AdaroundSupportedModules))
+
+    @staticmethod
     def _compute_param_encodings(quant_sim: QuantizationSimModel):
         for quantized in _quantized_modules(quant_sim.model):
             # only parameters are quantized while AdaRound runs: activation quantizers are taken out

@@ -166,6 +166,26 @@ class QuantizationSimModel:
 
     named_qmodules = qmodules
 
+    def exclude_layers_from_quantization(self, layers_to_exclude):
+        """The given quantized modules, and the quantized modules below the given containers, become plain modules
+        again (aimet_torch/v1/quantsim.py:731-751, which the v2 class inherits)."""
+        leaving = {id(m) for layer in layers_to_exclude for m in layer.modules()
+                   if isinstance(m, BaseQuantizationMixin)}
+
+        def restore(parent: nn.Module):
+            for name, child in list(parent.named_children()):
+                if id(child) in leaving:
+                    setattr(parent, name, child.get_original_module())
+                else:
+                    restore(child)
+        restore(self.model)
+
+    def exclude_param_from_quantization(self, param_name_to_exclude: str):
+        """No module quantizes its parameter of this name any more (reference v2 quantsim.py:288-298)."""
+        for _, module in self.qmodules():
+            if param_name_to_exclude in module.param_quantizers:
+                module.param_quantizers[param_name_to_exclude] = None
+
     def set_percentile_value(self, percentile_value: float):
         """Percentile of every percentile analyzer (reference v2 quantsim.py:270-278)."""
         if percentile_value < 90 or percentile_value > 100:

@@ -1,6 +1,7 @@
 """The end-to-end cases of the reference's AdaRound tests (TrainingExtensions/torch/test/python/
-test_adaround_weight.py:295-1045) on the GPU path, with the reference's test models, and the cases of
-test_adaround_optimizer.py / test_adaround_loss.py with the expected numbers those files hold."""
+test_adaround_weight.py:295-1045, and its copy for the v2 quantized modules, v2/test_adaround.py:281-1031) on the GPU
+path, with the reference's test models, each case once over the v1 wrappers and once over the v2 quantized modules, and
+the cases of test_adaround_optimizer.py / test_adaround_loss.py with the expected numbers those files hold."""
 import json
 import os
 from unittest.mock import patch
@@ -114,16 +115,28 @@ def _forward_fn(model, batch):
     return model(batch[0])
 
 
-@pytest.fixture(scope="module")
-def ada():
+@pytest.fixture(scope="module", params=["v1", "v2"])
+def ada(request):
+    """The AdaRound entry points over the v1 wrappers and over the v2 quantized modules: the reference keeps one copy
+    of these cases for each (test_adaround_weight.py and v2/test_adaround.py)."""
     from aimet_amd.common.defs import QuantScheme
-    from aimet_amd.v1.adaround import adaround_weight
 
     class Api:
         pass
     a = Api()
-    a.Adaround, a.AdaroundParameters, a.QuantScheme = adaround_weight.Adaround, adaround_weight.AdaroundParameters, \
-        QuantScheme
+    a.version, a.QuantScheme = request.param, QuantScheme
+    if request.param == "v1":
+        from aimet_amd.v1.adaround import adaround_weight as api
+        from aimet_amd.v1.qc_quantize_op import StaticGridQuantWrapper
+        from aimet_amd.v1.quantsim import QuantizationSimModel
+        a.quantized_module_type = StaticGridQuantWrapper
+    else:
+        from aimet_amd.v2 import adaround as api
+        from aimet_amd.v2.nn import BaseQuantizationMixin
+        from aimet_amd.v2.quantsim import QuantizationSimModel
+        a.quantized_module_type = BaseQuantizationMixin
+    a.Adaround, a.AdaroundParameters, a.QuantizationSimModel = api.Adaround, api.AdaroundParameters, \
+        QuantizationSimModel
     return a
 
 
@@ -177,12 +190,11 @@ def test_apply_adaround_per_channel(ada, tmp_path):
 def test_before_opt_mse(ada):
     # :518-563: soft rounding at initialisation reproduces the float layer; hard rounding the round-to-nearest one
     from aimet_amd.v1.qc_quantize_op import QcQuantizeOpMode, StaticGridQuantWrapper
-    from aimet_amd.v1.quantsim import QuantizationSimModel
     torch.manual_seed(0)
     model = TinyModel().eval().cuda()
     dummy_input = torch.randn(1, 3, 32, 32).cuda()
     out_float32 = model.conv1(dummy_input)
-    sim = QuantizationSimModel(model, dummy_input=dummy_input, default_param_bw=4)
+    sim = ada.QuantizationSimModel(model, dummy_input=dummy_input, default_param_bw=4)
     ada.Adaround._compute_param_encodings(sim)                      # pylint: disable=protected-access
     for w in sim.model.modules():
         if isinstance(w, StaticGridQuantWrapper):
@@ -260,18 +272,17 @@ def test_overriding_default_parameter_bitwidths(ada, tmp_path):
 
 def test_ignoring_ops_for_quantization(ada, tmp_path):
     # :810-872
-    from aimet_amd.v1.qc_quantize_op import StaticGridQuantWrapper
-    from aimet_amd.v1.quantsim import QuantizationSimModel
+    quantized = ada.quantized_module_type
     model = TinyModel().eval().cuda()
     x = torch.randn(1, 3, 32, 32).cuda()
-    sim = QuantizationSimModel(model, dummy_input=x, default_param_bw=8)
+    sim = ada.QuantizationSimModel(model, dummy_input=x, default_param_bw=8)
     for name in ("maxpool", "avgpool", "conv2", "relu3"):
-        assert isinstance(getattr(sim.model, name), StaticGridQuantWrapper)
+        assert isinstance(getattr(sim.model, name), quantized)
     ada.Adaround._exclude_modules(model, sim, [model.maxpool, model.avgpool])   # pylint: disable=protected-access
     sim.compute_encodings(lambda m, a: m(a), x)
-    assert not isinstance(sim.model.maxpool, StaticGridQuantWrapper)
-    assert not isinstance(sim.model.avgpool, StaticGridQuantWrapper)
-    assert isinstance(sim.model.conv2, StaticGridQuantWrapper) and isinstance(sim.model.relu3, StaticGridQuantWrapper)
+    assert not isinstance(sim.model.maxpool, quantized)
+    assert not isinstance(sim.model.avgpool, quantized)
+    assert isinstance(sim.model.conv2, quantized) and isinstance(sim.model.relu3, quantized)
     ada_model = ada.Adaround.apply_adaround(model=model, dummy_input=x, params=_params(ada, _loader()),
                                             path=str(tmp_path), filename_prefix='dummy',
                                             ignore_quant_ops_list=[model.relu1, model.bn2])
@@ -372,8 +383,9 @@ def test_compute_recon_loss():                      # test_adaround_loss.py:50-7
 
 
 @pytest.mark.parametrize("warm_start", [1.0, 0.2])  # test_adaround_optimizer.py:62-120
-def test_optimize_layer_rounding(ada, warm_start, tmp_path):
+def test_optimize_layer_rounding(warm_start, tmp_path):
     from aimet_amd.common import libpymo
+    from aimet_amd.v1.adaround.adaround_weight import Adaround
     from aimet_amd.utils import CachedDataset
     from aimet_amd.v1.adaround.adaround_loss import AdaroundHyperParameters
     from aimet_amd.v1.adaround.adaround_optimizer import AdaroundOptimizer
@@ -385,7 +397,7 @@ def test_optimize_layer_rounding(ada, warm_start, tmp_path):
     quantizer = sim.model.conv1.param_quantizers['weight']
     quantizer.encoding = libpymo.TfEncoding(-127.0 * 0.001551126479, (15 - 127.0) * 0.001551126479, 0.001551126479,
                                             -127.0, 4)
-    with ada.Adaround._replace_quantization_layer(sim.model, "conv1") as adaround_wrapper:
+    with Adaround._replace_quantization_layer(sim.model, "conv1") as adaround_wrapper:   # pylint: disable=protected-access
         alpha = torch.randn(adaround_wrapper.weight.shape, requires_grad=True, device='cuda')
         adaround_wrapper.alpha = nn.Parameter(alpha)
         before_opt = alpha.detach().clone()
