@@ -24,18 +24,22 @@ def dequantize(tensor, scale, offset, block_size=None):
 
 
 def _parse_args(args, kwargs):
-    """(qmin, qmax, block_size) from any of the three call forms (reference :334-356)."""
-    args = tuple(args) + (None,) * (3 - len(args))
-    first = kwargs.get('qmin', kwargs.get('bitwidth', args[0]))
-    second = kwargs.get('qmax', kwargs.get('signed', args[1]))
-    block_size = kwargs.get('block_size', None) or args[2]
-    if first is None:
-        qmin, qmax = _derive_qmin_qmax(num_steps=kwargs['num_steps'], signed=kwargs['signed'])
-    elif second is None or isinstance(second, bool):
-        qmin, qmax = _derive_qmin_qmax(bitwidth=first, signed=bool(second))
-    else:
-        qmin, qmax = first, second
-    return qmin, qmax, block_size
+    """(qmin, qmax, block_size) from any of the three call forms (reference :334-356): the first grid argument is
+    qmin or the bitwidth, the second qmax or the signed flag -- a bool (or nothing) there means the bitwidth form; with
+    no first argument at all the grid comes from the num_steps / signed keywords."""
+    slots = list(args[:3]) + [None] * max(0, 3 - len(args))
+    for position, names in enumerate((('qmin', 'bitwidth'), ('qmax', 'signed'))):
+        for name in names:
+            if name in kwargs:
+                slots[position] = kwargs[name]
+                break
+    lower, upper = slots[0], slots[1]
+    block_size = kwargs.get('block_size') or slots[2]
+    if lower is None:
+        return (*_derive_qmin_qmax(num_steps=kwargs['num_steps'], signed=kwargs['signed']), block_size)
+    if upper is None or isinstance(upper, bool):
+        return (*_derive_qmin_qmax(bitwidth=lower, signed=bool(upper)), block_size)
+    return lower, upper, block_size
 
 
 def _derive_qmin_qmax(*, bitwidth: int = None, num_steps: int = None, signed: bool):

@@ -1,0 +1,145 @@
+"""Training through the v2 simulation model, after the reference's
+TrainingExtensions/torch/test/python/v2/ab_test/test_quantsim_qat.py: which parameters ask for gradients under each quant
+scheme (:146-171), the gradients of the whole model against a quantize-dequantize written in plain torch operations with
+a straight-through round and differentiated by autograd (:174-203, :62-81), gradient accumulation (:205-224), one SGD
+step (:226-258), and the plain-torch formula against the blockwise kernel (:283-293).
+
+The reference runs these on torchvision's resnet18, which this image does not ship; the residual model of the
+configurator tests stands in (convolutions, batch norms, an element-wise add, pooling, a linear layer).  The data-parallel
+case needs a second GPU and is left out.
+"""
+import pytest
+import torch
+
+from test_gpu_reference_cases_quantsim_config import SingleResidual
+
+pytestmark = pytest.mark.gpu
+
+CONFIG = {"defaults": {"ops": {"is_output_quantized": "True", "is_symmetric": "False"},
+                       "params": {"is_quantized": "True", "is_symmetric": "True"}},
+          "params": {}, "op_type": {}, "supergroups": [], "model_input": {"is_input_quantized": "True"},
+          "model_output": {}}
+
+_SCHEMES = ("tf", "range_learning")
+
+
+def _scheme(name):
+    from aimet_amd.common.defs import QuantScheme
+    return QuantScheme.post_training_tf if name == "tf" else QuantScheme.training_range_learning_with_tf_init
+
+
+class _StraightThroughRound(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):                                            # pylint: disable=arguments-differ
+        return torch.round(x)
+
+    @staticmethod
+    def backward(ctx, grad):                                        # pylint: disable=arguments-differ
+        return grad
+
+
+def _plain_torch_qdq(tensor, scale, offset, qmin, qmax, block_size=None):
+    """The quantize-dequantize formula in torch operations; autograd differentiates it."""
+    from aimet_amd.v2.utils import get_encoding_shape_with_blocks, reshape_tensor_for_blocks
+    shape = tensor.shape
+    tensor = reshape_tensor_for_blocks(tensor, scale.shape, block_size)
+    scale = scale.view(get_encoding_shape_with_blocks(scale.shape, block_size))
+    offset = offset.view(get_encoding_shape_with_blocks(offset.shape, block_size))
+    on_grid = torch.clamp(_StraightThroughRound.apply(tensor / scale) - offset, qmin, qmax)
+    return ((on_grid + offset) * scale).view(shape)
+
+
+def _calibrated(quant_scheme, seed=0):
+    from aimet_amd.v2.quantsim import QuantizationSimModel
+    torch.manual_seed(seed)
+    model = SingleResidual().cuda()
+    x = torch.randn(4, 3, 32, 32).cuda()
+    sim = QuantizationSimModel(model, x, _scheme(quant_scheme), config_file=CONFIG, default_param_bw=8,
+                               default_output_bw=4)
+    sim.compute_encodings(lambda m, _: m(x), None)
+    return sim, x
+
+
+def _quantizers_of(module):
+    return [q for q in list(module.input_quantizers) + list(module.output_quantizers) +
+            list(module.param_quantizers.values()) if q is not None]
+
+
+@pytest.mark.parametrize("quant_scheme", _SCHEMES)
+def test_which_parameters_ask_for_gradients(quant_scheme):
+    sim, _ = _calibrated(quant_scheme)
+    modules = [m for _, m in sim.qmodules()]
+    assert modules
+    seen_ranges = 0
+    for module in modules:
+        ranges = {id(p) for q in _quantizers_of(module) for p in (q.min, q.max)}
+        for _, param in module.named_parameters():
+            if id(param) in ranges:
+                seen_ranges += 1
+                assert param.requires_grad == (quant_scheme == "range_learning")
+            else:
+                assert param.requires_grad
+    assert seen_ranges > 0
+
+
+@pytest.mark.parametrize("quant_scheme", _SCHEMES)
+def test_gradients_against_autograd(quant_scheme, monkeypatch):
+    from aimet_amd.v2.quantization.affine import quantizer as quantizer_module
+    with_kernels, x = _calibrated(quant_scheme)
+    with_autograd, _ = _calibrated(quant_scheme)
+    with_kernels.model.train()
+    with_autograd.model.train()
+    out = with_kernels.model(x)
+    out.sum().backward()
+    monkeypatch.setattr(quantizer_module, "quantize_dequantize", _plain_torch_qdq)
+    expected = with_autograd.model(x)
+    expected.sum().backward()
+    monkeypatch.undo()
+    assert torch.equal(out, expected)                               # the same arithmetic, to the bit
+    compared = 0
+    theirs = dict(with_autograd.model.named_parameters())
+    for name, param in with_kernels.model.named_parameters():
+        if not param.requires_grad and not theirs[name].requires_grad:
+            continue
+        assert torch.allclose(param.grad, theirs[name].grad, rtol=1e-3, atol=1e-3), name
+        compared += 1
+    assert compared > (20 if quant_scheme == "range_learning" else 10)
+
+
+@pytest.mark.parametrize("quant_scheme", _SCHEMES)
+def test_gradients_accumulate(quant_scheme):
+    sim, x = _calibrated(quant_scheme)
+    sim.model(x).sum().backward()
+    first = {n: p.grad.clone() for n, p in sim.model.named_parameters() if p.requires_grad}
+    sim.model(x).sum().backward()
+    for name, param in sim.model.named_parameters():
+        if param.requires_grad:
+            # convolution backward sums in an order that differs from run to run: twice the first gradient, to rounding
+            assert torch.allclose(2 * first[name], param.grad, rtol=1e-4, atol=1e-5), name
+
+
+@pytest.mark.parametrize("quant_scheme", _SCHEMES)
+def test_one_sgd_step(quant_scheme):
+    sim, x = _calibrated(quant_scheme)
+    before = {n: p.clone() for n, p in sim.model.named_parameters() if p.requires_grad}
+    rate = 0.01
+    optimizer = torch.optim.SGD(sim.model.parameters(), lr=rate)
+    sim.model(x).sum().backward()
+    grads = {n: p.grad.clone() for n, p in sim.model.named_parameters() if p.requires_grad}
+    optimizer.step()
+    for name, param in sim.model.named_parameters():
+        if param.requires_grad:
+            assert torch.allclose(param, before[name] - rate * grads[name]), name
+    assert torch.isfinite(sim.model(x)).all()                       # the moved weights and ranges are used as they are
+
+
+def test_plain_torch_formula_equals_the_blockwise_kernel():
+    from aimet_amd.v2.quantization import affine
+    torch.manual_seed(0)
+    tensor = torch.randn(4, 8, 12).cuda()
+    block_size = [2, 4, 3]
+    scale = torch.randn(2, 2, 4).cuda()
+    offset = torch.randint(low=-128, high=127, size=(2, 2, 4)).to(scale.dtype).cuda()
+    expected = _plain_torch_qdq(tensor, scale, offset, 0, 255, block_size)
+    out = affine.quantize_dequantize(tensor, scale, offset, bitwidth=8, signed=False, block_size=block_size)
+    assert torch.equal(expected, out)
