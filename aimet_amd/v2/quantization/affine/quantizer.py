@@ -21,6 +21,7 @@ from ...utils import (StatisticsNotFoundError, _is_expandable, get_encoding_shap
 from ..base import QuantizerBase
 from ..encoding_analyzer import EncodingAnalyzer, MinMaxEncodingAnalyzer
 from .backends import _derive_qmin_qmax, quantize, quantize_dequantize
+from .encoding import AffineEncoding, _GridMixin
 
 
 _pending_range_checks = None     # a list while batched_range_checks() is active
@@ -65,30 +66,6 @@ def batched_range_checks():
             _examine_bounds(torch.cat(tensors).cpu(), dtype)
 
 
-class _AffineEncoding:
-    """Value object returned by get_encoding(): scale, offset, grid."""
-
-    def __init__(self, scale, offset, qmin, qmax, symmetry, block_size=None):
-        self.scale, self.offset, self.qmin, self.qmax = scale, offset, qmin, qmax
-        self.symmetry, self.block_size = symmetry, block_size
-
-    @property
-    def num_steps(self):
-        return self.qmax - self.qmin
-
-    @property
-    def bitwidth(self):
-        return (self.qmax - self.qmin).bit_length()
-
-    @property
-    def min(self):
-        return self.scale * (self.offset + self.qmin)
-
-    @property
-    def max(self):
-        return self.scale * (self.offset + self.qmax)
-
-
 def _grid_arguments(owner: str, args, kwargs):
     """(qmin, qmax, symmetric, encoding_analyzer, block_size) from either call form of the constructor
     (reference affine/quantizer.py:91-140):
@@ -114,7 +91,7 @@ def _grid_arguments(owner: str, args, kwargs):
                         f"optionally followed by encoding_analyzer and block_size: {error}") from None
 
 
-class MinMaxQuantizer(QuantizerBase):
+class MinMaxQuantizer(_GridMixin, QuantizerBase):
     """Affine quantizer with min / max as trainable parameters."""
 
     def __init__(self, shape, *args, **kwargs):
@@ -151,49 +128,7 @@ class MinMaxQuantizer(QuantizerBase):
     def symmetric(self, symmetric: bool):
         self._symmetric = symmetric
 
-    def _grid_is_regular(self) -> bool:
-        return self.qmin + self.qmax == -1 or self.qmin == 0
-
-    @property
-    def bitwidth(self) -> int:
-        """B such that the grid is [0, 2^B - 1] or [-2^(B-1), 2^(B-1) - 1]; undefined for other grids
-        (reference affine/_utils.py:89-144)."""
-        if self._grid_is_regular():
-            bitwidth = math.log2(self.qmax - self.qmin + 1)
-            if bitwidth == int(bitwidth):
-                return int(bitwidth)
-        raise RuntimeError(f"bitwidth is undefined for a quantization grid of [{self.qmin}, {self.qmax}]")
-
-    @bitwidth.setter
-    def bitwidth(self, bitwidth: int):
-        if bitwidth == int(bitwidth):
-            bitwidth = int(bitwidth)
-        if not isinstance(bitwidth, int):
-            raise TypeError(f"Setting bitwidth to a non-integer value {bitwidth:.3f} is not supported; set "
-                            f"{type(self).__qualname__}.qmin and .qmax instead.")
-        if bitwidth < 1:
-            raise ValueError(f"Bitwidth can't be smaller than 1. Got {bitwidth}")
-        if self.qmin + self.qmax == -1:
-            self.qmin, self.qmax = -2 ** (bitwidth - 1), 2 ** (bitwidth - 1) - 1
-        elif self.qmin == 0:
-            self.qmin, self.qmax = 0, 2 ** bitwidth - 1
-        else:
-            raise RuntimeError(f"bitwidth is undefined for a quantization grid of [{self.qmin}, {self.qmax}]")
-
-    @property
-    def signed(self) -> bool:
-        if self._grid_is_regular():
-            return self.qmin < 0 <= self.qmax
-        raise RuntimeError(f"signed is undefined for a quantization grid of [{self.qmin}, {self.qmax}]")
-
-    @signed.setter
-    def signed(self, signed: bool):
-        """Shifts the grid between [0, 2^B - 1] and [-2^(B-1), 2^(B-1) - 1] (reference affine/_utils.py:170-188)."""
-        bitwidth = self.bitwidth
-        if signed:
-            self.qmin, self.qmax = -2 ** (bitwidth - 1), 2 ** (bitwidth - 1) - 1
-        else:
-            self.qmin, self.qmax = 0, 2 ** bitwidth - 1
+    # bitwidth / signed: views of (qmin, qmax), from _GridMixin
 
     # A parameter counts as initialised once it is no longer the untouched object it was created as: it has been
     # assigned anew, or modified in place (its version counter moved) -- reference base/quantizer.py:100-140.
@@ -324,7 +259,7 @@ class MinMaxQuantizer(QuantizerBase):
             return None
         return self.get_scale(dtype) * (self.get_offset(dtype) + self.qmax)
 
-    def get_encoding(self) -> Optional[_AffineEncoding]:
+    def get_encoding(self) -> Optional[AffineEncoding]:
         if not self.is_initialized():
             return None
         # Scale and offset are a handful of parameter-sized tensor operations per call (the reference performs them in
@@ -345,7 +280,7 @@ class MinMaxQuantizer(QuantizerBase):
                 with torch.no_grad():
                     scale, offset = scale.detach(), offset.detach()
                 self.__dict__['_kept_encoding'] = (key, mn, mx, scale, offset)
-        return _AffineEncoding(scale, offset, self.qmin, self.qmax, self._symmetric, self.block_size)
+        return AffineEncoding._on_grid(scale, offset, self.qmin, self.qmax, self._symmetric, self.block_size)  # pylint: disable=protected-access
 
     def lower_bound_is_zero(self) -> bool:
         """True when the kept encoding's grid starts exactly at zero (offset == -qmin everywhere), known on the host:
