@@ -78,6 +78,9 @@ _SIGNATURES = {
     "miq_v2_qdq_bwd_params_workspace_bytes": ([_i64, _i64, _i64], _i64),
     "miq_v2_qdq_bwd_params_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p, _p, _p, _p], _int),
     "miq_v2_qdq_bwd_params_bf16": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p, _p, _p, _p], _int),
+    "miq_range_to_grid_f32": ([_p, _p, _i64, _int, _int, _int, _int, _p, _p], _int),
+    "miq_qdq_bwd_range_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _int, _int, _int, _p, _p, _p, _p], _int),
+    "miq_qdq_bwd_range_bf16": ([_p, _p, _p, _i64, _i64, _i64, _p, _int, _int, _int, _p, _p, _p, _p], _int),
     "miq_fp16_round_trip_f32": ([_p, _p, _i64, _p], _int),
     "miq_bf16_round_trip_f32": ([_p, _p, _i64, _p], _int),
     "miq_fp8_fake_cast_f32": ([_p, _p, _i64, _i64, _i64, _p, _p, _p, _int, _p], _int),

@@ -46,6 +46,65 @@ struct LearnGeom
 
 constexpr int64_t kShortRow = 2048;
 
+// What becomes of a channel's two sums.  mode < 0: they are the results (scale_grad, offset_grad).  Otherwise they
+// are turned into the gradients of the encoding min / max the grid was made from, and those are stored in their place
+// (the formulas are stated with the modes in miq.h).
+struct RangeGrads
+{
+    int mode;
+    const float* enc_min;
+    const float* enc_max;
+    float steps;        // qmax - qmin
+    float steps_rcp;    // float32(1 / steps)
+    float half_steps;   // steps div 2
+};
+
+__device__ __forceinline__ void store_sums(const RangeGrads& r, const float* __restrict__ scale, uint32_t ch,
+                                           uint32_t at, float sum_s, float sum_o, float* __restrict__ out_a,
+                                           float* __restrict__ out_b)
+{
+    if (r.mode < 0)
+    {
+        if (out_a)
+            out_a[at] = sum_s;
+        if (out_b)
+            out_b[at] = sum_o;
+        return;
+    }
+    const float mn = r.enc_min[ch], mx = r.enc_max[ch];
+    float gmin, gmax;
+    switch (r.mode)
+    {
+    case MIQ_RANGE_V2_ASYMMETRIC:
+    {
+        const float sc = scale[ch];
+        const float s  = sum_s + -sum_o * ((mn / sc) / sc);
+        gmax           = s * r.steps_rcp;
+        gmin           = sum_o / sc + -gmax;
+        break;
+    }
+    case MIQ_RANGE_V2_SYMMETRIC:
+        gmax = sum_s * r.steps_rcp;
+        gmin = -gmax;
+        break;
+    case MIQ_RANGE_V1_ASYMMETRIC:
+    {
+        const float t1 = sum_s / r.steps;
+        const float d  = mx - mn;
+        const float t2 = r.steps / (d * d) * sum_o;
+        gmin           = -t1 + mx * t2;
+        gmax           = t1 - mn * t2;
+        break;
+    }
+    default:   // the two v1 symmetric modes
+        gmax = sum_s / r.half_steps;
+        gmin = -gmax;
+        break;
+    }
+    out_a[at] = gmin;
+    out_b[at] = gmax;
+}
+
 struct LearnParams
 {
     float scale, offset, rcp, lo, hi, qmin, qmax;
@@ -124,7 +183,7 @@ __global__ __launch_bounds__(kBlock) void learn_bwd_kernel(const IO* __restrict_
                                                            const float* __restrict__ offset, int qmin, int qmax,
                                                            LearnGeom geo, float2* __restrict__ partial,
                                                            float* __restrict__ scale_grad,
-                                                           float* __restrict__ offset_grad)
+                                                           float* __restrict__ offset_grad, RangeGrads range)
 {
     using T              = IOTraits<IO>;
     const uint32_t row   = fastdiv(blockIdx.x, geo.chunks_div);
@@ -238,13 +297,8 @@ __global__ __launch_bounds__(kBlock) void learn_bwd_kernel(const IO* __restrict_
             a += wave_sum[w].x;
             b += wave_sum[w].y;
         }
-        if (geo.direct)
-        {
-            if (scale_grad)
-                scale_grad[blockIdx.x] = a;
-            if (offset_grad)
-                offset_grad[blockIdx.x] = b;
-        }
+        if (geo.direct)   // one workgroup per channel, outer == 1: the block number is the channel
+            store_sums(range, scale, blockIdx.x, blockIdx.x, a, b, scale_grad, offset_grad);
         else
             partial[blockIdx.x] = make_float2(a, b);
     }
@@ -255,8 +309,9 @@ __global__ __launch_bounds__(kBlock) void learn_bwd_kernel(const IO* __restrict_
 // tree over the lanes -- the result does not depend on scheduling.
 template <int LANES>
 __global__ __launch_bounds__(kBlock) void learn_reduce_kernel(const float2* __restrict__ partial, LearnGeom geo,
+                                                              const float* __restrict__ scale,
                                                               float* __restrict__ scale_grad,
-                                                              float* __restrict__ offset_grad)
+                                                              float* __restrict__ offset_grad, RangeGrads range)
 {
     constexpr int kPerBlock = kBlock / LANES;
     const uint32_t ch       = blockIdx.x * kPerBlock + threadIdx.x / LANES;
@@ -298,12 +353,7 @@ __global__ __launch_bounds__(kBlock) void learn_reduce_kernel(const float2* __re
         }
     }
     if (lane == 0 && ch < geo.num_channel)
-    {
-        if (scale_grad)
-            scale_grad[ch] = (float) a;
-        if (offset_grad)
-            offset_grad[ch] = (float) b;
-    }
+        store_sums(range, scale, ch, ch, (float) a, (float) b, scale_grad, offset_grad);
 }
 
 // Short rows.  A group of geo.lanes lanes owns a row at a time; a workgroup owns rows_per_block consecutive rows, so
@@ -315,7 +365,7 @@ __global__ __launch_bounds__(kBlock) void learn_rows_kernel(const IO* __restrict
                                                             const float* __restrict__ offset, int qmin, int qmax,
                                                             LearnGeom geo, float2* __restrict__ partial,
                                                             float* __restrict__ scale_grad,
-                                                            float* __restrict__ offset_grad)
+                                                            float* __restrict__ offset_grad, RangeGrads range)
 {
     using T                 = IOTraits<IO>;
     constexpr int V         = VECTOR ? T::VEC : 1;
@@ -388,13 +438,8 @@ __global__ __launch_bounds__(kBlock) void learn_rows_kernel(const IO* __restrict
                 if (k == 1 && !two)
                     break;
                 const int64_t row = k ? row1 : row0;
-                if (geo.direct)
-                {
-                    if (scale_grad)
-                        scale_grad[row] = sg[k];
-                    if (offset_grad)
-                        offset_grad[row] = og[k];
-                }
+                if (geo.direct)   // outer == 1: the row number is the channel
+                    store_sums(range, scale, (uint32_t) row, (uint32_t) row, sg[k], og[k], scale_grad, offset_grad);
                 else
                     partial[row] = make_float2(sg[k], og[k]);
             }
@@ -455,7 +500,7 @@ int make_learn_geom(int64_t num_channel, int64_t n, int64_t npc, int vec, LearnG
 template <typename IO>
 int launch_learn(const IO* x, const IO* g, IO* gx, int64_t num_channel, int64_t n, int64_t npc, const float* scale,
                  const float* offset, int qmin, int qmax, float* scale_grad, float* offset_grad, void* workspace,
-                 hipStream_t stream)
+                 hipStream_t stream, const RangeGrads& range)
 {
     MIQ_CHECK_ARG(scale && offset, "null parameter pointer");
     MIQ_CHECK_ARG(qmin <= qmax, "qmin must not exceed qmax");
@@ -472,7 +517,7 @@ int launch_learn(const IO* x, const IO* g, IO* gx, int64_t num_channel, int64_t 
     {
 #define MIQ_LEARN(KERNEL, V, W)                                                                                        \
     KERNEL<IO, V, W><<<grid, kBlock, 0, stream>>>(x, g, gx, scale, offset, qmin, qmax, geo, partial, scale_grad,       \
-                                                  offset_grad)
+                                                  offset_grad, range)
 #define MIQ_LEARN_VARIANTS(KERNEL)                                                                                     \
     if (vector && gx)                                                                                                  \
         MIQ_LEARN(KERNEL, true, true);                                                                                 \
@@ -499,15 +544,104 @@ int launch_learn(const IO* x, const IO* g, IO* gx, int64_t num_channel, int64_t 
     if (!geo.direct)
     {
         if ((int64_t) geo.outer * geo.chunks >= 1024)
-            learn_reduce_kernel<kBlock><<<dim3(geo.num_channel), kBlock, 0, stream>>>(partial, geo, scale_grad,
-                                                                                      offset_grad);
+            learn_reduce_kernel<kBlock><<<dim3(geo.num_channel), kBlock, 0, stream>>>(partial, geo, scale, scale_grad,
+                                                                                      offset_grad, range);
         else
-            learn_reduce_kernel<64><<<dim3((geo.num_channel + 3) / 4), kBlock, 0, stream>>>(partial, geo, scale_grad,
-                                                                                            offset_grad);
+            learn_reduce_kernel<64><<<dim3((geo.num_channel + 3) / 4), kBlock, 0, stream>>>(
+                partial, geo, scale, scale_grad, offset_grad, range);
         MIQ_CHECK_LAUNCH();
     }
     return MIQ_OK;
 }
+constexpr RangeGrads kNoRange = {-1, nullptr, nullptr, 0.f, 0.f, 0.f};
+
+int make_range(RangeGrads& r, int mode, int qmin, int qmax, const float* grid, int64_t num_channel)
+{
+    MIQ_CHECK_ARG(mode >= MIQ_RANGE_V2_ASYMMETRIC && mode <= MIQ_RANGE_V1_UNSIGNED_SYMMETRIC, "unknown range mode %d",
+                  mode);
+    MIQ_CHECK_ARG(qmin < qmax, "qmin must be below qmax");
+    MIQ_CHECK_ARG(mode < MIQ_RANGE_V1_ASYMMETRIC || qmin == 0, "the v1 grids start at 0 (qmin = %d)", qmin);
+    MIQ_CHECK_ARG((int64_t) qmax - qmin < (1 << 24), "grid too wide for float32 (%d..%d)", qmin, qmax);
+    r.mode       = mode;
+    r.enc_min    = grid ? grid + 2 * num_channel : nullptr;
+    r.enc_max    = grid ? grid + 3 * num_channel : nullptr;
+    r.steps      = (float) (qmax - qmin);
+    r.steps_rcp  = 1.0f / r.steps;
+    r.half_steps = (float) ((qmax - qmin) / 2);
+    return MIQ_OK;
+}
+
+// torch.clamp / torch.maximum keep NaN
+__device__ __forceinline__ float max_keep_nan(float a, float b)
+{
+    return (a != a || b != b) ? NAN : fmaxf(a, b);
+}
+
+// One thread per channel: the range is put in order (gate), copied, and turned into scale and offset.
+__global__ __launch_bounds__(kBlock) void range_to_grid_kernel(float* __restrict__ enc_min, float* __restrict__ enc_max,
+                                                               int num_channel, float qmin, RangeGrads r, bool gate,
+                                                               float* __restrict__ grid)
+{
+    const int ch = blockIdx.x * kBlock + threadIdx.x;
+    if (ch >= num_channel)
+        return;
+    float mn = enc_min[ch], mx = enc_max[ch];
+    if (gate)
+    {
+        mn = (mn > 0.0f) ? 0.0f : mn;   // clamp_(max=0): a NaN compares false and stays
+        mx = (mx < 0.0f) ? 0.0f : mx;
+        mx = max_keep_nan(mx, mn + 1e-5f);
+        enc_min[ch] = mn;
+        enc_max[ch] = mx;
+    }
+    float scale, offset;
+    switch (r.mode)
+    {
+    case MIQ_RANGE_V2_ASYMMETRIC:
+        scale  = (mx - mn) * r.steps_rcp;
+        offset = rintf(mn / scale) - qmin;
+        break;
+    case MIQ_RANGE_V2_SYMMETRIC:
+        scale  = (mx - mn) * r.steps_rcp;
+        offset = 0.0f;
+        break;
+    case MIQ_RANGE_V1_ASYMMETRIC:
+    {
+        scale   = (mx - mn) / r.steps;
+        float z = rintf(-mn / scale);                 // torch.min(steps, torch.max(0, z)): NaN stays
+        z       = max_keep_nan(0.0f, z);
+        z       = (z != z) ? z : fminf(r.steps, z);
+        offset  = -z;
+        break;
+    }
+    case MIQ_RANGE_V1_SIGNED_SYMMETRIC:
+        scale  = mx / r.half_steps;                   // floor(steps / 2)
+        offset = -(r.steps - r.half_steps);           // -ceil(steps / 2)
+        break;
+    default:   // MIQ_RANGE_V1_UNSIGNED_SYMMETRIC
+        scale  = (mx - mn) / r.steps;
+        offset = mn / scale;
+        break;
+    }
+    grid[ch]                   = scale;
+    grid[num_channel + ch]     = offset;
+    grid[2 * num_channel + ch] = mn;
+    grid[3 * num_channel + ch] = mx;
+}
+template <typename IO>
+int bwd_range(const IO* x, const IO* grad_out, IO* grad_in, int64_t num_channel, int64_t num_element,
+                     int64_t num_element_per_channel, const float* grid, int qmin, int qmax, int mode, float* grad_min,
+                     float* grad_max, void* workspace, void* stream)
+{
+    MIQ_CHECK_ARG(grid && grad_min && grad_max, "null pointer");
+    MIQ_CHECK_ARG(num_channel >= 1, "bad channel count");
+    RangeGrads r;
+    if (int rc = make_range(r, mode, qmin, qmax, grid, num_channel))
+        return rc;
+    return launch_learn<IO>(x, grad_out, grad_in, num_channel, num_element, num_element_per_channel, grid,
+                            grid + num_channel, qmin, qmax, grad_min, grad_max, workspace, (hipStream_t) stream, r);
+}
+
 }   // namespace
 }   // namespace miq
 
@@ -532,7 +666,7 @@ int miq_v2_qdq_bwd_params_f32(const float* x, const float* grad_out, float* grad
                               void* workspace, void* stream)
 {
     return launch_learn<float>(x, grad_out, grad_in, num_channel, num_element, num_element_per_channel, scale, offset,
-                               qmin, qmax, scale_grad, offset_grad, workspace, (hipStream_t) stream);
+                               qmin, qmax, scale_grad, offset_grad, workspace, (hipStream_t) stream, kNoRange);
 }
 
 int miq_v2_qdq_bwd_params_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* grad_in, int64_t num_channel,
@@ -541,7 +675,39 @@ int miq_v2_qdq_bwd_params_bf16(const uint16_t* x, const uint16_t* grad_out, uint
                                void* workspace, void* stream)
 {
     return launch_learn<uint16_t>(x, grad_out, grad_in, num_channel, num_element, num_element_per_channel, scale,
-                                  offset, qmin, qmax, scale_grad, offset_grad, workspace, (hipStream_t) stream);
+                                  offset, qmin, qmax, scale_grad, offset_grad, workspace, (hipStream_t) stream,
+                                  kNoRange);
+}
+
+int miq_range_to_grid_f32(float* enc_min, float* enc_max, int64_t num_channel, int qmin, int qmax, int mode, int gate,
+                          float* grid, void* stream)
+{
+    MIQ_CHECK_ARG(num_channel >= 1 && num_channel <= 0x7fffffff, "bad channel count %lld", (long long) num_channel);
+    MIQ_CHECK_ARG(enc_min && enc_max && grid, "null pointer");
+    RangeGrads r;
+    if (int rc = make_range(r, mode, qmin, qmax, nullptr, num_channel))
+        return rc;
+    const dim3 blocks((uint32_t) ((num_channel + kBlock - 1) / kBlock));
+    range_to_grid_kernel<<<blocks, kBlock, 0, (hipStream_t) stream>>>(enc_min, enc_max, (int) num_channel,
+                                                                      (float) qmin, r, gate != 0, grid);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int miq_qdq_bwd_range_f32(const float* x, const float* grad_out, float* grad_in, int64_t num_channel,
+                          int64_t num_element, int64_t num_element_per_channel, const float* grid, int qmin, int qmax,
+                          int mode, float* grad_min, float* grad_max, void* workspace, void* stream)
+{
+    return bwd_range<float>(x, grad_out, grad_in, num_channel, num_element, num_element_per_channel, grid, qmin, qmax,
+                            mode, grad_min, grad_max, workspace, stream);
+}
+
+int miq_qdq_bwd_range_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* grad_in, int64_t num_channel,
+                           int64_t num_element, int64_t num_element_per_channel, const float* grid, int qmin,
+                           int qmax, int mode, float* grad_min, float* grad_max, void* workspace, void* stream)
+{
+    return bwd_range<uint16_t>(x, grad_out, grad_in, num_channel, num_element, num_element_per_channel, grid, qmin,
+                               qmax, mode, grad_min, grad_max, workspace, stream);
 }
 
 }   // extern "C"

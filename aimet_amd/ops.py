@@ -510,6 +510,51 @@ def v2_qdq_bwd_params(x, grad_out, num_channel, n_per_channel, scale, offset, qm
     return gin, grads[0], grads[1]
 
 
+# ---------------------------------------------------------------------------------------------------- range learning
+RANGE_V2_ASYMMETRIC, RANGE_V2_SYMMETRIC, RANGE_V1_ASYMMETRIC, RANGE_V1_SIGNED_SYMMETRIC, \
+    RANGE_V1_UNSIGNED_SYMMETRIC = range(5)
+
+
+def range_to_grid(enc_min, enc_max, qmin, qmax, mode, gate=False):
+    """float32 device tensor [4, C]: scale, offset and the encoding min / max they were made from, for the learnable
+    float32 min / max tensors of one quantizer (C elements each, contiguous).  gate=True first puts min <= 0 <= max and
+    max >= min + 1e-5 into the two tensors themselves, the way the v1 wrappers order their ranges before a forward
+    pass; their version counters are moved, as an in-place torch operation would move them."""
+    _require_gpu(enc_min, enc_max)
+    if enc_min.dtype != _F32 or enc_max.dtype != _F32 or not enc_min.is_contiguous() or not enc_max.is_contiguous() \
+            or enc_min.numel() != enc_max.numel():
+        raise ValueError("encoding min / max must be contiguous float32 tensors of one size")
+    c = enc_min.numel()
+    grid = torch.empty(4, c, dtype=_F32, device=enc_min.device)
+    with _OnDevice(enc_min.device):
+        check(lib.miq_range_to_grid_f32(_ptr(enc_min), _ptr(enc_max), c, int(qmin), int(qmax), int(mode),
+                                        1 if gate else 0, _ptr(grid), _stream(enc_min)))
+    if gate:
+        torch.autograd.graph.increment_version(enc_min)
+        torch.autograd.graph.increment_version(enc_max)
+    return grid
+
+
+def qdq_bwd_range(x, grad_out, num_channel, n_per_channel, grid, qmin, qmax, mode, want_grad_in=True):
+    """(grad_in or None, grad_min[C], grad_max[C]) of a quantize-dequantize whose grid range_to_grid() made: the
+    backward pass over x and grad_out, the channel sums and their conversion into the gradients of the encoding
+    min / max, in the two launches of v2_qdq_bwd_params (one where a channel is a single workgroup's work)."""
+    _require_gpu(x, grad_out, grid)
+    x, grad_out = x.contiguous(), grad_out.to(x.dtype).contiguous()
+    c, npc = int(num_channel), int(n_per_channel)
+    if grid.dtype != _F32 or tuple(grid.shape) != (4, c) or not grid.is_contiguous():
+        raise ValueError(f"grid must be the contiguous float32 [4, {c}] tensor of range_to_grid()")
+    gin = torch.empty_like(x) if want_grad_in else None
+    grads = torch.empty(2, c, dtype=_F32, device=x.device)
+    ws = torch.empty(int(lib.miq_v2_qdq_bwd_params_workspace_bytes(c, x.numel(), npc)), dtype=torch.uint8,
+                     device=x.device)
+    fn = getattr(lib, "miq_qdq_bwd_range_" + _suffix(x))
+    with _OnDevice(x.device):
+        check(fn(_ptr(x), _ptr(grad_out), _ptr(gin) if want_grad_in else None, c, x.numel(), npc, _ptr(grid),
+                 int(qmin), int(qmax), int(mode), _ptr(grads[0]), _ptr(grads[1]), _ptr(ws), _stream(x)))
+    return gin, grads[0], grads[1]
+
+
 # -------------------------------------------------------------------------------------------------------- statistics
 def _minmax_workspace(num_channel, n, n_per_channel, device):
     nbytes = int(lib.miq_minmax_workspace_bytes(int(num_channel), int(n), int(n_per_channel)))

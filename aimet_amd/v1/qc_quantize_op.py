@@ -632,8 +632,13 @@ class LearnedGridQuantWrapper(QcQuantizeWrapper):
         """Keeps every learned range ordered around zero before it is used (min <= 0 <= max, max > min)."""
         for name, quantizer in self._named_quantizers():
             if quantizer.enabled and quantizer.bitwidth != 32 and quantizer.data_type != QuantizationDataType.float:
-                set_encoding_min_max_gating_threshold(getattr(self, name + '_encoding_min'),
-                                                      getattr(self, name + '_encoding_max'))
+                encoding_min = getattr(self, name + '_encoding_min')
+                encoding_max = getattr(self, name + '_encoding_max')
+                if ste.grid_in_one_launch(encoding_min, encoding_max):
+                    # the same launch leaves delta / offset of the ordered range for the forward pass that follows
+                    ste.gate_and_prepare_grid(quantizer, encoding_min, encoding_max)
+                else:
+                    set_encoding_min_max_gating_threshold(encoding_min, encoding_max)
 
     def forward(self, *inputs, **kwargs):
         self.apply_gating_logic()

@@ -67,7 +67,8 @@ def get_computed_encodings(bitwidth, encoding_min, encoding_max, use_symmetric_e
     half = num_steps / 2
     steps = torch.full_like(encoding_min, float(num_steps))
     if use_symmetric_encodings and not is_unsigned_symmetric:
-        delta = encoding_max / float(math.floor(half))
+        # a tensor as divisor, as in the reference: torch's device kernels multiply by the reciprocal of a number
+        delta = encoding_max / torch.full_like(encoding_min, float(math.floor(half)))
         offset = torch.full_like(encoding_min, -float(math.ceil(half)))
     else:
         delta = (encoding_max - encoding_min) / steps
@@ -85,11 +86,52 @@ def _channel_geometry(tensor, num_param, ch_axis):
     return num_param, max(math.prod(tensor.shape[ch_axis + 1:]), 1)
 
 
+def range_mode(tensor_quantizer) -> int:
+    """Which of the library's grid formulas a learned-grid quantizer follows (get_computed_encodings' three cases)."""
+    if tensor_quantizer.use_symmetric_encodings:
+        return ops.RANGE_V1_UNSIGNED_SYMMETRIC if tensor_quantizer.is_unsigned_symmetric \
+            else ops.RANGE_V1_SIGNED_SYMMETRIC
+    return ops.RANGE_V1_ASYMMETRIC
+
+
+def _grid_key(tensor_quantizer, encoding_min, encoding_max):
+    # pylint: disable=protected-access
+    return (id(encoding_min), encoding_min._version, id(encoding_max), encoding_max._version,
+            tensor_quantizer.bitwidth, range_mode(tensor_quantizer), tensor_quantizer.use_strict_symmetric,
+            ops.current_stream_handle(encoding_min.device))
+
+
+def grid_in_one_launch(encoding_min, encoding_max) -> bool:
+    """The library forms delta / offset itself for float32 ranges held contiguously on the GPU."""
+    return encoding_min is not None and encoding_max is not None and encoding_min.is_cuda and \
+        encoding_min.dtype == encoding_max.dtype == torch.float32 and encoding_min.is_contiguous() and \
+        encoding_max.is_contiguous() and encoding_min.numel() == encoding_max.numel() and \
+        encoding_min.device == encoding_max.device
+
+
+def gate_and_prepare_grid(tensor_quantizer, encoding_min, encoding_max):
+    """The wrapper's ordering of a learned range (min <= 0 <= max, max >= min + 1e-5), in place, and the grid that
+    range gives -- one launch.  The grid is left with the quantizer for the forward pass that follows."""
+    grid = ops.range_to_grid(encoding_min.detach().reshape(-1), encoding_max.detach().reshape(-1), 0,
+                             _num_steps(tensor_quantizer), range_mode(tensor_quantizer), gate=True)
+    tensor_quantizer.__dict__['_prepared_grid'] = (_grid_key(tensor_quantizer, encoding_min, encoding_max), grid)
+
+
+def _grid_of(tensor_quantizer, encoding_min, encoding_max):
+    prepared = tensor_quantizer.__dict__.pop('_prepared_grid', None)
+    if prepared is not None and prepared[0] == _grid_key(tensor_quantizer, encoding_min, encoding_max):
+        return prepared[1]
+    return ops.range_to_grid(encoding_min.detach().reshape(-1), encoding_max.detach().reshape(-1), 0,
+                             _num_steps(tensor_quantizer), range_mode(tensor_quantizer))
+
+
 def learned_grid_forward(tensor, tensor_quantizer, encoding_min, encoding_max):
     """Forward of range learning (reference calculate_forward_pass :185-249):
     x_dequant = (clamp(round(x / delta) - offset, 0, steps) + offset) * delta, in one kernel.  Returns the output and
-    what backward needs (delta, offset, steps) -- no full-size intermediates are kept: the backward kernel recomputes
-    the grid position and the mask from the saved input."""
+    what backward needs -- no full-size intermediates are kept: the backward kernel recomputes the grid position and
+    the mask from the saved input.  What backward needs is (grid, steps, channels, elements per channel), grid being
+    the library's [4, C] table of delta, offset and the min / max they were made from, or, for ranges the library
+    does not take (not float32, not on the GPU), (delta, offset, steps, channels, elements per channel)."""
     if tensor.dtype not in (torch.float32, torch.float16, torch.bfloat16):
         raise RuntimeError("Invalid input data type. Expected torch.float32 or torch.float16. "
                            f"Got {tensor.dtype}.")
@@ -99,14 +141,19 @@ def learned_grid_forward(tensor, tensor_quantizer, encoding_min, encoding_max):
                            f"and {encoding_max.dtype} encoding_max")
     if tensor_quantizer.bitwidth >= 32:
         raise RuntimeError(f'Invalid bitwidth: {tensor_quantizer.bitwidth}')
-    delta, offset, steps = get_computed_encodings(tensor_quantizer.bitwidth, encoding_min.detach().float(),
-                                                  encoding_max.detach().float(),
-                                                  tensor_quantizer.use_symmetric_encodings,
-                                                  tensor_quantizer.use_strict_symmetric,
-                                                  tensor_quantizer.is_unsigned_symmetric)
     num_steps = _num_steps(tensor_quantizer)
-    c, npc = _channel_geometry(tensor, delta.numel(), tensor_quantizer.channel_axis)
     x = tensor if tensor.dtype != torch.float16 else tensor.float()
+    if grid_in_one_launch(encoding_min, encoding_max) and tensor.is_cuda:
+        grid = _grid_of(tensor_quantizer, encoding_min, encoding_max)
+        c, npc = _channel_geometry(tensor, grid.shape[1], tensor_quantizer.channel_axis)
+        out = ops.v2_qdq(x, c, npc, grid[0], grid[1], 0, num_steps)
+        return out.to(tensor.dtype), (grid, num_steps, c, npc)
+    delta, offset, _ = get_computed_encodings(tensor_quantizer.bitwidth, encoding_min.detach().float(),
+                                              encoding_max.detach().float(),
+                                              tensor_quantizer.use_symmetric_encodings,
+                                              tensor_quantizer.use_strict_symmetric,
+                                              tensor_quantizer.is_unsigned_symmetric)
+    c, npc = _channel_geometry(tensor, delta.numel(), tensor_quantizer.channel_axis)
     out = ops.v2_qdq(x, c, npc, delta, offset, 0, num_steps)
     return out.to(tensor.dtype), (delta, offset, num_steps, c, npc)
 
@@ -128,9 +175,21 @@ def learned_grid_backward(tensor, grad, saved, encoding_min, encoding_max, is_sy
                      d/dmin = -t1 + max * t2,  d/dmax = t1 - min * t2
         symmetric:   d/dmax = S / floor(steps / 2),  d/dmin = -d/dmax
     """
-    delta, offset, num_steps, c, npc = saved
     x = tensor if tensor.dtype != torch.float16 else tensor.float()
     g = grad.to(x.dtype)
+    if len(saved) == 4:
+        # the library's grid: the encoding gradients leave the kernel that adds up the channel sums
+        grid, num_steps, c, npc = saved
+        if not want_encoding_grads:
+            return ops.v2_qdq_bwd(x, g, c, npc, grid[0], grid[1], 0, num_steps).to(tensor.dtype), None, None
+        mode = ops.RANGE_V1_SIGNED_SYMMETRIC if is_symmetric else ops.RANGE_V1_ASYMMETRIC
+        tensor_grad, grad_min, grad_max = ops.qdq_bwd_range(x, g, c, npc, grid, 0, num_steps, mode,
+                                                            want_grad_in=want_tensor_grad)
+        if tensor_grad is not None:
+            tensor_grad = tensor_grad.to(tensor.dtype)
+        return (tensor_grad, grad_min.to(encoding_min.dtype).view_as(encoding_min),
+                grad_max.to(encoding_max.dtype).view_as(encoding_max))
+    delta, offset, num_steps, c, npc = saved
     if not want_encoding_grads:
         return ops.v2_qdq_bwd(x, g, c, npc, delta, offset, 0, num_steps).to(tensor.dtype), None, None
     tensor_grad, s_sum, o_sum = ops.v2_qdq_bwd_params(x, g, c, npc, delta, offset, 0, num_steps,
@@ -138,12 +197,13 @@ def learned_grid_backward(tensor, grad, saved, encoding_min, encoding_max, is_sy
     if tensor_grad is not None:
         tensor_grad = tensor_grad.to(tensor.dtype)
     emin, emax = encoding_min.detach().float().reshape(-1), encoding_max.detach().float().reshape(-1)
+    steps = torch.full_like(s_sum, float(num_steps))      # tensors as divisors, as in the reference
     if is_symmetric:
-        grad_max = s_sum / float(num_steps // 2)
+        grad_max = s_sum / torch.full_like(s_sum, float(num_steps // 2))
         grad_min = -grad_max
     else:
-        term1 = s_sum / float(num_steps)
-        term2 = float(num_steps) / (emax - emin) ** 2 * o_sum
+        term1 = s_sum / steps
+        term2 = steps / (emax - emin) ** 2 * o_sum
         grad_min = -term1 + emax * term2
         grad_max = term1 - emin * term2
     return (tensor_grad, grad_min.to(encoding_min.dtype).view_as(encoding_min),

@@ -850,23 +850,36 @@ class QuantizeDequantizeFunc(torch.autograd.Function):
             raise RuntimeError("Forward pass used for compute_encodings differs from forward pass used during "
                                "training")
         out, saved = grad_fn.learned_grid_forward(tensor, tensor_quantizer, encoding_min, encoding_max)
-        ctx.saved_geometry = saved[2:]
         ctx.is_symmetric = tensor_quantizer.use_symmetric_encodings
         # min / max are saved as copies: the wrapper clamps the parameters in place before every forward, also
-        # between the forward and the backward of a module that is used twice (reference :942-955)
-        ctx.save_for_backward(tensor, saved[0], saved[1], encoding_min.detach().clone(),
-                              encoding_max.detach().clone())
+        # between the forward and the backward of a module that is used twice (reference :942-955).  The library's
+        # grid table holds such copies.
+        if len(saved) == 4:
+            ctx.saved_geometry = saved[1:]
+            ctx.range_shapes = (encoding_min.shape, encoding_max.shape)
+            ctx.save_for_backward(tensor, saved[0])
+        else:
+            ctx.saved_geometry = saved[2:]
+            ctx.save_for_backward(tensor, saved[0], saved[1], encoding_min.detach().clone(),
+                                  encoding_max.detach().clone())
         return out
 
     @staticmethod
     def backward(ctx, grad):  # pylint: disable=arguments-differ
         if ctx.tensor_quantizer.bitwidth == 32:
             return grad, None, None, None
-        tensor, delta, offset, encoding_min, encoding_max = ctx.saved_tensors
         want_enc = ctx.needs_input_grad[1] or ctx.needs_input_grad[2]
+        if len(ctx.saved_tensors) == 2:
+            tensor, grid = ctx.saved_tensors
+            saved, encoding_min, encoding_max = (grid,) + tuple(ctx.saved_geometry), grid[2], grid[3]
+            shapes = ctx.range_shapes
+        else:
+            tensor, delta, offset, encoding_min, encoding_max = ctx.saved_tensors
+            saved, shapes = (delta, offset) + tuple(ctx.saved_geometry), None
         tensor_grad, grad_min, grad_max = grad_fn.learned_grid_backward(
-            tensor, grad, (delta, offset) + tuple(ctx.saved_geometry), encoding_min, encoding_max, ctx.is_symmetric,
-            ctx.needs_input_grad[0], want_enc)
+            tensor, grad, saved, encoding_min, encoding_max, ctx.is_symmetric, ctx.needs_input_grad[0], want_enc)
+        if shapes is not None and grad_min is not None:
+            grad_min, grad_max = grad_min.reshape(shapes[0]), grad_max.reshape(shapes[1])
         if not ctx.needs_input_grad[0]:
             tensor_grad = None
         return tensor_grad, grad_min if ctx.needs_input_grad[1] else None, \

@@ -19,7 +19,8 @@ last varying axis, e.g. weight [out, in] with scale [out, in / block]) without a
 copy each way.
 
 Gradients w.r.t. scale and offset (range learning, :329-344) come from one fused pass over the input and the
-incoming gradient, together with the input gradient.
+incoming gradient, together with the input gradient.  For the quantizer modules, whose scale and offset are functions
+of a learnable min / max, quantize_dequantize_learned_range() takes min / max themselves and returns their gradients.
 """
 import functools
 from typing import List, Optional
@@ -131,6 +132,57 @@ class _QuantDequantFunc(torch.autograd.Function):
         elif ctx.needs_input_grad[0]:
             tensor_grad = ops.v2_qdq_bwd(tensor, grad, c, npc, scale, offset, qmin, qmax)
         return tensor_grad, scale_grad, offset_grad, None, None
+
+
+class _LearnedRangeFunc(torch.autograd.Function):
+    """Quantize-dequantize as a function of (tensor, encoding min, encoding max): the grid is made from min / max by
+    one small launch, and backward returns the gradients of min / max straight from the kernel that reduces the
+    channel sums -- what autograd otherwise assembles from get_scale() / get_offset(), about ten tensor operations of
+    parameter size forward and as many backward, per quantizer and step."""
+
+    @staticmethod
+    def forward(ctx, tensor, enc_min, enc_max, qmin, qmax, symmetric):  # pylint: disable=arguments-differ
+        c, npc = tensor.shape[1], max(tensor.shape[2], 1)
+        mode = ops.RANGE_V2_SYMMETRIC if symmetric else ops.RANGE_V2_ASYMMETRIC
+        grid = ops.range_to_grid(enc_min.reshape(-1), enc_max.reshape(-1), qmin, qmax, mode)
+        ctx.geom = (c, npc, qmin, qmax, mode, enc_min.shape, enc_max.shape)
+        ctx.save_for_backward(tensor, grid)
+        return ops.v2_qdq(tensor, c, npc, grid[0], grid[1], qmin, qmax)
+
+    @staticmethod
+    def backward(ctx, grad):  # pylint: disable=arguments-differ
+        tensor, grid = ctx.saved_tensors
+        c, npc, qmin, qmax, mode, min_shape, max_shape = ctx.geom
+        tensor_grad, grad_min, grad_max = ops.qdq_bwd_range(tensor, grad, c, npc, grid, qmin, qmax, mode,
+                                                            want_grad_in=ctx.needs_input_grad[0])
+        return tensor_grad, (grad_min.reshape(min_shape) if ctx.needs_input_grad[1] else None), \
+            (grad_max.reshape(max_shape) if ctx.needs_input_grad[2] else None), None, None, None
+
+
+def takes_learned_range(tensor: torch.Tensor, enc_min: torch.Tensor, enc_max: torch.Tensor) -> bool:
+    """True where quantize_dequantize_learned_range() applies: float32 min / max of one shape, held contiguously on
+    the tensor's GPU."""
+    return tensor.is_cuda and tensor.is_floating_point() and enc_min.dtype == enc_max.dtype == torch.float32 and \
+        enc_min.shape == enc_max.shape and enc_min.device == enc_max.device == tensor.device and \
+        enc_min.is_contiguous() and enc_max.is_contiguous() and tensor.numel() > 0
+
+
+def quantize_dequantize_learned_range(tensor: torch.Tensor, enc_min: torch.Tensor, enc_max: torch.Tensor, qmin: int,
+                                      qmax: int, symmetric: bool, block_size: Optional[List] = None) -> torch.Tensor:
+    """quantize_dequantize(tensor, scale, offset, ...) with scale = (max - min) / (qmax - qmin) and
+    offset = round(min / scale) - qmin (0 for a symmetric quantizer), differentiable w.r.t. tensor, min and max: the
+    training-time forward of a quantizer with learnable range (reference affine/quantizer.py:404-436 followed by
+    :720-745)."""
+    _validate_arguments(tensor, enc_min, enc_max, qmin, qmax, block_size)
+    if not _is_grid_representable(torch.float32, qmin, qmax):
+        raise RuntimeError(f"{torch.float32} is unable to represent quantized output of range [{qmin}, {qmax}].")
+    x, orig = _prepare(tensor, enc_min, enc_max)
+    shape = x.shape
+    expanded = reshape_tensor_for_blocks(x, enc_min.shape, block_size)
+    tensor3, perm = channel_view(expanded, get_encoding_shape_with_blocks(enc_min.shape, block_size))
+    out = _LearnedRangeFunc.apply(tensor3, enc_min, enc_max, qmin, qmax, bool(symmetric))
+    out = channel_view_restore(out, expanded.shape, perm).reshape(shape)
+    return out.to(orig) if orig is not None else out
 
 
 class _QuantizeFunc(torch.autograd.Function):

@@ -20,7 +20,7 @@ from ...utils import (StatisticsNotFoundError, _is_expandable, get_encoding_shap
                       reshape_tensor_for_blocks, ste_round)
 from ..base import QuantizerBase
 from ..encoding_analyzer import EncodingAnalyzer, MinMaxEncodingAnalyzer
-from .backends import _derive_qmin_qmax, quantize, quantize_dequantize
+from .backends import _derive_qmin_qmax, get_backend, quantize, quantize_dequantize
 from .encoding import AffineEncoding, _GridMixin
 
 
@@ -333,10 +333,24 @@ class Quantize(MinMaxQuantizer):
 class QuantizeDequantize(MinMaxQuantizer):
     """out = (clamp(round(input / scale) - offset, qmin, qmax) + offset) * scale"""
 
+    # Training with a learnable range: min / max go to the backend as they are, which forms the grid and the range
+    # gradients in its kernels.  False: scale and offset are formed here by tensor operations, as in the reference, and
+    # autograd carries their gradients back to min / max.
+    fuse_range_learning = True
+
     def forward(self, input: torch.Tensor) -> torch.Tensor:  # pylint: disable=redefined-builtin
         if not self.is_initialized():
             raise RuntimeError('Failed to run QuantizeDequantize since quantization parameters are not initialized.'
                                ' Please initialize the quantization parameters using `compute_encodings()`.')
+        mn, mx = self.min, self.max
+        own_grid = type(self).get_scale is not MinMaxQuantizer.get_scale or \
+            type(self).get_offset is not MinMaxQuantizer.get_offset     # e.g. the grouped blockwise quantizer
+        if self.fuse_range_learning and torch.is_grad_enabled() and (mn.requires_grad or mx.requires_grad) and \
+                not own_grid:
+            backend = get_backend()
+            fused = getattr(backend, 'quantize_dequantize_learned_range', None)
+            if fused is not None and backend.takes_learned_range(input, mn, mx):
+                return fused(input, mn, mx, self.qmin, self.qmax, self._symmetric, block_size=self.block_size)
         encoding = self.get_encoding()
         return quantize_dequantize(input, encoding.scale, encoding.offset, encoding.qmin, encoding.qmax,
                                    block_size=self.block_size)

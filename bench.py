@@ -664,13 +664,16 @@ def _resnet50_shaped(torch):
     return Net().eval()
 
 
-def quantsim_resnet50_shaped(torch, batch=64):
+def quantsim_resnet50_shaped(torch, batch=64, quant_scheme='tf', v2=False):
     """The simulation-model workload: the ResNet-50-shaped net on the GPU, a QuantizationSimModel around it with int8
     per-channel symmetric weight quantizers and int8 per-tensor activation quantizers (Conv+ReLU and Add+ReLU
     supergroups, model input quantized), calibrated on 16 of the `batch` seeded N(0,1) images.
-    Returns (model, sim, images)."""
+    Returns (model, sim, images).  quant_scheme: a scheme's short name or a QuantScheme; v2: the v2 simulation model."""
     import tempfile
-    from aimet_amd.v1.quantsim import QuantizationSimModel
+    if v2:
+        from aimet_amd.v2.quantsim import QuantizationSimModel
+    else:
+        from aimet_amd.v1.quantsim import QuantizationSimModel
     dev = torch.device("cuda", 0)
     model = _resnet50_shaped(torch).to(dev)
     g = torch.Generator(device=dev).manual_seed(1004)
@@ -684,8 +687,8 @@ def quantsim_resnet50_shaped(torch, batch=64):
            "model_input": {"is_input_quantized": "True"}, "model_output": {}}
     with tempfile.NamedTemporaryFile("w", suffix=".json", delete=False) as f:
         json.dump(cfg, f)
-    sim = QuantizationSimModel(model, dummy_input=x[:2], quant_scheme='tf', default_output_bw=8, default_param_bw=8,
-                               config_file=f.name)
+    sim = QuantizationSimModel(model, dummy_input=x[:2], quant_scheme=quant_scheme, default_output_bw=8,
+                               default_param_bw=8, config_file=f.name)
     os.unlink(f.name)
     with torch.no_grad():
         sim.compute_encodings(lambda m, a: m(a), x[:16])
@@ -931,8 +934,36 @@ def bench_end_to_end(torch, ops):
     steps["v2_sim_ms"] = training_step(sim2.model.train())
     steps["note"] = ("min/max per-channel weight encodings; a v1 wrapper in training mode recomputes them in every "
                      "forward (as the reference does): one launch here, one host computation per channel there")
+    # ---- the same step while the ranges learn (the range-learning quant schemes): every quantizer's grid follows
+    # its encoding min / max, and backward returns their gradients
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1 import quantsim_straight_through_grad as ste
+    from aimet_amd.v2.quantization.affine import QuantizeDequantize
+    del sim_tf
+    gc.collect()
+    learning = QuantScheme.training_range_learning_with_tf_init
+    _, sim_rl, _ = quantsim_resnet50_shaped(torch, 32, learning)
+    steps["v1_range_learning_ms"] = training_step(sim_rl.model.train())
+    in_one_launch, ste.grid_in_one_launch = ste.grid_in_one_launch, lambda *_: False
+    try:
+        steps["v1_range_learning_grid_by_tensor_operations_ms"] = training_step(sim_rl.model)
+    finally:
+        ste.grid_in_one_launch = in_one_launch
+    del sim_rl
+    gc.collect()
+    _, sim2_rl, _ = quantsim_resnet50_shaped(torch, 32, learning, v2=True)
+    steps["v2_range_learning_ms"] = training_step(sim2_rl.model.train())
+    QuantizeDequantize.fuse_range_learning = False
+    try:
+        steps["v2_range_learning_grid_by_tensor_operations_ms"] = training_step(sim2_rl.model)
+    finally:
+        QuantizeDequantize.fuse_range_learning = True
+    del sim2_rl
+    steps["range_learning_note"] = (
+        "127 quantizers; per quantizer and step the grid is one launch and the encoding gradients leave the backward's "
+        "reduction kernel, against about twenty parameter-sized tensor operations")
     out["training_step_batch32_resnet50_shaped"] = steps
-    del sim2, sim_tf, model, data
+    del sim2, model, data
     gc.collect()
 
     # ---- apply_adaround

@@ -312,6 +312,51 @@ int miq_v2_qdq_bwd_params_bf16(const uint16_t* x, const uint16_t* grad_out, uint
                                void* workspace, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
+ * Range learning: the quantization grid is a function of a learnable encoding min / max per channel, and the
+ * gradients go back to that min / max.  The reference forms the grid and the encoding gradients with a dozen tensor
+ * operations of parameter size per quantizer and step; here the grid is one small launch and the encoding gradients
+ * leave the backward's reduction kernel directly.
+ *
+ * How (min, max) become (scale, offset), and (sum_s, sum_o) -- the two channel sums miq_v2_qdq_bwd_params_* returns
+ * as scale_grad / offset_grad -- become (grad_min, grad_max).  steps = qmax - qmin; every operation is float32.
+ *   MIQ_RANGE_V2_ASYMMETRIC (TORCH/v2/quantization/affine/quantizer.py:404-436, differentiated by autograd there;
+ *   "/ steps" is the product with float32(1 / steps), which is how torch's device kernels divide a tensor by a number,
+ *   so that the grid equals get_scale() / get_offset() of the same module to the bit)
+ *     scale = (max - min) / steps, offset = round(min / scale) - qmin (round straight-through)
+ *     s = sum_s - sum_o * ((min / scale) / scale); grad_max = s / steps; grad_min = sum_o / scale - s / steps
+ *   MIQ_RANGE_V2_SYMMETRIC: scale as above, offset = 0; grad_max = sum_s / steps, grad_min = -grad_max
+ *   MIQ_RANGE_V1_ASYMMETRIC (TORCH/v1/quantsim_straight_through_grad.py:121-162, :251-292; qmin must be 0; here and
+ *   below every "/" is a division, the reference's operands being tensors)
+ *     scale = (max - min) / steps, offset = -clamp(round(-min / scale), 0, steps)
+ *     t1 = sum_s / steps, t2 = steps / (max - min)^2 * sum_o
+ *     grad_min = -t1 + max * t2, grad_max = t1 - min * t2
+ *   MIQ_RANGE_V1_SIGNED_SYMMETRIC (:143-146, :296-325): scale = max / floor(steps / 2), offset = -ceil(steps / 2)
+ *     grad_max = sum_s / (steps div 2), grad_min = -grad_max
+ *   MIQ_RANGE_V1_UNSIGNED_SYMMETRIC (:148-151): scale = (max - min) / steps, offset = min / scale; gradients as for
+ *     the signed symmetric mode
+ * ------------------------------------------------------------------------------------------------------------- */
+#define MIQ_RANGE_V2_ASYMMETRIC 0
+#define MIQ_RANGE_V2_SYMMETRIC 1
+#define MIQ_RANGE_V1_ASYMMETRIC 2
+#define MIQ_RANGE_V1_SIGNED_SYMMETRIC 3
+#define MIQ_RANGE_V1_UNSIGNED_SYMMETRIC 4
+/* grid: device float[4 * num_channel] = {scale_0.., offset_0.., min_0.., max_0..}, min / max being the values the grid
+ * was made from.  gate != 0 first orders the range in place, in enc_min / enc_max themselves, as the v1 wrappers do
+ * before every forward pass (TORCH/v1/tensor_quantizer.py:1347-1359): min = min(min, 0), max = max(max, 0),
+ * max = max(max, min + 1e-5); NaN stays NaN. */
+int miq_range_to_grid_f32(float* enc_min, float* enc_max, int64_t num_channel, int qmin, int qmax, int mode, int gate,
+                          float* grid, void* stream);
+/* miq_v2_qdq_bwd_params_* with the encoding gradients in place of the scale / offset gradients: `grid` as
+ * miq_range_to_grid_f32 wrote it for the forward pass (scale and offset are read from it as well), grad_min /
+ * grad_max: device float[num_channel].  Workspace: miq_v2_qdq_bwd_params_workspace_bytes(). */
+int miq_qdq_bwd_range_f32(const float* x, const float* grad_out, float* grad_in, int64_t num_channel,
+                          int64_t num_element, int64_t num_element_per_channel, const float* grid, int qmin, int qmax,
+                          int mode, float* grad_min, float* grad_max, void* workspace, void* stream);
+int miq_qdq_bwd_range_bf16(const uint16_t* x, const uint16_t* grad_out, uint16_t* grad_in, int64_t num_channel,
+                           int64_t num_element, int64_t num_element_per_channel, const float* grid, int qmin,
+                           int qmax, int mode, float* grad_min, float* grad_max, void* workspace, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
  * Calibration statistics
  * ------------------------------------------------------------------------------------------------------------- */
 
