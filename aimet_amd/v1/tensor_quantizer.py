@@ -721,6 +721,12 @@ class LearnedGridTensorQuantizer(TensorQuantizer):
         return getattr(self.wrapper_ref, self.name + '_encoding_min'), \
             getattr(self.wrapper_ref, self.name + '_encoding_max')
 
+    def __getstate__(self):
+        # the grid a wrapper prepared for the forward pass in progress is not part of the quantizer
+        state = self.__dict__.copy()
+        state.pop('_prepared_grid', None)
+        return state
+
     def get_effective_encoding(self):
         """The encoding as the user's quant scheme means it: non-strict symmetric quantizers learn with max == -min
         and report min one step lower (reference :642-686)."""
