@@ -287,3 +287,56 @@ def test_v1_learned_grid_wrapper_with_and_without_the_library_grid(symmetric, pe
             # weight gradients come out of convolution kernels that add in no fixed order
             assert torch.allclose(grad, grads_b[name], rtol=1e-4, atol=1e-6), name
     assert checked >= 10
+
+
+# ------------------------------------------------------------------------------------------------- against the oracle
+@pytest.mark.parametrize("mode_name", ("RANGE_V2_ASYMMETRIC", "RANGE_V2_SYMMETRIC", "RANGE_V1_ASYMMETRIC",
+                                       "RANGE_V1_SIGNED_SYMMETRIC", "RANGE_V1_UNSIGNED_SYMMETRIC"))
+def test_grid_and_range_gradients_against_the_cpu_oracle(mode_name):
+    """The CPU restatement (numpy float32, one rounding per operation) gives the same grid, ordered range and range
+    gradients to the bit -- the v2 modes with "/ steps" as the product with float32(1 / steps), as the device kernels
+    of torch form it; with a division, as torch's CPU kernels do, scale is at most one ulp away."""
+    from aimet_amd import ops
+    from oracle import lib as oracle
+    from oracle import range_oracle
+    mode = getattr(ops, mode_name)
+    c, n = 24, 3000
+    rng = np.random.default_rng(mode)
+    enc_min = (-rng.uniform(0.2, 2.0, c)).astype(np.float32)
+    enc_max = rng.uniform(0.2, 2.0, c).astype(np.float32)
+    enc_min[3], enc_max[5] = 0.125, -0.5                                # out of order: put right by the gate
+    if mode == ops.RANGE_V1_SIGNED_SYMMETRIC:
+        enc_max[5] = 0.5                                                # (a max of 0 would be a step of 0 here)
+    qmin, qmax = (-128, 127) if mode == ops.RANGE_V2_SYMMETRIC else (0, 255)
+    want_min, want_max = range_oracle.ordered_range(enc_min, enc_max)
+    if mode in (ops.RANGE_V2_ASYMMETRIC, ops.RANGE_V2_SYMMETRIC):
+        symmetric = mode == ops.RANGE_V2_SYMMETRIC
+        scale, offset = range_oracle.grid_v2(want_min, want_max, qmin, qmax, symmetric, divide=False)
+        divided, _ = range_oracle.grid_v2(want_min, want_max, qmin, qmax, symmetric, divide=True)
+        assert np.all(np.abs(divided.view(np.int32) - scale.view(np.int32)) <= 1)
+    else:
+        symmetric = mode != ops.RANGE_V1_ASYMMETRIC
+        scale, offset, steps = range_oracle.grid_v1(want_min, want_max, 8, symmetric, False,
+                                                    mode == ops.RANGE_V1_UNSIGNED_SYMMETRIC)
+        assert steps == qmax
+    dev_min, dev_max = torch.from_numpy(enc_min).cuda(), torch.from_numpy(enc_max).cuda()
+    grid = ops.range_to_grid(dev_min, dev_max, qmin, qmax, mode, gate=True)
+    assert np.array_equal(dev_min.cpu().numpy(), want_min) and np.array_equal(dev_max.cpu().numpy(), want_max)
+    got = grid.cpu().numpy()
+    assert np.array_equal(got[0].view(np.int32), scale.view(np.int32))
+    assert np.array_equal(got[1], offset)           # (by value: max(0, -0) may be either zero, here and in torch)
+
+    x = (rng.standard_normal((c, n)) * 1.3).astype(np.float32)
+    g = rng.standard_normal((c, n)).astype(np.float32)
+    _, sum_s, sum_o = oracle.v2_qdq_bwd_params(x, g, c, n, scale, offset, qmin, qmax)
+    if mode in (ops.RANGE_V2_ASYMMETRIC, ops.RANGE_V2_SYMMETRIC):
+        want_gmin, want_gmax = range_oracle.range_grads_v2(sum_s, sum_o, want_min, scale, qmin, qmax, symmetric,
+                                                           divide=False)
+    else:
+        want_gmin, want_gmax = range_oracle.range_grads_v1(sum_s, sum_o, want_min, want_max, qmax, symmetric)
+    _, gmin, gmax = ops.qdq_bwd_range(torch.from_numpy(x).cuda(), torch.from_numpy(g).cuda(), c, n, grid, qmin, qmax,
+                                      mode, want_grad_in=False)
+    # the sums are float32 sums in another order: the bar of the scale / offset gradients (2e-5 of their magnitude)
+    for got_grad, want_grad in ((gmin, want_gmin), (gmax, want_gmax)):
+        bar = 2e-5 * max(float(np.abs(want_gmin).max()), float(np.abs(want_gmax).max()))
+        assert np.allclose(got_grad.cpu().numpy(), want_grad, rtol=2e-5, atol=bar)
