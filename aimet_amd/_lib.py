@@ -78,6 +78,7 @@ _SIGNATURES = {
     "miq_v2_qdq_bwd_params_workspace_bytes": ([_i64, _i64, _i64], _i64),
     "miq_v2_qdq_bwd_params_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p, _p, _p, _p], _int),
     "miq_v2_qdq_bwd_params_bf16": ([_p, _p, _p, _i64, _i64, _i64, _p, _p, _int, _int, _p, _p, _p, _p], _int),
+    "miq_adaround_recon_grad_f32": ([_p, _p, _p, _i64, _i64, _i64, _int, C.c_float, _p, _p], _int),
     "miq_range_to_grid_f32": ([_p, _p, _i64, _int, _int, _int, _int, _p, _p], _int),
     "miq_qdq_bwd_range_f32": ([_p, _p, _p, _i64, _i64, _i64, _p, _int, _int, _int, _p, _p, _p, _p], _int),
     "miq_qdq_bwd_range_bf16": ([_p, _p, _p, _i64, _i64, _i64, _p, _int, _int, _int, _p, _p, _p, _p], _int),

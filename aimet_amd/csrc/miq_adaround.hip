@@ -256,6 +256,62 @@ int make_geom(AdaGeom& g, int64_t num_channel, int64_t num_element, int64_t n_pe
     return MIQ_OK;
 }
 
+// relu as torch evaluates it: NaN stays NaN
+__device__ __forceinline__ float relu_keep_nan(float v)
+{
+    return (v > 0.0f || v != v) ? v : 0.0f;
+}
+
+// dLoss/dout of the reconstruction loss for one sample row of `per_sample` elements per workgroup row: the target row
+// is gathered from the cached outputs by the sample's number.  The operations, in the order autograd's backward of
+// relu / sub / square / sum / mean performs them: (act(out) - act(target)) * scale, then * (act(out) > 0) under relu.
+template <bool RELU, bool VEC>
+__global__ __launch_bounds__(kBlock) void recon_grad_kernel(const float* __restrict__ out,
+                                                            const float* __restrict__ target_all,
+                                                            const int64_t* __restrict__ index, int64_t num_cached,
+                                                            int64_t per_sample, float scale, float* __restrict__ grad)
+{
+    const int64_t sample = blockIdx.y;
+    int64_t row          = index ? index[sample] : sample;
+    row                  = row < 0 ? row + num_cached : row;    // as torch's indexing: negative numbers count from the end
+    const bool bad_row   = row < 0 || row >= num_cached;        // no such sample: the row of results becomes NaN
+    row                  = bad_row ? 0 : row;
+    const float* o       = out + sample * per_sample;
+    const float* t       = target_all + row * per_sample;
+    float* g             = grad + sample * per_sample;
+    constexpr int W      = VEC ? 4 : 1;
+    for (int64_t i = ((int64_t) blockIdx.x * kBlock + threadIdx.x) * W; i < per_sample;
+         i += (int64_t) gridDim.x * kBlock * W)
+    {
+        float ov[W], tv[W], gv[W];
+        if (VEC)
+        {
+            const float4 a = *reinterpret_cast<const float4*>(o + i), b = *reinterpret_cast<const float4*>(t + i);
+            ov[0] = a.x, ov[W > 1 ? 1 : 0] = a.y, ov[W > 1 ? 2 : 0] = a.z, ov[W > 1 ? 3 : 0] = a.w;
+            tv[0] = b.x, tv[W > 1 ? 1 : 0] = b.y, tv[W > 1 ? 2 : 0] = b.z, tv[W > 1 ? 3 : 0] = b.w;
+        }
+        else
+        {
+            ov[0] = o[i];
+            tv[0] = t[i];
+        }
+#pragma unroll
+        for (int j = 0; j < W; ++j)
+        {
+            const float qa = RELU ? relu_keep_nan(ov[j]) : ov[j];
+            const float ta = RELU ? relu_keep_nan(tv[j]) : tv[j];
+            float v        = (qa - ta) * scale;
+            if (RELU)
+                v = v * (qa > 0.0f ? 1.0f : 0.0f);
+            gv[j] = bad_row ? NAN : v;
+        }
+        if (VEC)
+            *reinterpret_cast<float4*>(g + i) = make_float4(gv[0], gv[W > 1 ? 1 : 0], gv[W > 1 ? 2 : 0], gv[W > 1 ? 3 : 0]);
+        else
+            g[i] = gv[0];
+    }
+}
+
 inline unsigned vec_blocks(int64_t n)
 {
     int64_t nvec = n / 4;
@@ -416,6 +472,44 @@ int miq_adaround_bwd_adam_f32(const float* weight, const float* grad_weight, flo
         return rc;
     hipLaunchKernelGGL(bwd_kernel<true>, dim3(vec_blocks(num_element)), dim3(kBlock), 0, (hipStream_t) stream, weight,
                        grad_weight, alpha, exp_avg, exp_avg_sq, grad_alpha, g, a, reg_partial);
+    MIQ_CHECK_LAUNCH();
+    return MIQ_OK;
+}
+
+int miq_adaround_recon_grad_f32(const float* out, const float* target, const int64_t* index, int64_t batch,
+                                int64_t num_cached, int64_t per_sample, int activation, float scale, float* grad_out,
+                                void* stream)
+{
+    MIQ_CHECK_ARG(batch >= 0 && batch <= 65535 && per_sample >= 0 && num_cached >= 1, "bad geometry");
+    MIQ_CHECK_ARG(activation == 0 || activation == 1, "activation must be 0 (none) or 1 (ReLU)");
+    MIQ_CHECK_ARG(index || num_cached >= batch, "without an index the target holds at least `batch` samples");
+    if (batch == 0 || per_sample == 0)
+        return MIQ_OK;
+    MIQ_CHECK_ARG(out && target && grad_out, "null tensor pointer");
+    const bool vec = per_sample % 4 == 0 && aligned16(out) && aligned16(target) && aligned16(grad_out);
+    const int64_t per_block = (int64_t) kBlock * (vec ? 4 : 1);
+    int64_t bx = (per_sample + per_block - 1) / per_block;
+    bx         = bx > 1024 ? 1024 : bx;
+    const dim3 grid((unsigned) bx, (unsigned) batch);
+    hipStream_t s = (hipStream_t) stream;
+#define MIQ_RECON(R, V)                                                                                                \
+    hipLaunchKernelGGL((recon_grad_kernel<R, V>), grid, dim3(kBlock), 0, s, out, target, index, num_cached,            \
+                       per_sample, scale, grad_out)
+    if (activation == 1)
+    {
+        if (vec)
+            MIQ_RECON(true, true);
+        else
+            MIQ_RECON(true, false);
+    }
+    else
+    {
+        if (vec)
+            MIQ_RECON(false, true);
+        else
+            MIQ_RECON(false, false);
+    }
+#undef MIQ_RECON
     MIQ_CHECK_LAUNCH();
     return MIQ_OK;
 }

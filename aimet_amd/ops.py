@@ -510,6 +510,31 @@ def v2_qdq_bwd_params(x, grad_out, num_channel, n_per_channel, scale, offset, qm
     return gin, grads[0], grads[1]
 
 
+def adaround_recon_grad(out, target_all, index, activation):
+    """dLoss/dout of AdaRound's reconstruction loss, (act(out) - act(target_all[index])) * 2 / (elements per channel)
+    [* (act(out) > 0) under ReLU], in one pass: `out` [batch, ...] float32 layer output, `target_all` the cached
+    float32 outputs of all samples [samples, ...], `index` int64 device tensor of `batch` sample numbers (None: the
+    first `batch` samples), activation 0 (none) or 1 (ReLU)."""
+    _require_gpu(out, target_all)
+    if out.dtype != _F32 or target_all.dtype != _F32 or not out.is_contiguous() or not target_all.is_contiguous():
+        raise ValueError("out and target_all must be contiguous float32 tensors")
+    batch = out.shape[0]
+    per_sample = out.numel() // max(batch, 1)
+    if tuple(out.shape[1:]) != tuple(target_all.shape[1:]):
+        raise ValueError(f"a sample of out is {tuple(out.shape[1:])}, of target_all {tuple(target_all.shape[1:])}")
+    if index is not None:
+        _require_gpu(index)
+        if index.dtype != torch.int64 or index.numel() != batch or not index.is_contiguous():
+            raise ValueError("index must hold one int64 sample number per row of out")
+    grad = torch.empty_like(out)
+    scale = 2.0 / (out.numel() // out.shape[1]) if out.numel() else 0.0
+    with _OnDevice(out.device):
+        check(lib.miq_adaround_recon_grad_f32(_ptr(out), _ptr(target_all), _ptr(index) if index is not None else None,
+                                              batch, target_all.shape[0], per_sample, int(activation), scale,
+                                              _ptr(grad), _stream(out)))
+    return grad
+
+
 # ---------------------------------------------------------------------------------------------------- range learning
 RANGE_V2_ASYMMETRIC, RANGE_V2_SYMMETRIC, RANGE_V1_ASYMMETRIC, RANGE_V1_SIGNED_SYMMETRIC, \
     RANGE_V1_UNSIGNED_SYMMETRIC = range(5)

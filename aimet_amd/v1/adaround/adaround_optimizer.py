@@ -146,13 +146,14 @@ class AdaroundOptimizer:
         for k, indices in enumerate(batches):
             indices = index_dev[k] if index_dev is not None else indices.to(device)
             inp_data = all_inp_data[indices]
-            orig_out_data = all_orig_out_data[indices]
 
             ada_weight = ops.adaround_soft_round(weight, alpha, qm.num_channel, qm.n_per_channel, qm.delta, qm.offset,
                                                  qm.clip_min, qm.clip_max, True)
             if explicit:
-                grad_weight = cls._recon_loss_weight_gradient(module, inp_data, orig_out_data, ada_weight, activation)
+                grad_weight = cls._recon_loss_weight_gradient(module, inp_data, all_orig_out_data, indices, ada_weight,
+                                                              activation)
             else:
+                orig_out_data = all_orig_out_data[indices]
                 ada_weight.requires_grad_(True)
                 quant_out_data = cls._layer_output(module, inp_data, ada_weight)
                 if act_func is not None:
@@ -174,6 +175,8 @@ class AdaroundOptimizer:
     # same numbers (torch's backward of square / sum / mean / relu / convolution performs exactly these), without the
     # graph and the engine's hand-over, which at 32 samples per iteration cost more than the kernels.  False: autograd.
     use_explicit_gradient = True
+    # dLoss/dout of that written-out gradient by one kernel (False: the five tensor operations it stands for)
+    use_fused_recon_gradient = True
 
     @staticmethod
     def _explicit_gradient_applies(module) -> bool:
@@ -184,16 +187,24 @@ class AdaroundOptimizer:
 
     @classmethod
     @torch.no_grad()
-    def _recon_loss_weight_gradient(cls, module, inp_data, orig_out_data, ada_weight, activation):
+    def _recon_loss_weight_gradient(cls, module, inp_data, all_orig_out_data, indices, ada_weight, activation):
         out = cls._layer_output(module, inp_data, ada_weight)
-        if activation == 1:
-            quant_act, orig_act = torch.relu(out), torch.relu(orig_out_data)
+        if cls.use_fused_recon_gradient and out.dtype == all_orig_out_data.dtype == torch.float32 and \
+                all_orig_out_data.device == out.device and all_orig_out_data.is_contiguous() and \
+                indices.dtype == torch.int64 and 0 < out.shape[0] <= 65535:
+            # both activations, the difference, the loss's factor and relu's mask in one pass over the output; the
+            # target rows are read where they lie in the cache
+            grad_out = ops.adaround_recon_grad(out.contiguous(), all_orig_out_data, indices.contiguous(), activation)
         else:
-            quant_act, orig_act = out, orig_out_data
-        # compute_recon_loss: squared error summed over dim 1, mean over the rest
-        grad_out = (quant_act - orig_act) * (2.0 / (out.numel() // out.shape[1]))
-        if activation == 1:
-            grad_out = grad_out * (quant_act > 0)              # relu's backward: the gradient where its result is positive
+            orig_out_data = all_orig_out_data[indices]
+            if activation == 1:
+                quant_act, orig_act = torch.relu(out), torch.relu(orig_out_data)
+            else:
+                quant_act, orig_act = out, orig_out_data
+            # compute_recon_loss: squared error summed over dim 1, mean over the rest
+            grad_out = (quant_act - orig_act) * (2.0 / (out.numel() // out.shape[1]))
+            if activation == 1:
+                grad_out = grad_out * (quant_act > 0)          # relu's backward: the gradient where its result is positive
         if isinstance(module, torch.nn.Linear):
             return grad_out.reshape(-1, grad_out.shape[-1]).t().mm(inp_data.reshape(-1, inp_data.shape[-1]))
         return torch.ops.aten.convolution_backward(

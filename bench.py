@@ -541,8 +541,11 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
         row = {"conv": [cout, cin, ksize, ksize], "input": [32, cin, hw, hw]}
         n_it = min(200, iterations)
         hp = AdaroundHyperParameters(n_it, 0.01, (20, 2), 0.2)
-        for name, explicit in (("ms_per_iteration", True), ("ms_per_iteration_through_autograd", False)):
+        for name, explicit, one_pass in (("ms_per_iteration", True, True),
+                                         ("ms_per_iteration_loss_gradient_by_tensor_operations", True, False),
+                                         ("ms_per_iteration_through_autograd", False, False)):
             AdaroundOptimizer.use_explicit_gradient = explicit
+            AdaroundOptimizer.use_fused_recon_gradient = one_pass
             alpha0 = layer.alpha.data.clone()
             AdaroundOptimizer.optimize_rounding_on_cached_acts(layer, torch.relu, xc, yc,
                                                                AdaroundHyperParameters(10, 0.01, (20, 2), 0.2))
@@ -553,6 +556,7 @@ def bench_adaround(torch, ops, iterations, timed_kernel_iters=50):
             row[name] = (time.perf_counter() - t0) * 1e3 / n_it
             layer.alpha.data.copy_(alpha0)
         AdaroundOptimizer.use_explicit_gradient = True
+        AdaroundOptimizer.use_fused_recon_gradient = True
         conv_rows.append(row)
     res["convolution_layers_general_path"] = conv_rows
 

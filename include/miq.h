@@ -545,6 +545,17 @@ int miq_adaround_bwd_f32(const float* weight, const float* grad_weight, const fl
                          double beta, float* reg_partial, void* stream);
 /* Number of workgroups (= partial sums) miq_adaround_bwd_adam_f32 / miq_adaround_bwd_f32 use for num_element elements. */
 int miq_adaround_blocks(int64_t num_element);
+/* dLoss/dout of the reconstruction loss (ADA/adaround_loss.py:71-80, after the activation of
+ * ADA/adaround_optimizer.py:194-200) in one pass, where autograd runs relu twice, a subtraction, two products and a
+ * comparison over the layer's output:
+ *   grad_out[b][j] = (act(out[b][j]) - act(target[index[b]][j])) * scale [ * (act(out[b][j]) > 0) under ReLU ]
+ * out / grad_out: [batch][per_sample]; target: the cached outputs of all num_cached samples, [num_cached][per_sample];
+ * index: device int64[batch] sample numbers (NULL: sample b is row b); negative numbers count from the end, as in
+ * torch's indexing, and a number outside [-num_cached, num_cached) turns its row of grad_out into NaN.  scale = 2 / (elements of `out` per channel), the factor the mean over all but dim 1 leaves.
+ * activation: 0 none, 1 ReLU.  batch <= 65535. */
+int miq_adaround_recon_grad_f32(const float* out, const float* target, const int64_t* index, int64_t batch,
+                                int64_t num_cached, int64_t per_sample, int activation, float scale, float* grad_out,
+                                void* stream);
 /* The per-element terms exactly as the kernels above evaluate them, for accuracy measurements (no counterpart in the
  * reference, whose terms are separate torch ops: ADA/adaround_wrapper.py:136-139, ADA/adaround_loss.py:100-106).
  *   what = 0: in = alpha[n]; out = float[3 n]: sigmoid(alpha), h(alpha), dh/dalpha
