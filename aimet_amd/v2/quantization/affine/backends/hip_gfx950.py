@@ -91,6 +91,25 @@ def _apply_per_channel(func, tensor, scale, offset, qmin, qmax, block_size):
     return channel_view_restore(out, expanded.shape, perm).reshape(shape)
 
 
+def _geometry_as_it_is(tensor: torch.Tensor, param: torch.Tensor):
+    """(num_channel, n_per_channel) of a tensor that _as_it_is() accepts"""
+    count = param.numel()
+    return count, max(tensor.numel() // count, 1)
+
+
+def _as_it_is(tensor: torch.Tensor, param: torch.Tensor, block_size) -> bool:
+    """True for a contiguous tensor whose parameter is one number, or one number per slice along the first axis (every
+    activation and every weight quantized per output channel): memory already is [channel][run], and the reshapes of
+    _apply_per_channel -- two view nodes forward, two backward -- have nothing to do."""
+    if block_size is not None or not tensor.is_contiguous() or tensor.numel() == 0:
+        return False
+    count = param.numel()
+    if count == 1:
+        return True
+    shape = param.shape
+    return len(shape) == tensor.dim() and shape[0] == tensor.shape[0] == count
+
+
 def _reduce_like(grad: torch.Tensor, shape) -> torch.Tensor:
     return grad.sum_to_size(shape) if tuple(grad.shape) != tuple(shape) else grad
 
@@ -102,8 +121,9 @@ class _QuantDequantFunc(torch.autograd.Function):
     save_mask = True
 
     @staticmethod
-    def forward(ctx, tensor, scale, offset, qmin, qmax):  # pylint: disable=arguments-differ
-        c, npc = _channel_geometry(tensor.shape, scale.shape)
+    def forward(ctx, tensor, scale, offset, qmin, qmax, geometry=None):  # pylint: disable=arguments-differ
+        # geometry: (channels, elements per channel) of a tensor handed over as it is; None: channel_view's layout
+        c, npc = geometry or _channel_geometry(tensor.shape, scale.shape)
         ctx.geom = (c, npc, qmin, qmax)
         ctx.masked = _QuantDequantFunc.save_mask and ctx.needs_input_grad[0] and \
             not (ctx.needs_input_grad[1] or ctx.needs_input_grad[2])
@@ -119,7 +139,7 @@ class _QuantDequantFunc(torch.autograd.Function):
     def backward(ctx, grad):  # pylint: disable=arguments-differ
         if ctx.masked:
             mask, = ctx.saved_tensors
-            return ops.ste_bwd_mask(mask, grad), None, None, None, None
+            return ops.ste_bwd_mask(mask, grad), None, None, None, None, None
         tensor, scale, offset = ctx.saved_tensors
         c, npc, qmin, qmax = ctx.geom
         tensor_grad = scale_grad = offset_grad = None
@@ -131,7 +151,7 @@ class _QuantDequantFunc(torch.autograd.Function):
             offset_grad = og.reshape(offset.shape).to(offset.dtype) if ctx.needs_input_grad[2] else None
         elif ctx.needs_input_grad[0]:
             tensor_grad = ops.v2_qdq_bwd(tensor, grad, c, npc, scale, offset, qmin, qmax)
-        return tensor_grad, scale_grad, offset_grad, None, None
+        return tensor_grad, scale_grad, offset_grad, None, None, None
 
 
 class _LearnedRangeFunc(torch.autograd.Function):
@@ -141,8 +161,8 @@ class _LearnedRangeFunc(torch.autograd.Function):
     parameter size forward and as many backward, per quantizer and step."""
 
     @staticmethod
-    def forward(ctx, tensor, enc_min, enc_max, qmin, qmax, symmetric):  # pylint: disable=arguments-differ
-        c, npc = tensor.shape[1], max(tensor.shape[2], 1)
+    def forward(ctx, tensor, enc_min, enc_max, qmin, qmax, symmetric, geometry=None):  # pylint: disable=arguments-differ
+        c, npc = geometry or (tensor.shape[1], max(tensor.shape[2], 1))
         mode = ops.RANGE_V2_SYMMETRIC if symmetric else ops.RANGE_V2_ASYMMETRIC
         grid = ops.range_to_grid(enc_min.reshape(-1), enc_max.reshape(-1), qmin, qmax, mode)
         ctx.geom = (c, npc, qmin, qmax, mode, enc_min.shape, enc_max.shape)
@@ -156,7 +176,7 @@ class _LearnedRangeFunc(torch.autograd.Function):
         tensor_grad, grad_min, grad_max = ops.qdq_bwd_range(tensor, grad, c, npc, grid, qmin, qmax, mode,
                                                             want_grad_in=ctx.needs_input_grad[0])
         return tensor_grad, (grad_min.reshape(min_shape) if ctx.needs_input_grad[1] else None), \
-            (grad_max.reshape(max_shape) if ctx.needs_input_grad[2] else None), None, None, None
+            (grad_max.reshape(max_shape) if ctx.needs_input_grad[2] else None), None, None, None, None
 
 
 def takes_learned_range(tensor: torch.Tensor, enc_min: torch.Tensor, enc_max: torch.Tensor) -> bool:
@@ -177,6 +197,10 @@ def quantize_dequantize_learned_range(tensor: torch.Tensor, enc_min: torch.Tenso
     if not _is_grid_representable(torch.float32, qmin, qmax):
         raise RuntimeError(f"{torch.float32} is unable to represent quantized output of range [{qmin}, {qmax}].")
     x, orig = _prepare(tensor, enc_min, enc_max)
+    if _as_it_is(x, enc_min, block_size):
+        out = _LearnedRangeFunc.apply(x, enc_min, enc_max, qmin, qmax, bool(symmetric),
+                                      _geometry_as_it_is(x, enc_min))
+        return out.to(orig) if orig is not None else out
     shape = x.shape
     expanded = reshape_tensor_for_blocks(x, enc_min.shape, block_size)
     tensor3, perm = channel_view(expanded, get_encoding_shape_with_blocks(enc_min.shape, block_size))
@@ -245,7 +269,10 @@ def quantize_dequantize(tensor: torch.Tensor, scale: torch.Tensor, offset: torch
     if not _is_grid_representable(torch.float32, qmin, qmax):
         raise RuntimeError(f"{torch.float32} is unable to represent quantized output of range [{qmin}, {qmax}].")
     x, orig = _prepare(tensor, scale, offset)
-    out = _apply_per_channel(_QuantDequantFunc, x, scale, offset, qmin, qmax, block_size)
+    if scale.shape == offset.shape and _as_it_is(x, scale, block_size) and torch.is_grad_enabled():
+        out = _QuantDequantFunc.apply(x, scale, offset, qmin, qmax, _geometry_as_it_is(x, scale))
+    else:
+        out = _apply_per_channel(_QuantDequantFunc, x, scale, offset, qmin, qmax, block_size)
     return out.to(orig) if orig is not None else out
 
 
