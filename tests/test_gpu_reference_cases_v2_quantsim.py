@@ -402,3 +402,45 @@ def test_models_that_are_quantized_already():
                   QuantizeDequantize((), 0, 255, False)):
         with pytest.raises(RuntimeError, match="WITHOUT quantized modules or quantizers"):
             _sim(model.cuda(), x)
+
+
+def test_grouped_blockwise_encodings_written_and_loaded(tmp_path):
+    """test_save_and_load_gbbq: a grouped blockwise weight quantizer exports one entry per block and takes them back."""
+    from aimet_amd.v2.quantization.affine import GroupedBlockQuantizeDequantize
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv, self.relu, self.pool = nn.Conv2d(3, 8, 3, padding=1), nn.ReLU(), nn.AdaptiveAvgPool2d(3)
+            self.flat, self.fc = nn.Flatten(), nn.Linear(72, 10)
+
+        def forward(self, x):
+            return self.fc(self.flat(self.pool(self.relu(self.conv(x)))))
+
+    x, other = torch.randn(1, 3, 28, 28).cuda(), torch.randn(1, 3, 28, 28).cuda()
+    sim = _sim(Net().eval().cuda(), x)
+    sim.model.fc.param_quantizers["weight"] = GroupedBlockQuantizeDequantize(
+        shape=(10, 6), bitwidth=4, symmetric=True, decompressed_bw=8, block_size=(1, 12), block_grouping=(1, 6)).cuda()
+    sim.compute_encodings(lambda m, _: m(x), None)
+    with torch.no_grad():
+        out1 = sim.model(x)
+    file = sim.export_encodings(str(tmp_path), "saved")
+    with open(file) as f:
+        assert len(json.load(f)["param_encodings"]["fc.weight"]) == 60
+
+    old_weight = sim.model.fc.weight
+    old_max = sim.model.fc.param_quantizers["weight"].get_max()[0][0].clone()
+    sim.model.fc.weight = nn.Parameter(torch.randn(old_weight.shape).cuda())
+    sim.compute_encodings(lambda m, _: m(other), None)
+    assert sim.model.fc.param_quantizers["weight"].get_max()[0][0] != old_max
+    with torch.no_grad():
+        assert not torch.equal(out1, sim.model(x))
+
+    sim.model.fc.weight = old_weight
+    sim.load_encodings(file)
+    assert sim.model.fc.param_quantizers["weight"].get_max()[0][0] == old_max
+    with torch.no_grad():
+        # (the file holds min / max as scale * (offset + qmin / qmax); the scale formed again from those two products
+        # may sit one ulp from the one that made them, so the grids agree to float rounding: one output step at most)
+        step = float(sim.model.fc.output_quantizers[0].get_scale())
+        assert (out1 - sim.model(x)).abs().max().item() <= 1.001 * step
