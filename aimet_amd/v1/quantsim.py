@@ -289,6 +289,7 @@ class QuantizationSimModel:
             for h in handles:
                 h.remove()
             model.train(was_training)
+        records = self._one_record_per_module(records)
         model_outputs = {producer.get(id(t)) for t in tensors_in(out)}
         for r in records:
             r["consumers"] = list(consumers.get(r["name"], []))
@@ -304,13 +305,34 @@ class QuantizationSimModel:
                                 "is_model_output": False})
         return records
 
+    @staticmethod
+    def _one_record_per_module(records):
+        """A module that the forward pass runs more than once gets one wrapper, as every module does, and that wrapper's
+        quantizers see all its uses (the reference does not stop at such a model either: its test
+        test_no_hard_stop_upon_reused_modules).  For the configuration it is one node at the place of its first use:
+        the readers of all its uses are its readers, a position that reads the model's input or a constant in a later
+        use only counts as reading it, and it has as many input / output quantizers as its widest use."""
+        first_use = {}
+        kept = []
+        for rec in records:
+            first = first_use.get(rec["name"])
+            if first is None:
+                first_use[rec["name"]] = rec
+                kept.append(rec)
+                continue
+            for position, source in enumerate(rec["inputs"]):
+                if position >= len(first["inputs"]):
+                    first["inputs"].append(source)
+                    first["singleton"].append(rec["singleton"][position])
+                elif first["inputs"][position] != source and (source == "__model_input__" or source is _CONSTANT):
+                    first["inputs"][position] = source
+                    first["singleton"][position] = rec["singleton"][position]
+            first["num_inputs"] = max(first["num_inputs"], rec["num_inputs"])
+            first["num_outputs"] = max(first["num_outputs"], rec["num_outputs"])
+        return kept
+
     def _add_quantization_wrappers(self):
-        seen = set()
         for rec in self._graph:
-            if rec["name"] in seen:
-                raise RuntimeError(f"module {rec['name']} is used more than once in the forward pass; "
-                                   "give each use its own module")
-            seen.add(rec["name"])
             # range-learning schemes start as static-grid wrappers of the scheme they are initialised from and are
             # swapped for learned-grid wrappers once encodings have been computed
             wrapper = StaticGridQuantWrapper(rec["module"], self._default_param_bw, self._default_output_bw,

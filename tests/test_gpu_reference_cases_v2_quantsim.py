@@ -444,3 +444,44 @@ def test_grouped_blockwise_encodings_written_and_loaded(tmp_path):
         # may sit one ulp from the one that made them, so the grids agree to float rounding: one output step at most)
         step = float(sim.model.fc.output_quantizers[0].get_scale())
         assert (out1 - sim.model(x)).abs().max().item() <= 1.001 * step
+
+
+@pytest.mark.parametrize("sim_kind", ("v1", "v2"))
+@pytest.mark.parametrize("scheme_name", ("post_training_tf", "training_range_learning_with_tf_init"))
+def test_modules_used_more_than_once(sim_kind, scheme_name):
+    """test_no_hard_stop_upon_reused_modules (v2/ab_test/test_quantizer_.py:3595-3612, and its v1 twin): a module that
+    the forward pass runs twice is one quantized module whose quantizers see both uses; calibration, forward, backward
+    and optimizer steps go through."""
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.quantsim import QuantizationSimModel as V1Sim
+    from aimet_amd.v2.quantsim import QuantizationSimModel as V2Sim
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv1 = nn.Conv2d(3, 8, kernel_size=2, stride=2, padding=2, bias=False)
+            self.bn1, self.relu1, self.relu2 = nn.BatchNorm2d(8), nn.ReLU(inplace=True), nn.ReLU(inplace=True)
+            self.fc = nn.Linear(2592, 10)
+
+        def forward(self, x):
+            x = self.relu1(self.conv1(x))
+            x = self.relu2(self.relu1(self.bn1(x)))
+            return self.fc(x.view(x.size(0), -1))
+
+    model = Net().cuda().eval()
+    x = torch.randn(1, 3, 32, 32).cuda()
+    sim = (V1Sim if sim_kind == "v1" else V2Sim)(model, x, quant_scheme=getattr(QuantScheme, scheme_name))
+    quantized = [n for n, m in sim.model.named_children() if type(m) is not type(getattr(model, n))]
+    assert quantized == ["conv1", "bn1", "relu1", "relu2", "fc"]
+    sim.compute_encodings(lambda m, _: m(x), None)
+    with torch.no_grad():
+        assert torch.isfinite(sim.model(x)).all()
+    sim.model.train()
+    optimizer = torch.optim.SGD(sim.model.parameters(), lr=0.05, momentum=0.5)
+    for _ in range(3):
+        sim.model(torch.randn(1, 3, 32, 32).cuda()).sum().backward()
+        optimizer.step()
+        optimizer.zero_grad()
+    # relu1's output quantizer has seen the rectified convolution output and the rectified batch norm output
+    out_q = sim.model.relu1.output_quantizers[0]
+    assert out_q is not None and (out_q.enabled if sim_kind == "v1" else out_q.is_initialized())
