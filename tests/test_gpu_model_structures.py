@@ -1,0 +1,205 @@
+"""Both simulation models over model structures beyond plain chains: calibration, inference, an export / load round trip
+of the encodings and two training steps must go through, for a post-training and a range-learning quant scheme.
+
+The structures are those the reference's simulation-model tests walk through one by one
+(TrainingExtensions/torch/test/python/v2/ab_test/test_quantizer_.py: several outputs :3023-3056, dictionary outputs
+:1717-1759, PReLU :2023-2054, a module taking a list :3619-3645, 3-d convolutions :3264-3286, two inputs :741-764,
+functional operators :1176-1481, embeddings :3647-3699), gathered here with small models of this file's own.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+pytestmark = pytest.mark.gpu
+
+
+def _custom():
+    from aimet_amd.v1.nn.modules import custom
+    return custom
+
+
+class MultiOut(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c1, self.c2, self.c3 = nn.Conv2d(3, 4, 3), nn.Conv2d(4, 4, 3), nn.Conv2d(4, 4, 3)
+
+    def forward(self, x):
+        a = self.c1(x)
+        b = self.c2(a)
+        return a, b, self.c3(b)
+
+
+class DictOut(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c1, self.c2 = nn.Conv2d(3, 4, 3), nn.Conv2d(4, 4, 3)
+
+    def forward(self, x):
+        a = self.c1(x)
+        return {"a": a, "b": self.c2(a)}
+
+
+class PReluUpsample(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c1, self.p, self.up, self.ps = nn.Conv2d(3, 4, 3), nn.PReLU(4), nn.Upsample(scale_factor=2), \
+            nn.PixelShuffle(2)
+
+    def forward(self, x):
+        return self.ps(self.up(self.p(self.c1(x))))
+
+
+class SplitConcat(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c1, self.c2, self.c3 = nn.Conv2d(3, 8, 3), nn.Conv2d(4, 4, 1), nn.Conv2d(4, 4, 1)
+        self.cat, self.head = _custom().Concat(1), nn.Conv2d(8, 2, 1)
+
+    def forward(self, x):
+        a, b = torch.split(self.c1(x), 4, dim=1)
+        return self.head(self.cat(self.c2(a), self.c3(b)))
+
+
+class NestedContainers(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.body = nn.Sequential(nn.Sequential(nn.Conv2d(3, 4, 3), nn.ReLU()), nn.Conv2d(4, 4, 3), nn.Hardtanh())
+        self.heads = nn.ModuleList([nn.Conv2d(4, 2, 1), nn.Conv2d(4, 2, 1)])
+
+    def forward(self, x):
+        y = self.body(x)
+        return self.heads[0](y) + self.heads[1](y)
+
+
+class KeywordsAndAttention(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c1, self.l, self.mha = nn.Conv2d(3, 4, 3), nn.Linear(4, 4), nn.MultiheadAttention(4, 2, batch_first=True)
+
+    def forward(self, x):
+        y = self.l(self.c1(input=x).flatten(2).transpose(1, 2))
+        return self.mha(y, y, y, need_weights=False)[0]
+
+
+class Functionals(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c1, self.c2 = nn.Conv2d(3, 4, 3, padding=1), nn.Conv2d(4, 4, 3, padding=1)
+
+    def forward(self, x):
+        y = F.interpolate(F.max_pool2d(F.relu(self.c1(x)), 2), scale_factor=2)
+        z = self.c2(y)
+        return torch.sigmoid(z) * y - z / 2 + torch.cat([y, z], 1).mean(1, keepdim=True)
+
+
+class TwoInputsOneModuleTwice(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c1, self.c2, self.add, self.mul = nn.Conv2d(3, 4, 3), nn.Conv2d(3, 4, 3), _custom().Add(), \
+            _custom().Multiply()
+
+    def forward(self, a, b):
+        return self.mul(self.add(self.c1(a), self.c2(b)), self.c1(a))
+
+
+class _Reshape(nn.Module):
+    @staticmethod
+    def forward(x, shape):
+        return x.reshape(shape)
+
+
+class ListArgument(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.reshape, self.conv = _Reshape(), nn.Conv2d(1, 16, 3)
+
+    def forward(self, x):
+        return self.conv(self.reshape(x, [-1, 1, 32, 128]))
+
+
+class Conv3dNet(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.conv1, self.bn1, self.relu1 = nn.Conv3d(3, 6, 3), nn.BatchNorm3d(6), nn.ReLU()
+        self.conv2, self.bn2, self.relu2 = nn.Conv3d(6, 8, 3), nn.BatchNorm3d(8), nn.ReLU()
+
+    def forward(self, x):
+        return self.relu2(self.bn2(self.conv2(self.relu1(self.bn1(self.conv1(x))))))
+
+
+class Conv1dNormGelu(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.c, self.ln, self.g, self.t = nn.Conv1d(4, 8, 3), nn.LayerNorm(14), nn.GELU(), nn.ConvTranspose1d(8, 4, 3)
+
+    def forward(self, x):
+        return self.t(self.g(self.ln(self.c(x))))
+
+
+class EmbeddingNet(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.embedding, self.linear, self.softmax = nn.Embedding(1000, 10), nn.Linear(10, 10), nn.Softmax(-1)
+
+    def forward(self, ids):
+        return self.softmax(self.linear(self.embedding(ids)))
+
+
+def _floats(*shapes):
+    return lambda: tuple(torch.randn(s).cuda() for s in shapes)
+
+
+_CASES = {
+    "several_outputs": (MultiOut, _floats((2, 3, 12, 12))),
+    "dictionary_output": (DictOut, _floats((2, 3, 12, 12))),
+    "prelu_upsample_pixelshuffle": (PReluUpsample, _floats((2, 3, 8, 8))),
+    "split_and_concat": (SplitConcat, _floats((2, 3, 8, 8))),
+    "nested_containers": (NestedContainers, _floats((2, 3, 12, 12))),
+    "keyword_arguments_and_attention": (KeywordsAndAttention, _floats((2, 3, 6, 6))),
+    "functional_operators": (Functionals, _floats((2, 3, 8, 8))),
+    "two_inputs_one_module_twice": (TwoInputsOneModuleTwice, _floats((2, 3, 8, 8), (2, 3, 8, 8))),
+    "list_argument": (ListArgument, _floats((1, 32, 128))),
+    "conv3d": (Conv3dNet, _floats((1, 3, 12, 12, 12))),
+    "conv1d_layernorm_gelu": (Conv1dNormGelu, _floats((2, 4, 16))),
+    "embedding": (EmbeddingNet, lambda: (torch.randint(0, 1000, (4, 7)).cuda(),)),
+}
+
+
+def _tensors(out):
+    if isinstance(out, torch.Tensor):
+        return [out]
+    return [t for item in (out.values() if isinstance(out, dict) else out) for t in _tensors(item)]
+
+
+@pytest.mark.parametrize("case", sorted(_CASES))
+@pytest.mark.parametrize("sim_kind", ("v1", "v2"))
+@pytest.mark.parametrize("scheme_name", ("post_training_tf_enhanced", "training_range_learning_with_tf_init"))
+def test_structure(case, sim_kind, scheme_name, tmp_path):
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.quantsim import QuantizationSimModel as V1Sim
+    from aimet_amd.v2.quantsim import QuantizationSimModel as V2Sim
+    model_cls, make = _CASES[case]
+    torch.manual_seed(0)
+    model = model_cls().cuda().eval()
+    x = make()
+    sim = (V1Sim if sim_kind == "v1" else V2Sim)(model, x if len(x) > 1 else x[0],
+                                                   quant_scheme=getattr(QuantScheme, scheme_name))
+    sim.compute_encodings(lambda m, _: m(*x), None)
+    with torch.no_grad():
+        before = _tensors(sim.model(*x))
+    assert before and all(torch.isfinite(t).all() for t in before)
+    file = sim.export_encodings(str(tmp_path), "structure")
+    sim.load_encodings(file)
+    with torch.no_grad():
+        after = _tensors(sim.model(*x))
+    # (encodings pass through the file as min / max: the grids agree to float rounding, outputs to a few steps)
+    for a, b in zip(before, after):
+        assert torch.allclose(a, b, rtol=0, atol=0.05 * float(a.abs().max()) + 1e-6)
+    sim.model.train()
+    optimizer = torch.optim.SGD(sim.model.parameters(), lr=0.01)
+    for _ in range(2):
+        sum(t.sum() for t in _tensors(sim.model(*make()))).backward()
+        optimizer.step()
+        optimizer.zero_grad()
+    assert all(torch.isfinite(p).all() for p in sim.model.parameters())
