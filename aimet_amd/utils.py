@@ -160,14 +160,17 @@ class ModuleData:
     def collect_inp_out_data(self, model_input, collect_input: bool, collect_output: bool):
         inp_data, out_data = [], []
 
-        def hook(_module, inputs, output):
+        def hook(_module, inputs, keywords, output):
             if collect_input:
+                if not inputs:
+                    # called with keyword arguments only (module(input=x)): the first tensor among them
+                    inputs = tuple(v for v in keywords.values() if isinstance(v, torch.Tensor))[:1]
                 inp_data.append(inputs[0] if isinstance(inputs, tuple) and len(inputs) == 1 else inputs)
             if collect_output:
                 out_data.append(output)
             raise StopForwardException
 
-        handle = self._module.register_forward_hook(hook)
+        handle = self._module.register_forward_hook(hook, with_kwargs=True)
         device = get_device(self._model)
         model_input = change_tensor_device_placement(model_input, device)
         try:

@@ -203,3 +203,68 @@ def test_structure(case, sim_kind, scheme_name, tmp_path):
         optimizer.step()
         optimizer.zero_grad()
     assert all(torch.isfinite(p).all() for p in sim.model.parameters())
+
+
+# ------------------------------------------------------------------------------------------------------- AdaRound
+class DepthwiseDilatedTransposed(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.dw, self.pw, self.r = nn.Conv2d(8, 8, 3, padding=1, groups=8), nn.Conv2d(8, 16, 1), nn.ReLU()
+        self.d, self.t = nn.Conv2d(16, 16, 3, dilation=2), nn.ConvTranspose2d(16, 8, 2, stride=2)
+
+    def forward(self, x):
+        return self.t(self.d(self.r(self.pw(self.dw(x)))))
+
+
+class TokenMlp(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.a, self.g, self.b = nn.Linear(64, 128), nn.GELU(), nn.Linear(128, 64)
+
+    def forward(self, x):
+        return self.b(self.g(self.a(x)))
+
+
+def _samples(*shapes):
+    return lambda n: tuple(torch.randn(n, *s).cuda() for s in shapes)
+
+
+# model, one batch of n samples, the layers AdaRound is expected to round
+_ADAROUND_CASES = {
+    "depthwise_dilated_transposed": (DepthwiseDilatedTransposed, _samples((8, 10, 10)), ["dw", "pw", "d", "t"]),
+    "linear_layers_on_tokens": (TokenMlp, _samples((16, 64)), ["a", "b"]),
+    "split_and_concat": (SplitConcat, _samples((3, 8, 8)), ["c1", "c2", "c3", "head"]),
+    "nested_containers": (NestedContainers, _samples((3, 12, 12)), ["body.0.0", "body.1", "heads.0", "heads.1"]),
+    "two_inputs_one_module_twice": (TwoInputsOneModuleTwice, _samples((3, 8, 8), (3, 8, 8)), ["c1", "c2"]),
+    # the attention block's output projection is a Linear that is never called as a module: left as it is
+    "keyword_arguments_and_attention": (KeywordsAndAttention, _samples((3, 6, 6)), ["c1", "l"]),
+    # layers AdaRound has no rule for stay as they are
+    "conv3d": (Conv3dNet, _samples((3, 12, 12, 12)), []),
+    "conv1d_layernorm_gelu": (Conv1dNormGelu, _samples((4, 16)), []),
+}
+
+
+@pytest.mark.parametrize("case", sorted(_ADAROUND_CASES))
+@pytest.mark.parametrize("kind", ("v1", "v2"))
+def test_apply_adaround_on_structure(case, kind, tmp_path):
+    import json
+    if kind == "v1":
+        from aimet_amd.v1.adaround.adaround_weight import Adaround, AdaroundParameters
+    else:
+        from aimet_amd.v2.adaround import Adaround, AdaroundParameters
+    model_cls, make, rounded = _ADAROUND_CASES[case]
+    torch.manual_seed(0)
+    model = model_cls().cuda().eval()
+    loader = [make(16) for _ in range(4)]
+    params = AdaroundParameters(loader, num_batches=4, default_num_iterations=30, forward_fn=lambda m, b: m(*b))
+    dummy = tuple(t[:2] for t in loader[0])
+    out = Adaround.apply_adaround(model, dummy if len(dummy) > 1 else dummy[0], params, str(tmp_path), "structure",
+                                  default_param_bw=4)
+    with open(tmp_path / "structure.encodings") as f:
+        encodings = json.load(f)["param_encodings"]
+    changed = sorted(n[:-len(".weight")] for (n, p), (_, q) in zip(model.named_parameters(), out.named_parameters())
+                     if n.endswith(".weight") and not torch.equal(p, q))
+    assert changed == sorted(rounded)
+    assert all(f"{name}.weight" in encodings for name in rounded)
+    with torch.no_grad():
+        assert all(torch.isfinite(t).all() for t in _tensors(out(*dummy)))
