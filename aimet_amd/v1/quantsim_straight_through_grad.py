@@ -45,12 +45,19 @@ def compute_dloss_by_dx(x, grad, encoding_min, encoding_max, ch_axis=0):
             # the reference compares against a 0-dim tensor, which torch's type promotion casts to x's dtype
             mn = float(torch.tensor(mn, dtype=torch.float32).to(x.dtype))
             mx = float(torch.tensor(mx, dtype=torch.float32).to(x.dtype))
+        if x.dtype == torch.float16:
+            # the kernels take float32 and bfloat16: a float16 value is the same number in float32, and the bounds
+            # have just been rounded to float16 as the reference's comparison rounds them
+            return ops.ste_bwd_per_tensor(x.float(), grad.float(), mn, mx).to(x.dtype)
         return ops.ste_bwd_per_tensor(x, grad, mn, mx)
     mn = torch.as_tensor(encoding_min, dtype=torch.float32).to(x.device)
     mx = torch.as_tensor(encoding_max, dtype=torch.float32).to(x.device)
     num_channel = x.shape[ch_axis]
     assert mn.numel() == num_channel and mx.numel() == num_channel
     n_per_channel = functools.reduce(lambda a, b: a * b, x.shape[ch_axis + 1:], 1)
+    if x.dtype == torch.float16:
+        # (one bound per channel is a tensor with a dimension: the reference's comparison promotes x to float32)
+        return ops.ste_bwd_per_channel(x.float(), grad.float(), num_channel, n_per_channel, mn, mx).to(x.dtype)
     return ops.ste_bwd_per_channel(x, grad, num_channel, n_per_channel, mn, mx)
 
 
