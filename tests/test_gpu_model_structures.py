@@ -322,3 +322,64 @@ def test_half_precision_model(dtype, sim_kind, scheme_name, per_channel):
         optimizer.step()
         optimizer.zero_grad()
     assert all(torch.isfinite(p).all() for p in sim.model.parameters())
+
+
+# ------------------------------------------------------------------------------------------------ ways of running
+@pytest.mark.parametrize("sim_kind", ("v1", "v2"))
+@pytest.mark.parametrize("scheme_name", ("post_training_tf", "training_range_learning_with_tf_init"))
+def test_ways_of_running_the_simulation(sim_kind, scheme_name):
+    """torch.inference_mode() (tensors made there track no version counter, which what the host layer keeps between
+    forwards is keyed on), inference tensors as input, channels-last inputs and weights, autocast, and a state
+    dictionary carried into a fresh simulation model."""
+    import io
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.quantsim import QuantizationSimModel as V1Sim
+    from aimet_amd.v2.quantsim import QuantizationSimModel as V2Sim
+    sim_cls = V1Sim if sim_kind == "v1" else V2Sim
+    scheme = getattr(QuantScheme, scheme_name)
+    learns = scheme_name.startswith("training_range_learning")
+    torch.manual_seed(0)
+    x = torch.randn(4, 3, 8, 8).cuda()
+    sim = sim_cls(_SmallNet().cuda().eval(), x, quant_scheme=scheme, config_file=_PER_CHANNEL)
+    sim.compute_encodings(lambda m, _: m(x), None)
+    with torch.no_grad():
+        expected = sim.model(x)
+
+    # a state dictionary holds the ranges of every v2 quantizer and of the v1 learned-grid wrappers
+    if sim_kind == "v2" or learns:
+        stored = io.BytesIO()
+        torch.save(sim.model.state_dict(), stored)
+        stored.seek(0)
+        fresh = sim_cls(_SmallNet().cuda().eval(), x, quant_scheme=scheme, config_file=_PER_CHANNEL)
+        if sim_kind == "v1":
+            fresh.compute_encodings(lambda m, _: m(torch.rand_like(x)), None)   # (creates the learned-grid wrappers)
+        result = fresh.model.load_state_dict(torch.load(stored, weights_only=True), strict=False)
+        assert not result.missing_keys and not result.unexpected_keys
+        with torch.no_grad():
+            assert torch.equal(fresh.model(x), expected)
+
+    with torch.inference_mode():
+        assert torch.equal(sim.model(x), expected) and torch.equal(sim.model(x), expected)
+        made_inside = x.clone()
+    with torch.no_grad():
+        assert torch.equal(sim.model(made_inside), expected)
+        channels_last = x.contiguous(memory_format=torch.channels_last)
+        assert torch.allclose(sim.model(channels_last), expected, atol=1e-5)
+        sim.model.to(memory_format=torch.channels_last)
+        assert torch.allclose(sim.model(channels_last), expected, atol=1e-4)
+        sim.model.to(memory_format=torch.contiguous_format)
+
+    if sim_kind == "v1" and learns:
+        # learned-grid quantizers want encoding parameters of the tensor's own type (as the reference's do)
+        with pytest.raises(RuntimeError, match="Data type mismatch"), torch.no_grad(), \
+                torch.autocast("cuda", dtype=torch.bfloat16):
+            sim.model(x)
+        return
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        out = sim.model(x)
+    assert out.dtype == torch.bfloat16 and torch.isfinite(out.float()).all()
+    sim.model.train()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = sim.model(x)
+    out.float().sum().backward()
+    assert all(p.grad is None or torch.isfinite(p.grad).all() for p in sim.model.parameters())
