@@ -711,6 +711,72 @@ class QuantizationSimModel:
             json.dump(self.get_encodings_dict(), f, sort_keys=True, indent=4)
         return file
 
+    def get_activation_param_encodings(self):
+        """(activation encodings, parameter encodings) by module / parameter name (reference quantsim.py:692-728)."""
+        exported = self.get_encodings_dict()
+        return exported['activation_encodings'], exported['param_encodings']
+
+    def save_encodings_to_json(self, path: str, filename_prefix: str):
+        """<path>/<filename_prefix>.json with the activation and parameter encodings (reference quantsim.py:680-690)."""
+        activation_encodings, param_encodings = self.get_activation_param_encodings()
+        os.makedirs(path, exist_ok=True)
+        with open(os.path.join(path, filename_prefix + '.json'), 'w') as f:
+            json.dump({'activation_encodings': activation_encodings, 'param_encodings': param_encodings}, f,
+                      sort_keys=True, indent=4)
+
+    @classmethod
+    def get_original_model(cls, model: nn.Module, qdq_weights: bool = False) -> nn.Module:
+        """A copy of the simulation's model without its quantization wrappers; with qdq_weights the parameters hold
+        their quantize-dequantized values (reference quantsim.py:1519-1533)."""
+        original = copy.deepcopy(model)
+        if qdq_weights:
+            cls._apply_qdq_to_model_parameters(original)
+        cls.remove_quantization_wrappers(original)
+        return original
+
+    @classmethod
+    @torch.no_grad()
+    def _apply_qdq_to_model_parameters(cls, model: nn.Module):
+        # pylint: disable=protected-access
+        for module in model.modules():
+            if not isinstance(module, QcQuantizeWrapper):
+                continue
+            was_training = module.training
+            module.eval()
+            try:
+                if isinstance(module, LearnedGridQuantWrapper):
+                    module._quantize_params()                       # leaves results of an autograd function in place
+                    wrapped = module._module_to_wrap
+                    for name, value in list(wrapped._parameters.items()):
+                        if value is not None and not isinstance(value, nn.Parameter):
+                            wrapped._parameters[name] = nn.Parameter(value.detach(), requires_grad=False)
+                else:
+                    module._quantize_dequantize_params()
+            finally:
+                module.train(was_training)
+
+    def export(self, path: str, filename_prefix: str, dummy_input=None, onnx_export_args=None,
+               propagate_encodings: bool = False, export_to_torchscript: bool = False,
+               use_embedded_encodings: bool = False, export_model: bool = True,
+               filename_prefix_encodings: str = None):
+        """Writes what the reference's export() (quantsim.py:486-560) writes on the torch side:
+        <filename_prefix>.pth, the model without quantization wrappers and with quantize-dequantized weights, and
+        <filename_prefix_encodings>_torch.encodings, the encodings by torch module and parameter names.
+
+        The reference goes on to trace an ONNX (or TorchScript) graph and to write a second encodings file keyed by
+        that graph's tensor names; graph export is not part of this library, and the arguments that only concern it
+        (dummy_input, onnx_export_args, propagate_encodings) are accepted and not used.  export_to_torchscript and
+        use_embedded_encodings, which ask for other kinds of graph, raise NotImplementedError."""
+        # pylint: disable=too-many-arguments, unused-argument
+        if export_to_torchscript or use_embedded_encodings:
+            raise NotImplementedError("TorchScript and embedded-encodings exports need the graph exporters, which "
+                                      "this library does not have")
+        os.makedirs(path, exist_ok=True)
+        if export_model:
+            torch.save(self.get_original_model(self.model, qdq_weights=True),
+                       os.path.join(path, filename_prefix + '.pth'))
+        return self.export_encodings(path, (filename_prefix_encodings or filename_prefix) + '_torch')
+
     def load_encodings(self, encodings, strict: bool = True, partial: bool = True, requires_grad=None,
                        allow_overwrite: bool = True):
         """Imports parameter and activation encodings from a dictionary or a JSON file

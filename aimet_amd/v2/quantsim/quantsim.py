@@ -9,6 +9,7 @@ symmetric, encoding analyzer of the quant scheme), shape () per tensor or [C, 1,
 unsigned-symmetric grids are refused for symmetric quantizers, as the reference's builder does.
 """
 import contextlib
+import copy
 import json
 import os
 from typing import Tuple, Union
@@ -243,6 +244,64 @@ class QuantizationSimModel:
         with open(file, 'w') as f:
             json.dump(self.get_encodings_dict(), f, sort_keys=True, indent=4)
         return file
+
+    def get_activation_param_encodings(self):
+        """(activation encodings, parameter encodings) by module / parameter name (v1 quantsim.py:692-728)."""
+        exported = self.get_encodings_dict()
+        return exported['activation_encodings'], exported['param_encodings']
+
+    def save_encodings_to_json(self, path: str, filename_prefix: str):
+        """<path>/<filename_prefix>.json with the activation and parameter encodings (v1 quantsim.py:680-690)."""
+        activation_encodings, param_encodings = self.get_activation_param_encodings()
+        os.makedirs(path, exist_ok=True)
+        with open(os.path.join(path, filename_prefix + '.json'), 'w') as f:
+            json.dump({'activation_encodings': activation_encodings, 'param_encodings': param_encodings}, f,
+                      sort_keys=True, indent=4)
+
+    @classmethod
+    def get_original_model(cls, model: nn.Module, qdq_weights: bool = False) -> nn.Module:
+        """A copy of the simulation's model made of plain modules again; with qdq_weights the parameters hold their
+        quantize-dequantized values (v1 quantsim.py:1519-1533, v2 quantsim.py:325-339)."""
+        original = copy.deepcopy(model)
+
+        @torch.no_grad()
+        def restore(parent: nn.Module):
+            for name, child in list(parent.named_children()):
+                if isinstance(child, BaseQuantizationMixin):
+                    if qdq_weights:
+                        with child._patch_quantized_parameters():       # pylint: disable=protected-access
+                            quantized = {n: getattr(child, n).detach().clone() for n, q in
+                                         child.param_quantizers.items() if q is not None and
+                                         getattr(child, n) is not None}
+                        for param_name, value in quantized.items():
+                            getattr(child, param_name).copy_(value)
+                    setattr(parent, name, child.get_original_module())
+                else:
+                    restore(child)
+        restore(original)
+        return original
+
+    def export(self, path: str, filename_prefix: str, dummy_input=None, onnx_export_args=None,
+               propagate_encodings: bool = False, export_to_torchscript: bool = False,
+               use_embedded_encodings: bool = False, export_model: bool = True,
+               filename_prefix_encodings: str = None):
+        """Writes what the reference's export() (v1 quantsim.py:486-560, v2 quantsim.py:226-268) writes on the torch
+        side: <filename_prefix>.pth, the model made of plain modules with quantize-dequantized weights, and
+        <filename_prefix_encodings>_torch.encodings, the encodings by torch module and parameter names.
+
+        The reference goes on to trace an ONNX (or TorchScript) graph and to write a second encodings file keyed by
+        that graph's tensor names; graph export is not part of this library, and the arguments that only concern it
+        (dummy_input, onnx_export_args, propagate_encodings) are accepted and not used.  export_to_torchscript and
+        use_embedded_encodings, which ask for other kinds of graph, raise NotImplementedError."""
+        # pylint: disable=too-many-arguments, unused-argument
+        if export_to_torchscript or use_embedded_encodings:
+            raise NotImplementedError("TorchScript and embedded-encodings exports need the graph exporters, which "
+                                      "this library does not have")
+        os.makedirs(path, exist_ok=True)
+        if export_model:
+            torch.save(self.get_original_model(self.model, qdq_weights=True),
+                       os.path.join(path, filename_prefix + '.pth'))
+        return self.export_encodings(path, (filename_prefix_encodings or filename_prefix) + '_torch')
 
     def load_encodings(self, encodings, strict: bool = True, partial: bool = True, requires_grad=None,
                        allow_overwrite: bool = True):
