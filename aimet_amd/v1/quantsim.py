@@ -16,6 +16,7 @@ import inspect
 import json
 import math
 import os
+import pickle
 from typing import Dict, List, Tuple, Union
 
 import torch
@@ -491,6 +492,12 @@ class QuantizationSimModel:
             if isinstance(module, QcQuantizeWrapper):
                 yield name, module
 
+    named_qmodules = quant_wrappers     # the newer name of the same generator (reference quantsim.py:1856-1868)
+
+    def qmodules(self):
+        """The wrappers without their names."""
+        yield from (wrapper for _, wrapper in self.quant_wrappers())
+
     _get_qc_quantized_layers = staticmethod(lambda model: [(n, m) for n, m in model.named_modules()
                                                            if isinstance(m, QcQuantizeWrapper)])
 
@@ -711,6 +718,12 @@ class QuantizationSimModel:
             json.dump(self.get_encodings_dict(), f, sort_keys=True, indent=4)
         return file
 
+    def exclude_param_from_quantization(self, param_name_to_exclude: str):
+        """Switches off every quantizer of parameters of this name (reference quantsim.py:753-762)."""
+        for _, wrapper in self.quant_wrappers():
+            if param_name_to_exclude in wrapper.param_quantizers:
+                wrapper.param_quantizers[param_name_to_exclude].enabled = False
+
     def get_activation_param_encodings(self):
         """(activation encodings, parameter encodings) by module / parameter name (reference quantsim.py:692-728)."""
         exported = self.get_encodings_dict()
@@ -845,6 +858,20 @@ def load_encodings_to_sim(quant_sim_model: QuantizationSimModel, pytorch_encodin
                                    allow_overwrite=None)
     if isinstance(quant_sim_model, QuantizationSimModel):
         quant_sim_model.replace_wrappers_for_quantize_dequantize()          # a v2 simulation has no wrappers
+
+
+def save_checkpoint(quant_sim_model, file_path: str):
+    """The whole simulation model, pickled, to continue fine-tuning later (reference quantsim.py:2215-2226).  Device
+    objects and what the host layer keeps between forwards are not part of the pickle; they are made again on use."""
+    with open(file_path, 'wb') as file:
+        pickle.dump(quant_sim_model, file)
+
+
+def load_checkpoint(file_path: str):
+    """A simulation model that save_checkpoint() wrote (reference quantsim.py:2229-2238).  As any pickle, only for
+    files you wrote yourself."""
+    with open(file_path, 'rb') as file:
+        return pickle.load(file)
 
 
 def has_valid_encodings(qc_quantize_op: QcQuantizeWrapper) -> bool:

@@ -251,8 +251,21 @@ class QuantizationMixin(BaseQuantizationMixin):
         """Creates (and registers) the quantized class of a single-input, single-output module class."""
         if module_cls in cls.cls_to_qcls:
             return cls.cls_to_qcls[module_cls]
-        quantized_cls = type(f"Quantized{module_cls.__name__}", (cls, module_cls), {})
+        quantized_cls = type(f"Quantized{module_cls.__name__}", (cls, module_cls), {"_wrapped_by": (cls, module_cls)})
         return cls.implements(module_cls)(quantized_cls)
+
+    def __reduce_ex__(self, protocol):
+        # A class that wrap() made has no name to import it by: pickles (and copies) name the mixin and the base class
+        # instead, and the class is made again where they are loaded.
+        made_by = type(self).__dict__.get("_wrapped_by")
+        if made_by is None:
+            return super().__reduce_ex__(protocol)
+        return _rebuild_wrapped, made_by, self.__getstate__()
+
+
+def _rebuild_wrapped(mixin_cls, module_cls):
+    quantized_cls = mixin_cls.wrap(module_cls)
+    return quantized_cls.__new__(quantized_cls)
 
 
 for _cls in (nn.Linear, nn.Conv1d, nn.Conv2d, nn.Conv3d, nn.ConvTranspose1d, nn.ConvTranspose2d, nn.ConvTranspose3d,

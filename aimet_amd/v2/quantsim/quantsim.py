@@ -160,12 +160,28 @@ class QuantizationSimModel:
         return quantizer
 
     # --------------------------------------------------------------------------------------------------- usage
-    def qmodules(self):
+    def named_qmodules(self):
+        """(name, quantized module) pairs (v1 quantsim.py:1856-1861)."""
         for name, module in self.model.named_modules():
             if isinstance(module, BaseQuantizationMixin):
                 yield name, module
 
-    named_qmodules = qmodules
+    def qmodules(self):
+        """The quantized modules (v1 quantsim.py:1863-1866)."""
+        yield from (module for _, module in self.named_qmodules())
+
+    quant_wrappers = named_qmodules     # the v1 name, which the reference keeps (deprecated) on the v2 class
+
+    @staticmethod
+    def compute_layer_encodings_for_sim(sim):
+        raise NotImplementedError("QuantizationSimModel.compute_layer_encodings_for_sim has been removed.")
+
+    @staticmethod
+    def prepare_sim_for_compute_encodings(sim):
+        """Nothing to prepare on the v2 classes (reference v2 quantsim.py:304-307)."""
+
+    def replace_wrappers_for_quantize_dequantize(self):
+        """The v2 quantizers learn their ranges as they are: nothing to replace."""
 
     def exclude_layers_from_quantization(self, layers_to_exclude):
         """The given quantized modules, and the quantized modules below the given containers, become plain modules
@@ -183,7 +199,7 @@ class QuantizationSimModel:
 
     def exclude_param_from_quantization(self, param_name_to_exclude: str):
         """No module quantizes its parameter of this name any more (reference v2 quantsim.py:288-298)."""
-        for _, module in self.qmodules():
+        for _, module in self.named_qmodules():
             if param_name_to_exclude in module.param_quantizers:
                 module.param_quantizers[param_name_to_exclude] = None
 
@@ -192,7 +208,7 @@ class QuantizationSimModel:
         if percentile_value < 90 or percentile_value > 100:
             raise ValueError("Percentile value must be in range [90, 100]")
         self._percentile_value = percentile_value
-        for _, module in self.qmodules():
+        for _, module in self.named_qmodules():
             for quantizer in list(module.input_quantizers) + list(module.output_quantizers) + \
                     list(module.param_quantizers.values()):
                 analyzer = getattr(quantizer, 'encoding_analyzer', None)
@@ -205,7 +221,7 @@ class QuantizationSimModel:
         # for the device for (has any observer seen only non-finite values, are the new ranges sane) is read for all
         # of them together
         with batched_range_checks(), contextlib.ExitStack() as stack:
-            for _, module in self.qmodules():
+            for _, module in self.named_qmodules():
                 stack.enter_context(module.compute_encodings())
             was_training = self.model.training
             self.model.eval()
@@ -215,7 +231,7 @@ class QuantizationSimModel:
             finally:
                 self.model.train(was_training)
             observers = [getattr(getattr(q, 'encoding_analyzer', None), 'observer', None) for _, module in
-                         self.qmodules() for q in list(module.input_quantizers) + list(module.output_quantizers) +
+                         self.named_qmodules() for q in list(module.input_quantizers) + list(module.output_quantizers) +
                          list(module.param_quantizers.values()) if q is not None]
             _HistogramObserver.read_flags_together([o for o in observers if isinstance(o, _HistogramObserver)])
 
@@ -223,7 +239,7 @@ class QuantizationSimModel:
         """The exported dictionary, laid out as the v1 simulation's: parameters by '<module>.<parameter>', activations
         by module with 'input' / 'output' entries per tensor index."""
         param_encodings, activation_encodings = {}, {}
-        for name, module in self.qmodules():
+        for name, module in self.named_qmodules():
             for pname, quantizer in module.param_quantizers.items():
                 if quantizer is not None and quantizer.is_initialized():
                     param_encodings[f"{name}.{pname}"] = quantizer.get_legacy_encodings()
@@ -331,7 +347,7 @@ class QuantizationSimModel:
                 raise RuntimeError("Encoding dictionary contains modules/parameters that doesn't exist in the "
                                    f"model: {', '.join(unknown)}")
         args = (strict, partial, requires_grad, allow_overwrite)
-        for name, module in self.qmodules():
+        for name, module in self.named_qmodules():
             prefix = f'{name}.'
             own = {key[len(prefix):]: value for key, value in for_params.items()
                    if key.startswith(prefix) and key[len(prefix):] in module.param_quantizers}

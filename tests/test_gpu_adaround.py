@@ -951,7 +951,7 @@ def test_v2_quantized_modules_and_sim():
         QuantizationMixin.from_module(torch.nn.Bilinear(2, 2, 2))
     model = _TinyNet().eval().cuda()
     sim = QuantizationSimModel(model, torch.randn(1, 3, 8, 8).cuda(), quant_scheme='tf', default_param_bw=8)
-    names = [n for n, _ in sim.qmodules()]
+    names = [n for n, _ in sim.named_qmodules()]
     assert names == ["conv1", "relu1", "pool", "flatten", "fc"]
     sim.compute_encodings(lambda m, a: m(a), torch.randn(8, 3, 8, 8).cuda())
     y = sim.model(torch.randn(2, 3, 8, 8).cuda())

@@ -171,7 +171,7 @@ def _placement_v1(sim):
 
 def _placement_v2(sim):
     out = {}
-    for name, m in sim.qmodules():
+    for name, m in sim.named_qmodules():
         out[name] = ([q is not None for q in m.input_quantizers], [q is not None for q in m.output_quantizers],
                      {p: q is not None for p, q in m.param_quantizers.items()})
     return out
@@ -205,7 +205,7 @@ def test_v2_sim_follows_the_configuration(tmp_path, per_channel):
     assert place["relu1"][1] == [True] and place["bn2"][2] == {"weight": False, "bias": False}
     assert place["add"] == ([False, False], [False], {}) and place["relu3"][1] == [True]   # Add+Relu
     assert place["flatten"][1] == [False] and place["drop"][1] == [False] and place["fc"][1] == [True]
-    qm = dict(v2.qmodules())
+    qm = dict(v2.named_qmodules())
     wq = qm["conv2"].param_quantizers["weight"]
     assert isinstance(wq, QuantizeDequantize) and wq.bitwidth == 4 and wq.symmetric
     assert tuple(wq.shape) == ((8, 1, 1, 1) if per_channel else ())
@@ -267,7 +267,7 @@ def test_v2_sim_schemes_and_refusals():
                                         (QuantScheme.training_range_learning_with_tf_init, MinMaxEncodingAnalyzer,
                                          True)):
         sim = V2Sim(model, dummy, quant_scheme=scheme)
-        q = dict(sim.qmodules())["relu1"].output_quantizers[0]
+        q = dict(sim.named_qmodules())["relu1"].output_quantizers[0]
         assert isinstance(q.encoding_analyzer, analyzer)
         assert all(p.requires_grad == trainable for p in q.parameters())
         if scheme == QuantScheme.post_training_percentile:
@@ -345,7 +345,7 @@ def test_v2_load_encodings_after_adaround(tmp_path):
 
     sim = V2Sim(rounded, dummy, quant_scheme='tf', default_param_bw=4)
     sim.load_encodings(file, allow_overwrite=False)
-    qm = dict(sim.qmodules())
+    qm = dict(sim.named_qmodules())
     for key, (entry,) in exported.items():
         layer = key.rsplit(".", 1)[0]
         q = qm[layer].param_quantizers["weight"]
@@ -376,7 +376,7 @@ def test_v2_load_encodings_after_adaround(tmp_path):
     # set_and_freeze_param_encodings is the same import under its older name
     sim2 = V2Sim(rounded, dummy, quant_scheme='tf', default_param_bw=4)
     sim2.set_and_freeze_param_encodings(file)
-    assert {k: dict(sim2.qmodules())[k.rsplit(".", 1)[0]].param_quantizers["weight"].get_legacy_encodings()
+    assert {k: dict(sim2.named_qmodules())[k.rsplit(".", 1)[0]].param_quantizers["weight"].get_legacy_encodings()
             for k in exported} == before
 
 
@@ -425,14 +425,14 @@ def test_v2_load_encodings_options(tmp_path):
     with pytest.raises(RuntimeError, match="bn2"):
         dst.load_encodings(stray)
     dst.load_encodings(stray, strict=False)
-    assert dict(dst.qmodules())["bn2"].output_quantizers[0] is None
+    assert dict(dst.named_qmodules())["bn2"].output_quantizers[0] is None
 
     # partial=False: only fc keeps quantizers; requires_grad reaches the imported min / max
     only_fc = {"param_encodings": {"fc.weight": full["param_encodings"]["fc.weight"]},
                "activation_encodings": {"fc": full["activation_encodings"]["fc"]}}
     part = V2Sim(model, dummy, quant_scheme='tf', default_param_bw=8, per_channel_quantization=True)
     part.load_encodings(only_fc, partial=False, requires_grad=True)
-    qm = dict(part.qmodules())
+    qm = dict(part.named_qmodules())
     assert qm["conv1"].param_quantizers["weight"] is None and qm["relu1"].output_quantizers[0] is None
     fcq = qm["fc"].param_quantizers["weight"]
     assert fcq is not None and all(p.requires_grad for p in fcq.parameters())
@@ -444,7 +444,7 @@ def test_v2_load_encodings_options(tmp_path):
     changed = {"param_encodings": {"fc.weight": [dict(e, min=2 * e["min"], max=2 * e["max"], scale=2 * e["scale"])
                                                  for e in full["param_encodings"]["fc.weight"]]}}
     frozen.load_encodings(changed)
-    got = dict(frozen.qmodules())["fc"].param_quantizers["weight"].get_legacy_encodings()
+    got = dict(frozen.named_qmodules())["fc"].param_quantizers["weight"].get_legacy_encodings()
     assert got[0]["scale"] == pytest.approx(full["param_encodings"]["fc.weight"][0]["scale"], rel=1e-6)
 
 

@@ -68,7 +68,7 @@ def _quantizers_of(module):
 @pytest.mark.parametrize("quant_scheme", _SCHEMES)
 def test_which_parameters_ask_for_gradients(quant_scheme):
     sim, _ = _calibrated(quant_scheme)
-    modules = [m for _, m in sim.qmodules()]
+    modules = [m for _, m in sim.named_qmodules()]
     assert modules
     seen_ranges = 0
     for module in modules:
