@@ -174,6 +174,14 @@ class AdaroundOptimizer:
     # layer's own weight-gradient routine -- instead of recorded and replayed by autograd: the same operations on the
     # same numbers (torch's backward of square / sum / mean / relu / convolution performs exactly these), without the
     # graph and the engine's hand-over, which at 32 samples per iteration cost more than the kernels.  False: autograd.
+    # The reference can gather a layer's activations batch by batch inside the loop instead of once per layer, to save
+    # host memory (:363-368); here they are always gathered once and stay on the GPU, whatever this says.
+    is_activation_caching_enabled = True
+
+    @staticmethod
+    def enable_caching_acts_data() -> bool:
+        return AdaroundOptimizer.is_activation_caching_enabled
+
     use_explicit_gradient = True
     # dLoss/dout of that written-out gradient by one kernel (False: the five tensor operations it stands for)
     use_fused_recon_gradient = True

@@ -587,6 +587,9 @@ def disable_recompute() -> _Handle:
     return _set_enable_recompute(False)
 
 
+no_recompute = disable_recompute       # the reference's name (:1439-1443)
+
+
 class LearnedGridQuantWrapper(QcQuantizeWrapper):
     """Wrapper whose enabled quantizers learn their encoding min / max (reference :947-1170).  The min / max of every
     quantizer are parameters of this module, named input<i>_encoding_min/max, output<i>_encoding_min/max and

@@ -1,6 +1,7 @@
 from .backends import dequantize, quantize, quantize_dequantize
 from .encoding import AffineEncoding
-from .quantizer import GroupedBlockQuantizeDequantize, Quantize, QuantizeDequantize
+from .quantizer import (AffineQuantizerBase, GroupedBlockQuantizeDequantize, MinMaxQuantizer, Quantize,
+                        QuantizeDequantize)
 
-__all__ = ['AffineEncoding', 'quantize', 'quantize_dequantize', 'dequantize', 'Quantize', 'QuantizeDequantize',
-           'GroupedBlockQuantizeDequantize']
+__all__ = ['AffineEncoding', 'quantize', 'quantize_dequantize', 'dequantize', 'AffineQuantizerBase', 'MinMaxQuantizer',
+           'Quantize', 'QuantizeDequantize', 'GroupedBlockQuantizeDequantize']

@@ -318,6 +318,11 @@ class MinMaxQuantizer(_GridMixin, QuantizerBase):
                        torch.tensor([e['max'] for e in encodings]).view(self.shape).to(dev))
 
 
+# The reference splits this class in two, AffineQuantizerBase (grid and encodings) and MinMaxQuantizer (min / max as
+# parameters, :62-300); here they are one, under both names.
+AffineQuantizerBase = MinMaxQuantizer
+
+
 class Quantize(MinMaxQuantizer):
     """out = clamp(round(input / scale) - offset, qmin, qmax)"""
 
