@@ -64,6 +64,49 @@ def tensor_quantizer_factory(bitwidth: int, round_mode, quant_scheme: QuantSchem
     raise AssertionError("Unsupported quant_scheme: " + str(quant_scheme))
 
 
+class QcQuantizeStandAloneBase(nn.Module):
+    """A quantization op that stands by itself in a model: one output quantizer applied to whatever tensors pass
+    through, with the wrappers' ANALYSIS / ACTIVE / PASSTHROUGH modes (reference :113-189)."""
+
+    def __init__(self, activation_bw, round_mode, quant_scheme, is_symmetric, data_type=QuantizationDataType.int):
+        super().__init__()
+        self.output_quantizers = [tensor_quantizer_factory(activation_bw, round_mode, quant_scheme, is_symmetric,
+                                                           enabled_by_default=True, data_type=data_type)]
+        self._mode = QcQuantizeOpMode.ANALYSIS
+
+    def forward(self, *inputs):
+        raise NotImplementedError
+
+    def set_output_bw(self, output_bw: int):
+        self.output_quantizers[0].bitwidth = output_bw
+
+    def set_mode(self, mode):
+        self._mode = mode
+
+    def _quantize_activation(self, tensor_quantizers, tensors_to_quantize):
+        outputs = []
+        for index, tensor in enumerate(tensors_to_quantize):
+            if self._mode is QcQuantizeOpMode.ANALYSIS:
+                tensor_quantizers[index].update_encoding_stats(tensor)
+            elif self._mode is QcQuantizeOpMode.ACTIVE:
+                # outside training only nearest rounding is used
+                round_mode = tensor_quantizers[index].round_mode if self.training else \
+                    libpymo.RoundingMode.ROUND_NEAREST
+                tensor = tensor_quantizers[index].quantize_dequantize(tensor, round_mode)
+            outputs.append(tensor)
+        return outputs[0] if len(outputs) == 1 else outputs
+
+
+class QcQuantizeStandalone(QcQuantizeStandAloneBase):
+    """Quantizes its inputs (reference :1290-1310)."""
+
+    def forward(self, *inputs):
+        return self._quantize_activation(self.output_quantizers, list(inputs))
+
+    def compute_encoding(self):
+        self.output_quantizers[0].compute_encoding()
+
+
 def get_encoding_by_quantizer(quantizer):
     """The encoding a quantizer is exported with: learned-grid quantizers report the one their quant scheme means
     (reference :1507-1519)."""

@@ -122,6 +122,16 @@ def _exported_encoding(quantizer):
     return quantizer.encoding
 
 
+class QuantParams:
+    """The quantization settings other techniques pass along to build a simulation model (reference :103-129)."""
+
+    def __init__(self, weight_bw: int = 8, act_bw: int = 8, round_mode: str = 'nearest',
+                 quant_scheme: Union[QuantScheme, str] = QuantScheme.post_training_tf_enhanced,
+                 config_file: str = None):
+        self.weight_bw, self.act_bw, self.round_mode = weight_bw, act_bw, round_mode
+        self.quant_scheme, self.config_file = quant_scheme, config_file
+
+
 class QuantizationSimModel:
     """Adds quantization simulation ops to a model for off-target simulation of quantized inference accuracy."""
 

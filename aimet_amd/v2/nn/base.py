@@ -15,7 +15,7 @@ from torch import nn
 
 from ... import ops
 from ..quantization.affine.quantizer import MinMaxQuantizer
-from ..utils import patch_attr
+from ..utils import _ContextManager, patch_attr
 
 
 def _no_op(input):  # pylint: disable=redefined-builtin
@@ -180,6 +180,24 @@ class BaseQuantizationMixin:
         module._buffers = dict(self._buffers)
         return module
 
+    # Taking quantizers out: each call empties the named slots at once and returns an object that puts the former
+    # quantizers back when used as a context manager (or as a decorator); ignored, the slots stay empty
+    # (reference :505-575).
+    def _remove_input_quantizers(self, indices=None):
+        return _emptied(self.input_quantizers, range(len(self.input_quantizers)), indices, int)
+
+    def _remove_output_quantizers(self, indices=None):
+        return _emptied(self.output_quantizers, range(len(self.output_quantizers)), indices, int)
+
+    def _remove_param_quantizers(self, keys=None):
+        return _emptied(self.param_quantizers, self.param_quantizers.keys(), keys, str)
+
+    def _remove_activation_quantizers(self):
+        return _all_of(self._remove_output_quantizers(), self._remove_input_quantizers())
+
+    def _remove_all_quantizers(self):
+        return _all_of(self._remove_activation_quantizers(), self._remove_param_quantizers())
+
     @classmethod
     def implements(cls, module_cls):
         """Decorator registering the quantized definition of a base class."""
@@ -261,6 +279,27 @@ class QuantizationMixin(BaseQuantizationMixin):
         if made_by is None:
             return super().__reduce_ex__(protocol)
         return _rebuild_wrapped, made_by, self.__getstate__()
+
+
+def _emptied(slots, every_key, keys, one_key_type):
+    """Sets slots[key] = None for the keys named (one key, several, or None for all of them)."""
+    if keys is None:
+        keys = every_key
+    elif isinstance(keys, one_key_type):
+        keys = (keys,)
+    keys = list(keys)
+    former = [(key, slots[key]) for key in keys]                    # a bad key raises before anything is changed
+
+    def put_back():
+        for key, quantizer in former:
+            slots[key] = quantizer
+    for key in keys:
+        slots[key] = None
+    return _ContextManager(action=lambda: None, cleanup=put_back)
+
+
+def _all_of(*undo):
+    return _ContextManager(action=lambda: None, cleanup=lambda: [u._cleanup() for u in undo])  # pylint: disable=protected-access
 
 
 def _rebuild_wrapped(mixin_cls, module_cls):

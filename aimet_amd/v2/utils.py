@@ -133,3 +133,50 @@ class _RoundSte(torch.autograd.Function):
 def ste_round(x):
     """Rounding (half to even) with a straight-through gradient."""
     return _RoundSte.apply(x)
+
+
+def _remove_from_qmodules(modules, kind: str):
+    """Calls `_remove_<kind>_quantizers()` on every quantized module under `modules` (a module or several); the result
+    puts all of them back when used as a context manager (reference v2/utils.py:283-344)."""
+    from .nn.base import BaseQuantizationMixin                      # pylint: disable=import-outside-toplevel
+    if isinstance(modules, torch.nn.Module):
+        modules = (modules,)
+    undo = []
+
+    def put_back():
+        while undo:
+            undo.pop()._cleanup()                                   # pylint: disable=protected-access
+    try:
+        for root in modules:
+            for module in root.modules():
+                if isinstance(module, BaseQuantizationMixin):
+                    undo.append(getattr(module, f"_remove_{kind}_quantizers")())
+    except Exception:
+        put_back()
+        raise
+    return _ContextManager(action=lambda: None, cleanup=put_back)
+
+
+def remove_input_quantizers(modules):
+    """Takes the input quantizers out of the quantized modules given."""
+    return _remove_from_qmodules(modules, "input")
+
+
+def remove_output_quantizers(modules):
+    """Takes the output quantizers out of the quantized modules given."""
+    return _remove_from_qmodules(modules, "output")
+
+
+def remove_param_quantizers(modules):
+    """Takes the parameter quantizers out of the quantized modules given."""
+    return _remove_from_qmodules(modules, "param")
+
+
+def remove_activation_quantizers(modules):
+    """Takes the input and output quantizers out of the quantized modules given."""
+    return _remove_from_qmodules(modules, "activation")
+
+
+def remove_all_quantizers(modules):
+    """Takes every quantizer out of the quantized modules given."""
+    return _remove_from_qmodules(modules, "all")

@@ -125,3 +125,83 @@ def test_softmax_quantizers(x):
         else:
             expected = _by_hand(a, F.softmax(x, dim=-1), quantizers[0])
         assert torch.equal(layer(x), expected)
+
+
+def test_quantizers_taken_out_and_put_back(x):
+    """After the reference's v2/nn/test_true_quant.py:567-636: under each `_remove_..._quantizers()` context the output
+    is computed without those quantizers and they come back afterwards; called without `with`, they stay out."""
+    a = _api()
+    layer = a.QuantizedLinear(10, 10, bias=False).cuda()
+    layer.input_quantizers[0], layer.output_quantizers[0] = q_in, q_out = a.activation(), a.activation()
+    layer.param_quantizers['weight'] = q_w = a.weight()
+    with layer.compute_encodings():
+        layer(x)
+    w = _by_hand(a, layer.weight, q_w, signed=True)
+    with layer._remove_input_quantizers(0):
+        assert layer.input_quantizers[0] is None
+        assert torch.equal(layer(x), _by_hand(a, F.linear(x, w), q_out))
+    assert layer.input_quantizers[0] is q_in
+    with layer._remove_param_quantizers('weight'):
+        assert layer.param_quantizers['weight'] is None
+        assert torch.equal(layer(x), _by_hand(a, F.linear(_by_hand(a, x, q_in), layer.weight), q_out))
+    assert layer.param_quantizers['weight'] is q_w
+    with layer._remove_output_quantizers(0):
+        assert layer.output_quantizers[0] is None
+        assert torch.equal(layer(x), F.linear(_by_hand(a, x, q_in), w))
+    assert layer.output_quantizers[0] is q_out
+    with layer._remove_activation_quantizers():
+        assert layer.input_quantizers[0] is None and layer.output_quantizers[0] is None
+        assert torch.equal(layer(x), F.linear(x, w))
+    assert layer.input_quantizers[0] is q_in and layer.output_quantizers[0] is q_out
+    with layer._remove_all_quantizers():
+        assert layer.param_quantizers['weight'] is None
+        assert torch.equal(layer(x), F.linear(x, layer.weight))
+    assert (layer.input_quantizers[0], layer.output_quantizers[0], layer.param_quantizers['weight']) == \
+        (q_in, q_out, q_w)
+    with pytest.raises(KeyError):
+        layer._remove_param_quantizers('bias')                      # no such parameter: nothing is changed
+    assert layer.param_quantizers['weight'] is q_w
+    layer._remove_input_quantizers(0)
+    layer._remove_param_quantizers('weight')
+    layer._remove_output_quantizers(0)
+    assert layer.input_quantizers[0] is None and layer.param_quantizers['weight'] is None
+    assert layer.output_quantizers[0] is None
+
+
+@pytest.mark.parametrize("which", ["input", "output", "param", "activation", "all"])
+def test_quantizers_taken_out_of_a_whole_model(which):
+    """After the reference's v2/test_utils_.py:229-353: the model-level helpers, as a context and for good."""
+    from aimet_amd.v2 import utils
+    from aimet_amd.v2.nn import BaseQuantizationMixin
+    from aimet_amd.v2.quantsim import QuantizationSimModel
+    torch.manual_seed(0)
+    model = nn.Sequential(nn.Conv2d(8, 8, 3), nn.BatchNorm2d(8), nn.ReLU()).cuda().eval()
+    dummy = torch.rand(1, 8, 16, 16).cuda()
+    sim = QuantizationSimModel(model, dummy)
+    sim.compute_encodings(lambda m, _: m(dummy), None)
+    remove = getattr(utils, f"remove_{which}_quantizers")
+    qmodules = [m for m in sim.model.modules() if isinstance(m, BaseQuantizationMixin)]
+    before = [(list(m.input_quantizers), list(m.output_quantizers), dict(m.param_quantizers)) for m in qmodules]
+    assert any(q is not None for ins, outs, params in before for q in ins + outs + list(params.values()))
+
+    def gone():
+        for m in qmodules:
+            if which in ("input", "activation", "all"):
+                assert all(q is None for q in m.input_quantizers)
+            if which in ("output", "activation", "all"):
+                assert all(q is None for q in m.output_quantizers)
+            if which in ("param", "all"):
+                assert all(q is None for q in m.param_quantizers.values())
+    modules_before = list(sim.model.modules())
+    quantized = sim.model(dummy)
+    with remove(sim.model):
+        gone()
+        if which == "all":
+            assert torch.equal(sim.model(dummy), model(dummy))
+    assert list(sim.model.modules()) == modules_before
+    now = [(list(m.input_quantizers), list(m.output_quantizers), dict(m.param_quantizers)) for m in qmodules]
+    assert all(x is y for (a1, b1, c1), (a2, b2, c2) in zip(before, now)
+               for x, y in zip(a1 + b1 + list(c1.values()), a2 + b2 + list(c2.values())))
+    assert torch.equal(sim.model(dummy), quantized)
+    remove(sim.model)
+    gone()

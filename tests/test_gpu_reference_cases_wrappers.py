@@ -404,3 +404,28 @@ def test_learned_grid_preserves_fp16(api, act_bw):
                                     for s in ('_encoding_min', '_encoding_max')]
     for g in grads:
         assert g.dtype == torch.float16 and torch.isfinite(g).all()
+
+
+def test_standalone_quantize_op(api):
+    """The op that stands by itself (reference v1/qc_quantize_op.py:113-189, :1290-1310): analysis passes tensors
+    through while it gathers statistics, active mode is the output quantizer's quantize-dequantize."""
+    torch.manual_seed(0)
+    op = api.qop.QcQuantizeStandalone(activation_bw=8, round_mode='nearest',
+                                      quant_scheme=api.QuantScheme.post_training_tf, is_symmetric=False).to(DEV)
+    x, y = torch.randn(4, 16, device=DEV), 3 * torch.randn(4, 16, device=DEV)
+    assert op(x) is x                                               # analysis: untouched
+    assert op(y) is y
+    with pytest.raises(IndexError):
+        op(x, y)                                                    # one quantizer, as in the reference: one tensor
+    op.compute_encoding()
+    encoding = op.output_quantizers[0].encoding
+    assert encoding.min <= float(torch.minimum(x.min(), y.min())) + encoding.delta
+    assert encoding.max >= float(torch.maximum(x.max(), y.max())) - encoding.delta
+    op.set_mode(api.qop.QcQuantizeOpMode.ACTIVE)
+    out = op(y)
+    assert torch.equal(out, op.output_quantizers[0].quantize_dequantize(y, api.nearest))
+    assert not torch.equal(out, y) and float((out - y).abs().max()) <= 0.5 * encoding.delta * 1.001
+    op.set_mode(api.qop.QcQuantizeOpMode.PASSTHROUGH)
+    assert op(y) is y
+    op.set_output_bw(4)
+    assert op.output_quantizers[0].bitwidth == 4
