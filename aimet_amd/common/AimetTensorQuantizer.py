@@ -15,7 +15,7 @@ from .. import ops
 from .libpymo import QuantizationMode, RoundingMode, TfEncoding
 
 _MODE_TO_MIQ = {QuantizationMode.QUANTIZATION_TF: 0, QuantizationMode.QUANTIZATION_TF_ENHANCED: 1,
-                QuantizationMode.QUANTIZATION_PERCENTILE: 2}
+                QuantizationMode.QUANTIZATION_PERCENTILE: 2, QuantizationMode.QUANTIZATION_MSE: 3}
 
 
 def _round_mode(round_mode) -> int:
@@ -34,7 +34,7 @@ class AimetTensorQuantizer:
     def __init__(self, quantizationScheme: QuantizationMode):
         if quantizationScheme not in _MODE_TO_MIQ:
             raise RuntimeError(f"{quantizationScheme} is not implemented: QUANTIZATION_TF, "
-                               "QUANTIZATION_TF_ENHANCED and QUANTIZATION_PERCENTILE are")
+                               "QUANTIZATION_TF_ENHANCED, QUANTIZATION_PERCENTILE and QUANTIZATION_MSE are")
         self._scheme = quantizationScheme
         self._percentile = 100.0
         self._analyzer = None          # created on the first updateStats, on that tensor's device

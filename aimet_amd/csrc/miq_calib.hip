@@ -18,6 +18,7 @@
 #include "miq_agent.h"
 #include "miq_fastmath.h"
 #include "miq_tfe_search.h"
+#include "miq_encoding_math.h"
 
 #include <algorithm>
 #include <cfloat>
@@ -878,6 +879,241 @@ __global__ __launch_bounds__(kBlock) void tfe_search_kernel(DevState* st, Search
     }
 }
 
+// ------------------------------------------------------------------------------------------------- MSE search
+// MseEncodingAnalyzer<float>::computeEncoding on the PDF the TF-Enhanced analyzer keeps (DLQ/src/MseEncodingAnalyzer.cpp
+// :78-262): every pair of one bucket edge below zero (or zero) and one above zero (or zero) inside the observed range
+// is a candidate (min, max); a candidate's cost is the PDF-weighted squared error of quantize-dequantizing the bucket
+// centres on its grid, accumulated bucket by bucket in the reference's types; the first candidate of least cost wins.
+// Three launches on one stream: the edge walk (sequential float additions, one lane), one lane per candidate, the pick.
+// The reference's edge walk `for (float i = histMin; i <= histMax; i += width)` has no end when `width` is below half
+// a unit in the last place of the edges; here it stops after kMseMaxWalk steps (a PDF needs 512 to 514).
+constexpr int kMseMaxWalk  = 1025;
+constexpr int kMseMaxEdges = kMseMaxWalk + 1;
+constexpr int kMseGrid     = 256;    // one workgroup per compute unit: 65536 candidates in one pass, more in strides
+struct MseScratch
+{
+    int n_min, n_max, n_center, pad;
+    float range_min, range_max;   // what the search returns when no candidate has a cost below FLT_MAX
+    float min_cand[kMseMaxEdges + 1];
+    float max_cand[kMseMaxEdges + 1];
+    float center[kMseMaxEdges];
+    float pdf_at[kMseMaxEdges];
+    float part_cost[kMseGrid];
+    int part_index[kMseGrid];
+};
+
+// (int) of a double or float the way x86-64 converts, where the reference runs: outside int -> INT_MIN
+__device__ __forceinline__ int to_int_x86(double v)
+{
+    return (v > -2147483649.0 && v < 2147483648.0) ? (int) v : INT_MIN;
+}
+
+__global__ __launch_bounds__(kBlock) void mse_prepare_kernel(const DevState* st, MseScratch* m)
+{
+    __shared__ float s_range[2];
+    __shared__ float s_walk[kMseMaxWalk];
+    __shared__ float s_center[kMseMaxWalk];
+    __shared__ int s_n_walk, s_n_center;
+    if (!st->initialized)
+    {
+        if (threadIdx.x == 0)
+            m->n_min = m->n_max = m->n_center = 0;
+        return;
+    }
+    const tfe::PdfView view{st->pdf, st->range_min, st->range_bucket};
+    const int lane = threadIdx.x;
+    if (lane < 64)
+    {
+        float lo, hi;
+        tfe::wave_range(view, lane, lo, hi);   // findOriginalRange<float>, DLQ/src/math_functions.cpp:400-433
+        if (lane == 0)
+            s_range[0] = lo, s_range[1] = hi;
+    }
+    __syncthreads();
+    const float width    = (float) (view.x_left(1) - view.x_left(0));
+    const float hist_min = (float) view.x_left(0);
+    const float min_val  = s_range[0];
+    const float max_val  = s_range[1] + width;
+    if (lane == 0)
+    {
+        // The two chains of float additions of _minimizeMSE: the walk over the bucket edges (:156-163) and the bucket
+        // centres (:172-183; at most as many centres as edges are used).  Nothing but additions, compares and LDS
+        // stores in the loop.
+        const float hist_max = (float) (view.x_left(kPdf - 1) + width);
+        int walked           = 0;
+        float c              = min_val + width / 2;
+        for (float i = hist_min; i <= hist_max && walked < kMseMaxWalk; i += width, ++walked)
+        {
+            s_walk[walked]   = i;
+            s_center[walked] = c;
+            c                = c + width;
+        }
+        s_n_walk = walked;
+    }
+    __syncthreads();
+    if (lane < 64)
+    {
+        // Edges in the reference's order: the observed minimum, then every walked value inside [min_val, max_val];
+        // those below zero are the min candidates, those above zero the max candidates, zero closes both lists
+        // (_pickMinMaxCandidatesMSECalib :202-234).  One wavefront compacts 64 entries at a time, order kept.
+        const int n_entries = s_n_walk + 1;
+        int n_min = 0, n_max = 0, n_edges = 0;
+        for (int base = 0; base < n_entries; base += 64)
+        {
+            const int j    = base + lane;
+            const bool in  = j < n_entries;
+            const float v  = !in ? 0.f : (j == 0 ? min_val : s_walk[j - 1]);
+            const bool keep = in && (j == 0 || (v >= min_val && v <= max_val));
+            const uint64_t below = __ballot(keep && v < 0);
+            const uint64_t above = __ballot(keep && v > 0);
+            const uint64_t before = (1ull << lane) - 1;
+            if (keep && v < 0)
+                m->min_cand[n_min + __popcll(below & before)] = v;
+            if (keep && v > 0)
+                m->max_cand[n_max + __popcll(above & before)] = v;
+            n_min += __popcll(below);
+            n_max += __popcll(above);
+            n_edges += __popcll(__ballot(keep));
+        }
+        if (lane == 0)
+        {
+            m->min_cand[n_min] = 0.f;
+            m->max_cand[n_max] = 0.f;
+            m->n_min           = n_min + 1;
+            m->n_max           = n_max + 1;
+            m->n_center        = n_edges - 1;
+            m->range_min       = min_val;
+            m->range_max       = max_val;
+            s_n_center         = n_edges - 1;
+        }
+    }
+    __syncthreads();
+    for (int k = lane; k < s_n_center; k += blockDim.x)
+    {
+        const float c = s_center[k];
+        int ind       = to_int_x86(floorf((c - hist_min) / width));
+        ind           = ind < 0 ? 0 : (ind > kPdf - 1 ? kPdf - 1 : ind);
+        m->center[k]  = c;
+        m->pdf_at[k]  = (float) st->pdf[ind];
+    }
+}
+
+struct MseArgs
+{
+    int bw, sym, strict, uns;
+    int int_steps;   // int(2^bw - 1), one less for strict symmetric, converted on the host
+};
+
+// _computeMSECost :236-262 for one candidate per lane; each workgroup keeps its first candidate of least cost.
+__global__ __launch_bounds__(kBlock) void mse_cost_kernel(MseScratch* m, MseArgs a)
+{
+    __shared__ float s_center[kMseMaxEdges];
+    __shared__ float s_pdf[kMseMaxEdges];
+    __shared__ float s_cost[kBlock / 64];
+    __shared__ int s_index[kBlock / 64];
+    const int n_center = m->n_center, n_min = m->n_min, n_max = m->n_max;
+    const int n_cand = n_min * n_max - 1;   // the last pair is {0, 0}: no candidate
+    for (int k = threadIdx.x; k < n_center; k += blockDim.x)
+    {
+        s_center[k] = m->center[k];
+        s_pdf[k]    = m->pdf_at[k];
+    }
+    __syncthreads();
+    float best = FLT_MAX;
+    int index  = INT_MAX;
+    for (int cand = blockIdx.x * blockDim.x + threadIdx.x; cand < n_cand; cand += gridDim.x * blockDim.x)
+    {
+        const float c_min = m->min_cand[cand / n_max];
+        const float c_max = m->max_cand[cand % n_max];
+        const EncodingD e = computed_encodings(a.bw, c_min, c_max, a.sym != 0, a.strict != 0, a.uns != 0);
+        float err         = 0.f;
+        for (int k = 0; k < n_center; ++k)
+        {
+            const float v       = s_center[k];
+            const float clamped = tfe::std_max(c_min, tfe::std_min(v, c_max));
+            const int q         = to_int_x86(round(clamped / e.delta - e.offset));
+            const float back    = (float) (e.delta * (q + e.offset));
+            const double diff   = (double) (v - back);
+            err                 = (float) (err + s_pdf[k] * (diff * diff));   // std::pow(float, 2) is exact in double
+        }
+        if (err < best)
+            best = err, index = cand;
+    }
+    // lowest cost, lowest candidate number among equals
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        const float oc = __shfl_xor(best, o);
+        const int oi   = __shfl_xor(index, o);
+        if (oc < best || (oc == best && oi < index))
+            best = oc, index = oi;
+    }
+    if ((threadIdx.x & 63) == 0)
+        s_cost[threadIdx.x >> 6] = best, s_index[threadIdx.x >> 6] = index;
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        for (int w = 1; w < kBlock / 64; ++w)
+            if (s_cost[w] < best || (s_cost[w] == best && s_index[w] < index))
+                best = s_cost[w], index = s_index[w];
+        m->part_cost[blockIdx.x]  = best;
+        m->part_index[blockIdx.x] = index;
+    }
+}
+
+// The winner among the workgroups' winners, zero gated into its range, the encoding of that range (computeEncoding
+// :78-130) written where the host reads it.
+__global__ __launch_bounds__(64) void mse_pick_kernel(DevState* st, const MseScratch* m, MseArgs a)
+{
+    const int lane = threadIdx.x;
+    float best     = FLT_MAX;
+    int index      = INT_MAX;
+    if (st->initialized)
+        for (int k = lane; k < kMseGrid; k += 64)
+        {
+            const float c = m->part_cost[k];
+            const int i   = m->part_index[k];
+            if (c < best || (c == best && i < index))
+                best = c, index = i;
+        }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        const float oc = __shfl_xor(best, o);
+        const int oi   = __shfl_xor(index, o);
+        if (oc < best || (oc == best && oi < index))
+            best = oc, index = oi;
+    }
+    if (lane != 0)
+        return;
+    double enc[4] = {0, 0, 0, 0};
+    if (!st->initialized)
+    {
+        if (st->stats_updated)
+        {
+            // only zeros were seen: an encoding that covers float 0 (:92-108)
+            const double d = (1.0 - -1.0) / a.int_steps;
+            const double o = floor(-1.0 / d);
+            enc[0] = o * d, enc[1] = enc[0] + a.int_steps * d, enc[2] = d, enc[3] = o;
+        }
+        st->enc_min = enc[0], st->enc_max = enc[1], st->enc_delta = enc[2], st->enc_offset = enc[3];
+        st->enc_bw     = st->stats_updated ? a.bw : 0;
+        st->best_index = -1;
+        st->n_cand     = 0;
+        return;
+    }
+    float a_min = m->range_min, a_max = m->range_max;
+    if (index != INT_MAX)
+        a_min = m->min_cand[index / m->n_max], a_max = m->max_cand[index % m->n_max];
+    a_min             = tfe::std_min(a_min, 0.f);
+    a_max             = tfe::std_max(a_max, 0.f);
+    const EncodingD e = computed_encodings(a.bw, a_min, a_max, a.sym != 0, a.strict != 0, a.uns != 0);
+    st->enc_min = e.min, st->enc_max = e.max, st->enc_delta = e.delta, st->enc_offset = e.offset;
+    st->enc_bw     = a.bw;
+    st->best_index = (index == INT_MAX) ? -1 : index;
+    st->n_cand     = m->n_min * m->n_max - 1;
+}
+
 __global__ void reset_state_kernel(DevState* st)
 {
     const int i = threadIdx.x;   // launched with kPdf threads
@@ -1024,6 +1260,7 @@ struct miq_analyzer
 {
     int mode;
     float percentile;    // percentile analyzer only
+    MseScratch* mse;     // MSE analyzer only: candidate lists, bucket centres, per-workgroup winners (device)
     int device;
     DevState* st;        // device
     void* pinned;        // host staging (pinned) for read-backs
@@ -1205,15 +1442,17 @@ int miq_analyzer_create_in(int quantization_mode, void* device_state, miq_analyz
     MIQ_CHECK_ARG(out != nullptr, "null output handle");
     MIQ_CHECK_ARG(device_state == nullptr || aligned16(device_state), "device_state must be 16-byte aligned");
     if (quantization_mode != MIQ_QUANTIZATION_TF && quantization_mode != MIQ_QUANTIZATION_TF_ENHANCED &&
-        quantization_mode != MIQ_QUANTIZATION_PERCENTILE)
+        quantization_mode != MIQ_QUANTIZATION_PERCENTILE && quantization_mode != MIQ_QUANTIZATION_MSE)
     {
-        set_error("quantization mode %d is not implemented (TF, TF_ENHANCED and PERCENTILE are)", quantization_mode);
+        set_error("quantization mode %d is not implemented (TF, TF_ENHANCED, PERCENTILE and MSE are)",
+                  quantization_mode);
         return MIQ_ERR_UNSUPPORTED;
     }
     miq_analyzer* a = new (std::nothrow) miq_analyzer();
     MIQ_CHECK_ARG(a != nullptr, "out of host memory");
     a->mode          = quantization_mode;
     a->percentile    = 100.0f;   // PercentileEncodingAnalyzer.h: the default clips nothing
+    a->mse           = nullptr;
     a->st            = static_cast<DevState*>(device_state);
     a->owns_state    = (device_state == nullptr);
     a->needs_reset   = true;
@@ -1230,6 +1469,8 @@ int miq_analyzer_create_in(int quantization_mode, void* device_state, miq_analyz
     hipError_t e     = hipGetDevice(&a->device);
     if (e == hipSuccess && a->owns_state)
         e = hipMalloc((void**) &a->st, sizeof(DevState));
+    if (e == hipSuccess && quantization_mode == MIQ_QUANTIZATION_MSE)
+        e = hipMalloc((void**) &a->mse, sizeof(MseScratch));   // every field is written before it is read
     if (e == hipSuccess)
         e = hipHostMalloc(&a->pinned, kInspectBytes + 64, hipHostMallocDefault);   // + 4 probe words
     if (e == hipSuccess)
@@ -1243,6 +1484,8 @@ int miq_analyzer_create_in(int quantization_mode, void* device_state, miq_analyz
         set_error("analyzer allocation failed: %s", hipGetErrorString(e));
         if (a->st && a->owns_state)
             (void) hipFree(a->st);
+        if (a->mse)
+            (void) hipFree(a->mse);
         if (a->pinned)
             (void) hipHostFree(a->pinned);
         delete a;
@@ -1268,6 +1511,8 @@ int miq_analyzer_destroy(miq_analyzer* a)
         return MIQ_OK;
     if (a->owns_state)
         (void) hipFree(a->st);
+    if (a->mse)
+        (void) hipFree(a->mse);
     (void) hipHostFree(a->pinned);
     delete a;
     return MIQ_OK;
@@ -1407,6 +1652,21 @@ static int queue_encoding(miq_analyzer* a, int bw, int use_symmetric, int use_st
         return rc;
     if (a->mode == MIQ_QUANTIZATION_PERCENTILE)
         return read_state(a, s, kInspectBytes, false);
+    if (a->mode == MIQ_QUANTIZATION_MSE)
+    {
+        float num_steps = (float) (std::pow(2, bw) - 1);
+        if (use_symmetric && use_strict_symmetric)
+            num_steps -= 1;
+        const MseArgs ma{bw, use_symmetric != 0, use_strict_symmetric != 0, use_unsigned_symmetric != 0,
+                         (int) num_steps};
+        hipLaunchKernelGGL(mse_prepare_kernel, dim3(1), dim3(kBlock), 0, s, a->st, a->mse);
+        MIQ_CHECK_LAUNCH();
+        hipLaunchKernelGGL(mse_cost_kernel, dim3(kMseGrid), dim3(kBlock), 0, s, a->mse, ma);
+        MIQ_CHECK_LAUNCH();
+        hipLaunchKernelGGL(mse_pick_kernel, dim3(1), dim3(64), 0, s, a->st, a->mse, ma);
+        MIQ_CHECK_LAUNCH();
+        return read_state(a, s, kHeadBytes, false);
+    }
     const SearchArgs sa = tfe::make_search_args(bw, use_symmetric, use_strict_symmetric, use_unsigned_symmetric);
     MIQ_CHECK_ARG(sa.n_cand <= kMaxCand, "internal: candidate grid too large");
     hipLaunchKernelGGL(tfe_search_kernel, dim3((sa.n_cand + kBlock / 64 - 1) / (kBlock / 64)), dim3(kBlock), 0, s, a->st,

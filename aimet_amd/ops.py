@@ -899,7 +899,7 @@ class _StateOwner:
 
 class Analyzer(_StateOwner):
     """Device-resident encoding analyzer: mode 0 = TF min/max, 1 = TF-Enhanced (512-bucket PDF + SQNR search),
-    2 = percentile on the same PDF."""
+    2 = percentile on the same PDF, 3 = least squared error over pairs of bucket edges of the same PDF."""
 
     def __init__(self, mode, device=None):
         self.mode = int(mode)

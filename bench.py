@@ -328,8 +328,26 @@ def bench_calibration(torch, ops, reps):
                 "update_us": ms * 1e3, "GBps": 4 * n * mult / ms / 1e6,
                 "frac_hbm": 4 * n * mult / ms / 1e6 / HBM_PEAK_GBPS}
         del bigs
+    # the other searches on the same PDF: percentile (host arithmetic on the buckets read back) and least squared error
+    # over pairs of bucket edges (three launches, one lane per pair); wall time of compute_encoding, statistics in place
+    other_searches = {}
+    for name, mode in (("percentile_99.9", 2), ("mse", 3)):
+        other = ops.Analyzer(mode, dev)
+        if mode == 2:
+            other.set_percentile(99.9)
+        for x in batches[:4]:
+            other.update_stats(x)
+        for bw in (8, 4):
+            other.compute_encoding(bw)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(10):
+                e, _ = other.compute_encoding(bw)
+            other_searches[f"{name}_bw{bw}"] = {"compute_encoding_us": (time.perf_counter() - t0) / 10 * 1e6,
+                                                "encoding": [e.min, e.max, e.delta, e.offset]}
+        del other
     return {"elements": elems, "accumulate_ms": acc, "search_ms_wall": sum(search_ms) / len(search_ms),
-            "update_by_batch_size": by_size,
+            "update_by_batch_size": by_size, "other_searches_on_the_same_pdf": other_searches,
             "total_ms_wall": tot, "elements_per_s": elems / (tot / 1e3),
             "accumulate_GBps": 17 * 4 * n / acc / 1e6, "accumulate_frac_hbm": 17 * 4 * n / acc / 1e6 / HBM_PEAK_GBPS,
             "encoding": [enc.min, enc.max, enc.delta, enc.offset]}

@@ -46,6 +46,7 @@ int miq_get_stochastic_state(uint64_t* seed /* host */, uint64_t* calls /* host 
 #define MIQ_QUANTIZATION_TF 0
 #define MIQ_QUANTIZATION_TF_ENHANCED 1
 #define MIQ_QUANTIZATION_PERCENTILE 2
+#define MIQ_QUANTIZATION_MSE 3
 
 #define MIQ_PDF_SIZE 512 /* DLQ/src/math_functions.hpp:80 */
 
@@ -392,7 +393,11 @@ int miq_minmax_per_channel_static_f32(const float* in, int64_t num_channel, int6
  * (TfEncodingAnalyzer, DLQ/src/TfEncodingAnalyzer.cpp:59-101) and QUANTIZATION_TF_ENHANCED
  * (TfEnhancedEncodingAnalyzer, DLQ/src/TfEnhancedEncodingAnalyzer.cpp:68-397) and QUANTIZATION_PERCENTILE
  * (PercentileEncodingAnalyzer, DLQ/src/PercentileEncodingAnalyzer.cpp:54-215: the same PDF, cut where its cumulative
- * sum reaches 100 - p and p percent).  All statistics (running min/max,
+ * sum reaches 100 - p and p percent) and QUANTIZATION_MSE (MseEncodingAnalyzer, DLQ/src/MseEncodingAnalyzer.cpp:54-262:
+ * the same PDF; every pair of one bucket edge below zero and one above, zero included on either side, is a candidate
+ * range, searched on the device for the least PDF-weighted squared quantization error of the bucket centres; this
+ * analyzer holds 25 KB more device memory than the others, allocated by the library also when the state is the
+ * caller's).  All statistics (running min/max,
  * the 512-bucket PDF, its range and iteration count) live in device memory owned by the object on the device that
  * was current at creation; update_stats enqueues work and never synchronises.  compute_encoding synchronises
  * `stream` once to read the result back.  An object must not be used from two threads at once. */

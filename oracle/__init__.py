@@ -83,6 +83,13 @@ class _Oracle:
         L.orc_tfe_cost.restype = C.c_double
         L.orc_tfe_compute_encoding.argtypes = [C.POINTER(_PdfStruct), C.c_int, C.c_int, C.c_int, C.c_int,
                                                C.POINTER(Encoding), C.c_void_p, C.POINTER(C.c_int)]
+        L.orc_mse_minimize.argtypes = [C.POINTER(_PdfStruct), C.c_int, C.c_int, C.c_int, C.c_int,
+                                       C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p, C.c_void_p, C.c_void_p,
+                                       C.POINTER(C.c_int)]
+        L.orc_mse_compute_encoding.argtypes = [C.POINTER(_PdfStruct), C.c_int, C.c_int, C.c_int, C.c_int,
+                                               C.POINTER(Encoding)]
+        L.orc_mse_cost.restype = C.c_float
+        L.orc_mse_cost.argtypes = [C.c_int, _f32p, _f32p, C.c_int, C.c_float, C.c_float, C.c_int, C.c_int, C.c_int]
         L.orc_v2_qdq_f32.argtypes = [_f32p, _i64, _i64, _i64, C.c_void_p, C.c_void_p, C.c_void_p, _f32p, _f32p,
                                      C.c_int, C.c_int]
         L.orc_v2_qdq_bf16.argtypes = [_u16p, _i64, _i64, _i64, _u16p, C.c_void_p, _f32p, _f32p, C.c_int, C.c_int]
@@ -327,6 +334,23 @@ class OraclePdf:
                                                  int(unsigned_sym), C.byref(e))
         return e
 
+    def mse_minimize(self, bw, sym=False, strict=False, unsigned_sym=False):
+        """MseEncodingAnalyzer<float>::_minimizeMSE on the same PDF: (best min, best max, min candidates, max
+        candidates, bucket centres)."""
+        a, b = C.c_float(), C.c_float()
+        mins, maxs, centers = (np.empty(1100, np.float32) for _ in range(3))
+        counts = (C.c_int * 3)()
+        self.o.L.orc_mse_minimize(C.byref(self.s), bw, int(sym), int(strict), int(unsigned_sym), C.byref(a),
+                                  C.byref(b), mins.ctypes.data, maxs.ctypes.data, centers.ctypes.data, counts)
+        return (np.float32(a.value), np.float32(b.value), mins[:counts[0]].copy(), maxs[:counts[1]].copy(),
+                centers[:counts[2]].copy())
+
+    def compute_mse_encoding(self, bw, sym=False, strict=False, unsigned_sym=False):
+        """MseEncodingAnalyzer<float>::computeEncoding on the same PDF."""
+        e = Encoding()
+        self.o.L.orc_mse_compute_encoding(C.byref(self.s), bw, int(sym), int(strict), int(unsigned_sym), C.byref(e))
+        return e
+
 
 class _Ref:
     """The reference's own CPU classes, compiled in place (present only where oracle/_ref was built)."""
@@ -437,6 +461,9 @@ class _Ref:
     def new_percentile(self, percentile):
         return _RefPercentile(self, percentile)
 
+    def new_mse(self):
+        return _RefMse(self)
+
 
 class _RefAnalyzer:
     def __init__(self, ref, enhanced):
@@ -503,6 +530,48 @@ class _RefPercentile:
         o = np.empty(5)
         self.L.ref_pct_compute(self.h, bw, int(sym), int(strict), int(unsigned_sym), o)
         return _Ref._enc(o)
+
+
+class _RefMse:
+    """The reference's MseEncodingAnalyzer<float>, compiled in place."""
+
+    def __init__(self, ref):
+        L = self.L = ref.L
+        L.ref_mse_create.restype = C.c_void_p
+        L.ref_mse_create.argtypes = []
+        L.ref_mse_destroy.argtypes = [C.c_void_p]
+        L.ref_mse_update.argtypes = [C.c_void_p, _f32p, _i64]
+        L.ref_mse_compute.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _f64p]
+        L.ref_mse_minimize.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float),
+                                       C.POINTER(C.c_float)]
+        L.ref_mse_cost.restype = C.c_float
+        L.ref_mse_cost.argtypes = [C.c_void_p, C.c_int, _f32p, _f32p, C.c_int, C.c_float, C.c_float, C.c_int, C.c_int,
+                                   C.c_int]
+        self.h = C.c_void_p(L.ref_mse_create())
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            self.L.ref_mse_destroy(self.h)
+            self.h = None
+
+    def update(self, x):
+        x = _f32(x)
+        self.L.ref_mse_update(self.h, x.reshape(-1), x.size)
+
+    def compute_encoding(self, bw, sym=False, strict=False, unsigned_sym=False):
+        o = np.empty(5)
+        self.L.ref_mse_compute(self.h, bw, int(sym), int(strict), int(unsigned_sym), o)
+        return _Ref._enc(o)
+
+    def minimize(self, bw, sym=False, strict=False, unsigned_sym=False):
+        a, b = C.c_float(), C.c_float()
+        self.L.ref_mse_minimize(self.h, bw, int(sym), int(strict), int(unsigned_sym), C.byref(a), C.byref(b))
+        return np.float32(a.value), np.float32(b.value)
+
+    def cost(self, bw, centers, pdf_at_center, cand_min, cand_max, sym=False, strict=False, unsigned_sym=False):
+        centers, pdf_at_center = _f32(centers), _f32(pdf_at_center)
+        return np.float32(self.L.ref_mse_cost(self.h, bw, centers, pdf_at_center, centers.size, cand_min, cand_max,
+                                              int(sym), int(strict), int(unsigned_sym)))
 
 
 def _load():

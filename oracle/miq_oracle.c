@@ -789,6 +789,152 @@ void orc_percentile_compute_encoding(const orc_pdf* p, float percentile, int bw,
 }
 
 /* ------------------------------------------------------------------------------------------------------------
+ * MSE calibration on the same 512-bucket PDF (MseEncodingAnalyzer<float>; DLQ/src/MseEncodingAnalyzer.cpp:78-262).
+ * Statistics are gathered by UpdatePdf with signed_vals = true, i.e. by orc_pdf_update_f32 above.  Every (min, max)
+ * pair made of one bucket edge below zero (or zero) and one above zero (or zero) is a candidate; its cost is the
+ * PDF-weighted squared error of quantize-dequantizing the bucket centres on the candidate's grid; the first candidate
+ * of least cost wins.
+ *
+ * The reference walks the edges with `for (float i = histMin; i <= histMax; i += histBinWidth)`, which does not end
+ * when the bucket width is below half a unit in the last place of the edges.  This restatement (and the library)
+ * stops the walk after ORC_MSE_MAX_WALK steps: a PDF laid out by UpdatePdf needs 512 to 514.
+ * ---------------------------------------------------------------------------------------------------------- */
+#define ORC_MSE_MAX_WALK 1025
+#define ORC_MSE_MAX_EDGES (ORC_MSE_MAX_WALK + 1)
+
+/* (int) of a double the way x86-64 converts (the reference runs there): values outside int are INT_MIN */
+static int orc_double_to_int(double v)
+{
+    if (!(v > -2147483649.0 && v < 2147483648.0))
+        return INT_MIN;
+    return (int) v;
+}
+
+/* _computeMSECost, :236-262 */
+float orc_mse_cost(int bw, const float* centers, const float* pdfAtCenter, int numCenters, float candMin,
+                   float candMax, int sym, int strict, int unsignedSym)
+{
+    orc_encoding e;
+    orc_get_computed_encodings(bw, candMin, candMax, sym, strict, unsignedSym, &e);
+    float weightedSquareErr = 0;
+    for (int i = 0; i < numCenters; ++i)
+    {
+        float floatVal = centers[i];
+        float inner    = STD_MIN(floatVal, candMax);
+        float clamped  = STD_MAX(candMin, inner);
+        int quantized  = orc_double_to_int(round(clamped / e.delta - e.offset));
+        float dequant  = (float) (e.delta * (quantized + e.offset));
+        float diff     = floatVal - dequant;
+        /* std::pow(float, int) is pow in double; the square of a float is exact there */
+        weightedSquareErr = (float) (weightedSquareErr + pdfAtCenter[i] * ((double) diff * (double) diff));
+    }
+    return weightedSquareErr;
+}
+
+/* _minimizeMSE + _pickMinMaxCandidatesMSECalib, :139-234.  Optional outputs: the candidate lists and bucket centres
+ * (arrays of ORC_MSE_MAX_EDGES + 1 floats) and their counts in counts[3] = {numMin, numMax, numCenters}. */
+void orc_mse_minimize(const orc_pdf* p, int bw, int sym, int strict, int unsignedSym, float* bestMin, float* bestMax,
+                      float* minCandOut, float* maxCandOut, float* centersOut, int* counts)
+{
+    const float histBinWidth = (float) (p->xLeft[1] - p->xLeft[0]);
+    float histMin            = (float) p->xLeft[0];
+    float histMax            = (float) (p->xLeft[ORC_PDF_SIZE - 1] + histBinWidth);
+    float minVal, maxVal;
+    orc_tfe_find_range(p, &minVal, &maxVal); /* findOriginalRange<float> (math_functions.cpp:400-433) */
+    maxVal = maxVal + histBinWidth;
+
+    float edges[ORC_MSE_MAX_EDGES];
+    float minCand[ORC_MSE_MAX_EDGES + 1], maxCand[ORC_MSE_MAX_EDGES + 1];
+    float centers[ORC_MSE_MAX_EDGES], pdfAt[ORC_MSE_MAX_EDGES];
+    int numEdges = 0;
+    edges[numEdges++] = minVal;
+    int walked        = 0;
+    for (float i = histMin; i <= histMax && walked < ORC_MSE_MAX_WALK; i += histBinWidth, ++walked)
+        if (i >= minVal && i <= maxVal)
+            edges[numEdges++] = i;
+
+    int numMin = 0, numMax = 0;
+    for (int k = 0; k < numEdges; ++k)
+    {
+        if (edges[k] < 0)
+            minCand[numMin++] = edges[k];
+        else if (edges[k] > 0)
+            maxCand[numMax++] = edges[k];
+    }
+    minCand[numMin++] = 0;
+    maxCand[numMax++] = 0;
+
+    float pdfStart          = (float) p->xLeft[0];
+    float pdfStep           = (float) (p->xLeft[1] - p->xLeft[0]);
+    const int numBinCenters = numEdges - 1;
+    for (int i = 0; i < numBinCenters; ++i)
+    {
+        centers[i] = (i == 0) ? minVal + histBinWidth / 2 : centers[i - 1] + histBinWidth;
+        int ind    = orc_double_to_int(floorf((centers[i] - pdfStart) / pdfStep));
+        ind        = STD_MIN(STD_MAX(0, ind), ORC_PDF_SIZE - 1);
+        pdfAt[i]   = (float) p->pdf[ind];
+    }
+
+    float mseMin = FLT_MAX;
+    *bestMin     = minVal;
+    *bestMax     = maxVal;
+    for (int i = 0; i < numMin; ++i)
+        for (int j = 0; j < numMax; ++j)
+        {
+            if (i == numMin - 1 && j == numMax - 1)
+                break; /* {0, 0} is no candidate */
+            float mse = orc_mse_cost(bw, centers, pdfAt, numBinCenters, minCand[i], maxCand[j], sym, strict,
+                                     unsignedSym);
+            if (mse < mseMin)
+            {
+                mseMin   = mse;
+                *bestMin = minCand[i];
+                *bestMax = maxCand[j];
+            }
+        }
+    if (counts)
+    {
+        counts[0] = numMin;
+        counts[1] = numMax;
+        counts[2] = numBinCenters;
+    }
+    if (minCandOut)
+        memcpy(minCandOut, minCand, sizeof(float) * (size_t) numMin);
+    if (maxCandOut)
+        memcpy(maxCandOut, maxCand, sizeof(float) * (size_t) numMax);
+    if (centersOut)
+        memcpy(centersOut, centers, sizeof(float) * (size_t) (numBinCenters > 0 ? numBinCenters : 0));
+}
+
+/* computeEncoding, :78-130 */
+void orc_mse_compute_encoding(const orc_pdf* p, int bw, int sym, int strict, int unsignedSym, orc_encoding* e)
+{
+    memset(e, 0, sizeof(*e));
+    float numSteps = (float) (pow(2, bw) - 1);
+    if (sym && strict)
+        numSteps -= 1;
+    if (!p->initialized)
+    {
+        if (p->stats_updated)
+        {
+            e->min    = -1;
+            e->max    = 1;
+            e->delta  = (e->max - e->min) / (int) numSteps;
+            e->offset = floor(e->min / e->delta);
+            e->min    = e->offset * e->delta;
+            e->max    = e->min + (int) numSteps * e->delta;
+            e->bw     = bw;
+        }
+        return;
+    }
+    float aMin, aMax;
+    orc_mse_minimize(p, bw, sym, strict, unsignedSym, &aMin, &aMax, NULL, NULL, NULL, NULL);
+    aMin = STD_MIN(aMin, 0.0f);
+    aMax = STD_MAX(aMax, 0.0f);
+    orc_get_computed_encodings(bw, aMin, aMax, sym, strict, unsignedSym, e);
+}
+
+/* ------------------------------------------------------------------------------------------------------------
  * a7  v2 quantize-dequantize (TORCH/v2/quantization/affine/backends/torch_builtins.py:303-344), float32 internal
  * dtype.  scale/offset are per "channel" with channel = (i / numElementPerChannel) % numChannel, which covers the
  * per-tensor ([1]) and per-output-channel ([C,1,...]) broadcast shapes.  torch.round is half-to-even (rintf under

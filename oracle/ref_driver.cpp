@@ -10,6 +10,7 @@
 //   TfEncodingAnalyzer<float>         ModelOptimizations/DlQuantization/src/TfEncodingAnalyzer.cpp:59-101
 //   TfEnhancedEncodingAnalyzer<float> ModelOptimizations/DlQuantization/src/TfEnhancedEncodingAnalyzer.cpp:68-397
 //   PercentileEncodingAnalyzer<float> ModelOptimizations/DlQuantization/src/PercentileEncodingAnalyzer.cpp:54-215
+//   MseEncodingAnalyzer<float>        ModelOptimizations/DlQuantization/src/MseEncodingAnalyzer.cpp:54-262
 //   getComputedEncodings              ModelOptimizations/DlQuantization/src/quantization_utils.cpp:58-143
 //   quantizeDequantizeBroadcastCpu    ModelOptimizations/DlQuantization/src/trim_functions.cpp:634-660
 
@@ -30,6 +31,7 @@
 // The analyzer keeps its PDF and its candidate/cost helpers private; the checks need to see them.
 #define private public
 #include "TfEnhancedEncodingAnalyzer.h"
+#include "MseEncodingAnalyzer.h"
 #undef private
 #include "TensorQuantizationSim.h"
 #include "PercentileEncodingAnalyzer.h"
@@ -242,5 +244,40 @@ void ref_pct_compute(void* h, int bw, int sym, int strict, int unsignedSym, doub
     TfEncoding e = static_cast<PercentileEncodingAnalyzer<float>*>(h)->computeEncoding((uint8_t) bw, sym != 0,
                                                                                        strict != 0, unsignedSym != 0);
     putEncoding(e, out5);
+}
+// ---- MseEncodingAnalyzer<float> ------------------------------------------------------------------
+void* ref_mse_create()
+{
+    return new MseEncodingAnalyzer<float>();
+}
+void ref_mse_destroy(void* h)
+{
+    delete static_cast<MseEncodingAnalyzer<float>*>(h);
+}
+void ref_mse_update(void* h, const float* data, int64_t n)
+{
+    static_cast<MseEncodingAnalyzer<float>*>(h)->updateStats(data, (size_t) n, COMP_MODE_CPU);
+}
+void ref_mse_compute(void* h, int bw, int sym, int strict, int unsignedSym, double* out5)
+{
+    TfEncoding e = static_cast<MseEncodingAnalyzer<float>*>(h)->computeEncoding((uint8_t) bw, sym != 0, strict != 0,
+                                                                                unsignedSym != 0);
+    putEncoding(e, out5);
+}
+// the (min, max) pair the search settles on, before zero is gated in and the grid is formed
+void ref_mse_minimize(void* h, int bw, int sym, int strict, int unsignedSym, float* bestMin, float* bestMax)
+{
+    auto* a                      = static_cast<MseEncodingAnalyzer<float>*>(h);
+    std::tie(*bestMin, *bestMax) = a->_minimizeMSE((uint8_t) bw, sym != 0, strict != 0, unsignedSym != 0);
+}
+// the cost of one candidate on explicit bucket centres
+float ref_mse_cost(void* h, int bw, const float* centers, const float* pdfAtCenter, int n, float candMin,
+                   float candMax, int sym, int strict, int unsignedSym)
+{
+    auto* a = static_cast<MseEncodingAnalyzer<float>*>(h);
+    std::vector<std::pair<float, float>> centersPdf((size_t) n);
+    for (int i = 0; i < n; ++i)
+        centersPdf[(size_t) i] = {centers[i], pdfAtCenter[i]};
+    return a->_computeMSECost((uint8_t) bw, centersPdf, candMin, candMax, sym != 0, strict != 0, unsignedSym != 0);
 }
 }   // extern "C"

@@ -424,3 +424,79 @@ def test_percentile_cases_of_the_reference_unit_tests(oracle):
     e = pdf.compute_percentile_encoding(8, 99.9999)
     assert e.min == pytest.approx(-1.00392, abs=1e-4) and e.max == pytest.approx(0.996078, abs=1e-4)
     assert e.offset == -128 and e.bw == 8
+
+
+def test_mse_cases_of_the_reference_unit_tests(oracle):
+    """ModelOptimizations/DlQuantization/test/TestMseEncodingAnalyzer.cpp:56-317: the assertions of its cases on data
+    of the same distributions (the reference draws from std::normal_distribution; the bounds it asserts hold for any
+    sample of that size)."""
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal(100000) * 2 + 2).astype(np.float32)
+    pdf = oracle.new_pdf()
+    pdf.update(x)
+    e = pdf.compute_mse_encoding(8)                                       # Asymmetric, :56-114
+    assert 2 - 12 < e.min < 2 - 4 and 2 + 4 < e.max < 2 + 12
+    # the reference also asserts min and max strictly inside the sample's extremes, which holds for its own draw; on
+    # any draw they lie within one bucket of them
+    bucket = pdf.x_left()[1] - pdf.x_left()[0]
+    assert e.min > x.min() - bucket and e.max < x.max() + bucket
+    x = (rng.standard_normal(6000) * 2 + 2).astype(np.float32)
+    pdf = oracle.new_pdf()
+    pdf.update(x)
+    e = pdf.compute_mse_encoding(8, sym=True)                             # Symmetric, :116-163
+    assert e.min > -np.abs(x).max() and e.max < np.abs(x).max() and e.offset == -128 and e.bw == 8
+    assert e.delta == pytest.approx((e.max - e.min) / 255, rel=1e-6)
+    assert e.offset == pytest.approx(e.min / e.delta, rel=1e-6)
+    x = (rng.standard_normal(6000) - 2).astype(np.float32)
+    pdf = oracle.new_pdf()
+    pdf.update(x)
+    e = pdf.compute_mse_encoding(8, sym=True, strict=True)                # StrictSymmetric, :165-211
+    assert e.min > -np.abs(x).max() and e.max < np.abs(x).max()
+    assert e.offset == -127 and e.min == -e.max and e.delta == pytest.approx((e.max - e.min) / 254, rel=1e-6)
+    pos = np.maximum(x, 0)
+    pdf = oracle.new_pdf()
+    pdf.update(pos)
+    e = pdf.compute_mse_encoding(8, sym=True, unsigned_sym=True)          # SymmetricUnsigned, :213-260
+    assert e.min == 0 and e.max < np.abs(x).max() and e.bw == 8
+    assert e.delta == pytest.approx((e.max - e.min) / 255, rel=1e-6) and e.offset == 0
+    pdf = oracle.new_pdf()                                                # AllSameValuesAsymmetric, :262-295
+    pdf.update(np.full(100, 4, np.float32))
+    e = pdf.compute_mse_encoding(8)
+    assert e.min <= 0 and e.max >= 3.9
+    pdf = oracle.new_pdf()
+    pdf.update(np.full(100, -5, np.float32))
+    e = pdf.compute_mse_encoding(8)
+    assert e.min <= -4.99992 and e.max >= 0
+    pdf = oracle.new_pdf()                                                # AllZeroesAsymmetric, :297-317
+    pdf.update(np.zeros(6000, np.float32))
+    e = pdf.compute_mse_encoding(8)
+    assert e.min == pytest.approx(-1.00392, abs=1e-4) and e.max == pytest.approx(0.996078, abs=1e-4)
+    assert e.offset == -128 and e.bw == 8
+
+
+def test_mse_search_against_brute_force(oracle):
+    """The pair the search returns has the least cost among all pairs, by a cost written here from the definition
+    (numpy, float64): quantize-dequantize of the bucket centres on the grid of (min, max), squared error weighted by
+    the PDF.  A wrong clamp, a missed candidate or a dropped weight moves the winner."""
+    rng = np.random.default_rng(3)
+    x = np.concatenate([rng.standard_normal(50000), 8 * rng.standard_normal(200)]).astype(np.float32)
+    pdf = oracle.new_pdf()
+    pdf.update(x)
+    best_min, best_max, mins, maxs, centers = pdf.mse_minimize(4)
+    x_left, p = pdf.x_left(), pdf.pdf()
+    index = np.clip(np.floor((centers.astype(np.float64) - x_left[0]) / (x_left[1] - x_left[0])), 0, 511).astype(int)
+    weight = p[index]
+    c = centers.astype(np.float64)
+
+    def cost(lo, hi):
+        delta = (hi - lo) / 15
+        offset = np.round(lo / delta)
+        if lo < 0 < hi:
+            offset = -min(15.0, max(0.0, np.round(-lo / delta)))
+        q = np.floor(np.clip(c, lo, hi) / delta - offset + 0.5)
+        return float(np.sum(weight * (c - delta * (q + offset)) ** 2))
+    costs = np.array([[cost(float(lo), float(hi)) if (lo, hi) != (0, 0) else np.inf for hi in maxs] for lo in mins])
+    i, j = np.unravel_index(np.argmin(costs), costs.shape)
+    assert costs[i, j] == pytest.approx(cost(float(best_min), float(best_max)), rel=1e-4)
+    assert best_min < 0 < best_max and best_max < x.max() and best_min > x.min()      # outliers are clipped
+    assert len(mins) + len(maxs) >= 100 and mins[-1] == 0 and maxs[-1] == 0

@@ -220,3 +220,69 @@ def test_percentile_analyzer_without_usable_statistics(oracle, ref):
     an.update(z)
     for bw, sym, strict in ((8, False, False), (8, True, True), (4, False, False)):
         assert pdf.compute_percentile_encoding(bw, 99.0, sym, strict).astuple() == an.compute_encoding(bw, sym, strict)
+
+
+def _mse_batches(rng, kind):
+    batches = []
+    for b in range(3):
+        x = (rng.standard_normal(20000) * (1 + b) + 0.5).astype(np.float32)
+        if kind == "relu":
+            x = np.maximum(x, 0)
+        elif kind == "negative":
+            x = -np.abs(x) - 0.25
+        elif kind == "outliers":
+            x[:5] = 300.0
+        elif kind == "constant":
+            x[:] = 4.0
+        elif kind == "zeros-then-data" and b == 0:
+            x[:] = 0.0
+        elif kind == "far-from-zero":
+            x = x * 0.01 + 50.0
+        batches.append(x)
+    return batches
+
+
+@pytest.mark.parametrize("kind", ["normal", "relu", "negative", "outliers", "constant", "zeros-then-data",
+                                  "far-from-zero"])
+def test_mse_analyzer(oracle, ref, kind):
+    """MseEncodingAnalyzer<float>: the PDF of TF-Enhanced, every pair of bucket edges either side of zero as a
+    candidate range, squared error of the bucket centres as cost.  The winning pair and every field of the encoding."""
+    rng = np.random.default_rng(len(kind))
+    pdf, an = oracle.new_pdf(), ref.new_mse()
+    for x in _mse_batches(rng, kind):
+        pdf.update(x)
+        an.update(x)
+    for bw in (4, 8, 16):
+        for sym, strict, uns in ((False, False, False), (True, False, False), (True, True, False), (True, False, True)):
+            best = pdf.mse_minimize(bw, sym, strict, uns)
+            assert (best[0], best[1]) == an.minimize(bw, sym, strict, uns), (kind, bw, sym, strict, uns)
+            got = pdf.compute_mse_encoding(bw, sym, strict, uns)
+            assert got.astuple() == an.compute_encoding(bw, sym, strict, uns), (kind, bw, sym, strict, uns)
+
+
+def test_mse_cost_of_single_candidates(oracle, ref):
+    """The cost function alone, on centres and weights that are not a PDF's: ranges that clip, that do not, one-sided
+    ranges, all four symmetry modes."""
+    rng = np.random.default_rng(5)
+    an = ref.new_mse()
+    centers = np.sort(rng.standard_normal(300).astype(np.float32) * 3)
+    weights = rng.random(300).astype(np.float32)
+    weights /= weights.sum()
+    for bw in (2, 4, 8, 16, 24):
+        for lo, hi in ((-1.0, 1.0), (-9.5, 0.25), (0.0, 2.0), (-3.0, 0.0), (-20.0, 20.0), (-1e-3, 1e-3)):
+            for sym, strict, uns in ((False, False, False), (True, False, False), (True, True, False),
+                                     (True, False, True)):
+                got = np.float32(oracle.L.orc_mse_cost(bw, centers, weights, centers.size, lo, hi, int(sym),
+                                                       int(strict), int(uns)))
+                want = an.cost(bw, centers, weights, lo, hi, sym, strict, uns)
+                assert got.tobytes() == want.tobytes(), (bw, lo, hi, sym, strict, uns)
+
+
+def test_mse_analyzer_without_usable_statistics(oracle, ref):
+    pdf, an = oracle.new_pdf(), ref.new_mse()
+    assert pdf.compute_mse_encoding(8).astuple() == an.compute_encoding(8)                   # nothing seen: zeros
+    z = np.zeros(100, np.float32)
+    pdf.update(z)
+    an.update(z)
+    for bw, sym, strict in ((8, False, False), (8, True, True), (4, False, False)):
+        assert pdf.compute_mse_encoding(bw, sym, strict).astuple() == an.compute_encoding(bw, sym, strict)
