@@ -15,7 +15,8 @@ from .. import ops
 from .libpymo import QuantizationMode, RoundingMode, TfEncoding
 
 _MODE_TO_MIQ = {QuantizationMode.QUANTIZATION_TF: 0, QuantizationMode.QUANTIZATION_TF_ENHANCED: 1,
-                QuantizationMode.QUANTIZATION_PERCENTILE: 2, QuantizationMode.QUANTIZATION_MSE: 3}
+                QuantizationMode.QUANTIZATION_PERCENTILE: 2, QuantizationMode.QUANTIZATION_MSE: 3,
+                QuantizationMode.QUANTIZATION_ENTROPY: 4}
 
 
 def _round_mode(round_mode) -> int:
@@ -33,8 +34,7 @@ class AimetTensorQuantizer:
 
     def __init__(self, quantizationScheme: QuantizationMode):
         if quantizationScheme not in _MODE_TO_MIQ:
-            raise RuntimeError(f"{quantizationScheme} is not implemented: QUANTIZATION_TF, "
-                               "QUANTIZATION_TF_ENHANCED, QUANTIZATION_PERCENTILE and QUANTIZATION_MSE are")
+            raise RuntimeError(f"{quantizationScheme} has no encoding analyzer")
         self._scheme = quantizationScheme
         self._percentile = 100.0
         self._analyzer = None          # created on the first updateStats, on that tensor's device

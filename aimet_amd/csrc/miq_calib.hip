@@ -19,6 +19,7 @@
 #include "miq_fastmath.h"
 #include "miq_tfe_search.h"
 #include "miq_encoding_math.h"
+#include "miq_entropy.h"
 
 #include <algorithm>
 #include <cfloat>
@@ -1261,6 +1262,7 @@ struct miq_analyzer
     int mode;
     float percentile;    // percentile analyzer only
     MseScratch* mse;     // MSE analyzer only: candidate lists, bucket centres, per-workgroup winners (device)
+    EntropyAnalyzer* entropy;   // entropy analyzer only: its own histogram and search; `st` is not used
     int device;
     DevState* st;        // device
     void* pinned;        // host staging (pinned) for read-backs
@@ -1442,9 +1444,10 @@ int miq_analyzer_create_in(int quantization_mode, void* device_state, miq_analyz
     MIQ_CHECK_ARG(out != nullptr, "null output handle");
     MIQ_CHECK_ARG(device_state == nullptr || aligned16(device_state), "device_state must be 16-byte aligned");
     if (quantization_mode != MIQ_QUANTIZATION_TF && quantization_mode != MIQ_QUANTIZATION_TF_ENHANCED &&
-        quantization_mode != MIQ_QUANTIZATION_PERCENTILE && quantization_mode != MIQ_QUANTIZATION_MSE)
+        quantization_mode != MIQ_QUANTIZATION_PERCENTILE && quantization_mode != MIQ_QUANTIZATION_MSE &&
+        quantization_mode != MIQ_QUANTIZATION_ENTROPY)
     {
-        set_error("quantization mode %d is not implemented (TF, TF_ENHANCED, PERCENTILE and MSE are)",
+        set_error("quantization mode %d is not implemented (TF, TF_ENHANCED, PERCENTILE, MSE and ENTROPY are)",
                   quantization_mode);
         return MIQ_ERR_UNSUPPORTED;
     }
@@ -1453,6 +1456,7 @@ int miq_analyzer_create_in(int quantization_mode, void* device_state, miq_analyz
     a->mode          = quantization_mode;
     a->percentile    = 100.0f;   // PercentileEncodingAnalyzer.h: the default clips nothing
     a->mse           = nullptr;
+    a->entropy       = nullptr;
     a->st            = static_cast<DevState*>(device_state);
     a->owns_state    = (device_state == nullptr);
     a->needs_reset   = true;
@@ -1467,6 +1471,19 @@ int miq_analyzer_create_in(int quantization_mode, void* device_state, miq_analyz
     a->seq           = 0;
     a->last_bw       = 0;
     hipError_t e     = hipGetDevice(&a->device);
+    if (e == hipSuccess && quantization_mode == MIQ_QUANTIZATION_ENTROPY)
+    {
+        // the entropy analyzer keeps a histogram of its own kind in memory of its own; a caller's state is left alone
+        a->owns_state = false;
+        a->st         = nullptr;
+        if (int rc = entropy_create(&a->entropy))
+        {
+            delete a;
+            return rc;
+        }
+        *out = a;
+        return MIQ_OK;
+    }
     if (e == hipSuccess && a->owns_state)
         e = hipMalloc((void**) &a->st, sizeof(DevState));
     if (e == hipSuccess && quantization_mode == MIQ_QUANTIZATION_MSE)
@@ -1513,7 +1530,9 @@ int miq_analyzer_destroy(miq_analyzer* a)
         (void) hipFree(a->st);
     if (a->mse)
         (void) hipFree(a->mse);
-    (void) hipHostFree(a->pinned);
+    entropy_destroy(a->entropy);
+    if (a->pinned)
+        (void) hipHostFree(a->pinned);
     delete a;
     return MIQ_OK;
 }
@@ -1521,6 +1540,12 @@ int miq_analyzer_destroy(miq_analyzer* a)
 int miq_analyzer_reset(miq_analyzer* a, void* stream)
 {
     MIQ_CHECK_ARG(a != nullptr, "null analyzer");
+    if (a->entropy)
+    {
+        a->stats_updated = false;
+        a->queued        = false;
+        return entropy_reset(a->entropy, (hipStream_t) stream);
+    }
     hipLaunchKernelGGL(reset_state_kernel, dim3(1), dim3(kPdf), 0, (hipStream_t) stream, a->st);
     MIQ_CHECK_LAUNCH();
     a->needs_reset = false;
@@ -1540,6 +1565,12 @@ int miq_analyzer_update_stats_f32(miq_analyzer* a, const float* data, int64_t n,
     MIQ_CHECK_ARG(n > 0 && data, "update_stats needs a non-empty tensor");
     hipStream_t s  = (hipStream_t) stream;
     const bool vec = aligned16(data);
+    if (a->entropy)
+    {
+        a->stats_updated = true;
+        a->queued        = false;
+        return entropy_update(a->entropy, data, n, s);
+    }
     if (int rc = ensure_reset(a, s))
         return rc;
     a->stats_updated = true;
@@ -1680,7 +1711,7 @@ int miq_analyzer_queue_encoding(miq_analyzer* a, int bw, int use_symmetric, int 
 {
     MIQ_CHECK_ARG(a != nullptr, "null argument");
     MIQ_CHECK_ARG(bw >= 1 && bw <= 32, "bitwidth must be in [1, 32] (got %d)", bw);
-    if (!a->stats_updated)
+    if (!a->stats_updated || a->entropy)   // the entropy search runs on the host: nothing to queue ahead
         return MIQ_OK;
     if (int rc = queue_encoding(a, bw, use_symmetric, use_strict_symmetric, use_unsigned_symmetric, (hipStream_t) stream))
         return rc;
@@ -1703,6 +1734,8 @@ int miq_analyzer_compute_encoding(miq_analyzer* a, int bw, int use_symmetric, in
     *is_valid = a->stats_updated ? 1 : 0;
     if (!a->stats_updated)
         return MIQ_OK;   // AimetTensorQuantizer::getEncoding returns a default encoding and valid = false
+    if (a->entropy)
+        return entropy_compute(a->entropy, bw, use_symmetric, use_strict_symmetric, use_unsigned_symmetric, out, s);
     const bool ahead = a->queued && a->queued_stream == s && a->queued_args[0] == bw &&
                        a->queued_args[1] == (use_symmetric != 0) && a->queued_args[2] == (use_strict_symmetric != 0) &&
                        a->queued_args[3] == (use_unsigned_symmetric != 0);
@@ -1741,6 +1774,14 @@ int miq_analyzer_get_stats_histogram(miq_analyzer* a, double* x_left, double* pd
         set_error("no histogram is kept by the TF (min/max) analyzer");
         return MIQ_ERR_UNSUPPORTED;
     }
+    if (a->entropy)
+    {
+        // the reference's getStatsHistogram for this analyzer appends to vectors it has already sized
+        // (DLQ/src/EntropyEncodingAnalyzer.cpp:54-78) and has no defined result; the counts themselves are read with
+        // miq_analyzer_entropy_histogram
+        set_error("the entropy analyzer keeps counts over a moving range, not a PDF: use miq_analyzer_entropy_histogram");
+        return MIQ_ERR_UNSUPPORTED;
+    }
     if (int rc = flush_pending(a, (hipStream_t) stream))
         return rc;
     if (int rc = read_state(a, (hipStream_t) stream))
@@ -1755,9 +1796,22 @@ int miq_analyzer_get_stats_histogram(miq_analyzer* a, double* x_left, double* pd
     return MIQ_OK;
 }
 
+int miq_analyzer_entropy_histogram(miq_analyzer* a, double* counts, double* range_min_max, int* initialized,
+                                   int* iterations, void* stream)
+{
+    MIQ_CHECK_ARG(a && counts && range_min_max && initialized && iterations, "null argument");
+    MIQ_CHECK_ARG(a->entropy != nullptr, "not an entropy analyzer");
+    return entropy_histogram(a->entropy, counts, range_min_max, initialized, iterations, (hipStream_t) stream);
+}
+
 int miq_analyzer_last_batch_counts(miq_analyzer* a, uint32_t* counts, void* stream)
 {
     MIQ_CHECK_ARG(a && counts, "null argument");
+    if (a->entropy)
+    {
+        set_error("the entropy analyzer does not keep the last batch apart: use miq_analyzer_entropy_histogram");
+        return MIQ_ERR_UNSUPPORTED;
+    }
     if (int rc = flush_pending(a, (hipStream_t) stream))
         return rc;
     if (int rc = read_state(a, (hipStream_t) stream))
@@ -1770,6 +1824,11 @@ int miq_analyzer_last_search(miq_analyzer* a, float* deltas, int32_t* offsets, d
                              int* best_index, void* stream)
 {
     MIQ_CHECK_ARG(a && deltas && offsets && costs && count && best_index && cap >= 0, "bad argument");
+    if (a->entropy)
+    {
+        set_error("the entropy analyzer has no candidate list");
+        return MIQ_ERR_UNSUPPORTED;
+    }
     if (int rc = read_state(a, (hipStream_t) stream))
         return rc;
     const DevState* h = static_cast<const DevState*>(a->pinned);

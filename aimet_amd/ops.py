@@ -899,7 +899,8 @@ class _StateOwner:
 
 class Analyzer(_StateOwner):
     """Device-resident encoding analyzer: mode 0 = TF min/max, 1 = TF-Enhanced (512-bucket PDF + SQNR search),
-    2 = percentile on the same PDF, 3 = least squared error over pairs of bucket edges of the same PDF."""
+    2 = percentile on the same PDF, 3 = least squared error over pairs of bucket edges of the same PDF, 4 = least KL
+    divergence over windows of a 512-bin histogram that follows the range of the data."""
 
     def __init__(self, mode, device=None):
         self.mode = int(mode)
@@ -974,6 +975,17 @@ class Analyzer(_StateOwner):
             check(lib.miq_analyzer_get_stats_histogram(self._h, xl.ctypes.data, pdf.ctypes.data, C.byref(n),
                                                        self._s()))
         return xl[:n.value], pdf[:n.value]
+
+    def entropy_histogram(self):
+        """Entropy analyzer only: (512 counts, (min, max) of the range they span, whether a batch other than all zeros
+        has been seen, number of batches counted)."""
+        import numpy as np
+        counts, span = np.zeros(_lib.PDF_SIZE), np.zeros(2)
+        seen, batches = C.c_int(0), C.c_int(0)
+        with torch.cuda.device(self.device):
+            check(lib.miq_analyzer_entropy_histogram(self._h, counts.ctypes.data, span.ctypes.data, C.byref(seen),
+                                                     C.byref(batches), self._s()))
+        return counts, (float(span[0]), float(span[1])), bool(seen.value), batches.value
 
     def last_batch_counts(self):
         import numpy as np

@@ -47,6 +47,7 @@ int miq_get_stochastic_state(uint64_t* seed /* host */, uint64_t* calls /* host 
 #define MIQ_QUANTIZATION_TF_ENHANCED 1
 #define MIQ_QUANTIZATION_PERCENTILE 2
 #define MIQ_QUANTIZATION_MSE 3
+#define MIQ_QUANTIZATION_ENTROPY 4
 
 #define MIQ_PDF_SIZE 512 /* DLQ/src/math_functions.hpp:80 */
 
@@ -397,7 +398,12 @@ int miq_minmax_per_channel_static_f32(const float* in, int64_t num_channel, int6
  * the same PDF; every pair of one bucket edge below zero and one above, zero included on either side, is a candidate
  * range, searched on the device for the least PDF-weighted squared quantization error of the bucket centres; this
  * analyzer holds 25 KB more device memory than the others, allocated by the library also when the state is the
- * caller's).  All statistics (running min/max,
+ * caller's) and QUANTIZATION_ENTROPY (EntropyEncodingAnalyzer, DLQ/src/EntropyEncodingAnalyzer.cpp:54-436, over
+ * updateTensorHistogram_cpu / rescaleHistogram, DLQ/src/math_functions.cpp:468-643: 512 counts over exactly the range
+ * seen so far, moved into new bins whenever a batch widens it; for 8 bits the range is narrowed to the window whose
+ * 255-level quantization has the least KL divergence from the histogram saturated into it, searched on the host over
+ * the counts read back; this analyzer allocates its own device state and ignores a caller's; samples are taken to be
+ * finite).  All statistics (running min/max,
  * the 512-bucket PDF, its range and iteration count) live in device memory owned by the object on the device that
  * was current at creation; update_stats enqueues work and never synchronises.  compute_encoding synchronises
  * `stream` once to read the result back.  An object must not be used from two threads at once. */
@@ -438,6 +444,13 @@ int miq_analyzer_queue_encoding(miq_analyzer* a, int bw, int use_symmetric, int 
  * has not been initialised. */
 int miq_analyzer_get_stats_histogram(miq_analyzer* a, double* x_left /* host[512] */, double* pdf /* host[512] */,
                                      int* num_buckets /* host */, void* stream);
+/* The entropy analyzer's histogram as it stands (TensorProfilingParams, DLQ/src/math_functions.hpp:69-77): 512
+ * counts, the range they span, whether a batch other than all zeros has been seen, and the number of batches counted.
+ * MIQ_ERR_INVALID_ARG for any other analyzer.  (miq_analyzer_get_stats_histogram is MIQ_ERR_UNSUPPORTED for the
+ * entropy analyzer: the reference's own getStatsHistogram for it has no defined result.) */
+int miq_analyzer_entropy_histogram(miq_analyzer* a, double* counts /* host[512] */,
+                                   double* range_min_max /* host[2] */, int* initialized /* host */,
+                                   int* iterations /* host */, void* stream);
 /* Test/inspection hooks: the integer bin counts of the most recent update_stats call (host uint32[512]) and the
  * TF-Enhanced candidate list with every candidate's cost from the most recent compute_encoding call
  * (host arrays of capacity `cap`; *count receives the number of candidates, *best_index the winner). */

@@ -46,6 +46,11 @@ class _PdfStruct(C.Structure):
                 ("initialized", C.c_int), ("stats_updated", C.c_int)]
 
 
+class _ProfileStruct(C.Structure):
+    _fields_ = [("min", C.c_double), ("max", C.c_double), ("histogram", C.c_double * PDF_SIZE),
+                ("iterations", C.c_int), ("initialized", C.c_int), ("stats_updated", C.c_int)]
+
+
 def _f32(a):
     return np.ascontiguousarray(a, dtype=np.float32)
 
@@ -90,6 +95,13 @@ class _Oracle:
                                                C.POINTER(Encoding)]
         L.orc_mse_cost.restype = C.c_float
         L.orc_mse_cost.argtypes = [C.c_int, _f32p, _f32p, C.c_int, C.c_float, C.c_float, C.c_int, C.c_int, C.c_int]
+        L.orc_profile_reset.argtypes = [C.POINTER(_ProfileStruct)]
+        L.orc_profile_update_f32.argtypes = [C.POINTER(_ProfileStruct), _f32p, _i64]
+        L.orc_entropy_optimize_kl.argtypes = [C.POINTER(_ProfileStruct), C.c_int, C.c_int, C.c_int, C.c_int,
+                                              C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p,
+                                              C.POINTER(C.c_int)]
+        L.orc_entropy_compute_encoding.argtypes = [C.POINTER(_ProfileStruct), C.c_int, C.c_int, C.c_int, C.c_int,
+                                                   C.POINTER(Encoding)]
         L.orc_v2_qdq_f32.argtypes = [_f32p, _i64, _i64, _i64, C.c_void_p, C.c_void_p, C.c_void_p, _f32p, _f32p,
                                      C.c_int, C.c_int]
         L.orc_v2_qdq_bf16.argtypes = [_u16p, _i64, _i64, _i64, _u16p, C.c_void_p, _f32p, _f32p, C.c_int, C.c_int]
@@ -223,6 +235,9 @@ class _Oracle:
     def new_pdf(self):
         return OraclePdf(self)
 
+    def new_profile(self):
+        return OracleProfile(self)
+
     # -- v2 ----------------------------------------------------------------------------------------------------
     def v2_qdq(self, x, num_channel, n_per_channel, scale, offset, qmin, qmax):
         """returns (dequantized, codes, mask)"""
@@ -352,6 +367,48 @@ class OraclePdf:
         return e
 
 
+class OracleProfile:
+    """The rescaling 512-bin histogram of the entropy analyzer (TensorProfilingParams) and its searches."""
+
+    def __init__(self, o):
+        self.o = o
+        self.s = _ProfileStruct()
+        o.L.orc_profile_reset(C.byref(self.s))
+
+    def update(self, x):
+        x = _f32(x)
+        self.o.L.orc_profile_update_f32(C.byref(self.s), x.reshape(-1), x.size)
+
+    @property
+    def initialized(self):
+        return bool(self.s.initialized)
+
+    @property
+    def iterations(self):
+        return self.s.iterations
+
+    def range(self):
+        return self.s.min, self.s.max
+
+    def histogram(self):
+        return np.array(self.s.histogram[:], np.float64)
+
+    def optimize_kl(self, bw, sym=False, strict=False, unsigned_sym=False):
+        """_optimizeKL: (min, max, divergence of every window tried)."""
+        a, b = C.c_float(), C.c_float()
+        div = np.empty(PDF_SIZE, np.float64)
+        n = C.c_int(0)
+        self.o.L.orc_entropy_optimize_kl(C.byref(self.s), bw, int(sym), int(strict), int(unsigned_sym), C.byref(a),
+                                         C.byref(b), div.ctypes.data, C.byref(n))
+        return np.float32(a.value), np.float32(b.value), div[:n.value].copy()
+
+    def compute_encoding(self, bw, sym=False, strict=False, unsigned_sym=False):
+        e = Encoding()
+        self.o.L.orc_entropy_compute_encoding(C.byref(self.s), bw, int(sym), int(strict), int(unsigned_sym),
+                                              C.byref(e))
+        return e
+
+
 class _Ref:
     """The reference's own CPU classes, compiled in place (present only where oracle/_ref was built)."""
 
@@ -464,6 +521,9 @@ class _Ref:
     def new_mse(self):
         return _RefMse(self)
 
+    def new_entropy(self):
+        return _RefEntropy(self)
+
 
 class _RefAnalyzer:
     def __init__(self, ref, enhanced):
@@ -572,6 +632,47 @@ class _RefMse:
         centers, pdf_at_center = _f32(centers), _f32(pdf_at_center)
         return np.float32(self.L.ref_mse_cost(self.h, bw, centers, pdf_at_center, centers.size, cand_min, cand_max,
                                               int(sym), int(strict), int(unsigned_sym)))
+
+
+class _RefEntropy:
+    """The reference's EntropyEncodingAnalyzer<float>, compiled in place."""
+
+    def __init__(self, ref):
+        L = self.L = ref.L
+        L.ref_entropy_create.restype = C.c_void_p
+        L.ref_entropy_create.argtypes = []
+        L.ref_entropy_destroy.argtypes = [C.c_void_p]
+        L.ref_entropy_update.argtypes = [C.c_void_p, _f32p, _i64]
+        L.ref_entropy_compute.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _f64p]
+        L.ref_entropy_get_histogram.argtypes = [C.c_void_p, _f64p, _f64p, C.POINTER(C.c_int)]
+        L.ref_entropy_optimize.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float),
+                                           C.POINTER(C.c_float)]
+        self.h = C.c_void_p(L.ref_entropy_create())
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            self.L.ref_entropy_destroy(self.h)
+            self.h = None
+
+    def update(self, x):
+        x = _f32(x)
+        self.L.ref_entropy_update(self.h, x.reshape(-1), x.size)
+
+    def compute_encoding(self, bw, sym=False, strict=False, unsigned_sym=False):
+        o = np.empty(5)
+        self.L.ref_entropy_compute(self.h, bw, int(sym), int(strict), int(unsigned_sym), o)
+        return _Ref._enc(o)
+
+    def histogram(self):
+        """(number of bins, histogram, (min, max), iterations)"""
+        hist, mm, it = np.zeros(PDF_SIZE), np.zeros(2), C.c_int(0)
+        n = self.L.ref_entropy_get_histogram(self.h, hist, mm, C.byref(it))
+        return n, hist, (mm[0], mm[1]), it.value
+
+    def optimize(self, bw, sym=False, strict=False, unsigned_sym=False):
+        a, b = C.c_float(), C.c_float()
+        self.L.ref_entropy_optimize(self.h, bw, int(sym), int(strict), int(unsigned_sym), C.byref(a), C.byref(b))
+        return np.float32(a.value), np.float32(b.value)
 
 
 def _load():

@@ -935,6 +935,335 @@ void orc_mse_compute_encoding(const orc_pdf* p, int bw, int sym, int strict, int
 }
 
 /* ------------------------------------------------------------------------------------------------------------
+ * Entropy (KL divergence) calibration: EntropyEncodingAnalyzer<float> (DLQ/src/EntropyEncodingAnalyzer.cpp:54-436)
+ * over the rescaling 512-bin histogram of updateTensorHistogram_cpu / rescaleHistogram
+ * (DLQ/src/math_functions.cpp:468-643).  The histogram spans exactly the range seen so far and is redistributed
+ * when a batch widens it; only for 8 bits is the range then narrowed, window by window, to the one whose 255-level
+ * quantization has the least KL divergence from the saturated histogram.
+ * Data are taken to be finite (the reference's bin index of a NaN or infinite sample is whatever the conversion of an
+ * out-of-range float to size_t yields).
+ * ---------------------------------------------------------------------------------------------------------- */
+typedef struct
+{
+    double min, max;
+    double histogram[ORC_PDF_SIZE];
+    int iterations;
+    int initialized;   /* histogram.size() != 0 in the reference */
+    int stats_updated; /* _statsUpdated */
+} orc_tensor_profile;  /* TensorProfilingParams, DLQ/src/math_functions.hpp:69-77 + EntropyEncodingAnalyzer.h */
+
+void orc_profile_reset(orc_tensor_profile* t)
+{
+    memset(t, 0, sizeof(*t));
+}
+
+/* getBin, math_functions.cpp:468-474: float arithmetic, the quotient truncated to size_t and capped at the last bin */
+static size_t orc_get_bin(size_t nBins, float binWidth, float minValue, float value)
+{
+    if (binWidth == 0)
+        return 0;
+    float q = (value - minValue) / binWidth;
+    if (!(q < (float) nBins) || q <= -1.0f)
+        return nBins - 1;
+    return (size_t) q;
+}
+
+/* std::accumulate(first, last, 0.f): the accumulator has the type of the initial value, float */
+static double orc_accumulate_in_float(const double* v, size_t n)
+{
+    float acc = 0.f;
+    for (size_t i = 0; i < n; ++i)
+        acc = (float) (acc + v[i]);
+    return acc;
+}
+
+/* updateTensorHistogram_cpu, math_functions.cpp:476-560 */
+void orc_profile_update_f32(orc_tensor_profile* t, const float* data, int64_t n)
+{
+    t->stats_updated = 1;
+    float mnf, mxf;
+    orc_minmax_f32(data, n, &mnf, &mxf);
+    double minInput = mnf, maxInput = mxf;
+    if (minInput == 0 && maxInput == 0)
+        return;
+    if (minInput == maxInput)
+    {
+        double widened = minInput + (float) 0.01;
+        maxInput       = STD_MAX(maxInput, widened);
+    }
+    if (!t->initialized)
+    {
+        memset(t->histogram, 0, sizeof(t->histogram));
+        t->min         = minInput;
+        t->max         = maxInput;
+        t->initialized = 1;
+    }
+    if (minInput < t->min || maxInput > t->max)
+    {
+        double newMin       = STD_MIN(minInput, t->min);
+        double newMax       = STD_MAX(maxInput, t->max);
+        double destBinWidth = (newMax - newMin) / ORC_PDF_SIZE;
+        double srcBinWidth  = (t->max - t->min) / ORC_PDF_SIZE;
+        double scaled[ORC_PDF_SIZE];
+        memset(scaled, 0, sizeof(scaled));
+        for (size_t i = 0; i < ORC_PDF_SIZE; ++i)
+        {
+            if (t->histogram[i] == 0)
+                continue;
+            double srcBinBegin = t->min + srcBinWidth * i;
+            size_t destBin     = (size_t) ((srcBinBegin - newMin) / destBinWidth);
+            double destBinEnd  = newMin + destBinWidth * (destBin + 1);
+            double share       = round((destBinEnd - srcBinBegin) / srcBinWidth * t->histogram[i]);
+            double dstBinCnt   = STD_MIN(share, t->histogram[i]);
+            size_t newBin      = orc_get_bin(ORC_PDF_SIZE, (float) destBinWidth, (float) newMin, (float) srcBinBegin);
+            scaled[newBin] += dstBinCnt;
+            if (dstBinCnt < t->histogram[i])
+            {
+                newBin = orc_get_bin(ORC_PDF_SIZE, (float) destBinWidth, (float) newMin,
+                                     (float) (srcBinBegin + destBinWidth));
+                scaled[newBin] += t->histogram[i] - dstBinCnt;
+            }
+        }
+        memcpy(t->histogram, scaled, sizeof(scaled));
+        t->min = newMin;
+        t->max = newMax;
+    }
+    float binWidth = (float) ((t->max - t->min) / ORC_PDF_SIZE);
+    for (int64_t i = 0; i < n; ++i)
+        t->histogram[orc_get_bin(ORC_PDF_SIZE, binWidth, (float) t->min, data[i])] += 1;
+    t->iterations++;
+}
+
+/* rescaleHistogram, math_functions.cpp:562-643 */
+static void orc_rescale_histogram(const double* srcHist, double srcHistMin, double srcHistMax, double destHistMin,
+                                  double destHistMax, double* destHist)
+{
+    const size_t numBins = ORC_PDF_SIZE;
+    if (srcHistMin == destHistMin && srcHistMax == destHistMax)
+    {
+        memcpy(destHist, srcHist, sizeof(double) * numBins);
+        return;
+    }
+    const double srcBinWidth  = (srcHistMax - srcHistMin) / numBins;
+    const double destBinWidth = (destHistMax - destHistMin) / numBins;
+    memset(destHist, 0, sizeof(double) * numBins);
+    for (size_t srcBinIdx = 0; srcBinIdx < numBins; srcBinIdx++)
+    {
+        double srcBinVal = srcHist[srcBinIdx];
+        if (srcBinVal == 0)
+            continue;
+        double srcBinStart     = srcHistMin + srcBinIdx * srcBinWidth;
+        double srcBinStop      = srcHistMin + (srcBinIdx + 1) * srcBinWidth;
+        double dstBinIdxStartF = floor((srcBinStart - destHistMin) / destBinWidth);
+        double dstBinIdxStopF  = ceil((srcBinStop - destHistMin) / destBinWidth);
+        size_t dstBinIdxStart  = (size_t) STD_MAX(dstBinIdxStartF, 0.0);
+        size_t dstBinIdxStop   = (size_t) STD_MAX(dstBinIdxStopF, 0.0);
+        if (dstBinIdxStart >= numBins)
+            dstBinIdxStart = numBins - 1;
+        if (dstBinIdxStop >= numBins)
+            dstBinIdxStop = numBins - 1;
+        double srcBinRem = srcBinVal;
+        for (size_t destBinIdx = dstBinIdxStart; destBinIdx <= dstBinIdxStop; destBinIdx++)
+        {
+            double destBinStart = destHistMin + destBinIdx * destBinWidth;
+            double destBinStop  = destHistMin + (destBinIdx + 1) * destBinWidth;
+            double overlapStart = STD_MAX(srcBinStart, destBinStart);
+            double overlapStop  = STD_MIN(srcBinStop, destBinStop);
+            double overlapRatio = (overlapStop - overlapStart) / srcBinWidth;
+            overlapRatio        = overlapRatio >= 0.0f ? overlapRatio : 0.0f;
+            overlapRatio        = overlapRatio <= 1.0f ? overlapRatio : 1.0f;
+            double distVal      = round(overlapRatio * srcBinVal);
+            distVal             = distVal <= srcBinRem ? distVal : srcBinRem;
+            destHist[destBinIdx] += distVal;
+            srcBinRem -= distVal;
+        }
+    }
+}
+
+/* _conditionHistogram, EntropyEncodingAnalyzer.cpp:153-200 */
+static void orc_condition_histogram(double* hist, size_t length)
+{
+    const double epsZero = 0.0001;
+    if (length == 0)
+        return;
+    size_t numZeros = 0;
+    for (size_t i = 0; i < length; ++i)
+        numZeros += (hist[i] == 0.f);
+    if (numZeros == length)
+        return;
+    size_t numNonZeros = length - numZeros;
+    double epsNonZero  = epsZero * (double) numZeros / (double) numNonZeros;
+    if (epsNonZero >= 1.0)
+        return;
+    for (size_t i = 0; i < length; ++i)
+    {
+        int isZero = (hist[i] == 0.f);
+        hist[i] += epsZero * isZero;
+        hist[i] -= epsNonZero * (1 - isZero);
+    }
+}
+
+/* _computeKL, :202-228 (P and Q are normalised in place) */
+static double orc_compute_kl(double* P, double* Q, size_t length)
+{
+    double sumP       = orc_accumulate_in_float(P, length);
+    double sumQ       = orc_accumulate_in_float(Q, length);
+    double divergence = 0;
+    for (size_t i = 0; i < length; ++i)
+    {
+        P[i] /= sumP;
+        Q[i] /= sumQ;
+        if (P[i] > 0 && Q[i] > 0)
+            divergence += P[i] * log(P[i] / Q[i]);
+    }
+    return divergence;
+}
+
+/* _optimizeKL, :230-431.  divergences (optional, ORC_PDF_SIZE doubles) receives the divergence of every window
+ * tried, in order; *numWindows their count. */
+void orc_entropy_optimize_kl(const orc_tensor_profile* t, int bw, int sym, int strict, int unsignedSym, float* minOut,
+                             float* maxOut, double* divergences, int* numWindows)
+{
+    double histMin = t->min, histMax = t->max;
+    double hist[ORC_PDF_SIZE];
+    if (numWindows)
+        *numWindows = 0;
+    if (sym && (histMin < 0.0 || !unsignedSym))
+    {
+        double absHi      = fabs(histMax), absLo = fabs(histMin);
+        float absoluteMax = (float) STD_MAX(absHi, absLo);
+        float absoluteMin = -absoluteMax;
+        orc_rescale_histogram(t->histogram, histMin, histMax, absoluteMin, absoluteMax, hist);
+        histMin = absoluteMin;
+        histMax = absoluteMax;
+    }
+    else
+        memcpy(hist, t->histogram, sizeof(hist));
+
+    const size_t numBins          = ORC_PDF_SIZE;
+    const size_t numQuantizedBins = 255;
+    if (bw != 8)
+    {
+        *minOut = (float) histMin;
+        *maxOut = (float) histMax;
+        return;
+    }
+    const double histBinWidth = (histMax - histMin) / (double) numBins;
+    double divergenceOpt      = INFINITY;
+    double thresholdMinOpt = histMin, thresholdMaxOpt = histMax;
+    size_t start = 0, stop = numBins - 1;
+    double P[ORC_PDF_SIZE], Q[ORC_PDF_SIZE];
+    while ((stop - start + 1) >= numQuantizedBins)
+    {
+        const size_t winSize = stop - start + 1;
+        const double* win    = hist + start;
+        memset(P, 0, sizeof(double) * winSize);
+        double leftSum = 0;
+        for (size_t i = 0; i <= start; i++)
+            leftSum += hist[i];
+        P[0] += leftSum;
+        for (size_t i = start + 1; i < stop; i++)
+            P[i - start] = hist[i];
+        double rightSum = 0;
+        for (size_t i = stop; i < numBins; i++)
+            rightSum += hist[i];
+        P[winSize - 1] += rightSum;
+
+        const double numMergedBins = (double) winSize / (double) numQuantizedBins;
+        memset(Q, 0, sizeof(double) * winSize);
+        for (size_t q = 0; q < numQuantizedBins; q++)
+        {
+            const size_t idxStart = (size_t) ceil(q * numMergedBins);
+            const size_t idxStop  = (q < numQuantizedBins - 1) ? (size_t) ceil((q + 1) * numMergedBins) : winSize;
+            double sum = 0, norm = 0;
+            for (size_t i = idxStart; i < idxStop; i++)
+            {
+                sum += win[i];
+                norm += (win[i] != 0);
+            }
+            if (norm != 0)
+                for (size_t i = idxStart; i < idxStop; i++)
+                    if (win[i])
+                        Q[i] = sum / norm;
+        }
+        double sumP = orc_accumulate_in_float(P, winSize);
+        double sumQ = orc_accumulate_in_float(Q, winSize);
+        if (sumP == 0 || sumQ == 0)
+            break;
+        orc_condition_histogram(P, winSize);
+        orc_condition_histogram(Q, winSize);
+        double divergence = orc_compute_kl(P, Q, winSize);
+        if (divergences && numWindows && *numWindows < ORC_PDF_SIZE)
+            divergences[(*numWindows)++] = divergence;
+        if (divergence < divergenceOpt)
+        {
+            divergenceOpt   = divergence;
+            thresholdMinOpt = histMin + start * histBinWidth;
+            thresholdMaxOpt = histMin + (stop + 1) * histBinWidth;
+        }
+        if (sym || strict)
+        {
+            start++;
+            stop--;
+        }
+        else
+        {
+            double loss[3] = {hist[start] + hist[stop], hist[start] + hist[start + 1], hist[stop] + hist[stop - 1]};
+            int lossMinIdx = 0; /* std::min_element: the first of equal minima */
+            for (int k = 1; k < 3; ++k)
+                if (loss[k] < loss[lossMinIdx])
+                    lossMinIdx = k;
+            if ((lossMinIdx == 0 && (histMin + (start + 1) * histBinWidth) > 0) ||
+                (lossMinIdx == 1 && (histMin + (start + 2) * histBinWidth) > 0))
+                lossMinIdx = 2;
+            else if ((lossMinIdx == 0 && (histMin + stop * histBinWidth) < 0) ||
+                     (lossMinIdx == 2 && (histMin + (stop - 1) * histBinWidth) < 0))
+                lossMinIdx = 1;
+            if (lossMinIdx == 0)
+            {
+                start++;
+                stop--;
+            }
+            else if (lossMinIdx == 1)
+                start += 2;
+            else
+                stop -= 2;
+        }
+    }
+    *minOut = (float) thresholdMinOpt;
+    *maxOut = (float) thresholdMaxOpt;
+}
+
+/* computeEncoding, :97-146 */
+void orc_entropy_compute_encoding(const orc_tensor_profile* t, int bw, int sym, int strict, int unsignedSym,
+                                  orc_encoding* e)
+{
+    memset(e, 0, sizeof(*e));
+    float numSteps = (float) (pow(2, bw) - 1);
+    if (sym && strict)
+        numSteps -= 1;
+    if (!t->initialized)
+    {
+        if (t->stats_updated)
+        {
+            e->min    = -1;
+            e->max    = 1;
+            e->delta  = (e->max - e->min) / (int) numSteps;
+            e->offset = floor(e->min / e->delta);
+            e->min    = e->offset * e->delta;
+            e->max    = e->min + (int) numSteps * e->delta;
+            e->bw     = bw;
+        }
+        return;
+    }
+    float aMin, aMax;
+    orc_entropy_optimize_kl(t, bw, sym, strict, unsignedSym, &aMin, &aMax, NULL, NULL);
+    aMin = STD_MIN(aMin, 0.0f);
+    aMax = STD_MAX(aMax, 0.0f);
+    orc_get_computed_encodings(bw, aMin, aMax, sym, strict, unsignedSym, e);
+}
+
+/* ------------------------------------------------------------------------------------------------------------
  * a7  v2 quantize-dequantize (TORCH/v2/quantization/affine/backends/torch_builtins.py:303-344), float32 internal
  * dtype.  scale/offset are per "channel" with channel = (i / numElementPerChannel) % numChannel, which covers the
  * per-tensor ([1]) and per-output-channel ([C,1,...]) broadcast shapes.  torch.round is half-to-even (rintf under

@@ -11,6 +11,7 @@
 //   TfEnhancedEncodingAnalyzer<float> ModelOptimizations/DlQuantization/src/TfEnhancedEncodingAnalyzer.cpp:68-397
 //   PercentileEncodingAnalyzer<float> ModelOptimizations/DlQuantization/src/PercentileEncodingAnalyzer.cpp:54-215
 //   MseEncodingAnalyzer<float>        ModelOptimizations/DlQuantization/src/MseEncodingAnalyzer.cpp:54-262
+//   EntropyEncodingAnalyzer<float>    ModelOptimizations/DlQuantization/src/EntropyEncodingAnalyzer.cpp:54-436
 //   getComputedEncodings              ModelOptimizations/DlQuantization/src/quantization_utils.cpp:58-143
 //   quantizeDequantizeBroadcastCpu    ModelOptimizations/DlQuantization/src/trim_functions.cpp:634-660
 
@@ -32,6 +33,7 @@
 #define private public
 #include "TfEnhancedEncodingAnalyzer.h"
 #include "MseEncodingAnalyzer.h"
+#include "EntropyEncodingAnalyzer.h"
 #undef private
 #include "TensorQuantizationSim.h"
 #include "PercentileEncodingAnalyzer.h"
@@ -279,5 +281,42 @@ float ref_mse_cost(void* h, int bw, const float* centers, const float* pdfAtCent
     for (int i = 0; i < n; ++i)
         centersPdf[(size_t) i] = {centers[i], pdfAtCenter[i]};
     return a->_computeMSECost((uint8_t) bw, centersPdf, candMin, candMax, sym != 0, strict != 0, unsignedSym != 0);
+}
+// ---- EntropyEncodingAnalyzer<float> --------------------------------------------------------------
+void* ref_entropy_create()
+{
+    return new EntropyEncodingAnalyzer<float>();
+}
+void ref_entropy_destroy(void* h)
+{
+    delete static_cast<EntropyEncodingAnalyzer<float>*>(h);
+}
+void ref_entropy_update(void* h, const float* data, int64_t n)
+{
+    static_cast<EntropyEncodingAnalyzer<float>*>(h)->updateStats(data, (size_t) n, COMP_MODE_CPU);
+}
+void ref_entropy_compute(void* h, int bw, int sym, int strict, int unsignedSym, double* out5)
+{
+    TfEncoding e = static_cast<EntropyEncodingAnalyzer<float>*>(h)->computeEncoding((uint8_t) bw, sym != 0,
+                                                                                    strict != 0, unsignedSym != 0);
+    putEncoding(e, out5);
+}
+// the rescaling histogram: returns the number of bins (0 before the first batch that is not all zeros)
+int ref_entropy_get_histogram(void* h, double* hist512, double* minMax2, int* iterations)
+{
+    auto* a    = static_cast<EntropyEncodingAnalyzer<float>*>(h);
+    auto& tpp  = a->_tensorProfilingParams;
+    minMax2[0] = tpp.min;
+    minMax2[1] = tpp.max;
+    *iterations = tpp.iterations;
+    for (size_t i = 0; i < tpp.histogram.size() && i < 512; ++i)
+        hist512[i] = tpp.histogram[i];
+    return (int) tpp.histogram.size();
+}
+// the range the window search settles on, before zero is gated in and the grid is formed
+void ref_entropy_optimize(void* h, int bw, int sym, int strict, int unsignedSym, float* bestMin, float* bestMax)
+{
+    auto* a                      = static_cast<EntropyEncodingAnalyzer<float>*>(h);
+    std::tie(*bestMin, *bestMax) = a->_optimizeKL((uint8_t) bw, sym != 0, strict != 0, unsignedSym != 0);
 }
 }   // extern "C"

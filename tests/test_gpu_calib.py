@@ -458,6 +458,101 @@ def test_mse_scheme_through_the_tensor_quantizer_object(oracle):
     assert valid and (encoding.min, encoding.max, encoding.delta, encoding.offset, encoding.bw) == want.astuple()
 
 
+# -------------------------------------------------------------------------------------------- entropy analyzer
+ENTROPY = 4
+
+
+def _entropy_cases(rng):
+    return {
+        "normal": [(rng.standard_normal(30000) * (1 + b) + 0.5).astype(np.float32) for b in range(3)],
+        "relu-pareto": [_relu_pareto(20 + b, 50000) for b in range(2)],
+        "negative": [(-np.abs(rng.standard_normal(10000)) - 0.25).astype(np.float32)],
+        "constant": [np.full(6000, 4, np.float32)],
+        "zeros": [np.zeros(6000, np.float32)],
+        "zeros-then-data": [np.zeros(100, np.float32), rng.standard_normal(9999).astype(np.float32)],
+        "far-from-zero": [(rng.standard_normal(20000) * 0.01 + 50).astype(np.float32)],
+        # every batch widens the range -- to the right, to the left, on both sides -- then one falls inside it
+        "growing-range": [(rng.standard_normal(5003) * s + m).astype(np.float32)
+                          for s, m in ((0.5, 0.0), (1.0, 2.0), (1.0, -3.0), (4.0, 0.0), (0.1, 0.0))],
+        "large": [rng.standard_normal(3_000_001).astype(np.float32)],
+    }
+
+
+@pytest.mark.parametrize("kind", ["normal", "relu-pareto", "negative", "constant", "zeros", "zeros-then-data",
+                                  "far-from-zero", "growing-range", "large"])
+def test_entropy_analyzer_matches_the_oracle(ops, oracle, kind):
+    """EntropyEncodingAnalyzer<float>: after every batch the histogram -- its range, each of the 512 counts, the
+    number of batches counted -- is the reference's, and so is every field of the encoding for each symmetry mode
+    (the KL window search runs for 8 bits; other bitwidths keep the histogram's range)."""
+    batches = _entropy_cases(np.random.default_rng(len(kind) + 7))[kind]
+    an, prof = ops.Analyzer(ENTROPY), oracle.new_profile()
+    for b in batches:
+        an.update_stats(_gpu(b))
+        prof.update(b)
+        counts, span, seen, batches_counted = an.entropy_histogram()
+        assert seen == prof.initialized and batches_counted == prof.iterations
+        if seen:
+            assert span == prof.range()
+            assert np.array_equal(counts, prof.histogram())
+    for bw, sym, strict, uns in ((8, 0, 0, 0), (8, 1, 0, 0), (8, 1, 1, 0), (8, 1, 0, 1), (4, 0, 0, 0), (16, 1, 0, 0)):
+        e, valid = an.compute_encoding(bw, sym, strict, uns)
+        want = prof.compute_encoding(bw, sym, strict, uns)
+        assert valid and (e.min, e.max, e.delta, e.offset, e.bw) == want.astuple(), (kind, bw, sym, strict, uns)
+
+
+def test_entropy_analyzer_on_views_and_unaligned_tensors(ops, oracle):
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal(40003).astype(np.float32)
+    an, prof = ops.Analyzer(ENTROPY), oracle.new_profile()
+    an.update_stats(_gpu(x)[1:])                                                  # not 16-byte aligned
+    prof.update(x[1:])
+    an.update_stats(_gpu(x)[:7])                                                  # fewer samples than one vector pass
+    prof.update(x[:7])
+    counts, span, _, _ = an.entropy_histogram()
+    assert span == prof.range() and np.array_equal(counts, prof.histogram())
+
+
+def test_entropy_analyzer_edge_behaviour(ops):
+    from aimet_amd._lib import MiqError
+    an = ops.Analyzer(ENTROPY)
+    e, valid = an.compute_encoding(8)
+    assert not valid and (e.min, e.max, e.delta, e.offset) == (0, 0, 0, 0)        # nothing seen
+    torch.manual_seed(0)
+    x = torch.cat([torch.randn(200000, device="cuda"), torch.tensor([14.0, -11.0], device="cuda")])
+    an.update_stats(x)
+    counts, span, seen, batches_counted = an.entropy_histogram()
+    assert seen and batches_counted == 1 and counts.sum() == x.numel() and span == (-11.0, 14.0)
+    e8, _ = an.compute_encoding(8)
+    assert -11 < e8.min < 0 < e8.max < 14                                         # the two outliers are cut off
+    e4, _ = an.compute_encoding(4)
+    assert e4.min <= -11 and e4.max >= 14 - e4.delta                              # no search below or above 8 bits
+    with pytest.raises(MiqError):
+        an.get_stats_histogram()                                                  # counts, not a PDF
+    with pytest.raises(MiqError):
+        ops.Analyzer(1).entropy_histogram()
+    an.reset()
+    assert not an.compute_encoding(8)[1]
+    an.update_stats(torch.zeros(100, device="cuda"))
+    e, valid = an.compute_encoding(8)
+    assert valid and e.offset == -128 and abs(e.min + 1.00392) < 1e-4             # only zeros: the range of [-1, 1]
+
+
+def test_entropy_scheme_through_the_tensor_quantizer_object(oracle):
+    """libpymo's QuantizationMode.QUANTIZATION_ENTROPY through the AimetTensorQuantizer object
+    (TrainingExtensions/torch/src/AimetTensorQuantizer.cpp:74-126 over DLQ/src/QuantizerFactory.cpp:89-92)."""
+    from aimet_amd.common import libpymo
+    from aimet_amd.common.AimetTensorQuantizer import AimetTensorQuantizer
+    rng = np.random.default_rng(9)
+    x = (rng.standard_normal(40000) * 2 - 1).astype(np.float32)
+    q = AimetTensorQuantizer(libpymo.QuantizationMode.QUANTIZATION_ENTROPY)
+    q.updateStats(_gpu(x), True)
+    encoding, valid = q.getEncoding(8, False, False, False)
+    prof = oracle.new_profile()
+    prof.update(x)
+    want = prof.compute_encoding(8)
+    assert valid and (encoding.min, encoding.max, encoding.delta, encoding.offset, encoding.bw) == want.astuple()
+
+
 def test_percentile_scheme_through_the_v1_quantizers():
     """test_tensor_quantizer / quantsim flow of the reference with quant_scheme = post_training_percentile."""
     from aimet_amd.common import libpymo

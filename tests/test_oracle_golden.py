@@ -500,3 +500,97 @@ def test_mse_search_against_brute_force(oracle):
     assert costs[i, j] == pytest.approx(cost(float(best_min), float(best_max)), rel=1e-4)
     assert best_min < 0 < best_max and best_max < x.max() and best_min > x.min()      # outliers are clipped
     assert len(mins) + len(maxs) >= 100 and mins[-1] == 0 and maxs[-1] == 0
+
+
+def test_entropy_cases_of_the_reference_unit_tests(oracle):
+    """ModelOptimizations/DlQuantization/test/TestEntropyEncodingAnalyzer.cpp:56-314: the assertions of its cases on
+    data of the same distributions."""
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal(100000) * 2 + 2).astype(np.float32)
+    top = np.abs(x).max()
+    prof = oracle.new_profile()
+    prof.update(x)
+    e = prof.compute_encoding(8)                                          # Asymmetric, :56-109
+    assert 2 - 12 < e.min < 2 - 4 and 2 + 4 < e.max < 2 + 12
+    e = prof.compute_encoding(8, sym=True)                                # Symmetric, :111-158
+    assert e.min > -top and e.max < top and e.offset == -128 and e.bw == 8
+    assert e.delta == pytest.approx((e.max - e.min) / 255, rel=1e-6)
+    assert e.offset == pytest.approx(e.min / e.delta, rel=1e-6)
+    e = prof.compute_encoding(8, sym=True, strict=True)                   # StrictSymmetric, :160-208
+    assert e.min > -top and e.max < top and e.offset == -127 and e.min == -e.max
+    assert e.delta == pytest.approx((e.max - e.min) / 254, rel=1e-6)
+    pos = np.maximum(x, 0)
+    prof = oracle.new_profile()
+    prof.update(pos)
+    e = prof.compute_encoding(8, sym=True, unsigned_sym=True)             # SymmetricUnsigned, :210-257
+    assert e.min == 0 and e.max <= top and e.offset == 0 and e.bw == 8
+    assert e.delta == pytest.approx((e.max - e.min) / 255, rel=1e-6)
+    prof = oracle.new_profile()                                           # AllSameValuesAsymmetric, :259-292
+    prof.update(np.full(100, 4, np.float32))
+    e = prof.compute_encoding(8)
+    assert e.min <= 0 and e.max >= 3.9
+    prof = oracle.new_profile()
+    prof.update(np.full(100, -5, np.float32))
+    e = prof.compute_encoding(8)
+    assert e.min <= -4.99992 and e.max >= 0
+    prof = oracle.new_profile()                                           # AllZeroesAsymmetric, :294-314
+    prof.update(np.zeros(6000, np.float32))
+    e = prof.compute_encoding(8)
+    assert e.min == pytest.approx(-1.00392, abs=1e-4) and e.max == pytest.approx(0.996078, abs=1e-4)
+    assert e.offset == -128 and e.bw == 8
+
+
+def test_entropy_histogram_invariants(oracle):
+    """What the arithmetic fixes about the rescaling histogram: it spans exactly the range seen, every sample is
+    counted once (redistribution moves whole counts: the total is the number of samples, exactly), a batch inside
+    the range leaves the range alone, and the bins agree with numpy's histogram away from bin edges."""
+    rng = np.random.default_rng(4)
+    prof = oracle.new_profile()
+    total, lo, hi = 0, np.inf, -np.inf
+    for scale, shift in ((1.0, 0.0), (0.2, 0.1), (3.0, -1.0), (1.0, 9.0)):
+        x = (rng.standard_normal(20000) * scale + shift).astype(np.float32)
+        prof.update(x)
+        total += x.size
+        lo, hi = min(lo, float(x.min())), max(hi, float(x.max()))
+        assert prof.range() == (lo, hi)
+        hist = prof.histogram()
+        assert hist.sum() == total and np.all(hist == np.round(hist)) and hist.min() >= 0
+    prof = oracle.new_profile()
+    x = rng.standard_normal(100000).astype(np.float32)
+    prof.update(x)
+    want, _ = np.histogram(x.astype(np.float64), bins=512, range=(float(x.min()), float(x.max())))
+    # float32 bin arithmetic against float64: a sample within rounding of an edge may land next door
+    assert np.abs(prof.histogram() - want).sum() <= 20 and prof.histogram().sum() == want.sum()
+
+
+def test_entropy_search_against_a_direct_kl(oracle):
+    """The divergence of the first window (the whole histogram, nothing saturated) against the KL divergence written
+    here from its definition in numpy: P = the histogram, Q = 255 merged levels spread back over their non-empty
+    bins, both smoothed by moving 1e-4 per empty bin from the non-empty ones, KL(P || Q) of the normalised two."""
+    rng = np.random.default_rng(8)
+    x = np.concatenate([rng.standard_normal(200000), [14.0, -11.0]]).astype(np.float32)
+    prof = oracle.new_profile()
+    prof.update(x)
+    lo, hi, divergences = prof.optimize_kl(8)
+    hist = prof.histogram()
+    edges = np.ceil(np.arange(256) * (512 / 255)).astype(int)
+    edges[-1] = 512
+    q = np.zeros(512)
+    for a, b in zip(edges[:-1], edges[1:]):
+        nz = hist[a:b] != 0
+        if nz.any():
+            q[a:b][nz] = hist[a:b].sum() / nz.sum()
+
+    def smooth(h):
+        zeros = h == 0
+        eps = 1e-4 * zeros.sum() / (~zeros).sum()
+        return np.where(zeros, 1e-4, h - eps)
+    p, q = smooth(hist.copy()), smooth(q)
+    p, q = p / p.sum(), q / q.sum()
+    assert divergences[0] == pytest.approx(float(np.sum(p * np.log(p / q))), rel=1e-5)
+    assert len(divergences) == 129                                        # 512, 510, ... 256 bins
+    # the winner is the window of least divergence, and it cuts the two far outliers off
+    assert -11 < lo < 0 < hi < 14
+    best = int(np.argmin(divergences))
+    width = (float(x.max()) - float(x.min())) / 512
+    assert hi - lo == pytest.approx((512 - 2 * best) * width, rel=1e-5)

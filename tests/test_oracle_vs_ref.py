@@ -286,3 +286,50 @@ def test_mse_analyzer_without_usable_statistics(oracle, ref):
     an.update(z)
     for bw, sym, strict in ((8, False, False), (8, True, True), (4, False, False)):
         assert pdf.compute_mse_encoding(bw, sym, strict).astuple() == an.compute_encoding(bw, sym, strict)
+
+
+_ENTROPY_KINDS = ["normal", "relu", "negative", "outliers", "constant", "zeros-then-data", "far-from-zero",
+                  "growing-range", "one-batch"]
+
+
+def _entropy_batches(rng, kind):
+    if kind == "growing-range":
+        # every batch widens the range, to the left, to the right, on both sides: the histogram is redistributed
+        return [(rng.standard_normal(5000) * s + m).astype(np.float32)
+                for s, m in ((0.5, 0.0), (1.0, 2.0), (1.0, -3.0), (4.0, 0.0), (0.1, 0.0))]
+    if kind == "one-batch":
+        return [rng.standard_normal(50000).astype(np.float32)]
+    return _mse_batches(rng, kind)
+
+
+@pytest.mark.parametrize("kind", _ENTROPY_KINDS)
+def test_entropy_analyzer(oracle, ref, kind):
+    """EntropyEncodingAnalyzer<float>: the histogram after every batch (range, every bin, batch count), the range the
+    KL window search returns, every field of the encoding."""
+    rng = np.random.default_rng(len(kind) + 100)
+    prof, an = oracle.new_profile(), ref.new_entropy()
+    for x in _entropy_batches(rng, kind):
+        prof.update(x)
+        an.update(x)
+        n, hist, rng_ref, it = an.histogram()
+        assert prof.initialized == (n == 512) and prof.iterations == it
+        if n:
+            assert prof.range() == rng_ref
+            assert np.array_equal(prof.histogram(), hist)
+    for bw in (8, 4, 16):
+        for sym, strict, uns in ((False, False, False), (True, False, False), (True, True, False), (True, False, True)):
+            lo, hi, _ = prof.optimize_kl(bw, sym, strict, uns)
+            assert (lo, hi) == an.optimize(bw, sym, strict, uns), (kind, bw, sym, strict, uns)
+            got = prof.compute_encoding(bw, sym, strict, uns)
+            assert got.astuple() == an.compute_encoding(bw, sym, strict, uns), (kind, bw, sym, strict, uns)
+
+
+def test_entropy_analyzer_without_usable_statistics(oracle, ref):
+    prof, an = oracle.new_profile(), ref.new_entropy()
+    assert prof.compute_encoding(8).astuple() == an.compute_encoding(8)                      # nothing seen: zeros
+    z = np.zeros(100, np.float32)
+    prof.update(z)
+    an.update(z)
+    assert prof.iterations == an.histogram()[3] == 0                                          # the batch is not counted
+    for bw, sym, strict in ((8, False, False), (8, True, True), (4, False, False)):
+        assert prof.compute_encoding(bw, sym, strict).astuple() == an.compute_encoding(bw, sym, strict)
