@@ -213,15 +213,19 @@ __global__ __launch_bounds__(kBins) void ent_range_kernel(EntState* st, int grou
     }
 }
 
+// Activations pile up in a few bins (after a ReLU, half of them in one): eight copies of the counters in LDS, picked by
+// lane, keep lanes of one wavefront from queueing on one address.
+constexpr int kEntCopies = 8;
 __global__ __launch_bounds__(kEntBlock) void ent_bin_kernel(const float* __restrict__ data, int64_t n, EntState* st,
                                                              int vec)
 {
     if (st->skip)
         return;
-    __shared__ unsigned int s_hist[kBins];
-    for (int k = threadIdx.x; k < kBins; k += kEntBlock)
-        s_hist[k] = 0;
+    __shared__ unsigned int s_hist[kEntCopies][kBins];
+    for (int k = threadIdx.x; k < kEntCopies * kBins; k += kEntBlock)
+        (&s_hist[0][0])[k] = 0;
     __syncthreads();
+    unsigned int* mine = s_hist[threadIdx.x & (kEntCopies - 1)];
     const float width = st->bin_width_f, low = st->min_f;
     const int64_t stride = (int64_t) gridDim.x * blockDim.x;
     const int64_t first  = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
@@ -233,19 +237,25 @@ __global__ __launch_bounds__(kEntBlock) void ent_bin_kernel(const float* __restr
         for (int64_t k = first; k < n4; k += stride)
         {
             const v4f v = __builtin_nontemporal_load(d4 + k);
-            atomicAdd(&s_hist[get_bin(width, low, v.x)], 1u);
-            atomicAdd(&s_hist[get_bin(width, low, v.y)], 1u);
-            atomicAdd(&s_hist[get_bin(width, low, v.z)], 1u);
-            atomicAdd(&s_hist[get_bin(width, low, v.w)], 1u);
+            atomicAdd(&mine[get_bin(width, low, v.x)], 1u);
+            atomicAdd(&mine[get_bin(width, low, v.y)], 1u);
+            atomicAdd(&mine[get_bin(width, low, v.z)], 1u);
+            atomicAdd(&mine[get_bin(width, low, v.w)], 1u);
         }
         done = n4 * 4;
     }
     for (int64_t k = done + first; k < n; k += stride)
-        atomicAdd(&s_hist[get_bin(width, low, data[k])], 1u);
+        atomicAdd(&mine[get_bin(width, low, data[k])], 1u);
     __syncthreads();
     for (int k = threadIdx.x; k < kBins; k += kEntBlock)
-        if (s_hist[k])
-            atomicAdd(&st->hist[k], (unsigned long long) s_hist[k]);
+    {
+        unsigned int sum = 0;
+#pragma unroll
+        for (int c = 0; c < kEntCopies; ++c)
+            sum += s_hist[c][k];
+        if (sum)
+            atomicAdd(&st->hist[k], (unsigned long long) sum);
+    }
 }
 
 __global__ void ent_reset_kernel(EntState* st)

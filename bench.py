@@ -346,8 +346,30 @@ def bench_calibration(torch, ops, reps):
             other_searches[f"{name}_bw{bw}"] = {"compute_encoding_us": (time.perf_counter() - t0) / 10 * 1e6,
                                                 "encoding": [e.min, e.max, e.delta, e.offset]}
         del other
+    # the entropy analyzer keeps a histogram of another kind (it follows the range of the data): two streaming passes
+    # and one small launch per batch, the KL window search on the host
+    ent = ops.Analyzer(4, dev)
+    for x in batches[:2]:
+        ent.update_stats(x)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for x in batches:
+        ent.update_stats(x)
+    e1.record()
+    torch.cuda.synchronize()
+    ent_update_ms = e0.elapsed_time(e1) / len(batches)
+    ent.compute_encoding(8)
+    t0 = time.perf_counter()
+    for _ in range(10):
+        e, _ = ent.compute_encoding(8)
+    entropy = {"update_us": ent_update_ms * 1e3, "update_GBps_of_one_read": 4 * n / ent_update_ms / 1e6,
+               "compute_encoding_us": (time.perf_counter() - t0) / 10 * 1e6,
+               "encoding": [e.min, e.max, e.delta, e.offset]}
+    del ent
     return {"elements": elems, "accumulate_ms": acc, "search_ms_wall": sum(search_ms) / len(search_ms),
             "update_by_batch_size": by_size, "other_searches_on_the_same_pdf": other_searches,
+            "entropy_analyzer": entropy,
             "total_ms_wall": tot, "elements_per_s": elems / (tot / 1e3),
             "accumulate_GBps": 17 * 4 * n / acc / 1e6, "accumulate_frac_hbm": 17 * 4 * n / acc / 1e6 / HBM_PEAK_GBPS,
             "encoding": [enc.min, enc.max, enc.delta, enc.offset]}
