@@ -7,6 +7,7 @@ Graph questions are answered with forward hooks on one pass of the model instead
 ConnectedGraph.
 """
 import contextlib
+import inspect
 from typing import Any, Callable, Dict, List, Tuple, Union
 
 import torch
@@ -147,6 +148,59 @@ class CachedDataset:
 
     def __iter__(self):
         return iter(self._batches)
+
+
+def add_foward_fn_kwargs_to_inputs(module: nn.Module, *args, **kwargs) -> Tuple:
+    """A call `module(*args, **kwargs)` as positional arguments only: the parameters of `module.forward` that `args`
+    does not reach take their keyword value, or else their default (reference aimet_torch/utils.py:1041-1061; the
+    misspelt name is the reference's)."""
+    parameters = [p for p in inspect.signature(module.forward).parameters.values()
+                  if p.name != 'self' and p.kind in (p.POSITIONAL_ONLY, p.POSITIONAL_OR_KEYWORD, p.KEYWORD_ONLY)]
+    extra = []
+    for parameter in parameters[len(args):]:
+        if parameter.name in kwargs:
+            extra.append(kwargs[parameter.name])
+        elif parameter.default is not inspect.Parameter.empty:
+            extra.append(parameter.default)
+    return (*args, *extra)
+
+
+def cache_intermediate_datasets(cached_dataset, cache_on_cpu: bool, model: nn.Module, module_name: str,
+                                forward_fn: Callable, path: str = None, incl_kwargs: bool = False) -> List[List]:
+    """What the module called `module_name` receives for every batch of `cached_dataset`: one list of its positional
+    inputs per batch (its keyword inputs laid behind them when `incl_kwargs`).  Each forward pass stops at that module.
+
+    The reference (aimet_torch/utils.py:1064-1105) keeps these lists in host memory when `cache_on_cpu`, and otherwise
+    pickles each to `path` and reads it back on every access.  Here `cache_on_cpu` decides between host memory and the
+    device the model runs on -- one GPU's 288 GB hold the block inputs of models that do not fit a host's page cache --
+    and `path` is accepted and ignored."""
+    # pylint: disable=too-many-arguments
+    del path
+    module = get_named_module(model, module_name)
+    forward_fn = forward_fn or _default_forward
+    cached = []
+
+    def keep_inputs_and_stop(_module, args, kwargs):
+        if incl_kwargs and kwargs:
+            args = add_foward_fn_kwargs_to_inputs(module, *args, **kwargs)
+        inputs = [*args]
+        cached.append(change_tensor_device_placement(inputs, torch.device('cpu')) if cache_on_cpu else inputs)
+        raise StopForwardException
+
+    handle = module.register_forward_pre_hook(keep_inputs_and_stop, with_kwargs=True)
+    try:
+        for batch in cached_dataset:
+            try:
+                with in_eval_mode(model), torch.no_grad():
+                    forward_fn(model, batch)
+            except StopForwardException:
+                pass
+    finally:
+        handle.remove()
+    if len(cached) != len(cached_dataset):
+        raise RuntimeError(f"module '{module_name}' was reached by {len(cached)} of {len(cached_dataset)} forward "
+                           "passes: a checkpoint has to lie on the path of every batch, once")
+    return cached
 
 
 class ModuleData:

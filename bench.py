@@ -1060,6 +1060,41 @@ def bench_end_to_end(torch, ops):
                                 default_param_bw=4)
         torch.cuda.synchronize()
         conv_total = time.perf_counter() - t0
+    # a deep chain through apply_adaround and through apply_adaround_with_cache (groups of four layers whose inputs are
+    # kept on the device): sampling a layer's activations costs a pass through every layer before it in the first
+    # and a pass through its own group in the second
+    depth, dwidth, deep_iters = 48, 1024, 50
+    torch.manual_seed(1005)
+    chain = []
+    for k in range(depth):
+        chain += [torch.nn.Linear(dwidth, dwidth), torch.nn.ReLU()]
+    deep = torch.nn.Sequential(*chain[:-1]).eval().to(dev)
+    dloader = [(torch.randn(256, dwidth, device=dev), torch.zeros(256)) for _ in range(4)]
+    unpack = lambda m, b: m(b[0]) if isinstance(b, (list, tuple)) else m(b)
+    names = [str(i) for i in range(len(deep))]
+    groups = {str(g): names[g * 8:(g + 1) * 8] for g in range((len(names) + 7) // 8)}
+    with tempfile.TemporaryDirectory() as tmp:
+        cfg = os.path.join(tmp, "checkpoints.json")
+        with open(cfg, "w") as f:
+            json.dump({"grouped_modules": groups, "include_static_inputs": ["False"] * len(groups),
+                        "cache_on_cpu": "False"}, f)
+        deep_s = {}
+        for label, call in (("apply_adaround_s", lambda it, pre: Adaround.apply_adaround(
+                                 deep, dloader[0][0][:2], AdaroundParameters(dloader, 4, it, forward_fn=unpack), tmp, pre,
+                                 default_param_bw=4)),
+                            ("apply_adaround_with_cache_s", lambda it, pre: Adaround.apply_adaround_with_cache(
+                                 deep, dloader[0][0][:2], AdaroundParameters(dloader, 4, it, forward_fn=unpack), tmp, pre,
+                                 default_param_bw=4, checkpoints_config=cfg))):
+            call(2, "warm")
+            gc.collect()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            call(deep_iters, "bench")
+            torch.cuda.synchronize()
+            deep_s[label] = time.perf_counter() - t0
+    out["apply_adaround_48x_linear_1024_whole_model_passes_against_kept_group_inputs"] = {
+        "layers": depth, "layer": [dwidth, dwidth], "samples": 1024, "iterations_per_layer": deep_iters,
+        "groups": len(groups), **deep_s}
     out["apply_adaround_6_convolutions"] = {
         "layers": 6, "input": [64, 3, 32, 32], "batches": 4, "iterations_per_layer": conv_iters, "bitwidth": 4,
         "apply_adaround_s": conv_total, "s_per_layer": conv_total / 6,
