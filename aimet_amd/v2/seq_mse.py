@@ -1,0 +1,213 @@
+"""Sequential MSE on the v2 quantized modules.
+
+Mirrors TrainingExtensions/torch/src/python/aimet_torch/v2/seq_mse.py: SequentialMse with the v2 overrides
+(apply_seq_mse :68-99, _get_grouped_convs_with_blockwise_quantization :101-118, _handle_grouped_block_quantizers
+:120-137, compute_all_param_encodings :139-148, temporarily_disable_quantizers :150-196, compute_param_encodings
+:198-216, get_min_and_max_for_candidate_selection :263-312, _get_candidate :314-323, _compute_loss :325-357,
+optimize_module :359-395).  Candidates are tensors of the weight quantizer's shape (per tensor, per channel) or of the
+weight's shape (blockwise: every element carries its block's extreme), the loss is kept per output channel and per
+block of input channels, and the winner is chosen per block.  The walk over the model, the sampling of layer inputs and
+the checkpointed flow are those of the v1 path.
+"""
+import contextlib
+from typing import List, Optional, Tuple
+
+import torch
+from torch import nn
+
+from ..v1.seq_mse import SUPPORTED_MODULES, SeqMseParams, SequentialMse as V1SequentialMse, default_forward_fn  # noqa: F401
+from .nn import BaseQuantizationMixin
+from .quantization.affine import GroupedBlockQuantizeDequantize, QuantizeDequantize
+from .quantsim import QuantizationSimModel
+from .utils import reshape_tensor_for_blocks
+
+
+def _reduced_to(tensor: torch.Tensor, shape, extreme) -> torch.Tensor:
+    """`tensor` reduced by `extreme` (torch.amax / torch.amin) over every axis along which `shape`, aligned from the
+    right, has one entry; the result has exactly `shape`."""
+    shape = tuple(shape)
+    aligned = (1,) * (tensor.dim() - len(shape)) + shape
+    axes = [axis for axis, (have, want) in enumerate(zip(tensor.shape, aligned)) if want == 1 and have != 1]
+    return (extreme(tensor, dim=axes, keepdim=True) if axes else tensor).reshape(shape)
+
+
+class SequentialMse(V1SequentialMse):
+    """Weight encodings of the v2 simulation model by minimizing each layer's output error, layer after layer."""
+
+    @classmethod
+    def apply_seq_mse(cls, model: nn.Module, sim: QuantizationSimModel, data_loader, params: SeqMseParams,
+                      modules_to_exclude: Optional[List[nn.Module]] = None, checkpoints_config: Optional[str] = None):
+        # pylint: disable=too-many-arguments
+        # grouped convolutions whose blocks cut through a group's input channels cannot be searched block by block
+        modules_to_exclude = list(modules_to_exclude or []) + cls._get_grouped_convs_with_blockwise_quantization(sim)
+        with cls._handle_grouped_block_quantizers(sim):
+            super().apply_seq_mse(model, sim, data_loader, params, modules_to_exclude, checkpoints_config)
+
+    @staticmethod
+    def _get_grouped_convs_with_blockwise_quantization(sim) -> List[nn.Module]:
+        found = []
+        for module in sim.model.modules():
+            if isinstance(module, nn.Conv2d) and isinstance(module, BaseQuantizationMixin) and module.groups != 1:
+                quantizer = module.param_quantizers['weight']
+                block_size = getattr(quantizer, 'block_size', None)
+                if block_size is not None and block_size[1] != module.weight.shape[1]:
+                    found.append(module)
+        return found
+
+    @staticmethod
+    @contextlib.contextmanager
+    def _handle_grouped_block_quantizers(sim: QuantizationSimModel):
+        """Inside the `with`, grouped blockwise quantizers behave as plain blockwise ones (every block its own group):
+        the search picks a range per block."""
+        grouped = [(q, q.block_grouping) for q in sim.model.modules() if isinstance(q, GroupedBlockQuantizeDequantize)]
+        for quantizer, _ in grouped:
+            quantizer.block_grouping = tuple(1 for _ in quantizer.shape)
+        try:
+            yield
+        finally:
+            for quantizer, grouping in grouped:
+                quantizer.block_grouping = grouping
+
+    @staticmethod
+    def compute_all_param_encodings(sim: QuantizationSimModel):
+        for _, qmodule in sim.named_qmodules():
+            qmodule._compute_param_encodings(overwrite=True)       # pylint: disable=protected-access
+
+    @staticmethod
+    @contextlib.contextmanager
+    def temporarily_disable_quantizers(model: nn.Module, sim: QuantizationSimModel, modules_to_exclude):
+        """Inside the `with`, activation quantizers are out of every quantized module, and so are the parameter
+        quantizers of unsupported module types and of the excluded modules (given as modules of `model`, or of the
+        simulation model)."""
+        # pylint: disable=protected-access, arguments-differ
+        float_modules = dict(model.named_modules())
+        excluded = modules_to_exclude or []
+        put_back = []
+        try:
+            for name, qmodule in sim.named_qmodules():
+                put_back.append(qmodule._remove_activation_quantizers())
+                skipped = any(other is qmodule or other is float_modules.get(name) for other in excluded)
+                if skipped or not isinstance(qmodule, SUPPORTED_MODULES):
+                    put_back.append(qmodule._remove_param_quantizers())
+            yield
+        finally:
+            for undo in reversed(put_back):
+                undo._cleanup()
+
+    @staticmethod
+    def _weight_bitwidth(quant_module) -> int:
+        quantizer = quant_module.param_quantizers['weight']
+        return quantizer.bitwidth if quantizer is not None else 1 << 30    # not quantized: never searched
+
+    @staticmethod
+    def compute_param_encodings(quantizer, x_min: torch.Tensor, x_max: torch.Tensor):
+        """min / max of `quantizer` as a fresh min-max quantizer of its geometry sets them on observing x_min, x_max."""
+        observer = QuantizeDequantize(quantizer.shape, quantizer.bitwidth, quantizer.symmetric,
+                                      block_size=quantizer.block_size).to(x_min.device)
+        with observer.compute_encodings():
+            observer(torch.stack([x_min, x_max]))
+        with torch.no_grad():
+            quantizer.min.copy_(observer.min)
+            quantizer.max.copy_(observer.max)
+
+    @staticmethod
+    def _is_symmetric_quantizer(quantizer) -> bool:
+        return quantizer.symmetric
+
+    @staticmethod
+    def _freeze_quantizer_encoding(quantizer):
+        quantizer.requires_grad_(False)
+        quantizer.allow_overwrite(False)
+
+    @staticmethod
+    def _get_quantized_weight(quant_module: BaseQuantizationMixin) -> torch.Tensor:
+        return quant_module.param_quantizers['weight'](quant_module.weight)
+
+    @staticmethod
+    def _get_original_module(quant_module: BaseQuantizationMixin) -> nn.Module:
+        return quant_module                                          # a v2 quantized module is the module
+
+    @staticmethod
+    def _get_input_channel_block_size(quant_module) -> int:
+        if not isinstance(quant_module, (nn.Linear, nn.Conv2d)):
+            raise NotImplementedError('Unsupported module type: ', type(quant_module))
+        quantizer = quant_module.param_quantizers['weight']
+        if quantizer.block_size is None:
+            return quant_module.weight.shape[1]
+        return quant_module.weight.shape[1] // quantizer.shape[1]
+
+    @classmethod
+    def get_min_and_max_for_candidate_selection(cls, quant_module: BaseQuantizationMixin) \
+            -> Tuple[torch.Tensor, torch.Tensor]:
+        """The extremes the candidates are fractions of: of the quantizer's shape without blocks; with blocks, of the
+        weight's shape, every element holding the extreme of its block."""
+        if not isinstance(quant_module, (nn.Conv2d, nn.Linear)):
+            raise ValueError('Unsupported module: ', quant_module)
+        quantizer = quant_module.param_quantizers['weight']
+        weight = quant_module.weight.detach()
+        symmetric = cls._is_symmetric_quantizer(quantizer)
+        if quantizer.block_size is None:
+            if symmetric:
+                top = _reduced_to(weight.abs(), quantizer.shape, torch.amax)
+                return -top, top
+            return _reduced_to(weight, quantizer.shape, torch.amin), _reduced_to(weight, quantizer.shape, torch.amax)
+        in_blocks = reshape_tensor_for_blocks(weight, quantizer.shape, quantizer.block_size)
+        # reshaped as (blocks, block size) pairs per axis: the block-size axes are every second one, from the last
+        within = [in_blocks.dim() - 1 - 2 * k for k in range(len(quantizer.block_size))][::-1]
+        if symmetric:
+            top = torch.maximum(in_blocks, torch.amax(in_blocks.abs(), within, keepdim=True)).reshape(weight.shape)
+            return -top, top
+        top = torch.maximum(in_blocks, torch.amax(in_blocks, within, keepdim=True)).reshape(weight.shape)
+        bottom = torch.minimum(in_blocks, torch.amin(in_blocks, within, keepdim=True)).reshape(weight.shape)
+        return bottom, top
+
+    @staticmethod
+    def _get_candidate(candidate_idx, num_candidates: int, min_tensor: torch.Tensor, max_tensor: torch.Tensor):
+        """Fraction (candidate_idx + 1) / num_candidates of the range; the index may be a tensor (one per block)."""
+        return min_tensor / num_candidates * (candidate_idx + 1), max_tensor / num_candidates * (candidate_idx + 1)
+
+    @classmethod
+    def _compute_loss(cls, quant_module, x, xq, w, wq, params) -> torch.Tensor:
+        """[output channels, blocks of input channels]: the loss of each block's partial product on its own."""
+        # pylint: disable=too-many-arguments
+        block = cls._get_input_channel_block_size(quant_module)
+        channel_axis = -1 if isinstance(quant_module, nn.Linear) else -3
+        losses = []
+        for w_part, wq_part, x_part, xq_part in zip(torch.split(w, block, dim=1), torch.split(wq, block, dim=1),
+                                                    torch.split(x, block, dim=channel_axis),
+                                                    torch.split(xq, block, dim=channel_axis)):
+            xqwq, xw = cls.compute_outputs(quant_module, x_part, xq_part, w_part, wq_part)
+            losses.append(cls.compute_recon_loss(xqwq, xw, params))
+        return torch.stack(losses, dim=-1)
+
+    @classmethod
+    def optimize_module(cls, quant_module: BaseQuantizationMixin, x: torch.Tensor, xq: torch.Tensor,
+                        params: SeqMseParams):
+        quantizer = quant_module.param_quantizers['weight']
+        min_tensor, max_tensor = cls.get_min_and_max_for_candidate_selection(quant_module)
+        total_loss = []
+        for index in range(params.num_candidates):
+            cand_min, cand_max = cls._get_candidate(index, params.num_candidates, min_tensor, max_tensor)
+            cls.compute_param_encodings(quantizer, cand_min, cand_max)
+            w = quant_module.weight
+            with torch.no_grad():
+                wq = cls._get_quantized_weight(quant_module)
+                loss = cls._compute_loss(quant_module, x[0], xq[0], w, wq, params)
+                for b in range(1, params.num_batches):
+                    loss += cls._compute_loss(quant_module, x[b], xq[b], w, wq, params)
+            total_loss.append(loss)
+        best = torch.stack(total_loss).min(0)[1]                     # [output channels, blocks]
+        block = cls._get_input_channel_block_size(quant_module)
+        if block != quant_module.weight.shape[1]:
+            best = best.repeat_interleave(block, dim=-1)             # one index per input channel
+        while best.dim() < max_tensor.dim():
+            best = best[..., None]
+        best_min, best_max = cls._get_candidate(best, params.num_candidates, min_tensor, max_tensor)
+        cls.compute_param_encodings(quantizer, best_min, best_max)
+        cls._freeze_quantizer_encoding(quantizer)
+
+
+# module-level names, as the reference offers them
+apply_seq_mse = SequentialMse.apply_seq_mse
+get_candidates = SequentialMse.get_candidates
+optimize_module = SequentialMse.optimize_module
