@@ -1112,7 +1112,7 @@ __global__ __launch_bounds__(64) void mse_pick_kernel(DevState* st, const MseScr
     st->enc_min = e.min, st->enc_max = e.max, st->enc_delta = e.delta, st->enc_offset = e.offset;
     st->enc_bw     = a.bw;
     st->best_index = (index == INT_MAX) ? -1 : index;
-    st->n_cand     = m->n_min * m->n_max - 1;
+    st->n_cand     = 0;   // the candidate arrays of the state belong to the TF-Enhanced search and stay empty
 }
 
 __global__ void reset_state_kernel(DevState* st)
@@ -1824,9 +1824,9 @@ int miq_analyzer_last_search(miq_analyzer* a, float* deltas, int32_t* offsets, d
                              int* best_index, void* stream)
 {
     MIQ_CHECK_ARG(a && deltas && offsets && costs && count && best_index && cap >= 0, "bad argument");
-    if (a->entropy)
+    if (a->entropy || a->mode == MIQ_QUANTIZATION_MSE)
     {
-        set_error("the entropy analyzer has no candidate list");
+        set_error("only the TF-Enhanced analyzer keeps its candidate list");
         return MIQ_ERR_UNSUPPORTED;
     }
     if (int rc = read_state(a, (hipStream_t) stream))
