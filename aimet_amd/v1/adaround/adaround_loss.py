@@ -5,7 +5,6 @@ Same names and values as TrainingExtensions/torch/src/python/aimet_torch/v1/adar
 :113-135).  The optimisation loop itself never evaluates the rounding loss: its gradient is part of the fused backward
 kernel (aimet_amd/csrc/miq_adaround_math.h), which also returns the sum this module's compute_round_loss forms.
 """
-import math
 from dataclasses import dataclass
 from typing import Tuple
 

@@ -14,7 +14,7 @@ from typing import Any, Callable, Tuple, Union
 import torch
 import torch.nn.functional as functional
 
-from ... import ops, utils
+from ... import ops
 from .activation_sampler import ActivationSampler
 from .adaround_loss import AdaroundHyperParameters, AdaroundLoss
 from .adaround_wrapper import AdaroundWrapper

@@ -7,7 +7,6 @@ context, get_min / get_max / get_scale / get_offset / set_range), Quantize (:448
 """
 import contextlib
 import functools
-import math
 import warnings
 import weakref
 from typing import Optional

@@ -14,7 +14,6 @@ from typing import Dict, List, Optional
 
 import numpy as np
 import torch
-from torch import nn
 
 from .... import ops
 from ...utils import StatisticsNotFoundError, patch_attr
