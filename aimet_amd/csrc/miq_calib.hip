@@ -935,15 +935,35 @@ __global__ __launch_bounds__(kBlock) void mse_prepare_kernel(const DevState* st,
     const float hist_min = (float) view.x_left(0);
     const float min_val  = s_range[0];
     const float max_val  = s_range[1] + width;
+    // The two chains of float additions of _minimizeMSE: the walk over the bucket edges (:156-163) and the bucket
+    // centres (:172-183; at most as many centres as edges are used).  The walk ends at the first value above hist_max,
+    // normally the 513th to 515th: kMseFastWalk steps of both chains run without a test on one lane (additions and LDS
+    // stores only), every lane then looks for the first value that ends the walk, and only a walk that has not ended
+    // by then goes on step by step.
+    constexpr int kMseFastWalk = 520;
+    const float hist_max       = (float) (view.x_left(kPdf - 1) + width);
     if (lane == 0)
     {
-        // The two chains of float additions of _minimizeMSE: the walk over the bucket edges (:156-163) and the bucket
-        // centres (:172-183; at most as many centres as edges are used).  Nothing but additions, compares and LDS
-        // stores in the loop.
-        const float hist_max = (float) (view.x_left(kPdf - 1) + width);
-        int walked           = 0;
-        float c              = min_val + width / 2;
-        for (float i = hist_min; i <= hist_max && walked < kMseMaxWalk; i += width, ++walked)
+        float i = hist_min, c = min_val + width / 2;
+        for (int k = 0; k < kMseFastWalk; ++k)
+        {
+            s_walk[k]   = i;
+            s_center[k] = c;
+            i += width;
+            c = c + width;
+        }
+        s_n_walk = kMseFastWalk;
+    }
+    __syncthreads();
+    for (int k = lane; k < kMseFastWalk; k += blockDim.x)
+        if (!(s_walk[k] <= hist_max))
+            atomicMin(&s_n_walk, k);
+    __syncthreads();
+    if (lane == 0 && s_n_walk == kMseFastWalk)
+    {
+        int walked = kMseFastWalk;
+        float c    = s_center[kMseFastWalk - 1] + width;
+        for (float i = s_walk[kMseFastWalk - 1] + width; i <= hist_max && walked < kMseMaxWalk; i += width, ++walked)
         {
             s_walk[walked]   = i;
             s_center[walked] = c;
