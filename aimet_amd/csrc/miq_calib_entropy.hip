@@ -30,6 +30,7 @@ namespace
 constexpr int kBins     = MIQ_PDF_SIZE;
 constexpr int kEntGrid  = 1024;   // workgroups of either streaming pass, at most
 constexpr int kEntBlock = 256;
+constexpr int kEntReplicas = 16;
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 struct EntState
@@ -41,6 +42,11 @@ struct EntState
     float bin_width_f, min_f;   // what getBin takes for the batch in flight
     unsigned long long hist[kBins];
     float2 partial[kEntGrid];
+    // Counts of the batch binned last, not yet added to `hist`: workgroup b of the bin pass adds to replica
+    // b % kEntReplicas.  Atomic adds of many workgroups to one address queue at about 15 ns each; with one set of 512
+    // counters, 1024 workgroups spent 15 us of a 19 us launch there.  Folded into `hist` by the next range kernel and
+    // before the histogram is read.
+    unsigned long long replica[kEntReplicas][kBins];
 };
 constexpr size_t kEntReadBytes = offsetof(EntState, partial);
 
@@ -117,6 +123,29 @@ enum
     kBatchWidens       // widens it: the counts move
 };
 
+// hist[t] += the replicas' counts of bin t, which are cleared (thread t of a 512-thread workgroup)
+__device__ __forceinline__ void fold_replicas(EntState* st, int t)
+{
+    // every load requested before the first is used: a dependent round trip to memory takes 1-2 us
+    unsigned long long part[kEntReplicas];
+#pragma unroll
+    for (int r = 0; r < kEntReplicas; ++r)
+        part[r] = st->replica[r][t];
+    unsigned long long sum = st->hist[t];
+#pragma unroll
+    for (int r = 0; r < kEntReplicas; ++r)
+    {
+        sum += part[r];
+        st->replica[r][t] = 0;
+    }
+    st->hist[t] = sum;
+}
+
+__global__ __launch_bounds__(kBins) void ent_fold_kernel(EntState* st)
+{
+    fold_replicas(st, threadIdx.x);
+}
+
 __global__ __launch_bounds__(kBins) void ent_range_kernel(EntState* st, int groups)
 {
     __shared__ float s_lo[kBins / 64], s_hi[kBins / 64];
@@ -124,6 +153,7 @@ __global__ __launch_bounds__(kBins) void ent_range_kernel(EntState* st, int grou
     __shared__ int s_kind;
     __shared__ double s_range[4];   // old min, old max, new min, new max
     const int t = threadIdx.x;
+    fold_replicas(st, t);   // the batch before this one; thread t alone touches hist[t] until the barriers below
     float lo = INFINITY, hi = -INFINITY;
     for (int k = t; k < groups; k += kBins)
     {
@@ -221,11 +251,13 @@ __global__ __launch_bounds__(kEntBlock) void ent_bin_kernel(const float* __restr
 {
     if (st->skip)
         return;
-    __shared__ unsigned int s_hist[kEntCopies][kBins];
+    // the copies of one bin sit side by side, in different LDS banks: laid out copy after copy, all copies of a bin
+    // share a bank and lanes on different copies still queue
+    __shared__ unsigned int s_hist[kBins * kEntCopies];
     for (int k = threadIdx.x; k < kEntCopies * kBins; k += kEntBlock)
-        (&s_hist[0][0])[k] = 0;
+        s_hist[k] = 0;
     __syncthreads();
-    unsigned int* mine = s_hist[threadIdx.x & (kEntCopies - 1)];
+    unsigned int* mine = s_hist + (threadIdx.x & (kEntCopies - 1));
     const float width = st->bin_width_f, low = st->min_f;
     const int64_t stride = (int64_t) gridDim.x * blockDim.x;
     const int64_t first  = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
@@ -234,27 +266,39 @@ __global__ __launch_bounds__(kEntBlock) void ent_bin_kernel(const float* __restr
     {
         const v4f* d4    = reinterpret_cast<const v4f*>(data);
         const int64_t n4 = n / 4;
-        for (int64_t k = first; k < n4; k += stride)
+        // four loads per lane in flight before the first of them is counted: one load at a time leaves the launch
+        // waiting on memory latency (12.8 us for 25.7 MB)
+        constexpr int kInFlight = 4;
+        for (int64_t k = first; k < n4; k += stride * kInFlight)
         {
-            const v4f v = __builtin_nontemporal_load(d4 + k);
-            atomicAdd(&mine[get_bin(width, low, v.x)], 1u);
-            atomicAdd(&mine[get_bin(width, low, v.y)], 1u);
-            atomicAdd(&mine[get_bin(width, low, v.z)], 1u);
-            atomicAdd(&mine[get_bin(width, low, v.w)], 1u);
+            v4f v[kInFlight];
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u)
+                if (k + u * stride < n4)
+                    v[u] = __builtin_nontemporal_load(d4 + k + u * stride);
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u)
+                if (k + u * stride < n4)
+                {
+                    atomicAdd(&mine[get_bin(width, low, v[u].x) * kEntCopies], 1u);
+                    atomicAdd(&mine[get_bin(width, low, v[u].y) * kEntCopies], 1u);
+                    atomicAdd(&mine[get_bin(width, low, v[u].z) * kEntCopies], 1u);
+                    atomicAdd(&mine[get_bin(width, low, v[u].w) * kEntCopies], 1u);
+                }
         }
         done = n4 * 4;
     }
     for (int64_t k = done + first; k < n; k += stride)
-        atomicAdd(&mine[get_bin(width, low, data[k])], 1u);
+        atomicAdd(&mine[get_bin(width, low, data[k]) * kEntCopies], 1u);
     __syncthreads();
     for (int k = threadIdx.x; k < kBins; k += kEntBlock)
     {
         unsigned int sum = 0;
 #pragma unroll
         for (int c = 0; c < kEntCopies; ++c)
-            sum += s_hist[c][k];
+            sum += s_hist[k * kEntCopies + c];
         if (sum)
-            atomicAdd(&st->hist[k], (unsigned long long) sum);
+            atomicAdd(&st->replica[blockIdx.x % kEntReplicas][k], (unsigned long long) sum);
     }
 }
 
@@ -262,6 +306,8 @@ __global__ void ent_reset_kernel(EntState* st)
 {
     const int t = threadIdx.x;   // launched with kBins threads
     st->hist[t] = 0;
+    for (int r = 0; r < kEntReplicas; ++r)
+        st->replica[r][t] = 0;
     if (t == 0)
     {
         st->min = st->max = 0;
@@ -512,6 +558,8 @@ static int read_back(EntropyAnalyzer* a, hipStream_t s)
     if (a->needs_reset)
         if (int rc = entropy_reset(a, s))
             return rc;
+    hipLaunchKernelGGL(ent_fold_kernel, dim3(1), dim3(kBins), 0, s, a->st);
+    MIQ_CHECK_LAUNCH();
     MIQ_CHECK_HIP(hipMemcpyAsync(a->pinned, a->st, kEntReadBytes, hipMemcpyDeviceToHost, s));
     MIQ_CHECK_HIP(hipStreamSynchronize(s));
     return MIQ_OK;
