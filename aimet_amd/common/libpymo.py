@@ -1,4 +1,5 @@
-"""Value types and enums of the reference's ``_libpymo`` pybind module that the hot path uses.
+"""Value types, enums and the array-fed encoding analyzer of the reference's ``_libpymo`` pybind module that the hot path
+uses.
 
 Mirrors ModelOptimizations/PyModelOptimizations/PyModelOptimizations.cpp:147-177, 232-258 (``TfEncoding`` and the
 enums) with identical field names and integer values (the pure-Python mirror of those values is
@@ -57,3 +58,38 @@ class TensorQuantizerOpMode(enum.Enum):
     oneShotQuantizeDequantize = 1
     quantizeDequantize = 2
     passThrough = 3
+
+
+class EncodingAnalyzerForPython:
+    """An encoding analyzer of any QuantizationMode fed with arrays: updateStats(array, use_cuda) gathers statistics,
+    computeEncoding(bitwidth, isSymmetric, useStrictSymmetric, useUnsignedSymmetric) returns (TfEncoding, is_valid)
+    (ModelOptimizations/DlQuantization/src/EncodingAnalyzerForPython.cpp:53-99, bound at
+    PyModelOptimizations.cpp:216-219).  The reference takes host arrays and computes on the host unless told to copy
+    them to the GPU; here a host array (numpy, or a CPU tensor) is copied to the current GPU, a GPU tensor is used where
+    it is, and `use_cuda` does not change where the statistics are gathered."""
+
+    _MODE_NUMBER = {QuantizationMode.QUANTIZATION_TF: 0, QuantizationMode.QUANTIZATION_TF_ENHANCED: 1,
+                    QuantizationMode.QUANTIZATION_PERCENTILE: 2, QuantizationMode.QUANTIZATION_MSE: 3,
+                    QuantizationMode.QUANTIZATION_ENTROPY: 4}
+
+    def __init__(self, quantizationScheme: QuantizationMode):
+        # every other mode gets the TF analyzer, as in getEncodingAnalyzerInstance (QuantizerFactory.cpp:74-97)
+        self._mode = self._MODE_NUMBER.get(quantizationScheme, 0)
+        self._analyzer = None
+        self._is_encoding_valid = False
+
+    def updateStats(self, input, use_cuda: bool = True):           # pylint: disable=redefined-builtin, unused-argument
+        import torch                                                 # pylint: disable=import-outside-toplevel
+        from .. import ops                                           # pylint: disable=import-outside-toplevel
+        tensor = input if isinstance(input, torch.Tensor) else torch.as_tensor(input)
+        tensor = tensor.detach().to(device="cuda" if not tensor.is_cuda else tensor.device, dtype=torch.float32)
+        if self._analyzer is None or self._analyzer.device != tensor.device:
+            self._analyzer = ops.Analyzer(self._mode, tensor.device)
+        self._is_encoding_valid = True
+        self._analyzer.update_stats(tensor.contiguous())
+
+    def computeEncoding(self, bitwidth: int, isSymmetric: bool, useStrictSymmetric: bool, useUnsignedSymmetric: bool):
+        if not self._is_encoding_valid:
+            return TfEncoding(), False
+        e, _ = self._analyzer.compute_encoding(bitwidth, isSymmetric, useStrictSymmetric, useUnsignedSymmetric)
+        return TfEncoding(e.min, e.max, e.delta, e.offset, e.bw), True

@@ -556,6 +556,39 @@ def test_entropy_scheme_through_the_tensor_quantizer_object(oracle):
     assert valid and (encoding.min, encoding.max, encoding.delta, encoding.offset, encoding.bw) == want.astuple()
 
 
+def test_encoding_analyzer_for_python(oracle):
+    """libpymo.EncodingAnalyzerForPython (PyModelOptimizations.cpp:216-219) with each mode of the factory, fed with a
+    numpy array as the reference's callers feed it: every field of the encoding against the oracle."""
+    from aimet_amd.common import libpymo
+    Mode = libpymo.QuantizationMode
+    rng = np.random.default_rng(12)
+    x = (rng.standard_normal(30000) * 1.5 + 0.25).astype(np.float32)
+    pdf, prof = oracle.new_pdf(), oracle.new_profile()
+    pdf.update(x)
+    prof.update(x)
+    expected = {Mode.QUANTIZATION_TF: oracle.tf_compute_encoding(float(x.min()), float(x.max()), 8),
+                Mode.QUANTIZATION_TF_ENHANCED: pdf.compute_encoding(8)[0],
+                Mode.QUANTIZATION_PERCENTILE: pdf.compute_percentile_encoding(8, 100.0),
+                Mode.QUANTIZATION_MSE: pdf.compute_mse_encoding(8),
+                Mode.QUANTIZATION_ENTROPY: prof.compute_encoding(8)}
+    for mode, want in expected.items():
+        analyzer = libpymo.EncodingAnalyzerForPython(mode)
+        encoding, valid = analyzer.computeEncoding(8, False, False, False)
+        assert not valid and encoding.delta == 0
+        analyzer.updateStats(x, False)
+        encoding, valid = analyzer.computeEncoding(8, False, False, False)
+        assert valid and encoding.bw == 8 and encoding.min <= 0 <= encoding.max
+        assert (encoding.min, encoding.max, encoding.delta, encoding.offset, encoding.bw) == want.astuple(), mode
+    # a mode without an analyzer of its own gets the TF analyzer
+    fallback = libpymo.EncodingAnalyzerForPython(Mode.QUANTIZATION_RANGE_LEARNING)
+    fallback.updateStats(torch.from_numpy(x), True)
+    tf = libpymo.EncodingAnalyzerForPython(Mode.QUANTIZATION_TF)
+    tf.updateStats(_gpu(x), True)
+    a, b = fallback.computeEncoding(8, False, False, False)[0], tf.computeEncoding(8, False, False, False)[0]
+    assert (a.min, a.max, a.delta, a.offset) == (b.min, b.max, b.delta, b.offset)
+    assert a.min <= float(x.min()) and a.max >= float(x.max()) - a.delta
+
+
 def test_percentile_scheme_through_the_v1_quantizers():
     """test_tensor_quantizer / quantsim flow of the reference with quant_scheme = post_training_percentile."""
     from aimet_amd.common import libpymo
