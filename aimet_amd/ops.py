@@ -897,6 +897,34 @@ class _StateOwner:
                 self._state.record_stream(current)
 
 
+# Destroying an analyzer frees pinned host memory (and, for some modes, device memory): calls the HIP runtime refuses
+# while a stream capture is under way -- they invalidate the capture.  The garbage collector can run a destructor in the
+# middle of somebody's `torch.cuda.graph(...)` block, so a handle that dies while the current stream is capturing is
+# parked and destroyed by the next creation or destruction that happens outside a capture.
+_parked_handles = []
+
+
+def _capturing() -> bool:
+    try:
+        return torch.cuda.is_current_stream_capturing()
+    except Exception:                             # pylint: disable=broad-except
+        return False                              # interpreter shutdown, or no usable device any more
+
+
+def _destroy_parked():
+    while _parked_handles and lib is not None:
+        destroy, handle = _parked_handles.pop()
+        destroy(handle)
+
+
+def _destroy_handle(destroy, handle):
+    if _capturing():
+        _parked_handles.append((destroy, handle))
+        return
+    _destroy_parked()
+    destroy(handle)
+
+
 class Analyzer(_StateOwner):
     """Device-resident encoding analyzer: mode 0 = TF min/max, 1 = TF-Enhanced (512-bucket PDF + SQNR search),
     2 = percentile on the same PDF, 3 = least squared error over pairs of bucket edges of the same PDF, 4 = least KL
@@ -910,6 +938,8 @@ class Analyzer(_StateOwner):
         if self.device.index is None:
             self.device = torch.device("cuda", torch.cuda.current_device())
         h = C.c_void_p()
+        if not _capturing():
+            _destroy_parked()
         # the device state comes from torch's caching allocator
         self._init_state(lib.miq_analyzer_state_bytes())
         with torch.cuda.device(self.device):
@@ -919,7 +949,7 @@ class Analyzer(_StateOwner):
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
         if h and lib is not None:                 # at interpreter shutdown the module's globals may already be gone
-            lib.miq_analyzer_destroy(h)
+            _destroy_handle(lib.miq_analyzer_destroy, h)
 
     def _s(self):
         handle = _stream_of(self.device)
@@ -1028,7 +1058,7 @@ class ChannelAnalyzer(_StateOwner):
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
         if h and lib is not None:
-            lib.miq_channel_analyzer_destroy(h)
+            _destroy_handle(lib.miq_channel_analyzer_destroy, h)
 
     def _s(self):
         handle = _stream_of(self.device)

@@ -589,6 +589,36 @@ def test_encoding_analyzer_for_python(oracle):
     assert a.min <= float(x.min()) and a.max >= float(x.max()) - a.delta
 
 
+def test_analyzer_dying_during_a_stream_capture(ops):
+    """Destroying an analyzer frees pinned memory, which the runtime refuses during a stream capture (the capture is
+    invalidated); the garbage collector may run the destructor right there.  A handle that dies while the current
+    stream is capturing is parked and destroyed later."""
+    import gc
+    x = torch.randn(4096, device="cuda")
+    doomed = [ops.Analyzer(mode) for mode in (0, 1, 2, 3, 4)]
+    for analyzer in doomed:
+        analyzer.update_stats(x)
+        analyzer.compute_encoding(8)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        y = x * 2
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = x * 2
+        del doomed, analyzer
+        gc.collect()
+        assert len(ops._parked_handles) == 5
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(y, x * 2)
+    survivor = ops.Analyzer(1)                                                    # outside a capture: parked handles go
+    assert not ops._parked_handles
+    survivor.update_stats(x)
+    assert survivor.compute_encoding(8)[1]
+
+
 def test_percentile_scheme_through_the_v1_quantizers():
     """test_tensor_quantizer / quantsim flow of the reference with quant_scheme = post_training_percentile."""
     from aimet_amd.common import libpymo

@@ -383,3 +383,64 @@ def test_ways_of_running_the_simulation(sim_kind, scheme_name):
         out = sim.model(x)
     out.float().sum().backward()
     assert all(p.grad is None or torch.isfinite(p.grad).all() for p in sim.model.parameters())
+
+
+@pytest.mark.parametrize("sim_kind", ("v1", "v2"))
+@pytest.mark.parametrize("scheme_name", ("post_training_tf", "training_range_learning_with_tf_init"))
+def test_training_step_in_a_hip_graph(sim_kind, scheme_name):
+    """A whole quantization-aware training step -- forward, backward, SGD update of weights and (while they learn) of
+    the ranges -- queues kernels and never waits for the device or allocates outside torch's allocator, so
+    `torch.cuda.graph` can capture it.  Replays are interleaved with eager steps of a copy of the model, which start
+    from the same state and see the same input: after every step the two agree to rounding (the convolutions'
+    backward sums in an order of its own from run to run)."""
+    import copy
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.quantsim import QuantizationSimModel as V1Sim
+    from aimet_amd.v2.quantsim import QuantizationSimModel as V2Sim
+    sim_cls = V1Sim if sim_kind == "v1" else V2Sim
+    torch.manual_seed(0)
+    x = torch.randn(8, 3, 8, 8).cuda()
+    sim = sim_cls(_SmallNet().cuda().eval(), x, quant_scheme=getattr(QuantScheme, scheme_name),
+                  config_file=_PER_CHANNEL)
+    sim.compute_encodings(lambda m, _: m(x), None)
+    in_graph = sim.model.train()
+    eager = copy.deepcopy(in_graph)
+
+    def one_step_of(model):
+        optimizer = torch.optim.SGD([p for p in model.parameters() if p.requires_grad], lr=0.05)
+
+        def step():
+            optimizer.zero_grad(set_to_none=True)
+            loss = model(static_x).float().pow(2).mean()
+            loss.backward()
+            optimizer.step()
+            return loss
+        return step
+    static_x = x.clone()
+    graph_step, eager_step = one_step_of(in_graph), one_step_of(eager)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            graph_step()                                           # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(3):
+        eager_step()
+    before = [p.detach().clone() for p in in_graph.parameters()]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_loss = graph_step()
+    for rep in range(5):
+        static_x.copy_(torch.randn(8, 3, 8, 8).cuda() * (1 + rep))
+        graph.replay()
+        eager_loss = eager_step()
+        torch.cuda.synchronize()
+        assert torch.allclose(static_loss, eager_loss, rtol=1e-4, atol=1e-6), rep
+        for (name, p), q in zip(in_graph.named_parameters(), eager.parameters()):
+            assert torch.allclose(p, q, rtol=1e-4, atol=1e-5), (rep, name)
+    moved = sum(int(not torch.equal(p, b)) for p, b in zip(in_graph.parameters(), before))
+    assert moved >= 4                                               # the replays did train the model
+    if scheme_name.startswith("training_range_learning"):
+        ranges = [(n, p) for n, p in in_graph.named_parameters() if n.endswith(("min", "max"))]
+        assert ranges and any(not torch.equal(p, b) for (n, p), b in
+                              zip(in_graph.named_parameters(), before) if n.endswith(("min", "max")))
