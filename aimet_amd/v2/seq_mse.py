@@ -99,11 +99,22 @@ class SequentialMse(V1SequentialMse):
         quantizer = quant_module.param_quantizers['weight']
         return quantizer.bitwidth if quantizer is not None else 1 << 30    # not quantized: never searched
 
+    _observers = {}
+
     @staticmethod
     def compute_param_encodings(quantizer, x_min: torch.Tensor, x_max: torch.Tensor):
         """min / max of `quantizer` as a fresh min-max quantizer of its geometry sets them on observing x_min, x_max."""
-        observer = QuantizeDequantize(quantizer.shape, quantizer.bitwidth, quantizer.symmetric,
-                                      block_size=quantizer.block_size).to(x_min.device)
+        # one observer per geometry serves every candidate of a search (and the next layer of the same geometry):
+        # building a quantizer module costs more than observing a candidate
+        block_size = None if quantizer.block_size is None else tuple(quantizer.block_size)
+        key = (tuple(quantizer.shape), quantizer.bitwidth, quantizer.symmetric, block_size, x_min.device)
+        observer = SequentialMse._observers.get(key)
+        if observer is None:
+            if len(SequentialMse._observers) >= 8:
+                SequentialMse._observers.clear()
+            observer = SequentialMse._observers[key] = QuantizeDequantize(
+                quantizer.shape, quantizer.bitwidth, quantizer.symmetric,
+                block_size=quantizer.block_size).to(x_min.device)
         with observer.compute_encodings():
             observer(torch.stack([x_min, x_max]))
         with torch.no_grad():
