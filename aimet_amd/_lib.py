@@ -102,6 +102,8 @@ _SIGNATURES = {
     "miq_analyzer_queue_encoding": ([_p, _int, _int, _int, _int, _p], _int),
     "miq_analyzer_compute_encoding": ([_p, _int, _int, _int, _int, C.POINTER(Encoding), C.POINTER(_int), _p], _int),
     "miq_analyzer_get_stats_histogram": ([_p, _p, _p, C.POINTER(_int), _p], _int),
+    "miq_column_error_splits": ([_i64, _i64, _i64], _i64),
+    "miq_column_error_f32": ([_p, _p, _i64, _i64, _i64, _int, _i64, _p, _p], _int),
     "miq_analyzer_entropy_histogram": ([_p, _p, _p, C.POINTER(_int), C.POINTER(_int), _p], _int),
     "miq_analyzer_last_batch_counts": ([_p, _p, _p], _int),
     "miq_analyzer_last_search": ([_p, _p, _p, _p, _int, C.POINTER(_int), C.POINTER(_int), _p], _int),

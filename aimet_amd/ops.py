@@ -535,6 +535,31 @@ def adaround_recon_grad(out, target_all, index, activation):
     return grad
 
 
+# ---------------------------------------------------------------------------------------------------- sequential MSE
+COLUMN_ERROR_SQUARED, COLUMN_ERROR_ABSOLUTE, COLUMN_ERROR_SQUARED_AND_SIGNAL = range(3)
+
+
+def column_error(a, b, kind):
+    """Per block and column, an error between `a` and `b` ([blocks, rows, cols] float32, contiguous) summed over rows,
+    both read once: squared (kind 0) or absolute (kind 1) differences -> [blocks, cols]; kind 2 -> [2, blocks, cols],
+    the squared differences and the squares of `b`."""
+    _require_gpu(a, b)
+    if a.dtype != _F32 or b.dtype != _F32 or a.dim() != 3 or a.shape != b.shape or not a.is_contiguous() \
+            or not b.is_contiguous():
+        raise ValueError("a and b must be contiguous float32 tensors of one shape [blocks, rows, cols]")
+    blocks, rows, cols = a.shape
+    planes = 2 if kind == COLUMN_ERROR_SQUARED_AND_SIGNAL else 1
+    if a.numel() == 0:
+        return a.new_zeros((planes, blocks, cols) if planes == 2 else (blocks, cols))
+    splits = lib.miq_column_error_splits(blocks, rows, cols)
+    partial = torch.empty((splits, planes, blocks, cols), dtype=_F32, device=a.device)
+    with _OnDevice(a.device):
+        check(lib.miq_column_error_f32(_ptr(a), _ptr(b), blocks, rows, cols, int(kind), splits, _ptr(partial),
+                                       _stream(a)))
+    total = partial[0] if splits == 1 else partial.sum(0)
+    return total if planes == 2 else total[0]
+
+
 # ---------------------------------------------------------------------------------------------------- range learning
 RANGE_V2_ASYMMETRIC, RANGE_V2_SYMMETRIC, RANGE_V1_ASYMMETRIC, RANGE_V1_SIGNED_SYMMETRIC, \
     RANGE_V1_UNSIGNED_SYMMETRIC = range(5)

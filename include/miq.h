@@ -690,6 +690,18 @@ int miq_v2_sqnr_search_f32(const float* hist, const float* minmax, int64_t num_h
                            int symmetric, double gamma, int asym_deltas, int sym_deltas, int offset_candidates,
                            float* out_min, float* out_max, double* noise, int32_t* best_index, void* stream);
 
+/* Sequential MSE's loss (SequentialMse.compute_recon_loss, aimet_torch/v1/seq_mse.py:557-581; neg_sqnr :602-615; per
+ * block of input channels in aimet_torch/v2/seq_mse.py:325-357): for two float32 tensors a, b of [blocks, rows, cols]
+ * -- a layer's output with the candidate weight and with the float weight, one slab per block of input channels --
+ * the error summed over rows, per block and column.  kind 0: (a - b)^2.  kind 1: |a - b|.  kind 2: two planes,
+ * (b - a)^2 and b^2, from which the caller forms -10 log10(mean b^2 / (mean (b - a)^2 + eps)).
+ * Rows are cut into `splits` pieces (miq_column_error_splits proposes a count that fills the device) whose sums land in
+ * partial[splits][planes][blocks][cols]; the caller adds the pieces.  Each sum runs over its rows in order: the result
+ * does not change from run to run. */
+int64_t miq_column_error_splits(int64_t blocks, int64_t rows, int64_t cols);
+int miq_column_error_f32(const float* a, const float* b, int64_t blocks, int64_t rows, int64_t cols, int kind,
+                         int64_t splits, float* partial, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

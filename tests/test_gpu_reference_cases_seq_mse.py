@@ -320,3 +320,28 @@ def test_search_lowers_the_output_error():
     before = error()
     optimize_module(wrapper, x, x, SeqMseParams(num_batches=4))
     assert error() < 0.9 * before
+
+
+@pytest.mark.parametrize("shape", [(1, 2048, 4096), (32, 512, 300), (3, 37, 5), (8, 31, 1024), (1, 1, 1)])
+def test_column_error_kernel(shape):
+    """The loss kernel against the tensor expressions of compute_recon_loss / neg_sqnr (reference v1/seq_mse.py
+    :557-581, :602-615): float32 sums in another order, so to rounding."""
+    from aimet_amd import ops
+    from aimet_amd.v1.seq_mse import neg_sqnr
+    torch.manual_seed(sum(shape))
+    a, b = torch.randn(shape).cuda(), torch.randn(shape).cuda()
+    a = b + 0.1 * a
+    squared = ops.column_error(a, b, ops.COLUMN_ERROR_SQUARED)
+    assert squared.shape == (shape[0], shape[2])
+    assert torch.allclose(squared, torch.nn.functional.mse_loss(a, b, reduction="none").sum(1), rtol=2e-5, atol=1e-6)
+    absolute = ops.column_error(a, b, ops.COLUMN_ERROR_ABSOLUTE)
+    assert torch.allclose(absolute, torch.nn.functional.l1_loss(a, b, reduction="none").sum(1), rtol=2e-5, atol=1e-6)
+    noise, signal = ops.column_error(a, b, ops.COLUMN_ERROR_SQUARED_AND_SIGNAL)
+    assert torch.equal(noise, squared)
+    sqnr = -10 * torch.log10((signal / shape[1]) / (noise / shape[1] + 1e-10))
+    for block in range(min(shape[0], 3)):
+        assert torch.allclose(sqnr[block], neg_sqnr(a[block], b[block]).sum(0), rtol=1e-4, atol=1e-4)
+    assert torch.equal(squared, ops.column_error(a, b, ops.COLUMN_ERROR_SQUARED))      # the same from run to run
+    if shape[1] > 1 and shape[2] > 1:
+        with pytest.raises(ValueError):
+            ops.column_error(a.transpose(1, 2), b.transpose(1, 2), 0)                  # not contiguous
