@@ -375,6 +375,78 @@ def bench_calibration(torch, ops, reps):
             "encoding": [enc.min, enc.max, enc.delta, enc.offset]}
 
 
+def bench_seq_mse(torch, ops):
+    """Sequential MSE's search on one Linear [4096, 4096] layer (4 bits, 20 candidates, 4 batches of [512, 4096]
+    inputs) over the v1 wrappers (per channel) and the v2 quantized modules (per channel, and blocks of 128 input
+    channels), beside the GEMMs alone; and the loss kernel on the blockwise search's [32, 512, 4096] products."""
+    from aimet_amd.common.defs import QuantScheme
+    from aimet_amd.v1.qc_quantize_op import StaticGridQuantWrapper
+    from aimet_amd.v1.seq_mse import SeqMseParams, optimize_module
+    from aimet_amd.v2 import seq_mse as v2
+    from aimet_amd.v2.nn import QuantizationMixin
+    from aimet_amd.v2.quantization.affine import QuantizeDequantize
+    dev = torch.device("cuda", 0)
+    torch.manual_seed(1006)
+    layer = torch.nn.Linear(4096, 4096).to(dev)
+    x = torch.randn(4, 512, 4096, device=dev)
+    params = SeqMseParams(num_batches=4)
+
+    def v1_search():
+        wrapper = StaticGridQuantWrapper(layer, 4, 16, 'nearest', QuantScheme.post_training_tf)
+        wrapper.enable_per_channel_quantization()
+        quantizer = wrapper.param_quantizers['weight']
+        quantizer.update_encoding_stats(layer.weight.data)
+        quantizer.compute_encoding()
+        return lambda: optimize_module(wrapper, x, x, params)
+
+    def v2_search(shape, block_size):
+        qmodule = QuantizationMixin.from_module(layer)
+        qmodule.param_quantizers['weight'] = quantizer = QuantizeDequantize(shape, 4, True,
+                                                                            block_size=block_size).to(dev)
+        with quantizer.compute_encodings():
+            quantizer(qmodule.weight.data)
+        return lambda: v2.optimize_module(qmodule, x, x, params)
+
+    def wall_ms(make):
+        make()()                                  # warm-up on a quantizer of its own: a search freezes its quantizer
+        search = make()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        search()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3
+
+    out = {"layer": [4096, 4096], "inputs": [4, 512, 4096], "candidates": 20, "bitwidth": 4,
+           "v1_per_channel_ms": wall_ms(v1_search),
+           "v2_per_channel_ms": wall_ms(lambda: v2_search([4096, 1], None)),
+           "v2_blocks_of_128_ms": wall_ms(lambda: v2_search([4096, 32], [-1, -1]))}
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(84):
+        torch.nn.functional.linear(x[0], layer.weight)
+    torch.cuda.synchronize()
+    out["the_84_gemms_alone_ms"] = (time.perf_counter() - t0) * 1e3
+    a, b = torch.randn(32, 512, 4096, device=dev), torch.randn(32, 512, 4096, device=dev)
+    for kind, name in ((ops.COLUMN_ERROR_SQUARED, "squared"), (ops.COLUMN_ERROR_SQUARED_AND_SIGNAL, "squared_and_signal")):
+        ops.column_error(a, b, kind)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            ops.column_error(a, b, kind)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / 10
+        out[f"column_error_{name}_32x512x4096"] = {"ms": ms, "GBps": 2 * a.numel() * 4 / ms / 1e6,
+                                                   "frac_hbm": 2 * a.numel() * 4 / ms / 1e6 / HBM_PEAK_GBPS}
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        (a - b).square_().sum(1)
+    torch.cuda.synchronize()
+    out["the_same_loss_by_tensor_operations_ms"] = (time.perf_counter() - t0) * 1e3 / 10
+    return out
+
+
 def _adaround_layer(torch, seed=1005, out_features=4096, in_features=4096, rows=2048):
     """cfg5 objects: Linear [4096,4096] fp32, W ~ N(0, 0.02); X [2048,4096] ~ N(0,1); Y = X W^T; 4-bit per-channel."""
     from aimet_amd.common.defs import QuantScheme
@@ -1568,6 +1640,8 @@ def main():
         extra["quantsim_resnet50_shaped"] = bench_quantsim(torch)
     if want("e2e"):
         extra["end_to_end"] = bench_end_to_end(torch, ops)
+    if want("seqmse"):
+        extra["sequential_mse"] = bench_seq_mse(torch, ops)
     if want("adaround"):
         extra["adaround_linear_4096"] = bench_adaround(torch, ops, 1000 if args.only is None else args.steps)
         extra["adaround_linear_4096"]["torch_ops_same_gpu"] = torch_ops_adaround_baseline(torch)
