@@ -436,3 +436,69 @@ def test_v2_grid_representability_is_memoised():
     assert not backend._is_grid_representable(torch.float16, 0, 2 ** 16 - 1)      # 65535 is not a float16
     assert backend._is_grid_representable(torch.bfloat16, -128, 127)
     assert not backend._is_grid_representable(torch.bfloat16, 0, 2 ** 9 - 1)       # 511 needs nine bits
+
+
+def test_checkpointed_flow_helpers_on_plain_modules():
+    """The helpers under apply_adaround_with_cache / checkpointed sequential MSE are tensor plumbing: what a block
+    receives per batch (keyword inputs laid behind the positional ones, host copies when asked), a block's outputs
+    handed on as the next block's inputs with and without the static inputs, and the cut of a model's layers into runs
+    per named block."""
+    from types import SimpleNamespace
+
+    from aimet_amd import utils
+    from aimet_amd.v1.adaround import activation_sampler as sampler
+
+    class Scaled(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc = nn.Linear(6, 6)
+
+        def forward(self, x, scale=None, shift=1.0):
+            return self.fc(x) * scale + shift, scale
+
+    class Stack(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.first, self.block_a, self.between, self.block_b = nn.Linear(6, 6), Scaled(), nn.Linear(6, 6), Scaled()
+
+        def forward(self, x, scale):
+            x, _ = self.block_a(self.first(x), scale=scale)
+            return self.block_b(self.between(x), scale=scale)[0]
+
+    torch.manual_seed(0)
+    model = Stack().eval()
+    other = Stack().eval()                                          # stands in for the simulation model
+    x, scale = torch.randn(3, 6), torch.full((3, 1), 2.0)
+    batches = [(x, scale), (x + 1, scale)]
+    forward = lambda m, batch: m(*batch)
+
+    assert utils.add_foward_fn_kwargs_to_inputs(model.block_a, x, scale=scale) == (x, scale, 1.0)
+    assert utils.add_foward_fn_kwargs_to_inputs(model.block_a, x, scale, 3.0) == (x, scale, 3.0)
+
+    fp_in, q_in = sampler.get_block_inputs(model, SimpleNamespace(model=other), "block_a", batches, True, forward, 2,
+                                           None, incl_kwargs=True)
+    assert len(fp_in) == len(q_in) == 2 and len(fp_in[0]) == 3
+    assert torch.equal(fp_in[1][0], model.first(x + 1)) and torch.equal(q_in[1][0], other.first(x + 1))
+    assert torch.equal(fp_in[0][1], scale) and fp_in[0][2] == 1.0
+    without_keywords = utils.cache_intermediate_datasets(batches, True, model, "block_a", forward)
+    assert len(without_keywords[0]) == 1                            # positional inputs only
+    model.unused = nn.Linear(6, 6)
+    with pytest.raises(RuntimeError):
+        utils.cache_intermediate_datasets(batches, True, model, "unused", forward)
+    del model.unused
+
+    fp_blocks, q_blocks = sampler.create_modulelist_for_group_modules(model, SimpleNamespace(model=other),
+                                                                      {"a": ["block_a"], "b": ["between"]})
+    assert fp_blocks[0][0] is model.block_a and q_blocks[1][0] is other.between
+    expected = model.block_a(*fp_in[0])[0]
+    run = lambda block, inputs: block[0](*inputs)
+    sampler.get_block_outputs(fp_blocks[0], q_blocks[0], "True", fp_in, q_in, True, run, torch.device("cpu"))
+    assert torch.equal(fp_in[0][0], expected) and len(fp_in[0]) == 3 and torch.equal(fp_in[0][1], scale)
+    fp_next, q_next = [[t[0]] for t in fp_in], [[t[0]] for t in q_in]
+    sampler.get_block_outputs(fp_blocks[1], q_blocks[1], "False", fp_next, q_next, True, run, torch.device("cpu"))
+    assert len(q_next[0]) == 1 and torch.equal(q_next[0][0], other.between(q_in[0][0]))
+    assert torch.equal(fp_next[1][0], model.between(fp_in[1][0]))
+
+    schedule = sampler.create_cached_block_schedule_list(model, (x, scale), ["block_a", "block_b"], (nn.Linear,))
+    assert [(b if b is None else b[0], [n for n, _ in layers]) for b, layers in schedule] == \
+        [(None, ["first"]), ("block_a", ["fc"]), (None, ["between"]), ("block_b", ["fc"])]
