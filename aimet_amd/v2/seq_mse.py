@@ -252,6 +252,33 @@ class SequentialMse(V1SequentialMse):
         return losses
 
     @classmethod
+    def _conv_candidate_losses(cls, quant_module, x, xq, params, candidates):
+        """For a convolution: `_compute_loss` per candidate and batch, with the float side -- the partial outputs of
+        every block of input channels, which no candidate changes -- formed once per batch while it fits."""
+        block = cls._get_input_channel_block_size(quant_module)
+        w = quant_module.weight.detach()
+        batches = range(params.num_batches)
+        parts = lambda t: torch.split(t, block, dim=-3)
+        w_parts = torch.split(w, block, dim=1)
+        outputs = lambda inputs, weights: [cls._layer_output(quant_module, i, k) for i, k in zip(inputs, weights)]
+        first = outputs(parts(x[0]), w_parts)
+        kept_bytes = sum(o.numel() for o in first) * w.element_size() * params.num_batches
+        keep = kept_bytes <= cls._FLOAT_PRODUCTS_BYTES
+        kept = [first] + [outputs(parts(x[b]), w_parts) for b in batches[1:]] if keep else None
+        del first
+        losses = []
+        for _ in candidates:
+            wq_parts = torch.split(cls._get_quantized_weight(quant_module), block, dim=1)
+            loss = None
+            for b in batches:
+                targets = kept[b] if keep else outputs(parts(x[b]), w_parts)
+                part = torch.stack([cls.compute_recon_loss(got, want, params)
+                                    for got, want in zip(outputs(parts(xq[b]), wq_parts), targets)], dim=-1)
+                loss = part if loss is None else loss.add_(part)
+            losses.append(loss)
+        return losses
+
+    @classmethod
     def optimize_module(cls, quant_module: BaseQuantizationMixin, x: torch.Tensor, xq: torch.Tensor,
                         params: SeqMseParams):
         quantizer = quant_module.param_quantizers['weight']
@@ -267,15 +294,8 @@ class SequentialMse(V1SequentialMse):
             with torch.no_grad():
                 total_loss = cls._linear_candidate_losses(quant_module, x, xq, params, candidates())
         else:
-            total_loss = []
-            for _ in candidates():
-                w = quant_module.weight
-                with torch.no_grad():
-                    wq = cls._get_quantized_weight(quant_module)
-                    loss = cls._compute_loss(quant_module, x[0], xq[0], w, wq, params)
-                    for b in range(1, params.num_batches):
-                        loss += cls._compute_loss(quant_module, x[b], xq[b], w, wq, params)
-                total_loss.append(loss)
+            with torch.no_grad():
+                total_loss = cls._conv_candidate_losses(quant_module, x, xq, params, candidates())
         best = torch.stack(total_loss).min(0)[1]                     # [output channels, blocks]
         block = cls._get_input_channel_block_size(quant_module)
         if block != quant_module.weight.shape[1]:
