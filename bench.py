@@ -1583,7 +1583,7 @@ def main():
     ap.add_argument("--full", action="store_true", help="(kept for old command lines: every cell is measured anyway)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default=None,
-                    help="run a subset of the legs, comma separated (main|pt|fp8|calib|chcalib|sqnr|learn|quantsim|e2e|adaround|floors|copyref), for profiling")
+                    help="run a subset of the legs, comma separated (main|pt|fp8|calib|chcalib|sqnr|learn|quantsim|e2e|seqmse|adaround|floors|copyref), for profiling")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
