@@ -112,10 +112,8 @@ class MinMaxQuantizer(_GridMixin, QuantizerBase):
             raise RuntimeError(f'Encoding analyzer of shape {self.encoding_analyzer.observer.shape} '
                                f'is incompatible with quantizer of shape {self.shape}.')
         self._initial_parameters = {}
-        self.min = nn.Parameter(-torch.ones(self.shape))
-        self.max = nn.Parameter(torch.ones(self.shape))
-        self._remember_initial('min', self.min)
-        self._remember_initial('max', self.max)
+        self.register_quantization_parameter('min', nn.Parameter(-torch.ones(self.shape)))
+        self.register_quantization_parameter('max', nn.Parameter(torch.ones(self.shape)))
         self._allow_overwrite = True
 
     # ---------------------------------------------------------------------------------------------- properties
@@ -131,6 +129,12 @@ class MinMaxQuantizer(_GridMixin, QuantizerBase):
 
     # A parameter counts as initialised once it is no longer the untouched object it was created as: it has been
     # assigned anew, or modified in place (its version counter moved) -- reference base/quantizer.py:100-140.
+    def register_quantization_parameter(self, name: str, param: nn.Parameter):
+        """A parameter of the module whose initialisation is tracked (reference base/quantizer.py:99-107); min and max
+        are registered this way, and a subclass may add its own."""
+        self.register_parameter(name, param)
+        self._remember_initial(name, getattr(self, name))
+
     def _remember_initial(self, name: str, param: nn.Parameter):
         self._initial_parameters[name] = (weakref.ref(param), param._version)  # pylint: disable=protected-access
 
@@ -143,18 +147,18 @@ class MinMaxQuantizer(_GridMixin, QuantizerBase):
         return not (current is initial and current._version == initial_version)  # pylint: disable=protected-access
 
     def is_initialized(self) -> bool:
-        return all(self._is_initialized(name) for name in ('min', 'max'))
+        return all(self._is_initialized(name) for name in self._initial_parameters)
 
     def allow_overwrite(self, mode: bool):
         """With False, compute_encodings() leaves the current parameters alone."""
         self._allow_overwrite = mode
 
     def get_extra_state(self):
-        return {name: torch.tensor(self._is_initialized(name)) for name in ('min', 'max')}
+        return {name: torch.tensor(self._is_initialized(name)) for name in self._initial_parameters}
 
     @torch.no_grad()
     def set_extra_state(self, state):
-        for name in ('min', 'max'):
+        for name in list(self._initial_parameters):
             if bool(state.get(name, False)):
                 self._initial_parameters[name] = (None, -1)
             else:
@@ -162,7 +166,7 @@ class MinMaxQuantizer(_GridMixin, QuantizerBase):
 
     def __getstate__(self):
         state = self.__dict__.copy()
-        state['_initial_parameters'] = {name: self._is_initialized(name) for name in ('min', 'max')}
+        state['_initial_parameters'] = {name: self._is_initialized(name) for name in self._initial_parameters}
         state.pop('_kept_encoding', None)
         return state
 

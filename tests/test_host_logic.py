@@ -502,3 +502,28 @@ def test_checkpointed_flow_helpers_on_plain_modules():
     schedule = sampler.create_cached_block_schedule_list(model, (x, scale), ["block_a", "block_b"], (nn.Linear,))
     assert [(b if b is None else b[0], [n for n, _ in layers]) for b, layers in schedule] == \
         [(None, ["first"]), ("block_a", ["fc"]), (None, ["between"]), ("block_b", ["fc"])]
+
+
+def test_v2_quantization_parameters_registered_by_a_subclass():
+    """register_quantization_parameter (reference v2/quantization/base/quantizer.py:99-135): a parameter registered
+    this way counts towards is_initialized(), travels in the extra state, and survives copies and pickles."""
+    import copy
+    import pickle
+    from aimet_amd.v2.quantization.affine import QuantizeDequantize
+    quantizer = QuantizeDequantize((), 8, False)
+    quantizer.register_quantization_parameter('gamma', nn.Parameter(torch.ones(())))
+    assert sorted(dict(quantizer.named_parameters())) == ['gamma', 'max', 'min']
+    with torch.no_grad():
+        quantizer.min.fill_(-1.)
+        quantizer.max.fill_(2.)
+    assert not quantizer.is_initialized()                           # gamma is still the object it was created as
+    with torch.no_grad():
+        quantizer.gamma.mul_(1.)
+    assert quantizer.is_initialized()
+    assert sorted(quantizer.get_extra_state()) == ['gamma', 'max', 'min']
+    assert copy.deepcopy(quantizer).is_initialized() and pickle.loads(pickle.dumps(quantizer)).is_initialized()
+    fresh = QuantizeDequantize((), 8, False)
+    fresh.register_quantization_parameter('gamma', nn.Parameter(torch.ones(())))
+    assert not fresh.is_initialized()
+    fresh.load_state_dict(quantizer.state_dict())
+    assert fresh.is_initialized() and float(fresh.max.detach()) == 2.0
