@@ -300,7 +300,9 @@ class QcQuantizeWrapper(nn.Module):
             if encoding[0]['dtype'] == 'int':
                 self._apply_int_encoding(quantizer, encoding, strict)
             elif encoding[0]['dtype'] == 'float':
-                raise RuntimeError("float encodings are not implemented")
+                # a float entry carries no range: the quantizer casts to the float type of that many bits
+                quantizer.bitwidth = encoding[0]['bitwidth']
+                quantizer.data_type = QuantizationDataType.float
             else:
                 raise RuntimeError("Data type does not match int or float in encodings file")
             self._finish_import(quantizer, requires_grad, allow_overwrite)
@@ -329,7 +331,8 @@ class QcQuantizeWrapper(nn.Module):
             if encoding['dtype'] == 'int':
                 self._apply_int_encoding(quantizer, [encoding], strict)
             elif encoding['dtype'] == 'float':
-                raise RuntimeError("float encodings are not implemented")
+                quantizer.bitwidth = encoding['bitwidth']
+                quantizer.data_type = QuantizationDataType.float
             else:
                 raise RuntimeError("Unrecognized encodings datatype")
             self._finish_import(quantizer, requires_grad, allow_overwrite)

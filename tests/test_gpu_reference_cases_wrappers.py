@@ -429,3 +429,39 @@ def test_standalone_quantize_op(api):
     assert op(y) is y
     op.set_output_bw(4)
     assert op.output_quantizers[0].bitwidth == 4
+
+
+def test_float_entries_of_an_encodings_file_round_trip(api, tmp_path):
+    """Float quantizers export {'bitwidth', 'dtype': 'float'} and nothing else; importing such an entry turns the
+    quantizer into a float quantizer of that bitwidth (reference v1/qc_quantize_op.py:555-563, 655-663)."""
+    import json
+    from aimet_amd.v1.quantsim import QuantizationSimModel
+    torch.manual_seed(0)
+    model = torch.nn.Sequential(torch.nn.Linear(16, 16), torch.nn.ReLU(), torch.nn.Linear(16, 4)).to(DEV).eval()
+    x = torch.randn(8, 16, device=DEV)
+    in_fp16 = QuantizationSimModel(model, x, quant_scheme=api.QuantScheme.post_training_tf, default_output_bw=16,
+                                   default_param_bw=16, default_data_type=api.QuantizationDataType.float)
+    in_fp16.compute_encodings(lambda m, _: m(x), None)
+    in_fp16.export(str(tmp_path), "fp16", x)
+    with open(tmp_path / "fp16_torch.encodings") as f:
+        exported = json.load(f)
+    entries = [e for group in (exported["activation_encodings"], exported["param_encodings"])
+               for value in group.values() for e in _flat_entries(value)]
+    assert entries and all(e == {"bitwidth": 16, "dtype": "float"} for e in entries)
+
+    in_int8 = QuantizationSimModel(model, x, quant_scheme=api.QuantScheme.post_training_tf)
+    in_int8.compute_encodings(lambda m, _: m(x), None)
+    assert not torch.equal(in_int8.model(x), in_fp16.model(x))
+    in_int8.load_encodings(str(tmp_path / "fp16_torch.encodings"), strict=False, partial=True)
+    turned = [q for _, w in in_int8.quant_wrappers() for q in (*w.output_quantizers, *w.param_quantizers.values())
+              if q.enabled and q.data_type == api.QuantizationDataType.float]
+    assert turned and all(q.bitwidth == 16 for q in turned)
+    assert torch.equal(in_int8.model(x), in_fp16.model(x))
+
+
+def _flat_entries(value):
+    if isinstance(value, dict):
+        if "dtype" in value:
+            return [value]
+        return [e for v in value.values() for e in _flat_entries(v)]
+    return [e for v in value for e in _flat_entries(v)]
