@@ -739,6 +739,15 @@ class QuantizationSimModel:
         exported = self.get_encodings_dict()
         return exported['activation_encodings'], exported['param_encodings']
 
+    def export_weights_to_safetensors(self, path: str, filename_prefix: str):
+        """The state dictionary of the model without its quantization wrappers, as `<path>/<prefix>.safetensors`
+        (reference :660-678; metadata from the model's `mpp_meta` attribute when it has one)."""
+        from safetensors.torch import save_file               # pylint: disable=import-outside-toplevel
+        plain = QuantizationSimModel.get_original_model(self.model)
+        tensors = {name: value.detach().cpu().contiguous() for name, value in plain.state_dict().items()}
+        metadata = {str(k): str(v) for k, v in getattr(self.model, 'mpp_meta', {}).items()}
+        save_file(tensors, os.path.join(path, filename_prefix + '.safetensors'), metadata=metadata or None)
+
     def save_encodings_to_json(self, path: str, filename_prefix: str):
         """<path>/<filename_prefix>.json with the activation and parameter encodings (reference quantsim.py:680-690)."""
         activation_encodings, param_encodings = self.get_activation_param_encodings()

@@ -444,3 +444,27 @@ def test_training_step_in_a_hip_graph(sim_kind, scheme_name):
         ranges = [(n, p) for n, p in in_graph.named_parameters() if n.endswith(("min", "max"))]
         assert ranges and any(not torch.equal(p, b) for (n, p), b in
                               zip(in_graph.named_parameters(), before) if n.endswith(("min", "max")))
+
+
+@pytest.mark.parametrize("sim_kind", ("v1", "v2"))
+def test_weights_to_safetensors(sim_kind, tmp_path):
+    """export_weights_to_safetensors (reference v1/quantsim.py:660-678): the plain model's state dictionary, names
+    and values, with the model's `mpp_meta` as metadata."""
+    from safetensors import safe_open
+    from safetensors.torch import load_file
+    from aimet_amd.v1.quantsim import QuantizationSimModel as V1Sim
+    from aimet_amd.v2.quantsim import QuantizationSimModel as V2Sim
+    torch.manual_seed(0)
+    x = torch.randn(4, 3, 8, 8).cuda()
+    model = _SmallNet().cuda().eval()
+    sim = (V1Sim if sim_kind == "v1" else V2Sim)(model, x, config_file=_PER_CHANNEL)
+    sim.compute_encodings(lambda m, _: m(x), None)
+    sim.model.mpp_meta = {"precision": "w8a8"}
+    sim.export_weights_to_safetensors(str(tmp_path), "weights")
+    stored = load_file(str(tmp_path / "weights.safetensors"))
+    expected = model.state_dict()
+    assert set(stored) == set(expected)
+    for name, value in expected.items():
+        assert torch.equal(stored[name], value.cpu()), name
+    with safe_open(str(tmp_path / "weights.safetensors"), framework="pt") as f:
+        assert f.metadata() == {"precision": "w8a8"}
